@@ -1,0 +1,171 @@
+/*
+ * ttq.h -- C ABI of libttq_hip.so: quantized-weight linear layer for AMD MI355X (gfx950).
+ *
+ * Drop-in boundary for the linear layer of the tattletale inference framework.  The
+ * reference operator is
+ *     Linear{weight (out,in), bias?, in_features, out_features}, init(weight, bias),
+ *     forward(x: (..., in)) -> (..., out)          workspace/transformers/src/layers/linear.nim:13-57
+ * whose arithmetic is one FFI call
+ *     torch::nn::functional::linear(input, weight[, bias])
+ *                                                  workspace/libtorch/src/abi/neural_nets.nim:64-81
+ * Each entry point below cites the reference interface it stands in for.  The reference
+ * binds C libraries with `{.pragma: x, importc: "prefix_$1", cdecl, dynlib: lib.}`
+ * (workspace/pcre2/pcre2.nim:376-384); every symbol here is plain C, `ttq_` prefixed and
+ * takes raw pointers and sizes only, so it binds the same way.
+ *
+ * Conventions
+ *   - All device pointers are HIP device memory on the current device; the library keeps
+ *     no pointer after a call returns (work may still be in flight on `stream`).
+ *   - `stream` is a hipStream_t passed as void*; NULL = the default stream.  Launches are
+ *     asynchronous; the caller synchronises (same contract as a torch tensor op).
+ *   - Return value: 0 on success, a negative ttq_status otherwise.  No C++ exception
+ *     crosses this boundary.
+ *   - Weights are (n_out, n_in) row-major; quantization blocks run along n_in.
+ *   - Base pointers must be 16-byte aligned (torch allocations are).
+ */
+#ifndef TTQ_H
+#define TTQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TTQ_VERSION 100 /* 0.1.0 */
+
+/* Exported symbols: the library is built with hidden visibility by default. */
+#if defined(TTQ_BUILD)
+#define TTQ_API __attribute__((visibility("default")))
+#else
+#define TTQ_API
+#endif
+
+typedef enum {
+  TTQ_OK = 0,
+  TTQ_ERR_NULL = -1,        /* a required pointer is NULL */
+  TTQ_ERR_SHAPE = -2,       /* dimension not positive / not a multiple of the block size */
+  TTQ_ERR_ALIGN = -3,       /* base pointer not 16-byte aligned */
+  TTQ_ERR_DTYPE = -4,       /* unknown or unsupported dtype code */
+  TTQ_ERR_FORMAT = -5,      /* unknown format / bits / codebook */
+  TTQ_ERR_UNSUPPORTED = -6, /* valid request outside what the kernels cover (size limits) */
+  TTQ_ERR_HIP = -7          /* a HIP runtime call failed; see ttq_last_hip_error() */
+} ttq_status;
+
+/* Element types of activation / output / bias buffers.  They correspond to the
+ * reference's ScalarKind members kFloat32, kFloat16, kBfloat16
+ * (workspace/libtorch/src/abi/torch_tensors.nim:114-130). */
+typedef enum { TTQ_F32 = 0, TTQ_F16 = 1, TTQ_BF16 = 2 } ttq_dtype;
+
+typedef enum { TTQ_Q8_0 = 0, TTQ_Q4_K = 1, TTQ_Q6_K = 2, TTQ_EXL3 = 3 } ttq_format;
+
+/* Codebook functions of the trellis format. */
+typedef enum { TTQ_CB_3INST = 0, TTQ_CB_MCG = 1 } ttq_codebook;
+
+/* ---- library ---------------------------------------------------------------------- */
+
+TTQ_API int ttq_version(void);
+TTQ_API const char* ttq_strerror(int status);
+/* hipError_t value of the most recent failed HIP call on this thread (0 if none). */
+TTQ_API int ttq_last_hip_error(void);
+
+/* Bytes of the packed weight buffer for an (n_out, n_in) matrix; negative status on bad
+ * arguments.  `bits` is used by TTQ_EXL3 only (1..8).  Replaces weight.nbytes of the dense
+ * tensor (workspace/libtorch/src/abi/torch_tensors.nim:192). */
+TTQ_API int64_t ttq_packed_nbytes(int format, int64_t n_out, int64_t n_in, int bits);
+
+/* ---- the operator ----------------------------------------------------------------- */
+
+/* Plain-data description of one quantized linear layer: the quantized counterpart of the
+ * reference's `Linear` object (linear.nim:13-27).  All pointers are device pointers owned
+ * by the caller. */
+typedef struct ttq_qlinear {
+  int32_t format;        /* ttq_format */
+  int32_t bits;          /* TTQ_EXL3: bits per weight (1..8); otherwise ignored */
+  int32_t codebook;      /* TTQ_EXL3: ttq_codebook; otherwise ignored */
+  int32_t bias_dtype;    /* ttq_dtype of `bias`; ignored when bias is NULL */
+  int64_t n_out;         /* out_features */
+  int64_t n_in;          /* in_features */
+  const void* qweight;   /* packed blocks (Q8_0/Q4_K/Q6_K) or trellis words (EXL3) */
+  const void* suh;       /* TTQ_EXL3: n_in fp16 input sign/scale vector, else NULL */
+  const void* svh;       /* TTQ_EXL3: n_out fp16 output sign/scale vector, else NULL */
+  const void* bias;      /* n_out values or NULL (linear.nim:26, Option[TorchTensor]) */
+} ttq_qlinear;
+
+/* y = x * W^T (+ bias) for x of shape (m, n_in), y of shape (m, n_out).
+ * Replaces Linear.forward (linear.nim:45-57) and the F.linear call under it
+ * (neural_nets.nim:64,73).  m == 1 runs the decode GEMV; m > 1 runs the prefill GEMM
+ * (MFMA kernel for Q4_K with bf16 activations, a batched GEMV otherwise) -- the same
+ * split the reference makes implicitly through x.size(1) (attn.nim:154-156). */
+TTQ_API int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int64_t m,
+                       void* y, int y_dtype, void* stream);
+
+/* ---- decode GEMV, one entry per block format (m rows of x, normally m == 1) -------- */
+/* y[m][n_out] (fp32) = x[m][n_in] * W^T.  Stand in for F.linear(x, weight) with a
+ * (1, n_in) activation (neural_nets.nim:64). */
+TTQ_API int ttq_gemv_q8_0(const void* w, const void* x, int x_dtype, float* y, int64_t m,
+                  int64_t n_out, int64_t n_in, void* stream);
+TTQ_API int ttq_gemv_q4_k(const void* w, const void* x, int x_dtype, float* y, int64_t m,
+                  int64_t n_out, int64_t n_in, void* stream);
+TTQ_API int ttq_gemv_q6_k(const void* w, const void* x, int x_dtype, float* y, int64_t m,
+                  int64_t n_out, int64_t n_in, void* stream);
+
+/* EXL3-style trellis GEMV: y = svh o H( T * H(suh o x) ), fp16 activations, fp32 output.
+ * n_in and n_out must be multiples of 128 (Hadamard groups). */
+TTQ_API int ttq_gemv_exl3(const uint16_t* trellis, const uint16_t* suh_f16, const uint16_t* svh_f16,
+                  const uint16_t* x_f16, float* y, int64_t m, int64_t n_out, int64_t n_in,
+                  int bits, int codebook, void* stream);
+
+/* ---- prefill GEMM ------------------------------------------------------------------ */
+/* Y[m][n_out] (bf16) = X[m][n_in] (bf16) * W^T, Q4_K weights dequantized to bf16 tiles and
+ * multiplied with bf16 MFMA, fp32 accumulation.  Stands in for F.linear(x, weight) with a
+ * (batch*seq, n_in) activation (neural_nets.nim:64; attn.nim:154-156 prefill case). */
+TTQ_API int ttq_gemm_q4_k(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m,
+                  int64_t n_out, int64_t n_in, void* stream);
+
+/* ---- device dequantizers (the bit-exactness contract made observable) -------------- */
+/* out[n_out][n_in] in `out_dtype`: TTQ_F32 gives the canonical values; TTQ_BF16 gives them
+ * rounded to nearest-even, i.e. exactly what the GEMM feeds to the matrix cores.  These
+ * produce the dense weight the reference's Linear would have held (linear.nim:19). */
+TTQ_API int ttq_dequant_q8_0(const void* w, void* out, int out_dtype, int64_t n_out, int64_t n_in, void* stream);
+TTQ_API int ttq_dequant_q4_k(const void* w, void* out, int out_dtype, int64_t n_out, int64_t n_in, void* stream);
+TTQ_API int ttq_dequant_q6_k(const void* w, void* out, int out_dtype, int64_t n_out, int64_t n_in, void* stream);
+/* Decoded (unscaled, unrotated) trellis values as fp16, shape (n_out, n_in). */
+TTQ_API int ttq_dequant_exl3(const uint16_t* trellis, uint16_t* out_f16, int64_t n_out, int64_t n_in,
+                     int bits, int codebook, void* stream);
+/* In-place orthonormal 128-group Hadamard transform of n fp32 values, optionally
+ * multiplying by an fp16 vector before (pre) and/or after (post) the transform. */
+TTQ_API int ttq_hadamard128_f32(float* v, const uint16_t* pre_f16, const uint16_t* post_f16,
+                        int64_t n, void* stream);
+
+/* ---- host-side preparation (CPU code; no GPU needed) ------------------------------- */
+/* Weight preparation happens once at load time, off the hot path; the reference's
+ * counterpart is building the dense weight tensor handed to Linear.init (linear.nim:29-43,
+ * mlp.nim:39-41).  All pointers here are HOST pointers. */
+
+/* Counter-based normal generator: out[i] = sigma * N(0,1) drawn from (seed, stream, i).
+ * Identical bytes on every machine with the same libm. */
+TTQ_API int ttq_host_fill_normal(uint64_t seed, uint64_t stream, float sigma, float* out, int64_t n);
+
+TTQ_API int ttq_host_quantize_q8_0(const float* w, void* out, int64_t n_out, int64_t n_in);
+TTQ_API int ttq_host_quantize_q4_k(const float* w, void* out, int64_t n_out, int64_t n_in);
+TTQ_API int ttq_host_quantize_q6_k(const float* w, void* out, int64_t n_out, int64_t n_in);
+/* Rotates and trellis-encodes w (n_out, n_in).  Writes trellis words
+ * [n_in/16][n_out/16][16*bits], suh (n_in fp16 signs drawn from `seed`) and svh (n_out
+ * fp16: sign * per-channel scale).  Encoder is a greedy search; only the decoder is a
+ * format contract. */
+TTQ_API int ttq_host_quantize_exl3(const float* w, uint16_t* trellis, uint16_t* suh_f16,
+                           uint16_t* svh_f16, int64_t n_out, int64_t n_in, int bits,
+                           int codebook, uint64_t seed);
+
+/* fp32 <-> 16-bit conversions, round-to-nearest-even. */
+TTQ_API int ttq_host_f32_to_bf16(const float* in, uint16_t* out, int64_t n);
+TTQ_API int ttq_host_f32_to_f16(const float* in, uint16_t* out, int64_t n);
+TTQ_API int ttq_host_bf16_to_f32(const uint16_t* in, float* out, int64_t n);
+TTQ_API int ttq_host_f16_to_f32(const uint16_t* in, float* out, int64_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TTQ_H */

@@ -1,0 +1,439 @@
+/*
+ * ttq_oracle.c -- CPU restatement of the quantized-linear path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This file is the checker for the HIP library, never the thing shipped or measured
+ * (except as the explicitly labelled CPU baseline).  Only tests, the smoke check and the
+ * CPU-baseline leg of the benchmark may load it.
+ *
+ * What it restates
+ *   - the operator semantics of the reference's linear layer, y = x * W^T (+ bias), with
+ *     weight (out_features, in_features) row-major:
+ *       /root/reference/workspace/transformers/src/layers/linear.nim:13-57
+ *       /root/reference/workspace/libtorch/src/abi/neural_nets.nim:64-81
+ *   - the block formats Q8_0 / Q4_K / Q6_K and the trellis-coded EXL3-style format.  The
+ *     reference snapshot holds NO implementation of these (only a quantization_config
+ *     JSON fixture, workspace/transformers/tests/fixtures/configs/
+ *     config-GLM-4.7-EXL3-3.84bpw.json:43-54), so the layouts below restate the public
+ *     ggml block layouts and a QTIP-style bit-shift trellis.  Parity with ggml and with
+ *     exllamav3 themselves is UNPINNED (neither is installed nor vendored); what is
+ *     pinned, and how, is listed per function.
+ *
+ * Canonical dequantisation arithmetic (the bit-exactness contract): every '*' and '-'
+ * is a separately rounded IEEE-754 binary32 operation, evaluated as written.  Compile
+ * with -ffp-contract=off.
+ *
+ * Pinning summary (tests/test_oracle_*.py):
+ *   f16/bf16 converters   exhaustive 65536 patterns vs numpy float16 / bit shifts
+ *   Q8_0/Q4_K/Q6_K        hand-computed known answers, brute-force scale pack/unpack
+ *                         round trip, bit-exact agreement with an independent
+ *                         vectorised closed-form restatement (oracle/np_oracle.py)
+ *   FWHT-128              scipy.linalg.hadamard, involution, norm preservation
+ *   trellis decode        brute force on one tile via python big-int bit arithmetic
+ *   codebooks             closed-form numpy restatement over all 65536 states
+ *   GEMV / GEMM           numpy float64 matmul on the dequantised weights
+ */
+#include <stdint.h>
+#include <stddef.h>
+#include <string.h>
+#include <math.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORA_API __attribute__((visibility("default")))
+
+/* ------------------------------------------------------------------ scalar converters */
+
+ORA_API float ora_f16_to_f32(uint16_t h) {
+  uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  uint32_t exp = (h >> 10) & 0x1Fu;
+  uint32_t man = h & 0x3FFu;
+  uint32_t bits;
+  if (exp == 0) {
+    if (man == 0) {
+      bits = sign;
+    } else { /* subnormal: normalise */
+      int e = -1;
+      do { man <<= 1; e++; } while (!(man & 0x400u));
+      man &= 0x3FFu;
+      bits = sign | ((uint32_t)(127 - 15 - e) << 23) | (man << 13);
+    }
+  } else if (exp == 31) {
+    bits = sign | 0x7F800000u | (man << 13);
+  } else {
+    bits = sign | ((exp + 127 - 15) << 23) | (man << 13);
+  }
+  float f; memcpy(&f, &bits, 4); return f;
+}
+
+/* round-to-nearest-even binary32 -> binary16 */
+ORA_API uint16_t ora_f32_to_f16(float f) {
+  uint32_t x; memcpy(&x, &f, 4);
+  uint32_t sign = (x >> 16) & 0x8000u;
+  uint32_t ax = x & 0x7FFFFFFFu;
+  if (ax >= 0x7F800000u) { /* inf / nan */
+    return (uint16_t)(sign | 0x7C00u | ((ax > 0x7F800000u) ? (0x200u | ((ax >> 13) & 0x3FFu)) : 0));
+  }
+  if (ax >= 0x477FF000u) { /* rounds to >= 65520 -> inf */
+    return (uint16_t)(sign | 0x7C00u);
+  }
+  if (ax < 0x33000001u) { /* < 2^-25 (or exactly 2^-25 -> ties to even 0) */
+    return (uint16_t)sign;
+  }
+  int e = (int)(ax >> 23) - 127;
+  uint32_t man = (ax & 0x7FFFFFu) | 0x800000u; /* 24-bit significand */
+  int shift;     /* number of low bits dropped */
+  uint32_t hexp;
+  if (e < -14) { shift = 13 + (-14 - e); hexp = 0; }
+  else { shift = 13; hexp = (uint32_t)(e + 15); }
+  uint32_t kept = man >> shift;
+  uint32_t rem = man & ((1u << shift) - 1u);
+  uint32_t half = 1u << (shift - 1);
+  if (rem > half || (rem == half && (kept & 1u))) kept++;
+  uint32_t h;
+  if (hexp == 0) h = kept;                       /* subnormal (may carry into exp=1) */
+  else h = ((hexp << 10) + (kept - 0x400u));     /* carry propagates into exponent */
+  return (uint16_t)(sign | h);
+}
+
+ORA_API float ora_bf16_to_f32(uint16_t b) {
+  uint32_t bits = (uint32_t)b << 16; float f; memcpy(&f, &bits, 4); return f;
+}
+
+/* round-to-nearest-even binary32 -> bfloat16 */
+ORA_API uint16_t ora_f32_to_bf16(float f) {
+  uint32_t x; memcpy(&x, &f, 4);
+  if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((x >> 16) | 0x40u); /* quiet nan */
+  uint32_t lsb = (x >> 16) & 1u;
+  x += 0x7FFFu + lsb;
+  return (uint16_t)(x >> 16);
+}
+
+ORA_API void ora_f16_to_f32_array(const uint16_t* in, float* out, int64_t n) {
+  for (int64_t i = 0; i < n; i++) out[i] = ora_f16_to_f32(in[i]);
+}
+ORA_API void ora_f32_to_f16_array(const float* in, uint16_t* out, int64_t n) {
+  for (int64_t i = 0; i < n; i++) out[i] = ora_f32_to_f16(in[i]);
+}
+ORA_API void ora_bf16_to_f32_array(const uint16_t* in, float* out, int64_t n) {
+  for (int64_t i = 0; i < n; i++) out[i] = ora_bf16_to_f32(in[i]);
+}
+ORA_API void ora_f32_to_bf16_array(const float* in, uint16_t* out, int64_t n) {
+  for (int64_t i = 0; i < n; i++) out[i] = ora_f32_to_bf16(in[i]);
+}
+
+/* ------------------------------------------------------------------ Q8_0
+ * 32 weights / 34 bytes: { f16 d; i8 qs[32]; }      y[i] = f32(d) * (f32)qs[i]          */
+
+ORA_API void ora_dequant_q8_0(const uint8_t* blocks, int64_t nblocks, float* out) {
+  for (int64_t b = 0; b < nblocks; b++) {
+    const uint8_t* p = blocks + 34 * b;
+    uint16_t dh; memcpy(&dh, p, 2);
+    const float d = ora_f16_to_f32(dh);
+    const int8_t* qs = (const int8_t*)(p + 2);
+    for (int i = 0; i < 32; i++) out[32 * b + i] = d * (float)qs[i];
+  }
+}
+
+/* ------------------------------------------------------------------ Q4_K
+ * 256 weights / 144 bytes: { f16 d; f16 dmin; u8 scales[12]; u8 qs[128]; }
+ * eight sub-blocks of 32, each with a 6-bit scale sc_j and a 6-bit min m_j.              */
+
+ORA_API void ora_q4k_unpack_scales(const uint8_t scales[12], uint8_t sc[8], uint8_t mn[8]) {
+  for (int j = 0; j < 8; j++) {
+    if (j < 4) {
+      sc[j] = scales[j] & 63;
+      mn[j] = scales[j + 4] & 63;
+    } else {
+      sc[j] = (uint8_t)((scales[j + 4] & 0x0F) | ((scales[j - 4] >> 6) << 4));
+      mn[j] = (uint8_t)((scales[j + 4] >> 4) | ((scales[j] >> 6) << 4));
+    }
+  }
+}
+
+ORA_API void ora_dequant_q4_k(const uint8_t* blocks, int64_t nblocks, float* out) {
+  for (int64_t b = 0; b < nblocks; b++) {
+    const uint8_t* p = blocks + 144 * b;
+    uint16_t dh, mh; memcpy(&dh, p, 2); memcpy(&mh, p + 2, 2);
+    const float d = ora_f16_to_f32(dh);
+    const float dmin = ora_f16_to_f32(mh);
+    uint8_t sc[8], mn[8];
+    ora_q4k_unpack_scales(p + 4, sc, mn);
+    const uint8_t* qs = p + 16;
+    float* y = out + 256 * b;
+    for (int c = 0; c < 4; c++) {
+      const float d1 = d * (float)sc[2 * c], m1 = dmin * (float)mn[2 * c];
+      const float d2 = d * (float)sc[2 * c + 1], m2 = dmin * (float)mn[2 * c + 1];
+      const uint8_t* q = qs + 32 * c;
+      for (int l = 0; l < 32; l++) {
+        float t1 = d1 * (float)(q[l] & 0xF);
+        float t2 = d2 * (float)(q[l] >> 4);
+        y[64 * c + l] = t1 - m1;
+        y[64 * c + 32 + l] = t2 - m2;
+      }
+    }
+  }
+}
+
+/* ------------------------------------------------------------------ Q6_K
+ * 256 weights / 210 bytes: { u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d; }              */
+
+ORA_API void ora_dequant_q6_k(const uint8_t* blocks, int64_t nblocks, float* out) {
+  for (int64_t b = 0; b < nblocks; b++) {
+    const uint8_t* p = blocks + 210 * b;
+    const uint8_t* ql = p;
+    const uint8_t* qh = p + 128;
+    const int8_t* sc = (const int8_t*)(p + 192);
+    uint16_t dh; memcpy(&dh, p + 208, 2);
+    const float d = ora_f16_to_f32(dh);
+    float* y = out + 256 * b;
+    for (int h = 0; h < 2; h++) {
+      for (int l = 0; l < 32; l++) {
+        const int is = l / 16;
+        const int q1 = (int)((ql[l] & 0xF) | (((qh[l] >> 0) & 3) << 4)) - 32;
+        const int q2 = (int)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32;
+        const int q3 = (int)((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32;
+        const int q4 = (int)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32;
+        const float s1 = d * (float)sc[is + 0];
+        const float s2 = d * (float)sc[is + 2];
+        const float s3 = d * (float)sc[is + 4];
+        const float s4 = d * (float)sc[is + 6];
+        y[l] = s1 * (float)q1;
+        y[l + 32] = s2 * (float)q2;
+        y[l + 64] = s3 * (float)q3;
+        y[l + 96] = s4 * (float)q4;
+      }
+      y += 128; ql += 64; qh += 32; sc += 8;
+    }
+  }
+}
+
+/* ------------------------------------------------------------------ dense reference
+ * y[m][n] = sum_k x[m][k] * w[n][k] (+ bias[n]), float64 accumulation in index order.
+ * Follows linear.nim:45-57 / neural_nets.nim:64-81 (y = input * weight^T + bias).       */
+
+ORA_API void ora_linear_f64(const float* w, const float* x, const float* bias, double* y,
+                            int64_t m, int64_t n_out, int64_t n_in) {
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int64_t i = 0; i < m; i++) {
+    for (int64_t n = 0; n < n_out; n++) {
+      const float* wr = w + n * n_in;
+      const float* xr = x + i * n_in;
+      double acc = 0.0;
+      for (int64_t k = 0; k < n_in; k++) acc += (double)xr[k] * (double)wr[k];
+      if (bias) acc += (double)bias[n];
+      y[i * n_out + n] = acc;
+    }
+  }
+}
+
+/* Same product for a chosen subset of output rows (full-size spot checks). */
+ORA_API void ora_linear_rows_f64(const float* w_rows, const float* x, double* y,
+                                 int64_t m, int64_t n_rows, int64_t n_in) {
+  ora_linear_f64(w_rows, x, NULL, y, m, n_rows, n_in);
+}
+
+/* ------------------------------------------------------------------ fused CPU GEMV
+ * Streams the packed blocks once (no dense intermediate), float32 accumulation per block,
+ * one row per task.  Used as the like-for-like "reads packed bytes" CPU baseline.        */
+
+static float dot_q8_0_row(const uint8_t* row, const float* x, int64_t nb) {
+  float acc = 0.f;
+  for (int64_t b = 0; b < nb; b++) {
+    const uint8_t* p = row + 34 * b;
+    uint16_t dh; memcpy(&dh, p, 2);
+    const float d = ora_f16_to_f32(dh);
+    const int8_t* qs = (const int8_t*)(p + 2);
+    float s = 0.f;
+    for (int i = 0; i < 32; i++) s += (float)qs[i] * x[32 * b + i];
+    acc += d * s;
+  }
+  return acc;
+}
+
+static float dot_q4_k_row(const uint8_t* row, const float* x, int64_t nb) {
+  float acc = 0.f;
+  for (int64_t b = 0; b < nb; b++) {
+    const uint8_t* p = row + 144 * b;
+    uint16_t dh, mh; memcpy(&dh, p, 2); memcpy(&mh, p + 2, 2);
+    const float d = ora_f16_to_f32(dh), dmin = ora_f16_to_f32(mh);
+    uint8_t sc[8], mn[8];
+    ora_q4k_unpack_scales(p + 4, sc, mn);
+    const uint8_t* qs = p + 16;
+    const float* xb = x + 256 * b;
+    for (int c = 0; c < 4; c++) {
+      const uint8_t* q = qs + 32 * c;
+      float s1 = 0.f, s2 = 0.f, x1 = 0.f, x2 = 0.f;
+      for (int l = 0; l < 32; l++) {
+        const float xa = xb[64 * c + l], xc = xb[64 * c + 32 + l];
+        s1 += (float)(q[l] & 0xF) * xa; x1 += xa;
+        s2 += (float)(q[l] >> 4) * xc; x2 += xc;
+      }
+      acc += d * (float)sc[2 * c] * s1 - dmin * (float)mn[2 * c] * x1;
+      acc += d * (float)sc[2 * c + 1] * s2 - dmin * (float)mn[2 * c + 1] * x2;
+    }
+  }
+  return acc;
+}
+
+static float dot_q6_k_row(const uint8_t* row, const float* x, int64_t nb) {
+  float acc = 0.f;
+  for (int64_t b = 0; b < nb; b++) {
+    const uint8_t* p = row + 210 * b;
+    const uint8_t* ql = p; const uint8_t* qh = p + 128;
+    const int8_t* sc = (const int8_t*)(p + 192);
+    uint16_t dh; memcpy(&dh, p + 208, 2);
+    const float d = ora_f16_to_f32(dh);
+    const float* xb = x + 256 * b;
+    float blk = 0.f;
+    for (int h = 0; h < 2; h++) {
+      float s[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+      for (int l = 0; l < 32; l++) {
+        const int is = l / 16;
+        const int q1 = (int)((ql[l] & 0xF) | (((qh[l] >> 0) & 3) << 4)) - 32;
+        const int q2 = (int)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32;
+        const int q3 = (int)((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32;
+        const int q4 = (int)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32;
+        s[is + 0] += (float)q1 * xb[l];
+        s[is + 2] += (float)q2 * xb[l + 32];
+        s[is + 4] += (float)q3 * xb[l + 64];
+        s[is + 6] += (float)q4 * xb[l + 96];
+      }
+      for (int j = 0; j < 8; j++) blk += (float)sc[j] * s[j];
+      xb += 128; ql += 64; qh += 32; sc += 8;
+    }
+    acc += d * blk;
+  }
+  return acc;
+}
+
+/* format: 0 = Q8_0, 1 = Q4_K, 2 = Q6_K.  x is float32 (already widened from its dtype). */
+ORA_API int ora_gemv_fused(int format, const uint8_t* w, const float* x, float* y,
+                           int64_t n_out, int64_t n_in, int nthreads) {
+  int64_t row_bytes, nb;
+  if (format == 0) { nb = n_in / 32; row_bytes = nb * 34; }
+  else if (format == 1) { nb = n_in / 256; row_bytes = nb * 144; }
+  else if (format == 2) { nb = n_in / 256; row_bytes = nb * 210; }
+  else return -1;
+#ifdef _OPENMP
+  if (nthreads > 0) omp_set_num_threads(nthreads);
+#else
+  (void)nthreads;
+#endif
+#pragma omp parallel for schedule(static)
+  for (int64_t n = 0; n < n_out; n++) {
+    const uint8_t* row = w + n * row_bytes;
+    y[n] = (format == 0) ? dot_q8_0_row(row, x, nb)
+         : (format == 1) ? dot_q4_k_row(row, x, nb)
+                         : dot_q6_k_row(row, x, nb);
+  }
+  return 0;
+}
+
+ORA_API int ora_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+/* ------------------------------------------------------------------ Hadamard
+ * Orthonormal Sylvester-Hadamard on each consecutive group of 128 values:
+ * 7 butterfly stages, then scale by 1/sqrt(128).  Stage s pairs i and i + 2^s.           */
+
+ORA_API void ora_fwht128_f64(double* v, int64_t n) {
+  for (int64_t g = 0; g + 128 <= n; g += 128) {
+    double* p = v + g;
+    for (int len = 1; len < 128; len <<= 1) {
+      for (int i = 0; i < 128; i += 2 * len) {
+        for (int j = i; j < i + len; j++) {
+          const double a = p[j], b = p[j + len];
+          p[j] = a + b; p[j + len] = a - b;
+        }
+      }
+    }
+    const double s = 0.08838834764831845; /* 1/sqrt(128) */
+    for (int i = 0; i < 128; i++) p[i] *= s;
+  }
+}
+
+/* ------------------------------------------------------------------ EXL3-style trellis
+ * A 16x16 tile of weights is one cyclic bit string of 256*bits bits, stored as 16*bits
+ * little-endian u16 words, most significant bit of each word first:
+ *     bit(p) = (word[p / 16] >> (15 - p % 16)) & 1,   p taken mod 256*bits.
+ * Weight i (0..255) is decoded from the 16-bit window starting at bit i*bits, first bit
+ * as MSB, so consecutive states obey  s[i+1] = ((s[i] << bits) | next bits) & 0xFFFF.
+ * Index map inside the tile: i = 16 * n_local + k_local  (the 16 input positions of one
+ * output channel are consecutive in the stream).
+ * Tensor layout: trellis[k_tile][n_tile][16*bits] u16, k_tile = in/16, n_tile = out/16.
+ *
+ * Codebook (pure function of the state, result is an IEEE binary16 bit pattern):
+ *   cb 0 ("3inst"): u = s * 89226354 + 64248484 (mod 2^32)
+ *   cb 1 ("mcg")  : u = s * 0xCBAC1FED           (mod 2^32)
+ *   then u = (u & 0x8FFF8FFF) ^ 0x3B603B60; value = f16(lo16(u)) + f16(hi16(u)),
+ *   the sum rounded to binary16 (round-to-nearest-even).
+ * The constants follow the published QTIP / exllamav3 designs as recalled; parity with
+ * those projects is unpinned.                                                            */
+
+ORA_API uint16_t ora_exl3_codebook(uint32_t state, int cb) {
+  uint32_t u = (cb == 0) ? (state * 89226354u + 64248484u) : (state * 0xCBAC1FEDu);
+  u = (u & 0x8FFF8FFFu) ^ 0x3B603B60u;
+  const float lo = ora_f16_to_f32((uint16_t)(u & 0xFFFFu));
+  const float hi = ora_f16_to_f32((uint16_t)(u >> 16));
+  /* both halves have exponent field 12..15, so lo + hi is exact in binary32 */
+  return ora_f32_to_f16(lo + hi);
+}
+
+static inline int tile_bit(const uint16_t* tile, int p) {
+  return (tile[p >> 4] >> (15 - (p & 15))) & 1;
+}
+
+ORA_API void ora_exl3_tile_states(const uint16_t* tile, int bits, uint16_t states[256]) {
+  const int total = 256 * bits;
+  for (int i = 0; i < 256; i++) {
+    uint32_t s = 0;
+    for (int j = 0; j < 16; j++) s = (s << 1) | (uint32_t)tile_bit(tile, (i * bits + j) % total);
+    states[i] = (uint16_t)s;
+  }
+}
+
+/* Decoded (unscaled) trellis values as binary16 bit patterns, shape (n_out, n_in). */
+ORA_API void ora_exl3_decode(const uint16_t* trellis, uint16_t* out_f16,
+                             int64_t n_out, int64_t n_in, int bits, int cb) {
+  const int64_t kt_n = n_in / 16, nt_n = n_out / 16;
+  const int words = 16 * bits;
+  for (int64_t kt = 0; kt < kt_n; kt++) {
+    for (int64_t nt = 0; nt < nt_n; nt++) {
+      const uint16_t* tile = trellis + (kt * nt_n + nt) * words;
+      uint16_t st[256];
+      ora_exl3_tile_states(tile, bits, st);
+      for (int i = 0; i < 256; i++) {
+        const int64_t n = nt * 16 + (i >> 4), k = kt * 16 + (i & 15);
+        out_f16[n * n_in + k] = ora_exl3_codebook(st[i], cb);
+      }
+    }
+  }
+}
+
+/* y = svh o H( T * H(suh o x) ): float64 reference of the run-time formula.
+ * t_f32: decoded trellis values widened to f32 (n_out, n_in); suh (n_in), svh (n_out),
+ * x (n_in) all already widened to f32.                                                   */
+ORA_API void ora_exl3_gemv_f64(const float* t_f32, const float* suh, const float* svh,
+                               const float* x, double* y, double* xrot_scratch,
+                               int64_t n_out, int64_t n_in) {
+  for (int64_t k = 0; k < n_in; k++) xrot_scratch[k] = (double)suh[k] * (double)x[k];
+  ora_fwht128_f64(xrot_scratch, n_in);
+#pragma omp parallel for schedule(static)
+  for (int64_t n = 0; n < n_out; n++) {
+    double acc = 0.0;
+    const float* tr = t_f32 + n * n_in;
+    for (int64_t k = 0; k < n_in; k++) acc += (double)tr[k] * xrot_scratch[k];
+    y[n] = acc;
+  }
+  ora_fwht128_f64(y, n_out);
+  for (int64_t n = 0; n < n_out; n++) y[n] *= (double)svh[n];
+}
+
+ORA_API int ora_version(void) { return 1; }

@@ -1,0 +1,110 @@
+"""ctypes binding of ``libttq_hip.so`` -- the C ABI declared in ``include/ttq.h``.
+
+The library is the product; there is no Python or CPU fallback for any device entry point.
+If the shared library is missing, loading raises ``TtqLibraryError``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libttq_hip.so")
+
+# status / dtype / format codes (include/ttq.h)
+OK = 0
+ERR_NULL, ERR_SHAPE, ERR_ALIGN, ERR_DTYPE, ERR_FORMAT, ERR_UNSUPPORTED, ERR_HIP = -1, -2, -3, -4, -5, -6, -7
+F32, F16, BF16 = 0, 1, 2
+Q8_0, Q4_K, Q6_K, EXL3 = 0, 1, 2, 3
+CB_3INST, CB_MCG = 0, 1
+
+
+class TtqLibraryError(RuntimeError):
+    """libttq_hip.so is missing or cannot be loaded."""
+
+
+class QLinearStruct(C.Structure):
+    """``ttq_qlinear`` of include/ttq.h."""
+
+    _fields_ = [
+        ("format", C.c_int32),
+        ("bits", C.c_int32),
+        ("codebook", C.c_int32),
+        ("bias_dtype", C.c_int32),
+        ("n_out", C.c_int64),
+        ("n_in", C.c_int64),
+        ("qweight", C.c_void_p),
+        ("suh", C.c_void_p),
+        ("svh", C.c_void_p),
+        ("bias", C.c_void_p),
+    ]
+
+
+_vp, _i64, _i32, _u64 = C.c_void_p, C.c_int64, C.c_int, C.c_uint64
+
+# name -> (restype, argtypes); every symbol include/ttq.h declares
+SIGNATURES = {
+    "ttq_version": (_i32, []),
+    "ttq_strerror": (C.c_char_p, [_i32]),
+    "ttq_last_hip_error": (_i32, []),
+    "ttq_packed_nbytes": (_i64, [_i32, _i64, _i64, _i32]),
+    "ttq_linear_forward": (_i32, [C.POINTER(QLinearStruct), _vp, _i32, _i64, _vp, _i32, _vp]),
+    "ttq_gemv_q8_0": (_i32, [_vp, _vp, _i32, _vp, _i64, _i64, _i64, _vp]),
+    "ttq_gemv_q4_k": (_i32, [_vp, _vp, _i32, _vp, _i64, _i64, _i64, _vp]),
+    "ttq_gemv_q6_k": (_i32, [_vp, _vp, _i32, _vp, _i64, _i64, _i64, _vp]),
+    "ttq_gemv_exl3": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32, _vp]),
+    "ttq_gemm_q4_k": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "ttq_dequant_q8_0": (_i32, [_vp, _vp, _i32, _i64, _i64, _vp]),
+    "ttq_dequant_q4_k": (_i32, [_vp, _vp, _i32, _i64, _i64, _vp]),
+    "ttq_dequant_q6_k": (_i32, [_vp, _vp, _i32, _i64, _i64, _vp]),
+    "ttq_dequant_exl3": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _vp]),
+    "ttq_hadamard128_f32": (_i32, [_vp, _vp, _vp, _i64, _vp]),
+    "ttq_host_fill_normal": (_i32, [_u64, _u64, C.c_float, _vp, _i64]),
+    "ttq_host_quantize_q8_0": (_i32, [_vp, _vp, _i64, _i64]),
+    "ttq_host_quantize_q4_k": (_i32, [_vp, _vp, _i64, _i64]),
+    "ttq_host_quantize_q6_k": (_i32, [_vp, _vp, _i64, _i64]),
+    "ttq_host_quantize_exl3": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _u64]),
+    "ttq_host_f32_to_bf16": (_i32, [_vp, _vp, _i64]),
+    "ttq_host_f32_to_f16": (_i32, [_vp, _vp, _i64]),
+    "ttq_host_bf16_to_f32": (_i32, [_vp, _vp, _i64]),
+    "ttq_host_f16_to_f32": (_i32, [_vp, _vp, _i64]),
+}
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    """The loaded library with argument types set.  Raises if it is not built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise TtqLibraryError(
+                "%s not found: build it with `python -m tattletale_amd.build` "
+                "(there is no fallback implementation)" % LIB_PATH)
+        try:
+            L = C.CDLL(LIB_PATH)
+        except OSError as e:  # pragma: no cover - depends on the host
+            raise TtqLibraryError("cannot load %s: %s" % (LIB_PATH, e)) from e
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+class TtqError(ValueError):
+    """A ttq_* call returned a non-zero status (the counterpart of the reference raising
+    from F.linear on bad shapes)."""
+
+    def __init__(self, status: int, where: str):
+        self.status = status
+        msg = lib().ttq_strerror(status).decode()
+        if status == ERR_HIP:
+            msg += " [hipError %d]" % lib().ttq_last_hip_error()
+        super().__init__("%s: %s (status %d)" % (where, msg, status))
+
+
+def check(status: int, where: str) -> None:
+    if status != OK:
+        raise TtqError(status, where)

@@ -1,0 +1,76 @@
+"""Builds ``libttq_hip.so`` (gfx950 only) with hipcc.  ``python -m tattletale_amd.build``.
+
+hipcc cross-compiles without a GPU, so this runs on any host with ROCm installed.  The
+library is written in-tree, next to this file.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libttq_hip.so")
+
+SOURCES = [
+    "ttq_api.hip",
+    "ttq_dequant.hip",
+    "ttq_gemv.hip",
+    "ttq_gemm_q4k.hip",
+    "ttq_exl3.hip",
+    "ttq_host.cpp",
+]
+
+# -ffp-contract=off: float expressions round per operation, as the canonical dequantizer
+# does; fused multiply-adds are written explicitly in the kernels.
+# packed-fp32-ops is switched off so the compiler never forms v_pk_*_f32 instructions.
+COMMON = ["-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fno-fast-math", "-fvisibility=hidden",
+          "-Wall", "-Wno-unused-function"]
+DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; ROCm is required to build libttq_hip.so")
+    return exe
+
+
+def _compile(src: str, obj: str) -> None:
+    cmd = [hipcc()] + COMMON
+    if src.endswith(".hip"):
+        cmd += DEVICE
+    cmd += ["-DTTQ_BUILD", "-c", src, "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))
+
+
+def build_library(force: bool = True, verbose: bool = False) -> str:
+    """Compile every source and link the shared library.  Returns its path."""
+    srcs = [os.path.join(CSRC, s) for s in SOURCES]
+    deps = srcs + [os.path.join(CSRC, h) for h in os.listdir(CSRC) if h.endswith(".h")]
+    deps.append(os.path.join(HERE, "..", "include", "ttq.h"))
+    if not force and os.path.exists(LIB):
+        newest = max(os.path.getmtime(d) for d in deps)
+        if os.path.getmtime(LIB) >= newest:
+            return LIB
+    objdir = os.path.join(CSRC, "build")
+    os.makedirs(objdir, exist_ok=True)
+    objs = [os.path.join(objdir, os.path.basename(s) + ".o") for s in srcs]
+    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
+        list(ex.map(lambda so: _compile(*so), zip(srcs, objs)))
+    cmd = [hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs + ["-lpthread"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n%s\n%s" % (r.stdout, r.stderr))
+    if verbose:
+        print("built", LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    build_library(force="--if-stale" not in sys.argv, verbose=True)

@@ -1,0 +1,201 @@
+// C-ABI layer of libttq_hip.so: argument validation, GEMV/GEMM dispatch, error codes.
+// Declarations and the reference interfaces they replace are in include/ttq.h.
+//
+// The dispatch in ttq_linear_forward mirrors the reference's Linear.forward
+// (workspace/transformers/src/layers/linear.nim:45-57): one operator, bias optional, the
+// number of activation rows decides between the decode (GEMV) and prefill (GEMM) kernels.
+#include "../../include/ttq.h"
+#include "ttq_internal.h"
+
+namespace {
+
+thread_local int g_last_hip_error = 0;
+
+int hip_status(hipError_t e) {
+  if (e == hipSuccess) return TTQ_OK;
+  g_last_hip_error = (int)e;
+  return TTQ_ERR_HIP;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+bool valid_dtype(int d) { return d == TTQ_F32 || d == TTQ_F16 || d == TTQ_BF16; }
+
+// Shape rules of each format along n_in / n_out.
+int check_shape(int format, int64_t m, int64_t n_out, int64_t n_in, int bits, int cb) {
+  if (m < 0 || n_out < 0 || n_in <= 0) return TTQ_ERR_SHAPE;
+  if (n_out > 0x7FFFFFFF || n_in > 0x7FFFFFFF || m > 65535) return TTQ_ERR_UNSUPPORTED;
+  switch (format) {
+    case TTQ_Q8_0: return (n_in % 32 == 0) ? TTQ_OK : TTQ_ERR_SHAPE;
+    case TTQ_Q4_K:
+    case TTQ_Q6_K: return (n_in % 256 == 0) ? TTQ_OK : TTQ_ERR_SHAPE;
+    case TTQ_EXL3:
+      if (bits < 1 || bits > 8) return TTQ_ERR_FORMAT;
+      if (cb != TTQ_CB_3INST && cb != TTQ_CB_MCG) return TTQ_ERR_FORMAT;
+      return (n_in % 128 == 0 && n_out % 128 == 0) ? TTQ_OK : TTQ_ERR_SHAPE;
+    default: return TTQ_ERR_FORMAT;
+  }
+}
+
+int check_gemv_limits(int x_dtype, int64_t n_in) {
+  const int64_t lim = (x_dtype == TTQ_F32) ? ttq::kMaxGemvInF32 : ttq::kMaxGemvInF32;
+  return n_in <= lim ? TTQ_OK : TTQ_ERR_UNSUPPORTED;
+}
+
+int gemv_block(int format, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+               const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+               void* stream) {
+  if (!w || !x || !y) return TTQ_ERR_NULL;
+  if (!valid_dtype(x_dtype) || !valid_dtype(y_dtype)) return TTQ_ERR_DTYPE;
+  if (bias && !valid_dtype(bias_dtype)) return TTQ_ERR_DTYPE;
+  int rc = check_shape(format, m, n_out, n_in, 0, 0);
+  if (rc != TTQ_OK) return rc;
+  if (!aligned16(w) || !aligned16(x) || !aligned16(y)) return TTQ_ERR_ALIGN;
+  rc = check_gemv_limits(x_dtype, n_in);
+  if (rc != TTQ_OK) return rc;
+  return hip_status(ttq::launch_gemv(format, w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out,
+                                     n_in, static_cast<hipStream_t>(stream)));
+}
+
+int dequant_block(int format, const void* w, void* out, int out_dtype, int64_t n_out, int64_t n_in,
+                  void* stream) {
+  if (!w || !out) return TTQ_ERR_NULL;
+  if (!valid_dtype(out_dtype)) return TTQ_ERR_DTYPE;
+  const int rc = check_shape(format, 1, n_out, n_in, 0, 0);
+  if (rc != TTQ_OK) return rc;
+  if (!aligned16(w) || !aligned16(out)) return TTQ_ERR_ALIGN;
+  return hip_status(ttq::launch_dequant(format, w, out, out_dtype, n_out, n_in,
+                                        static_cast<hipStream_t>(stream)));
+}
+
+}  // namespace
+
+extern "C" {
+
+int ttq_version(void) { return TTQ_VERSION; }
+
+const char* ttq_strerror(int status) {
+  switch (status) {
+    case TTQ_OK: return "ok";
+    case TTQ_ERR_NULL: return "required pointer is NULL";
+    case TTQ_ERR_SHAPE: return "bad shape: dimension negative or not a multiple of the block size";
+    case TTQ_ERR_ALIGN: return "base pointer is not 16-byte aligned";
+    case TTQ_ERR_DTYPE: return "unknown or unsupported dtype";
+    case TTQ_ERR_FORMAT: return "unknown format, bit width or codebook";
+    case TTQ_ERR_UNSUPPORTED: return "request outside the supported size limits";
+    case TTQ_ERR_HIP: return "HIP runtime error (see ttq_last_hip_error)";
+    default: return "unknown status";
+  }
+}
+
+int ttq_last_hip_error(void) { return g_last_hip_error; }
+
+int64_t ttq_packed_nbytes(int format, int64_t n_out, int64_t n_in, int bits) {
+  const int rc = check_shape(format, 1, n_out, n_in, bits, TTQ_CB_MCG);
+  if (rc != TTQ_OK) return rc;
+  switch (format) {
+    case TTQ_Q8_0: return n_out * (n_in / 32) * 34;
+    case TTQ_Q4_K: return n_out * (n_in / 256) * 144;
+    case TTQ_Q6_K: return n_out * (n_in / 256) * 210;
+    case TTQ_EXL3: return (n_out / 16) * (n_in / 16) * 32 * bits;
+    default: return TTQ_ERR_FORMAT;
+  }
+}
+
+int ttq_gemv_q8_0(const void* w, const void* x, int x_dtype, float* y, int64_t m, int64_t n_out,
+                  int64_t n_in, void* stream) {
+  return gemv_block(TTQ_Q8_0, w, x, x_dtype, y, TTQ_F32, nullptr, 0, m, n_out, n_in, stream);
+}
+int ttq_gemv_q4_k(const void* w, const void* x, int x_dtype, float* y, int64_t m, int64_t n_out,
+                  int64_t n_in, void* stream) {
+  return gemv_block(TTQ_Q4_K, w, x, x_dtype, y, TTQ_F32, nullptr, 0, m, n_out, n_in, stream);
+}
+int ttq_gemv_q6_k(const void* w, const void* x, int x_dtype, float* y, int64_t m, int64_t n_out,
+                  int64_t n_in, void* stream) {
+  return gemv_block(TTQ_Q6_K, w, x, x_dtype, y, TTQ_F32, nullptr, 0, m, n_out, n_in, stream);
+}
+
+int ttq_gemv_exl3(const uint16_t* trellis, const uint16_t* suh_f16, const uint16_t* svh_f16,
+                  const uint16_t* x_f16, float* y, int64_t m, int64_t n_out, int64_t n_in, int bits,
+                  int codebook, void* stream) {
+  if (!trellis || !suh_f16 || !svh_f16 || !x_f16 || !y) return TTQ_ERR_NULL;
+  const int rc = check_shape(TTQ_EXL3, m, n_out, n_in, bits, codebook);
+  if (rc != TTQ_OK) return rc;
+  if (!aligned16(trellis) || !aligned16(x_f16) || !aligned16(y)) return TTQ_ERR_ALIGN;
+  if (n_in > ttq::kMaxGemvInF32) return TTQ_ERR_UNSUPPORTED;
+  return hip_status(ttq::launch_gemv_exl3(trellis, suh_f16, svh_f16, x_f16, TTQ_F16, y, TTQ_F32,
+                                          nullptr, 0, m, n_out, n_in, bits, codebook,
+                                          static_cast<hipStream_t>(stream)));
+}
+
+int ttq_gemm_q4_k(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m, int64_t n_out,
+                  int64_t n_in, void* stream) {
+  if (!w || !x_bf16 || !y_bf16) return TTQ_ERR_NULL;
+  const int rc = check_shape(TTQ_Q4_K, m, n_out, n_in, 0, 0);
+  if (rc != TTQ_OK) return rc;
+  if (!aligned16(w) || !aligned16(x_bf16) || !aligned16(y_bf16)) return TTQ_ERR_ALIGN;
+  return hip_status(ttq::launch_gemm_q4k(w, x_bf16, y_bf16, TTQ_BF16, nullptr, 0, m, n_out, n_in,
+                                         static_cast<hipStream_t>(stream)));
+}
+
+int ttq_dequant_q8_0(const void* w, void* out, int out_dtype, int64_t n_out, int64_t n_in, void* stream) {
+  return dequant_block(TTQ_Q8_0, w, out, out_dtype, n_out, n_in, stream);
+}
+int ttq_dequant_q4_k(const void* w, void* out, int out_dtype, int64_t n_out, int64_t n_in, void* stream) {
+  return dequant_block(TTQ_Q4_K, w, out, out_dtype, n_out, n_in, stream);
+}
+int ttq_dequant_q6_k(const void* w, void* out, int out_dtype, int64_t n_out, int64_t n_in, void* stream) {
+  return dequant_block(TTQ_Q6_K, w, out, out_dtype, n_out, n_in, stream);
+}
+
+int ttq_dequant_exl3(const uint16_t* trellis, uint16_t* out_f16, int64_t n_out, int64_t n_in, int bits,
+                     int codebook, void* stream) {
+  if (!trellis || !out_f16) return TTQ_ERR_NULL;
+  const int rc = check_shape(TTQ_EXL3, 1, n_out, n_in, bits, codebook);
+  if (rc != TTQ_OK) return rc;
+  if (!aligned16(trellis) || !aligned16(out_f16)) return TTQ_ERR_ALIGN;
+  return hip_status(ttq::launch_dequant_exl3(trellis, out_f16, n_out, n_in, bits, codebook,
+                                             static_cast<hipStream_t>(stream)));
+}
+
+int ttq_hadamard128_f32(float* v, const uint16_t* pre_f16, const uint16_t* post_f16, int64_t n,
+                        void* stream) {
+  if (!v) return TTQ_ERR_NULL;
+  if (n < 0 || n % 128 != 0) return TTQ_ERR_SHAPE;
+  if (!aligned16(v)) return TTQ_ERR_ALIGN;
+  return hip_status(ttq::launch_hadamard128(v, pre_f16, post_f16, n, static_cast<hipStream_t>(stream)));
+}
+
+int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int64_t m, void* y,
+                       int y_dtype, void* stream) {
+  if (!layer || !x || !y || !layer->qweight) return TTQ_ERR_NULL;
+  if (!valid_dtype(x_dtype) || !valid_dtype(y_dtype)) return TTQ_ERR_DTYPE;
+  if (layer->bias && !valid_dtype(layer->bias_dtype)) return TTQ_ERR_DTYPE;
+  const int rc = check_shape(layer->format, m, layer->n_out, layer->n_in, layer->bits, layer->codebook);
+  if (rc != TTQ_OK) return rc;
+  if (!aligned16(layer->qweight) || !aligned16(x) || !aligned16(y)) return TTQ_ERR_ALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t n_out = layer->n_out, n_in = layer->n_in;
+
+  if (layer->format == TTQ_EXL3) {
+    if (!layer->suh || !layer->svh) return TTQ_ERR_NULL;
+    if (y_dtype != TTQ_F32) return TTQ_ERR_UNSUPPORTED;  // output rotation runs in place on fp32
+    if (n_in > ttq::kMaxGemvInF32) return TTQ_ERR_UNSUPPORTED;
+    return hip_status(ttq::launch_gemv_exl3(
+        static_cast<const uint16_t*>(layer->qweight), static_cast<const uint16_t*>(layer->suh),
+        static_cast<const uint16_t*>(layer->svh), x, x_dtype, y, y_dtype, layer->bias,
+        layer->bias_dtype, m, n_out, n_in, layer->bits, layer->codebook, s));
+  }
+
+  // Prefill: MFMA kernel for Q4_K with bf16 activations once there are enough rows to fill a tile.
+  if (layer->format == TTQ_Q4_K && x_dtype == TTQ_BF16 && m >= 16 &&
+      (y_dtype == TTQ_BF16 || y_dtype == TTQ_F32)) {
+    return hip_status(ttq::launch_gemm_q4k(layer->qweight, static_cast<const uint16_t*>(x), y, y_dtype,
+                                           layer->bias, layer->bias_dtype, m, n_out, n_in, s));
+  }
+  const int lim = check_gemv_limits(x_dtype, n_in);
+  if (lim != TTQ_OK) return lim;
+  return hip_status(ttq::launch_gemv(layer->format, layer->qweight, x, x_dtype, y, y_dtype, layer->bias,
+                                     layer->bias_dtype, m, n_out, n_in, s));
+}
+
+}  // extern "C"

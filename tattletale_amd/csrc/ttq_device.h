@@ -1,0 +1,125 @@
+// Device-side helpers shared by the gfx950 kernels: 16-bit float handling, wavefront
+// reductions, unaligned vector loads and the block-format field decoders.
+//
+// Arithmetic contract: this library is compiled with -ffp-contract=off, so every float
+// operator below rounds once, exactly like the canonical CPU dequantizer; fused
+// multiply-adds are written explicitly with fmaf_() where they are wanted.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ttq {
+
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float fmaf_(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
+  _Float16 v;
+  __builtin_memcpy(&v, &h, 2);
+  return (float)v;
+}
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+  _Float16 v = (_Float16)f;  // round-to-nearest-even
+  uint16_t h;
+  __builtin_memcpy(&h, &v, 2);
+  return h;
+}
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) {
+  return __uint_as_float((uint32_t)b << 16);
+}
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  __bf16 v = (__bf16)f;  // v_cvt_pk_bf16_f32: round-to-nearest-even
+  uint16_t h;
+  __builtin_memcpy(&h, &v, 2);
+  return h;
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  bf16x2_t r;
+  r[0] = (__bf16)lo;
+  r[1] = (__bf16)hi;
+  uint32_t u;
+  __builtin_memcpy(&u, &r, 4);
+  return u;
+}
+
+// Activation element -> float, by buffer element type.
+template <typename T> struct XElem;
+template <> struct XElem<float> {
+  static __device__ __forceinline__ float load(const float* p, int64_t i) { return p[i]; }
+};
+struct f16_tag { uint16_t v; };
+struct bf16_tag { uint16_t v; };
+template <> struct XElem<f16_tag> {
+  static __device__ __forceinline__ float load(const f16_tag* p, int64_t i) { return f16_bits_to_f32(p[i].v); }
+};
+template <> struct XElem<bf16_tag> {
+  static __device__ __forceinline__ float load(const bf16_tag* p, int64_t i) { return bf16_bits_to_f32(p[i].v); }
+};
+
+// Output element <- float.
+template <typename T> struct YElem;
+template <> struct YElem<float> {
+  static __device__ __forceinline__ void store(float* p, int64_t i, float v) { p[i] = v; }
+};
+template <> struct YElem<f16_tag> {
+  static __device__ __forceinline__ void store(f16_tag* p, int64_t i, float v) { p[i].v = f32_to_f16_bits(v); }
+};
+template <> struct YElem<bf16_tag> {
+  static __device__ __forceinline__ void store(bf16_tag* p, int64_t i, float v) { p[i].v = f32_to_bf16_bits(v); }
+};
+
+// 16-byte load from an address that is only 2-byte aligned (Q6_K / Q8_0 blocks).  gfx950
+// global loads accept any alignment; the builtin copy keeps the compiler honest about it.
+__device__ __forceinline__ uint4 load16_a2(const uint8_t* p) {
+  uint4 v;
+  __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 16);
+  return v;
+}
+__device__ __forceinline__ uint4 load16_a4(const uint8_t* p) {
+  uint4 v;
+  __builtin_memcpy(&v, __builtin_assume_aligned(p, 4), 16);
+  return v;
+}
+__device__ __forceinline__ uint4 load16_a16(const uint8_t* p) {
+  return *reinterpret_cast<const uint4*>(__builtin_assume_aligned(p, 16));
+}
+__device__ __forceinline__ uint32_t load4_a2(const uint8_t* p) {
+  uint32_t v;
+  __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 4);
+  return v;
+}
+__device__ __forceinline__ uint16_t load2(const uint8_t* p) {
+  uint16_t v;
+  __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 2);
+  return v;
+}
+
+// Sum over the 64 lanes of a wavefront; every lane gets the total.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+
+// Q4_K: 6-bit scale and min of sub-block j (0..7) from the 12 packed bytes held as three
+// little-endian dwords s0 (bytes 0-3), s1 (4-7), s2 (8-11).
+__device__ __forceinline__ void q4k_scale_min(uint32_t s0, uint32_t s1, uint32_t s2, int j,
+                                              uint32_t& sc, uint32_t& mn) {
+  if (j < 4) {
+    sc = (s0 >> (8 * j)) & 63u;
+    mn = (s1 >> (8 * j)) & 63u;
+  } else {
+    const int jj = j - 4;
+    sc = ((s2 >> (8 * jj)) & 0xFu) | (((s0 >> (8 * jj + 6)) & 3u) << 4);
+    mn = ((s2 >> (8 * jj + 4)) & 0xFu) | (((s1 >> (8 * jj + 6)) & 3u) << 4);
+  }
+}
+
+}  // namespace ttq

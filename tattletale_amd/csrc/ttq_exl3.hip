@@ -1,0 +1,291 @@
+// EXL3-style trellis-coded weights on gfx950: tile decoder, decode GEMV with the input-side
+// Hadamard rotation fused into its prologue, and the 128-group Hadamard epilogue.
+//
+//   y = svh o H( T * H(suh o x) )
+//
+// T (n_out, n_in) are the decoded trellis values, H the orthonormal Sylvester-Hadamard
+// transform applied to each group of 128, suh/svh fp16 vectors.  This is the quantized
+// counterpart of F.linear(x, weight) (workspace/libtorch/src/abi/neural_nets.nim:64-81);
+// the reference holds only the format's metadata
+// (workspace/transformers/tests/fixtures/configs/config-GLM-4.7-EXL3-3.84bpw.json:43-54).
+//
+// Format.  A 16x16 tile is one cyclic string of 256*bits bits kept in 16*bits u16 words,
+// most significant bit of each word first.  Weight i = 16*n_local + k_local is decoded
+// from the 16-bit window that starts at bit i*bits.  Tiles are laid out
+// trellis[k_tile][n_tile][16*bits].  Because 16*bits is a multiple of 16, the 16 weights
+// of one output channel inside a tile start on a word boundary and span bits+1 words; one
+// lane decodes exactly those 16 weights, so all window shifts are compile-time constants.
+#include "ttq_device.h"
+#include "ttq_internal.h"
+
+namespace ttq {
+
+typedef __attribute__((ext_vector_type(2))) _Float16 half2_t;
+
+template <int CB>
+__device__ __forceinline__ _Float16 exl3_code(uint32_t state) {
+  uint32_t u = (CB == 0) ? (state * 89226354u + 64248484u) : (state * 0xCBAC1FEDu);
+  u = (u & 0x8FFF8FFFu) ^ 0x3B603B60u;
+  half2_t h;
+  __builtin_memcpy(&h, &u, 4);
+  return h[0] + h[1];  // fp16 add, round-to-nearest-even
+}
+
+// The bits+1 words that hold the 16 windows of output channel j of a tile, as big-endian
+// 32-bit chunks (first stream bit = bit 31 of chunk 0).
+template <int BITS>
+struct LaneBits {
+  static constexpr int kWords = BITS + 1;
+  static constexpr int kChunks = (kWords + 1) / 2;
+  uint32_t c[kChunks];
+  __device__ __forceinline__ void load(const uint16_t* tile, int j) {
+    constexpr int words = 16 * BITS;
+    uint32_t w[2 * kChunks];
+#pragma unroll
+    for (int t = 0; t < 2 * kChunks; t++) {
+      int idx = j * BITS + t;
+      if (idx >= words) idx -= words;  // cyclic wrap (only channel 15 reaches it)
+      w[t] = (t < kWords) ? (uint32_t)tile[idx] : 0u;
+    }
+#pragma unroll
+    for (int t = 0; t < kChunks; t++) c[t] = (w[2 * t] << 16) | w[2 * t + 1];
+  }
+  template <int KK>
+  __device__ __forceinline__ uint32_t state() const {
+    constexpr int q = KK * BITS;
+    constexpr int ci = q >> 5, o = q & 31;
+    if constexpr (o <= 16) {
+      return (c[ci] >> (16 - o)) & 0xFFFFu;
+    } else {
+      return __builtin_amdgcn_alignbit(c[ci], c[ci + 1 < kChunks ? ci + 1 : ci], 48 - o) & 0xFFFFu;
+    }
+  }
+};
+
+template <int BITS, int CB, int KK>
+struct DecodeLoop {
+  static __device__ __forceinline__ void run(const LaneBits<BITS>& lb, _Float16* out) {
+    out[KK] = exl3_code<CB>(lb.template state<KK>());
+    if constexpr (KK + 1 < 16) DecodeLoop<BITS, CB, KK + 1>::run(lb, out);
+  }
+};
+
+// ------------------------------------------------------------------ tile decoder
+// One thread per (tile, output channel): writes 16 consecutive fp16 values of a row.
+template <int BITS, int CB>
+__global__ void __launch_bounds__(256) dequant_exl3_kernel(const uint16_t* __restrict__ trellis,
+                                                           uint16_t* __restrict__ out, int nt_n,
+                                                           int64_t nthreads, int n_in) {
+  const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (g >= nthreads) return;
+  const int j = (int)(g & 15);
+  const int64_t tile = g >> 4;
+  const int64_t kt = tile / nt_n, nt = tile % nt_n;
+  LaneBits<BITS> lb;
+  lb.load(trellis + tile * (16 * BITS), j);
+  _Float16 v[16];
+  DecodeLoop<BITS, CB, 0>::run(lb, v);
+  uint16_t* o = out + (nt * 16 + j) * (int64_t)n_in + kt * 16;
+#pragma unroll
+  for (int kk = 0; kk < 16; kk++) {
+    uint16_t b;
+    __builtin_memcpy(&b, &v[kk], 2);
+    o[kk] = b;
+  }
+}
+
+// ------------------------------------------------------------------ GEMV
+constexpr int kExl3Threads = 1024;
+constexpr int kExl3Waves = kExl3Threads / kWave;
+
+// In-LDS orthonormal FWHT of every 128-group of xs[0..n), all threads of the block.
+__device__ __forceinline__ void fwht128_lds(float* xs, int n, int tid, int nthreads) {
+  for (int len = 1; len < 128; len <<= 1) {
+    __syncthreads();
+    for (int p = tid; p < n / 2; p += nthreads) {
+      // pair p of its stage: insert a zero bit at position log2(len)
+      const int lo = p & (len - 1);
+      const int i = ((p - lo) << 1) | lo;
+      const float a = xs[i], b = xs[i + len];
+      xs[i] = a + b;
+      xs[i + len] = a - b;
+    }
+  }
+  __syncthreads();
+}
+
+// One workgroup per n_tile (16 output channels).  Lane = (k-tile slot g = lane/16, channel
+// j = lane%16); the 16 waves times 4 slots walk the k tiles 64 at a time.  Partial sums are
+// combined across slots with lane shuffles and across waves through LDS.
+template <int BITS, int CB, typename XT>
+__global__ void __launch_bounds__(kExl3Threads)
+gemv_exl3_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __restrict__ suh,
+                 const XT* __restrict__ x, float* __restrict__ y, int n_out, int n_in) {
+  extern __shared__ float xs[];          // n_in rotated activations, then kExl3Waves*16 partials
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const XT* xm = x + (int64_t)blockIdx.y * n_in;
+  float* ym = y + (int64_t)blockIdx.y * n_out;
+  for (int k = tid; k < n_in; k += kExl3Threads)
+    xs[k] = XElem<XT>::load(xm, k) * f16_bits_to_f32(suh[k]);
+  fwht128_lds(xs, n_in, tid, kExl3Threads);
+  const float kNorm = 0.08838834764831845f;  // 1/sqrt(128), applied to the dot product
+
+  const int nt = blockIdx.x, nt_n = n_out >> 4, kt_n = n_in >> 4;
+  const int g = lane >> 4, j = lane & 15;
+  float acc = 0.f;
+  for (int kt = wave * 4 + g; kt < kt_n; kt += kExl3Waves * 4) {
+    LaneBits<BITS> lb;
+    lb.load(trellis + ((int64_t)kt * nt_n + nt) * (16 * BITS), j);
+    _Float16 v[16];
+    DecodeLoop<BITS, CB, 0>::run(lb, v);
+    const float4* xv = reinterpret_cast<const float4*>(xs + 16 * kt);
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const float4 xq = xv[q];
+      acc = fmaf_((float)v[4 * q + 0], xq.x, acc);
+      acc = fmaf_((float)v[4 * q + 1], xq.y, acc);
+      acc = fmaf_((float)v[4 * q + 2], xq.z, acc);
+      acc = fmaf_((float)v[4 * q + 3], xq.w, acc);
+    }
+  }
+  acc += __shfl_xor(acc, 16, kWave);
+  acc += __shfl_xor(acc, 32, kWave);
+  float* red = xs + n_in;
+  if (lane < 16) red[wave * 16 + lane] = acc;
+  __syncthreads();
+  if (tid < 16) {
+    float s = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < kExl3Waves; wv++) s += red[wv * 16 + tid];
+    ym[nt * 16 + tid] = s * kNorm;
+  }
+}
+
+// ------------------------------------------------------------------ Hadamard epilogue
+// One workgroup of 128 threads per 128-group: v <- post o H(pre o v) (+ bias), in place.
+// `period` is the length after which pre/post/bias repeat (n_out for batched outputs).
+__global__ void __launch_bounds__(128)
+hadamard128_kernel(float* __restrict__ v, const uint16_t* __restrict__ pre,
+                   const uint16_t* __restrict__ post, const void* __restrict__ bias, int bias_dtype,
+                   int64_t period) {
+  __shared__ float s[128];
+  const int t = threadIdx.x;
+  const int64_t idx = (int64_t)blockIdx.x * 128 + t;
+  const int64_t ch = idx % period;
+  float a = v[idx];
+  if (pre) a *= f16_bits_to_f32(pre[ch]);
+  s[t] = a;
+  for (int len = 1; len < 128; len <<= 1) {
+    __syncthreads();
+    const float mine = s[t], other = s[t ^ len];
+    __syncthreads();
+    s[t] = (t & len) ? (other - mine) : (mine + other);
+  }
+  float r = s[t] * 0.08838834764831845f;
+  if (post) r *= f16_bits_to_f32(post[ch]);
+  if (bias) {
+    if (bias_dtype == kF32) r += static_cast<const float*>(bias)[ch];
+    else {
+      const uint16_t b = static_cast<const uint16_t*>(bias)[ch];
+      r += (bias_dtype == kF16) ? f16_bits_to_f32(b) : bf16_bits_to_f32(b);
+    }
+  }
+  v[idx] = r;
+}
+
+// ------------------------------------------------------------------ launchers
+template <int BITS>
+static hipError_t dequant_bits(const uint16_t* trellis, uint16_t* out, int64_t n_out, int64_t n_in,
+                               int cb, hipStream_t s) {
+  const int nt_n = (int)(n_out / 16);
+  const int64_t nthreads = (n_out / 16) * (n_in / 16) * 16;
+  if (nthreads == 0) return hipSuccess;
+  const dim3 grid((unsigned)((nthreads + 255) / 256)), block(256);
+  if (cb == 0)
+    hipLaunchKernelGGL((dequant_exl3_kernel<BITS, 0>), grid, block, 0, s, trellis, out, nt_n, nthreads, (int)n_in);
+  else
+    hipLaunchKernelGGL((dequant_exl3_kernel<BITS, 1>), grid, block, 0, s, trellis, out, nt_n, nthreads, (int)n_in);
+  return hipGetLastError();
+}
+
+hipError_t launch_dequant_exl3(const uint16_t* trellis, uint16_t* out_f16, int64_t n_out, int64_t n_in,
+                               int bits, int cb, hipStream_t s) {
+  switch (bits) {
+    case 1: return dequant_bits<1>(trellis, out_f16, n_out, n_in, cb, s);
+    case 2: return dequant_bits<2>(trellis, out_f16, n_out, n_in, cb, s);
+    case 3: return dequant_bits<3>(trellis, out_f16, n_out, n_in, cb, s);
+    case 4: return dequant_bits<4>(trellis, out_f16, n_out, n_in, cb, s);
+    case 5: return dequant_bits<5>(trellis, out_f16, n_out, n_in, cb, s);
+    case 6: return dequant_bits<6>(trellis, out_f16, n_out, n_in, cb, s);
+    case 7: return dequant_bits<7>(trellis, out_f16, n_out, n_in, cb, s);
+    case 8: return dequant_bits<8>(trellis, out_f16, n_out, n_in, cb, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+template <int BITS, int CB>
+static hipError_t gemv_bits_cb(const uint16_t* trellis, const uint16_t* suh, const void* x, int x_dtype,
+                               float* y, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+  const dim3 grid((unsigned)(n_out / 16), (unsigned)m), block(kExl3Threads);
+  const size_t lds = ((size_t)n_in + kExl3Waves * 16) * sizeof(float);
+  switch (x_dtype) {
+    case kF32:
+      hipLaunchKernelGGL((gemv_exl3_kernel<BITS, CB, float>), grid, block, lds, s, trellis, suh,
+                         static_cast<const float*>(x), y, (int)n_out, (int)n_in);
+      break;
+    case kF16:
+      hipLaunchKernelGGL((gemv_exl3_kernel<BITS, CB, f16_tag>), grid, block, lds, s, trellis, suh,
+                         static_cast<const f16_tag*>(x), y, (int)n_out, (int)n_in);
+      break;
+    case kBF16:
+      hipLaunchKernelGGL((gemv_exl3_kernel<BITS, CB, bf16_tag>), grid, block, lds, s, trellis, suh,
+                         static_cast<const bf16_tag*>(x), y, (int)n_out, (int)n_in);
+      break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+template <int BITS>
+static hipError_t gemv_bits(const uint16_t* trellis, const uint16_t* suh, const void* x, int x_dtype,
+                            float* y, int64_t m, int64_t n_out, int64_t n_in, int cb, hipStream_t s) {
+  return cb == 0 ? gemv_bits_cb<BITS, 0>(trellis, suh, x, x_dtype, y, m, n_out, n_in, s)
+                 : gemv_bits_cb<BITS, 1>(trellis, suh, x, x_dtype, y, m, n_out, n_in, s);
+}
+
+hipError_t launch_gemv_exl3(const uint16_t* trellis, const uint16_t* suh, const uint16_t* svh,
+                            const void* x, int x_dtype, void* y, int y_dtype, const void* bias,
+                            int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, int bits, int cb,
+                            hipStream_t s) {
+  if (m == 0 || n_out == 0) return hipSuccess;
+  if (y_dtype != kF32) return hipErrorInvalidValue;
+  if (n_in > 16000) return hipErrorInvalidValue;  // activations + partials must fit 64 KiB of LDS
+  float* yf = static_cast<float*>(y);
+  hipError_t e;
+  switch (bits) {
+    case 1: e = gemv_bits<1>(trellis, suh, x, x_dtype, yf, m, n_out, n_in, cb, s); break;
+    case 2: e = gemv_bits<2>(trellis, suh, x, x_dtype, yf, m, n_out, n_in, cb, s); break;
+    case 3: e = gemv_bits<3>(trellis, suh, x, x_dtype, yf, m, n_out, n_in, cb, s); break;
+    case 4: e = gemv_bits<4>(trellis, suh, x, x_dtype, yf, m, n_out, n_in, cb, s); break;
+    case 5: e = gemv_bits<5>(trellis, suh, x, x_dtype, yf, m, n_out, n_in, cb, s); break;
+    case 6: e = gemv_bits<6>(trellis, suh, x, x_dtype, yf, m, n_out, n_in, cb, s); break;
+    case 7: e = gemv_bits<7>(trellis, suh, x, x_dtype, yf, m, n_out, n_in, cb, s); break;
+    case 8: e = gemv_bits<8>(trellis, suh, x, x_dtype, yf, m, n_out, n_in, cb, s); break;
+    default: return hipErrorInvalidValue;
+  }
+  if (e != hipSuccess) return e;
+  const int64_t groups = m * n_out / 128;
+  hipLaunchKernelGGL(hadamard128_kernel, dim3((unsigned)groups), dim3(128), 0, s, yf,
+                     (const uint16_t*)nullptr, svh, bias, bias_dtype, n_out);
+  return hipGetLastError();
+}
+
+hipError_t launch_hadamard128(float* v, const uint16_t* pre, const uint16_t* post, int64_t n,
+                              hipStream_t s) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(hadamard128_kernel, dim3((unsigned)(n / 128)), dim3(128), 0, s, v, pre, post,
+                     (const void*)nullptr, 0, n);
+  return hipGetLastError();
+}
+
+}  // namespace ttq

@@ -1,0 +1,353 @@
+// Decode GEMV for the block formats Q8_0 / Q4_K / Q6_K on gfx950.
+//
+//   y[n] = sum_k W^[n][k] * x[k] (+ bias[n])        W^ = dequantized weight, never stored
+//
+// replaces F.linear(x, weight) for a single-token activation
+// (workspace/libtorch/src/abi/neural_nets.nim:64-81, called from
+//  workspace/transformers/src/layers/linear.nim:45-57).
+//
+// Mapping.  A row of W is cut into "units" of 64 weights; unit u of every row is always
+// handled by lane u % 64, so the 64 activations a lane needs never change from row to row.
+// A workgroup first stages x in LDS in a lane-major permutation; when a row has at most 64
+// units (n_in <= 4096) each lane then pulls its 64 activations into VGPRs once and the row
+// loop touches only HBM: per row a wavefront issues 16-byte loads that cover the packed row
+// contiguously, unpacks in registers, and finishes with a cross-lane sum.  Rows are dealt
+// to wavefronts round-robin, so at any moment the whole chip streams one contiguous span
+// of the weight buffer.
+//
+// Two arithmetic paths:
+//   generic : x widened to fp32, fp32 FMA per weight.  Any activation dtype.
+//   dot2    : bf16 activations kept as packed pairs, weights turned into bf16 pairs with
+//             one AND-OR each (0x4300 | q is the bf16 value 128 + q) and multiplied with
+//             v_dot2_f32_bf16; the 128 offset is removed with a per-unit sum of x.
+// Both compute sum(q*x) per sub-block first and apply the block scales once per sub-block,
+// so for a unit-vector activation the result equals the canonical dequantized weight bit
+// for bit.
+#include "ttq_device.h"
+#include "ttq_internal.h"
+
+#include <stdlib.h>
+
+namespace ttq {
+
+constexpr int kGemvThreads = 256;
+constexpr int kGemvWaves = kGemvThreads / kWave;
+
+// LDS slot of activation p (0..63) of unit u, fp32 layout: [u/64][p/4][u%64][p%4]
+__device__ __forceinline__ int xslot_f32(int u, int p) {
+  return ((((u >> 6) * 16 + (p >> 2)) * 64 + (u & 63)) << 2) + (p & 3);
+}
+
+// ------------------------------------------------------------------------------- formats
+struct FmtQ8_0 {
+  // unit = two consecutive 34-byte blocks (64 weights); the second may be absent at row end
+  static __device__ __forceinline__ int units(int n_in) { return (n_in + 63) >> 6; }
+  static __device__ __forceinline__ int64_t row_bytes(int n_in) { return (int64_t)(n_in >> 5) * 34; }
+  static __device__ __forceinline__ void kmap(int k, int& u, int& p) { u = k >> 6; p = k & 63; }
+  struct Raw { uint4 a0, a1, b0, b1; uint32_t d0, d1; };
+  static __device__ __forceinline__ Raw load(const uint8_t* row, int u, int n_in) {
+    Raw r;
+    const uint8_t* p = row + 68 * (int64_t)u;
+    r.d0 = load2(p);
+    r.a0 = load16_a2(p + 2);
+    r.a1 = load16_a2(p + 18);
+    const bool second = (64 * u + 32) < n_in;
+    if (second) {
+      r.d1 = load2(p + 34);
+      r.b0 = load16_a4(p + 36);
+      r.b1 = load16_a4(p + 52);
+    } else {
+      r.d1 = 0;
+      r.b0 = make_uint4(0, 0, 0, 0);
+      r.b1 = r.b0;
+    }
+    return r;
+  }
+  static __device__ __forceinline__ float dot32(const uint4& q0, const uint4& q1, const float* x) {
+    const uint32_t dw[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        const int q = (int)(int8_t)((dw[i] >> (8 * k)) & 0xFFu);
+        s = fmaf_((float)q, x[4 * i + k], s);
+      }
+    }
+    return s;
+  }
+  static __device__ __forceinline__ float dot(const Raw& r, const float (&x)[64]) {
+    const float s0 = dot32(r.a0, r.a1, &x[0]);
+    const float s1 = dot32(r.b0, r.b1, &x[32]);
+    const float d0 = f16_bits_to_f32((uint16_t)r.d0), d1 = f16_bits_to_f32((uint16_t)r.d1);
+    return d0 * s0 + d1 * s1;
+  }
+};
+
+struct FmtQ4_K {
+  // unit = chunk c of a super-block: 32 qs bytes -> sub-blocks 2c (low nibbles), 2c+1 (high)
+  static __device__ __forceinline__ int units(int n_in) { return n_in >> 6; }
+  static __device__ __forceinline__ int64_t row_bytes(int n_in) { return (int64_t)(n_in >> 8) * 144; }
+  static __device__ __forceinline__ void kmap(int k, int& u, int& p) { u = k >> 6; p = k & 63; }
+  struct Raw { uint4 hdr, q0, q1; int c; };
+  static __device__ __forceinline__ Raw load(const uint8_t* row, int u, int) {
+    Raw r;
+    const uint8_t* p = row + 144 * (int64_t)(u >> 2);
+    r.c = u & 3;
+    r.hdr = load16_a16(p);
+    r.q0 = load16_a16(p + 16 + 32 * r.c);
+    r.q1 = load16_a16(p + 32 + 32 * r.c);
+    return r;
+  }
+  static __device__ __forceinline__ float dot(const Raw& r, const float (&x)[64]) {
+    const uint32_t dw[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+    float s1 = 0.f, s2 = 0.f, x1 = 0.f, x2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        const uint32_t b = (dw[i] >> (8 * k)) & 0xFFu;
+        s1 = fmaf_((float)(b & 0xFu), x[4 * i + k], s1);
+        s2 = fmaf_((float)(b >> 4), x[32 + 4 * i + k], s2);
+        x1 += x[4 * i + k];
+        x2 += x[32 + 4 * i + k];
+      }
+    }
+    const float d = f16_bits_to_f32((uint16_t)(r.hdr.x & 0xFFFF));
+    const float dmin = f16_bits_to_f32((uint16_t)(r.hdr.x >> 16));
+    uint32_t sc1, mn1, sc2, mn2;
+    q4k_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, 2 * r.c, sc1, mn1);
+    q4k_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, 2 * r.c + 1, sc2, mn2);
+    const float t1 = (d * (float)sc1) * s1 - (dmin * (float)mn1) * x1;
+    const float t2 = (d * (float)sc2) * s2 - (dmin * (float)mn2) * x2;
+    return t1 + t2;
+  }
+};
+
+struct FmtQ6_K {
+  // unit = (block b, half h, 16-wide l range s): weights 128h + 32j + 16s + i, j=0..3, i=0..15
+  // unit index u = 4b + 2h + s; activation slot p = 16j + i
+  static __device__ __forceinline__ int units(int n_in) { return n_in >> 6; }
+  static __device__ __forceinline__ int64_t row_bytes(int n_in) { return (int64_t)(n_in >> 8) * 210; }
+  static __device__ __forceinline__ void kmap(int k, int& u, int& p) {
+    const int b = k >> 8, r = k & 255;
+    const int h = r >> 7, rr = r & 127;
+    const int j = rr >> 5, l = rr & 31;
+    u = 4 * b + 2 * h + (l >> 4);
+    p = 16 * j + (l & 15);
+  }
+  struct Raw { uint4 a, b, h; uint32_t sc0, sc1; uint32_t d; int s; };
+  static __device__ __forceinline__ Raw load(const uint8_t* row, int u, int) {
+    Raw r;
+    const uint8_t* p = row + 210 * (int64_t)(u >> 2);
+    const int h = (u >> 1) & 1;
+    r.s = u & 1;
+    r.a = load16_a2(p + 64 * h + 16 * r.s);
+    r.b = load16_a2(p + 64 * h + 32 + 16 * r.s);
+    r.h = load16_a2(p + 128 + 32 * h + 16 * r.s);
+    r.sc0 = load4_a2(p + 192 + 8 * h);
+    r.sc1 = load4_a2(p + 196 + 8 * h);
+    r.d = load2(p + 208);
+    return r;
+  }
+  static __device__ __forceinline__ float dot(const Raw& r, const float (&x)[64]) {
+    const uint32_t A[4] = {r.a.x, r.a.y, r.a.z, r.a.w};
+    const uint32_t B[4] = {r.b.x, r.b.y, r.b.z, r.b.w};
+    const uint32_t H[4] = {r.h.x, r.h.y, r.h.z, r.h.w};
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        const uint32_t a = (A[i] >> (8 * k)) & 0xFFu, b = (B[i] >> (8 * k)) & 0xFFu;
+        const uint32_t h = (H[i] >> (8 * k)) & 0xFFu;
+        const int q1 = (int)((a & 0xF) | (((h >> 0) & 3) << 4)) - 32;
+        const int q2 = (int)((b & 0xF) | (((h >> 2) & 3) << 4)) - 32;
+        const int q3 = (int)((a >> 4) | (((h >> 4) & 3) << 4)) - 32;
+        const int q4 = (int)((b >> 4) | (((h >> 6) & 3) << 4)) - 32;
+        const int l = 4 * i + k;
+        s[0] = fmaf_((float)q1, x[l], s[0]);
+        s[1] = fmaf_((float)q2, x[16 + l], s[1]);
+        s[2] = fmaf_((float)q3, x[32 + l], s[2]);
+        s[3] = fmaf_((float)q4, x[48 + l], s[3]);
+      }
+    }
+    const float d = f16_bits_to_f32((uint16_t)r.d);
+    // scale bytes of this half: index s + 2j
+    const uint32_t lo = r.sc0 >> (8 * r.s), hi = r.sc1 >> (8 * r.s);
+    const float c0 = (float)(int8_t)(lo & 0xFF), c1 = (float)(int8_t)((lo >> 16) & 0xFF);
+    const float c2 = (float)(int8_t)(hi & 0xFF), c3 = (float)(int8_t)((hi >> 16) & 0xFF);
+    return ((d * c0) * s[0] + (d * c1) * s[1]) + ((d * c2) * s[2] + (d * c3) * s[3]);
+  }
+};
+
+__device__ __forceinline__ float load_bias(const void* bias, int bias_dtype, int64_t n) {
+  if (bias == nullptr) return 0.f;
+  if (bias_dtype == kF32) return static_cast<const float*>(bias)[n];
+  const uint16_t b = static_cast<const uint16_t*>(bias)[n];
+  return bias_dtype == kF16 ? f16_bits_to_f32(b) : bf16_bits_to_f32(b);
+}
+
+// ------------------------------------------------------------------------- generic kernel
+// XREG: a row has at most 64 units, so each lane keeps its activations in registers.
+template <class F, typename XT, typename YT, bool XREG>
+__global__ void __launch_bounds__(kGemvThreads)
+gemv_generic_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, YT* __restrict__ y,
+                    const void* __restrict__ bias, int bias_dtype, int n_out, int n_in) {
+  extern __shared__ float xs[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const XT* xm = x + (int64_t)blockIdx.y * n_in;
+  YT* ym = y + (int64_t)blockIdx.y * n_out;
+  const int units = F::units(n_in);
+  const int nit = (units + 63) >> 6;
+
+  for (int k = tid; k < nit * 4096; k += kGemvThreads) {
+    const float v = (k < n_in) ? XElem<XT>::load(xm, k) : 0.f;
+    int u, p;
+    F::kmap(k, u, p);
+    xs[xslot_f32(u, p)] = v;
+  }
+  __syncthreads();
+
+  const int64_t rb = F::row_bytes(n_in);
+  const int first = blockIdx.x * kGemvWaves + wave;
+  const int stride = gridDim.x * kGemvWaves;
+  const float4* xs4 = reinterpret_cast<const float4*>(xs);
+
+  if constexpr (XREG) {
+    float xr[64];
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const float4 v = xs4[r * 64 + lane];
+      xr[4 * r] = v.x; xr[4 * r + 1] = v.y; xr[4 * r + 2] = v.z; xr[4 * r + 3] = v.w;
+    }
+    const bool active = lane < units;
+    int row = first;
+    // two rows per trip keeps more loads in flight
+    for (; row + stride < n_out; row += 2 * stride) {
+      float a0 = 0.f, a1 = 0.f;
+      if (active) {
+        const typename F::Raw r0 = F::load(w + rb * row, lane, n_in);
+        const typename F::Raw r1 = F::load(w + rb * (row + stride), lane, n_in);
+        a0 = F::dot(r0, xr);
+        a1 = F::dot(r1, xr);
+      }
+      a0 = wave_sum(a0);
+      a1 = wave_sum(a1);
+      if (lane == 0) {
+        YElem<YT>::store(ym, row, a0 + load_bias(bias, bias_dtype, row));
+        YElem<YT>::store(ym, row + stride, a1 + load_bias(bias, bias_dtype, row + stride));
+      }
+    }
+    for (; row < n_out; row += stride) {
+      float a0 = 0.f;
+      if (active) a0 = F::dot(F::load(w + rb * row, lane, n_in), xr);
+      a0 = wave_sum(a0);
+      if (lane == 0) YElem<YT>::store(ym, row, a0 + load_bias(bias, bias_dtype, row));
+    }
+  } else {
+    for (int row = first; row < n_out; row += stride) {
+      float acc = 0.f;
+      for (int it = 0; it < nit; it++) {
+        const int u = it * 64 + lane;
+        if (u < units) {
+          const typename F::Raw r = F::load(w + rb * row, u, n_in);
+          float xr[64];
+#pragma unroll
+          for (int q = 0; q < 16; q++) {
+            const float4 v = xs4[(it * 16 + q) * 64 + lane];
+            xr[4 * q] = v.x; xr[4 * q + 1] = v.y; xr[4 * q + 2] = v.z; xr[4 * q + 3] = v.w;
+          }
+          acc += F::dot(r, xr);
+        }
+      }
+      acc = wave_sum(acc);
+      if (lane == 0) YElem<YT>::store(ym, row, acc + load_bias(bias, bias_dtype, row));
+    }
+  }
+}
+
+// Launch geometry: enough workgroups to give every SIMD several wavefronts, never more
+// wavefronts than rows.  TTQ_GEMV_WG_PER_CU overrides the per-CU workgroup count.
+static int gemv_grid(int64_t n_out, int default_per_cu) {
+  static int per_cu_env = -1;
+  if (per_cu_env < 0) {
+    const char* e = getenv("TTQ_GEMV_WG_PER_CU");
+    per_cu_env = e ? atoi(e) : 0;
+  }
+  const int per_cu = per_cu_env > 0 ? per_cu_env : default_per_cu;
+  int cus = 256;
+  int dev = 0;
+  hipDeviceProp_t prop;
+  static int cached_cus = 0;
+  if (cached_cus == 0) {
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      cached_cus = prop.multiProcessorCount;
+    else
+      cached_cus = cus;
+  }
+  cus = cached_cus;
+  int64_t g = (int64_t)cus * per_cu;
+  const int64_t need = (n_out + kGemvWaves - 1) / kGemvWaves;
+  if (g > need) g = need;
+  if (g < 1) g = 1;
+  return (int)g;
+}
+
+template <class F, typename XT, typename YT>
+static hipError_t launch_generic(const void* w, const void* x, void* y, const void* bias,
+                                 int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                                 hipStream_t s) {
+  const int units = (int)((n_in + 63) / 64);
+  const int nit = (units + 63) / 64;
+  const size_t lds = (size_t)nit * 4096 * sizeof(float);
+  const dim3 grid(gemv_grid(n_out, 4), (unsigned)m), block(kGemvThreads);
+  if (nit == 1) {
+    hipLaunchKernelGGL((gemv_generic_kernel<F, XT, YT, true>), grid, block, lds, s,
+                       static_cast<const uint8_t*>(w), static_cast<const XT*>(x),
+                       static_cast<YT*>(y), bias, bias_dtype, (int)n_out, (int)n_in);
+  } else {
+    hipLaunchKernelGGL((gemv_generic_kernel<F, XT, YT, false>), grid, block, lds, s,
+                       static_cast<const uint8_t*>(w), static_cast<const XT*>(x),
+                       static_cast<YT*>(y), bias, bias_dtype, (int)n_out, (int)n_in);
+  }
+  return hipGetLastError();
+}
+
+template <class F, typename XT>
+static hipError_t launch_generic_y(const void* w, const void* x, void* y, int y_dtype,
+                                   const void* bias, int bias_dtype, int64_t m, int64_t n_out,
+                                   int64_t n_in, hipStream_t s) {
+  switch (y_dtype) {
+    case kF32: return launch_generic<F, XT, float>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kF16: return launch_generic<F, XT, f16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kBF16: return launch_generic<F, XT, bf16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+template <class F>
+static hipError_t launch_generic_xy(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                                    const void* bias, int bias_dtype, int64_t m, int64_t n_out,
+                                    int64_t n_in, hipStream_t s) {
+  switch (x_dtype) {
+    case kF32: return launch_generic_y<F, float>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kF16: return launch_generic_y<F, f16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kBF16: return launch_generic_y<F, bf16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+hipError_t launch_gemv(int format, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                       const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                       hipStream_t s) {
+  if (m == 0 || n_out == 0) return hipSuccess;
+  switch (format) {
+    case kQ8_0: return launch_generic_xy<FmtQ8_0>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kQ4_K: return launch_generic_xy<FmtQ4_K>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kQ6_K: return launch_generic_xy<FmtQ6_K>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace ttq

@@ -1,0 +1,40 @@
+// Internal launcher interface between the C-ABI layer (ttq_api.hip) and the kernel files.
+// Every launcher assumes its arguments were validated by the caller and returns the
+// hipError_t of the launch.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ttq {
+
+// dtype codes as in ttq.h (TTQ_F32 = 0, TTQ_F16 = 1, TTQ_BF16 = 2)
+enum : int { kF32 = 0, kF16 = 1, kBF16 = 2 };
+// format codes as in ttq.h
+enum : int { kQ8_0 = 0, kQ4_K = 1, kQ6_K = 2, kEXL3 = 3 };
+
+constexpr int64_t kMaxGemvInF32 = 16384;    // activations staged in 64 KiB of LDS
+constexpr int64_t kMaxGemvIn16 = 32768;
+
+hipError_t launch_dequant(int format, const void* w, void* out, int out_dtype, int64_t n_out,
+                          int64_t n_in, hipStream_t s);
+
+// y (m, n_out) in y_dtype = x (m, n_in) in x_dtype times W^T, optional bias (n_out).
+hipError_t launch_gemv(int format, const void* w, const void* x, int x_dtype, void* y,
+                       int y_dtype, const void* bias, int bias_dtype, int64_t m, int64_t n_out,
+                       int64_t n_in, hipStream_t s);
+
+hipError_t launch_gemm_q4k(const void* w, const uint16_t* x_bf16, void* y, int y_dtype,
+                           const void* bias, int bias_dtype, int64_t m, int64_t n_out,
+                           int64_t n_in, hipStream_t s);
+
+hipError_t launch_dequant_exl3(const uint16_t* trellis, uint16_t* out_f16, int64_t n_out,
+                               int64_t n_in, int bits, int cb, hipStream_t s);
+hipError_t launch_gemv_exl3(const uint16_t* trellis, const uint16_t* suh, const uint16_t* svh,
+                            const void* x, int x_dtype, void* y, int y_dtype, const void* bias,
+                            int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, int bits,
+                            int cb, hipStream_t s);
+hipError_t launch_hadamard128(float* v, const uint16_t* pre, const uint16_t* post, int64_t n,
+                              hipStream_t s);
+
+}  // namespace ttq

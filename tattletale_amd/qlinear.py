@@ -1,0 +1,210 @@
+"""``QuantLinear`` -- host-side mirror of the reference's ``Linear`` layer over the C ABI.
+
+Reference interface (workspace/transformers/src/layers/linear.nim:13-57)::
+
+    Linear{weight, bias, in_features, out_features}
+    Linear.init(weight, bias = none)      # weight (out_features, in_features)
+    forward(self, x)                      # x (..., in_features) -> (..., out_features)
+
+``QuantLinear`` keeps the same shape contract and the same two verbs.  The dense weight is
+replaced by a packed buffer (uint8 blocks for Q8_0/Q4_K/Q6_K, u16 trellis words plus the
+``suh``/``svh`` vectors for EXL3), so ``init`` takes the dimensions explicitly.  ``forward``
+makes one ``ttq_linear_forward`` call; like ``Linear.forward`` it launches asynchronously on
+the current stream and returns a tensor.  torch is used for device memory and streams only.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from . import _lib
+from ._lib import BF16, F16, F32, QLinearStruct, TtqError, check
+
+_DTYPE_CODE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
+
+
+def _code(dt: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dt]
+    except KeyError:
+        raise TtqError(_lib.ERR_DTYPE, "dtype %s" % dt) from None
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _stream(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _require_device(*tensors: Optional[torch.Tensor]) -> torch.device:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise TtqError(_lib.ERR_UNSUPPORTED, "tensor is not on a GPU (no CPU fallback exists)")
+        if dev is not None and t.device != dev:
+            raise TtqError(_lib.ERR_UNSUPPORTED, "tensors on different devices")
+        dev = t.device
+        if not t.is_contiguous():
+            raise TtqError(_lib.ERR_SHAPE, "tensor must be contiguous")
+    return dev
+
+
+@dataclass
+class QuantLinear:
+    """Quantized linear layer; fields follow ``Linear`` (linear.nim:13-27)."""
+
+    qweight: torch.Tensor                 # packed bytes / trellis words, on the GPU
+    format: int                           # _lib.Q8_0 | Q4_K | Q6_K | EXL3
+    in_features: int
+    out_features: int
+    bias: Optional[torch.Tensor] = None   # (out_features,)
+    suh: Optional[torch.Tensor] = None    # EXL3: (in_features,) float16
+    svh: Optional[torch.Tensor] = None    # EXL3: (out_features,) float16
+    bits: int = 0
+    codebook: int = _lib.CB_MCG
+
+    @classmethod
+    def init(cls, qweight: torch.Tensor, format: int, in_features: int, out_features: int,
+             bias: Optional[torch.Tensor] = None, suh: Optional[torch.Tensor] = None,
+             svh: Optional[torch.Tensor] = None, bits: int = 0,
+             codebook: int = _lib.CB_MCG) -> "QuantLinear":
+        """Creates the layer from existing packed weights (no copy, no repacking), as
+        ``Linear.init`` does from a dense weight (linear.nim:29-43)."""
+        _require_device(qweight, bias, suh, svh)
+        need = _lib.lib().ttq_packed_nbytes(format, out_features, in_features, bits)
+        if need < 0:
+            raise TtqError(int(need), "QuantLinear.init")
+        have = qweight.numel() * qweight.element_size()
+        if have != need:
+            raise TtqError(_lib.ERR_SHAPE, "QuantLinear.init: packed buffer holds %d bytes, %d expected"
+                           % (have, need))
+        if bias is not None and bias.numel() != out_features:
+            raise TtqError(_lib.ERR_SHAPE, "QuantLinear.init: bias length")
+        if format == _lib.EXL3:
+            if suh is None or svh is None:
+                raise TtqError(_lib.ERR_NULL, "QuantLinear.init: EXL3 needs suh and svh")
+            if suh.dtype != torch.float16 or svh.dtype != torch.float16:
+                raise TtqError(_lib.ERR_DTYPE, "QuantLinear.init: suh/svh must be float16")
+            if suh.numel() != in_features or svh.numel() != out_features:
+                raise TtqError(_lib.ERR_SHAPE, "QuantLinear.init: suh/svh length")
+        return cls(qweight, format, in_features, out_features, bias, suh, svh, bits, codebook)
+
+    def _struct(self) -> QLinearStruct:
+        return QLinearStruct(
+            format=self.format, bits=self.bits, codebook=self.codebook,
+            bias_dtype=_code(self.bias.dtype) if self.bias is not None else 0,
+            n_out=self.out_features, n_in=self.in_features,
+            qweight=_ptr(self.qweight), suh=_ptr(self.suh), svh=_ptr(self.svh), bias=_ptr(self.bias))
+
+    def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        """x (..., in_features) -> (..., out_features)  (linear.nim:45-57).
+
+        ``out_dtype`` defaults to ``x.dtype`` (what ``F.linear`` returns); pass
+        ``torch.float32`` for fp32 logits from 16-bit activations."""
+        if x.shape[-1] != self.in_features:
+            raise TtqError(_lib.ERR_SHAPE, "QuantLinear.forward: last dim %d != in_features %d"
+                           % (x.shape[-1], self.in_features))
+        dev = _require_device(self.qweight, x)
+        out_dtype = out_dtype or x.dtype
+        m = x.numel() // self.in_features
+        # the trellis path rotates its output in place in fp32
+        y_dtype = torch.float32 if self.format == _lib.EXL3 else out_dtype
+        y = torch.empty(x.shape[:-1] + (self.out_features,), dtype=y_dtype, device=dev)
+        st = self._struct()
+        with torch.cuda.device(dev):
+            check(_lib.lib().ttq_linear_forward(C.byref(st), x.data_ptr(), _code(x.dtype), m, y.data_ptr(),
+                                                _code(y_dtype), _stream(dev)), "ttq_linear_forward")
+        return y if y_dtype == out_dtype else y.to(out_dtype)
+
+    __call__ = forward
+
+
+# ------------------------------------------------------------------------- functional API
+_GEMV = {_lib.Q8_0: "ttq_gemv_q8_0", _lib.Q4_K: "ttq_gemv_q4_k", _lib.Q6_K: "ttq_gemv_q6_k"}
+_DEQ = {_lib.Q8_0: "ttq_dequant_q8_0", _lib.Q4_K: "ttq_dequant_q4_k", _lib.Q6_K: "ttq_dequant_q6_k"}
+
+
+def gemv(fmt: int, qweight: torch.Tensor, x: torch.Tensor, n_out: int, n_in: int,
+         out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 y (m, n_out) = x (m, n_in) * W^T through ``ttq_gemv_<fmt>``."""
+    dev = _require_device(qweight, x, out)
+    m = x.numel() // n_in
+    if out is None:
+        out = torch.empty((m, n_out), dtype=torch.float32, device=dev)
+    fn = getattr(_lib.lib(), _GEMV[fmt])
+    with torch.cuda.device(dev):
+        check(fn(qweight.data_ptr(), x.data_ptr(), _code(x.dtype), out.data_ptr(), m, n_out, n_in,
+                 _stream(dev)), _GEMV[fmt])
+    return out
+
+
+def gemv_exl3(trellis: torch.Tensor, suh: torch.Tensor, svh: torch.Tensor, x: torch.Tensor,
+              n_out: int, n_in: int, bits: int, codebook: int = _lib.CB_MCG,
+              out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    dev = _require_device(trellis, suh, svh, x, out)
+    if x.dtype != torch.float16:
+        raise TtqError(_lib.ERR_DTYPE, "ttq_gemv_exl3 takes float16 activations")
+    m = x.numel() // n_in
+    if out is None:
+        out = torch.empty((m, n_out), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        check(_lib.lib().ttq_gemv_exl3(trellis.data_ptr(), suh.data_ptr(), svh.data_ptr(), x.data_ptr(),
+                                       out.data_ptr(), m, n_out, n_in, bits, codebook, _stream(dev)),
+              "ttq_gemv_exl3")
+    return out
+
+
+def gemm_q4_k(qweight: torch.Tensor, x: torch.Tensor, n_out: int, n_in: int,
+              out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """bf16 Y (m, n_out) = bf16 X (m, n_in) * W^T through ``ttq_gemm_q4_k``."""
+    dev = _require_device(qweight, x, out)
+    if x.dtype != torch.bfloat16:
+        raise TtqError(_lib.ERR_DTYPE, "ttq_gemm_q4_k takes bfloat16 activations")
+    m = x.numel() // n_in
+    if out is None:
+        out = torch.empty((m, n_out), dtype=torch.bfloat16, device=dev)
+    with torch.cuda.device(dev):
+        check(_lib.lib().ttq_gemm_q4_k(qweight.data_ptr(), x.data_ptr(), out.data_ptr(), m, n_out, n_in,
+                                       _stream(dev)), "ttq_gemm_q4_k")
+    return out
+
+
+def dequantize(fmt: int, qweight: torch.Tensor, n_out: int, n_in: int,
+               dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """Dense (n_out, n_in) weight from packed blocks through ``ttq_dequant_<fmt>``."""
+    dev = _require_device(qweight)
+    out = torch.empty((n_out, n_in), dtype=dtype, device=dev)
+    fn = getattr(_lib.lib(), _DEQ[fmt])
+    with torch.cuda.device(dev):
+        check(fn(qweight.data_ptr(), out.data_ptr(), _code(dtype), n_out, n_in, _stream(dev)), _DEQ[fmt])
+    return out
+
+
+def dequantize_exl3(trellis: torch.Tensor, n_out: int, n_in: int, bits: int,
+                    codebook: int = _lib.CB_MCG) -> torch.Tensor:
+    """Decoded (unscaled, unrotated) trellis values, float16 (n_out, n_in)."""
+    dev = _require_device(trellis)
+    out = torch.empty((n_out, n_in), dtype=torch.float16, device=dev)
+    with torch.cuda.device(dev):
+        check(_lib.lib().ttq_dequant_exl3(trellis.data_ptr(), out.data_ptr(), n_out, n_in, bits, codebook,
+                                          _stream(dev)), "ttq_dequant_exl3")
+    return out
+
+
+def hadamard128_(v: torch.Tensor, pre: Optional[torch.Tensor] = None,
+                 post: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """In-place 128-group Hadamard transform of a float32 tensor (optional fp16 pre/post scale)."""
+    dev = _require_device(v, pre, post)
+    if v.dtype != torch.float32:
+        raise TtqError(_lib.ERR_DTYPE, "hadamard128_ takes float32")
+    with torch.cuda.device(dev):
+        check(_lib.lib().ttq_hadamard128_f32(v.data_ptr(), _ptr(pre), _ptr(post), v.numel(), _stream(dev)),
+              "ttq_hadamard128_f32")
+    return v

@@ -1,0 +1,85 @@
+"""Q4_K prefill GEMM on the GPU against the CPU oracle, through the C ABI.
+
+Tolerance: relative L2 error <= 2e-2 against the float64 product over oracle-dequantized
+weights (bf16 MFMA inputs, fp32 accumulation, bf16 output).  With X = [I; 0] each output is
+a single bf16-rounded weight, which must match the oracle exactly."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from tattletale_amd import QuantLinear, formats as F
+from tattletale_amd import configs as CFG
+from tattletale_amd import qlinear as QL
+from tattletale_amd import quantize as Q
+
+from util import DEV, bits_to_dev, dev_bits, packed_to_dev, rel_l2, x_to_dev, random_blocks
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-2
+
+
+@pytest.mark.parametrize("m,n_out,n_in", [(64, 256, 1024), (128, 128, 256), (16, 384, 512), (100, 200, 768),
+                                          (257, 130, 1024), (512, 512, 4096)])
+def test_gemm_random(m, n_out, n_in):
+    w = Q.fill_normal(300 + m, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
+    p = Q.quantize(F.Q4_K, w)
+    what = oracle.dequant(F.Q4_K, p, n_out, n_in)
+    xd, xf = x_to_dev(Q.fill_normal(301 + m, 1, 1.0, m * n_in).reshape(m, n_in), "bf16")
+    y = QL.gemm_q4_k(packed_to_dev(p), xd, n_out, n_in)
+    assert y.shape == (m, n_out) and y.dtype == torch.bfloat16
+    got = oracle.bf16_to_f32(dev_bits(y))
+    want = oracle.linear_f64(what, xf)
+    assert rel_l2(got, want) <= TOL
+    # against the bf16-rounded weights the kernel really multiplies, only output rounding remains
+    want_r = oracle.linear_f64(oracle.bf16_to_f32(oracle.f32_to_bf16(what)), xf)
+    assert rel_l2(got, want_r) <= 4e-3
+
+
+@pytest.mark.parametrize("n_in", [256, 1024])
+def test_gemm_identity_activations_give_bf16_weights_exactly(n_in):
+    n_out = 192
+    p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=17)
+    what = oracle.dequant(F.Q4_K, p, n_out, n_in)
+    m = n_in + 32                                    # [I; 0]: extra zero rows
+    x = np.zeros((m, n_in), np.float32)
+    x[np.arange(n_in), np.arange(n_in)] = 1.0
+    xd, _ = x_to_dev(x, "bf16")
+    y = dev_bits(QL.gemm_q4_k(packed_to_dev(p), xd, n_out, n_in))
+    assert np.array_equal(y[:n_in], oracle.f32_to_bf16(what).T)
+    assert not (y[n_in:] & 0x7FFF).any()
+
+
+def test_forward_dispatches_prefill_to_gemm_and_matches_gemv():
+    n_out, n_in, m = 256, 1024, 48
+    w = Q.fill_normal(400, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
+    p = Q.quantize(F.Q4_K, w)
+    what = oracle.dequant(F.Q4_K, p, n_out, n_in)
+    bias = Q.fill_normal(401, 2, 0.5, n_out)
+    xd, xf = x_to_dev(Q.fill_normal(402, 1, 1.0, m * n_in).reshape(4, 12, n_in), "bf16")
+    bd, bf = x_to_dev(bias, "f32")
+    layer = QuantLinear.init(packed_to_dev(p), F.Q4_K, n_in, n_out, bias=bd)
+    y = layer.forward(xd)
+    assert y.shape == (4, 12, n_out) and y.dtype == torch.bfloat16
+    want = oracle.linear_f64(what, xf.reshape(m, n_in), bf).reshape(4, 12, n_out)
+    assert rel_l2(oracle.bf16_to_f32(dev_bits(y)), want) <= TOL
+    y32 = layer.forward(xd, out_dtype=torch.float32)
+    assert rel_l2(y32.cpu().numpy(), want) <= TOL
+    # decode of one of the rows agrees with its prefill row up to bf16 weight rounding
+    row = layer.forward(xd[1, 5], out_dtype=torch.float32).cpu().numpy()
+    assert rel_l2(row, y32[1, 5].cpu().numpy()) <= 5e-3
+
+
+@pytest.mark.parametrize("name,step", [("q4_k_gemm_m64", 7), ("q4_k_gemm_m512", 29), ("q4_k_gemm_m2048", 113)])
+def test_full_shape_sampled_columns(name, step):
+    cfg = CFG.CONFIGS[name]
+    p = CFG.packed_weights(cfg)
+    xbits = CFG.activations(cfg)
+    y = QL.gemm_q4_k(packed_to_dev(p), bits_to_dev(xbits, "bf16"), cfg.n_out, cfg.n_in)
+    cols = np.unique(np.concatenate([np.arange(0, cfg.n_out, step), np.arange(cfg.n_out - 130, cfg.n_out)]))
+    sub = np.ascontiguousarray(p.reshape(cfg.n_out, -1)[cols])
+    what = oracle.dequant(F.Q4_K, sub, cols.size, cfg.n_in)
+    rows = np.unique(np.concatenate([np.arange(0, cfg.m, max(1, cfg.m // 64)), [cfg.m - 1]]))
+    want = oracle.linear_f64(what, oracle.bf16_to_f32(xbits[rows]))
+    got = oracle.bf16_to_f32(dev_bits(y[torch.from_numpy(rows).to(DEV)][:, torch.from_numpy(cols).to(DEV)]))
+    assert rel_l2(got, want) <= TOL

@@ -1,0 +1,147 @@
+"""Decode GEMV on the GPU against the CPU oracle, through the C ABI.
+
+Tolerance: relative L2 error <= 1e-3 against the float64-accumulated product over
+oracle-dequantized weights (fp32 accumulation on the GPU).  Unit-vector activations must
+reproduce the dequantized column bit for bit, which pins the fused in-register dequant."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from tattletale_amd import QuantLinear, TtqError, formats as F
+from tattletale_amd import configs as CFG
+from tattletale_amd import qlinear as QL
+from tattletale_amd import quantize as Q
+
+from util import DEV, dev_bits, packed_to_dev, rel_l2, x_to_dev, random_blocks
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+FMTS = [F.Q8_0, F.Q4_K, F.Q6_K]
+
+
+def make(fmt, n_out, n_in, seed):
+    w = Q.fill_normal(seed, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
+    p = Q.quantize(fmt, w)
+    return p, oracle.dequant(fmt, p, n_out, n_in)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("xk", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("n_out,n_in", [(64, 256), (131, 1024), (1000, 4096), (77, 4096 + 512), (33, 14336)])
+def test_gemv_random_activations(fmt, xk, n_out, n_in):
+    p, what = make(fmt, n_out, n_in, 1000 + fmt)
+    xd, xf = x_to_dev(Q.fill_normal(2000 + fmt, 1, 1.0, n_in), xk)
+    y = QL.gemv(fmt, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()[0]
+    assert rel_l2(y, oracle.linear_f64(what, xf)[0]) <= TOL
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("xk", ["f32", "bf16"])
+@pytest.mark.parametrize("n_in", [1024, 4096, 8192])
+def test_gemv_unit_vectors_reproduce_columns_bit_exactly(fmt, xk, n_in):
+    n_out = 70
+    p = random_blocks(fmt, n_out * (n_in // (32 if fmt == F.Q8_0 else 256)), seed=7 + fmt)
+    what = oracle.dequant(fmt, p, n_out, n_in)
+    cols = [0, 1, 31, 32, 33, 63, 64, 95, 127, 128, 255, 256, 300, n_in - 129, n_in - 33, n_in - 1]
+    x = np.zeros((len(cols), n_in), np.float32)
+    for i, c in enumerate(cols):
+        x[i, c] = 1.0
+    xd, _ = x_to_dev(x, xk)
+    y = QL.gemv(fmt, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()       # batched rows, m = 16
+    for i, c in enumerate(cols):
+        assert np.array_equal(y[i].view(np.uint32), what[:, c].copy().view(np.uint32)), (fmt, c)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_gemv_linearity_and_ones(fmt):
+    n_out, n_in = 256, 4096
+    p, what = make(fmt, n_out, n_in, 55)
+    pd = packed_to_dev(p)
+    ones, _ = x_to_dev(np.ones(n_in, np.float32), "bf16")
+    y1 = QL.gemv(fmt, pd, ones, n_out, n_in).cpu().numpy()[0]
+    assert rel_l2(y1, what.astype(np.float64).sum(axis=1)) <= TOL             # row sums
+    a = Q.fill_normal(56, 1, 1.0, n_in)
+    xa, af = x_to_dev(a, "f32")
+    x2, _ = x_to_dev(2.0 * af, "f32")
+    ya = QL.gemv(fmt, pd, xa, n_out, n_in).cpu().numpy()[0]
+    y2 = QL.gemv(fmt, pd, x2, n_out, n_in).cpu().numpy()[0]
+    assert np.array_equal(y2, 2.0 * ya)                                       # exact power-of-two scaling
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_quantlinear_forward_shapes_bias_and_dtypes(fmt):
+    """The operator-level entry: (..., in) -> (..., out), optional bias, output dtype."""
+    n_out, n_in = 200, 1024
+    p, what = make(fmt, n_out, n_in, 90)
+    bias = Q.fill_normal(91, 2, 0.5, n_out)
+    x = Q.fill_normal(92, 1, 1.0, 2 * 3 * n_in).reshape(2, 3, n_in)
+    xd, xf = x_to_dev(x, "bf16")
+    bd, bf = x_to_dev(bias, "bf16")
+    layer = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out, bias=bd)
+    want = oracle.linear_f64(what, xf.reshape(6, n_in), bf).reshape(2, 3, n_out)
+    y32 = layer.forward(xd, out_dtype=torch.float32)
+    assert y32.shape == (2, 3, n_out) and y32.dtype == torch.float32
+    assert rel_l2(y32.cpu().numpy(), want) <= TOL
+    y16 = layer.forward(xd)                                                   # dtype follows x
+    assert y16.dtype == torch.bfloat16
+    assert rel_l2(oracle.bf16_to_f32(dev_bits(y16)), want) <= 1e-2            # bf16 output rounding
+    nobias = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out)
+    y0 = nobias.forward(xd[0, 0], out_dtype=torch.float32)
+    assert y0.shape == (n_out,)
+    assert rel_l2(y0.cpu().numpy(), oracle.linear_f64(what, xf[0, 0])[0]) <= TOL
+    with pytest.raises(TtqError):
+        layer.forward(xd[..., :-1].contiguous())
+
+
+def test_row_concatenation_of_packed_weights_is_a_fused_layer():
+    """gate||up fusion by concatenating rows (mlp.nim:39) stays valid on packed bytes."""
+    n_in = 1024
+    pg, wg = make(F.Q4_K, 96, n_in, 60)
+    pu, wu = make(F.Q4_K, 160, n_in, 61)
+    fused = np.concatenate([pg, pu])
+    xd, xf = x_to_dev(Q.fill_normal(62, 1, 1.0, n_in), "bf16")
+    y = QL.gemv(F.Q4_K, packed_to_dev(fused), xd, 256, n_in).cpu().numpy()[0]
+    yg = QL.gemv(F.Q4_K, packed_to_dev(pg), xd, 96, n_in).cpu().numpy()[0]
+    yu = QL.gemv(F.Q4_K, packed_to_dev(pu), xd, 160, n_in).cpu().numpy()[0]
+    assert np.array_equal(y, np.concatenate([yg, yu]))
+
+
+def test_gemv_rejects_oversized_rows():
+    with pytest.raises(TtqError) as e:
+        QL.gemv(F.Q4_K, torch.zeros(144 * 4 * 128, dtype=torch.uint8, device=DEV),
+                torch.zeros(32768, dtype=torch.float32, device=DEV), 1, 32768)
+    assert e.value.status == F.ERR_UNSUPPORTED
+
+
+# ------------------------------------------------------------------- full benchmark shapes
+def _full(cfg_name, row_step):
+    cfg = CFG.CONFIGS[cfg_name]
+    p = CFG.packed_weights(cfg)
+    xbits = CFG.activations(cfg)
+    if cfg.x_dtype == "f32":
+        xd, xf = torch.from_numpy(xbits).to(DEV), xbits
+    else:
+        from util import bits_to_dev
+        xd = bits_to_dev(xbits, cfg.x_dtype)
+        xf = oracle.bf16_to_f32(xbits) if cfg.x_dtype == "bf16" else oracle.f16_to_f32(xbits)
+    y = QL.gemv(cfg.fmt, packed_to_dev(p), xd, cfg.n_out, cfg.n_in).cpu().numpy()[0]
+    rows = np.unique(np.concatenate([np.arange(0, cfg.n_out, row_step), np.arange(cfg.n_out - 300, cfg.n_out)]))
+    rb = p.size // cfg.n_out
+    sub = np.ascontiguousarray(p.reshape(cfg.n_out, rb)[rows])
+    what = oracle.dequant(cfg.fmt, sub, rows.size, cfg.n_in)
+    want = oracle.linear_f64(what, xf)[0]
+    assert np.all(np.isfinite(y))
+    return rel_l2(y[rows], want)
+
+
+def test_full_shape_q8_0_4096x4096():
+    assert _full("q8_0_gemv", 1) <= TOL
+
+
+def test_full_shape_q4_k_14336x4096():
+    assert _full("q4_k_gemv", 1) <= TOL
+
+
+def test_full_shape_q6_k_128256x4096_sampled_rows():
+    assert _full("q6_k_gemv", 37) <= TOL
