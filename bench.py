@@ -1,0 +1,236 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME] [--no-cpu] [--no-extra]
+
+Headline workload (`value`): Q4_K decode GEMV, W 14336x4096, batch 1, bf16 activations, fp32
+output -- weight-stream GB/s.  One step = one GEMV call.  Steps rotate through enough distinct
+copies of the packed weight (> 256 MiB in total) that the Infinity Cache cannot serve the
+stream, and are replayed from a HIP graph so that host launch cost does not starve a kernel
+that runs for a few microseconds.  All inputs are resident in HBM before the timed region.
+
+The same line carries the other configurations (Q8_0 / Q6_K / EXL3 GEMV, Q4_K GEMM at
+M = 64 / 512 / 2048) under "extra", the roofline of the dominant kernel and a CPU baseline
+timed on this machine's host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+MALL_BYTES = 256 << 20
+METRIC = "Q4_K GEMV weight GB/s (% of HBM peak); Q4_K GEMM M=512 TFLOP/s"
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--only", default=None, help="run a single configuration (name in tattletale_amd.configs)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-extra", action="store_true", help="headline workload only")
+    ap.add_argument("--eager", action="store_true", help="time plain launches instead of a HIP graph")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path runs on ONE GPU; --gpus %d is not supported "
+              "(see DESIGN.md, 'More than one GPU')" % args.gpus, file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    from tattletale_amd import configs as CFG
+    from tattletale_amd import formats as F
+    from tattletale_amd import qlinear as QL
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    TD = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
+
+    def to_dev(a: "np.ndarray", kind: str | None = None):
+        if a.dtype == np.uint16:
+            t = torch.from_numpy(a.view(np.int16)).to(dev)
+            return t.view(TD[kind]) if kind in ("f16", "bf16") else t
+        return torch.from_numpy(a).to(dev)
+
+    def time_steps(step_fn, steps: int, warmup: int, use_graph: bool):
+        """Runs `warmup` untimed and exactly `steps` timed calls of step_fn(i).
+        Returns (wall ms per step, HIP-event ms per step)."""
+        stream = torch.cuda.current_stream(dev)
+        for i in range(warmup):
+            step_fn(i)
+        torch.cuda.synchronize()
+        graph = None
+        if use_graph:
+            graph = torch.cuda.CUDAGraph()
+            side = torch.cuda.Stream(dev)
+            side.wait_stream(stream)
+            with torch.cuda.stream(side):
+                step_fn(0)
+                torch.cuda.synchronize()
+                with torch.cuda.graph(graph, stream=side):
+                    for i in range(steps):
+                        step_fn(i)
+            stream.wait_stream(side)
+            torch.cuda.synchronize()
+            graph.replay()            # untimed replay: uploads the graph
+            torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record(stream)
+        if graph is not None:
+            graph.replay()
+        else:
+            for i in range(steps):
+                step_fn(i)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
+
+    def run_config(name: str, steps: int, warmup: int):
+        cfg = CFG.CONFIGS[name]
+        t0 = time.time()
+        packed = CFG.packed_weights(cfg)
+        xh = CFG.activations(cfg)
+        log("[%s] inputs generated in %.1f s" % (name, time.time() - t0))
+        x = to_dev(xh, cfg.x_dtype)
+        if cfg.fmt == F.EXL3:
+            trellis, suh, svh = packed
+            wbytes = trellis.nbytes
+            ncopies = max(2, -(-2 * MALL_BYTES // wbytes))
+            ncopies = min(ncopies, 96)
+            tr = [to_dev(trellis) for _ in range(ncopies)]
+            suh_d, svh_d = to_dev(suh, "f16"), to_dev(svh, "f16")
+            y = torch.empty((cfg.m, cfg.n_out), dtype=torch.float32, device=dev)
+
+            def step(i):
+                QL.gemv_exl3(tr[i % ncopies], suh_d, svh_d, x, cfg.n_out, cfg.n_in, cfg.bits, F.CB_MCG, out=y)
+        else:
+            wbytes = packed.nbytes
+            ncopies = 1 if wbytes > MALL_BYTES else max(2, -(-2 * MALL_BYTES // wbytes))
+            ws = [to_dev(packed) for _ in range(ncopies)]
+            if cfg.m == 1:
+                y = torch.empty((1, cfg.n_out), dtype=torch.float32, device=dev)
+
+                def step(i):
+                    QL.gemv(cfg.fmt, ws[i % ncopies], x, cfg.n_out, cfg.n_in, out=y)
+            else:
+                y = torch.empty((cfg.m, cfg.n_out), dtype=torch.bfloat16, device=dev)
+
+                def step(i):
+                    QL.gemm_q4_k(ws[i % ncopies], x, cfg.n_out, cfg.n_in, out=y)
+        wall_ms, ev_ms = time_steps(step, steps, warmup, use_graph=not args.eager)
+        flops = 2.0 * cfg.m * cfg.n_out * cfg.n_in
+        res = {
+            "name": name, "steps": steps, "weight_bytes": int(wbytes), "weight_copies": ncopies,
+            "ms_per_step": ev_ms, "wall_ms_per_step": wall_ms,
+            "weight_GBps": wbytes / (ev_ms * 1e-3) / 1e9,
+            "TFLOPs": flops / (ev_ms * 1e-3) / 1e12,
+        }
+        if cfg.m == 1:
+            res["hbm_frac"] = res["weight_GBps"] / HBM_PEAK_GBPS
+        else:
+            res["mfma_frac"] = res["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS
+        log("[%s] %.3f us/step  %.0f GB/s  %.1f TFLOP/s" % (name, ev_ms * 1e3, res["weight_GBps"], res["TFLOPs"]))
+        del y
+        torch.cuda.empty_cache()
+        return res
+
+    def cpu_baseline():
+        """The oracle's fused packed-weight GEMV (a port of the same op to plain C) on the host
+        cores, plus ATen's dense linear on dequantized weights (what the reference runs on CPU)."""
+        import oracle
+        cfg = CFG.CONFIGS["q4_k_gemv"]
+        packed = CFG.packed_weights(cfg)
+        xf = oracle.bf16_to_f32(CFG.activations(cfg))[0]
+        threads = min(os.cpu_count() or 1, 16)
+        oracle.gemv_fused(cfg.fmt, packed, xf, cfg.n_out, cfg.n_in, threads)
+        n, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < 8.0:
+            oracle.gemv_fused(cfg.fmt, packed, xf, cfg.n_out, cfg.n_in, threads)
+            n += 1
+        dt = (time.perf_counter() - t0) / n
+        out = {"value": packed.nbytes / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+               "sample": "%d calls of the full 14336x4096 Q4_K GEMV (fused C port, OpenMP)" % n,
+               "us_per_call": dt * 1e6}
+        # reference CPU path: dense linear on the dequantized weight (ATen)
+        what = torch.from_numpy(oracle.dequant(cfg.fmt, packed, cfg.n_out, cfg.n_in)).to(torch.bfloat16)
+        xb = torch.from_numpy(xf).to(torch.bfloat16)[None, :]
+        torch.set_num_threads(threads)
+        torch.nn.functional.linear(xb, what)
+        n, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < 6.0:
+            torch.nn.functional.linear(xb, what)
+            n += 1
+        dt2 = (time.perf_counter() - t0) / n
+        out["aten_dense_bf16_us_per_call"] = dt2 * 1e6
+        out["aten_dense_bf16_weight_GBps"] = what.numel() * 2 / dt2 / 1e9
+        return out
+
+    names = [args.only] if args.only else ["q4_k_gemv"]
+    if not args.only and not args.no_extra:
+        names += ["q4_k_gemm_m512", "q8_0_gemv", "q6_k_gemv", "exl3_gemv", "q4_k_gemm_m64", "q4_k_gemm_m2048"]
+    results = {}
+    for nme in names:
+        cfg = CFG.CONFIGS[nme]
+        steps = args.steps
+        if cfg.m > 1 or nme == "q6_k_gemv":
+            steps = max(20, args.steps // 10)     # longer kernels need fewer launches
+        if cfg.m >= 2048:
+            steps = max(10, args.steps // 40)
+        results[nme] = run_config(nme, steps, max(3, args.warmup * steps // max(1, args.steps)))
+    head = results[names[0]]
+    hc = CFG.CONFIGS[names[0]]
+
+    line = {
+        "metric": METRIC,
+        "value": head["weight_GBps"] if hc.m == 1 else head["TFLOPs"],
+        "unit": "GB/s" if hc.m == 1 else "TFLOP/s",
+        "n_gpus": 1, "steps": head["steps"], "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "%s: W %dx%d %s, x %dx%d %s, y %s" % (
+            hc.name, hc.n_out, hc.n_in, {0: "Q8_0", 1: "Q4_K", 2: "Q6_K", 3: "EXL3"}[hc.fmt], hc.m, hc.n_in,
+            hc.x_dtype, hc.y_dtype),
+            "launch": "eager" if args.eager else "hip-graph replay of %d launches" % head["steps"],
+            "weight_copies_rotated": head["weight_copies"]},
+    }
+    if hc.m == 1:
+        line["roofline"] = {"bound": "hbm", "achieved": head["weight_GBps"], "peak": HBM_PEAK_GBPS,
+                            "unit": "GB/s", "frac": head["weight_GBps"] / HBM_PEAK_GBPS, "traffic": None}
+    else:
+        line["roofline"] = {"bound": "mfma", "achieved": head["TFLOPs"], "peak": MFMA_BF16_PEAK_TFLOPS,
+                            "unit": "TFLOP/s", "frac": head["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS, "traffic": None}
+    if "q4_k_gemm_m512" in results:
+        g = results["q4_k_gemm_m512"]
+        line["gemm_m512_TFLOPs"] = g["TFLOPs"]
+        line["gemm_m512_mfma_frac"] = g["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline()
+    line["extra"] = {k: v for k, v in results.items() if k != names[0]}
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -44,11 +44,12 @@ int check_gemv_limits(int x_dtype, int64_t n_in) {
 int gemv_block(int format, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
                const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                void* stream) {
-  if (!w || !x || !y) return TTQ_ERR_NULL;
   if (!valid_dtype(x_dtype) || !valid_dtype(y_dtype)) return TTQ_ERR_DTYPE;
   if (bias && !valid_dtype(bias_dtype)) return TTQ_ERR_DTYPE;
   int rc = check_shape(format, m, n_out, n_in, 0, 0);
   if (rc != TTQ_OK) return rc;
+  if (m == 0 || n_out == 0) return TTQ_OK;  // empty output: nothing to read or write
+  if (!w || !x || !y) return TTQ_ERR_NULL;
   if (!aligned16(w) || !aligned16(x) || !aligned16(y)) return TTQ_ERR_ALIGN;
   rc = check_gemv_limits(x_dtype, n_in);
   if (rc != TTQ_OK) return rc;
@@ -58,10 +59,11 @@ int gemv_block(int format, const void* w, const void* x, int x_dtype, void* y, i
 
 int dequant_block(int format, const void* w, void* out, int out_dtype, int64_t n_out, int64_t n_in,
                   void* stream) {
-  if (!w || !out) return TTQ_ERR_NULL;
   if (!valid_dtype(out_dtype)) return TTQ_ERR_DTYPE;
   const int rc = check_shape(format, 1, n_out, n_in, 0, 0);
   if (rc != TTQ_OK) return rc;
+  if (n_out == 0) return TTQ_OK;  // empty matrix
+  if (!w || !out) return TTQ_ERR_NULL;
   if (!aligned16(w) || !aligned16(out)) return TTQ_ERR_ALIGN;
   return hip_status(ttq::launch_dequant(format, w, out, out_dtype, n_out, n_in,
                                         static_cast<hipStream_t>(stream)));

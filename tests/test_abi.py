@@ -49,6 +49,7 @@ def test_gemv_validation_order(name):
     p = buf.ctypes.data
     p += (-p) % 16
     assert fn(None, p, _lib.F32, p, 1, 4, 256, None) == _lib.ERR_NULL
+    assert fn(None, None, _lib.F32, None, 0, 4, 256, None) == _lib.OK     # empty batch: nothing to do
     assert fn(p, p, 7, p, 1, 4, 256, None) == _lib.ERR_DTYPE
     assert fn(p, p, _lib.F32, p, 1, 4, 100, None) == _lib.ERR_SHAPE
     assert fn(p, p, _lib.F32, p, -1, 4, 256, None) == _lib.ERR_SHAPE
