@@ -19,6 +19,7 @@ SOURCES = [
     "ttq_api.hip",
     "ttq_dequant.hip",
     "ttq_gemv.hip",
+    "ttq_gemv_dot2.hip",
     "ttq_gemm_q4k.hip",
     "ttq_exl3.hip",
     "ttq_host.cpp",

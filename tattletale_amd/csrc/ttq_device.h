@@ -75,6 +75,14 @@ template <> struct YElem<bf16_tag> {
   static __device__ __forceinline__ void store(bf16_tag* p, int64_t i, float v) { p[i].v = f32_to_bf16_bits(v); }
 };
 
+// Optional bias element n as float (dtype codes: 0 = fp32, 1 = fp16, 2 = bf16).
+__device__ __forceinline__ float load_bias(const void* bias, int bias_dtype, int64_t n) {
+  if (bias == nullptr) return 0.f;
+  if (bias_dtype == 0) return static_cast<const float*>(bias)[n];
+  const uint16_t b = static_cast<const uint16_t*>(bias)[n];
+  return bias_dtype == 1 ? f16_bits_to_f32(b) : bf16_bits_to_f32(b);
+}
+
 // 16-byte load from an address that is only 2-byte aligned (Q6_K / Q8_0 blocks).  gfx950
 // global loads accept any alignment; the builtin copy keeps the compiler honest about it.
 __device__ __forceinline__ uint4 load16_a2(const uint8_t* p) {

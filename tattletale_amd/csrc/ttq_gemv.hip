@@ -181,13 +181,6 @@ struct FmtQ6_K {
   }
 };
 
-__device__ __forceinline__ float load_bias(const void* bias, int bias_dtype, int64_t n) {
-  if (bias == nullptr) return 0.f;
-  if (bias_dtype == kF32) return static_cast<const float*>(bias)[n];
-  const uint16_t b = static_cast<const uint16_t*>(bias)[n];
-  return bias_dtype == kF16 ? f16_bits_to_f32(b) : bf16_bits_to_f32(b);
-}
-
 // ------------------------------------------------------------------------- generic kernel
 // XREG: a row has at most 64 units, so each lane keeps its activations in registers.
 template <class F, typename XT, typename YT, bool XREG>
@@ -342,6 +335,8 @@ hipError_t launch_gemv(int format, const void* w, const void* x, int x_dtype, vo
                        const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                        hipStream_t s) {
   if (m == 0 || n_out == 0) return hipSuccess;
+  if (gemv_dot2_supported(format, x_dtype, n_in))
+    return launch_gemv_dot2(format, w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   switch (format) {
     case kQ8_0: return launch_generic_xy<FmtQ8_0>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
     case kQ4_K: return launch_generic_xy<FmtQ4_K>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);

@@ -1,0 +1,414 @@
+// Decode GEMV fast path for 16-bit activations (bf16 / fp16) on gfx950: packed dot products.
+//
+// Same operator as ttq_gemv.hip (F.linear with a single-token activation,
+// workspace/libtorch/src/abi/neural_nets.nim:64-81), different arithmetic:
+// the activations stay 16-bit, packed two to a register, and the quantized integers are
+// turned into 16-bit floats with ONE and-or each, using the fact that OR-ing a small
+// integer q into the mantissa of a suitable power of two gives an exact float:
+//       bf16:  0x4300 | q  ==  128 + q      (q < 128)
+//       fp16:  0x6400 | q  ==  1024 + q     (q < 1024)
+// v_dot2_f32_{bf16,f16} then multiplies two weights by two activations per instruction
+// and accumulates in fp32; the constant offset is removed with a per-lane sum of the
+// activations (computed once, the activations never change from row to row):
+//       sum (OFF + q) x  -  OFF * sum x  =  sum q x.
+// Scales are applied once per sub-block, so a unit-vector activation still reproduces
+// the canonical dequantized weight exactly.
+//
+// Work distribution.  Lane l always owns unit l (mod 64) of a row (a unit = 64 weights),
+// so when a row has at most 64 units the lane's 32 activation registers are loaded once.
+// Each wavefront owns a contiguous range of rows and walks it in batches of four rows,
+// double-buffered: the 16-byte loads of the next batch are in flight while the current
+// batch is unpacked, so HBM never waits for the ALUs.  The first batch is requested
+// before the activations are staged, hiding that latency too.
+#include "ttq_device.h"
+#include "ttq_internal.h"
+
+#include <stdlib.h>
+
+namespace ttq {
+
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+
+struct OpsBF16 {
+  static constexpr uint32_t kMagic = 0x43004300u;   // (128.0, 128.0)
+  static constexpr float kOffset = 128.f;
+  static constexpr uint32_t kOnes = 0x3F803F80u;    // (1.0, 1.0)
+  static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+    bf16x2_t x, y;
+    __builtin_memcpy(&x, &a, 4);
+    __builtin_memcpy(&y, &b, 4);
+    return __builtin_amdgcn_fdot2_f32_bf16(x, y, c, false);
+  }
+};
+struct OpsF16 {
+  static constexpr uint32_t kMagic = 0x64006400u;   // (1024.0, 1024.0)
+  static constexpr float kOffset = 1024.f;
+  static constexpr uint32_t kOnes = 0x3C003C00u;
+  static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+    f16x2_t x, y;
+    __builtin_memcpy(&x, &a, 4);
+    __builtin_memcpy(&y, &b, 4);
+    return __builtin_amdgcn_fdot2(x, y, c, false);
+  }
+};
+
+// (v & mask) | magic is a single v_and_or_b32 when `magic` lives in a VGPR (the instruction
+// takes no literal and only one scalar operand; with two literals the compiler falls back to
+// v_and + v_or).  opaque_vgpr() pins a constant into a VGPR without emitting anything.
+__device__ __forceinline__ uint32_t opaque_vgpr(uint32_t v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+__device__ __forceinline__ uint32_t and_or(uint32_t v, uint32_t mask, uint32_t magic_vgpr) {
+  return (v & mask) | magic_vgpr;
+}
+
+// Sum over the 64 lanes with DPP adds; the total lands in lane 63.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xF, false);
+  return v + __int_as_float(moved);
+}
+__device__ __forceinline__ float wave_sum_to_lane63(float v) {
+  v = dpp_add<0xB1, 0xF>(v);    // quad_perm [1,0,3,2]
+  v = dpp_add<0x4E, 0xF>(v);    // quad_perm [2,3,0,1]
+  v = dpp_add<0x141, 0xF>(v);   // row_half_mirror
+  v = dpp_add<0x140, 0xF>(v);   // row_mirror: every lane holds its row's sum
+  v = dpp_add<0x142, 0xA>(v);   // row_bcast:15 into rows 1 and 3
+  v = dpp_add<0x143, 0xC>(v);   // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
+// Developer timeline instrumentation, compiled in only with -DTTQ_PHASE_TRACE: lane 0 of every
+// wavefront stores the 100 MHz real-time counter at a few phase boundaries.
+#ifdef TTQ_PHASE_TRACE
+__device__ unsigned long long* g_phase_trace = nullptr;
+#define TTQ_TRACE_POINT(wave_id, slot)                                                          \
+  do {                                                                                          \
+    if (g_phase_trace != nullptr && (threadIdx.x & 63) == 0)                                    \
+      g_phase_trace[(size_t)(wave_id) * 8 + (slot)] = __builtin_amdgcn_s_memrealtime();         \
+  } while (0)
+#else
+#define TTQ_TRACE_POINT(wave_id, slot) do { } while (0)
+#endif
+
+constexpr int kFastThreads = 512;
+constexpr int kFastWaves = kFastThreads / kWave;
+constexpr int kBatch = 4;     // rows per pass when activations are re-read from LDS
+constexpr int kRing = 4;      // row buffers per wavefront when activations sit in registers
+constexpr int kEarlyRows = 1; // rows requested before the activations are staged
+
+// -------------------------------------------------------------------------------- Q4_K
+// unit u = (super-block u/4, chunk c = u%4): 32 qs bytes; low nibbles -> sub-block 2c,
+// high nibbles -> sub-block 2c+1.  Activation pairs of a unit, register 4i+kind for qs dword
+// i: kind 0 = (x[4i], x[4i+2]), 1 = (x[4i+1], x[4i+3]), 2/3 = the same 32 positions further.
+struct Q4KRaw { uint4 hdr, q0, q1; };
+
+// Per-lane constants.  A lane always decodes chunk c = lane % 4, so the bit positions of its
+// two 6-bit scales and mins inside the 12 packed bytes never change: sub-blocks 0..3 keep
+// the whole field in bytes 0..7, sub-blocks 4..7 keep 4 bits in bytes 8..11 and 2 bits on top
+// of bytes 0..7.  Written as two bit-field extracts (the second with width 0 for the simple
+// case) so that no branch is needed.
+struct Q4KLane {
+  uint32_t off_hdr, off_q;        // byte offsets of the header and the 32 qs bytes in the row
+  bool upper;                     // sub-blocks 4..7
+  uint32_t wl, wh;                // widths of the low and the high part
+  uint32_t sc_lo[2], mn_lo[2], hi[2];  // bit offsets, for sub-blocks 2c and 2c+1
+  __device__ __forceinline__ void init(int u) {
+    const int c = u & 3;
+    off_hdr = 144u * (uint32_t)(u >> 2);
+    off_q = off_hdr + 16u + 32u * (uint32_t)c;
+    upper = c >= 2;
+    wl = upper ? 4u : 6u;
+    wh = upper ? 2u : 0u;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      const uint32_t j = 2u * c + h, jj = j & 3u;
+      sc_lo[h] = 8u * jj;
+      mn_lo[h] = upper ? 8u * jj + 4u : 8u * jj;
+      hi[h] = 8u * jj + 6u;
+    }
+  }
+};
+
+__device__ __forceinline__ void q4k_load(Q4KRaw& r, const uint8_t* row, const Q4KLane& L) {
+  r.hdr = load16_a16(row + L.off_hdr);
+  r.q0 = load16_a16(row + L.off_q);
+  r.q1 = load16_a16(row + L.off_q + 16);
+}
+
+// Dot product of one unit (64 weights) with the lane's activations.  off1/off2 are
+// kOffset * sx1 / sx2.
+template <class Ops>
+__device__ __forceinline__ float q4k_unit_dot(const Q4KRaw& r, const Q4KLane& L, const uint32_t (&xr)[32],
+                                              float sx1, float sx2, float off1, float off2, uint32_t magic) {
+  const uint32_t dw[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+  constexpr uint32_t M = 0x000F000Fu;
+  float s1a = 0.f, s1b = 0.f, s2a = 0.f, s2b = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const uint32_t q = dw[i];
+    s1a = Ops::dot2(and_or(q, M, magic), xr[4 * i + 0], s1a);
+    s1b = Ops::dot2(and_or(q >> 8, M, magic), xr[4 * i + 1], s1b);
+    s2a = Ops::dot2(and_or(q >> 4, M, magic), xr[4 * i + 2], s2a);
+    s2b = Ops::dot2(and_or(q >> 12, M, magic), xr[4 * i + 3], s2b);
+  }
+  const float q1 = (s1a + s1b) - off1;   // sum q*x over sub-block 2c
+  const float q2 = (s2a + s2b) - off2;   // sub-block 2c+1
+  const float d = f16_bits_to_f32((uint16_t)(r.hdr.x & 0xFFFF));
+  const float dmin = f16_bits_to_f32((uint16_t)(r.hdr.x >> 16));
+  const uint32_t a_sc = L.upper ? r.hdr.w : r.hdr.y;   // bytes 8-11 or 0-3
+  const uint32_t a_mn = L.upper ? r.hdr.w : r.hdr.z;   // bytes 8-11 or 4-7
+  const uint32_t sc1 = __builtin_amdgcn_ubfe(a_sc, L.sc_lo[0], L.wl) | (__builtin_amdgcn_ubfe(r.hdr.y, L.hi[0], L.wh) << 4);
+  const uint32_t sc2 = __builtin_amdgcn_ubfe(a_sc, L.sc_lo[1], L.wl) | (__builtin_amdgcn_ubfe(r.hdr.y, L.hi[1], L.wh) << 4);
+  const uint32_t mn1 = __builtin_amdgcn_ubfe(a_mn, L.mn_lo[0], L.wl) | (__builtin_amdgcn_ubfe(r.hdr.z, L.hi[0], L.wh) << 4);
+  const uint32_t mn2 = __builtin_amdgcn_ubfe(a_mn, L.mn_lo[1], L.wl) | (__builtin_amdgcn_ubfe(r.hdr.z, L.hi[1], L.wh) << 4);
+  const float t1 = (d * (float)sc1) * q1 - (dmin * (float)mn1) * sx1;
+  const float t2 = (d * (float)sc2) * q2 - (dmin * (float)mn2) * sx2;
+  return t1 + t2;
+}
+
+// LDS slot (dword) of activation-pair register `reg` of unit u: [u/64][reg/4][u%64][reg%4]
+__device__ __forceinline__ int xpair_slot(int u, int reg) {
+  return ((((u >> 6) * 8 + (reg >> 2)) * 64 + (u & 63)) << 2) + (reg & 3);
+}
+
+template <class Ops>
+__device__ __forceinline__ void load_x_regs(const uint32_t* xs, int it, int lane, uint32_t (&xr)[32],
+                                            float& sx1, float& sx2) {
+  const uint4* xs4 = reinterpret_cast<const uint4*>(xs);
+#pragma unroll
+  for (int r = 0; r < 8; r++) {
+    const uint4 v = xs4[(it * 8 + r) * 64 + lane];
+    xr[4 * r] = v.x; xr[4 * r + 1] = v.y; xr[4 * r + 2] = v.z; xr[4 * r + 3] = v.w;
+  }
+  float a = 0.f, b = 0.f, c = 0.f, d = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    a = Ops::dot2(xr[4 * i + 0], Ops::kOnes, a);
+    b = Ops::dot2(xr[4 * i + 1], Ops::kOnes, b);
+    c = Ops::dot2(xr[4 * i + 2], Ops::kOnes, c);
+    d = Ops::dot2(xr[4 * i + 3], Ops::kOnes, d);
+  }
+  sx1 = a + b;
+  sx2 = c + d;
+}
+
+template <class Ops, typename YT, bool XREG>
+__global__ void __launch_bounds__(kFastThreads)
+gemv_q4k_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
+                     const void* __restrict__ bias, int bias_dtype, int n_out, int n_in,
+                     int rows_per_wave) {
+  extern __shared__ uint32_t xs[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  // the wave index is the same in all 64 lanes: keep it (and every row address) scalar
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint16_t* xm = x + (int64_t)blockIdx.y * n_in;
+  YT* ym = y + (int64_t)blockIdx.y * n_out;
+  const int units = n_in >> 6;
+  const int nit = (units + 63) >> 6;
+  const int64_t rb = (int64_t)(n_in >> 8) * 144;
+
+  const int gw = blockIdx.x * kFastWaves + wave;
+  TTQ_TRACE_POINT(gw, 0);
+  const int row0 = gw * rows_per_wave;
+  const int row_end = min(row0 + rows_per_wave, n_out);
+  const int last = n_out - 1;
+
+  // lanes beyond the last unit of a short row read unit 0 and are given zero activations
+  const bool active = lane < units;
+  Q4KLane L;
+  L.init(active ? lane : 0);
+
+  Q4KRaw bufA[XREG ? kRing : 1];
+
+  // stage x as permuted pairs: one 16-byte load (8 activations) per thread and 4096-chunk,
+  // all chunks requested before the first is consumed
+  {
+    constexpr int kMaxChunks = XREG ? 1 : (int)(kMaxGemvIn16 / 4096);
+    uint4 xv[kMaxChunks];
+#pragma unroll
+    for (int ch = 0; ch < kMaxChunks; ch++) {
+      // unconditional loads from a clamped address keep the control flow straight, so the
+      // compiler can wait for exactly these loads and not for the weight loads behind them
+      const int k0 = ch * 4096 + 8 * tid;
+      const bool ok = ch < nit && k0 < n_in;
+      const uint4 v = *reinterpret_cast<const uint4*>(xm + (ok ? k0 : 0));
+      xv[ch] = ok ? v : make_uint4(0, 0, 0, 0);
+    }
+    // XREG: request the first kEarlyRows rows right behind the activations and the rest of the
+    // batch only once x is staged.  Under a full-rate weight stream every request waits in
+    // queues as deep as the bytes already asked for, so x must not be asked for behind a
+    // whole batch; a bare s_barrier (no memory wait) also makes sure every wavefront's x request
+    // is queued before any weight request of this workgroup.  The weight loads are
+    // unconditional and clamped to the last row, to keep the control flow straight.
+    if constexpr (XREG) {
+      __builtin_amdgcn_s_barrier();
+#pragma unroll
+      for (int r = 0; r < kEarlyRows; r++) q4k_load(bufA[r], w + rb * min(row0 + r, last), L);
+    }
+#pragma unroll
+    for (int ch = 0; ch < kMaxChunks; ch++) {
+      if (ch < nit) {
+        // thread holds x[k0 .. k0+8): unit u, qs dwords i0 = (k0 % 32) / 4 and i0 + 1
+        const int k0 = ch * 4096 + 8 * tid;
+        const int u = k0 >> 6, o = k0 & 63;
+        const int kbase = (o >> 5) << 1;          // kinds 0/1 for the low half, 2/3 for the high
+        const int i0 = (o & 31) >> 2;
+        const uint4 v = xv[ch];
+        uint2 p0, p1;
+        p0.x = (v.x & 0xFFFFu) | (v.y << 16);      // (x0, x2)
+        p0.y = (v.x >> 16) | (v.y & 0xFFFF0000u);  // (x1, x3)
+        p1.x = (v.z & 0xFFFFu) | (v.w << 16);      // (x4, x6)
+        p1.y = (v.z >> 16) | (v.w & 0xFFFF0000u);  // (x5, x7)
+        *reinterpret_cast<uint2*>(&xs[xpair_slot(u, 4 * i0 + kbase)]) = p0;
+        *reinterpret_cast<uint2*>(&xs[xpair_slot(u, 4 * (i0 + 1) + kbase)]) = p1;
+      }
+    }
+  }
+  __syncthreads();
+  TTQ_TRACE_POINT(gw, 1);
+  // wavefronts without rows fall through: their loads are clamped and their stores masked
+
+  const uint32_t magic = opaque_vgpr(Ops::kMagic);
+  auto store_rows = [&](auto& acc, int base) {
+    constexpr int kN = (int)(sizeof(acc) / sizeof(float));
+#pragma unroll
+    for (int r = 0; r < kN; r++) acc[r] = wave_sum_to_lane63(acc[r]);
+    if (lane == 63) {
+#pragma unroll
+      for (int r = 0; r < kN; r++) {
+        const int row = base + r;
+        if (row < row_end) YElem<YT>::store(ym, row, acc[r] + load_bias(bias, bias_dtype, row));
+      }
+    }
+  };
+
+  if constexpr (XREG) {
+    uint32_t xr[32];
+    float sx1, sx2;
+    load_x_regs<Ops>(xs, 0, lane, xr, sx1, sx2);
+    const float off1 = Ops::kOffset * sx1, off2 = Ops::kOffset * sx2;
+    TTQ_TRACE_POINT(gw, 2);
+
+    // Row-granular software pipeline over a ring of kRing row buffers: while row r is unpacked,
+    // rows r+1 .. r+kRing-1 are in flight (loads return in request order).  Keeping only a few
+    // rows in flight per wavefront matters: asking for everything at once fills the memory
+    // queues so deeply that issuing the requests itself stalls the wavefront for microseconds.
+    // Loads are always issued (rows past the end fetch one harmless line) so that the
+    // compiler's load counting stays exact; only the arithmetic is skipped.
+    auto fetch = [&](Q4KRaw& dst, int row) {
+      const bool valid = row < row_end;
+      const uint8_t* rp = w + rb * (valid ? row : min(row0, last));
+      const uint32_t keep = valid ? 0xFFFFFFFFu : 0u;
+      dst.hdr = load16_a16(rp + (L.off_hdr & keep));
+      dst.q0 = load16_a16(rp + (L.off_q & keep));
+      dst.q1 = load16_a16(rp + ((L.off_q + 16) & keep));
+    };
+#pragma unroll
+    for (int r = kEarlyRows; r < kRing - 1; r++) fetch(bufA[r], row0 + r);
+    for (int base = row0; base < row_end; base += kRing) {
+      float acc[kRing];
+#pragma unroll
+      for (int i = 0; i < kRing; i++) {
+        fetch(bufA[(i + kRing - 1) % kRing], base + i + kRing - 1);
+        acc[i] = 0.f;
+        if (base + i < row_end) acc[i] = q4k_unit_dot<Ops>(bufA[i], L, xr, sx1, sx2, off1, off2, magic);
+      }
+      store_rows(acc, base);
+    }
+    TTQ_TRACE_POINT(gw, 5);
+  } else {
+    // long rows: activations come from LDS for every unit
+    for (int base = row0; base < row_end; base += kBatch) {
+      float acc[kBatch];
+#pragma unroll
+      for (int r = 0; r < kBatch; r++) acc[r] = 0.f;
+      for (int it = 0; it < nit; it++) {
+        const int u = it * 64 + lane;
+        Q4KLane Lu;
+        Lu.init(u < units ? u : 0);
+        Q4KRaw buf[kBatch];
+#pragma unroll
+        for (int r = 0; r < kBatch; r++) q4k_load(buf[r], w + rb * min(base + r, last), Lu);
+        uint32_t xr[32];
+        float sx1, sx2;
+        load_x_regs<Ops>(xs, it, lane, xr, sx1, sx2);
+        const float off1 = Ops::kOffset * sx1, off2 = Ops::kOffset * sx2;
+#pragma unroll
+        for (int r = 0; r < kBatch; r++) acc[r] += q4k_unit_dot<Ops>(buf[r], Lu, xr, sx1, sx2, off1, off2, magic);
+      }
+      store_rows(acc, base);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------ launch
+static int num_cus() {
+  static int cached = 0;
+  if (cached == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      cached = prop.multiProcessorCount;
+    else
+      cached = 256;
+  }
+  return cached;
+}
+
+static int env_int(const char* name, int dflt) {
+  const char* e = getenv(name);
+  return e ? atoi(e) : dflt;
+}
+
+template <class Ops, typename YT>
+static hipError_t launch_q4k_t(const void* w, const void* x, void* y, const void* bias, int bias_dtype,
+                               int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+  static const int wg_per_cu = env_int("TTQ_GEMV_WG_PER_CU", 1);
+  const int units = (int)(n_in / 64);
+  const int nit = (units + 63) / 64;
+  int64_t waves = (int64_t)num_cus() * wg_per_cu * kFastWaves;
+  if (waves > n_out) waves = n_out;
+  int rows_per_wave = (int)((n_out + waves - 1) / waves);
+  const int64_t used_waves = (n_out + rows_per_wave - 1) / rows_per_wave;
+  const dim3 grid((unsigned)((used_waves + kFastWaves - 1) / kFastWaves), (unsigned)m), block(kFastThreads);
+  const size_t lds = (size_t)nit * 2048 * sizeof(uint32_t);
+  const uint8_t* wb = static_cast<const uint8_t*>(w);
+  const uint16_t* xb = static_cast<const uint16_t*>(x);
+  if (nit == 1)
+    hipLaunchKernelGGL((gemv_q4k_dot2_kernel<Ops, YT, true>), grid, block, lds, s, wb, xb,
+                       static_cast<YT*>(y), bias, bias_dtype, (int)n_out, (int)n_in, rows_per_wave);
+  else
+    hipLaunchKernelGGL((gemv_q4k_dot2_kernel<Ops, YT, false>), grid, block, lds, s, wb, xb,
+                       static_cast<YT*>(y), bias, bias_dtype, (int)n_out, (int)n_in, rows_per_wave);
+  return hipGetLastError();
+}
+
+template <class Ops>
+static hipError_t launch_q4k_y(const void* w, const void* x, void* y, int y_dtype, const void* bias,
+                               int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+  switch (y_dtype) {
+    case kF32: return launch_q4k_t<Ops, float>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kF16: return launch_q4k_t<Ops, f16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kBF16: return launch_q4k_t<Ops, bf16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+bool gemv_dot2_supported(int format, int x_dtype, int64_t n_in) {
+  static const int disabled = env_int("TTQ_GEMV_NO_DOT2", 0);
+  if (disabled) return false;
+  return format == kQ4_K && (x_dtype == kBF16 || x_dtype == kF16) && n_in <= kMaxGemvIn16;
+}
+
+hipError_t launch_gemv_dot2(int format, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                            const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                            hipStream_t s) {
+  if (format != kQ4_K) return hipErrorInvalidValue;
+  if (x_dtype == kBF16) return launch_q4k_y<OpsBF16>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  if (x_dtype == kF16) return launch_q4k_y<OpsF16>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  return hipErrorInvalidValue;
+}
+
+}  // namespace ttq
