@@ -44,6 +44,9 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-extra", action="store_true", help="headline workload only")
     ap.add_argument("--eager", action="store_true", help="time plain launches instead of a HIP graph")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run a plain device copy of 256 MiB a few times and exit (reference point for "
+                         "scaling the FETCH_SIZE / WRITE_SIZE counters of rocprofv3)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on ONE GPU; --gpus %d is not supported "
@@ -63,6 +66,15 @@ def main() -> int:
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     TD = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
+
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes": 256 << 20, "launches": 10}))
+        return 0
 
     def to_dev(a: "np.ndarray", kind: str | None = None):
         if a.dtype == np.uint16:
@@ -215,12 +227,22 @@ def main() -> int:
             "launch": "eager" if args.eager else "hip-graph replay of %d launches" % head["steps"],
             "weight_copies_rotated": head["weight_copies"]},
     }
+    # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (committed summary)
+    traffic = None
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            t = json.load(f).get(hc.name)
+        if t:
+            traffic = t["hbm_read_bytes"] + t["hbm_write_bytes"]
+    except (OSError, ValueError):
+        pass
     if hc.m == 1:
         line["roofline"] = {"bound": "hbm", "achieved": head["weight_GBps"], "peak": HBM_PEAK_GBPS,
-                            "unit": "GB/s", "frac": head["weight_GBps"] / HBM_PEAK_GBPS, "traffic": None}
+                            "unit": "GB/s", "frac": head["weight_GBps"] / HBM_PEAK_GBPS, "traffic": traffic,
+                            "algorithmic_bytes": head["weight_bytes"]}
     else:
         line["roofline"] = {"bound": "mfma", "achieved": head["TFLOPs"], "peak": MFMA_BF16_PEAK_TFLOPS,
-                            "unit": "TFLOP/s", "frac": head["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS, "traffic": None}
+                            "unit": "TFLOP/s", "frac": head["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS, "traffic": traffic}
     if "q4_k_gemm_m512" in results:
         g = results["q4_k_gemm_m512"]
         line["gemm_m512_TFLOPs"] = g["TFLOPs"]
