@@ -26,6 +26,19 @@
 
 namespace ttq {
 
+// Developer timeline instrumentation, compiled in only with -DTTQ_PHASE_TRACE: wavefront 0 of
+// workgroup 0 stores the shader clock at a few points of every step.
+#ifdef TTQ_PHASE_TRACE
+__device__ long long* g_gemm_trace = nullptr;
+#define TTQ_GEMM_TRACE(idx)                                                                     \
+  do {                                                                                          \
+    if (g_gemm_trace != nullptr && blockIdx.x == 0 && threadIdx.x == 0)                         \
+      g_gemm_trace[(idx)] = __builtin_readcyclecounter();                                       \
+  } while (0)
+#else
+#define TTQ_GEMM_TRACE(idx) do { } while (0)
+#endif
+
 constexpr int kGemmThreads = 256;
 constexpr int kGemmBM = 256;      // rows of X per workgroup (4 wavefronts x 64)
 constexpr int kWaveM = 64;
@@ -224,28 +237,46 @@ gemm_q4k_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, Y
   constexpr int kMfmas = 8 * NJ;
 
   // MFMA t = (s*4 + i)*NJ + j of a step, followed by the dequant pieces that fall into its slot
-  auto step_slot = [&](auto tt, const uint4 (&xa)[2][4], const bf16x8_t (&bf)[2][NJ], DqState& st,
-                       const WRaw& r, auto cc, int buf_next) {
+  // The global loads of a step are spread over the slots as well: a wavefront that issues its
+  // eight X-fragment loads back to back sits in the issue stage for about a thousand cycles
+  // (the vector-memory unit takes ~128 clk per such load), and no MFMA goes out meanwhile.
+  auto step_slot = [&](auto tt, const uint4 (&xa)[2][4], uint4 (&xdst)[2][4], int ks_next, WRaw& wdst,
+                       int b_next, auto loadw, const bf16x8_t (&bf)[2][NJ], DqState& st, const WRaw& r,
+                       auto cc, int buf_next) {
     constexpr int t = decltype(tt)::value;
     constexpr int s = t / (4 * NJ), i = (t / NJ) % 4, j = t % NJ;
+    constexpr bool kLoadW = decltype(loadw)::value;
     bf16x8_t afrag;
     __builtin_memcpy(&afrag, &xa[s][i], 16);
     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag, bf[s][j], acc[i][j], 0, 0, 0);
+    if constexpr (t == 1) TTQ_GEMM_TRACE(4 * ks_next + 1);
+    if constexpr (t == 4 * NJ + 1) TTQ_GEMM_TRACE(4 * ks_next + 3);
+    if constexpr (j == 0)
+      xdst[s][i] = *reinterpret_cast<const uint4*>(xptr[i] + ks_next * 64 + 32 * s);
+    if constexpr (kLoadW && j == 3 && (t / NJ) < 5) {
+      constexpr int piece = t / NJ;   // 0: header, 1..4: the thread's 16 bytes of chunk piece-1
+      const uint8_t* p = wptr + 144 * (int64_t)b_next;
+      if constexpr (piece == 0) wdst.hdr = load16_a16(p);
+      else wdst.q[piece - 1] = load16_a16(p + 16 + 32 * (piece - 1) + 16 * whalf);
+    }
     constexpr int p0 = t * kPieces / kMfmas, p1 = (t + 1) * kPieces / kMfmas;
     if constexpr (p1 > p0) dq_piece(st, r, cc, std::integral_constant<int, p0>{}, buf_next);
     if constexpr (p1 > p0 + 1) dq_piece(st, r, cc, std::integral_constant<int, p0 + 1>{}, buf_next);
     __builtin_amdgcn_sched_barrier(0);
   };
-  auto run_slots = [&](auto self, auto tt, const uint4 (&xa)[2][4], const bf16x8_t (&bf)[2][NJ],
-                       DqState& st, const WRaw& r, auto cc, int buf_next) -> void {
+  auto run_slots = [&](auto self, auto tt, const uint4 (&xa)[2][4], uint4 (&xdst)[2][4], int ks_next,
+                       WRaw& wdst, int b_next, auto loadw, const bf16x8_t (&bf)[2][NJ], DqState& st,
+                       const WRaw& r, auto cc, int buf_next) -> void {
     constexpr int t = decltype(tt)::value;
     if constexpr (t < kMfmas) {
-      step_slot(tt, xa, bf, st, r, cc, buf_next);
-      self(self, std::integral_constant<int, t + 1>{}, xa, bf, st, r, cc, buf_next);
+      step_slot(tt, xa, xdst, ks_next, wdst, b_next, loadw, bf, st, r, cc, buf_next);
+      self(self, std::integral_constant<int, t + 1>{}, xa, xdst, ks_next, wdst, b_next, loadw, bf, st, r, cc,
+           buf_next);
     }
   };
   // step: B fragments of both k halves are read from LDS buffer `buf` up front, then the slots
-  auto step = [&](const uint4 (&xa)[2][4], int buf, const WRaw& r, auto cc) {
+  auto step = [&](const uint4 (&xa)[2][4], uint4 (&xdst)[2][4], int ks_next, WRaw& wdst, int b_next,
+                  auto loadw, int buf, const WRaw& r, auto cc) {
     bf16x8_t bf[2][NJ];
 #pragma unroll
     for (int s = 0; s < 2; s++)
@@ -256,7 +287,10 @@ gemm_q4k_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, Y
       }
     DqState st;
     __builtin_amdgcn_sched_barrier(0);
-    run_slots(run_slots, std::integral_constant<int, 0>{}, xa, bf, st, r, cc, buf ^ 1);
+    TTQ_GEMM_TRACE(4 * ks_next + 0);
+    run_slots(run_slots, std::integral_constant<int, 0>{}, xa, xdst, ks_next, wdst, b_next, loadw, bf, st, r,
+              cc, buf ^ 1);
+    TTQ_GEMM_TRACE(4 * ks_next + 2);
   };
 
   // Software pipeline, one super-block (4 steps of 64 k) per outer iteration.  X fragments
@@ -280,27 +314,33 @@ gemm_q4k_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, Y
     const int ks = 4 * b;
     // loads past the end are clamped to the last block / step: harmless re-reads that keep the
     // step bodies straight-line (the chunk dequantized from them in the last step is never read)
-    load_w(wnext, min(b + 1, nblocks - 1));
-    // step 0
-    load_x(xr[3], min(ks + 3, ksteps - 1));
-    if constexpr (WEAVE) step(xr[0], 0, wcur, std::integral_constant<int, 1>{});
-    else { mfma_step(xr[0], 0); dequant_to_lds(wcur, std::integral_constant<int, 1>{}, 1); }
-    __syncthreads();
-    // step 1
-    load_x(xr[0], min(ks + 4, ksteps - 1));
-    if constexpr (WEAVE) step(xr[1], 1, wcur, std::integral_constant<int, 2>{});
-    else { mfma_step(xr[1], 1); dequant_to_lds(wcur, std::integral_constant<int, 2>{}, 0); }
-    __syncthreads();
-    // step 2
-    load_x(xr[1], min(ks + 5, ksteps - 1));
-    if constexpr (WEAVE) step(xr[2], 0, wcur, std::integral_constant<int, 3>{});
-    else { mfma_step(xr[2], 0); dequant_to_lds(wcur, std::integral_constant<int, 3>{}, 1); }
-    __syncthreads();
-    // step 3
-    load_x(xr[2], min(ks + 6, ksteps - 1));
-    if constexpr (WEAVE) step(xr[3], 1, wnext, std::integral_constant<int, 0>{});
-    else { mfma_step(xr[3], 1); dequant_to_lds(wnext, std::integral_constant<int, 0>{}, 0); }
-    __syncthreads();
+    const int bn = min(b + 1, nblocks - 1);
+    using T = std::true_type;
+    using Fz = std::false_type;
+    if constexpr (WEAVE) {
+      step(xr[0], xr[3], min(ks + 3, ksteps - 1), wnext, bn, T{}, 0, wcur, std::integral_constant<int, 1>{});
+      __syncthreads();
+      step(xr[1], xr[0], min(ks + 4, ksteps - 1), wnext, bn, Fz{}, 1, wcur, std::integral_constant<int, 2>{});
+      __syncthreads();
+      step(xr[2], xr[1], min(ks + 5, ksteps - 1), wnext, bn, Fz{}, 0, wcur, std::integral_constant<int, 3>{});
+      __syncthreads();
+      step(xr[3], xr[2], min(ks + 6, ksteps - 1), wnext, bn, Fz{}, 1, wnext, std::integral_constant<int, 0>{});
+      __syncthreads();
+    } else {
+      load_w(wnext, bn);
+      load_x(xr[3], min(ks + 3, ksteps - 1));
+      mfma_step(xr[0], 0); dequant_to_lds(wcur, std::integral_constant<int, 1>{}, 1);
+      __syncthreads();
+      load_x(xr[0], min(ks + 4, ksteps - 1));
+      mfma_step(xr[1], 1); dequant_to_lds(wcur, std::integral_constant<int, 2>{}, 0);
+      __syncthreads();
+      load_x(xr[1], min(ks + 5, ksteps - 1));
+      mfma_step(xr[2], 0); dequant_to_lds(wcur, std::integral_constant<int, 3>{}, 1);
+      __syncthreads();
+      load_x(xr[2], min(ks + 6, ksteps - 1));
+      mfma_step(xr[3], 1); dequant_to_lds(wnext, std::integral_constant<int, 0>{}, 0);
+      __syncthreads();
+    }
     wcur = wnext;
   }
 

@@ -93,6 +93,7 @@ __device__ unsigned long long* g_phase_trace = nullptr;
 #endif
 
 constexpr int kFastThreads = 512;
+constexpr int kStageChunk = kFastThreads * 8;   // activations staged per pass of the workgroup
 constexpr int kFastWaves = kFastThreads / kWave;
 constexpr int kBatch = 4;     // rows per pass when activations are re-read from LDS
 constexpr int kRing = 4;      // row buffers per wavefront when activations sit in registers
@@ -222,17 +223,17 @@ gemv_q4k_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
 
   Q4KRaw bufA[XREG ? kRing : 1];
 
-  // stage x as permuted pairs: one 16-byte load (8 activations) per thread and 4096-chunk,
+  // stage x as permuted pairs: one 16-byte load (8 activations) per thread and pass,
   // all chunks requested before the first is consumed
   {
-    constexpr int kMaxChunks = XREG ? 1 : (int)(kMaxGemvIn16 / 4096);
+    constexpr int kMaxChunks = XREG ? 1 : (int)(kMaxGemvIn16 / kStageChunk);
     uint4 xv[kMaxChunks];
 #pragma unroll
     for (int ch = 0; ch < kMaxChunks; ch++) {
       // unconditional loads from a clamped address keep the control flow straight, so the
       // compiler can wait for exactly these loads and not for the weight loads behind them
-      const int k0 = ch * 4096 + 8 * tid;
-      const bool ok = ch < nit && k0 < n_in;
+      const int k0 = ch * kStageChunk + 8 * tid;
+      const bool ok = k0 < n_in;
       const uint4 v = *reinterpret_cast<const uint4*>(xm + (ok ? k0 : 0));
       xv[ch] = ok ? v : make_uint4(0, 0, 0, 0);
     }
@@ -249,9 +250,9 @@ gemv_q4k_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
     }
 #pragma unroll
     for (int ch = 0; ch < kMaxChunks; ch++) {
-      if (ch < nit) {
+      const int k0 = ch * kStageChunk + 8 * tid;
+      if (k0 < nit * 4096) {
         // thread holds x[k0 .. k0+8): unit u, qs dwords i0 = (k0 % 32) / 4 and i0 + 1
-        const int k0 = ch * 4096 + 8 * tid;
         const int u = k0 >> 6, o = k0 & 63;
         const int kbase = (o >> 5) << 1;          // kinds 0/1 for the low half, 2/3 for the high
         const int i0 = (o & 31) >> 2;
