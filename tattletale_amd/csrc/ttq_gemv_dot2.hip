@@ -99,107 +99,231 @@ constexpr int kBatch = 4;     // rows per pass when activations are re-read from
 constexpr int kRing = 4;      // row buffers per wavefront when activations sit in registers
 constexpr int kEarlyRows = 1; // rows requested before the activations are staged
 
-// -------------------------------------------------------------------------------- Q4_K
-// unit u = (super-block u/4, chunk c = u%4): 32 qs bytes; low nibbles -> sub-block 2c,
-// high nibbles -> sub-block 2c+1.  Activation pairs of a unit, register 4i+kind for qs dword
-// i: kind 0 = (x[4i], x[4i+2]), 1 = (x[4i+1], x[4i+3]), 2/3 = the same 32 positions further.
-struct Q4KRaw { uint4 hdr, q0, q1; };
-
-// Per-lane constants.  A lane always decodes chunk c = lane % 4, so the bit positions of its
-// two 6-bit scales and mins inside the 12 packed bytes never change: sub-blocks 0..3 keep
-// the whole field in bytes 0..7, sub-blocks 4..7 keep 4 bits in bytes 8..11 and 2 bits on top
-// of bytes 0..7.  Written as two bit-field extracts (the second with width 0 for the simple
-// case) so that no branch is needed.
-struct Q4KLane {
-  uint32_t off_hdr, off_q;        // byte offsets of the header and the 32 qs bytes in the row
-  bool upper;                     // sub-blocks 4..7
-  uint32_t wl, wh;                // widths of the low and the high part
-  uint32_t sc_lo[2], mn_lo[2], hi[2];  // bit offsets, for sub-blocks 2c and 2c+1
-  __device__ __forceinline__ void init(int u) {
-    const int c = u & 3;
-    off_hdr = 144u * (uint32_t)(u >> 2);
-    off_q = off_hdr + 16u + 32u * (uint32_t)c;
-    upper = c >= 2;
-    wl = upper ? 4u : 6u;
-    wh = upper ? 2u : 0u;
-#pragma unroll
-    for (int h = 0; h < 2; h++) {
-      const uint32_t j = 2u * c + h, jj = j & 3u;
-      sc_lo[h] = 8u * jj;
-      mn_lo[h] = upper ? 8u * jj + 4u : 8u * jj;
-      hi[h] = 8u * jj + 6u;
-    }
-  }
-};
-
-__device__ __forceinline__ void q4k_load(Q4KRaw& r, const uint8_t* row, const Q4KLane& L) {
-  r.hdr = load16_a16(row + L.off_hdr);
-  r.q0 = load16_a16(row + L.off_q);
-  r.q1 = load16_a16(row + L.off_q + 16);
-}
-
-// Dot product of one unit (64 weights) with the lane's activations.  off1/off2 are
-// kOffset * sx1 / sx2.
-template <class Ops>
-__device__ __forceinline__ float q4k_unit_dot(const Q4KRaw& r, const Q4KLane& L, const uint32_t (&xr)[32],
-                                              float sx1, float sx2, float off1, float off2, uint32_t magic) {
-  const uint32_t dw[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
-  constexpr uint32_t M = 0x000F000Fu;
-  float s1a = 0.f, s1b = 0.f, s2a = 0.f, s2b = 0.f;
-#pragma unroll
-  for (int i = 0; i < 8; i++) {
-    const uint32_t q = dw[i];
-    s1a = Ops::dot2(and_or(q, M, magic), xr[4 * i + 0], s1a);
-    s1b = Ops::dot2(and_or(q >> 8, M, magic), xr[4 * i + 1], s1b);
-    s2a = Ops::dot2(and_or(q >> 4, M, magic), xr[4 * i + 2], s2a);
-    s2b = Ops::dot2(and_or(q >> 12, M, magic), xr[4 * i + 3], s2b);
-  }
-  const float q1 = (s1a + s1b) - off1;   // sum q*x over sub-block 2c
-  const float q2 = (s2a + s2b) - off2;   // sub-block 2c+1
-  const float d = f16_bits_to_f32((uint16_t)(r.hdr.x & 0xFFFF));
-  const float dmin = f16_bits_to_f32((uint16_t)(r.hdr.x >> 16));
-  const uint32_t a_sc = L.upper ? r.hdr.w : r.hdr.y;   // bytes 8-11 or 0-3
-  const uint32_t a_mn = L.upper ? r.hdr.w : r.hdr.z;   // bytes 8-11 or 4-7
-  const uint32_t sc1 = __builtin_amdgcn_ubfe(a_sc, L.sc_lo[0], L.wl) | (__builtin_amdgcn_ubfe(r.hdr.y, L.hi[0], L.wh) << 4);
-  const uint32_t sc2 = __builtin_amdgcn_ubfe(a_sc, L.sc_lo[1], L.wl) | (__builtin_amdgcn_ubfe(r.hdr.y, L.hi[1], L.wh) << 4);
-  const uint32_t mn1 = __builtin_amdgcn_ubfe(a_mn, L.mn_lo[0], L.wl) | (__builtin_amdgcn_ubfe(r.hdr.z, L.hi[0], L.wh) << 4);
-  const uint32_t mn2 = __builtin_amdgcn_ubfe(a_mn, L.mn_lo[1], L.wl) | (__builtin_amdgcn_ubfe(r.hdr.z, L.hi[1], L.wh) << 4);
-  const float t1 = (d * (float)sc1) * q1 - (dmin * (float)mn1) * sx1;
-  const float t2 = (d * (float)sc2) * q2 - (dmin * (float)mn2) * sx2;
-  return t1 + t2;
-}
-
 // LDS slot (dword) of activation-pair register `reg` of unit u: [u/64][reg/4][u%64][reg%4]
 __device__ __forceinline__ int xpair_slot(int u, int reg) {
   return ((((u >> 6) * 8 + (reg >> 2)) * 64 + (u & 63)) << 2) + (reg & 3);
 }
 
-template <class Ops>
-__device__ __forceinline__ void load_x_regs(const uint32_t* xs, int it, int lane, uint32_t (&xr)[32],
-                                            float& sx1, float& sx2) {
+// Pairs (x0,x2), (x1,x3), (x4,x6), (x5,x7) of eight consecutive 16-bit activations
+__device__ __forceinline__ void make_pairs(const uint4& v, uint2& p0, uint2& p1) {
+  p0.x = (v.x & 0xFFFFu) | (v.y << 16);
+  p0.y = (v.x >> 16) | (v.y & 0xFFFF0000u);
+  p1.x = (v.z & 0xFFFFu) | (v.w << 16);
+  p1.y = (v.z >> 16) | (v.w & 0xFFFF0000u);
+}
+
+// -------------------------------------------------------------------------------- Q4_K
+// unit u = (super-block u/4, chunk c = u%4): 32 qs bytes; low nibbles -> sub-block 2c,
+// high nibbles -> sub-block 2c+1.  Activation pairs of a unit, register 4i+kind for qs dword
+// i: kind 0 = (x[4i], x[4i+2]), 1 = (x[4i+1], x[4i+3]), 2/3 = the same 32 positions further.
+struct DotQ4K {
+  static constexpr int kSums = 2;
+  static __device__ __forceinline__ int64_t row_bytes(int n_in) { return (int64_t)(n_in >> 8) * 144; }
+  struct Raw { uint4 hdr, q0, q1; };
+
+  // Per-lane constants.  A lane always decodes chunk c = lane % 4, so the bit positions of its
+  // two 6-bit scales and mins inside the 12 packed bytes never change: sub-blocks 0..3 keep
+  // the whole field in bytes 0..7, sub-blocks 4..7 keep 4 bits in bytes 8..11 and 2 bits on top
+  // of bytes 0..7.  Written as two bit-field extracts (the second with width 0 for the simple
+  // case) so that no branch is needed.
+  struct Lane {
+    uint32_t off_hdr, off_q;        // byte offsets of the header and the 32 qs bytes in the row
+    bool upper;                     // sub-blocks 4..7
+    uint32_t wl, wh;                // widths of the low and the high part
+    uint32_t sc_lo[2], mn_lo[2], hi[2];  // bit offsets, for sub-blocks 2c and 2c+1
+    __device__ __forceinline__ void init(int u) {
+      const int c = u & 3;
+      off_hdr = 144u * (uint32_t)(u >> 2);
+      off_q = off_hdr + 16u + 32u * (uint32_t)c;
+      upper = c >= 2;
+      wl = upper ? 4u : 6u;
+      wh = upper ? 2u : 0u;
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const uint32_t j = 2u * c + h, jj = j & 3u;
+        sc_lo[h] = 8u * jj;
+        mn_lo[h] = upper ? 8u * jj + 4u : 8u * jj;
+        hi[h] = 8u * jj + 6u;
+      }
+    }
+  };
+
+  // `keep` is all ones for a real row and zero for a row past the end (every lane then reads
+  // the first bytes of a valid row: one harmless cache line)
+  static __device__ __forceinline__ void fetch(Raw& r, const uint8_t* rp, const Lane& L, uint32_t keep) {
+    r.hdr = load16_a16(rp + (L.off_hdr & keep));
+    r.q0 = load16_a16(rp + (L.off_q & keep));
+    r.q1 = load16_a16(rp + ((L.off_q + 16) & keep));
+  }
+
+  // thread holds x[k0 .. k0+8): unit k0/64, qs dwords i0 = (k0 % 32) / 4 and i0 + 1
+  static __device__ __forceinline__ void stage(uint32_t* xs, int k0, const uint4& v) {
+    const int u = k0 >> 6, o = k0 & 63;
+    const int kbase = (o >> 5) << 1;          // kinds 0/1 for the low half, 2/3 for the high
+    const int i0 = (o & 31) >> 2;
+    uint2 p0, p1;
+    make_pairs(v, p0, p1);
+    *reinterpret_cast<uint2*>(&xs[xpair_slot(u, 4 * i0 + kbase)]) = p0;
+    *reinterpret_cast<uint2*>(&xs[xpair_slot(u, 4 * (i0 + 1) + kbase)]) = p1;
+  }
+
+  template <class Ops>
+  static __device__ __forceinline__ void sums(const uint32_t (&xr)[32], float (&sx)[kSums]) {
+    float a = 0.f, b = 0.f, c = 0.f, d = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      a = Ops::dot2(xr[4 * i + 0], Ops::kOnes, a);
+      b = Ops::dot2(xr[4 * i + 1], Ops::kOnes, b);
+      c = Ops::dot2(xr[4 * i + 2], Ops::kOnes, c);
+      d = Ops::dot2(xr[4 * i + 3], Ops::kOnes, d);
+    }
+    sx[0] = a + b;
+    sx[1] = c + d;
+  }
+
+  // Dot product of one unit (64 weights) with the lane's activations; off = kOffset * sx.
+  template <class Ops>
+  static __device__ __forceinline__ float unit_dot(const Raw& r, const Lane& L, const uint32_t (&xr)[32],
+                                                   const float (&sx)[kSums], const float (&off)[kSums],
+                                                   uint32_t magic) {
+    const uint32_t dw[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+    constexpr uint32_t M = 0x000F000Fu;
+    float s1a = 0.f, s1b = 0.f, s2a = 0.f, s2b = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const uint32_t q = dw[i];
+      s1a = Ops::dot2(and_or(q, M, magic), xr[4 * i + 0], s1a);
+      s1b = Ops::dot2(and_or(q >> 8, M, magic), xr[4 * i + 1], s1b);
+      s2a = Ops::dot2(and_or(q >> 4, M, magic), xr[4 * i + 2], s2a);
+      s2b = Ops::dot2(and_or(q >> 12, M, magic), xr[4 * i + 3], s2b);
+    }
+    const float q1 = (s1a + s1b) - off[0];   // sum q*x over sub-block 2c
+    const float q2 = (s2a + s2b) - off[1];   // sub-block 2c+1
+    const float d = f16_bits_to_f32((uint16_t)(r.hdr.x & 0xFFFF));
+    const float dmin = f16_bits_to_f32((uint16_t)(r.hdr.x >> 16));
+    const uint32_t a_sc = L.upper ? r.hdr.w : r.hdr.y;   // bytes 8-11 or 0-3
+    const uint32_t a_mn = L.upper ? r.hdr.w : r.hdr.z;   // bytes 8-11 or 4-7
+    const uint32_t sc1 = __builtin_amdgcn_ubfe(a_sc, L.sc_lo[0], L.wl) | (__builtin_amdgcn_ubfe(r.hdr.y, L.hi[0], L.wh) << 4);
+    const uint32_t sc2 = __builtin_amdgcn_ubfe(a_sc, L.sc_lo[1], L.wl) | (__builtin_amdgcn_ubfe(r.hdr.y, L.hi[1], L.wh) << 4);
+    const uint32_t mn1 = __builtin_amdgcn_ubfe(a_mn, L.mn_lo[0], L.wl) | (__builtin_amdgcn_ubfe(r.hdr.z, L.hi[0], L.wh) << 4);
+    const uint32_t mn2 = __builtin_amdgcn_ubfe(a_mn, L.mn_lo[1], L.wl) | (__builtin_amdgcn_ubfe(r.hdr.z, L.hi[1], L.wh) << 4);
+    const float t1 = (d * (float)sc1) * q1 - (dmin * (float)mn1) * sx[0];
+    const float t2 = (d * (float)sc2) * q2 - (dmin * (float)mn2) * sx[1];
+    return t1 + t2;
+  }
+};
+
+// -------------------------------------------------------------------------------- Q6_K
+// unit u = 4b + 2h + s of block b: the 64 weights 128h + 32j + 16s + i (j = 0..3, i = 0..15).
+// They come from 16 bytes of ql (low nibbles: j = 0, high: j = 2), the 16 bytes 32 further
+// (j = 1, 3) and 16 bytes of qh (2 bits per j).  Four bytes of each give one dword of four
+// 6-bit values per j; (Q & 0x00FF00FF) | magic and ((Q >> 8) & 0x00FF00FF) | magic turn it into
+// two float pairs.  Register 8j + 2d + parity holds (x[16j+4d+parity], x[16j+4d+parity+2]).
+// The weights are q - 32 and the magic adds 128 (bf16) or 1024 (fp16): the offset removed per j
+// is (kOffset + 32) * sum(x).
+struct DotQ6K {
+  static constexpr int kSums = 4;
+  static __device__ __forceinline__ int64_t row_bytes(int n_in) { return (int64_t)(n_in >> 8) * 210; }
+  struct Raw { uint4 a, b, h; uint2 sc; uint32_t d; };
+  struct Lane {
+    uint32_t off_a, off_h, off_sc, off_d;
+    uint32_t sbit;   // 8*s: bit offset of the lane's first scale byte inside each scale dword
+    __device__ __forceinline__ void init(int u) {
+      const uint32_t blk = 210u * (uint32_t)(u >> 2);
+      const uint32_t h = (u >> 1) & 1, s = u & 1;
+      off_a = blk + 64u * h + 16u * s;
+      off_h = blk + 128u + 32u * h + 16u * s;
+      off_sc = blk + 192u + 8u * h;
+      off_d = blk + 208u;
+      sbit = 8u * s;
+    }
+  };
+  static __device__ __forceinline__ void fetch(Raw& r, const uint8_t* rp, const Lane& L, uint32_t keep) {
+    r.a = load16_a2(rp + (L.off_a & keep));
+    r.b = load16_a2(rp + ((L.off_a + 32) & keep));
+    r.h = load16_a2(rp + (L.off_h & keep));
+    uint2 sc;
+    __builtin_memcpy(&sc, __builtin_assume_aligned(rp + (L.off_sc & keep), 2), 8);
+    r.sc = sc;
+    r.d = load2(rp + (L.off_d & keep));
+  }
+  // thread holds x[k0 .. k0+8): block, half, j, s and the dwords d0 = (k0 % 16) / 4, d0 + 1
+  static __device__ __forceinline__ void stage(uint32_t* xs, int k0, const uint4& v) {
+    const int b = k0 >> 8, r = k0 & 255;
+    const int h = r >> 7, j = (r >> 5) & 3, s = (r >> 4) & 1, d0 = (r & 15) >> 2;
+    const int u = 4 * b + 2 * h + s;
+    uint2 p0, p1;
+    make_pairs(v, p0, p1);
+    *reinterpret_cast<uint4*>(&xs[xpair_slot(u, 8 * j + 2 * d0)]) = make_uint4(p0.x, p0.y, p1.x, p1.y);
+  }
+  template <class Ops>
+  static __device__ __forceinline__ void sums(const uint32_t (&xr)[32], float (&sx)[kSums]) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      float a = 0.f, b = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        a = Ops::dot2(xr[8 * j + 2 * i], Ops::kOnes, a);
+        b = Ops::dot2(xr[8 * j + 2 * i + 1], Ops::kOnes, b);
+      }
+      sx[j] = a + b;
+    }
+  }
+  template <class Ops>
+  static __device__ __forceinline__ float unit_dot(const Raw& r, const Lane& L, const uint32_t (&xr)[32],
+                                                   const float (&sx)[kSums], const float (&off)[kSums],
+                                                   uint32_t magic) {
+    const uint32_t A[4] = {r.a.x, r.a.y, r.a.z, r.a.w};
+    const uint32_t B[4] = {r.b.x, r.b.y, r.b.z, r.b.w};
+    const uint32_t H[4] = {r.h.x, r.h.y, r.h.z, r.h.w};
+    constexpr uint32_t N4 = 0x0F0F0F0Fu, H2 = 0x30303030u, M = 0x00FF00FFu;
+    float acc[4][2];
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[j][0] = acc[j][1] = 0.f;
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+      uint32_t Q[4];
+      Q[0] = (A[d] & N4) | ((H[d] << 4) & H2);
+      Q[1] = (B[d] & N4) | ((H[d] << 2) & H2);
+      Q[2] = ((A[d] >> 4) & N4) | (H[d] & H2);
+      Q[3] = ((B[d] >> 4) & N4) | ((H[d] >> 2) & H2);
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        acc[j][0] = Ops::dot2(and_or(Q[j], M, magic), xr[8 * j + 2 * d], acc[j][0]);
+        acc[j][1] = Ops::dot2(and_or(Q[j] >> 8, M, magic), xr[8 * j + 2 * d + 1], acc[j][1]);
+      }
+    }
+    const float dd = f16_bits_to_f32((uint16_t)r.d);
+    // scale bytes s, s+2 of the low dword (j = 0, 1) and of the high dword (j = 2, 3)
+    const float c0 = (float)(int)__builtin_amdgcn_sbfe((int)r.sc.x, L.sbit, 8);
+    const float c1 = (float)(int)__builtin_amdgcn_sbfe((int)r.sc.x, L.sbit + 16, 8);
+    const float c2 = (float)(int)__builtin_amdgcn_sbfe((int)r.sc.y, L.sbit, 8);
+    const float c3 = (float)(int)__builtin_amdgcn_sbfe((int)r.sc.y, L.sbit + 16, 8);
+    const float t0 = (dd * c0) * ((acc[0][0] + acc[0][1]) - off[0]);
+    const float t1 = (dd * c1) * ((acc[1][0] + acc[1][1]) - off[1]);
+    const float t2 = (dd * c2) * ((acc[2][0] + acc[2][1]) - off[2]);
+    const float t3 = (dd * c3) * ((acc[3][0] + acc[3][1]) - off[3]);
+    return (t0 + t1) + (t2 + t3);
+  }
+  static constexpr float kExtraOffset = 32.f;
+};
+
+template <class F> struct ExtraOffset { static constexpr float value = 0.f; };
+template <> struct ExtraOffset<DotQ6K> { static constexpr float value = 32.f; };
+
+__device__ __forceinline__ void load_x_regs(const uint32_t* xs, int it, int lane, uint32_t (&xr)[32]) {
   const uint4* xs4 = reinterpret_cast<const uint4*>(xs);
 #pragma unroll
   for (int r = 0; r < 8; r++) {
     const uint4 v = xs4[(it * 8 + r) * 64 + lane];
     xr[4 * r] = v.x; xr[4 * r + 1] = v.y; xr[4 * r + 2] = v.z; xr[4 * r + 3] = v.w;
   }
-  float a = 0.f, b = 0.f, c = 0.f, d = 0.f;
-#pragma unroll
-  for (int i = 0; i < 8; i++) {
-    a = Ops::dot2(xr[4 * i + 0], Ops::kOnes, a);
-    b = Ops::dot2(xr[4 * i + 1], Ops::kOnes, b);
-    c = Ops::dot2(xr[4 * i + 2], Ops::kOnes, c);
-    d = Ops::dot2(xr[4 * i + 3], Ops::kOnes, d);
-  }
-  sx1 = a + b;
-  sx2 = c + d;
 }
 
-template <class Ops, typename YT, bool XREG>
+template <class F, class Ops, typename YT, bool XREG>
 __global__ void __launch_bounds__(kFastThreads)
-gemv_q4k_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
-                     const void* __restrict__ bias, int bias_dtype, int n_out, int n_in,
-                     int rows_per_wave) {
+gemv_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
+                 const void* __restrict__ bias, int bias_dtype, int n_out, int n_in, int rows_per_wave) {
   extern __shared__ uint32_t xs[];
   const int tid = threadIdx.x, lane = tid & 63;
   // the wave index is the same in all 64 lanes: keep it (and every row address) scalar
@@ -208,7 +332,7 @@ gemv_q4k_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
   YT* ym = y + (int64_t)blockIdx.y * n_out;
   const int units = n_in >> 6;
   const int nit = (units + 63) >> 6;
-  const int64_t rb = (int64_t)(n_in >> 8) * 144;
+  const int64_t rb = F::row_bytes(n_in);
 
   const int gw = blockIdx.x * kFastWaves + wave;
   TTQ_TRACE_POINT(gw, 0);
@@ -218,13 +342,13 @@ gemv_q4k_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
 
   // lanes beyond the last unit of a short row read unit 0 and are given zero activations
   const bool active = lane < units;
-  Q4KLane L;
+  typename F::Lane L;
   L.init(active ? lane : 0);
 
-  Q4KRaw bufA[XREG ? kRing : 1];
+  typename F::Raw ring[XREG ? kRing : 1];
 
   // stage x as permuted pairs: one 16-byte load (8 activations) per thread and pass,
-  // all chunks requested before the first is consumed
+  // all passes requested before the first is consumed
   {
     constexpr int kMaxChunks = XREG ? 1 : (int)(kMaxGemvIn16 / kStageChunk);
     uint4 xv[kMaxChunks];
@@ -238,7 +362,7 @@ gemv_q4k_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
       xv[ch] = ok ? v : make_uint4(0, 0, 0, 0);
     }
     // XREG: request the first kEarlyRows rows right behind the activations and the rest of the
-    // batch only once x is staged.  Under a full-rate weight stream every request waits in
+    // ring only once x is staged.  Under a full-rate weight stream every request waits in
     // queues as deep as the bytes already asked for, so x must not be asked for behind a
     // whole batch; a bare s_barrier (no memory wait) also makes sure every wavefront's x request
     // is queued before any weight request of this workgroup.  The weight loads are
@@ -246,25 +370,12 @@ gemv_q4k_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
     if constexpr (XREG) {
       __builtin_amdgcn_s_barrier();
 #pragma unroll
-      for (int r = 0; r < kEarlyRows; r++) q4k_load(bufA[r], w + rb * min(row0 + r, last), L);
+      for (int r = 0; r < kEarlyRows; r++) F::fetch(ring[r], w + rb * min(row0 + r, last), L, 0xFFFFFFFFu);
     }
 #pragma unroll
     for (int ch = 0; ch < kMaxChunks; ch++) {
       const int k0 = ch * kStageChunk + 8 * tid;
-      if (k0 < nit * 4096) {
-        // thread holds x[k0 .. k0+8): unit u, qs dwords i0 = (k0 % 32) / 4 and i0 + 1
-        const int u = k0 >> 6, o = k0 & 63;
-        const int kbase = (o >> 5) << 1;          // kinds 0/1 for the low half, 2/3 for the high
-        const int i0 = (o & 31) >> 2;
-        const uint4 v = xv[ch];
-        uint2 p0, p1;
-        p0.x = (v.x & 0xFFFFu) | (v.y << 16);      // (x0, x2)
-        p0.y = (v.x >> 16) | (v.y & 0xFFFF0000u);  // (x1, x3)
-        p1.x = (v.z & 0xFFFFu) | (v.w << 16);      // (x4, x6)
-        p1.y = (v.z >> 16) | (v.w & 0xFFFF0000u);  // (x5, x7)
-        *reinterpret_cast<uint2*>(&xs[xpair_slot(u, 4 * i0 + kbase)]) = p0;
-        *reinterpret_cast<uint2*>(&xs[xpair_slot(u, 4 * (i0 + 1) + kbase)]) = p1;
-      }
+      if (k0 < nit * 4096) F::stage(xs, k0, xv[ch]);
     }
   }
   __syncthreads();
@@ -272,6 +383,7 @@ gemv_q4k_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
   // wavefronts without rows fall through: their loads are clamped and their stores masked
 
   const uint32_t magic = opaque_vgpr(Ops::kMagic);
+  constexpr float kOff = Ops::kOffset + ExtraOffset<F>::value;
   auto store_rows = [&](auto& acc, int base) {
     constexpr int kN = (int)(sizeof(acc) / sizeof(float));
 #pragma unroll
@@ -287,9 +399,11 @@ gemv_q4k_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
 
   if constexpr (XREG) {
     uint32_t xr[32];
-    float sx1, sx2;
-    load_x_regs<Ops>(xs, 0, lane, xr, sx1, sx2);
-    const float off1 = Ops::kOffset * sx1, off2 = Ops::kOffset * sx2;
+    float sx[F::kSums], off[F::kSums];
+    load_x_regs(xs, 0, lane, xr);
+    F::template sums<Ops>(xr, sx);
+#pragma unroll
+    for (int i = 0; i < F::kSums; i++) off[i] = kOff * sx[i];
     TTQ_TRACE_POINT(gw, 2);
 
     // Row-granular software pipeline over a ring of kRing row buffers: while row r is unpacked,
@@ -298,23 +412,19 @@ gemv_q4k_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
     // queues so deeply that issuing the requests itself stalls the wavefront for microseconds.
     // Loads are always issued (rows past the end fetch one harmless line) so that the
     // compiler's load counting stays exact; only the arithmetic is skipped.
-    auto fetch = [&](Q4KRaw& dst, int row) {
+    auto fetch = [&](typename F::Raw& dst, int row) {
       const bool valid = row < row_end;
-      const uint8_t* rp = w + rb * (valid ? row : min(row0, last));
-      const uint32_t keep = valid ? 0xFFFFFFFFu : 0u;
-      dst.hdr = load16_a16(rp + (L.off_hdr & keep));
-      dst.q0 = load16_a16(rp + (L.off_q & keep));
-      dst.q1 = load16_a16(rp + ((L.off_q + 16) & keep));
+      F::fetch(dst, w + rb * (valid ? row : min(row0, last)), L, valid ? 0xFFFFFFFFu : 0u);
     };
 #pragma unroll
-    for (int r = kEarlyRows; r < kRing - 1; r++) fetch(bufA[r], row0 + r);
+    for (int r = kEarlyRows; r < kRing - 1; r++) fetch(ring[r], row0 + r);
     for (int base = row0; base < row_end; base += kRing) {
       float acc[kRing];
 #pragma unroll
       for (int i = 0; i < kRing; i++) {
-        fetch(bufA[(i + kRing - 1) % kRing], base + i + kRing - 1);
+        fetch(ring[(i + kRing - 1) % kRing], base + i + kRing - 1);
         acc[i] = 0.f;
-        if (base + i < row_end) acc[i] = q4k_unit_dot<Ops>(bufA[i], L, xr, sx1, sx2, off1, off2, magic);
+        if (base + i < row_end) acc[i] = F::template unit_dot<Ops>(ring[i], L, xr, sx, off, magic);
       }
       store_rows(acc, base);
     }
@@ -327,17 +437,19 @@ gemv_q4k_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
       for (int r = 0; r < kBatch; r++) acc[r] = 0.f;
       for (int it = 0; it < nit; it++) {
         const int u = it * 64 + lane;
-        Q4KLane Lu;
+        typename F::Lane Lu;
         Lu.init(u < units ? u : 0);
-        Q4KRaw buf[kBatch];
+        typename F::Raw buf[kBatch];
 #pragma unroll
-        for (int r = 0; r < kBatch; r++) q4k_load(buf[r], w + rb * min(base + r, last), Lu);
+        for (int r = 0; r < kBatch; r++) F::fetch(buf[r], w + rb * min(base + r, last), Lu, 0xFFFFFFFFu);
         uint32_t xr[32];
-        float sx1, sx2;
-        load_x_regs<Ops>(xs, it, lane, xr, sx1, sx2);
-        const float off1 = Ops::kOffset * sx1, off2 = Ops::kOffset * sx2;
+        float sx[F::kSums], off[F::kSums];
+        load_x_regs(xs, it, lane, xr);
+        F::template sums<Ops>(xr, sx);
 #pragma unroll
-        for (int r = 0; r < kBatch; r++) acc[r] += q4k_unit_dot<Ops>(buf[r], Lu, xr, sx1, sx2, off1, off2, magic);
+        for (int i = 0; i < F::kSums; i++) off[i] = kOff * sx[i];
+#pragma unroll
+        for (int r = 0; r < kBatch; r++) acc[r] += F::template unit_dot<Ops>(buf[r], Lu, xr, sx, off, magic);
       }
       store_rows(acc, base);
     }
@@ -363,8 +475,8 @@ static int env_int(const char* name, int dflt) {
   return e ? atoi(e) : dflt;
 }
 
-template <class Ops, typename YT>
-static hipError_t launch_q4k_t(const void* w, const void* x, void* y, const void* bias, int bias_dtype,
+template <class F, class Ops, typename YT>
+static hipError_t launch_fmt_t(const void* w, const void* x, void* y, const void* bias, int bias_dtype,
                                int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
   static const int wg_per_cu = env_int("TTQ_GEMV_WG_PER_CU", 1);
   const int units = (int)(n_in / 64);
@@ -378,21 +490,21 @@ static hipError_t launch_q4k_t(const void* w, const void* x, void* y, const void
   const uint8_t* wb = static_cast<const uint8_t*>(w);
   const uint16_t* xb = static_cast<const uint16_t*>(x);
   if (nit == 1)
-    hipLaunchKernelGGL((gemv_q4k_dot2_kernel<Ops, YT, true>), grid, block, lds, s, wb, xb,
+    hipLaunchKernelGGL((gemv_dot2_kernel<F, Ops, YT, true>), grid, block, lds, s, wb, xb,
                        static_cast<YT*>(y), bias, bias_dtype, (int)n_out, (int)n_in, rows_per_wave);
   else
-    hipLaunchKernelGGL((gemv_q4k_dot2_kernel<Ops, YT, false>), grid, block, lds, s, wb, xb,
+    hipLaunchKernelGGL((gemv_dot2_kernel<F, Ops, YT, false>), grid, block, lds, s, wb, xb,
                        static_cast<YT*>(y), bias, bias_dtype, (int)n_out, (int)n_in, rows_per_wave);
   return hipGetLastError();
 }
 
-template <class Ops>
-static hipError_t launch_q4k_y(const void* w, const void* x, void* y, int y_dtype, const void* bias,
+template <class F, class Ops>
+static hipError_t launch_fmt_y(const void* w, const void* x, void* y, int y_dtype, const void* bias,
                                int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
   switch (y_dtype) {
-    case kF32: return launch_q4k_t<Ops, float>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
-    case kF16: return launch_q4k_t<Ops, f16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
-    case kBF16: return launch_q4k_t<Ops, bf16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kF32: return launch_fmt_t<F, Ops, float>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kF16: return launch_fmt_t<F, Ops, f16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kBF16: return launch_fmt_t<F, Ops, bf16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
     default: return hipErrorInvalidValue;
   }
 }
@@ -400,15 +512,19 @@ static hipError_t launch_q4k_y(const void* w, const void* x, void* y, int y_dtyp
 bool gemv_dot2_supported(int format, int x_dtype, int64_t n_in) {
   static const int disabled = env_int("TTQ_GEMV_NO_DOT2", 0);
   if (disabled) return false;
-  return format == kQ4_K && (x_dtype == kBF16 || x_dtype == kF16) && n_in <= kMaxGemvIn16;
+  return (format == kQ4_K || format == kQ6_K) && (x_dtype == kBF16 || x_dtype == kF16) && n_in <= kMaxGemvIn16;
 }
 
 hipError_t launch_gemv_dot2(int format, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
                             const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                             hipStream_t s) {
-  if (format != kQ4_K) return hipErrorInvalidValue;
-  if (x_dtype == kBF16) return launch_q4k_y<OpsBF16>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-  if (x_dtype == kF16) return launch_q4k_y<OpsF16>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  if (format == kQ4_K) {
+    if (x_dtype == kBF16) return launch_fmt_y<DotQ4K, OpsBF16>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    if (x_dtype == kF16) return launch_fmt_y<DotQ4K, OpsF16>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  } else if (format == kQ6_K) {
+    if (x_dtype == kBF16) return launch_fmt_y<DotQ6K, OpsBF16>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    if (x_dtype == kF16) return launch_fmt_y<DotQ6K, OpsF16>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  }
   return hipErrorInvalidValue;
 }
 
