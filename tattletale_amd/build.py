@@ -20,6 +20,7 @@ SOURCES = [
     "ttq_dequant.hip",
     "ttq_gemv.hip",
     "ttq_gemv_dot2.hip",
+    "ttq_gemv_mfma.hip",
     "ttq_gemm_q4k.hip",
     "ttq_exl3.hip",
     "ttq_host.cpp",

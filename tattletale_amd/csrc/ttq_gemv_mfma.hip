@@ -1,0 +1,390 @@
+// Decode GEMV for Q4_K weights and 16-bit activations on gfx950 through the int8 matrix cores.
+//
+// Same operator as ttq_gemv.hip (F.linear with a single-token activation,
+// workspace/libtorch/src/abi/neural_nets.nim:64-81).  The packed-dot kernel in
+// ttq_gemv_dot2.hip needs about 2.6 vector-ALU instructions per weight byte and is bound by
+// them; this kernel leaves only the nibble split (3 instructions per 8 weights) on the
+// vector ALU and hands the multiply-adds AND the reduction along the row to
+// v_mfma_i32_16x16x64_i8.
+//
+// Arithmetic.  Per sub-block of 32 activations the kernel picks the power of two 2^E just
+// below the largest |x| and turns every activation into a 15-bit integer
+// v = rint(x * 2^(13-E)), split into two signed bytes v = 256*hi + lo (lo in [-128,127],
+// |hi| <= 64).  sum(q*v) over a sub-block is then an exact integer (< 2^24), and
+//       sum(q*x) = 2^(E-13) * (256 * sum(q*hi) + sum(q*lo))
+// carries only the rounding of x to 14 bits below its sub-block maximum (relative error
+// about 3e-5 of the row product; a unit-vector activation is exact, so the canonical
+// dequantized weight d*sc*q - dmin*m is still reproduced bit for bit).  Scales and mins are
+// applied once per sub-block in fp32, in the canonical order.
+//
+// Matrix shapes.  One MFMA multiplies A (16 x 64, the activations) by B (64 x 16, weights of
+// 16 rows) into C (16 x 16).  The 16 rows of A are (sub-block j, plane t) = (0..7) x (hi, lo)
+// of ONE super-block; a row is zero wherever the 64 k-positions of this MFMA do not belong to
+// its sub-block, so C[2j+t][n] = sum over sub-block j of plane_t(x) * q for weight row n.
+// Four MFMAs (two 64-byte halves of the 128 qs bytes, low and high nibbles) cover a
+// super-block of 16 weight rows; 15/16 of the multiplies are by zero, which costs nothing that
+// matters (the matrix cores are otherwise idle) and buys the per-sub-block separation the
+// block scales need.  Lane (n = lane%16, g = lane/16) loads 16 qs bytes of weight row n,
+// supplies them as B, and receives C rows 4g..4g+3, i.e. both planes of sub-blocks 2g and
+// 2g+1 of its own row, whose scales it decodes from the header it loaded itself: no
+// cross-lane traffic until the row is finished.
+//
+// Work distribution.  One workgroup of 16 wavefronts per CU.  A wavefront owns a group of 16
+// consecutive rows and one of SL interleaved slices of the super-blocks, and walks it one
+// step (16 rows x one super-block, 3 x 16 bytes per lane) at a time.  SL is chosen so that
+// all 16 wavefronts have work even when a workgroup owns few rows.
+#include "ttq_device.h"
+#include "ttq_internal.h"
+
+#include <stdlib.h>
+
+namespace ttq {
+
+typedef int v4i_t __attribute__((ext_vector_type(4)));
+
+constexpr int kMfmaThreads = 1024;
+constexpr int kMfmaWaves = kMfmaThreads / kWave;
+// Steps in flight per wavefront.  One is best: with 16 wavefronts that is 48 KiB requested per
+// CU; asking for more lets the memory system serve the CUs unevenly, and the ones served last
+// unpack their whole share after the stream has ended.
+constexpr int kMfmaRing = 1;
+constexpr int64_t kMaxMfmaIn = 8192;            // activation table: 4 KiB of LDS per super-block
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_quad(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
+}
+
+// Bit positions of the two 6-bit scales and mins a lane needs (sub-blocks 2g and 2g+1) inside
+// the 12 packed bytes: sub-blocks 0..3 keep the whole field in bytes 0..7, sub-blocks 4..7
+// keep 4 bits in bytes 8..11 and 2 bits on top of bytes 0..7.  Two bit-field extracts each,
+// the second with width 0 in the simple case, so no branch is needed.
+struct ScaleBits {
+  bool upper;
+  uint32_t wl, wh;
+  uint32_t sc_lo[2], mn_lo[2], hi[2];
+  __device__ __forceinline__ void init(int g) {
+    upper = g >= 2;
+    wl = upper ? 4u : 6u;
+    wh = upper ? 2u : 0u;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      const uint32_t jj = (2u * g + h) & 3u;
+      sc_lo[h] = 8u * jj;
+      mn_lo[h] = upper ? 8u * jj + 4u : 8u * jj;
+      hi[h] = 8u * jj + 6u;
+    }
+  }
+};
+
+struct StepRaw { uint4 hdr, c0, c1; };
+
+template <typename XT> __device__ __forceinline__ void widen8(const uint4& v, float (&f)[8]);
+template <> __device__ __forceinline__ void widen8<bf16_tag>(const uint4& v, float (&f)[8]) {
+  const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    f[2 * i] = __uint_as_float(d[i] << 16);
+    f[2 * i + 1] = __uint_as_float(d[i] & 0xFFFF0000u);
+  }
+}
+template <> __device__ __forceinline__ void widen8<f16_tag>(const uint4& v, float (&f)[8]) {
+  const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    f[2 * i] = f16_bits_to_f32((uint16_t)(d[i] & 0xFFFFu));
+    f[2 * i + 1] = f16_bits_to_f32((uint16_t)(d[i] >> 16));
+  }
+}
+
+// bytes 0 of a, b, c, d -> one dword (a lowest)
+__device__ __forceinline__ uint32_t pack_low_bytes(int a, int b, int c, int d) {
+  const uint32_t p01 = __builtin_amdgcn_perm((uint32_t)b, (uint32_t)a, 0x0c0c0400u);
+  const uint32_t p23 = __builtin_amdgcn_perm((uint32_t)d, (uint32_t)c, 0x0c0c0400u);
+  return p01 | (p23 << 16);
+}
+
+// LDS layout (bytes): plane table [nsb][4 MFMAs][64 lanes] x 16, then the per-sub-block
+// constants [nsb][4] x float4 {2^(E-13) of sub-blocks 2g, 2g+1, sum(x) of 2g, 2g+1}, then
+// the partial row sums of the wavefronts [W][16] floats.
+//
+// W wavefronts per workgroup, R steps in flight per wavefront.
+template <int W, int R, typename XT, typename YT>
+__global__ void __launch_bounds__(W * 64)
+gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
+                     const void* __restrict__ bias, int bias_dtype, int n_out, int nsb, int rows_per_wg,
+                     int sl_log2) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  v4i_t* xa = reinterpret_cast<v4i_t*>(smem);
+  float* tab = reinterpret_cast<float*>(smem + (size_t)nsb * 4096);
+  float* part = reinterpret_cast<float*>(smem + (size_t)nsb * 4096 + (size_t)nsb * 64);
+
+  constexpr int kThreads = W * 64;
+  constexpr int XP = (int)(kMaxMfmaIn / (8 * kThreads));   // staging passes
+  const int SL = 1 << sl_log2;          // slices of the super-blocks
+  const int G = W >> sl_log2;           // row groups per round
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int gi = wave >> sl_log2, sl = wave & (SL - 1);
+  const int n = lane & 15, g = lane >> 4;
+  const int n_in = nsb * 256;
+  const uint16_t* xm = x + (int64_t)blockIdx.y * n_in;
+  YT* ym = y + (int64_t)blockIdx.y * n_out;
+  const uint32_t rb = (uint32_t)nsb * 144u;
+  const int S = (nsb + SL - 1) >> sl_log2;
+  const int wg_row0 = blockIdx.x * rows_per_wg;
+  const int wg_row_end = min(wg_row0 + rows_per_wg, n_out);
+  const int rounds = (rows_per_wg + 16 * G - 1) / (16 * G);
+  const int t_total = rounds * S;
+  const int last = wg_row_end - 1;   // rows past the workgroup's share re-read its last row
+
+  // ---- activations: 16-byte loads (8 values) per thread, requested before any weights
+  uint4 xraw[XP];
+#pragma unroll
+  for (int p = 0; p < XP; p++) {
+    const int k0 = 8 * (tid + p * kThreads);
+    xraw[p] = *reinterpret_cast<const uint4*>(xm + (k0 < n_in ? k0 : 0));
+  }
+  // every wavefront's x request is queued before any weight request of this workgroup
+  __builtin_amdgcn_s_barrier();
+
+  // ---- weight stream: step t = (round r, slice step si); loads are unconditional (clamped)
+  StepRaw ring[R];
+  int ir = 0, isi = 0;                  // round and step-in-round of the next request
+  auto issue = [&](StepRaw& dst) {
+    const int sb = (isi << sl_log2) + sl;
+    const bool ok = ir < rounds && sb < nsb;
+    const int row = min(wg_row0 + (ir * G + gi) * 16 + n, last);
+    const uint32_t o_hdr = ok ? (uint32_t)row * rb + (uint32_t)sb * 144u : 0u;
+    const uint32_t o_q = o_hdr + 16u + 16u * (uint32_t)g;
+    dst.hdr = load16_a16(w + o_hdr);
+    dst.c0 = load16_a16(w + o_q);
+    dst.c1 = load16_a16(w + (o_q + 64u));
+    if (++isi == S) { isi = 0; ir++; }
+  };
+#pragma unroll
+  for (int i = 0; i < R; i++) issue(ring[i]);
+
+  // ---- zero the plane-table entries that stay zero.  Entry (b, q, la): la = 16*ga + m,
+  // m = 2j + t.  MFMA q = 2P + nib covers, in k-group ga, sub-block 4P + 2(ga/2) + nib.
+  {
+    const int la = tid & 63, q = (tid >> 6) & 3;
+    const int j = (la & 15) >> 1, ga = la >> 4;
+    const bool nonzero = (q == 2 * (j >> 2) + (j & 1)) && ((ga >> 1) == ((j & 3) >> 1));
+    if (!nonzero) {
+      const v4i_t z = {0, 0, 0, 0};
+      for (int b = tid >> 8; b < nsb; b += W / 4) xa[(b * 4 + q) * 64 + la] = z;
+    }
+  }
+
+  // ---- quantize the activations into the two byte planes
+#pragma unroll
+  for (int p = 0; p < XP; p++) {
+    const int k0 = 8 * (tid + p * kThreads);
+    if (k0 < n_in) {
+      float xf[8];
+      widen8<XT>(xraw[p], xf);
+      float amax = 0.f, sum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        amax = fmaxf(amax, fabsf(xf[i]));
+        sum += xf[i];
+      }
+      // the four threads of a sub-block are an aligned quad
+      amax = fmaxf(amax, dpp_quad<0xB1>(amax));
+      amax = fmaxf(amax, dpp_quad<0x4E>(amax));
+      sum += dpp_quad<0xB1>(sum);
+      sum += dpp_quad<0x4E>(sum);
+      const uint32_t eb = __float_as_uint(amax) >> 23;      // biased exponent (amax >= 0)
+      const uint32_t ec = eb < 14u ? 14u : eb;
+      const float mul = __uint_as_float((267u - ec) << 23);  // 2^(13-E)
+      // non-finite activations poison the sub-block instead of being clipped
+      const float f = eb == 255u ? __uint_as_float(0x7FC00000u) : __uint_as_float((ec - 13u) << 23);
+      int hi[8], lo[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        const int v = (int)rintf(xf[i] * mul);
+        hi[i] = (v + 128) >> 8;
+        lo[i] = v;                     // only the low byte is used
+      }
+      const int b = k0 >> 8, j = (k0 >> 5) & 7, h = (k0 >> 4) & 1, half8 = (k0 >> 3) & 1;
+      const int q = 2 * (j >> 2) + (j & 1);
+      const int ga = 2 * ((j & 3) >> 1) + h;
+      const int e_hi = ((b * 4 + q) * 64 + 16 * ga + 2 * j) * 2 + half8;   // in 8-byte units
+      uint2* xa8 = reinterpret_cast<uint2*>(smem);
+      xa8[e_hi] = make_uint2(pack_low_bytes(hi[0], hi[1], hi[2], hi[3]), pack_low_bytes(hi[4], hi[5], hi[6], hi[7]));
+      xa8[e_hi + 2] = make_uint2(pack_low_bytes(lo[0], lo[1], lo[2], lo[3]), pack_low_bytes(lo[4], lo[5], lo[6], lo[7]));
+      if ((tid & 3) == 0) {
+        float* e = tab + (b * 4 + (j >> 1)) * 4 + (j & 1);
+        e[0] = f;
+        e[2] = sum;
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- main loop
+  ScaleBits B;
+  B.init(g);
+  constexpr uint32_t N4 = 0x0F0F0F0Fu;
+  int cr = 0, csi = 0;                  // round and step-in-round being consumed
+  float acc = 0.f;
+
+  auto consume = [&](const StepRaw& s) {
+    const int sb = (csi << sl_log2) + sl;
+    if (cr < rounds && sb < nsb) {
+      const v4i_t* xe = xa + (size_t)sb * 256 + lane;
+      const v4i_t a0 = xe[0], a1 = xe[64], a2 = xe[128], a3 = xe[192];
+      const float4 cst = *reinterpret_cast<const float4*>(tab + (sb * 4 + g) * 4);
+      v4i_t L0, H0, L1, H1;
+      L0[0] = (int)(s.c0.x & N4); H0[0] = (int)((s.c0.x >> 4) & N4);
+      L0[1] = (int)(s.c0.y & N4); H0[1] = (int)((s.c0.y >> 4) & N4);
+      L0[2] = (int)(s.c0.z & N4); H0[2] = (int)((s.c0.z >> 4) & N4);
+      L0[3] = (int)(s.c0.w & N4); H0[3] = (int)((s.c0.w >> 4) & N4);
+      L1[0] = (int)(s.c1.x & N4); H1[0] = (int)((s.c1.x >> 4) & N4);
+      L1[1] = (int)(s.c1.y & N4); H1[1] = (int)((s.c1.y >> 4) & N4);
+      L1[2] = (int)(s.c1.z & N4); H1[2] = (int)((s.c1.z >> 4) & N4);
+      L1[3] = (int)(s.c1.w & N4); H1[3] = (int)((s.c1.w >> 4) & N4);
+      // two independent chains; their non-zero rows are disjoint (sub-blocks 0-3 and 4-7)
+      const v4i_t zero = {0, 0, 0, 0};
+      v4i_t Ca = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, L0, zero, 0, 0, 0);
+      v4i_t Cb = __builtin_amdgcn_mfma_i32_16x16x64_i8(a2, L1, zero, 0, 0, 0);
+      Ca = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, H0, Ca, 0, 0, 0);
+      Cb = __builtin_amdgcn_mfma_i32_16x16x64_i8(a3, H1, Cb, 0, 0, 0);
+      const v4i_t C = Ca + Cb;
+
+      const float d = f16_bits_to_f32((uint16_t)(s.hdr.x & 0xFFFFu));
+      const float dmin = f16_bits_to_f32((uint16_t)(s.hdr.x >> 16));
+      const uint32_t a_sc = B.upper ? s.hdr.w : s.hdr.y;   // bytes 8-11 or 0-3
+      const uint32_t a_mn = B.upper ? s.hdr.w : s.hdr.z;   // bytes 8-11 or 4-7
+      const uint32_t sc1 = __builtin_amdgcn_ubfe(a_sc, B.sc_lo[0], B.wl) | (__builtin_amdgcn_ubfe(s.hdr.y, B.hi[0], B.wh) << 4);
+      const uint32_t sc2 = __builtin_amdgcn_ubfe(a_sc, B.sc_lo[1], B.wl) | (__builtin_amdgcn_ubfe(s.hdr.y, B.hi[1], B.wh) << 4);
+      const uint32_t mn1 = __builtin_amdgcn_ubfe(a_mn, B.mn_lo[0], B.wl) | (__builtin_amdgcn_ubfe(s.hdr.z, B.hi[0], B.wh) << 4);
+      const uint32_t mn2 = __builtin_amdgcn_ubfe(a_mn, B.mn_lo[1], B.wl) | (__builtin_amdgcn_ubfe(s.hdr.z, B.hi[1], B.wh) << 4);
+      // exact integers below 2^24, scaled by a power of two: sum(q*x) of the sub-block
+      const float q1 = (float)(C[0] * 256 + C[1]) * cst.x;
+      const float q2 = (float)(C[2] * 256 + C[3]) * cst.y;
+      acc = acc + (d * (float)sc1) * q1;
+      acc = acc - (dmin * (float)mn1) * cst.z;
+      acc = acc + (d * (float)sc2) * q2;
+      acc = acc - (dmin * (float)mn2) * cst.w;
+    }
+    if (++csi == S) {
+      // the row group is finished for this wavefront's slice: add the four k-groups
+      float v = acc;
+      v += __shfl_xor(v, 16, kWave);
+      v += __shfl_xor(v, 32, kWave);
+      if (cr < rounds) {
+        if (sl_log2 == 0) {
+          const int row = wg_row0 + (cr * G + gi) * 16 + n;
+          if (lane < 16 && row < wg_row_end) YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
+        } else {
+          if (lane < 16) part[wave * 16 + n] = v;
+        }
+      }
+      acc = 0.f;
+      csi = 0;
+      cr++;
+    }
+  };
+
+  // steady state: every consumed slot is re-requested R steps ahead; the last R steps drain
+  for (int t0 = R; t0 < t_total; t0 += R) {
+#pragma unroll
+    for (int i = 0; i < R; i++) {
+      consume(ring[i]);
+      issue(ring[i]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < R; i++) consume(ring[i]);
+
+  if (sl_log2 != 0) {
+    // one round only: add the slices in a fixed order
+    __syncthreads();
+    if (tid < 16 * G) {
+      const int grp = tid >> 4, nn = tid & 15;
+      float v = 0.f;
+      for (int s2 = 0; s2 < SL; s2++) v += part[(grp * SL + s2) * 16 + nn];
+      const int row = wg_row0 + grp * 16 + nn;
+      if (row < wg_row_end) YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------ launch
+static int mfma_num_cus() {
+  static int cached = 0;
+  if (cached == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      cached = prop.multiProcessorCount;
+    else
+      cached = 256;
+  }
+  return cached;
+}
+
+static int mfma_env_int(const char* name, int dflt) {
+  const char* e = getenv(name);
+  return e ? atoi(e) : dflt;
+}
+
+template <typename XT, typename YT>
+static hipError_t launch_xy(const void* w, const void* x, void* y, const void* bias, int bias_dtype,
+                            int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+  constexpr int W = kMfmaWaves;
+  const int nsb = (int)(n_in / 256);
+  int num_wg = mfma_num_cus();
+  const int64_t groups = (n_out + 15) / 16;
+  if (num_wg > groups) num_wg = (int)groups;
+  const int rows_per_wg = (int)((n_out + num_wg - 1) / num_wg);
+  num_wg = (int)((n_out + rows_per_wg - 1) / rows_per_wg);
+  // the most slices that still leave room for all the workgroup's rows in one round
+  int sl_log2 = 0;
+  while ((2 << sl_log2) <= W && (2 << sl_log2) <= nsb && (16 * W >> (sl_log2 + 1)) >= rows_per_wg) sl_log2++;
+  const size_t lds = (size_t)nsb * 4096 + (size_t)nsb * 64 + 1024;
+  auto kernel = gemv_q4k_mfma_kernel<W, kMfmaRing, XT, YT>;
+  static bool configured = false;
+  if (!configured) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
+  const dim3 grid((unsigned)num_wg, (unsigned)m), block(W * 64);
+  hipLaunchKernelGGL(kernel, grid, block, lds, s, static_cast<const uint8_t*>(w),
+                     static_cast<const uint16_t*>(x), static_cast<YT*>(y), bias, bias_dtype, (int)n_out, nsb,
+                     rows_per_wg, sl_log2);
+  return hipGetLastError();
+}
+
+template <typename XT>
+static hipError_t launch_x(const void* w, const void* x, void* y, int y_dtype, const void* bias, int bias_dtype,
+                           int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+  switch (y_dtype) {
+    case kF32: return launch_xy<XT, float>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kF16: return launch_xy<XT, f16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kBF16: return launch_xy<XT, bf16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+bool gemv_mfma_supported(int format, int x_dtype, int64_t n_out, int64_t n_in) {
+  static const int disabled = mfma_env_int("TTQ_GEMV_NO_MFMA", 0);
+  if (disabled) return false;
+  // byte offsets into the weight buffer are 32-bit in the kernel; with fewer than eight rows per
+  // CU the per-workgroup activation set-up outweighs the saving
+  return n_out >= 2048 && format == kQ4_K && (x_dtype == kBF16 || x_dtype == kF16) && n_in % 256 == 0 && n_in <= kMaxMfmaIn &&
+         n_out * (n_in / 256) * 144 < ((int64_t)1 << 32);
+}
+
+hipError_t launch_gemv_mfma(const void* w, const void* x, int x_dtype, void* y, int y_dtype, const void* bias,
+                            int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+  if (x_dtype == kBF16) return launch_x<bf16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  if (x_dtype == kF16) return launch_x<f16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  return hipErrorInvalidValue;
+}
+
+}  // namespace ttq

@@ -30,6 +30,12 @@ hipError_t launch_gemv_dot2(int format, const void* w, const void* x, int x_dtyp
                             int y_dtype, const void* bias, int bias_dtype, int64_t m, int64_t n_out,
                             int64_t n_in, hipStream_t s);
 
+// int8 matrix-core path for Q4_K and 16-bit activations (ttq_gemv_mfma.hip).
+bool gemv_mfma_supported(int format, int x_dtype, int64_t n_out, int64_t n_in);
+hipError_t launch_gemv_mfma(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                            const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                            hipStream_t s);
+
 hipError_t launch_gemm_q4k(const void* w, const uint16_t* x_bf16, void* y, int y_dtype,
                            const void* bias, int bias_dtype, int64_t m, int64_t n_out,
                            int64_t n_in, hipStream_t s);

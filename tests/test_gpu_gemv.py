@@ -111,6 +111,67 @@ def test_row_concatenation_of_packed_weights_is_a_fused_layer():
     assert np.array_equal(y, np.concatenate([yg, yu]))
 
 
+@pytest.mark.parametrize("xk", ["bf16", "f16"])
+@pytest.mark.parametrize("n_out,n_in", [(70000, 256), (25600, 512), (14336 + 8, 1024), (2500, 8192), (5000, 1280)])
+def test_q4_k_16bit_work_distributions(xk, n_out, n_in):
+    """Shapes that exercise every split of rows and super-blocks over the wavefronts of the
+    matrix-core kernel: several rounds per workgroup, 1/2/4/16 slices, ragged last groups,
+    a super-block count that is not a power of two; two activation rows."""
+    rng = np.random.default_rng(n_out + n_in)
+    p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=n_out)
+    rows = np.unique(np.concatenate([rng.integers(0, n_out, 400), np.arange(n_out - 40, n_out), np.arange(40)]))
+    sub = np.ascontiguousarray(p.reshape(n_out, -1)[rows])
+    what = oracle.dequant(F.Q4_K, sub, rows.size, n_in)
+    x = Q.fill_normal(n_in + 5, 1, 1.0, 2 * n_in).reshape(2, n_in)
+    x[1, ::7] *= 37.0       # uneven magnitudes across sub-blocks
+    xd, xf = x_to_dev(x, xk)
+    y = QL.gemv(F.Q4_K, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()
+    assert np.all(np.isfinite(y))
+    want = oracle.linear_f64(what, xf)
+    for r in range(2):
+        assert rel_l2(y[r][rows], want[r]) <= TOL
+
+
+@pytest.mark.parametrize("xk", ["bf16", "f16"])
+@pytest.mark.parametrize("n_in", [1024, 8192])
+def test_q4_k_unit_vectors_many_rows(xk, n_in):
+    """Bit-exact columns again, with enough rows that the matrix-core kernel is the one that runs."""
+    n_out = 2100
+    p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=11)
+    what = oracle.dequant(F.Q4_K, p, n_out, n_in)
+    cols = [0, 1, 15, 16, 31, 32, 33, 63, 64, 95, 127, 128, 255, 256, 300, n_in - 129, n_in - 33, n_in - 1]
+    x = np.zeros((len(cols), n_in), np.float32)
+    for i, c in enumerate(cols):
+        x[i, c] = 1.0 if i % 2 == 0 else -0.5
+    xd, _ = x_to_dev(x, xk)
+    y = QL.gemv(F.Q4_K, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()
+    for i, c in enumerate(cols):
+        col = what[:, c] * np.float32(1.0 if i % 2 == 0 else -0.5)
+        assert np.array_equal(y[i], col), c
+        nz = col != 0
+        assert np.array_equal(y[i][nz].view(np.uint32), col[nz].view(np.uint32)), c
+
+
+def test_q4_k_16bit_activation_extremes():
+    """Zero activations, one huge value among tiny ones, and non-finite values: the fixed-point
+    planes of the matrix-core kernel must neither overflow nor hide an Inf/NaN."""
+    n_out, n_in = 2048 + 64, 1024
+    p, what = make(F.Q4_K, n_out, n_in, 77)
+    x = np.zeros((4, n_in), np.float32)
+    x[1] = Q.fill_normal(78, 1, 1e-3, n_in)
+    x[1, 100] = 3.0e4
+    x[2] = Q.fill_normal(79, 1, 1.0, n_in)
+    x[2, 5] = np.inf
+    x[3] = Q.fill_normal(80, 1, 1.0, n_in) * 1e-30
+    xd, xf = x_to_dev(x, "bf16")
+    y = QL.gemv(F.Q4_K, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()
+    want = oracle.linear_f64(what, xf[[0, 1, 3]])
+    assert np.array_equal(y[0], np.zeros(n_out, np.float32))
+    assert rel_l2(y[1], want[1]) <= TOL
+    assert not np.any(np.isfinite(y[2]))
+    assert rel_l2(y[3], want[2]) <= TOL
+
+
 def test_gemv_rejects_oversized_rows():
     with pytest.raises(TtqError) as e:
         QL.gemv(F.Q4_K, torch.zeros(144 * 4 * 128, dtype=torch.uint8, device=DEV),
