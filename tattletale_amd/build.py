@@ -22,6 +22,7 @@ SOURCES = [
     "ttq_gemv_dot2.hip",
     "ttq_gemv_mfma.hip",
     "ttq_gemm_q4k.hip",
+    "ttq_gemm_q4k_pc.hip",
     "ttq_exl3.hip",
     "ttq_host.cpp",
 ]

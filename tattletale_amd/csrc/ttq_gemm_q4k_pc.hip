@@ -1,0 +1,358 @@
+// Prefill GEMM for Q4_K weights on gfx950, producer/consumer form:  Y (m, n_out) = X (m, n_in) * W^T.
+//
+// Replaces F.linear(x, weight) for a multi-row bf16 activation
+// (workspace/libtorch/src/abi/neural_nets.nim:64-81; the prefill case of
+//  workspace/transformers/src/layers/attn.nim:154-156).
+//
+// A wavefront issues its instructions in order, so one that loads, dequantizes AND multiplies
+// leaves the matrix pipe idle whenever it is busy with the other two.  Here a workgroup of
+// eight wavefronts (two per SIMD) owns a 256 x BN tile of Y and splits the roles:
+//   consumers (wavefronts 0-3, 64 rows of the tile each): nothing but LDS fragment reads and
+//       v_mfma_f32_16x16x32_bf16.  Their 64 rows x 64 k of X per step come from global memory
+//       straight into a private LDS ring (global_load_lds, no registers, whole 128-byte
+//       lines per row), three steps ahead; the 16-byte chunks of a row are XOR-swizzled on the
+//       way in so that the fragment reads (16 rows x one chunk) hit 16 different banks.
+//   producers (wavefronts 4-7): load the tile's packed super-blocks once per 256 k, dequantize
+//       64 k per step with the canonical arithmetic (d*sc*q - dmin*m; one fused multiply-add
+//       reproduces it exactly because d*sc*q has at most 21 significant bits), round to bf16
+//       nearest-even and write the B fragments to a double-buffered LDS tile.
+// The hardware interleaves the two kinds of wavefront on each SIMD: the vector ALU and memory
+// work of the producers runs in the shadow of the consumers' MFMAs.  One barrier per 64-k step.
+#include "ttq_device.h"
+#include "ttq_internal.h"
+
+#include <stdlib.h>
+#include <type_traits>
+
+namespace ttq {
+
+constexpr int kPcThreads = 768;          // 4 consumers, 4 W producers, 4 X movers
+constexpr int kPcBM = 256;               // rows of X per workgroup (4 consumer wavefronts x 64)
+constexpr int kXStage = 64 * 128;        // bytes: one consumer's 64 rows x 64 k of bf16
+constexpr int kXStages = 4;
+constexpr int kXRingBytes = 4 * kXStages * kXStage;
+
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+// s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8)
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+  asm volatile("" ::: "memory");
+}
+
+// The barrier of this kernel.  __syncthreads() would also wait for every outstanding
+// global_load_lds (they write LDS, so a release fence drains them), which is exactly the
+// prefetch this kernel lives on; all that is needed is that the wavefront's own LDS accesses
+// are done and that the compiler moves no LDS access across.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// 16-byte LDS store the compiler does not see as one.  It cannot tell a store to the W tile
+// from the asynchronous global_load_lds writes into the X ring and would wait for ALL
+// outstanding requests before every visible LDS store; the barrier protocol below already
+// orders the two.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void lds_store16(uint32_t lds_addr, uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+  const u32x4_t v = {a, b, c, d};
+  asm volatile("ds_write_b128 %0, %1" : : "v"(lds_addr), "v"(v) : "memory");
+}
+
+// W tile in LDS: [ksub 2][j NJ][g 4][n 16] units of 16 bytes (8 consecutive k of one column),
+// i.e. exactly the B operand of lane g*16+n for column block j.
+template <int NJ>
+__global__ void __launch_bounds__(kPcThreads)
+gemm_q4k_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, void* __restrict__ yv,
+                   int y_dtype, const void* __restrict__ bias, int bias_dtype, int m, int n_out, int n_in,
+                   int n_tiles, int m_tiles, int xcds_per_mtile) {
+  constexpr int BN = NJ * 16;
+  constexpr int kWUnits = 2 * NJ * 64;
+  // two separate arrays, so that the compiler can tell LDS writes to the W tile from the
+  // asynchronous global_load_lds writes into the X ring (otherwise it drains every outstanding
+  // request before each W write)
+  __shared__ __attribute__((aligned(16))) uint8_t smem[kXRingBytes];
+  __shared__ uint4 sw[2 * kWUnits];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // Tile assignment.  Workgroups are dealt to the 8 XCDs round-robin (XCD = id % 8) and every XCD
+  // has its own L2.  All workgroups of one row tile read the same 256 x n_in slab of X, so when
+  // the row tiles divide the XCDs evenly each XCD is given workgroups of ONE row tile only.
+  int n_tile, m_tile;
+  if (xcds_per_mtile > 0) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    m_tile = xcd / xcds_per_mtile;
+    n_tile = slot * xcds_per_mtile + xcd % xcds_per_mtile;
+  } else {
+    m_tile = blockIdx.x % m_tiles;
+    n_tile = blockIdx.x / m_tiles;
+  }
+  if (n_tile >= n_tiles) return;
+  const int n0 = n_tile * BN;
+  const int ksteps = n_in >> 6;
+  const int nblocks = n_in >> 8;
+
+  // One barrier per 64-k step, numbered s = -1 .. ksteps-1.  Barrier s means: the data of step
+  // s+1 is complete in LDS (W buffer (s+1)%2, X stage (s+1)%3) and every LDS read of step s has
+  // finished.  The consumers pass it in the MIDDLE of step s (between the MFMAs of the two 32-k
+  // halves), the producers after preparing step s+1.
+
+  if (wave >= 8) {
+    // ------------------------------------------------------------------ X mover
+    // Mover p feeds consumer p.  DMA instruction i covers rows 8i .. 8i+7 of the consumer's 64,
+    // lane l the LDS slot (row 8i + l/8, position l%8); the chunk stored there is
+    // position ^ key(row), key = row & 7: eight
+    // consecutive rows then hold a given chunk in eight different 16-byte bank groups.  (One wavefront gets a 16-byte-per-lane request
+    // out every 64 cycles at best, so the 32 requests of a step need four of them.)
+    const int pc = wave - 8;
+    const uint8_t* xb = reinterpret_cast<const uint8_t*>(x);
+    uint8_t* ring = smem + pc * (kXStages * kXStage);
+    uint32_t xoff[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const int rl = 8 * i + (lane >> 3);
+      const int key = rl & 7;
+      const int row = min(m_tile * kPcBM + pc * 64 + rl, m - 1);   // clamped: never stored
+      xoff[i] = (uint32_t)row * (uint32_t)(n_in * 2) + (uint32_t)(((lane & 7) ^ key) * 16);
+    }
+    const int klast = ksteps - 1;
+    auto dma_step = [&](int ks, int stage) {
+      const uint32_t koff = (uint32_t)min(ks, klast) * 128u;   // past the end: a harmless re-read
+#pragma unroll
+      for (int i = 0; i < 8; i++)
+        __builtin_amdgcn_global_load_lds((gptr_t)(xb + (size_t)(xoff[i] + koff)),
+                                         (lptr_t)(ring + stage * kXStage + i * 1024), 16, 0, 0);
+    };
+    // Requests complete in order, so "all but the youngest N have landed" is the only wait there
+    // is.  Iteration s requests step s+3 into the stage that barrier s-1 freed and then makes
+    // sure step s+1 has landed: 16 younger requests (steps s+2, s+3) may stay in flight.
+    dma_step(0, 0);
+    dma_step(1, 1);
+    dma_step(2, 2);
+    wait_vmcnt<16>();
+    lds_barrier();                       // barrier -1
+    int st = 3;
+    for (int s2 = 0; s2 < ksteps; s2++) {
+      dma_step(s2 + 3, st);
+      st = (st + 1) & (kXStages - 1);
+      wait_vmcnt<16>();
+      lds_barrier();                     // barrier s
+    }
+    // outstanding DMA writes target this workgroup's LDS: let them land before the wavefront ends
+    wait_vmcnt<0>();
+    return;
+  }
+
+  if (wave >= 4) {
+    // ------------------------------------------------------------------ W producer
+    const int pt = tid - 256;
+    // thread -> (tile row, 16-byte half of every 32-byte chunk); with BN = 112 the last 32
+    // threads mirror threads 0..31 (same loads, same LDS writes of the same values)
+    const int wt = pt < 2 * BN ? pt : pt - 2 * BN;
+    const int wr = wt % BN, whalf = wt / BN;
+    const int wrow = min(n0 + wr, n_out - 1);           // clamped: rows past the end are never stored
+    const uint8_t* wptr = w + (int64_t)nblocks * 144 * (int64_t)wrow;
+    const int wj = wr >> 4, wn = wr & 15;
+    const uint32_t sw_addr = (uint32_t)(size_t)(lptr_t)(&sw[0]);
+    struct WRaw { uint4 hdr, q[4]; };
+    auto load_w = [&](WRaw& dst, int b) {
+      const uint8_t* p = wptr + 144 * (int64_t)min(b, nblocks - 1);   // past the end: a harmless re-read
+      dst.hdr = load16_a16(p);
+#pragma unroll
+      for (int c = 0; c < 4; c++) dst.q[c] = load16_a16(p + 16 + 32 * c + 16 * whalf);
+    };
+    auto dequant_to_lds = [&](const WRaw& r, auto cc, int buf) {
+      constexpr int c = decltype(cc)::value;
+      const float d = f16_bits_to_f32((uint16_t)(r.hdr.x & 0xFFFF));
+      const float dmin = f16_bits_to_f32((uint16_t)(r.hdr.x >> 16));
+      uint32_t sc1, mn1, sc2, mn2;
+      q4k_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, 2 * c, sc1, mn1);
+      q4k_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, 2 * c + 1, sc2, mn2);
+      const float d1 = d * (float)sc1, nm1 = -(dmin * (float)mn1);
+      const float d2 = d * (float)sc2, nm2 = -(dmin * (float)mn2);
+      const uint32_t qd[4] = {r.q[c].x, r.q[c].y, r.q[c].z, r.q[c].w};
+      uint32_t lo[8], hi[8];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const uint32_t l4 = qd[i] & 0x0F0F0F0Fu, h4 = (qd[i] >> 4) & 0x0F0F0F0Fu;
+        float fl[4], fh[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+          // fused multiply-add == canonical two-step form here (the product is exact)
+          fl[k] = fmaf_(d1, (float)((l4 >> (8 * k)) & 0xFFu), nm1);
+          fh[k] = fmaf_(d2, (float)((h4 >> (8 * k)) & 0xFFu), nm2);
+        }
+        lo[2 * i] = pack_bf16x2(fl[0], fl[1]);
+        lo[2 * i + 1] = pack_bf16x2(fl[2], fl[3]);
+        hi[2 * i] = pack_bf16x2(fh[0], fh[1]);
+        hi[2 * i + 1] = pack_bf16x2(fh[2], fh[3]);
+      }
+      // low nibbles: k = 16*half + e  -> ksub 0, groups 2*half and 2*half+1; high nibbles: ksub 1
+      const uint32_t base = sw_addr + (uint32_t)(buf * kWUnits + (wj * 4 + 2 * whalf) * 16 + wn) * 16u;
+      lds_store16(base, lo[0], lo[1], lo[2], lo[3]);
+      lds_store16(base + 256u, lo[4], lo[5], lo[6], lo[7]);
+      lds_store16(base + NJ * 1024u, hi[0], hi[1], hi[2], hi[3]);
+      lds_store16(base + NJ * 1024u + 256u, hi[4], hi[5], hi[6], hi[7]);
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+    // The packed super-blocks come from HBM (about 2 us away): block b+2 is requested at the
+    // start of block b, into the register set block b-1 used.  Three sets rotate by name, so no
+    // copy ever forces a request to complete early.  These wavefronts issue no other global
+    // loads, so the compiler's own counting of outstanding requests is exact.
+    // Iteration s prepares step s+1: chunks 1..3 of block b, then chunk 0 of block b+1.
+    auto do_block = [&](const WRaw& cur, const WRaw& nxt, WRaw& into, int b) {
+      load_w(into, b + 2);
+      dequant_to_lds(cur, I1{}, 1);
+      lds_barrier();
+      dequant_to_lds(cur, I2{}, 0);
+      lds_barrier();
+      dequant_to_lds(cur, I3{}, 1);
+      lds_barrier();
+      dequant_to_lds(nxt, I0{}, 0);      // the chunk written in the very last iteration is never read
+      lds_barrier();
+    };
+    WRaw wa, wb, wc;
+    load_w(wa, 0);
+    load_w(wb, 1);
+    dequant_to_lds(wa, I0{}, 0);
+    lds_barrier();                       // barrier -1
+    for (int b = 0; b < nblocks; b += 3) {
+      do_block(wa, wb, wc, b);
+      if (b + 1 < nblocks) do_block(wb, wc, wa, b + 1);
+      if (b + 2 < nblocks) do_block(wc, wa, wb, b + 2);
+    }
+    return;
+  }
+
+  // -------------------------------------------------------------------- consumer
+  const int m0 = m_tile * kPcBM + wave * 64;
+  const uint8_t* myx = smem + wave * (kXStages * kXStage);
+  const int fr = lane & 15, fg = lane >> 4;
+  // A fragments: row 16*ib + fr, chunk 4*half + fg, stored at position chunk ^ key(row)
+  const int akey = fr & 7;
+  const int apos[2] = {(fr * 8 + (fg ^ akey)) * 16, (fr * 8 + ((4 + fg) ^ akey)) * 16};
+  // A step is 2*NJ groups of four MFMAs: group g uses the A fragments of half g/NJ (four row
+  // blocks) and the B fragment of column block g%NJ.  B fragments are read two groups ahead
+  // into a ring of four, A fragments half a step ahead, and __builtin_amdgcn_sched_barrier
+  // pins that order: left alone the compiler sinks every read to just before its use and the
+  // wavefront then waits out the LDS latency fourteen times per step.
+  constexpr int G = 2 * NJ;
+  uint4 afr[2][4];                      // A fragments of half 0 / half 1
+  bf16x8_t bring[4];
+  auto read_a = [&](uint4 (&dst)[4], int stage, int half) {
+    const uint8_t* xbase = myx + stage * kXStage + apos[half];
+#pragma unroll
+    for (int ib = 0; ib < 4; ib++) dst[ib] = *reinterpret_cast<const uint4*>(xbase + ib * 2048);
+  };
+  auto read_b = [&](bf16x8_t& dst, int buf, int g) {   // g = half * NJ + j
+    const uint4 v = sw[buf * kWUnits + g * 64 + lane];
+    __builtin_memcpy(&dst, &v, 16);
+  };
+
+  f32x4_t acc[4][NJ];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < NJ; j++) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  // one step; everything that selects a buffer is a compile-time constant, so that every LDS
+  // address is one register plus an immediate.  SO = ring slot of the step's group 0: 2*NJ is
+  // not always a multiple of four, and the first two groups of the next step are read while
+  // the last two of this one still hold their slots.
+  auto step = [&](auto so, auto stage, auto bufc) {
+    constexpr int SO = decltype(so)::value, ST = decltype(stage)::value, BUF = decltype(bufc)::value;
+    constexpr int STN = (ST + 1) & (kXStages - 1);
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+      if (g == G - 2) lds_barrier();     // barrier ks: step ks+1 is in LDS, reads of step ks done
+      if (g + 2 < G) read_b(bring[(g + 2 + SO) & 3], BUF, g + 2);
+      else read_b(bring[(g + 2 + SO) & 3], BUF ^ 1, g + 2 - G);
+      if (g == (NJ > 3 ? NJ - 3 : 0)) read_a(afr[1], ST, 1);
+      if (g == G - 2) read_a(afr[0], STN, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      const int half = g / NJ, j = g % NJ;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        bf16x8_t a;
+        __builtin_memcpy(&a, &afr[half][i], 16);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bring[(g + SO) & 3], acc[i][j], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  lds_barrier();                         // barrier -1: step 0 is in LDS
+  read_a(afr[0], 0, 0);
+  read_b(bring[0], 0, 0);
+  read_b(bring[1], 0, 1);
+  static_assert(kXStages == 4, "the step loop is unrolled over the four X stages");
+  using C0 = std::integral_constant<int, 0>;
+  using C1 = std::integral_constant<int, 1>;
+  using C2 = std::integral_constant<int, 2>;
+  using C3 = std::integral_constant<int, 3>;
+  for (int ks = 0; ks < ksteps; ks += 4) {   // ksteps is a multiple of four
+    step(std::integral_constant<int, 0>{}, C0{}, C0{});
+    step(std::integral_constant<int, (G & 3)>{}, C1{}, C1{});
+    step(std::integral_constant<int, ((2 * G) & 3)>{}, C2{}, C0{});
+    step(std::integral_constant<int, ((3 * G) & 3)>{}, C3{}, C1{});   // after the last step: stale reads, never used
+  }
+
+  // ---- epilogue: lane holds Y[m0 + 16i + 4*(lane/16) + r][n0 + 16j + lane%16], r = 0..3
+  const int cn = lane & 15, rb4 = (lane >> 4) * 4;
+#pragma unroll
+  for (int j = 0; j < NJ; j++) {
+    const int n = n0 + 16 * j + cn;
+    if (n >= n_out) continue;
+    const float bv = load_bias(bias, bias_dtype, n);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int mm = m0 + 16 * i + rb4 + r;
+        if (mm < m) {
+          const float v = acc[i][j][r] + bv;
+          if (y_dtype == kBF16) YElem<bf16_tag>::store(static_cast<bf16_tag*>(yv), (int64_t)mm * n_out + n, v);
+          else YElem<float>::store(static_cast<float*>(yv), (int64_t)mm * n_out + n, v);
+        }
+      }
+    }
+  }
+}
+
+static hipError_t launch_pc_112(const uint8_t* wb, const uint16_t* x, void* y, int y_dtype, const void* bias,
+                                int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+  constexpr int NJ = 7, BN = NJ * 16;
+  const int n_tiles = (int)((n_out + BN - 1) / BN), m_tiles = (int)((m + kPcBM - 1) / kPcBM);
+  int xcds_per_mtile = 0;
+  unsigned nwg = (unsigned)(n_tiles * m_tiles);
+  if (m_tiles >= 2 && m_tiles <= 8 && 8 % m_tiles == 0) {
+    xcds_per_mtile = 8 / m_tiles;
+    nwg = (unsigned)(((n_tiles + xcds_per_mtile - 1) / xcds_per_mtile) * 8);
+  }
+  hipLaunchKernelGGL(gemm_q4k_pc_kernel<NJ>, dim3(nwg), dim3(kPcThreads), 0, s, wb, x, y, y_dtype, bias,
+                     bias_dtype, (int)m, (int)n_out, (int)n_in, n_tiles, m_tiles, xcds_per_mtile);
+  return hipGetLastError();
+}
+
+// Only the 112-column tile is built in this form: with 128 columns the consumers' 128
+// accumulator registers plus the fragment rings do not fit the 168 registers a wavefront gets
+// when twelve of them share a CU.
+bool gemm_q4k_pc_supported(int64_t m, int64_t n_out, int64_t n_in, int bn) {
+  static const int disabled = [] { const char* e = getenv("TTQ_GEMM_NO_PC"); return e ? atoi(e) : 0; }();
+  // activation byte offsets are 32-bit in the kernel
+  return !disabled && bn == 112 && m * n_in * 2 < ((int64_t)1 << 32) && n_out > 0;
+}
+
+hipError_t launch_gemm_q4k_pc(const void* w, const uint16_t* x_bf16, void* y, int y_dtype, const void* bias,
+                              int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+  if (m == 0 || n_out == 0) return hipSuccess;
+  if (y_dtype != kBF16 && y_dtype != kF32) return hipErrorInvalidValue;
+  return launch_pc_112(static_cast<const uint8_t*>(w), x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+}
+
+}  // namespace ttq

@@ -20,8 +20,9 @@ TOL = 2e-2
 
 
 @pytest.mark.parametrize("m,n_out,n_in", [(64, 256, 1024), (128, 128, 256), (16, 384, 512), (100, 200, 768),
-                                          (257, 130, 1024), (512, 512, 4096)])
+                                          (257, 130, 1024), (512, 512, 4096), (300, 16384, 256)])
 def test_gemm_random(m, n_out, n_in):
+    # (300, 16384, 256) is the one shape here for which the 128-column tile is chosen
     w = Q.fill_normal(300 + m, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
     p = Q.quantize(F.Q4_K, w)
     what = oracle.dequant(F.Q4_K, p, n_out, n_in)
