@@ -103,9 +103,9 @@ gemm_q4k_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
     // ------------------------------------------------------------------ X mover
     // Mover p feeds consumer p.  DMA instruction i covers rows 8i .. 8i+7 of the consumer's 64,
     // lane l the LDS slot (row 8i + l/8, position l%8); the chunk stored there is
-    // position ^ key(row), key = row & 7: eight
-    // consecutive rows then hold a given chunk in eight different 16-byte bank groups.  (One wavefront gets a 16-byte-per-lane request
-    // out every 64 cycles at best, so the 32 requests of a step need four of them.)
+    // position ^ key(row), key = row & 7: eight consecutive rows then hold a given chunk in
+    // eight different 16-byte bank groups.  (One wavefront gets a 16-byte-per-lane request out
+    // every 64 cycles at best, so the 32 requests of a step need four of them.)
     const int pc = wave - 8;
     const uint8_t* xb = reinterpret_cast<const uint8_t*>(x);
     uint8_t* ring = smem + pc * (kXStages * kXStage);
@@ -117,9 +117,8 @@ gemm_q4k_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
       const int row = min(m_tile * kPcBM + pc * 64 + rl, m - 1);   // clamped: never stored
       xoff[i] = (uint32_t)row * (uint32_t)(n_in * 2) + (uint32_t)(((lane & 7) ^ key) * 16);
     }
-    const int klast = ksteps - 1;
     auto dma_step = [&](int ks, int stage) {
-      const uint32_t koff = (uint32_t)min(ks, klast) * 128u;   // past the end: a harmless re-read
+      const uint32_t koff = (uint32_t)ks * 128u;
 #pragma unroll
       for (int i = 0; i < 8; i++)
         __builtin_amdgcn_global_load_lds((gptr_t)(xb + (size_t)(xoff[i] + koff)),
@@ -128,20 +127,24 @@ gemm_q4k_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
     // Requests complete in order, so "all but the youngest N have landed" is the only wait there
     // is.  Iteration s requests step s+3 into the stage that barrier s-1 freed and then makes
     // sure step s+1 has landed: 16 younger requests (steps s+2, s+3) may stay in flight.
+    // Nothing is requested past the last step: the consumers reuse their rings in the epilogue.
     dma_step(0, 0);
     dma_step(1, 1);
     dma_step(2, 2);
     wait_vmcnt<16>();
     lds_barrier();                       // barrier -1
     int st = 3;
-    for (int s2 = 0; s2 < ksteps; s2++) {
+    for (int s2 = 0; s2 < ksteps - 3; s2++) {
       dma_step(s2 + 3, st);
       st = (st + 1) & (kXStages - 1);
       wait_vmcnt<16>();
       lds_barrier();                     // barrier s
     }
-    // outstanding DMA writes target this workgroup's LDS: let them land before the wavefront ends
+    wait_vmcnt<8>();
+    lds_barrier();                       // barrier ksteps-3: step ksteps-2 has landed
     wait_vmcnt<0>();
+    lds_barrier();                       // barrier ksteps-2: the last step has landed
+    lds_barrier();                       // barrier ksteps-1
     return;
   }
 
@@ -304,6 +307,34 @@ gemm_q4k_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
 
   // ---- epilogue: lane holds Y[m0 + 16i + 4*(lane/16) + r][n0 + 16j + lane%16], r = 0..3
   const int cn = lane & 15, rb4 = (lane >> 4) * 4;
+  if (y_dtype == kBF16 && n0 + BN <= n_out && (n_out & 7) == 0) {
+    // Full tile of bf16: transpose through the wavefront's own (now idle) X ring, so that global
+    // memory sees 16-byte stores along the rows instead of 2-byte ones.  Row stride 240 bytes.
+    constexpr int kRowBytes = BN * 2 + 16;
+    uint8_t* stg = smem + wave * (kXStages * kXStage);
+#pragma unroll
+    for (int j = 0; j < NJ; j++) {
+      const float bv = load_bias(bias, bias_dtype, n0 + 16 * j + cn);
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+          *reinterpret_cast<uint16_t*>(stg + (16 * i + rb4 + r) * kRowBytes + (16 * j + cn) * 2) =
+              f32_to_bf16_bits(acc[i][j][r] + bv);
+    }
+    // same wavefront wrote and reads: LDS keeps program order, no barrier needed
+    uint8_t* yb = static_cast<uint8_t*>(yv);
+    constexpr int kChunks = BN / 8;      // 16-byte chunks per row
+#pragma unroll
+    for (int t = 0; t < kChunks; t++) {
+      const int c = t * 64 + lane;
+      const int row = c / kChunks, ch = c - row * kChunks;
+      const uint4 v = *reinterpret_cast<const uint4*>(stg + row * kRowBytes + ch * 16);
+      if (m0 + row < m)
+        *reinterpret_cast<uint4*>(yb + ((int64_t)(m0 + row) * n_out + n0 + ch * 8) * 2) = v;
+    }
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < NJ; j++) {
     const int n = n0 + 16 * j + cn;
