@@ -59,6 +59,8 @@ def main() -> int:
     from tattletale_amd import configs as CFG
     from tattletale_amd import formats as F
     from tattletale_amd import qlinear as QL
+    from tattletale_amd import quantize as Q
+    from tattletale_amd import _lib
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -198,6 +200,53 @@ def main() -> int:
         out["aten_dense_bf16_weight_GBps"] = what.numel() * 2 / dt2 / 1e9
         return out
 
+    def run_gate_up(steps: int, warmup: int):
+        """Llama-3-8B FFN decode: the 28672 x 4096 gate/up matrix, silu_and_mul fused into the GEMV
+        (one launch) against the GEMV followed by ttq_silu_and_mul (two launches)."""
+        n_ff, n_in = 14336, 4096
+        cfg = CFG.CONFIGS["q4_k_gemv"]
+        t0 = time.time()
+        w = Q.fill_normal(cfg.seed + 50, 0, 0.02, 2 * n_ff * n_in).reshape(2 * n_ff, n_in)
+        packed = Q.quantize(F.Q4_K, w)
+        del w
+        log("[q4_k_gate_up_silu_gemv] inputs generated in %.1f s" % (time.time() - t0))
+        x = to_dev(CFG.activations(cfg), "bf16")
+        ncopies = max(2, -(-2 * MALL_BYTES // packed.nbytes))
+        ws = [to_dev(packed) for _ in range(ncopies)]
+        y = torch.empty((1, n_ff), dtype=torch.bfloat16, device=dev)
+        gu = torch.empty((1, 2 * n_ff), dtype=torch.float32, device=dev)
+        L = _lib.lib()
+        sp = torch.cuda.current_stream(dev).cuda_stream
+
+        def fused(i):
+            _lib.check(L.ttq_gemv_q4_k_silu_mul(ws[i % ncopies].data_ptr(), x.data_ptr(), F.BF16, y.data_ptr(),
+                                                F.BF16, 1, n_ff, n_in, torch.cuda.current_stream(dev).cuda_stream),
+                       "ttq_gemv_q4_k_silu_mul")
+
+        gu16 = torch.empty((1, 2 * n_ff), dtype=torch.bfloat16, device=dev)
+        st = _lib.QLinearStruct(format=F.Q4_K, n_out=2 * n_ff, n_in=n_in)
+        import ctypes as C
+
+        def unfused(i):
+            cur = torch.cuda.current_stream(dev).cuda_stream
+            st.qweight = ws[i % ncopies].data_ptr()
+            _lib.check(L.ttq_linear_forward(C.byref(st), x.data_ptr(), F.BF16, 1, gu16.data_ptr(), F.BF16, cur),
+                       "ttq_linear_forward")
+            _lib.check(L.ttq_silu_and_mul(gu16.data_ptr(), y.data_ptr(), F.BF16, 1, n_ff, cur), "ttq_silu_and_mul")
+
+        _, f_ms = time_steps(fused, steps, warmup, use_graph=not args.eager)
+        _, u_ms = time_steps(unfused, steps, warmup, use_graph=not args.eager)
+        res = {"name": "q4_k_gate_up_silu_gemv", "steps": steps, "weight_bytes": int(packed.nbytes),
+               "weight_copies": ncopies, "ms_per_step": f_ms, "weight_GBps": packed.nbytes / (f_ms * 1e-3) / 1e9,
+               "hbm_frac": packed.nbytes / (f_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+               "unfused_two_launches_ms_per_step": u_ms}
+        log("[q4_k_gate_up_silu_gemv] fused %.3f us/step (%.0f GB/s), GEMV + silu_and_mul %.3f us/step"
+            % (f_ms * 1e3, res["weight_GBps"], u_ms * 1e3))
+        return res
+
+    if args.only == "q4_k_gate_up_silu_gemv":
+        print(json.dumps(run_gate_up(max(20, args.steps // 4), max(3, args.warmup // 4))), flush=True)
+        return 0
     names = [args.only] if args.only else ["q4_k_gemv"]
     if not args.only and not args.no_extra:
         names += ["q4_k_gemm_m512", "q8_0_gemv", "q6_k_gemv", "exl3_gemv", "q4_k_gemm_m64", "q4_k_gemm_m2048"]
@@ -250,6 +299,8 @@ def main() -> int:
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline()
     line["extra"] = {k: v for k, v in results.items() if k != names[0]}
+    if not args.only and not args.no_extra:
+        line["extra"]["q4_k_gate_up_silu_gemv"] = run_gate_up(max(20, args.steps // 4), max(3, args.warmup // 4))
     print(json.dumps(line), flush=True)
     return 0
 

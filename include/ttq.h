@@ -139,6 +139,19 @@ TTQ_API int ttq_dequant_exl3(const uint16_t* trellis, uint16_t* out_f16, int64_t
 TTQ_API int ttq_hadamard128_f32(float* v, const uint16_t* pre_f16, const uint16_t* post_f16,
                         int64_t n, void* stream);
 
+/* ---- gated MLP: activation and its fusion into the decode GEMV ---------------------- */
+/* out[m][h] = silu(in[m][0:h]) * in[m][h:2h], in and out of the same dtype.  Stands in for
+ * silu_and_mul (workspace/transformers/src/kernels/activations.nim:14-38), applied by
+ * GatedMLP.forward to the output of the fused gate/up projection (mlp.nim:56-60). */
+TTQ_API int ttq_silu_and_mul(const void* in, void* out, int dtype, int64_t m, int64_t h, void* stream);
+/* y[m][n_ff] = silu(x Wg^T) * (x Wu^T) in one kernel, W = [Wg; Wu] the (2*n_ff, n_in) Q4_K
+ * matrix GatedMLP.init builds by row concatenation (mlp.nim:39).  Replaces
+ * gate_up_proj.forward followed by silu_and_mul (mlp.nim:56-59) for decode.  16-bit
+ * activations only; returns TTQ_ERR_UNSUPPORTED for shapes the fused kernel does not cover
+ * (n_in > 8192, n_ff < 16, fp32 activations): call ttq_gemv_q4_k + ttq_silu_and_mul then. */
+TTQ_API int ttq_gemv_q4_k_silu_mul(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                           int64_t m, int64_t n_ff, int64_t n_in, void* stream);
+
 /* ---- host-side preparation (CPU code; no GPU needed) ------------------------------- */
 /* Weight preparation happens once at load time, off the hot path; the reference's
  * counterpart is building the dense weight tensor handed to Linear.init (linear.nim:29-43,

@@ -53,6 +53,8 @@ def lib() -> C.CDLL:
             getattr(L, name).argtypes = [vp, i64, vp]
         L.ora_q4k_unpack_scales.restype = None
         L.ora_q4k_unpack_scales.argtypes = [vp, vp, vp]
+        L.ora_silu_and_mul_f64.restype = None
+        L.ora_silu_and_mul_f64.argtypes = [vp, vp, i64, i64]
         L.ora_linear_f64.restype = None
         L.ora_linear_f64.argtypes = [vp, vp, vp, vp, i64, i64, i64]
         L.ora_gemv_fused.restype = i32
@@ -147,6 +149,18 @@ def linear_f64(w_f32, x_f32, bias_f32=None) -> np.ndarray:
     b = None if bias_f32 is None else _c(bias_f32, np.float32)
     lib().ora_linear_f64(_p(w), _p(x), _p(b) if b is not None else None, _p(y), m, n_out, n_in)
     return y
+
+
+def silu_and_mul_f64(x) -> np.ndarray:
+    """(m, 2h) -> (m, h): silu(x[:, :h]) * x[:, h:] in float64 (activations.nim:14-38)."""
+    a = _c(x, np.float64)
+    if a.ndim == 1:
+        a = a[None, :]
+    m, h2 = a.shape
+    assert h2 % 2 == 0
+    out = np.empty((m, h2 // 2), np.float64)
+    lib().ora_silu_and_mul_f64(_p(a), _p(out), m, h2 // 2)
+    return out
 
 
 def gemv_fused(fmt: int, packed, x_f32, n_out: int, n_in: int, nthreads: int = 0) -> np.ndarray:

@@ -27,6 +27,7 @@
  *   Q8_0/Q4_K/Q6_K        hand-computed known answers, brute-force scale pack/unpack
  *                         round trip, bit-exact agreement with an independent
  *                         vectorised closed-form restatement (oracle/np_oracle.py)
+ *   silu_and_mul          scipy.special.expit, fixed points and asymptotes
  *   FWHT-128              scipy.linalg.hadamard, involution, norm preservation
  *   trellis decode        brute force on one tile via python big-int bit arithmetic
  *   codebooks             closed-form numpy restatement over all 65536 states
@@ -226,6 +227,18 @@ ORA_API void ora_linear_f64(const float* w, const float* x, const float* bias, d
       y[i * n_out + n] = acc;
     }
   }
+}
+
+/* silu_and_mul: out[i][c] = silu(in[i][c]) * in[i][h + c], silu(g) = g / (1 + exp(-g)), in
+ * float64.  Follows workspace/transformers/src/kernels/activations.nim:14-38
+ * (x.chunk(2, -1); silu(chunks[0]) * chunks[1]).  Pinned by scipy.special.expit
+ * (silu(g) = g * expit(g)), silu(0) = 0, the asymptotes and the minimum near -1.2785.     */
+ORA_API void ora_silu_and_mul_f64(const double* in, double* out, int64_t m, int64_t h) {
+  for (int64_t i = 0; i < m; i++)
+    for (int64_t c = 0; c < h; c++) {
+      const double g = in[i * 2 * h + c], u = in[i * 2 * h + h + c];
+      out[i * h + c] = g / (1.0 + exp(-g)) * u;
+    }
 }
 
 /* Same product for a chosen subset of output rows (full-size spot checks). */

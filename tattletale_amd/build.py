@@ -24,6 +24,7 @@ SOURCES = [
     "ttq_gemm_q4k.hip",
     "ttq_gemm_q4k_pc.hip",
     "ttq_exl3.hip",
+    "ttq_activations.hip",
     "ttq_host.cpp",
 ]
 

@@ -1,0 +1,77 @@
+// silu_and_mul on the GPU: out[..., :h] = silu(in[..., :h]) * in[..., h:2h].
+//
+// Stand-in for workspace/transformers/src/kernels/activations.nim:14-38, which GatedMLP
+// applies to the output of the fused gate/up projection
+// (workspace/transformers/src/layers/mlp.nim:56-60).  The arithmetic is fp32 with one
+// rounding to the output type (the reference rounds silu(gate) to the tensor type first).
+// Memory-bound elementwise work: 16-byte loads and stores when the width allows.
+#include "ttq_device.h"
+#include "ttq_internal.h"
+
+namespace ttq {
+
+__device__ __forceinline__ float silu_mul(float g, float u) { return (g / (1.f + expf(-g))) * u; }
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+silu_and_mul_kernel(const T* __restrict__ in, T* __restrict__ out, int64_t m, int64_t h) {
+  const int64_t total = m * h;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / h, c = i - r * h;
+    const float g = XElem<T>::load(in, r * 2 * h + c), u = XElem<T>::load(in, r * 2 * h + h + c);
+    YElem<T>::store(out, i, silu_mul(g, u));
+  }
+}
+
+// eight 16-bit elements per thread; h must be a multiple of 8 and the rows 16-byte aligned
+template <bool BF16>
+__global__ void __launch_bounds__(256)
+silu_and_mul16_kernel(const uint16_t* __restrict__ in, uint16_t* __restrict__ out, int64_t m, int64_t h8) {
+  const int64_t total = m * h8;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / h8, c = i - r * h8;
+    const uint4 gv = *reinterpret_cast<const uint4*>(in + (r * 2 * h8 + c) * 8);
+    const uint4 uv = *reinterpret_cast<const uint4*>(in + (r * 2 * h8 + h8 + c) * 8);
+    const uint32_t gd[4] = {gv.x, gv.y, gv.z, gv.w}, ud[4] = {uv.x, uv.y, uv.z, uv.w};
+    uint32_t od[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      float g0, g1, u0, u1;
+      if (BF16) {
+        g0 = bf16_bits_to_f32((uint16_t)gd[k]); g1 = bf16_bits_to_f32((uint16_t)(gd[k] >> 16));
+        u0 = bf16_bits_to_f32((uint16_t)ud[k]); u1 = bf16_bits_to_f32((uint16_t)(ud[k] >> 16));
+        od[k] = (uint32_t)f32_to_bf16_bits(silu_mul(g0, u0)) | ((uint32_t)f32_to_bf16_bits(silu_mul(g1, u1)) << 16);
+      } else {
+        g0 = f16_bits_to_f32((uint16_t)gd[k]); g1 = f16_bits_to_f32((uint16_t)(gd[k] >> 16));
+        u0 = f16_bits_to_f32((uint16_t)ud[k]); u1 = f16_bits_to_f32((uint16_t)(ud[k] >> 16));
+        od[k] = (uint32_t)f32_to_f16_bits(silu_mul(g0, u0)) | ((uint32_t)f32_to_f16_bits(silu_mul(g1, u1)) << 16);
+      }
+    }
+    *reinterpret_cast<uint4*>(out + i * 8) = make_uint4(od[0], od[1], od[2], od[3]);
+  }
+}
+
+hipError_t launch_silu_and_mul(const void* in, void* out, int dtype, int64_t m, int64_t h, hipStream_t s) {
+  if (m == 0 || h == 0) return hipSuccess;
+  const auto blocks = [](int64_t work) { return (unsigned)((work + 255) / 256 < 65536 ? (work + 255) / 256 : 65536); };
+  if (dtype == kF32) {
+    hipLaunchKernelGGL(silu_and_mul_kernel<float>, dim3(blocks(m * h)), dim3(256), 0, s,
+                       static_cast<const float*>(in), static_cast<float*>(out), m, h);
+  } else if (h % 8 == 0) {
+    const uint16_t* i16 = static_cast<const uint16_t*>(in);
+    uint16_t* o16 = static_cast<uint16_t*>(out);
+    if (dtype == kBF16)
+      hipLaunchKernelGGL(silu_and_mul16_kernel<true>, dim3(blocks(m * h / 8)), dim3(256), 0, s, i16, o16, m, h / 8);
+    else
+      hipLaunchKernelGGL(silu_and_mul16_kernel<false>, dim3(blocks(m * h / 8)), dim3(256), 0, s, i16, o16, m, h / 8);
+  } else if (dtype == kBF16) {
+    hipLaunchKernelGGL(silu_and_mul_kernel<bf16_tag>, dim3(blocks(m * h)), dim3(256), 0, s,
+                       static_cast<const bf16_tag*>(in), static_cast<bf16_tag*>(out), m, h);
+  } else {
+    hipLaunchKernelGGL(silu_and_mul_kernel<f16_tag>, dim3(blocks(m * h)), dim3(256), 0, s,
+                       static_cast<const f16_tag*>(in), static_cast<f16_tag*>(out), m, h);
+  }
+  return hipGetLastError();
+}
+
+}  // namespace ttq

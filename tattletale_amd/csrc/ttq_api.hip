@@ -129,6 +129,29 @@ int ttq_gemv_exl3(const uint16_t* trellis, const uint16_t* suh_f16, const uint16
                                           static_cast<hipStream_t>(stream)));
 }
 
+int ttq_silu_and_mul(const void* in, void* out, int dtype, int64_t m, int64_t h, void* stream) {
+  if (!valid_dtype(dtype)) return TTQ_ERR_DTYPE;
+  if (m < 0 || h < 0) return TTQ_ERR_SHAPE;
+  if (m == 0 || h == 0) return TTQ_OK;
+  if (!in || !out) return TTQ_ERR_NULL;
+  if (!aligned16(in) || !aligned16(out)) return TTQ_ERR_ALIGN;
+  return hip_status(ttq::launch_silu_and_mul(in, out, dtype, m, h, static_cast<hipStream_t>(stream)));
+}
+
+int ttq_gemv_q4_k_silu_mul(const void* w, const void* x, int x_dtype, void* y, int y_dtype, int64_t m,
+                           int64_t n_ff, int64_t n_in, void* stream) {
+  if (!valid_dtype(x_dtype) || !valid_dtype(y_dtype)) return TTQ_ERR_DTYPE;
+  if (n_ff < 0 || n_ff > (INT64_MAX >> 2)) return TTQ_ERR_SHAPE;
+  const int rc = check_shape(TTQ_Q4_K, m, 2 * n_ff, n_in, 0, 0);
+  if (rc != TTQ_OK) return rc;
+  if (m == 0 || n_ff == 0) return TTQ_OK;
+  if (!w || !x || !y) return TTQ_ERR_NULL;
+  if (!aligned16(w) || !aligned16(x) || !aligned16(y)) return TTQ_ERR_ALIGN;
+  if (!ttq::gemv_silu_mul_supported(TTQ_Q4_K, x_dtype, n_ff, n_in)) return TTQ_ERR_UNSUPPORTED;
+  return hip_status(ttq::launch_gemv_silu_mul(w, x, x_dtype, y, y_dtype, nullptr, 0, m, n_ff, n_in,
+                                              static_cast<hipStream_t>(stream)));
+}
+
 int ttq_gemm_q4_k(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m, int64_t n_out,
                   int64_t n_in, void* stream) {
   if (!w || !x_bf16 || !y_bf16) return TTQ_ERR_NULL;

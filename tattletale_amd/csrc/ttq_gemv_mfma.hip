@@ -109,7 +109,14 @@ __device__ __forceinline__ uint32_t pack_low_bytes(int a, int b, int c, int d) {
 // the partial row sums of the wavefronts [W][16] floats.
 //
 // W wavefronts per workgroup, R steps in flight per wavefront.
-template <int W, int R, typename XT, typename YT>
+//
+// FUSE: the weight holds gate rows [0, n_out) followed by up rows [n_out, 2*n_out), as
+// GatedMLP builds it (workspace/transformers/src/layers/mlp.nim:39), and the kernel writes
+// silu(gate . x) * (up . x), the silu_and_mul of
+// workspace/transformers/src/kernels/activations.nim:14-38, for its n_out outputs: row groups
+// alternate between the gate rows and the up rows of the same 16 outputs, and the wavefronts'
+// row sums meet in LDS at the end of every round.  rows_per_wg then counts outputs.
+template <int W, int R, bool FUSE, typename XT, typename YT>
 __global__ void __launch_bounds__(W * 64)
 gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
                      const void* __restrict__ bias, int bias_dtype, int n_out, int nsb, int rows_per_wg,
@@ -134,9 +141,15 @@ gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
   const int S = (nsb + SL - 1) >> sl_log2;
   const int wg_row0 = blockIdx.x * rows_per_wg;
   const int wg_row_end = min(wg_row0 + rows_per_wg, n_out);
-  const int rounds = (rows_per_wg + 16 * G - 1) / (16 * G);
+  const int per_round = FUSE ? 8 * G : 16 * G;   // rows (outputs when fused) of the workgroup per round
+  const int rounds = (rows_per_wg + per_round - 1) / per_round;
   const int t_total = rounds * S;
   const int last = wg_row_end - 1;   // rows past the workgroup's share re-read its last row
+  // weight row of lane n in row group `grp` of the workgroup
+  auto group_row = [&](int grp) {
+    if constexpr (FUSE) return min(wg_row0 + (grp >> 1) * 16 + n, last) + (grp & 1) * n_out;
+    else return min(wg_row0 + grp * 16 + n, last);
+  };
 
   // ---- activations: 16-byte loads (8 values) per thread, requested before any weights
   uint4 xraw[XP];
@@ -154,7 +167,7 @@ gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
   auto issue = [&](StepRaw& dst) {
     const int sb = (isi << sl_log2) + sl;
     const bool ok = ir < rounds && sb < nsb;
-    const int row = min(wg_row0 + (ir * G + gi) * 16 + n, last);
+    const int row = group_row(ir * G + gi);
     const uint32_t o_hdr = ok ? (uint32_t)row * rb + (uint32_t)sb * 144u : 0u;
     const uint32_t o_q = o_hdr + 16u + 16u * (uint32_t)g;
     dst.hdr = load16_a16(w + o_hdr);
@@ -274,7 +287,26 @@ gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
       float v = acc;
       v += __shfl_xor(v, 16, kWave);
       v += __shfl_xor(v, 32, kWave);
-      if (cr < rounds) {
+      if constexpr (FUSE) {
+        // every wavefront ends its round after the same number of steps
+        if (lane < 16) part[wave * 16 + n] = v;
+        __syncthreads();
+        if (cr < rounds && tid < 8 * G) {
+          const int pair = tid >> 4, nn = tid & 15;
+          float gate = 0.f, up = 0.f;
+          for (int s2 = 0; s2 < SL; s2++) {
+            gate += part[((2 * pair) * SL + s2) * 16 + nn];
+            up += part[((2 * pair + 1) * SL + s2) * 16 + nn];
+          }
+          const int o = wg_row0 + (cr * (G >> 1) + pair) * 16 + nn;
+          if (o < wg_row_end) {
+            gate += load_bias(bias, bias_dtype, o);
+            up += load_bias(bias, bias_dtype, (int64_t)n_out + o);
+            YElem<YT>::store(ym, o, (gate / (1.f + expf(-gate))) * up);
+          }
+        }
+        __syncthreads();
+      } else if (cr < rounds) {
         if (sl_log2 == 0) {
           const int row = wg_row0 + (cr * G + gi) * 16 + n;
           if (lane < 16 && row < wg_row_end) YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
@@ -299,7 +331,7 @@ gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
 #pragma unroll
   for (int i = 0; i < R; i++) consume(ring[i]);
 
-  if (sl_log2 != 0) {
+  if (!FUSE && sl_log2 != 0) {
     // one round only: add the slices in a fixed order
     __syncthreads();
     if (tid < 16 * G) {
@@ -331,7 +363,7 @@ static int mfma_env_int(const char* name, int dflt) {
   return e ? atoi(e) : dflt;
 }
 
-template <typename XT, typename YT>
+template <bool FUSE, typename XT, typename YT>
 static hipError_t launch_xy(const void* w, const void* x, void* y, const void* bias, int bias_dtype,
                             int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
   constexpr int W = kMfmaWaves;
@@ -341,11 +373,15 @@ static hipError_t launch_xy(const void* w, const void* x, void* y, const void* b
   if (num_wg > groups) num_wg = (int)groups;
   const int rows_per_wg = (int)((n_out + num_wg - 1) / num_wg);
   num_wg = (int)((n_out + rows_per_wg - 1) / rows_per_wg);
-  // the most slices that still leave room for all the workgroup's rows in one round
+  // the most slices that still leave room for all the workgroup's rows (outputs when fused: each
+  // needs a gate and an up row group) in one round
+  constexpr int kMaxSl = FUSE ? W / 2 : W;
+  constexpr int kRowsAllWaves = FUSE ? 8 * W : 16 * W;
   int sl_log2 = 0;
-  while ((2 << sl_log2) <= W && (2 << sl_log2) <= nsb && (16 * W >> (sl_log2 + 1)) >= rows_per_wg) sl_log2++;
+  while ((2 << sl_log2) <= kMaxSl && (2 << sl_log2) <= nsb && (kRowsAllWaves >> (sl_log2 + 1)) >= rows_per_wg)
+    sl_log2++;
   const size_t lds = (size_t)nsb * 4096 + (size_t)nsb * 64 + 1024;
-  auto kernel = gemv_q4k_mfma_kernel<W, kMfmaRing, XT, YT>;
+  auto kernel = gemv_q4k_mfma_kernel<W, kMfmaRing, FUSE, XT, YT>;
   static bool configured = false;
   if (!configured) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -360,13 +396,13 @@ static hipError_t launch_xy(const void* w, const void* x, void* y, const void* b
   return hipGetLastError();
 }
 
-template <typename XT>
+template <bool FUSE, typename XT>
 static hipError_t launch_x(const void* w, const void* x, void* y, int y_dtype, const void* bias, int bias_dtype,
                            int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
   switch (y_dtype) {
-    case kF32: return launch_xy<XT, float>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
-    case kF16: return launch_xy<XT, f16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
-    case kBF16: return launch_xy<XT, bf16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kF32: return launch_xy<FUSE, XT, float>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kF16: return launch_xy<FUSE, XT, f16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kBF16: return launch_xy<FUSE, XT, bf16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
     default: return hipErrorInvalidValue;
   }
 }
@@ -376,14 +412,29 @@ bool gemv_mfma_supported(int format, int x_dtype, int64_t n_out, int64_t n_in) {
   if (disabled) return false;
   // byte offsets into the weight buffer are 32-bit in the kernel; with fewer than eight rows per
   // CU the per-workgroup activation set-up outweighs the saving
-  return n_out >= 2048 && format == kQ4_K && (x_dtype == kBF16 || x_dtype == kF16) && n_in % 256 == 0 && n_in <= kMaxMfmaIn &&
-         n_out * (n_in / 256) * 144 < ((int64_t)1 << 32);
+  return n_out >= 2048 && format == kQ4_K && (x_dtype == kBF16 || x_dtype == kF16) && n_in % 256 == 0 &&
+         n_in <= kMaxMfmaIn && n_out * (n_in / 256) * 144 < ((int64_t)1 << 32);
 }
 
 hipError_t launch_gemv_mfma(const void* w, const void* x, int x_dtype, void* y, int y_dtype, const void* bias,
                             int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
-  if (x_dtype == kBF16) return launch_x<bf16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-  if (x_dtype == kF16) return launch_x<f16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  if (x_dtype == kBF16) return launch_x<false, bf16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  if (x_dtype == kF16) return launch_x<false, f16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  return hipErrorInvalidValue;
+}
+
+// Fused gate/up projection + silu_and_mul: w holds 2*n_ff rows (gate rows first), y has n_ff
+// columns.  Supported wherever the plain kernel is, for any n_ff >= 16.
+bool gemv_silu_mul_supported(int format, int x_dtype, int64_t n_ff, int64_t n_in) {
+  return format == kQ4_K && (x_dtype == kBF16 || x_dtype == kF16) && n_in % 256 == 0 && n_in <= kMaxMfmaIn &&
+         n_ff >= 16 && 2 * n_ff * (n_in / 256) * 144 < ((int64_t)1 << 32);
+}
+
+hipError_t launch_gemv_silu_mul(const void* w, const void* x, int x_dtype, void* y, int y_dtype, const void* bias,
+                                int bias_dtype, int64_t m, int64_t n_ff, int64_t n_in, hipStream_t s) {
+  if (m == 0 || n_ff == 0) return hipSuccess;
+  if (x_dtype == kBF16) return launch_x<true, bf16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_ff, n_in, s);
+  if (x_dtype == kF16) return launch_x<true, f16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_ff, n_in, s);
   return hipErrorInvalidValue;
 }
 

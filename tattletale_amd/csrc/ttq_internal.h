@@ -36,6 +36,14 @@ hipError_t launch_gemv_mfma(const void* w, const void* x, int x_dtype, void* y, 
                             const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                             hipStream_t s);
 
+// Fused gate/up GEMV + silu_and_mul for Q4_K (ttq_gemv_mfma.hip): w holds 2*n_ff rows, gate first.
+bool gemv_silu_mul_supported(int format, int x_dtype, int64_t n_ff, int64_t n_in);
+hipError_t launch_gemv_silu_mul(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                                const void* bias, int bias_dtype, int64_t m, int64_t n_ff,
+                                int64_t n_in, hipStream_t s);
+// out (m, h) = silu(in[:, :h]) * in[:, h:], in (m, 2h), same dtype (ttq_activations.hip).
+hipError_t launch_silu_and_mul(const void* in, void* out, int dtype, int64_t m, int64_t h, hipStream_t s);
+
 hipError_t launch_gemm_q4k(const void* w, const uint16_t* x_bf16, void* y, int y_dtype,
                            const void* bias, int bias_dtype, int64_t m, int64_t n_out,
                            int64_t n_in, hipStream_t s);

@@ -39,6 +39,9 @@ proc dequant_q8_0*(w, dst: pointer, out_dtype: cint, n_out, n_in: int64, stream:
 proc dequant_q4_k*(w, dst: pointer, out_dtype: cint, n_out, n_in: int64, stream: pointer): cint {.ttq.}
 proc dequant_q6_k*(w, dst: pointer, out_dtype: cint, n_out, n_in: int64, stream: pointer): cint {.ttq.}
 proc dequant_exl3*(trellis, dst: ptr uint16, n_out, n_in: int64, bits, codebook: cint, stream: pointer): cint {.ttq.}
+proc silu_and_mul*(src, dst: pointer, dtype: cint, m, h: int64, stream: pointer): cint {.ttq.}
+proc gemv_q4_k_silu_mul*(w, x: pointer, x_dtype: cint, y: pointer, y_dtype: cint, m, n_ff, n_in: int64,
+                         stream: pointer): cint {.ttq.}
 
 func ttqDtype(k: ScalarKind): cint =
   case k
@@ -88,3 +91,48 @@ proc forward*(self: QuantLinear, x: TorchTensor): TorchTensor =
   if rc != 0:
     raise newException(QuantLinearError, "ttq_linear_forward: " & $strerror(rc))
   if outKind != x.scalarType(): result = result.to(x.scalarType())
+
+# ---------------------------------------------------------------------------- gated MLP
+# Shaped like GatedMLP (workspace/transformers/src/layers/mlp.nim:25-60): one fused gate/up
+# projection, silu_and_mul (workspace/transformers/src/kernels/activations.nim:14-38), down.
+
+const kTtqErrUnsupported = -6
+
+type
+  QuantGatedMLP* = object
+    gate_up_proj*: QuantLinear    ## (2 * intermediate, hidden), gate rows first (mlp.nim:39)
+    down_proj*: QuantLinear       ## (hidden, intermediate)
+
+func init*(_: type QuantGatedMLP, gate_up_proj, down_proj: QuantLinear): QuantGatedMLP =
+  ## Row-wise block formats concatenate as bytes, so the caller builds gate_up_proj.qweight
+  ## with F.cat([gate_packed, up_packed], 0) exactly as mlp.nim:39 does for dense weights.
+  if gate_up_proj.out_features != 2 * down_proj.in_features or
+     gate_up_proj.in_features != down_proj.out_features:
+    raise newException(QuantLinearError, "gate_up / down shapes do not form a gated MLP")
+  QuantGatedMLP(gate_up_proj: gate_up_proj, down_proj: down_proj)
+
+proc quant_silu_and_mul*(x: TorchTensor): TorchTensor =
+  ## (..., 2h) -> (..., h), drop-in for silu_and_mul.
+  var shape = x.sizes().asNimView().toSeq()
+  let h = shape[^1] div 2
+  shape[^1] = h
+  result = F.empty(shape, x.options())
+  let rc = silu_and_mul(x.data_ptr(byte), result.data_ptr(byte), ttqDtype(x.scalarType()),
+                        x.numel() div (2 * h), h, nil)
+  if rc != 0: raise newException(QuantLinearError, "ttq_silu_and_mul: " & $strerror(rc))
+
+proc forward*(self: QuantGatedMLP, x: TorchTensor): TorchTensor =
+  ## x (..., hidden) -> (..., hidden).  Decode on Q4_K weights takes the fused kernel.
+  let gu = self.gate_up_proj
+  let nff = self.down_proj.in_features
+  let m = x.numel() div gu.in_features
+  if gu.format == kQ4_K and gu.bias.isNone and m == 1:
+    var shape = x.sizes().asNimView().toSeq()
+    shape[^1] = nff
+    let act = F.empty(shape, x.options())
+    let rc = gemv_q4_k_silu_mul(gu.qweight.data_ptr(byte), x.data_ptr(byte), ttqDtype(x.scalarType()),
+                                act.data_ptr(byte), ttqDtype(x.scalarType()), m, nff, gu.in_features, nil)
+    if rc == 0: return self.down_proj.forward(act)
+    if rc != kTtqErrUnsupported:
+      raise newException(QuantLinearError, "ttq_gemv_q4_k_silu_mul: " & $strerror(rc))
+  result = self.down_proj.forward(quant_silu_and_mul(gu.forward(x)))

@@ -208,3 +208,72 @@ def hadamard128_(v: torch.Tensor, pre: Optional[torch.Tensor] = None,
         check(_lib.lib().ttq_hadamard128_f32(v.data_ptr(), _ptr(pre), _ptr(post), v.numel(), _stream(dev)),
               "ttq_hadamard128_f32")
     return v
+
+
+# ------------------------------------------------------------------------------ gated MLP
+def silu_and_mul(x: torch.Tensor) -> torch.Tensor:
+    """(..., 2h) -> (..., h): silu(x[..., :h]) * x[..., h:]
+    (workspace/transformers/src/kernels/activations.nim:14-38), through ``ttq_silu_and_mul``."""
+    dev = _require_device(x)
+    if x.shape[-1] % 2:
+        raise TtqError(_lib.ERR_SHAPE, "silu_and_mul: last dim must be even")
+    h = x.shape[-1] // 2
+    out = torch.empty(x.shape[:-1] + (h,), dtype=x.dtype, device=dev)
+    with torch.cuda.device(dev):
+        check(_lib.lib().ttq_silu_and_mul(x.data_ptr(), out.data_ptr(), _code(x.dtype), x.numel() // (2 * h), h,
+                                          _stream(dev)), "ttq_silu_and_mul")
+    return out
+
+
+def gemv_q4_k_silu_mul(qweight: torch.Tensor, x: torch.Tensor, n_ff: int, n_in: int,
+                       out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """y (m, n_ff) = silu(x Wg^T) * (x Wu^T) for the packed (2*n_ff, n_in) Q4_K matrix [Wg; Wu],
+    one kernel (``ttq_gemv_q4_k_silu_mul``)."""
+    dev = _require_device(qweight, x)
+    m = x.numel() // n_in
+    out = torch.empty((m, n_ff), dtype=out_dtype, device=dev)
+    with torch.cuda.device(dev):
+        check(_lib.lib().ttq_gemv_q4_k_silu_mul(qweight.data_ptr(), x.data_ptr(), _code(x.dtype), out.data_ptr(),
+                                                _code(out_dtype), m, n_ff, n_in, _stream(dev)),
+              "ttq_gemv_q4_k_silu_mul")
+    return out
+
+
+@dataclass
+class QuantGatedMLP:
+    """Quantized counterpart of ``GatedMLP`` (workspace/transformers/src/layers/mlp.nim:25-60):
+    one fused gate/up projection, silu_and_mul, down projection."""
+
+    gate_up_proj: QuantLinear            # (2 * intermediate, hidden), gate rows first (mlp.nim:39)
+    down_proj: QuantLinear               # (hidden, intermediate)
+
+    @classmethod
+    def init(cls, gate_up_proj: QuantLinear, down_proj: QuantLinear) -> "QuantGatedMLP":
+        """Takes the already concatenated gate/up weight: rows of the block formats concatenate
+        as bytes, so ``torch.cat([gate_packed, up_packed])`` is the ``F.cat`` of mlp.nim:39."""
+        if gate_up_proj.out_features != 2 * down_proj.in_features:
+            raise TtqError(_lib.ERR_SHAPE, "QuantGatedMLP.init: gate_up rows != 2 * down columns")
+        if gate_up_proj.in_features != down_proj.out_features:
+            raise TtqError(_lib.ERR_SHAPE, "QuantGatedMLP.init: hidden sizes differ")
+        return cls(gate_up_proj, down_proj)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """x (..., hidden) -> (..., hidden)  (mlp.nim:43-60).  A single-token 16-bit activation
+        on Q4_K weights takes the fused GEMV + silu_and_mul kernel; everything else runs the
+        projection, ``silu_and_mul`` and the down projection as three launches."""
+        gu = self.gate_up_proj
+        n_ff = self.down_proj.in_features
+        m = x.numel() // gu.in_features
+        act = None
+        if gu.format == _lib.Q4_K and gu.bias is None and m == 1 and x.dtype in (torch.bfloat16, torch.float16):
+            try:
+                act = gemv_q4_k_silu_mul(gu.qweight, x.reshape(m, gu.in_features), n_ff, gu.in_features,
+                                         out_dtype=x.dtype).reshape(x.shape[:-1] + (n_ff,))
+            except TtqError as e:
+                if e.status != _lib.ERR_UNSUPPORTED:
+                    raise
+        if act is None:
+            act = silu_and_mul(gu.forward(x))
+        return self.down_proj.forward(act)
+
+    __call__ = forward

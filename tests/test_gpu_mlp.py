@@ -1,0 +1,116 @@
+"""Gated MLP pieces on the GPU against the CPU oracle, through the C ABI: silu_and_mul
+(workspace/transformers/src/kernels/activations.nim:14-38), its fusion into the Q4_K gate/up
+decode GEMV, and the GatedMLP mirror (workspace/transformers/src/layers/mlp.nim:25-60).
+
+Tolerances: fused GEMV + activation, fp32 output: relative L2 <= 1e-3 against silu(g) * u formed
+in float64 from the float64 products over oracle-dequantized weights.  Elementwise kernel: one
+rounding to the output type, so <= 1 ulp of it (2^-8 relative for bf16, 2^-11 for fp16; fp32: a
+few ulp from expf and the division)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from tattletale_amd import QuantGatedMLP, QuantLinear, TtqError, formats as F
+from tattletale_amd import qlinear as QL
+from tattletale_amd import quantize as Q
+
+from util import DEV, dev_bits, packed_to_dev, rel_l2, x_to_dev, random_blocks
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dt,ulp,tiny", [("f32", 2.0 ** -22, 1e-37), ("bf16", 2.0 ** -8, 1e-37), ("f16", 2.0 ** -11, 2.0 ** -24)])
+@pytest.mark.parametrize("m,h", [(1, 14336), (3, 40), (5, 7), (64, 1024)])
+def test_silu_and_mul_elementwise(dt, ulp, tiny, m, h):
+    x = Q.fill_normal(900 + h, 1, 2.5, m * 2 * h).reshape(m, 2 * h)
+    x[0, :4] = [0.0, -30.0, 30.0, -1.2784645]
+    xd, xf = x_to_dev(x, dt)
+    y = QL.silu_and_mul(xd)
+    assert y.shape == (m, h) and y.dtype == xd.dtype
+    got = y.float().cpu().numpy().astype(np.float64)
+    want = oracle.silu_and_mul_f64(xf.astype(np.float64))
+    # `tiny`: results below the type's smallest subnormal round to zero
+    assert np.all(np.abs(got - want) <= ulp * np.abs(want) + tiny)
+
+
+@pytest.mark.parametrize("xk", ["bf16", "f16"])
+@pytest.mark.parametrize("n_ff,n_in", [(16, 256), (100, 1024), (1000, 4096), (3000, 512), (20000, 256), (777, 8192)])
+def test_fused_gate_up_silu_mul_gemv(xk, n_ff, n_in):
+    """Every split of outputs and super-blocks over the wavefronts (one or several rounds, 1 to 8
+    slices, ragged last group), two activation rows."""
+    rng = np.random.default_rng(n_ff)
+    p = random_blocks(F.Q4_K, 2 * n_ff * (n_in // 256), seed=n_ff + 1)
+    outs = np.unique(np.concatenate([rng.integers(0, n_ff, 300), np.arange(max(0, n_ff - 20), n_ff), np.arange(min(20, n_ff))]))
+    rows = np.concatenate([outs, n_ff + outs])
+    what = oracle.dequant(F.Q4_K, np.ascontiguousarray(p.reshape(2 * n_ff, -1)[rows]), rows.size, n_in)
+    x = Q.fill_normal(n_in + 9, 1, 1.0, 2 * n_in).reshape(2, n_in) * np.float32(0.05)
+    xd, xf = x_to_dev(x, xk)
+    y = QL.gemv_q4_k_silu_mul(packed_to_dev(p), xd, n_ff, n_in).cpu().numpy()
+    assert y.shape == (2, n_ff) and np.all(np.isfinite(y))
+    gu = oracle.linear_f64(what, xf)                                  # (2, 2*len(outs)): gates then ups
+    want = oracle.silu_and_mul_f64(gu)
+    for r in range(2):
+        assert rel_l2(y[r][outs], want[r]) <= 1e-3
+    # and it is the same function as the two separate kernels (which accumulate differently)
+    sep = QL.silu_and_mul(QL.gemv(F.Q4_K, packed_to_dev(p), xd, 2 * n_ff, n_in)).cpu().numpy()
+    assert rel_l2(y, sep) <= 2e-4
+
+
+def test_fused_gemv_output_dtypes_and_refusals():
+    n_ff, n_in = 256, 1024
+    p = random_blocks(F.Q4_K, 2 * n_ff * (n_in // 256), seed=3)
+    xd, _ = x_to_dev(Q.fill_normal(4, 1, 0.05, n_in).reshape(1, n_in), "bf16")
+    y32 = QL.gemv_q4_k_silu_mul(packed_to_dev(p), xd, n_ff, n_in)
+    y16 = QL.gemv_q4_k_silu_mul(packed_to_dev(p), xd, n_ff, n_in, out_dtype=torch.bfloat16)
+    assert torch.equal(y16, y32.to(torch.bfloat16))
+    with pytest.raises(TtqError) as e:
+        QL.gemv_q4_k_silu_mul(packed_to_dev(p), xd.float(), n_ff, n_in)
+    assert e.value.status == F.ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("shape", [(1,), (1, 1), (2, 3), (40,)])
+def test_gated_mlp_forward(shape):
+    """(..., hidden) -> (..., hidden); decode takes the fused kernel, everything else the three
+    launches; both against the oracle's float64 chain on the same quantized weights."""
+    hidden, inter = 512, 1280
+    wg = Q.fill_normal(70, 0, 0.05, inter * hidden).reshape(inter, hidden)
+    wu = Q.fill_normal(71, 0, 0.05, inter * hidden).reshape(inter, hidden)
+    wd = Q.fill_normal(72, 0, 0.05, hidden * inter).reshape(hidden, inter)
+    pgu = np.concatenate([Q.quantize(F.Q4_K, wg), Q.quantize(F.Q4_K, wu)])     # F.cat of mlp.nim:39 on bytes
+    pd = Q.quantize(F.Q4_K, wd)
+    mlp = QuantGatedMLP.init(QuantLinear.init(packed_to_dev(pgu), F.Q4_K, hidden, 2 * inter),
+                             QuantLinear.init(packed_to_dev(pd), F.Q4_K, inter, hidden))
+    x = Q.fill_normal(73, 1, 1.0, int(np.prod(shape)) * hidden).reshape(shape + (hidden,))
+    xd, xf = x_to_dev(x, "bf16")
+    y = mlp.forward(xd)
+    assert y.shape == shape + (hidden,) and y.dtype == torch.bfloat16
+    wgu = oracle.dequant(F.Q4_K, pgu, 2 * inter, hidden)
+    wdd = oracle.dequant(F.Q4_K, pd, hidden, inter)
+    act = oracle.silu_and_mul_f64(oracle.linear_f64(wgu, xf.reshape(-1, hidden)))
+    # the activation travels as bf16 between the projections, as in the reference
+    act16 = oracle.bf16_to_f32(oracle.f32_to_bf16(act.astype(np.float32)))
+    want = oracle.linear_f64(wdd, act16)
+    got = oracle.bf16_to_f32(dev_bits(y)).reshape(-1, hidden)
+    assert rel_l2(got, want) <= 2e-2
+
+
+def test_gated_mlp_rejects_mismatched_layers():
+    a = QuantLinear.init(torch.zeros(144 * 64, dtype=torch.uint8, device=DEV), F.Q4_K, 256, 64)
+    b = QuantLinear.init(torch.zeros(144 * 16, dtype=torch.uint8, device=DEV), F.Q4_K, 256, 16)
+    with pytest.raises(TtqError):
+        QuantGatedMLP.init(a, b)
+
+
+def test_fused_full_shape_llama3_8b_ffn():
+    """28672 x 4096 (gate and up of 14336 each): finite everywhere, sampled outputs against the oracle."""
+    n_ff, n_in = 14336, 4096
+    p = random_blocks(F.Q4_K, 2 * n_ff * (n_in // 256), seed=99)
+    xd, xf = x_to_dev(Q.fill_normal(98, 1, 0.02, n_in).reshape(1, n_in), "bf16")
+    y = QL.gemv_q4_k_silu_mul(packed_to_dev(p), xd, n_ff, n_in).cpu().numpy()[0]
+    assert np.all(np.isfinite(y))
+    outs = np.unique(np.concatenate([np.arange(0, n_ff, 61), np.arange(n_ff - 64, n_ff)]))
+    rows = np.concatenate([outs, n_ff + outs])
+    what = oracle.dequant(F.Q4_K, np.ascontiguousarray(p.reshape(2 * n_ff, -1)[rows]), rows.size, n_in)
+    want = oracle.silu_and_mul_f64(oracle.linear_f64(what, xf))[0]
+    assert rel_l2(y[outs], want) <= 1e-3

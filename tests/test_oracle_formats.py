@@ -218,3 +218,22 @@ def test_fused_cpu_gemv_matches_dense(fmt):
     y = oracle.gemv_fused(fmt, p, x, 64, 512, nthreads=2)
     ref = oracle.linear_f64(oracle.dequant(fmt, p, 64, 512), x)[0]
     assert np.linalg.norm(y - ref) / np.linalg.norm(ref) < 1e-5
+
+
+def test_silu_and_mul_against_library_sigmoid_and_fixed_points():
+    """silu(g) = g * expit(g) (scipy), silu(0) = 0, silu(g) -> g and -> 0 at the ends, minimum
+    -0.27846 at g = -1.27846; the second half of the last axis multiplies
+    (kernels/activations.nim:14-38: silu(chunks[0]) * chunks[1])."""
+    from scipy.special import expit
+    rng = np.random.default_rng(5)
+    x = rng.normal(0, 3, (7, 64))
+    got = oracle.silu_and_mul_f64(x)
+    want = x[:, :32] * expit(x[:, :32]) * x[:, 32:]
+    assert got.shape == (7, 32)
+    assert np.allclose(got, want, rtol=1e-14, atol=1e-300)
+    one = lambda g, u: oracle.silu_and_mul_f64(np.array([[g, u]]))[0, 0]
+    assert one(0.0, 5.0) == 0.0
+    assert abs(one(40.0, 1.0) - 40.0) < 1e-12 and abs(one(-40.0, 1.0)) < 1e-12
+    assert abs(one(-1.2784645427610738, 1.0) + 0.27846454276107374) < 1e-12
+    # swapping the halves is a different function: gate is the FIRST half
+    assert one(2.0, 3.0) != one(3.0, 2.0)
