@@ -148,7 +148,7 @@ TTQ_API int ttq_silu_and_mul(const void* in, void* out, int dtype, int64_t m, in
  * matrix GatedMLP.init builds by row concatenation (mlp.nim:39).  Replaces
  * gate_up_proj.forward followed by silu_and_mul (mlp.nim:56-59) for decode.  16-bit
  * activations only; returns TTQ_ERR_UNSUPPORTED for shapes the fused kernel does not cover
- * (n_in > 8192, n_ff < 16, fp32 activations): call ttq_gemv_q4_k + ttq_silu_and_mul then. */
+ * (n_ff < 16, fp32 activations): call ttq_gemv_q4_k + ttq_silu_and_mul then. */
 TTQ_API int ttq_gemv_q4_k_silu_mul(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
                            int64_t m, int64_t n_ff, int64_t n_in, void* stream);
 

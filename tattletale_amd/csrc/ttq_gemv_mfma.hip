@@ -48,7 +48,8 @@ constexpr int kMfmaWaves = kMfmaThreads / kWave;
 // CU; asking for more lets the memory system serve the CUs unevenly, and the ones served last
 // unpack their whole share after the stream has ended.
 constexpr int kMfmaRing = 1;
-constexpr int64_t kMaxMfmaIn = 8192;            // activation table: 4 KiB of LDS per super-block
+constexpr int64_t kMaxMfmaIn = 16384;           // the limit of the GEMV entry points
+constexpr int kMaxWideSb = 32;                  // up to here the 4 KiB-per-super-block plane table fits LDS
 
 template <int CTRL>
 __device__ __forceinline__ float dpp_quad(float v) {
@@ -104,9 +105,20 @@ __device__ __forceinline__ uint32_t pack_low_bytes(int a, int b, int c, int d) {
   return p01 | (p23 << 16);
 }
 
-// LDS layout (bytes): plane table [nsb][4 MFMAs][64 lanes] x 16, then the per-sub-block
-// constants [nsb][4] x float4 {2^(E-13) of sub-blocks 2g, 2g+1, sum(x) of 2g, 2g+1}, then
-// the partial row sums of the wavefronts [W][16] floats.
+// LDS layout (bytes): plane table, then the per-sub-block constants [nsb][4] x float4
+// {2^(E-13) of sub-blocks 2g, 2g+1, sum(x) of 2g, 2g+1}, then the partial row sums of the
+// wavefronts [W][16] floats.
+// The plane table holds, per super-block b, the A operands of its four MFMAs.  Entry (b, m, h),
+// m = 2j + t, is plane t (0 = hi, 1 = lo) of the 16 activations x[256b + 32j + 16h ..]; as the A
+// operand of MFMA q = 2P + nib (P = which 64 bytes of qs, nib = low/high nibbles), lane (m, ga)
+// supplies that entry when k-group ga of this MFMA is sub-block j (j = 4P + 2(ga/2) + nib,
+// h = ga%2) and zeros otherwise.  Two layouts:
+//   wide    [nsb][4 MFMAs][64 lanes] x 16 bytes, zeros stored: every address is one register
+//           plus an immediate.  4 KiB per super-block, so only for n_in <= 8192.
+//   compact [nsb][32] x 16 bytes plus one zero entry.  A lane has at most one non-zero MFMA out
+//           of the four and reads `base_q + sb * stride_q` with (base, stride) = (its entry, 512)
+//           for that one and (the zero entry, 0) for the others: four more VALU instructions
+//           per step (about 3 % at 14336 x 4096), any n_in the entry points accept.
 //
 // W wavefronts per workgroup, R steps in flight per wavefront.
 //
@@ -116,18 +128,20 @@ __device__ __forceinline__ uint32_t pack_low_bytes(int a, int b, int c, int d) {
 // workspace/transformers/src/kernels/activations.nim:14-38, for its n_out outputs: row groups
 // alternate between the gate rows and the up rows of the same 16 outputs, and the wavefronts'
 // row sums meet in LDS at the end of every round.  rows_per_wg then counts outputs.
-template <int W, int R, bool FUSE, typename XT, typename YT>
+template <int W, int R, bool FUSE, bool COMPACT, typename XT, typename YT>
 __global__ void __launch_bounds__(W * 64)
 gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
                      const void* __restrict__ bias, int bias_dtype, int n_out, int nsb, int rows_per_wg,
                      int sl_log2) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const size_t table_bytes = COMPACT ? (size_t)nsb * 512 + 16 : (size_t)nsb * 4096;
   v4i_t* xa = reinterpret_cast<v4i_t*>(smem);
-  float* tab = reinterpret_cast<float*>(smem + (size_t)nsb * 4096);
-  float* part = reinterpret_cast<float*>(smem + (size_t)nsb * 4096 + (size_t)nsb * 64);
+  float* tab = reinterpret_cast<float*>(smem + table_bytes);
+  float* part = reinterpret_cast<float*>(smem + table_bytes + (size_t)nsb * 64);
 
   constexpr int kThreads = W * 64;
-  constexpr int XP = (int)(kMaxMfmaIn / (8 * kThreads));   // staging passes
+  // staging passes of 8 activations per thread: one covers everything the wide table can hold
+  constexpr int XP = COMPACT ? (int)(kMaxMfmaIn / (8 * kThreads)) : (kMaxWideSb * 256 + 8 * kThreads - 1) / (8 * kThreads);
   const int SL = 1 << sl_log2;          // slices of the super-blocks
   const int G = W >> sl_log2;           // row groups per round
   const int tid = threadIdx.x, lane = tid & 63;
@@ -156,7 +170,9 @@ gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
 #pragma unroll
   for (int p = 0; p < XP; p++) {
     const int k0 = 8 * (tid + p * kThreads);
-    xraw[p] = *reinterpret_cast<const uint4*>(xm + (k0 < n_in ? k0 : 0));
+    // a pass past the end re-reads the first pass's data (the compact table means n_in > 8192;
+    // spread addresses, never used)
+    xraw[p] = *reinterpret_cast<const uint4*>(xm + (k0 < n_in ? k0 : (COMPACT ? (k0 & (8 * kThreads - 1)) : 0)));
   }
   // every wavefront's x request is queued before any weight request of this workgroup
   __builtin_amdgcn_s_barrier();
@@ -178,9 +194,11 @@ gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
 #pragma unroll
   for (int i = 0; i < R; i++) issue(ring[i]);
 
-  // ---- zero the plane-table entries that stay zero.  Entry (b, q, la): la = 16*ga + m,
+  // ---- zero the plane-table entries that stay zero.  Wide entry (b, q, la): la = 16*ga + m,
   // m = 2j + t.  MFMA q = 2P + nib covers, in k-group ga, sub-block 4P + 2(ga/2) + nib.
-  {
+  if constexpr (COMPACT) {
+    if (tid < 4) reinterpret_cast<uint32_t*>(smem + (size_t)nsb * 512)[tid] = 0u;
+  } else {
     const int la = tid & 63, q = (tid >> 6) & 3;
     const int j = (la & 15) >> 1, ga = la >> 4;
     const bool nonzero = (q == 2 * (j >> 2) + (j & 1)) && ((ga >> 1) == ((j & 3) >> 1));
@@ -223,10 +241,12 @@ gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
       const int b = k0 >> 8, j = (k0 >> 5) & 7, h = (k0 >> 4) & 1, half8 = (k0 >> 3) & 1;
       const int q = 2 * (j >> 2) + (j & 1);
       const int ga = 2 * ((j & 3) >> 1) + h;
-      const int e_hi = ((b * 4 + q) * 64 + 16 * ga + 2 * j) * 2 + half8;   // in 8-byte units
+      // entry of the hi plane in 8-byte units, and the distance to the lo plane's
+      const int e_hi = COMPACT ? (b * 32 + 4 * j + h) * 2 + half8 : ((b * 4 + q) * 64 + 16 * ga + 2 * j) * 2 + half8;
+      constexpr int kLoStep = COMPACT ? 4 : 2;
       uint2* xa8 = reinterpret_cast<uint2*>(smem);
       xa8[e_hi] = make_uint2(pack_low_bytes(hi[0], hi[1], hi[2], hi[3]), pack_low_bytes(hi[4], hi[5], hi[6], hi[7]));
-      xa8[e_hi + 2] = make_uint2(pack_low_bytes(lo[0], lo[1], lo[2], lo[3]), pack_low_bytes(lo[4], lo[5], lo[6], lo[7]));
+      xa8[e_hi + kLoStep] = make_uint2(pack_low_bytes(lo[0], lo[1], lo[2], lo[3]), pack_low_bytes(lo[4], lo[5], lo[6], lo[7]));
       if ((tid & 3) == 0) {
         float* e = tab + (b * 4 + (j >> 1)) * 4 + (j & 1);
         e[0] = f;
@@ -240,14 +260,35 @@ gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
   ScaleBits B;
   B.init(g);
   constexpr uint32_t N4 = 0x0F0F0F0Fu;
+  // compact table: A-operand addresses of this lane (m = lane%16, ga = lane/16) for the four MFMAs
+  uint32_t a_base[4], a_stride[4];
+  {
+    const int mrow = lane & 15, ga = lane >> 4, j = mrow >> 1;
+    const bool valid = (ga >> 1) == ((j & 3) >> 1);
+    const int qstar = 2 * (j >> 2) + (j & 1);
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const bool mine = valid && q == qstar;
+      a_base[q] = mine ? (uint32_t)(mrow * 2 + (ga & 1)) * 16u : (uint32_t)nsb * 512u;
+      a_stride[q] = mine ? 512u : 0u;
+    }
+  }
   int cr = 0, csi = 0;                  // round and step-in-round being consumed
   float acc = 0.f;
 
   auto consume = [&](const StepRaw& s) {
     const int sb = (csi << sl_log2) + sl;
     if (cr < rounds && sb < nsb) {
-      const v4i_t* xe = xa + (size_t)sb * 256 + lane;
-      const v4i_t a0 = xe[0], a1 = xe[64], a2 = xe[128], a3 = xe[192];
+      v4i_t a0, a1, a2, a3;
+      if constexpr (COMPACT) {
+        a0 = *reinterpret_cast<const v4i_t*>(smem + a_base[0] + (uint32_t)sb * a_stride[0]);
+        a1 = *reinterpret_cast<const v4i_t*>(smem + a_base[1] + (uint32_t)sb * a_stride[1]);
+        a2 = *reinterpret_cast<const v4i_t*>(smem + a_base[2] + (uint32_t)sb * a_stride[2]);
+        a3 = *reinterpret_cast<const v4i_t*>(smem + a_base[3] + (uint32_t)sb * a_stride[3]);
+      } else {
+        const v4i_t* xe = xa + (size_t)sb * 256 + lane;
+        a0 = xe[0]; a1 = xe[64]; a2 = xe[128]; a3 = xe[192];
+      }
       const float4 cst = *reinterpret_cast<const float4*>(tab + (sb * 4 + g) * 4);
       v4i_t L0, H0, L1, H1;
       L0[0] = (int)(s.c0.x & N4); H0[0] = (int)((s.c0.x >> 4) & N4);
@@ -380,20 +421,24 @@ static hipError_t launch_xy(const void* w, const void* x, void* y, const void* b
   int sl_log2 = 0;
   while ((2 << sl_log2) <= kMaxSl && (2 << sl_log2) <= nsb && (kRowsAllWaves >> (sl_log2 + 1)) >= rows_per_wg)
     sl_log2++;
-  const size_t lds = (size_t)nsb * 4096 + (size_t)nsb * 64 + 1024;
-  auto kernel = gemv_q4k_mfma_kernel<W, kMfmaRing, FUSE, XT, YT>;
-  static bool configured = false;
-  if (!configured) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
+  const bool compact = nsb > kMaxWideSb;
+  const size_t lds = (compact ? (size_t)nsb * 512 + 16 : (size_t)nsb * 4096) + (size_t)nsb * 64 + 1024;
   const dim3 grid((unsigned)num_wg, (unsigned)m), block(W * 64);
-  hipLaunchKernelGGL(kernel, grid, block, lds, s, static_cast<const uint8_t*>(w),
-                     static_cast<const uint16_t*>(x), static_cast<YT*>(y), bias, bias_dtype, (int)n_out, nsb,
-                     rows_per_wg, sl_log2);
-  return hipGetLastError();
+  const auto launch = [&](auto kernel, bool& configured) -> hipError_t {
+    if (!configured) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      if (e != hipSuccess) return e;
+      configured = true;
+    }
+    hipLaunchKernelGGL(kernel, grid, block, lds, s, static_cast<const uint8_t*>(w),
+                       static_cast<const uint16_t*>(x), static_cast<YT*>(y), bias, bias_dtype, (int)n_out, nsb,
+                       rows_per_wg, sl_log2);
+    return hipGetLastError();
+  };
+  static bool configured_wide = false, configured_compact = false;
+  if (compact) return launch(gemv_q4k_mfma_kernel<W, kMfmaRing, FUSE, true, XT, YT>, configured_compact);
+  return launch(gemv_q4k_mfma_kernel<W, kMfmaRing, FUSE, false, XT, YT>, configured_wide);
 }
 
 template <bool FUSE, typename XT>

@@ -82,7 +82,7 @@ def test_other_entry_points_validate():
     assert L.ttq_gemv_q4_k_silu_mul(p, p, _lib.BF16, p, _lib.F32, 1, 0, 256, None) == _lib.OK
     # shapes the fused kernel does not cover are refused, not silently computed some other way
     assert L.ttq_gemv_q4_k_silu_mul(p, p, _lib.F32, p, _lib.F32, 1, 16, 256, None) == _lib.ERR_UNSUPPORTED
-    assert L.ttq_gemv_q4_k_silu_mul(p, p, _lib.BF16, p, _lib.F32, 1, 16, 16384, None) == _lib.ERR_UNSUPPORTED
+    assert L.ttq_gemv_q4_k_silu_mul(p, p, _lib.BF16, p, _lib.F32, 1, 8, 256, None) == _lib.ERR_UNSUPPORTED
     st = QLinearStruct(format=_lib.Q4_K, n_out=16, n_in=100, qweight=p)
     assert L.ttq_linear_forward(C.byref(st), p, _lib.BF16, 1, p, _lib.F32, None) == _lib.ERR_SHAPE
     st = QLinearStruct(format=42, n_out=16, n_in=256, qweight=p)

@@ -112,7 +112,7 @@ def test_row_concatenation_of_packed_weights_is_a_fused_layer():
 
 
 @pytest.mark.parametrize("xk", ["bf16", "f16"])
-@pytest.mark.parametrize("n_out,n_in", [(70000, 256), (25600, 512), (14336 + 8, 1024), (2500, 8192), (5000, 1280)])
+@pytest.mark.parametrize("n_out,n_in", [(70000, 256), (25600, 512), (14336 + 8, 1024), (2500, 8192), (5000, 1280), (4096, 14336), (2050, 16384)])
 def test_q4_k_16bit_work_distributions(xk, n_out, n_in):
     """Shapes that exercise every split of rows and super-blocks over the wavefronts of the
     matrix-core kernel: several rounds per workgroup, 1/2/4/16 slices, ragged last groups,

@@ -35,7 +35,7 @@ def test_silu_and_mul_elementwise(dt, ulp, tiny, m, h):
 
 
 @pytest.mark.parametrize("xk", ["bf16", "f16"])
-@pytest.mark.parametrize("n_ff,n_in", [(16, 256), (100, 1024), (1000, 4096), (3000, 512), (20000, 256), (777, 8192)])
+@pytest.mark.parametrize("n_ff,n_in", [(16, 256), (100, 1024), (1000, 4096), (3000, 512), (20000, 256), (777, 8192), (520, 14336)])
 def test_fused_gate_up_silu_mul_gemv(xk, n_ff, n_in):
     """Every split of outputs and super-blocks over the wavefronts (one or several rounds, 1 to 8
     slices, ragged last group), two activation rows."""
