@@ -234,14 +234,39 @@ def main() -> int:
                        "ttq_linear_forward")
             _lib.check(L.ttq_silu_and_mul(gu16.data_ptr(), y.data_ptr(), F.BF16, 1, n_ff, cur), "ttq_silu_and_mul")
 
+        # the same with the block's add + RMSNorm in front: one launch against four
+        res_in = torch.randn((1, n_in), device=dev).to(torch.bfloat16)
+        gamma = torch.ones(n_in, dtype=torch.bfloat16, device=dev)
+        new_res = torch.empty_like(res_in)
+        normed = torch.empty_like(res_in)
+
+        def norm_fused(i):
+            cur = torch.cuda.current_stream(dev).cuda_stream
+            _lib.check(L.ttq_gemv_q4_k_rmsnorm(ws[i % ncopies].data_ptr(), x.data_ptr(), res_in.data_ptr(),
+                                               gamma.data_ptr(), 1e-5, F.BF16, new_res.data_ptr(), None,
+                                               y.data_ptr(), F.BF16, 1, n_ff, n_in, 1, cur), "ttq_gemv_q4_k_rmsnorm")
+
+        def norm_unfused(i):
+            cur = torch.cuda.current_stream(dev).cuda_stream
+            _lib.check(L.ttq_rmsnorm(x.data_ptr(), res_in.data_ptr(), gamma.data_ptr(), 1e-5, F.BF16,
+                                     new_res.data_ptr(), normed.data_ptr(), 1, n_in, cur), "ttq_rmsnorm")
+            st.qweight = ws[i % ncopies].data_ptr()
+            _lib.check(L.ttq_linear_forward(C.byref(st), normed.data_ptr(), F.BF16, 1, gu16.data_ptr(), F.BF16, cur),
+                       "ttq_linear_forward")
+            _lib.check(L.ttq_silu_and_mul(gu16.data_ptr(), y.data_ptr(), F.BF16, 1, n_ff, cur), "ttq_silu_and_mul")
+
         _, f_ms = time_steps(fused, steps, warmup, use_graph=not args.eager)
         _, u_ms = time_steps(unfused, steps, warmup, use_graph=not args.eager)
+        _, nf_ms = time_steps(norm_fused, steps, warmup, use_graph=not args.eager)
+        _, nu_ms = time_steps(norm_unfused, steps, warmup, use_graph=not args.eager)
         res = {"name": "q4_k_gate_up_silu_gemv", "steps": steps, "weight_bytes": int(packed.nbytes),
                "weight_copies": ncopies, "ms_per_step": f_ms, "weight_GBps": packed.nbytes / (f_ms * 1e-3) / 1e9,
                "hbm_frac": packed.nbytes / (f_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-               "unfused_two_launches_ms_per_step": u_ms}
-        log("[q4_k_gate_up_silu_gemv] fused %.3f us/step (%.0f GB/s), GEMV + silu_and_mul %.3f us/step"
-            % (f_ms * 1e3, res["weight_GBps"], u_ms * 1e3))
+               "unfused_two_launches_ms_per_step": u_ms,
+               "with_add_rmsnorm_fused_ms_per_step": nf_ms, "with_add_rmsnorm_three_launches_ms_per_step": nu_ms}
+        log("[q4_k_gate_up_silu_gemv] fused %.3f us/step (%.0f GB/s), GEMV + silu_and_mul %.3f us/step; "
+            "with add+RMSNorm in front: one launch %.3f us/step, three launches %.3f us/step"
+            % (f_ms * 1e3, res["weight_GBps"], u_ms * 1e3, nf_ms * 1e3, nu_ms * 1e3))
         return res
 
     if args.only == "q4_k_gate_up_silu_gemv":

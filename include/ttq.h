@@ -152,6 +152,25 @@ TTQ_API int ttq_silu_and_mul(const void* in, void* out, int dtype, int64_t m, in
 TTQ_API int ttq_gemv_q4_k_silu_mul(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
                            int64_t m, int64_t n_ff, int64_t n_in, void* stream);
 
+/* ---- RMSNorm and its fusion into the decode GEMV -------------------------------------- */
+/* t = x (+ residual, rounded to dtype); normed = t * rsqrt(mean(t^2) + eps) * gamma, fp32
+ * arithmetic, one rounding to dtype.  x, residual, new_residual_out, normed_out are (m, n);
+ * gamma is (n).  Stands in for RmsNorm.forward (residual = NULL) and
+ * RmsNorm.forward_with_residual, which returns (normalized, new_residual)
+ * (workspace/transformers/src/layers/norm.nim:23-38; torch::rms_norm,
+ * workspace/libtorch/src/abi/neural_nets.nim:144-146).  new_residual_out may be NULL. */
+TTQ_API int ttq_rmsnorm(const void* x, const void* residual, const void* gamma, float eps, int dtype,
+                void* new_residual_out, void* normed_out, int64_t m, int64_t n, void* stream);
+/* y = Linear(RmsNorm(x [, residual])) in one kernel for a Q4_K weight and 16-bit activations:
+ * the "fused add + RMSNorm" that norm.nim:35 leaves as a TODO, placed in front of the decode
+ * GEMV.  With silu_mul != 0 the weight is the (2*n_out, n_in) gate/up matrix and y is
+ * silu_and_mul of the projection (mlp.nim:56-59).  residual, new_residual_out and normed_out
+ * may be NULL; normed_out receives the normalized row the GEMV consumed (other projections of
+ * the same block read it).  Returns TTQ_ERR_UNSUPPORTED for fp32 activations or n_out < 16. */
+TTQ_API int ttq_gemv_q4_k_rmsnorm(const void* w, const void* x, const void* residual, const void* gamma,
+                          float eps, int x_dtype, void* new_residual_out, void* normed_out, void* y,
+                          int y_dtype, int64_t m, int64_t n_out, int64_t n_in, int silu_mul, void* stream);
+
 /* ---- host-side preparation (CPU code; no GPU needed) ------------------------------- */
 /* Weight preparation happens once at load time, off the hot path; the reference's
  * counterpart is building the dense weight tensor handed to Linear.init (linear.nim:29-43,

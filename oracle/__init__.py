@@ -53,6 +53,8 @@ def lib() -> C.CDLL:
             getattr(L, name).argtypes = [vp, i64, vp]
         L.ora_q4k_unpack_scales.restype = None
         L.ora_q4k_unpack_scales.argtypes = [vp, vp, vp]
+        L.ora_rmsnorm_f64.restype = None
+        L.ora_rmsnorm_f64.argtypes = [vp, vp, C.c_double, vp, i64, i64]
         L.ora_silu_and_mul_f64.restype = None
         L.ora_silu_and_mul_f64.argtypes = [vp, vp, i64, i64]
         L.ora_linear_f64.restype = None
@@ -149,6 +151,19 @@ def linear_f64(w_f32, x_f32, bias_f32=None) -> np.ndarray:
     b = None if bias_f32 is None else _c(bias_f32, np.float32)
     lib().ora_linear_f64(_p(w), _p(x), _p(b) if b is not None else None, _p(y), m, n_out, n_in)
     return y
+
+
+def rmsnorm_f64(x, gamma, eps: float) -> np.ndarray:
+    """(m, n) -> (m, n): x / sqrt(mean(x^2) + eps) * gamma in float64 (norm.nim:23-25)."""
+    a = _c(x, np.float64)
+    if a.ndim == 1:
+        a = a[None, :]
+    g = _c(gamma, np.float64)
+    m, n = a.shape
+    assert g.shape == (n,)
+    out = np.empty((m, n), np.float64)
+    lib().ora_rmsnorm_f64(_p(a), _p(g), float(eps), _p(out), m, n)
+    return out
 
 
 def silu_and_mul_f64(x) -> np.ndarray:

@@ -28,6 +28,7 @@
  *                         round trip, bit-exact agreement with an independent
  *                         vectorised closed-form restatement (oracle/np_oracle.py)
  *   silu_and_mul          scipy.special.expit, fixed points and asymptotes
+ *   RMSNorm               numpy closed form, scale invariance, unit output RMS
  *   FWHT-128              scipy.linalg.hadamard, involution, norm preservation
  *   trellis decode        brute force on one tile via python big-int bit arithmetic
  *   codebooks             closed-form numpy restatement over all 65536 states
@@ -239,6 +240,21 @@ ORA_API void ora_silu_and_mul_f64(const double* in, double* out, int64_t m, int6
       const double g = in[i * 2 * h + c], u = in[i * 2 * h + h + c];
       out[i * h + c] = g / (1.0 + exp(-g)) * u;
     }
+}
+
+/* RMSNorm: out[i][k] = x[i][k] / sqrt(mean_k(x[i][k]^2) + eps) * gamma[k], float64.
+ * Follows RmsNorm.forward (workspace/transformers/src/layers/norm.nim:23-25), i.e.
+ * torch::rms_norm(input, {hidden}, weight, eps) (neural_nets.nim:144-146).  Pinned by a numpy
+ * closed form, scale invariance at eps = 0, unit RMS of the output for gamma = 1 and a
+ * constant-vector known answer.                                                          */
+ORA_API void ora_rmsnorm_f64(const double* x, const double* gamma, double eps, double* out,
+                             int64_t m, int64_t n) {
+  for (int64_t i = 0; i < m; i++) {
+    double ss = 0.0;
+    for (int64_t k = 0; k < n; k++) ss += x[i * n + k] * x[i * n + k];
+    const double rs = 1.0 / sqrt(ss / (double)n + eps);
+    for (int64_t k = 0; k < n; k++) out[i * n + k] = x[i * n + k] * rs * gamma[k];
+  }
 }
 
 /* Same product for a chosen subset of output rows (full-size spot checks). */

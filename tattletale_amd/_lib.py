@@ -60,6 +60,9 @@ SIGNATURES = {
     "ttq_dequant_exl3": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _vp]),
     "ttq_hadamard128_f32": (_i32, [_vp, _vp, _vp, _i64, _vp]),
     "ttq_silu_and_mul": (_i32, [_vp, _vp, _i32, _i64, _i64, _vp]),
+    "ttq_rmsnorm": (_i32, [_vp, _vp, _vp, C.c_float, _i32, _vp, _vp, _i64, _i64, _vp]),
+    "ttq_gemv_q4_k_rmsnorm": (_i32, [_vp, _vp, _vp, _vp, C.c_float, _i32, _vp, _vp, _vp, _i32, _i64, _i64, _i64,
+                                     _i32, _vp]),
     "ttq_gemv_q4_k_silu_mul": (_i32, [_vp, _vp, _i32, _vp, _i32, _i64, _i64, _i64, _vp]),
     "ttq_host_fill_normal": (_i32, [_u64, _u64, C.c_float, _vp, _i64]),
     "ttq_host_quantize_q8_0": (_i32, [_vp, _vp, _i64, _i64]),

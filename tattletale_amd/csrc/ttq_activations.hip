@@ -1,4 +1,6 @@
-// silu_and_mul on the GPU: out[..., :h] = silu(in[..., :h]) * in[..., h:2h].
+// Elementwise / row-wise pieces around the linear layers: silu_and_mul and RMSNorm.
+//
+// silu_and_mul: out[..., :h] = silu(in[..., :h]) * in[..., h:2h].
 //
 // Stand-in for workspace/transformers/src/kernels/activations.nim:14-38, which GatedMLP
 // applies to the output of the fused gate/up projection
@@ -71,6 +73,64 @@ hipError_t launch_silu_and_mul(const void* in, void* out, int dtype, int64_t m, 
     hipLaunchKernelGGL(silu_and_mul_kernel<f16_tag>, dim3(blocks(m * h)), dim3(256), 0, s,
                        static_cast<const f16_tag*>(in), static_cast<f16_tag*>(out), m, h);
   }
+  return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------ RMSNorm
+// One workgroup per row: t = x (+ residual, rounded to the tensor type, as the reference's
+// separate add does), normalized = t * rsqrt(mean(t^2) + eps) * gamma in fp32, one rounding.
+// Stand-in for RmsNorm.forward / forward_with_residual
+// (workspace/transformers/src/layers/norm.nim:23-38).  Two passes over the row (the second one
+// hits in cache: a row is a few KiB).
+template <typename T> __device__ __forceinline__ float round_as(float v);
+template <> __device__ __forceinline__ float round_as<float>(float v) { return v; }
+template <> __device__ __forceinline__ float round_as<f16_tag>(float v) { return f16_bits_to_f32(f32_to_f16_bits(v)); }
+template <> __device__ __forceinline__ float round_as<bf16_tag>(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+rmsnorm_kernel(const T* x, const T* residual, const T* __restrict__ gamma, float eps, T* new_residual,
+               T* normed, int64_t n) {   // new_residual / normed may be x or residual (same index, same thread)
+  __shared__ float red[4];
+  const int tid = threadIdx.x;
+  const int64_t row = (int64_t)blockIdx.x * n;
+  auto value = [&](int64_t k) {
+    const float t = XElem<T>::load(x, row + k);
+    return residual != nullptr ? round_as<T>(t + XElem<T>::load(residual, row + k)) : t;
+  };
+  float ss = 0.f;
+  for (int64_t k = tid; k < n; k += 256) {
+    const float t = value(k);
+    ss += t * t;
+  }
+  ss = wave_sum(ss);
+  if ((tid & 63) == 0) red[tid >> 6] = ss;
+  __syncthreads();
+  const float total = (red[0] + red[1]) + (red[2] + red[3]);
+  const float rs = 1.f / sqrtf(total / (float)n + eps);
+  for (int64_t k = tid; k < n; k += 256) {
+    const float t = value(k);
+    if (new_residual != nullptr) YElem<T>::store(new_residual, row + k, t);
+    YElem<T>::store(normed, row + k, (t * rs) * XElem<T>::load(gamma, k));
+  }
+}
+
+hipError_t launch_rmsnorm(const void* x, const void* residual, const void* gamma, float eps, int dtype,
+                          void* new_residual_out, void* normed_out, int64_t m, int64_t n, hipStream_t s) {
+  if (m == 0 || n == 0) return hipSuccess;
+  const dim3 grid((unsigned)m), block(256);
+  if (dtype == kF32)
+    hipLaunchKernelGGL(rmsnorm_kernel<float>, grid, block, 0, s, static_cast<const float*>(x),
+                       static_cast<const float*>(residual), static_cast<const float*>(gamma), eps,
+                       static_cast<float*>(new_residual_out), static_cast<float*>(normed_out), n);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(rmsnorm_kernel<bf16_tag>, grid, block, 0, s, static_cast<const bf16_tag*>(x),
+                       static_cast<const bf16_tag*>(residual), static_cast<const bf16_tag*>(gamma), eps,
+                       static_cast<bf16_tag*>(new_residual_out), static_cast<bf16_tag*>(normed_out), n);
+  else
+    hipLaunchKernelGGL(rmsnorm_kernel<f16_tag>, grid, block, 0, s, static_cast<const f16_tag*>(x),
+                       static_cast<const f16_tag*>(residual), static_cast<const f16_tag*>(gamma), eps,
+                       static_cast<f16_tag*>(new_residual_out), static_cast<f16_tag*>(normed_out), n);
   return hipGetLastError();
 }
 

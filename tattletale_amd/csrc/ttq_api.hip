@@ -147,9 +147,40 @@ int ttq_gemv_q4_k_silu_mul(const void* w, const void* x, int x_dtype, void* y, i
   if (m == 0 || n_ff == 0) return TTQ_OK;
   if (!w || !x || !y) return TTQ_ERR_NULL;
   if (!aligned16(w) || !aligned16(x) || !aligned16(y)) return TTQ_ERR_ALIGN;
-  if (!ttq::gemv_silu_mul_supported(TTQ_Q4_K, x_dtype, n_ff, n_in)) return TTQ_ERR_UNSUPPORTED;
-  return hip_status(ttq::launch_gemv_silu_mul(w, x, x_dtype, y, y_dtype, nullptr, 0, m, n_ff, n_in,
-                                              static_cast<hipStream_t>(stream)));
+  if (!ttq::gemv_fused_supported(TTQ_Q4_K, x_dtype, n_ff, n_in, true)) return TTQ_ERR_UNSUPPORTED;
+  return hip_status(ttq::launch_gemv_fused(w, x, x_dtype, y, y_dtype, nullptr, 0, m, n_ff, n_in, true, nullptr,
+                                           nullptr, 0.f, nullptr, nullptr, static_cast<hipStream_t>(stream)));
+}
+
+int ttq_rmsnorm(const void* x, const void* residual, const void* gamma, float eps, int dtype,
+                void* new_residual_out, void* normed_out, int64_t m, int64_t n, void* stream) {
+  if (!valid_dtype(dtype)) return TTQ_ERR_DTYPE;
+  if (m < 0 || n < 0 || !(eps >= 0.f)) return TTQ_ERR_SHAPE;
+  if (m == 0 || n == 0) return TTQ_OK;
+  if (!x || !gamma || !normed_out) return TTQ_ERR_NULL;
+  if (!aligned16(x) || !aligned16(gamma) || !aligned16(normed_out) || (residual && !aligned16(residual)) ||
+      (new_residual_out && !aligned16(new_residual_out)))
+    return TTQ_ERR_ALIGN;
+  return hip_status(ttq::launch_rmsnorm(x, residual, gamma, eps, dtype, new_residual_out, normed_out, m, n,
+                                        static_cast<hipStream_t>(stream)));
+}
+
+int ttq_gemv_q4_k_rmsnorm(const void* w, const void* x, const void* residual, const void* gamma, float eps,
+                          int x_dtype, void* new_residual_out, void* normed_out, void* y, int y_dtype,
+                          int64_t m, int64_t n_out, int64_t n_in, int silu_mul, void* stream) {
+  if (!valid_dtype(x_dtype) || !valid_dtype(y_dtype)) return TTQ_ERR_DTYPE;
+  if (n_out < 0 || n_out > (INT64_MAX >> 2) || !(eps >= 0.f)) return TTQ_ERR_SHAPE;
+  const int rc = check_shape(TTQ_Q4_K, m, silu_mul ? 2 * n_out : n_out, n_in, 0, 0);
+  if (rc != TTQ_OK) return rc;
+  if (m == 0 || n_out == 0) return TTQ_OK;
+  if (!w || !x || !gamma || !y) return TTQ_ERR_NULL;
+  if (!aligned16(w) || !aligned16(x) || !aligned16(gamma) || !aligned16(y) || (residual && !aligned16(residual)) ||
+      (new_residual_out && !aligned16(new_residual_out)) || (normed_out && !aligned16(normed_out)))
+    return TTQ_ERR_ALIGN;
+  if (!ttq::gemv_fused_supported(TTQ_Q4_K, x_dtype, n_out, n_in, silu_mul != 0)) return TTQ_ERR_UNSUPPORTED;
+  return hip_status(ttq::launch_gemv_fused(w, x, x_dtype, y, y_dtype, nullptr, 0, m, n_out, n_in, silu_mul != 0,
+                                           residual, gamma, eps, new_residual_out, normed_out,
+                                           static_cast<hipStream_t>(stream)));
 }
 
 int ttq_gemm_q4_k(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m, int64_t n_out,

@@ -98,6 +98,37 @@ template <> __device__ __forceinline__ void widen8<f16_tag>(const uint4& v, floa
   }
 }
 
+// float -> the 16-bit activation type and back (one rounding, nearest-even)
+template <typename XT> __device__ __forceinline__ uint16_t narrow1(float v);
+template <> __device__ __forceinline__ uint16_t narrow1<bf16_tag>(float v) { return f32_to_bf16_bits(v); }
+template <> __device__ __forceinline__ uint16_t narrow1<f16_tag>(float v) { return f32_to_f16_bits(v); }
+template <typename XT> __device__ __forceinline__ float widen1(uint16_t b);
+template <> __device__ __forceinline__ float widen1<bf16_tag>(uint16_t b) { return bf16_bits_to_f32(b); }
+template <> __device__ __forceinline__ float widen1<f16_tag>(uint16_t b) { return f16_bits_to_f32(b); }
+// rounds eight floats to the 16-bit type in place and returns their packed bits
+template <typename XT> __device__ __forceinline__ uint4 narrow8(float (&f)[8]) {
+  uint32_t d[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const uint16_t lo = narrow1<XT>(f[2 * i]), hi = narrow1<XT>(f[2 * i + 1]);
+    f[2 * i] = widen1<XT>(lo);
+    f[2 * i + 1] = widen1<XT>(hi);
+    d[i] = (uint32_t)lo | ((uint32_t)hi << 16);
+  }
+  return make_uint4(d[0], d[1], d[2], d[3]);
+}
+
+// Optional RMSNorm in front of the GEMV (NORM kernels): normalized = rms_norm(x [+ residual]) *
+// gamma, as RmsNorm.forward / forward_with_residual compute it before a Linear
+// (workspace/transformers/src/layers/norm.nim:23-38).  All buffers hold the activation type.
+struct GemvNormArgs {
+  const uint16_t* residual;     // (m, n_in) or null
+  const uint16_t* gamma;        // (n_in)
+  uint16_t* new_residual;       // (m, n_in) or null: x + residual
+  uint16_t* normed;             // (m, n_in) or null: the normalized activations the GEMV consumed
+  float eps;
+};
+
 // bytes 0 of a, b, c, d -> one dword (a lowest)
 __device__ __forceinline__ uint32_t pack_low_bytes(int a, int b, int c, int d) {
   const uint32_t p01 = __builtin_amdgcn_perm((uint32_t)b, (uint32_t)a, 0x0c0c0400u);
@@ -128,11 +159,16 @@ __device__ __forceinline__ uint32_t pack_low_bytes(int a, int b, int c, int d) {
 // workspace/transformers/src/kernels/activations.nim:14-38, for its n_out outputs: row groups
 // alternate between the gate rows and the up rows of the same 16 outputs, and the wavefronts'
 // row sums meet in LDS at the end of every round.  rows_per_wg then counts outputs.
-template <int W, int R, bool FUSE, bool COMPACT, typename XT, typename YT>
+//
+// NORM: every workgroup first normalizes the activation row itself (8 to 32 KiB, cheaper than a
+// kernel launch): t = x + residual rounded to the activation type, normalized =
+// t * rsqrt(mean(t^2) + eps) * gamma in fp32, rounded once to the activation type; the GEMV
+// then consumes exactly those rounded values.  Workgroup 0 writes t and the normalized row out.
+template <int W, int R, bool FUSE, bool COMPACT, bool NORM, typename XT, typename YT>
 __global__ void __launch_bounds__(W * 64)
 gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
                      const void* __restrict__ bias, int bias_dtype, int n_out, int nsb, int rows_per_wg,
-                     int sl_log2) {
+                     int sl_log2, GemvNormArgs na) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const size_t table_bytes = COMPACT ? (size_t)nsb * 512 + 16 : (size_t)nsb * 4096;
   v4i_t* xa = reinterpret_cast<v4i_t*>(smem);
@@ -174,6 +210,17 @@ gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
     // spread addresses, never used)
     xraw[p] = *reinterpret_cast<const uint4*>(xm + (k0 < n_in ? k0 : (COMPACT ? (k0 & (8 * kThreads - 1)) : 0)));
   }
+  uint4 rraw[NORM ? XP : 1], graw[NORM ? XP : 1];
+  if constexpr (NORM) {
+#pragma unroll
+    for (int p = 0; p < XP; p++) {
+      const int k0 = 8 * (tid + p * kThreads);
+      const int kc = k0 < n_in ? k0 : (COMPACT ? (k0 & (8 * kThreads - 1)) : 0);
+      graw[p] = *reinterpret_cast<const uint4*>(na.gamma + kc);
+      rraw[p] = make_uint4(0, 0, 0, 0);
+      if (na.residual != nullptr) rraw[p] = *reinterpret_cast<const uint4*>(na.residual + (int64_t)blockIdx.y * n_in + kc);
+    }
+  }
   // every wavefront's x request is queued before any weight request of this workgroup
   __builtin_amdgcn_s_barrier();
 
@@ -208,13 +255,57 @@ gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
     }
   }
 
+  // ---- the activations as floats, normalized first if asked
+  float xv[XP][8];
+#pragma unroll
+  for (int p = 0; p < XP; p++) widen8<XT>(xraw[p], xv[p]);
+  if constexpr (NORM) {
+    float ss = 0.f;
+#pragma unroll
+    for (int p = 0; p < XP; p++) {
+      const int k0 = 8 * (tid + p * kThreads);
+      if (k0 < n_in) {
+        if (na.residual != nullptr) {
+          float rf[8];
+          widen8<XT>(rraw[p], rf);
+#pragma unroll
+          for (int i = 0; i < 8; i++) xv[p][i] += rf[i];
+          const uint4 t = narrow8<XT>(xv[p]);     // the new residual, as the reference's add rounds it
+          if (blockIdx.x == 0 && na.new_residual != nullptr)
+            *reinterpret_cast<uint4*>(na.new_residual + (int64_t)blockIdx.y * n_in + k0) = t;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) ss += xv[p][i] * xv[p][i];
+      }
+    }
+    ss = wave_sum(ss);
+    if (lane == 0) part[wave] = ss;
+    __syncthreads();
+    float total = 0.f;
+#pragma unroll
+    for (int i = 0; i < W; i++) total += part[i];
+    const float rs = 1.f / sqrtf(total / (float)n_in + na.eps);
+#pragma unroll
+    for (int p = 0; p < XP; p++) {
+      const int k0 = 8 * (tid + p * kThreads);
+      if (k0 < n_in) {
+        float gf[8];
+        widen8<XT>(graw[p], gf);
+#pragma unroll
+        for (int i = 0; i < 8; i++) xv[p][i] = (xv[p][i] * rs) * gf[i];
+        const uint4 t = narrow8<XT>(xv[p]);
+        if (blockIdx.x == 0 && na.normed != nullptr)
+          *reinterpret_cast<uint4*>(na.normed + (int64_t)blockIdx.y * n_in + k0) = t;
+      }
+    }
+  }
+
   // ---- quantize the activations into the two byte planes
 #pragma unroll
   for (int p = 0; p < XP; p++) {
     const int k0 = 8 * (tid + p * kThreads);
     if (k0 < n_in) {
-      float xf[8];
-      widen8<XT>(xraw[p], xf);
+      float (&xf)[8] = xv[p];
       float amax = 0.f, sum = 0.f;
 #pragma unroll
       for (int i = 0; i < 8; i++) {
@@ -404,9 +495,9 @@ static int mfma_env_int(const char* name, int dflt) {
   return e ? atoi(e) : dflt;
 }
 
-template <bool FUSE, typename XT, typename YT>
+template <bool FUSE, bool NORM, typename XT, typename YT>
 static hipError_t launch_xy(const void* w, const void* x, void* y, const void* bias, int bias_dtype,
-                            int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+                            int64_t m, int64_t n_out, int64_t n_in, const GemvNormArgs& na, hipStream_t s) {
   constexpr int W = kMfmaWaves;
   const int nsb = (int)(n_in / 256);
   int num_wg = mfma_num_cus();
@@ -433,23 +524,32 @@ static hipError_t launch_xy(const void* w, const void* x, void* y, const void* b
     }
     hipLaunchKernelGGL(kernel, grid, block, lds, s, static_cast<const uint8_t*>(w),
                        static_cast<const uint16_t*>(x), static_cast<YT*>(y), bias, bias_dtype, (int)n_out, nsb,
-                       rows_per_wg, sl_log2);
+                       rows_per_wg, sl_log2, na);
     return hipGetLastError();
   };
   static bool configured_wide = false, configured_compact = false;
-  if (compact) return launch(gemv_q4k_mfma_kernel<W, kMfmaRing, FUSE, true, XT, YT>, configured_compact);
-  return launch(gemv_q4k_mfma_kernel<W, kMfmaRing, FUSE, false, XT, YT>, configured_wide);
+  if (compact) return launch(gemv_q4k_mfma_kernel<W, kMfmaRing, FUSE, true, NORM, XT, YT>, configured_compact);
+  return launch(gemv_q4k_mfma_kernel<W, kMfmaRing, FUSE, false, NORM, XT, YT>, configured_wide);
 }
 
-template <bool FUSE, typename XT>
+template <bool FUSE, bool NORM, typename XT>
 static hipError_t launch_x(const void* w, const void* x, void* y, int y_dtype, const void* bias, int bias_dtype,
-                           int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+                           int64_t m, int64_t n_out, int64_t n_in, const GemvNormArgs& na, hipStream_t s) {
   switch (y_dtype) {
-    case kF32: return launch_xy<FUSE, XT, float>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
-    case kF16: return launch_xy<FUSE, XT, f16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
-    case kBF16: return launch_xy<FUSE, XT, bf16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kF32: return launch_xy<FUSE, NORM, XT, float>(w, x, y, bias, bias_dtype, m, n_out, n_in, na, s);
+    case kF16: return launch_xy<FUSE, NORM, XT, f16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, na, s);
+    case kBF16: return launch_xy<FUSE, NORM, XT, bf16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, na, s);
     default: return hipErrorInvalidValue;
   }
+}
+
+template <bool FUSE, bool NORM>
+static hipError_t launch_any(const void* w, const void* x, int x_dtype, void* y, int y_dtype, const void* bias,
+                             int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, const GemvNormArgs& na,
+                             hipStream_t s) {
+  if (x_dtype == kBF16) return launch_x<FUSE, NORM, bf16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, na, s);
+  if (x_dtype == kF16) return launch_x<FUSE, NORM, f16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, na, s);
+  return hipErrorInvalidValue;
 }
 
 bool gemv_mfma_supported(int format, int x_dtype, int64_t n_out, int64_t n_in) {
@@ -463,24 +563,34 @@ bool gemv_mfma_supported(int format, int x_dtype, int64_t n_out, int64_t n_in) {
 
 hipError_t launch_gemv_mfma(const void* w, const void* x, int x_dtype, void* y, int y_dtype, const void* bias,
                             int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
-  if (x_dtype == kBF16) return launch_x<false, bf16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-  if (x_dtype == kF16) return launch_x<false, f16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-  return hipErrorInvalidValue;
+  return launch_any<false, false>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, GemvNormArgs{}, s);
 }
 
-// Fused gate/up projection + silu_and_mul: w holds 2*n_ff rows (gate rows first), y has n_ff
-// columns.  Supported wherever the plain kernel is, for any n_ff >= 16.
-bool gemv_silu_mul_supported(int format, int x_dtype, int64_t n_ff, int64_t n_in) {
+// Fused variants: gate/up projection + silu_and_mul (w holds 2*n_out rows, gate rows first,
+// y has n_out columns) and/or RMSNorm in front (norm_gamma != null).  Supported for 16-bit
+// activations, any n_in the entry points accept, n_out >= 16.
+bool gemv_fused_supported(int format, int x_dtype, int64_t n_out, int64_t n_in, bool silu_mul) {
   return format == kQ4_K && (x_dtype == kBF16 || x_dtype == kF16) && n_in % 256 == 0 && n_in <= kMaxMfmaIn &&
-         n_ff >= 16 && 2 * n_ff * (n_in / 256) * 144 < ((int64_t)1 << 32);
+         n_out >= 16 && (silu_mul ? 2 : 1) * n_out * (n_in / 256) * 144 < ((int64_t)1 << 32);
 }
 
-hipError_t launch_gemv_silu_mul(const void* w, const void* x, int x_dtype, void* y, int y_dtype, const void* bias,
-                                int bias_dtype, int64_t m, int64_t n_ff, int64_t n_in, hipStream_t s) {
-  if (m == 0 || n_ff == 0) return hipSuccess;
-  if (x_dtype == kBF16) return launch_x<true, bf16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_ff, n_in, s);
-  if (x_dtype == kF16) return launch_x<true, f16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_ff, n_in, s);
-  return hipErrorInvalidValue;
+hipError_t launch_gemv_fused(const void* w, const void* x, int x_dtype, void* y, int y_dtype, const void* bias,
+                             int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, bool silu_mul,
+                             const void* norm_residual, const void* norm_gamma, float norm_eps,
+                             void* new_residual_out, void* normed_out, hipStream_t s) {
+  if (m == 0 || n_out == 0) return hipSuccess;
+  GemvNormArgs na{};
+  na.residual = static_cast<const uint16_t*>(norm_residual);
+  na.gamma = static_cast<const uint16_t*>(norm_gamma);
+  na.new_residual = static_cast<uint16_t*>(new_residual_out);
+  na.normed = static_cast<uint16_t*>(normed_out);
+  na.eps = norm_eps;
+  if (norm_gamma != nullptr) {
+    if (silu_mul) return launch_any<true, true>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, na, s);
+    return launch_any<false, true>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, na, s);
+  }
+  if (silu_mul) return launch_any<true, false>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, na, s);
+  return launch_any<false, false>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, na, s);
 }
 
 }  // namespace ttq

@@ -36,11 +36,17 @@ hipError_t launch_gemv_mfma(const void* w, const void* x, int x_dtype, void* y, 
                             const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                             hipStream_t s);
 
-// Fused gate/up GEMV + silu_and_mul for Q4_K (ttq_gemv_mfma.hip): w holds 2*n_ff rows, gate first.
-bool gemv_silu_mul_supported(int format, int x_dtype, int64_t n_ff, int64_t n_in);
-hipError_t launch_gemv_silu_mul(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
-                                const void* bias, int bias_dtype, int64_t m, int64_t n_ff,
-                                int64_t n_in, hipStream_t s);
+// Fused decode kernels for Q4_K (ttq_gemv_mfma.hip): optional RMSNorm of the activation row in
+// front (norm_gamma != null; residual / outputs optional) and optional gate/up + silu_and_mul
+// behind (w then holds 2*n_out rows, gate rows first).
+bool gemv_fused_supported(int format, int x_dtype, int64_t n_out, int64_t n_in, bool silu_mul);
+hipError_t launch_gemv_fused(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                             const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                             bool silu_mul, const void* norm_residual, const void* norm_gamma,
+                             float norm_eps, void* new_residual_out, void* normed_out, hipStream_t s);
+// RMSNorm alone (ttq_activations.hip): t = x (+ residual), normed = t * rsqrt(mean(t^2) + eps) * gamma.
+hipError_t launch_rmsnorm(const void* x, const void* residual, const void* gamma, float eps, int dtype,
+                          void* new_residual_out, void* normed_out, int64_t m, int64_t n, hipStream_t s);
 // out (m, h) = silu(in[:, :h]) * in[:, h:], in (m, 2h), same dtype (ttq_activations.hip).
 hipError_t launch_silu_and_mul(const void* in, void* out, int dtype, int64_t m, int64_t h, hipStream_t s);
 

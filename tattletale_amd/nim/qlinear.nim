@@ -42,6 +42,11 @@ proc dequant_exl3*(trellis, dst: ptr uint16, n_out, n_in: int64, bits, codebook:
 proc silu_and_mul*(src, dst: pointer, dtype: cint, m, h: int64, stream: pointer): cint {.ttq.}
 proc gemv_q4_k_silu_mul*(w, x: pointer, x_dtype: cint, y: pointer, y_dtype: cint, m, n_ff, n_in: int64,
                          stream: pointer): cint {.ttq.}
+proc rmsnorm*(x, residual, gamma: pointer, eps: cfloat, dtype: cint, new_residual_out, normed_out: pointer,
+              m, n: int64, stream: pointer): cint {.ttq.}
+proc gemv_q4_k_rmsnorm*(w, x, residual, gamma: pointer, eps: cfloat, x_dtype: cint,
+                        new_residual_out, normed_out, y: pointer, y_dtype: cint, m, n_out, n_in: int64,
+                        silu_mul: cint, stream: pointer): cint {.ttq.}
 
 func ttqDtype(k: ScalarKind): cint =
   case k
@@ -136,3 +141,43 @@ proc forward*(self: QuantGatedMLP, x: TorchTensor): TorchTensor =
     if rc != kTtqErrUnsupported:
       raise newException(QuantLinearError, "ttq_gemv_q4_k_silu_mul: " & $strerror(rc))
   result = self.down_proj.forward(quant_silu_and_mul(gu.forward(x)))
+
+# ------------------------------------------------------------------------------ RMSNorm
+# Shaped like RmsNorm (workspace/transformers/src/layers/norm.nim:13-38).
+
+type
+  QuantRmsNorm* = object
+    weight*: TorchTensor
+    eps*: float
+    hidden_size*: int
+
+func init*(_: type QuantRmsNorm, weight: TorchTensor, eps: float = 1e-6): QuantRmsNorm =
+  QuantRmsNorm(weight: weight, eps: eps, hidden_size: weight.size(0))
+
+proc forward_with_residual*(self: QuantRmsNorm, hidden_state, residual: TorchTensor): (TorchTensor, TorchTensor) =
+  ## (normalized, new_residual), one kernel instead of an add and an rms_norm (the TODO of norm.nim:35).
+  let normalized = F.empty(hidden_state.sizes(), hidden_state.options())
+  let new_residual = F.empty(hidden_state.sizes(), hidden_state.options())
+  let rc = rmsnorm(hidden_state.data_ptr(byte), residual.data_ptr(byte), self.weight.data_ptr(byte),
+                   self.eps.cfloat, ttqDtype(hidden_state.scalarType()), new_residual.data_ptr(byte),
+                   normalized.data_ptr(byte), hidden_state.numel() div self.hidden_size, self.hidden_size, nil)
+  if rc != 0: raise newException(QuantLinearError, "ttq_rmsnorm: " & $strerror(rc))
+  (normalized, new_residual)
+
+proc forward_norm_gate_up*(norm: QuantRmsNorm, mlp: QuantGatedMLP,
+                           hidden_state, residual: TorchTensor): (TorchTensor, TorchTensor) =
+  ## Decode: add + RMSNorm + gate/up projection + silu_and_mul in ONE launch, then the down
+  ## projection.  Returns (mlp output, new_residual).
+  let gu = mlp.gate_up_proj
+  let nff = mlp.down_proj.in_features
+  var shape = hidden_state.sizes().asNimView().toSeq()
+  shape[^1] = nff
+  let act = F.empty(shape, hidden_state.options())
+  let new_residual = F.empty(hidden_state.sizes(), hidden_state.options())
+  let rc = gemv_q4_k_rmsnorm(gu.qweight.data_ptr(byte), hidden_state.data_ptr(byte), residual.data_ptr(byte),
+                             norm.weight.data_ptr(byte), norm.eps.cfloat, ttqDtype(hidden_state.scalarType()),
+                             new_residual.data_ptr(byte), nil, act.data_ptr(byte),
+                             ttqDtype(hidden_state.scalarType()), hidden_state.numel() div gu.in_features,
+                             nff, gu.in_features, 1, nil)
+  if rc != 0: raise newException(QuantLinearError, "ttq_gemv_q4_k_rmsnorm: " & $strerror(rc))
+  (mlp.down_proj.forward(act), new_residual)

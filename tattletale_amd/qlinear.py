@@ -239,6 +239,42 @@ def gemv_q4_k_silu_mul(qweight: torch.Tensor, x: torch.Tensor, n_ff: int, n_in: 
     return out
 
 
+def rmsnorm(x: torch.Tensor, gamma: torch.Tensor, eps: float, residual: Optional[torch.Tensor] = None):
+    """``RmsNorm.forward`` (residual None) / ``forward_with_residual``
+    (workspace/transformers/src/layers/norm.nim:23-38) through ``ttq_rmsnorm``.
+    Returns (normalized, new_residual or None)."""
+    dev = _require_device(x, gamma, residual)
+    n = x.shape[-1]
+    if gamma.numel() != n or gamma.dtype != x.dtype or (residual is not None and residual.shape != x.shape):
+        raise TtqError(_lib.ERR_SHAPE, "rmsnorm: gamma / residual do not match x")
+    normed = torch.empty_like(x)
+    new_res = torch.empty_like(x) if residual is not None else None
+    with torch.cuda.device(dev):
+        check(_lib.lib().ttq_rmsnorm(x.data_ptr(), _ptr(residual), gamma.data_ptr(), eps, _code(x.dtype),
+                                     _ptr(new_res), normed.data_ptr(), x.numel() // n, n, _stream(dev)),
+              "ttq_rmsnorm")
+    return normed, new_res
+
+
+def gemv_q4_k_rmsnorm(qweight: torch.Tensor, x: torch.Tensor, gamma: torch.Tensor, eps: float, n_out: int,
+                      n_in: int, residual: Optional[torch.Tensor] = None, silu_mul: bool = False,
+                      out_dtype: torch.dtype = torch.float32, want_normed: bool = True):
+    """y = Linear(RmsNorm(x [, residual])) (optionally followed by silu_and_mul over a gate/up
+    weight of 2*n_out rows) in one kernel (``ttq_gemv_q4_k_rmsnorm``).
+    Returns (y, normalized or None, new_residual or None)."""
+    dev = _require_device(qweight, x, gamma, residual)
+    m = x.numel() // n_in
+    y = torch.empty((m, n_out), dtype=out_dtype, device=dev)
+    normed = torch.empty_like(x) if want_normed else None
+    new_res = torch.empty_like(x) if residual is not None else None
+    with torch.cuda.device(dev):
+        check(_lib.lib().ttq_gemv_q4_k_rmsnorm(qweight.data_ptr(), x.data_ptr(), _ptr(residual), gamma.data_ptr(),
+                                               eps, _code(x.dtype), _ptr(new_res), _ptr(normed), y.data_ptr(),
+                                               _code(out_dtype), m, n_out, n_in, 1 if silu_mul else 0,
+                                               _stream(dev)), "ttq_gemv_q4_k_rmsnorm")
+    return y, normed, new_res
+
+
 @dataclass
 class QuantGatedMLP:
     """Quantized counterpart of ``GatedMLP`` (workspace/transformers/src/layers/mlp.nim:25-60):

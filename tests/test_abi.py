@@ -83,6 +83,16 @@ def test_other_entry_points_validate():
     # shapes the fused kernel does not cover are refused, not silently computed some other way
     assert L.ttq_gemv_q4_k_silu_mul(p, p, _lib.F32, p, _lib.F32, 1, 16, 256, None) == _lib.ERR_UNSUPPORTED
     assert L.ttq_gemv_q4_k_silu_mul(p, p, _lib.BF16, p, _lib.F32, 1, 8, 256, None) == _lib.ERR_UNSUPPORTED
+    assert L.ttq_rmsnorm(p, None, p, 1e-6, 9, None, p, 1, 8, None) == _lib.ERR_DTYPE
+    assert L.ttq_rmsnorm(p, None, p, -1.0, _lib.BF16, None, p, 1, 8, None) == _lib.ERR_SHAPE
+    assert L.ttq_rmsnorm(p, None, None, 1e-6, _lib.BF16, None, p, 1, 8, None) == _lib.ERR_NULL
+    assert L.ttq_rmsnorm(p, None, p, 1e-6, _lib.BF16, None, None, 1, 8, None) == _lib.ERR_NULL
+    assert L.ttq_rmsnorm(p, p + 2, p, 1e-6, _lib.BF16, None, p, 1, 8, None) == _lib.ERR_ALIGN
+    assert L.ttq_rmsnorm(p, None, p, 1e-6, _lib.BF16, None, p, 0, 8, None) == _lib.OK
+    assert L.ttq_gemv_q4_k_rmsnorm(p, p, None, None, 1e-6, _lib.BF16, None, None, p, _lib.F32, 1, 16, 256, 0, None) == _lib.ERR_NULL
+    assert L.ttq_gemv_q4_k_rmsnorm(p, p, None, p, 1e-6, _lib.BF16, None, None, p, _lib.F32, 1, 16, 100, 0, None) == _lib.ERR_SHAPE
+    assert L.ttq_gemv_q4_k_rmsnorm(p, p, None, p, 1e-6, _lib.F32, None, None, p, _lib.F32, 1, 16, 256, 0, None) == _lib.ERR_UNSUPPORTED
+    assert L.ttq_gemv_q4_k_rmsnorm(p, p, None, p, 1e-6, _lib.BF16, None, None, p, _lib.F32, 0, 16, 256, 1, None) == _lib.OK
     st = QLinearStruct(format=_lib.Q4_K, n_out=16, n_in=100, qweight=p)
     assert L.ttq_linear_forward(C.byref(st), p, _lib.BF16, 1, p, _lib.F32, None) == _lib.ERR_SHAPE
     st = QLinearStruct(format=42, n_out=16, n_in=256, qweight=p)

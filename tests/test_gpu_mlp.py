@@ -1,4 +1,4 @@
-"""Gated MLP pieces on the GPU against the CPU oracle, through the C ABI: silu_and_mul
+"""Gated MLP and RMSNorm pieces on the GPU against the CPU oracle, through the C ABI: silu_and_mul
 (workspace/transformers/src/kernels/activations.nim:14-38), its fusion into the Q4_K gate/up
 decode GEMV, and the GatedMLP mirror (workspace/transformers/src/layers/mlp.nim:25-60).
 
@@ -114,3 +114,99 @@ def test_fused_full_shape_llama3_8b_ffn():
     what = oracle.dequant(F.Q4_K, np.ascontiguousarray(p.reshape(2 * n_ff, -1)[rows]), rows.size, n_in)
     want = oracle.silu_and_mul_f64(oracle.linear_f64(what, xf))[0]
     assert rel_l2(y[outs], want) <= 1e-3
+
+
+# ------------------------------------------------------------------------------ RMSNorm
+def _round(a, dt):
+    if dt == "bf16":
+        return oracle.bf16_to_f32(oracle.f32_to_bf16(np.asarray(a, np.float32)))
+    if dt == "f16":
+        return oracle.f16_to_f32(oracle.f32_to_f16(np.asarray(a, np.float32)))
+    return np.asarray(a, np.float32)
+
+
+@pytest.mark.parametrize("dt,ulp", [("f32", 2.0 ** -21), ("bf16", 2.0 ** -8), ("f16", 2.0 ** -11)])
+@pytest.mark.parametrize("m,n", [(1, 4096), (3, 1000), (2, 14336)])
+@pytest.mark.parametrize("with_residual", [False, True])
+def test_rmsnorm_kernel(dt, ulp, m, n, with_residual):
+    """RmsNorm.forward / forward_with_residual (norm.nim:23-38): new_residual = x + residual rounded
+    to the tensor type (exactly what a separate add gives), normalized within one rounding of the
+    float64 formula applied to that new residual."""
+    x = Q.fill_normal(500 + n, 1, 1.5, m * n).reshape(m, n)
+    r = Q.fill_normal(501 + n, 1, 0.7, m * n).reshape(m, n)
+    g = 1.0 + Q.fill_normal(502 + n, 2, 0.1, n)
+    xd, xf = x_to_dev(x, dt)
+    rd, rf = x_to_dev(r, dt)
+    gd, gf = x_to_dev(g, dt)
+    normed, new_res = QL.rmsnorm(xd, gd.reshape(-1), 1e-5, rd if with_residual else None)
+    t = _round(xf + rf, dt) if with_residual else xf
+    if with_residual:
+        assert np.array_equal(new_res.float().cpu().numpy(), t)
+    else:
+        assert new_res is None
+    want = oracle.rmsnorm_f64(t.astype(np.float64), gf.reshape(-1).astype(np.float64), 1e-5)
+    got = normed.float().cpu().numpy().astype(np.float64)
+    assert np.all(np.abs(got - want) <= ulp * np.abs(want) + 1e-30)
+
+
+@pytest.mark.parametrize("xk", ["bf16", "f16"])
+@pytest.mark.parametrize("n_out,n_in,silu", [(100, 1024, False), (3000, 4096, False), (520, 14336, False),
+                                             (1000, 4096, True), (64, 256, True)])
+@pytest.mark.parametrize("with_residual", [False, True])
+def test_fused_rmsnorm_gemv(xk, n_out, n_in, silu, with_residual):
+    """One kernel for [add +] RMSNorm + GEMV [+ silu_and_mul].  The normalized row it reports must be
+    what the standalone kernel gives (to one unit in the last place) and y must be the GEMV of
+    exactly that row."""
+    rows = (2 if silu else 1) * n_out
+    p = random_blocks(F.Q4_K, rows * (n_in // 256), seed=n_out + 7)
+    x = Q.fill_normal(600 + n_in, 1, 2.0, 2 * n_in).reshape(2, n_in)
+    r = Q.fill_normal(601 + n_in, 1, 1.0, 2 * n_in).reshape(2, n_in)
+    g = 0.05 * (1.0 + Q.fill_normal(602 + n_in, 2, 0.2, n_in))
+    xd, _ = x_to_dev(x, xk)
+    rd, _ = x_to_dev(r, xk)
+    gd, _ = x_to_dev(g, xk)
+    gd = gd.reshape(-1)
+    res = rd if with_residual else None
+    y, normed, new_res = QL.gemv_q4_k_rmsnorm(packed_to_dev(p), xd, gd, 1e-5, n_out, n_in, residual=res, silu_mul=silu)
+    normed_ref, new_res_ref = QL.rmsnorm(xd, gd, 1e-5, res)
+    # the two kernels add the squares in different orders: the rows agree to one unit in the last place
+    a, b = normed.float(), normed_ref.float()
+    assert bool(((a - b).abs() <= (2.0 ** -7 if xk == "bf16" else 2.0 ** -10) * b.abs() + 1e-30).all())
+    if with_residual:
+        assert torch.equal(new_res, new_res_ref)
+    else:
+        assert new_res is None
+    # the same GEMV kernel on the row this kernel reported: identical arithmetic, identical bits
+    if silu:
+        y_ref = QL.gemv_q4_k_silu_mul(packed_to_dev(p), normed, n_out, n_in)
+    else:
+        y_ref = QL.gemv(F.Q4_K, packed_to_dev(p), normed, n_out, n_in)
+    if n_out >= 2048 or silu:
+        assert torch.equal(y, y_ref)
+    # and against the oracle on a sample of outputs
+    outs = np.unique(np.concatenate([np.arange(0, n_out, 17), np.arange(max(0, n_out - 20), n_out)]))
+    sel = np.concatenate([outs, n_out + outs]) if silu else outs
+    what = oracle.dequant(F.Q4_K, np.ascontiguousarray(p.reshape(rows, -1)[sel]), sel.size, n_in)
+    nf = normed.float().cpu().numpy()
+    prod = oracle.linear_f64(what, nf)
+    want = oracle.silu_and_mul_f64(prod) if silu else prod
+    got = y.cpu().numpy()
+    for i in range(2):
+        assert rel_l2(got[i][outs], want[i]) <= 1e-3
+
+
+def test_fused_rmsnorm_full_shape_gate_up():
+    """Llama-3-8B decode front half of the MLP in one launch: add + RMSNorm + gate/up + SiLU*mul."""
+    n_ff, n_in = 14336, 4096
+    p = random_blocks(F.Q4_K, 2 * n_ff * (n_in // 256), seed=123)
+    xd, _ = x_to_dev(Q.fill_normal(124, 1, 1.0, n_in).reshape(1, n_in), "bf16")
+    rd, _ = x_to_dev(Q.fill_normal(125, 1, 1.0, n_in).reshape(1, n_in), "bf16")
+    gd, _ = x_to_dev(0.02 * np.ones(n_in, np.float32), "bf16")
+    gd = gd.reshape(-1)
+    y, normed, new_res = QL.gemv_q4_k_rmsnorm(packed_to_dev(p), xd, gd, 1e-5, n_ff, n_in, residual=rd, silu_mul=True,
+                                              out_dtype=torch.bfloat16)
+    normed_ref, new_res_ref = QL.rmsnorm(xd, gd, 1e-5, rd)
+    assert torch.equal(new_res, new_res_ref)
+    assert bool(((normed.float() - normed_ref.float()).abs() <= 2.0 ** -7 * normed_ref.float().abs()).all())
+    y_ref = QL.gemv_q4_k_silu_mul(packed_to_dev(p), normed, n_ff, n_in, out_dtype=torch.bfloat16)
+    assert torch.equal(y, y_ref) and bool(torch.isfinite(y.float()).all())

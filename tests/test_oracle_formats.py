@@ -237,3 +237,21 @@ def test_silu_and_mul_against_library_sigmoid_and_fixed_points():
     assert abs(one(-1.2784645427610738, 1.0) + 0.27846454276107374) < 1e-12
     # swapping the halves is a different function: gate is the FIRST half
     assert one(2.0, 3.0) != one(3.0, 2.0)
+
+
+def test_rmsnorm_against_closed_form_and_invariants():
+    """x / sqrt(mean(x^2) + eps) * gamma (norm.nim:23-25 -> torch::rms_norm): numpy closed form,
+    scale invariance at eps = 0, unit RMS for gamma = 1, a constant vector, and eps actually used."""
+    rng = np.random.default_rng(6)
+    x = rng.normal(0, 2, (5, 96))
+    g = rng.normal(1, 0.2, 96)
+    got = oracle.rmsnorm_f64(x, g, 1e-6)
+    want = x / np.sqrt((x * x).mean(axis=1, keepdims=True) + 1e-6) * g
+    assert np.allclose(got, want, rtol=1e-14, atol=0)
+    assert np.allclose(oracle.rmsnorm_f64(37.5 * x, g, 0.0), oracle.rmsnorm_f64(x, g, 0.0), rtol=1e-13)
+    ones = np.ones(96)
+    out = oracle.rmsnorm_f64(x, ones, 0.0)
+    assert np.allclose(np.sqrt((out * out).mean(axis=1)), 1.0, rtol=1e-13)
+    assert np.allclose(oracle.rmsnorm_f64(np.full((1, 8), -3.0), np.arange(8.0), 0.0), -np.arange(8.0))
+    # mean, not sum; eps inside the root
+    assert np.allclose(oracle.rmsnorm_f64(np.full((1, 4), 2.0), np.ones(4), 5.0), 2.0 / 3.0)
