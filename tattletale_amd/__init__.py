@@ -9,12 +9,12 @@ import importlib
 from . import _lib as formats  # format / dtype / status codes
 from ._lib import TtqError, TtqLibraryError, lib
 
-__all__ = ["formats", "TtqError", "TtqLibraryError", "lib", "QuantLinear", "QuantGatedMLP", "quantize", "qlinear"]
+__all__ = ["formats", "TtqError", "TtqLibraryError", "lib", "QuantLinear", "QuantGatedMLP", "quantize", "qlinear", "gguf"]
 
 
 def __getattr__(name):
     # torch is only needed by the device-facing half; keep `import tattletale_amd` light
-    if name in ("quantize", "qlinear"):
+    if name in ("quantize", "qlinear", "gguf"):
         return importlib.import_module("." + name, __name__)
     if name in ("QuantLinear", "QuantGatedMLP"):
         return getattr(importlib.import_module(".qlinear", __name__), name)
