@@ -36,6 +36,12 @@ hipError_t launch_gemv_mfma(const void* w, const void* x, int x_dtype, void* y, 
                             const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                             hipStream_t s);
 
+// int8 matrix-core path for Q8_0, any activation dtype (ttq_gemv_q8_mfma.hip).
+bool gemv_q8_mfma_supported(int format, int64_t n_out, int64_t n_in);
+hipError_t launch_gemv_q8_mfma(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                               const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                               hipStream_t s);
+
 // Fused decode kernels for Q4_K (ttq_gemv_mfma.hip): optional RMSNorm of the activation row in
 // front (norm_gamma != null; residual / outputs optional) and optional gate/up + silu_and_mul
 // behind (w then holds 2*n_out rows, gate rows first).

@@ -172,6 +172,50 @@ def test_q4_k_16bit_activation_extremes():
     assert rel_l2(y[3], want[2]) <= TOL
 
 
+@pytest.mark.parametrize("xk", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("n_out,n_in", [(70000, 128), (25600, 256), (4096 + 8, 1024), (2500, 8192), (5000, 640)])
+def test_q8_0_work_distributions(xk, n_out, n_in):
+    """Q8_0 through the matrix cores (enough rows for that kernel): every split of rows and steps
+    over the wavefronts, all activation types, two activation rows of uneven magnitude."""
+    rng = np.random.default_rng(n_out + n_in)
+    p = random_blocks(F.Q8_0, n_out * (n_in // 32), seed=n_out)
+    rows = np.unique(np.concatenate([rng.integers(0, n_out, 400), np.arange(n_out - 40, n_out), np.arange(40)]))
+    what = oracle.dequant(F.Q8_0, np.ascontiguousarray(p.reshape(n_out, -1)[rows]), rows.size, n_in)
+    x = Q.fill_normal(n_in + 5, 1, 1.0, 2 * n_in).reshape(2, n_in)
+    x[1, ::7] *= 37.0
+    xd, xf = x_to_dev(x, xk)
+    y = QL.gemv(F.Q8_0, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()
+    assert np.all(np.isfinite(y))
+    want = oracle.linear_f64(what, xf)
+    for r in range(2):
+        assert rel_l2(y[r][rows], want[r]) <= (1e-6 if xk == "f32" else TOL)
+
+
+@pytest.mark.parametrize("xk", ["f32", "bf16"])
+def test_q8_0_unit_vectors_and_extremes_many_rows(xk):
+    n_out, n_in = 2100, 1024
+    p = random_blocks(F.Q8_0, n_out * (n_in // 32), seed=13)
+    what = oracle.dequant(F.Q8_0, p, n_out, n_in)
+    cols = [0, 1, 15, 16, 31, 32, 33, 127, 128, 500, n_in - 33, n_in - 1]
+    x = np.zeros((len(cols) + 3, n_in), np.float32)
+    for i, c in enumerate(cols):
+        x[i, c] = 1.0 if i % 2 == 0 else -0.5
+    x[-3] = Q.fill_normal(14, 1, 1e-3, n_in)
+    x[-3, 100] = 3.0e4                       # one huge value among tiny ones
+    x[-2] = Q.fill_normal(15, 1, 1.0, n_in)
+    x[-2, 5] = np.inf
+    x[-1] = Q.fill_normal(16, 1, 1.0, n_in) * 1e-30
+    xd, xf = x_to_dev(x, xk)
+    y = QL.gemv(F.Q8_0, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()
+    for i, c in enumerate(cols):
+        col = what[:, c] * np.float32(1.0 if i % 2 == 0 else -0.5)
+        assert np.array_equal(y[i], col), c
+    want = oracle.linear_f64(what, xf[[-3, -1]])
+    assert rel_l2(y[-3], want[0]) <= TOL
+    assert not np.any(np.isfinite(y[-2]))
+    assert rel_l2(y[-1], want[1]) <= TOL
+
+
 def test_gemv_rejects_oversized_rows():
     with pytest.raises(TtqError) as e:
         QL.gemv(F.Q4_K, torch.zeros(144 * 4 * 128, dtype=torch.uint8, device=DEV),
