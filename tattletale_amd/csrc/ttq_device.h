@@ -103,6 +103,9 @@ __device__ __forceinline__ uint32_t load4_a2(const uint8_t* p) {
   __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 4);
   return v;
 }
+__device__ __forceinline__ uint32_t load4_a4(const uint8_t* p) {
+  return *reinterpret_cast<const uint32_t*>(__builtin_assume_aligned(p, 4));
+}
 __device__ __forceinline__ uint16_t load2(const uint8_t* p) {
   uint16_t v;
   __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 2);

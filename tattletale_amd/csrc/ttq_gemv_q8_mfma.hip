@@ -47,7 +47,9 @@ template <> struct Q8X<f16_tag> {
   }
 };
 
-struct Q8Step { uint4 q0, q1; uint32_t d; };
+// q0/q1: the 16 bytes from the 4-byte aligned address at or below the lane's quants, e0/e1 the
+// dword after them (needed when the quants start 2 bytes into q0/q1)
+struct Q8Step { uint4 q0, q1; uint32_t e0, e1, d; };
 
 // LDS layout (bytes): plane table [nst][2 MFMAs][64 lanes] x 16 (entry (s, q, la): la = 16*ga + m,
 // m = 4b + t; MFMA q covers blocks 2q and 2q+1 of the step, k-group ga the half ga%2 of block
@@ -96,9 +98,14 @@ gemv_q8_mfma_kernel(const uint8_t* __restrict__ w, const typename Q8X<XT>::elem_
     const bool ok = ir < rounds && st < nst;
     const int row = min(wg_row0 + (ir * G + gi) * 16 + n, last);
     const uint32_t o = ok ? (uint32_t)row * rb + (uint32_t)st * 136u : 0u;
-    const uint32_t oq = o + 34u * (uint32_t)(g >> 1) + 2u + 16u * (uint32_t)(g & 1);
-    dst.q0 = load16_a2(w + oq);
-    dst.q1 = load16_a2(w + (oq + 68u));
+    // a step's 136 bytes start 8-byte aligned; the quants of blocks 0 and 2 sit 2 bytes past a
+    // dword boundary, those of blocks 1 and 3 on one
+    const uint32_t oq = o + 34u * (uint32_t)(g >> 1) + 16u * (uint32_t)(g & 1) + (g >= 2 ? 2u : 0u);
+    const uint32_t oe = oq + (g >= 2 ? 0u : 16u);
+    dst.q0 = load16_a4(w + oq);
+    dst.q1 = load16_a4(w + (oq + 68u));
+    dst.e0 = load4_a4(w + oe);
+    dst.e1 = load4_a4(w + (oe + 68u));
     dst.d = load2(w + (o + 34u * (uint32_t)g));
     if (++isi == S) { isi = 0; ir++; }
   };
@@ -166,8 +173,15 @@ gemv_q8_mfma_kernel(const uint8_t* __restrict__ w, const typename Q8X<XT>::elem_
       const v4i_t a0 = xe[0], a1 = xe[64];
       const float f = tab[st * 4 + g];
       v4i_t b0, b1;
-      b0[0] = (int)s.q0.x; b0[1] = (int)s.q0.y; b0[2] = (int)s.q0.z; b0[3] = (int)s.q0.w;
-      b1[0] = (int)s.q1.x; b1[1] = (int)s.q1.y; b1[2] = (int)s.q1.z; b1[3] = (int)s.q1.w;
+      const uint32_t sh = g >= 2 ? 0u : 16u;
+      b0[0] = (int)__builtin_amdgcn_alignbit(s.q0.y, s.q0.x, sh);
+      b0[1] = (int)__builtin_amdgcn_alignbit(s.q0.z, s.q0.y, sh);
+      b0[2] = (int)__builtin_amdgcn_alignbit(s.q0.w, s.q0.z, sh);
+      b0[3] = (int)__builtin_amdgcn_alignbit(s.e0, s.q0.w, sh);
+      b1[0] = (int)__builtin_amdgcn_alignbit(s.q1.y, s.q1.x, sh);
+      b1[1] = (int)__builtin_amdgcn_alignbit(s.q1.z, s.q1.y, sh);
+      b1[2] = (int)__builtin_amdgcn_alignbit(s.q1.w, s.q1.z, sh);
+      b1[3] = (int)__builtin_amdgcn_alignbit(s.e1, s.q1.w, sh);
       const v4i_t zero = {0, 0, 0, 0};
       // the non-zero rows of the two products are disjoint (blocks 0-1 and 2-3)
       const v4i_t Ca = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b0, zero, 0, 0, 0);
