@@ -123,6 +123,13 @@ TTQ_API int ttq_gemv_exl3(const uint16_t* trellis, const uint16_t* suh_f16, cons
  * (batch*seq, n_in) activation (neural_nets.nim:64; attn.nim:154-156 prefill case). */
 TTQ_API int ttq_gemm_q4_k(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m,
                   int64_t n_out, int64_t n_in, void* stream);
+/* The same operator for Q6_K and Q8_0 weights (a GGUF "Q4_K_M" file mixes Q4_K and Q6_K tensors;
+ * every projection of attn.nim:154-156,189 and mlp.nim:56,60 sees seq_len > 1 at prefill).
+ * n_in must be a multiple of 256. */
+TTQ_API int ttq_gemm_q6_k(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m,
+                  int64_t n_out, int64_t n_in, void* stream);
+TTQ_API int ttq_gemm_q8_0(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m,
+                  int64_t n_out, int64_t n_in, void* stream);
 
 /* ---- device dequantizers (the bit-exactness contract made observable) -------------- */
 /* out[n_out][n_in] in `out_dtype`: TTQ_F32 gives the canonical values; TTQ_BF16 gives them

@@ -23,7 +23,7 @@ SOURCES = [
     "ttq_gemv_mfma.hip",
     "ttq_gemv_q8_mfma.hip",
     "ttq_gemm_q4k.hip",
-    "ttq_gemm_q4k_pc.hip",
+    "ttq_gemm_pc.hip",
     "ttq_exl3.hip",
     "ttq_activations.hip",
     "ttq_host.cpp",

@@ -193,6 +193,25 @@ int ttq_gemm_q4_k(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64
                                          static_cast<hipStream_t>(stream)));
 }
 
+static int gemm_block(int format, const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m,
+                      int64_t n_out, int64_t n_in, void* stream) {
+  if (!w || !x_bf16 || !y_bf16) return TTQ_ERR_NULL;
+  const int rc = check_shape(format, m, n_out, n_in, 0, 0);
+  if (rc != TTQ_OK) return rc;
+  if (!aligned16(w) || !aligned16(x_bf16) || !aligned16(y_bf16)) return TTQ_ERR_ALIGN;
+  if (!ttq::gemm_pc_supported(format, m, n_out, n_in, 112)) return TTQ_ERR_UNSUPPORTED;
+  return hip_status(ttq::launch_gemm_pc(format, w, x_bf16, y_bf16, TTQ_BF16, nullptr, 0, m, n_out, n_in,
+                                        static_cast<hipStream_t>(stream)));
+}
+int ttq_gemm_q6_k(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m, int64_t n_out,
+                  int64_t n_in, void* stream) {
+  return gemm_block(TTQ_Q6_K, w, x_bf16, y_bf16, m, n_out, n_in, stream);
+}
+int ttq_gemm_q8_0(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m, int64_t n_out,
+                  int64_t n_in, void* stream) {
+  return gemm_block(TTQ_Q8_0, w, x_bf16, y_bf16, m, n_out, n_in, stream);
+}
+
 int ttq_dequant_q8_0(const void* w, void* out, int out_dtype, int64_t n_out, int64_t n_in, void* stream) {
   return dequant_block(TTQ_Q8_0, w, out, out_dtype, n_out, n_in, stream);
 }
@@ -247,6 +266,11 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
       (y_dtype == TTQ_BF16 || y_dtype == TTQ_F32)) {
     return hip_status(ttq::launch_gemm_q4k(layer->qweight, static_cast<const uint16_t*>(x), y, y_dtype,
                                            layer->bias, layer->bias_dtype, m, n_out, n_in, s));
+  }
+  if ((layer->format == TTQ_Q6_K || layer->format == TTQ_Q8_0) && x_dtype == TTQ_BF16 && m >= 16 &&
+      (y_dtype == TTQ_BF16 || y_dtype == TTQ_F32) && ttq::gemm_pc_supported(layer->format, m, n_out, n_in, 112)) {
+    return hip_status(ttq::launch_gemm_pc(layer->format, layer->qweight, static_cast<const uint16_t*>(x), y,
+                                          y_dtype, layer->bias, layer->bias_dtype, m, n_out, n_in, s));
   }
   const int lim = check_gemv_limits(x_dtype, n_in);
   if (lim != TTQ_OK) return lim;

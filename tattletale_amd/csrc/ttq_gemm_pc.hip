@@ -1,4 +1,5 @@
-// Prefill GEMM for Q4_K weights on gfx950, producer/consumer form:  Y (m, n_out) = X (m, n_in) * W^T.
+// Prefill GEMM for Q4_K, Q6_K and Q8_0 weights on gfx950, producer/consumer form:
+// Y (m, n_out) = X (m, n_in) * W^T.
 //
 // Replaces F.linear(x, weight) for a multi-row bf16 activation
 // (workspace/libtorch/src/abi/neural_nets.nim:64-81; the prefill case of
@@ -12,10 +13,11 @@
 //       straight into a private LDS ring (global_load_lds, no registers, whole 128-byte
 //       lines per row), three steps ahead; the 16-byte chunks of a row are XOR-swizzled on the
 //       way in so that the fragment reads (16 rows x one chunk) hit 16 different banks.
-//   producers (wavefronts 4-7): load the tile's packed super-blocks once per 256 k, dequantize
-//       64 k per step with the canonical arithmetic (d*sc*q - dmin*m; one fused multiply-add
-//       reproduces it exactly because d*sc*q has at most 21 significant bits), round to bf16
-//       nearest-even and write the B fragments to a double-buffered LDS tile.
+//   producers (wavefronts 4-7): load the tile's packed blocks once per 256 k, dequantize
+//       64 k per step with the format's canonical arithmetic (Q4_K: d*sc*q - dmin*m, where one
+//       fused multiply-add reproduces it exactly because d*sc*q has at most 21 significant bits;
+//       Q6_K: (d*sc)*(q-32); Q8_0: d*q), round to bf16 nearest-even and write the B fragments to
+//       a double-buffered LDS tile.  Only this role knows the weight format.
 // The hardware interleaves the two kinds of wavefront on each SIMD: the vector ALU and memory
 // work of the producers runs in the shadow of the consumers' MFMAs.  One barrier per 64-k step.
 #include "ttq_device.h"
@@ -60,11 +62,134 @@ __device__ __forceinline__ void lds_store16(uint32_t lds_addr, uint32_t a, uint3
   asm volatile("ds_write_b128 %0, %1" : : "v"(lds_addr), "v"(v) : "memory");
 }
 
+// ---- what the W producers know about a format.  A producer thread owns one row of the tile
+// and, of every 64-k step, the weights k = 16*whalf + e and k = 32 + 16*whalf + e (e = 0..15):
+// `lo` and `hi` below, 8 bf16 pairs each.  Raw holds the thread's share of 256 k of its row.
+template <int FMT> struct WFmt;
+
+template <> struct WFmt<kQ4_K> {
+  static constexpr int kUnitBytes = 144;               // one super-block
+  struct Raw { uint4 hdr, q[4]; };
+  static __device__ __forceinline__ void load(Raw& dst, const uint8_t* p, int whalf) {
+    dst.hdr = load16_a16(p);
+#pragma unroll
+    for (int c = 0; c < 4; c++) dst.q[c] = load16_a16(p + 16 + 32 * c + 16 * whalf);
+  }
+  template <int C>
+  static __device__ __forceinline__ void dequant(const Raw& r, int, uint32_t (&lo)[8], uint32_t (&hi)[8]) {
+    const float d = f16_bits_to_f32((uint16_t)(r.hdr.x & 0xFFFF));
+    const float dmin = f16_bits_to_f32((uint16_t)(r.hdr.x >> 16));
+    uint32_t sc1, mn1, sc2, mn2;
+    q4k_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, 2 * C, sc1, mn1);
+    q4k_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, 2 * C + 1, sc2, mn2);
+    const float d1 = d * (float)sc1, nm1 = -(dmin * (float)mn1);
+    const float d2 = d * (float)sc2, nm2 = -(dmin * (float)mn2);
+    const uint32_t qd[4] = {r.q[C].x, r.q[C].y, r.q[C].z, r.q[C].w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      // low nibbles are sub-block 2C (the first 32 k of the step), high nibbles sub-block 2C+1
+      const uint32_t l4 = qd[i] & 0x0F0F0F0Fu, h4 = (qd[i] >> 4) & 0x0F0F0F0Fu;
+      float fl[4], fh[4];
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        // fused multiply-add == canonical two-step form here (the product is exact)
+        fl[k] = fmaf_(d1, (float)((l4 >> (8 * k)) & 0xFFu), nm1);
+        fh[k] = fmaf_(d2, (float)((h4 >> (8 * k)) & 0xFFu), nm2);
+      }
+      lo[2 * i] = pack_bf16x2(fl[0], fl[1]);
+      lo[2 * i + 1] = pack_bf16x2(fl[2], fl[3]);
+      hi[2 * i] = pack_bf16x2(fh[0], fh[1]);
+      hi[2 * i + 1] = pack_bf16x2(fh[2], fh[3]);
+    }
+  }
+};
+
+// Q6_K super-block: ql[128] qh[64] scales[16] d.  Of each 128-weight half, weight l (< 32) is
+// the low nibble of ql[l], weight 32+l the low nibble of ql[32+l], weights 64+l and 96+l the
+// high nibbles of the same two bytes; qh[l] holds their four 2-bit tops.  Step C of the
+// super-block is weights 64*(C&1) .. +63 of half C/2, so the thread needs ql[l], ql[32+l] and
+// qh[l] for its l = 16*whalf + e; the scale of weight group t (32 weights) and this l is
+// scales[8*half + 2*t + whalf].
+template <> struct WFmt<kQ6_K> {
+  static constexpr int kUnitBytes = 210;
+  struct Raw { uint4 ql[4], qh[2], sc; uint32_t d; };
+  static __device__ __forceinline__ void load(Raw& dst, const uint8_t* p, int whalf) {
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      dst.ql[2 * h] = load16_a2(p + 64 * h + 16 * whalf);
+      dst.ql[2 * h + 1] = load16_a2(p + 64 * h + 32 + 16 * whalf);
+      dst.qh[h] = load16_a2(p + 128 + 32 * h + 16 * whalf);
+    }
+    dst.sc = load16_a2(p + 192);
+    dst.d = load2(p + 208);
+  }
+  template <int C>
+  static __device__ __forceinline__ void dequant(const Raw& r, int whalf, uint32_t (&lo)[8], uint32_t (&hi)[8]) {
+    constexpr int H = C >> 1, ODD = C & 1;
+    const float d = f16_bits_to_f32((uint16_t)r.d);
+    const uint32_t scw[4] = {r.sc.x, r.sc.y, r.sc.z, r.sc.w};
+    const uint32_t sw4 = scw[2 * H + ODD] >> (8 * whalf);       // scales 8H + 4*ODD + whalf (+2)
+    const float s1 = d * (float)(int)(int8_t)(sw4 & 0xFFu);
+    const float s2 = d * (float)(int)(int8_t)((sw4 >> 16) & 0xFFu);
+    const uint32_t a4[4] = {r.ql[2 * H].x, r.ql[2 * H].y, r.ql[2 * H].z, r.ql[2 * H].w};
+    const uint32_t b4[4] = {r.ql[2 * H + 1].x, r.ql[2 * H + 1].y, r.ql[2 * H + 1].z, r.ql[2 * H + 1].w};
+    const uint32_t h4[4] = {r.qh[H].x, r.qh[H].y, r.qh[H].z, r.qh[H].w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t qa = ((a4[i] >> (4 * ODD)) & 0x0F0F0F0Fu) | (((h4[i] >> (4 * ODD)) & 0x03030303u) << 4);
+      const uint32_t qb = ((b4[i] >> (4 * ODD)) & 0x0F0F0F0Fu) | (((h4[i] >> (4 * ODD + 2)) & 0x03030303u) << 4);
+      float fl[4], fh[4];
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        fl[k] = s1 * ((float)((qa >> (8 * k)) & 0xFFu) - 32.f);
+        fh[k] = s2 * ((float)((qb >> (8 * k)) & 0xFFu) - 32.f);
+      }
+      lo[2 * i] = pack_bf16x2(fl[0], fl[1]);
+      lo[2 * i + 1] = pack_bf16x2(fl[2], fl[3]);
+      hi[2 * i] = pack_bf16x2(fh[0], fh[1]);
+      hi[2 * i + 1] = pack_bf16x2(fh[2], fh[3]);
+    }
+  }
+};
+
+// Q8_0: eight 34-byte blocks { d, q[32] } per 256 k; step C is blocks 2C and 2C+1.
+template <> struct WFmt<kQ8_0> {
+  static constexpr int kUnitBytes = 8 * 34;
+  struct Raw { uint4 q[8]; uint32_t d[8]; };
+  static __device__ __forceinline__ void load(Raw& dst, const uint8_t* p, int whalf) {
+#pragma unroll
+    for (int b = 0; b < 8; b++) {
+      dst.q[b] = load16_a2(p + 34 * b + 2 + 16 * whalf);
+      dst.d[b] = load2(p + 34 * b);
+    }
+  }
+  template <int C>
+  static __device__ __forceinline__ void dequant(const Raw& r, int, uint32_t (&lo)[8], uint32_t (&hi)[8]) {
+    const float d0 = f16_bits_to_f32((uint16_t)r.d[2 * C]), d1 = f16_bits_to_f32((uint16_t)r.d[2 * C + 1]);
+    const uint32_t a4[4] = {r.q[2 * C].x, r.q[2 * C].y, r.q[2 * C].z, r.q[2 * C].w};
+    const uint32_t b4[4] = {r.q[2 * C + 1].x, r.q[2 * C + 1].y, r.q[2 * C + 1].z, r.q[2 * C + 1].w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      float fl[4], fh[4];
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        fl[k] = d0 * (float)(int)(int8_t)((a4[i] >> (8 * k)) & 0xFFu);
+        fh[k] = d1 * (float)(int)(int8_t)((b4[i] >> (8 * k)) & 0xFFu);
+      }
+      lo[2 * i] = pack_bf16x2(fl[0], fl[1]);
+      lo[2 * i + 1] = pack_bf16x2(fl[2], fl[3]);
+      hi[2 * i] = pack_bf16x2(fh[0], fh[1]);
+      hi[2 * i + 1] = pack_bf16x2(fh[2], fh[3]);
+    }
+  }
+};
+
+
 // W tile in LDS: [ksub 2][j NJ][g 4][n 16] units of 16 bytes (8 consecutive k of one column),
 // i.e. exactly the B operand of lane g*16+n for column block j.
-template <int NJ>
+template <int NJ, int FMT>
 __global__ void __launch_bounds__(kPcThreads)
-gemm_q4k_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, void* __restrict__ yv,
+gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, void* __restrict__ yv,
                    int y_dtype, const void* __restrict__ bias, int bias_dtype, int m, int n_out, int n_in,
                    int n_tiles, int m_tiles, int xcds_per_mtile) {
   constexpr int BN = NJ * 16;
@@ -156,43 +281,20 @@ gemm_q4k_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
     const int wt = pt < 2 * BN ? pt : pt - 2 * BN;
     const int wr = wt % BN, whalf = wt / BN;
     const int wrow = min(n0 + wr, n_out - 1);           // clamped: rows past the end are never stored
-    const uint8_t* wptr = w + (int64_t)nblocks * 144 * (int64_t)wrow;
+    using WF = WFmt<FMT>;
+    using WRaw = typename WF::Raw;
+    const uint8_t* wptr = w + (int64_t)nblocks * WF::kUnitBytes * (int64_t)wrow;
     const int wj = wr >> 4, wn = wr & 15;
     const uint32_t sw_addr = (uint32_t)(size_t)(lptr_t)(&sw[0]);
-    struct WRaw { uint4 hdr, q[4]; };
     auto load_w = [&](WRaw& dst, int b) {
-      const uint8_t* p = wptr + 144 * (int64_t)min(b, nblocks - 1);   // past the end: a harmless re-read
-      dst.hdr = load16_a16(p);
-#pragma unroll
-      for (int c = 0; c < 4; c++) dst.q[c] = load16_a16(p + 16 + 32 * c + 16 * whalf);
+      // past the end: a harmless re-read
+      WF::load(dst, wptr + WF::kUnitBytes * (int64_t)min(b, nblocks - 1), whalf);
     };
     auto dequant_to_lds = [&](const WRaw& r, auto cc, int buf) {
       constexpr int c = decltype(cc)::value;
-      const float d = f16_bits_to_f32((uint16_t)(r.hdr.x & 0xFFFF));
-      const float dmin = f16_bits_to_f32((uint16_t)(r.hdr.x >> 16));
-      uint32_t sc1, mn1, sc2, mn2;
-      q4k_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, 2 * c, sc1, mn1);
-      q4k_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, 2 * c + 1, sc2, mn2);
-      const float d1 = d * (float)sc1, nm1 = -(dmin * (float)mn1);
-      const float d2 = d * (float)sc2, nm2 = -(dmin * (float)mn2);
-      const uint32_t qd[4] = {r.q[c].x, r.q[c].y, r.q[c].z, r.q[c].w};
       uint32_t lo[8], hi[8];
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const uint32_t l4 = qd[i] & 0x0F0F0F0Fu, h4 = (qd[i] >> 4) & 0x0F0F0F0Fu;
-        float fl[4], fh[4];
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-          // fused multiply-add == canonical two-step form here (the product is exact)
-          fl[k] = fmaf_(d1, (float)((l4 >> (8 * k)) & 0xFFu), nm1);
-          fh[k] = fmaf_(d2, (float)((h4 >> (8 * k)) & 0xFFu), nm2);
-        }
-        lo[2 * i] = pack_bf16x2(fl[0], fl[1]);
-        lo[2 * i + 1] = pack_bf16x2(fl[2], fl[3]);
-        hi[2 * i] = pack_bf16x2(fh[0], fh[1]);
-        hi[2 * i + 1] = pack_bf16x2(fh[2], fh[3]);
-      }
-      // low nibbles: k = 16*half + e  -> ksub 0, groups 2*half and 2*half+1; high nibbles: ksub 1
+      WF::template dequant<c>(r, whalf, lo, hi);
+      // k = 16*half + e  -> ksub 0, groups 2*half and 2*half+1; k = 32 + 16*half + e: ksub 1
       const uint32_t base = sw_addr + (uint32_t)(buf * kWUnits + (wj * 4 + 2 * whalf) * 16 + wn) * 16u;
       lds_store16(base, lo[0], lo[1], lo[2], lo[3]);
       lds_store16(base + 256u, lo[4], lo[5], lo[6], lo[7]);
@@ -203,7 +305,7 @@ gemm_q4k_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
     using I1 = std::integral_constant<int, 1>;
     using I2 = std::integral_constant<int, 2>;
     using I3 = std::integral_constant<int, 3>;
-    // The packed super-blocks come from HBM (about 2 us away): block b+2 is requested at the
+    // The packed blocks come from HBM (about 2 us away): block b+2 is requested at the
     // start of block b, into the register set block b-1 used.  Three sets rotate by name, so no
     // copy ever forces a request to complete early.  These wavefronts issue no other global
     // loads, so the compiler's own counting of outstanding requests is exact.
@@ -355,6 +457,7 @@ gemm_q4k_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
   }
 }
 
+template <int FMT>
 static hipError_t launch_pc_112(const uint8_t* wb, const uint16_t* x, void* y, int y_dtype, const void* bias,
                                 int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
   constexpr int NJ = 7, BN = NJ * 16;
@@ -365,7 +468,7 @@ static hipError_t launch_pc_112(const uint8_t* wb, const uint16_t* x, void* y, i
     xcds_per_mtile = 8 / m_tiles;
     nwg = (unsigned)(((n_tiles + xcds_per_mtile - 1) / xcds_per_mtile) * 8);
   }
-  hipLaunchKernelGGL(gemm_q4k_pc_kernel<NJ>, dim3(nwg), dim3(kPcThreads), 0, s, wb, x, y, y_dtype, bias,
+  hipLaunchKernelGGL((gemm_pc_kernel<NJ, FMT>), dim3(nwg), dim3(kPcThreads), 0, s, wb, x, y, y_dtype, bias,
                      bias_dtype, (int)m, (int)n_out, (int)n_in, n_tiles, m_tiles, xcds_per_mtile);
   return hipGetLastError();
 }
@@ -373,17 +476,25 @@ static hipError_t launch_pc_112(const uint8_t* wb, const uint16_t* x, void* y, i
 // Only the 112-column tile is built in this form: with 128 columns the consumers' 128
 // accumulator registers plus the fragment rings do not fit the 168 registers a wavefront gets
 // when twelve of them share a CU.
-bool gemm_q4k_pc_supported(int64_t m, int64_t n_out, int64_t n_in, int bn) {
+bool gemm_pc_supported(int format, int64_t m, int64_t n_out, int64_t n_in, int bn) {
   static const int disabled = [] { const char* e = getenv("TTQ_GEMM_NO_PC"); return e ? atoi(e) : 0; }();
-  // activation byte offsets are 32-bit in the kernel
-  return !disabled && bn == 112 && m * n_in * 2 < ((int64_t)1 << 32) && n_out > 0;
+  // activation byte offsets are 32-bit in the kernel; a step loop iteration is 256 k
+  return !disabled && (format == kQ4_K || format == kQ6_K || format == kQ8_0) && bn == 112 &&
+         m * n_in * 2 < ((int64_t)1 << 32) && n_out > 0 && n_in > 0 && n_in % 256 == 0;
 }
 
-hipError_t launch_gemm_q4k_pc(const void* w, const uint16_t* x_bf16, void* y, int y_dtype, const void* bias,
-                              int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+hipError_t launch_gemm_pc(int format, const void* w, const uint16_t* x_bf16, void* y, int y_dtype,
+                          const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                          hipStream_t s) {
   if (m == 0 || n_out == 0) return hipSuccess;
   if (y_dtype != kBF16 && y_dtype != kF32) return hipErrorInvalidValue;
-  return launch_pc_112(static_cast<const uint8_t*>(w), x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  const uint8_t* wb = static_cast<const uint8_t*>(w);
+  switch (format) {
+    case kQ4_K: return launch_pc_112<kQ4_K>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kQ6_K: return launch_pc_112<kQ6_K>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kQ8_0: return launch_pc_112<kQ8_0>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    default: return hipErrorInvalidValue;
+  }
 }
 
 }  // namespace ttq

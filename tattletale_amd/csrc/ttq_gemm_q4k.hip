@@ -421,9 +421,9 @@ hipError_t launch_gemm_q4k(const void* w, const uint16_t* x_bf16, void* y, int y
   auto cost = [&](int64_t bn) { return ((((n_out + bn - 1) / bn) * mt + cus - 1) / cus) * bn; };
   static const int forced = [] { const char* e = getenv("TTQ_GEMM_BN"); return e ? atoi(e) : 0; }();
   const bool use112 = forced ? forced == 112 : cost(112) < cost(128);
-  // the producer/consumer kernel (ttq_gemm_q4k_pc.hip) exists for the 112-column tile
-  if (gemm_q4k_pc_supported(m, n_out, n_in, use112 ? 112 : 128))
-    return launch_gemm_q4k_pc(w, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  // the producer/consumer kernel (ttq_gemm_pc.hip) exists for the 112-column tile
+  if (gemm_pc_supported(kQ4_K, m, n_out, n_in, use112 ? 112 : 128))
+    return launch_gemm_pc(kQ4_K, w, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   const uint8_t* wb = static_cast<const uint8_t*>(w);
   return use112 ? launch_nj<7>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s)
                 : launch_nj<8>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);

@@ -60,11 +60,11 @@ hipError_t launch_gemm_q4k(const void* w, const uint16_t* x_bf16, void* y, int y
                            const void* bias, int bias_dtype, int64_t m, int64_t n_out,
                            int64_t n_in, hipStream_t s);
 
-// Producer/consumer form of the Q4_K GEMM (ttq_gemm_q4k_pc.hip).
-bool gemm_q4k_pc_supported(int64_t m, int64_t n_out, int64_t n_in, int bn);
-hipError_t launch_gemm_q4k_pc(const void* w, const uint16_t* x_bf16, void* y, int y_dtype,
-                              const void* bias, int bias_dtype, int64_t m, int64_t n_out,
-                              int64_t n_in, hipStream_t s);
+// Producer/consumer GEMM for Q4_K / Q6_K / Q8_0 weights and bf16 activations (ttq_gemm_pc.hip).
+bool gemm_pc_supported(int format, int64_t m, int64_t n_out, int64_t n_in, int bn);
+hipError_t launch_gemm_pc(int format, const void* w, const uint16_t* x_bf16, void* y, int y_dtype,
+                          const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                          hipStream_t s);
 
 hipError_t launch_dequant_exl3(const uint16_t* trellis, uint16_t* out_f16, int64_t n_out,
                                int64_t n_in, int bits, int cb, hipStream_t s);

@@ -35,6 +35,8 @@ proc gemv_q6_k*(w, x: pointer, x_dtype: cint, y: ptr cfloat, m, n_out, n_in: int
 proc gemv_exl3*(trellis, suh, svh, x: ptr uint16, y: ptr cfloat, m, n_out, n_in: int64,
                 bits, codebook: cint, stream: pointer): cint {.ttq.}
 proc gemm_q4_k*(w: pointer, x, y: ptr uint16, m, n_out, n_in: int64, stream: pointer): cint {.ttq.}
+proc gemm_q6_k*(w: pointer, x, y: ptr uint16, m, n_out, n_in: int64, stream: pointer): cint {.ttq.}
+proc gemm_q8_0*(w: pointer, x, y: ptr uint16, m, n_out, n_in: int64, stream: pointer): cint {.ttq.}
 proc dequant_q8_0*(w, dst: pointer, out_dtype: cint, n_out, n_in: int64, stream: pointer): cint {.ttq.}
 proc dequant_q4_k*(w, dst: pointer, out_dtype: cint, n_out, n_in: int64, stream: pointer): cint {.ttq.}
 proc dequant_q6_k*(w, dst: pointer, out_dtype: cint, n_out, n_in: int64, stream: pointer): cint {.ttq.}

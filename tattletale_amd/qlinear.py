@@ -161,19 +161,31 @@ def gemv_exl3(trellis: torch.Tensor, suh: torch.Tensor, svh: torch.Tensor, x: to
     return out
 
 
-def gemm_q4_k(qweight: torch.Tensor, x: torch.Tensor, n_out: int, n_in: int,
-              out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """bf16 Y (m, n_out) = bf16 X (m, n_in) * W^T through ``ttq_gemm_q4_k``."""
+_GEMM_ENTRY = {_lib.Q4_K: "ttq_gemm_q4_k", _lib.Q6_K: "ttq_gemm_q6_k", _lib.Q8_0: "ttq_gemm_q8_0"}
+
+
+def gemm(fmt: int, qweight: torch.Tensor, x: torch.Tensor, n_out: int, n_in: int,
+         out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """bf16 Y (m, n_out) = bf16 X (m, n_in) * W^T through ``ttq_gemm_<format>``."""
+    name = _GEMM_ENTRY.get(fmt)
+    if name is None:
+        raise TtqError(_lib.ERR_FORMAT, f"no prefill GEMM for format {fmt}")
     dev = _require_device(qweight, x, out)
     if x.dtype != torch.bfloat16:
-        raise TtqError(_lib.ERR_DTYPE, "ttq_gemm_q4_k takes bfloat16 activations")
+        raise TtqError(_lib.ERR_DTYPE, f"{name} takes bfloat16 activations")
     m = x.numel() // n_in
     if out is None:
         out = torch.empty((m, n_out), dtype=torch.bfloat16, device=dev)
     with torch.cuda.device(dev):
-        check(_lib.lib().ttq_gemm_q4_k(qweight.data_ptr(), x.data_ptr(), out.data_ptr(), m, n_out, n_in,
-                                       _stream(dev)), "ttq_gemm_q4_k")
+        check(getattr(_lib.lib(), name)(qweight.data_ptr(), x.data_ptr(), out.data_ptr(), m, n_out, n_in,
+                                        _stream(dev)), name)
     return out
+
+
+def gemm_q4_k(qweight: torch.Tensor, x: torch.Tensor, n_out: int, n_in: int,
+              out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """bf16 Y (m, n_out) = bf16 X (m, n_in) * W^T through ``ttq_gemm_q4_k``."""
+    return gemm(_lib.Q4_K, qweight, x, n_out, n_in, out)
 
 
 def dequantize(fmt: int, qweight: torch.Tensor, n_out: int, n_in: int,

@@ -64,6 +64,11 @@ def test_other_entry_points_validate():
     p += (-p) % 16
     assert L.ttq_gemm_q4_k(p, None, p, 16, 16, 256, None) == _lib.ERR_NULL
     assert L.ttq_gemm_q4_k(p, p, p, 16, 16, 100, None) == _lib.ERR_SHAPE
+    for fn in (L.ttq_gemm_q6_k, L.ttq_gemm_q8_0):
+        assert fn(p, None, p, 16, 16, 256, None) == _lib.ERR_NULL
+        assert fn(p, p, p, 16, 16, 100, None) == _lib.ERR_SHAPE
+        assert fn(p, p + 2, p, 16, 16, 256, None) == _lib.ERR_ALIGN
+    assert L.ttq_gemm_q8_0(p, p, p, 16, 16, 32, None) == _lib.ERR_UNSUPPORTED   # needs n_in % 256 == 0
     assert L.ttq_gemv_exl3(p, p, p, p, p, 1, 100, 128, 3, 1, None) == _lib.ERR_SHAPE
     assert L.ttq_gemv_exl3(p, p, p, p, p, 1, 128, 128, 0, 1, None) == _lib.ERR_FORMAT
     assert L.ttq_gemv_exl3(p, p, p, p, p, 1, 128, 128, 3, 5, None) == _lib.ERR_FORMAT

@@ -51,6 +51,60 @@ def test_gemm_identity_activations_give_bf16_weights_exactly(n_in):
     assert not (y[n_in:] & 0x7FFF).any()
 
 
+@pytest.mark.parametrize("fmt", [F.Q6_K, F.Q8_0])
+@pytest.mark.parametrize("m,n_out,n_in", [(64, 256, 1024), (16, 384, 512), (100, 200, 768), (257, 130, 1024),
+                                          (512, 512, 4096), (300, 1000, 256)])
+def test_gemm_random_other_formats(fmt, m, n_out, n_in):
+    w = Q.fill_normal(700 + m + fmt, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
+    p = Q.quantize(fmt, w)
+    what = oracle.dequant(fmt, p, n_out, n_in)
+    xd, xf = x_to_dev(Q.fill_normal(701 + m, 1, 1.0, m * n_in).reshape(m, n_in), "bf16")
+    y = QL.gemm(fmt, packed_to_dev(p), xd, n_out, n_in)
+    assert y.shape == (m, n_out) and y.dtype == torch.bfloat16
+    got = oracle.bf16_to_f32(dev_bits(y))
+    assert rel_l2(got, oracle.linear_f64(what, xf)) <= TOL
+    want_r = oracle.linear_f64(oracle.bf16_to_f32(oracle.f32_to_bf16(what)), xf)
+    assert rel_l2(got, want_r) <= 4e-3
+
+
+@pytest.mark.parametrize("fmt", [F.Q6_K, F.Q8_0])
+@pytest.mark.parametrize("n_in", [256, 1024])
+def test_gemm_identity_activations_other_formats(fmt, n_in):
+    # random block bytes: every scale sign, every quant value, every position of the block layout
+    n_out = 192
+    p = random_blocks(fmt, n_out * (n_in // {F.Q6_K: 256, F.Q8_0: 32}[fmt]), seed=23 + fmt)
+    what = oracle.dequant(fmt, p, n_out, n_in)
+    m = n_in + 32
+    x = np.zeros((m, n_in), np.float32)
+    x[np.arange(n_in), np.arange(n_in)] = 1.0
+    xd, _ = x_to_dev(x, "bf16")
+    y = dev_bits(QL.gemm(fmt, packed_to_dev(p), xd, n_out, n_in))
+    want = oracle.f32_to_bf16(what).T.copy()
+    want[want == 0x8000] = 0         # a sum that starts at +0 cannot end at -0 (negative scale x zero quant)
+    assert np.array_equal(y[:n_in], want)
+    assert not (y[n_in:] & 0x7FFF).any()
+
+
+@pytest.mark.parametrize("fmt", [F.Q6_K, F.Q8_0])
+def test_forward_prefill_other_formats(fmt):
+    n_out, n_in, m = 256, 1024, 48
+    w = Q.fill_normal(410 + fmt, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
+    p = Q.quantize(fmt, w)
+    what = oracle.dequant(fmt, p, n_out, n_in)
+    bias = Q.fill_normal(411, 2, 0.5, n_out)
+    xd, xf = x_to_dev(Q.fill_normal(412, 1, 1.0, m * n_in).reshape(4, 12, n_in), "bf16")
+    bd, bf = x_to_dev(bias, "f32")
+    layer = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out, bias=bd)
+    y = layer.forward(xd)
+    assert y.shape == (4, 12, n_out) and y.dtype == torch.bfloat16
+    want = oracle.linear_f64(what, xf.reshape(m, n_in), bf).reshape(4, 12, n_out)
+    assert rel_l2(oracle.bf16_to_f32(dev_bits(y)), want) <= TOL
+    y32 = layer.forward(xd, out_dtype=torch.float32)
+    assert rel_l2(y32.cpu().numpy(), want) <= TOL
+    row = layer.forward(xd[1, 5], out_dtype=torch.float32).cpu().numpy()
+    assert rel_l2(row, y32[1, 5].cpu().numpy()) <= 5e-3
+
+
 def test_forward_dispatches_prefill_to_gemm_and_matches_gemv():
     n_out, n_in, m = 256, 1024, 48
     w = Q.fill_normal(400, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
@@ -81,6 +135,23 @@ def test_full_shape_sampled_columns(name, step):
     sub = np.ascontiguousarray(p.reshape(cfg.n_out, -1)[cols])
     what = oracle.dequant(F.Q4_K, sub, cols.size, cfg.n_in)
     rows = np.unique(np.concatenate([np.arange(0, cfg.m, max(1, cfg.m // 64)), [cfg.m - 1]]))
+    want = oracle.linear_f64(what, oracle.bf16_to_f32(xbits[rows]))
+    got = oracle.bf16_to_f32(dev_bits(y[torch.from_numpy(rows).to(DEV)][:, torch.from_numpy(cols).to(DEV)]))
+    assert rel_l2(got, want) <= TOL
+
+
+@pytest.mark.parametrize("name,n_out", [("q8_0_gemv", 4096), ("q6_k_gemv", 14336)])
+def test_full_shape_other_formats_sampled_columns(name, n_out):
+    # the weights of the decode configurations (Q6_K: the first 14336 rows) under a 512-row activation
+    cfg = CFG.CONFIGS[name]
+    m = 512
+    p = CFG.packed_weights(cfg, n_out)
+    xbits = Q.f32_to_bf16(Q.fill_normal(cfg.seed, 1, 1.0, m * cfg.n_in).reshape(m, cfg.n_in))
+    y = QL.gemm(cfg.fmt, packed_to_dev(p), bits_to_dev(xbits, "bf16"), n_out, cfg.n_in)
+    cols = np.unique(np.concatenate([np.arange(0, n_out, 13), np.arange(n_out - 130, n_out)]))
+    sub = np.ascontiguousarray(p.reshape(n_out, -1)[cols])
+    what = oracle.dequant(cfg.fmt, sub, cols.size, cfg.n_in)
+    rows = np.arange(0, m, 8)
     want = oracle.linear_f64(what, oracle.bf16_to_f32(xbits[rows]))
     got = oracle.bf16_to_f32(dev_bits(y[torch.from_numpy(rows).to(DEV)][:, torch.from_numpy(cols).to(DEV)]))
     assert rel_l2(got, want) <= TOL
