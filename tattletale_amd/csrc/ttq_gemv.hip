@@ -335,6 +335,8 @@ hipError_t launch_gemv(int format, const void* w, const void* x, int x_dtype, vo
                        const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                        hipStream_t s) {
   if (m == 0 || n_out == 0) return hipSuccess;
+  if (gemv_q4k_batch_supported(format, x_dtype, m, n_out, n_in))
+    return launch_gemv_q4k_batch(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   if (gemv_mfma_supported(format, x_dtype, n_out, n_in))
     return launch_gemv_mfma(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   if (gemv_q8_mfma_supported(format, n_out, n_in))

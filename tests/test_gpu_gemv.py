@@ -20,6 +20,12 @@ TOL = 1e-3
 FMTS = [F.Q8_0, F.Q4_K, F.Q6_K]
 
 
+def gemv_row_by_row(fmt, wd, xd, n_out, n_in):
+    """One call per activation row: the single-row kernels (several rows in one call may take the
+    batched kernel instead)."""
+    return torch.cat([QL.gemv(fmt, wd, xd[r:r + 1], n_out, n_in) for r in range(xd.shape[0])]).cpu().numpy()
+
+
 def make(fmt, n_out, n_in, seed):
     w = Q.fill_normal(seed, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
     p = Q.quantize(fmt, w)
@@ -125,11 +131,12 @@ def test_q4_k_16bit_work_distributions(xk, n_out, n_in):
     x = Q.fill_normal(n_in + 5, 1, 1.0, 2 * n_in).reshape(2, n_in)
     x[1, ::7] *= 37.0       # uneven magnitudes across sub-blocks
     xd, xf = x_to_dev(x, xk)
-    y = QL.gemv(F.Q4_K, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()
-    assert np.all(np.isfinite(y))
+    wd = packed_to_dev(p)
     want = oracle.linear_f64(what, xf)
-    for r in range(2):
-        assert rel_l2(y[r][rows], want[r]) <= TOL
+    for y in (QL.gemv(F.Q4_K, wd, xd, n_out, n_in).cpu().numpy(), gemv_row_by_row(F.Q4_K, wd, xd, n_out, n_in)):
+        assert np.all(np.isfinite(y))
+        for r in range(2):
+            assert rel_l2(y[r][rows], want[r]) <= TOL
 
 
 @pytest.mark.parametrize("xk", ["bf16", "f16"])
@@ -144,12 +151,13 @@ def test_q4_k_unit_vectors_many_rows(xk, n_in):
     for i, c in enumerate(cols):
         x[i, c] = 1.0 if i % 2 == 0 else -0.5
     xd, _ = x_to_dev(x, xk)
-    y = QL.gemv(F.Q4_K, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()
-    for i, c in enumerate(cols):
-        col = what[:, c] * np.float32(1.0 if i % 2 == 0 else -0.5)
-        assert np.array_equal(y[i], col), c
-        nz = col != 0
-        assert np.array_equal(y[i][nz].view(np.uint32), col[nz].view(np.uint32)), c
+    wd = packed_to_dev(p)
+    for y in (QL.gemv(F.Q4_K, wd, xd, n_out, n_in).cpu().numpy(), gemv_row_by_row(F.Q4_K, wd, xd, n_out, n_in)):
+        for i, c in enumerate(cols):
+            col = what[:, c] * np.float32(1.0 if i % 2 == 0 else -0.5)
+            assert np.array_equal(y[i], col), c
+            nz = col != 0
+            assert np.array_equal(y[i][nz].view(np.uint32), col[nz].view(np.uint32)), c
 
 
 def test_q4_k_16bit_activation_extremes():
@@ -164,12 +172,13 @@ def test_q4_k_16bit_activation_extremes():
     x[2, 5] = np.inf
     x[3] = Q.fill_normal(80, 1, 1.0, n_in) * 1e-30
     xd, xf = x_to_dev(x, "bf16")
-    y = QL.gemv(F.Q4_K, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()
+    wd = packed_to_dev(p)
     want = oracle.linear_f64(what, xf[[0, 1, 3]])
-    assert np.array_equal(y[0], np.zeros(n_out, np.float32))
-    assert rel_l2(y[1], want[1]) <= TOL
-    assert not np.any(np.isfinite(y[2]))
-    assert rel_l2(y[3], want[2]) <= TOL
+    for y in (QL.gemv(F.Q4_K, wd, xd, n_out, n_in).cpu().numpy(), gemv_row_by_row(F.Q4_K, wd, xd, n_out, n_in)):
+        assert np.array_equal(y[0], np.zeros(n_out, np.float32))
+        assert rel_l2(y[1], want[1]) <= TOL
+        assert not np.any(np.isfinite(y[2]))
+        assert rel_l2(y[3], want[2]) <= TOL
 
 
 @pytest.mark.parametrize("xk", ["f32", "bf16", "f16"])

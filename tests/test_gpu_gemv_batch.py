@@ -1,0 +1,127 @@
+"""Q4_K decode GEMV for a few activation rows at once (batched decode) against the CPU oracle,
+through the C ABI.
+
+Same bar as the single-row GEMV: relative L2 error <= 1e-3 against the float64 product over
+oracle-dequantized weights; rows that are unit vectors reproduce the dequantized column bit for
+bit.  Every row of a batched call must also agree with the single-row kernel on that row to
+fp32 summation-order noise (both compute the same exact integer sums per sub-block)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from tattletale_amd import QuantLinear, formats as F
+from tattletale_amd import configs as CFG
+from tattletale_amd import qlinear as QL
+from tattletale_amd import quantize as Q
+
+from util import DEV, dev_bits, packed_to_dev, rel_l2, x_to_dev, random_blocks
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+@pytest.mark.parametrize("xk", ["bf16", "f16"])
+@pytest.mark.parametrize("m", [2, 3, 7, 8, 9, 16, 17, 31])
+@pytest.mark.parametrize("n_out,n_in", [(2048, 256), (4096 + 8, 1024), (2500, 4096), (25600, 512), (2304, 8192),
+                                        (5000, 1280)])
+def test_batch_random(xk, m, n_out, n_in):
+    """Row counts around the 8- and 16-token groups, shapes with 1/2/4/16 slices of the
+    super-blocks, several rounds per workgroup, ragged last row groups."""
+    rng = np.random.default_rng(n_out + n_in + m)
+    p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=n_out + m)
+    rows = np.unique(np.concatenate([rng.integers(0, n_out, 300), np.arange(n_out - 40, n_out), np.arange(40)]))
+    what = oracle.dequant(F.Q4_K, np.ascontiguousarray(p.reshape(n_out, -1)[rows]), rows.size, n_in)
+    x = Q.fill_normal(n_in + m, 1, 1.0, m * n_in).reshape(m, n_in)
+    x[m - 1, ::7] *= 37.0            # uneven magnitudes across sub-blocks
+    xd, xf = x_to_dev(x, xk)
+    wd = packed_to_dev(p)
+    y = QL.gemv(F.Q4_K, wd, xd, n_out, n_in)
+    assert y.shape == (m, n_out) and y.dtype == torch.float32
+    y = y.cpu().numpy()
+    assert np.all(np.isfinite(y))
+    want = oracle.linear_f64(what, xf)
+    for r in range(m):
+        assert rel_l2(y[r][rows], want[r]) <= TOL, r
+    # the single-row kernel on three of the rows
+    for r in {0, m // 2, m - 1}:
+        y1 = QL.gemv(F.Q4_K, wd, xd[r:r + 1], n_out, n_in).cpu().numpy()[0]
+        assert rel_l2(y[r], y1) <= 2e-6, r
+
+
+@pytest.mark.parametrize("xk", ["bf16", "f16"])
+@pytest.mark.parametrize("n_in", [1024, 4096, 8192])
+def test_batch_unit_vectors_reproduce_columns_bit_exactly(xk, n_in):
+    n_out = 2100
+    p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=13)
+    what = oracle.dequant(F.Q4_K, p, n_out, n_in)
+    cols = [0, 1, 15, 16, 31, 32, 33, 63, 64, 95, 96, 127, 128, 159, 160, 191, 192, 223, 224, 255, 256, 300,
+            n_in - 129, n_in - 33, n_in - 1]
+    x = np.zeros((len(cols), n_in), np.float32)
+    for i, c in enumerate(cols):
+        x[i, c] = 1.0 if i % 2 == 0 else -0.5
+    xd, _ = x_to_dev(x, xk)
+    y = QL.gemv(F.Q4_K, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()
+    for i, c in enumerate(cols):
+        col = what[:, c] * np.float32(1.0 if i % 2 == 0 else -0.5)
+        assert np.array_equal(y[i], col), c
+        nz = col != 0
+        assert np.array_equal(y[i][nz].view(np.uint32), col[nz].view(np.uint32)), c
+
+
+def test_batch_rows_do_not_leak_into_each_other():
+    """A row of zeros between ordinary rows, a row with an Inf, tiny and huge rows."""
+    n_out, n_in = 2048 + 64, 1024
+    w = Q.fill_normal(77, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
+    p = Q.quantize(F.Q4_K, w)
+    what = oracle.dequant(F.Q4_K, p, n_out, n_in)
+    x = np.zeros((6, n_in), np.float32)
+    x[1] = Q.fill_normal(78, 1, 1e-3, n_in)
+    x[1, 100] = 3.0e4
+    x[2] = Q.fill_normal(79, 1, 1.0, n_in)
+    x[2, 5] = np.inf
+    x[3] = Q.fill_normal(80, 1, 1.0, n_in) * 1e-30
+    x[5] = Q.fill_normal(81, 1, 1.0, n_in)
+    xd, xf = x_to_dev(x, "bf16")
+    y = QL.gemv(F.Q4_K, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()
+    want = oracle.linear_f64(what, xf[[1, 3, 5]])
+    assert np.array_equal(y[0], np.zeros(n_out, np.float32))
+    assert np.array_equal(y[4], np.zeros(n_out, np.float32))
+    assert rel_l2(y[1], want[0]) <= TOL
+    assert not np.any(np.isfinite(y[2]))
+    assert rel_l2(y[3], want[1]) <= TOL
+    assert rel_l2(y[5], want[2]) <= TOL
+
+
+@pytest.mark.parametrize("m", [5, 20, 32])
+def test_forward_few_rows_bias_and_output_types(m):
+    n_out, n_in = 2304, 1024
+    w = Q.fill_normal(500, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
+    p = Q.quantize(F.Q4_K, w)
+    what = oracle.dequant(F.Q4_K, p, n_out, n_in)
+    bias = Q.fill_normal(501, 2, 0.5, n_out)
+    xd, xf = x_to_dev(Q.fill_normal(502, 1, 1.0, m * n_in).reshape(m, n_in), "bf16")
+    bd, bf = x_to_dev(bias, "f32")
+    layer = QuantLinear.init(packed_to_dev(p), F.Q4_K, n_in, n_out, bias=bd)
+    want = oracle.linear_f64(what, xf, bf)
+    y32 = layer.forward(xd, out_dtype=torch.float32)
+    assert rel_l2(y32.cpu().numpy(), want) <= TOL          # decode-class accuracy: not the bf16-weight GEMM
+    y16 = layer.forward(xd)
+    assert y16.dtype == torch.bfloat16
+    assert np.array_equal(dev_bits(y16), oracle.f32_to_bf16(y32.cpu().numpy()))
+    yh = layer.forward(xd, out_dtype=torch.float16)
+    assert rel_l2(yh.float().cpu().numpy(), want) <= 2e-3
+
+
+@pytest.mark.parametrize("m", [4, 16])
+def test_batch_full_shape_14336x4096(m):
+    cfg = CFG.CONFIGS["q4_k_gemv"]
+    p = CFG.packed_weights(cfg)
+    x = Q.fill_normal(cfg.seed, 1, 1.0, m * cfg.n_in).reshape(m, cfg.n_in)
+    xd, xf = x_to_dev(x, "bf16")
+    y = QL.gemv(F.Q4_K, packed_to_dev(p), xd, cfg.n_out, cfg.n_in).cpu().numpy()
+    rows = np.unique(np.concatenate([np.arange(0, cfg.n_out, 11), np.arange(cfg.n_out - 60, cfg.n_out)]))
+    what = oracle.dequant(F.Q4_K, np.ascontiguousarray(p.reshape(cfg.n_out, -1)[rows]), rows.size, cfg.n_in)
+    want = oracle.linear_f64(what, xf)
+    for r in range(m):
+        assert rel_l2(y[r][rows], want[r]) <= TOL
