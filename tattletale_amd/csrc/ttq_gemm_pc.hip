@@ -199,6 +199,7 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
   // request before each W write)
   __shared__ __attribute__((aligned(16))) uint8_t smem[kXRingBytes];
   __shared__ uint4 sw[2 * kWUnits];
+  __shared__ uint32_t pf_sink[4 * 64];   // where the movers' L2 prefetch requests land (never read)
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -242,30 +243,40 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
       const int row = min(m_tile * kPcBM + pc * 64 + rl, m - 1);   // clamped: never stored
       xoff[i] = (uint32_t)row * (uint32_t)(n_in * 2) + (uint32_t)(((lane & 7) ^ key) * 16);
     }
+    // L2 prefetch.  All workgroups of an XCD walk the same slab of X in step, so a line that is
+    // not in their L2 yet is missed by all of them at once and every one waits out the HBM
+    // latency, which is longer than the three stages of lookahead.  Each mover therefore also
+    // touches the line (64 k of one row = 128 bytes) of its consumer's 64 rows kPf steps ahead,
+    // as one 4-byte request per lane into a scratch LDS word: no register, nothing to wait for.
+    constexpr int kPf = 8;
+    const uint8_t* pf_row = xb + (size_t)min(m_tile * kPcBM + pc * 64 + lane, m - 1) * (size_t)(n_in * 2);
     auto dma_step = [&](int ks, int stage) {
       const uint32_t koff = (uint32_t)ks * 128u;
 #pragma unroll
       for (int i = 0; i < 8; i++)
         __builtin_amdgcn_global_load_lds((gptr_t)(xb + (size_t)(xoff[i] + koff)),
                                          (lptr_t)(ring + stage * kXStage + i * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_t)(pf_row + (size_t)min(ks + kPf, ksteps - 1) * 128),
+                                       (lptr_t)(pf_sink + pc * 64), 4, 0, 0);
     };
     // Requests complete in order, so "all but the youngest N have landed" is the only wait there
-    // is.  Iteration s requests step s+3 into the stage that barrier s-1 freed and then makes
-    // sure step s+1 has landed: 16 younger requests (steps s+2, s+3) may stay in flight.
+    // is.  A step is nine requests (eight data, one prefetch).  Iteration s requests step s+3
+    // into the stage that barrier s-1 freed and then makes sure step s+1 has landed: the
+    // prefetch that followed it and steps s+2, s+3 (19 requests) may stay in flight.
     // Nothing is requested past the last step: the consumers reuse their rings in the epilogue.
     dma_step(0, 0);
     dma_step(1, 1);
     dma_step(2, 2);
-    wait_vmcnt<16>();
+    wait_vmcnt<19>();
     lds_barrier();                       // barrier -1
     int st = 3;
     for (int s2 = 0; s2 < ksteps - 3; s2++) {
       dma_step(s2 + 3, st);
       st = (st + 1) & (kXStages - 1);
-      wait_vmcnt<16>();
+      wait_vmcnt<19>();
       lds_barrier();                     // barrier s
     }
-    wait_vmcnt<8>();
+    wait_vmcnt<10>();
     lds_barrier();                       // barrier ksteps-3: step ksteps-2 has landed
     wait_vmcnt<0>();
     lds_barrier();                       // barrier ksteps-2: the last step has landed
