@@ -269,6 +269,48 @@ def main() -> int:
             % (f_ms * 1e3, res["weight_GBps"], u_ms * 1e3, nf_ms * 1e3, nu_ms * 1e3))
         return res
 
+    def run_widened(steps: int, warmup: int):
+        """Rows next to the headline ones, on random packed bytes with finite scale fields (timing
+        only): the few-row decode GEMV (8 and 16 activation rows at once) and the prefill GEMM for
+        Q6_K and Q8_0 weights, all 14336 x 4096."""
+        n_out, n_in = 14336, 4096
+        rng = np.random.default_rng(1234)
+        res = {}
+
+        def random_packed(fmt):
+            nbytes, wpb, scale_hi = {F.Q8_0: (34, 32, [1]), F.Q4_K: (144, 256, [1, 3]), F.Q6_K: (210, 256, [209])}[fmt]
+            raw = rng.integers(0, 256, (n_out * (n_in // wpb), nbytes), dtype=np.uint8)
+            for off in scale_hi:
+                raw[:, off] &= 0x3F            # |fp16 scale| < 2
+            return raw.reshape(-1)
+
+        def timed(name, fmt, m, fn_of):
+            packed = random_packed(fmt)
+            ncopies = max(2, -(-2 * MALL_BYTES // packed.nbytes))
+            ws = [to_dev(packed) for _ in range(ncopies)]
+            x = torch.randn((m, n_in), device=dev).to(torch.bfloat16)
+            step = fn_of(ws, x, ncopies)
+            _, ev_ms = time_steps(step, steps, warmup, use_graph=not args.eager)
+            res[name] = {"us_per_step": ev_ms * 1e3, "weight_GBps": packed.nbytes / (ev_ms * 1e-3) / 1e9,
+                         "TFLOPs": 2.0 * m * n_out * n_in / (ev_ms * 1e-3) / 1e12}
+            log("[%s] %.2f us/step  %.0f GB/s  %.1f TFLOP/s" % (name, ev_ms * 1e3, res[name]["weight_GBps"],
+                                                              res[name]["TFLOPs"]))
+            del ws
+            torch.cuda.empty_cache()
+
+        for m in (8, 16):
+            y = torch.empty((m, n_out), dtype=torch.float32, device=dev)
+            timed("q4_k_gemv_m%d" % m, F.Q4_K, m,
+                  lambda ws, x, nc, y=y: (lambda i: QL.gemv(F.Q4_K, ws[i % nc], x, n_out, n_in, out=y)))
+        for fmt, nm in ((F.Q6_K, "q6_k_gemm_m512"), (F.Q8_0, "q8_0_gemm_m512")):
+            y = torch.empty((512, n_out), dtype=torch.bfloat16, device=dev)
+            timed(nm, fmt, 512,
+                  lambda ws, x, nc, y=y, fmt=fmt: (lambda i: QL.gemm(fmt, ws[i % nc], x, n_out, n_in, out=y)))
+        return res
+
+    if args.only == "widened":
+        print(json.dumps(run_widened(max(20, args.steps // 4), max(3, args.warmup // 4))), flush=True)
+        return 0
     if args.only == "q4_k_gate_up_silu_gemv":
         print(json.dumps(run_gate_up(max(20, args.steps // 4), max(3, args.warmup // 4))), flush=True)
         return 0
@@ -326,6 +368,7 @@ def main() -> int:
     line["extra"] = {k: v for k, v in results.items() if k != names[0]}
     if not args.only and not args.no_extra:
         line["extra"]["q4_k_gate_up_silu_gemv"] = run_gate_up(max(20, args.steps // 4), max(3, args.warmup // 4))
+        line["extra"]["widened"] = run_widened(max(20, args.steps // 4), max(3, args.warmup // 4))
     print(json.dumps(line), flush=True)
     return 0
 
