@@ -98,54 +98,92 @@ __global__ void __launch_bounds__(256) dequant_exl3_kernel(const uint16_t* __res
 constexpr int kExl3Threads = 1024;
 constexpr int kExl3Waves = kExl3Threads / kWave;
 
-// In-LDS orthonormal FWHT of every 128-group of xs[0..n), all threads of the block.
-__device__ __forceinline__ void fwht128_lds(float* xs, int n, int tid, int nthreads) {
-  for (int len = 1; len < 128; len <<= 1) {
-    __syncthreads();
-    for (int p = tid; p < n / 2; p += nthreads) {
-      // pair p of its stage: insert a zero bit at position log2(len)
-      const int lo = p & (len - 1);
-      const int i = ((p - lo) << 1) | lo;
-      const float a = xs[i], b = xs[i + len];
-      xs[i] = a + b;
-      xs[i + len] = a - b;
+// Unnormalized FWHT of a 128-group held as 4 consecutive values in each of 32 consecutive lanes
+// (value index = 4*lane + i): stages 1 and 2 inside the lane, stages 4..64 against the lane
+// 1, 2, 4, 8, 16 away.  Same stage order and operand order as the textbook loop
+// (lower index gets a+b, upper a-b), so the results do not depend on how it is laid out.
+__device__ __forceinline__ void fwht128_quad(float (&v)[4], int lane) {
+  float t;
+  t = v[0]; v[0] = t + v[1]; v[1] = t - v[1];
+  t = v[2]; v[2] = t + v[3]; v[3] = t - v[3];
+  t = v[0]; v[0] = t + v[2]; v[2] = t - v[2];
+  t = v[1]; v[1] = t + v[3]; v[3] = t - v[3];
+#pragma unroll
+  for (int d = 1; d < 32; d <<= 1) {
+    const bool upper = (lane & d) != 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const float o = __shfl_xor(v[i], d, kWave);
+      v[i] = upper ? (o - v[i]) : (v[i] + o);
     }
   }
-  __syncthreads();
 }
 
 // One workgroup per n_tile (16 output channels).  Lane = (k-tile slot g = lane/16, channel
 // j = lane%16); the 16 waves times 4 slots walk the k tiles 64 at a time.  Partial sums are
 // combined across slots with lane shuffles and across waves through LDS.
+// The packed bits of a lane's first kPre tiles are requested before anything else, so that they
+// travel while the activations are loaded and rotated; later tiles are requested one batch ahead.
 template <int BITS, int CB, typename XT>
 __global__ void __launch_bounds__(kExl3Threads)
 gemv_exl3_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __restrict__ suh,
                  const XT* __restrict__ x, float* __restrict__ y, int n_out, int n_in) {
   extern __shared__ float xs[];          // n_in rotated activations, then kExl3Waves*16 partials
+  constexpr int kPre = 4;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const XT* xm = x + (int64_t)blockIdx.y * n_in;
   float* ym = y + (int64_t)blockIdx.y * n_out;
-  for (int k = tid; k < n_in; k += kExl3Threads)
-    xs[k] = XElem<XT>::load(xm, k) * f16_bits_to_f32(suh[k]);
-  fwht128_lds(xs, n_in, tid, kExl3Threads);
-  const float kNorm = 0.08838834764831845f;  // 1/sqrt(128), applied to the dot product
-
   const int nt = blockIdx.x, nt_n = n_out >> 4, kt_n = n_in >> 4;
   const int g = lane >> 4, j = lane & 15;
-  float acc = 0.f;
-  for (int kt = wave * 4 + g; kt < kt_n; kt += kExl3Waves * 4) {
-    LaneBits<BITS> lb;
-    lb.load(trellis + ((int64_t)kt * nt_n + nt) * (16 * BITS), j);
-    _Float16 v[16];
-    DecodeLoop<BITS, CB, 0>::run(lb, v);
-    const float4* xv = reinterpret_cast<const float4*>(xs + 16 * kt);
+  const int kt0 = wave * 4 + g;
+  constexpr int kStride = kExl3Waves * 4;
+
+  LaneBits<BITS> cur[kPre];
+  auto load_batch = [&](LaneBits<BITS> (&dst)[kPre], int kt_first) {
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-      const float4 xq = xv[q];
-      acc = fmaf_((float)v[4 * q + 0], xq.x, acc);
-      acc = fmaf_((float)v[4 * q + 1], xq.y, acc);
-      acc = fmaf_((float)v[4 * q + 2], xq.z, acc);
-      acc = fmaf_((float)v[4 * q + 3], xq.w, acc);
+    for (int i = 0; i < kPre; i++) {
+      const int kt = min(kt_first + i * kStride, kt_n - 1);     // past the end: a harmless re-read
+      dst[i].load(trellis + ((int64_t)kt * nt_n + nt) * (16 * BITS), j);
+    }
+  };
+  load_batch(cur, kt0);
+
+  // input side: x o suh, then the Hadamard rotation of every group of 128 (32 lanes x 4 values)
+  for (int k4 = tid * 4; k4 < n_in; k4 += kExl3Threads * 4) {
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) v[i] = XElem<XT>::load(xm, k4 + i) * f16_bits_to_f32(suh[k4 + i]);
+    fwht128_quad(v, lane);
+    *reinterpret_cast<float4*>(xs + k4) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+  __syncthreads();
+  const float kNorm = 0.08838834764831845f;  // 1/sqrt(128), applied to the dot product
+
+  float acc = 0.f;
+  for (int ktb = kt0; ktb < kt_n; ktb += kPre * kStride) {
+    LaneBits<BITS> nxt[kPre];
+    const bool more = ktb + kPre * kStride < kt_n;
+    if (more) load_batch(nxt, ktb + kPre * kStride);
+#pragma unroll
+    for (int i = 0; i < kPre; i++) {
+      const int kt = ktb + i * kStride;
+      if (kt < kt_n) {
+        _Float16 v[16];
+        DecodeLoop<BITS, CB, 0>::run(cur[i], v);
+        const float4* xv = reinterpret_cast<const float4*>(xs + 16 * kt);
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const float4 xq = xv[q];
+          acc = fmaf_((float)v[4 * q + 0], xq.x, acc);
+          acc = fmaf_((float)v[4 * q + 1], xq.y, acc);
+          acc = fmaf_((float)v[4 * q + 2], xq.z, acc);
+          acc = fmaf_((float)v[4 * q + 3], xq.w, acc);
+        }
+      }
+    }
+    if (more) {
+#pragma unroll
+      for (int i = 0; i < kPre; i++) cur[i] = nxt[i];
     }
   }
   acc += __shfl_xor(acc, 16, kWave);
@@ -162,35 +200,52 @@ gemv_exl3_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __restric
 }
 
 // ------------------------------------------------------------------ Hadamard epilogue
-// One workgroup of 128 threads per 128-group: v <- post o H(pre o v) (+ bias), in place.
-// `period` is the length after which pre/post/bias repeat (n_out for batched outputs).
-__global__ void __launch_bounds__(128)
+// One wavefront per 128-group: v <- post o H(pre o v) (+ bias), in place.  Lane l holds elements
+// l and l + 64: stages 1..32 against the lanes 1..32 away, stage 64 inside the lane (the stage
+// order of the textbook loop).  `period` is the length after which pre/post/bias repeat (n_out
+// for batched outputs).
+constexpr int kHadThreads = 256;
+__global__ void __launch_bounds__(kHadThreads)
 hadamard128_kernel(float* __restrict__ v, const uint16_t* __restrict__ pre,
                    const uint16_t* __restrict__ post, const void* __restrict__ bias, int bias_dtype,
-                   int64_t period) {
-  __shared__ float s[128];
-  const int t = threadIdx.x;
-  const int64_t idx = (int64_t)blockIdx.x * 128 + t;
-  const int64_t ch = idx % period;
-  float a = v[idx];
-  if (pre) a *= f16_bits_to_f32(pre[ch]);
-  s[t] = a;
-  for (int len = 1; len < 128; len <<= 1) {
-    __syncthreads();
-    const float mine = s[t], other = s[t ^ len];
-    __syncthreads();
-    s[t] = (t & len) ? (other - mine) : (mine + other);
+                   int64_t period, int64_t groups) {
+  const int lane = threadIdx.x & 63;
+  const int64_t grp = (int64_t)blockIdx.x * (kHadThreads / kWave) + (threadIdx.x >> 6);
+  if (grp >= groups) return;
+  float a[2];
+  int64_t ch[2];
+#pragma unroll
+  for (int h = 0; h < 2; h++) {
+    const int64_t idx = grp * 128 + lane + 64 * h;
+    ch[h] = idx % period;
+    a[h] = v[idx];
+    if (pre) a[h] *= f16_bits_to_f32(pre[ch[h]]);
   }
-  float r = s[t] * 0.08838834764831845f;
-  if (post) r *= f16_bits_to_f32(post[ch]);
-  if (bias) {
-    if (bias_dtype == kF32) r += static_cast<const float*>(bias)[ch];
-    else {
-      const uint16_t b = static_cast<const uint16_t*>(bias)[ch];
-      r += (bias_dtype == kF16) ? f16_bits_to_f32(b) : bf16_bits_to_f32(b);
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const bool upper = (lane & d) != 0;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      const float o = __shfl_xor(a[h], d, kWave);
+      a[h] = upper ? (o - a[h]) : (a[h] + o);
     }
   }
-  v[idx] = r;
+  const float lo = a[0] + a[1], hi = a[0] - a[1];
+  a[0] = lo;
+  a[1] = hi;
+#pragma unroll
+  for (int h = 0; h < 2; h++) {
+    float r = a[h] * 0.08838834764831845f;
+    if (post) r *= f16_bits_to_f32(post[ch[h]]);
+    if (bias) {
+      if (bias_dtype == kF32) r += static_cast<const float*>(bias)[ch[h]];
+      else {
+        const uint16_t b = static_cast<const uint16_t*>(bias)[ch[h]];
+        r += (bias_dtype == kF16) ? f16_bits_to_f32(b) : bf16_bits_to_f32(b);
+      }
+    }
+    v[grp * 128 + lane + 64 * h] = r;
+  }
 }
 
 // ------------------------------------------------------------------ launchers
@@ -275,16 +330,19 @@ hipError_t launch_gemv_exl3(const uint16_t* trellis, const uint16_t* suh, const 
   }
   if (e != hipSuccess) return e;
   const int64_t groups = m * n_out / 128;
-  hipLaunchKernelGGL(hadamard128_kernel, dim3((unsigned)groups), dim3(128), 0, s, yf,
-                     (const uint16_t*)nullptr, svh, bias, bias_dtype, n_out);
+  constexpr int kPerBlock = kHadThreads / kWave;
+  hipLaunchKernelGGL(hadamard128_kernel, dim3((unsigned)((groups + kPerBlock - 1) / kPerBlock)), dim3(kHadThreads), 0,
+                     s, yf, (const uint16_t*)nullptr, svh, bias, bias_dtype, n_out, groups);
   return hipGetLastError();
 }
 
 hipError_t launch_hadamard128(float* v, const uint16_t* pre, const uint16_t* post, int64_t n,
                               hipStream_t s) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(hadamard128_kernel, dim3((unsigned)(n / 128)), dim3(128), 0, s, v, pre, post,
-                     (const void*)nullptr, 0, n);
+  constexpr int kPerBlock = kHadThreads / kWave;
+  const int64_t groups = n / 128;
+  hipLaunchKernelGGL(hadamard128_kernel, dim3((unsigned)((groups + kPerBlock - 1) / kPerBlock)), dim3(kHadThreads), 0,
+                     s, v, pre, post, (const void*)nullptr, 0, n, groups);
   return hipGetLastError();
 }
 
