@@ -17,8 +17,9 @@
 // reads its table entry or one shared zero entry).  Eight (sixteen) MFMAs per super-block of 16
 // weight rows.  Lane (n = lane%16, g = lane/16) loads 16 qs bytes of weight row n, supplies
 // them as B and receives C rows 4g..4g+3 of column n: everything of tokens 2g, 2g+1 (TOK = 8)
-// or the plane sums of tokens 4g..4g+3 (TOK = 16) for its own weight row, whose scales it
-// decodes from the header it loaded itself.  No cross-lane traffic at all.
+// or the plane sums of tokens 4g..4g+3 (TOK = 16) for its own weight row.  The vector ALU is
+// the bottleneck of this kernel, so the sub-block scales are decoded once per row (two per lane)
+// and spread over the row's four lanes, and the min term is summed, by fp32 matrix instructions.
 //
 // Work distribution as in ttq_gemv_mfma.hip, two steps in flight per wavefront; blockIdx.y walks
 // the groups of TOK tokens.
@@ -27,6 +28,7 @@
 namespace ttq {
 
 struct BatchStep { uint4 hdr, c0, c1; };
+typedef float v4f_t __attribute__((ext_vector_type(4)));
 
 // LDS (bytes): plane table [nsb*8 sub-blocks][TOK/8 planes-in-own-slab][16 rows][2 halves] x 16,
 // one zero entry (64 bytes reserved), then f = 2^(E-13) and sum(x) per (sub-block, token) as two
@@ -79,8 +81,9 @@ gemv_q4k_batch_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
   __builtin_amdgcn_s_barrier();
 
   // ---- weight stream; loads are unconditional (clamped)
-  // two steps in flight per wavefront: a step of this kernel keeps the vector ALU busy for long
-  // enough that the next one has to be on its way meanwhile
+  // Two steps in flight per wavefront: a step keeps the wavefront busy for long enough that the
+  // next one has to be on its way meanwhile.  (Four, i.e. nearly the whole share of a workgroup
+  // requested before the activations are staged, measured slower.)
   constexpr int R = 2;
   BatchStep ring[R];
   int ir = 0, isi = 0;
@@ -157,10 +160,28 @@ gemv_q4k_batch_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
   // A operand of this lane (row = lane%16, k-group ga = lane/16): its entry inside a sub-block
   const uint32_t act_off = (uint32_t)((lane & 15) * 2 + (g & 1)) * 16u;
   const bool upper_half = (g >> 1) != 0;         // k-groups 2, 3 carry sub-blocks 2, 3 (6, 7)
+  // The fp32 matrix instruction v_mfma_f32_16x16x4_f32 does two side jobs per step (A operand:
+  // lane (i = lane%16, kk = lane/16) supplies A[i][kk]; B operand: lane (n, kk) supplies B[kk][n]):
+  //  * all-gather of the sub-block scales: every lane decodes d*sc of sub-blocks g and 4+g of its
+  //    own row; with A[i][kk] = (kk == i%4) the product hands lane (n, g) the values of lanes
+  //    (n, 0..3) in its four C registers (1.0 * value + zeros: exact);
+  //  * the min term sum_j dmin*m_j * sum(x) of sub-block j: A[i][kk] = sum(x) of the token that C
+  //    row i belongs to (sub-block kk, then 4+kk), B[kk][n] = dmin*m of sub-block kk of row n,
+  //    accumulated over the whole round in fp32.
+  const float sel = ((lane >> 4) == (lane & 3)) ? 1.f : 0.f;
+  // token of C row i = lane%16 (TOK = 8: rows 4g', 4g'+1 are tokens 2g', 2g'+1, the others unused)
+  const int mrow = lane & 15;
+  const bool row_used = TOK == 16 || (mrow & 3) < 2;
+  const int row_tok = TOK == 16 ? mrow : 2 * (mrow >> 2) + (mrow & 3);
+  // byte offset of ts[(sb*8 + kk) * TOK + token] relative to ts + sb*8*TOK (unused rows: zero entry)
+  const uint32_t ts_base = (uint32_t)(reinterpret_cast<uint8_t*>(ts) - smem);
+  const uint32_t ts_lane = row_used ? ts_base + (uint32_t)(g * TOK + row_tok) * 4u : zero_off;
+  const uint32_t ts_step = row_used ? (uint32_t)(8 * TOK * 4) : 0u;
   int cr = 0, csi = 0;
   float acc[TPL];
 #pragma unroll
   for (int i = 0; i < TPL; i++) acc[i] = 0.f;
+  v4f_t cmin = {0.f, 0.f, 0.f, 0.f};
 
   auto store_row = [&](int row, int tk, float v) {
     if (row < wg_row_end && t0 + tk < m)
@@ -181,43 +202,75 @@ gemv_q4k_batch_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
       }
       const float d = f16_bits_to_f32((uint16_t)(s.hdr.x & 0xFFFFu));
       const float dmin = f16_bits_to_f32((uint16_t)(s.hdr.x >> 16));
+      // scales and mins of sub-blocks g and 4+g of this lane's row (the 6-bit fields of
+      // q4k_scale_min with a run-time sub-block)
+      const uint32_t sh = 8u * (uint32_t)g;
+      const uint32_t sc_lo = (s.hdr.y >> sh) & 63u, mn_lo = (s.hdr.z >> sh) & 63u;
+      const uint32_t sc_hi = ((s.hdr.w >> sh) & 0xFu) | (((s.hdr.y >> (sh + 6u)) & 3u) << 4);
+      const uint32_t mn_hi = ((s.hdr.w >> (sh + 4u)) & 0xFu) | (((s.hdr.z >> (sh + 6u)) & 3u) << 4);
+      const v4f_t fzero = {0.f, 0.f, 0.f, 0.f};
+      const v4f_t dsc03 = __builtin_amdgcn_mfma_f32_16x16x4f32(sel, d * (float)sc_lo, fzero, 0, 0, 0);
+      const v4f_t dsc47 = __builtin_amdgcn_mfma_f32_16x16x4f32(sel, d * (float)sc_hi, fzero, 0, 0, 0);
+      {
+        const uint32_t ta = ts_lane + (uint32_t)sb * ts_step;
+        const float s_lo = *reinterpret_cast<const float*>(smem + ta);
+        const float s_hi = *reinterpret_cast<const float*>(smem + ta + (row_used ? (uint32_t)(4 * TOK * 4) : 0u));
+        cmin = __builtin_amdgcn_mfma_f32_16x16x4f32(s_lo, dmin * (float)mn_lo, cmin, 0, 0, 0);
+        cmin = __builtin_amdgcn_mfma_f32_16x16x4f32(s_hi, dmin * (float)mn_hi, cmin, 0, 0, 0);
+      }
       const v4i_t zero = {0, 0, 0, 0};
+      // Sub-block j: nibble plane j%2 of qs bytes 64*(j/4) + 32*((j%4)/2) .. +32, i.e. B operand
+      // 2*(j/4) + j%2, k-groups 2*((j%4)/2) and +1.  The sub-blocks are taken kGroup at a time:
+      // all LDS reads of a group, then its MFMAs back to back, then the scaling -- left alone the
+      // compiler issues read, wait, MFMA, wait, scale for one sub-block after the other and the
+      // wavefront sits out every latency eight times per step.
+      constexpr int kGroup = TOK == 8 ? 4 : 2;
 #pragma unroll
-      for (int j = 0; j < 8; j++) {
-        // sub-block j: nibble plane j%2 of qs bytes 64*(j/4) + 32*((j%4)/2) .. +32, i.e. B operand
-        // 2*(j/4) + j%2, k-groups 2*((j%4)/2) and +1
-        uint32_t sc, mn;
-        q4k_scale_min(s.hdr.y, s.hdr.z, s.hdr.w, j, sc, mn);
-        const float dsc = d * (float)sc, dm = dmin * (float)mn;
-        const bool mine = (((j & 3) >> 1) != 0) == upper_half;
-        const uint32_t sbg = (uint32_t)sb * 8u + j;
-        const uint32_t a_addr = mine ? sbg * kSubBytes + act_off : zero_off;
-        const v4i_t& B = Bq[2 * (j >> 2) + (j & 1)];
-        if (TOK == 8) {
-          const v4i_t a = *reinterpret_cast<const v4i_t*>(smem + a_addr);
-          const v4i_t C = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, B, zero, 0, 0, 0);
-          const float2 f2 = *reinterpret_cast<const float2*>(tf + sbg * TOK + 2 * g);
-          const float2 s2 = *reinterpret_cast<const float2*>(ts + sbg * TOK + 2 * g);
+      for (int j0 = 0; j0 < 8; j0 += kGroup) {
+        v4i_t A[kGroup][TOK / 8];
+        float ff[kGroup][TPL];
+#pragma unroll
+        for (int jj = 0; jj < kGroup; jj++) {
+          const int j = j0 + jj;
+          const bool mine = (((j & 3) >> 1) != 0) == upper_half;
+          const uint32_t sbg = (uint32_t)sb * 8u + j;
+          const uint32_t a_addr = mine ? sbg * kSubBytes + act_off : zero_off;
+          A[jj][0] = *reinterpret_cast<const v4i_t*>(smem + a_addr);
+          if (TOK == 16) A[jj][TOK / 8 - 1] = *reinterpret_cast<const v4i_t*>(smem + a_addr + (mine ? 512u : 0u));
+          if (TOK == 8) {
+            const float2 f2 = *reinterpret_cast<const float2*>(tf + sbg * TOK + 2 * g);
+            ff[jj][0] = f2.x; ff[jj][TPL - 1] = f2.y;
+          } else {
+            const float4 f4 = *reinterpret_cast<const float4*>(tf + sbg * TOK + 4 * g);
+            ff[jj][0] = f4.x; ff[jj][1] = f4.y; ff[jj][TPL - 2] = f4.z; ff[jj][TPL - 1] = f4.w;
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        v4i_t C[kGroup][TOK / 8];
+#pragma unroll
+        for (int jj = 0; jj < kGroup; jj++) {
+          const int j = j0 + jj;
+          const v4i_t& B = Bq[2 * (j >> 2) + (j & 1)];
+#pragma unroll
+          for (int pl = 0; pl < TOK / 8; pl++) C[jj][pl] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[jj][pl], B, zero, 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int jj = 0; jj < kGroup; jj++) {
+          const int j = j0 + jj;
+          const float dsc = j < 4 ? dsc03[j & 3] : dsc47[j & 3];
           // exact integers below 2^24, scaled by a power of two: sum(q*x) of the sub-block
-          const float q0 = (float)(C[0] * 256 + C[1]) * f2.x;
-          const float q1 = (float)(C[2] * 256 + C[3]) * f2.y;
-          acc[0] = acc[0] + dsc * q0;
-          acc[0] = acc[0] - dm * s2.x;
-          acc[1] = acc[1] + dsc * q1;
-          acc[1] = acc[1] - dm * s2.y;
-        } else {
-          const v4i_t ah = *reinterpret_cast<const v4i_t*>(smem + a_addr);
-          const v4i_t al = *reinterpret_cast<const v4i_t*>(smem + a_addr + (mine ? 512u : 0u));
-          const v4i_t Ch = __builtin_amdgcn_mfma_i32_16x16x64_i8(ah, B, zero, 0, 0, 0);
-          const v4i_t Cl = __builtin_amdgcn_mfma_i32_16x16x64_i8(al, B, zero, 0, 0, 0);
-          const float4 f4 = *reinterpret_cast<const float4*>(tf + sbg * TOK + 4 * g);
-          const float4 s4 = *reinterpret_cast<const float4*>(ts + sbg * TOK + 4 * g);
-          const float ff[4] = {f4.x, f4.y, f4.z, f4.w}, ss[4] = {s4.x, s4.y, s4.z, s4.w};
+          if (TOK == 8) {
+            const float q0 = (float)(C[jj][0][0] * 256 + C[jj][0][1]) * ff[jj][0];
+            const float q1 = (float)(C[jj][0][2] * 256 + C[jj][0][3]) * ff[jj][TPL - 1];
+            acc[0] = acc[0] + dsc * q0;
+            acc[TPL - 1] = acc[TPL - 1] + dsc * q1;
+          } else {
 #pragma unroll
-          for (int i = 0; i < 4; i++) {
-            const float q = (float)(Ch[i] * 256 + Cl[i]) * ff[i];
-            acc[i] = acc[i] + dsc * q;
-            acc[i] = acc[i] - dm * ss[i];
+            for (int i = 0; i < TPL; i++) {
+              const float q = (float)(C[jj][0][i] * 256 + C[jj][TOK / 8 - 1][i]) * ff[jj][i];
+              acc[i] = acc[i] + dsc * q;
+            }
           }
         }
       }
@@ -228,10 +281,11 @@ gemv_q4k_batch_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
         if (cr < rounds) {
           const int row = wg_row0 + (cr * G + gi) * 16 + n;
 #pragma unroll
-          for (int i = 0; i < TPL; i++) store_row(row, TPL * g + i, acc[i]);
+          for (int i = 0; i < TPL; i++) store_row(row, TPL * g + i, acc[i] - cmin[i]);
         }
 #pragma unroll
         for (int i = 0; i < TPL; i++) acc[i] = 0.f;
+        cmin = v4f_t{0.f, 0.f, 0.f, 0.f};
       }
       // with slices there is one round only: the sums stay in registers until the table is free
       csi = 0;
@@ -254,7 +308,7 @@ gemv_q4k_batch_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
   if (sl_log2 != 0) {
     __syncthreads();                   // every wavefront is done with the plane table
 #pragma unroll
-    for (int i = 0; i < TPL; i++) part[(wave * 64 + lane) * TPL + i] = acc[i];
+    for (int i = 0; i < TPL; i++) part[(wave * 64 + lane) * TPL + i] = acc[i] - cmin[i];
     __syncthreads();
     // add the slices in a fixed order
     for (int idx = tid; idx < 16 * G * TOK; idx += kMfmaThreads) {
