@@ -29,10 +29,11 @@
 namespace ttq {
 
 constexpr int kPcThreads = 768;          // 4 consumers, 4 W producers, 4 X movers
-constexpr int kPcBM = 256;               // rows of X per workgroup (4 consumer wavefronts x 64)
-constexpr int kXStage = 64 * 128;        // bytes: one consumer's 64 rows x 64 k of bf16
+// MB = blocks of 16 rows per consumer wavefront: 4 (a 256-row tile of X per workgroup) for prefill,
+// 1 (64 rows) when the whole activation has no more rows than that.
 constexpr int kXStages = 4;
-constexpr int kXRingBytes = 4 * kXStages * kXStage;
+constexpr int pc_bm(int mb) { return 64 * mb; }            // rows of X per workgroup
+constexpr int pc_xstage(int mb) { return 16 * mb * 128; }  // bytes: one consumer's rows x 64 k of bf16
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
@@ -187,13 +188,15 @@ template <> struct WFmt<kQ8_0> {
 
 // W tile in LDS: [ksub 2][j NJ][g 4][n 16] units of 16 bytes (8 consecutive k of one column),
 // i.e. exactly the B operand of lane g*16+n for column block j.
-template <int NJ, int FMT>
+template <int NJ, int FMT, int MB>
 __global__ void __launch_bounds__(kPcThreads)
 gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, void* __restrict__ yv,
                    int y_dtype, const void* __restrict__ bias, int bias_dtype, int m, int n_out, int n_in,
                    int n_tiles, int m_tiles, int xcds_per_mtile) {
   constexpr int BN = NJ * 16;
   constexpr int kWUnits = 2 * NJ * 64;
+  constexpr int kPcBM = pc_bm(MB), kXStage = pc_xstage(MB), kXRingBytes = 4 * kXStages * kXStage;
+  constexpr int kDma = 2 * MB;           // 8-row DMA requests per consumer and step
   // two separate arrays, so that the compiler can tell LDS writes to the W tile from the
   // asynchronous global_load_lds writes into the X ring (otherwise it drains every outstanding
   // request before each W write)
@@ -235,12 +238,12 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
     const int pc = wave - 8;
     const uint8_t* xb = reinterpret_cast<const uint8_t*>(x);
     uint8_t* ring = smem + pc * (kXStages * kXStage);
-    uint32_t xoff[8];
+    uint32_t xoff[kDma];
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
+    for (int i = 0; i < kDma; i++) {
       const int rl = 8 * i + (lane >> 3);
       const int key = rl & 7;
-      const int row = min(m_tile * kPcBM + pc * 64 + rl, m - 1);   // clamped: never stored
+      const int row = min(m_tile * kPcBM + pc * (16 * MB) + rl, m - 1);   // clamped: never stored
       xoff[i] = (uint32_t)row * (uint32_t)(n_in * 2) + (uint32_t)(((lane & 7) ^ key) * 16);
     }
     // L2 prefetch.  All workgroups of an XCD walk the same slab of X in step, so a line that is
@@ -249,34 +252,35 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
     // touches the line (64 k of one row = 128 bytes) of its consumer's 64 rows kPf steps ahead,
     // as one 4-byte request per lane into a scratch LDS word: no register, nothing to wait for.
     constexpr int kPf = 8;
-    const uint8_t* pf_row = xb + (size_t)min(m_tile * kPcBM + pc * 64 + lane, m - 1) * (size_t)(n_in * 2);
+    const uint8_t* pf_row =
+        xb + (size_t)min(m_tile * kPcBM + pc * (16 * MB) + (lane & (16 * MB - 1)), m - 1) * (size_t)(n_in * 2);
     auto dma_step = [&](int ks, int stage) {
       const uint32_t koff = (uint32_t)ks * 128u;
 #pragma unroll
-      for (int i = 0; i < 8; i++)
+      for (int i = 0; i < kDma; i++)
         __builtin_amdgcn_global_load_lds((gptr_t)(xb + (size_t)(xoff[i] + koff)),
                                          (lptr_t)(ring + stage * kXStage + i * 1024), 16, 0, 0);
       __builtin_amdgcn_global_load_lds((gptr_t)(pf_row + (size_t)min(ks + kPf, ksteps - 1) * 128),
                                        (lptr_t)(pf_sink + pc * 64), 4, 0, 0);
     };
     // Requests complete in order, so "all but the youngest N have landed" is the only wait there
-    // is.  A step is nine requests (eight data, one prefetch).  Iteration s requests step s+3
+    // is.  A step is kDma data requests and one prefetch.  Iteration s requests step s+3
     // into the stage that barrier s-1 freed and then makes sure step s+1 has landed: the
-    // prefetch that followed it and steps s+2, s+3 (19 requests) may stay in flight.
+    // prefetch that followed it and steps s+2, s+3 (2 * (kDma + 1) + 1 requests) may stay in flight.
     // Nothing is requested past the last step: the consumers reuse their rings in the epilogue.
     dma_step(0, 0);
     dma_step(1, 1);
     dma_step(2, 2);
-    wait_vmcnt<19>();
+    wait_vmcnt<2 * (kDma + 1) + 1>();
     lds_barrier();                       // barrier -1
     int st = 3;
     for (int s2 = 0; s2 < ksteps - 3; s2++) {
       dma_step(s2 + 3, st);
       st = (st + 1) & (kXStages - 1);
-      wait_vmcnt<19>();
+      wait_vmcnt<2 * (kDma + 1) + 1>();
       lds_barrier();                     // barrier s
     }
-    wait_vmcnt<10>();
+    wait_vmcnt<kDma + 2>();
     lds_barrier();                       // barrier ksteps-3: step ksteps-2 has landed
     wait_vmcnt<0>();
     lds_barrier();                       // barrier ksteps-2: the last step has landed
@@ -346,7 +350,7 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
   }
 
   // -------------------------------------------------------------------- consumer
-  const int m0 = m_tile * kPcBM + wave * 64;
+  const int m0 = m_tile * kPcBM + wave * (16 * MB);
   const uint8_t* myx = smem + wave * (kXStages * kXStage);
   const int fr = lane & 15, fg = lane >> 4;
   // A fragments: row 16*ib + fr, chunk 4*half + fg, stored at position chunk ^ key(row)
@@ -358,21 +362,21 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
   // pins that order: left alone the compiler sinks every read to just before its use and the
   // wavefront then waits out the LDS latency fourteen times per step.
   constexpr int G = 2 * NJ;
-  uint4 afr[2][4];                      // A fragments of half 0 / half 1
+  uint4 afr[2][MB];                     // A fragments of half 0 / half 1
   bf16x8_t bring[4];
-  auto read_a = [&](uint4 (&dst)[4], int stage, int half) {
+  auto read_a = [&](uint4 (&dst)[MB], int stage, int half) {
     const uint8_t* xbase = myx + stage * kXStage + apos[half];
 #pragma unroll
-    for (int ib = 0; ib < 4; ib++) dst[ib] = *reinterpret_cast<const uint4*>(xbase + ib * 2048);
+    for (int ib = 0; ib < MB; ib++) dst[ib] = *reinterpret_cast<const uint4*>(xbase + ib * 2048);
   };
   auto read_b = [&](bf16x8_t& dst, int buf, int g) {   // g = half * NJ + j
     const uint4 v = sw[buf * kWUnits + g * 64 + lane];
     __builtin_memcpy(&dst, &v, 16);
   };
 
-  f32x4_t acc[4][NJ];
+  f32x4_t acc[MB][NJ];
 #pragma unroll
-  for (int i = 0; i < 4; i++)
+  for (int i = 0; i < MB; i++)
 #pragma unroll
     for (int j = 0; j < NJ; j++) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
@@ -393,7 +397,7 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
       __builtin_amdgcn_sched_barrier(0);
       const int half = g / NJ, j = g % NJ;
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
+      for (int i = 0; i < MB; i++) {
         bf16x8_t a;
         __builtin_memcpy(&a, &afr[half][i], 16);
         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bring[(g + SO) & 3], acc[i][j], 0, 0, 0);
@@ -429,7 +433,7 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
     for (int j = 0; j < NJ; j++) {
       const float bv = load_bias(bias, bias_dtype, n0 + 16 * j + cn);
 #pragma unroll
-      for (int i = 0; i < 4; i++)
+      for (int i = 0; i < MB; i++)
 #pragma unroll
         for (int r = 0; r < 4; r++)
           *reinterpret_cast<uint16_t*>(stg + (16 * i + rb4 + r) * kRowBytes + (16 * j + cn) * 2) =
@@ -438,10 +442,12 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
     // same wavefront wrote and reads: LDS keeps program order, no barrier needed
     uint8_t* yb = static_cast<uint8_t*>(yv);
     constexpr int kChunks = BN / 8;      // 16-byte chunks per row
+    constexpr int kSlots = 16 * MB * kChunks;
 #pragma unroll
-    for (int t = 0; t < kChunks; t++) {
+    for (int t = 0; t < (kSlots + 63) / 64; t++) {
       const int c = t * 64 + lane;
       const int row = c / kChunks, ch = c - row * kChunks;
+      if (c >= kSlots) break;
       const uint4 v = *reinterpret_cast<const uint4*>(stg + row * kRowBytes + ch * 16);
       if (m0 + row < m)
         *reinterpret_cast<uint4*>(yb + ((int64_t)(m0 + row) * n_out + n0 + ch * 8) * 2) = v;
@@ -454,7 +460,7 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
     if (n >= n_out) continue;
     const float bv = load_bias(bias, bias_dtype, n);
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < MB; i++) {
 #pragma unroll
       for (int r = 0; r < 4; r++) {
         const int mm = m0 + 16 * i + rb4 + r;
@@ -468,20 +474,30 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
   }
 }
 
-template <int FMT>
+template <int FMT, int MB>
 static hipError_t launch_pc_112(const uint8_t* wb, const uint16_t* x, void* y, int y_dtype, const void* bias,
                                 int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
-  constexpr int NJ = 7, BN = NJ * 16;
-  const int n_tiles = (int)((n_out + BN - 1) / BN), m_tiles = (int)((m + kPcBM - 1) / kPcBM);
+  constexpr int NJ = 7, BN = NJ * 16, BM = pc_bm(MB);
+  const int n_tiles = (int)((n_out + BN - 1) / BN), m_tiles = (int)((m + BM - 1) / BM);
   int xcds_per_mtile = 0;
   unsigned nwg = (unsigned)(n_tiles * m_tiles);
   if (m_tiles >= 2 && m_tiles <= 8 && 8 % m_tiles == 0) {
     xcds_per_mtile = 8 / m_tiles;
     nwg = (unsigned)(((n_tiles + xcds_per_mtile - 1) / xcds_per_mtile) * 8);
   }
-  hipLaunchKernelGGL((gemm_pc_kernel<NJ, FMT>), dim3(nwg), dim3(kPcThreads), 0, s, wb, x, y, y_dtype, bias,
+  hipLaunchKernelGGL((gemm_pc_kernel<NJ, FMT, MB>), dim3(nwg), dim3(kPcThreads), 0, s, wb, x, y, y_dtype, bias,
                      bias_dtype, (int)m, (int)n_out, (int)n_in, n_tiles, m_tiles, xcds_per_mtile);
   return hipGetLastError();
+}
+
+// Few rows (up to kPcSkinnyRows) take 64-row tiles: a quarter of the MFMA and activation traffic
+// per step, and twice the workgroups when there are more than 64 rows.
+static const int64_t kPcSkinnyRows = [] { const char* e = getenv("TTQ_GEMM_SKINNY_ROWS"); return e ? atoi(e) : 128; }();
+template <int FMT>
+static hipError_t launch_pc_fmt(const uint8_t* wb, const uint16_t* x, void* y, int y_dtype, const void* bias,
+                                int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+  if (m <= kPcSkinnyRows) return launch_pc_112<FMT, 1>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  return launch_pc_112<FMT, 4>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
 }
 
 // Only the 112-column tile is built in this form: with 128 columns the consumers' 128
@@ -501,9 +517,9 @@ hipError_t launch_gemm_pc(int format, const void* w, const uint16_t* x_bf16, voi
   if (y_dtype != kBF16 && y_dtype != kF32) return hipErrorInvalidValue;
   const uint8_t* wb = static_cast<const uint8_t*>(w);
   switch (format) {
-    case kQ4_K: return launch_pc_112<kQ4_K>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-    case kQ6_K: return launch_pc_112<kQ6_K>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-    case kQ8_0: return launch_pc_112<kQ8_0>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kQ4_K: return launch_pc_fmt<kQ4_K>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kQ6_K: return launch_pc_fmt<kQ6_K>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kQ8_0: return launch_pc_fmt<kQ8_0>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
     default: return hipErrorInvalidValue;
   }
 }
