@@ -22,6 +22,7 @@ SOURCES = [
     "ttq_gemv_dot2.hip",
     "ttq_gemv_mfma.hip",
     "ttq_gemv_q8_mfma.hip",
+    "ttq_gemv_q8_win.hip",
     "ttq_gemv_q4k_batch.hip",
     "ttq_gemm_q4k.hip",
     "ttq_gemm_pc.hip",

@@ -182,7 +182,8 @@ def test_q4_k_16bit_activation_extremes():
 
 
 @pytest.mark.parametrize("xk", ["f32", "bf16", "f16"])
-@pytest.mark.parametrize("n_out,n_in", [(70000, 128), (25600, 256), (4096 + 8, 1024), (2500, 8192), (5000, 640)])
+@pytest.mark.parametrize("n_out,n_in", [(70000, 128), (25600, 256), (4096 + 8, 1024), (2500, 8192), (5000, 640),
+                                        (3000, 2048), (2304, 6144), (2048 + 16, 4096), (9000, 512)])
 def test_q8_0_work_distributions(xk, n_out, n_in):
     """Q8_0 through the matrix cores (enough rows for that kernel): every split of rows and steps
     over the wavefronts, all activation types, two activation rows of uneven magnitude."""
@@ -201,11 +202,15 @@ def test_q8_0_work_distributions(xk, n_out, n_in):
 
 
 @pytest.mark.parametrize("xk", ["f32", "bf16"])
-def test_q8_0_unit_vectors_and_extremes_many_rows(xk):
-    n_out, n_in = 2100, 1024
+@pytest.mark.parametrize("n_in", [1024, 1024 + 128])
+def test_q8_0_unit_vectors_and_extremes_many_rows(xk, n_in):
+    # 1024: whole chunks of 8 blocks (the aligned-window kernel); 1152: the block-wise kernel
+    n_out = 2100
     p = random_blocks(F.Q8_0, n_out * (n_in // 32), seed=13)
     what = oracle.dequant(F.Q8_0, p, n_out, n_in)
-    cols = [0, 1, 15, 16, 31, 32, 33, 127, 128, 500, n_in - 33, n_in - 1]
+    # every position of a chunk's windows: block starts and ends, 16-byte piece and 64-byte window edges
+    cols = [0, 1, 13, 14, 15, 16, 29, 30, 31, 32, 33, 59, 60, 61, 62, 63, 64, 91, 92, 95, 96, 119, 120, 121,
+            127, 128, 151, 152, 159, 160, 179, 180, 191, 192, 223, 224, 239, 240, 255, 256, 500, n_in - 33, n_in - 1]
     x = np.zeros((len(cols) + 3, n_in), np.float32)
     for i, c in enumerate(cols):
         x[i, c] = 1.0 if i % 2 == 0 else -0.5
