@@ -65,11 +65,13 @@ __device__ __forceinline__ void lds_store16(uint32_t lds_addr, uint32_t a, uint3
 
 // ---- what the W producers know about a format.  A producer thread owns one row of the tile
 // and, of every 64-k step, the weights k = 16*whalf + e and k = 32 + 16*whalf + e (e = 0..15):
-// `lo` and `hi` below, 8 bf16 pairs each.  Raw holds the thread's share of 256 k of its row.
+// `lo` and `hi` below, 8 bf16 pairs each (kWholeKsub formats: k = 32*whalf + e, e = 0..31 instead).
+// Raw holds the thread's share of 256 k of its row.
 template <int FMT> struct WFmt;
 
 template <> struct WFmt<kQ4_K> {
   static constexpr int kUnitBytes = 144;               // one super-block
+  static constexpr bool kWholeKsub = false;
   struct Raw { uint4 hdr, q[4]; };
   static __device__ __forceinline__ void load(Raw& dst, const uint8_t* p, int whalf) {
     dst.hdr = load16_a16(p);
@@ -113,6 +115,7 @@ template <> struct WFmt<kQ4_K> {
 // scales[8*half + 2*t + whalf].
 template <> struct WFmt<kQ6_K> {
   static constexpr int kUnitBytes = 210;
+  static constexpr bool kWholeKsub = false;
   struct Raw { uint4 ql[4], qh[2], sc; uint32_t d; };
   static __device__ __forceinline__ void load(Raw& dst, const uint8_t* p, int whalf) {
 #pragma unroll
@@ -132,6 +135,7 @@ template <> struct WFmt<kQ6_K> {
     const uint32_t sw4 = scw[2 * H + ODD] >> (8 * whalf);       // scales 8H + 4*ODD + whalf (+2)
     const float s1 = d * (float)(int)(int8_t)(sw4 & 0xFFu);
     const float s2 = d * (float)(int)(int8_t)((sw4 >> 16) & 0xFFu);
+    const float m1 = -32.f * s1, m2 = -32.f * s2;
     const uint32_t a4[4] = {r.ql[2 * H].x, r.ql[2 * H].y, r.ql[2 * H].z, r.ql[2 * H].w};
     const uint32_t b4[4] = {r.ql[2 * H + 1].x, r.ql[2 * H + 1].y, r.ql[2 * H + 1].z, r.ql[2 * H + 1].w};
     const uint32_t h4[4] = {r.qh[H].x, r.qh[H].y, r.qh[H].z, r.qh[H].w};
@@ -142,8 +146,10 @@ template <> struct WFmt<kQ6_K> {
       float fl[4], fh[4];
 #pragma unroll
       for (int k = 0; k < 4; k++) {
-        fl[k] = s1 * ((float)((qa >> (8 * k)) & 0xFFu) - 32.f);
-        fh[k] = s2 * ((float)((qb >> (8 * k)) & 0xFFu) - 32.f);
+        // s * (u - 32) in one fused multiply-add: -32 * s is exact, so the single rounding is
+        // that of the canonical product s * (float)(u - 32)
+        fl[k] = fmaf_(s1, (float)((qa >> (8 * k)) & 0xFFu), m1);
+        fh[k] = fmaf_(s2, (float)((qb >> (8 * k)) & 0xFFu), m2);
       }
       lo[2 * i] = pack_bf16x2(fl[0], fl[1]);
       lo[2 * i + 1] = pack_bf16x2(fl[2], fl[3]);
@@ -153,29 +159,38 @@ template <> struct WFmt<kQ6_K> {
   }
 };
 
-// Q8_0: eight 34-byte blocks { d, q[32] } per 256 k; step C is blocks 2C and 2C+1.
+// Q8_0: eight 34-byte blocks { d, q[32] } per 256 k; step C is blocks 2C and 2C+1.  Here a thread
+// takes the whole block 2C + whalf of every step (kWholeKsub: its 32 weights are k = 32*whalf + e,
+// `lo` the first 16, `hi` the last 16): one scale and three loads per block.
 template <> struct WFmt<kQ8_0> {
   static constexpr int kUnitBytes = 8 * 34;
-  struct Raw { uint4 q[8]; uint32_t d[8]; };
+  static constexpr bool kWholeKsub = true;
+  struct Raw { uint4 q[8]; uint32_t d[4]; };
   static __device__ __forceinline__ void load(Raw& dst, const uint8_t* p, int whalf) {
 #pragma unroll
-    for (int b = 0; b < 8; b++) {
-      dst.q[b] = load16_a2(p + 34 * b + 2 + 16 * whalf);
-      dst.d[b] = load2(p + 34 * b);
+    for (int c = 0; c < 4; c++) {
+      const uint8_t* blk = p + 34 * (2 * c + whalf);
+      dst.d[c] = load2(blk);
+      dst.q[2 * c] = load16_a2(blk + 2);
+      dst.q[2 * c + 1] = load16_a2(blk + 18);
     }
   }
   template <int C>
   static __device__ __forceinline__ void dequant(const Raw& r, int, uint32_t (&lo)[8], uint32_t (&hi)[8]) {
-    const float d0 = f16_bits_to_f32((uint16_t)r.d[2 * C]), d1 = f16_bits_to_f32((uint16_t)r.d[2 * C + 1]);
+    const float d = f16_bits_to_f32((uint16_t)r.d[C]);
+    const float md = -128.f * d;
     const uint32_t a4[4] = {r.q[2 * C].x, r.q[2 * C].y, r.q[2 * C].z, r.q[2 * C].w};
     const uint32_t b4[4] = {r.q[2 * C + 1].x, r.q[2 * C + 1].y, r.q[2 * C + 1].z, r.q[2 * C + 1].w};
 #pragma unroll
     for (int i = 0; i < 4; i++) {
+      // q + 128 as an unsigned byte converts in one instruction; d * (u - 128) as one fused
+      // multiply-add rounds once, like the canonical d * q (128 * d is exact)
+      const uint32_t ua = a4[i] ^ 0x80808080u, ub = b4[i] ^ 0x80808080u;
       float fl[4], fh[4];
 #pragma unroll
       for (int k = 0; k < 4; k++) {
-        fl[k] = d0 * (float)(int)(int8_t)((a4[i] >> (8 * k)) & 0xFFu);
-        fh[k] = d1 * (float)(int)(int8_t)((b4[i] >> (8 * k)) & 0xFFu);
+        fl[k] = fmaf_(d, (float)((ua >> (8 * k)) & 0xFFu), md);
+        fh[k] = fmaf_(d, (float)((ub >> (8 * k)) & 0xFFu), md);
       }
       lo[2 * i] = pack_bf16x2(fl[0], fl[1]);
       lo[2 * i + 1] = pack_bf16x2(fl[2], fl[3]);
@@ -184,7 +199,6 @@ template <> struct WFmt<kQ8_0> {
     }
   }
 };
-
 
 // W tile in LDS: [ksub 2][j NJ][g 4][n 16] units of 16 bytes (8 consecutive k of one column),
 // i.e. exactly the B operand of lane g*16+n for column block j.
@@ -309,12 +323,21 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
       constexpr int c = decltype(cc)::value;
       uint32_t lo[8], hi[8];
       WF::template dequant<c>(r, whalf, lo, hi);
-      // k = 16*half + e  -> ksub 0, groups 2*half and 2*half+1; k = 32 + 16*half + e: ksub 1
-      const uint32_t base = sw_addr + (uint32_t)(buf * kWUnits + (wj * 4 + 2 * whalf) * 16 + wn) * 16u;
-      lds_store16(base, lo[0], lo[1], lo[2], lo[3]);
-      lds_store16(base + 256u, lo[4], lo[5], lo[6], lo[7]);
-      lds_store16(base + NJ * 1024u, hi[0], hi[1], hi[2], hi[3]);
-      lds_store16(base + NJ * 1024u + 256u, hi[4], hi[5], hi[6], hi[7]);
+      if constexpr (WF::kWholeKsub) {
+        // k = 32*half + e -> ksub `half`, groups 0..3
+        const uint32_t base = sw_addr + (uint32_t)(buf * kWUnits + whalf * (NJ * 64) + wj * 64 + wn) * 16u;
+        lds_store16(base, lo[0], lo[1], lo[2], lo[3]);
+        lds_store16(base + 256u, lo[4], lo[5], lo[6], lo[7]);
+        lds_store16(base + 512u, hi[0], hi[1], hi[2], hi[3]);
+        lds_store16(base + 768u, hi[4], hi[5], hi[6], hi[7]);
+      } else {
+        // k = 16*half + e  -> ksub 0, groups 2*half and 2*half+1; k = 32 + 16*half + e: ksub 1
+        const uint32_t base = sw_addr + (uint32_t)(buf * kWUnits + (wj * 4 + 2 * whalf) * 16 + wn) * 16u;
+        lds_store16(base, lo[0], lo[1], lo[2], lo[3]);
+        lds_store16(base + 256u, lo[4], lo[5], lo[6], lo[7]);
+        lds_store16(base + NJ * 1024u, hi[0], hi[1], hi[2], hi[3]);
+        lds_store16(base + NJ * 1024u + 256u, hi[4], hi[5], hi[6], hi[7]);
+      }
     };
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
