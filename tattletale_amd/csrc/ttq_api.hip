@@ -270,7 +270,9 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
     return hip_status(ttq::launch_gemm_q4k(layer->qweight, static_cast<const uint16_t*>(x), y, y_dtype,
                                            layer->bias, layer->bias_dtype, m, n_out, n_in, s));
   }
-  if ((layer->format == TTQ_Q6_K || layer->format == TTQ_Q8_0) && x_dtype == TTQ_BF16 && m >= 16 &&
+  // Q6_K / Q8_0 have no few-row decode kernel: from eight rows on the 64-row GEMM tile is faster
+  // than one GEMV pass per row
+  if ((layer->format == TTQ_Q6_K || layer->format == TTQ_Q8_0) && x_dtype == TTQ_BF16 && m >= 8 &&
       (y_dtype == TTQ_BF16 || y_dtype == TTQ_F32) && ttq::gemm_pc_supported(layer->format, m, n_out, n_in, 112)) {
     return hip_status(ttq::launch_gemm_pc(layer->format, layer->qweight, static_cast<const uint16_t*>(x), y,
                                           y_dtype, layer->bias, layer->bias_dtype, m, n_out, n_in, s));

@@ -86,23 +86,26 @@ def test_gemm_identity_activations_other_formats(fmt, n_in):
 
 
 @pytest.mark.parametrize("fmt", [F.Q6_K, F.Q8_0])
-def test_forward_prefill_other_formats(fmt):
-    n_out, n_in, m = 256, 1024, 48
+@pytest.mark.parametrize("lead", [(4, 12), (2, 5), (8,)])
+def test_forward_prefill_other_formats(fmt, lead):
+    # 48 rows, and 10 / 8 rows: from eight rows on these formats take the GEMM (64-row tiles)
+    n_out, n_in, m = 256, 1024, int(np.prod(lead))
     w = Q.fill_normal(410 + fmt, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
     p = Q.quantize(fmt, w)
     what = oracle.dequant(fmt, p, n_out, n_in)
     bias = Q.fill_normal(411, 2, 0.5, n_out)
-    xd, xf = x_to_dev(Q.fill_normal(412, 1, 1.0, m * n_in).reshape(4, 12, n_in), "bf16")
+    xd, xf = x_to_dev(Q.fill_normal(412, 1, 1.0, m * n_in).reshape(lead + (n_in,)), "bf16")
     bd, bf = x_to_dev(bias, "f32")
     layer = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out, bias=bd)
     y = layer.forward(xd)
-    assert y.shape == (4, 12, n_out) and y.dtype == torch.bfloat16
-    want = oracle.linear_f64(what, xf.reshape(m, n_in), bf).reshape(4, 12, n_out)
+    assert y.shape == lead + (n_out,) and y.dtype == torch.bfloat16
+    want = oracle.linear_f64(what, xf.reshape(m, n_in), bf).reshape(lead + (n_out,))
     assert rel_l2(oracle.bf16_to_f32(dev_bits(y)), want) <= TOL
     y32 = layer.forward(xd, out_dtype=torch.float32)
     assert rel_l2(y32.cpu().numpy(), want) <= TOL
-    row = layer.forward(xd[1, 5], out_dtype=torch.float32).cpu().numpy()
-    assert rel_l2(row, y32[1, 5].cpu().numpy()) <= 5e-3
+    idx = tuple(d - 1 for d in lead)
+    row = layer.forward(xd[idx], out_dtype=torch.float32).cpu().numpy()
+    assert rel_l2(row, y32[idx].cpu().numpy()) <= 5e-3
 
 
 def test_forward_dispatches_prefill_to_gemm_and_matches_gemv():
