@@ -49,8 +49,8 @@ def main() -> int:
                          "scaling the FETCH_SIZE / WRITE_SIZE counters of rocprofv3)")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this path runs on ONE GPU; --gpus %d is not supported "
-              "(see DESIGN.md, 'More than one GPU')" % args.gpus, file=sys.stderr)
+        print("bench.py: this path runs on ONE GPU; --gpus %d is not supported (the operator shards by "
+              "output rows with no exchange; nothing here uses a second device)" % args.gpus, file=sys.stderr)
         return 2
 
     import numpy as np
