@@ -267,6 +267,22 @@ def main() -> int:
         log("[q4_k_gate_up_silu_gemv] fused %.3f us/step (%.0f GB/s), GEMV + silu_and_mul %.3f us/step; "
             "with add+RMSNorm in front: one launch %.3f us/step, three launches %.3f us/step"
             % (f_ms * 1e3, res["weight_GBps"], u_ms * 1e3, nf_ms * 1e3, nu_ms * 1e3))
+        # prefill, M = 2048: silu_and_mul in the GEMM epilogue against GEMM + ttq_silu_and_mul
+        xm = torch.randn((2048, n_in), device=dev).mul_(0.05).to(torch.bfloat16)
+
+        def pre_fused(i):
+            QL.gemm_q4_k_silu_mul(ws[i % ncopies], xm, n_ff, n_in)
+
+        def pre_unfused(i):
+            QL.silu_and_mul(QL.gemm_q4_k(ws[i % ncopies], xm, 2 * n_ff, n_in))
+
+        _, pf_ms = time_steps(pre_fused, 20, 3, use_graph=not args.eager)
+        _, pu_ms = time_steps(pre_unfused, 20, 3, use_graph=not args.eager)
+        res["prefill_m2048_fused_gemm_ms_per_step"] = pf_ms
+        res["prefill_m2048_gemm_plus_silu_ms_per_step"] = pu_ms
+        res["prefill_m2048_fused_TFLOPs"] = 2.0 * 2048 * 2 * n_ff * n_in / (pf_ms * 1e-3) / 1e12
+        log("[q4_k_gate_up_silu_gemm M=2048] fused %.1f us/step (%.0f TFLOP/s), GEMM + silu_and_mul %.1f us/step"
+            % (pf_ms * 1e3, res["prefill_m2048_fused_TFLOPs"], pu_ms * 1e3))
         return res
 
     def run_widened(steps: int, warmup: int):

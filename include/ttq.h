@@ -130,6 +130,12 @@ TTQ_API int ttq_gemm_q6_k(const void* w, const uint16_t* x_bf16, uint16_t* y_bf1
                   int64_t n_out, int64_t n_in, void* stream);
 TTQ_API int ttq_gemm_q8_0(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m,
                   int64_t n_out, int64_t n_in, void* stream);
+/* Prefill half of GatedMLP.forward in one kernel: y (m, n_ff) = silu(x Wg^T) * (x Wu^T) with the
+ * fused gate||up weight of mlp.nim:39 (2*n_ff rows, gate rows first) -- gate_up_proj.forward
+ * followed by silu_and_mul (mlp.nim:56-59, activations.nim:14-38), silu(g)*u formed in fp32 from
+ * the fp32 accumulators and rounded once to bf16.  n_in a multiple of 256. */
+TTQ_API int ttq_gemm_q4_k_silu_mul(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m,
+                  int64_t n_ff, int64_t n_in, void* stream);
 
 /* ---- device dequantizers (the bit-exactness contract made observable) -------------- */
 /* out[n_out][n_in] in `out_dtype`: TTQ_F32 gives the canonical values; TTQ_BF16 gives them

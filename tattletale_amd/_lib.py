@@ -56,6 +56,7 @@ SIGNATURES = {
     "ttq_gemm_q4_k": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "ttq_gemm_q6_k": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "ttq_gemm_q8_0": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "ttq_gemm_q4_k_silu_mul": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "ttq_dequant_q8_0": (_i32, [_vp, _vp, _i32, _i64, _i64, _vp]),
     "ttq_dequant_q4_k": (_i32, [_vp, _vp, _i32, _i64, _i64, _vp]),
     "ttq_dequant_q6_k": (_i32, [_vp, _vp, _i32, _i64, _i64, _vp]),

@@ -193,6 +193,18 @@ int ttq_gemm_q4_k(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64
                                          static_cast<hipStream_t>(stream)));
 }
 
+int ttq_gemm_q4_k_silu_mul(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m, int64_t n_ff,
+                           int64_t n_in, void* stream) {
+  if (!w || !x_bf16 || !y_bf16) return TTQ_ERR_NULL;
+  const int rc = check_shape(TTQ_Q4_K, m, n_ff, n_in, 0, 0);
+  if (rc != TTQ_OK) return rc;
+  if (n_ff > 0x3FFFFFFF) return TTQ_ERR_UNSUPPORTED;
+  if (!aligned16(w) || !aligned16(x_bf16) || !aligned16(y_bf16)) return TTQ_ERR_ALIGN;
+  if (!ttq::gemm_pc_supported(TTQ_Q4_K, m, 2 * n_ff, n_in, 112)) return TTQ_ERR_UNSUPPORTED;
+  return hip_status(ttq::launch_gemm_pc_silu_mul(w, x_bf16, y_bf16, TTQ_BF16, nullptr, 0, m, n_ff, n_in,
+                                                 static_cast<hipStream_t>(stream)));
+}
+
 static int gemm_block(int format, const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m,
                       int64_t n_out, int64_t n_in, void* stream) {
   if (!w || !x_bf16 || !y_bf16) return TTQ_ERR_NULL;

@@ -202,7 +202,14 @@ template <> struct WFmt<kQ8_0> {
 
 // W tile in LDS: [ksub 2][j NJ][g 4][n 16] units of 16 bytes (8 consecutive k of one column),
 // i.e. exactly the B operand of lane g*16+n for column block j.
-template <int NJ, int FMT, int MB>
+// FUSE: the weight holds gate rows [0, n_out) followed by up rows [n_out, 2*n_out), as GatedMLP
+// builds it (workspace/transformers/src/layers/mlp.nim:39), and the kernel writes
+// silu(gate . x) * (up . x), the silu_and_mul of
+// workspace/transformers/src/kernels/activations.nim:14-38, for n_out outputs.  A tile then covers
+// BN / 2 outputs: column 16j + c of the tile is output n0 + 8j + c%8, its gate row for c < 8 and
+// its up row for c >= 8, so that a gate value and its up value meet eight lanes apart in the same
+// accumulator register.
+template <int NJ, int FMT, int MB, bool FUSE>
 __global__ void __launch_bounds__(kPcThreads)
 gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, void* __restrict__ yv,
                    int y_dtype, const void* __restrict__ bias, int bias_dtype, int m, int n_out, int n_in,
@@ -233,7 +240,8 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
     n_tile = blockIdx.x / m_tiles;
   }
   if (n_tile >= n_tiles) return;
-  const int n0 = n_tile * BN;
+  constexpr int BO = FUSE ? BN / 2 : BN;     // outputs per tile
+  const int n0 = n_tile * BO;
   const int ksteps = n_in >> 6;
   const int nblocks = n_in >> 8;
 
@@ -309,7 +317,9 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
     // threads mirror threads 0..31 (same loads, same LDS writes of the same values)
     const int wt = pt < 2 * BN ? pt : pt - 2 * BN;
     const int wr = wt % BN, whalf = wt / BN;
-    const int wrow = min(n0 + wr, n_out - 1);           // clamped: rows past the end are never stored
+    // clamped: rows past the end are never stored
+    const int wrow = FUSE ? min(n0 + 8 * (wr >> 4) + (wr & 7), n_out - 1) + ((wr >> 3) & 1) * n_out
+                          : min(n0 + wr, n_out - 1);
     using WF = WFmt<FMT>;
     using WRaw = typename WF::Raw;
     const uint8_t* wptr = w + (int64_t)nblocks * WF::kUnitBytes * (int64_t)wrow;
@@ -447,6 +457,65 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
 
   // ---- epilogue: lane holds Y[m0 + 16i + 4*(lane/16) + r][n0 + 16j + lane%16], r = 0..3
   const int cn = lane & 15, rb4 = (lane >> 4) * 4;
+  if constexpr (FUSE) {
+    // gate in lanes cn < 8, the matching up eight lanes further; silu(g) * u in fp32, one rounding.
+    const bool full = y_dtype == kBF16 && n0 + BO <= n_out && (n_out & 7) == 0;
+    constexpr int kRowBytes = BO * 2 + 16;
+    uint8_t* stg = smem + wave * (kXStages * kXStage);
+    // Column blocks are taken in pairs: lanes cn < 8 finish block j (own gate, up from eight lanes
+    // further), lanes cn >= 8 block j+1 (own up, gate from eight lanes back), so that the exp2 and
+    // reciprocal -- quarter-rate instructions -- run once per output and not twice.  Both halves
+    // write output column n0 + 8j + cn.
+#pragma unroll
+    for (int j = 0; j < NJ; j += 2) {
+      const bool pair = j + 1 < NJ;
+      const bool lowhalf = cn < 8;
+      const int o = n0 + 8 * j + cn;
+      const bool live = lowhalf || pair;
+      const int oc = min(o, n_out - 1);
+      const float bg = load_bias(bias, bias_dtype, (int64_t)oc);
+      const float bu = load_bias(bias, bias_dtype, (int64_t)oc + (int64_t)n_out);
+#pragma unroll
+      for (int i = 0; i < MB; i++) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const float a0 = acc[i][j][r];
+          const float a1 = pair ? acc[i][j + 1 < NJ ? j + 1 : j][r] : 0.f;
+          const float up0 = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(a0), 0x108, 0xF, 0xF, false));
+          const float gt1 = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(a1), 0x118, 0xF, 0xF, false));
+          const float g = (lowhalf ? a0 : gt1) + bg;
+          const float u = (lowhalf ? up0 : a1) + bu;
+          // silu with the hardware exp2 / reciprocal (1 ulp each): the result is rounded to bf16 or
+          // is one term of a 2e-2 comparison, and the library versions cost five times as much
+          const float res = (g * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(g * -1.4426950408889634f))) * u;
+          if (live) {
+            const int row = 16 * i + rb4 + r;
+            if (full) {
+              *reinterpret_cast<uint16_t*>(stg + row * kRowBytes + (8 * j + cn) * 2) = f32_to_bf16_bits(res);
+            } else if (o < n_out && m0 + row < m) {
+              if (y_dtype == kBF16) YElem<bf16_tag>::store(static_cast<bf16_tag*>(yv), (int64_t)(m0 + row) * n_out + o, res);
+              else YElem<float>::store(static_cast<float*>(yv), (int64_t)(m0 + row) * n_out + o, res);
+            }
+          }
+        }
+      }
+    }
+    if (full) {
+      uint8_t* yb = static_cast<uint8_t*>(yv);
+      constexpr int kChunks = BO / 8;      // 16-byte chunks per row
+      constexpr int kSlots = 16 * MB * kChunks;
+#pragma unroll
+      for (int t = 0; t < (kSlots + 63) / 64; t++) {
+        const int c = t * 64 + lane;
+        const int row = c / kChunks, ch = c - row * kChunks;
+        if (c >= kSlots) break;
+        const uint4 v = *reinterpret_cast<const uint4*>(stg + row * kRowBytes + ch * 16);
+        if (m0 + row < m)
+          *reinterpret_cast<uint4*>(yb + ((int64_t)(m0 + row) * n_out + n0 + ch * 8) * 2) = v;
+      }
+    }
+    return;
+  }
   if (y_dtype == kBF16 && n0 + BN <= n_out && (n_out & 7) == 0) {
     // Full tile of bf16: transpose through the wavefront's own (now idle) X ring, so that global
     // memory sees 16-byte stores along the rows instead of 2-byte ones.  Row stride 240 bytes.
@@ -497,30 +566,30 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
   }
 }
 
-template <int FMT, int MB>
+template <int FMT, int MB, bool FUSE>
 static hipError_t launch_pc_112(const uint8_t* wb, const uint16_t* x, void* y, int y_dtype, const void* bias,
                                 int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
-  constexpr int NJ = 7, BN = NJ * 16, BM = pc_bm(MB);
-  const int n_tiles = (int)((n_out + BN - 1) / BN), m_tiles = (int)((m + BM - 1) / BM);
+  constexpr int NJ = 7, BO = FUSE ? NJ * 8 : NJ * 16, BM = pc_bm(MB);
+  const int n_tiles = (int)((n_out + BO - 1) / BO), m_tiles = (int)((m + BM - 1) / BM);
   int xcds_per_mtile = 0;
   unsigned nwg = (unsigned)(n_tiles * m_tiles);
   if (m_tiles >= 2 && m_tiles <= 8 && 8 % m_tiles == 0) {
     xcds_per_mtile = 8 / m_tiles;
     nwg = (unsigned)(((n_tiles + xcds_per_mtile - 1) / xcds_per_mtile) * 8);
   }
-  hipLaunchKernelGGL((gemm_pc_kernel<NJ, FMT, MB>), dim3(nwg), dim3(kPcThreads), 0, s, wb, x, y, y_dtype, bias,
-                     bias_dtype, (int)m, (int)n_out, (int)n_in, n_tiles, m_tiles, xcds_per_mtile);
+  hipLaunchKernelGGL((gemm_pc_kernel<NJ, FMT, MB, FUSE>), dim3(nwg), dim3(kPcThreads), 0, s, wb, x, y, y_dtype,
+                     bias, bias_dtype, (int)m, (int)n_out, (int)n_in, n_tiles, m_tiles, xcds_per_mtile);
   return hipGetLastError();
 }
 
 // Few rows (up to kPcSkinnyRows) take 64-row tiles: a quarter of the MFMA and activation traffic
 // per step, and twice the workgroups when there are more than 64 rows.
 static const int64_t kPcSkinnyRows = [] { const char* e = getenv("TTQ_GEMM_SKINNY_ROWS"); return e ? atoi(e) : 128; }();
-template <int FMT>
+template <int FMT, bool FUSE>
 static hipError_t launch_pc_fmt(const uint8_t* wb, const uint16_t* x, void* y, int y_dtype, const void* bias,
                                 int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
-  if (m <= kPcSkinnyRows) return launch_pc_112<FMT, 1>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-  return launch_pc_112<FMT, 4>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  if (m <= kPcSkinnyRows) return launch_pc_112<FMT, 1, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  return launch_pc_112<FMT, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
 }
 
 // Only the 112-column tile is built in this form: with 128 columns the consumers' 128
@@ -540,11 +609,22 @@ hipError_t launch_gemm_pc(int format, const void* w, const uint16_t* x_bf16, voi
   if (y_dtype != kBF16 && y_dtype != kF32) return hipErrorInvalidValue;
   const uint8_t* wb = static_cast<const uint8_t*>(w);
   switch (format) {
-    case kQ4_K: return launch_pc_fmt<kQ4_K>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-    case kQ6_K: return launch_pc_fmt<kQ6_K>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-    case kQ8_0: return launch_pc_fmt<kQ8_0>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kQ4_K: return launch_pc_fmt<kQ4_K, false>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kQ6_K: return launch_pc_fmt<kQ6_K, false>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kQ8_0: return launch_pc_fmt<kQ8_0, false>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
     default: return hipErrorInvalidValue;
   }
+}
+
+
+// gate||up projection + silu_and_mul in the GEMM epilogue: w holds 2*n_ff rows (gate rows first),
+// y is (m, n_ff).  Q4_K weights.
+hipError_t launch_gemm_pc_silu_mul(const void* w, const uint16_t* x_bf16, void* y, int y_dtype, const void* bias,
+                                   int bias_dtype, int64_t m, int64_t n_ff, int64_t n_in, hipStream_t s) {
+  if (m == 0 || n_ff == 0) return hipSuccess;
+  if (y_dtype != kBF16 && y_dtype != kF32) return hipErrorInvalidValue;
+  return launch_pc_fmt<kQ4_K, true>(static_cast<const uint8_t*>(w), x_bf16, y, y_dtype, bias, bias_dtype, m, n_ff,
+                                    n_in, s);
 }
 
 }  // namespace ttq

@@ -80,6 +80,11 @@ hipError_t launch_gemm_pc(int format, const void* w, const uint16_t* x_bf16, voi
                           const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                           hipStream_t s);
 
+// The same GEMM with silu_and_mul in the epilogue: Q4_K weight of 2*n_ff rows (gate rows first).
+hipError_t launch_gemm_pc_silu_mul(const void* w, const uint16_t* x_bf16, void* y, int y_dtype,
+                                   const void* bias, int bias_dtype, int64_t m, int64_t n_ff,
+                                   int64_t n_in, hipStream_t s);
+
 hipError_t launch_dequant_exl3(const uint16_t* trellis, uint16_t* out_f16, int64_t n_out,
                                int64_t n_in, int bits, int cb, hipStream_t s);
 hipError_t launch_gemv_exl3(const uint16_t* trellis, const uint16_t* suh, const uint16_t* svh,

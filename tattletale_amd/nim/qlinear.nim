@@ -42,6 +42,7 @@ proc dequant_q4_k*(w, dst: pointer, out_dtype: cint, n_out, n_in: int64, stream:
 proc dequant_q6_k*(w, dst: pointer, out_dtype: cint, n_out, n_in: int64, stream: pointer): cint {.ttq.}
 proc dequant_exl3*(trellis, dst: ptr uint16, n_out, n_in: int64, bits, codebook: cint, stream: pointer): cint {.ttq.}
 proc silu_and_mul*(src, dst: pointer, dtype: cint, m, h: int64, stream: pointer): cint {.ttq.}
+proc gemm_q4_k_silu_mul*(w: pointer, x, y: ptr uint16, m, n_ff, n_in: int64, stream: pointer): cint {.ttq.}
 proc gemv_q4_k_silu_mul*(w, x: pointer, x_dtype: cint, y: pointer, y_dtype: cint, m, n_ff, n_in: int64,
                          stream: pointer): cint {.ttq.}
 proc rmsnorm*(x, residual, gamma: pointer, eps: cfloat, dtype: cint, new_residual_out, normed_out: pointer,
@@ -104,6 +105,7 @@ proc forward*(self: QuantLinear, x: TorchTensor): TorchTensor =
 # projection, silu_and_mul (workspace/transformers/src/kernels/activations.nim:14-38), down.
 
 const kTtqErrUnsupported = -6
+const kFusedGemmMinRows = 512
 
 type
   QuantGatedMLP* = object
@@ -142,6 +144,16 @@ proc forward*(self: QuantGatedMLP, x: TorchTensor): TorchTensor =
     if rc == 0: return self.down_proj.forward(act)
     if rc != kTtqErrUnsupported:
       raise newException(QuantLinearError, "ttq_gemv_q4_k_silu_mul: " & $strerror(rc))
+  elif gu.format == kQ4_K and gu.bias.isNone and m >= kFusedGemmMinRows and x.scalarType() == kBfloat16:
+    # prefill: silu_and_mul in the GEMM epilogue (breaks even at 512 rows, 15 % faster at 2048)
+    var shape = x.sizes().asNimView().toSeq()
+    shape[^1] = nff
+    let act = F.empty(shape, x.options())
+    let rc = gemm_q4_k_silu_mul(gu.qweight.data_ptr(byte), cast[ptr uint16](x.data_ptr(byte)),
+                                cast[ptr uint16](act.data_ptr(byte)), m, nff, gu.in_features, nil)
+    if rc == 0: return self.down_proj.forward(act)
+    if rc != kTtqErrUnsupported:
+      raise newException(QuantLinearError, "ttq_gemm_q4_k_silu_mul: " & $strerror(rc))
   result = self.down_proj.forward(quant_silu_and_mul(gu.forward(x)))
 
 # ------------------------------------------------------------------------------ RMSNorm

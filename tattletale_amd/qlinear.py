@@ -251,6 +251,21 @@ def gemv_q4_k_silu_mul(qweight: torch.Tensor, x: torch.Tensor, n_ff: int, n_in: 
     return out
 
 
+def gemm_q4_k_silu_mul(qweight: torch.Tensor, x: torch.Tensor, n_ff: int, n_in: int) -> torch.Tensor:
+    """bf16 y (m, n_ff) = silu(x Wg^T) * (x Wu^T) for the packed (2*n_ff, n_in) Q4_K matrix [Wg; Wu] and a
+    multi-row bf16 activation: the prefill GEMM with silu_and_mul in its epilogue
+    (``ttq_gemm_q4_k_silu_mul``)."""
+    dev = _require_device(qweight, x)
+    if x.dtype != torch.bfloat16:
+        raise TtqError(_lib.ERR_DTYPE, "ttq_gemm_q4_k_silu_mul takes bfloat16 activations")
+    m = x.numel() // n_in
+    out = torch.empty((m, n_ff), dtype=torch.bfloat16, device=dev)
+    with torch.cuda.device(dev):
+        check(_lib.lib().ttq_gemm_q4_k_silu_mul(qweight.data_ptr(), x.data_ptr(), out.data_ptr(), m, n_ff, n_in,
+                                                _stream(dev)), "ttq_gemm_q4_k_silu_mul")
+    return out
+
+
 def rmsnorm(x: torch.Tensor, gamma: torch.Tensor, eps: float, residual: Optional[torch.Tensor] = None):
     """``RmsNorm.forward`` (residual None) / ``forward_with_residual``
     (workspace/transformers/src/layers/norm.nim:23-38) through ``ttq_rmsnorm``.
@@ -305,10 +320,16 @@ class QuantGatedMLP:
             raise TtqError(_lib.ERR_SHAPE, "QuantGatedMLP.init: hidden sizes differ")
         return cls(gate_up_proj, down_proj)
 
+    # The fused GEMM pays for the activation with quarter-rate exp2 / reciprocal in its epilogue and
+    # wins once the (rows, 2 * intermediate) tensor it saves no longer fits the caches: at
+    # 28672 x 4096 it breaks even at 512 rows and is 15 % faster at 2048.
+    FUSED_GEMM_MIN_ROWS = 512
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        """x (..., hidden) -> (..., hidden)  (mlp.nim:43-60).  A single-token 16-bit activation
-        on Q4_K weights takes the fused GEMV + silu_and_mul kernel; everything else runs the
-        projection, ``silu_and_mul`` and the down projection as three launches."""
+        """x (..., hidden) -> (..., hidden)  (mlp.nim:43-60).  On Q4_K weights a single-token 16-bit
+        activation takes the fused GEMV + silu_and_mul kernel and a bf16 activation of at least
+        ``FUSED_GEMM_MIN_ROWS`` rows the GEMM with silu_and_mul in its epilogue; everything else runs
+        the projection, ``silu_and_mul`` and the down projection as three launches."""
         gu = self.gate_up_proj
         n_ff = self.down_proj.in_features
         m = x.numel() // gu.in_features
@@ -317,6 +338,14 @@ class QuantGatedMLP:
             try:
                 act = gemv_q4_k_silu_mul(gu.qweight, x.reshape(m, gu.in_features), n_ff, gu.in_features,
                                          out_dtype=x.dtype).reshape(x.shape[:-1] + (n_ff,))
+            except TtqError as e:
+                if e.status != _lib.ERR_UNSUPPORTED:
+                    raise
+        elif (gu.format == _lib.Q4_K and gu.bias is None and m >= self.FUSED_GEMM_MIN_ROWS
+              and x.dtype == torch.bfloat16 and gu.in_features % 256 == 0):
+            try:
+                act = gemm_q4_k_silu_mul(gu.qweight, x.reshape(m, gu.in_features), n_ff,
+                                         gu.in_features).reshape(x.shape[:-1] + (n_ff,))
             except TtqError as e:
                 if e.status != _lib.ERR_UNSUPPORTED:
                     raise

@@ -64,7 +64,7 @@ def test_other_entry_points_validate():
     p += (-p) % 16
     assert L.ttq_gemm_q4_k(p, None, p, 16, 16, 256, None) == _lib.ERR_NULL
     assert L.ttq_gemm_q4_k(p, p, p, 16, 16, 100, None) == _lib.ERR_SHAPE
-    for fn in (L.ttq_gemm_q6_k, L.ttq_gemm_q8_0):
+    for fn in (L.ttq_gemm_q6_k, L.ttq_gemm_q8_0, L.ttq_gemm_q4_k_silu_mul):
         assert fn(p, None, p, 16, 16, 256, None) == _lib.ERR_NULL
         assert fn(p, p, p, 16, 16, 100, None) == _lib.ERR_SHAPE
         assert fn(p, p + 2, p, 16, 16, 256, None) == _lib.ERR_ALIGN

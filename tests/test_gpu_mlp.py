@@ -212,3 +212,60 @@ def test_fused_rmsnorm_full_shape_gate_up():
     assert bool(((normed.float() - normed_ref.float()).abs() <= 2.0 ** -7 * normed_ref.float().abs()).all())
     y_ref = QL.gemv_q4_k_silu_mul(packed_to_dev(p), normed, n_ff, n_in, out_dtype=torch.bfloat16)
     assert torch.equal(y, y_ref) and bool(torch.isfinite(y.float()).all())
+
+
+# ------------------------------------------------------------------ prefill: silu_and_mul in the GEMM epilogue
+@pytest.mark.parametrize("m,n_ff,n_in", [(64, 256, 1024), (16, 56, 256), (100, 200, 768), (257, 130, 1024),
+                                         (512, 1000, 2048), (300, 3000, 256)])
+def test_fused_gate_up_silu_mul_gemm(m, n_ff, n_in):
+    """Tiles of 56 outputs (full, ragged, a single partial one), 64- and 256-row tiles, ragged rows."""
+    p = random_blocks(F.Q4_K, 2 * n_ff * (n_in // 256), seed=n_ff + m)
+    what = oracle.dequant(F.Q4_K, p, 2 * n_ff, n_in)
+    xd, xf = x_to_dev(Q.fill_normal(n_in + m, 1, 1.0, m * n_in).reshape(m, n_in) * np.float32(0.05), "bf16")
+    y = QL.gemm_q4_k_silu_mul(packed_to_dev(p), xd, n_ff, n_in)
+    assert y.shape == (m, n_ff) and y.dtype == torch.bfloat16
+    got = oracle.bf16_to_f32(dev_bits(y))
+    assert np.all(np.isfinite(got))
+    want = oracle.silu_and_mul_f64(oracle.linear_f64(what, xf))
+    assert rel_l2(got, want) <= 2e-2
+    # against the bf16-rounded weights the kernel really multiplies, only the output rounding remains
+    want_r = oracle.silu_and_mul_f64(oracle.linear_f64(oracle.bf16_to_f32(oracle.f32_to_bf16(what)), xf))
+    assert rel_l2(got, want_r) <= 4e-3
+    # and it is the same function as GEMM followed by the elementwise kernel (which rounds twice)
+    sep = QL.silu_and_mul(QL.gemm_q4_k(packed_to_dev(p), xd, 2 * n_ff, n_in))
+    assert rel_l2(got, oracle.bf16_to_f32(dev_bits(sep))) <= 1e-2
+
+
+def test_gated_mlp_prefill_takes_the_fused_gemm(monkeypatch):
+    monkeypatch.setattr(QuantGatedMLP, "FUSED_GEMM_MIN_ROWS", 32)
+    hidden, inter, m = 512, 1280, 96
+    wg = Q.fill_normal(70, 0, 0.05, inter * hidden).reshape(inter, hidden)
+    wu = Q.fill_normal(71, 0, 0.05, inter * hidden).reshape(inter, hidden)
+    wd = Q.fill_normal(72, 0, 0.05, hidden * inter).reshape(hidden, inter)
+    pgu = np.concatenate([Q.quantize(F.Q4_K, wg), Q.quantize(F.Q4_K, wu)])
+    pd = Q.quantize(F.Q4_K, wd)
+    mlp = QuantGatedMLP.init(QuantLinear.init(packed_to_dev(pgu), F.Q4_K, hidden, 2 * inter),
+                             QuantLinear.init(packed_to_dev(pd), F.Q4_K, inter, hidden))
+    xd, xf = x_to_dev(Q.fill_normal(73, 1, 1.0, m * hidden).reshape(2, m // 2, hidden), "bf16")
+    y = mlp.forward(xd)
+    assert y.shape == (2, m // 2, hidden) and y.dtype == torch.bfloat16
+    wgu = oracle.dequant(F.Q4_K, pgu, 2 * inter, hidden)
+    wdd = oracle.dequant(F.Q4_K, pd, hidden, inter)
+    act = oracle.silu_and_mul_f64(oracle.linear_f64(wgu, xf.reshape(-1, hidden)))
+    act16 = oracle.bf16_to_f32(oracle.f32_to_bf16(act.astype(np.float32)))
+    want = oracle.linear_f64(wdd, act16)
+    assert rel_l2(oracle.bf16_to_f32(dev_bits(y)).reshape(-1, hidden), want) <= 2e-2
+
+
+def test_fused_gemm_full_shape_llama3_8b_ffn():
+    n_ff, n_in, m = 14336, 4096, 512
+    p = random_blocks(F.Q4_K, 2 * n_ff * (n_in // 256), seed=99)
+    xd, xf = x_to_dev(Q.fill_normal(97, 1, 0.02, m * n_in).reshape(m, n_in), "bf16")
+    y = QL.gemm_q4_k_silu_mul(packed_to_dev(p), xd, n_ff, n_in)
+    outs = np.unique(np.concatenate([np.arange(0, n_ff, 97), np.arange(n_ff - 60, n_ff)]))
+    rows = np.concatenate([outs, n_ff + outs])
+    what = oracle.dequant(F.Q4_K, np.ascontiguousarray(p.reshape(2 * n_ff, -1)[rows]), rows.size, n_in)
+    tok = np.arange(0, m, 16)
+    want = oracle.silu_and_mul_f64(oracle.linear_f64(what, xf[tok]))
+    got = oracle.bf16_to_f32(dev_bits(y[torch.from_numpy(tok).to(DEV)][:, torch.from_numpy(outs).to(DEV)]))
+    assert rel_l2(got, want) <= 2e-2
