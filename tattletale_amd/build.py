@@ -24,6 +24,7 @@ SOURCES = [
     "ttq_gemv_q8_mfma.hip",
     "ttq_gemv_q8_win.hip",
     "ttq_gemv_q4k_batch.hip",
+    "ttq_gemv_q4k_batch4.hip",
     "ttq_gemm_q4k.hip",
     "ttq_gemm_pc.hip",
     "ttq_exl3.hip",

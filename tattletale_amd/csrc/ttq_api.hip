@@ -275,8 +275,10 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
 
   // Prefill: MFMA kernel for Q4_K with bf16 activations once there are enough rows to fill a tile.
   // (a few rows more than that still go through the batched decode kernel when it applies)
-  const bool few_rows = m <= ttq::kBatchGemvMaxRows &&
-                        ttq::gemv_q4k_batch_supported(layer->format, x_dtype, m, n_out, n_in);
+  const bool few_rows = (m <= ttq::kBatchGemvMaxRows &&
+                         ttq::gemv_q4k_batch_supported(layer->format, x_dtype, m, n_out, n_in)) ||
+                        (m <= ttq::kBatch4GemvMaxRows &&
+                         ttq::gemv_q4k_batch4_supported(layer->format, x_dtype, m, n_out, n_in));
   if (layer->format == TTQ_Q4_K && x_dtype == TTQ_BF16 && m >= 16 && !few_rows &&
       (y_dtype == TTQ_BF16 || y_dtype == TTQ_F32)) {
     return hip_status(ttq::launch_gemm_q4k(layer->qweight, static_cast<const uint16_t*>(x), y, y_dtype,

@@ -335,8 +335,15 @@ hipError_t launch_gemv(int format, const void* w, const void* x, int x_dtype, vo
                        const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                        hipStream_t s) {
   if (m == 0 || n_out == 0) return hipSuccess;
+  // a few rows at once: four per pass for up to four rows and for rows too long for the 8- and
+  // 16-token tables, else eight or sixteen per pass
+  static const int batch4_max = [] { const char* e = getenv("TTQ_GEMV_BATCH4_MAX_ROWS"); return e ? atoi(e) : 4; }();
+  const bool b4 = gemv_q4k_batch4_supported(format, x_dtype, m, n_out, n_in);
+  if (b4 && m <= batch4_max)
+    return launch_gemv_q4k_batch4(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   if (gemv_q4k_batch_supported(format, x_dtype, m, n_out, n_in))
     return launch_gemv_q4k_batch(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  if (b4) return launch_gemv_q4k_batch4(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   if (gemv_mfma_supported(format, x_dtype, n_out, n_in))
     return launch_gemv_mfma(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   if (gemv_q8_win_supported(format, n_out, n_in))

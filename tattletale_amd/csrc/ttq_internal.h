@@ -69,10 +69,17 @@ hipError_t launch_gemm_q4k(const void* w, const uint16_t* x_bf16, void* y, int y
 // read and unpacked once per 8 or 16 rows.
 // ttq_linear_forward prefers it to the prefill GEMM up to this many rows
 constexpr int64_t kBatchGemvMaxRows = 32;
+constexpr int64_t kBatch4GemvMaxRows = 16;   // four rows per pass (long rows)
 bool gemv_q4k_batch_supported(int format, int x_dtype, int64_t m, int64_t n_out, int64_t n_in);
 hipError_t launch_gemv_q4k_batch(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
                                  const void* bias, int bias_dtype, int64_t m, int64_t n_out,
                                  int64_t n_in, hipStream_t s);
+
+// The same with four rows per pass, for rows up to the GEMV limit (ttq_gemv_q4k_batch4.hip).
+bool gemv_q4k_batch4_supported(int format, int x_dtype, int64_t m, int64_t n_out, int64_t n_in);
+hipError_t launch_gemv_q4k_batch4(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                                  const void* bias, int bias_dtype, int64_t m, int64_t n_out,
+                                  int64_t n_in, hipStream_t s);
 
 // Producer/consumer GEMM for Q4_K / Q6_K / Q8_0 weights and bf16 activations (ttq_gemm_pc.hip).
 bool gemm_pc_supported(int format, int64_t m, int64_t n_out, int64_t n_in, int bn);

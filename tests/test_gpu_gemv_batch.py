@@ -24,7 +24,7 @@ TOL = 1e-3
 @pytest.mark.parametrize("xk", ["bf16", "f16"])
 @pytest.mark.parametrize("m", [2, 3, 7, 8, 9, 16, 17, 31])
 @pytest.mark.parametrize("n_out,n_in", [(2048, 256), (4096 + 8, 1024), (2500, 4096), (25600, 512), (2304, 8192),
-                                        (5000, 1280)])
+                                        (5000, 1280), (4096, 14336), (2050, 16384)])
 def test_batch_random(xk, m, n_out, n_in):
     """Row counts around the 8- and 16-token groups, shapes with 1/2/4/16 slices of the
     super-blocks, several rounds per workgroup, ragged last row groups."""
@@ -50,7 +50,7 @@ def test_batch_random(xk, m, n_out, n_in):
 
 
 @pytest.mark.parametrize("xk", ["bf16", "f16"])
-@pytest.mark.parametrize("n_in", [1024, 4096, 8192])
+@pytest.mark.parametrize("n_in", [1024, 4096, 8192, 14336])
 def test_batch_unit_vectors_reproduce_columns_bit_exactly(xk, n_in):
     n_out = 2100
     p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=13)
@@ -67,6 +67,9 @@ def test_batch_unit_vectors_reproduce_columns_bit_exactly(xk, n_in):
         assert np.array_equal(y[i], col), c
         nz = col != 0
         assert np.array_equal(y[i][nz].view(np.uint32), col[nz].view(np.uint32)), c
+    # four rows or fewer in one call: the four-token kernel
+    y4 = QL.gemv(F.Q4_K, packed_to_dev(p), xd[3:7], n_out, n_in).cpu().numpy()
+    assert np.array_equal(y4, y[3:7])
 
 
 def test_batch_rows_do_not_leak_into_each_other():
@@ -91,6 +94,10 @@ def test_batch_rows_do_not_leak_into_each_other():
     assert not np.any(np.isfinite(y[2]))
     assert rel_l2(y[3], want[1]) <= TOL
     assert rel_l2(y[5], want[2]) <= TOL
+    y3 = QL.gemv(F.Q4_K, packed_to_dev(p), xd[:3], n_out, n_in).cpu().numpy()      # the four-token kernel
+    assert np.array_equal(y3[0], np.zeros(n_out, np.float32))
+    assert rel_l2(y3[1], want[0]) <= TOL
+    assert not np.any(np.isfinite(y3[2]))
 
 
 @pytest.mark.parametrize("m", [5, 20, 32])
