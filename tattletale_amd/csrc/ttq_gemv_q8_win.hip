@@ -10,7 +10,7 @@
 // loads per lane and 16 rows, each touching one 64-byte segment per row.  The bytes then go into
 // the MFMA as they are -- quants AND scale bytes -- and the A operand sorts them out:
 //   * window w (the 64 bytes 64w .. 64w+63 of the chunk, w = 0..3, plus the 16 bytes of piece 16)
-//     holds parts of up to three blocks.  Its plane table has, for a k position that is quant q of
+//     holds parts of up to three blocks.  Its A operand has, for a k position that is quant q of
 //     block b, plane t of x[32b + q] in row 4*(b%4) + t and zero elsewhere (so also at the
 //     positions of scale bytes).  Block b always lands in C rows 4*(b%4) .. +3, i.e. in lane
 //     (n, g = b%4); blocks 0-3 accumulate in one C, blocks 4-7 in another (window 2 holds a part
@@ -23,7 +23,7 @@
 
 namespace ttq {
 
-constexpr int kQ8WinMaxChunks = 24;     // plane tables: 6 KiB of LDS per chunk of 256 activations
+constexpr int kQ8WinMaxChunks = 64;     // n_in <= 16384, the limit of the GEMV entry points
 
 template <typename XT> struct Q8WX;
 template <> struct Q8WX<float> {
@@ -51,17 +51,31 @@ template <> struct Q8WX<f16_tag> {
 
 struct Q8WinStep { uint4 p[5]; };
 
-// table index of the window that holds chunk byte `byte` of block `b` (b = 0..7): windows 0, 1,
-// 2 (block 3 only), 2 (blocks 4, 5), 3, 4
+// The plane tables are stored compactly.  Block b has quants in the 16-byte pieces
+// (34b+2)/16 .. (34b+33)/16 of the chunk: three pieces each for blocks 0-6, two for block 7, 23
+// (block, piece) pairs in all.  A pair holds one 16-byte entry per plane: the plane bytes at the
+// positions of the block's quants in that piece, zero elsewhere.  As the A operand of the MFMA for
+// window w, lane (row = 4*slot + plane, k-group ga) supplies the entry of (the block of that slot
+// in piece 4w + ga, plane) if there is one, else zeros.
+__device__ __forceinline__ int q8win_first_piece(int b) { return (34 * b + 2) >> 4; }
+__device__ __forceinline__ int q8win_pair(int b, int piece) { return 3 * b + (piece - q8win_first_piece(b)); }
+constexpr int kQ8WinPairs = 23;
+// For short rows the tables are kept wide instead: [nch][6 MFMAs][64 lanes] x 16 bytes with the
+// zeros stored, so that every A address is one register plus an immediate (6 KiB per chunk;
+// 0.35 us faster at 4096 x 4096).
+constexpr int kQ8WinMaxWideChunks = 24;
+
+// wide layout: table index of the window that holds chunk byte `byte` of block `b` (b = 0..7):
+// windows 0, 1, 2 (block 3 only), 2 (blocks 4, 5), 3, 4
 __device__ __forceinline__ int q8win_table(int byte, int b) {
   const int w = byte >> 6;
   return w < 2 ? w : (w == 2 ? (b == 3 ? 2 : 3) : w + 1);
 }
 
-// LDS layout (bytes): plane tables [nch][6 tables][64 lanes] x 16 (lane la = 16*ga + row supplies
-// k positions 16*ga .. +15 of its row), then the per-block factors [nch][8] floats 2^(E - shift),
-// then the partial row sums of the wavefronts [16][16] floats.
-template <typename XT, typename YT>
+// LDS layout (bytes): plane tables [nch][23 pairs][T planes] x 16, one zero entry (64 bytes
+// reserved), then the per-block factors [nch][8] floats 2^(E - shift), then the partial row sums of
+// the wavefronts [16][16] floats.
+template <bool COMPACT, typename XT, typename YT>
 __global__ void __launch_bounds__(kMfmaThreads)
 gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_t* __restrict__ x,
                    YT* __restrict__ y, const void* __restrict__ bias, int bias_dtype, int n_out, int nch,
@@ -69,9 +83,11 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
   using X = Q8WX<XT>;
   constexpr int W = kMfmaWaves, T = X::kPlanes;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  const uint32_t table_bytes = (uint32_t)nch * 6u * 1024u;
-  float* tab = reinterpret_cast<float*>(smem + table_bytes);
-  float* part = reinterpret_cast<float*>(smem + table_bytes + (size_t)nch * 32);
+  constexpr uint32_t kChunkBytes = COMPACT ? kQ8WinPairs * T * 16 : 6 * 1024;
+  const uint32_t table_bytes = (uint32_t)nch * kChunkBytes;
+  const uint32_t zero_off = table_bytes;
+  float* tab = reinterpret_cast<float*>(smem + table_bytes + 64);
+  float* part = reinterpret_cast<float*>(smem + table_bytes + 64 + (size_t)nch * 32);
 
   const int SL = 1 << sl_log2, G = W >> sl_log2;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -90,7 +106,7 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
   const int last = wg_row_end - 1;   // rows past the workgroup's share re-read its last row
 
   // ---- activations: 8 values per thread and pass, requested before any weights
-  constexpr int XP = (kQ8WinMaxChunks * 256 + 8 * kMfmaThreads - 1) / (8 * kMfmaThreads);
+  constexpr int XP = ((COMPACT ? kQ8WinMaxChunks : kQ8WinMaxWideChunks) * 256 + 8 * kMfmaThreads - 1) / (8 * kMfmaThreads);
   float xf[XP][8];
 #pragma unroll
   for (int p = 0; p < XP; p++) {
@@ -118,7 +134,7 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
   {
     const v4i_t z = {0, 0, 0, 0};
     v4i_t* xa = reinterpret_cast<v4i_t*>(smem);
-    for (int e = tid; e < nch * 6 * 64; e += kMfmaThreads) xa[e] = z;
+    for (int e = tid; e < nch * (int)(kChunkBytes / 16) + 1; e += kMfmaThreads) xa[e] = z;   // + the zero entry
   }
   __syncthreads();
 
@@ -154,14 +170,15 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
         }
       }
       const int blk = k0 >> 5, ch = blk >> 3, b = blk & 7, q0 = k0 & 31;
-      const int row0 = 4 * (b & 3);
       // the 8 quants sit at chunk bytes 34b + 2 + q0 .. +7: an even start, so pairs of bytes never
       // straddle a 16-byte piece (nor a window)
 #pragma unroll
       for (int i2 = 0; i2 < 4; i2++) {
         const int byte = 34 * b + 2 + q0 + 2 * i2;
-        const int tb = q8win_table(byte, b), pos = byte & 63;
-        uint8_t* e = smem + (size_t)(((ch * 6 + tb) * 64 + 16 * (pos >> 4) + row0) * 16 + (pos & 15));
+        const int pos = byte & 63;
+        uint8_t* e = smem + (size_t)ch * kChunkBytes +
+                     (COMPACT ? (size_t)(q8win_pair(b, byte >> 4) * T * 16 + (byte & 15))
+                              : (size_t)((q8win_table(byte, b) * 64 + 16 * (pos >> 4) + 4 * (b & 3)) * 16 + (pos & 15)));
 #pragma unroll
         for (int t = 0; t < T; t++)
           *reinterpret_cast<uint16_t*>(e + 16 * t) =
@@ -190,6 +207,29 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
     }
   }
 
+  // ---- A operand addresses of this lane for the six plane MFMAs: windows 0, 1, 2 (block 3 only),
+  // 2 (blocks 4, 5), 3, 4
+  uint32_t a_base[6], a_stride[6];
+  {
+    const int slot = (lane & 15) >> 2, t = lane & 3;
+#pragma unroll
+    for (int ti = 0; ti < 6; ti++) {
+      const int wdw = ti < 2 ? ti : (ti < 4 ? 2 : ti - 1);
+      const int piece = 4 * wdw + g;
+      int off = -1;
+#pragma unroll
+      for (int hh = 0; hh < 2; hh++) {
+        const int b = slot + 4 * hh;
+        const bool in_table = ti == 2 ? b == 3 : (ti == 3 ? b >= 4 : true);
+        const bool touches = piece >= q8win_first_piece(b) && piece <= ((34 * b + 33) >> 4) && (wdw < 4 || g == 0);
+        if (t < T && in_table && touches) off = (q8win_pair(b, piece) * T + t) * 16;
+      }
+      if (!COMPACT) off = (ti * 64 + lane) * 16;
+      a_base[ti] = off >= 0 ? (uint32_t)off : zero_off;
+      a_stride[ti] = off >= 0 ? kChunkBytes : 0u;
+    }
+  }
+
   // ---- main loop
   int cr = 0, csi = 0;
   float acc = 0.f;
@@ -201,16 +241,21 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
       for (int i = 0; i < 5; i++) {
         B[i][0] = (int)s.p[i].x; B[i][1] = (int)s.p[i].y; B[i][2] = (int)s.p[i].z; B[i][3] = (int)s.p[i].w;
       }
-      const v4i_t* xe = reinterpret_cast<const v4i_t*>(smem) + (size_t)ch * 384 + lane;
+      v4i_t A[6];
+#pragma unroll
+      for (int ti = 0; ti < 6; ti++) {
+        if (COMPACT) A[ti] = *reinterpret_cast<const v4i_t*>(smem + a_base[ti] + (uint32_t)ch * a_stride[ti]);
+        else A[ti] = reinterpret_cast<const v4i_t*>(smem)[(size_t)ch * 384 + ti * 64 + lane];
+      }
       const v4i_t zero = {0, 0, 0, 0};
-      v4i_t c03 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xe[0], B[0], zero, 0, 0, 0);
-      v4i_t c47 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xe[192], B[2], zero, 0, 0, 0);
+      v4i_t c03 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[0], B[0], zero, 0, 0, 0);
+      v4i_t c47 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[3], B[2], zero, 0, 0, 0);
       v4i_t cd = __builtin_amdgcn_mfma_i32_16x16x64_i8(sel[0], B[0], zero, 0, 0, 0);
-      c03 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xe[64], B[1], c03, 0, 0, 0);
-      c47 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xe[256], B[3], c47, 0, 0, 0);
+      c03 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[1], B[1], c03, 0, 0, 0);
+      c47 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[4], B[3], c47, 0, 0, 0);
       cd = __builtin_amdgcn_mfma_i32_16x16x64_i8(sel[1], B[1], cd, 0, 0, 0);
-      c03 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xe[128], B[2], c03, 0, 0, 0);
-      c47 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xe[320], B[4], c47, 0, 0, 0);
+      c03 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[2], B[2], c03, 0, 0, 0);
+      c47 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[5], B[4], c47, 0, 0, 0);
       cd = __builtin_amdgcn_mfma_i32_16x16x64_i8(sel[2], B[2], cd, 0, 0, 0);
       cd = __builtin_amdgcn_mfma_i32_16x16x64_i8(sel[3], B[3], cd, 0, 0, 0);
       const float f0 = tab[ch * 8 + g], f1 = tab[ch * 8 + 4 + g];
@@ -276,19 +321,24 @@ static hipError_t q8win_launch_xy(const void* w, const void* x, void* y, const v
   num_wg = (int)((n_out + rows_per_wg - 1) / rows_per_wg);
   int sl_log2 = 0;
   while ((2 << sl_log2) <= W && (2 << sl_log2) <= nch && (16 * W >> (sl_log2 + 1)) >= rows_per_wg) sl_log2++;
-  const size_t lds = (size_t)nch * 6 * 1024 + (size_t)nch * 32 + 1024;
-  auto kernel = gemv_q8_win_kernel<XT, YT>;
-  static bool configured = false;
-  if (!configured) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
-  hipLaunchKernelGGL(kernel, dim3((unsigned)num_wg, (unsigned)m), dim3(W * 64), lds, s,
-                     static_cast<const uint8_t*>(w), static_cast<const typename Q8WX<XT>::elem_t*>(x),
-                     static_cast<YT*>(y), bias, bias_dtype, (int)n_out, nch, rows_per_wg, sl_log2);
-  return hipGetLastError();
+  const bool compact = nch > kQ8WinMaxWideChunks;
+  const size_t lds = (size_t)nch * (compact ? kQ8WinPairs * Q8WX<XT>::kPlanes * 16 : 6 * 1024) + 64 +
+                     (size_t)nch * 32 + 1024;
+  const auto launch = [&](auto kernel, bool& configured) -> hipError_t {
+    if (!configured) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      if (e != hipSuccess) return e;
+      configured = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3((unsigned)num_wg, (unsigned)m), dim3(W * 64), lds, s,
+                       static_cast<const uint8_t*>(w), static_cast<const typename Q8WX<XT>::elem_t*>(x),
+                       static_cast<YT*>(y), bias, bias_dtype, (int)n_out, nch, rows_per_wg, sl_log2);
+    return hipGetLastError();
+  };
+  static bool configured_wide = false, configured_compact = false;
+  if (compact) return launch(gemv_q8_win_kernel<true, XT, YT>, configured_compact);
+  return launch(gemv_q8_win_kernel<false, XT, YT>, configured_wide);
 }
 
 template <typename XT>

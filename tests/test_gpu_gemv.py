@@ -183,7 +183,7 @@ def test_q4_k_16bit_activation_extremes():
 
 @pytest.mark.parametrize("xk", ["f32", "bf16", "f16"])
 @pytest.mark.parametrize("n_out,n_in", [(70000, 128), (25600, 256), (4096 + 8, 1024), (2500, 8192), (5000, 640),
-                                        (3000, 2048), (2304, 6144), (2048 + 16, 4096), (9000, 512)])
+                                        (3000, 2048), (2304, 6144), (2048 + 16, 4096), (9000, 512), (4096, 14336), (2050, 16384)])
 def test_q8_0_work_distributions(xk, n_out, n_in):
     """Q8_0 through the matrix cores (enough rows for that kernel): every split of rows and steps
     over the wavefronts, all activation types, two activation rows of uneven magnitude."""
