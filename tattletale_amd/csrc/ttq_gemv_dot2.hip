@@ -431,6 +431,37 @@ gemv_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, 
     TTQ_TRACE_POINT(gw, 5);
   } else {
     // long rows: activations come from LDS for every unit
+    if (row_end - row0 < kBatch) {
+      // fewer rows than a batch (many CUs, few rows each): the batch runs along the row instead,
+      // kBatch groups of 64 units requested together
+      for (int row = row0; row < row_end; row++) {
+        float acc1[1] = {0.f};
+        for (int it0 = 0; it0 < nit; it0 += kBatch) {
+          typename F::Raw buf[kBatch];
+          typename F::Lane Ls[kBatch];
+#pragma unroll
+          for (int j = 0; j < kBatch; j++) {
+            const int u = min(it0 + j, nit - 1) * 64 + lane;
+            Ls[j].init(u < units ? u : 0);
+            F::fetch(buf[j], w + rb * row, Ls[j], 0xFFFFFFFFu);
+          }
+#pragma unroll
+          for (int j = 0; j < kBatch; j++) {
+            if (it0 + j < nit) {
+              uint32_t xr[32];
+              float sx[F::kSums], off[F::kSums];
+              load_x_regs(xs, it0 + j, lane, xr);
+              F::template sums<Ops>(xr, sx);
+#pragma unroll
+              for (int i = 0; i < F::kSums; i++) off[i] = kOff * sx[i];
+              acc1[0] += F::template unit_dot<Ops>(buf[j], Ls[j], xr, sx, off, magic);
+            }
+          }
+        }
+        store_rows(acc1, row);
+      }
+      return;
+    }
     for (int base = row0; base < row_end; base += kBatch) {
       float acc[kBatch];
 #pragma unroll
@@ -441,7 +472,8 @@ gemv_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, 
         Lu.init(u < units ? u : 0);
         typename F::Raw buf[kBatch];
 #pragma unroll
-        for (int r = 0; r < kBatch; r++) F::fetch(buf[r], w + rb * min(base + r, last), Lu, 0xFFFFFFFFu);
+        for (int r = 0; r < kBatch; r++)      // rows past the wavefront's share: its own last row again (cache hits)
+          F::fetch(buf[r], w + rb * min(base + r, row_end - 1), Lu, 0xFFFFFFFFu);
         uint32_t xr[32];
         float sx[F::kSums], off[F::kSums];
         load_x_regs(xs, it, lane, xr);
@@ -449,7 +481,8 @@ gemv_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, 
 #pragma unroll
         for (int i = 0; i < F::kSums; i++) off[i] = kOff * sx[i];
 #pragma unroll
-        for (int r = 0; r < kBatch; r++) acc[r] += F::template unit_dot<Ops>(buf[r], Lu, xr, sx, off, magic);
+        for (int r = 0; r < kBatch; r++)
+          if (base + r < row_end) acc[r] += F::template unit_dot<Ops>(buf[r], Lu, xr, sx, off, magic);
       }
       store_rows(acc, base);
     }
