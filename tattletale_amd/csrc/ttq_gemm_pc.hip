@@ -315,7 +315,10 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
     const int pt = tid - 256;
     // thread -> (tile row, 16-byte half of every 32-byte chunk); with BN = 112 the last 32
     // threads mirror threads 0..31 (same loads, same LDS writes of the same values)
-    const int wt = pt < 2 * BN ? pt : pt - 2 * BN;
+    // (a 64-column tile needs only half of the producer threads: the others just keep the barriers)
+    constexpr bool kSpare = 4 * BN <= 256;
+    const bool widle = kSpare && pt >= 2 * BN;
+    const int wt = pt < 2 * BN ? pt : (kSpare ? pt % (2 * BN) : pt - 2 * BN);
     const int wr = wt % BN, whalf = wt / BN;
     // clamped: rows past the end are never stored
     const int wrow = FUSE ? min(n0 + 8 * (wr >> 4) + (wr & 7), n_out - 1) + ((wr >> 3) & 1) * n_out
@@ -326,11 +329,13 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
     const int wj = wr >> 4, wn = wr & 15;
     const uint32_t sw_addr = (uint32_t)(size_t)(lptr_t)(&sw[0]);
     auto load_w = [&](WRaw& dst, int b) {
+      if (widle) return;
       // past the end: a harmless re-read
       WF::load(dst, wptr + WF::kUnitBytes * (int64_t)min(b, nblocks - 1), whalf);
     };
     auto dequant_to_lds = [&](const WRaw& r, auto cc, int buf) {
       constexpr int c = decltype(cc)::value;
+      if (widle) return;
       uint32_t lo[8], hi[8];
       WF::template dequant<c>(r, whalf, lo, hi);
       if constexpr (WF::kWholeKsub) {
@@ -566,10 +571,10 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
   }
 }
 
-template <int FMT, int MB, bool FUSE>
-static hipError_t launch_pc_112(const uint8_t* wb, const uint16_t* x, void* y, int y_dtype, const void* bias,
-                                int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
-  constexpr int NJ = 7, BO = FUSE ? NJ * 8 : NJ * 16, BM = pc_bm(MB);
+template <int FMT, int MB, int NJ, bool FUSE>
+static hipError_t launch_pc_tile(const uint8_t* wb, const uint16_t* x, void* y, int y_dtype, const void* bias,
+                                 int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+  constexpr int BO = FUSE ? NJ * 8 : NJ * 16, BM = pc_bm(MB);
   const int n_tiles = (int)((n_out + BO - 1) / BO), m_tiles = (int)((m + BM - 1) / BM);
   int xcds_per_mtile = 0;
   unsigned nwg = (unsigned)(n_tiles * m_tiles);
@@ -582,17 +587,55 @@ static hipError_t launch_pc_112(const uint8_t* wb, const uint16_t* x, void* y, i
   return hipGetLastError();
 }
 
-// Few rows (up to kPcSkinnyRows) take 64-row tiles: a quarter of the MFMA and activation traffic
-// per step, and twice the workgroups when there are more than 64 rows.
-static const int64_t kPcSkinnyRows = [] { const char* e = getenv("TTQ_GEMM_SKINNY_ROWS"); return e ? atoi(e) : 128; }();
+// Tile choice.  A workgroup owns 64*MB rows x 16*NJ columns (8*NJ outputs when fused); the grid
+// should fill the 256 CUs without a nearly empty last round.  Cost model: rounds of workgroups x
+// (64-k steps x time per step of the tile shape + a fixed cost per workgroup), both measured
+// (microseconds; 14336 x 4096 and x 8192 at 2048 rows).  Smaller tiles are cheaper per step --
+// down to the latency of the producers' load / dequantize / store / barrier chain, about 0.45 us
+// -- but dequantize every weight for fewer rows.
+struct PcTile { int mb, nj; float step_us; };
+static const PcTile kPcTiles[] = {{4, 7, 0.87f}, {4, 4, 0.68f}, {2, 7, 0.585f}, {2, 4, 0.55f}, {1, 7, 0.46f}, {1, 4, 0.52f}};
+constexpr float kPcFixedUs = 6.f;
+
+static int pc_choose_tile(int64_t m, int64_t n_out, int64_t n_in, bool fuse) {
+  static const int forced = [] { const char* e = getenv("TTQ_GEMM_TILE"); return e ? atoi(e) : -1; }();
+  if (forced >= 0 && forced < (int)(sizeof(kPcTiles) / sizeof(kPcTiles[0]))) return forced;
+  int cus = 256;
+  {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    static int cached = 0;
+    if (cached == 0 && hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      cached = prop.multiProcessorCount;
+    if (cached > 0) cus = cached;
+  }
+  int best = 0;
+  float best_cost = 1e30f;
+  for (int i = 0; i < (int)(sizeof(kPcTiles) / sizeof(kPcTiles[0])); i++) {
+    const PcTile& t = kPcTiles[i];
+    const int64_t bo = fuse ? t.nj * 8 : t.nj * 16, bm = pc_bm(t.mb);
+    const int64_t wgs = ((n_out + bo - 1) / bo) * ((m + bm - 1) / bm);
+    const int64_t rounds = (wgs + cus - 1) / cus;
+    const float cost = (float)rounds * ((float)(n_in / 64) * t.step_us + kPcFixedUs);
+    if (cost < best_cost * 0.999f) { best_cost = cost; best = i; }
+  }
+  return best;
+}
+
 template <int FMT, bool FUSE>
 static hipError_t launch_pc_fmt(const uint8_t* wb, const uint16_t* x, void* y, int y_dtype, const void* bias,
                                 int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
-  if (m <= kPcSkinnyRows) return launch_pc_112<FMT, 1, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-  return launch_pc_112<FMT, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  switch (pc_choose_tile(m, n_out, n_in, FUSE)) {
+    case 0: return launch_pc_tile<FMT, 4, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case 1: return launch_pc_tile<FMT, 4, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case 2: return launch_pc_tile<FMT, 2, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case 3: return launch_pc_tile<FMT, 2, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case 4: return launch_pc_tile<FMT, 1, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    default: return launch_pc_tile<FMT, 1, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  }
 }
 
-// Only the 112-column tile is built in this form: with 128 columns the consumers' 128
+// 112- and 64-column tiles are built in this form: with 128 columns the consumers' 128
 // accumulator registers plus the fragment rings do not fit the 168 registers a wavefront gets
 // when twelve of them share a CU.
 bool gemm_pc_supported(int format, int64_t m, int64_t n_out, int64_t n_in, int bn) {
