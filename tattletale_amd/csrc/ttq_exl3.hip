@@ -124,15 +124,18 @@ __device__ __forceinline__ void fwht128_quad(float (&v)[4], int lane) {
 // combined across slots with lane shuffles and across waves through LDS.
 // The packed bits of a lane's first kPre tiles are requested before anything else, so that they
 // travel while the activations are loaded and rotated; later tiles are requested one batch ahead.
-template <int BITS, int CB, typename XT>
+// TOK activation rows ("tokens") per workgroup: decoding a weight costs about ten vector-ALU
+// issue slots, multiplying it one per token, so the decode is shared by up to eight tokens
+// (blockIdx.y walks the groups of TOK tokens; the last group may hold fewer).
+template <int BITS, int CB, typename XT, int TOK>
 __global__ void __launch_bounds__(kExl3Threads)
 gemv_exl3_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __restrict__ suh,
-                 const XT* __restrict__ x, float* __restrict__ y, int n_out, int n_in) {
-  extern __shared__ float xs[];          // n_in rotated activations, then kExl3Waves*16 partials
+                 const XT* __restrict__ x, float* __restrict__ y, int m, int n_out, int n_in) {
+  extern __shared__ float xs[];          // TOK x n_in rotated activations, then kExl3Waves*16*TOK partials
   constexpr int kPre = 4;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const XT* xm = x + (int64_t)blockIdx.y * n_in;
-  float* ym = y + (int64_t)blockIdx.y * n_out;
+  const int t0 = blockIdx.y * TOK;
+  const int ntok = min(TOK, m - t0);       // tokens of this group that exist
   const int nt = blockIdx.x, nt_n = n_out >> 4, kt_n = n_in >> 4;
   const int g = lane >> 4, j = lane & 15;
   const int kt0 = wave * 4 + g;
@@ -150,16 +153,27 @@ gemv_exl3_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __restric
 
   // input side: x o suh, then the Hadamard rotation of every group of 128 (32 lanes x 4 values)
   for (int k4 = tid * 4; k4 < n_in; k4 += kExl3Threads * 4) {
-    float v[4];
+    float sg[4];
 #pragma unroll
-    for (int i = 0; i < 4; i++) v[i] = XElem<XT>::load(xm, k4 + i) * f16_bits_to_f32(suh[k4 + i]);
-    fwht128_quad(v, lane);
-    *reinterpret_cast<float4*>(xs + k4) = make_float4(v[0], v[1], v[2], v[3]);
+    for (int i = 0; i < 4; i++) sg[i] = f16_bits_to_f32(suh[k4 + i]);
+#pragma unroll
+    for (int t = 0; t < TOK; t++) {
+      if (t < ntok) {          // uniform; no `break`, so that the loop unrolls and acc[] stays in registers
+        const XT* xm = x + (int64_t)(t0 + t) * n_in;
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) v[i] = XElem<XT>::load(xm, k4 + i) * sg[i];
+        fwht128_quad(v, lane);
+        *reinterpret_cast<float4*>(xs + (size_t)t * n_in + k4) = make_float4(v[0], v[1], v[2], v[3]);
+      }
+    }
   }
   __syncthreads();
   const float kNorm = 0.08838834764831845f;  // 1/sqrt(128), applied to the dot product
 
-  float acc = 0.f;
+  float acc[TOK];
+#pragma unroll
+  for (int t = 0; t < TOK; t++) acc[t] = 0.f;
   for (int ktb = kt0; ktb < kt_n; ktb += kPre * kStride) {
     LaneBits<BITS> nxt[kPre];
     const bool more = ktb + kPre * kStride < kt_n;
@@ -170,14 +184,24 @@ gemv_exl3_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __restric
       if (kt < kt_n) {
         _Float16 v[16];
         DecodeLoop<BITS, CB, 0>::run(cur[i], v);
-        const float4* xv = reinterpret_cast<const float4*>(xs + 16 * kt);
+        float vf[16];
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-          const float4 xq = xv[q];
-          acc = fmaf_((float)v[4 * q + 0], xq.x, acc);
-          acc = fmaf_((float)v[4 * q + 1], xq.y, acc);
-          acc = fmaf_((float)v[4 * q + 2], xq.z, acc);
-          acc = fmaf_((float)v[4 * q + 3], xq.w, acc);
+        for (int e = 0; e < 16; e++) vf[e] = (float)v[e];
+#pragma unroll
+        for (int t = 0; t < TOK; t++) {
+          if (t < ntok) {
+            const float4* xv = reinterpret_cast<const float4*>(xs + (size_t)t * n_in + 16 * kt);
+            float a = acc[t];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+              const float4 xq = xv[q];
+              a = fmaf_(vf[4 * q + 0], xq.x, a);
+              a = fmaf_(vf[4 * q + 1], xq.y, a);
+              a = fmaf_(vf[4 * q + 2], xq.z, a);
+              a = fmaf_(vf[4 * q + 3], xq.w, a);
+            }
+            acc[t] = a;
+          }
         }
       }
     }
@@ -186,16 +210,21 @@ gemv_exl3_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __restric
       for (int i = 0; i < kPre; i++) cur[i] = nxt[i];
     }
   }
-  acc += __shfl_xor(acc, 16, kWave);
-  acc += __shfl_xor(acc, 32, kWave);
-  float* red = xs + n_in;
-  if (lane < 16) red[wave * 16 + lane] = acc;
+  float* red = xs + (size_t)TOK * n_in;
+#pragma unroll
+  for (int t = 0; t < TOK; t++) {
+    float a = acc[t];
+    a += __shfl_xor(a, 16, kWave);
+    a += __shfl_xor(a, 32, kWave);
+    if (lane < 16) red[(t * kExl3Waves + wave) * 16 + lane] = a;
+  }
   __syncthreads();
-  if (tid < 16) {
+  if (tid < 16 * TOK) {
+    const int t = tid >> 4, c = tid & 15;
     float s = 0.f;
 #pragma unroll
-    for (int wv = 0; wv < kExl3Waves; wv++) s += red[wv * 16 + tid];
-    ym[nt * 16 + tid] = s * kNorm;
+    for (int wv = 0; wv < kExl3Waves; wv++) s += red[(t * kExl3Waves + wv) * 16 + c];
+    if (t0 + t < m) y[(int64_t)(t0 + t) * n_out + nt * 16 + c] = s * kNorm;
   }
 }
 
@@ -278,27 +307,45 @@ hipError_t launch_dequant_exl3(const uint16_t* trellis, uint16_t* out_f16, int64
   }
 }
 
+constexpr int kExl3Tok = 8;              // tokens per workgroup when there are several and they fit LDS
+template <int BITS, int CB, typename XT, int TOK>
+static hipError_t gemv_bits_cb_t(const uint16_t* trellis, const uint16_t* suh, const void* x, float* y, int64_t m,
+                                 int64_t n_out, int64_t n_in, hipStream_t s) {
+  const dim3 grid((unsigned)(n_out / 16), (unsigned)((m + TOK - 1) / TOK)), block(kExl3Threads);
+  const size_t lds = ((size_t)TOK * n_in + (size_t)kExl3Waves * 16 * TOK) * sizeof(float);
+  auto kernel = gemv_exl3_kernel<BITS, CB, XT, TOK>;
+  if (lds > 64 * 1024) {
+    static bool configured = false;
+    if (!configured) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      if (e != hipSuccess) return e;
+      configured = true;
+    }
+  }
+  hipLaunchKernelGGL(kernel, grid, block, lds, s, trellis, suh, static_cast<const XT*>(x), y, (int)m, (int)n_out,
+                     (int)n_in);
+  return hipGetLastError();
+}
+
+template <int BITS, int CB, typename XT>
+static hipError_t gemv_bits_cb_x(const uint16_t* trellis, const uint16_t* suh, const void* x, float* y, int64_t m,
+                                 int64_t n_out, int64_t n_in, hipStream_t s) {
+  const size_t lds8 = ((size_t)kExl3Tok * n_in + (size_t)kExl3Waves * 16 * kExl3Tok) * sizeof(float);
+  if (m >= 2 && lds8 <= 150 * 1024)
+    return gemv_bits_cb_t<BITS, CB, XT, kExl3Tok>(trellis, suh, x, y, m, n_out, n_in, s);
+  return gemv_bits_cb_t<BITS, CB, XT, 1>(trellis, suh, x, y, m, n_out, n_in, s);
+}
+
 template <int BITS, int CB>
 static hipError_t gemv_bits_cb(const uint16_t* trellis, const uint16_t* suh, const void* x, int x_dtype,
                                float* y, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
-  const dim3 grid((unsigned)(n_out / 16), (unsigned)m), block(kExl3Threads);
-  const size_t lds = ((size_t)n_in + kExl3Waves * 16) * sizeof(float);
   switch (x_dtype) {
-    case kF32:
-      hipLaunchKernelGGL((gemv_exl3_kernel<BITS, CB, float>), grid, block, lds, s, trellis, suh,
-                         static_cast<const float*>(x), y, (int)n_out, (int)n_in);
-      break;
-    case kF16:
-      hipLaunchKernelGGL((gemv_exl3_kernel<BITS, CB, f16_tag>), grid, block, lds, s, trellis, suh,
-                         static_cast<const f16_tag*>(x), y, (int)n_out, (int)n_in);
-      break;
-    case kBF16:
-      hipLaunchKernelGGL((gemv_exl3_kernel<BITS, CB, bf16_tag>), grid, block, lds, s, trellis, suh,
-                         static_cast<const bf16_tag*>(x), y, (int)n_out, (int)n_in);
-      break;
+    case kF32: return gemv_bits_cb_x<BITS, CB, float>(trellis, suh, x, y, m, n_out, n_in, s);
+    case kF16: return gemv_bits_cb_x<BITS, CB, f16_tag>(trellis, suh, x, y, m, n_out, n_in, s);
+    case kBF16: return gemv_bits_cb_x<BITS, CB, bf16_tag>(trellis, suh, x, y, m, n_out, n_in, s);
     default: return hipErrorInvalidValue;
   }
-  return hipGetLastError();
 }
 
 template <int BITS>

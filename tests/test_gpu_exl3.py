@@ -57,3 +57,22 @@ def test_full_shape_exl3_4096x4096():
     y = QL.gemv_exl3(packed_to_dev(tr), bits_to_dev(suh, "f16"), bits_to_dev(svh, "f16"),
                      bits_to_dev(x, "f16"), cfg.n_out, cfg.n_in, cfg.bits, F.CB_MCG).cpu().numpy()[0]
     assert rel_l2(y, oracle.exl3_gemv_f64(T, suh, svh, x)) <= TOL
+
+
+@pytest.mark.parametrize("m", [2, 8, 9, 19])
+def test_exl3_several_rows_share_the_decode(m):
+    """Several activation rows in one call (the trellis is decoded once per eight rows): each row
+    against the oracle, and bit for bit equal to the same row on its own."""
+    n_out, n_in, bits = 384, 1024, 3
+    w = Q.fill_normal(520, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
+    tr, suh, svh = Q.quantize_exl3(w, bits, F.CB_MCG, seed=2)
+    T = oracle.exl3_decode(tr, n_out, n_in, bits, F.CB_MCG)
+    x = Q.f32_to_f16(Q.fill_normal(521 + m, 1, 1.0, m * n_in).reshape(m, n_in))
+    trd, sud, svd, xd = packed_to_dev(tr), bits_to_dev(suh, "f16"), bits_to_dev(svh, "f16"), bits_to_dev(x, "f16")
+    y = QL.gemv_exl3(trd, sud, svd, xd, n_out, n_in, bits, F.CB_MCG)
+    assert y.shape == (m, n_out)
+    for i in range(m):
+        assert rel_l2(y[i].cpu().numpy(), oracle.exl3_gemv_f64(T, suh, svh, x[i])) <= TOL
+    for i in {0, m // 2, m - 1}:
+        y1 = QL.gemv_exl3(trd, sud, svd, xd[i:i + 1], n_out, n_in, bits, F.CB_MCG)
+        assert torch.equal(y1[0], y[i])
