@@ -273,23 +273,22 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
         layer->bias_dtype, m, n_out, n_in, layer->bits, layer->codebook, s));
   }
 
-  // Prefill: MFMA kernel for Q4_K with bf16 activations once there are enough rows to fill a tile.
-  // (a few rows more than that still go through the batched decode kernel when it applies)
-  const bool few_rows = (m <= ttq::kBatchGemvMaxRows &&
-                         ttq::gemv_q4k_batch_supported(layer->format, x_dtype, m, n_out, n_in)) ||
-                        (m <= ttq::kBatch4GemvMaxRows &&
-                         ttq::gemv_q4k_batch4_supported(layer->format, x_dtype, m, n_out, n_in));
-  if (layer->format == TTQ_Q4_K && x_dtype == TTQ_BF16 && m >= 16 && !few_rows &&
-      (y_dtype == TTQ_BF16 || y_dtype == TTQ_F32)) {
-    return hip_status(ttq::launch_gemm_q4k(layer->qweight, static_cast<const uint16_t*>(x), y, y_dtype,
-                                           layer->bias, layer->bias_dtype, m, n_out, n_in, s));
-  }
-  // Q6_K / Q8_0 have no few-row decode kernel: from eight rows on the 64-row GEMM tile is faster
-  // than one GEMV pass per row
-  if ((layer->format == TTQ_Q6_K || layer->format == TTQ_Q8_0) && x_dtype == TTQ_BF16 && m >= 8 &&
-      (y_dtype == TTQ_BF16 || y_dtype == TTQ_F32) && ttq::gemm_pc_supported(layer->format, m, n_out, n_in, 112)) {
-    return hip_status(ttq::launch_gemm_pc(layer->format, layer->qweight, static_cast<const uint16_t*>(x), y,
-                                          y_dtype, layer->bias, layer->bias_dtype, m, n_out, n_in, s));
+  // Several rows of bf16 activations: the prefill GEMM (weights rounded to bf16) or a few passes of
+  // the decode kernels (fp32 scales), whichever the shape makes cheaper.  Up to four rows always
+  // decode; a GEMV that the row length rules out leaves only the GEMM.
+  const bool gemm_ok = x_dtype == TTQ_BF16 && (y_dtype == TTQ_BF16 || y_dtype == TTQ_F32) &&
+                       (layer->format == TTQ_Q4_K || layer->format == TTQ_Q6_K || layer->format == TTQ_Q8_0) &&
+                       ttq::gemm_pc_supported(layer->format, m, n_out, n_in, 112);
+  if (gemm_ok && m >= 5) {
+    const bool gemv_ok = check_gemv_limits(x_dtype, n_in) == TTQ_OK;
+    if (!gemv_ok || ttq::gemm_pc_estimate_us(layer->format, m, n_out, n_in) <
+                        ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in)) {
+      if (layer->format == TTQ_Q4_K)
+        return hip_status(ttq::launch_gemm_q4k(layer->qweight, static_cast<const uint16_t*>(x), y, y_dtype,
+                                               layer->bias, layer->bias_dtype, m, n_out, n_in, s));
+      return hip_status(ttq::launch_gemm_pc(layer->format, layer->qweight, static_cast<const uint16_t*>(x), y,
+                                            y_dtype, layer->bias, layer->bias_dtype, m, n_out, n_in, s));
+    }
   }
   const int lim = check_gemv_limits(x_dtype, n_in);
   if (lim != TTQ_OK) return lim;

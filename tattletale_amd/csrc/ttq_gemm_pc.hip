@@ -597,9 +597,8 @@ struct PcTile { int mb, nj; float step_us; };
 static const PcTile kPcTiles[] = {{4, 7, 0.87f}, {4, 4, 0.68f}, {2, 7, 0.585f}, {2, 4, 0.55f}, {1, 7, 0.46f}, {1, 4, 0.52f}};
 constexpr float kPcFixedUs = 6.f;
 
-static int pc_choose_tile(int64_t m, int64_t n_out, int64_t n_in, bool fuse) {
+static int pc_choose_tile(int64_t m, int64_t n_out, int64_t n_in, bool fuse, float* cost_us = nullptr) {
   static const int forced = [] { const char* e = getenv("TTQ_GEMM_TILE"); return e ? atoi(e) : -1; }();
-  if (forced >= 0 && forced < (int)(sizeof(kPcTiles) / sizeof(kPcTiles[0]))) return forced;
   int cus = 256;
   {
     int dev = 0;
@@ -612,6 +611,7 @@ static int pc_choose_tile(int64_t m, int64_t n_out, int64_t n_in, bool fuse) {
   int best = 0;
   float best_cost = 1e30f;
   for (int i = 0; i < (int)(sizeof(kPcTiles) / sizeof(kPcTiles[0])); i++) {
+    if (forced >= 0 && forced < (int)(sizeof(kPcTiles) / sizeof(kPcTiles[0])) && i != forced) continue;
     const PcTile& t = kPcTiles[i];
     const int64_t bo = fuse ? t.nj * 8 : t.nj * 16, bm = pc_bm(t.mb);
     const int64_t wgs = ((n_out + bo - 1) / bo) * ((m + bm - 1) / bm);
@@ -619,7 +619,16 @@ static int pc_choose_tile(int64_t m, int64_t n_out, int64_t n_in, bool fuse) {
     const float cost = (float)rounds * ((float)(n_in / 64) * t.step_us + kPcFixedUs);
     if (cost < best_cost * 0.999f) { best_cost = cost; best = i; }
   }
+  if (cost_us) *cost_us = best_cost;
   return best;
+}
+
+// Rough time of the GEMM for this shape (microseconds), for callers that can also run the
+// operator as a few GEMV passes.  The Q6_K and Q8_0 producers are slower than the Q4_K one.
+float gemm_pc_estimate_us(int format, int64_t m, int64_t n_out, int64_t n_in) {
+  float c = 0.f;
+  pc_choose_tile(m, n_out, n_in, false, &c);
+  return c * (format == kQ8_0 ? 2.1f : (format == kQ6_K ? 1.5f : 1.f)) + 2.f;
 }
 
 template <int FMT, bool FUSE>

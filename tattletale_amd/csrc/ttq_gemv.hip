@@ -344,6 +344,8 @@ hipError_t launch_gemv(int format, const void* w, const void* x, int x_dtype, vo
   if (gemv_q4k_batch_supported(format, x_dtype, m, n_out, n_in))
     return launch_gemv_q4k_batch(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   if (b4) return launch_gemv_q4k_batch4(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  if (gemv_dot2_multi_supported(format, x_dtype, m, n_in))
+    return launch_gemv_dot2_multi(format, w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   if (gemv_mfma_supported(format, x_dtype, n_out, n_in))
     return launch_gemv_mfma(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   if (gemv_q8_win_supported(format, n_out, n_in))
@@ -358,6 +360,29 @@ hipError_t launch_gemv(int format, const void* w, const void* x, int x_dtype, vo
     case kQ6_K: return launch_generic_xy<FmtQ6_K>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
     default: return hipErrorInvalidValue;
   }
+}
+
+
+// Rough time (microseconds) of launch_gemv for m >= 2 activation rows, following the dispatch
+// above: passes over the weights x (packed megabytes / measured rate of the kernel that runs
+// + a fixed cost).  ttq_linear_forward weighs it against the prefill GEMM.
+float gemv_estimate_us(int format, int x_dtype, int64_t m, int64_t n_out, int64_t n_in) {
+  const int64_t per = format == kQ8_0 ? 32 : 256, blk = format == kQ8_0 ? 34 : (format == kQ4_K ? 144 : 210);
+  const float mb = (float)(n_out * (n_in / per) * blk) * 1e-6f;
+  const bool b4 = gemv_q4k_batch4_supported(format, x_dtype, m, n_out, n_in);
+  if (b4 && m <= 4) return mb / 2.75f + 2.f;
+  if (gemv_q4k_batch_supported(format, x_dtype, m, n_out, n_in)) {
+    const int tok = gemv_q4k_batch_tokens(m, n_in);
+    return (float)((m + tok - 1) / tok) * (mb / (tok == 16 ? 1.73f : 2.4f) + 2.f);
+  }
+  if (b4) return (float)((m + 3) / 4) * (mb / 2.4f + 2.f);
+  if (gemv_dot2_multi_supported(format, x_dtype, m, n_in))
+    return m <= 2 ? mb / 2.6f + 2.f : (float)((m + 3) / 4) * (mb / 1.7f + 2.f);
+  if (gemv_q8_win_supported(format, n_out, n_in)) {
+    const int tok = gemv_q8_win_tokens(x_dtype, m, n_in);
+    return (float)((m + tok - 1) / tok) * (mb / (tok == 4 ? 3.1f : 3.6f) + 2.f);
+  }
+  return (float)m * (mb / 3.2f + 3.f);
 }
 
 }  // namespace ttq

@@ -489,6 +489,112 @@ gemv_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, 
   }
 }
 
+// ------------------------------------------------------------------------------ a few rows at once
+// The same arithmetic for TOK activation rows ("tokens") per pass over the weights: the activations
+// of all tokens are staged in LDS as permuted pairs, a unit's packed bytes are loaded and unpacked
+// once (the unpacking of unit_dot is common to the TOK calls and is shared by the compiler), and
+// only the dot products and the per-token offsets repeat.  A pass costs about 1.4 times a
+// single-row pass for two tokens and 2.2 times for four.  blockIdx.y walks the groups of TOK
+// tokens; tokens past the end re-read the last one and are not stored.
+template <class F, class Ops, typename YT, int TOK>
+__global__ void __launch_bounds__(kFastThreads)
+gemv_dot2_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
+                       const void* __restrict__ bias, int bias_dtype, int m, int n_out, int n_in,
+                       int rows_per_wave) {
+  extern __shared__ uint32_t xs[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int t0 = blockIdx.y * TOK;
+  const int units = n_in >> 6;
+  const int nit = (units + 63) >> 6;
+  const int tok_dwords = nit * 2048;            // LDS dwords per token
+  const int64_t rb = F::row_bytes(n_in);
+  const int gw = blockIdx.x * kFastWaves + wave;
+  const int row0 = gw * rows_per_wave;
+  const int row_end = min(row0 + rows_per_wave, n_out);
+
+  // stage the activations: one 16-byte load (8 activations) per thread, token and pass
+  for (int k0 = 8 * tid; k0 < nit * 4096; k0 += kStageChunk) {
+    uint4 xv[TOK];
+#pragma unroll
+    for (int t = 0; t < TOK; t++) {
+      const uint4 v = *reinterpret_cast<const uint4*>(x + (int64_t)min(t0 + t, m - 1) * n_in + (k0 < n_in ? k0 : 0));
+      xv[t] = k0 < n_in ? v : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int t = 0; t < TOK; t++) F::stage(xs + t * tok_dwords, k0, xv[t]);
+  }
+  __syncthreads();
+
+  const uint32_t magic = opaque_vgpr(Ops::kMagic);
+  constexpr float kOff = Ops::kOffset + ExtraOffset<F>::value;
+  auto store = [&](int row, int t, float v) {
+    v = wave_sum_to_lane63(v);
+    if (lane == 63 && row < row_end && t0 + t < m)
+      YElem<YT>::store(y + (int64_t)(t0 + t) * n_out, row, v + load_bias(bias, bias_dtype, row));
+  };
+  // dot products of one unit of one row with every token
+  auto unit_tokens = [&](const typename F::Raw& buf, const typename F::Lane& Lu, int it, float (&acc)[TOK]) {
+#pragma unroll
+    for (int t = 0; t < TOK; t++) {
+      uint32_t xr[32];
+      float sx[F::kSums], off[F::kSums];
+      load_x_regs(xs + t * tok_dwords, it, lane, xr);
+      F::template sums<Ops>(xr, sx);
+#pragma unroll
+      for (int i = 0; i < F::kSums; i++) off[i] = kOff * sx[i];
+      acc[t] += F::template unit_dot<Ops>(buf, Lu, xr, sx, off, magic);
+    }
+  };
+
+  if (row_end - row0 < kBatch) {
+    // few rows per wavefront: the batch runs along the row, kBatch groups of 64 units at a time
+    for (int row = row0; row < row_end; row++) {
+      float acc[TOK];
+#pragma unroll
+      for (int t = 0; t < TOK; t++) acc[t] = 0.f;
+      for (int it0 = 0; it0 < nit; it0 += kBatch) {
+        typename F::Raw buf[kBatch];
+        typename F::Lane Ls[kBatch];
+#pragma unroll
+        for (int j = 0; j < kBatch; j++) {
+          const int u = min(it0 + j, nit - 1) * 64 + lane;
+          Ls[j].init(u < units ? u : 0);
+          F::fetch(buf[j], w + rb * row, Ls[j], 0xFFFFFFFFu);
+        }
+#pragma unroll
+        for (int j = 0; j < kBatch; j++)
+          if (it0 + j < nit) unit_tokens(buf[j], Ls[j], it0 + j, acc);
+      }
+#pragma unroll
+      for (int t = 0; t < TOK; t++) store(row, t, acc[t]);
+    }
+    return;
+  }
+  for (int base = row0; base < row_end; base += kBatch) {
+    float acc[kBatch][TOK];
+#pragma unroll
+    for (int r = 0; r < kBatch; r++)
+#pragma unroll
+      for (int t = 0; t < TOK; t++) acc[r][t] = 0.f;
+    for (int it = 0; it < nit; it++) {
+      const int u = it * 64 + lane;
+      typename F::Lane Lu;
+      Lu.init(u < units ? u : 0);
+      typename F::Raw buf[kBatch];
+#pragma unroll
+      for (int r = 0; r < kBatch; r++) F::fetch(buf[r], w + rb * min(base + r, row_end - 1), Lu, 0xFFFFFFFFu);
+#pragma unroll
+      for (int r = 0; r < kBatch; r++)
+        if (base + r < row_end) unit_tokens(buf[r], Lu, it, acc[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < kBatch; r++)
+#pragma unroll
+      for (int t = 0; t < TOK; t++) store(base + r, t, acc[r][t]);
+  }
+}
+
 // ------------------------------------------------------------------------------ launch
 static int num_cus() {
   static int cached = 0;
@@ -557,6 +663,80 @@ hipError_t launch_gemv_dot2(int format, const void* w, const void* x, int x_dtyp
   } else if (format == kQ6_K) {
     if (x_dtype == kBF16) return launch_fmt_y<DotQ6K, OpsBF16>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
     if (x_dtype == kF16) return launch_fmt_y<DotQ6K, OpsF16>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  }
+  return hipErrorInvalidValue;
+}
+
+
+// ---- launch of the few-rows kernel
+template <class F, class Ops, typename YT, int TOK>
+static hipError_t launch_multi_t(const void* w, const void* x, void* y, const void* bias, int bias_dtype,
+                                 int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+  const int units = (int)(n_in / 64);
+  const int nit = (units + 63) / 64;
+  int64_t waves = (int64_t)num_cus() * kFastWaves;
+  if (waves > n_out) waves = n_out;
+  const int rows_per_wave = (int)((n_out + waves - 1) / waves);
+  const int64_t used_waves = (n_out + rows_per_wave - 1) / rows_per_wave;
+  const dim3 grid((unsigned)((used_waves + kFastWaves - 1) / kFastWaves), (unsigned)((m + TOK - 1) / TOK)),
+      block(kFastThreads);
+  const size_t lds = (size_t)TOK * nit * 2048 * sizeof(uint32_t);
+  auto kernel = gemv_dot2_multi_kernel<F, Ops, YT, TOK>;
+  static bool configured = false;
+  if (lds > 64 * 1024 && !configured) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
+  hipLaunchKernelGGL(kernel, grid, block, lds, s, static_cast<const uint8_t*>(w), static_cast<const uint16_t*>(x),
+                     static_cast<YT*>(y), bias, bias_dtype, (int)m, (int)n_out, (int)n_in, rows_per_wave);
+  return hipGetLastError();
+}
+
+template <class F, class Ops, int TOK>
+static hipError_t launch_multi_y(const void* w, const void* x, void* y, int y_dtype, const void* bias,
+                                 int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+  switch (y_dtype) {
+    case kF32: return launch_multi_t<F, Ops, float, TOK>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kF16: return launch_multi_t<F, Ops, f16_tag, TOK>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kBF16: return launch_multi_t<F, Ops, bf16_tag, TOK>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+template <class F, int TOK>
+static hipError_t launch_multi_x(const void* w, const void* x, int x_dtype, void* y, int y_dtype, const void* bias,
+                                 int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+  if (x_dtype == kBF16) return launch_multi_y<F, OpsBF16, TOK>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  if (x_dtype == kF16) return launch_multi_y<F, OpsF16, TOK>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  return hipErrorInvalidValue;
+}
+
+// Four tokens per pass while their staged activations fit LDS (n_in <= 16384), else two.
+static int multi_tokens(int64_t m, int64_t n_in) {
+  const int nit = (int)((n_in / 64 + 63) / 64);
+  const size_t per_tok = (size_t)nit * 2048 * sizeof(uint32_t);
+  if (m > 2 && 4 * per_tok <= 150 * 1024) return 4;
+  return 2 * per_tok <= 150 * 1024 ? 2 : 0;
+}
+
+bool gemv_dot2_multi_supported(int format, int x_dtype, int64_t m, int64_t n_in) {
+  static const int disabled = env_int("TTQ_GEMV_NO_BATCH", 0);
+  return !disabled && m >= 2 && gemv_dot2_supported(format, x_dtype, n_in) && multi_tokens(m, n_in) != 0;
+}
+
+hipError_t launch_gemv_dot2_multi(int format, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                                  const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                                  hipStream_t s) {
+  const int tok = multi_tokens(m, n_in);
+  if (format == kQ6_K) {
+    if (tok == 4) return launch_multi_x<DotQ6K, 4>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    return launch_multi_x<DotQ6K, 2>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  }
+  if (format == kQ4_K) {
+    if (tok == 4) return launch_multi_x<DotQ4K, 4>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    return launch_multi_x<DotQ4K, 2>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   }
   return hipErrorInvalidValue;
 }

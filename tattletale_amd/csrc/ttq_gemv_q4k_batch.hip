@@ -375,6 +375,8 @@ static int batch_tokens(int64_t m, int64_t n_in) {
   return fits8 ? 8 : 0;
 }
 
+int gemv_q4k_batch_tokens(int64_t m, int64_t n_in) { return batch_tokens(m, n_in); }
+
 bool gemv_q4k_batch_supported(int format, int x_dtype, int64_t m, int64_t n_out, int64_t n_in) {
   static const int disabled = mfma_env_int("TTQ_GEMV_NO_BATCH", 0) || mfma_env_int("TTQ_GEMV_NO_MFMA", 0);
   // one staging pass of 8 activations per thread; 32-bit byte offsets into the weights

@@ -75,19 +75,25 @@ __device__ __forceinline__ int q8win_table(int byte, int b) {
 // LDS layout (bytes): plane tables [nch][23 pairs][T planes] x 16, one zero entry (64 bytes
 // reserved), then the per-block factors [nch][8] floats 2^(E - shift), then the partial row sums of
 // the wavefronts [16][16] floats.
-template <bool COMPACT, typename XT, typename YT>
+// TOK activation rows ("tokens") per pass over the weights (compact tables only when TOK > 1): the
+// B operands and the scale MFMAs are shared, every token has its own plane tables, six plane
+// MFMAs and two scalings per step.  blockIdx.y walks the groups of TOK tokens; tokens past the
+// end re-read the last one and are not stored.
+template <bool COMPACT, int TOK, typename XT, typename YT>
 __global__ void __launch_bounds__(kMfmaThreads)
 gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_t* __restrict__ x,
-                   YT* __restrict__ y, const void* __restrict__ bias, int bias_dtype, int n_out, int nch,
+                   YT* __restrict__ y, const void* __restrict__ bias, int bias_dtype, int m, int n_out, int nch,
                    int rows_per_wg, int sl_log2) {
+  static_assert(COMPACT || TOK == 1, "several tokens use the compact tables");
   using X = Q8WX<XT>;
   constexpr int W = kMfmaWaves, T = X::kPlanes;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   constexpr uint32_t kChunkBytes = COMPACT ? kQ8WinPairs * T * 16 : 6 * 1024;
-  const uint32_t table_bytes = (uint32_t)nch * kChunkBytes;
+  const uint32_t tok_bytes = (uint32_t)nch * kChunkBytes;          // plane tables of one token
+  const uint32_t table_bytes = TOK * tok_bytes;
   const uint32_t zero_off = table_bytes;
-  float* tab = reinterpret_cast<float*>(smem + table_bytes + 64);
-  float* part = reinterpret_cast<float*>(smem + table_bytes + 64 + (size_t)nch * 32);
+  float* tab = reinterpret_cast<float*>(smem + table_bytes + 64);   // [TOK][nch * 8]
+  float* part = reinterpret_cast<float*>(smem + table_bytes + 64 + (size_t)TOK * nch * 32);   // [TOK][16][16]
 
   const int SL = 1 << sl_log2, G = W >> sl_log2;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -95,8 +101,7 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
   const int gi = wave >> sl_log2, sl = wave & (SL - 1);
   const int n = lane & 15, g = lane >> 4;
   const int n_in = nch * 256;
-  const typename X::elem_t* xm = x + (int64_t)blockIdx.y * n_in;
-  YT* ym = y + (int64_t)blockIdx.y * n_out;
+  const int t0 = blockIdx.y * TOK;
   const uint32_t rb = (uint32_t)nch * 272u;
   const int S = (nch + SL - 1) >> sl_log2;
   const int wg_row0 = blockIdx.x * rows_per_wg;
@@ -107,11 +112,15 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
 
   // ---- activations: 8 values per thread and pass, requested before any weights
   constexpr int XP = ((COMPACT ? kQ8WinMaxChunks : kQ8WinMaxWideChunks) * 256 + 8 * kMfmaThreads - 1) / (8 * kMfmaThreads);
-  float xf[XP][8];
+  float xf[TOK][XP][8];
 #pragma unroll
-  for (int p = 0; p < XP; p++) {
-    const int k0 = 8 * (tid + p * kMfmaThreads);
-    X::load8(xm + (k0 < n_in ? k0 : 0), xf[p]);
+  for (int t = 0; t < TOK; t++) {
+    const typename X::elem_t* xm = x + (int64_t)min(t0 + t, m - 1) * n_in;
+#pragma unroll
+    for (int p = 0; p < XP; p++) {
+      const int k0 = 8 * (tid + p * kMfmaThreads);
+      X::load8(xm + (k0 < n_in ? k0 : 0), xf[t][p]);
+    }
   }
   __builtin_amdgcn_s_barrier();
 
@@ -134,18 +143,20 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
   {
     const v4i_t z = {0, 0, 0, 0};
     v4i_t* xa = reinterpret_cast<v4i_t*>(smem);
-    for (int e = tid; e < nch * (int)(kChunkBytes / 16) + 1; e += kMfmaThreads) xa[e] = z;   // + the zero entry
+    for (int e = tid; e < TOK * nch * (int)(kChunkBytes / 16) + 1; e += kMfmaThreads) xa[e] = z;   // + the zero entry
   }
   __syncthreads();
 
   // ---- quantize the activations into byte planes and scatter them to their windows
+#pragma unroll
+  for (int t = 0; t < TOK; t++)
 #pragma unroll
   for (int p = 0; p < XP; p++) {
     const int k0 = 8 * (tid + p * kMfmaThreads);
     if (k0 < n_in) {
       float amax = 0.f;
 #pragma unroll
-      for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(xf[p][i]));
+      for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(xf[t][p][i]));
       // the four threads of a block are an aligned quad
       amax = fmaxf(amax, dpp_quad<0xB1>(amax));
       amax = fmaxf(amax, dpp_quad<0x4E>(amax));
@@ -157,7 +168,7 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
       int pl[3][8];
 #pragma unroll
       for (int i = 0; i < 8; i++) {
-        const int v = (int)rintf(xf[p][i] * mul);
+        const int v = (int)rintf(xf[t][p][i] * mul);
         if (T == 3) {
           const int v1 = (v + 128) >> 8;
           pl[2][i] = v;                  // only the low byte is used
@@ -176,15 +187,15 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
       for (int i2 = 0; i2 < 4; i2++) {
         const int byte = 34 * b + 2 + q0 + 2 * i2;
         const int pos = byte & 63;
-        uint8_t* e = smem + (size_t)ch * kChunkBytes +
+        uint8_t* e = smem + (size_t)t * tok_bytes + (size_t)ch * kChunkBytes +
                      (COMPACT ? (size_t)(q8win_pair(b, byte >> 4) * T * 16 + (byte & 15))
                               : (size_t)((q8win_table(byte, b) * 64 + 16 * (pos >> 4) + 4 * (b & 3)) * 16 + (pos & 15)));
 #pragma unroll
-        for (int t = 0; t < T; t++)
-          *reinterpret_cast<uint16_t*>(e + 16 * t) =
-              (uint16_t)((pl[t][2 * i2] & 0xFF) | ((pl[t][2 * i2 + 1] & 0xFF) << 8));
+        for (int pi = 0; pi < T; pi++)
+          *reinterpret_cast<uint16_t*>(e + 16 * pi) =
+              (uint16_t)((pl[pi][2 * i2] & 0xFF) | ((pl[pi][2 * i2 + 1] & 0xFF) << 8));
       }
-      if ((tid & 3) == 0) tab[blk] = f;
+      if ((tid & 3) == 0) tab[t * nch * 8 + blk] = f;
     }
   }
   __syncthreads();
@@ -209,9 +220,9 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
 
   // ---- A operand addresses of this lane for the six plane MFMAs: windows 0, 1, 2 (block 3 only),
   // 2 (blocks 4, 5), 3, 4
-  uint32_t a_base[6], a_stride[6];
+  uint32_t a_base[6], a_stride[6], a_tok[6];
   {
-    const int slot = (lane & 15) >> 2, t = lane & 3;
+    const int slot = (lane & 15) >> 2, pln = lane & 3;
 #pragma unroll
     for (int ti = 0; ti < 6; ti++) {
       const int wdw = ti < 2 ? ti : (ti < 4 ? 2 : ti - 1);
@@ -222,17 +233,24 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
         const int b = slot + 4 * hh;
         const bool in_table = ti == 2 ? b == 3 : (ti == 3 ? b >= 4 : true);
         const bool touches = piece >= q8win_first_piece(b) && piece <= ((34 * b + 33) >> 4) && (wdw < 4 || g == 0);
-        if (t < T && in_table && touches) off = (q8win_pair(b, piece) * T + t) * 16;
+        if (pln < T && in_table && touches) off = (q8win_pair(b, piece) * T + pln) * 16;
       }
       if (!COMPACT) off = (ti * 64 + lane) * 16;
       a_base[ti] = off >= 0 ? (uint32_t)off : zero_off;
       a_stride[ti] = off >= 0 ? kChunkBytes : 0u;
+      a_tok[ti] = off >= 0 ? tok_bytes : 0u;
     }
   }
 
   // ---- main loop
   int cr = 0, csi = 0;
-  float acc = 0.f;
+  float acc[TOK];
+#pragma unroll
+  for (int t = 0; t < TOK; t++) acc[t] = 0.f;
+  auto store_row = [&](int row, int t, float v) {
+    if (row < wg_row_end && t0 + t < m)
+      YElem<YT>::store(y + (int64_t)(t0 + t) * n_out, row, v + load_bias(bias, bias_dtype, row));
+  };
   auto consume = [&](const Q8WinStep& s) {
     const int ch = (csi << sl_log2) + sl;
     if (cr < rounds && ch < nch) {
@@ -241,50 +259,57 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
       for (int i = 0; i < 5; i++) {
         B[i][0] = (int)s.p[i].x; B[i][1] = (int)s.p[i].y; B[i][2] = (int)s.p[i].z; B[i][3] = (int)s.p[i].w;
       }
-      v4i_t A[6];
-#pragma unroll
-      for (int ti = 0; ti < 6; ti++) {
-        if (COMPACT) A[ti] = *reinterpret_cast<const v4i_t*>(smem + a_base[ti] + (uint32_t)ch * a_stride[ti]);
-        else A[ti] = reinterpret_cast<const v4i_t*>(smem)[(size_t)ch * 384 + ti * 64 + lane];
-      }
       const v4i_t zero = {0, 0, 0, 0};
-      v4i_t c03 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[0], B[0], zero, 0, 0, 0);
-      v4i_t c47 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[3], B[2], zero, 0, 0, 0);
       v4i_t cd = __builtin_amdgcn_mfma_i32_16x16x64_i8(sel[0], B[0], zero, 0, 0, 0);
-      c03 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[1], B[1], c03, 0, 0, 0);
-      c47 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[4], B[3], c47, 0, 0, 0);
       cd = __builtin_amdgcn_mfma_i32_16x16x64_i8(sel[1], B[1], cd, 0, 0, 0);
-      c03 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[2], B[2], c03, 0, 0, 0);
-      c47 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[5], B[4], c47, 0, 0, 0);
       cd = __builtin_amdgcn_mfma_i32_16x16x64_i8(sel[2], B[2], cd, 0, 0, 0);
       cd = __builtin_amdgcn_mfma_i32_16x16x64_i8(sel[3], B[3], cd, 0, 0, 0);
-      const float f0 = tab[ch * 8 + g], f1 = tab[ch * 8 + 4 + g];
       const float d0 = f16_bits_to_f32((uint16_t)(((uint32_t)cd[1] & 0xFFu) << 8 | ((uint32_t)cd[0] & 0xFFu)));
       const float d1 = f16_bits_to_f32((uint16_t)(((uint32_t)cd[3] & 0xFFu) << 8 | ((uint32_t)cd[2] & 0xFFu)));
-      float s0, s1;
-      if (T == 3) {
-        s0 = ((float)c03[0] * 65536.f + (float)c03[1] * 256.f) + (float)c03[2];
-        s1 = ((float)c47[0] * 65536.f + (float)c47[1] * 256.f) + (float)c47[2];
-      } else {
-        s0 = (float)(c03[0] * 256 + c03[1]);
-        s1 = (float)(c47[0] * 256 + c47[1]);
+#pragma unroll
+      for (int t = 0; t < TOK; t++) {
+        v4i_t A[6];
+#pragma unroll
+        for (int ti = 0; ti < 6; ti++) {
+          if (COMPACT)
+            A[ti] = *reinterpret_cast<const v4i_t*>(smem + a_base[ti] + (uint32_t)ch * a_stride[ti] + (uint32_t)t * a_tok[ti]);
+          else
+            A[ti] = reinterpret_cast<const v4i_t*>(smem)[(size_t)ch * 384 + ti * 64 + lane];
+        }
+        v4i_t c03 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[0], B[0], zero, 0, 0, 0);
+        v4i_t c47 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[3], B[2], zero, 0, 0, 0);
+        c03 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[1], B[1], c03, 0, 0, 0);
+        c47 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[4], B[3], c47, 0, 0, 0);
+        c03 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[2], B[2], c03, 0, 0, 0);
+        c47 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[5], B[4], c47, 0, 0, 0);
+        const float f0 = tab[t * nch * 8 + ch * 8 + g], f1 = tab[t * nch * 8 + ch * 8 + 4 + g];
+        float s0, s1;
+        if (T == 3) {
+          s0 = ((float)c03[0] * 65536.f + (float)c03[1] * 256.f) + (float)c03[2];
+          s1 = ((float)c47[0] * 65536.f + (float)c47[1] * 256.f) + (float)c47[2];
+        } else {
+          s0 = (float)(c03[0] * 256 + c03[1]);
+          s1 = (float)(c47[0] * 256 + c47[1]);
+        }
+        acc[t] = acc[t] + d0 * (s0 * f0);
+        acc[t] = acc[t] + d1 * (s1 * f1);
       }
-      acc = acc + d0 * (s0 * f0);
-      acc = acc + d1 * (s1 * f1);
     }
     if (++csi == S) {
-      float v = acc;
-      v += __shfl_xor(v, 16, kWave);
-      v += __shfl_xor(v, 32, kWave);
-      if (cr < rounds) {
-        if (sl_log2 == 0) {
-          const int row = wg_row0 + (cr * G + gi) * 16 + n;
-          if (lane < 16 && row < wg_row_end) YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
-        } else {
-          if (lane < 16) part[wave * 16 + n] = v;
+#pragma unroll
+      for (int t = 0; t < TOK; t++) {
+        float v = acc[t];
+        v += __shfl_xor(v, 16, kWave);
+        v += __shfl_xor(v, 32, kWave);
+        if (cr < rounds) {
+          if (sl_log2 == 0) {
+            if (lane < 16) store_row(wg_row0 + (cr * G + gi) * 16 + n, t, v);
+          } else {
+            if (lane < 16) part[(t * W + wave) * 16 + n] = v;
+          }
         }
+        acc[t] = 0.f;
       }
-      acc = 0.f;
       csi = 0;
       cr++;
     }
@@ -298,12 +323,11 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
   if (sl_log2 != 0) {
     // one round only: add the slices in a fixed order
     __syncthreads();
-    if (tid < 16 * G) {
-      const int grp = tid >> 4, nn = tid & 15;
+    for (int idx = tid; idx < 16 * G * TOK; idx += kMfmaThreads) {
+      const int nn = idx & 15, grp = (idx >> 4) % G, t = idx / (16 * G);
       float v = 0.f;
-      for (int s2 = 0; s2 < SL; s2++) v += part[(grp * SL + s2) * 16 + nn];
-      const int row = wg_row0 + grp * 16 + nn;
-      if (row < wg_row_end) YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
+      for (int s2 = 0; s2 < SL; s2++) v += part[(t * W + grp * SL + s2) * 16 + nn];
+      store_row(wg_row0 + grp * 16 + nn, t, v);
     }
   }
 }
@@ -321,9 +345,17 @@ static hipError_t q8win_launch_xy(const void* w, const void* x, void* y, const v
   num_wg = (int)((n_out + rows_per_wg - 1) / rows_per_wg);
   int sl_log2 = 0;
   while ((2 << sl_log2) <= W && (2 << sl_log2) <= nch && (16 * W >> (sl_log2 + 1)) >= rows_per_wg) sl_log2++;
-  const bool compact = nch > kQ8WinMaxWideChunks;
-  const size_t lds = (size_t)nch * (compact ? kQ8WinPairs * Q8WX<XT>::kPlanes * 16 : 6 * 1024) + 64 +
-                     (size_t)nch * 32 + 1024;
+  constexpr int T = Q8WX<XT>::kPlanes;
+  const auto lds_for = [&](bool compact, int tok) {
+    return (size_t)tok * nch * (compact ? kQ8WinPairs * T * 16 : 6 * 1024) + 64 + (size_t)tok * nch * 32 +
+           (size_t)tok * 1024;
+  };
+  // tokens per pass: four (two) when their compact tables fit LDS
+  int tok = 1;
+  if (m >= 2) tok = (m > 2 && lds_for(true, 4) <= 150 * 1024) ? 4 : (lds_for(true, 2) <= 150 * 1024 ? 2 : 1);
+  const bool compact = tok > 1 || nch > kQ8WinMaxWideChunks;
+  const size_t lds = lds_for(compact, tok);
+  const dim3 grid((unsigned)num_wg, (unsigned)((m + tok - 1) / tok));
   const auto launch = [&](auto kernel, bool& configured) -> hipError_t {
     if (!configured) {
       const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -331,14 +363,16 @@ static hipError_t q8win_launch_xy(const void* w, const void* x, void* y, const v
       if (e != hipSuccess) return e;
       configured = true;
     }
-    hipLaunchKernelGGL(kernel, dim3((unsigned)num_wg, (unsigned)m), dim3(W * 64), lds, s,
-                       static_cast<const uint8_t*>(w), static_cast<const typename Q8WX<XT>::elem_t*>(x),
-                       static_cast<YT*>(y), bias, bias_dtype, (int)n_out, nch, rows_per_wg, sl_log2);
+    hipLaunchKernelGGL(kernel, grid, dim3(W * 64), lds, s, static_cast<const uint8_t*>(w),
+                       static_cast<const typename Q8WX<XT>::elem_t*>(x), static_cast<YT*>(y), bias, bias_dtype, (int)m,
+                       (int)n_out, nch, rows_per_wg, sl_log2);
     return hipGetLastError();
   };
-  static bool configured_wide = false, configured_compact = false;
-  if (compact) return launch(gemv_q8_win_kernel<true, XT, YT>, configured_compact);
-  return launch(gemv_q8_win_kernel<false, XT, YT>, configured_wide);
+  static bool configured_wide = false, configured_compact = false, configured_2 = false, configured_4 = false;
+  if (tok == 4) return launch(gemv_q8_win_kernel<true, 4, XT, YT>, configured_4);
+  if (tok == 2) return launch(gemv_q8_win_kernel<true, 2, XT, YT>, configured_2);
+  if (compact) return launch(gemv_q8_win_kernel<true, 1, XT, YT>, configured_compact);
+  return launch(gemv_q8_win_kernel<false, 1, XT, YT>, configured_wide);
 }
 
 template <typename XT>
@@ -350,6 +384,16 @@ static hipError_t q8win_launch_x(const void* w, const void* x, void* y, int y_dt
     case kBF16: return q8win_launch_xy<XT, bf16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
     default: return hipErrorInvalidValue;
   }
+}
+
+// Tokens per pass the launcher above picks (see q8win_launch_xy).
+int gemv_q8_win_tokens(int x_dtype, int64_t m, int64_t n_in) {
+  const int nch = (int)(n_in / 256), planes = x_dtype == kF32 ? 3 : 2;
+  const auto lds_for = [&](int tok) {
+    return (size_t)tok * nch * kQ8WinPairs * planes * 16 + 64 + (size_t)tok * nch * 32 + (size_t)tok * 1024;
+  };
+  if (m < 2) return 1;
+  return (m > 2 && lds_for(4) <= 150 * 1024) ? 4 : (lds_for(2) <= 150 * 1024 ? 2 : 1);
 }
 
 bool gemv_q8_win_supported(int format, int64_t n_out, int64_t n_in) {

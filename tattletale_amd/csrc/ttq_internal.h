@@ -25,6 +25,12 @@ hipError_t launch_gemv(int format, const void* w, const void* x, int x_dtype, vo
                        int64_t n_in, hipStream_t s);
 
 // Packed-dot fast path for 16-bit activations (ttq_gemv_dot2.hip).
+// Packed-dot GEMV for two or four activation rows per pass over the weights (Q4_K shapes the
+// matrix-core few-row kernels do not take, Q6_K).
+bool gemv_dot2_multi_supported(int format, int x_dtype, int64_t m, int64_t n_in);
+hipError_t launch_gemv_dot2_multi(int format, const void* w, const void* x, int x_dtype, void* y,
+                                  int y_dtype, const void* bias, int bias_dtype, int64_t m,
+                                  int64_t n_out, int64_t n_in, hipStream_t s);
 bool gemv_dot2_supported(int format, int x_dtype, int64_t n_in);
 hipError_t launch_gemv_dot2(int format, const void* w, const void* x, int x_dtype, void* y,
                             int y_dtype, const void* bias, int bias_dtype, int64_t m, int64_t n_out,
@@ -39,6 +45,7 @@ hipError_t launch_gemv_mfma(const void* w, const void* x, int x_dtype, void* y, 
 // int8 matrix-core path for Q8_0, any activation dtype (ttq_gemv_q8_mfma.hip).
 // Q8_0 through the matrix cores, rows read as aligned 64-byte windows (ttq_gemv_q8_win.hip).
 bool gemv_q8_win_supported(int format, int64_t n_out, int64_t n_in);
+int gemv_q8_win_tokens(int x_dtype, int64_t m, int64_t n_in);
 hipError_t launch_gemv_q8_win(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
                               const void* bias, int bias_dtype, int64_t m, int64_t n_out,
                               int64_t n_in, hipStream_t s);
@@ -67,9 +74,6 @@ hipError_t launch_gemm_q4k(const void* w, const uint16_t* x_bf16, void* y, int y
 
 // Q4_K decode GEMV for a few activation rows at once (ttq_gemv_q4k_batch.hip): the weights are
 // read and unpacked once per 8 or 16 rows.
-// ttq_linear_forward prefers it to the prefill GEMM up to this many rows
-constexpr int64_t kBatchGemvMaxRows = 32;
-constexpr int64_t kBatch4GemvMaxRows = 16;   // four rows per pass (long rows)
 bool gemv_q4k_batch_supported(int format, int x_dtype, int64_t m, int64_t n_out, int64_t n_in);
 hipError_t launch_gemv_q4k_batch(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
                                  const void* bias, int bias_dtype, int64_t m, int64_t n_out,
@@ -80,6 +84,11 @@ bool gemv_q4k_batch4_supported(int format, int x_dtype, int64_t m, int64_t n_out
 hipError_t launch_gemv_q4k_batch4(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
                                   const void* bias, int bias_dtype, int64_t m, int64_t n_out,
                                   int64_t n_in, hipStream_t s);
+
+// Rough times (microseconds) of the two ways to run a few activation rows.
+float gemv_estimate_us(int format, int x_dtype, int64_t m, int64_t n_out, int64_t n_in);
+float gemm_pc_estimate_us(int format, int64_t m, int64_t n_out, int64_t n_in);
+int gemv_q4k_batch_tokens(int64_t m, int64_t n_in);
 
 // Producer/consumer GEMM for Q4_K / Q6_K / Q8_0 weights and bf16 activations (ttq_gemm_pc.hip).
 bool gemm_pc_supported(int format, int64_t m, int64_t n_out, int64_t n_in, int bn);

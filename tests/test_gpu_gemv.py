@@ -194,11 +194,13 @@ def test_q8_0_work_distributions(xk, n_out, n_in):
     x = Q.fill_normal(n_in + 5, 1, 1.0, 2 * n_in).reshape(2, n_in)
     x[1, ::7] *= 37.0
     xd, xf = x_to_dev(x, xk)
-    y = QL.gemv(F.Q8_0, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()
-    assert np.all(np.isfinite(y))
+    wd = packed_to_dev(p)
     want = oracle.linear_f64(what, xf)
-    for r in range(2):
-        assert rel_l2(y[r][rows], want[r]) <= (1e-6 if xk == "f32" else TOL)
+    # both rows in one call (two tokens per pass where the kernel allows) and one call per row
+    for y in (QL.gemv(F.Q8_0, wd, xd, n_out, n_in).cpu().numpy(), gemv_row_by_row(F.Q8_0, wd, xd, n_out, n_in)):
+        assert np.all(np.isfinite(y))
+        for r in range(2):
+            assert rel_l2(y[r][rows], want[r]) <= (1e-6 if xk == "f32" else TOL)
 
 
 @pytest.mark.parametrize("xk", ["f32", "bf16"])
@@ -220,14 +222,16 @@ def test_q8_0_unit_vectors_and_extremes_many_rows(xk, n_in):
     x[-2, 5] = np.inf
     x[-1] = Q.fill_normal(16, 1, 1.0, n_in) * 1e-30
     xd, xf = x_to_dev(x, xk)
-    y = QL.gemv(F.Q8_0, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()
-    for i, c in enumerate(cols):
-        col = what[:, c] * np.float32(1.0 if i % 2 == 0 else -0.5)
-        assert np.array_equal(y[i], col), c
+    wd = packed_to_dev(p)
     want = oracle.linear_f64(what, xf[[-3, -1]])
-    assert rel_l2(y[-3], want[0]) <= TOL
-    assert not np.any(np.isfinite(y[-2]))
-    assert rel_l2(y[-1], want[1]) <= TOL
+    # all rows in one call (four tokens per pass) and one call per row
+    for y in (QL.gemv(F.Q8_0, wd, xd, n_out, n_in).cpu().numpy(), gemv_row_by_row(F.Q8_0, wd, xd, n_out, n_in)):
+        for i, c in enumerate(cols):
+            col = what[:, c] * np.float32(1.0 if i % 2 == 0 else -0.5)
+            assert np.array_equal(y[i], col), c
+        assert rel_l2(y[-3], want[0]) <= TOL
+        assert not np.any(np.isfinite(y[-2]))
+        assert rel_l2(y[-1], want[1]) <= TOL
 
 
 def test_gemv_rejects_oversized_rows():

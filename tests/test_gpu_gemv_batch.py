@@ -132,3 +132,69 @@ def test_batch_full_shape_14336x4096(m):
     want = oracle.linear_f64(what, xf)
     for r in range(m):
         assert rel_l2(y[r][rows], want[r]) <= TOL
+
+
+@pytest.mark.parametrize("fmt,n_out,n_in", [(F.Q6_K, 2500, 4096), (F.Q6_K, 4096, 14336), (F.Q6_K, 300, 1280),
+                                           (F.Q6_K, 40000, 256), (F.Q4_K, 1000, 4096), (F.Q4_K, 33, 14336),
+                                           (F.Q6_K, 2050, 16384)])
+@pytest.mark.parametrize("xk", ["bf16", "f16"])
+@pytest.mark.parametrize("m", [2, 3, 4, 7])
+def test_packed_dot_few_rows(fmt, n_out, n_in, xk, m):
+    """Q6_K, and the Q4_K shapes the matrix-core few-row kernels do not take: two or four rows per
+    pass over the weights.  Each row against the oracle and against the same row on its own."""
+    rng = np.random.default_rng(n_out + n_in + m)
+    p = random_blocks(fmt, n_out * (n_in // 256), seed=n_out + m)
+    rows = np.unique(np.concatenate([rng.integers(0, n_out, 200), np.arange(max(0, n_out - 30), n_out), np.arange(min(30, n_out))]))
+    what = oracle.dequant(fmt, np.ascontiguousarray(p.reshape(n_out, -1)[rows]), rows.size, n_in)
+    x = Q.fill_normal(n_in + m, 1, 1.0, m * n_in).reshape(m, n_in)
+    x[m - 1, ::5] *= 21.0
+    xd, xf = x_to_dev(x, xk)
+    wd = packed_to_dev(p)
+    y = QL.gemv(fmt, wd, xd, n_out, n_in).cpu().numpy()
+    assert y.shape == (m, n_out) and np.all(np.isfinite(y))
+    want = oracle.linear_f64(what, xf)
+    for r in range(m):
+        assert rel_l2(y[r][rows], want[r]) <= TOL, r
+    for r in {0, m - 1}:
+        y1 = QL.gemv(fmt, wd, xd[r:r + 1], n_out, n_in).cpu().numpy()[0]
+        assert rel_l2(y[r], y1) <= 2e-6, r
+
+
+@pytest.mark.parametrize("n_in", [1024, 8192])
+def test_packed_dot_few_rows_unit_vectors(n_in):
+    n_out = 700
+    p = random_blocks(F.Q6_K, n_out * (n_in // 256), seed=31)
+    what = oracle.dequant(F.Q6_K, p, n_out, n_in)
+    cols = [0, 1, 15, 16, 31, 32, 63, 64, 127, 128, 255, 256, n_in - 1]
+    x = np.zeros((len(cols), n_in), np.float32)
+    for i, c in enumerate(cols):
+        x[i, c] = 1.0 if i % 2 == 0 else -0.5
+    xd, _ = x_to_dev(x, "bf16")
+    y = QL.gemv(F.Q6_K, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()
+    for i, c in enumerate(cols):
+        col = what[:, c] * np.float32(1.0 if i % 2 == 0 else -0.5)
+        assert np.array_equal(y[i], col), c
+
+
+@pytest.mark.parametrize("n_out,n_in", [(2100, 1024), (4096, 4096), (2304, 8192), (4096, 14336), (25600, 256)])
+@pytest.mark.parametrize("xk", ["f32", "bf16"])
+@pytest.mark.parametrize("m", [2, 3, 4, 7])
+def test_q8_0_few_rows(n_out, n_in, xk, m):
+    """Q8_0: four (two, for long rows) tokens per pass in the aligned-window kernel; each row against
+    the oracle and against the same row on its own."""
+    rng = np.random.default_rng(n_out + n_in + m)
+    p = random_blocks(F.Q8_0, n_out * (n_in // 32), seed=n_out + m)
+    rows = np.unique(np.concatenate([rng.integers(0, n_out, 200), np.arange(n_out - 30, n_out), np.arange(30)]))
+    what = oracle.dequant(F.Q8_0, np.ascontiguousarray(p.reshape(n_out, -1)[rows]), rows.size, n_in)
+    x = Q.fill_normal(n_in + m, 1, 1.0, m * n_in).reshape(m, n_in)
+    x[m - 1, ::5] *= 21.0
+    xd, xf = x_to_dev(x, xk)
+    wd = packed_to_dev(p)
+    y = QL.gemv(F.Q8_0, wd, xd, n_out, n_in).cpu().numpy()
+    assert y.shape == (m, n_out) and np.all(np.isfinite(y))
+    want = oracle.linear_f64(what, xf)
+    for r in range(m):
+        assert rel_l2(y[r][rows], want[r]) <= (1e-6 if xk == "f32" else TOL), r
+    for r in {0, m - 1}:
+        y1 = QL.gemv(F.Q8_0, wd, xd[r:r + 1], n_out, n_in).cpu().numpy()[0]
+        assert np.array_equal(y[r], y1), r        # same sums in the same order
