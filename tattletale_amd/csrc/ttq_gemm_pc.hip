@@ -319,7 +319,8 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
     constexpr bool kSpare = 4 * BN <= 256;
     const bool widle = kSpare && pt >= 2 * BN;
     const int wt = pt < 2 * BN ? pt : (kSpare ? pt % (2 * BN) : pt - 2 * BN);
-    const int wr = wt % BN, whalf = wt / BN;
+    // the two halves of a row in adjacent lanes: a 64-lane load then touches 32 rows, not 64
+    const int wr = wt >> 1, whalf = wt & 1;
     // clamped: rows past the end are never stored
     const int wrow = FUSE ? min(n0 + 8 * (wr >> 4) + (wr & 7), n_out - 1) + ((wr >> 3) & 1) * n_out
                           : min(n0 + wr, n_out - 1);
