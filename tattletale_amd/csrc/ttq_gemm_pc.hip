@@ -629,7 +629,7 @@ static int pc_choose_tile(int64_t m, int64_t n_out, int64_t n_in, bool fuse, flo
 float gemm_pc_estimate_us(int format, int64_t m, int64_t n_out, int64_t n_in) {
   float c = 0.f;
   pc_choose_tile(m, n_out, n_in, false, &c);
-  return c * (format == kQ8_0 ? 2.1f : (format == kQ6_K ? 1.5f : 1.f)) + 2.f;
+  return c * (format == kQ8_0 ? 1.9f : (format == kQ6_K ? 1.4f : 1.f)) + 2.f;
 }
 
 template <int FMT, bool FUSE>
