@@ -11,7 +11,7 @@ import pytest
 import torch
 
 import oracle
-from tattletale_amd import QuantGatedMLP, QuantLinear, TtqError, formats as F
+from tattletale_amd import QuantGatedMLP, QuantLinear, TtqError, _lib, formats as F
 from tattletale_amd import qlinear as QL
 from tattletale_amd import quantize as Q
 
@@ -126,7 +126,7 @@ def _round(a, dt):
 
 
 @pytest.mark.parametrize("dt,ulp", [("f32", 2.0 ** -21), ("bf16", 2.0 ** -8), ("f16", 2.0 ** -11)])
-@pytest.mark.parametrize("m,n", [(1, 4096), (3, 1000), (2, 14336)])
+@pytest.mark.parametrize("m,n", [(1, 4096), (3, 1000), (2, 14336), (3, 1001), (5, 8), (2, 40000), (1, 70004)])
 @pytest.mark.parametrize("with_residual", [False, True])
 def test_rmsnorm_kernel(dt, ulp, m, n, with_residual):
     """RmsNorm.forward / forward_with_residual (norm.nim:23-38): new_residual = x + residual rounded
@@ -146,7 +146,32 @@ def test_rmsnorm_kernel(dt, ulp, m, n, with_residual):
         assert new_res is None
     want = oracle.rmsnorm_f64(t.astype(np.float64), gf.reshape(-1).astype(np.float64), 1e-5)
     got = normed.float().cpu().numpy().astype(np.float64)
-    assert np.all(np.abs(got - want) <= ulp * np.abs(want) + 1e-30)
+    # half a unit in the last place of the output type, plus the kernel's own fp32 arithmetic (the
+    # sum of squares, rsqrt and two products) ahead of that rounding
+    floor = 2.0 ** -25 if dt == "f16" else 1e-30    # f16 results under 2^-14 are subnormal: spacing 2^-24
+    assert np.all(np.abs(got - want) <= (ulp + 2.0 ** -19) * np.abs(want) + floor)
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("n", [4096, 12288, 1001])
+def test_rmsnorm_in_place(dt, n):
+    """The C entry point allows normed_out == x and new_residual_out == residual (the reference adds
+    into the residual stream in place, norm.nim:31-38): same bits as the out-of-place call."""
+    m = 3
+    dev = torch.device("cuda:0")
+    xd, _ = x_to_dev(Q.fill_normal(700 + n, 1, 1.5, m * n).reshape(m, n), dt)
+    rd, _ = x_to_dev(Q.fill_normal(701 + n, 1, 0.7, m * n).reshape(m, n), dt)
+    gd, _ = x_to_dev(1.0 + Q.fill_normal(702 + n, 2, 0.1, n), dt)
+    gd = gd.reshape(-1)
+    normed_ref, new_res_ref = QL.rmsnorm(xd, gd, 1e-5, rd)
+    xs, rs = xd.clone(), rd.clone()
+    code = {"f32": _lib.F32, "bf16": _lib.BF16, "f16": _lib.F16}[dt]
+    with torch.cuda.device(dev):
+        rc = _lib.lib().ttq_rmsnorm(xs.data_ptr(), rs.data_ptr(), gd.data_ptr(), 1e-5, code, rs.data_ptr(),
+                                    xs.data_ptr(), m, n, torch.cuda.current_stream(dev).cuda_stream)
+    assert rc == _lib.OK
+    assert torch.equal(rs, new_res_ref)
+    assert torch.equal(xs, normed_ref)
 
 
 @pytest.mark.parametrize("xk", ["bf16", "f16"])
