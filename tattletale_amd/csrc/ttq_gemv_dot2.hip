@@ -98,6 +98,8 @@ constexpr int kFastWaves = kFastThreads / kWave;
 constexpr int kBatch = 4;     // rows per pass when activations are re-read from LDS
 constexpr int kRing = 4;      // row buffers per wavefront when activations sit in registers
 constexpr int kEarlyRows = 1; // rows requested before the activations are staged
+constexpr int kLongRing = 6;  // unit-group buffers per wavefront on the long-row path
+constexpr int kLongEarly = 2; // of them requested before the activations are staged
 
 // LDS slot (dword) of activation-pair register `reg` of unit u: [u/64][reg/4][u%64][reg%4]
 __device__ __forceinline__ int xpair_slot(int u, int reg) {
@@ -119,6 +121,7 @@ __device__ __forceinline__ void make_pairs(const uint4& v, uint2& p0, uint2& p1)
 struct DotQ4K {
   static constexpr int kSums = 2;
   static __device__ __forceinline__ int64_t row_bytes(int n_in) { return (int64_t)(n_in >> 8) * 144; }
+  static constexpr uint32_t kGroupBytes = 16 * 144;   // 64 units
   struct Raw { uint4 hdr, q0, q1; };
 
   // Per-lane constants.  A lane always decodes chunk c = lane % 4, so the bit positions of its
@@ -224,6 +227,7 @@ struct DotQ4K {
 struct DotQ6K {
   static constexpr int kSums = 4;
   static __device__ __forceinline__ int64_t row_bytes(int n_in) { return (int64_t)(n_in >> 8) * 210; }
+  static constexpr uint32_t kGroupBytes = 16 * 210;   // 64 units
   struct Raw { uint4 a, b, h; uint2 sc; uint32_t d; };
   struct Lane {
     uint32_t off_a, off_h, off_sc, off_d;
@@ -323,7 +327,8 @@ __device__ __forceinline__ void load_x_regs(const uint32_t* xs, int it, int lane
 template <class F, class Ops, typename YT, bool XREG>
 __global__ void __launch_bounds__(kFastThreads)
 gemv_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
-                 const void* __restrict__ bias, int bias_dtype, int n_out, int n_in, int rows_per_wave) {
+                 const void* __restrict__ bias, int bias_dtype, int n_out, int n_in, int rows_per_wave,
+                 int flat) {
   extern __shared__ uint32_t xs[];
   const int tid = threadIdx.x, lane = tid & 63;
   // the wave index is the same in all 64 lanes: keep it (and every row address) scalar
@@ -345,7 +350,19 @@ gemv_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, 
   typename F::Lane L;
   L.init(active ? lane : 0);
 
-  typename F::Raw ring[XREG ? kRing : 1];
+  typename F::Raw ring[XREG ? kRing : kLongRing];
+
+  // Long rows, flat order: the wavefront's work is the sequence of items (row, group of 64 units),
+  // row by row.  next_item() requests the next one (items past the end fetch one harmless line,
+  // so that the compiler's load counting stays exact).  A lane whose unit lies beyond the row's
+  // last one reads its unit of group 0 instead (valid packed bytes; its activations are zero).
+  int f_row = row0, f_it = 0;
+  auto next_item = [&](typename F::Raw& dst) {
+    const bool valid = f_row < row_end;
+    const uint32_t group = (f_it * 64 + lane < units) ? (uint32_t)f_it * F::kGroupBytes : 0u;
+    F::fetch(dst, w + rb * (valid ? f_row : min(row0, last)) + (valid ? group : 0u), L, valid ? 0xFFFFFFFFu : 0u);
+    if (++f_it == nit) { f_it = 0; f_row++; }
+  };
 
   // stage x as permuted pairs: one 16-byte load (8 activations) per thread and pass,
   // all passes requested before the first is consumed
@@ -371,6 +388,10 @@ gemv_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, 
       __builtin_amdgcn_s_barrier();
 #pragma unroll
       for (int r = 0; r < kEarlyRows; r++) F::fetch(ring[r], w + rb * min(row0 + r, last), L, 0xFFFFFFFFu);
+    } else if (flat) {
+      __builtin_amdgcn_s_barrier();
+#pragma unroll
+      for (int r = 0; r < kLongEarly; r++) next_item(ring[r]);
     }
 #pragma unroll
     for (int ch = 0; ch < kMaxChunks; ch++) {
@@ -431,6 +452,49 @@ gemv_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, 
     TTQ_TRACE_POINT(gw, 5);
   } else {
     // long rows: activations come from LDS for every unit
+    if (flat) {
+      // The per-group activation sums do not depend on the row: each wavefront works out a share
+      // of them once, into LDS behind the staged pairs ([group][sum][lane]).
+      float* xsum = reinterpret_cast<float*>(xs + nit * 2048);
+      for (int it = wave; it < nit; it += kFastWaves) {
+        uint32_t xr[32];
+        float sx[F::kSums];
+        load_x_regs(xs, it, lane, xr);
+        F::template sums<Ops>(xr, sx);
+#pragma unroll
+        for (int i = 0; i < F::kSums; i++) xsum[(it * F::kSums + i) * 64 + lane] = sx[i];
+      }
+      __syncthreads();
+      // Ring of kLongRing items: while one is unpacked the next kLongRing-1 are in flight.
+#pragma unroll
+      for (int r = kLongEarly; r < kLongRing - 1; r++) next_item(ring[r]);
+      int c_row = row0, c_it = 0;
+      float acc1[1] = {0.f};
+      while (c_row < row_end) {
+#pragma unroll
+        for (int i = 0; i < kLongRing; i++) {
+          next_item(ring[(i + kLongRing - 1) % kLongRing]);
+          if (c_row < row_end) {
+            uint32_t xr[32];
+            float sx[F::kSums], off[F::kSums];
+            load_x_regs(xs, c_it, lane, xr);
+#pragma unroll
+            for (int k = 0; k < F::kSums; k++) {
+              sx[k] = xsum[(c_it * F::kSums + k) * 64 + lane];
+              off[k] = kOff * sx[k];
+            }
+            acc1[0] += F::template unit_dot<Ops>(ring[i], L, xr, sx, off, magic);
+            if (++c_it == nit) {
+              store_rows(acc1, c_row);
+              acc1[0] = 0.f;
+              c_it = 0;
+              c_row++;
+            }
+          }
+        }
+      }
+      return;
+    }
     if (row_end - row0 < kBatch) {
       // fewer rows than a batch (many CUs, few rows each): the batch runs along the row instead,
       // kBatch groups of 64 units requested together
@@ -625,15 +689,30 @@ static hipError_t launch_fmt_t(const void* w, const void* x, void* y, const void
   int rows_per_wave = (int)((n_out + waves - 1) / waves);
   const int64_t used_waves = (n_out + rows_per_wave - 1) / rows_per_wave;
   const dim3 grid((unsigned)((used_waves + kFastWaves - 1) / kFastWaves), (unsigned)m), block(kFastThreads);
-  const size_t lds = (size_t)nit * 2048 * sizeof(uint32_t);
+  // staged pairs, and behind them the per-group activation sums of the long-row path
+  const size_t lds = (size_t)nit * 2048 * sizeof(uint32_t) + (nit > 1 ? (size_t)nit * F::kSums * 64 * sizeof(float) : 0);
+  // Long rows: with a batch of rows or more per wavefront the flat item ring (requests running
+  // ahead across rows) wins (28672x8192 Q6_K: 46.6 -> 42.8 us); with fewer, one request of a
+  // whole batch along the row does.  TTQ_GEMV_LONG_FLAT=0/1 forces either.
+  static const int flat_env = env_int("TTQ_GEMV_LONG_FLAT", -1);
+  const int flat = flat_env >= 0 ? flat_env : (rows_per_wave >= kBatch ? 1 : 0);
   const uint8_t* wb = static_cast<const uint8_t*>(w);
   const uint16_t* xb = static_cast<const uint16_t*>(x);
   if (nit == 1)
     hipLaunchKernelGGL((gemv_dot2_kernel<F, Ops, YT, true>), grid, block, lds, s, wb, xb,
-                       static_cast<YT*>(y), bias, bias_dtype, (int)n_out, (int)n_in, rows_per_wave);
-  else
-    hipLaunchKernelGGL((gemv_dot2_kernel<F, Ops, YT, false>), grid, block, lds, s, wb, xb,
-                       static_cast<YT*>(y), bias, bias_dtype, (int)n_out, (int)n_in, rows_per_wave);
+                       static_cast<YT*>(y), bias, bias_dtype, (int)n_out, (int)n_in, rows_per_wave, 0);
+  else {
+    auto kernel = gemv_dot2_kernel<F, Ops, YT, false>;
+    static bool configured = false;
+    if (lds > 64 * 1024 && !configured) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      if (e != hipSuccess) return e;
+      configured = true;
+    }
+    hipLaunchKernelGGL(kernel, grid, block, lds, s, wb, xb, static_cast<YT*>(y), bias, bias_dtype, (int)n_out,
+                       (int)n_in, rows_per_wave, flat);
+  }
   return hipGetLastError();
 }
 

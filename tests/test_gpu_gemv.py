@@ -140,6 +140,36 @@ def test_q4_k_16bit_work_distributions(xk, n_out, n_in):
 
 
 @pytest.mark.parametrize("xk", ["bf16", "f16"])
+@pytest.mark.parametrize("fmt,n_out,n_in", [(F.Q6_K, 9000, 8192), (F.Q6_K, 4096, 14336), (F.Q6_K, 2500, 5120),
+                                            (F.Q6_K, 10001, 4096 + 256), (F.Q6_K, 300, 16384),
+                                            (F.Q4_K, 2000, 16384), (F.Q4_K, 1500, 8192 + 1024)])
+def test_long_row_work_distributions(fmt, xk, n_out, n_in):
+    """Rows longer than one pass of a wavefront (more than 64 units of 64 weights) on the packed-dot
+    kernels: many rows per wavefront (requests run ahead across rows) and few (a batch along the
+    row), last groups of units that are full, half full and nearly empty; two activation rows."""
+    rng = np.random.default_rng(n_out + n_in)
+    p = random_blocks(fmt, n_out * (n_in // 256), seed=n_out + 1)
+    rows = np.unique(np.concatenate([rng.integers(0, n_out, 300), np.arange(n_out - 40, n_out), np.arange(40)]))
+    sub = np.ascontiguousarray(p.reshape(n_out, -1)[rows])
+    what = oracle.dequant(fmt, sub, rows.size, n_in)
+    x = Q.fill_normal(n_in + 6, 1, 1.0, 2 * n_in).reshape(2, n_in)
+    x[1, ::5] *= 29.0
+    xd, xf = x_to_dev(x, xk)
+    wd = packed_to_dev(p)
+    want = oracle.linear_f64(what, xf)
+    y = gemv_row_by_row(fmt, wd, xd, n_out, n_in)
+    assert np.all(np.isfinite(y))
+    for r in range(2):
+        assert rel_l2(y[r][rows], want[r]) <= TOL
+    # a unit vector in the last group of units reproduces that column of the canonical weights
+    e = np.zeros((1, n_in), np.float32)
+    e[0, n_in - 3] = 1.0
+    ed, _ = x_to_dev(e, xk)
+    col = QL.gemv(fmt, wd, ed, n_out, n_in).cpu().numpy()[0]
+    assert np.array_equal(col[rows], what[:, n_in - 3])
+
+
+@pytest.mark.parametrize("xk", ["bf16", "f16"])
 @pytest.mark.parametrize("n_in", [1024, 8192])
 def test_q4_k_unit_vectors_many_rows(xk, n_in):
     """Bit-exact columns again, with enough rows that the matrix-core kernel is the one that runs."""
