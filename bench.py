@@ -288,7 +288,7 @@ def main() -> int:
     def run_widened(steps: int, warmup: int):
         """Rows next to the headline ones, on random packed bytes with finite scale fields (timing
         only): the few-row decode GEMV (8 and 16 activation rows at once) and the prefill GEMM for
-        Q6_K and Q8_0 weights, all 14336 x 4096."""
+        Q6_K and Q8_0 weights, all 14336 x 4096; add + RMSNorm on rows of 4096."""
         n_out, n_in = 14336, 4096
         rng = np.random.default_rng(1234)
         res = {}
@@ -322,6 +322,27 @@ def main() -> int:
             y = torch.empty((512, n_out), dtype=torch.bfloat16, device=dev)
             timed(nm, fmt, 512,
                   lambda ws, x, nc, y=y, fmt=fmt: (lambda i: QL.gemm(fmt, ws[i % nc], x, n_out, n_in, out=y)))
+        # add + RMSNorm alone (ttq_rmsnorm with a residual): one decode row and a prefill block.
+        # Algorithmic bytes: x and residual read, new residual and normalized row written.
+        L = _lib.lib()
+        gamma = torch.ones(n_in, dtype=torch.bfloat16, device=dev)
+        for m in (1, 2048):
+            nbuf = max(2, -(-2 * MALL_BYTES // (4 * m * n_in * 2))) if m > 1 else 2
+            xs = [torch.randn((m, n_in), device=dev).to(torch.bfloat16) for _ in range(nbuf)]
+            rs = [torch.randn((m, n_in), device=dev).to(torch.bfloat16) for _ in range(nbuf)]
+            new_res, normed = torch.empty_like(xs[0]), torch.empty_like(xs[0])
+
+            def norm_step(i, m=m, xs=xs, rs=rs, new_res=new_res, normed=normed, nbuf=nbuf):
+                _lib.check(L.ttq_rmsnorm(xs[i % nbuf].data_ptr(), rs[i % nbuf].data_ptr(), gamma.data_ptr(), 1e-5,
+                                         F.BF16, new_res.data_ptr(), normed.data_ptr(), m, n_in,
+                                         torch.cuda.current_stream(dev).cuda_stream), "ttq_rmsnorm")
+
+            _, ev_ms = time_steps(norm_step, steps, warmup, use_graph=not args.eager)
+            nm = "add_rmsnorm_m%d" % m
+            res[nm] = {"us_per_step": ev_ms * 1e3, "GBps": 4.0 * m * n_in * 2 / (ev_ms * 1e-3) / 1e9}
+            log("[%s] %.2f us/step  %.0f GB/s" % (nm, ev_ms * 1e3, res[nm]["GBps"]))
+            del xs, rs
+            torch.cuda.empty_cache()
         return res
 
     if args.only == "widened":
