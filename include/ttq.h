@@ -171,7 +171,9 @@ TTQ_API int ttq_gemv_q4_k_silu_mul(const void* w, const void* x, int x_dtype, vo
  * gamma is (n).  Stands in for RmsNorm.forward (residual = NULL) and
  * RmsNorm.forward_with_residual, which returns (normalized, new_residual)
  * (workspace/transformers/src/layers/norm.nim:23-38; torch::rms_norm,
- * workspace/libtorch/src/abi/neural_nets.nim:144-146).  new_residual_out may be NULL. */
+ * workspace/libtorch/src/abi/neural_nets.nim:144-146).  new_residual_out may be NULL.
+ * The outputs may be the inputs (normed_out == x, new_residual_out == residual: the in-place
+ * add of the residual stream); other overlaps are not allowed.  All pointers 16-byte aligned. */
 TTQ_API int ttq_rmsnorm(const void* x, const void* residual, const void* gamma, float eps, int dtype,
                 void* new_residual_out, void* normed_out, int64_t m, int64_t n, void* stream);
 /* y = Linear(RmsNorm(x [, residual])) in one kernel for a Q4_K weight and 16-bit activations:
