@@ -287,21 +287,22 @@ def main() -> int:
 
     def run_widened(steps: int, warmup: int):
         """Rows next to the headline ones, on random packed bytes with finite scale fields (timing
-        only): the few-row decode GEMV (8 and 16 activation rows at once) and the prefill GEMM for
-        Q6_K and Q8_0 weights, all 14336 x 4096; add + RMSNorm on rows of 4096."""
+        only): the few-row decode GEMV (8 and 16 activation rows at once), the few-row form of the
+        prefill operator (32 rows) and the prefill GEMM for Q6_K and Q8_0 weights, 14336 x 4096 unless
+        named otherwise; add + RMSNorm on rows of 4096."""
         n_out, n_in = 14336, 4096
         rng = np.random.default_rng(1234)
         res = {}
 
-        def random_packed(fmt):
+        def random_packed(fmt, n_out=n_out, n_in=n_in):
             nbytes, wpb, scale_hi = {F.Q8_0: (34, 32, [1]), F.Q4_K: (144, 256, [1, 3]), F.Q6_K: (210, 256, [209])}[fmt]
             raw = rng.integers(0, 256, (n_out * (n_in // wpb), nbytes), dtype=np.uint8)
             for off in scale_hi:
                 raw[:, off] &= 0x3F            # |fp16 scale| < 2
             return raw.reshape(-1)
 
-        def timed(name, fmt, m, fn_of):
-            packed = random_packed(fmt)
+        def timed(name, fmt, m, fn_of, n_out=n_out, n_in=n_in):
+            packed = random_packed(fmt, n_out, n_in)
             ncopies = max(2, -(-2 * MALL_BYTES // packed.nbytes))
             ws = [to_dev(packed) for _ in range(ncopies)]
             x = torch.randn((m, n_in), device=dev).to(torch.bfloat16)
@@ -318,6 +319,13 @@ def main() -> int:
             y = torch.empty((m, n_out), dtype=torch.float32, device=dev)
             timed("q4_k_gemv_m%d" % m, F.Q4_K, m,
                   lambda ws, x, nc, y=y: (lambda i: QL.gemv(F.Q4_K, ws[i % nc], x, n_out, n_in, out=y)))
+        # 17..64 rows: the prefill operator's few-row kernel (weights dequantized in registers), on the
+        # up/gate shape and on the down projection (few weight rows, long K)
+        for nm, (no, ni) in (("q4_k_gemm_m32", (n_out, n_in)), ("q4_k_gemm_m32_down_4096x14336", (n_in, n_out))):
+            y = torch.empty((32, no), dtype=torch.bfloat16, device=dev)
+            timed(nm, F.Q4_K, 32,
+                  lambda ws, x, nc, y=y, no=no, ni=ni: (lambda i: QL.gemm(F.Q4_K, ws[i % nc], x, no, ni, out=y)),
+                  n_out=no, n_in=ni)
         for fmt, nm in ((F.Q6_K, "q6_k_gemm_m512"), (F.Q8_0, "q8_0_gemm_m512")):
             y = torch.empty((512, n_out), dtype=torch.bfloat16, device=dev)
             timed(nm, fmt, 512,

@@ -27,6 +27,7 @@ SOURCES = [
     "ttq_gemv_q4k_batch4.hip",
     "ttq_gemm_q4k.hip",
     "ttq_gemm_pc.hip",
+    "ttq_gemm_skinny.hip",
     "ttq_exl3.hip",
     "ttq_activations.hip",
     "ttq_host.cpp",

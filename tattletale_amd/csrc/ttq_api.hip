@@ -7,6 +7,22 @@
 #include "../../include/ttq.h"
 #include "ttq_internal.h"
 
+namespace ttq {
+
+int device_num_cus() {
+  static int cached = 0;
+  if (cached == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    cached = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+              prop.multiProcessorCount > 0)
+                 ? prop.multiProcessorCount : 256;
+  }
+  return cached;
+}
+
+}  // namespace ttq
+
 namespace {
 
 thread_local int g_last_hip_error = 0;
@@ -281,8 +297,10 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
                        ttq::gemm_pc_supported(layer->format, m, n_out, n_in, 112);
   if (gemm_ok && m >= 5) {
     const bool gemv_ok = check_gemv_limits(x_dtype, n_in) == TTQ_OK;
-    if (!gemv_ok || ttq::gemm_pc_estimate_us(layer->format, m, n_out, n_in) <
-                        ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in)) {
+    float gemm_us = ttq::gemm_pc_estimate_us(layer->format, m, n_out, n_in);
+    if (ttq::gemm_skinny_supported(layer->format, m, n_out, n_in))
+      gemm_us = fminf(gemm_us, ttq::gemm_skinny_estimate_us(m, n_out, n_in));
+    if (!gemv_ok || gemm_us < ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in)) {
       if (layer->format == TTQ_Q4_K)
         return hip_status(ttq::launch_gemm_q4k(layer->qweight, static_cast<const uint16_t*>(x), y, y_dtype,
                                                layer->bias, layer->bias_dtype, m, n_out, n_in, s));

@@ -600,15 +600,7 @@ constexpr float kPcFixedUs = 6.f;
 
 static int pc_choose_tile(int64_t m, int64_t n_out, int64_t n_in, bool fuse, float* cost_us = nullptr) {
   static const int forced = [] { const char* e = getenv("TTQ_GEMM_TILE"); return e ? atoi(e) : -1; }();
-  int cus = 256;
-  {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    static int cached = 0;
-    if (cached == 0 && hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-      cached = prop.multiProcessorCount;
-    if (cached > 0) cus = cached;
-  }
+  const int cus = device_num_cus();
   int best = 0;
   float best_cost = 1e30f;
   for (int i = 0; i < (int)(sizeof(kPcTiles) / sizeof(kPcTiles[0])); i++) {

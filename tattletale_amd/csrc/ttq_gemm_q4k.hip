@@ -362,17 +362,6 @@ gemm_q4k_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, Y
   }
 }
 
-static int gemm_num_cus() {
-  static int cached = 0;
-  if (cached == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    cached = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-                 ? prop.multiProcessorCount : 256;
-  }
-  return cached;
-}
-
 static int env_flag(const char* name, int dflt) {
   const char* e = getenv(name);
   return e ? atoi(e) : dflt;
@@ -415,8 +404,14 @@ hipError_t launch_gemm_q4k(const void* w, const uint16_t* x_bf16, void* y, int y
                            const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                            hipStream_t s) {
   if (m == 0 || n_out == 0) return hipSuccess;
+  // up to 64 rows: weights dequantized in registers, no tile of W in LDS (ttq_gemm_skinny.hip),
+  // where that is estimated to be faster than the tiled kernel
+  if (gemm_skinny_supported(kQ4_K, m, n_out, n_in) &&
+      (!gemm_pc_supported(kQ4_K, m, n_out, n_in, 112) ||
+       gemm_skinny_estimate_us(m, n_out, n_in) < gemm_pc_estimate_us(kQ4_K, m, n_out, n_in)))
+    return launch_gemm_skinny(w, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   // Pick the tile width that needs the least time: rounds of tiles over the CUs times tile width.
-  const int64_t cus = gemm_num_cus();
+  const int64_t cus = device_num_cus();
   const int64_t mt = (m + kGemmBM - 1) / kGemmBM;
   auto cost = [&](int64_t bn) { return ((((n_out + bn - 1) / bn) * mt + cus - 1) / cus) * bn; };
   static const int forced = [] { const char* e = getenv("TTQ_GEMM_BN"); return e ? atoi(e) : 0; }();

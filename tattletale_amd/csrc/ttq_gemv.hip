@@ -269,17 +269,7 @@ static int gemv_grid(int64_t n_out, int default_per_cu) {
     per_cu_env = e ? atoi(e) : 0;
   }
   const int per_cu = per_cu_env > 0 ? per_cu_env : default_per_cu;
-  int cus = 256;
-  int dev = 0;
-  hipDeviceProp_t prop;
-  static int cached_cus = 0;
-  if (cached_cus == 0) {
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-      cached_cus = prop.multiProcessorCount;
-    else
-      cached_cus = cus;
-  }
-  cus = cached_cus;
+  const int cus = device_num_cus();
   int64_t g = (int64_t)cus * per_cu;
   const int64_t need = (n_out + kGemvWaves - 1) / kGemvWaves;
   if (g > need) g = need;

@@ -660,19 +660,6 @@ gemv_dot2_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
 }
 
 // ------------------------------------------------------------------------------ launch
-static int num_cus() {
-  static int cached = 0;
-  if (cached == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-      cached = prop.multiProcessorCount;
-    else
-      cached = 256;
-  }
-  return cached;
-}
-
 static int env_int(const char* name, int dflt) {
   const char* e = getenv(name);
   return e ? atoi(e) : dflt;
@@ -684,7 +671,7 @@ static hipError_t launch_fmt_t(const void* w, const void* x, void* y, const void
   static const int wg_per_cu = env_int("TTQ_GEMV_WG_PER_CU", 1);
   const int units = (int)(n_in / 64);
   const int nit = (units + 63) / 64;
-  int64_t waves = (int64_t)num_cus() * wg_per_cu * kFastWaves;
+  int64_t waves = (int64_t)device_num_cus() * wg_per_cu * kFastWaves;
   if (waves > n_out) waves = n_out;
   int rows_per_wave = (int)((n_out + waves - 1) / waves);
   const int64_t used_waves = (n_out + rows_per_wave - 1) / rows_per_wave;
@@ -753,7 +740,7 @@ static hipError_t launch_multi_t(const void* w, const void* x, void* y, const vo
                                  int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
   const int units = (int)(n_in / 64);
   const int nit = (units + 63) / 64;
-  int64_t waves = (int64_t)num_cus() * kFastWaves;
+  int64_t waves = (int64_t)device_num_cus() * kFastWaves;
   if (waves > n_out) waves = n_out;
   const int rows_per_wave = (int)((n_out + waves - 1) / waves);
   const int64_t used_waves = (n_out + rows_per_wave - 1) / rows_per_wave;

@@ -90,6 +90,16 @@ float gemv_estimate_us(int format, int x_dtype, int64_t m, int64_t n_out, int64_
 float gemm_pc_estimate_us(int format, int64_t m, int64_t n_out, int64_t n_in);
 int gemv_q4k_batch_tokens(int64_t m, int64_t n_in);
 
+// Compute units of the current device (256 when the query fails); cached after the first call.
+int device_num_cus();
+
+// Q4_K linear layer for up to 64 rows of bf16 activations, weights dequantized in registers
+// (ttq_gemm_skinny.hip).
+bool gemm_skinny_supported(int format, int64_t m, int64_t n_out, int64_t n_in);
+float gemm_skinny_estimate_us(int64_t m, int64_t n_out, int64_t n_in);
+hipError_t launch_gemm_skinny(const void* w, const uint16_t* x_bf16, void* y, int y_dtype, const void* bias,
+                              int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s);
+
 // Producer/consumer GEMM for Q4_K / Q6_K / Q8_0 weights and bf16 activations (ttq_gemm_pc.hip).
 bool gemm_pc_supported(int format, int64_t m, int64_t n_out, int64_t n_in, int bn);
 hipError_t launch_gemm_pc(int format, const void* w, const uint16_t* x_bf16, void* y, int y_dtype,
