@@ -22,14 +22,22 @@ namespace ttq {
 
 typedef __attribute__((ext_vector_type(2))) _Float16 half2_t;
 
+// The codebook: a pure function of the 16-bit trellis state (bits 16..31 of `state` are ignored).
+// The 32-bit multiply is not what limits the decode here: splitting it into two 16-bit
+// multiply-adds was measured slower.
 template <int CB>
-__device__ __forceinline__ _Float16 exl3_code(uint32_t state) {
-  uint32_t u = (CB == 0) ? (state * 89226354u + 64248484u) : (state * 0xCBAC1FEDu);
-  u = (u & 0x8FFF8FFFu) ^ 0x3B603B60u;
-  half2_t h;
-  __builtin_memcpy(&h, &u, 4);
-  return h[0] + h[1];  // fp16 add, round-to-nearest-even
-}
+struct Codebook {
+  static constexpr uint32_t kMul = (CB == 0) ? 89226354u : 0xCBAC1FEDu;
+  __device__ __forceinline__ void init() {}
+  __device__ __forceinline__ _Float16 code(uint32_t state) const {
+    uint32_t u = (state & 0xFFFFu) * kMul;
+    if (CB == 0) u += 64248484u;
+    u = (u & 0x8FFF8FFFu) ^ 0x3B603B60u;
+    half2_t h;
+    __builtin_memcpy(&h, &u, 4);
+    return h[0] + h[1];  // fp16 add, round-to-nearest-even
+  }
+};
 
 // The bits+1 words that hold the 16 windows of output channel j of a tile, as big-endian
 // 32-bit chunks (first stream bit = bit 31 of chunk 0).
@@ -38,35 +46,49 @@ struct LaneBits {
   static constexpr int kWords = BITS + 1;
   static constexpr int kChunks = (kWords + 1) / 2;
   uint32_t c[kChunks];
+  // One load of the 2 * kWords bytes plus the tile's first word.  Channels 0..14 read their words
+  // where they lie; channel 15, whose last word is the tile's first (the string is cyclic), starts
+  // one word early so that it never reads past the tile, and shifts by a word while the 16-bit
+  // halves are swapped into stream order (a byte permute either way).
   __device__ __forceinline__ void load(const uint16_t* tile, int j) {
-    constexpr int words = 16 * BITS;
-    uint32_t w[2 * kChunks];
+    const bool last = j == 15;
+    const uint16_t* p = tile + j * BITS - (last ? 1 : 0);
+    uint16_t w[kWords];
+    __builtin_memcpy(w, __builtin_assume_aligned(p, 2), 2 * kWords);
+    const uint32_t wrap = tile[0];
+    // little-endian dwords of the words, continued by the wrap word: d[i] = w[2i] | w[2i+1] << 16
+    uint32_t d[kChunks + 1];
 #pragma unroll
-    for (int t = 0; t < 2 * kChunks; t++) {
-      int idx = j * BITS + t;
-      if (idx >= words) idx -= words;  // cyclic wrap (only channel 15 reaches it)
-      w[t] = (t < kWords) ? (uint32_t)tile[idx] : 0u;
+    for (int i = 0; i <= kChunks; i++) {
+      const uint32_t lo = 2 * i < kWords ? (uint32_t)w[2 * i] : (2 * i == kWords ? wrap : 0u);
+      const uint32_t hi = 2 * i + 1 < kWords ? (uint32_t)w[2 * i + 1] : (2 * i + 1 == kWords ? wrap : 0u);
+      d[i] = lo | (hi << 16);
     }
+    // channels 0..14: (w[2t] << 16) | w[2t+1]; channel 15: (w[2t+1] << 16) | w[2t+2]
+    const uint32_t sel = last ? 0x03020504u : 0x01000302u;
 #pragma unroll
-    for (int t = 0; t < kChunks; t++) c[t] = (w[2 * t] << 16) | w[2 * t + 1];
+    for (int t = 0; t < kChunks; t++) c[t] = __builtin_amdgcn_perm(d[t + 1], d[t], sel);
   }
+  // the window of weight KK in bits 0..15; bits 16..31 hold whatever precedes it in the stream
   template <int KK>
   __device__ __forceinline__ uint32_t state() const {
     constexpr int q = KK * BITS;
     constexpr int ci = q >> 5, o = q & 31;
-    if constexpr (o <= 16) {
-      return (c[ci] >> (16 - o)) & 0xFFFFu;
+    if constexpr (o == 16) {
+      return c[ci];
+    } else if constexpr (o < 16) {
+      return c[ci] >> (16 - o);
     } else {
-      return __builtin_amdgcn_alignbit(c[ci], c[ci + 1 < kChunks ? ci + 1 : ci], 48 - o) & 0xFFFFu;
+      return __builtin_amdgcn_alignbit(c[ci], c[ci + 1 < kChunks ? ci + 1 : ci], 48 - o);
     }
   }
 };
 
 template <int BITS, int CB, int KK>
 struct DecodeLoop {
-  static __device__ __forceinline__ void run(const LaneBits<BITS>& lb, _Float16* out) {
-    out[KK] = exl3_code<CB>(lb.template state<KK>());
-    if constexpr (KK + 1 < 16) DecodeLoop<BITS, CB, KK + 1>::run(lb, out);
+  static __device__ __forceinline__ void run(const LaneBits<BITS>& lb, const Codebook<CB>& cb, _Float16* out) {
+    out[KK] = cb.code(lb.template state<KK>());
+    if constexpr (KK + 1 < 16) DecodeLoop<BITS, CB, KK + 1>::run(lb, cb, out);
   }
 };
 
@@ -83,8 +105,10 @@ __global__ void __launch_bounds__(256) dequant_exl3_kernel(const uint16_t* __res
   const int64_t kt = tile / nt_n, nt = tile % nt_n;
   LaneBits<BITS> lb;
   lb.load(trellis + tile * (16 * BITS), j);
+  Codebook<CB> cb;
+  cb.init();
   _Float16 v[16];
-  DecodeLoop<BITS, CB, 0>::run(lb, v);
+  DecodeLoop<BITS, CB, 0>::run(lb, cb, v);
   uint16_t* o = out + (nt * 16 + j) * (int64_t)n_in + kt * 16;
 #pragma unroll
   for (int kk = 0; kk < 16; kk++) {
@@ -117,6 +141,24 @@ __device__ __forceinline__ void fwht128_quad(float (&v)[4], int lane) {
       v[i] = upper ? (o - v[i]) : (v[i] + o);
     }
   }
+}
+
+// Four consecutive activations (a multiple of four elements from the row start) as floats.
+__device__ __forceinline__ void load_x4(const float* p, float (&v)[4]) {
+  const float4 t = *reinterpret_cast<const float4*>(__builtin_assume_aligned(p, 16));
+  v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+__device__ __forceinline__ void load_x4(const f16_tag* p, float (&v)[4]) {
+  uint2 r;
+  __builtin_memcpy(&r, __builtin_assume_aligned(p, 8), 8);
+  v[0] = f16_bits_to_f32((uint16_t)r.x); v[1] = f16_bits_to_f32((uint16_t)(r.x >> 16));
+  v[2] = f16_bits_to_f32((uint16_t)r.y); v[3] = f16_bits_to_f32((uint16_t)(r.y >> 16));
+}
+__device__ __forceinline__ void load_x4(const bf16_tag* p, float (&v)[4]) {
+  uint2 r;
+  __builtin_memcpy(&r, __builtin_assume_aligned(p, 8), 8);
+  v[0] = bf16_bits_to_f32((uint16_t)r.x); v[1] = bf16_bits_to_f32((uint16_t)(r.x >> 16));
+  v[2] = bf16_bits_to_f32((uint16_t)r.y); v[3] = bf16_bits_to_f32((uint16_t)(r.y >> 16));
 }
 
 // One workgroup per n_tile (16 output channels).  Lane = (k-tile slot g = lane/16, channel
@@ -153,16 +195,18 @@ gemv_exl3_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __restric
 
   // input side: x o suh, then the Hadamard rotation of every group of 128 (32 lanes x 4 values)
   for (int k4 = tid * 4; k4 < n_in; k4 += kExl3Threads * 4) {
-    float sg[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) sg[i] = f16_bits_to_f32(suh[k4 + i]);
+    uint2 sraw;
+    __builtin_memcpy(&sraw, __builtin_assume_aligned(suh + k4, 8), 8);
+    const float sg[4] = {f16_bits_to_f32((uint16_t)sraw.x), f16_bits_to_f32((uint16_t)(sraw.x >> 16)),
+                         f16_bits_to_f32((uint16_t)sraw.y), f16_bits_to_f32((uint16_t)(sraw.y >> 16))};
 #pragma unroll
     for (int t = 0; t < TOK; t++) {
       if (t < ntok) {          // uniform; no `break`, so that the loop unrolls and acc[] stays in registers
         const XT* xm = x + (int64_t)(t0 + t) * n_in;
         float v[4];
+        load_x4(xm + k4, v);
 #pragma unroll
-        for (int i = 0; i < 4; i++) v[i] = XElem<XT>::load(xm, k4 + i) * sg[i];
+        for (int i = 0; i < 4; i++) v[i] *= sg[i];
         fwht128_quad(v, lane);
         *reinterpret_cast<float4*>(xs + (size_t)t * n_in + k4) = make_float4(v[0], v[1], v[2], v[3]);
       }
@@ -171,9 +215,13 @@ gemv_exl3_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __restric
   __syncthreads();
   const float kNorm = 0.08838834764831845f;  // 1/sqrt(128), applied to the dot product
 
-  float acc[TOK];
+  Codebook<CB> cb;
+  cb.init();
+  // two partial sums per token (even and odd quads of the tile row): independent chains for the
+  // multiply-adds
+  float acc[TOK][2];
 #pragma unroll
-  for (int t = 0; t < TOK; t++) acc[t] = 0.f;
+  for (int t = 0; t < TOK; t++) acc[t][0] = acc[t][1] = 0.f;
   for (int ktb = kt0; ktb < kt_n; ktb += kPre * kStride) {
     LaneBits<BITS> nxt[kPre];
     const bool more = ktb + kPre * kStride < kt_n;
@@ -183,24 +231,21 @@ gemv_exl3_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __restric
       const int kt = ktb + i * kStride;
       if (kt < kt_n) {
         _Float16 v[16];
-        DecodeLoop<BITS, CB, 0>::run(cur[i], v);
-        float vf[16];
-#pragma unroll
-        for (int e = 0; e < 16; e++) vf[e] = (float)v[e];
+        DecodeLoop<BITS, CB, 0>::run(cur[i], cb, v);
 #pragma unroll
         for (int t = 0; t < TOK; t++) {
           if (t < ntok) {
             const float4* xv = reinterpret_cast<const float4*>(xs + (size_t)t * n_in + 16 * kt);
-            float a = acc[t];
 #pragma unroll
             for (int q = 0; q < 4; q++) {
               const float4 xq = xv[q];
-              a = fmaf_(vf[4 * q + 0], xq.x, a);
-              a = fmaf_(vf[4 * q + 1], xq.y, a);
-              a = fmaf_(vf[4 * q + 2], xq.z, a);
-              a = fmaf_(vf[4 * q + 3], xq.w, a);
+              float a = acc[t][q & 1];
+              a = fmaf_((float)v[4 * q + 0], xq.x, a);
+              a = fmaf_((float)v[4 * q + 1], xq.y, a);
+              a = fmaf_((float)v[4 * q + 2], xq.z, a);
+              a = fmaf_((float)v[4 * q + 3], xq.w, a);
+              acc[t][q & 1] = a;
             }
-            acc[t] = a;
           }
         }
       }
@@ -213,7 +258,7 @@ gemv_exl3_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __restric
   float* red = xs + (size_t)TOK * n_in;
 #pragma unroll
   for (int t = 0; t < TOK; t++) {
-    float a = acc[t];
+    float a = acc[t][0] + acc[t][1];
     a += __shfl_xor(a, 16, kWave);
     a += __shfl_xor(a, 32, kWave);
     if (lane < 16) red[(t * kExl3Waves + wave) * 16 + lane] = a;
