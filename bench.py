@@ -353,6 +353,31 @@ def main() -> int:
             torch.cuda.empty_cache()
         return res
 
+    def run_dense_reference(steps: int, warmup: int):
+        """Context, not the product: the vendor library's plain bf16 linear (torch -> hipBLASLt) on
+        dense 14336 x 4096 weights, i.e. what the reference's Linear.forward would run on this GPU
+        after dequantizing once.  Same timing method, weight copies rotated past the cache."""
+        n_out, n_in = 14336, 4096
+        ncopies = max(2, -(-2 * MALL_BYTES // (n_out * n_in * 2)))
+        ws = [torch.randn((n_out, n_in), device=dev).mul_(0.02).to(torch.bfloat16) for _ in range(ncopies)]
+        res = {}
+        for m in (1, 512, 2048):
+            x = torch.randn((m, n_in), device=dev).to(torch.bfloat16)
+            y = torch.empty((m, n_out), dtype=torch.bfloat16, device=dev)
+            n = max(10, steps // (1 if m == 1 else 4))
+            _, ev_ms = time_steps(lambda i: torch.matmul(x, ws[i % ncopies].t(), out=y), n, warmup,
+                                  use_graph=not args.eager)
+            res["m%d" % m] = {"us_per_step": ev_ms * 1e3, "TFLOPs": 2.0 * m * n_out * n_in / (ev_ms * 1e-3) / 1e12,
+                              "weight_GBps": n_out * n_in * 2 / (ev_ms * 1e-3) / 1e9}
+            log("[dense_bf16_library m=%d] %.2f us/step  %.1f TFLOP/s  %.0f GB/s of bf16 weights" % (
+                m, ev_ms * 1e3, res["m%d" % m]["TFLOPs"], res["m%d" % m]["weight_GBps"]))
+        del ws
+        torch.cuda.empty_cache()
+        return res
+
+    if args.only == "dense_reference":
+        print(json.dumps(run_dense_reference(max(20, args.steps // 10), max(3, args.warmup // 10))), flush=True)
+        return 0
     if args.only == "widened":
         print(json.dumps(run_widened(max(20, args.steps // 4), max(3, args.warmup // 4))), flush=True)
         return 0
@@ -414,6 +439,8 @@ def main() -> int:
     if not args.only and not args.no_extra:
         line["extra"]["q4_k_gate_up_silu_gemv"] = run_gate_up(max(20, args.steps // 4), max(3, args.warmup // 4))
         line["extra"]["widened"] = run_widened(max(20, args.steps // 4), max(3, args.warmup // 4))
+        line["extra"]["dense_bf16_library_14336x4096"] = run_dense_reference(max(20, args.steps // 10),
+                                                                             max(3, args.warmup // 10))
     print(json.dumps(line), flush=True)
     return 0
 
