@@ -10,15 +10,30 @@
 namespace ttq {
 
 int device_num_cus() {
-  static int cached = 0;
-  if (cached == 0) {
-    int dev = 0;
+  static std::atomic<int> cached[64];     // by device ordinal; 0 = not asked yet
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 256;
+  std::atomic<int>& slot = cached[dev & 63];
+  int cus = slot.load(std::memory_order_relaxed);
+  if (cus == 0) {
     hipDeviceProp_t prop;
-    cached = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
-              prop.multiProcessorCount > 0)
-                 ? prop.multiProcessorCount : 256;
+    cus = (hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0)
+              ? prop.multiProcessorCount : 256;
+    slot.store(cus, std::memory_order_relaxed);
   }
-  return cached;
+  return cus;
+}
+
+hipError_t allow_large_lds(const void* kernel, LargeLds& state) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (state.done.load(std::memory_order_relaxed) & bit) return hipSuccess;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  if (e != hipSuccess) return e;
+  state.done.fetch_or(bit, std::memory_order_relaxed);
+  return hipSuccess;
 }
 
 }  // namespace ttq

@@ -360,12 +360,10 @@ static hipError_t gemv_bits_cb_t(const uint16_t* trellis, const uint16_t* suh, c
   const size_t lds = ((size_t)TOK * n_in + (size_t)kExl3Waves * 16 * TOK) * sizeof(float);
   auto kernel = gemv_exl3_kernel<BITS, CB, XT, TOK>;
   if (lds > 64 * 1024) {
-    static bool configured = false;
-    if (!configured) {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    static LargeLds configured;
+    {
+      const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), configured);
       if (e != hipSuccess) return e;
-      configured = true;
     }
   }
   hipLaunchKernelGGL(kernel, grid, block, lds, s, trellis, suh, static_cast<const XT*>(x), y, (int)m, (int)n_out,

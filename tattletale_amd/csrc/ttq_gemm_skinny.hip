@@ -228,12 +228,10 @@ hipError_t launch_skinny_tb(const uint8_t* w, const uint16_t* x, void* y, int y_
                             int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
   auto kernel = gemm_q4k_skinny_kernel<RB, TB, WD, XB>;
   const size_t lds = (size_t)(kSkWaves * RB * TB * 4 * 64 + 16 * TB * (16 * RB + 1)) * sizeof(float);
-  static bool configured = false;
-  if (lds > 64 * 1024 && !configured) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  static LargeLds configured;
+  if (lds > 64 * 1024) {
+    const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), configured);
     if (e != hipSuccess) return e;
-    configured = true;
   }
   const dim3 grid((unsigned)((n_out + 16 * RB - 1) / (16 * RB))), block(kSkThreads);
   hipLaunchKernelGGL(kernel, grid, block, lds, s, w, x, y, y_dtype, bias, bias_dtype, (int)m, (int)n_out, (int)n_in);

@@ -690,12 +690,10 @@ static hipError_t launch_fmt_t(const void* w, const void* x, void* y, const void
                        static_cast<YT*>(y), bias, bias_dtype, (int)n_out, (int)n_in, rows_per_wave, 0);
   else {
     auto kernel = gemv_dot2_kernel<F, Ops, YT, false>;
-    static bool configured = false;
-    if (lds > 64 * 1024 && !configured) {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    static LargeLds configured;
+    if (lds > 64 * 1024) {
+      const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), configured);
       if (e != hipSuccess) return e;
-      configured = true;
     }
     hipLaunchKernelGGL(kernel, grid, block, lds, s, wb, xb, static_cast<YT*>(y), bias, bias_dtype, (int)n_out,
                        (int)n_in, rows_per_wave, flat);
@@ -748,12 +746,10 @@ static hipError_t launch_multi_t(const void* w, const void* x, void* y, const vo
       block(kFastThreads);
   const size_t lds = (size_t)TOK * nit * 2048 * sizeof(uint32_t);
   auto kernel = gemv_dot2_multi_kernel<F, Ops, YT, TOK>;
-  static bool configured = false;
-  if (lds > 64 * 1024 && !configured) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  static LargeLds configured;
+  if (lds > 64 * 1024) {
+    const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), configured);
     if (e != hipSuccess) return e;
-    configured = true;
   }
   hipLaunchKernelGGL(kernel, grid, block, lds, s, static_cast<const uint8_t*>(w), static_cast<const uint16_t*>(x),
                      static_cast<YT*>(y), bias, bias_dtype, (int)m, (int)n_out, (int)n_in, rows_per_wave);

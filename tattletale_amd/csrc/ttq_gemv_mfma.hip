@@ -433,19 +433,17 @@ static hipError_t launch_xy(const void* w, const void* x, void* y, const void* b
   const bool compact = nsb > kMaxWideSb;
   const size_t lds = (compact ? (size_t)nsb * 512 + 16 : (size_t)nsb * 4096) + (size_t)nsb * 64 + 1024;
   const dim3 grid((unsigned)num_wg, (unsigned)m), block(W * 64);
-  const auto launch = [&](auto kernel, bool& configured) -> hipError_t {
-    if (!configured) {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  const auto launch = [&](auto kernel, LargeLds& configured) -> hipError_t {
+    {
+      const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), configured);
       if (e != hipSuccess) return e;
-      configured = true;
     }
     hipLaunchKernelGGL(kernel, grid, block, lds, s, static_cast<const uint8_t*>(w),
                        static_cast<const uint16_t*>(x), static_cast<YT*>(y), bias, bias_dtype, (int)n_out, nsb,
                        rows_per_wg, sl_log2, na);
     return hipGetLastError();
   };
-  static bool configured_wide = false, configured_compact = false;
+  static LargeLds configured_wide, configured_compact;
   if (compact) return launch(gemv_q4k_mfma_kernel<W, kMfmaRing, FUSE, true, NORM, XT, YT>, configured_compact);
   return launch(gemv_q4k_mfma_kernel<W, kMfmaRing, FUSE, false, NORM, XT, YT>, configured_wide);
 }

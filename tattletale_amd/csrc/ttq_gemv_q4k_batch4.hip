@@ -247,12 +247,10 @@ static hipError_t batch4_launch_xy(const void* w, const void* x, void* y, const 
   int sl_log2 = 0;
   while ((2 << sl_log2) <= W && (2 << sl_log2) <= nsb && (16 * W >> (sl_log2 + 1)) >= rows_per_wg) sl_log2++;
   auto kernel = gemv_q4k_batch4_kernel<XT, YT>;
-  static bool configured = false;
-  if (!configured) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  static LargeLds configured;
+  {
+    const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), configured);
     if (e != hipSuccess) return e;
-    configured = true;
   }
   hipLaunchKernelGGL(kernel, dim3((unsigned)num_wg, (unsigned)((m + 3) / 4)), dim3(W * 64), batch4_lds_bytes(nsb), s,
                      static_cast<const uint8_t*>(w), static_cast<const uint16_t*>(x), static_cast<YT*>(y), bias,

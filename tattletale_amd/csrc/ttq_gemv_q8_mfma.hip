@@ -247,12 +247,10 @@ static hipError_t q8_launch_xy(const void* w, const void* x, void* y, const void
   int sl_log2 = 0;
   while ((2 << sl_log2) <= W && (2 << sl_log2) <= nst && (16 * W >> (sl_log2 + 1)) >= rows_per_wg) sl_log2++;
   const size_t lds = (size_t)nst * 2048 + (size_t)nst * 16 + 1024;
-  const auto launch = [&](auto kernel, bool& configured) -> hipError_t {
-    if (!configured) {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  const auto launch = [&](auto kernel, LargeLds& configured) -> hipError_t {
+    {
+      const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), configured);
       if (e != hipSuccess) return e;
-      configured = true;
     }
     hipLaunchKernelGGL(kernel, dim3((unsigned)num_wg, (unsigned)m), dim3(W * 64), lds, s,
                        static_cast<const uint8_t*>(w), static_cast<const typename Q8X<XT>::elem_t*>(x),
@@ -266,7 +264,7 @@ static hipError_t q8_launch_xy(const void* w, const void* x, void* y, const void
   const int rounds = (rows_per_wg + (16 * W >> sl_log2) - 1) / (16 * W >> sl_log2);
   static const int forced = mfma_env_int("TTQ_GEMV_Q8_RING", 0);
   const bool two = forced ? forced == 2 : rounds * S <= 2;
-  static bool configured1 = false, configured2 = false;
+  static LargeLds configured1, configured2;
   if (two) return launch(gemv_q8_mfma_kernel<2, XT, YT>, configured2);
   return launch(gemv_q8_mfma_kernel<1, XT, YT>, configured1);
 }

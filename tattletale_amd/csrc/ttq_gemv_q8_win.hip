@@ -356,19 +356,17 @@ static hipError_t q8win_launch_xy(const void* w, const void* x, void* y, const v
   const bool compact = tok > 1 || nch > kQ8WinMaxWideChunks;
   const size_t lds = lds_for(compact, tok);
   const dim3 grid((unsigned)num_wg, (unsigned)((m + tok - 1) / tok));
-  const auto launch = [&](auto kernel, bool& configured) -> hipError_t {
-    if (!configured) {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  const auto launch = [&](auto kernel, LargeLds& configured) -> hipError_t {
+    {
+      const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), configured);
       if (e != hipSuccess) return e;
-      configured = true;
     }
     hipLaunchKernelGGL(kernel, grid, dim3(W * 64), lds, s, static_cast<const uint8_t*>(w),
                        static_cast<const typename Q8WX<XT>::elem_t*>(x), static_cast<YT*>(y), bias, bias_dtype, (int)m,
                        (int)n_out, nch, rows_per_wg, sl_log2);
     return hipGetLastError();
   };
-  static bool configured_wide = false, configured_compact = false, configured_2 = false, configured_4 = false;
+  static LargeLds configured_wide, configured_compact, configured_2, configured_4;
   if (tok == 4) return launch(gemv_q8_win_kernel<true, 4, XT, YT>, configured_4);
   if (tok == 2) return launch(gemv_q8_win_kernel<true, 2, XT, YT>, configured_2);
   if (compact) return launch(gemv_q8_win_kernel<true, 1, XT, YT>, configured_compact);

@@ -6,6 +6,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace ttq {
 
 // dtype codes as in ttq.h (TTQ_F32 = 0, TTQ_F16 = 1, TTQ_BF16 = 2)
@@ -90,8 +92,14 @@ float gemv_estimate_us(int format, int x_dtype, int64_t m, int64_t n_out, int64_
 float gemm_pc_estimate_us(int format, int64_t m, int64_t n_out, int64_t n_in);
 int gemv_q4k_batch_tokens(int64_t m, int64_t n_in);
 
-// Compute units of the current device (256 when the query fails); cached after the first call.
+// Compute units of the current device (256 when the query fails); cached per device ordinal.
 int device_num_cus();
+
+// Kernels that use more than 64 KiB of dynamic LDS must be allowed to, once per device.  One
+// LargeLds per kernel instantiation (a function-local static) remembers on which device ordinals
+// that has been done.
+struct LargeLds { std::atomic<uint64_t> done{0}; };
+hipError_t allow_large_lds(const void* kernel, LargeLds& state);
 
 // Q4_K linear layer for up to 64 rows of bf16 activations, weights dequantized in registers
 // (ttq_gemm_skinny.hip).
