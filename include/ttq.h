@@ -120,7 +120,9 @@ TTQ_API int ttq_gemv_exl3(const uint16_t* trellis, const uint16_t* suh_f16, cons
 /* ---- prefill GEMM ------------------------------------------------------------------ */
 /* Y[m][n_out] (bf16) = X[m][n_in] (bf16) * W^T, Q4_K weights dequantized to bf16 tiles and
  * multiplied with bf16 MFMA, fp32 accumulation.  Stands in for F.linear(x, weight) with a
- * (batch*seq, n_in) activation (neural_nets.nim:64; attn.nim:154-156 prefill case). */
+ * (batch*seq, n_in) activation (neural_nets.nim:64; attn.nim:154-156 prefill case).
+ * Up to 64 rows may run a kernel that dequantizes in registers instead of tiling W through LDS
+ * (same arithmetic: weights rounded to bf16 once, fp32 accumulation); the library picks by shape. */
 TTQ_API int ttq_gemm_q4_k(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m,
                   int64_t n_out, int64_t n_in, void* stream);
 /* The same operator for Q6_K and Q8_0 weights (a GGUF "Q4_K_M" file mixes Q4_K and Q6_K tensors;

@@ -220,8 +220,8 @@ int ttq_gemm_q4_k(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64
   const int rc = check_shape(TTQ_Q4_K, m, n_out, n_in, 0, 0);
   if (rc != TTQ_OK) return rc;
   if (!aligned16(w) || !aligned16(x_bf16) || !aligned16(y_bf16)) return TTQ_ERR_ALIGN;
-  return hip_status(ttq::launch_gemm_q4k(w, x_bf16, y_bf16, TTQ_BF16, nullptr, 0, m, n_out, n_in,
-                                         static_cast<hipStream_t>(stream)));
+  return hip_status(ttq::launch_gemm(TTQ_Q4_K, w, x_bf16, y_bf16, TTQ_BF16, nullptr, 0, m, n_out, n_in,
+                                     static_cast<hipStream_t>(stream)));
 }
 
 int ttq_gemm_q4_k_silu_mul(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m, int64_t n_ff,
@@ -242,9 +242,9 @@ static int gemm_block(int format, const void* w, const uint16_t* x_bf16, uint16_
   const int rc = check_shape(format, m, n_out, n_in, 0, 0);
   if (rc != TTQ_OK) return rc;
   if (!aligned16(w) || !aligned16(x_bf16) || !aligned16(y_bf16)) return TTQ_ERR_ALIGN;
-  if (!ttq::gemm_pc_supported(format, m, n_out, n_in, 112)) return TTQ_ERR_UNSUPPORTED;
-  return hip_status(ttq::launch_gemm_pc(format, w, x_bf16, y_bf16, TTQ_BF16, nullptr, 0, m, n_out, n_in,
-                                        static_cast<hipStream_t>(stream)));
+  if (!ttq::gemm_supported(format, m, n_out, n_in)) return TTQ_ERR_UNSUPPORTED;
+  return hip_status(ttq::launch_gemm(format, w, x_bf16, y_bf16, TTQ_BF16, nullptr, 0, m, n_out, n_in,
+                                     static_cast<hipStream_t>(stream)));
 }
 int ttq_gemm_q6_k(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m, int64_t n_out,
                   int64_t n_in, void* stream) {
@@ -309,19 +309,13 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
   // decode; a GEMV that the row length rules out leaves only the GEMM.
   const bool gemm_ok = x_dtype == TTQ_BF16 && (y_dtype == TTQ_BF16 || y_dtype == TTQ_F32) &&
                        (layer->format == TTQ_Q4_K || layer->format == TTQ_Q6_K || layer->format == TTQ_Q8_0) &&
-                       ttq::gemm_pc_supported(layer->format, m, n_out, n_in, 112);
+                       ttq::gemm_supported(layer->format, m, n_out, n_in);
   if (gemm_ok && m >= 5) {
     const bool gemv_ok = check_gemv_limits(x_dtype, n_in) == TTQ_OK;
-    float gemm_us = ttq::gemm_pc_estimate_us(layer->format, m, n_out, n_in);
-    if (ttq::gemm_skinny_supported(layer->format, m, n_out, n_in))
-      gemm_us = fminf(gemm_us, ttq::gemm_skinny_estimate_us(m, n_out, n_in));
-    if (!gemv_ok || gemm_us < ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in)) {
-      if (layer->format == TTQ_Q4_K)
-        return hip_status(ttq::launch_gemm_q4k(layer->qweight, static_cast<const uint16_t*>(x), y, y_dtype,
-                                               layer->bias, layer->bias_dtype, m, n_out, n_in, s));
-      return hip_status(ttq::launch_gemm_pc(layer->format, layer->qweight, static_cast<const uint16_t*>(x), y,
-                                            y_dtype, layer->bias, layer->bias_dtype, m, n_out, n_in, s));
-    }
+    if (!gemv_ok || ttq::gemm_estimate_us(layer->format, m, n_out, n_in) <
+                        ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in))
+      return hip_status(ttq::launch_gemm(layer->format, layer->qweight, static_cast<const uint16_t*>(x), y, y_dtype,
+                                         layer->bias, layer->bias_dtype, m, n_out, n_in, s));
   }
   const int lim = check_gemv_limits(x_dtype, n_in);
   if (lim != TTQ_OK) return lim;

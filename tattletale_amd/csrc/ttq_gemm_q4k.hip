@@ -400,16 +400,35 @@ static hipError_t launch_nj(const uint8_t* wb, const uint16_t* x, void* y, int y
   return hipErrorInvalidValue;
 }
 
-hipError_t launch_gemm_q4k(const void* w, const uint16_t* x_bf16, void* y, int y_dtype,
-                           const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
-                           hipStream_t s) {
+// The few-row kernel (ttq_gemm_skinny.hip: up to 64 rows, weights dequantized in registers, no tile
+// of W in LDS) where it exists for the shape and is estimated to be faster than the tiled kernel.
+static bool prefer_skinny(int format, int64_t m, int64_t n_out, int64_t n_in) {
+  return gemm_skinny_supported(format, m, n_out, n_in) &&
+         (!gemm_pc_supported(format, m, n_out, n_in, 112) ||
+          gemm_skinny_estimate_us(format, m, n_out, n_in) < gemm_pc_estimate_us(format, m, n_out, n_in));
+}
+
+bool gemm_supported(int format, int64_t m, int64_t n_out, int64_t n_in) {
+  // Q4_K also has the single-role tiled kernel of this file, which takes any size
+  return format == kQ4_K || gemm_skinny_supported(format, m, n_out, n_in) ||
+         gemm_pc_supported(format, m, n_out, n_in, 112);
+}
+
+float gemm_estimate_us(int format, int64_t m, int64_t n_out, int64_t n_in) {
+  float us = gemm_pc_estimate_us(format, m, n_out, n_in);
+  if (gemm_skinny_supported(format, m, n_out, n_in)) us = fminf(us, gemm_skinny_estimate_us(format, m, n_out, n_in));
+  return us;
+}
+
+hipError_t launch_gemm(int format, const void* w, const uint16_t* x_bf16, void* y, int y_dtype, const void* bias,
+                       int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
   if (m == 0 || n_out == 0) return hipSuccess;
-  // up to 64 rows: weights dequantized in registers, no tile of W in LDS (ttq_gemm_skinny.hip),
-  // where that is estimated to be faster than the tiled kernel
-  if (gemm_skinny_supported(kQ4_K, m, n_out, n_in) &&
-      (!gemm_pc_supported(kQ4_K, m, n_out, n_in, 112) ||
-       gemm_skinny_estimate_us(m, n_out, n_in) < gemm_pc_estimate_us(kQ4_K, m, n_out, n_in)))
-    return launch_gemm_skinny(w, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  if (prefer_skinny(format, m, n_out, n_in))
+    return launch_gemm_skinny(format, w, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  if (format != kQ4_K) {
+    if (!gemm_pc_supported(format, m, n_out, n_in, 112)) return hipErrorInvalidValue;
+    return launch_gemm_pc(format, w, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  }
   // Pick the tile width that needs the least time: rounds of tiles over the CUs times tile width.
   const int64_t cus = device_num_cus();
   const int64_t mt = (m + kGemmBM - 1) / kGemmBM;

@@ -1,5 +1,5 @@
-// Q4_K linear layer for a handful of activation rows (up to 64): the regime between the decode
-// GEMV and the prefill GEMM (batched decoding, speculative verification, short prompts).
+// Q4_K / Q6_K / Q8_0 linear layer for a handful of activation rows (up to 64): the regime between
+// the decode GEMV and the prefill GEMM (batched decoding, speculative verification, short prompts).
 //
 // Same operator as ttq_gemm_q4k.hip (F.linear with seq_len > 1,
 // workspace/libtorch/src/abi/neural_nets.nim:64-81, reached from
@@ -15,12 +15,15 @@
 //     16-byte load per step, and the four lanes of a token read 64 consecutive bytes, so a load
 //     instruction touches 16 cache lines (what such loads cost is lines looked up, not bytes);
 //     the 128 bytes per token block stay in registers for all row blocks of the workgroup;
-//   * for the weights it is the 8 bytes 8*g .. 8*g+7 of each of the four 32-byte qs chunks: low
-//     nibbles for the even sub-block of the chunk, high nibbles for the odd one, dequantized in
-//     registers (canonical arithmetic, one bf16 rounding);
-//   * each lane decodes the scale and min of two sub-blocks (2g, 2g+1) of its row and the four
-//     lanes of a row exchange them through v_mfma_f32_16x16x4_f32 with a 0/1 selector as the other
-//     operand (D[4g'+r][row] = value of lane g = r: an exact all-gather);
+//   * for the weights it is the 8 weights at those k of the lane's row, dequantized in registers
+//     (canonical arithmetic written as one exact fused multiply-add, one bf16 rounding).  Q4_K: the
+//     8 bytes 8*g .. 8*g+7 of each of the four 32-byte qs chunks, low nibbles for the even sub-block
+//     of the chunk, high nibbles for the odd one.  Q6_K: 8 bytes of each ql half-row and 8 of qh per
+//     128 weights.  Q8_0: 8 of the 32 bytes of each block;
+//   * Q4_K: each lane decodes the scale and min of two sub-blocks (2g, 2g+1) of its row and the
+//     four lanes of a row exchange them through v_mfma_f32_16x16x4_f32 with a 0/1 selector as the
+//     other operand (D[4g'+r][row] = value of lane g = r: an exact all-gather).  Q8_0 does the same
+//     with the block scales (two per lane); Q6_K lanes read the row's 16 scale bytes themselves;
 //   * the eight wavefronts' partial sums meet in LDS once, at the end; the sums are transposed
 //     through LDS so that every thread stores 8 consecutive outputs of one token.
 //
@@ -37,16 +40,187 @@ namespace {
 
 constexpr int kSkThreads = 512;
 constexpr int kSkWaves = kSkThreads / 64;
+// time per row block relative to Q4_K (cost model): more unpacking for Q6_K, eighteen small loads per
+// lane and super-block for Q8_0
+constexpr float kSkQ6KWeightFactor = 1.6f, kSkQ8WeightFactor = 3.5f;
 
-struct SkRaw { uint4 hdr; uint2 q[4]; };
+__device__ __forceinline__ uint2 load8_a2(const uint8_t* p) {
+  uint2 v;
+  __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 8);
+  return v;
+}
+
+// D[4g'+r][row] = value of the row's lane g = r, for every g': the four lanes of a row exchange a
+// float each (v_mfma_f32_16x16x4_f32 against a 0/1 selector, exact).
+__device__ __forceinline__ f32x4_t gather_row4(float sel, float v) {
+  const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+  return __builtin_amdgcn_mfma_f32_16x16x4f32(sel, v, zero, 0, 0, 0);
+}
+
+// 8 weights -> 8 bf16 as scale * u + offset for the bytes u of q0 (weights 0..3) and q1 (4..7).
+__device__ __forceinline__ void fma_bytes_to_bf16(uint32_t q0, uint32_t q1, float scale, float offset,
+                                                  uint32_t (&au)[4]) {
+  // keep the words opaque: byte k of them converts with one v_cvt_f32_ubyte<k>
+  asm volatile("" : "+v"(q0), "+v"(q1));
+  float f[8];
+#pragma unroll
+  for (int k = 0; k < 4; k++) {
+    f[k] = fmaf_(scale, (float)((q0 >> (8 * k)) & 0xFFu), offset);
+    f[4 + k] = fmaf_(scale, (float)((q1 >> (8 * k)) & 0xFFu), offset);
+  }
+  au[0] = pack_bf16x2(f[0], f[1]);
+  au[1] = pack_bf16x2(f[2], f[3]);
+  au[2] = pack_bf16x2(f[4], f[5]);
+  au[3] = pack_bf16x2(f[6], f[7]);
+}
+
+// A format supplies: the bytes of 256 weights of a row (kBlockBytes), what lane (row, kg) keeps of
+// them (Raw, fetch), the per-super-block preparation of scales (Prep, prepare) and the 8 bf16
+// weights k = 32*i + 8*kg .. +7 of step i (dequant).
+struct SkQ4K {
+  static constexpr uint32_t kBlockBytes = 144;
+  struct Raw { uint4 hdr; uint2 q[4]; };
+  struct Prep { f32x4_t de, dd, me, md; };
+  // Bit positions of the 6-bit scale and min of sub-blocks 2kg and 2kg+1 in the 12 packed bytes:
+  // sub-blocks 0..3 have the field whole in bytes 0..7, sub-blocks 4..7 four bits in bytes 8..11 and
+  // two on top of bytes 0..7.  Two bit-field extracts each, the second of width 0 in the simple case.
+  struct Lane {
+    float sel;
+    bool upper;
+    uint32_t kg8, wl, wh, sh_sc[2], sh_mn[2], sh_hi[2];
+    __device__ __forceinline__ void init(int li, int kg) {
+      sel = ((li & 3) == kg) ? 1.f : 0.f;
+      kg8 = 8u * kg;
+      upper = kg >= 2;
+      wl = upper ? 4u : 6u;
+      wh = upper ? 2u : 0u;
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const uint32_t jj = (2u * kg + h) & 3u;
+        sh_sc[h] = 8u * jj;
+        sh_mn[h] = upper ? 8u * jj + 4u : 8u * jj;
+        sh_hi[h] = 8u * jj + 6u;
+      }
+    }
+  };
+  static __device__ __forceinline__ void fetch(Raw& r, const uint8_t* p, const Lane& L) {
+    r.hdr = load16_a16(p);
+#pragma unroll
+    for (int c = 0; c < 4; c++) r.q[c] = *reinterpret_cast<const uint2*>(p + 16 + 32 * c + L.kg8);
+  }
+  // this lane: sub-blocks 2kg and 2kg+1 of its row; then all eight from the row's four lanes
+  static __device__ __forceinline__ void prepare(const Raw& r, const Lane& L, Prep& P) {
+    const float d = f16_bits_to_f32((uint16_t)(r.hdr.x & 0xFFFF));
+    const float dmin = f16_bits_to_f32((uint16_t)(r.hdr.x >> 16));
+    const uint32_t a_sc = L.upper ? r.hdr.w : r.hdr.y;   // bytes 8-11 or 0-3
+    const uint32_t a_mn = L.upper ? r.hdr.w : r.hdr.z;   // bytes 8-11 or 4-7
+    const uint32_t sc1 = __builtin_amdgcn_ubfe(a_sc, L.sh_sc[0], L.wl) | (__builtin_amdgcn_ubfe(r.hdr.y, L.sh_hi[0], L.wh) << 4);
+    const uint32_t sc2 = __builtin_amdgcn_ubfe(a_sc, L.sh_sc[1], L.wl) | (__builtin_amdgcn_ubfe(r.hdr.y, L.sh_hi[1], L.wh) << 4);
+    const uint32_t mn1 = __builtin_amdgcn_ubfe(a_mn, L.sh_mn[0], L.wl) | (__builtin_amdgcn_ubfe(r.hdr.z, L.sh_hi[0], L.wh) << 4);
+    const uint32_t mn2 = __builtin_amdgcn_ubfe(a_mn, L.sh_mn[1], L.wl) | (__builtin_amdgcn_ubfe(r.hdr.z, L.sh_hi[1], L.wh) << 4);
+    P.de = gather_row4(L.sel, d * (float)sc1);
+    P.dd = gather_row4(L.sel, d * (float)sc2);
+    P.me = gather_row4(L.sel, -(dmin * (float)mn1));
+    P.md = gather_row4(L.sel, -(dmin * (float)mn2));
+  }
+  // fused multiply-add == the canonical two-step form: d is an f16, sc has 6 bits and q 4, so the
+  // product is exact in fp32
+  static __device__ __forceinline__ void dequant(const Raw& r, const Prep& P, const Lane&, int i, uint32_t (&au)[4]) {
+    const int c = i >> 1;
+    const float ds = (i & 1) ? P.dd[c] : P.de[c], nm = (i & 1) ? P.md[c] : P.me[c];
+    const uint32_t q0 = ((i & 1) ? (r.q[c].x >> 4) : r.q[c].x) & 0x0F0F0F0Fu;
+    const uint32_t q1 = ((i & 1) ? (r.q[c].y >> 4) : r.q[c].y) & 0x0F0F0F0Fu;
+    fma_bytes_to_bf16(q0, q1, ds, nm, au);
+  }
+};
+
+// Q6_K super-block: ql[128] qh[64] scales[16] d; weight 128h + 32j + l (l < 32) is
+// (nibble j/2 of ql[64h + 32(j%2) + l]) | (bits 2j, 2j+1 of qh[32h + l]) << 4, minus 32, times
+// d * scales[8h + 2j + l/16].  Step i = 4h + j, l = 8kg .. 8kg+7.
+struct SkQ6K {
+  static constexpr uint32_t kBlockBytes = 210;
+  struct Raw { uint2 qa[2], qb[2], qh[2]; uint4 sc; uint32_t d; };
+  struct Prep { float ds[8], off[8]; };
+  struct Lane {
+    uint32_t kg8, sbit;
+    __device__ __forceinline__ void init(int, int kg) {
+      kg8 = 8u * kg;
+      sbit = 8u * (uint32_t)(kg >> 1);      // scale byte l/16 inside each pair of scale bytes
+    }
+  };
+  static __device__ __forceinline__ void fetch(Raw& r, const uint8_t* p, const Lane& L) {
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      r.qa[h] = load8_a2(p + 64 * h + L.kg8);
+      r.qb[h] = load8_a2(p + 64 * h + 32 + L.kg8);
+      r.qh[h] = load8_a2(p + 128 + 32 * h + L.kg8);
+    }
+    r.sc = load16_a2(p + 192);
+    r.d = load2(p + 208);
+  }
+  static __device__ __forceinline__ void prepare(const Raw& r, const Lane& L, Prep& P) {
+    const float d = f16_bits_to_f32((uint16_t)r.d);
+    const uint32_t w[4] = {r.sc.x, r.sc.y, r.sc.z, r.sc.w};
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      // scale byte 8h + 2j + l/16 = dword 2h + j/2, byte 2(j%2) + l/16
+      const int h = i >> 2, j = i & 3;
+      const float sc = (float)(int)__builtin_amdgcn_sbfe((int)w[2 * h + (j >> 1)], 16u * (j & 1) + L.sbit, 8);
+      P.ds[i] = d * sc;
+      P.off[i] = -32.f * P.ds[i];
+    }
+  }
+  // (d * sc) * (q - 32) as one fused multiply-add on the unsigned q: the same exact product
+  static __device__ __forceinline__ void dequant(const Raw& r, const Prep& P, const Lane&, int i, uint32_t (&au)[4]) {
+    const int h = i >> 2, j = i & 3;
+    const uint2 ql = (j & 1) ? r.qb[h] : r.qa[h];
+    const uint32_t n0 = ((j >> 1) ? (ql.x >> 4) : ql.x) & 0x0F0F0F0Fu;
+    const uint32_t n1 = ((j >> 1) ? (ql.y >> 4) : ql.y) & 0x0F0F0F0Fu;
+    const uint32_t h0 = (r.qh[h].x >> (2 * j)) & 0x03030303u;
+    const uint32_t h1 = (r.qh[h].y >> (2 * j)) & 0x03030303u;
+    fma_bytes_to_bf16((h0 << 4) | n0, (h1 << 4) | n1, P.ds[i], P.off[i], au);
+  }
+};
+
+// Q8_0: eight blocks of {fp16 d, 32 int8} per 256 weights.  Step i is block i; the lane keeps bytes
+// 8kg .. 8kg+7 of each block and the scales of blocks 2kg, 2kg+1, exchanged like the Q4_K scales.
+struct SkQ8_0 {
+  static constexpr uint32_t kBlockBytes = 8 * 34;
+  struct Raw { uint2 q[8]; uint32_t d0, d1; };
+  struct Prep { f32x4_t de, dd; };
+  struct Lane {
+    float sel;
+    uint32_t kg8, dofs;
+    __device__ __forceinline__ void init(int li, int kg) {
+      sel = ((li & 3) == kg) ? 1.f : 0.f;
+      kg8 = 8u * kg;
+      dofs = 68u * kg;
+    }
+  };
+  static __device__ __forceinline__ void fetch(Raw& r, const uint8_t* p, const Lane& L) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) r.q[i] = load8_a2(p + 34 * i + 2 + L.kg8);
+    r.d0 = load2(p + L.dofs);
+    r.d1 = load2(p + L.dofs + 34);
+  }
+  static __device__ __forceinline__ void prepare(const Raw& r, const Lane& L, Prep& P) {
+    P.de = gather_row4(L.sel, f16_bits_to_f32((uint16_t)r.d0));
+    P.dd = gather_row4(L.sel, f16_bits_to_f32((uint16_t)r.d1));
+  }
+  // d * q as one fused multiply-add on u = q + 128 (the sign bit flipped): d * u - 128 d
+  static __device__ __forceinline__ void dequant(const Raw& r, const Prep& P, const Lane&, int i, uint32_t (&au)[4]) {
+    const float d = (i & 1) ? P.dd[i >> 1] : P.de[i >> 1];
+    fma_bytes_to_bf16(r.q[i].x ^ 0x80808080u, r.q[i].y ^ 0x80808080u, d, -128.f * d, au);
+  }
+};
 
 // RB: blocks of 16 weight rows per workgroup; TB: blocks of 16 tokens (m <= 16 * TB); WD: ring of
 // (super-block, row block) items of packed weights per wavefront, WD - 1 of them in flight; XB:
 // buffers for a super-block's activations (2: the next super-block's are requested while this one
 // is multiplied).
-template <int RB, int TB, int WD, int XB>
+template <class WF, int RB, int TB, int WD, int XB>
 __global__ void __launch_bounds__(kSkThreads)
-gemm_q4k_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, void* __restrict__ yv,
+gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, void* __restrict__ yv,
                        int y_dtype, const void* __restrict__ bias, int bias_dtype, int m, int n_out, int n_in) {
   static_assert((WD == 2 || WD == 4) && (2 * RB) % WD == 0 && (XB == 1 || XB == 2), "ring sizes");
   extern __shared__ float smem[];
@@ -59,7 +233,7 @@ gemm_q4k_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   // byte offset of (row, super-block 0) and element offset of (token, k = 8*kg)
   uint32_t wofs[RB], xofs[TB];
 #pragma unroll
-  for (int rb = 0; rb < RB; rb++) wofs[rb] = (uint32_t)min(n0 + 16 * rb + li, n_out - 1) * (uint32_t)(nsb * 144);
+  for (int rb = 0; rb < RB; rb++) wofs[rb] = (uint32_t)min(n0 + 16 * rb + li, n_out - 1) * ((uint32_t)nsb * WF::kBlockBytes);
 #pragma unroll
   for (int tb = 0; tb < TB; tb++) xofs[tb] = (uint32_t)min(16 * tb + li, m - 1) * (uint32_t)n_in + 8u * kg;
 
@@ -69,27 +243,10 @@ gemm_q4k_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
 #pragma unroll
     for (int tb = 0; tb < TB; tb++) acc[rb][tb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  // selector of the all-gather: as the A operand of the 16x16x4 MFMA (row i = lane % 16, k = lane / 16)
-  const float gather_sel = ((li & 3) == kg) ? 1.f : 0.f;
-  // Bit positions of the 6-bit scale and min of sub-blocks 2kg and 2kg+1 in the 12 packed bytes:
-  // sub-blocks 0..3 have the field whole in bytes 0..7, sub-blocks 4..7 four bits in bytes 8..11 and
-  // two on top of bytes 0..7.  Two bit-field extracts each, the second of width 0 in the simple case.
-  const bool upper = kg >= 2;
-  const uint32_t wl = upper ? 4u : 6u, wh = upper ? 2u : 0u;
-  uint32_t sh_sc[2], sh_mn[2], sh_hi[2];
-#pragma unroll
-  for (int h = 0; h < 2; h++) {
-    const uint32_t jj = (2u * kg + h) & 3u;
-    sh_sc[h] = 8u * jj;
-    sh_mn[h] = upper ? 8u * jj + 4u : 8u * jj;
-    sh_hi[h] = 8u * jj + 6u;
-  }
-
-  auto fetch = [&](SkRaw& r, int sb, int rb) {
-    const uint8_t* p = w + wofs[rb] + (uint32_t)sb * 144u;
-    r.hdr = load16_a16(p);
-#pragma unroll
-    for (int c = 0; c < 4; c++) r.q[c] = *reinterpret_cast<const uint2*>(p + 16 + 32 * c + 8 * kg);
+  typename WF::Lane L;
+  L.init(li, kg);
+  auto fetch = [&](typename WF::Raw& r, int sb, int rb) {
+    WF::fetch(r, w + wofs[rb] + (uint32_t)sb * WF::kBlockBytes, L);
   };
   // a super-block's activations: piece i is k = 32*i + 8*kg .. +7 of the lane's token
   auto load_x = [&](uint4 (&xf)[TB][8], int sb) {
@@ -100,7 +257,7 @@ gemm_q4k_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
         xf[tb][i] = *reinterpret_cast<const uint4*>(x + xofs[tb] + 256u * (uint32_t)sb + 32u * i);
   };
 
-  SkRaw raw[WD];
+  typename WF::Raw raw[WD];
   uint4 xfr[XB][TB][8];
 
   // The wavefront's items in order: (super-block, row block), row blocks innermost.  Item rb of a
@@ -122,39 +279,13 @@ gemm_q4k_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
         if (kMaxOff > 1 || off > 0) sb_a = sb_a < nsb ? sb_a : sb;
         fetch(raw[(XI * RB + rb + kAhead) % WD], sb_a, (rb + kAhead) % RB);
       }
-      const SkRaw& r = raw[(XI * RB + rb) % WD];
-      // this lane: sub-blocks 2kg and 2kg+1 of its row; then all eight from the row's four lanes
-      const float d = f16_bits_to_f32((uint16_t)(r.hdr.x & 0xFFFF));
-      const float dmin = f16_bits_to_f32((uint16_t)(r.hdr.x >> 16));
-      const uint32_t a_sc = upper ? r.hdr.w : r.hdr.y;   // bytes 8-11 or 0-3
-      const uint32_t a_mn = upper ? r.hdr.w : r.hdr.z;   // bytes 8-11 or 4-7
-      const uint32_t sc1 = __builtin_amdgcn_ubfe(a_sc, sh_sc[0], wl) | (__builtin_amdgcn_ubfe(r.hdr.y, sh_hi[0], wh) << 4);
-      const uint32_t sc2 = __builtin_amdgcn_ubfe(a_sc, sh_sc[1], wl) | (__builtin_amdgcn_ubfe(r.hdr.y, sh_hi[1], wh) << 4);
-      const uint32_t mn1 = __builtin_amdgcn_ubfe(a_mn, sh_mn[0], wl) | (__builtin_amdgcn_ubfe(r.hdr.z, sh_hi[0], wh) << 4);
-      const uint32_t mn2 = __builtin_amdgcn_ubfe(a_mn, sh_mn[1], wl) | (__builtin_amdgcn_ubfe(r.hdr.z, sh_hi[1], wh) << 4);
-      const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
-      const f32x4_t de = __builtin_amdgcn_mfma_f32_16x16x4f32(gather_sel, d * (float)sc1, zero, 0, 0, 0);
-      const f32x4_t dd = __builtin_amdgcn_mfma_f32_16x16x4f32(gather_sel, d * (float)sc2, zero, 0, 0, 0);
-      const f32x4_t me = __builtin_amdgcn_mfma_f32_16x16x4f32(gather_sel, -(dmin * (float)mn1), zero, 0, 0, 0);
-      const f32x4_t md = __builtin_amdgcn_mfma_f32_16x16x4f32(gather_sel, -(dmin * (float)mn2), zero, 0, 0, 0);
+      const typename WF::Raw& r = raw[(XI * RB + rb) % WD];
+      typename WF::Prep P;
+      WF::prepare(r, L, P);
 #pragma unroll
       for (int i = 0; i < 8; i++) {
-        const int c = i >> 1;
-        const float ds = (i & 1) ? dd[c] : de[c], nm = (i & 1) ? md[c] : me[c];
-        uint32_t q0 = ((i & 1) ? (r.q[c].x >> 4) : r.q[c].x) & 0x0F0F0F0Fu;
-        uint32_t q1 = ((i & 1) ? (r.q[c].y >> 4) : r.q[c].y) & 0x0F0F0F0Fu;
-        // keep the masked words opaque: byte k of them converts with one v_cvt_f32_ubyte<k>
-        asm volatile("" : "+v"(q0), "+v"(q1));
-        float f[8];
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-          // fused multiply-add == the canonical two-step form: d is an f16, sc has 6 bits and q 4,
-          // so the product is exact in fp32
-          f[k] = fmaf_(ds, (float)((q0 >> (8 * k)) & 0xFFu), nm);
-          f[4 + k] = fmaf_(ds, (float)((q1 >> (8 * k)) & 0xFFu), nm);
-        }
-        const uint32_t au[4] = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]),
-                                pack_bf16x2(f[4], f[5]), pack_bf16x2(f[6], f[7])};
+        uint32_t au[4];
+        WF::dequant(r, P, L, i, au);
         bf16x8_t a;
         __builtin_memcpy(&a, au, 16);
 #pragma unroll
@@ -223,10 +354,10 @@ gemm_q4k_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   }
 }
 
-template <int RB, int TB, int WD, int XB>
+template <class WF, int RB, int TB, int WD, int XB>
 hipError_t launch_skinny_tb(const uint8_t* w, const uint16_t* x, void* y, int y_dtype, const void* bias,
                             int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
-  auto kernel = gemm_q4k_skinny_kernel<RB, TB, WD, XB>;
+  auto kernel = gemm_skinny_kernel<WF, RB, TB, WD, XB>;
   const size_t lds = (size_t)(kSkWaves * RB * TB * 4 * 64 + 16 * TB * (16 * RB + 1)) * sizeof(float);
   static LargeLds configured;
   if (lds > 64 * 1024) {
@@ -238,64 +369,81 @@ hipError_t launch_skinny_tb(const uint8_t* w, const uint16_t* x, void* y, int y_
   return hipGetLastError();
 }
 
-}  // namespace
-
-bool gemm_skinny_supported(int format, int64_t m, int64_t n_out, int64_t n_in) {
-  static const int disabled = [] { const char* e = getenv("TTQ_GEMM_NO_SKINNY"); return e ? atoi(e) : 0; }();
-  // weight byte offsets and activation element offsets are 32-bit in the kernel; outputs are stored
-  // eight at a time
-  return !disabled && format == kQ4_K && m >= 1 && m <= 64 && n_out > 0 && n_out % 8 == 0 && n_in > 0 &&
-         n_in % 256 == 0 && n_out * (n_in / 256) * 144 < ((int64_t)1 << 32) && m * n_in < ((int64_t)1 << 31);
-}
-
-// Cost model (microseconds), fitted to 4096 x 4096, 4096 x 14336 and 14336 x 4096: rounds of workgroups
-// over the CUs x (fixed + super-blocks per wavefront x (activation loads + row blocks x weights)).
-// The activations of a super-block are re-read from L2 by every workgroup, which is what makes
-// more rows per workgroup cheaper per row, as long as every CU still gets a workgroup.
-static float skinny_cost_us(int rb, int64_t m, int64_t n_out, int64_t n_in) {
+// Cost model (microseconds), fitted to 4096 x 4096, 4096 x 14336 and 14336 x 4096 with Q4_K weights:
+// rounds of workgroups over the CUs x (fixed + super-blocks per wavefront x (activation loads + row
+// blocks x weights)).  The activations of a super-block are re-read from L2 by every workgroup,
+// which is what makes more rows per workgroup cheaper per row, as long as every CU still gets a
+// workgroup.  The weight term is scaled for the other formats' dequantization.
+float skinny_cost_us(int format, int rb, int64_t m, int64_t n_out, int64_t n_in) {
   static const float kX[4] = {1.46f, 2.73f, 4.9f, 6.25f}, kW[4] = {1.13f, 1.14f, 1.28f, 1.6f};
   static const float kF0[4] = {4.5f, 7.8f, 4.2f, 4.7f}, kF1[4] = {1.0f, 0.6f, 0.f, 0.f};
+  const float wf = format == kQ6_K ? kSkQ6KWeightFactor : (format == kQ8_0 ? kSkQ8WeightFactor : 1.f);
   const int t = (int)((m + 15) / 16) - 1;
   const int64_t wgs = (n_out + 16 * rb - 1) / (16 * rb), cus = device_num_cus();
   const int64_t iters = ((n_in >> 8) + kSkWaves - 1) / kSkWaves;
-  return (float)((wgs + cus - 1) / cus) * (kF0[t] + kF1[t] * rb + (float)iters * (kX[t] + rb * kW[t]));
+  return (float)((wgs + cus - 1) / cus) * (kF0[t] + kF1[t] * rb + (float)iters * (kX[t] + rb * wf * kW[t]));
 }
 
-static int skinny_choose_rb(int64_t m, int64_t n_out, int64_t n_in, float* cost_us = nullptr) {
+int skinny_choose_rb(int format, int64_t m, int64_t n_out, int64_t n_in, float* cost_us = nullptr) {
   static const int forced_rb = [] { const char* e = getenv("TTQ_SK_RB"); return e ? atoi(e) : 0; }();
   int best = 4;
   float best_cost = 1e30f;
   for (int rb = 4; rb >= 1; rb >>= 1) {
     if (forced_rb > 0 && rb != forced_rb) continue;
-    const float c = skinny_cost_us(rb, m, n_out, n_in);
+    const float c = skinny_cost_us(format, rb, m, n_out, n_in);
     if (c < best_cost) { best_cost = c; best = rb; }
   }
   if (cost_us) *cost_us = best_cost;
   return best;
 }
 
-float gemm_skinny_estimate_us(int64_t m, int64_t n_out, int64_t n_in) {
-  float c = 0.f;
-  skinny_choose_rb(m, n_out, n_in, &c);
-  return c;
-}
-
-hipError_t launch_gemm_skinny(const void* w, const uint16_t* x_bf16, void* y, int y_dtype, const void* bias,
-                              int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
-  if (m == 0 || n_out == 0) return hipSuccess;
-  if (y_dtype != kBF16 && y_dtype != kF32) return hipErrorInvalidValue;
-  const uint8_t* wb = static_cast<const uint8_t*>(w);
-  // Registers decide how far ahead a wavefront can request: 64 per token block for the activations.
-  const int rb = skinny_choose_rb(m, n_out, n_in);
+// Registers decide how far ahead a wavefront can request: 64 per token block for the activations.
+template <class WF>
+hipError_t launch_skinny_fmt(int format, const uint8_t* wb, const uint16_t* x_bf16, void* y, int y_dtype,
+                             const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                             hipStream_t s) {
+  const int rb = skinny_choose_rb(format, m, n_out, n_in);
   const int tb = (int)((m + 15) / 16);
 #define TTQ_SK_CASE(RBv, TBv, WDv, XBv) \
   if (rb == RBv && tb == TBv)            \
-    return launch_skinny_tb<RBv, TBv, WDv, XBv>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    return launch_skinny_tb<WF, RBv, TBv, WDv, XBv>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   TTQ_SK_CASE(4, 1, 4, 2) TTQ_SK_CASE(4, 2, 4, 2) TTQ_SK_CASE(4, 3, 2, 1) TTQ_SK_CASE(4, 4, 2, 1)
   TTQ_SK_CASE(2, 1, 4, 2) TTQ_SK_CASE(2, 2, 4, 2) TTQ_SK_CASE(2, 3, 2, 1) TTQ_SK_CASE(2, 4, 2, 1)
   TTQ_SK_CASE(1, 1, 2, 2) TTQ_SK_CASE(1, 2, 2, 2) TTQ_SK_CASE(1, 3, 2, 1) TTQ_SK_CASE(1, 4, 2, 1)
 #undef TTQ_SK_CASE
   return hipErrorInvalidValue;
+}
+
+}  // namespace
+
+bool gemm_skinny_supported(int format, int64_t m, int64_t n_out, int64_t n_in) {
+  static const int disabled = [] { const char* e = getenv("TTQ_GEMM_NO_SKINNY"); return e ? atoi(e) : 0; }();
+  const int64_t block_bytes = format == kQ4_K ? 144 : (format == kQ6_K ? 210 : 272);
+  // weight byte offsets and activation element offsets are 32-bit in the kernel; outputs are stored
+  // eight at a time
+  return !disabled && (format == kQ4_K || format == kQ6_K || format == kQ8_0) && m >= 1 && m <= 64 && n_out > 0 &&
+         n_out % 8 == 0 && n_in > 0 && n_in % 256 == 0 && n_out * (n_in / 256) * block_bytes < ((int64_t)1 << 32) &&
+         m * n_in < ((int64_t)1 << 31);
+}
+
+float gemm_skinny_estimate_us(int format, int64_t m, int64_t n_out, int64_t n_in) {
+  float c = 0.f;
+  skinny_choose_rb(format, m, n_out, n_in, &c);
+  return c;
+}
+
+hipError_t launch_gemm_skinny(int format, const void* w, const uint16_t* x_bf16, void* y, int y_dtype,
+                              const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                              hipStream_t s) {
+  if (m == 0 || n_out == 0) return hipSuccess;
+  if (y_dtype != kBF16 && y_dtype != kF32) return hipErrorInvalidValue;
+  const uint8_t* wb = static_cast<const uint8_t*>(w);
+  switch (format) {
+    case kQ4_K: return launch_skinny_fmt<SkQ4K>(format, wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kQ6_K: return launch_skinny_fmt<SkQ6K>(format, wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kQ8_0: return launch_skinny_fmt<SkQ8_0>(format, wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    default: return hipErrorInvalidValue;
+  }
 }
 
 }  // namespace ttq

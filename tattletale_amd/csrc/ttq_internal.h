@@ -70,10 +70,6 @@ hipError_t launch_rmsnorm(const void* x, const void* residual, const void* gamma
 // out (m, h) = silu(in[:, :h]) * in[:, h:], in (m, 2h), same dtype (ttq_activations.hip).
 hipError_t launch_silu_and_mul(const void* in, void* out, int dtype, int64_t m, int64_t h, hipStream_t s);
 
-hipError_t launch_gemm_q4k(const void* w, const uint16_t* x_bf16, void* y, int y_dtype,
-                           const void* bias, int bias_dtype, int64_t m, int64_t n_out,
-                           int64_t n_in, hipStream_t s);
-
 // Q4_K decode GEMV for a few activation rows at once (ttq_gemv_q4k_batch.hip): the weights are
 // read and unpacked once per 8 or 16 rows.
 bool gemv_q4k_batch_supported(int format, int x_dtype, int64_t m, int64_t n_out, int64_t n_in);
@@ -101,12 +97,20 @@ int device_num_cus();
 struct LargeLds { std::atomic<uint64_t> done{0}; };
 hipError_t allow_large_lds(const void* kernel, LargeLds& state);
 
-// Q4_K linear layer for up to 64 rows of bf16 activations, weights dequantized in registers
-// (ttq_gemm_skinny.hip).
+// Q4_K / Q6_K / Q8_0 linear layer for up to 64 rows of bf16 activations, weights dequantized in
+// registers (ttq_gemm_skinny.hip).
 bool gemm_skinny_supported(int format, int64_t m, int64_t n_out, int64_t n_in);
-float gemm_skinny_estimate_us(int64_t m, int64_t n_out, int64_t n_in);
-hipError_t launch_gemm_skinny(const void* w, const uint16_t* x_bf16, void* y, int y_dtype, const void* bias,
-                              int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s);
+float gemm_skinny_estimate_us(int format, int64_t m, int64_t n_out, int64_t n_in);
+hipError_t launch_gemm_skinny(int format, const void* w, const uint16_t* x_bf16, void* y, int y_dtype,
+                              const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                              hipStream_t s);
+
+// The multi-row operator for block formats and bf16 activations: the few-row kernel or the tiled
+// GEMM, whichever is estimated to be faster for the shape (ttq_gemm_q4k.hip).
+bool gemm_supported(int format, int64_t m, int64_t n_out, int64_t n_in);
+float gemm_estimate_us(int format, int64_t m, int64_t n_out, int64_t n_in);
+hipError_t launch_gemm(int format, const void* w, const uint16_t* x_bf16, void* y, int y_dtype, const void* bias,
+                       int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s);
 
 // Producer/consumer GEMM for Q4_K / Q6_K / Q8_0 weights and bf16 activations (ttq_gemm_pc.hip).
 bool gemm_pc_supported(int format, int64_t m, int64_t n_out, int64_t n_in, int bn);

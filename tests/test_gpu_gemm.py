@@ -17,6 +17,7 @@ from util import DEV, bits_to_dev, dev_bits, packed_to_dev, rel_l2, x_to_dev, ra
 
 pytestmark = pytest.mark.gpu
 TOL = 2e-2
+BLOCK_WEIGHTS = {F.Q8_0: 32, F.Q4_K: 256, F.Q6_K: 256}      # weights per packed block
 
 
 @pytest.mark.parametrize("m,n_out,n_in", [(64, 256, 1024), (128, 128, 256), (16, 384, 512), (100, 200, 768),
@@ -55,15 +56,16 @@ def test_gemm_identity_activations_give_bf16_weights_exactly(n_in):
 # 16, 32 or 64 weight rows per workgroup: n_out <= 4096 gives 16, 6144 gives 32, 12288 and up 64 on
 # a 256-CU device.  Token blocks of 16: m = 1..16, 17..32, 33..48, 49..64.  n_out not a multiple of
 # the workgroup's rows, super-block counts below / not a multiple of the 8 wavefronts.
+@pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
 @pytest.mark.parametrize("m,n_out,n_in", [(1, 64, 256), (7, 200, 768), (16, 4096, 2304), (17, 1048, 256),
                                           (32, 6152, 512), (33, 6144, 256), (48, 12296, 512), (49, 136, 4352),
                                           (64, 12288, 256), (64, 16384, 256), (5, 12288, 256)])
-def test_gemm_few_rows(m, n_out, n_in):
-    p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=500 + m)
-    what = oracle.dequant(F.Q4_K, p, n_out, n_in)
+def test_gemm_few_rows(fmt, m, n_out, n_in):
+    p = random_blocks(fmt, n_out * (n_in // BLOCK_WEIGHTS[fmt]), seed=500 + m)
+    what = oracle.dequant(fmt, p, n_out, n_in)
     what_r = oracle.bf16_to_f32(oracle.f32_to_bf16(what))
     xd, xf = x_to_dev(Q.fill_normal(501 + m, 1, 1.0, m * n_in).reshape(m, n_in), "bf16")
-    y = QL.gemm_q4_k(packed_to_dev(p), xd, n_out, n_in)
+    y = QL.gemm(fmt, packed_to_dev(p), xd, n_out, n_in)
     assert y.shape == (m, n_out) and y.dtype == torch.bfloat16
     got = oracle.bf16_to_f32(dev_bits(y))
     assert rel_l2(got, oracle.linear_f64(what, xf)) <= TOL
@@ -74,29 +76,31 @@ def test_gemm_few_rows(m, n_out, n_in):
         assert rel_l2(got[i], want_r[i]) <= 6e-3, i
 
 
+@pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
 @pytest.mark.parametrize("m,n_out", [(64, 192), (40, 6144), (16, 12304)])
-def test_gemm_few_rows_unit_vectors_give_bf16_weights_exactly(m, n_out):
+def test_gemm_few_rows_unit_vectors_give_bf16_weights_exactly(fmt, m, n_out):
     n_in = 2560                                      # ten super-blocks: wavefronts 0 and 1 take two each
-    p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=23)
-    what = oracle.dequant(F.Q4_K, p, n_out, n_in)
+    p = random_blocks(fmt, n_out * (n_in // BLOCK_WEIGHTS[fmt]), seed=23)
+    what = oracle.dequant(fmt, p, n_out, n_in)
     ks = (np.arange(m) * 397 + 5) % n_in             # distinct k over all super-blocks and sub-blocks
     assert np.unique(ks).size == m
     x = np.zeros((m, n_in), np.float32)
     x[np.arange(m), ks] = 1.0
     xd, _ = x_to_dev(x, "bf16")
-    y = dev_bits(QL.gemm_q4_k(packed_to_dev(p), xd, n_out, n_in))
+    y = dev_bits(QL.gemm(fmt, packed_to_dev(p), xd, n_out, n_in))
     want = oracle.f32_to_bf16(what)[:, ks].T
     # up to the sign of a zero: the other 2559 products of the sum are +0
     assert np.array_equal(y + (y == 0x8000) * np.uint16(0x8000), want + (want == 0x8000) * np.uint16(0x8000))
 
 
-def test_forward_few_rows_f32_output_with_bias():
+@pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
+def test_forward_few_rows_f32_output_with_bias(fmt):
     n_out, n_in, m = 4096, 1024, 24
-    p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=29)
-    what = oracle.dequant(F.Q4_K, p, n_out, n_in)
+    p = random_blocks(fmt, n_out * (n_in // BLOCK_WEIGHTS[fmt]), seed=29)
+    what = oracle.dequant(fmt, p, n_out, n_in)
     bd, bf = x_to_dev(Q.fill_normal(31, 2, 0.5, n_out), "f32")
     xd, xf = x_to_dev(Q.fill_normal(32, 1, 1.0, m * n_in).reshape(2, 12, n_in), "bf16")
-    layer = QuantLinear.init(packed_to_dev(p), F.Q4_K, n_in, n_out, bias=bd)
+    layer = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out, bias=bd)
     want = oracle.linear_f64(what, xf.reshape(m, n_in), bf).reshape(2, 12, n_out)
     y32 = layer.forward(xd, out_dtype=torch.float32)
     assert y32.dtype == torch.float32 and rel_l2(y32.cpu().numpy(), want) <= 4e-3

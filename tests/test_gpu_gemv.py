@@ -85,14 +85,21 @@ def test_quantlinear_forward_shapes_bias_and_dtypes(fmt):
     n_out, n_in = 200, 1024
     p, what = make(fmt, n_out, n_in, 90)
     bias = Q.fill_normal(91, 2, 0.5, n_out)
-    x = Q.fill_normal(92, 1, 1.0, 2 * 3 * n_in).reshape(2, 3, n_in)
+    # up to four rows always run the decode kernels (fp32 scales: the 1e-3 class)
+    x = Q.fill_normal(92, 1, 1.0, 2 * 2 * n_in).reshape(2, 2, n_in)
     xd, xf = x_to_dev(x, "bf16")
     bd, bf = x_to_dev(bias, "bf16")
     layer = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out, bias=bd)
-    want = oracle.linear_f64(what, xf.reshape(6, n_in), bf).reshape(2, 3, n_out)
+    want = oracle.linear_f64(what, xf.reshape(4, n_in), bf).reshape(2, 2, n_out)
     y32 = layer.forward(xd, out_dtype=torch.float32)
-    assert y32.shape == (2, 3, n_out) and y32.dtype == torch.float32
+    assert y32.shape == (2, 2, n_out) and y32.dtype == torch.float32
     assert rel_l2(y32.cpu().numpy(), want) <= TOL
+    # five or more rows of bf16 activations may take the bf16 matrix-core kernels (weights rounded to
+    # bf16: the 2e-2 class), whichever the cost estimate prefers for the shape
+    x6d, x6f = x_to_dev(Q.fill_normal(93, 1, 1.0, 2 * 3 * n_in).reshape(2, 3, n_in), "bf16")
+    y6 = layer.forward(x6d, out_dtype=torch.float32)
+    assert y6.shape == (2, 3, n_out) and y6.dtype == torch.float32
+    assert rel_l2(y6.cpu().numpy(), oracle.linear_f64(what, x6f.reshape(6, n_in), bf).reshape(2, 3, n_out)) <= 2e-2
     y16 = layer.forward(xd)                                                   # dtype follows x
     assert y16.dtype == torch.bfloat16
     assert rel_l2(oracle.bf16_to_f32(dev_bits(y16)), want) <= 1e-2            # bf16 output rounding
