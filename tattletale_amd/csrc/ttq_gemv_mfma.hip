@@ -418,7 +418,8 @@ static hipError_t launch_xy(const void* w, const void* x, void* y, const void* b
                             int64_t m, int64_t n_out, int64_t n_in, const GemvNormArgs& na, hipStream_t s) {
   constexpr int W = kMfmaWaves;
   const int nsb = (int)(n_in / 256);
-  int num_wg = mfma_num_cus();
+  static const int forced_wgs = mfma_env_int("TTQ_GEMV_MFMA_WGS", 0);
+  int num_wg = forced_wgs > 0 ? forced_wgs : device_num_cus();
   const int64_t groups = (n_out + 15) / 16;
   if (num_wg > groups) num_wg = (int)groups;
   const int rows_per_wg = (int)((n_out + num_wg - 1) / num_wg);

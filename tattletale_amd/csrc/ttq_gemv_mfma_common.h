@@ -70,19 +70,6 @@ __device__ __forceinline__ uint32_t pack_low_bytes(int a, int b, int c, int d) {
   return p01 | (p23 << 16);
 }
 
-inline int mfma_num_cus() {
-  static int cached = 0;
-  if (cached == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-      cached = prop.multiProcessorCount;
-    else
-      cached = 256;
-  }
-  return cached;
-}
-
 inline int mfma_env_int(const char* name, int dflt) {
   const char* e = getenv(name);
   return e ? atoi(e) : dflt;

@@ -239,7 +239,7 @@ static hipError_t q8_launch_xy(const void* w, const void* x, void* y, const void
                                int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
   constexpr int W = kMfmaWaves;
   const int nst = (int)(n_in / 128);
-  int num_wg = mfma_num_cus();
+  int num_wg = device_num_cus();
   const int64_t groups = (n_out + 15) / 16;
   if (num_wg > groups) num_wg = (int)groups;
   const int rows_per_wg = (int)((n_out + num_wg - 1) / num_wg);
