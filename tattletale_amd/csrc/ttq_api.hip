@@ -7,6 +7,8 @@
 #include "../../include/ttq.h"
 #include "ttq_internal.h"
 
+#include <stdlib.h>
+
 namespace ttq {
 
 int device_num_cus() {
@@ -310,10 +312,12 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
   const bool gemm_ok = x_dtype == TTQ_BF16 && (y_dtype == TTQ_BF16 || y_dtype == TTQ_F32) &&
                        (layer->format == TTQ_Q4_K || layer->format == TTQ_Q6_K || layer->format == TTQ_Q8_0) &&
                        ttq::gemm_supported(layer->format, m, n_out, n_in);
-  if (gemm_ok && m >= 5) {
+  // TTQ_FORWARD_ROUTE (for A/B measurements): 1 = always the decode kernels, 2 = the GEMM whenever it exists
+  static const int route = [] { const char* e = getenv("TTQ_FORWARD_ROUTE"); return e ? atoi(e) : 0; }();
+  if (gemm_ok && m >= 5 && route != 1) {
     const bool gemv_ok = check_gemv_limits(x_dtype, n_in) == TTQ_OK;
-    if (!gemv_ok || ttq::gemm_estimate_us(layer->format, m, n_out, n_in) <
-                        ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in))
+    if (!gemv_ok || route == 2 ||
+        ttq::gemm_estimate_us(layer->format, m, n_out, n_in) < ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in))
       return hip_status(ttq::launch_gemm(layer->format, layer->qweight, static_cast<const uint16_t*>(x), y, y_dtype,
                                          layer->bias, layer->bias_dtype, m, n_out, n_in, s));
   }

@@ -111,13 +111,19 @@ def test_forward_few_rows_bias_and_output_types(m):
     bd, bf = x_to_dev(bias, "f32")
     layer = QuantLinear.init(packed_to_dev(p), F.Q4_K, n_in, n_out, bias=bd)
     want = oracle.linear_f64(what, xf, bf)
+    # From five rows of bf16 activations on the operator takes whichever of the few-row decode
+    # kernels (fp32 scales, 1e-3 class) and the bf16 matrix-core kernels (weights rounded to bf16
+    # once: about 1.3e-3 with fp32 output) its cost estimate prefers for the shape.
     y32 = layer.forward(xd, out_dtype=torch.float32)
-    assert rel_l2(y32.cpu().numpy(), want) <= TOL          # decode-class accuracy: not the bf16-weight GEMM
+    assert rel_l2(y32.cpu().numpy(), want) <= 4e-3
     y16 = layer.forward(xd)
     assert y16.dtype == torch.bfloat16
     assert np.array_equal(dev_bits(y16), oracle.f32_to_bf16(y32.cpu().numpy()))
     yh = layer.forward(xd, out_dtype=torch.float16)
-    assert rel_l2(yh.float().cpu().numpy(), want) <= 2e-3
+    assert rel_l2(yh.float().cpu().numpy(), want) <= 4e-3
+    # the decode entry point itself stays in the 1e-3 class whatever the row count
+    yg = QL.gemv(F.Q4_K, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()
+    assert rel_l2(yg, oracle.linear_f64(what, xf)) <= TOL
 
 
 @pytest.mark.parametrize("m", [4, 16])
