@@ -19,11 +19,11 @@
 //     (canonical arithmetic written as one exact fused multiply-add, one bf16 rounding).  Q4_K: the
 //     8 bytes 8*g .. 8*g+7 of each of the four 32-byte qs chunks, low nibbles for the even sub-block
 //     of the chunk, high nibbles for the odd one.  Q6_K: 8 bytes of each ql half-row and 8 of qh per
-//     128 weights.  Q8_0: 8 of the 32 bytes of each block;
+//     128 weights.  Q8_0: half a block (16 bytes) per pair of steps;
 //   * Q4_K: each lane decodes the scale and min of two sub-blocks (2g, 2g+1) of its row and the
 //     four lanes of a row exchange them through v_mfma_f32_16x16x4_f32 with a 0/1 selector as the
-//     other operand (D[4g'+r][row] = value of lane g = r: an exact all-gather).  Q8_0 does the same
-//     with the block scales (two per lane); Q6_K lanes read the row's 16 scale bytes themselves;
+//     other operand (D[4g'+r][row] = value of lane g = r: an exact all-gather).  Q6_K lanes read
+//     the row's 16 scale bytes themselves, Q8_0 lanes the scale of the block they hold;
 //   * the eight wavefronts' partial sums meet in LDS once, at the end; the sums are transposed
 //     through LDS so that every thread stores 8 consecutive outputs of one token.
 //
@@ -40,14 +40,22 @@ namespace {
 
 constexpr int kSkThreads = 512;
 constexpr int kSkWaves = kSkThreads / 64;
-// time per row block relative to Q4_K (cost model): more unpacking for Q6_K, eighteen small loads per
-// lane and super-block for Q8_0
-constexpr float kSkQ6KWeightFactor = 1.6f, kSkQ8WeightFactor = 3.5f;
+// time per row block relative to Q4_K (cost model)
+constexpr float kSkQ6KWeightFactor = 1.2f, kSkQ8WeightFactor = 2.2f;
 
 __device__ __forceinline__ uint2 load8_a2(const uint8_t* p) {
   uint2 v;
   __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 8);
   return v;
+}
+
+// Lane exchange: every lane receives `v` of lane `src_lane4 / 4`.
+__device__ __forceinline__ uint32_t pull_lane(uint32_t src_lane4, uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_ds_bpermute((int)src_lane4, (int)v);
+}
+__device__ __forceinline__ void pull_lane(uint32_t s4, uint2& v) { v.x = pull_lane(s4, v.x); v.y = pull_lane(s4, v.y); }
+__device__ __forceinline__ void pull_lane(uint32_t s4, uint4& v) {
+  v.x = pull_lane(s4, v.x); v.y = pull_lane(s4, v.y); v.z = pull_lane(s4, v.z); v.w = pull_lane(s4, v.w);
 }
 
 // D[4g'+r][row] = value of the row's lane g = r, for every g': the four lanes of a row exchange a
@@ -79,6 +87,8 @@ __device__ __forceinline__ void fma_bytes_to_bf16(uint32_t q0, uint32_t q1, floa
 // weights k = 32*i + 8*kg .. +7 of step i (dequant).
 struct SkQ4K {
   static constexpr uint32_t kBlockBytes = 144;
+  static __device__ __forceinline__ uint32_t x_lane_k(int kg) { return 8u * kg; }
+  static __device__ __forceinline__ constexpr uint32_t x_step_k(int i) { return 32u * i; }
   struct Raw { uint4 hdr; uint2 q[4]; };
   struct Prep { f32x4_t de, dd, me, md; };
   // Bit positions of the 6-bit scale and min of sub-blocks 2kg and 2kg+1 in the 12 packed bytes:
@@ -88,9 +98,9 @@ struct SkQ4K {
     float sel;
     bool upper;
     uint32_t kg8, wl, wh, sh_sc[2], sh_mn[2], sh_hi[2];
-    __device__ __forceinline__ void init(int li, int kg) {
+    __device__ __forceinline__ void init(int li, int kg, int load_kg) {
       sel = ((li & 3) == kg) ? 1.f : 0.f;
-      kg8 = 8u * kg;
+      kg8 = 8u * load_kg;
       upper = kg >= 2;
       wl = upper ? 4u : 6u;
       wh = upper ? 2u : 0u;
@@ -107,6 +117,11 @@ struct SkQ4K {
     r.hdr = load16_a16(p);
 #pragma unroll
     for (int c = 0; c < 4; c++) r.q[c] = *reinterpret_cast<const uint2*>(p + 16 + 32 * c + L.kg8);
+  }
+  static __device__ __forceinline__ void exchange(Raw& r, uint32_t s4) {
+    pull_lane(s4, r.hdr);
+#pragma unroll
+    for (int c = 0; c < 4; c++) pull_lane(s4, r.q[c]);
   }
   // this lane: sub-blocks 2kg and 2kg+1 of its row; then all eight from the row's four lanes
   static __device__ __forceinline__ void prepare(const Raw& r, const Lane& L, Prep& P) {
@@ -139,15 +154,23 @@ struct SkQ4K {
 // d * scales[8h + 2j + l/16].  Step i = 4h + j, l = 8kg .. 8kg+7.
 struct SkQ6K {
   static constexpr uint32_t kBlockBytes = 210;
+  static __device__ __forceinline__ uint32_t x_lane_k(int kg) { return 8u * kg; }
+  static __device__ __forceinline__ constexpr uint32_t x_step_k(int i) { return 32u * i; }
   struct Raw { uint2 qa[2], qb[2], qh[2]; uint4 sc; uint32_t d; };
   struct Prep { float ds[8], off[8]; };
   struct Lane {
     uint32_t kg8, sbit;
-    __device__ __forceinline__ void init(int, int kg) {
-      kg8 = 8u * kg;
+    __device__ __forceinline__ void init(int, int kg, int load_kg) {
+      kg8 = 8u * load_kg;
       sbit = 8u * (uint32_t)(kg >> 1);      // scale byte l/16 inside each pair of scale bytes
     }
   };
+  static __device__ __forceinline__ void exchange(Raw& r, uint32_t s4) {
+#pragma unroll
+    for (int h = 0; h < 2; h++) { pull_lane(s4, r.qa[h]); pull_lane(s4, r.qb[h]); pull_lane(s4, r.qh[h]); }
+    pull_lane(s4, r.sc);
+    r.d = pull_lane(s4, r.d);
+  }
   static __device__ __forceinline__ void fetch(Raw& r, const uint8_t* p, const Lane& L) {
 #pragma unroll
     for (int h = 0; h < 2; h++) {
@@ -182,35 +205,47 @@ struct SkQ6K {
   }
 };
 
-// Q8_0: eight blocks of {fp16 d, 32 int8} per 256 weights.  Step i is block i; the lane keeps bytes
-// 8kg .. 8kg+7 of each block and the scales of blocks 2kg, 2kg+1, exchanged like the Q4_K scales.
+// Q8_0: eight blocks of {fp16 d, 32 int8} per 256 weights.  Lane kg keeps half a block per pair of
+// steps -- bytes 16(kg%2) .. +15 of block 2p + kg/2 for steps 2p, 2p+1 -- and that block's scale, so
+// a pair costs one 16-byte and one 2-byte load.  Step 2p + s then multiplies
+// k = 32(2p + kg/2) + 16(kg%2) + 8s .. +7, and the activations are read at the same k.
 struct SkQ8_0 {
   static constexpr uint32_t kBlockBytes = 8 * 34;
-  struct Raw { uint2 q[8]; uint32_t d0, d1; };
-  struct Prep { f32x4_t de, dd; };
+  static __device__ __forceinline__ uint32_t x_lane_k(int kg) { return 32u * (kg >> 1) + 16u * (kg & 1); }
+  static __device__ __forceinline__ constexpr uint32_t x_step_k(int i) { return 64u * (i >> 1) + 8u * (i & 1); }
+  struct Raw { uint4 q[4]; uint32_t d[4]; };
+  struct Prep { float d[4], off[4]; };
   struct Lane {
-    float sel;
-    uint32_t kg8, dofs;
-    __device__ __forceinline__ void init(int li, int kg) {
-      sel = ((li & 3) == kg) ? 1.f : 0.f;
-      kg8 = 8u * kg;
-      dofs = 68u * kg;
+    uint32_t bofs;     // byte offset of the lane's block of pair 0
+    uint32_t qofs;     // of its 16 quant bytes in it
+    __device__ __forceinline__ void init(int, int, int load_kg) {
+      bofs = 34u * (uint32_t)(load_kg >> 1);
+      qofs = bofs + 2u + 16u * (uint32_t)(load_kg & 1);
     }
   };
+  static __device__ __forceinline__ void exchange(Raw& r, uint32_t s4) {
+#pragma unroll
+    for (int pr = 0; pr < 4; pr++) { pull_lane(s4, r.q[pr]); r.d[pr] = pull_lane(s4, r.d[pr]); }
+  }
   static __device__ __forceinline__ void fetch(Raw& r, const uint8_t* p, const Lane& L) {
 #pragma unroll
-    for (int i = 0; i < 8; i++) r.q[i] = load8_a2(p + 34 * i + 2 + L.kg8);
-    r.d0 = load2(p + L.dofs);
-    r.d1 = load2(p + L.dofs + 34);
+    for (int pr = 0; pr < 4; pr++) {
+      r.q[pr] = load16_a2(p + 68 * pr + L.qofs);
+      r.d[pr] = load2(p + 68 * pr + L.bofs);
+    }
   }
-  static __device__ __forceinline__ void prepare(const Raw& r, const Lane& L, Prep& P) {
-    P.de = gather_row4(L.sel, f16_bits_to_f32((uint16_t)r.d0));
-    P.dd = gather_row4(L.sel, f16_bits_to_f32((uint16_t)r.d1));
+  static __device__ __forceinline__ void prepare(const Raw& r, const Lane&, Prep& P) {
+#pragma unroll
+    for (int pr = 0; pr < 4; pr++) {
+      P.d[pr] = f16_bits_to_f32((uint16_t)r.d[pr]);
+      P.off[pr] = -128.f * P.d[pr];
+    }
   }
   // d * q as one fused multiply-add on u = q + 128 (the sign bit flipped): d * u - 128 d
   static __device__ __forceinline__ void dequant(const Raw& r, const Prep& P, const Lane&, int i, uint32_t (&au)[4]) {
-    const float d = (i & 1) ? P.dd[i >> 1] : P.de[i >> 1];
-    fma_bytes_to_bf16(r.q[i].x ^ 0x80808080u, r.q[i].y ^ 0x80808080u, d, -128.f * d, au);
+    const int pr = i >> 1;
+    const uint32_t q0 = (i & 1) ? r.q[pr].z : r.q[pr].x, q1 = (i & 1) ? r.q[pr].w : r.q[pr].y;
+    fma_bytes_to_bf16(q0 ^ 0x80808080u, q1 ^ 0x80808080u, P.d[pr], P.off[pr], au);
   }
 };
 
@@ -232,10 +267,18 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
 
   // byte offset of (row, super-block 0) and element offset of (token, k = 8*kg)
   uint32_t wofs[RB], xofs[TB];
+  // Weights and activations are requested with the four pieces of a row (token) in adjacent lanes
+  // (lane = 4 * row + piece: one 64-byte run per row and quad of lanes) and exchanged into the MFMA
+  // operand layout (lane = row + 16 * piece) when they are used: the memory pipeline merges the
+  // accesses of neighbouring lanes only.
+  const int load_row = lane >> 2, load_kg = lane & 3;
+  const uint32_t from_lane4 = 4u * (uint32_t)(4 * li + kg);
 #pragma unroll
-  for (int rb = 0; rb < RB; rb++) wofs[rb] = (uint32_t)min(n0 + 16 * rb + li, n_out - 1) * ((uint32_t)nsb * WF::kBlockBytes);
+  for (int rb = 0; rb < RB; rb++)
+    wofs[rb] = (uint32_t)min(n0 + 16 * rb + load_row, n_out - 1) * ((uint32_t)nsb * WF::kBlockBytes);
 #pragma unroll
-  for (int tb = 0; tb < TB; tb++) xofs[tb] = (uint32_t)min(16 * tb + li, m - 1) * (uint32_t)n_in + 8u * kg;
+  for (int tb = 0; tb < TB; tb++)
+    xofs[tb] = (uint32_t)min(16 * tb + load_row, m - 1) * (uint32_t)n_in + WF::x_lane_k(load_kg);
 
   f32x4_t acc[RB][TB];
 #pragma unroll
@@ -244,17 +287,19 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
     for (int tb = 0; tb < TB; tb++) acc[rb][tb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
   typename WF::Lane L;
-  L.init(li, kg);
+  L.init(li, kg, load_kg);
   auto fetch = [&](typename WF::Raw& r, int sb, int rb) {
     WF::fetch(r, w + wofs[rb] + (uint32_t)sb * WF::kBlockBytes, L);
   };
-  // a super-block's activations: piece i is k = 32*i + 8*kg .. +7 of the lane's token
+  // a super-block's activations: piece i is the lane's token at the eight k of step i (for Q4_K and
+  // Q6_K k = 32*i + 8*kg .. +7; any assignment of k to (step, kg) works as long as weights and
+  // activations agree, and Q8_0 uses one that makes its loads 16 bytes long)
   auto load_x = [&](uint4 (&xf)[TB][8], int sb) {
 #pragma unroll
     for (int tb = 0; tb < TB; tb++)
 #pragma unroll
       for (int i = 0; i < 8; i++)
-        xf[tb][i] = *reinterpret_cast<const uint4*>(x + xofs[tb] + 256u * (uint32_t)sb + 32u * i);
+        xf[tb][i] = *reinterpret_cast<const uint4*>(x + xofs[tb] + 256u * (uint32_t)sb + WF::x_step_k(i));
   };
 
   typename WF::Raw raw[WD];
@@ -269,7 +314,13 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
     constexpr int kAhead = WD - 1;
     const int sb_next = sb + kSkWaves < nsb ? sb + kSkWaves : sb;
     if (XB == 1) load_x(xfr[0], sb);
-    else load_x(xfr[XI ^ 1], sb_next);
+    // this super-block's activations into the operand layout (they were requested one super-block
+    // ago when there are two buffers)
+#pragma unroll
+    for (int tb = 0; tb < TB; tb++)
+#pragma unroll
+      for (int i = 0; i < 8; i++) pull_lane(from_lane4, xfr[XB == 1 ? 0 : XI][tb][i]);
+    if (XB == 2) load_x(xfr[XI ^ 1], sb_next);
 #pragma unroll
     for (int rb = 0; rb < RB; rb++) {
       {
@@ -279,7 +330,8 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
         if (kMaxOff > 1 || off > 0) sb_a = sb_a < nsb ? sb_a : sb;
         fetch(raw[(XI * RB + rb + kAhead) % WD], sb_a, (rb + kAhead) % RB);
       }
-      const typename WF::Raw& r = raw[(XI * RB + rb) % WD];
+      typename WF::Raw& r = raw[(XI * RB + rb) % WD];
+      WF::exchange(r, from_lane4);
       typename WF::Prep P;
       WF::prepare(r, L, P);
 #pragma unroll
@@ -354,12 +406,11 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
   }
 }
 
-template <class WF, int RB, int TB, int WD, int XB>
-hipError_t launch_skinny_tb(const uint8_t* w, const uint16_t* x, void* y, int y_dtype, const void* bias,
-                            int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
-  auto kernel = gemm_skinny_kernel<WF, RB, TB, WD, XB>;
+template <int RB, int TB, class K>
+hipError_t launch_skinny_k(K kernel, const uint8_t* w, const uint16_t* x, void* y, int y_dtype, const void* bias,
+                           int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
   const size_t lds = (size_t)(kSkWaves * RB * TB * 4 * 64 + 16 * TB * (16 * RB + 1)) * sizeof(float);
-  static LargeLds configured;
+  static LargeLds configured;          // one per kernel instantiation: K is part of this function's type
   if (lds > 64 * 1024) {
     const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), configured);
     if (e != hipSuccess) return e;
@@ -369,19 +420,29 @@ hipError_t launch_skinny_tb(const uint8_t* w, const uint16_t* x, void* y, int y_
   return hipGetLastError();
 }
 
-// Cost model (microseconds), fitted to 4096 x 4096, 4096 x 14336 and 14336 x 4096 with Q4_K weights:
-// rounds of workgroups over the CUs x (fixed + super-blocks per wavefront x (activation loads + row
-// blocks x weights)).  The activations of a super-block are re-read from L2 by every workgroup,
-// which is what makes more rows per workgroup cheaper per row, as long as every CU still gets a
-// workgroup.  The weight term is scaled for the other formats' dequantization.
+template <class WF, int RB, int TB, int WD, int XB>
+hipError_t launch_skinny_tb(const uint8_t* w, const uint16_t* x, void* y, int y_dtype, const void* bias,
+                            int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+  return launch_skinny_k<RB, TB>(gemm_skinny_kernel<WF, RB, TB, WD, XB>, w, x, y, y_dtype, bias, bias_dtype, m, n_out,
+                                 n_in, s);
+}
+
+// Cost model (microseconds), a least-squares fit to 4096 x 4096, 4096 x 14336 and 14336 x 4096 with
+// Q4_K weights, 16 and 64 weight rows per workgroup: rounds of workgroups over the CUs x (fixed +
+// super-blocks per wavefront x (activation loads + row blocks x weights)) + packed megabytes x
+// 0.2 (the stream itself, about 5 TB/s).  The activations of a super-block are re-read from L2 by
+// every workgroup, which is what makes more rows per workgroup cheaper per row, as long as every
+// CU still gets a workgroup.  The weight term is scaled for the other formats.
 float skinny_cost_us(int format, int rb, int64_t m, int64_t n_out, int64_t n_in) {
-  static const float kX[4] = {1.46f, 2.73f, 4.9f, 6.25f}, kW[4] = {1.13f, 1.14f, 1.28f, 1.6f};
-  static const float kF0[4] = {4.5f, 7.8f, 4.2f, 4.7f}, kF1[4] = {1.0f, 0.6f, 0.f, 0.f};
+  static const float kF0[4] = {1.95f, 2.78f, 2.11f, 2.51f}, kX[4] = {0.44f, 1.30f, 1.87f, 2.36f};
+  static const float kW[4] = {0.97f, 0.88f, 1.10f, 1.31f};
   const float wf = format == kQ6_K ? kSkQ6KWeightFactor : (format == kQ8_0 ? kSkQ8WeightFactor : 1.f);
+  const int64_t block_bytes = format == kQ4_K ? 144 : (format == kQ6_K ? 210 : 272);
+  const float mb = (float)(n_out * (n_in >> 8) * block_bytes) * 1e-6f;
   const int t = (int)((m + 15) / 16) - 1;
   const int64_t wgs = (n_out + 16 * rb - 1) / (16 * rb), cus = device_num_cus();
   const int64_t iters = ((n_in >> 8) + kSkWaves - 1) / kSkWaves;
-  return (float)((wgs + cus - 1) / cus) * (kF0[t] + kF1[t] * rb + (float)iters * (kX[t] + rb * wf * kW[t]));
+  return (float)((wgs + cus - 1) / cus) * (kF0[t] + (float)iters * (kX[t] + rb * wf * kW[t])) + 0.2f * mb;
 }
 
 int skinny_choose_rb(int format, int64_t m, int64_t n_out, int64_t n_in, float* cost_us = nullptr) {
