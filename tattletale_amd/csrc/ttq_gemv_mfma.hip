@@ -131,10 +131,16 @@ gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
   const int rounds = (rows_per_wg + per_round - 1) / per_round;
   const int t_total = rounds * S;
   const int last = wg_row_end - 1;   // rows past the workgroup's share re-read its last row
-  // weight row of lane n in row group `grp` of the workgroup
-  auto group_row = [&](int grp) {
-    if constexpr (FUSE) return min(wg_row0 + (grp >> 1) * 16 + n, last) + (grp & 1) * n_out;
-    else return min(wg_row0 + grp * 16 + n, last);
+  // Weights are requested with lane = 4 * row + k-group (the 64 bytes of a row that one request
+  // covers lie in a quad of neighbouring lanes: the memory pipeline merges neighbours' accesses only,
+  // so this is one look-up per row instead of four) and exchanged into the MFMA operand layout
+  // lane = row + 16 * k-group when the step is consumed.
+  const int ln = lane >> 2, lg = lane & 3;
+  const int from_lane4 = 4 * (4 * n + g);
+  // weight row that this lane requests in row group `grp` of the workgroup
+  auto group_row_of = [&](int grp, int r) {
+    if constexpr (FUSE) return min(wg_row0 + (grp >> 1) * 16 + r, last) + (grp & 1) * n_out;
+    else return min(wg_row0 + grp * 16 + r, last);
   };
 
   // ---- activations: 16-byte loads (8 values) per thread, requested before any weights
@@ -166,9 +172,9 @@ gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
   auto issue = [&](StepRaw& dst) {
     const int sb = (isi << sl_log2) + sl;
     const bool ok = ir < rounds && sb < nsb;
-    const int row = group_row(ir * G + gi);
-    const uint32_t o_hdr = ok ? (uint32_t)row * rb + (uint32_t)sb * 144u : 0u;
-    const uint32_t o_q = o_hdr + 16u + 16u * (uint32_t)g;
+    const int row = group_row_of(ir * G + gi, ln), hrow = group_row_of(ir * G + gi, n);
+    const uint32_t o_hdr = ok ? (uint32_t)hrow * rb + (uint32_t)sb * 144u : 0u;
+    const uint32_t o_q = (ok ? (uint32_t)row * rb + (uint32_t)sb * 144u : 0u) + 16u + 16u * (uint32_t)lg;
     dst.hdr = load16_a16(w + o_hdr);
     dst.c0 = load16_a16(w + o_q);
     dst.c1 = load16_a16(w + (o_q + 64u));
@@ -303,6 +309,13 @@ gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
   int cr = 0, csi = 0;                  // round and step-in-round being consumed
   float acc = 0.f;
 
+  auto pull = [&](uint4& v) {
+    v.x = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane4, (int)v.x);
+    v.y = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane4, (int)v.y);
+    v.z = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane4, (int)v.z);
+    v.w = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane4, (int)v.w);
+  };
+  // `s` is the step in operand layout (see exchange below)
   auto consume = [&](const StepRaw& s) {
     const int sb = (csi << sl_log2) + sl;
     if (cr < rounds && sb < nsb) {
@@ -392,12 +405,19 @@ gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
   for (int t0 = R; t0 < t_total; t0 += R) {
 #pragma unroll
     for (int i = 0; i < R; i++) {
-      consume(ring[i]);
+      // exchange into operand layout, re-request the slot, then do the arithmetic
+      StepRaw t = ring[i];
+      pull(t.c0); pull(t.c1);
       issue(ring[i]);
+      consume(t);
     }
   }
 #pragma unroll
-  for (int i = 0; i < R; i++) consume(ring[i]);
+  for (int i = 0; i < R; i++) {
+    StepRaw t = ring[i];
+    pull(t.c0); pull(t.c1);
+    consume(t);
+  }
 
   if (!FUSE && sl_log2 != 0) {
     // one round only: add the slices in a fixed order
