@@ -83,7 +83,7 @@ template <bool COMPACT, int TOK, typename XT, typename YT>
 __global__ void __launch_bounds__(kMfmaThreads)
 gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_t* __restrict__ x,
                    YT* __restrict__ y, const void* __restrict__ bias, int bias_dtype, int m, int n_out, int nch,
-                   int rows_per_wg, int sl_log2) {
+                   int rows_per_wg, int sl_log2, int exch_min_steps) {
   static_assert(COMPACT || TOK == 1, "several tokens use the compact tables");
   using X = Q8WX<XT>;
   constexpr int W = kMfmaWaves, T = X::kPlanes;
@@ -108,6 +108,7 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
   const int wg_row_end = min(wg_row0 + rows_per_wg, n_out);
   const int rounds = (rows_per_wg + 16 * G - 1) / (16 * G);
   const int t_total = rounds * S;
+  const bool exch = t_total >= exch_min_steps;
   const int last = wg_row_end - 1;   // rows past the workgroup's share re-read its last row
 
   // ---- activations: 8 values per thread and pass, requested before any weights
@@ -130,11 +131,18 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
   auto issue = [&](Q8WinStep& dst) {
     const int ch = (isi << sl_log2) + sl;
     const bool ok = ir < rounds && ch < nch;
+    // pieces 0..15 with lane = 4 * row + k-group, so that the 64 bytes of a row that one request
+    // covers lie in a quad of neighbouring lanes (the memory pipeline merges neighbours' accesses
+    // only); they are exchanged into the operand layout lane = row + 16 * k-group when the step is
+    // consumed.  Piece 16 is the same for a row's four lanes and is requested in operand layout.
+    // The exchange costs a wavefront latency once per step, which only pays when it has several
+    // steps to overlap it with; with fewer, everything is requested in operand layout.
     const int row = min(wg_row0 + (ir * G + gi) * 16 + n, last);
-    const uint32_t o = (ok ? (uint32_t)row * rb + (uint32_t)ch * 272u : 0u) + 16u * (uint32_t)g;
+    const int qrow = min(wg_row0 + (ir * G + gi) * 16 + (exch ? lane >> 2 : n), last);
+    const uint32_t o = (ok ? (uint32_t)qrow * rb + (uint32_t)ch * 272u : 0u) + 16u * (uint32_t)(exch ? lane & 3 : g);
 #pragma unroll
     for (int i = 0; i < 4; i++) dst.p[i] = load16_a16(w + (o + 64u * i));
-    dst.p[4] = load16_a16(w + (o - 16u * (uint32_t)g + 256u));     // piece 16, the same for all four lanes
+    dst.p[4] = load16_a16(w + ((ok ? (uint32_t)row * rb + (uint32_t)ch * 272u : 0u) + 256u));
     if (++isi == S) { isi = 0; ir++; }
   };
   issue(cur);
@@ -251,6 +259,16 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
     if (row < wg_row_end && t0 + t < m)
       YElem<YT>::store(y + (int64_t)(t0 + t) * n_out, row, v + load_bias(bias, bias_dtype, row));
   };
+  const int from_lane4 = 4 * (4 * n + g);
+  auto exchange = [&](Q8WinStep& t) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      t.p[i].x = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane4, (int)t.p[i].x);
+      t.p[i].y = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane4, (int)t.p[i].y);
+      t.p[i].z = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane4, (int)t.p[i].z);
+      t.p[i].w = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane4, (int)t.p[i].w);
+    }
+  };
   auto consume = [&](const Q8WinStep& s) {
     const int ch = (csi << sl_log2) + sl;
     if (cr < rounds && ch < nch) {
@@ -315,9 +333,12 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
     }
   };
   for (int t = 1; t < t_total; t++) {
-    consume(cur);
+    Q8WinStep now = cur;
+    if (exch) exchange(now);
     issue(cur);
+    consume(now);
   }
+  if (exch) exchange(cur);
   consume(cur);
 
   if (sl_log2 != 0) {
@@ -356,6 +377,7 @@ static hipError_t q8win_launch_xy(const void* w, const void* x, void* y, const v
   const bool compact = tok > 1 || nch > kQ8WinMaxWideChunks;
   const size_t lds = lds_for(compact, tok);
   const dim3 grid((unsigned)num_wg, (unsigned)((m + tok - 1) / tok));
+  static const int exch_min_steps = mfma_env_int("TTQ_GEMV_Q8_EXCHANGE_MIN_STEPS", 2);
   const auto launch = [&](auto kernel, LargeLds& configured) -> hipError_t {
     {
       const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), configured);
@@ -363,7 +385,7 @@ static hipError_t q8win_launch_xy(const void* w, const void* x, void* y, const v
     }
     hipLaunchKernelGGL(kernel, grid, dim3(W * 64), lds, s, static_cast<const uint8_t*>(w),
                        static_cast<const typename Q8WX<XT>::elem_t*>(x), static_cast<YT*>(y), bias, bias_dtype, (int)m,
-                       (int)n_out, nch, rows_per_wg, sl_log2);
+                       (int)n_out, nch, rows_per_wg, sl_log2, exch_min_steps);
     return hipGetLastError();
   };
   static LargeLds configured_wide, configured_compact, configured_2, configured_4;
