@@ -135,7 +135,8 @@ TTQ_API int ttq_gemm_q8_0(const void* w, const uint16_t* x_bf16, uint16_t* y_bf1
 /* Prefill half of GatedMLP.forward in one kernel: y (m, n_ff) = silu(x Wg^T) * (x Wu^T) with the
  * fused gate||up weight of mlp.nim:39 (2*n_ff rows, gate rows first) -- gate_up_proj.forward
  * followed by silu_and_mul (mlp.nim:56-59, activations.nim:14-38), silu(g)*u formed in fp32 from
- * the fp32 accumulators and rounded once to bf16.  n_in a multiple of 256. */
+ * the fp32 accumulators and rounded once to bf16.  n_in a multiple of 256. 
+ * Up to 64 rows may run the few-row kernel (see ttq_gemm_q4_k), same arithmetic. */
 TTQ_API int ttq_gemm_q4_k_silu_mul(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m,
                   int64_t n_ff, int64_t n_in, void* stream);
 

@@ -233,7 +233,14 @@ int ttq_gemm_q4_k_silu_mul(const void* w, const uint16_t* x_bf16, uint16_t* y_bf
   if (rc != TTQ_OK) return rc;
   if (n_ff > 0x3FFFFFFF) return TTQ_ERR_UNSUPPORTED;
   if (!aligned16(w) || !aligned16(x_bf16) || !aligned16(y_bf16)) return TTQ_ERR_ALIGN;
-  if (!ttq::gemm_pc_supported(TTQ_Q4_K, m, 2 * n_ff, n_in, 112)) return TTQ_ERR_UNSUPPORTED;
+  // up to 64 rows: the few-row kernel where it is estimated to be faster than the tiled one
+  const bool pc_ok = ttq::gemm_pc_supported(TTQ_Q4_K, m, 2 * n_ff, n_in, 112);
+  if (ttq::gemm_skinny_silu_mul_supported(m, n_ff, n_in) &&
+      (!pc_ok || ttq::gemm_skinny_silu_mul_estimate_us(m, n_ff, n_in) <
+                     ttq::gemm_pc_estimate_us(TTQ_Q4_K, m, 2 * n_ff, n_in)))
+    return hip_status(ttq::launch_gemm_skinny_silu_mul(w, x_bf16, y_bf16, TTQ_BF16, nullptr, 0, m, n_ff, n_in,
+                                                       static_cast<hipStream_t>(stream)));
+  if (!pc_ok) return TTQ_ERR_UNSUPPORTED;
   return hip_status(ttq::launch_gemm_pc_silu_mul(w, x_bf16, y_bf16, TTQ_BF16, nullptr, 0, m, n_ff, n_in,
                                                  static_cast<hipStream_t>(stream)));
 }

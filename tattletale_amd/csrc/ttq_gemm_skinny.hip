@@ -253,7 +253,7 @@ struct SkQ8_0 {
 // (super-block, row block) items of packed weights per wavefront, WD - 1 of them in flight; XB:
 // buffers for a super-block's activations (2: the next super-block's are requested while this one
 // is multiplied).
-template <class WF, int RB, int TB, int WD, int XB>
+template <class WF, int RB, int TB, int WD, int XB, bool FUSE>
 __global__ void __launch_bounds__(kSkThreads)
 gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, void* __restrict__ yv,
                        int y_dtype, const void* __restrict__ bias, int bias_dtype, int m, int n_out, int n_in) {
@@ -263,7 +263,13 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int li = lane & 15, kg = lane >> 4;
   const int nsb = n_in >> 8;
-  const int n0 = blockIdx.x * (16 * RB);
+  // FUSE: the weight holds gate rows [0, n_out) then up rows [n_out, 2 * n_out) (the fused
+  // gate||up projection of workspace/transformers/src/layers/mlp.nim:39) and the kernel writes
+  // silu(gate . x) * (up . x) for its 8 * RB outputs: row blocks alternate between the gate rows
+  // and the up rows of the same 16 outputs.
+  static_assert(!FUSE || RB % 2 == 0, "a fused workgroup needs gate and up row blocks in pairs");
+  constexpr int kOutPerWg = FUSE ? 8 * RB : 16 * RB;
+  const int n0 = blockIdx.x * kOutPerWg;
 
   // byte offset of (row, super-block 0) and element offset of (token, k = 8*kg)
   uint32_t wofs[RB], xofs[TB];
@@ -275,7 +281,9 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
   const uint32_t from_lane4 = 4u * (uint32_t)(4 * li + kg);
 #pragma unroll
   for (int rb = 0; rb < RB; rb++)
-    wofs[rb] = (uint32_t)min(n0 + 16 * rb + load_row, n_out - 1) * ((uint32_t)nsb * WF::kBlockBytes);
+    wofs[rb] = (uint32_t)(FUSE ? min(n0 + 16 * (rb >> 1) + load_row, n_out - 1) + (rb & 1) * n_out
+                               : min(n0 + 16 * rb + load_row, n_out - 1)) *
+               ((uint32_t)nsb * WF::kBlockBytes);
 #pragma unroll
   for (int tb = 0; tb < TB; tb++)
     xofs[tb] = (uint32_t)min(16 * tb + load_row, m - 1) * (uint32_t)n_in + WF::x_lane_k(load_kg);
@@ -387,13 +395,26 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
   }
   __syncthreads();
   // 8 consecutive outputs of one token per thread
-  for (int t = tid; t < 16 * TB * 2 * RB; t += kSkThreads) {
-    const int tok = t / (2 * RB), g = t % (2 * RB);
+  constexpr int kGroups = kOutPerWg / 8;
+  for (int t = tid; t < 16 * TB * kGroups; t += kSkThreads) {
+    const int tok = t / kGroups, g = t % kGroups;
     const int col = n0 + 8 * g;
     if (tok >= m || col >= n_out) continue;      // n_out is a multiple of 8: a group is all in or all out
     float v[8];
+    if constexpr (FUSE) {
+      // outputs 8g .. 8g+7 of the workgroup: gate in row block 2 * (g / 2), up in the next one
+      const int lr = 32 * (g >> 1) + 8 * (g & 1);
 #pragma unroll
-    for (int k = 0; k < 8; k++) v[k] = tile[tok * kTileLd + 8 * g + k] + load_bias(bias, bias_dtype, col + k);
+      for (int k = 0; k < 8; k++) {
+        const float gt = tile[tok * kTileLd + lr + k] + load_bias(bias, bias_dtype, col + k);
+        const float up = tile[tok * kTileLd + lr + 16 + k] + load_bias(bias, bias_dtype, (int64_t)n_out + col + k);
+        // silu with the hardware exp2 / reciprocal, as the tiled kernel's epilogue forms it
+        v[k] = (gt * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(gt * -1.4426950408889634f))) * up;
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < 8; k++) v[k] = tile[tok * kTileLd + 8 * g + k] + load_bias(bias, bias_dtype, col + k);
+    }
     const int64_t o = (int64_t)tok * n_out + col;
     if (y_dtype == kBF16) {
       *reinterpret_cast<uint4*>(static_cast<uint16_t*>(yv) + o) =
@@ -406,7 +427,8 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
   }
 }
 
-template <int RB, int TB, class K>
+// n_out counts outputs: weight rows, or gate/up pairs when fused.
+template <int RB, int TB, bool FUSE, class K>
 hipError_t launch_skinny_k(K kernel, const uint8_t* w, const uint16_t* x, void* y, int y_dtype, const void* bias,
                            int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
   const size_t lds = (size_t)(kSkWaves * RB * TB * 4 * 64 + 16 * TB * (16 * RB + 1)) * sizeof(float);
@@ -415,16 +437,17 @@ hipError_t launch_skinny_k(K kernel, const uint8_t* w, const uint16_t* x, void* 
     const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), configured);
     if (e != hipSuccess) return e;
   }
-  const dim3 grid((unsigned)((n_out + 16 * RB - 1) / (16 * RB))), block(kSkThreads);
+  constexpr int kOutPerWg = FUSE ? 8 * RB : 16 * RB;
+  const dim3 grid((unsigned)((n_out + kOutPerWg - 1) / kOutPerWg)), block(kSkThreads);
   hipLaunchKernelGGL(kernel, grid, block, lds, s, w, x, y, y_dtype, bias, bias_dtype, (int)m, (int)n_out, (int)n_in);
   return hipGetLastError();
 }
 
-template <class WF, int RB, int TB, int WD, int XB>
+template <class WF, int RB, int TB, int WD, int XB, bool FUSE>
 hipError_t launch_skinny_tb(const uint8_t* w, const uint16_t* x, void* y, int y_dtype, const void* bias,
                             int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
-  return launch_skinny_k<RB, TB>(gemm_skinny_kernel<WF, RB, TB, WD, XB>, w, x, y, y_dtype, bias, bias_dtype, m, n_out,
-                                 n_in, s);
+  return launch_skinny_k<RB, TB, FUSE>(gemm_skinny_kernel<WF, RB, TB, WD, XB, FUSE>, w, x, y, y_dtype, bias,
+                                       bias_dtype, m, n_out, n_in, s);
 }
 
 // Cost model (microseconds), a least-squares fit to 4096 x 4096, 4096 x 14336 and 14336 x 4096 with
@@ -445,13 +468,14 @@ float skinny_cost_us(int format, int rb, int64_t m, int64_t n_out, int64_t n_in)
   return (float)((wgs + cus - 1) / cus) * (kF0[t] + (float)iters * (kX[t] + rb * wf * kW[t])) + 0.2f * mb;
 }
 
-int skinny_choose_rb(int format, int64_t m, int64_t n_out, int64_t n_in, float* cost_us = nullptr) {
+// rows = weight rows (twice the outputs when fused, which also rules out single row blocks)
+int skinny_choose_rb(int format, int64_t m, int64_t rows, int64_t n_in, bool fuse, float* cost_us = nullptr) {
   static const int forced_rb = [] { const char* e = getenv("TTQ_SK_RB"); return e ? atoi(e) : 0; }();
   int best = 4;
   float best_cost = 1e30f;
-  for (int rb = 4; rb >= 1; rb >>= 1) {
-    if (forced_rb > 0 && rb != forced_rb) continue;
-    const float c = skinny_cost_us(format, rb, m, n_out, n_in);
+  for (int rb = 4; rb >= (fuse ? 2 : 1); rb >>= 1) {
+    if (forced_rb > 0 && rb != forced_rb && !(fuse && forced_rb == 1)) continue;
+    const float c = skinny_cost_us(format, rb, m, rows, n_in);
     if (c < best_cost) { best_cost = c; best = rb; }
   }
   if (cost_us) *cost_us = best_cost;
@@ -459,18 +483,20 @@ int skinny_choose_rb(int format, int64_t m, int64_t n_out, int64_t n_in, float* 
 }
 
 // Registers decide how far ahead a wavefront can request: 64 per token block for the activations.
-template <class WF>
+template <class WF, bool FUSE>
 hipError_t launch_skinny_fmt(int format, const uint8_t* wb, const uint16_t* x_bf16, void* y, int y_dtype,
                              const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                              hipStream_t s) {
-  const int rb = skinny_choose_rb(format, m, n_out, n_in);
+  const int rb = skinny_choose_rb(format, m, FUSE ? 2 * n_out : n_out, n_in, FUSE);
   const int tb = (int)((m + 15) / 16);
 #define TTQ_SK_CASE(RBv, TBv, WDv, XBv) \
   if (rb == RBv && tb == TBv)            \
-    return launch_skinny_tb<WF, RBv, TBv, WDv, XBv>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    return launch_skinny_tb<WF, RBv, TBv, WDv, XBv, FUSE>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   TTQ_SK_CASE(4, 1, 4, 2) TTQ_SK_CASE(4, 2, 4, 2) TTQ_SK_CASE(4, 3, 2, 1) TTQ_SK_CASE(4, 4, 2, 1)
   TTQ_SK_CASE(2, 1, 4, 2) TTQ_SK_CASE(2, 2, 4, 2) TTQ_SK_CASE(2, 3, 2, 1) TTQ_SK_CASE(2, 4, 2, 1)
-  TTQ_SK_CASE(1, 1, 2, 2) TTQ_SK_CASE(1, 2, 2, 2) TTQ_SK_CASE(1, 3, 2, 1) TTQ_SK_CASE(1, 4, 2, 1)
+  if constexpr (!FUSE) {
+    TTQ_SK_CASE(1, 1, 2, 2) TTQ_SK_CASE(1, 2, 2, 2) TTQ_SK_CASE(1, 3, 2, 1) TTQ_SK_CASE(1, 4, 2, 1)
+  }
 #undef TTQ_SK_CASE
   return hipErrorInvalidValue;
 }
@@ -489,8 +515,27 @@ bool gemm_skinny_supported(int format, int64_t m, int64_t n_out, int64_t n_in) {
 
 float gemm_skinny_estimate_us(int format, int64_t m, int64_t n_out, int64_t n_in) {
   float c = 0.f;
-  skinny_choose_rb(format, m, n_out, n_in, &c);
+  skinny_choose_rb(format, m, n_out, n_in, false, &c);
   return c;
+}
+
+// The fused gate||up + silu_and_mul form: n_ff outputs from 2 * n_ff weight rows (Q4_K).
+bool gemm_skinny_silu_mul_supported(int64_t m, int64_t n_ff, int64_t n_in) {
+  return gemm_skinny_supported(kQ4_K, m, 2 * n_ff, n_in) && n_ff % 8 == 0;
+}
+
+float gemm_skinny_silu_mul_estimate_us(int64_t m, int64_t n_ff, int64_t n_in) {
+  float c = 0.f;
+  skinny_choose_rb(kQ4_K, m, 2 * n_ff, n_in, true, &c);
+  return c;
+}
+
+hipError_t launch_gemm_skinny_silu_mul(const void* w, const uint16_t* x_bf16, void* y, int y_dtype, const void* bias,
+                                       int bias_dtype, int64_t m, int64_t n_ff, int64_t n_in, hipStream_t s) {
+  if (m == 0 || n_ff == 0) return hipSuccess;
+  if (y_dtype != kBF16 && y_dtype != kF32) return hipErrorInvalidValue;
+  return launch_skinny_fmt<SkQ4K, true>(kQ4_K, static_cast<const uint8_t*>(w), x_bf16, y, y_dtype, bias, bias_dtype, m,
+                                        n_ff, n_in, s);
 }
 
 hipError_t launch_gemm_skinny(int format, const void* w, const uint16_t* x_bf16, void* y, int y_dtype,
@@ -500,9 +545,9 @@ hipError_t launch_gemm_skinny(int format, const void* w, const uint16_t* x_bf16,
   if (y_dtype != kBF16 && y_dtype != kF32) return hipErrorInvalidValue;
   const uint8_t* wb = static_cast<const uint8_t*>(w);
   switch (format) {
-    case kQ4_K: return launch_skinny_fmt<SkQ4K>(format, wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-    case kQ6_K: return launch_skinny_fmt<SkQ6K>(format, wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-    case kQ8_0: return launch_skinny_fmt<SkQ8_0>(format, wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kQ4_K: return launch_skinny_fmt<SkQ4K, false>(format, wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kQ6_K: return launch_skinny_fmt<SkQ6K, false>(format, wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kQ8_0: return launch_skinny_fmt<SkQ8_0, false>(format, wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
     default: return hipErrorInvalidValue;
   }
 }

@@ -105,6 +105,13 @@ hipError_t launch_gemm_skinny(int format, const void* w, const uint16_t* x_bf16,
                               const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                               hipStream_t s);
 
+// The same kernel with the fused gate||up weight (2 * n_ff rows, gate rows first) and silu_and_mul
+// in its epilogue: y is (m, n_ff).  Q4_K.
+bool gemm_skinny_silu_mul_supported(int64_t m, int64_t n_ff, int64_t n_in);
+float gemm_skinny_silu_mul_estimate_us(int64_t m, int64_t n_ff, int64_t n_in);
+hipError_t launch_gemm_skinny_silu_mul(const void* w, const uint16_t* x_bf16, void* y, int y_dtype, const void* bias,
+                                       int bias_dtype, int64_t m, int64_t n_ff, int64_t n_in, hipStream_t s);
+
 // The multi-row operator for block formats and bf16 activations: the few-row kernel or the tiled
 // GEMM, whichever is estimated to be faster for the shape (ttq_gemm_q4k.hip).
 bool gemm_supported(int format, int64_t m, int64_t n_out, int64_t n_in);

@@ -106,6 +106,8 @@ proc forward*(self: QuantLinear, x: TorchTensor): TorchTensor =
 
 const kTtqErrUnsupported = -6
 const kFusedGemmMinRows = 512
+const kFusedFewRowsMin = 17     # 17..64 rows: the few-row kernel with silu_and_mul in its epilogue
+const kFusedFewRowsMax = 64
 
 type
   QuantGatedMLP* = object
@@ -144,8 +146,10 @@ proc forward*(self: QuantGatedMLP, x: TorchTensor): TorchTensor =
     if rc == 0: return self.down_proj.forward(act)
     if rc != kTtqErrUnsupported:
       raise newException(QuantLinearError, "ttq_gemv_q4_k_silu_mul: " & $strerror(rc))
-  elif gu.format == kQ4_K and gu.bias.isNone and m >= kFusedGemmMinRows and x.scalarType() == kBfloat16:
-    # prefill: silu_and_mul in the GEMM epilogue (breaks even at 512 rows, 15 % faster at 2048)
+  elif gu.format == kQ4_K and gu.bias.isNone and x.scalarType() == kBfloat16 and
+       (m >= kFusedGemmMinRows or (m >= kFusedFewRowsMin and m <= kFusedFewRowsMax)):
+    # prefill: silu_and_mul in the GEMM epilogue (breaks even at 512 rows, 15 % faster at 2048);
+    # 17..64 rows: the same entry point runs the few-row kernel
     var shape = x.sizes().asNimView().toSeq()
     shape[^1] = nff
     let act = F.empty(shape, x.options())

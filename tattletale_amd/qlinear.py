@@ -324,10 +324,14 @@ class QuantGatedMLP:
     # wins once the (rows, 2 * intermediate) tensor it saves no longer fits the caches: at
     # 28672 x 4096 it breaks even at 512 rows and is 15 % faster at 2048.
     FUSED_GEMM_MIN_ROWS = 512
+    # 17..64 rows: the same entry point runs the few-row kernel with the activation in its epilogue (one
+    # launch and one (rows, 2 * intermediate) round trip less); up to 16 rows the few-row GEMV passes
+    # plus silu_and_mul are faster.
+    FUSED_FEW_ROWS = (17, 64)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """x (..., hidden) -> (..., hidden)  (mlp.nim:43-60).  On Q4_K weights a single-token 16-bit
-        activation takes the fused GEMV + silu_and_mul kernel and a bf16 activation of at least
+        activation takes the fused GEMV + silu_and_mul kernel and a bf16 activation of 17 to 64 or at least
         ``FUSED_GEMM_MIN_ROWS`` rows the GEMM with silu_and_mul in its epilogue; everything else runs
         the projection, ``silu_and_mul`` and the down projection as three launches."""
         gu = self.gate_up_proj
@@ -341,7 +345,8 @@ class QuantGatedMLP:
             except TtqError as e:
                 if e.status != _lib.ERR_UNSUPPORTED:
                     raise
-        elif (gu.format == _lib.Q4_K and gu.bias is None and m >= self.FUSED_GEMM_MIN_ROWS
+        elif (gu.format == _lib.Q4_K and gu.bias is None
+              and (m >= self.FUSED_GEMM_MIN_ROWS or self.FUSED_FEW_ROWS[0] <= m <= self.FUSED_FEW_ROWS[1])
               and x.dtype == torch.bfloat16 and gu.in_features % 256 == 0):
             try:
                 act = gemm_q4_k_silu_mul(gu.qweight, x.reshape(m, gu.in_features), n_ff,

@@ -241,9 +241,13 @@ def test_fused_rmsnorm_full_shape_gate_up():
 
 # ------------------------------------------------------------------ prefill: silu_and_mul in the GEMM epilogue
 @pytest.mark.parametrize("m,n_ff,n_in", [(64, 256, 1024), (16, 56, 256), (100, 200, 768), (257, 130, 1024),
-                                         (512, 1000, 2048), (300, 3000, 256)])
+                                         (512, 1000, 2048), (300, 3000, 256),
+                                         (17, 200, 768), (33, 3080, 256), (49, 4104, 256), (64, 6152, 512),
+                                         (5, 72, 2304)])
 def test_fused_gate_up_silu_mul_gemm(m, n_ff, n_in):
-    """Tiles of 56 outputs (full, ragged, a single partial one), 64- and 256-row tiles, ragged rows."""
+    """Tiles of 56 outputs (full, ragged, a single partial one), 64- and 256-row tiles, ragged rows.
+    Up to 64 rows the entry point may run the few-row kernel (16 or 32 outputs per workgroup, one to
+    four token blocks): the last five shapes, with outputs that do not fill the last workgroup."""
     p = random_blocks(F.Q4_K, 2 * n_ff * (n_in // 256), seed=n_ff + m)
     what = oracle.dequant(F.Q4_K, p, 2 * n_ff, n_in)
     xd, xf = x_to_dev(Q.fill_normal(n_in + m, 1, 1.0, m * n_in).reshape(m, n_in) * np.float32(0.05), "bf16")
