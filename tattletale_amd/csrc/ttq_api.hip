@@ -233,6 +233,7 @@ int ttq_gemm_q4_k_silu_mul(const void* w, const uint16_t* x_bf16, uint16_t* y_bf
   if (rc != TTQ_OK) return rc;
   if (n_ff > 0x3FFFFFFF) return TTQ_ERR_UNSUPPORTED;
   if (!aligned16(w) || !aligned16(x_bf16) || !aligned16(y_bf16)) return TTQ_ERR_ALIGN;
+  if (m == 0 || n_ff == 0) return TTQ_OK;
   // up to 64 rows: the few-row kernel where it is estimated to be faster than the tiled one
   const bool pc_ok = ttq::gemm_pc_supported(TTQ_Q4_K, m, 2 * n_ff, n_in, 112);
   if (ttq::gemm_skinny_silu_mul_supported(m, n_ff, n_in) &&
@@ -251,6 +252,7 @@ static int gemm_block(int format, const void* w, const uint16_t* x_bf16, uint16_
   const int rc = check_shape(format, m, n_out, n_in, 0, 0);
   if (rc != TTQ_OK) return rc;
   if (!aligned16(w) || !aligned16(x_bf16) || !aligned16(y_bf16)) return TTQ_ERR_ALIGN;
+  if (m == 0 || n_out == 0) return TTQ_OK;
   if (!ttq::gemm_supported(format, m, n_out, n_in)) return TTQ_ERR_UNSUPPORTED;
   return hip_status(ttq::launch_gemm(format, w, x_bf16, y_bf16, TTQ_BF16, nullptr, 0, m, n_out, n_in,
                                      static_cast<hipStream_t>(stream)));

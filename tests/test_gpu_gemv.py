@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import oracle
-from tattletale_amd import QuantLinear, TtqError, formats as F
+from tattletale_amd import QuantLinear, TtqError, _lib, formats as F
 from tattletale_amd import configs as CFG
 from tattletale_amd import qlinear as QL
 from tattletale_amd import quantize as Q
@@ -309,3 +309,24 @@ def test_full_shape_q4_k_14336x4096():
 
 def test_full_shape_q6_k_128256x4096_sampled_rows():
     assert _full("q6_k_gemv", 37) <= TOL
+
+
+def test_zero_rows_and_zero_outputs_are_no_ops():
+    """m == 0 or n_out == 0: status OK, nothing launched that writes (the reference's F.linear returns an
+    empty tensor for an empty batch)."""
+    L = _lib.lib()
+    n_in = 1024
+    w = torch.zeros(64 * 4 * 210, dtype=torch.uint8, device=DEV)           # room for any block format
+    x = torch.zeros(n_in, dtype=torch.bfloat16, device=DEV)
+    y = torch.full((64,), 7.0, dtype=torch.float32, device=DEV)
+    s = torch.cuda.current_stream().cuda_stream
+    for m, n_out in ((0, 64), (1, 0), (0, 0)):
+        for fn in (L.ttq_gemv_q8_0, L.ttq_gemv_q4_k, L.ttq_gemv_q6_k):
+            assert fn(w.data_ptr(), x.data_ptr(), _lib.BF16, y.data_ptr(), m, n_out, n_in, s) == _lib.OK
+        for fn in (L.ttq_gemm_q4_k, L.ttq_gemm_q6_k, L.ttq_gemm_q8_0, L.ttq_gemm_q4_k_silu_mul):
+            assert fn(w.data_ptr(), x.data_ptr(), y.data_ptr(), m, n_out, n_in, s) == _lib.OK
+        st = _lib.QLinearStruct(format=F.Q4_K, bits=0, codebook=0, bias_dtype=0, n_out=n_out, n_in=n_in,
+                                qweight=w.data_ptr(), suh=None, svh=None, bias=None)
+        assert L.ttq_linear_forward(st, x.data_ptr(), _lib.BF16, m, y.data_ptr(), _lib.F32, s) == _lib.OK
+    torch.cuda.synchronize()
+    assert bool((y == 7.0).all())
