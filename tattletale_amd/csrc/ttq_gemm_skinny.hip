@@ -12,9 +12,12 @@
 //   * one step of v_mfma_f32_16x16x32_bf16 is one sub-block (32 k): lane (i = lane % 16, g = lane / 16)
 //     supplies k = 32*step + 8*g + {0..7}, for weight row 16*rb + i as the A operand and for
 //     activation row ("token") 16*tb + i as the B operand.  For the activations that is one
-//     16-byte load per step, and the four lanes of a token read 64 consecutive bytes, so a load
-//     instruction touches 16 cache lines (what such loads cost is lines looked up, not bytes);
-//     the 128 bytes per token block stay in registers for all row blocks of the workgroup;
+//     16-byte piece per step; the 128 bytes per token block stay in registers for all row blocks
+//     of the workgroup;
+//   * the four pieces of a row (or token) that one request covers are 64 consecutive bytes, but in
+//     operand layout they belong to lanes 16 apart, and the memory pipeline merges the accesses of
+//     neighbouring lanes only.  So every request is made with lane = 4 * row + piece and the data
+//     is exchanged into lane = row + 16 * piece with ds_bpermute when it is used;
 //   * for the weights it is the 8 weights at those k of the lane's row, dequantized in registers
 //     (canonical arithmetic written as one exact fused multiply-add, one bf16 rounding).  Q4_K: the
 //     8 bytes 8*g .. 8*g+7 of each of the four 32-byte qs chunks, low nibbles for the even sub-block
@@ -27,9 +30,13 @@
 //   * the eight wavefronts' partial sums meet in LDS once, at the end; the sums are transposed
 //     through LDS so that every thread stores 8 consecutive outputs of one token.
 //
-// Algorithmic bytes: the packed weights once (n_out * n_in * 0.5625) plus m * n_out outputs; the
-// activations (m * n_in * 2 per workgroup) come from L2.  The kernel is bound by the
-// dequantization (about 3 vector instructions per weight), not by HBM or the matrix cores.
+//   * with the fused gate||up weight (FUSE) row blocks alternate between gate rows and up rows of the
+//     same outputs and silu(gate) * up is formed where the partial sums meet.
+//
+// Algorithmic bytes: the packed weights once (n_out * n_in * 0.5625 for Q4_K) plus m * n_out
+// outputs; the activations (m * n_in * 2 per workgroup) come from L2.  The kernel is bound by the
+// dequantization (about 3 vector instructions per weight) and the activation re-reads, not by HBM
+// or the matrix cores.
 #include <type_traits>
 
 #include "ttq_device.h"
