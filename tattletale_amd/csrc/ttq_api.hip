@@ -330,6 +330,19 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
       return hip_status(ttq::launch_gemm(layer->format, layer->qweight, static_cast<const uint16_t*>(x), y, y_dtype,
                                          layer->bias, layer->bias_dtype, m, n_out, n_in, s));
   }
+  // fp16 activations: no tiled GEMM, but the few-row kernel takes them, 64 rows per launch
+  const bool block_format = layer->format == TTQ_Q4_K || layer->format == TTQ_Q6_K || layer->format == TTQ_Q8_0;
+  if (x_dtype == TTQ_F16 && block_format && m >= 5 && route != 1 &&
+      ttq::gemm_skinny_supported(layer->format, m < 64 ? m : 64, n_out, n_in)) {
+    const int64_t full = m / 64, rest = m % 64;
+    float us = (float)full * ttq::gemm_skinny_estimate_us(layer->format, 64, n_out, n_in);
+    if (rest) us += ttq::gemm_skinny_estimate_us(layer->format, rest, n_out, n_in);
+    const bool gemv_ok = check_gemv_limits(x_dtype, n_in) == TTQ_OK;
+    if (!gemv_ok || route == 2 || us < ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in))
+      return hip_status(ttq::launch_gemm_skinny_chunked(layer->format, layer->qweight, static_cast<const uint16_t*>(x),
+                                                        x_dtype, y, y_dtype, layer->bias, layer->bias_dtype, m, n_out,
+                                                        n_in, s));
+  }
   const int lim = check_gemv_limits(x_dtype, n_in);
   if (lim != TTQ_OK) return lim;
   return hip_status(ttq::launch_gemv(layer->format, layer->qweight, x, x_dtype, y, y_dtype, layer->bias,

@@ -424,7 +424,7 @@ hipError_t launch_gemm(int format, const void* w, const uint16_t* x_bf16, void* 
                        int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
   if (m == 0 || n_out == 0) return hipSuccess;
   if (prefer_skinny(format, m, n_out, n_in))
-    return launch_gemm_skinny(format, w, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    return launch_gemm_skinny(format, w, x_bf16, kBF16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   if (format != kQ4_K) {
     if (!gemm_pc_supported(format, m, n_out, n_in, 112)) return hipErrorInvalidValue;
     return launch_gemm_pc(format, w, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);

@@ -72,26 +72,51 @@ __device__ __forceinline__ f32x4_t gather_row4(float sel, float v) {
   return __builtin_amdgcn_mfma_f32_16x16x4f32(sel, v, zero, 0, 0, 0);
 }
 
-// 8 weights -> 8 bf16 as scale * u + offset for the bytes u of q0 (weights 0..3) and q1 (4..7).
-__device__ __forceinline__ void fma_bytes_to_bf16(uint32_t q0, uint32_t q1, float scale, float offset,
-                                                  uint32_t (&au)[4]) {
+// 8 weights as scale * u + offset for the bytes u of q0 (weights 0..3) and q1 (4..7).
+__device__ __forceinline__ void fma_bytes(uint32_t q0, uint32_t q1, float scale, float offset, float (&f)[8]) {
   // keep the words opaque: byte k of them converts with one v_cvt_f32_ubyte<k>
   asm volatile("" : "+v"(q0), "+v"(q1));
-  float f[8];
 #pragma unroll
   for (int k = 0; k < 4; k++) {
     f[k] = fmaf_(scale, (float)((q0 >> (8 * k)) & 0xFFu), offset);
     f[4 + k] = fmaf_(scale, (float)((q1 >> (8 * k)) & 0xFFu), offset);
   }
-  au[0] = pack_bf16x2(f[0], f[1]);
-  au[1] = pack_bf16x2(f[2], f[3]);
-  au[2] = pack_bf16x2(f[4], f[5]);
-  au[3] = pack_bf16x2(f[6], f[7]);
+}
+
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+  f16x2_t r;
+  r[0] = (_Float16)lo;      // round-to-nearest-even
+  r[1] = (_Float16)hi;
+  uint32_t u;
+  __builtin_memcpy(&u, &r, 4);
+  return u;
+}
+// two floats -> one dword of the activation type XT (bf16_tag / f16_tag), one rounding each
+template <class XT> __device__ __forceinline__ uint32_t pack_x2(float lo, float hi) {
+  if constexpr (std::is_same<XT, f16_tag>::value) return pack_f16x2(lo, hi);
+  else return pack_bf16x2(lo, hi);
+}
+// acc += A(16 x 32) * B(32 x 16) with both operands of the activation type
+template <class XT>
+__device__ __forceinline__ f32x4_t mfma_16x16x32(const uint32_t (&a)[4], const uint4& b, f32x4_t acc) {
+  if constexpr (std::is_same<XT, f16_tag>::value) {
+    f16x8_t av, bv;
+    __builtin_memcpy(&av, a, 16);
+    __builtin_memcpy(&bv, &b, 16);
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bv, acc, 0, 0, 0);
+  } else {
+    bf16x8_t av, bv;
+    __builtin_memcpy(&av, a, 16);
+    __builtin_memcpy(&bv, &b, 16);
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, acc, 0, 0, 0);
+  }
 }
 
 // A format supplies: the bytes of 256 weights of a row (kBlockBytes), what lane (row, kg) keeps of
-// them (Raw, fetch), the per-super-block preparation of scales (Prep, prepare) and the 8 bf16
-// weights k = 32*i + 8*kg .. +7 of step i (dequant).
+// them (Raw, fetch), the per-super-block preparation of scales (Prep, prepare) and the 8 weights
+// of step i as floats (dequant; the kernel rounds them once to the activation type).
 struct SkQ4K {
   static constexpr uint32_t kBlockBytes = 144;
   static __device__ __forceinline__ uint32_t x_lane_k(int kg) { return 8u * kg; }
@@ -147,12 +172,12 @@ struct SkQ4K {
   }
   // fused multiply-add == the canonical two-step form: d is an f16, sc has 6 bits and q 4, so the
   // product is exact in fp32
-  static __device__ __forceinline__ void dequant(const Raw& r, const Prep& P, const Lane&, int i, uint32_t (&au)[4]) {
+  static __device__ __forceinline__ void dequant(const Raw& r, const Prep& P, const Lane&, int i, float (&f)[8]) {
     const int c = i >> 1;
     const float ds = (i & 1) ? P.dd[c] : P.de[c], nm = (i & 1) ? P.md[c] : P.me[c];
     const uint32_t q0 = ((i & 1) ? (r.q[c].x >> 4) : r.q[c].x) & 0x0F0F0F0Fu;
     const uint32_t q1 = ((i & 1) ? (r.q[c].y >> 4) : r.q[c].y) & 0x0F0F0F0Fu;
-    fma_bytes_to_bf16(q0, q1, ds, nm, au);
+    fma_bytes(q0, q1, ds, nm, f);
   }
 };
 
@@ -201,14 +226,14 @@ struct SkQ6K {
     }
   }
   // (d * sc) * (q - 32) as one fused multiply-add on the unsigned q: the same exact product
-  static __device__ __forceinline__ void dequant(const Raw& r, const Prep& P, const Lane&, int i, uint32_t (&au)[4]) {
+  static __device__ __forceinline__ void dequant(const Raw& r, const Prep& P, const Lane&, int i, float (&f)[8]) {
     const int h = i >> 2, j = i & 3;
     const uint2 ql = (j & 1) ? r.qb[h] : r.qa[h];
     const uint32_t n0 = ((j >> 1) ? (ql.x >> 4) : ql.x) & 0x0F0F0F0Fu;
     const uint32_t n1 = ((j >> 1) ? (ql.y >> 4) : ql.y) & 0x0F0F0F0Fu;
     const uint32_t h0 = (r.qh[h].x >> (2 * j)) & 0x03030303u;
     const uint32_t h1 = (r.qh[h].y >> (2 * j)) & 0x03030303u;
-    fma_bytes_to_bf16((h0 << 4) | n0, (h1 << 4) | n1, P.ds[i], P.off[i], au);
+    fma_bytes((h0 << 4) | n0, (h1 << 4) | n1, P.ds[i], P.off[i], f);
   }
 };
 
@@ -249,10 +274,10 @@ struct SkQ8_0 {
     }
   }
   // d * q as one fused multiply-add on u = q + 128 (the sign bit flipped): d * u - 128 d
-  static __device__ __forceinline__ void dequant(const Raw& r, const Prep& P, const Lane&, int i, uint32_t (&au)[4]) {
+  static __device__ __forceinline__ void dequant(const Raw& r, const Prep& P, const Lane&, int i, float (&f)[8]) {
     const int pr = i >> 1;
     const uint32_t q0 = (i & 1) ? r.q[pr].z : r.q[pr].x, q1 = (i & 1) ? r.q[pr].w : r.q[pr].y;
-    fma_bytes_to_bf16(q0 ^ 0x80808080u, q1 ^ 0x80808080u, P.d[pr], P.off[pr], au);
+    fma_bytes(q0 ^ 0x80808080u, q1 ^ 0x80808080u, P.d[pr], P.off[pr], f);
   }
 };
 
@@ -260,7 +285,7 @@ struct SkQ8_0 {
 // (super-block, row block) items of packed weights per wavefront, WD - 1 of them in flight; XB:
 // buffers for a super-block's activations (2: the next super-block's are requested while this one
 // is multiplied).
-template <class WF, int RB, int TB, int WD, int XB, bool FUSE>
+template <class WF, class XT, int RB, int TB, int WD, int XB, bool FUSE>
 __global__ void __launch_bounds__(kSkThreads)
 gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, void* __restrict__ yv,
                        int y_dtype, const void* __restrict__ bias, int bias_dtype, int m, int n_out, int n_in) {
@@ -328,14 +353,14 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
     constexpr int XI = decltype(xi_c)::value;
     constexpr int kAhead = WD - 1;
     const int sb_next = sb + kSkWaves < nsb ? sb + kSkWaves : sb;
-    if (XB == 1) load_x(xfr[0], sb);
+    if constexpr (XB == 1) load_x(xfr[0], sb);
     // this super-block's activations into the operand layout (they were requested one super-block
     // ago when there are two buffers)
 #pragma unroll
     for (int tb = 0; tb < TB; tb++)
 #pragma unroll
       for (int i = 0; i < 8; i++) pull_lane(from_lane4, xfr[XB == 1 ? 0 : XI][tb][i]);
-    if (XB == 2) load_x(xfr[XI ^ 1], sb_next);
+    if constexpr (XB == 2) load_x(xfr[XI ^ 1], sb_next);
 #pragma unroll
     for (int rb = 0; rb < RB; rb++) {
       {
@@ -351,16 +376,13 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
       WF::prepare(r, L, P);
 #pragma unroll
       for (int i = 0; i < 8; i++) {
-        uint32_t au[4];
-        WF::dequant(r, P, L, i, au);
-        bf16x8_t a;
-        __builtin_memcpy(&a, au, 16);
+        float f[8];
+        WF::dequant(r, P, L, i, f);
+        const uint32_t au[4] = {pack_x2<XT>(f[0], f[1]), pack_x2<XT>(f[2], f[3]), pack_x2<XT>(f[4], f[5]),
+                                pack_x2<XT>(f[6], f[7])};
 #pragma unroll
-        for (int tb = 0; tb < TB; tb++) {
-          bf16x8_t b;
-          __builtin_memcpy(&b, &xfr[XB == 1 ? 0 : XI][tb][i], 16);
-          acc[rb][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[rb][tb], 0, 0, 0);
-        }
+        for (int tb = 0; tb < TB; tb++)
+          acc[rb][tb] = mfma_16x16x32<XT>(au, xfr[XB == 1 ? 0 : XI][tb][i], acc[rb][tb]);
       }
     }
   };
@@ -426,6 +448,9 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
     if (y_dtype == kBF16) {
       *reinterpret_cast<uint4*>(static_cast<uint16_t*>(yv) + o) =
           make_uint4(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7]));
+    } else if (y_dtype == kF16) {
+      *reinterpret_cast<uint4*>(static_cast<uint16_t*>(yv) + o) =
+          make_uint4(pack_f16x2(v[0], v[1]), pack_f16x2(v[2], v[3]), pack_f16x2(v[4], v[5]), pack_f16x2(v[6], v[7]));
     } else {
       float4* yo = reinterpret_cast<float4*>(static_cast<float*>(yv) + o);
       yo[0] = make_float4(v[0], v[1], v[2], v[3]);
@@ -450,10 +475,10 @@ hipError_t launch_skinny_k(K kernel, const uint8_t* w, const uint16_t* x, void* 
   return hipGetLastError();
 }
 
-template <class WF, int RB, int TB, int WD, int XB, bool FUSE>
+template <class WF, class XT, int RB, int TB, int WD, int XB, bool FUSE>
 hipError_t launch_skinny_tb(const uint8_t* w, const uint16_t* x, void* y, int y_dtype, const void* bias,
                             int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
-  return launch_skinny_k<RB, TB, FUSE>(gemm_skinny_kernel<WF, RB, TB, WD, XB, FUSE>, w, x, y, y_dtype, bias,
+  return launch_skinny_k<RB, TB, FUSE>(gemm_skinny_kernel<WF, XT, RB, TB, WD, XB, FUSE>, w, x, y, y_dtype, bias,
                                        bias_dtype, m, n_out, n_in, s);
 }
 
@@ -490,7 +515,7 @@ int skinny_choose_rb(int format, int64_t m, int64_t rows, int64_t n_in, bool fus
 }
 
 // Registers decide how far ahead a wavefront can request: 64 per token block for the activations.
-template <class WF, bool FUSE>
+template <class WF, class XT, bool FUSE>
 hipError_t launch_skinny_fmt(int format, const uint8_t* wb, const uint16_t* x_bf16, void* y, int y_dtype,
                              const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                              hipStream_t s) {
@@ -498,7 +523,7 @@ hipError_t launch_skinny_fmt(int format, const uint8_t* wb, const uint16_t* x_bf
   const int tb = (int)((m + 15) / 16);
 #define TTQ_SK_CASE(RBv, TBv, WDv, XBv) \
   if (rb == RBv && tb == TBv)            \
-    return launch_skinny_tb<WF, RBv, TBv, WDv, XBv, FUSE>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    return launch_skinny_tb<WF, XT, RBv, TBv, WDv, XBv, FUSE>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   TTQ_SK_CASE(4, 1, 4, 2) TTQ_SK_CASE(4, 2, 4, 2) TTQ_SK_CASE(4, 3, 2, 1) TTQ_SK_CASE(4, 4, 2, 1)
   TTQ_SK_CASE(2, 1, 4, 2) TTQ_SK_CASE(2, 2, 4, 2) TTQ_SK_CASE(2, 3, 2, 1) TTQ_SK_CASE(2, 4, 2, 1)
   if constexpr (!FUSE) {
@@ -541,22 +566,48 @@ hipError_t launch_gemm_skinny_silu_mul(const void* w, const uint16_t* x_bf16, vo
                                        int bias_dtype, int64_t m, int64_t n_ff, int64_t n_in, hipStream_t s) {
   if (m == 0 || n_ff == 0) return hipSuccess;
   if (y_dtype != kBF16 && y_dtype != kF32) return hipErrorInvalidValue;
-  return launch_skinny_fmt<SkQ4K, true>(kQ4_K, static_cast<const uint8_t*>(w), x_bf16, y, y_dtype, bias, bias_dtype, m,
+  return launch_skinny_fmt<SkQ4K, bf16_tag, true>(kQ4_K, static_cast<const uint8_t*>(w), x_bf16, y, y_dtype, bias, bias_dtype, m,
                                         n_ff, n_in, s);
 }
 
-hipError_t launch_gemm_skinny(int format, const void* w, const uint16_t* x_bf16, void* y, int y_dtype,
+hipError_t launch_gemm_skinny(int format, const void* w, const uint16_t* x, int x_dtype, void* y, int y_dtype,
                               const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                               hipStream_t s) {
   if (m == 0 || n_out == 0) return hipSuccess;
-  if (y_dtype != kBF16 && y_dtype != kF32) return hipErrorInvalidValue;
+  if (y_dtype != kBF16 && y_dtype != kF32 && y_dtype != kF16) return hipErrorInvalidValue;
   const uint8_t* wb = static_cast<const uint8_t*>(w);
-  switch (format) {
-    case kQ4_K: return launch_skinny_fmt<SkQ4K, false>(format, wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-    case kQ6_K: return launch_skinny_fmt<SkQ6K, false>(format, wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-    case kQ8_0: return launch_skinny_fmt<SkQ8_0, false>(format, wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-    default: return hipErrorInvalidValue;
+  if (x_dtype == kBF16) {
+    switch (format) {
+      case kQ4_K: return launch_skinny_fmt<SkQ4K, bf16_tag, false>(format, wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+      case kQ6_K: return launch_skinny_fmt<SkQ6K, bf16_tag, false>(format, wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+      case kQ8_0: return launch_skinny_fmt<SkQ8_0, bf16_tag, false>(format, wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+      default: return hipErrorInvalidValue;
+    }
   }
+  if (x_dtype == kF16) {
+    switch (format) {
+      case kQ4_K: return launch_skinny_fmt<SkQ4K, f16_tag, false>(format, wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+      case kQ6_K: return launch_skinny_fmt<SkQ6K, f16_tag, false>(format, wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+      case kQ8_0: return launch_skinny_fmt<SkQ8_0, f16_tag, false>(format, wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+      default: return hipErrorInvalidValue;
+    }
+  }
+  return hipErrorInvalidValue;
+}
+
+// More than 64 rows of fp16 activations, for which no tiled GEMM exists: one launch per 64 rows.
+hipError_t launch_gemm_skinny_chunked(int format, const void* w, const uint16_t* x, int x_dtype, void* y, int y_dtype,
+                                      const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                                      hipStream_t s) {
+  const int64_t ysize = y_dtype == kF32 ? 4 : 2;
+  for (int64_t r0 = 0; r0 < m; r0 += 64) {
+    const int64_t rows = m - r0 < 64 ? m - r0 : 64;
+    const hipError_t e = launch_gemm_skinny(format, w, x + r0 * n_in, x_dtype,
+                                            static_cast<uint8_t*>(y) + r0 * n_out * ysize, y_dtype, bias, bias_dtype,
+                                            rows, n_out, n_in, s);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
 }
 
 }  // namespace ttq

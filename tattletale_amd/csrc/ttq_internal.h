@@ -97,13 +97,18 @@ int device_num_cus();
 struct LargeLds { std::atomic<uint64_t> done{0}; };
 hipError_t allow_large_lds(const void* kernel, LargeLds& state);
 
-// Q4_K / Q6_K / Q8_0 linear layer for up to 64 rows of bf16 activations, weights dequantized in
+// Q4_K / Q6_K / Q8_0 linear layer for up to 64 rows of 16-bit activations, weights dequantized in
 // registers (ttq_gemm_skinny.hip).
 bool gemm_skinny_supported(int format, int64_t m, int64_t n_out, int64_t n_in);
 float gemm_skinny_estimate_us(int format, int64_t m, int64_t n_out, int64_t n_in);
-hipError_t launch_gemm_skinny(int format, const void* w, const uint16_t* x_bf16, void* y, int y_dtype,
+// x: bf16 or fp16 activations (the weights are rounded once to the same type); y: bf16, fp16 or fp32.
+hipError_t launch_gemm_skinny(int format, const void* w, const uint16_t* x, int x_dtype, void* y, int y_dtype,
                               const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                               hipStream_t s);
+// Any number of rows, 64 per launch (fp16 activations have no tiled GEMM).
+hipError_t launch_gemm_skinny_chunked(int format, const void* w, const uint16_t* x, int x_dtype, void* y, int y_dtype,
+                                      const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                                      hipStream_t s);
 
 // The same kernel with the fused gate||up weight (2 * n_ff rows, gate rows first) and silu_and_mul
 // in its epilogue: y is (m, n_ff).  Q4_K.

@@ -215,3 +215,48 @@ def test_full_shape_other_formats_sampled_columns(name, n_out):
     want = oracle.linear_f64(what, oracle.bf16_to_f32(xbits[rows]))
     got = oracle.bf16_to_f32(dev_bits(y[torch.from_numpy(rows).to(DEV)][:, torch.from_numpy(cols).to(DEV)]))
     assert rel_l2(got, want) <= TOL
+
+
+# fp16 activations have no tiled GEMM; from five rows on the operator may run the few-row kernel on
+# them, 64 rows per launch, with the weights rounded once to fp16 (11 significant bits: closer to the
+# canonical weights than the bf16 kernels).
+@pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
+@pytest.mark.parametrize("m,n_out,n_in", [(5, 200, 768), (17, 4096, 512), (64, 12296, 256), (100, 1048, 1024),
+                                          (200, 6144, 256)])
+def test_forward_fp16_activations_few_row_kernel(fmt, m, n_out, n_in):
+    p = random_blocks(fmt, n_out * (n_in // BLOCK_WEIGHTS[fmt]), seed=700 + m)
+    what = oracle.dequant(fmt, p, n_out, n_in)
+    bd, bf = x_to_dev(Q.fill_normal(701, 2, 0.5, n_out), "f32")
+    # small activations: the random blocks hold weights up to a few hundred and the fp16 output must
+    # stay finite
+    xd, xf = x_to_dev(Q.fill_normal(702 + m, 1, 1.0, m * n_in).reshape(m, n_in) * np.float32(0.02), "f16")
+    layer = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out, bias=bd)
+    want = oracle.linear_f64(what, xf, bf)
+    y32 = layer.forward(xd, out_dtype=torch.float32)
+    assert y32.shape == (m, n_out) and y32.dtype == torch.float32
+    got = y32.cpu().numpy()
+    assert rel_l2(got, want) <= 1e-3
+    for i in range(0, m, 7):
+        assert rel_l2(got[i], want[i]) <= 2e-3, i
+    y16 = layer.forward(xd)
+    assert y16.dtype == torch.float16
+    assert rel_l2(oracle.f16_to_f32(dev_bits(y16)), want) <= 2e-3
+    ybf = layer.forward(xd, out_dtype=torch.bfloat16)
+    assert rel_l2(oracle.bf16_to_f32(dev_bits(ybf)), want) <= TOL
+
+
+@pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
+def test_forward_fp16_unit_vectors_give_fp16_weights_exactly(fmt):
+    m, n_out, n_in = 40, 6144, 2560
+    p = random_blocks(fmt, n_out * (n_in // BLOCK_WEIGHTS[fmt]), seed=31)
+    what = oracle.dequant(fmt, p, n_out, n_in)
+    ks = (np.arange(m) * 397 + 5) % n_in
+    x = np.zeros((m, n_in), np.float32)
+    x[np.arange(m), ks] = 1.0
+    xd, _ = x_to_dev(x, "f16")
+    layer = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out)
+    y = layer.forward(xd, out_dtype=torch.float32).cpu().numpy()
+    want = oracle.f16_to_f32(oracle.f32_to_f16(what))[:, ks].T
+    # the library decides between this kernel and decode passes by cost; both reproduce the weight up to
+    # its rounding to fp16 at most
+    assert np.array_equal(y, want) or np.array_equal(y, what[:, ks].T)
