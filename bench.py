@@ -361,10 +361,10 @@ def main() -> int:
         ncopies = max(2, -(-2 * MALL_BYTES // (n_out * n_in * 2)))
         ws = [torch.randn((n_out, n_in), device=dev).mul_(0.02).to(torch.bfloat16) for _ in range(ncopies)]
         res = {}
-        for m in (1, 512, 2048):
+        for m in (1, 64, 512, 2048):
             x = torch.randn((m, n_in), device=dev).to(torch.bfloat16)
             y = torch.empty((m, n_out), dtype=torch.bfloat16, device=dev)
-            n = max(10, steps // (1 if m == 1 else 4))
+            n = max(10, steps // (1 if m <= 64 else 4))
             _, ev_ms = time_steps(lambda i: torch.matmul(x, ws[i % ncopies].t(), out=y), n, warmup,
                                   use_graph=not args.eager)
             res["m%d" % m] = {"us_per_step": ev_ms * 1e3, "TFLOPs": 2.0 * m * n_out * n_in / (ev_ms * 1e-3) / 1e12,
