@@ -87,18 +87,22 @@ template <> struct WFmt<kQ4_K> {
     q4k_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, 2 * C + 1, sc2, mn2);
     const float d1 = d * (float)sc1, nm1 = -(dmin * (float)mn1);
     const float d2 = d * (float)sc2, nm2 = -(dmin * (float)mn2);
+    // Nibble bytes (0..15) read as 8-bit floats (4 exponent, 3 mantissa bits) are the subnormals and
+    // the first binade: multiples of one step, so the packed conversion to fp32 gives byte * step
+    // exactly, two bytes per instruction; the step (a power of two) is divided out of the scale.
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    const float inv_step = 1.f / __builtin_amdgcn_cvt_pk_f32_fp8(1, false)[0];
+    const float e1 = d1 * inv_step, e2 = d2 * inv_step;
     const uint32_t qd[4] = {r.q[C].x, r.q[C].y, r.q[C].z, r.q[C].w};
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       // low nibbles are sub-block 2C (the first 32 k of the step), high nibbles sub-block 2C+1
       const uint32_t l4 = qd[i] & 0x0F0F0F0Fu, h4 = (qd[i] >> 4) & 0x0F0F0F0Fu;
-      float fl[4], fh[4];
-#pragma unroll
-      for (int k = 0; k < 4; k++) {
-        // fused multiply-add == canonical two-step form here (the product is exact)
-        fl[k] = fmaf_(d1, (float)((l4 >> (8 * k)) & 0xFFu), nm1);
-        fh[k] = fmaf_(d2, (float)((h4 >> (8 * k)) & 0xFFu), nm2);
-      }
+      const f32x2_t la = __builtin_amdgcn_cvt_pk_f32_fp8((int)l4, false), lb = __builtin_amdgcn_cvt_pk_f32_fp8((int)l4, true);
+      const f32x2_t ha = __builtin_amdgcn_cvt_pk_f32_fp8((int)h4, false), hb = __builtin_amdgcn_cvt_pk_f32_fp8((int)h4, true);
+      // fused multiply-add == canonical two-step form here (the product is exact)
+      const float fl[4] = {fmaf_(e1, la[0], nm1), fmaf_(e1, la[1], nm1), fmaf_(e1, lb[0], nm1), fmaf_(e1, lb[1], nm1)};
+      const float fh[4] = {fmaf_(e2, ha[0], nm2), fmaf_(e2, ha[1], nm2), fmaf_(e2, hb[0], nm2), fmaf_(e2, hb[1], nm2)};
       lo[2 * i] = pack_bf16x2(fl[0], fl[1]);
       lo[2 * i + 1] = pack_bf16x2(fl[2], fl[3]);
       hi[2 * i] = pack_bf16x2(fh[0], fh[1]);

@@ -83,6 +83,22 @@ __device__ __forceinline__ void fma_bytes(uint32_t q0, uint32_t q1, float scale,
   }
 }
 
+// The same for nibbles (bytes 0..15).  Read as an 8-bit float (4 exponent, 3 mantissa bits) the codes
+// 0..15 are the subnormals and the first binade, all multiples of one step, so the packed
+// conversion to fp32 turns two bytes into (byte * step) exactly with one instruction; the step is
+// measured on the constant 0x01 and divided out of the scale (a power of two: exact).
+__device__ __forceinline__ void fma_nibbles(uint32_t q0, uint32_t q1, float scale, float offset, float (&f)[8]) {
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  const float step = __builtin_amdgcn_cvt_pk_f32_fp8(1, false)[0];
+  const float s = scale * (1.f / step);
+  const f32x2_t a = __builtin_amdgcn_cvt_pk_f32_fp8((int)q0, false), b = __builtin_amdgcn_cvt_pk_f32_fp8((int)q0, true);
+  const f32x2_t c = __builtin_amdgcn_cvt_pk_f32_fp8((int)q1, false), d = __builtin_amdgcn_cvt_pk_f32_fp8((int)q1, true);
+  f[0] = fmaf_(s, a[0], offset); f[1] = fmaf_(s, a[1], offset);
+  f[2] = fmaf_(s, b[0], offset); f[3] = fmaf_(s, b[1], offset);
+  f[4] = fmaf_(s, c[0], offset); f[5] = fmaf_(s, c[1], offset);
+  f[6] = fmaf_(s, d[0], offset); f[7] = fmaf_(s, d[1], offset);
+}
+
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
 typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
 __device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
@@ -177,7 +193,7 @@ struct SkQ4K {
     const float ds = (i & 1) ? P.dd[c] : P.de[c], nm = (i & 1) ? P.md[c] : P.me[c];
     const uint32_t q0 = ((i & 1) ? (r.q[c].x >> 4) : r.q[c].x) & 0x0F0F0F0Fu;
     const uint32_t q1 = ((i & 1) ? (r.q[c].y >> 4) : r.q[c].y) & 0x0F0F0F0Fu;
-    fma_bytes(q0, q1, ds, nm, f);
+    fma_nibbles(q0, q1, ds, nm, f);
   }
 };
 
