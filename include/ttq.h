@@ -97,7 +97,11 @@ typedef struct ttq_qlinear {
  * Replaces Linear.forward (linear.nim:45-57) and the F.linear call under it
  * (neural_nets.nim:64,73).  m == 1 runs the decode GEMV; m > 1 runs the prefill GEMM
  * (MFMA kernel for Q4_K with bf16 activations, a batched GEMV otherwise) -- the same
- * split the reference makes implicitly through x.size(1) (attn.nim:154-156). */
+ * split the reference makes implicitly through x.size(1) (attn.nim:154-156).
+ * Accuracy: up to four rows always run the decode kernels (fp32 scales; rel-L2 <= 1e-3 against the
+ * canonical dequantized weights).  From five rows of bf16 (fp16) activations on, the library may
+ * run matrix-core kernels that round each dequantized weight once to bf16 (fp16) -- the 2e-2 class
+ * of the GEMM entry points -- when its cost estimate prefers them for the shape. */
 TTQ_API int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int64_t m,
                        void* y, int y_dtype, void* stream);
 
