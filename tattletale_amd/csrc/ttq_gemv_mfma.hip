@@ -33,6 +33,8 @@
 // consecutive rows and one of SL interleaved slices of the super-blocks, and walks it one
 // step (16 rows x one super-block, 3 x 16 bytes per lane) at a time.  SL is chosen so that
 // all 16 wavefronts have work even when a workgroup owns few rows.
+#include <type_traits>
+
 #include "ttq_gemv_mfma_common.h"
 
 namespace ttq {
@@ -144,13 +146,23 @@ gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
   };
 
   // ---- activations: 16-byte loads (8 values) per thread, requested before any weights
-  uint4 xraw[XP];
+  // (fp32 activations, plain kernel only: 32 bytes per thread; `x` then points at floats)
+  constexpr bool kX32 = std::is_same<XT, float>::value;
+  static_assert(!kX32 || !NORM, "the fused RMSNorm takes 16-bit activations");
+  uint4 xraw[XP], xraw2[kX32 ? XP : 1];
 #pragma unroll
   for (int p = 0; p < XP; p++) {
     const int k0 = 8 * (tid + p * kThreads);
     // a pass past the end re-reads the first pass's data (the compact table means n_in > 8192;
     // spread addresses, never used)
-    xraw[p] = *reinterpret_cast<const uint4*>(xm + (k0 < n_in ? k0 : (COMPACT ? (k0 & (8 * kThreads - 1)) : 0)));
+    const int kc = k0 < n_in ? k0 : (COMPACT ? (k0 & (8 * kThreads - 1)) : 0);
+    if constexpr (kX32) {
+      const float* xf = reinterpret_cast<const float*>(x) + (int64_t)blockIdx.y * n_in + kc;
+      xraw[p] = *reinterpret_cast<const uint4*>(xf);
+      xraw2[p] = *reinterpret_cast<const uint4*>(xf + 4);
+    } else {
+      xraw[p] = *reinterpret_cast<const uint4*>(xm + kc);
+    }
   }
   uint4 rraw[NORM ? XP : 1], graw[NORM ? XP : 1];
   if constexpr (NORM) {
@@ -200,7 +212,15 @@ gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
   // ---- the activations as floats, normalized first if asked
   float xv[XP][8];
 #pragma unroll
-  for (int p = 0; p < XP; p++) widen8<XT>(xraw[p], xv[p]);
+  for (int p = 0; p < XP; p++) {
+    if constexpr (kX32) {
+      const uint32_t d[8] = {xraw[p].x, xraw[p].y, xraw[p].z, xraw[p].w, xraw2[p].x, xraw2[p].y, xraw2[p].z, xraw2[p].w};
+#pragma unroll
+      for (int i = 0; i < 8; i++) xv[p][i] = __uint_as_float(d[i]);
+    } else {
+      widen8<XT>(xraw[p], xv[p]);
+    }
+  }
   if constexpr (NORM) {
     float ss = 0.f;
 #pragma unroll
@@ -486,6 +506,9 @@ static hipError_t launch_any(const void* w, const void* x, int x_dtype, void* y,
                              hipStream_t s) {
   if (x_dtype == kBF16) return launch_x<FUSE, NORM, bf16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, na, s);
   if (x_dtype == kF16) return launch_x<FUSE, NORM, f16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, na, s);
+  if constexpr (!FUSE && !NORM) {
+    if (x_dtype == kF32) return launch_x<false, false, float>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, na, s);
+  }
   return hipErrorInvalidValue;
 }
 
@@ -494,7 +517,7 @@ bool gemv_mfma_supported(int format, int x_dtype, int64_t n_out, int64_t n_in) {
   if (disabled) return false;
   // byte offsets into the weight buffer are 32-bit in the kernel; with fewer than eight rows per
   // CU the per-workgroup activation set-up outweighs the saving
-  return n_out >= 2048 && format == kQ4_K && (x_dtype == kBF16 || x_dtype == kF16) && n_in % 256 == 0 &&
+  return n_out >= 2048 && format == kQ4_K && (x_dtype == kBF16 || x_dtype == kF16 || x_dtype == kF32) && n_in % 256 == 0 &&
          n_in <= kMaxMfmaIn && n_out * (n_in / 256) * 144 < ((int64_t)1 << 32);
 }
 

@@ -124,12 +124,13 @@ def test_row_concatenation_of_packed_weights_is_a_fused_layer():
     assert np.array_equal(y, np.concatenate([yg, yu]))
 
 
-@pytest.mark.parametrize("xk", ["bf16", "f16"])
+@pytest.mark.parametrize("xk", ["bf16", "f16", "f32"])
 @pytest.mark.parametrize("n_out,n_in", [(70000, 256), (25600, 512), (14336 + 8, 1024), (2500, 8192), (5000, 1280), (4096, 14336), (2050, 16384)])
 def test_q4_k_16bit_work_distributions(xk, n_out, n_in):
     """Shapes that exercise every split of rows and super-blocks over the wavefronts of the
     matrix-core kernel: several rounds per workgroup, 1/2/4/16 slices, ragged last groups,
-    a super-block count that is not a power of two; two activation rows."""
+    a super-block count that is not a power of two; two activation rows.  fp32 activations take
+    the same kernel one row at a time."""
     rng = np.random.default_rng(n_out + n_in)
     p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=n_out)
     rows = np.unique(np.concatenate([rng.integers(0, n_out, 400), np.arange(n_out - 40, n_out), np.arange(40)]))
@@ -330,3 +331,18 @@ def test_zero_rows_and_zero_outputs_are_no_ops():
         assert L.ttq_linear_forward(st, x.data_ptr(), _lib.BF16, m, y.data_ptr(), _lib.F32, s) == _lib.OK
     torch.cuda.synchronize()
     assert bool((y == 7.0).all())
+
+
+def test_q4_k_fp32_activations_matrix_core_kernel_unit_vectors():
+    """fp32 activations on a matrix large enough for the matrix-core kernel: unit vectors (also scaled
+    by a power of two) reproduce the canonical column bit for bit."""
+    n_out, n_in = 2304, 1024
+    p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=41)
+    what = oracle.dequant(F.Q4_K, p, n_out, n_in)
+    wd = packed_to_dev(p)
+    for c, scale in ((0, 1.0), (31, 1.0), (32, -0.5), (255, 1.0), (256, 4.0), (n_in - 1, 1.0)):
+        x = np.zeros((1, n_in), np.float32)
+        x[0, c] = scale
+        xd, _ = x_to_dev(x, "f32")
+        y = QL.gemv(F.Q4_K, wd, xd, n_out, n_in).cpu().numpy()[0]
+        assert np.array_equal(y, np.float32(scale) * what[:, c]), (c, scale)
