@@ -44,6 +44,13 @@ hipError_t launch_gemv_mfma(const void* w, const void* x, int x_dtype, void* y, 
                             const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                             hipStream_t s);
 
+// The same arithmetic with the weights streamed through LDS as whole cache lines (ttq_gemv_q4k_stream.hip):
+// 16-bit activations, n_in 2048 or 4096.
+bool gemv_q4k_stream_supported(int format, int x_dtype, int64_t n_out, int64_t n_in);
+hipError_t launch_gemv_q4k_stream(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                                  const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                                  hipStream_t s);
+
 // int8 matrix-core path for Q8_0, any activation dtype (ttq_gemv_q8_mfma.hip).
 // Q8_0 through the matrix cores, rows read as aligned 64-byte windows (ttq_gemv_q8_win.hip).
 bool gemv_q8_win_supported(int format, int64_t n_out, int64_t n_in);
