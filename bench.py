@@ -1,21 +1,38 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-linear hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--replays R] [--only NAME] [--no-cpu] [--no-extra]
 
 Headline workload (`value`): Q4_K decode GEMV, W 14336x4096, batch 1, bf16 activations, fp32
 output -- weight-stream GB/s.  One step = one GEMV call.  Steps rotate through enough distinct
-copies of the packed weight (> 256 MiB in total) that the Infinity Cache cannot serve the
-stream, and are replayed from a HIP graph so that host launch cost does not starve a kernel
-that runs for a few microseconds.  All inputs are resident in HBM before the timed region.
+copies of the packed weight (> 2 x 256 MiB in total) that the Infinity Cache cannot serve the
+stream.  All inputs are resident in HBM before the timed region.
+
+Launch: K >= 200 steps are captured into one HIP graph and replayed; fewer steps are launched one
+by one through the C ABI (ctypes, no Python wrapper in the loop).  A graph launch costs about one
+kernel duration (7 us) per replay on this runtime whatever K is, which a 20-step region cannot
+amortize; plain launches cost about 0.15 us more per step but nothing per region.  --graph and
+--eager force either way; `config.launch` says which one ran.
+
+Timing: W untimed warm-up steps, a fixed untimed conditioning phase (the same K steps repeated
+for about 0.4 s, so that a short run is not timed on clocks that have not ramped yet), then R
+timed passes of exactly K steps.  A timed pass is bracketed by synchronization on both sides and
+by HIP events on the stream the kernels run on; one untimed pass is queued in front of the first
+event, so that the K timed steps follow it back to back and the host's submission is not part of a
+20-step measurement.  `ms_per_step` is the median timed pass divided by K; minimum and maximum
+are reported beside it.
 
 The same line carries the other configurations (Q8_0 / Q6_K / EXL3 GEMV, Q4_K GEMM at
-M = 64 / 512 / 2048) under "extra", the roofline of the dominant kernel and a CPU baseline
-timed on this machine's host cores.
+M = 64 / 512 / 2048, attention-shaped GEMVs) under "extra", a roofline object for the GEMV and one
+for the GEMM, and a CPU baseline timed on this machine's host cores.
+
+    python bench.py --only ladder     the roofline ladder of the headline kernel (see csrc/ttq_ladder.hip);
+                                      --only ladder_14336x4096 runs one shape (for a kernel trace)
 """
 from __future__ import annotations
 
 import argparse
+import ctypes as C
 import json
 import os
 import sys
@@ -28,11 +45,29 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 MALL_BYTES = 256 << 20
+CONDITIONING_S = 0.4
+GRAPH_MIN_STEPS = 200     # fewer timed steps than this are launched one by one (a graph launch costs ~7 us per replay)
 METRIC = "Q4_K GEMV weight GB/s (% of HBM peak); Q4_K GEMM M=512 TFLOP/s"
+FMT_NAME = {0: "Q8_0", 1: "Q4_K", 2: "Q6_K", 3: "EXL3"}
+# what the kernels compute in (not a precision claim)
+GEMV_DTYPE = ("i8 (bf16 activations as 15-bit block fixed point in two int8 planes, 4-bit weights, "
+              "int32 MFMA accumulate; fp32 scales and row sums)")
+GEMM_DTYPE = "bf16 (weights dequantized in fp32 and rounded once to bf16; fp32 MFMA accumulate)"
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
+
+
+def cpu_brand() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def main() -> int:
@@ -40,10 +75,13 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--only", default=None, help="run a single configuration (name in tattletale_amd.configs)")
+    ap.add_argument("--replays", type=int, default=7, help="timed replays of the K-step graph (median reported)")
+    ap.add_argument("--only", default=None, help="run a single configuration (name in tattletale_amd.configs), "
+                                                 "or one of: ladder, widened, q4_k_gate_up_silu_gemv, dense_reference")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-extra", action="store_true", help="headline workload only")
-    ap.add_argument("--eager", action="store_true", help="time plain launches instead of a HIP graph")
+    ap.add_argument("--eager", action="store_true", help="always time plain launches")
+    ap.add_argument("--graph", action="store_true", help="always time replays of a HIP graph of K launches")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run a plain device copy of 256 MiB a few times and exit (reference point for "
                          "scaling the FETCH_SIZE / WRITE_SIZE counters of rocprofv3)")
@@ -84,14 +122,22 @@ def main() -> int:
             return t.view(TD[kind]) if kind in ("f16", "bf16") else t
         return torch.from_numpy(a).to(dev)
 
-    def time_steps(step_fn, steps: int, warmup: int, use_graph: bool):
-        """Runs `warmup` untimed and exactly `steps` timed calls of step_fn(i).
-        Returns (wall ms per step, HIP-event ms per step)."""
+    def time_steps(step_fn, steps: int, warmup: int, use_graph: bool = True, replays: int | None = None,
+                   direct_fn=None):
+        """`warmup` untimed calls of step_fn(i), a graph of exactly `steps` calls (or, for few steps and
+        when a `direct_fn(i)` that goes straight to the C ABI is given, plain launches), an untimed
+        conditioning phase, then `replays` timed passes.  Returns a dict with the per-step times
+        (milliseconds, HIP events on the launch stream): median, min, max over the passes."""
+        replays = args.replays if replays is None else replays
         stream = torch.cuda.current_stream(dev)
         for i in range(warmup):
             step_fn(i)
         torch.cuda.synchronize()
         graph = None
+        if args.eager or (direct_fn is not None and steps < GRAPH_MIN_STEPS and not args.graph):
+            use_graph = False
+            if direct_fn is not None:
+                step_fn = direct_fn
         if use_graph:
             graph = torch.cuda.CUDAGraph()
             side = torch.cuda.Stream(dev)
@@ -104,21 +150,49 @@ def main() -> int:
                         step_fn(i)
             stream.wait_stream(side)
             torch.cuda.synchronize()
-            graph.replay()            # untimed replay: uploads the graph
+
+        def run_once():
+            if graph is not None:
+                graph.replay()
+            else:
+                for i in range(steps):
+                    step_fn(i)
+
+        # conditioning: same launches, untimed, a fixed wall-clock budget
+        run_once()
+        torch.cuda.synchronize()
+        t_end = time.perf_counter() + CONDITIONING_S
+        n_cond = 1
+        while time.perf_counter() < t_end:
+            run_once()
             torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        e0.record(stream)
-        if graph is not None:
-            graph.replay()
-        else:
-            for i in range(steps):
-                step_fn(i)
-        e1.record(stream)
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
+            n_cond += 1
+        per = []
+        wall = []
+        for _ in range(max(1, replays)):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            # an untimed replay runs while the host submits the timed one, so that the K timed steps
+            # start back to back with the first event instead of waiting for the submission
+            run_once()
+            e0.record(stream)
+            run_once()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            wall.append((time.perf_counter() - t0) * 1e3 / (2 * steps))
+            per.append(e0.elapsed_time(e1) / steps)
+        per.sort()
+        wall.sort()
+        return {"ms": per[len(per) // 2], "ms_min": per[0], "ms_max": per[-1], "wall_ms": wall[len(wall) // 2],
+                "replays": len(per), "conditioning_replays": n_cond,
+                "launch": ("hip-graph replay of %d launches" % steps) if graph is not None else
+                          ("%d plain stream launches through the C ABI" % steps if step_fn is direct_fn else
+                           "%d plain stream launches through the Python wrapper" % steps)}
+
+    def rotated(nbytes: int) -> int:
+        """Copies of a weight of nbytes to rotate through so that the Infinity Cache cannot serve it."""
+        return 1 if nbytes > MALL_BYTES else min(96, max(2, -(-2 * MALL_BYTES // nbytes)))
 
     def run_config(name: str, steps: int, warmup: int):
         cfg = CFG.CONFIGS[name]
@@ -127,11 +201,11 @@ def main() -> int:
         xh = CFG.activations(cfg)
         log("[%s] inputs generated in %.1f s" % (name, time.time() - t0))
         x = to_dev(xh, cfg.x_dtype)
+        direct = None
         if cfg.fmt == F.EXL3:
             trellis, suh, svh = packed
             wbytes = trellis.nbytes
-            ncopies = max(2, -(-2 * MALL_BYTES // wbytes))
-            ncopies = min(ncopies, 96)
+            ncopies = rotated(wbytes)
             tr = [to_dev(trellis) for _ in range(ncopies)]
             suh_d, svh_d = to_dev(suh, "f16"), to_dev(svh, "f16")
             y = torch.empty((cfg.m, cfg.n_out), dtype=torch.float32, device=dev)
@@ -140,65 +214,129 @@ def main() -> int:
                 QL.gemv_exl3(tr[i % ncopies], suh_d, svh_d, x, cfg.n_out, cfg.n_in, cfg.bits, F.CB_MCG, out=y)
         else:
             wbytes = packed.nbytes
-            ncopies = 1 if wbytes > MALL_BYTES else max(2, -(-2 * MALL_BYTES // wbytes))
+            ncopies = rotated(wbytes)
             ws = [to_dev(packed) for _ in range(ncopies)]
             if cfg.m == 1:
                 y = torch.empty((1, cfg.n_out), dtype=torch.float32, device=dev)
 
                 def step(i):
                     QL.gemv(cfg.fmt, ws[i % ncopies], x, cfg.n_out, cfg.n_in, out=y)
+                entry = getattr(_lib.lib(), {F.Q8_0: "ttq_gemv_q8_0", F.Q4_K: "ttq_gemv_q4_k",
+                                             F.Q6_K: "ttq_gemv_q6_k"}[cfg.fmt])
+                wp, xp, yp = [w.data_ptr() for w in ws], x.data_ptr(), y.data_ptr()
+                xcode = {"f32": _lib.F32, "f16": _lib.F16, "bf16": _lib.BF16}[cfg.x_dtype]
+                sp = torch.cuda.current_stream(dev).cuda_stream
+
+                def direct(i):
+                    rc = entry(wp[i % ncopies], xp, xcode, yp, 1, cfg.n_out, cfg.n_in, sp)
+                    if rc:
+                        raise RuntimeError("%s returned %d" % (name, rc))
             else:
                 y = torch.empty((cfg.m, cfg.n_out), dtype=torch.bfloat16, device=dev)
 
                 def step(i):
                     QL.gemm_q4_k(ws[i % ncopies], x, cfg.n_out, cfg.n_in, out=y)
-        wall_ms, ev_ms = time_steps(step, steps, warmup, use_graph=not args.eager)
+        t = time_steps(step, steps, warmup, direct_fn=direct)
         flops = 2.0 * cfg.m * cfg.n_out * cfg.n_in
         res = {
-            "name": name, "steps": steps, "weight_bytes": int(wbytes), "weight_copies": ncopies,
-            "ms_per_step": ev_ms, "wall_ms_per_step": wall_ms,
-            "weight_GBps": wbytes / (ev_ms * 1e-3) / 1e9,
-            "TFLOPs": flops / (ev_ms * 1e-3) / 1e12,
+            "name": name, "steps": steps, "replays": t["replays"], "launch": t["launch"], "weight_bytes": int(wbytes),
+            "weight_copies": ncopies,
+            "ms_per_step": t["ms"], "ms_per_step_min": t["ms_min"], "ms_per_step_max": t["ms_max"],
+            "wall_ms_per_step": t["wall_ms"],
+            "weight_GBps": wbytes / (t["ms"] * 1e-3) / 1e9,
+            "TFLOPs": flops / (t["ms"] * 1e-3) / 1e12,
         }
         if cfg.m == 1:
             res["hbm_frac"] = res["weight_GBps"] / HBM_PEAK_GBPS
         else:
             res["mfma_frac"] = res["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS
-        log("[%s] %.3f us/step  %.0f GB/s  %.1f TFLOP/s" % (name, ev_ms * 1e3, res["weight_GBps"], res["TFLOPs"]))
+        log("[%s] %.3f us/step (min %.3f, max %.3f over %d replays)  %.0f GB/s  %.1f TFLOP/s" % (
+            name, t["ms"] * 1e3, t["ms_min"] * 1e3, t["ms_max"] * 1e3, t["replays"], res["weight_GBps"],
+            res["TFLOPs"]))
         del y
         torch.cuda.empty_cache()
         return res
 
+    def random_packed(rng, fmt, n_out, n_in):
+        """Random packed bytes with finite scale fields (timing only)."""
+        nbytes, wpb, scale_hi = {F.Q8_0: (34, 32, [1]), F.Q4_K: (144, 256, [1, 3]), F.Q6_K: (210, 256, [209])}[fmt]
+        raw = rng.integers(0, 256, (n_out * (n_in // wpb), nbytes), dtype=np.uint8)
+        for off in scale_hi:
+            raw[:, off] &= 0x3F            # |fp16 scale| < 2
+        return raw.reshape(-1)
+
     def cpu_baseline():
-        """The oracle's fused packed-weight GEMV (a port of the same op to plain C) on the host
-        cores, plus ATen's dense linear on dequantized weights (what the reference runs on CPU)."""
+        """The same operator on this machine's host cores, in the probes-table style of the reference
+        (workspace/probes/src/reports.nim:27-46: name, calls, time per call, rate).
+
+        kind "port": the oracle's fused packed-weight GEMV (plain C, OpenMP), all host cores and one
+        thread, for the four GEMV configurations; plus ATen's dense bf16 linear on dequantized weights
+        for the headline shape, which is what the reference's Linear.forward runs on a CPU."""
         import oracle
+        ncores = os.cpu_count() or 1
+        table = []
+
+        def timed(label, fn, nbytes, flops, threads, budget_s):
+            fn()
+            n, t0 = 0, time.perf_counter()
+            while True:
+                fn()
+                n += 1
+                dt = time.perf_counter() - t0
+                if dt >= budget_s:
+                    break
+            per = dt / n
+            row = {"name": label, "threads": threads, "calls": n, "us_per_call": per * 1e6,
+                   "weight_GBps": nbytes / per / 1e9, "GFLOPs": flops / per / 1e9}
+            table.append(row)
+            log("  %-34s %3d thr %5d calls %12.1f us/call %8.2f GB/s %8.2f GFLOP/s" % (
+                label, threads, n, row["us_per_call"], row["weight_GBps"], row["GFLOPs"]))
+            return row
+
+        log("[cpu_baseline] %s, %d logical cores" % (cpu_brand(), ncores))
+        head_all = head_one = None
+        for name, budget in (("q4_k_gemv", 3.0), ("q8_0_gemv", 1.5), ("q6_k_gemv", 3.0)):
+            cfg = CFG.CONFIGS[name]
+            packed = CFG.packed_weights(cfg)
+            xh = CFG.activations(cfg)
+            xf = (oracle.bf16_to_f32(xh) if cfg.x_dtype == "bf16" else np.asarray(xh, np.float32))[0]
+            flops = 2.0 * cfg.n_out * cfg.n_in
+            for thr in (ncores, 1):
+                r = timed("%s %dx%d" % (name, cfg.n_out, cfg.n_in),
+                          lambda: oracle.gemv_fused(cfg.fmt, packed, xf, cfg.n_out, cfg.n_in, thr),
+                          packed.nbytes, flops, thr, budget)
+                if name == "q4_k_gemv":
+                    if thr == ncores:
+                        head_all = r
+                    else:
+                        head_one = r
+        # EXL3: decode the trellis and multiply (the oracle has no fused form; one thread)
+        cfg = CFG.CONFIGS["exl3_gemv"]
+        trellis, suh, svh = CFG.packed_weights(cfg)
+        xh = CFG.activations(cfg)
+
+        def exl3_once():
+            t = oracle.exl3_decode(trellis, cfg.n_out, cfg.n_in, cfg.bits, oracle.CB_MCG)
+            oracle.exl3_gemv_f64(t, suh, svh, xh[0])
+
+        timed("exl3_gemv %dx%d (decode + multiply)" % (cfg.n_out, cfg.n_in), exl3_once, trellis.nbytes,
+              2.0 * cfg.n_out * cfg.n_in, 1, 2.0)
+        # reference CPU path: dense linear on the dequantized weight (ATen), headline shape
         cfg = CFG.CONFIGS["q4_k_gemv"]
         packed = CFG.packed_weights(cfg)
-        xf = oracle.bf16_to_f32(CFG.activations(cfg))[0]
-        threads = min(os.cpu_count() or 1, 16)
-        oracle.gemv_fused(cfg.fmt, packed, xf, cfg.n_out, cfg.n_in, threads)
-        n, t0 = 0, time.perf_counter()
-        while time.perf_counter() - t0 < 8.0:
-            oracle.gemv_fused(cfg.fmt, packed, xf, cfg.n_out, cfg.n_in, threads)
-            n += 1
-        dt = (time.perf_counter() - t0) / n
-        out = {"value": packed.nbytes / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
-               "sample": "%d calls of the full 14336x4096 Q4_K GEMV (fused C port, OpenMP)" % n,
-               "us_per_call": dt * 1e6}
-        # reference CPU path: dense linear on the dequantized weight (ATen)
         what = torch.from_numpy(oracle.dequant(cfg.fmt, packed, cfg.n_out, cfg.n_in)).to(torch.bfloat16)
-        xb = torch.from_numpy(xf).to(torch.bfloat16)[None, :]
-        torch.set_num_threads(threads)
-        torch.nn.functional.linear(xb, what)
-        n, t0 = 0, time.perf_counter()
-        while time.perf_counter() - t0 < 6.0:
-            torch.nn.functional.linear(xb, what)
-            n += 1
-        dt2 = (time.perf_counter() - t0) / n
-        out["aten_dense_bf16_us_per_call"] = dt2 * 1e6
-        out["aten_dense_bf16_weight_GBps"] = what.numel() * 2 / dt2 / 1e9
-        return out
+        xb = torch.from_numpy(oracle.bf16_to_f32(CFG.activations(cfg))[0]).to(torch.bfloat16)[None, :]
+        for thr in (ncores, 1):
+            torch.set_num_threads(thr)
+            timed("aten dense bf16 linear 14336x4096", lambda: torch.nn.functional.linear(xb, what),
+                  what.numel() * 2, 2.0 * cfg.n_out * cfg.n_in, thr, 2.0)
+        torch.set_num_threads(ncores)
+        return {"value": head_all["weight_GBps"], "unit": "GB/s", "cores": ncores, "kind": "port",
+                "sample": "%d calls of the full 14336x4096 Q4_K GEMV (the oracle's fused C restatement, OpenMP, "
+                          "%d threads); the table has one thread and the other GEMV configurations"
+                          % (head_all["calls"], ncores),
+                "us_per_call": head_all["us_per_call"],
+                "single_thread_value": head_one["weight_GBps"], "cpu": cpu_brand(), "table": table}
 
     def run_gate_up(steps: int, warmup: int):
         """Llama-3-8B FFN decode: the 28672 x 4096 gate/up matrix, silu_and_mul fused into the GEMV
@@ -211,12 +349,10 @@ def main() -> int:
         del w
         log("[q4_k_gate_up_silu_gemv] inputs generated in %.1f s" % (time.time() - t0))
         x = to_dev(CFG.activations(cfg), "bf16")
-        ncopies = max(2, -(-2 * MALL_BYTES // packed.nbytes))
+        ncopies = rotated(packed.nbytes)
         ws = [to_dev(packed) for _ in range(ncopies)]
         y = torch.empty((1, n_ff), dtype=torch.bfloat16, device=dev)
-        gu = torch.empty((1, 2 * n_ff), dtype=torch.float32, device=dev)
         L = _lib.lib()
-        sp = torch.cuda.current_stream(dev).cuda_stream
 
         def fused(i):
             _lib.check(L.ttq_gemv_q4_k_silu_mul(ws[i % ncopies].data_ptr(), x.data_ptr(), F.BF16, y.data_ptr(),
@@ -225,7 +361,6 @@ def main() -> int:
 
         gu16 = torch.empty((1, 2 * n_ff), dtype=torch.bfloat16, device=dev)
         st = _lib.QLinearStruct(format=F.Q4_K, n_out=2 * n_ff, n_in=n_in)
-        import ctypes as C
 
         def unfused(i):
             cur = torch.cuda.current_stream(dev).cuda_stream
@@ -234,7 +369,7 @@ def main() -> int:
                        "ttq_linear_forward")
             _lib.check(L.ttq_silu_and_mul(gu16.data_ptr(), y.data_ptr(), F.BF16, 1, n_ff, cur), "ttq_silu_and_mul")
 
-        # the same with the block's add + RMSNorm in front: one launch against four
+        # the same with the block's add + RMSNorm in front: one launch against three
         res_in = torch.randn((1, n_in), device=dev).to(torch.bfloat16)
         gamma = torch.ones(n_in, dtype=torch.bfloat16, device=dev)
         new_res = torch.empty_like(res_in)
@@ -255,10 +390,10 @@ def main() -> int:
                        "ttq_linear_forward")
             _lib.check(L.ttq_silu_and_mul(gu16.data_ptr(), y.data_ptr(), F.BF16, 1, n_ff, cur), "ttq_silu_and_mul")
 
-        _, f_ms = time_steps(fused, steps, warmup, use_graph=not args.eager)
-        _, u_ms = time_steps(unfused, steps, warmup, use_graph=not args.eager)
-        _, nf_ms = time_steps(norm_fused, steps, warmup, use_graph=not args.eager)
-        _, nu_ms = time_steps(norm_unfused, steps, warmup, use_graph=not args.eager)
+        f_ms = time_steps(fused, steps, warmup)["ms"]
+        u_ms = time_steps(unfused, steps, warmup)["ms"]
+        nf_ms = time_steps(norm_fused, steps, warmup)["ms"]
+        nu_ms = time_steps(norm_unfused, steps, warmup)["ms"]
         res = {"name": "q4_k_gate_up_silu_gemv", "steps": steps, "weight_bytes": int(packed.nbytes),
                "weight_copies": ncopies, "ms_per_step": f_ms, "weight_GBps": packed.nbytes / (f_ms * 1e-3) / 1e9,
                "hbm_frac": packed.nbytes / (f_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
@@ -276,8 +411,8 @@ def main() -> int:
         def pre_unfused(i):
             QL.silu_and_mul(QL.gemm_q4_k(ws[i % ncopies], xm, 2 * n_ff, n_in))
 
-        _, pf_ms = time_steps(pre_fused, 20, 3, use_graph=not args.eager)
-        _, pu_ms = time_steps(pre_unfused, 20, 3, use_graph=not args.eager)
+        pf_ms = time_steps(pre_fused, 20, 3, replays=3)["ms"]
+        pu_ms = time_steps(pre_unfused, 20, 3, replays=3)["ms"]
         res["prefill_m2048_fused_gemm_ms_per_step"] = pf_ms
         res["prefill_m2048_gemm_plus_silu_ms_per_step"] = pu_ms
         res["prefill_m2048_fused_TFLOPs"] = 2.0 * 2048 * 2 * n_ff * n_in / (pf_ms * 1e-3) / 1e12
@@ -287,34 +422,37 @@ def main() -> int:
 
     def run_widened(steps: int, warmup: int):
         """Rows next to the headline ones, on random packed bytes with finite scale fields (timing
-        only): the few-row decode GEMV (8 and 16 activation rows at once), the few-row form of the
+        only): the attention projections as decode GEMVs (q/o 4096x4096, k/v 1024x4096, reference call
+        sites workspace/transformers/src/layers/attn.nim:113-116,154-156,189), the LM-head-sized Q4_K
+        stream, the few-row decode GEMV (8 and 16 activation rows at once), the few-row form of the
         prefill operator (32 rows) and the prefill GEMM for Q6_K and Q8_0 weights, 14336 x 4096 unless
         named otherwise; add + RMSNorm on rows of 4096."""
         n_out, n_in = 14336, 4096
         rng = np.random.default_rng(1234)
         res = {}
 
-        def random_packed(fmt, n_out=n_out, n_in=n_in):
-            nbytes, wpb, scale_hi = {F.Q8_0: (34, 32, [1]), F.Q4_K: (144, 256, [1, 3]), F.Q6_K: (210, 256, [209])}[fmt]
-            raw = rng.integers(0, 256, (n_out * (n_in // wpb), nbytes), dtype=np.uint8)
-            for off in scale_hi:
-                raw[:, off] &= 0x3F            # |fp16 scale| < 2
-            return raw.reshape(-1)
-
-        def timed(name, fmt, m, fn_of, n_out=n_out, n_in=n_in):
-            packed = random_packed(fmt, n_out, n_in)
-            ncopies = max(2, -(-2 * MALL_BYTES // packed.nbytes))
+        def timed(name, fmt, m, fn_of, n_out=n_out, n_in=n_in, steps=steps):
+            packed = random_packed(rng, fmt, n_out, n_in)
+            ncopies = rotated(packed.nbytes)
             ws = [to_dev(packed) for _ in range(ncopies)]
             x = torch.randn((m, n_in), device=dev).to(torch.bfloat16)
             step = fn_of(ws, x, ncopies)
-            _, ev_ms = time_steps(step, steps, warmup, use_graph=not args.eager)
-            res[name] = {"us_per_step": ev_ms * 1e3, "weight_GBps": packed.nbytes / (ev_ms * 1e-3) / 1e9,
-                         "TFLOPs": 2.0 * m * n_out * n_in / (ev_ms * 1e-3) / 1e12}
-            log("[%s] %.2f us/step  %.0f GB/s  %.1f TFLOP/s" % (name, ev_ms * 1e3, res[name]["weight_GBps"],
+            ms = time_steps(step, steps, warmup)["ms"]
+            res[name] = {"us_per_step": ms * 1e3, "weight_GBps": packed.nbytes / (ms * 1e-3) / 1e9,
+                         "hbm_frac": packed.nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                         "TFLOPs": 2.0 * m * n_out * n_in / (ms * 1e-3) / 1e12}
+            log("[%s] %.2f us/step  %.0f GB/s  %.1f TFLOP/s" % (name, ms * 1e3, res[name]["weight_GBps"],
                                                               res[name]["TFLOPs"]))
             del ws
             torch.cuda.empty_cache()
 
+        for nm, (no, ni) in (("q4_k_gemv_o_4096x4096", (4096, 4096)), ("q4_k_gemv_kv_1024x4096", (1024, 4096)),
+                             ("q4_k_gemv_down_4096x14336", (4096, 14336)),
+                             ("q4_k_gemv_lm_head_128256x4096", (128256, 4096))):
+            y = torch.empty((1, no), dtype=torch.float32, device=dev)
+            timed(nm, F.Q4_K, 1,
+                  lambda ws, x, nc, y=y, no=no, ni=ni: (lambda i: QL.gemv(F.Q4_K, ws[i % nc], x, no, ni, out=y)),
+                  n_out=no, n_in=ni, steps=steps if no < 100000 else max(20, steps // 10))
         for m in (8, 16):
             y = torch.empty((m, n_out), dtype=torch.float32, device=dev)
             timed("q4_k_gemv_m%d" % m, F.Q4_K, m,
@@ -329,7 +467,8 @@ def main() -> int:
         for fmt, nm in ((F.Q6_K, "q6_k_gemm_m512"), (F.Q8_0, "q8_0_gemm_m512")):
             y = torch.empty((512, n_out), dtype=torch.bfloat16, device=dev)
             timed(nm, fmt, 512,
-                  lambda ws, x, nc, y=y, fmt=fmt: (lambda i: QL.gemm(fmt, ws[i % nc], x, n_out, n_in, out=y)))
+                  lambda ws, x, nc, y=y, fmt=fmt: (lambda i: QL.gemm(fmt, ws[i % nc], x, n_out, n_in, out=y)),
+                  steps=max(20, steps // 4))
         # add + RMSNorm alone (ttq_rmsnorm with a residual): one decode row and a prefill block.
         # Algorithmic bytes: x and residual read, new residual and normalized row written.
         L = _lib.lib()
@@ -345,10 +484,10 @@ def main() -> int:
                                          F.BF16, new_res.data_ptr(), normed.data_ptr(), m, n_in,
                                          torch.cuda.current_stream(dev).cuda_stream), "ttq_rmsnorm")
 
-            _, ev_ms = time_steps(norm_step, steps, warmup, use_graph=not args.eager)
+            ms = time_steps(norm_step, steps, warmup)["ms"]
             nm = "add_rmsnorm_m%d" % m
-            res[nm] = {"us_per_step": ev_ms * 1e3, "GBps": 4.0 * m * n_in * 2 / (ev_ms * 1e-3) / 1e9}
-            log("[%s] %.2f us/step  %.0f GB/s" % (nm, ev_ms * 1e3, res[nm]["GBps"]))
+            res[nm] = {"us_per_step": ms * 1e3, "GBps": 4.0 * m * n_in * 2 / (ms * 1e-3) / 1e9}
+            log("[%s] %.2f us/step  %.0f GB/s" % (nm, ms * 1e3, res[nm]["GBps"]))
             del xs, rs
             torch.cuda.empty_cache()
         return res
@@ -358,31 +497,86 @@ def main() -> int:
         dense 14336 x 4096 weights, i.e. what the reference's Linear.forward would run on this GPU
         after dequantizing once.  Same timing method, weight copies rotated past the cache."""
         n_out, n_in = 14336, 4096
-        ncopies = max(2, -(-2 * MALL_BYTES // (n_out * n_in * 2)))
+        ncopies = rotated(n_out * n_in * 2)
         ws = [torch.randn((n_out, n_in), device=dev).mul_(0.02).to(torch.bfloat16) for _ in range(ncopies)]
         res = {}
         for m in (1, 64, 512, 2048):
             x = torch.randn((m, n_in), device=dev).to(torch.bfloat16)
             y = torch.empty((m, n_out), dtype=torch.bfloat16, device=dev)
             n = max(10, steps // (1 if m <= 64 else 4))
-            _, ev_ms = time_steps(lambda i: torch.matmul(x, ws[i % ncopies].t(), out=y), n, warmup,
-                                  use_graph=not args.eager)
-            res["m%d" % m] = {"us_per_step": ev_ms * 1e3, "TFLOPs": 2.0 * m * n_out * n_in / (ev_ms * 1e-3) / 1e12,
-                              "weight_GBps": n_out * n_in * 2 / (ev_ms * 1e-3) / 1e9}
+            ms = time_steps(lambda i: torch.matmul(x, ws[i % ncopies].t(), out=y), n, warmup)["ms"]
+            res["m%d" % m] = {"us_per_step": ms * 1e3, "TFLOPs": 2.0 * m * n_out * n_in / (ms * 1e-3) / 1e12,
+                              "weight_GBps": n_out * n_in * 2 / (ms * 1e-3) / 1e9}
             log("[dense_bf16_library m=%d] %.2f us/step  %.1f TFLOP/s  %.0f GB/s of bf16 weights" % (
-                m, ev_ms * 1e3, res["m%d" % m]["TFLOPs"], res["m%d" % m]["weight_GBps"]))
+                m, ms * 1e3, res["m%d" % m]["TFLOPs"], res["m%d" % m]["weight_GBps"]))
         del ws
         torch.cuda.empty_cache()
         return res
 
+    def run_ladder(steps: int, warmup: int, shapes=((14336, 4096), (128256, 4096))):
+        """What each stage of the headline kernel costs on its own (tattletale_amd/csrc/ttq_ladder.hip):
+        empty launch, the kernel's requests alone, + the y store, the kernel without arithmetic, the
+        kernel; at the headline shape and on a 295 MB Q4_K matrix (128256 x 4096)."""
+        lad_path = os.path.join(ROOT, "tattletale_amd", "libttq_ladder.so")
+        if not os.path.exists(lad_path):
+            raise RuntimeError("%s not found: build it with `python -m tattletale_amd.build`" % lad_path)
+        LAD = C.CDLL(lad_path)
+        LAD.ttq_ladder_launch.restype = C.c_int
+        LAD.ttq_ladder_launch.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p]
+        L = _lib.lib()
+        rng = np.random.default_rng(99)
+        names = ["0 empty launch (grid, workgroup and LDS of the GEMV)", "1 requests only (HBM -> LDS, all at once)",
+                 "2 requests + y store", "3 GEMV without arithmetic", "4 GEMV (ttq_gemv_q4_k)"]
+        out = {}
+        for n_out, n_in in shapes:
+            st = steps if n_out < 100000 else max(20, steps // 10)
+            packed = random_packed(rng, F.Q4_K, n_out, n_in)
+            ncopies = rotated(packed.nbytes)
+            ws = [to_dev(packed) for _ in range(ncopies)]
+            x = torch.randn((1, n_in), device=dev).to(torch.bfloat16)
+            y = torch.empty((1, n_out), dtype=torch.float32, device=dev)
+            rows = []
+            for rung in range(5):
+                if rung < 4:
+                    def step(i, rung=rung):
+                        rc = LAD.ttq_ladder_launch(rung, ws[i % ncopies].data_ptr(), x.data_ptr(), y.data_ptr(), n_out,
+                                                   n_in, torch.cuda.current_stream(dev).cuda_stream)
+                        if rc != 0:
+                            raise RuntimeError("ttq_ladder_launch(%d) returned %d" % (rung, rc))
+                else:
+                    def step(i):
+                        _lib.check(L.ttq_gemv_q4_k(ws[i % ncopies].data_ptr(), x.data_ptr(), F.BF16, y.data_ptr(), 1,
+                                                   n_out, n_in, torch.cuda.current_stream(dev).cuda_stream),
+                                   "ttq_gemv_q4_k")
+                t = time_steps(step, st, warmup)
+                gbps = packed.nbytes / (t["ms"] * 1e-3) / 1e9
+                rows.append({"rung": names[rung], "us_per_launch": t["ms"] * 1e3, "us_min": t["ms_min"] * 1e3,
+                             "us_max": t["ms_max"] * 1e3, "weight_GBps": gbps if rung else None,
+                             "hbm_frac": gbps / HBM_PEAK_GBPS if rung else None})
+                log("[ladder %dx%d] %-58s %8.3f us  %s" % (n_out, n_in, names[rung], t["ms"] * 1e3,
+                                                          ("%.0f GB/s (%.3f of peak)" % (gbps, gbps / HBM_PEAK_GBPS))
+                                                          if rung else ""))
+            out["%dx%d" % (n_out, n_in)] = {"weight_bytes": int(packed.nbytes), "weight_copies": ncopies,
+                                           "steps": st, "rungs": rows}
+            del ws
+            torch.cuda.empty_cache()
+        return out
+
+    if args.only == "ladder":
+        print(json.dumps(run_ladder(args.steps, args.warmup)), flush=True)
+        return 0
+    if args.only and args.only.startswith("ladder_"):      # one shape, e.g. ladder_14336x4096 (for a kernel trace)
+        no, ni = (int(v) for v in args.only[len("ladder_"):].split("x"))
+        print(json.dumps(run_ladder(args.steps, args.warmup, shapes=((no, ni),))), flush=True)
+        return 0
     if args.only == "dense_reference":
         print(json.dumps(run_dense_reference(max(20, args.steps // 10), max(3, args.warmup // 10))), flush=True)
         return 0
     if args.only == "widened":
-        print(json.dumps(run_widened(max(20, args.steps // 4), max(3, args.warmup // 4))), flush=True)
+        print(json.dumps(run_widened(max(GRAPH_MIN_STEPS, args.steps // 4), max(3, args.warmup // 4))), flush=True)
         return 0
     if args.only == "q4_k_gate_up_silu_gemv":
-        print(json.dumps(run_gate_up(max(20, args.steps // 4), max(3, args.warmup // 4))), flush=True)
+        print(json.dumps(run_gate_up(max(GRAPH_MIN_STEPS, args.steps // 4), max(3, args.warmup // 4))), flush=True)
         return 0
     names = [args.only] if args.only else ["q4_k_gemv"]
     if not args.only and not args.no_extra:
@@ -391,11 +585,16 @@ def main() -> int:
     for nme in names:
         cfg = CFG.CONFIGS[nme]
         steps = args.steps
-        if cfg.m > 1 or nme == "q6_k_gemv":
-            steps = max(20, args.steps // 10)     # longer kernels need fewer launches
-        if cfg.m >= 2048:
-            steps = max(10, args.steps // 40)
-        results[nme] = run_config(nme, steps, max(3, args.warmup * steps // max(1, args.steps)))
+        if nme != names[0]:
+            # the other rows: fewer launches for longer kernels (the headline keeps K as passed)
+            if cfg.m > 1 or nme == "q6_k_gemv":
+                steps = max(20, args.steps // 10)
+            else:
+                steps = max(GRAPH_MIN_STEPS, args.steps)     # microsecond kernels: enough to amortize the graph launch
+            if cfg.m >= 2048:
+                steps = max(10, args.steps // 40)
+        results[nme] = run_config(nme, steps, max(3, args.warmup * steps // max(1, args.steps)) if nme != names[0]
+                                  else args.warmup)
     head = results[names[0]]
     hc = CFG.CONFIGS[names[0]]
 
@@ -405,40 +604,54 @@ def main() -> int:
         "unit": "GB/s" if hc.m == 1 else "TFLOP/s",
         "n_gpus": 1, "steps": head["steps"], "warmup": args.warmup,
         "ms_per_step": head["ms_per_step"],
+        "ms_per_step_min": head["ms_per_step_min"], "ms_per_step_max": head["ms_per_step_max"],
+        "replays": head["replays"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
+        "dtype": GEMV_DTYPE if hc.m == 1 else GEMM_DTYPE, "data": "synthetic",
         "config": {"workload": "%s: W %dx%d %s, x %dx%d %s, y %s" % (
-            hc.name, hc.n_out, hc.n_in, {0: "Q8_0", 1: "Q4_K", 2: "Q6_K", 3: "EXL3"}[hc.fmt], hc.m, hc.n_in,
-            hc.x_dtype, hc.y_dtype),
-            "launch": "eager" if args.eager else "hip-graph replay of %d launches" % head["steps"],
+            hc.name, hc.n_out, hc.n_in, FMT_NAME[hc.fmt], hc.m, hc.n_in, hc.x_dtype, hc.y_dtype),
+            "launch": head["launch"],
+            "timing": "median of %d timed passes of K steps; each is bracketed by synchronization and by "
+                      "HIP events on the launch stream, with one untimed pass queued in front of the first event"
+                      % head["replays"],
+            "conditioning": "%.1f s of untimed passes of the same K steps before the timed ones" % CONDITIONING_S,
             "weight_copies_rotated": head["weight_copies"]},
     }
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (committed summary)
-    traffic = None
+    traffic = {}
     try:
         with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
-            t = json.load(f).get(hc.name)
-        if t:
-            traffic = t["hbm_read_bytes"] + t["hbm_write_bytes"]
+            traffic = json.load(f)
     except (OSError, ValueError):
         pass
-    if hc.m == 1:
-        line["roofline"] = {"bound": "hbm", "achieved": head["weight_GBps"], "peak": HBM_PEAK_GBPS,
-                            "unit": "GB/s", "frac": head["weight_GBps"] / HBM_PEAK_GBPS, "traffic": traffic,
-                            "algorithmic_bytes": head["weight_bytes"]}
-    else:
-        line["roofline"] = {"bound": "mfma", "achieved": head["TFLOPs"], "peak": MFMA_BF16_PEAK_TFLOPS,
-                            "unit": "TFLOP/s", "frac": head["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS, "traffic": traffic}
-    if "q4_k_gemm_m512" in results:
+
+    def traffic_of(name):
+        t = traffic.get(name)
+        return t["hbm_read_bytes"] + t["hbm_write_bytes"] if t else None
+
+    def gemv_roofline(r, name):
+        return {"bound": "hbm", "kernel": name, "achieved": r["weight_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": r["weight_GBps"] / HBM_PEAK_GBPS, "traffic": traffic_of(name),
+                "algorithmic_bytes": r["weight_bytes"]}
+
+    def gemm_roofline(r, name):
+        c = CFG.CONFIGS[name]
+        return {"bound": "mfma", "kernel": name, "achieved": r["TFLOPs"], "peak": MFMA_BF16_PEAK_TFLOPS,
+                "unit": "TFLOP/s", "frac": r["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS, "traffic": traffic_of(name),
+                "algorithmic_flops": 2.0 * c.m * c.n_out * c.n_in, "dtype": GEMM_DTYPE}
+
+    line["roofline"] = gemv_roofline(head, hc.name) if hc.m == 1 else gemm_roofline(head, hc.name)
+    if "q4_k_gemm_m512" in results and names[0] != "q4_k_gemm_m512":
         g = results["q4_k_gemm_m512"]
+        line["roofline_gemm"] = gemm_roofline(g, "q4_k_gemm_m512")
         line["gemm_m512_TFLOPs"] = g["TFLOPs"]
         line["gemm_m512_mfma_frac"] = g["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline()
     line["extra"] = {k: v for k, v in results.items() if k != names[0]}
     if not args.only and not args.no_extra:
-        line["extra"]["q4_k_gate_up_silu_gemv"] = run_gate_up(max(20, args.steps // 4), max(3, args.warmup // 4))
-        line["extra"]["widened"] = run_widened(max(20, args.steps // 4), max(3, args.warmup // 4))
+        line["extra"]["q4_k_gate_up_silu_gemv"] = run_gate_up(max(GRAPH_MIN_STEPS, args.steps // 4), max(3, args.warmup // 4))
+        line["extra"]["widened"] = run_widened(max(GRAPH_MIN_STEPS, args.steps // 4), max(3, args.warmup // 4))
         line["extra"]["dense_bf16_library_14336x4096"] = run_dense_reference(max(20, args.steps // 10),
                                                                              max(3, args.warmup // 10))
     print(json.dumps(line), flush=True)

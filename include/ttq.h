@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define TTQ_VERSION 100 /* 0.1.0 */
+#define TTQ_VERSION 110 /* 0.1.1 */
 
 /* Exported symbols: the library is built with hidden visibility by default. */
 #if defined(TTQ_BUILD)
@@ -50,7 +50,8 @@ typedef enum {
   TTQ_ERR_DTYPE = -4,       /* unknown or unsupported dtype code */
   TTQ_ERR_FORMAT = -5,      /* unknown format / bits / codebook */
   TTQ_ERR_UNSUPPORTED = -6, /* valid request outside what the kernels cover (size limits) */
-  TTQ_ERR_HIP = -7          /* a HIP runtime call failed; see ttq_last_hip_error() */
+  TTQ_ERR_HIP = -7,         /* a HIP runtime call failed; see ttq_last_hip_error() */
+  TTQ_ERR_ALIAS = -8        /* an output overlaps an input in a call that must run out of place */
 } ttq_status;
 
 /* Element types of activation / output / bias buffers.  They correspond to the
@@ -59,6 +60,12 @@ typedef enum {
 typedef enum { TTQ_F32 = 0, TTQ_F16 = 1, TTQ_BF16 = 2 } ttq_dtype;
 
 typedef enum { TTQ_Q8_0 = 0, TTQ_Q4_K = 1, TTQ_Q6_K = 2, TTQ_EXL3 = 3 } ttq_format;
+
+/* How ttq_linear_forward may trade accuracy for speed when there are several activation rows. */
+typedef enum {
+  TTQ_PRECISION_AUTO = 0,       /* from five rows on, whichever kernel the shape makes cheaper */
+  TTQ_PRECISION_F32_SCALES = 1  /* always the decode kernels: fp32 scales, rel-L2 <= 1e-3 whatever m is */
+} ttq_precision;
 
 /* Codebook functions of the trellis format. */
 typedef enum { TTQ_CB_3INST = 0, TTQ_CB_MCG = 1 } ttq_codebook;
@@ -85,6 +92,8 @@ typedef struct ttq_qlinear {
   int32_t bits;          /* TTQ_EXL3: bits per weight (1..8); otherwise ignored */
   int32_t codebook;      /* TTQ_EXL3: ttq_codebook; otherwise ignored */
   int32_t bias_dtype;    /* ttq_dtype of `bias`; ignored when bias is NULL */
+  int32_t precision;     /* ttq_precision */
+  int32_t reserved;      /* 0 */
   int64_t n_out;         /* out_features */
   int64_t n_in;          /* in_features */
   const void* qweight;   /* packed blocks (Q8_0/Q4_K/Q6_K) or trellis words (EXL3) */
@@ -101,13 +110,19 @@ typedef struct ttq_qlinear {
  * Accuracy: up to four rows always run the decode kernels (fp32 scales; rel-L2 <= 1e-3 against the
  * canonical dequantized weights).  From five rows of bf16 (fp16) activations on, the library may
  * run matrix-core kernels that round each dequantized weight once to bf16 (fp16) -- the 2e-2 class
- * of the GEMM entry points -- when its cost estimate prefers them for the shape. */
+ * of the GEMM entry points -- when its cost estimate prefers them for the shape.  A layer with
+ * precision == TTQ_PRECISION_F32_SCALES keeps the decode kernels, and with them the 1e-3 class,
+ * for every m.
+ * Limits (TTQ_ERR_UNSUPPORTED beyond): the decode kernels take n_in <= 32768 for Q4_K / Q6_K with
+ * 16-bit activations and n_in <= 16384 otherwise; any m (rows are taken 65535 at a time where a
+ * kernel needs that).  m == 0 or n_out == 0 returns TTQ_OK without touching a pointer. */
 TTQ_API int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int64_t m,
                        void* y, int y_dtype, void* stream);
 
 /* ---- decode GEMV, one entry per block format (m rows of x, normally m == 1) -------- */
 /* y[m][n_out] (fp32) = x[m][n_in] * W^T.  Stand in for F.linear(x, weight) with a
- * (1, n_in) activation (neural_nets.nim:64). */
+ * (1, n_in) activation (neural_nets.nim:64).  n_in <= 32768 for Q4_K / Q6_K with 16-bit
+ * activations, <= 16384 otherwise. */
 TTQ_API int ttq_gemv_q8_0(const void* w, const void* x, int x_dtype, float* y, int64_t m,
                   int64_t n_out, int64_t n_in, void* stream);
 TTQ_API int ttq_gemv_q4_k(const void* w, const void* x, int x_dtype, float* y, int64_t m,
@@ -188,7 +203,10 @@ TTQ_API int ttq_rmsnorm(const void* x, const void* residual, const void* gamma, 
  * GEMV.  With silu_mul != 0 the weight is the (2*n_out, n_in) gate/up matrix and y is
  * silu_and_mul of the projection (mlp.nim:56-59).  residual, new_residual_out and normed_out
  * may be NULL; normed_out receives the normalized row the GEMV consumed (other projections of
- * the same block read it).  Returns TTQ_ERR_UNSUPPORTED for fp32 activations or n_out < 16. */
+ * the same block read it).  Returns TTQ_ERR_UNSUPPORTED for fp32 activations or n_out < 16.
+ * Out of place only: every workgroup re-reads x and residual while the outputs are written, so
+ * new_residual_out and normed_out must not overlap x, residual or each other (TTQ_ERR_ALIAS);
+ * use ttq_rmsnorm for the in-place form. */
 TTQ_API int ttq_gemv_q4_k_rmsnorm(const void* w, const void* x, const void* residual, const void* gamma,
                           float eps, int x_dtype, void* new_residual_out, void* normed_out, void* y,
                           int y_dtype, int64_t m, int64_t n_out, int64_t n_in, int silu_mul, void* stream);

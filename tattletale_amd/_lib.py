@@ -13,10 +13,11 @@ LIB_PATH = os.path.join(HERE, "libttq_hip.so")
 
 # status / dtype / format codes (include/ttq.h)
 OK = 0
-ERR_NULL, ERR_SHAPE, ERR_ALIGN, ERR_DTYPE, ERR_FORMAT, ERR_UNSUPPORTED, ERR_HIP = -1, -2, -3, -4, -5, -6, -7
+ERR_NULL, ERR_SHAPE, ERR_ALIGN, ERR_DTYPE, ERR_FORMAT, ERR_UNSUPPORTED, ERR_HIP, ERR_ALIAS = -1, -2, -3, -4, -5, -6, -7, -8
 F32, F16, BF16 = 0, 1, 2
 Q8_0, Q4_K, Q6_K, EXL3 = 0, 1, 2, 3
 CB_3INST, CB_MCG = 0, 1
+PRECISION_AUTO, PRECISION_F32_SCALES = 0, 1
 
 
 class TtqLibraryError(RuntimeError):
@@ -31,6 +32,8 @@ class QLinearStruct(C.Structure):
         ("bits", C.c_int32),
         ("codebook", C.c_int32),
         ("bias_dtype", C.c_int32),
+        ("precision", C.c_int32),
+        ("reserved", C.c_int32),
         ("n_out", C.c_int64),
         ("n_in", C.c_int64),
         ("qweight", C.c_void_p),

@@ -14,6 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libttq_hip.so")
+LADDER_LIB = os.path.join(HERE, "libttq_ladder.so")      # bench.py's roofline ladder, not the product
 
 SOURCES = [
     "ttq_api.hip",
@@ -79,6 +80,15 @@ def build_library(force: bool = True, verbose: bool = False) -> str:
         raise RuntimeError("link failed:\n%s\n%s" % (r.stdout, r.stderr))
     if verbose:
         print("built", LIB)
+    # the measurement-only ladder kernels (bench.py --only ladder)
+    lobj = os.path.join(objdir, "ttq_ladder.hip.o")
+    _compile(os.path.join(CSRC, "ttq_ladder.hip"), lobj)
+    r = subprocess.run([hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LADDER_LIB, lobj],
+                       capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n%s\n%s" % (r.stdout, r.stderr))
+    if verbose:
+        print("built", LADDER_LIB)
     return LIB
 
 

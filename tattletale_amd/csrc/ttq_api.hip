@@ -51,12 +51,20 @@ int hip_status(hipError_t e) {
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+bool aligned8(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }
+int64_t dtype_size(int d) { return d == TTQ_F32 ? 4 : 2; }
+// do [a, a + an) and [b, b + bn) share a byte?  (null pointers never overlap anything)
+bool overlaps(const void* a, int64_t an, const void* b, int64_t bn) {
+  if (!a || !b || an <= 0 || bn <= 0) return false;
+  const uintptr_t pa = reinterpret_cast<uintptr_t>(a), pb = reinterpret_cast<uintptr_t>(b);
+  return pa < pb + (uintptr_t)bn && pb < pa + (uintptr_t)an;
+}
 bool valid_dtype(int d) { return d == TTQ_F32 || d == TTQ_F16 || d == TTQ_BF16; }
 
 // Shape rules of each format along n_in / n_out.
 int check_shape(int format, int64_t m, int64_t n_out, int64_t n_in, int bits, int cb) {
   if (m < 0 || n_out < 0 || n_in <= 0) return TTQ_ERR_SHAPE;
-  if (n_out > 0x7FFFFFFF || n_in > 0x7FFFFFFF || m > 65535) return TTQ_ERR_UNSUPPORTED;
+  if (n_out > 0x7FFFFFFF || n_in > 0x7FFFFFFF || m > 0x7FFFFFFF) return TTQ_ERR_UNSUPPORTED;
   switch (format) {
     case TTQ_Q8_0: return (n_in % 32 == 0) ? TTQ_OK : TTQ_ERR_SHAPE;
     case TTQ_Q4_K:
@@ -69,9 +77,29 @@ int check_shape(int format, int64_t m, int64_t n_out, int64_t n_in, int bits, in
   }
 }
 
-int check_gemv_limits(int x_dtype, int64_t n_in) {
-  const int64_t lim = (x_dtype == TTQ_F32) ? ttq::kMaxGemvInF32 : ttq::kMaxGemvInF32;
+// Longest row the decode kernels take: the packed-dot kernel (Q4_K / Q6_K, 16-bit activations)
+// stages 32768 activations in 64 KiB of LDS, everything else 16384.
+int check_gemv_limits(int format, int x_dtype, int64_t n_in) {
+  const bool long_rows = (format == TTQ_Q4_K || format == TTQ_Q6_K) && (x_dtype == TTQ_F16 || x_dtype == TTQ_BF16);
+  const int64_t lim = long_rows ? ttq::kMaxGemvIn16 : ttq::kMaxGemvInF32;
   return n_in <= lim ? TTQ_OK : TTQ_ERR_UNSUPPORTED;
+}
+
+// launch_gemv puts the activation rows (or passes over them) on gridDim.y, which ends at 65535
+hipError_t launch_gemv_any_m(int format, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                             const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                             hipStream_t s) {
+  constexpr int64_t kChunk = 65520;   // a multiple of the 4, 8 and 16 rows the few-row kernels take per pass
+  const char* xb = static_cast<const char*>(x);
+  char* yb = static_cast<char*>(y);
+  for (int64_t r = 0; r < m; r += kChunk) {
+    const int64_t rows = m - r < kChunk ? m - r : kChunk;
+    const hipError_t e = ttq::launch_gemv(format, w, xb + r * n_in * dtype_size(x_dtype), x_dtype,
+                                          yb + r * n_out * dtype_size(y_dtype), y_dtype, bias, bias_dtype, rows,
+                                          n_out, n_in, s);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
 }
 
 int gemv_block(int format, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
@@ -84,10 +112,10 @@ int gemv_block(int format, const void* w, const void* x, int x_dtype, void* y, i
   if (m == 0 || n_out == 0) return TTQ_OK;  // empty output: nothing to read or write
   if (!w || !x || !y) return TTQ_ERR_NULL;
   if (!aligned16(w) || !aligned16(x) || !aligned16(y)) return TTQ_ERR_ALIGN;
-  rc = check_gemv_limits(x_dtype, n_in);
+  rc = check_gemv_limits(format, x_dtype, n_in);
   if (rc != TTQ_OK) return rc;
-  return hip_status(ttq::launch_gemv(format, w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out,
-                                     n_in, static_cast<hipStream_t>(stream)));
+  return hip_status(launch_gemv_any_m(format, w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in,
+                                      static_cast<hipStream_t>(stream)));
 }
 
 int dequant_block(int format, const void* w, void* out, int out_dtype, int64_t n_out, int64_t n_in,
@@ -118,6 +146,7 @@ const char* ttq_strerror(int status) {
     case TTQ_ERR_FORMAT: return "unknown format, bit width or codebook";
     case TTQ_ERR_UNSUPPORTED: return "request outside the supported size limits";
     case TTQ_ERR_HIP: return "HIP runtime error (see ttq_last_hip_error)";
+    case TTQ_ERR_ALIAS: return "output buffer overlaps an input where that is not allowed";
     default: return "unknown status";
   }
 }
@@ -152,10 +181,12 @@ int ttq_gemv_q6_k(const void* w, const void* x, int x_dtype, float* y, int64_t m
 int ttq_gemv_exl3(const uint16_t* trellis, const uint16_t* suh_f16, const uint16_t* svh_f16,
                   const uint16_t* x_f16, float* y, int64_t m, int64_t n_out, int64_t n_in, int bits,
                   int codebook, void* stream) {
-  if (!trellis || !suh_f16 || !svh_f16 || !x_f16 || !y) return TTQ_ERR_NULL;
   const int rc = check_shape(TTQ_EXL3, m, n_out, n_in, bits, codebook);
   if (rc != TTQ_OK) return rc;
-  if (!aligned16(trellis) || !aligned16(x_f16) || !aligned16(y)) return TTQ_ERR_ALIGN;
+  if (m == 0 || n_out == 0) return TTQ_OK;
+  if (!trellis || !suh_f16 || !svh_f16 || !x_f16 || !y) return TTQ_ERR_NULL;
+  if (!aligned16(trellis) || !aligned16(x_f16) || !aligned16(y) || !aligned8(suh_f16) || !aligned8(svh_f16))
+    return TTQ_ERR_ALIGN;
   if (n_in > ttq::kMaxGemvInF32) return TTQ_ERR_UNSUPPORTED;
   return hip_status(ttq::launch_gemv_exl3(trellis, suh_f16, svh_f16, x_f16, TTQ_F16, y, TTQ_F32,
                                           nullptr, 0, m, n_out, n_in, bits, codebook,
@@ -210,30 +241,29 @@ int ttq_gemv_q4_k_rmsnorm(const void* w, const void* x, const void* residual, co
   if (!aligned16(w) || !aligned16(x) || !aligned16(gamma) || !aligned16(y) || (residual && !aligned16(residual)) ||
       (new_residual_out && !aligned16(new_residual_out)) || (normed_out && !aligned16(normed_out)))
     return TTQ_ERR_ALIGN;
+  // every workgroup re-reads x and residual while workgroup 0 writes the two outputs: in-place use
+  // (allowed for ttq_rmsnorm) would race here
+  {
+    const int64_t nb = m * n_in * dtype_size(x_dtype);
+    if (overlaps(new_residual_out, nb, x, nb) || overlaps(new_residual_out, nb, residual, nb) ||
+        overlaps(normed_out, nb, x, nb) || overlaps(normed_out, nb, residual, nb) ||
+        overlaps(normed_out, nb, new_residual_out, nb))
+      return TTQ_ERR_ALIAS;
+  }
   if (!ttq::gemv_fused_supported(TTQ_Q4_K, x_dtype, n_out, n_in, silu_mul != 0)) return TTQ_ERR_UNSUPPORTED;
   return hip_status(ttq::launch_gemv_fused(w, x, x_dtype, y, y_dtype, nullptr, 0, m, n_out, n_in, silu_mul != 0,
                                            residual, gamma, eps, new_residual_out, normed_out,
                                            static_cast<hipStream_t>(stream)));
 }
 
-int ttq_gemm_q4_k(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m, int64_t n_out,
-                  int64_t n_in, void* stream) {
-  if (!w || !x_bf16 || !y_bf16) return TTQ_ERR_NULL;
-  const int rc = check_shape(TTQ_Q4_K, m, n_out, n_in, 0, 0);
-  if (rc != TTQ_OK) return rc;
-  if (!aligned16(w) || !aligned16(x_bf16) || !aligned16(y_bf16)) return TTQ_ERR_ALIGN;
-  return hip_status(ttq::launch_gemm(TTQ_Q4_K, w, x_bf16, y_bf16, TTQ_BF16, nullptr, 0, m, n_out, n_in,
-                                     static_cast<hipStream_t>(stream)));
-}
-
 int ttq_gemm_q4_k_silu_mul(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m, int64_t n_ff,
                            int64_t n_in, void* stream) {
-  if (!w || !x_bf16 || !y_bf16) return TTQ_ERR_NULL;
   const int rc = check_shape(TTQ_Q4_K, m, n_ff, n_in, 0, 0);
   if (rc != TTQ_OK) return rc;
   if (n_ff > 0x3FFFFFFF) return TTQ_ERR_UNSUPPORTED;
-  if (!aligned16(w) || !aligned16(x_bf16) || !aligned16(y_bf16)) return TTQ_ERR_ALIGN;
   if (m == 0 || n_ff == 0) return TTQ_OK;
+  if (!w || !x_bf16 || !y_bf16) return TTQ_ERR_NULL;
+  if (!aligned16(w) || !aligned16(x_bf16) || !aligned16(y_bf16)) return TTQ_ERR_ALIGN;
   // up to 64 rows: the few-row kernel where it is estimated to be faster than the tiled one
   const bool pc_ok = ttq::gemm_pc_supported(TTQ_Q4_K, m, 2 * n_ff, n_in, 112);
   if (ttq::gemm_skinny_silu_mul_supported(m, n_ff, n_in) &&
@@ -248,14 +278,18 @@ int ttq_gemm_q4_k_silu_mul(const void* w, const uint16_t* x_bf16, uint16_t* y_bf
 
 static int gemm_block(int format, const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m,
                       int64_t n_out, int64_t n_in, void* stream) {
-  if (!w || !x_bf16 || !y_bf16) return TTQ_ERR_NULL;
   const int rc = check_shape(format, m, n_out, n_in, 0, 0);
   if (rc != TTQ_OK) return rc;
+  if (m == 0 || n_out == 0) return TTQ_OK;    // empty output: nothing to read or write
+  if (!w || !x_bf16 || !y_bf16) return TTQ_ERR_NULL;
   if (!aligned16(w) || !aligned16(x_bf16) || !aligned16(y_bf16)) return TTQ_ERR_ALIGN;
-  if (m == 0 || n_out == 0) return TTQ_OK;
   if (!ttq::gemm_supported(format, m, n_out, n_in)) return TTQ_ERR_UNSUPPORTED;
   return hip_status(ttq::launch_gemm(format, w, x_bf16, y_bf16, TTQ_BF16, nullptr, 0, m, n_out, n_in,
                                      static_cast<hipStream_t>(stream)));
+}
+int ttq_gemm_q4_k(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m, int64_t n_out,
+                  int64_t n_in, void* stream) {
+  return gemm_block(TTQ_Q4_K, w, x_bf16, y_bf16, m, n_out, n_in, stream);
 }
 int ttq_gemm_q6_k(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m, int64_t n_out,
                   int64_t n_in, void* stream) {
@@ -296,17 +330,21 @@ int ttq_hadamard128_f32(float* v, const uint16_t* pre_f16, const uint16_t* post_
 
 int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int64_t m, void* y,
                        int y_dtype, void* stream) {
-  if (!layer || !x || !y || !layer->qweight) return TTQ_ERR_NULL;
+  if (!layer) return TTQ_ERR_NULL;
   if (!valid_dtype(x_dtype) || !valid_dtype(y_dtype)) return TTQ_ERR_DTYPE;
   if (layer->bias && !valid_dtype(layer->bias_dtype)) return TTQ_ERR_DTYPE;
+  if (layer->precision != TTQ_PRECISION_AUTO && layer->precision != TTQ_PRECISION_F32_SCALES) return TTQ_ERR_FORMAT;
   const int rc = check_shape(layer->format, m, layer->n_out, layer->n_in, layer->bits, layer->codebook);
   if (rc != TTQ_OK) return rc;
+  if (m == 0 || layer->n_out == 0) return TTQ_OK;   // an empty batch gives an empty output, as F.linear does
+  if (!x || !y || !layer->qweight) return TTQ_ERR_NULL;
   if (!aligned16(layer->qweight) || !aligned16(x) || !aligned16(y)) return TTQ_ERR_ALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t n_out = layer->n_out, n_in = layer->n_in;
 
   if (layer->format == TTQ_EXL3) {
     if (!layer->suh || !layer->svh) return TTQ_ERR_NULL;
+    if (!aligned8(layer->suh) || !aligned8(layer->svh)) return TTQ_ERR_ALIGN;
     if (y_dtype != TTQ_F32) return TTQ_ERR_UNSUPPORTED;  // output rotation runs in place on fp32
     if (n_in > ttq::kMaxGemvInF32) return TTQ_ERR_UNSUPPORTED;
     return hip_status(ttq::launch_gemv_exl3(
@@ -321,10 +359,11 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
   const bool gemm_ok = x_dtype == TTQ_BF16 && (y_dtype == TTQ_BF16 || y_dtype == TTQ_F32) &&
                        (layer->format == TTQ_Q4_K || layer->format == TTQ_Q6_K || layer->format == TTQ_Q8_0) &&
                        ttq::gemm_supported(layer->format, m, n_out, n_in);
-  // TTQ_FORWARD_ROUTE (for A/B measurements): 1 = always the decode kernels, 2 = the GEMM whenever it exists
-  static const int route = [] { const char* e = getenv("TTQ_FORWARD_ROUTE"); return e ? atoi(e) : 0; }();
+  // TTQ_FORWARD_ROUTE (developer builds, A/B measurements): 1 = always the decode kernels, 2 = the GEMM whenever it exists
+  static const int knob = ttq::dev_knob("TTQ_FORWARD_ROUTE", 0);
+  const int route = layer->precision == TTQ_PRECISION_F32_SCALES ? 1 : knob;
   if (gemm_ok && m >= 5 && route != 1) {
-    const bool gemv_ok = check_gemv_limits(x_dtype, n_in) == TTQ_OK;
+    const bool gemv_ok = check_gemv_limits(layer->format, x_dtype, n_in) == TTQ_OK;
     if (!gemv_ok || route == 2 ||
         ttq::gemm_estimate_us(layer->format, m, n_out, n_in) < ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in))
       return hip_status(ttq::launch_gemm(layer->format, layer->qweight, static_cast<const uint16_t*>(x), y, y_dtype,
@@ -337,16 +376,16 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
     const int64_t full = m / 64, rest = m % 64;
     float us = (float)full * ttq::gemm_skinny_estimate_us(layer->format, 64, n_out, n_in);
     if (rest) us += ttq::gemm_skinny_estimate_us(layer->format, rest, n_out, n_in);
-    const bool gemv_ok = check_gemv_limits(x_dtype, n_in) == TTQ_OK;
+    const bool gemv_ok = check_gemv_limits(layer->format, x_dtype, n_in) == TTQ_OK;
     if (!gemv_ok || route == 2 || us < ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in))
       return hip_status(ttq::launch_gemm_skinny_chunked(layer->format, layer->qweight, static_cast<const uint16_t*>(x),
                                                         x_dtype, y, y_dtype, layer->bias, layer->bias_dtype, m, n_out,
                                                         n_in, s));
   }
-  const int lim = check_gemv_limits(x_dtype, n_in);
+  const int lim = check_gemv_limits(layer->format, x_dtype, n_in);
   if (lim != TTQ_OK) return lim;
-  return hip_status(ttq::launch_gemv(layer->format, layer->qweight, x, x_dtype, y, y_dtype, layer->bias,
-                                     layer->bias_dtype, m, n_out, n_in, s));
+  return hip_status(launch_gemv_any_m(layer->format, layer->qweight, x, x_dtype, y, y_dtype, layer->bias,
+                                      layer->bias_dtype, m, n_out, n_in, s));
 }
 
 }  // extern "C"

@@ -404,7 +404,6 @@ hipError_t launch_gemv_exl3(const uint16_t* trellis, const uint16_t* suh, const 
                             hipStream_t s) {
   if (m == 0 || n_out == 0) return hipSuccess;
   if (y_dtype != kF32) return hipErrorInvalidValue;
-  if (n_in > 16000) return hipErrorInvalidValue;  // activations + partials must fit 64 KiB of LDS
   float* yf = static_cast<float*>(y);
   hipError_t e;
   switch (bits) {

@@ -603,7 +603,7 @@ static const PcTile kPcTiles[] = {{4, 7, 0.87f}, {4, 4, 0.68f}, {2, 7, 0.585f}, 
 constexpr float kPcFixedUs = 6.f;
 
 static int pc_choose_tile(int64_t m, int64_t n_out, int64_t n_in, bool fuse, float* cost_us = nullptr) {
-  static const int forced = [] { const char* e = getenv("TTQ_GEMM_TILE"); return e ? atoi(e) : -1; }();
+  static const int forced = dev_knob("TTQ_GEMM_TILE", -1);
   const int cus = device_num_cus();
   int best = 0;
   float best_cost = 1e30f;
@@ -645,7 +645,7 @@ static hipError_t launch_pc_fmt(const uint8_t* wb, const uint16_t* x, void* y, i
 // accumulator registers plus the fragment rings do not fit the 168 registers a wavefront gets
 // when twelve of them share a CU.
 bool gemm_pc_supported(int format, int64_t m, int64_t n_out, int64_t n_in, int bn) {
-  static const int disabled = [] { const char* e = getenv("TTQ_GEMM_NO_PC"); return e ? atoi(e) : 0; }();
+  static const int disabled = dev_knob("TTQ_GEMM_NO_PC", 0);
   // activation byte offsets are 32-bit in the kernel; a step loop iteration is 256 k
   return !disabled && (format == kQ4_K || format == kQ6_K || format == kQ8_0) && bn == 112 &&
          m * n_in * 2 < ((int64_t)1 << 32) && n_out > 0 && n_in > 0 && n_in % 256 == 0;

@@ -362,10 +362,7 @@ gemm_q4k_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, Y
   }
 }
 
-static int env_flag(const char* name, int dflt) {
-  const char* e = getenv(name);
-  return e ? atoi(e) : dflt;
-}
+static int env_flag(const char* name, int dflt) { return dev_knob(name, dflt); }
 
 template <int NJ, typename YT>
 static hipError_t launch_nj_y(const uint8_t* wb, const uint16_t* x, YT* y, const void* bias, int bias_dtype,
@@ -433,7 +430,7 @@ hipError_t launch_gemm(int format, const void* w, const uint16_t* x_bf16, void* 
   const int64_t cus = device_num_cus();
   const int64_t mt = (m + kGemmBM - 1) / kGemmBM;
   auto cost = [&](int64_t bn) { return ((((n_out + bn - 1) / bn) * mt + cus - 1) / cus) * bn; };
-  static const int forced = [] { const char* e = getenv("TTQ_GEMM_BN"); return e ? atoi(e) : 0; }();
+  static const int forced = dev_knob("TTQ_GEMM_BN", 0);
   const bool use112 = forced ? forced == 112 : cost(112) < cost(128);
   // the producer/consumer kernel (ttq_gemm_pc.hip) exists for the 112-column tile
   if (gemm_pc_supported(kQ4_K, m, n_out, n_in, use112 ? 112 : 128))

@@ -525,7 +525,7 @@ float skinny_cost_us(int format, int rb, int64_t m, int64_t n_out, int64_t n_in)
 
 // rows = weight rows (twice the outputs when fused, which also rules out single row blocks)
 int skinny_choose_rb(int format, int64_t m, int64_t rows, int64_t n_in, bool fuse, float* cost_us = nullptr) {
-  static const int forced_rb = [] { const char* e = getenv("TTQ_SK_RB"); return e ? atoi(e) : 0; }();
+  static const int forced_rb = dev_knob("TTQ_SK_RB", 0);
   int best = 4;
   float best_cost = 1e30f;
   for (int rb = 4; rb >= (fuse ? 2 : 1); rb >>= 1) {
@@ -559,7 +559,7 @@ hipError_t launch_skinny_fmt(int format, const uint8_t* wb, const uint16_t* x_bf
 }  // namespace
 
 bool gemm_skinny_supported(int format, int64_t m, int64_t n_out, int64_t n_in) {
-  static const int disabled = [] { const char* e = getenv("TTQ_GEMM_NO_SKINNY"); return e ? atoi(e) : 0; }();
+  static const int disabled = dev_knob("TTQ_GEMM_NO_SKINNY", 0);
   const int64_t block_bytes = format == kQ4_K ? 144 : (format == kQ6_K ? 210 : 272);
   // weight byte offsets and activation element offsets are 32-bit in the kernel; outputs are stored
   // eight at a time

@@ -265,8 +265,7 @@ gemv_generic_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, YT*
 static int gemv_grid(int64_t n_out, int default_per_cu) {
   static int per_cu_env = -1;
   if (per_cu_env < 0) {
-    const char* e = getenv("TTQ_GEMV_WG_PER_CU");
-    per_cu_env = e ? atoi(e) : 0;
+    per_cu_env = dev_knob("TTQ_GEMV_WG_PER_CU", 0);
   }
   const int per_cu = per_cu_env > 0 ? per_cu_env : default_per_cu;
   const int cus = device_num_cus();
@@ -327,7 +326,7 @@ hipError_t launch_gemv(int format, const void* w, const void* x, int x_dtype, vo
   if (m == 0 || n_out == 0) return hipSuccess;
   // a few rows at once: four per pass for up to four rows and for rows too long for the 8- and
   // 16-token tables, else eight or sixteen per pass
-  static const int batch4_max = [] { const char* e = getenv("TTQ_GEMV_BATCH4_MAX_ROWS"); return e ? atoi(e) : 4; }();
+  static const int batch4_max = dev_knob("TTQ_GEMV_BATCH4_MAX_ROWS", 4);
   const bool b4 = gemv_q4k_batch4_supported(format, x_dtype, m, n_out, n_in);
   if (b4 && m <= batch4_max)
     return launch_gemv_q4k_batch4(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);

@@ -660,10 +660,7 @@ gemv_dot2_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
 }
 
 // ------------------------------------------------------------------------------ launch
-static int env_int(const char* name, int dflt) {
-  const char* e = getenv(name);
-  return e ? atoi(e) : dflt;
-}
+static int env_int(const char* name, int dflt) { return dev_knob(name, dflt); }
 
 template <class F, class Ops, typename YT>
 static hipError_t launch_fmt_t(const void* w, const void* x, void* y, const void* bias, int bias_dtype,

@@ -70,9 +70,6 @@ __device__ __forceinline__ uint32_t pack_low_bytes(int a, int b, int c, int d) {
   return p01 | (p23 << 16);
 }
 
-inline int mfma_env_int(const char* name, int dflt) {
-  const char* e = getenv(name);
-  return e ? atoi(e) : dflt;
-}
+inline int mfma_env_int(const char* name, int dflt) { return dev_knob(name, dflt); }
 
 }  // namespace ttq

@@ -6,9 +6,24 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <stdlib.h>
+
 #include <atomic>
 
 namespace ttq {
+
+// Developer A/B switches.  They are read from the environment only in builds made with
+// -DTTQ_DEV_KNOBS; the product build (tattletale_amd/build.py) leaves that off, so what the library
+// does never depends on the process environment.
+inline int dev_knob(const char* name, int dflt) {
+#ifdef TTQ_DEV_KNOBS
+  const char* e = getenv(name);
+  return e ? atoi(e) : dflt;
+#else
+  (void)name;
+  return dflt;
+#endif
+}
 
 // dtype codes as in ttq.h (TTQ_F32 = 0, TTQ_F16 = 1, TTQ_BF16 = 2)
 enum : int { kF32 = 0, kF16 = 1, kBF16 = 2 };

@@ -17,8 +17,11 @@ type
     kQ8_0 = 0, kQ4_K = 1, kQ6_K = 2, kEXL3 = 3
   TtqDtype* {.size: sizeof(cint).} = enum
     kTtqF32 = 0, kTtqF16 = 1, kTtqBF16 = 2
+  TtqPrecision* {.size: sizeof(cint).} = enum
+    kTtqAuto = 0, kTtqF32Scales = 1    ## kTtqF32Scales: decode kernels (fp32 scales) for every batch size
   TtqQLinear* {.bycopy.} = object      ## struct ttq_qlinear
     format*, bits*, codebook*, bias_dtype*: int32
+    precision*, reserved*: int32       ## ttq_precision, 0
     n_out*, n_in*: int64
     qweight*, suh*, svh*, bias*: pointer
   QuantLinearError* = object of ValueError
@@ -41,6 +44,7 @@ proc dequant_q8_0*(w, dst: pointer, out_dtype: cint, n_out, n_in: int64, stream:
 proc dequant_q4_k*(w, dst: pointer, out_dtype: cint, n_out, n_in: int64, stream: pointer): cint {.ttq.}
 proc dequant_q6_k*(w, dst: pointer, out_dtype: cint, n_out, n_in: int64, stream: pointer): cint {.ttq.}
 proc dequant_exl3*(trellis, dst: ptr uint16, n_out, n_in: int64, bits, codebook: cint, stream: pointer): cint {.ttq.}
+proc hadamard128_f32*(v: ptr cfloat, pre_f16, post_f16: ptr uint16, n: int64, stream: pointer): cint {.ttq.}
 proc silu_and_mul*(src, dst: pointer, dtype: cint, m, h: int64, stream: pointer): cint {.ttq.}
 proc gemm_q4_k_silu_mul*(w: pointer, x, y: ptr uint16, m, n_ff, n_in: int64, stream: pointer): cint {.ttq.}
 proc gemv_q4_k_silu_mul*(w, x: pointer, x_dtype: cint, y: pointer, y_dtype: cint, m, n_ff, n_in: int64,
@@ -50,6 +54,22 @@ proc rmsnorm*(x, residual, gamma: pointer, eps: cfloat, dtype: cint, new_residua
 proc gemv_q4_k_rmsnorm*(w, x, residual, gamma: pointer, eps: cfloat, x_dtype: cint,
                         new_residual_out, normed_out, y: pointer, y_dtype: cint, m, n_out, n_in: int64,
                         silu_mul: cint, stream: pointer): cint {.ttq.}
+# host-side preparation (CPU code)
+proc host_fill_normal*(seed, stream: uint64, sigma: cfloat, dst: ptr cfloat, n: int64): cint {.ttq.}
+proc host_quantize_q8_0*(w: ptr cfloat, dst: pointer, n_out, n_in: int64): cint {.ttq.}
+proc host_quantize_q4_k*(w: ptr cfloat, dst: pointer, n_out, n_in: int64): cint {.ttq.}
+proc host_quantize_q6_k*(w: ptr cfloat, dst: pointer, n_out, n_in: int64): cint {.ttq.}
+proc host_quantize_exl3*(w: ptr cfloat, trellis, suh_f16, svh_f16: ptr uint16, n_out, n_in: int64,
+                         bits, codebook: cint, seed: uint64): cint {.ttq.}
+proc host_f32_to_bf16*(src: ptr cfloat, dst: ptr uint16, n: int64): cint {.ttq.}
+proc host_f32_to_f16*(src: ptr cfloat, dst: ptr uint16, n: int64): cint {.ttq.}
+proc host_bf16_to_f32*(src: ptr uint16, dst: ptr cfloat, n: int64): cint {.ttq.}
+proc host_f16_to_f32*(src: ptr uint16, dst: ptr cfloat, n: int64): cint {.ttq.}
+
+# The stream torch's own kernels of this thread run on, so that a layer keeps its place in the
+# caller's stream order (a ROCm build of libtorch names its HIP streams c10::cuda as well).
+proc currentStream*(): pointer {.importcpp: "((void*)c10::cuda::getCurrentCUDAStream().stream())",
+                                 header: "<c10/cuda/CUDAStream.h>".}
 
 func ttqDtype(k: ScalarKind): cint =
   case k
@@ -67,20 +87,22 @@ type
     suh*, svh*: Option[TorchTensor] ## EXL3 only, kFloat16
     bits*, codebook*: int
     in_features*, out_features*: int
+    precision*: TtqPrecision
 
 func init*(_: type QuantLinear, qweight: TorchTensor, format: QuantFormat,
            in_features, out_features: int, bias = none(TorchTensor),
            suh = none(TorchTensor), svh = none(TorchTensor),
-           bits = 0, codebook = 1): QuantLinear =
+           bits = 0, codebook = 1, precision = kTtqAuto): QuantLinear =
   ## Creates the layer from existing packed weights (no copy), as Linear.init does.
   let need = packed_nbytes(format.cint, out_features, in_features, bits.cint)
   if need < 0 or need != qweight.nbytes.int64:
     raise newException(QuantLinearError, "packed buffer size does not match the dimensions")
   QuantLinear(qweight: qweight, format: format, bias: bias, suh: suh, svh: svh, bits: bits,
-              codebook: codebook, in_features: in_features, out_features: out_features)
+              codebook: codebook, in_features: in_features, out_features: out_features,
+              precision: precision)
 
 proc forward*(self: QuantLinear, x: TorchTensor): TorchTensor =
-  ## x: (..., in_features) -> (..., out_features); launches on the current stream.
+  ## x: (..., in_features) -> (..., out_features); launches on torch's current stream.
   var shape = x.sizes().asNimView().toSeq()      # (..., in) -> (..., out)
   shape[^1] = self.out_features
   let m = x.numel() div self.in_features
@@ -89,13 +111,14 @@ proc forward*(self: QuantLinear, x: TorchTensor): TorchTensor =
   var desc = TtqQLinear(
     format: self.format.int32, bits: self.bits.int32, codebook: self.codebook.int32,
     bias_dtype: (if self.bias.isSome: ttqDtype(self.bias.get().scalarType()).int32 else: 0),
+    precision: self.precision.int32, reserved: 0,
     n_out: self.out_features, n_in: self.in_features,
     qweight: self.qweight.data_ptr(byte),
     suh: (if self.suh.isSome: self.suh.get().data_ptr(byte) else: nil),
     svh: (if self.svh.isSome: self.svh.get().data_ptr(byte) else: nil),
     bias: (if self.bias.isSome: self.bias.get().data_ptr(byte) else: nil))
   let rc = linear_forward(addr desc, x.data_ptr(byte), ttqDtype(x.scalarType()), m,
-                          result.data_ptr(byte), ttqDtype(outKind), nil)
+                          result.data_ptr(byte), ttqDtype(outKind), currentStream())
   if rc != 0:
     raise newException(QuantLinearError, "ttq_linear_forward: " & $strerror(rc))
   if outKind != x.scalarType(): result = result.to(x.scalarType())
@@ -129,7 +152,7 @@ proc quant_silu_and_mul*(x: TorchTensor): TorchTensor =
   shape[^1] = h
   result = F.empty(shape, x.options())
   let rc = silu_and_mul(x.data_ptr(byte), result.data_ptr(byte), ttqDtype(x.scalarType()),
-                        x.numel() div (2 * h), h, nil)
+                        x.numel() div (2 * h), h, currentStream())
   if rc != 0: raise newException(QuantLinearError, "ttq_silu_and_mul: " & $strerror(rc))
 
 proc forward*(self: QuantGatedMLP, x: TorchTensor): TorchTensor =
@@ -142,7 +165,7 @@ proc forward*(self: QuantGatedMLP, x: TorchTensor): TorchTensor =
     shape[^1] = nff
     let act = F.empty(shape, x.options())
     let rc = gemv_q4_k_silu_mul(gu.qweight.data_ptr(byte), x.data_ptr(byte), ttqDtype(x.scalarType()),
-                                act.data_ptr(byte), ttqDtype(x.scalarType()), m, nff, gu.in_features, nil)
+                                act.data_ptr(byte), ttqDtype(x.scalarType()), m, nff, gu.in_features, currentStream())
     if rc == 0: return self.down_proj.forward(act)
     if rc != kTtqErrUnsupported:
       raise newException(QuantLinearError, "ttq_gemv_q4_k_silu_mul: " & $strerror(rc))
@@ -154,7 +177,7 @@ proc forward*(self: QuantGatedMLP, x: TorchTensor): TorchTensor =
     shape[^1] = nff
     let act = F.empty(shape, x.options())
     let rc = gemm_q4_k_silu_mul(gu.qweight.data_ptr(byte), cast[ptr uint16](x.data_ptr(byte)),
-                                cast[ptr uint16](act.data_ptr(byte)), m, nff, gu.in_features, nil)
+                                cast[ptr uint16](act.data_ptr(byte)), m, nff, gu.in_features, currentStream())
     if rc == 0: return self.down_proj.forward(act)
     if rc != kTtqErrUnsupported:
       raise newException(QuantLinearError, "ttq_gemm_q4_k_silu_mul: " & $strerror(rc))
@@ -178,7 +201,7 @@ proc forward_with_residual*(self: QuantRmsNorm, hidden_state, residual: TorchTen
   let new_residual = F.empty(hidden_state.sizes(), hidden_state.options())
   let rc = rmsnorm(hidden_state.data_ptr(byte), residual.data_ptr(byte), self.weight.data_ptr(byte),
                    self.eps.cfloat, ttqDtype(hidden_state.scalarType()), new_residual.data_ptr(byte),
-                   normalized.data_ptr(byte), hidden_state.numel() div self.hidden_size, self.hidden_size, nil)
+                   normalized.data_ptr(byte), hidden_state.numel() div self.hidden_size, self.hidden_size, currentStream())
   if rc != 0: raise newException(QuantLinearError, "ttq_rmsnorm: " & $strerror(rc))
   (normalized, new_residual)
 
@@ -196,6 +219,6 @@ proc forward_norm_gate_up*(norm: QuantRmsNorm, mlp: QuantGatedMLP,
                              norm.weight.data_ptr(byte), norm.eps.cfloat, ttqDtype(hidden_state.scalarType()),
                              new_residual.data_ptr(byte), nil, act.data_ptr(byte),
                              ttqDtype(hidden_state.scalarType()), hidden_state.numel() div gu.in_features,
-                             nff, gu.in_features, 1, nil)
+                             nff, gu.in_features, 1, currentStream())
   if rc != 0: raise newException(QuantLinearError, "ttq_gemv_q4_k_rmsnorm: " & $strerror(rc))
   (mlp.down_proj.forward(act), new_residual)

@@ -69,12 +69,13 @@ class QuantLinear:
     svh: Optional[torch.Tensor] = None    # EXL3: (out_features,) float16
     bits: int = 0
     codebook: int = _lib.CB_MCG
+    precision: int = _lib.PRECISION_AUTO  # PRECISION_F32_SCALES keeps the decode kernels for every batch
 
     @classmethod
     def init(cls, qweight: torch.Tensor, format: int, in_features: int, out_features: int,
              bias: Optional[torch.Tensor] = None, suh: Optional[torch.Tensor] = None,
              svh: Optional[torch.Tensor] = None, bits: int = 0,
-             codebook: int = _lib.CB_MCG) -> "QuantLinear":
+             codebook: int = _lib.CB_MCG, precision: int = _lib.PRECISION_AUTO) -> "QuantLinear":
         """Creates the layer from existing packed weights (no copy, no repacking), as
         ``Linear.init`` does from a dense weight (linear.nim:29-43)."""
         _require_device(qweight, bias, suh, svh)
@@ -94,12 +95,13 @@ class QuantLinear:
                 raise TtqError(_lib.ERR_DTYPE, "QuantLinear.init: suh/svh must be float16")
             if suh.numel() != in_features or svh.numel() != out_features:
                 raise TtqError(_lib.ERR_SHAPE, "QuantLinear.init: suh/svh length")
-        return cls(qweight, format, in_features, out_features, bias, suh, svh, bits, codebook)
+        return cls(qweight, format, in_features, out_features, bias, suh, svh, bits, codebook, precision)
 
     def _struct(self) -> QLinearStruct:
         return QLinearStruct(
             format=self.format, bits=self.bits, codebook=self.codebook,
             bias_dtype=_code(self.bias.dtype) if self.bias is not None else 0,
+            precision=self.precision, reserved=0,
             n_out=self.out_features, n_in=self.in_features,
             qweight=_ptr(self.qweight), suh=_ptr(self.suh), svh=_ptr(self.svh), bias=_ptr(self.bias))
 
@@ -127,6 +129,35 @@ class QuantLinear:
 
 
 # ------------------------------------------------------------------------- functional API
+def _nbytes(t: torch.Tensor) -> int:
+    return t.numel() * t.element_size()
+
+
+def _check_packed(what: str, qweight: torch.Tensor, fmt: int, n_out: int, n_in: int, bits: int = 0) -> None:
+    """The packed buffer must hold exactly the (n_out, n_in) matrix the kernels will index."""
+    need = _lib.lib().ttq_packed_nbytes(fmt, n_out, n_in, bits)
+    if need < 0:
+        raise TtqError(int(need), what)
+    if need and _nbytes(qweight) != need:     # an empty matrix reads nothing, whatever stands in for it
+        raise TtqError(_lib.ERR_SHAPE, "%s: packed buffer holds %d bytes, %d expected for (%d, %d)"
+                       % (what, _nbytes(qweight), need, n_out, n_in))
+
+
+def _rows(what: str, x: torch.Tensor, n_in: int) -> int:
+    if x.dim() == 0 or x.shape[-1] != n_in:
+        raise TtqError(_lib.ERR_SHAPE, "%s: last dim of x is %s, n_in is %d"
+                       % (what, x.shape[-1] if x.dim() else "missing", n_in))
+    return x.numel() // n_in
+
+
+def _check_out(what: str, out: torch.Tensor, m: int, n_out: int, dtype: torch.dtype) -> None:
+    if out.dtype != dtype:
+        raise TtqError(_lib.ERR_DTYPE, "%s: out is %s, %s expected" % (what, out.dtype, dtype))
+    if out.numel() != m * n_out or (out.dim() > 0 and n_out and out.shape[-1] != n_out):
+        raise TtqError(_lib.ERR_SHAPE, "%s: out has shape %s, (%d, %d) expected"
+                       % (what, tuple(out.shape), m, n_out))
+
+
 _GEMV = {_lib.Q8_0: "ttq_gemv_q8_0", _lib.Q4_K: "ttq_gemv_q4_k", _lib.Q6_K: "ttq_gemv_q6_k"}
 _DEQ = {_lib.Q8_0: "ttq_dequant_q8_0", _lib.Q4_K: "ttq_dequant_q4_k", _lib.Q6_K: "ttq_dequant_q6_k"}
 
@@ -134,10 +165,15 @@ _DEQ = {_lib.Q8_0: "ttq_dequant_q8_0", _lib.Q4_K: "ttq_dequant_q4_k", _lib.Q6_K:
 def gemv(fmt: int, qweight: torch.Tensor, x: torch.Tensor, n_out: int, n_in: int,
          out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """fp32 y (m, n_out) = x (m, n_in) * W^T through ``ttq_gemv_<fmt>``."""
+    if fmt not in _GEMV:
+        raise TtqError(_lib.ERR_FORMAT, f"no block-format GEMV for format {fmt}")
     dev = _require_device(qweight, x, out)
-    m = x.numel() // n_in
+    _check_packed(_GEMV[fmt], qweight, fmt, n_out, n_in)
+    m = _rows(_GEMV[fmt], x, n_in)
     if out is None:
         out = torch.empty((m, n_out), dtype=torch.float32, device=dev)
+    else:
+        _check_out(_GEMV[fmt], out, m, n_out, torch.float32)
     fn = getattr(_lib.lib(), _GEMV[fmt])
     with torch.cuda.device(dev):
         check(fn(qweight.data_ptr(), x.data_ptr(), _code(x.dtype), out.data_ptr(), m, n_out, n_in,
@@ -151,9 +187,16 @@ def gemv_exl3(trellis: torch.Tensor, suh: torch.Tensor, svh: torch.Tensor, x: to
     dev = _require_device(trellis, suh, svh, x, out)
     if x.dtype != torch.float16:
         raise TtqError(_lib.ERR_DTYPE, "ttq_gemv_exl3 takes float16 activations")
-    m = x.numel() // n_in
+    if suh.dtype != torch.float16 or svh.dtype != torch.float16:
+        raise TtqError(_lib.ERR_DTYPE, "ttq_gemv_exl3: suh/svh must be float16")
+    if suh.numel() != n_in or svh.numel() != n_out:
+        raise TtqError(_lib.ERR_SHAPE, "ttq_gemv_exl3: suh/svh length")
+    _check_packed("ttq_gemv_exl3", trellis, _lib.EXL3, n_out, n_in, bits)
+    m = _rows("ttq_gemv_exl3", x, n_in)
     if out is None:
         out = torch.empty((m, n_out), dtype=torch.float32, device=dev)
+    else:
+        _check_out("ttq_gemv_exl3", out, m, n_out, torch.float32)
     with torch.cuda.device(dev):
         check(_lib.lib().ttq_gemv_exl3(trellis.data_ptr(), suh.data_ptr(), svh.data_ptr(), x.data_ptr(),
                                        out.data_ptr(), m, n_out, n_in, bits, codebook, _stream(dev)),
@@ -173,9 +216,12 @@ def gemm(fmt: int, qweight: torch.Tensor, x: torch.Tensor, n_out: int, n_in: int
     dev = _require_device(qweight, x, out)
     if x.dtype != torch.bfloat16:
         raise TtqError(_lib.ERR_DTYPE, f"{name} takes bfloat16 activations")
-    m = x.numel() // n_in
+    _check_packed(name, qweight, fmt, n_out, n_in)
+    m = _rows(name, x, n_in)
     if out is None:
         out = torch.empty((m, n_out), dtype=torch.bfloat16, device=dev)
+    else:
+        _check_out(name, out, m, n_out, torch.bfloat16)
     with torch.cuda.device(dev):
         check(getattr(_lib.lib(), name)(qweight.data_ptr(), x.data_ptr(), out.data_ptr(), m, n_out, n_in,
                                         _stream(dev)), name)
@@ -191,7 +237,10 @@ def gemm_q4_k(qweight: torch.Tensor, x: torch.Tensor, n_out: int, n_in: int,
 def dequantize(fmt: int, qweight: torch.Tensor, n_out: int, n_in: int,
                dtype: torch.dtype = torch.float32) -> torch.Tensor:
     """Dense (n_out, n_in) weight from packed blocks through ``ttq_dequant_<fmt>``."""
+    if fmt not in _DEQ:
+        raise TtqError(_lib.ERR_FORMAT, f"no block-format dequantizer for format {fmt}")
     dev = _require_device(qweight)
+    _check_packed(_DEQ[fmt], qweight, fmt, n_out, n_in)
     out = torch.empty((n_out, n_in), dtype=dtype, device=dev)
     fn = getattr(_lib.lib(), _DEQ[fmt])
     with torch.cuda.device(dev):
@@ -203,6 +252,7 @@ def dequantize_exl3(trellis: torch.Tensor, n_out: int, n_in: int, bits: int,
                     codebook: int = _lib.CB_MCG) -> torch.Tensor:
     """Decoded (unscaled, unrotated) trellis values, float16 (n_out, n_in)."""
     dev = _require_device(trellis)
+    _check_packed("ttq_dequant_exl3", trellis, _lib.EXL3, n_out, n_in, bits)
     out = torch.empty((n_out, n_in), dtype=torch.float16, device=dev)
     with torch.cuda.device(dev):
         check(_lib.lib().ttq_dequant_exl3(trellis.data_ptr(), out.data_ptr(), n_out, n_in, bits, codebook,
@@ -216,6 +266,9 @@ def hadamard128_(v: torch.Tensor, pre: Optional[torch.Tensor] = None,
     dev = _require_device(v, pre, post)
     if v.dtype != torch.float32:
         raise TtqError(_lib.ERR_DTYPE, "hadamard128_ takes float32")
+    for t in (pre, post):
+        if t is not None and (t.dtype != torch.float16 or t.numel() != v.numel()):
+            raise TtqError(_lib.ERR_SHAPE, "hadamard128_: pre/post must be float16 vectors as long as v")
     with torch.cuda.device(dev):
         check(_lib.lib().ttq_hadamard128_f32(v.data_ptr(), _ptr(pre), _ptr(post), v.numel(), _stream(dev)),
               "ttq_hadamard128_f32")
@@ -242,7 +295,8 @@ def gemv_q4_k_silu_mul(qweight: torch.Tensor, x: torch.Tensor, n_ff: int, n_in: 
     """y (m, n_ff) = silu(x Wg^T) * (x Wu^T) for the packed (2*n_ff, n_in) Q4_K matrix [Wg; Wu],
     one kernel (``ttq_gemv_q4_k_silu_mul``)."""
     dev = _require_device(qweight, x)
-    m = x.numel() // n_in
+    _check_packed("ttq_gemv_q4_k_silu_mul", qweight, _lib.Q4_K, 2 * n_ff, n_in)
+    m = _rows("ttq_gemv_q4_k_silu_mul", x, n_in)
     out = torch.empty((m, n_ff), dtype=out_dtype, device=dev)
     with torch.cuda.device(dev):
         check(_lib.lib().ttq_gemv_q4_k_silu_mul(qweight.data_ptr(), x.data_ptr(), _code(x.dtype), out.data_ptr(),
@@ -258,7 +312,8 @@ def gemm_q4_k_silu_mul(qweight: torch.Tensor, x: torch.Tensor, n_ff: int, n_in: 
     dev = _require_device(qweight, x)
     if x.dtype != torch.bfloat16:
         raise TtqError(_lib.ERR_DTYPE, "ttq_gemm_q4_k_silu_mul takes bfloat16 activations")
-    m = x.numel() // n_in
+    _check_packed("ttq_gemm_q4_k_silu_mul", qweight, _lib.Q4_K, 2 * n_ff, n_in)
+    m = _rows("ttq_gemm_q4_k_silu_mul", x, n_in)
     out = torch.empty((m, n_ff), dtype=torch.bfloat16, device=dev)
     with torch.cuda.device(dev):
         check(_lib.lib().ttq_gemm_q4_k_silu_mul(qweight.data_ptr(), x.data_ptr(), out.data_ptr(), m, n_ff, n_in,
@@ -290,7 +345,11 @@ def gemv_q4_k_rmsnorm(qweight: torch.Tensor, x: torch.Tensor, gamma: torch.Tenso
     weight of 2*n_out rows) in one kernel (``ttq_gemv_q4_k_rmsnorm``).
     Returns (y, normalized or None, new_residual or None)."""
     dev = _require_device(qweight, x, gamma, residual)
-    m = x.numel() // n_in
+    _check_packed("ttq_gemv_q4_k_rmsnorm", qweight, _lib.Q4_K, (2 if silu_mul else 1) * n_out, n_in)
+    m = _rows("ttq_gemv_q4_k_rmsnorm", x, n_in)
+    if gamma.numel() != n_in or gamma.dtype != x.dtype or (residual is not None and
+                                                          (residual.shape != x.shape or residual.dtype != x.dtype)):
+        raise TtqError(_lib.ERR_SHAPE, "ttq_gemv_q4_k_rmsnorm: gamma / residual do not match x")
     y = torch.empty((m, n_out), dtype=out_dtype, device=dev)
     normed = torch.empty_like(x) if want_normed else None
     new_res = torch.empty_like(x) if residual is not None else None

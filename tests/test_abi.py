@@ -30,16 +30,17 @@ def test_every_declared_symbol_is_exported_and_bound():
 
 def test_version_and_strerror():
     L = _lib.lib()
-    assert L.ttq_version() == 100
+    assert L.ttq_version() == 110
     assert L.ttq_strerror(0) == b"ok"
-    for code in range(-7, 0):
+    for code in range(-8, 0):
         assert len(L.ttq_strerror(code)) > 3
     assert L.ttq_strerror(-99) == b"unknown status"
 
 
 def test_struct_layout_matches_header():
-    assert C.sizeof(QLinearStruct) == 4 * 4 + 2 * 8 + 4 * 8
-    assert QLinearStruct.n_out.offset == 16 and QLinearStruct.qweight.offset == 32
+    assert C.sizeof(QLinearStruct) == 6 * 4 + 2 * 8 + 4 * 8
+    assert QLinearStruct.precision.offset == 16
+    assert QLinearStruct.n_out.offset == 24 and QLinearStruct.qweight.offset == 40
 
 
 @pytest.mark.parametrize("name", ["ttq_gemv_q8_0", "ttq_gemv_q4_k", "ttq_gemv_q6_k"])
@@ -105,6 +106,83 @@ def test_other_entry_points_validate():
     st = QLinearStruct(format=_lib.EXL3, bits=3, codebook=1, n_out=128, n_in=128, qweight=p)
     assert L.ttq_linear_forward(C.byref(st), p, _lib.F16, 1, p, _lib.F32, None) == _lib.ERR_NULL
     assert L.ttq_linear_forward(None, p, _lib.F16, 1, p, _lib.F32, None) == _lib.ERR_NULL
+
+
+def test_empty_batches_return_ok_before_any_pointer_check():
+    """F.linear of a (0, n_in) activation gives an empty tensor, whose data pointer is NULL."""
+    L = _lib.lib()
+    for fn in (L.ttq_gemm_q4_k, L.ttq_gemm_q6_k, L.ttq_gemm_q8_0, L.ttq_gemm_q4_k_silu_mul):
+        assert fn(None, None, None, 0, 16, 256, None) == _lib.OK
+        assert fn(None, None, None, 16, 0, 256, None) == _lib.OK
+        assert fn(None, None, None, 0, 16, 100, None) == _lib.ERR_SHAPE      # dimensions still checked
+    assert L.ttq_gemv_exl3(None, None, None, None, None, 0, 128, 128, 3, 1, None) == _lib.OK
+    assert L.ttq_gemv_exl3(None, None, None, None, None, 0, 128, 128, 9, 1, None) == _lib.ERR_FORMAT
+    for fmt, kw in ((_lib.Q4_K, {}), (_lib.Q6_K, {}), (_lib.Q8_0, {}), (_lib.EXL3, dict(bits=3, codebook=1))):
+        st = QLinearStruct(format=fmt, n_out=128, n_in=256, **kw)
+        assert L.ttq_linear_forward(C.byref(st), None, _lib.BF16, 0, None, _lib.BF16, None) == _lib.OK
+        st = QLinearStruct(format=fmt, n_out=0, n_in=256, **kw)
+        assert L.ttq_linear_forward(C.byref(st), None, _lib.BF16, 3, None, _lib.BF16, None) == _lib.OK
+
+
+def test_large_batches_pass_the_shape_check():
+    """Rows beyond gridDim.y's 65535 are accepted (taken a slice at a time); the checks that follow
+    the shape check answer here, since there is no buffer behind the pointers."""
+    L = _lib.lib()
+    buf = np.zeros(4096, np.uint8)
+    p = buf.ctypes.data
+    p += (-p) % 16
+    assert L.ttq_gemm_q4_k(p, p + 2, p, 1 << 20, 16, 256, None) == _lib.ERR_ALIGN
+    assert L.ttq_gemv_q4_k(p, p + 2, _lib.BF16, p, 70000, 16, 256, None) == _lib.ERR_ALIGN
+    st = QLinearStruct(format=_lib.Q4_K, n_out=16, n_in=256, qweight=p)
+    assert L.ttq_linear_forward(C.byref(st), p + 2, _lib.BF16, 1 << 20, p, _lib.BF16, None) == _lib.ERR_ALIGN
+
+
+def test_row_length_limits():
+    L = _lib.lib()
+    buf = np.zeros(4096, np.uint8)
+    p = buf.ctypes.data
+    p += (-p) % 16
+    # 16-bit activations on the K-quants: 32768; everything else 16384 (misalignment answers when the
+    # limit lets the call through)
+    assert L.ttq_gemv_q4_k(p, p + 2, _lib.BF16, p, 1, 16, 32768, None) == _lib.ERR_ALIGN
+    assert L.ttq_gemv_q6_k(p, p + 2, _lib.F16, p, 1, 16, 28672, None) == _lib.ERR_ALIGN
+    assert L.ttq_gemv_q4_k(p, p, _lib.BF16, p, 1, 16, 32768 + 256, None) == _lib.ERR_UNSUPPORTED
+    assert L.ttq_gemv_q4_k(p, p, _lib.F32, p, 1, 16, 16384 + 256, None) == _lib.ERR_UNSUPPORTED
+    assert L.ttq_gemv_q8_0(p, p, _lib.BF16, p, 1, 16, 16384 + 256, None) == _lib.ERR_UNSUPPORTED
+    st = QLinearStruct(format=_lib.EXL3, bits=3, codebook=1, n_out=128, n_in=16384 + 128, qweight=p, suh=p, svh=p)
+    assert L.ttq_linear_forward(C.byref(st), p, _lib.F16, 1, p, _lib.F32, None) == _lib.ERR_UNSUPPORTED
+
+
+def test_fused_rmsnorm_gemv_rejects_in_place_outputs():
+    """Every workgroup re-reads x and residual while one of them writes the outputs, so the fused
+    call is out of place only."""
+    L = _lib.lib()
+    buf = np.zeros(1 << 16, np.uint8)
+    p = buf.ctypes.data
+    p += (-p) % 16
+    w, x, res, gamma, nres, normed, y = (p + i * 4096 for i in range(7))
+    n_in, n_out = 256, 16
+
+    def call(new_res, nrm, residual=res):
+        return L.ttq_gemv_q4_k_rmsnorm(w, x, residual, gamma, 1e-6, _lib.BF16, new_res, nrm, y, _lib.F32,
+                                       2, n_out, n_in, 0, None)
+    assert call(res, normed) == _lib.ERR_ALIAS          # new_residual_out == residual
+    assert call(nres, x) == _lib.ERR_ALIAS              # normed_out == x
+    assert call(x, normed) == _lib.ERR_ALIAS
+    assert call(nres, res) == _lib.ERR_ALIAS
+    assert call(nres, nres) == _lib.ERR_ALIAS           # the two outputs on each other
+    assert call(x + 2 * n_in * 2 - 16, normed) == _lib.ERR_ALIAS    # partial overlap with x's last bytes
+    assert call(None, x, residual=None) == _lib.ERR_ALIAS
+    assert L.ttq_strerror(_lib.ERR_ALIAS) not in (b"unknown status", b"ok")
+
+
+def test_linear_forward_rejects_unknown_precision():
+    L = _lib.lib()
+    buf = np.zeros(4096, np.uint8)
+    p = buf.ctypes.data
+    p += (-p) % 16
+    st = QLinearStruct(format=_lib.Q4_K, n_out=16, n_in=256, qweight=p, precision=7)
+    assert L.ttq_linear_forward(C.byref(st), p, _lib.BF16, 1, p, _lib.F32, None) == _lib.ERR_FORMAT
 
 
 def test_missing_library_fails_loudly(monkeypatch):

@@ -274,7 +274,7 @@ def test_q8_0_unit_vectors_and_extremes_many_rows(xk, n_in):
 
 def test_gemv_rejects_oversized_rows():
     with pytest.raises(TtqError) as e:
-        QL.gemv(F.Q4_K, torch.zeros(144 * 4 * 128, dtype=torch.uint8, device=DEV),
+        QL.gemv(F.Q4_K, torch.zeros(144 * 128, dtype=torch.uint8, device=DEV),
                 torch.zeros(32768, dtype=torch.float32, device=DEV), 1, 32768)
     assert e.value.status == F.ERR_UNSUPPORTED
 
