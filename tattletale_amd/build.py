@@ -31,6 +31,7 @@ SOURCES = [
     "ttq_gemm_pc.hip",
     "ttq_gemm_skinny.hip",
     "ttq_exl3.hip",
+    "ttq_exl3_mfma.hip",
     "ttq_activations.hip",
     "ttq_host.cpp",
 ]

@@ -15,29 +15,9 @@
 // trellis[k_tile][n_tile][16*bits].  Because 16*bits is a multiple of 16, the 16 weights
 // of one output channel inside a tile start on a word boundary and span bits+1 words; one
 // lane decodes exactly those 16 weights, so all window shifts are compile-time constants.
-#include "ttq_device.h"
-#include "ttq_internal.h"
+#include "ttq_exl3_common.h"
 
 namespace ttq {
-
-typedef __attribute__((ext_vector_type(2))) _Float16 half2_t;
-
-// The codebook: a pure function of the 16-bit trellis state (bits 16..31 of `state` are ignored).
-// The 32-bit multiply is not what limits the decode here: splitting it into two 16-bit
-// multiply-adds was measured slower.
-template <int CB>
-struct Codebook {
-  static constexpr uint32_t kMul = (CB == 0) ? 89226354u : 0xCBAC1FEDu;
-  __device__ __forceinline__ void init() {}
-  __device__ __forceinline__ _Float16 code(uint32_t state) const {
-    uint32_t u = (state & 0xFFFFu) * kMul;
-    if (CB == 0) u += 64248484u;
-    u = (u & 0x8FFF8FFFu) ^ 0x3B603B60u;
-    half2_t h;
-    __builtin_memcpy(&h, &u, 4);
-    return h[0] + h[1];  // fp16 add, round-to-nearest-even
-  }
-};
 
 // The bits+1 words that hold the 16 windows of output channel j of a tile, as big-endian
 // 32-bit chunks (first stream bit = bit 31 of chunk 0).
@@ -121,45 +101,6 @@ __global__ void __launch_bounds__(256) dequant_exl3_kernel(const uint16_t* __res
 // ------------------------------------------------------------------ GEMV
 constexpr int kExl3Threads = 1024;
 constexpr int kExl3Waves = kExl3Threads / kWave;
-
-// Unnormalized FWHT of a 128-group held as 4 consecutive values in each of 32 consecutive lanes
-// (value index = 4*lane + i): stages 1 and 2 inside the lane, stages 4..64 against the lane
-// 1, 2, 4, 8, 16 away.  Same stage order and operand order as the textbook loop
-// (lower index gets a+b, upper a-b), so the results do not depend on how it is laid out.
-__device__ __forceinline__ void fwht128_quad(float (&v)[4], int lane) {
-  float t;
-  t = v[0]; v[0] = t + v[1]; v[1] = t - v[1];
-  t = v[2]; v[2] = t + v[3]; v[3] = t - v[3];
-  t = v[0]; v[0] = t + v[2]; v[2] = t - v[2];
-  t = v[1]; v[1] = t + v[3]; v[3] = t - v[3];
-#pragma unroll
-  for (int d = 1; d < 32; d <<= 1) {
-    const bool upper = (lane & d) != 0;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const float o = __shfl_xor(v[i], d, kWave);
-      v[i] = upper ? (o - v[i]) : (v[i] + o);
-    }
-  }
-}
-
-// Four consecutive activations (a multiple of four elements from the row start) as floats.
-__device__ __forceinline__ void load_x4(const float* p, float (&v)[4]) {
-  const float4 t = *reinterpret_cast<const float4*>(__builtin_assume_aligned(p, 16));
-  v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-}
-__device__ __forceinline__ void load_x4(const f16_tag* p, float (&v)[4]) {
-  uint2 r;
-  __builtin_memcpy(&r, __builtin_assume_aligned(p, 8), 8);
-  v[0] = f16_bits_to_f32((uint16_t)r.x); v[1] = f16_bits_to_f32((uint16_t)(r.x >> 16));
-  v[2] = f16_bits_to_f32((uint16_t)r.y); v[3] = f16_bits_to_f32((uint16_t)(r.y >> 16));
-}
-__device__ __forceinline__ void load_x4(const bf16_tag* p, float (&v)[4]) {
-  uint2 r;
-  __builtin_memcpy(&r, __builtin_assume_aligned(p, 8), 8);
-  v[0] = bf16_bits_to_f32((uint16_t)r.x); v[1] = bf16_bits_to_f32((uint16_t)(r.x >> 16));
-  v[2] = bf16_bits_to_f32((uint16_t)r.y); v[3] = bf16_bits_to_f32((uint16_t)(r.y >> 16));
-}
 
 // One workgroup per n_tile (16 output channels).  Lane = (k-tile slot g = lane/16, channel
 // j = lane%16); the 16 waves times 4 slots walk the k tiles 64 at a time.  Partial sums are
@@ -406,6 +347,17 @@ hipError_t launch_gemv_exl3(const uint16_t* trellis, const uint16_t* suh, const 
   if (y_dtype != kF32) return hipErrorInvalidValue;
   float* yf = static_cast<float*>(y);
   hipError_t e;
+  static const int two_launches = dev_knob("TTQ_EXL3_TWO_LAUNCHES", 0);
+  if (!two_launches) {
+    const Exl3Plan plan = exl3_mfma_plan(m, n_out, n_in);
+    unsigned long long* accum = nullptr;
+    if (plan.slices > 1) {
+      e = exl3_workspace(s, &accum);
+      if (e != hipSuccess) return e;
+    }
+    return launch_gemv_exl3_mfma(plan, trellis, suh, svh, x, x_dtype, yf, bias, bias_dtype, m, n_out, n_in, bits, cb,
+                                 accum, s);
+  }
   switch (bits) {
     case 1: e = gemv_bits<1>(trellis, suh, x, x_dtype, yf, m, n_out, n_in, cb, s); break;
     case 2: e = gemv_bits<2>(trellis, suh, x, x_dtype, yf, m, n_out, n_in, cb, s); break;

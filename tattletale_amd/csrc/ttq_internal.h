@@ -166,4 +166,20 @@ hipError_t launch_gemv_exl3(const uint16_t* trellis, const uint16_t* suh, const 
 hipError_t launch_hadamard128(float* v, const uint16_t* pre, const uint16_t* post, int64_t n,
                               hipStream_t s);
 
+// Matrix-core trellis GEMV in one launch (ttq_exl3_mfma.hip).  The plan says how the reduction
+// dimension is sliced and how many 64-bit accumulator words a sliced launch needs (zero before and
+// after every launch).
+struct Exl3Plan {
+  int groups, row_groups, slices, slice_tiles;
+  int64_t accum_words;
+};
+Exl3Plan exl3_mfma_plan(int64_t m, int64_t n_out, int64_t n_in);
+hipError_t launch_gemv_exl3_mfma(const Exl3Plan& p, const uint16_t* trellis, const uint16_t* suh,
+                                 const uint16_t* svh, const void* x, int x_dtype, float* y, const void* bias,
+                                 int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, int bits, int cb,
+                                 unsigned long long* accum, hipStream_t s);
+// The library's own accumulator words for the calling thread's device and this stream, allocated and
+// cleared on first use.
+hipError_t exl3_workspace(hipStream_t s, unsigned long long** accum);
+
 }  // namespace ttq

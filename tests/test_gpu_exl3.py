@@ -76,3 +76,66 @@ def test_exl3_several_rows_share_the_decode(m):
     for i in {0, m // 2, m - 1}:
         y1 = QL.gemv_exl3(trd, sud, svd, xd[i:i + 1], n_out, n_in, bits, F.CB_MCG)
         assert torch.equal(y1[0], y[i])
+
+
+@pytest.mark.parametrize("bits,cb", [(1, F.CB_MCG), (7, F.CB_3INST), (7, F.CB_MCG), (4, F.CB_3INST)])
+@pytest.mark.parametrize("n_out,n_in,m", [(128, 128, 1), (128, 2048, 3), (1024, 2176, 1), (256, 4096 + 128, 9)])
+def test_exl3_gemv_slicing_of_the_reduction(bits, cb, n_out, n_in, m):
+    """Shapes that split the reduction over several workgroups per output group (few outputs), with a
+    last slice shorter than the others, and one with more than one LDS pass per slice."""
+    w = Q.fill_normal(600 + bits, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
+    tr, suh, svh = Q.quantize_exl3(w, bits, cb, seed=bits)
+    T = oracle.exl3_decode(tr, n_out, n_in, bits, cb)
+    x = Q.f32_to_f16(Q.fill_normal(601, 1, 1.0, m * n_in).reshape(m, n_in))
+    args = (packed_to_dev(tr), bits_to_dev(suh, "f16"), bits_to_dev(svh, "f16"), bits_to_dev(x, "f16"))
+    y = QL.gemv_exl3(*args, n_out, n_in, bits, cb)
+    for i in range(m):
+        assert rel_l2(y[i].cpu().numpy(), oracle.exl3_gemv_f64(T, suh, svh, x[i])) <= TOL
+    # the arrival counters are back at zero after every launch: the same call again gives the same bits
+    for _ in range(3):
+        assert torch.equal(QL.gemv_exl3(*args, n_out, n_in, bits, cb), y)
+
+
+def test_exl3_many_rows_take_whole_slices():
+    """Enough (output group, row group) units to fill the GPU: no slicing, eight LDS passes per workgroup."""
+    n_out, n_in, bits, m = 1024, 4096, 2, 8 * 33 + 5
+    w = Q.fill_normal(610, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
+    tr, suh, svh = Q.quantize_exl3(w, bits, F.CB_MCG, seed=3)
+    T = oracle.exl3_decode(tr, n_out, n_in, bits, F.CB_MCG)
+    x = Q.f32_to_f16(Q.fill_normal(611, 1, 1.0, m * n_in).reshape(m, n_in))
+    y = QL.gemv_exl3(packed_to_dev(tr), bits_to_dev(suh, "f16"), bits_to_dev(svh, "f16"), bits_to_dev(x, "f16"),
+                     n_out, n_in, bits, F.CB_MCG).cpu().numpy()
+    for i in (0, 7, 8, 100, m - 6, m - 1):
+        assert rel_l2(y[i], oracle.exl3_gemv_f64(T, suh, svh, x[i])) <= TOL, i
+
+
+@pytest.mark.parametrize("xk", ["bf16", "f32"])
+def test_exl3_forward_other_activation_types_and_ranges(xk):
+    """bf16 / fp32 activations through the operator, with rows scaled far outside fp16's range: the
+    per-group power-of-two scale keeps the two-term split exact enough at any magnitude."""
+    n_out, n_in, bits = 256, 1024, 3
+    w = Q.fill_normal(620, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
+    tr, suh, svh = Q.quantize_exl3(w, bits, F.CB_MCG, seed=4)
+    T = oracle.exl3_decode(tr, n_out, n_in, bits, F.CB_MCG)
+    x = Q.fill_normal(621, 1, 1.0, 4 * n_in).reshape(4, n_in)
+    x[1] *= 1e-12
+    x[2] *= 3e9
+    x[3, ::2] = 0.0
+    from scipy.linalg import hadamard
+    from util import x_to_dev
+    xd, xf = x_to_dev(x, xk)
+    H = hadamard(128).astype(np.float64) / np.sqrt(128.0)
+    Tf = oracle.f16_to_f32(T).astype(np.float64)
+    su, sv = oracle.f16_to_f32(suh).astype(np.float64), oracle.f16_to_f32(svh).astype(np.float64)
+
+    def by_matrices(xrow):
+        xr = ((xrow.astype(np.float64) * su).reshape(-1, 128) @ H.T).reshape(-1)
+        return ((Tf @ xr).reshape(-1, 128) @ H.T).reshape(-1) * sv
+    # the matrix form is the oracle's function: same answer on a row the oracle can take
+    probe = Q.f32_to_f16(x[0])
+    assert rel_l2(by_matrices(oracle.f16_to_f32(probe)), oracle.exl3_gemv_f64(T, suh, svh, probe)) <= 1e-12
+    layer = QuantLinear.init(packed_to_dev(tr), F.EXL3, n_in, n_out, suh=bits_to_dev(suh, "f16"),
+                             svh=bits_to_dev(svh, "f16"), bits=bits)
+    y = layer.forward(xd, out_dtype=torch.float32).cpu().numpy()
+    for i in range(4):
+        assert rel_l2(y[i], by_matrices(xf[i])) <= TOL, i
