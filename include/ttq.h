@@ -136,6 +136,20 @@ TTQ_API int ttq_gemv_exl3(const uint16_t* trellis, const uint16_t* suh_f16, cons
                   const uint16_t* x_f16, float* y, int64_t m, int64_t n_out, int64_t n_in,
                   int bits, int codebook, void* stream);
 
+/* ttq_gemv_exl3 for callers that cannot allocate device memory: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments,
+ * same results bit for bit; m <= 8.  Where ttq_gemv_exl3 takes its workspace (the words through which
+ * the slices of the reduction meet) from hipMalloc on first use, this entry point uses a 4 MiB array
+ * that is part of the library's device image: every GPU the library runs on holds one from the first
+ * call there until the process ends.  It calls no allocating routine.  Returns TTQ_ERR_UNSUPPORTED
+ * for m > 8 and for a launch that would need more than the 4 MiB (a device with more than 256
+ * compute units).  All calls on one GPU share the array: calls that may overlap there (different
+ * streams, different threads) race; calls on one stream do not.  Every call leaves the words it used
+ * at zero, which is what the next call expects. */
+TTQ_API int ttq_gemv_exl3_noalloc(const uint16_t* trellis, const uint16_t* suh_f16, const uint16_t* svh_f16,
+                  const uint16_t* x_f16, float* y, int64_t m, int64_t n_out, int64_t n_in,
+                  int bits, int codebook, void* stream);
+
 /* ---- prefill GEMM ------------------------------------------------------------------ */
 /* Y[m][n_out] (bf16) = X[m][n_in] (bf16) * W^T, Q4_K weights dequantized to bf16 tiles and
  * multiplied with bf16 MFMA, fp32 accumulation.  Stands in for F.linear(x, weight) with a

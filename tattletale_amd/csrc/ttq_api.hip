@@ -193,6 +193,29 @@ int ttq_gemv_exl3(const uint16_t* trellis, const uint16_t* suh_f16, const uint16
                                           static_cast<hipStream_t>(stream)));
 }
 
+int ttq_gemv_exl3_noalloc(const uint16_t* trellis, const uint16_t* suh_f16, const uint16_t* svh_f16,
+                          const uint16_t* x_f16, float* y, int64_t m, int64_t n_out, int64_t n_in, int bits,
+                          int codebook, void* stream) {
+  const int rc = check_shape(TTQ_EXL3, m, n_out, n_in, bits, codebook);
+  if (rc != TTQ_OK) return rc;
+  if (m == 0 || n_out == 0) return TTQ_OK;
+  if (!trellis || !suh_f16 || !svh_f16 || !x_f16 || !y) return TTQ_ERR_NULL;
+  if (!aligned16(trellis) || !aligned16(x_f16) || !aligned16(y) || !aligned8(suh_f16) || !aligned8(svh_f16))
+    return TTQ_ERR_ALIGN;
+  if (n_in > ttq::kMaxGemvInF32) return TTQ_ERR_UNSUPPORTED;
+  if (m > 8) return TTQ_ERR_UNSUPPORTED;        // one group of activation rows: the decode case
+  const ttq::Exl3Plan plan = ttq::exl3_mfma_plan(m, n_out, n_in);
+  if (plan.accum_words > ttq::exl3_resident_words()) return TTQ_ERR_UNSUPPORTED;
+  unsigned long long* accum = nullptr;
+  if (plan.slices > 1) {
+    const hipError_t e = ttq::exl3_resident_workspace(&accum);
+    if (e != hipSuccess) return hip_status(e);
+  }
+  return hip_status(ttq::launch_gemv_exl3_mfma(plan, trellis, suh_f16, svh_f16, x_f16, TTQ_F16, y, nullptr, 0, m,
+                                               n_out, n_in, bits, codebook, accum,
+                                               static_cast<hipStream_t>(stream)));
+}
+
 int ttq_silu_and_mul(const void* in, void* out, int dtype, int64_t m, int64_t h, void* stream) {
   if (!valid_dtype(dtype)) return TTQ_ERR_DTYPE;
   if (m < 0 || h < 0) return TTQ_ERR_SHAPE;

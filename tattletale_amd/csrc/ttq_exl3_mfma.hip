@@ -509,4 +509,37 @@ hipError_t exl3_workspace(hipStream_t s, unsigned long long** accum) {
   return hipSuccess;
 }
 
+// ------------------------------------------------------------------------------ resident workspace
+// The same words as a file-scope array in device memory, for the entry point that must not allocate:
+// every GPU the library runs on holds its own copy from the moment the code object is loaded there
+// until the process ends, zero-initialised, and every launch leaves the words it used at zero again.
+// The array's name is only a handle in host code; the address on a device comes from
+// hipGetSymbolAddress, asked once per device with that device current.
+constexpr int64_t kXmResidentWords = (int64_t)256 * kXmKSplit * kXmTok * 128;      // 4 MiB
+static __device__ __align__(256) unsigned long long scratch[kXmResidentWords];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_resident_mutex;
+unsigned long long* g_resident[kMaxDevices] = {};
+}  // namespace
+
+int64_t exl3_resident_words() { return kXmResidentWords; }
+
+hipError_t exl3_resident_workspace(unsigned long long** accum) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(g_resident_mutex);
+  if (!g_resident[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    g_resident[dev] = static_cast<unsigned long long*>(p);
+  }
+  *accum = g_resident[dev];
+  return hipSuccess;
+}
+
 }  // namespace ttq

@@ -181,5 +181,8 @@ hipError_t launch_gemv_exl3_mfma(const Exl3Plan& p, const uint16_t* trellis, con
 // The library's own accumulator words for the calling thread's device and this stream, allocated and
 // cleared on first use.
 hipError_t exl3_workspace(hipStream_t s, unsigned long long** accum);
+// The workspace that lives in the library's own device image (one per GPU, nothing allocated), and its size.
+hipError_t exl3_resident_workspace(unsigned long long** accum);
+int64_t exl3_resident_words();
 
 }  // namespace ttq
