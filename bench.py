@@ -469,6 +469,34 @@ def main() -> int:
             timed(nm, fmt, 512,
                   lambda ws, x, nc, y=y, fmt=fmt: (lambda i: QL.gemm(fmt, ws[i % nc], x, n_out, n_in, out=y)),
                   steps=max(20, steps // 4))
+        # trellis weights, 4096 x 4096 at 3 bits: 8 rows through the decode kernel (one decode of the weights
+        # for all 8), 512 rows through the prefill path, and the Q4_K GEMM at the same shape beside it
+        ecfg = CFG.CONFIGS["exl3_gemv"]
+        etr, esuh, esvh = CFG.packed_weights(ecfg)
+        enc = rotated(etr.nbytes)
+        etrs = [to_dev(etr) for _ in range(enc)]
+        esu, esv = to_dev(esuh, "f16"), to_dev(esvh, "f16")
+        for m in (8, 512):
+            xe = torch.randn((m, ecfg.n_in), device=dev).to(torch.float16)
+            if m == 8:
+                ye = torch.empty((m, ecfg.n_out), dtype=torch.float32, device=dev)
+
+                def estep(i, xe=xe, ye=ye):
+                    QL.gemv_exl3(etrs[i % enc], esu, esv, xe, ecfg.n_out, ecfg.n_in, ecfg.bits, F.CB_MCG, out=ye)
+            else:
+                def estep(i, xe=xe):
+                    QL.gemm_exl3(etrs[i % enc], esu, esv, xe, ecfg.n_out, ecfg.n_in, ecfg.bits, F.CB_MCG)
+            ms = time_steps(estep, steps if m == 8 else max(20, steps // 4), warmup)["ms"]
+            nm = "exl3_gemv_m8_4096x4096" if m == 8 else "exl3_prefill_m512_4096x4096"
+            res[nm] = {"us_per_step": ms * 1e3, "weight_GBps": etr.nbytes / (ms * 1e-3) / 1e9,
+                       "TFLOPs": 2.0 * m * ecfg.n_out * ecfg.n_in / (ms * 1e-3) / 1e12}
+            log("[%s] %.2f us/step  %.1f TFLOP/s" % (nm, ms * 1e3, res[nm]["TFLOPs"]))
+        del etrs
+        torch.cuda.empty_cache()
+        y = torch.empty((512, 4096), dtype=torch.bfloat16, device=dev)
+        timed("q4_k_gemm_m512_4096x4096", F.Q4_K, 512,
+              lambda ws, x, nc, y=y: (lambda i: QL.gemm(F.Q4_K, ws[i % nc], x, 4096, 4096, out=y)),
+              n_out=4096, n_in=4096, steps=max(20, steps // 4))
         # add + RMSNorm alone (ttq_rmsnorm with a residual): one decode row and a prefill block.
         # Algorithmic bytes: x and residual read, new residual and normalized row written.
         L = _lib.lib()

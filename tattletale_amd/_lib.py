@@ -57,6 +57,7 @@ SIGNATURES = {
     "ttq_gemv_q6_k": (_i32, [_vp, _vp, _i32, _vp, _i64, _i64, _i64, _vp]),
     "ttq_gemv_exl3": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32, _vp]),
     "ttq_gemv_exl3_noalloc": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32, _vp]),
+    "ttq_gemm_exl3": (_i32, [_vp, _vp, _vp, _vp, _i32, _vp, _i64, _i64, _i64, _i32, _i32, _vp]),
     "ttq_gemm_q4_k": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "ttq_gemm_q6_k": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "ttq_gemm_q8_0": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),

@@ -32,6 +32,7 @@ SOURCES = [
     "ttq_gemm_skinny.hip",
     "ttq_exl3.hip",
     "ttq_exl3_mfma.hip",
+    "ttq_exl3_prefill.hip",
     "ttq_activations.hip",
     "ttq_host.cpp",
 ]

@@ -1,0 +1,313 @@
+// Trellis-coded (EXL3-style) linear layer for many activation rows: Y = svh o H( T * H(suh o X^T) ),
+// the prefill side of Linear.forward (workspace/transformers/src/layers/linear.nim:45-57; the
+// projections see seq_len rows at prefill, attn.nim:154-156).
+//
+// Two launches.  The first rotates the activations once -- x o suh, the 128-group butterfly, 1/sqrt(128),
+// rounded to fp16 -- into a workspace: every output group needs every rotated row, and the rotation of a
+// pass of 64 rows would cost a workgroup more vector work than decoding the pass's weights.  The second
+// is the decode GEMV's workgroup (128 output channels, 16 wavefronts, weights staged through LDS as a
+// big-endian bit string, four weights per lane decoded into an A fragment) with 64 rows per workgroup:
+// each decoded fragment feeds four v_mfma_f32_16x16x16_f16, one per block of 16 rows, so the decode --
+// which bounds the single-row kernel -- is paid once per 64 rows.  A workgroup covers the whole
+// reduction, rotates its 64 x 128 sums and writes y; no workspace is shared between workgroups.
+//
+// Accuracy: the rotated activations are rounded to fp16 once (2^-11 relative per element, about 3e-4
+// on a row product); weights are exact fp16, sums fp32.  The decode kernel's two-term split is for
+// callers that ask for its accuracy class whatever the row count.
+#include "ttq_exl3_common.h"
+
+#include <mutex>
+#include <unordered_map>
+
+namespace ttq {
+
+constexpr int kXpRows = 64;                                   // activation rows per workgroup
+constexpr int kXpRowBlocks = kXpRows / 16;
+constexpr int kXpXPieces = kXpRows * (kXmChunkK / 8) / kXmThreads;   // 16-byte pieces of X per thread and pass
+
+// ---- pass one: Xr[row][k] = fp16( H(x o suh) / sqrt(128) ), one 32-lane half wavefront per (row, 128-group)
+template <typename XT>
+__global__ void __launch_bounds__(256)
+exl3_rotate_rows_kernel(const XT* __restrict__ x, const uint16_t* __restrict__ suh, uint16_t* __restrict__ xr,
+                        int64_t items, int groups_per_row, int64_t n_in) {
+  const int lane = threadIdx.x & 63, l32 = threadIdx.x & 31;
+  const int64_t item = (int64_t)blockIdx.x * (256 / 32) + (threadIdx.x >> 5);
+  if (item >= items) return;
+  const int64_t row = item / groups_per_row;
+  const int64_t k = (item - row * groups_per_row) * 128 + 4 * l32;
+  uint2 sraw;
+  __builtin_memcpy(&sraw, __builtin_assume_aligned(suh + k, 8), 8);
+  float v[4];
+  load_x4(x + row * n_in + k, v);
+  v[0] *= f16_bits_to_f32((uint16_t)sraw.x);
+  v[1] *= f16_bits_to_f32((uint16_t)(sraw.x >> 16));
+  v[2] *= f16_bits_to_f32((uint16_t)sraw.y);
+  v[3] *= f16_bits_to_f32((uint16_t)(sraw.y >> 16));
+  fwht128_quad(v, lane);
+  uint2 o;
+  o.x = (uint32_t)f32_to_f16_bits(v[0] * 0.08838834764831845f) | ((uint32_t)f32_to_f16_bits(v[1] * 0.08838834764831845f) << 16);
+  o.y = (uint32_t)f32_to_f16_bits(v[2] * 0.08838834764831845f) | ((uint32_t)f32_to_f16_bits(v[3] * 0.08838834764831845f) << 16);
+  __builtin_memcpy(__builtin_assume_aligned(xr + row * n_in + k, 8), &o, 8);
+}
+
+// ---- pass two
+template <int BITS, int CB>
+__global__ void __launch_bounds__(kXmThreads)
+gemm_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __restrict__ svh,
+                      const uint16_t* __restrict__ xr, float* __restrict__ y, const void* __restrict__ bias,
+                      int bias_dtype, int m, int n_out, int n_in) {
+  using G = XmGeom<BITS>;
+  // one pass of tiles, then 64 rows of rotated activations; the epilogue's sums reuse the activations' space
+  __shared__ uint32_t slab[G::kSlabDw];
+  __shared__ __attribute__((aligned(16))) _Float16 xs[kXpRows * kXmColStride];
+  static_assert(sizeof(_Float16) * kXpRows * kXmColStride >= sizeof(float) * kXmKSplit * kXpRows * 128, "sums fit");
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int grp = blockIdx.x;
+  const int t0 = blockIdx.y * kXpRows;
+  const int rows = min(kXpRows, m - t0);
+  const int nt_n = n_out >> 4, kt_n = n_in >> 4;
+  const int col = lane & 15, q = lane >> 4;
+  const int tcol = wave & 7, kpart = wave >> 3;
+
+  XmLane<BITS> ln;
+  ln.init(lane);
+
+  const char* wbase = reinterpret_cast<const char*>(trellis) + (int64_t)grp * 8 * (32 * BITS);
+  const int64_t row_bytes = (int64_t)nt_n * (32 * BITS);
+  uint4 pre[G::kSets];
+  uint4 xpre[kXpXPieces];
+  auto request = [&](int kt_first, int cnt) {
+    // activations first: piece p = (row, 8 columns); rows past the end re-read the last row
+#pragma unroll
+    for (int i = 0; i < kXpXPieces; i++) {
+      const int p = tid + i * kXmThreads;
+      const int r = p >> 6, c = p & 63;
+      xpre[i] = *reinterpret_cast<const uint4*>(xr + (int64_t)(t0 + min(r, rows - 1)) * n_in + (int64_t)kt_first * 16 +
+                                                min(c, 2 * cnt - 1) * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < G::kSets; i++) {
+      const int p = tid + i * kXmThreads;
+      const int ktl = p / G::kRunPieces, r = p - ktl * G::kRunPieces;
+      pre[i] = *reinterpret_cast<const uint4*>(wbase + (int64_t)(kt_first + min(ktl, cnt - 1)) * row_bytes + r * 16);
+    }
+  };
+  auto stage = [&](int cnt) {
+#pragma unroll
+    for (int i = 0; i < kXpXPieces; i++) {
+      const int p = tid + i * kXmThreads;
+      const int r = p >> 6, c = p & 63;
+      *reinterpret_cast<uint4*>(xs + r * kXmColStride + c * 8) = xpre[i];
+    }
+#pragma unroll
+    for (int i = 0; i < G::kSets; i++) {
+      const int p = tid + i * kXmThreads;
+      const int ktl = p / G::kRunPieces, r = p - ktl * G::kRunPieces;
+      if (ktl < cnt) {
+        const int nt = r / (2 * BITS), ci = r - nt * (2 * BITS);
+        uint32_t* dst = slab + 1 + (ktl * 8 + nt) * G::kTileStride + 4 * ci;
+        const uint32_t c0 = __builtin_amdgcn_alignbit(pre[i].x, pre[i].x, 16);
+        dst[0] = c0;
+        dst[1] = __builtin_amdgcn_alignbit(pre[i].y, pre[i].y, 16);
+        dst[2] = __builtin_amdgcn_alignbit(pre[i].z, pre[i].z, 16);
+        dst[3] = __builtin_amdgcn_alignbit(pre[i].w, pre[i].w, 16);
+        if (ci == 0) dst[G::kTileDw] = c0;
+      }
+    }
+  };
+
+  request(0, min(kXmChunkTiles, kt_n));
+
+  f32x4_t acc[kXpRowBlocks];
+#pragma unroll
+  for (int rb = 0; rb < kXpRowBlocks; rb++) acc[rb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  constexpr int kWin = XmLane<BITS>::kWin;
+  const uint32_t* wcol = slab + 1 + (kpart * kXmTilesPerWave * 8 + tcol) * G::kTileStride;
+  const _Float16* xcol = xs + col * kXmColStride + kpart * kXmTilesPerWave * 16 + 4 * q;
+
+  for (int kt0 = 0; kt0 < kt_n; kt0 += kXmChunkTiles) {
+    const int cnt = min(kXmChunkTiles, kt_n - kt0);       // a multiple of 8
+    const int ngl = cnt >> 3;
+    if (kt0 != 0) __syncthreads();                          // the previous pass has been read
+    stage(cnt);
+    if (kt0 + kXmChunkTiles < kt_n) request(kt0 + kXmChunkTiles, min(kXmChunkTiles, kt_n - kt0 - kXmChunkTiles));
+    __syncthreads();
+    // this wavefront's tile column and its share of every group's 8 k-tiles; a group's window dwords are
+    // read while the group before it is decoded, the B fragments right before their matrix instructions
+    uint32_t cw[2][kXmTilesPerWave][kWin][2];
+    auto fetch_group = [&](int gl, int buf) {
+#pragma unroll
+      for (int i = 0; i < kXmTilesPerWave; i++) ln.fetch(wcol + (gl * 8 + i) * 8 * G::kTileStride, cw[buf][i]);
+    };
+    auto compute_group = [&](int gl, int buf) {
+#pragma unroll
+      for (int i = 0; i < kXmTilesPerWave; i++) {
+        const f16x4_t a = ln.template decode<CB>(cw[buf][i]);
+        const _Float16* xb = xcol + (gl * 8 + i) * 16;
+#pragma unroll
+        for (int rb = 0; rb < kXpRowBlocks; rb++) {
+          const f16x4_t b = *reinterpret_cast<const f16x4_t*>(xb + rb * 16 * kXmColStride);
+          acc[rb] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, acc[rb], 0, 0, 0);
+        }
+      }
+    };
+    fetch_group(0, 0);
+    for (int gl = 0; gl < ngl; gl += 2) {
+      if (gl + 1 < ngl) fetch_group(gl + 1, 1);
+      compute_group(gl, 0);
+      if (gl + 1 < ngl) {
+        if (gl + 2 < ngl) fetch_group(gl + 2, 0);
+        compute_group(gl + 1, 1);
+      }
+    }
+  }
+
+  // ---- the sums of the workgroup's k parts meet in LDS (over the activations, which are done with)
+  __syncthreads();
+  float* yp = reinterpret_cast<float*>(xs);
+  {
+    float* dst = yp + kpart * (kXpRows * 128);
+#pragma unroll
+    for (int rb = 0; rb < kXpRowBlocks; rb++) {
+      const int r = rb * 16 + col;
+      if (r < rows)
+        *reinterpret_cast<float4*>(dst + r * 128 + tcol * 16 + 4 * q) = make_float4(acc[rb][0], acc[rb][1], acc[rb][2], acc[rb][3]);
+    }
+  }
+  __syncthreads();
+  // ---- output side: rotate the 128 sums of each row, svh, bias; 32 lanes per row
+  {
+    const int hw = tid >> 5, l32 = tid & 31;
+    const int n = grp * 128 + 4 * l32;
+    uint2 sraw;
+    __builtin_memcpy(&sraw, __builtin_assume_aligned(svh + n, 8), 8);
+    const float svf[4] = {f16_bits_to_f32((uint16_t)sraw.x), f16_bits_to_f32((uint16_t)(sraw.x >> 16)),
+                          f16_bits_to_f32((uint16_t)sraw.y), f16_bits_to_f32((uint16_t)(sraw.y >> 16))};
+    float bv[4] = {0.f, 0.f, 0.f, 0.f};
+    if (bias) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) bv[i] = load_bias(bias, bias_dtype, n + i);
+    }
+    for (int r = hw; r < rows; r += kXmThreads / 32) {
+      float v[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kp = 0; kp < kXmKSplit; kp++) {
+        const float4 t = *reinterpret_cast<const float4*>(yp + kp * (kXpRows * 128) + r * 128 + 4 * l32);
+        v[0] += t.x; v[1] += t.y; v[2] += t.z; v[3] += t.w;
+      }
+      fwht128_quad(v, lane);
+      float o[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) o[i] = v[i] * 0.08838834764831845f * svf[i] + bv[i];
+      *reinterpret_cast<float4*>(y + (int64_t)(t0 + r) * n_out + n) = make_float4(o[0], o[1], o[2], o[3]);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------ launch
+bool gemm_exl3_preferred(int64_t m, int64_t n_out, int64_t n_in) {
+  // worth it once the 64-row workgroups cover at least half of the compute units; below that the decode
+  // kernel's 8-row groups spread over more of them
+  const int64_t wgs = (n_out / 128) * ((m + kXpRows - 1) / kXpRows);
+  return m >= 16 && n_in % 128 == 0 && wgs * 2 >= device_num_cus();
+}
+
+template <int BITS>
+static hipError_t xp_launch(const uint16_t* trellis, const uint16_t* svh, const uint16_t* xr, float* y,
+                            const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, int cb,
+                            hipStream_t s) {
+  const dim3 grid((unsigned)(n_out / 128), (unsigned)((m + kXpRows - 1) / kXpRows)), block(kXmThreads);
+  if (cb == 0)
+    hipLaunchKernelGGL((gemm_exl3_mfma_kernel<BITS, 0>), grid, block, 0, s, trellis, svh, xr, y, bias, bias_dtype,
+                       (int)m, (int)n_out, (int)n_in);
+  else
+    hipLaunchKernelGGL((gemm_exl3_mfma_kernel<BITS, 1>), grid, block, 0, s, trellis, svh, xr, y, bias, bias_dtype,
+                       (int)m, (int)n_out, (int)n_in);
+  return hipGetLastError();
+}
+
+// The rotated activations of up to kXpMaxRows rows, per (device, stream), grown on demand.
+namespace {
+constexpr int64_t kXpMaxRows = 4096;
+struct XrBuf { uint16_t* p; size_t bytes; };
+std::mutex g_xr_mutex;
+std::unordered_map<uint64_t, XrBuf> g_xr;
+
+hipError_t xr_workspace(hipStream_t s, size_t bytes, uint16_t** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t key = ((uint64_t)(uint32_t)dev << 48) ^ (uint64_t)reinterpret_cast<uintptr_t>(s);
+  std::lock_guard<std::mutex> lock(g_xr_mutex);
+  XrBuf& b = g_xr[key];
+  if (b.bytes < bytes) {
+    if (b.p) {
+      // earlier launches on the stream may still read the old buffer
+      e = hipStreamSynchronize(s);
+      if (e != hipSuccess) return e;
+      (void)hipFree(b.p);
+      b.p = nullptr;
+      b.bytes = 0;
+    }
+    void* p = nullptr;
+    e = hipMalloc(&p, bytes);
+    if (e != hipSuccess) return e;
+    b.p = static_cast<uint16_t*>(p);
+    b.bytes = bytes;
+  }
+  *out = b.p;
+  return hipSuccess;
+}
+}  // namespace
+
+hipError_t launch_gemm_exl3(const uint16_t* trellis, const uint16_t* suh, const uint16_t* svh, const void* x,
+                            int x_dtype, float* y, const void* bias, int bias_dtype, int64_t m, int64_t n_out,
+                            int64_t n_in, int bits, int cb, hipStream_t s) {
+  if (m == 0 || n_out == 0) return hipSuccess;
+  const int64_t block_rows = m < kXpMaxRows ? m : kXpMaxRows;
+  uint16_t* xr = nullptr;
+  hipError_t e = xr_workspace(s, (size_t)block_rows * n_in * sizeof(uint16_t), &xr);
+  if (e != hipSuccess) return e;
+  const int64_t xsize = x_dtype == kF32 ? 4 : 2;
+  for (int64_t r0 = 0; r0 < m; r0 += kXpMaxRows) {
+    const int64_t rows = m - r0 < kXpMaxRows ? m - r0 : kXpMaxRows;
+    const char* xb = static_cast<const char*>(x) + r0 * n_in * xsize;
+    const int groups_per_row = (int)(n_in / 128);
+    const int64_t items = rows * groups_per_row;
+    const dim3 rgrid((unsigned)((items + 7) / 8)), rblock(256);
+    switch (x_dtype) {
+      case kF32:
+        hipLaunchKernelGGL(exl3_rotate_rows_kernel<float>, rgrid, rblock, 0, s, reinterpret_cast<const float*>(xb), suh,
+                           xr, items, groups_per_row, n_in);
+        break;
+      case kF16:
+        hipLaunchKernelGGL(exl3_rotate_rows_kernel<f16_tag>, rgrid, rblock, 0, s, reinterpret_cast<const f16_tag*>(xb),
+                           suh, xr, items, groups_per_row, n_in);
+        break;
+      case kBF16:
+        hipLaunchKernelGGL(exl3_rotate_rows_kernel<bf16_tag>, rgrid, rblock, 0, s, reinterpret_cast<const bf16_tag*>(xb),
+                           suh, xr, items, groups_per_row, n_in);
+        break;
+      default: return hipErrorInvalidValue;
+    }
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    float* yb = y + r0 * n_out;
+    switch (bits) {
+      case 1: e = xp_launch<1>(trellis, svh, xr, yb, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
+      case 2: e = xp_launch<2>(trellis, svh, xr, yb, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
+      case 3: e = xp_launch<3>(trellis, svh, xr, yb, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
+      case 4: e = xp_launch<4>(trellis, svh, xr, yb, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
+      case 5: e = xp_launch<5>(trellis, svh, xr, yb, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
+      case 6: e = xp_launch<6>(trellis, svh, xr, yb, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
+      case 7: e = xp_launch<7>(trellis, svh, xr, yb, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
+      case 8: e = xp_launch<8>(trellis, svh, xr, yb, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
+      default: return hipErrorInvalidValue;
+    }
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+
+}  // namespace ttq

@@ -166,6 +166,13 @@ hipError_t launch_gemv_exl3(const uint16_t* trellis, const uint16_t* suh, const 
 hipError_t launch_hadamard128(float* v, const uint16_t* pre, const uint16_t* post, int64_t n,
                               hipStream_t s);
 
+// Trellis layer for many activation rows (ttq_exl3_prefill.hip): activations rotated once into a workspace
+// the library keeps per (device, stream), then 64 rows per decoded weight.  y fp32.
+bool gemm_exl3_preferred(int64_t m, int64_t n_out, int64_t n_in);
+hipError_t launch_gemm_exl3(const uint16_t* trellis, const uint16_t* suh, const uint16_t* svh, const void* x,
+                            int x_dtype, float* y, const void* bias, int bias_dtype, int64_t m, int64_t n_out,
+                            int64_t n_in, int bits, int cb, hipStream_t s);
+
 // Matrix-core trellis GEMV in one launch (ttq_exl3_mfma.hip).  The plan says how the reduction
 // dimension is sliced and how many 64-bit accumulator words a sliced launch needs (zero before and
 // after every launch).

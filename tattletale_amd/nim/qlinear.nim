@@ -39,6 +39,8 @@ proc gemv_exl3*(trellis, suh, svh, x: ptr uint16, y: ptr cfloat, m, n_out, n_in:
                 bits, codebook: cint, stream: pointer): cint {.ttq.}
 proc gemv_exl3_noalloc*(trellis, suh, svh, x: ptr uint16, y: ptr cfloat, m, n_out, n_in: int64,
                         bits, codebook: cint, stream: pointer): cint {.ttq.}
+proc gemm_exl3*(trellis, suh, svh: ptr uint16, x: pointer, x_dtype: cint, y: ptr cfloat, m, n_out, n_in: int64,
+                bits, codebook: cint, stream: pointer): cint {.ttq.}
 proc gemm_q4_k*(w: pointer, x, y: ptr uint16, m, n_out, n_in: int64, stream: pointer): cint {.ttq.}
 proc gemm_q6_k*(w: pointer, x, y: ptr uint16, m, n_out, n_in: int64, stream: pointer): cint {.ttq.}
 proc gemm_q8_0*(w: pointer, x, y: ptr uint16, m, n_out, n_in: int64, stream: pointer): cint {.ttq.}

@@ -204,6 +204,25 @@ def gemv_exl3(trellis: torch.Tensor, suh: torch.Tensor, svh: torch.Tensor, x: to
     return out
 
 
+def gemm_exl3(trellis: torch.Tensor, suh: torch.Tensor, svh: torch.Tensor, x: torch.Tensor,
+              n_out: int, n_in: int, bits: int, codebook: int = _lib.CB_MCG) -> torch.Tensor:
+    """fp32 y (m, n_out) for many activation rows through ``ttq_gemm_exl3`` (activations rotated once,
+    rounded to float16; every weight decoded once per 64 rows)."""
+    dev = _require_device(trellis, suh, svh, x)
+    if suh.dtype != torch.float16 or svh.dtype != torch.float16:
+        raise TtqError(_lib.ERR_DTYPE, "ttq_gemm_exl3: suh/svh must be float16")
+    if suh.numel() != n_in or svh.numel() != n_out:
+        raise TtqError(_lib.ERR_SHAPE, "ttq_gemm_exl3: suh/svh length")
+    _check_packed("ttq_gemm_exl3", trellis, _lib.EXL3, n_out, n_in, bits)
+    m = _rows("ttq_gemm_exl3", x, n_in)
+    out = torch.empty((m, n_out), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        check(_lib.lib().ttq_gemm_exl3(trellis.data_ptr(), suh.data_ptr(), svh.data_ptr(), x.data_ptr(),
+                                       _code(x.dtype), out.data_ptr(), m, n_out, n_in, bits, codebook,
+                                       _stream(dev)), "ttq_gemm_exl3")
+    return out
+
+
 _GEMM_ENTRY = {_lib.Q4_K: "ttq_gemm_q4_k", _lib.Q6_K: "ttq_gemm_q6_k", _lib.Q8_0: "ttq_gemm_q8_0"}
 
 

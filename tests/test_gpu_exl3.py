@@ -139,3 +139,66 @@ def test_exl3_forward_other_activation_types_and_ranges(xk):
     y = layer.forward(xd, out_dtype=torch.float32).cpu().numpy()
     for i in range(4):
         assert rel_l2(y[i], by_matrices(xf[i])) <= TOL, i
+
+
+def _exl3_f64_rows(T_bits, suh_bits, svh_bits, xf):
+    """The oracle's operator in matrix form, for many rows at once (pinned against ora_exl3_gemv_f64 below)."""
+    from scipy.linalg import hadamard
+    H = hadamard(128).astype(np.float64) / np.sqrt(128.0)
+    Tf = oracle.f16_to_f32(T_bits).astype(np.float64)
+    su, sv = oracle.f16_to_f32(suh_bits).astype(np.float64), oracle.f16_to_f32(svh_bits).astype(np.float64)
+    m = xf.shape[0]
+    xr = ((xf.astype(np.float64) * su).reshape(m, -1, 128) @ H.T).reshape(m, -1)
+    return ((xr @ Tf.T).reshape(m, -1, 128) @ H.T).reshape(m, -1) * sv
+
+
+@pytest.mark.parametrize("bits,cb", [(3, F.CB_MCG), (2, F.CB_3INST), (4, F.CB_MCG), (6, F.CB_3INST), (8, F.CB_MCG)])
+@pytest.mark.parametrize("n_out,n_in,m", [(256, 512, 16), (384, 1024 + 128, 70), (1024, 2048, 333)])
+def test_exl3_prefill_rows(bits, cb, n_out, n_in, m):
+    """Many activation rows through ttq_gemm_exl3 (activations rotated once and rounded to fp16: the
+    2e-2 class, in practice below 1e-3), row by row against the oracle."""
+    w = Q.fill_normal(800 + bits, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
+    tr, suh, svh = Q.quantize_exl3(w, bits, cb, seed=bits)
+    T = oracle.exl3_decode(tr, n_out, n_in, bits, cb)
+    x = Q.f32_to_f16(Q.fill_normal(801, 1, 1.0, m * n_in).reshape(m, n_in))
+    y = QL.gemm_exl3(packed_to_dev(tr), bits_to_dev(suh, "f16"), bits_to_dev(svh, "f16"), bits_to_dev(x, "f16"),
+                     n_out, n_in, bits, cb).cpu().numpy()
+    want = _exl3_f64_rows(T, suh, svh, oracle.f16_to_f32(x))
+    for i in (0, m // 2, m - 1):        # the matrix form is the oracle's function
+        assert rel_l2(want[i], oracle.exl3_gemv_f64(T, suh, svh, x[i])) <= 1e-12
+    worst = max(rel_l2(y[i], want[i]) for i in range(m))
+    assert worst <= 2e-2
+    assert worst <= 1.5e-3                # what the fp16 rounding of the rotated activations costs
+
+
+@pytest.mark.parametrize("xk", ["bf16", "f32", "f16"])
+def test_exl3_forward_takes_the_prefill_path_and_the_flag_pins_the_decode_class(xk):
+    from util import x_to_dev
+    n_out, n_in, bits, m = 4096, 1024, 3, 512
+    w = Q.fill_normal(810, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
+    tr, suh, svh = Q.quantize_exl3(w, bits, F.CB_MCG, seed=5)
+    T = oracle.exl3_decode(tr, n_out, n_in, bits, F.CB_MCG)
+    bias = Q.fill_normal(811, 2, 0.5, n_out)
+    xd, xf = x_to_dev(Q.fill_normal(812, 1, 1.0, m * n_in).reshape(m, n_in), xk)
+    want = _exl3_f64_rows(T, suh, svh, xf) + bias
+    common = dict(bias=torch.from_numpy(bias).to(DEV), suh=bits_to_dev(suh, "f16"), svh=bits_to_dev(svh, "f16"), bits=bits)
+    auto = QuantLinear.init(packed_to_dev(tr), F.EXL3, n_in, n_out, **common)
+    y = auto.forward(xd, out_dtype=torch.float32).cpu().numpy()
+    assert max(rel_l2(y[i], want[i]) for i in range(0, m, 7)) <= 2e-2
+    exact = QuantLinear.init(packed_to_dev(tr), F.EXL3, n_in, n_out, precision=F.PRECISION_F32_SCALES, **common)
+    ye = exact.forward(xd, out_dtype=torch.float32).cpu().numpy()
+    assert max(rel_l2(ye[i], want[i]) for i in range(0, m, 7)) <= 1e-4       # two-term activations: fp32 class
+    assert not np.array_equal(y, ye)                                          # the two paths really differ
+
+
+def test_exl3_prefill_full_shape_4096x4096_m512_sampled_rows():
+    cfg = CFG.CONFIGS["exl3_gemv"]
+    tr, suh, svh = CFG.packed_weights(cfg)
+    T = oracle.exl3_decode(tr, cfg.n_out, cfg.n_in, cfg.bits, F.CB_MCG)
+    m = 512
+    x = Q.f32_to_f16(Q.fill_normal(820, 1, 1.0, m * cfg.n_in).reshape(m, cfg.n_in))
+    y = QL.gemm_exl3(packed_to_dev(tr), bits_to_dev(suh, "f16"), bits_to_dev(svh, "f16"), bits_to_dev(x, "f16"),
+                     cfg.n_out, cfg.n_in, cfg.bits, F.CB_MCG).cpu().numpy()
+    assert np.all(np.isfinite(y))
+    for i in (0, 63, 64, 255, 448, 511):
+        assert rel_l2(y[i], oracle.exl3_gemv_f64(T, suh, svh, x[i])) <= 2e-2, i
