@@ -248,6 +248,9 @@ int ttq_gemv_q4_k_silu_mul(const void* w, const void* x, int x_dtype, void* y, i
   if (m == 0 || n_ff == 0) return TTQ_OK;
   if (!w || !x || !y) return TTQ_ERR_NULL;
   if (!aligned16(w) || !aligned16(x) || !aligned16(y)) return TTQ_ERR_ALIGN;
+  if (m <= 4 && ttq::gemv_q4k_stream_fused_supported(x_dtype, n_ff, n_in))
+    return hip_status(ttq::launch_gemv_q4k_stream_fused(w, x, x_dtype, y, y_dtype, m, n_ff, n_in,
+                                                        static_cast<hipStream_t>(stream)));
   if (!ttq::gemv_fused_supported(TTQ_Q4_K, x_dtype, n_ff, n_in, true)) return TTQ_ERR_UNSUPPORTED;
   return hip_status(ttq::launch_gemv_fused(w, x, x_dtype, y, y_dtype, nullptr, 0, m, n_ff, n_in, true, nullptr,
                                            nullptr, 0.f, nullptr, nullptr, static_cast<hipStream_t>(stream)));

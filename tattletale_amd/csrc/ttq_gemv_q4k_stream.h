@@ -69,7 +69,12 @@ __device__ __forceinline__ st_u32x4 st_read1(uint32_t a) {
 
 // XT: bf16 or fp16 activations.  STAGE 0 is the GEMV; STAGE 1 leaves out the arithmetic (requests,
 // waits, LDS reads and the activation prologue stay) and exists for the roofline ladder of bench.py.
-template <typename XT, typename YT, int STAGE>
+// FUSE: the weight holds gate rows [0, n_out) followed by up rows [n_out, 2 n_out), as GatedMLP builds it
+// (workspace/transformers/src/layers/mlp.nim:39), and the kernel writes silu(gate . x) * (up . x), the
+// silu_and_mul of workspace/transformers/src/kernels/activations.nim:14-38: a workgroup takes the gate row
+// groups of its outputs, then the up row groups of the same outputs, and pairs their sums at the end.
+// n_out and rows_per_wg count outputs.
+template <typename XT, typename YT, int STAGE, bool FUSE = false>
 __global__ void __launch_bounds__(kStThreads)
 gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
                        const void* __restrict__ bias, int bias_dtype, int n_out, int nsb, int rows_per_wg) {
@@ -89,7 +94,8 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   const int wg_row0 = blockIdx.x * rows_per_wg;
   const int wg_row_end = min(wg_row0 + rows_per_wg, n_out);
   const int last = wg_row_end - 1;
-  const int nblocks = ((wg_row_end - wg_row0 + 15) >> 4) << nks_log2;    // <= kStMaxBlocks (the launcher sees to it)
+  const int ngroups = (wg_row_end - wg_row0 + 15) >> 4;                  // row groups of 16 outputs
+  const int nblocks = ((FUSE ? 2 : 1) * ngroups) << nks_log2;            // <= kStMaxBlocks (the launcher sees to it)
   uint8_t* mybuf = wbuf + wave * kStBlockBytes;
 
   // ---- activations first, also as an LDS request (a register load among the weight requests
@@ -114,7 +120,14 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
 #pragma unroll
     for (int o = 0; o < 2; o++) {
       const int row16 = 8 * o + r8;
-      const int row = min(wg_row0 + rg * 16 + row16, last);   // past the end: the last row again, never used
+      // past the end: the last row again, never used
+      int row;
+      if (FUSE) {
+        const int up = rg >= ngroups ? 1 : 0;
+        row = up * n_out + min(wg_row0 + (rg - up * ngroups) * 16 + row16, last);
+      } else {
+        row = min(wg_row0 + rg * 16 + row16, last);
+      }
       lane_off[o] = (uint32_t)row * rb + (uint32_t)(ks * kStSegBytes) + (uint32_t)(((lane & 7) ^ ((row16 >> 1) & 7)) * 16);
     }
   };
@@ -347,12 +360,18 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   for (; blk < nblocks; blk += kStWaves) run_block(blk);
   // every request has landed (plain loads and barriers are safe again); the blocks of a row group add up
   __syncthreads();
-  for (int t = tid; t < (nblocks >> nks_log2) * 16; t += kStThreads) {
+  for (int t = tid; t < ngroups * 16; t += kStThreads) {
     const int grp = t >> 4, nn = t & 15;
     float v = part[grp << nks_log2][nn];
     if (nks_log2) v += part[(grp << 1) + 1][nn];
     const int row = wg_row0 + t;
-    if (row < wg_row_end) YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
+    if (FUSE) {
+      float u = part[(ngroups + grp) << nks_log2][nn];
+      if (nks_log2) u += part[((ngroups + grp) << 1) + 1][nn];
+      if (row < wg_row_end) YElem<YT>::store(ym, row, (v / (1.f + expf(-v))) * u);
+    } else {
+      if (row < wg_row_end) YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
+    }
   }
 }
 
@@ -366,13 +385,13 @@ inline int st_rows_per_wg(int64_t n_out, int* num_wg_out) {
   return rows_per_wg;
 }
 
-template <typename XT, typename YT, int STAGE>
+template <typename XT, typename YT, int STAGE, bool FUSE = false>
 inline hipError_t st_launch_xy(const void* w, const void* x, void* y, const void* bias, int bias_dtype, int64_t m,
                                int64_t n_out, int64_t n_in, hipStream_t s) {
   int num_wg = 0;
   const int rows_per_wg = st_rows_per_wg(n_out, &num_wg);
   const dim3 grid((unsigned)num_wg, (unsigned)m), block(kStThreads);
-  hipLaunchKernelGGL((gemv_q4k_stream_kernel<XT, YT, STAGE>), grid, block, 0, s, static_cast<const uint8_t*>(w),
+  hipLaunchKernelGGL((gemv_q4k_stream_kernel<XT, YT, STAGE, FUSE>), grid, block, 0, s, static_cast<const uint8_t*>(w),
                      static_cast<const uint16_t*>(x), static_cast<YT*>(y), bias, bias_dtype, (int)n_out,
                      (int)(n_in / 256), rows_per_wg);
   return hipGetLastError();

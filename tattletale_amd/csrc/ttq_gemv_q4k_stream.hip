@@ -13,6 +13,33 @@ bool gemv_q4k_stream_supported(int format, int x_dtype, int64_t n_out, int64_t n
   return n_out >= 16 * device_num_cus() && blocks <= kStMaxBlocks && n_out * (n_in / 256) * 144 < ((int64_t)1 << 32);
 }
 
+// The gate || up form: n_ff outputs from 2 n_ff weight rows.  At least 8 outputs per compute unit (16 weight rows),
+// and the two parts' row groups together within the block table.
+bool gemv_q4k_stream_fused_supported(int x_dtype, int64_t n_ff, int64_t n_in) {
+  if (!(x_dtype == kBF16 || x_dtype == kF16)) return false;
+  if (n_in != 4096 && n_in != 2048) return false;
+  const int64_t blocks = 2 * (((int64_t)st_rows_per_wg(n_ff, nullptr) + 15) / 16) * (n_in / 2048);
+  return n_ff >= 8 * device_num_cus() && blocks <= kStMaxBlocks && 2 * n_ff * (n_in / 256) * 144 < ((int64_t)1 << 32);
+}
+
+template <typename XT>
+static hipError_t st_launch_fused_x(const void* w, const void* x, void* y, int y_dtype, int64_t m, int64_t n_ff,
+                                    int64_t n_in, hipStream_t s) {
+  switch (y_dtype) {
+    case kF32: return st_launch_xy<XT, float, 0, true>(w, x, y, nullptr, 0, m, n_ff, n_in, s);
+    case kF16: return st_launch_xy<XT, f16_tag, 0, true>(w, x, y, nullptr, 0, m, n_ff, n_in, s);
+    case kBF16: return st_launch_xy<XT, bf16_tag, 0, true>(w, x, y, nullptr, 0, m, n_ff, n_in, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+hipError_t launch_gemv_q4k_stream_fused(const void* w, const void* x, int x_dtype, void* y, int y_dtype, int64_t m,
+                                        int64_t n_ff, int64_t n_in, hipStream_t s) {
+  if (x_dtype == kBF16) return st_launch_fused_x<bf16_tag>(w, x, y, y_dtype, m, n_ff, n_in, s);
+  if (x_dtype == kF16) return st_launch_fused_x<f16_tag>(w, x, y, y_dtype, m, n_ff, n_in, s);
+  return hipErrorInvalidValue;
+}
+
 template <typename XT>
 static hipError_t st_launch_x(const void* w, const void* x, void* y, int y_dtype, const void* bias, int bias_dtype,
                               int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {

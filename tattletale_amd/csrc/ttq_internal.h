@@ -82,6 +82,10 @@ hipError_t launch_gemv_q8_mfma(const void* w, const void* x, int x_dtype, void* 
 // front (norm_gamma != null; residual / outputs optional) and optional gate/up + silu_and_mul
 // behind (w then holds 2*n_out rows, gate rows first).
 bool gemv_fused_supported(int format, int x_dtype, int64_t n_out, int64_t n_in, bool silu_mul);
+// gate || up + silu_and_mul on the LDS-streamed kernel (ttq_gemv_q4k_stream.hip): Q4_K, 16-bit activations
+bool gemv_q4k_stream_fused_supported(int x_dtype, int64_t n_ff, int64_t n_in);
+hipError_t launch_gemv_q4k_stream_fused(const void* w, const void* x, int x_dtype, void* y, int y_dtype, int64_t m,
+                                        int64_t n_ff, int64_t n_in, hipStream_t s);
 hipError_t launch_gemv_fused(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
                              const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                              bool silu_mul, const void* norm_residual, const void* norm_gamma,

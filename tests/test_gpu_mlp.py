@@ -35,7 +35,8 @@ def test_silu_and_mul_elementwise(dt, ulp, tiny, m, h):
 
 
 @pytest.mark.parametrize("xk", ["bf16", "f16"])
-@pytest.mark.parametrize("n_ff,n_in", [(16, 256), (100, 1024), (1000, 4096), (3000, 512), (20000, 256), (777, 8192), (520, 14336)])
+@pytest.mark.parametrize("n_ff,n_in", [(16, 256), (100, 1024), (1000, 4096), (3000, 512), (20000, 256), (777, 8192), (520, 14336),
+                                       (2048, 4096), (2100, 2048), (5000, 4096), (7177, 2048)])
 def test_fused_gate_up_silu_mul_gemv(xk, n_ff, n_in):
     """Every split of outputs and super-blocks over the wavefronts (one or several rounds, 1 to 8
     slices, ragged last group), two activation rows."""
@@ -236,7 +237,12 @@ def test_fused_rmsnorm_full_shape_gate_up():
     assert torch.equal(new_res, new_res_ref)
     assert bool(((normed.float() - normed_ref.float()).abs() <= 2.0 ** -7 * normed_ref.float().abs()).all())
     y_ref = QL.gemv_q4_k_silu_mul(packed_to_dev(p), normed, n_ff, n_in, out_dtype=torch.bfloat16)
-    assert torch.equal(y, y_ref) and bool(torch.isfinite(y.float()).all())
+    # the two entry points may run different kernels (different summation order): equal to the rounding of
+    # the bf16 output, and against each other well inside the decode tolerance
+    assert bool(torch.isfinite(y.float()).all())
+    yf, yr = y.float().cpu().numpy(), y_ref.float().cpu().numpy()
+    assert rel_l2(yf, yr) <= 1e-3
+    assert np.all(np.abs(yf - yr) <= 2.0 ** -7 * np.abs(yr) + 1e-30)
 
 
 # ------------------------------------------------------------------ prefill: silu_and_mul in the GEMM epilogue
