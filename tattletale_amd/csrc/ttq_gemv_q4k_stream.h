@@ -40,6 +40,12 @@ constexpr int kStHalfBytes = 8 * kStSegBytes;             // eight rows: [line 9
 constexpr int kStBlockBytes = 2 * kStHalfBytes;           // 18432
 constexpr int kStBlockRequests = 2 * kStLines;            // 18
 constexpr int kStUpFront = 6;                             // requests before the first super-block (even)
+// With one or two blocks per workgroup only one or two wavefronts carry the whole stream, and six requests in
+// flight each would leave it latency-bound: those launches ask for 16 of a block's 18 at once (the last
+// request's slot holds the activations until they have been read back).  4096x4096: 4.53 -> 4.28 us.  Sharing
+// the landed super-blocks among all 8 wavefronts after a wait-for-all and a barrier was measured too: slower
+// (4.54 us; 6144x4096 4.77 -> 6.03 us), the pipelined consumption by the owners wins.
+constexpr int kStUpFrontFew = 16;
 constexpr int kStMaxSb = 16;                              // n_in <= 4096: one staging pass, 8 KiB table
 constexpr int kStMaxBlocks = 80;                          // blocks of a workgroup (their row sums wait in LDS)
 
@@ -74,7 +80,7 @@ __device__ __forceinline__ st_u32x4 st_read1(uint32_t a) {
 // silu_and_mul of workspace/transformers/src/kernels/activations.nim:14-38: a workgroup takes the gate row
 // groups of its outputs, then the up row groups of the same outputs, and pairs their sums at the end.
 // n_out and rows_per_wg count outputs.
-template <typename XT, typename YT, int STAGE, bool FUSE = false>
+template <typename XT, typename YT, int STAGE, bool FUSE = false, int UP = kStUpFront>
 __global__ void __launch_bounds__(kStThreads)
 gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
                        const void* __restrict__ bias, int bias_dtype, int n_out, int nsb, int rows_per_wg) {
@@ -142,13 +148,13 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   if (have_block) {
     set_block(blk);
 #pragma unroll
-    for (int i = 0; i < kStUpFront; i++) request(i);
+    for (int i = 0; i < UP; i++) request(i);
   }
 
   // ---- the raw activations back into registers
   float xf[8];
   if (xok) {
-    if (have_block) st_wait_vmcnt<kStUpFront>();
+    if (have_block) st_wait_vmcnt<UP>();
     else st_wait_vmcnt<0>();
     const st_u32x4 r = st_read1((uint32_t)(size_t)(st_lptr_t)(xland) + (uint32_t)(lane * 16));
     widen8<XT>(make_uint4(r[0], r[1], r[2], r[3]), xf);
@@ -238,15 +244,15 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   uint32_t a_addr[4], tab_addr = tab_addr0;
   auto topup = [&](auto sc) {
     constexpr int s = decltype(sc)::value;
-    if constexpr (kStUpFront + 2 * s < kStBlockRequests) {
-      request(kStUpFront + 2 * s);
-      request(kStUpFront + 2 * s + 1);
+    if constexpr (UP + 2 * s < kStBlockRequests) {
+      request(UP + 2 * s);
+      request(UP + 2 * s + 1);
     }
   };
   auto issue = [&](auto sc, Regs& r) {
     constexpr int s = decltype(sc)::value;
     // super-block s needs requests 0 .. 2 s + 3; two more are made first while there are any
-    constexpr int kIssued = kStUpFront + 2 * (s + 1) < kStBlockRequests ? kStUpFront + 2 * (s + 1) : kStBlockRequests;
+    constexpr int kIssued = UP + 2 * (s + 1) < kStBlockRequests ? UP + 2 * (s + 1) : kStBlockRequests;
     topup(sc);
     st_wait_vmcnt<kIssued - (2 * s + 4)>();
     const uint32_t ta = tab_addr;
@@ -344,7 +350,7 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
     if (next < nblocks) {
       set_block(next);
 #pragma unroll
-      for (int i = 0; i < kStUpFront; i++) request(i);
+      for (int i = 0; i < UP; i++) request(i);
     }
     compute(rb2);
     // the four k-groups of a row
@@ -391,9 +397,15 @@ inline hipError_t st_launch_xy(const void* w, const void* x, void* y, const void
   int num_wg = 0;
   const int rows_per_wg = st_rows_per_wg(n_out, &num_wg);
   const dim3 grid((unsigned)num_wg, (unsigned)m), block(kStThreads);
-  hipLaunchKernelGGL((gemv_q4k_stream_kernel<XT, YT, STAGE, FUSE>), grid, block, 0, s, static_cast<const uint8_t*>(w),
-                     static_cast<const uint16_t*>(x), static_cast<YT*>(y), bias, bias_dtype, (int)n_out,
-                     (int)(n_in / 256), rows_per_wg);
+  const int blocks = (FUSE ? 2 : 1) * ((rows_per_wg + 15) / 16) * (int)(n_in / 2048);
+  if (blocks <= 2)
+    hipLaunchKernelGGL((gemv_q4k_stream_kernel<XT, YT, STAGE, FUSE, kStUpFrontFew>), grid, block, 0, s,
+                       static_cast<const uint8_t*>(w), static_cast<const uint16_t*>(x), static_cast<YT*>(y), bias,
+                       bias_dtype, (int)n_out, (int)(n_in / 256), rows_per_wg);
+  else
+    hipLaunchKernelGGL((gemv_q4k_stream_kernel<XT, YT, STAGE, FUSE>), grid, block, 0, s, static_cast<const uint8_t*>(w),
+                       static_cast<const uint16_t*>(x), static_cast<YT*>(y), bias, bias_dtype, (int)n_out,
+                       (int)(n_in / 256), rows_per_wg);
   return hipGetLastError();
 }
 
