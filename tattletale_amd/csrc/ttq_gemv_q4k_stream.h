@@ -402,6 +402,10 @@ inline hipError_t st_launch_xy(const void* w, const void* x, void* y, const void
     hipLaunchKernelGGL((gemv_q4k_stream_kernel<XT, YT, STAGE, FUSE, kStUpFrontFew>), grid, block, 0, s,
                        static_cast<const uint8_t*>(w), static_cast<const uint16_t*>(x), static_cast<YT*>(y), bias,
                        bias_dtype, (int)n_out, (int)(n_in / 256), rows_per_wg);
+  else if (blocks <= 4)
+    hipLaunchKernelGGL((gemv_q4k_stream_kernel<XT, YT, STAGE, FUSE, 12>), grid, block, 0, s,
+                       static_cast<const uint8_t*>(w), static_cast<const uint16_t*>(x), static_cast<YT*>(y), bias,
+                       bias_dtype, (int)n_out, (int)(n_in / 256), rows_per_wg);
   else
     hipLaunchKernelGGL((gemv_q4k_stream_kernel<XT, YT, STAGE, FUSE>), grid, block, 0, s, static_cast<const uint8_t*>(w),
                        static_cast<const uint16_t*>(x), static_cast<YT*>(y), bias, bias_dtype, (int)n_out,
