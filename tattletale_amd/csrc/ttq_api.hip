@@ -211,7 +211,7 @@ int ttq_gemv_exl3_noalloc(const uint16_t* trellis, const uint16_t* suh_f16, cons
     const hipError_t e = ttq::exl3_resident_workspace(&accum);
     if (e != hipSuccess) return hip_status(e);
   }
-  return hip_status(ttq::launch_gemv_exl3_mfma(plan, trellis, suh_f16, svh_f16, x_f16, TTQ_F16, y, nullptr, 0, m,
+  return hip_status(ttq::launch_gemv_exl3_mfma(plan, trellis, suh_f16, svh_f16, x_f16, TTQ_F16, y, TTQ_F32, nullptr, 0, m,
                                                n_out, n_in, bits, codebook, accum,
                                                static_cast<hipStream_t>(stream)));
 }
@@ -226,7 +226,7 @@ int ttq_gemm_exl3(const uint16_t* trellis, const uint16_t* suh_f16, const uint16
   if (!trellis || !suh_f16 || !svh_f16 || !x || !y) return TTQ_ERR_NULL;
   if (!aligned16(trellis) || !aligned16(x) || !aligned16(y) || !aligned8(suh_f16) || !aligned8(svh_f16))
     return TTQ_ERR_ALIGN;
-  return hip_status(ttq::launch_gemm_exl3(trellis, suh_f16, svh_f16, x, x_dtype, y, nullptr, 0, m, n_out, n_in, bits,
+  return hip_status(ttq::launch_gemm_exl3(trellis, suh_f16, svh_f16, x, x_dtype, y, TTQ_F32, nullptr, 0, m, n_out, n_in, bits,
                                           codebook, static_cast<hipStream_t>(stream)));
 }
 
@@ -385,14 +385,13 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
   if (layer->format == TTQ_EXL3) {
     if (!layer->suh || !layer->svh) return TTQ_ERR_NULL;
     if (!aligned8(layer->suh) || !aligned8(layer->svh)) return TTQ_ERR_ALIGN;
-    if (y_dtype != TTQ_F32) return TTQ_ERR_UNSUPPORTED;  // output rotation runs in place on fp32
     if (n_in > ttq::kMaxGemvInF32) return TTQ_ERR_UNSUPPORTED;
     // many rows: rotate the activations once (rounded to fp16) and decode every weight once per 64 rows
     if (layer->precision != TTQ_PRECISION_F32_SCALES && ttq::gemm_exl3_preferred(m, n_out, n_in))
       return hip_status(ttq::launch_gemm_exl3(
           static_cast<const uint16_t*>(layer->qweight), static_cast<const uint16_t*>(layer->suh),
-          static_cast<const uint16_t*>(layer->svh), x, x_dtype, static_cast<float*>(y), layer->bias,
-          layer->bias_dtype, m, n_out, n_in, layer->bits, layer->codebook, s));
+          static_cast<const uint16_t*>(layer->svh), x, x_dtype, y, y_dtype, layer->bias, layer->bias_dtype, m, n_out,
+          n_in, layer->bits, layer->codebook, s));
     return hip_status(ttq::launch_gemv_exl3(
         static_cast<const uint16_t*>(layer->qweight), static_cast<const uint16_t*>(layer->suh),
         static_cast<const uint16_t*>(layer->svh), x, x_dtype, y, y_dtype, layer->bias,

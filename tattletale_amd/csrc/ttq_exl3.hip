@@ -344,8 +344,6 @@ hipError_t launch_gemv_exl3(const uint16_t* trellis, const uint16_t* suh, const 
                             int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, int bits, int cb,
                             hipStream_t s) {
   if (m == 0 || n_out == 0) return hipSuccess;
-  if (y_dtype != kF32) return hipErrorInvalidValue;
-  float* yf = static_cast<float*>(y);
   hipError_t e;
   static const int two_launches = dev_knob("TTQ_EXL3_TWO_LAUNCHES", 0);
   if (!two_launches) {
@@ -355,9 +353,11 @@ hipError_t launch_gemv_exl3(const uint16_t* trellis, const uint16_t* suh, const 
       e = exl3_workspace(s, &accum);
       if (e != hipSuccess) return e;
     }
-    return launch_gemv_exl3_mfma(plan, trellis, suh, svh, x, x_dtype, yf, bias, bias_dtype, m, n_out, n_in, bits, cb,
-                                 accum, s);
+    return launch_gemv_exl3_mfma(plan, trellis, suh, svh, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, bits,
+                                 cb, accum, s);
   }
+  if (y_dtype != kF32) return hipErrorInvalidValue;     // the two-kernel form rotates an fp32 buffer in place
+  float* yf = static_cast<float*>(y);
   switch (bits) {
     case 1: e = gemv_bits<1>(trellis, suh, x, x_dtype, yf, m, n_out, n_in, cb, s); break;
     case 2: e = gemv_bits<2>(trellis, suh, x, x_dtype, yf, m, n_out, n_in, cb, s); break;

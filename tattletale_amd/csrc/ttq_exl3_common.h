@@ -100,6 +100,23 @@ __device__ __forceinline__ void xm_code(uint32_t w, uint32_t& dst) {
         : "+v"(dst) : "v"(u));
 }
 
+// Four consecutive outputs (idx a multiple of four) in the output buffer's element type.
+__device__ __forceinline__ void xm_store4(void* y, int y_dtype, int64_t idx, const float (&o)[4]) {
+  if (y_dtype == kF32) {
+    *reinterpret_cast<float4*>(static_cast<float*>(y) + idx) = make_float4(o[0], o[1], o[2], o[3]);
+  } else {
+    uint2 v;
+    if (y_dtype == kF16) {
+      v.x = (uint32_t)f32_to_f16_bits(o[0]) | ((uint32_t)f32_to_f16_bits(o[1]) << 16);
+      v.y = (uint32_t)f32_to_f16_bits(o[2]) | ((uint32_t)f32_to_f16_bits(o[3]) << 16);
+    } else {
+      v.x = pack_bf16x2(o[0], o[1]);
+      v.y = pack_bf16x2(o[2], o[3]);
+    }
+    *reinterpret_cast<uint2*>(static_cast<uint16_t*>(y) + idx) = v;
+  }
+}
+
 // Four consecutive activations as loaded (converted when they are used, so that the load can stay in flight).
 template <typename XT> struct XmRaw;
 template <> struct XmRaw<float> {

@@ -36,7 +36,7 @@ namespace ttq {
 template <int BITS, int CB, typename XT>
 __global__ void __launch_bounds__(kXmThreads)
 gemv_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __restrict__ suh,
-                      const uint16_t* __restrict__ svh, const XT* __restrict__ x, float* __restrict__ y,
+                      const uint16_t* __restrict__ svh, const XT* __restrict__ x, void* __restrict__ y, int y_dtype,
                       const void* __restrict__ bias, int bias_dtype, int m, int n_out, int n_in, int slice_tiles,
                       unsigned long long* __restrict__ accum) {
   using G = XmGeom<BITS>;
@@ -283,7 +283,7 @@ gemv_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __re
       o[i] = v[i] * 0.08838834764831845f * svf[i];
       if (bias) o[i] += load_bias(bias, bias_dtype, n + i);
     }
-    *reinterpret_cast<float4*>(y + (int64_t)(t0 + hw) * n_out + n) = make_float4(o[0], o[1], o[2], o[3]);
+    xm_store4(y, y_dtype, (int64_t)(t0 + hw) * n_out + n, o);
   }
 }
 
@@ -308,50 +308,50 @@ Exl3Plan exl3_mfma_plan(int64_t m, int64_t n_out, int64_t n_in) {
 
 template <int BITS, int CB, typename XT>
 static hipError_t xm_launch(const Exl3Plan& p, const uint16_t* trellis, const uint16_t* suh, const uint16_t* svh,
-                            const void* x, float* y, const void* bias, int bias_dtype, int64_t m, int64_t n_out,
-                            int64_t n_in, unsigned long long* accum, hipStream_t s) {
+                            const void* x, void* y, int y_dtype, const void* bias, int bias_dtype, int64_t m,
+                            int64_t n_out, int64_t n_in, unsigned long long* accum, hipStream_t s) {
   const dim3 grid((unsigned)p.groups, (unsigned)p.slices, (unsigned)p.row_groups), block(kXmThreads);
   hipLaunchKernelGGL((gemv_exl3_mfma_kernel<BITS, CB, XT>), grid, block, 0, s, trellis, suh, svh,
-                     static_cast<const XT*>(x), y, bias, bias_dtype, (int)m, (int)n_out, (int)n_in, p.slice_tiles,
+                     static_cast<const XT*>(x), y, y_dtype, bias, bias_dtype, (int)m, (int)n_out, (int)n_in, p.slice_tiles,
                      accum);
   return hipGetLastError();
 }
 
 template <int BITS, int CB>
 static hipError_t xm_launch_x(const Exl3Plan& p, const uint16_t* trellis, const uint16_t* suh, const uint16_t* svh,
-                              const void* x, int x_dtype, float* y, const void* bias, int bias_dtype, int64_t m,
+                              const void* x, int x_dtype, void* y, int y_dtype, const void* bias, int bias_dtype, int64_t m,
                               int64_t n_out, int64_t n_in, unsigned long long* accum, hipStream_t s) {
   switch (x_dtype) {
-    case kF32: return xm_launch<BITS, CB, float>(p, trellis, suh, svh, x, y, bias, bias_dtype, m, n_out, n_in, accum, s);
-    case kF16: return xm_launch<BITS, CB, f16_tag>(p, trellis, suh, svh, x, y, bias, bias_dtype, m, n_out, n_in, accum, s);
-    case kBF16: return xm_launch<BITS, CB, bf16_tag>(p, trellis, suh, svh, x, y, bias, bias_dtype, m, n_out, n_in, accum, s);
+    case kF32: return xm_launch<BITS, CB, float>(p, trellis, suh, svh, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, accum, s);
+    case kF16: return xm_launch<BITS, CB, f16_tag>(p, trellis, suh, svh, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, accum, s);
+    case kBF16: return xm_launch<BITS, CB, bf16_tag>(p, trellis, suh, svh, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, accum, s);
     default: return hipErrorInvalidValue;
   }
 }
 
 template <int BITS>
 static hipError_t xm_launch_cb(const Exl3Plan& p, const uint16_t* trellis, const uint16_t* suh, const uint16_t* svh,
-                               const void* x, int x_dtype, float* y, const void* bias, int bias_dtype, int64_t m,
+                               const void* x, int x_dtype, void* y, int y_dtype, const void* bias, int bias_dtype, int64_t m,
                                int64_t n_out, int64_t n_in, int cb, unsigned long long* accum, hipStream_t s) {
-  return cb == 0 ? xm_launch_x<BITS, 0>(p, trellis, suh, svh, x, x_dtype, y, bias, bias_dtype, m, n_out, n_in, accum, s)
-                 : xm_launch_x<BITS, 1>(p, trellis, suh, svh, x, x_dtype, y, bias, bias_dtype, m, n_out, n_in, accum, s);
+  return cb == 0 ? xm_launch_x<BITS, 0>(p, trellis, suh, svh, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, accum, s)
+                 : xm_launch_x<BITS, 1>(p, trellis, suh, svh, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, accum, s);
 }
 
 hipError_t launch_gemv_exl3_mfma(const Exl3Plan& p, const uint16_t* trellis, const uint16_t* suh,
-                                 const uint16_t* svh, const void* x, int x_dtype, float* y, const void* bias,
+                                 const uint16_t* svh, const void* x, int x_dtype, void* y, int y_dtype, const void* bias,
                                  int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, int bits, int cb,
                                  unsigned long long* accum, hipStream_t s) {
   if (m == 0 || n_out == 0) return hipSuccess;
   if (p.slices > 1 && !accum) return hipErrorInvalidValue;
   switch (bits) {
-    case 1: return xm_launch_cb<1>(p, trellis, suh, svh, x, x_dtype, y, bias, bias_dtype, m, n_out, n_in, cb, accum, s);
-    case 2: return xm_launch_cb<2>(p, trellis, suh, svh, x, x_dtype, y, bias, bias_dtype, m, n_out, n_in, cb, accum, s);
-    case 3: return xm_launch_cb<3>(p, trellis, suh, svh, x, x_dtype, y, bias, bias_dtype, m, n_out, n_in, cb, accum, s);
-    case 4: return xm_launch_cb<4>(p, trellis, suh, svh, x, x_dtype, y, bias, bias_dtype, m, n_out, n_in, cb, accum, s);
-    case 5: return xm_launch_cb<5>(p, trellis, suh, svh, x, x_dtype, y, bias, bias_dtype, m, n_out, n_in, cb, accum, s);
-    case 6: return xm_launch_cb<6>(p, trellis, suh, svh, x, x_dtype, y, bias, bias_dtype, m, n_out, n_in, cb, accum, s);
-    case 7: return xm_launch_cb<7>(p, trellis, suh, svh, x, x_dtype, y, bias, bias_dtype, m, n_out, n_in, cb, accum, s);
-    case 8: return xm_launch_cb<8>(p, trellis, suh, svh, x, x_dtype, y, bias, bias_dtype, m, n_out, n_in, cb, accum, s);
+    case 1: return xm_launch_cb<1>(p, trellis, suh, svh, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, cb, accum, s);
+    case 2: return xm_launch_cb<2>(p, trellis, suh, svh, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, cb, accum, s);
+    case 3: return xm_launch_cb<3>(p, trellis, suh, svh, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, cb, accum, s);
+    case 4: return xm_launch_cb<4>(p, trellis, suh, svh, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, cb, accum, s);
+    case 5: return xm_launch_cb<5>(p, trellis, suh, svh, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, cb, accum, s);
+    case 6: return xm_launch_cb<6>(p, trellis, suh, svh, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, cb, accum, s);
+    case 7: return xm_launch_cb<7>(p, trellis, suh, svh, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, cb, accum, s);
+    case 8: return xm_launch_cb<8>(p, trellis, suh, svh, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, cb, accum, s);
     default: return hipErrorInvalidValue;
   }
 }

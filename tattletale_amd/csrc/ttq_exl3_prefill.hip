@@ -54,7 +54,7 @@ exl3_rotate_rows_kernel(const XT* __restrict__ x, const uint16_t* __restrict__ s
 template <int BITS, int CB>
 __global__ void __launch_bounds__(kXmThreads)
 gemm_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __restrict__ svh,
-                      const uint16_t* __restrict__ xr, float* __restrict__ y, const void* __restrict__ bias,
+                      const uint16_t* __restrict__ xr, void* __restrict__ y, int y_dtype, const void* __restrict__ bias,
                       int bias_dtype, int m, int n_out, int n_in) {
   using G = XmGeom<BITS>;
   // one pass of tiles, then 64 rows of rotated activations; the epilogue's sums reuse the activations' space
@@ -200,7 +200,7 @@ gemm_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __re
       float o[4];
 #pragma unroll
       for (int i = 0; i < 4; i++) o[i] = v[i] * 0.08838834764831845f * svf[i] + bv[i];
-      *reinterpret_cast<float4*>(y + (int64_t)(t0 + r) * n_out + n) = make_float4(o[0], o[1], o[2], o[3]);
+      xm_store4(y, y_dtype, (int64_t)(t0 + r) * n_out + n, o);
     }
   }
 }
@@ -214,16 +214,16 @@ bool gemm_exl3_preferred(int64_t m, int64_t n_out, int64_t n_in) {
 }
 
 template <int BITS>
-static hipError_t xp_launch(const uint16_t* trellis, const uint16_t* svh, const uint16_t* xr, float* y,
+static hipError_t xp_launch(const uint16_t* trellis, const uint16_t* svh, const uint16_t* xr, void* y, int y_dtype,
                             const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, int cb,
                             hipStream_t s) {
   const dim3 grid((unsigned)(n_out / 128), (unsigned)((m + kXpRows - 1) / kXpRows)), block(kXmThreads);
   if (cb == 0)
-    hipLaunchKernelGGL((gemm_exl3_mfma_kernel<BITS, 0>), grid, block, 0, s, trellis, svh, xr, y, bias, bias_dtype,
-                       (int)m, (int)n_out, (int)n_in);
+    hipLaunchKernelGGL((gemm_exl3_mfma_kernel<BITS, 0>), grid, block, 0, s, trellis, svh, xr, y, y_dtype, bias,
+                       bias_dtype, (int)m, (int)n_out, (int)n_in);
   else
-    hipLaunchKernelGGL((gemm_exl3_mfma_kernel<BITS, 1>), grid, block, 0, s, trellis, svh, xr, y, bias, bias_dtype,
-                       (int)m, (int)n_out, (int)n_in);
+    hipLaunchKernelGGL((gemm_exl3_mfma_kernel<BITS, 1>), grid, block, 0, s, trellis, svh, xr, y, y_dtype, bias,
+                       bias_dtype, (int)m, (int)n_out, (int)n_in);
   return hipGetLastError();
 }
 
@@ -262,8 +262,8 @@ hipError_t xr_workspace(hipStream_t s, size_t bytes, uint16_t** out) {
 }  // namespace
 
 hipError_t launch_gemm_exl3(const uint16_t* trellis, const uint16_t* suh, const uint16_t* svh, const void* x,
-                            int x_dtype, float* y, const void* bias, int bias_dtype, int64_t m, int64_t n_out,
-                            int64_t n_in, int bits, int cb, hipStream_t s) {
+                            int x_dtype, void* y, int y_dtype, const void* bias, int bias_dtype, int64_t m,
+                            int64_t n_out, int64_t n_in, int bits, int cb, hipStream_t s) {
   if (m == 0 || n_out == 0) return hipSuccess;
   const int64_t block_rows = m < kXpMaxRows ? m : kXpMaxRows;
   uint16_t* xr = nullptr;
@@ -293,16 +293,16 @@ hipError_t launch_gemm_exl3(const uint16_t* trellis, const uint16_t* suh, const 
     }
     e = hipGetLastError();
     if (e != hipSuccess) return e;
-    float* yb = y + r0 * n_out;
+    void* yb = static_cast<char*>(y) + r0 * n_out * (y_dtype == kF32 ? 4 : 2);
     switch (bits) {
-      case 1: e = xp_launch<1>(trellis, svh, xr, yb, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
-      case 2: e = xp_launch<2>(trellis, svh, xr, yb, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
-      case 3: e = xp_launch<3>(trellis, svh, xr, yb, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
-      case 4: e = xp_launch<4>(trellis, svh, xr, yb, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
-      case 5: e = xp_launch<5>(trellis, svh, xr, yb, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
-      case 6: e = xp_launch<6>(trellis, svh, xr, yb, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
-      case 7: e = xp_launch<7>(trellis, svh, xr, yb, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
-      case 8: e = xp_launch<8>(trellis, svh, xr, yb, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
+      case 1: e = xp_launch<1>(trellis, svh, xr, yb, y_dtype, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
+      case 2: e = xp_launch<2>(trellis, svh, xr, yb, y_dtype, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
+      case 3: e = xp_launch<3>(trellis, svh, xr, yb, y_dtype, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
+      case 4: e = xp_launch<4>(trellis, svh, xr, yb, y_dtype, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
+      case 5: e = xp_launch<5>(trellis, svh, xr, yb, y_dtype, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
+      case 6: e = xp_launch<6>(trellis, svh, xr, yb, y_dtype, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
+      case 7: e = xp_launch<7>(trellis, svh, xr, yb, y_dtype, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
+      case 8: e = xp_launch<8>(trellis, svh, xr, yb, y_dtype, bias, bias_dtype, rows, n_out, n_in, cb, s); break;
       default: return hipErrorInvalidValue;
     }
     if (e != hipSuccess) return e;

@@ -174,8 +174,8 @@ hipError_t launch_hadamard128(float* v, const uint16_t* pre, const uint16_t* pos
 // the library keeps per (device, stream), then 64 rows per decoded weight.  y fp32.
 bool gemm_exl3_preferred(int64_t m, int64_t n_out, int64_t n_in);
 hipError_t launch_gemm_exl3(const uint16_t* trellis, const uint16_t* suh, const uint16_t* svh, const void* x,
-                            int x_dtype, float* y, const void* bias, int bias_dtype, int64_t m, int64_t n_out,
-                            int64_t n_in, int bits, int cb, hipStream_t s);
+                            int x_dtype, void* y, int y_dtype, const void* bias, int bias_dtype, int64_t m,
+                            int64_t n_out, int64_t n_in, int bits, int cb, hipStream_t s);
 
 // Matrix-core trellis GEMV in one launch (ttq_exl3_mfma.hip).  The plan says how the reduction
 // dimension is sliced and how many 64-bit accumulator words a sliced launch needs (zero before and
@@ -186,7 +186,7 @@ struct Exl3Plan {
 };
 Exl3Plan exl3_mfma_plan(int64_t m, int64_t n_out, int64_t n_in);
 hipError_t launch_gemv_exl3_mfma(const Exl3Plan& p, const uint16_t* trellis, const uint16_t* suh,
-                                 const uint16_t* svh, const void* x, int x_dtype, float* y, const void* bias,
+                                 const uint16_t* svh, const void* x, int x_dtype, void* y, int y_dtype, const void* bias,
                                  int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, int bits, int cb,
                                  unsigned long long* accum, hipStream_t s);
 // The library's own accumulator words for the calling thread's device and this stream, allocated and

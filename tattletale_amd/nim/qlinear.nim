@@ -110,8 +110,7 @@ proc forward*(self: QuantLinear, x: TorchTensor): TorchTensor =
   var shape = x.sizes().asNimView().toSeq()      # (..., in) -> (..., out)
   shape[^1] = self.out_features
   let m = x.numel() div self.in_features
-  let outKind = if self.format == kEXL3: kFloat32 else: x.scalarType()
-  result = F.empty(shape, x.options().dtype(outKind))
+  result = F.empty(shape, x.options())
   var desc = TtqQLinear(
     format: self.format.int32, bits: self.bits.int32, codebook: self.codebook.int32,
     bias_dtype: (if self.bias.isSome: ttqDtype(self.bias.get().scalarType()).int32 else: 0),
@@ -122,10 +121,9 @@ proc forward*(self: QuantLinear, x: TorchTensor): TorchTensor =
     svh: (if self.svh.isSome: self.svh.get().data_ptr(byte) else: nil),
     bias: (if self.bias.isSome: self.bias.get().data_ptr(byte) else: nil))
   let rc = linear_forward(addr desc, x.data_ptr(byte), ttqDtype(x.scalarType()), m,
-                          result.data_ptr(byte), ttqDtype(outKind), currentStream())
+                          result.data_ptr(byte), ttqDtype(x.scalarType()), currentStream())
   if rc != 0:
     raise newException(QuantLinearError, "ttq_linear_forward: " & $strerror(rc))
-  if outKind != x.scalarType(): result = result.to(x.scalarType())
 
 # ---------------------------------------------------------------------------- gated MLP
 # Shaped like GatedMLP (workspace/transformers/src/layers/mlp.nim:25-60): one fused gate/up

@@ -116,14 +116,12 @@ class QuantLinear:
         dev = _require_device(self.qweight, x)
         out_dtype = out_dtype or x.dtype
         m = x.numel() // self.in_features
-        # the trellis path rotates its output in place in fp32
-        y_dtype = torch.float32 if self.format == _lib.EXL3 else out_dtype
-        y = torch.empty(x.shape[:-1] + (self.out_features,), dtype=y_dtype, device=dev)
+        y = torch.empty(x.shape[:-1] + (self.out_features,), dtype=out_dtype, device=dev)
         st = self._struct()
         with torch.cuda.device(dev):
             check(_lib.lib().ttq_linear_forward(C.byref(st), x.data_ptr(), _code(x.dtype), m, y.data_ptr(),
-                                                _code(y_dtype), _stream(dev)), "ttq_linear_forward")
-        return y if y_dtype == out_dtype else y.to(out_dtype)
+                                                _code(out_dtype), _stream(dev)), "ttq_linear_forward")
+        return y
 
     __call__ = forward
 

@@ -46,7 +46,13 @@ def test_exl3_quantlinear_forward_and_bias():
     # the layer approximates the dense weights it was built from
     dense = oracle.linear_f64(w, oracle.f16_to_f32(x))[0] + bias
     assert rel_l2(y, dense) < 0.7
-    assert layer.forward(bits_to_dev(x, "f16")).dtype == torch.float16
+    yh = layer.forward(bits_to_dev(x, "f16"))
+    assert yh.dtype == torch.float16
+    # the 16-bit outputs are the fp32 result rounded once, written by the same launch
+    y32 = layer.forward(bits_to_dev(x, "f16"), out_dtype=torch.float32)
+    assert torch.equal(yh, y32.to(torch.float16))
+    yb = layer.forward(bits_to_dev(x, "f16"), out_dtype=torch.bfloat16)
+    assert yb.dtype == torch.bfloat16 and torch.equal(yb, y32.to(torch.bfloat16))
 
 
 def test_full_shape_exl3_4096x4096():
@@ -189,6 +195,8 @@ def test_exl3_forward_takes_the_prefill_path_and_the_flag_pins_the_decode_class(
     ye = exact.forward(xd, out_dtype=torch.float32).cpu().numpy()
     assert max(rel_l2(ye[i], want[i]) for i in range(0, m, 7)) <= 1e-4       # two-term activations: fp32 class
     assert not np.array_equal(y, ye)                                          # the two paths really differ
+    y16 = auto.forward(xd, out_dtype=torch.bfloat16)                           # prefill path, 16-bit output
+    assert torch.equal(y16, torch.from_numpy(y).to(DEV).to(torch.bfloat16))
 
 
 def test_exl3_prefill_full_shape_4096x4096_m512_sampled_rows():
