@@ -290,6 +290,11 @@ int ttq_gemv_q4_k_rmsnorm(const void* w, const void* x, const void* residual, co
         overlaps(normed_out, nb, new_residual_out, nb))
       return TTQ_ERR_ALIAS;
   }
+  if (m <= 4 && (silu_mul ? ttq::gemv_q4k_stream_fused_supported(x_dtype, n_out, n_in)
+                          : ttq::gemv_q4k_stream_supported(TTQ_Q4_K, x_dtype, n_out, n_in)))
+    return hip_status(ttq::launch_gemv_q4k_stream_norm(w, x, x_dtype, y, y_dtype, m, n_out, n_in, silu_mul != 0, residual,
+                                                       gamma, eps, new_residual_out, normed_out,
+                                                       static_cast<hipStream_t>(stream)));
   if (!ttq::gemv_fused_supported(TTQ_Q4_K, x_dtype, n_out, n_in, silu_mul != 0)) return TTQ_ERR_UNSUPPORTED;
   return hip_status(ttq::launch_gemv_fused(w, x, x_dtype, y, y_dtype, nullptr, 0, m, n_out, n_in, silu_mul != 0,
                                            residual, gamma, eps, new_residual_out, normed_out,

@@ -66,13 +66,6 @@ struct StepRaw { uint4 hdr, c0, c1; };
 // Optional RMSNorm in front of the GEMV (NORM kernels): normalized = rms_norm(x [+ residual]) *
 // gamma, as RmsNorm.forward / forward_with_residual compute it before a Linear
 // (workspace/transformers/src/layers/norm.nim:23-38).  All buffers hold the activation type.
-struct GemvNormArgs {
-  const uint16_t* residual;     // (m, n_in) or null
-  const uint16_t* gamma;        // (n_in)
-  uint16_t* new_residual;       // (m, n_in) or null: x + residual
-  uint16_t* normed;             // (m, n_in) or null: the normalized activations the GEMV consumed
-  float eps;
-};
 
 // LDS layout (bytes): plane table, then the per-sub-block constants [nsb][4] x float4
 // {2^(E-13) of sub-blocks 2g, 2g+1, sum(x) of 2g, 2g+1}, then the partial row sums of the

@@ -70,6 +70,15 @@ __device__ __forceinline__ uint32_t pack_low_bytes(int a, int b, int c, int d) {
   return p01 | (p23 << 16);
 }
 
+// Optional RMSNorm in front of a GEMV: what the kernels that normalize the activation row themselves need.
+struct GemvNormArgs {
+  const uint16_t* residual;     // (m, n_in) or null
+  const uint16_t* gamma;        // (n_in)
+  uint16_t* new_residual;       // (m, n_in) or null: x + residual
+  uint16_t* normed;             // (m, n_in) or null: the normalized activations the GEMV consumed
+  float eps;
+};
+
 inline int mfma_env_int(const char* name, int dflt) { return dev_knob(name, dflt); }
 
 }  // namespace ttq

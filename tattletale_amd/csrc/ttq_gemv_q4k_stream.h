@@ -80,10 +80,16 @@ __device__ __forceinline__ st_u32x4 st_read1(uint32_t a) {
 // silu_and_mul of workspace/transformers/src/kernels/activations.nim:14-38: a workgroup takes the gate row
 // groups of its outputs, then the up row groups of the same outputs, and pairs their sums at the end.
 // n_out and rows_per_wg count outputs.
-template <typename XT, typename YT, int STAGE, bool FUSE = false, int UP = kStUpFront>
+// NORM: every workgroup first normalizes the activation row itself: t = x + residual rounded to the activation
+// type, normalized = t * rsqrt(mean(t^2) + eps) * gamma in fp32, rounded once to the activation type; the GEMV
+// consumes exactly those rounded values, and workgroup 0 writes t and the normalized row out.  Residual and
+// gamma arrive like the activations, as LDS requests into the slots of the block's last requests.
+template <typename XT, typename YT, int STAGE, bool FUSE = false, int UP = kStUpFront, bool NORM = false>
 __global__ void __launch_bounds__(kStThreads)
 gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
-                       const void* __restrict__ bias, int bias_dtype, int n_out, int nsb, int rows_per_wg) {
+                       const void* __restrict__ bias, int bias_dtype, int n_out, int nsb, int rows_per_wg,
+                       GemvNormArgs na) {
+  static_assert(!NORM || UP + 3 <= kStBlockRequests, "three slots stay free for x, residual and gamma");
   __shared__ __attribute__((aligned(1024))) uint8_t wbuf[kStWaves * kStBlockBytes];
   __shared__ __attribute__((aligned(16))) v4i_t xa[kStMaxSb * 32 + 1];   // plane table + one zero entry
   __shared__ __attribute__((aligned(16))) float tab[kStMaxSb * 32];
@@ -112,6 +118,15 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   const bool xok = k0 < n_in;                             // whole wavefronts: n_in is a multiple of 512
   uint8_t* xland = mybuf + kStHalfBytes + (kStLines - 1) * 1024;
   if (xok) __builtin_amdgcn_global_load_lds((st_gptr_t)(xm + k0), (st_lptr_t)xland, 16, 0, 0);
+  uint8_t* rland = mybuf + (kStLines - 1) * 1024;                      // request 16's slot
+  uint8_t* gland = mybuf + kStHalfBytes + (kStLines - 2) * 1024;       // request 15's slot
+  if constexpr (NORM) {
+    if (xok) {
+      if (na.residual != nullptr)
+        __builtin_amdgcn_global_load_lds((st_gptr_t)(na.residual + (int64_t)blockIdx.y * n_in + k0), (st_lptr_t)rland, 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((st_gptr_t)(na.gamma + k0), (st_lptr_t)gland, 16, 0, 0);
+    }
+  }
   // a compute unit serves its requests in the order they were made: every wavefront's activation
   // request is queued before any weight request of the workgroup
   asm volatile("s_barrier" ::: "memory");
@@ -158,6 +173,39 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
     else st_wait_vmcnt<0>();
     const st_u32x4 r = st_read1((uint32_t)(size_t)(st_lptr_t)(xland) + (uint32_t)(lane * 16));
     widen8<XT>(make_uint4(r[0], r[1], r[2], r[3]), xf);
+  }
+  if constexpr (NORM) {
+    float ss = 0.f, gf[8];
+    if (xok) {
+      if (na.residual != nullptr) {
+        const st_u32x4 rr = st_read1((uint32_t)(size_t)(st_lptr_t)(rland) + (uint32_t)(lane * 16));
+        float rf[8];
+        widen8<XT>(make_uint4(rr[0], rr[1], rr[2], rr[3]), rf);
+#pragma unroll
+        for (int i = 0; i < 8; i++) xf[i] += rf[i];
+        const uint4 t = narrow8<XT>(xf);          // the new residual, as the reference's add rounds it
+        if (blockIdx.x == 0 && na.new_residual != nullptr)
+          *reinterpret_cast<uint4*>(na.new_residual + (int64_t)blockIdx.y * n_in + k0) = t;
+      }
+      const st_u32x4 gr = st_read1((uint32_t)(size_t)(st_lptr_t)(gland) + (uint32_t)(lane * 16));
+      widen8<XT>(make_uint4(gr[0], gr[1], gr[2], gr[3]), gf);
+#pragma unroll
+      for (int i = 0; i < 8; i++) ss += xf[i] * xf[i];
+    }
+    ss = wave_sum(ss);
+    if (lane == 0) part[0][wave] = ss;
+    st_barrier();
+    float total = 0.f;
+#pragma unroll
+    for (int i = 0; i < kStWaves; i++) total += part[0][i];
+    const float rs = 1.f / sqrtf(total / (float)n_in + na.eps);
+    if (xok) {
+#pragma unroll
+      for (int i = 0; i < 8; i++) xf[i] = (xf[i] * rs) * gf[i];
+      const uint4 t = narrow8<XT>(xf);
+      if (blockIdx.x == 0 && na.normed != nullptr)
+        *reinterpret_cast<uint4*>(na.normed + (int64_t)blockIdx.y * n_in + k0) = t;
+    }
   }
 
   // ---- quantize the activations into the two byte planes (compact table: entry (b, j, t, h) =
@@ -391,25 +439,21 @@ inline int st_rows_per_wg(int64_t n_out, int* num_wg_out) {
   return rows_per_wg;
 }
 
-template <typename XT, typename YT, int STAGE, bool FUSE = false>
+template <typename XT, typename YT, int STAGE, bool FUSE = false, bool NORM = false>
 inline hipError_t st_launch_xy(const void* w, const void* x, void* y, const void* bias, int bias_dtype, int64_t m,
-                               int64_t n_out, int64_t n_in, hipStream_t s) {
+                               int64_t n_out, int64_t n_in, hipStream_t s, GemvNormArgs na = GemvNormArgs{}) {
   int num_wg = 0;
   const int rows_per_wg = st_rows_per_wg(n_out, &num_wg);
   const dim3 grid((unsigned)num_wg, (unsigned)m), block(kStThreads);
   const int blocks = (FUSE ? 2 : 1) * ((rows_per_wg + 15) / 16) * (int)(n_in / 2048);
-  if (blocks <= 2)
-    hipLaunchKernelGGL((gemv_q4k_stream_kernel<XT, YT, STAGE, FUSE, kStUpFrontFew>), grid, block, 0, s,
-                       static_cast<const uint8_t*>(w), static_cast<const uint16_t*>(x), static_cast<YT*>(y), bias,
-                       bias_dtype, (int)n_out, (int)(n_in / 256), rows_per_wg);
-  else if (blocks <= 4)
-    hipLaunchKernelGGL((gemv_q4k_stream_kernel<XT, YT, STAGE, FUSE, 12>), grid, block, 0, s,
-                       static_cast<const uint8_t*>(w), static_cast<const uint16_t*>(x), static_cast<YT*>(y), bias,
-                       bias_dtype, (int)n_out, (int)(n_in / 256), rows_per_wg);
-  else
-    hipLaunchKernelGGL((gemv_q4k_stream_kernel<XT, YT, STAGE, FUSE>), grid, block, 0, s, static_cast<const uint8_t*>(w),
-                       static_cast<const uint16_t*>(x), static_cast<YT*>(y), bias, bias_dtype, (int)n_out,
-                       (int)(n_in / 256), rows_per_wg);
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, block, 0, s, static_cast<const uint8_t*>(w), static_cast<const uint16_t*>(x),
+                       static_cast<YT*>(y), bias, bias_dtype, (int)n_out, (int)(n_in / 256), rows_per_wg, na);
+  };
+  // (the normalizing form keeps three request slots free for x, residual and gamma)
+  if (blocks <= 2 && !NORM) go(gemv_q4k_stream_kernel<XT, YT, STAGE, FUSE, NORM ? 12 : kStUpFrontFew, NORM>);
+  else if (blocks <= 4) go(gemv_q4k_stream_kernel<XT, YT, STAGE, FUSE, 12, NORM>);
+  else go(gemv_q4k_stream_kernel<XT, YT, STAGE, FUSE, kStUpFront, NORM>);
   return hipGetLastError();
 }
 

@@ -40,6 +40,37 @@ hipError_t launch_gemv_q4k_stream_fused(const void* w, const void* x, int x_dtyp
   return hipErrorInvalidValue;
 }
 
+// add + RMSNorm in front (and optionally silu_and_mul behind) on the same kernel
+template <typename XT, bool FUSE>
+static hipError_t st_launch_norm_x(const void* w, const void* x, void* y, int y_dtype, int64_t m, int64_t n_out,
+                                   int64_t n_in, const GemvNormArgs& na, hipStream_t s) {
+  switch (y_dtype) {
+    case kF32: return st_launch_xy<XT, float, 0, FUSE, true>(w, x, y, nullptr, 0, m, n_out, n_in, s, na);
+    case kF16: return st_launch_xy<XT, f16_tag, 0, FUSE, true>(w, x, y, nullptr, 0, m, n_out, n_in, s, na);
+    case kBF16: return st_launch_xy<XT, bf16_tag, 0, FUSE, true>(w, x, y, nullptr, 0, m, n_out, n_in, s, na);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+hipError_t launch_gemv_q4k_stream_norm(const void* w, const void* x, int x_dtype, void* y, int y_dtype, int64_t m,
+                                       int64_t n_out, int64_t n_in, bool silu_mul, const void* norm_residual,
+                                       const void* norm_gamma, float norm_eps, void* new_residual_out,
+                                       void* normed_out, hipStream_t s) {
+  GemvNormArgs na{};
+  na.residual = static_cast<const uint16_t*>(norm_residual);
+  na.gamma = static_cast<const uint16_t*>(norm_gamma);
+  na.new_residual = static_cast<uint16_t*>(new_residual_out);
+  na.normed = static_cast<uint16_t*>(normed_out);
+  na.eps = norm_eps;
+  if (x_dtype == kBF16)
+    return silu_mul ? st_launch_norm_x<bf16_tag, true>(w, x, y, y_dtype, m, n_out, n_in, na, s)
+                    : st_launch_norm_x<bf16_tag, false>(w, x, y, y_dtype, m, n_out, n_in, na, s);
+  if (x_dtype == kF16)
+    return silu_mul ? st_launch_norm_x<f16_tag, true>(w, x, y, y_dtype, m, n_out, n_in, na, s)
+                    : st_launch_norm_x<f16_tag, false>(w, x, y, y_dtype, m, n_out, n_in, na, s);
+  return hipErrorInvalidValue;
+}
+
 template <typename XT>
 static hipError_t st_launch_x(const void* w, const void* x, void* y, int y_dtype, const void* bias, int bias_dtype,
                               int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {

@@ -86,6 +86,11 @@ bool gemv_fused_supported(int format, int x_dtype, int64_t n_out, int64_t n_in, 
 bool gemv_q4k_stream_fused_supported(int x_dtype, int64_t n_ff, int64_t n_in);
 hipError_t launch_gemv_q4k_stream_fused(const void* w, const void* x, int x_dtype, void* y, int y_dtype, int64_t m,
                                         int64_t n_ff, int64_t n_in, hipStream_t s);
+// add + RMSNorm in front of either form (the shapes the two predicates above accept)
+hipError_t launch_gemv_q4k_stream_norm(const void* w, const void* x, int x_dtype, void* y, int y_dtype, int64_t m,
+                                       int64_t n_out, int64_t n_in, bool silu_mul, const void* norm_residual,
+                                       const void* norm_gamma, float norm_eps, void* new_residual_out,
+                                       void* normed_out, hipStream_t s);
 hipError_t launch_gemv_fused(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
                              const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                              bool silu_mul, const void* norm_residual, const void* norm_gamma,

@@ -177,7 +177,9 @@ def test_rmsnorm_in_place(dt, n):
 
 @pytest.mark.parametrize("xk", ["bf16", "f16"])
 @pytest.mark.parametrize("n_out,n_in,silu", [(100, 1024, False), (3000, 4096, False), (520, 14336, False),
-                                             (1000, 4096, True), (64, 256, True)])
+                                             (1000, 4096, True), (64, 256, True),
+                                             (4096, 4096, False), (5000, 2048, False), (14336, 4096, False),
+                                             (2048, 4096, True), (7177, 2048, True)])
 @pytest.mark.parametrize("with_residual", [False, True])
 def test_fused_rmsnorm_gemv(xk, n_out, n_in, silu, with_residual):
     """One kernel for [add +] RMSNorm + GEMV [+ silu_and_mul].  The normalized row it reports must be
