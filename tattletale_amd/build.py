@@ -34,6 +34,7 @@ SOURCES = [
     "ttq_exl3_mfma.hip",
     "ttq_exl3_prefill.hip",
     "ttq_activations.hip",
+    "ttq_workspace.hip",
     "ttq_host.cpp",
 ]
 

@@ -419,7 +419,30 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
       return hip_status(ttq::launch_gemm(layer->format, layer->qweight, static_cast<const uint16_t*>(x), y, y_dtype,
                                          layer->bias, layer->bias_dtype, m, n_out, n_in, s));
   }
-  // fp16 activations: no tiled GEMM, but the few-row kernel takes them, 64 rows per launch
+  // fp16 / fp32 activations, 256 rows or more (four launches of the few-row kernel): round them to bf16 into the library's
+  // workspace (4096 rows at a time) and run the bf16 matrix-core GEMM (weights and activations rounded to bf16:
+  // the 2e-2 class, like the GEMM entry points)
+  const bool block_fmt = layer->format == TTQ_Q4_K || layer->format == TTQ_Q6_K || layer->format == TTQ_Q8_0;
+  if ((x_dtype == TTQ_F16 || x_dtype == TTQ_F32) && block_fmt && m >= 256 && route != 1 && n_in % 8 == 0 &&
+      ttq::gemm_pc_supported(layer->format, m < 4096 ? m : 4096, n_out, n_in, 112)) {
+    constexpr int64_t kRows = 4096;
+    void* ws = nullptr;
+    const int64_t block_rows = m < kRows ? m : kRows;
+    hipError_t e = ttq::stream_workspace(ttq::kWsBf16Activations, s, (size_t)block_rows * n_in * 2, &ws);
+    if (e != hipSuccess) return hip_status(e);
+    for (int64_t r0 = 0; r0 < m; r0 += kRows) {
+      const int64_t rows = m - r0 < kRows ? m - r0 : kRows;
+      e = ttq::launch_to_bf16(static_cast<const char*>(x) + r0 * n_in * dtype_size(x_dtype), x_dtype,
+                              static_cast<uint16_t*>(ws), rows * n_in, s);
+      if (e != hipSuccess) return hip_status(e);
+      e = ttq::launch_gemm_pc(layer->format, layer->qweight, static_cast<const uint16_t*>(ws),
+                              static_cast<char*>(y) + r0 * n_out * dtype_size(y_dtype), y_dtype, layer->bias,
+                              layer->bias_dtype, rows, n_out, n_in, s);
+      if (e != hipSuccess) return hip_status(e);
+    }
+    return TTQ_OK;
+  }
+  // fp16 activations, up to 64 rows: the few-row kernel takes them as they are
   const bool block_format = layer->format == TTQ_Q4_K || layer->format == TTQ_Q6_K || layer->format == TTQ_Q8_0;
   if (x_dtype == TTQ_F16 && block_format && m >= 5 && route != 1 &&
       ttq::gemm_skinny_supported(layer->format, m < 64 ? m : 64, n_out, n_in)) {

@@ -16,9 +16,6 @@
 // callers that ask for its accuracy class whatever the row count.
 #include "ttq_exl3_common.h"
 
-#include <mutex>
-#include <unordered_map>
-
 namespace ttq {
 
 constexpr int kXpRows = 64;                                   // activation rows per workgroup
@@ -227,47 +224,16 @@ static hipError_t xp_launch(const uint16_t* trellis, const uint16_t* svh, const 
   return hipGetLastError();
 }
 
-// The rotated activations of up to kXpMaxRows rows, per (device, stream), grown on demand.
-namespace {
-constexpr int64_t kXpMaxRows = 4096;
-struct XrBuf { uint16_t* p; size_t bytes; };
-std::mutex g_xr_mutex;
-std::unordered_map<uint64_t, XrBuf> g_xr;
-
-hipError_t xr_workspace(hipStream_t s, size_t bytes, uint16_t** out) {
-  int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return e;
-  const uint64_t key = ((uint64_t)(uint32_t)dev << 48) ^ (uint64_t)reinterpret_cast<uintptr_t>(s);
-  std::lock_guard<std::mutex> lock(g_xr_mutex);
-  XrBuf& b = g_xr[key];
-  if (b.bytes < bytes) {
-    if (b.p) {
-      // earlier launches on the stream may still read the old buffer
-      e = hipStreamSynchronize(s);
-      if (e != hipSuccess) return e;
-      (void)hipFree(b.p);
-      b.p = nullptr;
-      b.bytes = 0;
-    }
-    void* p = nullptr;
-    e = hipMalloc(&p, bytes);
-    if (e != hipSuccess) return e;
-    b.p = static_cast<uint16_t*>(p);
-    b.bytes = bytes;
-  }
-  *out = b.p;
-  return hipSuccess;
-}
-}  // namespace
+constexpr int64_t kXpMaxRows = 4096;       // rows rotated into the workspace at a time
 
 hipError_t launch_gemm_exl3(const uint16_t* trellis, const uint16_t* suh, const uint16_t* svh, const void* x,
                             int x_dtype, void* y, int y_dtype, const void* bias, int bias_dtype, int64_t m,
                             int64_t n_out, int64_t n_in, int bits, int cb, hipStream_t s) {
   if (m == 0 || n_out == 0) return hipSuccess;
   const int64_t block_rows = m < kXpMaxRows ? m : kXpMaxRows;
-  uint16_t* xr = nullptr;
-  hipError_t e = xr_workspace(s, (size_t)block_rows * n_in * sizeof(uint16_t), &xr);
+  void* ws = nullptr;
+  hipError_t e = stream_workspace(kWsExl3Rotated, s, (size_t)block_rows * n_in * sizeof(uint16_t), &ws);
+  uint16_t* xr = static_cast<uint16_t*>(ws);
   if (e != hipSuccess) return e;
   const int64_t xsize = x_dtype == kF32 ? 4 : 2;
   for (int64_t r0 = 0; r0 < m; r0 += kXpMaxRows) {

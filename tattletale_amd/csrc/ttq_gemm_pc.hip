@@ -504,6 +504,7 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
               *reinterpret_cast<uint16_t*>(stg + row * kRowBytes + (8 * j + cn) * 2) = f32_to_bf16_bits(res);
             } else if (o < n_out && m0 + row < m) {
               if (y_dtype == kBF16) YElem<bf16_tag>::store(static_cast<bf16_tag*>(yv), (int64_t)(m0 + row) * n_out + o, res);
+              else if (y_dtype == kF16) YElem<f16_tag>::store(static_cast<f16_tag*>(yv), (int64_t)(m0 + row) * n_out + o, res);
               else YElem<float>::store(static_cast<float*>(yv), (int64_t)(m0 + row) * n_out + o, res);
             }
           }
@@ -569,6 +570,7 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
         if (mm < m) {
           const float v = acc[i][j][r] + bv;
           if (y_dtype == kBF16) YElem<bf16_tag>::store(static_cast<bf16_tag*>(yv), (int64_t)mm * n_out + n, v);
+          else if (y_dtype == kF16) YElem<f16_tag>::store(static_cast<f16_tag*>(yv), (int64_t)mm * n_out + n, v);
           else YElem<float>::store(static_cast<float*>(yv), (int64_t)mm * n_out + n, v);
         }
       }
@@ -655,7 +657,7 @@ hipError_t launch_gemm_pc(int format, const void* w, const uint16_t* x_bf16, voi
                           const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                           hipStream_t s) {
   if (m == 0 || n_out == 0) return hipSuccess;
-  if (y_dtype != kBF16 && y_dtype != kF32) return hipErrorInvalidValue;
+  if (y_dtype != kBF16 && y_dtype != kF32 && y_dtype != kF16) return hipErrorInvalidValue;
   const uint8_t* wb = static_cast<const uint8_t*>(w);
   switch (format) {
     case kQ4_K: return launch_pc_fmt<kQ4_K, false>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);

@@ -175,6 +175,12 @@ hipError_t launch_gemv_exl3(const uint16_t* trellis, const uint16_t* suh, const 
 hipError_t launch_hadamard128(float* v, const uint16_t* pre, const uint16_t* post, int64_t n,
                               hipStream_t s);
 
+// Workspaces the library keeps per (slot, device, stream), grown on demand (ttq_workspace.hip).
+constexpr int kWsExl3Rotated = 0, kWsBf16Activations = 1;
+hipError_t stream_workspace(int slot, hipStream_t s, size_t bytes, void** out);
+// n fp16 or fp32 values (n a multiple of 8) rounded to bf16
+hipError_t launch_to_bf16(const void* x, int x_dtype, uint16_t* out, int64_t n, hipStream_t s);
+
 // Trellis layer for many activation rows (ttq_exl3_prefill.hip): activations rotated once into a workspace
 // the library keeps per (device, stream), then 64 rows per decoded weight.  y fp32.
 bool gemm_exl3_preferred(int64_t m, int64_t n_out, int64_t n_in);

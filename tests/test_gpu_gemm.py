@@ -260,3 +260,29 @@ def test_forward_fp16_unit_vectors_give_fp16_weights_exactly(fmt):
     # the library decides between this kernel and decode passes by cost; both reproduce the weight up to
     # its rounding to fp16 at most
     assert np.array_equal(y, want) or np.array_equal(y, what[:, ks].T)
+
+
+@pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
+@pytest.mark.parametrize("xk", ["f16", "f32"])
+@pytest.mark.parametrize("m,n_out,n_in", [(256, 1048, 1024), (600, 4096, 512)])
+def test_forward_fp16_fp32_activations_many_rows_take_the_bf16_gemm(fmt, xk, m, n_out, n_in):
+    """From 256 rows on, fp16 and fp32 activations are rounded to bf16 into the library's workspace and run
+    the matrix-core GEMM (2e-2 class: weights and activations rounded to bf16 once); every output type."""
+    p = random_blocks(fmt, n_out * (n_in // BLOCK_WEIGHTS[fmt]), seed=900 + m)
+    what = oracle.dequant(fmt, p, n_out, n_in)
+    bd, bf = x_to_dev(Q.fill_normal(901, 2, 0.5, n_out), "f32")
+    xd, xf = x_to_dev(Q.fill_normal(902 + m, 1, 1.0, m * n_in).reshape(m, n_in) * np.float32(0.02), xk)
+    layer = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out, bias=bd)
+    want = oracle.linear_f64(what, xf, bf)
+    y32 = layer.forward(xd, out_dtype=torch.float32).cpu().numpy()
+    assert rel_l2(y32, want) <= TOL
+    for i in (0, 63, 64, 255, m - 1):
+        assert rel_l2(y32[i], want[i]) <= TOL, i
+    y16 = layer.forward(xd, out_dtype=torch.float16)
+    assert y16.dtype == torch.float16 and rel_l2(oracle.f16_to_f32(dev_bits(y16)), want) <= TOL
+    ybf = layer.forward(xd, out_dtype=torch.bfloat16)
+    assert rel_l2(oracle.bf16_to_f32(dev_bits(ybf)), want) <= TOL
+    # a layer that pins the decode accuracy class keeps it
+    exact = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out, bias=bd, precision=F.PRECISION_F32_SCALES)
+    ye = exact.forward(xd, out_dtype=torch.float32).cpu().numpy()
+    assert rel_l2(ye, want) <= 1e-3
