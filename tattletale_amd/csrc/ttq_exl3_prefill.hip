@@ -8,7 +8,8 @@
 // is the decode GEMV's workgroup (128 output channels, 16 wavefronts, weights staged through LDS as a
 // big-endian bit string, four weights per lane decoded into an A fragment) with 64 rows per workgroup:
 // each decoded fragment feeds four v_mfma_f32_16x16x16_f16, one per block of 16 rows, so the decode --
-// which bounds the single-row kernel -- is paid once per 64 rows.  A workgroup covers the whole
+// which bounds the single-row kernel -- is paid once per 64 rows; a wavefront takes two tile columns, so
+// that every activation fragment it reads from LDS serves two of them.  A workgroup covers the whole
 // reduction, rotates its 64 x 128 sums and writes y; no workspace is shared between workgroups.
 //
 // Accuracy: the rotated activations are rounded to fp16 once (2^-11 relative per element, about 3e-4
@@ -20,6 +21,11 @@ namespace ttq {
 
 constexpr int kXpRows = 64;                                   // activation rows per workgroup
 constexpr int kXpRowBlocks = kXpRows / 16;
+// A wavefront takes two adjacent tile columns and two of every group's eight k-tiles: a B fragment (16 rows x 16 k
+// of activations) read from LDS then serves two matrix instructions instead of one.
+constexpr int kXpCols = 2;                                    // tile columns per wavefront
+constexpr int kXpKParts = kXmThreads / kWave / (8 / kXpCols); // wavefronts along k: 4
+constexpr int kXpTiles = 8 / kXpKParts;                       // k-tiles of a group per wavefront: 2
 constexpr int kXpXPieces = kXpRows * (kXmChunkK / 8) / kXmThreads;   // 16-byte pieces of X per thread and pass
 
 // ---- pass one: Xr[row][k] = fp16( H(x o suh) / sqrt(128) ), one 32-lane half wavefront per (row, 128-group)
@@ -57,7 +63,7 @@ gemm_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __re
   // one pass of tiles, then 64 rows of rotated activations; the epilogue's sums reuse the activations' space
   __shared__ uint32_t slab[G::kSlabDw];
   __shared__ __attribute__((aligned(16))) _Float16 xs[kXpRows * kXmColStride];
-  static_assert(sizeof(_Float16) * kXpRows * kXmColStride >= sizeof(float) * kXmKSplit * kXpRows * 128, "sums fit");
+  static_assert(sizeof(_Float16) * kXpRows * kXmColStride >= sizeof(float) * 2 * kXpRows * 128, "two copies of the sums fit");
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int grp = blockIdx.x;
@@ -65,7 +71,7 @@ gemm_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __re
   const int rows = min(kXpRows, m - t0);
   const int nt_n = n_out >> 4, kt_n = n_in >> 4;
   const int col = lane & 15, q = lane >> 4;
-  const int tcol = wave & 7, kpart = wave >> 3;
+  const int tcol0 = (wave & 3) * kXpCols, kpart = wave >> 2;
 
   XmLane<BITS> ln;
   ln.init(lane);
@@ -116,12 +122,14 @@ gemm_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __re
 
   request(0, min(kXmChunkTiles, kt_n));
 
-  f32x4_t acc[kXpRowBlocks];
+  f32x4_t acc[kXpCols][kXpRowBlocks];
 #pragma unroll
-  for (int rb = 0; rb < kXpRowBlocks; rb++) acc[rb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int c = 0; c < kXpCols; c++)
+#pragma unroll
+    for (int rb = 0; rb < kXpRowBlocks; rb++) acc[c][rb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   constexpr int kWin = XmLane<BITS>::kWin;
-  const uint32_t* wcol = slab + 1 + (kpart * kXmTilesPerWave * 8 + tcol) * G::kTileStride;
-  const _Float16* xcol = xs + col * kXmColStride + kpart * kXmTilesPerWave * 16 + 4 * q;
+  const uint32_t* wcol = slab + 1 + (kpart * kXpTiles * 8 + tcol0) * G::kTileStride;
+  const _Float16* xcol = xs + col * kXmColStride + kpart * kXpTiles * 16 + 4 * q;
 
   for (int kt0 = 0; kt0 < kt_n; kt0 += kXmChunkTiles) {
     const int cnt = min(kXmChunkTiles, kt_n - kt0);       // a multiple of 8
@@ -132,20 +140,25 @@ gemm_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __re
     __syncthreads();
     // this wavefront's tile column and its share of every group's 8 k-tiles; a group's window dwords are
     // read while the group before it is decoded, the B fragments right before their matrix instructions
-    uint32_t cw[2][kXmTilesPerWave][kWin][2];
+    uint32_t cw[2][kXpTiles][kXpCols][kWin][2];
     auto fetch_group = [&](int gl, int buf) {
 #pragma unroll
-      for (int i = 0; i < kXmTilesPerWave; i++) ln.fetch(wcol + (gl * 8 + i) * 8 * G::kTileStride, cw[buf][i]);
+      for (int i = 0; i < kXpTiles; i++)
+#pragma unroll
+        for (int c = 0; c < kXpCols; c++) ln.fetch(wcol + ((gl * 8 + i) * 8 + c) * G::kTileStride, cw[buf][i][c]);
     };
     auto compute_group = [&](int gl, int buf) {
 #pragma unroll
-      for (int i = 0; i < kXmTilesPerWave; i++) {
-        const f16x4_t a = ln.template decode<CB>(cw[buf][i]);
+      for (int i = 0; i < kXpTiles; i++) {
+        f16x4_t a[kXpCols];
+#pragma unroll
+        for (int c = 0; c < kXpCols; c++) a[c] = ln.template decode<CB>(cw[buf][i][c]);
         const _Float16* xb = xcol + (gl * 8 + i) * 16;
 #pragma unroll
         for (int rb = 0; rb < kXpRowBlocks; rb++) {
           const f16x4_t b = *reinterpret_cast<const f16x4_t*>(xb + rb * 16 * kXmColStride);
-          acc[rb] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, acc[rb], 0, 0, 0);
+#pragma unroll
+          for (int c = 0; c < kXpCols; c++) acc[c][rb] = __builtin_amdgcn_mfma_f32_16x16x16f16(a[c], b, acc[c][rb], 0, 0, 0);
         }
       }
     };
@@ -160,19 +173,32 @@ gemm_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __re
     }
   }
 
-  // ---- the sums of the workgroup's k parts meet in LDS (over the activations, which are done with)
+  // ---- the sums of the workgroup's four k parts meet in LDS (over the activations, which are done with): parts 0
+  // and 1 write a copy each, then parts 2 and 3 add theirs onto them -- every element by the lane that owns it
   __syncthreads();
   float* yp = reinterpret_cast<float*>(xs);
-  {
-    float* dst = yp + kpart * (kXpRows * 128);
 #pragma unroll
-    for (int rb = 0; rb < kXpRowBlocks; rb++) {
-      const int r = rb * 16 + col;
-      if (r < rows)
-        *reinterpret_cast<float4*>(dst + r * 128 + tcol * 16 + 4 * q) = make_float4(acc[rb][0], acc[rb][1], acc[rb][2], acc[rb][3]);
+  for (int round = 0; round < 2; round++) {
+    if ((kpart >> 1) == round) {
+      float* dst = yp + (kpart & 1) * (kXpRows * 128);
+#pragma unroll
+      for (int c = 0; c < kXpCols; c++)
+#pragma unroll
+        for (int rb = 0; rb < kXpRowBlocks; rb++) {
+          const int r = rb * 16 + col;
+          if (r < rows) {
+            float4* p4 = reinterpret_cast<float4*>(dst + r * 128 + (tcol0 + c) * 16 + 4 * q);
+            float4 v = make_float4(acc[c][rb][0], acc[c][rb][1], acc[c][rb][2], acc[c][rb][3]);
+            if (round == 1) {
+              const float4 o = *p4;
+              v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
+            }
+            *p4 = v;
+          }
+        }
     }
+    __syncthreads();
   }
-  __syncthreads();
   // ---- output side: rotate the 128 sums of each row, svh, bias; 32 lanes per row
   {
     const int hw = tid >> 5, l32 = tid & 31;
@@ -189,7 +215,7 @@ gemm_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __re
     for (int r = hw; r < rows; r += kXmThreads / 32) {
       float v[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int kp = 0; kp < kXmKSplit; kp++) {
+      for (int kp = 0; kp < 2; kp++) {
         const float4 t = *reinterpret_cast<const float4*>(yp + kp * (kXpRows * 128) + r * 128 + 4 * l32);
         v[0] += t.x; v[1] += t.y; v[2] += t.z; v[3] += t.w;
       }
