@@ -299,9 +299,8 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   };
   auto issue = [&](auto sc, Regs& r) {
     constexpr int s = decltype(sc)::value;
-    // super-block s needs requests 0 .. 2 s + 3; two more are made first while there are any
+    // super-block s needs requests 0 .. 2 s + 3 (its two top-up requests have been made by now)
     constexpr int kIssued = UP + 2 * (s + 1) < kStBlockRequests ? UP + 2 * (s + 1) : kStBlockRequests;
-    topup(sc);
     st_wait_vmcnt<kIssued - (2 * s + 4)>();
     const uint32_t ta = tab_addr;
     // (s + c) ^ key, c = 1 + g or 5 + g: bits 0-2 are the slot, bit 3 says "next line"
@@ -384,14 +383,17 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
     Regs ra, rb2;
     using I0 = std::integral_constant<int, 0>;
     using I9 = std::integral_constant<int, 9>;
-    issue(std::integral_constant<int, 0>{}, ra);
-    issue(std::integral_constant<int, 1>{}, rb2); settle(I9{}, ra); compute(ra);
-    issue(std::integral_constant<int, 2>{}, ra); settle(I9{}, rb2); compute(rb2);
-    issue(std::integral_constant<int, 3>{}, rb2); settle(I9{}, ra); compute(ra);
-    issue(std::integral_constant<int, 4>{}, ra); settle(I9{}, rb2); compute(rb2);
-    issue(std::integral_constant<int, 5>{}, rb2); settle(I9{}, ra); compute(ra);
-    issue(std::integral_constant<int, 6>{}, ra); settle(I9{}, rb2); compute(rb2);
-    issue(std::integral_constant<int, 7>{}, rb2); settle(I9{}, ra); compute(ra);
+    // per super-block: its top-up requests, then the arithmetic of the one before (whose operands were read a step
+    // ago), and only then the wait for its own bytes -- so that when the block's last bytes land, one super-block
+    // of arithmetic is left, not two
+    topup(std::integral_constant<int, 0>{}); issue(std::integral_constant<int, 0>{}, ra);
+    topup(std::integral_constant<int, 1>{}); settle(I0{}, ra); compute(ra); issue(std::integral_constant<int, 1>{}, rb2);
+    topup(std::integral_constant<int, 2>{}); settle(I0{}, rb2); compute(rb2); issue(std::integral_constant<int, 2>{}, ra);
+    topup(std::integral_constant<int, 3>{}); settle(I0{}, ra); compute(ra); issue(std::integral_constant<int, 3>{}, rb2);
+    topup(std::integral_constant<int, 4>{}); settle(I0{}, rb2); compute(rb2); issue(std::integral_constant<int, 4>{}, ra);
+    topup(std::integral_constant<int, 5>{}); settle(I0{}, ra); compute(ra); issue(std::integral_constant<int, 5>{}, rb2);
+    topup(std::integral_constant<int, 6>{}); settle(I0{}, rb2); compute(rb2); issue(std::integral_constant<int, 6>{}, ra);
+    topup(std::integral_constant<int, 7>{}); settle(I0{}, ra); compute(ra); issue(std::integral_constant<int, 7>{}, rb2);
     settle(I0{}, rb2);
     // every request of the block has landed and been read: the next block may use the buffer
     const int next = blk + kStWaves;
