@@ -382,18 +382,31 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
     acc = 0.f;
     Regs ra, rb2;
     using I0 = std::integral_constant<int, 0>;
-    using I9 = std::integral_constant<int, 9>;
-    // per super-block: its top-up requests, then the arithmetic of the one before (whose operands were read a step
-    // ago), and only then the wait for its own bytes -- so that when the block's last bytes land, one super-block
-    // of arithmetic is left, not two
-    topup(std::integral_constant<int, 0>{}); issue(std::integral_constant<int, 0>{}, ra);
-    topup(std::integral_constant<int, 1>{}); settle(I0{}, ra); compute(ra); issue(std::integral_constant<int, 1>{}, rb2);
-    topup(std::integral_constant<int, 2>{}); settle(I0{}, rb2); compute(rb2); issue(std::integral_constant<int, 2>{}, ra);
-    topup(std::integral_constant<int, 3>{}); settle(I0{}, ra); compute(ra); issue(std::integral_constant<int, 3>{}, rb2);
-    topup(std::integral_constant<int, 4>{}); settle(I0{}, rb2); compute(rb2); issue(std::integral_constant<int, 4>{}, ra);
-    topup(std::integral_constant<int, 5>{}); settle(I0{}, ra); compute(ra); issue(std::integral_constant<int, 5>{}, rb2);
-    topup(std::integral_constant<int, 6>{}); settle(I0{}, rb2); compute(rb2); issue(std::integral_constant<int, 6>{}, ra);
-    topup(std::integral_constant<int, 7>{}); settle(I0{}, ra); compute(ra); issue(std::integral_constant<int, 7>{}, rb2);
+    if constexpr (UP == kStUpFront) {
+      // per super-block: its top-up requests, then the arithmetic of the one before (whose operands were read a step
+      // ago), and only then the wait for its own bytes -- so that when the block's last bytes land, one super-block
+      // of arithmetic is left, not two
+      topup(std::integral_constant<int, 0>{}); issue(std::integral_constant<int, 0>{}, ra);
+      topup(std::integral_constant<int, 1>{}); settle(I0{}, ra); compute(ra); issue(std::integral_constant<int, 1>{}, rb2);
+      topup(std::integral_constant<int, 2>{}); settle(I0{}, rb2); compute(rb2); issue(std::integral_constant<int, 2>{}, ra);
+      topup(std::integral_constant<int, 3>{}); settle(I0{}, ra); compute(ra); issue(std::integral_constant<int, 3>{}, rb2);
+      topup(std::integral_constant<int, 4>{}); settle(I0{}, rb2); compute(rb2); issue(std::integral_constant<int, 4>{}, ra);
+      topup(std::integral_constant<int, 5>{}); settle(I0{}, ra); compute(ra); issue(std::integral_constant<int, 5>{}, rb2);
+      topup(std::integral_constant<int, 6>{}); settle(I0{}, rb2); compute(rb2); issue(std::integral_constant<int, 6>{}, ra);
+      topup(std::integral_constant<int, 7>{}); settle(I0{}, ra); compute(ra); issue(std::integral_constant<int, 7>{}, rb2);
+    } else {
+      // few blocks per workgroup: the bytes arrive in one burst and the wavefronts that own them multiply eight
+      // super-blocks back to back, so the operand reads of a super-block overlap the arithmetic of the one before
+      using I9 = std::integral_constant<int, 9>;
+      topup(std::integral_constant<int, 0>{}); issue(std::integral_constant<int, 0>{}, ra);
+      topup(std::integral_constant<int, 1>{}); issue(std::integral_constant<int, 1>{}, rb2); settle(I9{}, ra); compute(ra);
+      topup(std::integral_constant<int, 2>{}); issue(std::integral_constant<int, 2>{}, ra); settle(I9{}, rb2); compute(rb2);
+      topup(std::integral_constant<int, 3>{}); issue(std::integral_constant<int, 3>{}, rb2); settle(I9{}, ra); compute(ra);
+      topup(std::integral_constant<int, 4>{}); issue(std::integral_constant<int, 4>{}, ra); settle(I9{}, rb2); compute(rb2);
+      topup(std::integral_constant<int, 5>{}); issue(std::integral_constant<int, 5>{}, rb2); settle(I9{}, ra); compute(ra);
+      topup(std::integral_constant<int, 6>{}); issue(std::integral_constant<int, 6>{}, ra); settle(I9{}, rb2); compute(rb2);
+      topup(std::integral_constant<int, 7>{}); issue(std::integral_constant<int, 7>{}, rb2); settle(I9{}, ra); compute(ra);
+    }
     settle(I0{}, rb2);
     // every request of the block has landed and been read: the next block may use the buffer
     const int next = blk + kStWaves;
