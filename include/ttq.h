@@ -112,7 +112,10 @@ typedef struct ttq_qlinear {
  * run matrix-core kernels that round each dequantized weight once to bf16 (fp16) -- the 2e-2 class
  * of the GEMM entry points -- when its cost estimate prefers them for the shape.  A layer with
  * precision == TTQ_PRECISION_F32_SCALES keeps the decode kernels, and with them the 1e-3 class,
- * for every m.
+ * for every m.  From 256 rows of fp16 / fp32 activations on (GGUF formats, no F32_SCALES), the rows
+ * are first rounded to bf16 into a workspace the library keeps per (device, stream) -- allocated on
+ * first use and grown on demand, so that first call must not happen under graph capture -- and the
+ * bf16 matrix-core GEMM runs on the copy.
  * Limits (TTQ_ERR_UNSUPPORTED beyond): the decode kernels take n_in <= 32768 for Q4_K / Q6_K with
  * 16-bit activations and n_in <= 16384 otherwise; any m (rows are taken 65535 at a time where a
  * kernel needs that).  m == 0 or n_out == 0 returns TTQ_OK without touching a pointer. */
