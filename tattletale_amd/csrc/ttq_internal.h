@@ -66,6 +66,13 @@ hipError_t launch_gemv_q4k_stream(const void* w, const void* x, int x_dtype, voi
                                   const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                                   hipStream_t s);
 
+// Q6_K through the int8 matrix cores, 16 rows at a time streamed linearly through two LDS buffers
+// (ttq_gemv_q6k_stream.hip): 16-bit activations, n_in 4096, whole groups of 16 rows, at least two per compute unit.
+bool gemv_q6k_stream_supported(int format, int x_dtype, int64_t n_out, int64_t n_in);
+hipError_t launch_gemv_q6k_stream(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                                  const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                                  hipStream_t s);
+
 // int8 matrix-core path for Q8_0, any activation dtype (ttq_gemv_q8_mfma.hip).
 // Q8_0 through the matrix cores, rows read as aligned 64-byte windows (ttq_gemv_q8_win.hip).
 bool gemv_q8_win_supported(int format, int64_t n_out, int64_t n_in);

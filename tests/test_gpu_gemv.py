@@ -346,3 +346,80 @@ def test_q4_k_fp32_activations_matrix_core_kernel_unit_vectors():
         xd, _ = x_to_dev(x, "f32")
         y = QL.gemv(F.Q4_K, wd, xd, n_out, n_in).cpu().numpy()[0]
         assert np.array_equal(y, np.float32(scale) * what[:, c]), (c, scale)
+
+
+# ------------------------------------------------------------------- Q6_K, LDS-streamed kernel
+# (rows of 4096 values, whole groups of 16 rows, at least two groups per compute unit)
+def _q6k_stream_rows(extra_groups):
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    return 16 * (2 * cus + extra_groups)
+
+
+@pytest.mark.parametrize("xk", ["bf16", "f16"])
+def test_q6_k_streamed_unit_vectors_reproduce_columns(xk):
+    """Random block bytes (every scale, bit pair and nibble value, negative scales and d): a unit vector,
+    also scaled by a power of two, reproduces the canonical column bit for bit -- for columns in every
+    nibble / bit-pair position of a block, in odd blocks (which sit at 2 mod 4 in memory) and in every
+    wavefront's share of K.  The row count leaves the workgroups with two or three groups each."""
+    n_in = 4096
+    n_out = _q6k_stream_rows(37)
+    p = random_blocks(F.Q6_K, n_out * (n_in // 256), seed=23)
+    what = oracle.dequant(F.Q6_K, p, n_out, n_in)
+    wd = packed_to_dev(p)
+    cols = [0, 1, 15, 16, 31, 32, 47, 63, 64, 80, 95, 96, 127, 128, 129, 191, 255, 256, 257, 300, 511, 512 + 77,
+            1024 + 200, 1535, 2048, 2048 + 255, 3000, 3583, 3584 + 100, n_in - 257, n_in - 129, n_in - 33, n_in - 1]
+    for i, c in enumerate(cols):
+        s = (1.0, -0.5, 4.0)[i % 3]
+        x = np.zeros((1, n_in), np.float32)
+        x[0, c] = s
+        xd, _ = x_to_dev(x, xk)
+        y = QL.gemv(F.Q6_K, wd, xd, n_out, n_in).cpu().numpy()[0]
+        col = what[:, c] * np.float32(s)
+        assert np.array_equal(y, col), c
+        nz = col != 0
+        assert np.array_equal(y[nz].view(np.uint32), col[nz].view(np.uint32)), c
+
+
+@pytest.mark.parametrize("xk", ["bf16", "f16"])
+@pytest.mark.parametrize("extra_groups", [0, 1, 255, 300])
+def test_q6_k_streamed_random_activations(xk, extra_groups):
+    """Quantized normal weights, normal activations: 1e-3 against the float64 product; every output row is
+    checked, for group counts that divide evenly among the compute units and ones that do not."""
+    n_in = 4096
+    n_out = _q6k_stream_rows(extra_groups)
+    p, what = make(F.Q6_K, n_out, n_in, 300 + extra_groups)
+    xd, xf = x_to_dev(Q.fill_normal(301, 1, 1.0, n_in), xk)
+    y = QL.gemv(F.Q6_K, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()[0]
+    want = oracle.linear_f64(what, xf)[0]
+    assert rel_l2(y, want) <= TOL
+    # no row may be off by more than the activations' fixed-point step allows
+    assert np.max(np.abs(y - want)) <= 2e-3 * np.sqrt(np.mean(want ** 2)) * 4
+
+
+def test_q6_k_streamed_activation_extremes_bias_and_output_types():
+    """Zero activations, one huge value among tiny ones (its 64 values share a scale), non-finite values,
+    tiny values; bias and 16-bit outputs through the layer entry point."""
+    n_in = 4096
+    n_out = _q6k_stream_rows(5)
+    p, what = make(F.Q6_K, n_out, n_in, 91)
+    wd = packed_to_dev(p)
+    x = np.zeros((4, n_in), np.float32)
+    x[1] = Q.fill_normal(92, 1, 1e-3, n_in)
+    x[1, 100] = 3.0e4
+    x[2] = Q.fill_normal(93, 1, 1.0, n_in)
+    x[2, 4095] = np.inf
+    x[3] = Q.fill_normal(94, 1, 1.0, n_in) * 1e-30
+    xd, xf = x_to_dev(x, "bf16")
+    y = gemv_row_by_row(F.Q6_K, wd, xd, n_out, n_in)
+    want = oracle.linear_f64(what, xf[[0, 1, 3]])
+    assert np.array_equal(y[0], np.zeros(n_out, np.float32))
+    assert rel_l2(y[1], want[1]) <= TOL
+    assert not np.any(np.isfinite(y[2]))
+    assert rel_l2(y[3], want[2]) <= TOL
+    bias = Q.fill_normal(95, 0, 0.5, n_out)
+    xd1, xf1 = x_to_dev(Q.fill_normal(96, 1, 1.0, n_in), "f16")
+    want1 = oracle.linear_f64(what, xf1).reshape(-1) + bias
+    for out_dtype, tol in ((torch.float32, TOL), (torch.bfloat16, 4e-3), (torch.float16, 1e-3)):
+        layer = QuantLinear.init(wd, F.Q6_K, n_in, n_out, bias=torch.from_numpy(bias).to(DEV))
+        yy = layer.forward(xd1, out_dtype=out_dtype).float().cpu().numpy().reshape(-1)
+        assert rel_l2(yy, want1) <= tol, out_dtype
