@@ -8,18 +8,21 @@
 // A 210-byte block is neither a multiple of a cache line nor of a dword, so the per-wavefront line rings of the
 // Q4_K kernel (ttq_gemv_q4k_stream.h) do not carry over.  What is line-shaped is a group of 16 rows: 53 760
 // contiguous bytes = 420 lines.  So here the eight wavefronts of a workgroup share the stream:
-//   * a round is one group of 16 rows, copied in memory order into one of two LDS buffers by 57 requests of
-//     1 KiB (global_load_lds_dwordx4, no registers), eight or seven per wavefront.  On the way in every block
-//     is moved to a 16-byte boundary: it lands in a slot of 14 chunks of 16 bytes, 13 fetched from its first
-//     208 bytes and one from its last 16 (the fetch addresses are 2-byte aligned, the landing addresses
-//     16-byte aligned), and every row gets 16 bytes of padding, which puts the 16 rows of an operand read
-//     into 16 different bank groups.  Operand reads that are not dword aligned, which the packed layout
-//     would need for every other block, were measured at three times the cost of the whole stream;
-//   * while one buffer is multiplied the other one's requests are in flight; a wavefront waits for its own
-//     requests on its own counter, a barrier makes the buffer whole, a second one frees it for the round after
-//     next;
-//   * along K the group is split: wavefront w multiplies blocks 2 w and 2 w + 1 of all 16 rows, four units
-//     of 16 rows x 128 weights, two v_mfma_i32_16x16x64_i8 each.
+//   * a round is half of K of one group of 16 rows: 16 runs of 1680 contiguous bytes, copied into one of three
+//     LDS buffers by 28 requests of 1 KiB (global_load_lds_dwordx4, no registers), four or three per
+//     wavefront.  On the way in every block is moved to a 16-byte boundary: it lands in a slot of 14 chunks
+//     of 16 bytes, 13 fetched from consecutive addresses and one that ends with the block's last bytes, and
+//     row n is rotated by n chunks, which puts the 16 rows of an operand read into 16 different bank groups.
+//     Fetch addresses are rounded down to a dword: requests at 2 mod 4 were measured 15 % slower than
+//     dword-aligned ones, and operand reads at 2 mod 4 -- which the packed layout would need for every other
+//     block -- at three times the cost of the whole stream.  So an odd block lands two bytes into its slot,
+//     and the wavefronts that multiply odd blocks (the odd ones: block = 8 * half + wavefront) shift their
+//     operands by 16 bits in registers;
+//   * while one buffer is multiplied, the next two rounds are in flight or landed (a compute unit takes about
+//     64 KiB of outstanding requests); a wavefront waits for its own requests on its own counter, a barrier
+//     makes the buffer whole, a second one frees it for the round three later;
+//   * along K a round is split: wavefront w multiplies block w of the half for all 16 rows, two units of
+//     16 rows x 128 weights, two v_mfma_i32_16x16x64_i8 each.
 // Arithmetic.  The activations are block fixed point, 15 bits in two byte planes with one power-of-two scale
 // per 64 values.  A weight reaches the matrix core as the signed byte 4 * (q6 - 32) = ((q6 << 2) ^ 0x80), built
 // from the nibble and the bit pair with four instructions per dword.  The 16 columns of the MFMA that a GEMV
@@ -39,20 +42,31 @@ constexpr int kQ6Waves = 8;
 constexpr int kQ6Threads = kQ6Waves * 64;
 constexpr int kQ6Nb = 16;                                  // blocks per row: n_in = 4096
 constexpr int kQ6RowBytes = kQ6Nb * 210;                   // 3360
-constexpr int kQ6SlotChunks = 14;                          // a block in LDS: 224 bytes
-constexpr int kQ6SlotBytes = kQ6SlotChunks * 16;
-constexpr int kQ6TailAt = 194;                             // chunk 13 holds bytes 194..209: d sits at its byte 14
-constexpr int kQ6DAt = 13 * 16 + (208 - kQ6TailAt);        // 222
-constexpr int kQ6RowChunks = kQ6Nb * kQ6SlotChunks + 1;    // 225 with the pad chunk
-constexpr int kQ6LdsRow = kQ6RowChunks * 16;               // 3600: 16 mod 256, rows 0..15 cover the 16 bank groups
 constexpr int kQ6GroupBytes = 16 * kQ6RowBytes;            // 53760 in memory
-constexpr int kQ6GroupChunks = 16 * kQ6RowChunks;          // 3600 in LDS
-constexpr int kQ6Requests = (kQ6GroupChunks + 63) / 64;    // 57
-constexpr int kQ6BufBytes = kQ6Requests * 1024;            // 58368
-constexpr int kQ6ReqMax = (kQ6Requests + kQ6Waves - 1) / kQ6Waves;   // 8
-constexpr int kQ6FullWaves = kQ6Requests - (kQ6ReqMax - 1) * kQ6Waves;   // wavefront 0 makes 8 requests, the others 7
-constexpr int kQ6MaxGroups = 40;                           // row groups of a workgroup (their partial sums wait in LDS)
+constexpr int kQ6HalfBlocks = kQ6Nb / 2;                   // blocks of a row in one round: one per wavefront
+constexpr int kQ6SlotChunks = 14;                          // a block in LDS: 224 bytes
+constexpr int kQ6TailAt = 196;                             // chunk 13 starts here, counted from the slot's first byte
+constexpr int kQ6DAt = 208 - kQ6TailAt;                    // d in chunk 13 (+ 2 for an odd block)
+constexpr int kQ6RowChunks = kQ6HalfBlocks * kQ6SlotChunks;   // 112
+constexpr int kQ6Requests = 16 * kQ6RowChunks / 64;        // 28
+constexpr int kQ6BufBytes = kQ6Requests * 1024;            // 28672
+#ifndef Q6_ORDER
+#define Q6_ORDER 0
+#endif
+#ifndef Q6_BUFS
+#define Q6_BUFS 2
+#endif
+#ifndef Q6_WGS_PER_CU
+#define Q6_WGS_PER_CU 2
+#endif
+constexpr int kQ6Bufs = Q6_BUFS;
+constexpr int kQ6ReqMax = (kQ6Requests + kQ6Waves - 1) / kQ6Waves;   // 4
+constexpr int kQ6FullWaves = kQ6Requests - (kQ6ReqMax - 1) * kQ6Waves;   // wavefronts 0..3 make 4 requests, the others 3
+constexpr int kQ6WgsPerCu = Q6_WGS_PER_CU;
+constexpr int kQ6MaxGroups = 40 / kQ6WgsPerCu;                           // row groups of a workgroup (their partial sums wait in LDS)
 constexpr int kQ6MinGroups = 2;
+static_assert(kQ6HalfBlocks == kQ6Waves, "one block of the half per wavefront");
+static_assert(kQ6Bufs >= 2 && kQ6Bufs <= 4, "the waits below count up to three later rounds");
 
 typedef const __attribute__((address_space(1))) void* q6_gptr_t;
 typedef __attribute__((address_space(3))) void* q6_lptr_t;
@@ -88,14 +102,16 @@ __device__ __forceinline__ void q6_write_f32(uint32_t a, float v) {
 // STAGE 0 is the GEMV; STAGE 1 leaves out the arithmetic on the operands, STAGE 2 the operand reads as well
 // (requests, waits and barriers stay): what each part costs is measured by leaving it out.
 template <typename XT, typename YT, int STAGE = 0>
-__global__ void __launch_bounds__(kQ6Threads)
+__global__ void __launch_bounds__(kQ6Threads) __attribute__((amdgpu_waves_per_eu(2 * kQ6WgsPerCu, 2 * kQ6WgsPerCu)))
 gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
                        const void* __restrict__ bias, int bias_dtype, int n_out, int groups_per_wg, int groups_rem) {
-  __shared__ __attribute__((aligned(1024))) uint8_t wbuf[2 * kQ6BufBytes];
-  __shared__ __attribute__((aligned(1024))) uint8_t xstage[kQ6Threads * 16];
+  __shared__ __attribute__((aligned(1024))) uint8_t wbuf[kQ6Bufs * kQ6BufBytes];
   __shared__ __attribute__((aligned(16))) v4i_t xa[kQ6Nb * 32 + 1];    // (16 values, plane) entries + one of zeros
   __shared__ __attribute__((aligned(16))) float fac[kQ6Nb * 4 * 2];    // (64 values, plane): scale of the integer sum
-  __shared__ float part[kQ6MaxGroups][kQ6Waves][16];
+  // (the raw activations land here first: the partial sums are written after they have been read back)
+  __shared__ __attribute__((aligned(1024))) float part[kQ6MaxGroups][kQ6Waves][16];
+  static_assert(sizeof(part) >= kQ6Threads * 16, "room for the staged activations");
+  uint8_t* xstage = reinterpret_cast<uint8_t*>(&part[0][0][0]);
 
   constexpr int n_in = kQ6Nb * 256;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -106,6 +122,7 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   const int bx = blockIdx.x;
   const int grp0 = bx * groups_per_wg + min(bx, groups_rem);
   const int ng = groups_per_wg + (bx < groups_rem ? 1 : 0);            // kQ6MinGroups .. kQ6MaxGroups
+  const int nrounds = 2 * ng;
 
   // ---- the activations, as an LDS request too (a register load among the weight requests would make the
   // compiler wait for all of them at its first use): thread t stages x[8 t .. 8 t + 7]
@@ -115,20 +132,24 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   // queued before any weight request of the workgroup
   asm volatile("s_barrier" ::: "memory");
 
-  // ---- requests of a group: request q = wave + 8 i fills LDS chunks 64 q .. 64 q + 63 of the layout above
-  // (row = chunk / 225; the pad chunk and the chunks past the group fetch a valid chunk again)
+  // ---- requests of a round: request q = wave + 8 i fills LDS chunks 64 q .. 64 q + 63 of the buffer.  Chunk
+  // position 112 n + (c + n) % 112 holds chunk c of row n's eight slots.
   uint32_t src_off[kQ6ReqMax];
 #pragma unroll
   for (int i = 0; i < kQ6ReqMax; i++) {
-    int p = 64 * (wave + kQ6Waves * i) + lane;
-    p = min(p, kQ6GroupChunks - 1);
-    const int row = p / kQ6RowChunks, c = min(p - row * kQ6RowChunks, kQ6RowChunks - 2);
+    const int p = min(64 * (wave + kQ6Waves * i) + lane, 16 * kQ6RowChunks - 1);
+    const int row = p / kQ6RowChunks, pos = p - row * kQ6RowChunks;
+    const int c = pos >= row ? pos - row : pos - row + kQ6RowChunks;
     const int b = c / kQ6SlotChunks, j = c - b * kQ6SlotChunks;
-    src_off[i] = (uint32_t)(row * kQ6RowBytes + b * 210 + (j < kQ6SlotChunks - 1 ? 16 * j : kQ6TailAt));
+    // an odd block starts at 2 mod 4: its slot starts two bytes early.  The last chunk of an even block reads two
+    // bytes into the next block of the row; the last chunk of an odd block ends with the block.
+    src_off[i] = (uint32_t)(row * kQ6RowBytes + b * 210 - 2 * (b & 1) + (j < kQ6SlotChunks - 1 ? 16 * j : kQ6TailAt));
   }
   const bool full = wave < kQ6FullWaves;
-  auto request_group = [&](int grp, int buf) {
-    const uint8_t* src = w + (size_t)((uint32_t)grp * (uint32_t)kQ6GroupBytes);
+  // round rr = 2 * (group - grp0) + (half of K)
+  auto request_round = [&](int rr, int buf) {
+    const uint8_t* src = w + (size_t)((uint32_t)(grp0 + (rr >> 1)) * (uint32_t)kQ6GroupBytes +
+                                      (uint32_t)((rr & 1) * (kQ6HalfBlocks * 210)));
     uint8_t* dst = wbuf + buf * kQ6BufBytes + wave * 1024;
 #pragma unroll
     for (int i = 0; i < kQ6ReqMax - 1; i++)
@@ -137,22 +158,23 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
       __builtin_amdgcn_global_load_lds((q6_gptr_t)(src + src_off[kQ6ReqMax - 1]),
                                        (q6_lptr_t)(dst + (kQ6ReqMax - 1) * (kQ6Waves * 1024)), 16, 0, 2);
   };
-  // all but the youngest `groups_after` groups of requests of this wavefront have landed
-  auto wait_groups = [&](auto groups_after) {
-    constexpr int A = decltype(groups_after)::value;
+  // all but the youngest `rounds_after` rounds of requests of this wavefront have landed
+  auto wait_rounds = [&](auto rounds_after) {
+    constexpr int A = decltype(rounds_after)::value;
     if (full) q6_wait_vmcnt<A * kQ6ReqMax>();
     else q6_wait_vmcnt<A * (kQ6ReqMax - 1)>();
   };
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
   using I2 = std::integral_constant<int, 2>;
-  request_group(grp0, 0);
-  request_group(grp0 + 1, 1);
+  using I3 = std::integral_constant<int, 3>;
+#pragma unroll
+  for (int i = 0; i < kQ6Bufs; i++) request_round(i, i);      // nrounds >= 4
 
   // ---- the raw activations back into registers, then into the two byte planes
   float xf[8];
   {
-    wait_groups(I2{});
+    wait_rounds(std::integral_constant<int, kQ6Bufs>{});
     const q6_u32x4 r = q6_read16(q6_lds(xstage) + (uint32_t)(tid * 16));
     widen8<XT>(make_uint4(r[0], r[1], r[2], r[3]), xf);
   }
@@ -193,115 +215,176 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   // weight operand: row n, values 16 g .. 16 g + 15 of the k-set: ql bytes 16 g, qh bytes 16 (g % 2), bit pair
   // g / 2 (low nibbles) or 2 + g / 2 (high nibbles)
   const uint32_t sh1 = 6u - 2u * (uint32_t)(g >> 1), sh2 = 2u - 2u * (uint32_t)(g >> 1);
-  const uint32_t row_off = (uint32_t)(n * kQ6LdsRow + 2 * wave * kQ6SlotBytes);
-  const uint32_t ql_off = row_off + (uint32_t)(16 * g);
-  const uint32_t qh_off = row_off + 128u + (uint32_t)(16 * (g & 1));
-  // accumulator lane (n, g): row n, k-set g / 2, plane g % 2; its four scales are consecutive bytes
-  const uint32_t sc_off = row_off + 192u + (uint32_t)(4 * (g >> 1));
-  const uint32_t d_off = row_off + (uint32_t)kQ6DAt;
+  // chunk c of row n's slots, as a byte offset into the buffer
+  auto chunk_at = [&](int c) {
+    const int pos = c + n < kQ6RowChunks ? c + n : c + n - kQ6RowChunks;
+    return (uint32_t)((n * kQ6RowChunks + pos) * 16);
+  };
+  const int slot = wave * kQ6SlotChunks;                   // the wavefront's block of the half
   // activation operand: lane (i, g) of the first MFMA holds something only if i < 8 and i % 4 == g, of the
-  // second only if i >= 8 and i % 4 == g; plane (i / 4) % 2.  Unit u = 2 b + half starts at value 128 u.
+  // second only if i >= 8 and i % 4 == g; plane (i / 4) % 2.  Unit u = 2 block + half starts at value 128 u.
   const uint32_t xa_base = q6_lds(&xa[0]);
   const uint32_t zero_entry = xa_base + (uint32_t)(kQ6Nb * 32 * 16);
   const bool mine = (n & 3) == g;
   const uint32_t plane16 = (uint32_t)(((n >> 2) & 1) * 16);
   const bool act1 = mine && n < 8, act2 = mine && n >= 8;
-  const uint32_t u0 = (uint32_t)(4 * wave);                // the wavefront's first unit
+  const uint32_t u0 = (uint32_t)(2 * wave);                // the wavefront's first unit of a first half of K
   const uint32_t a1_addr = act1 ? xa_base + 256u * u0 + 32u * (uint32_t)g + plane16 : zero_entry;
   const uint32_t a2_addr = act2 ? xa_base + 256u * u0 + 128u + 32u * (uint32_t)g + plane16 : zero_entry;
+  // per unit 256 bytes of table, per half of K 16 units
   const uint32_t a1_step = act1 ? 256u : 0u, a2_step = act2 ? 256u : 0u;
-  const uint32_t fac_addr = q6_lds(&fac[0]) + 16u * u0 + 4u * (uint32_t)g;
+  const uint32_t fac_addr0 = q6_lds(&fac[0]) + 16u * u0 + 4u * (uint32_t)g;
   const uint32_t wbuf_base = q6_lds(wbuf);
 
   q6_barrier();                         // the plane table is complete
 
-  struct Regs { q6_u32x4 ql, qh, a1, a2; uint32_t sc, d, f; };
-  // unit i of the wavefront: block 2 wave + i / 2, half i % 2
-  auto issue = [&](auto ic, uint32_t buf, Regs& r) {
-    constexpr int i = decltype(ic)::value;
-    constexpr int boff = (i >> 1) * kQ6SlotBytes, hf = i & 1;
-    const uint32_t a_ql = buf + ql_off, a_qh = buf + qh_off, a_sc = buf + sc_off, a_d = buf + d_off;
-    const uint32_t x1 = a1_addr + (uint32_t)i * a1_step, x2 = a2_addr + (uint32_t)i * a2_step;
-    const uint32_t fa = fac_addr;
-    if constexpr (STAGE >= 2) return;
-    asm volatile(
-        "ds_read_b128 %0, %7 offset:%13\n\t"
-        "ds_read_b128 %1, %8 offset:%14\n\t"
-        "ds_read_b128 %2, %9\n\t"
-        "ds_read_b128 %3, %10\n\t"
-        "ds_read_b32 %4, %11 offset:%15\n\t"
-        "ds_read_u16 %5, %12 offset:%16\n\t"
-        "ds_read_b32 %6, %17 offset:%18"
-        : "=&v"(r.ql), "=&v"(r.qh), "=&v"(r.a1), "=&v"(r.a2), "=&v"(r.sc), "=&v"(r.d), "=&v"(r.f)
-        : "v"(a_ql), "v"(a_qh), "v"(x1), "v"(x2), "v"(a_sc), "v"(a_d), "n"(boff + 64 * hf), "n"(boff + 32 * hf),
-          "n"(boff + 8 * hf), "n"(boff), "v"(fa), "n"(16 * i)
-        : "memory");
-  };
-  auto settle = [&](auto pending, Regs& r) {
-    constexpr int P = decltype(pending)::value;
-    if constexpr (STAGE >= 2) return;
-    asm volatile("s_waitcnt lgkmcnt(%7)"
-                 : "+v"(r.ql), "+v"(r.qh), "+v"(r.a1), "+v"(r.a2), "+v"(r.sc), "+v"(r.d), "+v"(r.f)
-                 : "n"(P)
-                 : "memory");
-  };
-  float acc = 0.f;
-  auto compute = [&](const Regs& r) {
-    if constexpr (STAGE >= 1) return;
-    const uint32_t ql[4] = {r.ql[0], r.ql[1], r.ql[2], r.ql[3]};
-    const uint32_t qh[4] = {r.qh[0], r.qh[1], r.qh[2], r.qh[3]};
-    v4i_t B1, B2, A1, A2;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      // 4 * (q - 32) as a signed byte: nibble into bits 2-5, bit pair into bits 6-7, top bit flipped
-      B1[i] = (int)(((ql[i] << 2) & 0x3C3C3C3Cu) | (((qh[i] << sh1) & 0xC0C0C0C0u) ^ 0x80808080u));
-      B2[i] = (int)(((ql[i] >> 2) & 0x3C3C3C3Cu) | (((qh[i] << sh2) & 0xC0C0C0C0u) ^ 0x80808080u));
-      A1[i] = (int)r.a1[i];
-      A2[i] = (int)r.a2[i];
-    }
-    const v4i_t zero = {0, 0, 0, 0};
-    v4i_t C = __builtin_amdgcn_mfma_i32_16x16x64_i8(A1, B1, zero, 0, 0, 0);
-    C = __builtin_amdgcn_mfma_i32_16x16x64_i8(A2, B2, C, 0, 0, 0);
-    const int sc = (int)r.sc;
-    int t = (int)(int8_t)(sc & 0xFF) * C[0];
-    t += (int)(int8_t)((sc >> 8) & 0xFF) * C[1];
-    t += (int)(int8_t)((sc >> 16) & 0xFF) * C[2];
-    t += (sc >> 24) * C[3];
-    const float d = f16_bits_to_f32((uint16_t)(r.d & 0xFFFFu));
-    acc = fmaf_((float)t * __uint_as_float(r.f), d, acc);
-    // pins the arithmetic here: left alone the compiler moves it behind later waits
-    asm volatile("" : "+v"(acc));
-  };
-
-  using U0 = std::integral_constant<int, 0>;
-  using U1 = std::integral_constant<int, 1>;
-  using U2 = std::integral_constant<int, 2>;
-  using U3 = std::integral_constant<int, 3>;
-  using I7 = std::integral_constant<int, 7>;
   const uint32_t part_addr = q6_lds(&part[0][0][0]) + (uint32_t)((wave * 16 + n) * 4);
-  for (int r = 0; r < ng; r++) {
-    const int cur = r & 1;
-    // the round's buffer: own requests landed, then everybody's
-    if (r + 1 < ng) wait_groups(I1{});
-    else wait_groups(I0{});
-    q6_barrier();
-    const uint32_t buf = wbuf_base + (uint32_t)(cur * kQ6BufBytes);
-    acc = 0.f;
-    Regs ra, rb;
-    issue(U0{}, buf, ra);
-    issue(U1{}, buf, rb); settle(I7{}, ra); compute(ra);
-    issue(U2{}, buf, ra); settle(I7{}, rb); compute(rb);
-    issue(U3{}, buf, rb); settle(I7{}, ra); compute(ra);
-    settle(I0{}, rb);
-    // every wavefront has read what it needs of the buffer: the group after next may land there
-    q6_barrier();
-    if (r + 2 < ng) request_group(grp0 + r + 2, cur);
-    compute(rb);
-    // the four accumulator lanes of a row
-    acc += __shfl_xor(acc, 16, kWave);
-    acc += __shfl_xor(acc, 32, kWave);
-    if (lane < 16) q6_write_f32(part_addr + (uint32_t)(r * (kQ6Waves * 16 * 4)), acc);
-  }
+  // ODD: the wavefront's blocks sit two bytes into their slots
+  auto run_rounds = [&](auto oddc) {
+    constexpr bool ODD = decltype(oddc)::value;
+    // unit hf (half of the block): ql chunk 4 hf + g, qh chunk 8 + 2 hf + g % 2 (plus the first dword of the
+    // chunk after it when the block is shifted); scales in chunk 12 (accumulator lane (n, g): row n, k-set
+    // g / 2, plane g % 2; its four scales are consecutive bytes); d near the end of chunk 13
+    const uint32_t ql_off0 = chunk_at(slot + g), ql_off1 = chunk_at(slot + 4 + g);
+    const uint32_t qh_off0 = chunk_at(slot + 8 + (g & 1)), qh_off1 = chunk_at(slot + 10 + (g & 1));
+    const uint32_t qlx_off0 = chunk_at(slot + g + 1), qlx_off1 = chunk_at(slot + 4 + g + 1);
+    const uint32_t qhx_off0 = chunk_at(slot + 8 + (g & 1) + 1), qhx_off1 = chunk_at(slot + 10 + (g & 1) + 1);
+    const uint32_t sc_off = chunk_at(slot + 12) + (uint32_t)(4 * (g >> 1));
+    // shifted: the dword after the scales' (for the last one of the block that is byte 12 of chunk 13, which holds
+    // the block's bytes 194..209)
+    const uint32_t scx_off0 = sc_off + 4u;
+    const uint32_t scx_off1 = (g >> 1) ? chunk_at(slot + 13) + 12u : sc_off + 12u;
+    const uint32_t d_off = chunk_at(slot + 13) + (uint32_t)(kQ6DAt + (ODD ? 2 : 0));
+
+    struct Regs { q6_u32x4 ql, qh, a1, a2; uint32_t sc, d, f, qlx, qhx, scx; };
+    // unit hf of the round, k-half kh
+    auto issue = [&](auto hc, uint32_t buf, uint32_t kh, Regs& r) {
+      constexpr int hf = decltype(hc)::value;
+      const uint32_t a_ql = buf + (hf ? ql_off1 : ql_off0), a_qh = buf + (hf ? qh_off1 : qh_off0);
+      const uint32_t a_sc = buf + sc_off, a_d = buf + d_off;
+      const uint32_t ui = 16u * kh + (uint32_t)hf;
+      const uint32_t x1 = a1_addr + ui * a1_step, x2 = a2_addr + ui * a2_step;
+      const uint32_t fa = fac_addr0 + 16u * ui;
+      if constexpr (STAGE >= 2) return;
+      asm volatile(
+          "ds_read_b128 %0, %7\n\t"
+          "ds_read_b128 %1, %8\n\t"
+          "ds_read_b128 %2, %9\n\t"
+          "ds_read_b128 %3, %10\n\t"
+          "ds_read_b32 %4, %11 offset:%13\n\t"
+          "ds_read_u16 %5, %12\n\t"
+          "ds_read_b32 %6, %14"
+          : "=&v"(r.ql), "=&v"(r.qh), "=&v"(r.a1), "=&v"(r.a2), "=&v"(r.sc), "=&v"(r.d), "=&v"(r.f)
+          : "v"(a_ql), "v"(a_qh), "v"(x1), "v"(x2), "v"(a_sc), "v"(a_d), "n"(8 * hf), "v"(fa)
+          : "memory");
+      if constexpr (ODD) {
+        const uint32_t a_qlx = buf + (hf ? qlx_off1 : qlx_off0), a_qhx = buf + (hf ? qhx_off1 : qhx_off0);
+        const uint32_t a_scx = buf + (hf ? scx_off1 : scx_off0);
+        asm volatile(
+            "ds_read_b32 %0, %3\n\t"
+            "ds_read_b32 %1, %4\n\t"
+            "ds_read_b32 %2, %5"
+            : "=&v"(r.qlx), "=&v"(r.qhx), "=&v"(r.scx)
+            : "v"(a_qlx), "v"(a_qhx), "v"(a_scx)
+            : "memory");
+      }
+    };
+    constexpr int kReads = ODD ? 10 : 7;                   // LDS reads of a unit
+    auto settle = [&](auto pending, Regs& r) {
+      constexpr int P = decltype(pending)::value;
+      if constexpr (STAGE >= 2) return;
+      if constexpr (ODD)
+        asm volatile("s_waitcnt lgkmcnt(%10)"
+                     : "+v"(r.ql), "+v"(r.qh), "+v"(r.a1), "+v"(r.a2), "+v"(r.sc), "+v"(r.d), "+v"(r.f), "+v"(r.qlx),
+                       "+v"(r.qhx), "+v"(r.scx)
+                     : "n"(P)
+                     : "memory");
+      else
+        asm volatile("s_waitcnt lgkmcnt(%7)"
+                     : "+v"(r.ql), "+v"(r.qh), "+v"(r.a1), "+v"(r.a2), "+v"(r.sc), "+v"(r.d), "+v"(r.f)
+                     : "n"(P)
+                     : "memory");
+    };
+    float acc = 0.f;
+    auto compute = [&](const Regs& r) {
+      if constexpr (STAGE >= 1) return;
+      uint32_t ql[4], qh[4], sc4;
+      if constexpr (ODD) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          ql[i] = __builtin_amdgcn_alignbit(i < 3 ? r.ql[i + 1] : r.qlx, r.ql[i], 16);
+          qh[i] = __builtin_amdgcn_alignbit(i < 3 ? r.qh[i + 1] : r.qhx, r.qh[i], 16);
+        }
+        sc4 = __builtin_amdgcn_alignbit(r.scx, r.sc, 16);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          ql[i] = r.ql[i];
+          qh[i] = r.qh[i];
+        }
+        sc4 = r.sc;
+      }
+      v4i_t B1, B2, A1, A2;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        // 4 * (q - 32) as a signed byte: nibble into bits 2-5, bit pair into bits 6-7, low bits cleared and
+        // the top bit flipped
+        const uint32_t t1 = ((ql[i] << 2) & 0x3C3C3C3Cu) | ((qh[i] << sh1) & ~0x3C3C3C3Cu);
+        const uint32_t t2 = ((ql[i] >> 2) & 0x3C3C3C3Cu) | ((qh[i] << sh2) & ~0x3C3C3C3Cu);
+        B1[i] = (int)((t1 & 0xFCFCFCFCu) ^ 0x80808080u);
+        B2[i] = (int)((t2 & 0xFCFCFCFCu) ^ 0x80808080u);
+        A1[i] = (int)r.a1[i];
+        A2[i] = (int)r.a2[i];
+      }
+      const v4i_t zero = {0, 0, 0, 0};
+      v4i_t C = __builtin_amdgcn_mfma_i32_16x16x64_i8(A1, B1, zero, 0, 0, 0);
+      C = __builtin_amdgcn_mfma_i32_16x16x64_i8(A2, B2, C, 0, 0, 0);
+      const int sc = (int)sc4;
+      int t = (int)(int8_t)(sc & 0xFF) * C[0];
+      t += (int)(int8_t)((sc >> 8) & 0xFF) * C[1];
+      t += (int)(int8_t)((sc >> 16) & 0xFF) * C[2];
+      t += (sc >> 24) * C[3];
+      const float d = f16_bits_to_f32((uint16_t)(r.d & 0xFFFFu));
+      acc = fmaf_((float)t * __uint_as_float(r.f), d, acc);
+      // pins the arithmetic here: left alone the compiler moves it behind later waits
+      asm volatile("" : "+v"(acc));
+    };
+
+    using U0 = std::integral_constant<int, 0>;
+    using U1 = std::integral_constant<int, 1>;
+    int bufi = 0;
+    for (int rr = 0; rr < nrounds; rr++) {
+      // the round's buffer: own requests landed, then everybody's
+      const int later = min(nrounds - 1 - rr, kQ6Bufs - 1);        // rounds requested after this one
+      if (later == 3) wait_rounds(I3{});
+      else if (later == 2) wait_rounds(I2{});
+      else if (later == 1) wait_rounds(I1{});
+      else wait_rounds(I0{});
+      q6_barrier();
+      const uint32_t buf = wbuf_base + (uint32_t)(bufi * kQ6BufBytes);
+      const uint32_t kh = (uint32_t)(rr & 1);
+      Regs ra, rb;
+      issue(U0{}, buf, kh, ra);
+      issue(U1{}, buf, kh, rb);
+      settle(std::integral_constant<int, kReads>{}, ra);
+      compute(ra);
+      settle(I0{}, rb);
+      // every wavefront has read what it needs of the buffer: the round kQ6Bufs later may land there
+      q6_barrier();
+      if (rr + kQ6Bufs < nrounds) request_round(rr + kQ6Bufs, bufi);
+      bufi = bufi == kQ6Bufs - 1 ? 0 : bufi + 1;
+      compute(rb);
+      if (kh) {
+        // the four accumulator lanes of a row
+        acc += __shfl_xor(acc, 16, kWave);
+        acc += __shfl_xor(acc, 32, kWave);
+        if (lane < 16) q6_write_f32(part_addr + (uint32_t)((rr >> 1) * (kQ6Waves * 16 * 4)), acc);
+        acc = 0.f;
+      }
+    }
+  };
+  if (wave & 1) run_rounds(std::true_type{});
+  else run_rounds(std::false_type{});
   // every request has landed (plain loads are safe again); the eight K-slices of a row add up in a fixed order
   __syncthreads();
   for (int t = tid; t < ng * 16; t += kQ6Threads) {
@@ -318,7 +401,8 @@ template <typename XT, typename YT>
 hipError_t q6_launch_xy(const void* w, const void* x, void* y, const void* bias, int bias_dtype, int64_t m, int64_t n_out,
                         hipStream_t s) {
   const int groups = (int)(n_out / 16);
-  int num_wg = device_num_cus();
+  // two workgroups per compute unit when every one of them still gets two groups: their rounds interleave
+  int num_wg = min(kQ6WgsPerCu * device_num_cus(), groups / kQ6MinGroups);
   if ((groups + num_wg - 1) / num_wg > kQ6MaxGroups) num_wg = (groups + kQ6MaxGroups - 1) / kQ6MaxGroups;
   const dim3 grid((unsigned)num_wg, (unsigned)m), block(kQ6Threads);
   hipLaunchKernelGGL((gemv_q6k_stream_kernel<XT, YT>), grid, block, 0, s, static_cast<const uint8_t*>(w),
