@@ -424,7 +424,7 @@ def main() -> int:
         """Rows next to the headline ones, on random packed bytes with finite scale fields (timing
         only): the attention projections as decode GEMVs (q/o 4096x4096, k/v 1024x4096, reference call
         sites workspace/transformers/src/layers/attn.nim:113-116,154-156,189), the LM-head-sized Q4_K
-        stream, the few-row decode GEMV (8 and 16 activation rows at once), the few-row form of the
+        stream, a Q6_K down projection (mlp.nim:60), the few-row decode GEMV (8 and 16 activation rows at once), the few-row form of the
         prefill operator (32 rows) and the prefill GEMM for Q6_K and Q8_0 weights, 14336 x 4096 unless
         named otherwise; add + RMSNorm on rows of 4096."""
         n_out, n_in = 14336, 4096
@@ -453,6 +453,11 @@ def main() -> int:
             timed(nm, F.Q4_K, 1,
                   lambda ws, x, nc, y=y, no=no, ni=ni: (lambda i: QL.gemv(F.Q4_K, ws[i % nc], x, no, ni, out=y)),
                   n_out=no, n_in=ni, steps=steps if no < 100000 else max(20, steps // 10))
+        # Q6_K decode beside the LM head: the down projection of the layers that a "Q4_K_M" file stores as Q6_K
+        y = torch.empty((1, 4096), dtype=torch.float32, device=dev)
+        timed("q6_k_gemv_down_4096x14336", F.Q6_K, 1,
+              lambda ws, x, nc, y=y: (lambda i: QL.gemv(F.Q6_K, ws[i % nc], x, 4096, 14336, out=y)),
+              n_out=4096, n_in=14336)
         for m in (8, 16):
             y = torch.empty((m, n_out), dtype=torch.float32, device=dev)
             timed("q4_k_gemv_m%d" % m, F.Q4_K, m,

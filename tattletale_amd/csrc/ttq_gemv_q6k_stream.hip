@@ -1,5 +1,6 @@
-// Decode GEMV for Q6_K weights on gfx950 with rows of 4096 values (the LM head of a "Q4_K_M" file):
-// the weight stream goes HBM -> LDS as whole cache lines and feeds the int8 matrix cores.
+// Decode GEMV for Q6_K weights on gfx950 with rows of 2048 to 14336 values (in a "Q4_K_M" file: the LM head
+// and half of the down projections): the weight stream goes HBM -> LDS as whole cache lines and feeds the int8
+// matrix cores.
 //
 // Operator: F.linear with a single-token activation (workspace/libtorch/src/abi/neural_nets.nim:64-81) over a
 // weight stored as GGUF Q6_K blocks { u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d } of 256 weights,
@@ -8,21 +9,23 @@
 // A 210-byte block is neither a multiple of a cache line nor of a dword, so the per-wavefront line rings of the
 // Q4_K kernel (ttq_gemv_q4k_stream.h) do not carry over.  What is line-shaped is a group of 16 rows: 53 760
 // contiguous bytes = 420 lines.  So here the eight wavefronts of a workgroup share the stream:
-//   * a round is half of K of one group of 16 rows: 16 runs of 1680 contiguous bytes, copied into one of three
-//     LDS buffers by 28 requests of 1 KiB (global_load_lds_dwordx4, no registers), four or three per
+//   * a round is eight blocks (2048 values) of one group of 16 rows: 16 runs of 1680 contiguous bytes, copied
+//     into one of two or three LDS buffers by 28 requests of 1 KiB (global_load_lds_dwordx4, no registers), four or three per
 //     wavefront.  On the way in every block is moved to a 16-byte boundary: it lands in a slot of 14 chunks
 //     of 16 bytes, 13 fetched from consecutive addresses and one that ends with the block's last bytes, and
 //     row n is rotated by n chunks, which puts the 16 rows of an operand read into 16 different bank groups.
 //     Fetch addresses are rounded down to a dword: requests at 2 mod 4 were measured 15 % slower than
 //     dword-aligned ones, and operand reads at 2 mod 4 -- which the packed layout would need for every other
 //     block -- at three times the cost of the whole stream.  So an odd block lands two bytes into its slot,
-//     and the wavefronts that multiply odd blocks (the odd ones: block = 8 * half + wavefront) shift their
+//     and the wavefronts that multiply odd blocks (the odd ones: block = 8 * round + wavefront) shift their
 //     operands by 16 bits in registers;
-//   * while one buffer is multiplied, the next two rounds are in flight or landed (a compute unit takes about
+//   * while one buffer is multiplied, the next rounds are in flight or landed (a compute unit takes about
 //     64 KiB of outstanding requests); a wavefront waits for its own requests on its own counter, a barrier
-//     makes the buffer whole, a second one frees it for the round three later;
-//   * along K a round is split: wavefront w multiplies block w of the half for all 16 rows, two units of
-//     16 rows x 128 weights, two v_mfma_i32_16x16x64_i8 each.
+//     makes the buffer whole, a second one frees it for a later round;
+//   * along K a round is split: wavefront w multiplies block w of the eight for all 16 rows, two units of
+//     16 rows x 128 weights, two v_mfma_i32_16x16x64_i8 each;
+//   * rows of 4096 values and many of them (the LM head): two workgroups per compute unit with two buffers
+//     each, so that one's arithmetic falls into the other's waits; otherwise one workgroup with three buffers.
 // Arithmetic.  The activations are block fixed point, 15 bits in two byte planes with one power-of-two scale
 // per 64 values.  A weight reaches the matrix core as the signed byte 4 * (q6 - 32) = ((q6 << 2) ^ 0x80), built
 // from the nibble and the bit pair with four instructions per dword.  The 16 columns of the MFMA that a GEMV
@@ -40,33 +43,23 @@ namespace {
 
 constexpr int kQ6Waves = 8;
 constexpr int kQ6Threads = kQ6Waves * 64;
-constexpr int kQ6Nb = 16;                                  // blocks per row: n_in = 4096
-constexpr int kQ6RowBytes = kQ6Nb * 210;                   // 3360
-constexpr int kQ6GroupBytes = 16 * kQ6RowBytes;            // 53760 in memory
-constexpr int kQ6HalfBlocks = kQ6Nb / 2;                   // blocks of a row in one round: one per wavefront
+constexpr int kQ6RoundBlocks = 8;                          // blocks of a row in one round: one per wavefront
 constexpr int kQ6SlotChunks = 14;                          // a block in LDS: 224 bytes
 constexpr int kQ6TailAt = 196;                             // chunk 13 starts here, counted from the slot's first byte
 constexpr int kQ6DAt = 208 - kQ6TailAt;                    // d in chunk 13 (+ 2 for an odd block)
-constexpr int kQ6RowChunks = kQ6HalfBlocks * kQ6SlotChunks;   // 112
+constexpr int kQ6RowChunks = kQ6RoundBlocks * kQ6SlotChunks;   // 112
 constexpr int kQ6Requests = 16 * kQ6RowChunks / 64;        // 28
 constexpr int kQ6BufBytes = kQ6Requests * 1024;            // 28672
-#ifndef Q6_ORDER
-#define Q6_ORDER 0
-#endif
-#ifndef Q6_BUFS
-#define Q6_BUFS 2
-#endif
-#ifndef Q6_WGS_PER_CU
-#define Q6_WGS_PER_CU 2
-#endif
-constexpr int kQ6Bufs = Q6_BUFS;
 constexpr int kQ6ReqMax = (kQ6Requests + kQ6Waves - 1) / kQ6Waves;   // 4
 constexpr int kQ6FullWaves = kQ6Requests - (kQ6ReqMax - 1) * kQ6Waves;   // wavefronts 0..3 make 4 requests, the others 3
-constexpr int kQ6WgsPerCu = Q6_WGS_PER_CU;
-constexpr int kQ6MaxGroups = 40 / kQ6WgsPerCu;                           // row groups of a workgroup (their partial sums wait in LDS)
-constexpr int kQ6MinGroups = 2;
-static_assert(kQ6HalfBlocks == kQ6Waves, "one block of the half per wavefront");
-static_assert(kQ6Bufs >= 2 && kQ6Bufs <= 4, "the waits below count up to three later rounds");
+static_assert(kQ6RoundBlocks == kQ6Waves, "one block of the round per wavefront");
+
+// The two shapes of the kernel.  NBMAX: blocks per row it has tables for; BUFS: LDS buffers; WGS: workgroups per
+// compute unit; MAXG: row groups of a workgroup (their partial sums wait in LDS, in the space where the raw
+// activations land first).
+// FIXED: the row length is NBMAX blocks, known at compile time.
+struct Q6Head { static constexpr int NBMAX = 16, BUFS = 2, WGS = 2, MAXG = 20; static constexpr bool FIXED = true; };    // rows of 4096, many rows
+struct Q6Wide { static constexpr int NBMAX = 56, BUFS = 3, WGS = 1, MAXG = 56; static constexpr bool FIXED = false; };   // rows up to 14336
 
 typedef const __attribute__((address_space(1))) void* q6_gptr_t;
 typedef __attribute__((address_space(3))) void* q6_lptr_t;
@@ -98,22 +91,28 @@ __device__ __forceinline__ void q6_write_f32(uint32_t a, float v) {
 }
 
 // XT: bf16 or fp16 activations.  The row groups are dealt out in runs: the first groups_rem workgroups take
-// groups_per_wg + 1 each, the others groups_per_wg.
+// groups_per_wg + 1 each, the others groups_per_wg.  nb: blocks per row, a multiple of eight.
 // STAGE 0 is the GEMV; STAGE 1 leaves out the arithmetic on the operands, STAGE 2 the operand reads as well
 // (requests, waits and barriers stay): what each part costs is measured by leaving it out.
-template <typename XT, typename YT, int STAGE = 0>
-__global__ void __launch_bounds__(kQ6Threads) __attribute__((amdgpu_waves_per_eu(2 * kQ6WgsPerCu, 2 * kQ6WgsPerCu)))
+template <typename XT, typename YT, typename CFG, int STAGE = 0>
+__global__ void __launch_bounds__(kQ6Threads) __attribute__((amdgpu_waves_per_eu(2 * CFG::WGS, 2 * CFG::WGS)))
 gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
-                       const void* __restrict__ bias, int bias_dtype, int n_out, int groups_per_wg, int groups_rem) {
-  __shared__ __attribute__((aligned(1024))) uint8_t wbuf[kQ6Bufs * kQ6BufBytes];
-  __shared__ __attribute__((aligned(16))) v4i_t xa[kQ6Nb * 32 + 1];    // (16 values, plane) entries + one of zeros
-  __shared__ __attribute__((aligned(16))) float fac[kQ6Nb * 4 * 2];    // (64 values, plane): scale of the integer sum
+                       const void* __restrict__ bias, int bias_dtype, int n_out, int nb_arg, int groups_per_wg,
+                       int groups_rem) {
+  const int nb = CFG::FIXED ? CFG::NBMAX : nb_arg;
+  constexpr int kBufs = CFG::BUFS;
+  static_assert(kBufs >= 2 && kBufs <= 4, "the waits below count up to three later rounds");
+  __shared__ __attribute__((aligned(1024))) uint8_t wbuf[kBufs * kQ6BufBytes];
+  __shared__ __attribute__((aligned(16))) v4i_t xa[CFG::NBMAX * 32 + 1];   // (16 values, plane) entries + one of zeros
+  __shared__ __attribute__((aligned(16))) float fac[CFG::NBMAX * 4 * 2];   // (64 values, plane): scale of the integer sum
   // (the raw activations land here first: the partial sums are written after they have been read back)
-  __shared__ __attribute__((aligned(1024))) float part[kQ6MaxGroups][kQ6Waves][16];
-  static_assert(sizeof(part) >= kQ6Threads * 16, "room for the staged activations");
+  __shared__ __attribute__((aligned(1024))) float part[CFG::MAXG][kQ6Waves][16];
+  static_assert(sizeof(part) >= CFG::NBMAX * 512, "room for the staged activations");
   uint8_t* xstage = reinterpret_cast<uint8_t*>(&part[0][0][0]);
 
-  constexpr int n_in = kQ6Nb * 256;
+  const int n_in = nb * 256;
+  const int rpg = nb >> 3;                                // rounds per group
+  const uint32_t row_bytes = (uint32_t)nb * 210u;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 15, g = lane >> 4;
@@ -121,14 +120,19 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   YT* ym = y + (int64_t)blockIdx.y * n_out;
   const int bx = blockIdx.x;
   const int grp0 = bx * groups_per_wg + min(bx, groups_rem);
-  const int ng = groups_per_wg + (bx < groups_rem ? 1 : 0);            // kQ6MinGroups .. kQ6MaxGroups
-  const int nrounds = 2 * ng;
+  const int ng = groups_per_wg + (bx < groups_rem ? 1 : 0);            // 1 .. CFG::MAXG
+  const int nrounds = rpg * ng;                                          // >= kBufs (the launcher sees to it)
 
-  // ---- the activations, as an LDS request too (a register load among the weight requests would make the
-  // compiler wait for all of them at its first use): thread t stages x[8 t .. 8 t + 7]
-  const int k0 = 8 * tid;
-  __builtin_amdgcn_global_load_lds((q6_gptr_t)(xm + k0), (q6_lptr_t)(xstage + wave * 1024), 16, 0, 0);
-  // a compute unit serves its requests in the order they were made: every wavefront's activation request is
+  // ---- the activations, as LDS requests too (a register load among the weight requests would make the
+  // compiler wait for all of them at its first use): thread t stages x[8 t + 4096 i .. + 7]
+  constexpr int kXPasses = (CFG::NBMAX * 256 + 8 * kQ6Threads - 1) / (8 * kQ6Threads);
+#pragma unroll
+  for (int i = 0; i < kXPasses; i++) {
+    const int k0 = 8 * tid + i * (8 * kQ6Threads);
+    if (k0 < n_in)                                        // whole wavefronts: n_in is a multiple of 512
+      __builtin_amdgcn_global_load_lds((q6_gptr_t)(xm + k0), (q6_lptr_t)(xstage + i * (16 * kQ6Threads) + wave * 1024), 16, 0, 0);
+  }
+  // a compute unit serves its requests in the order they were made: every wavefront's activation requests are
   // queued before any weight request of the workgroup
   asm volatile("s_barrier" ::: "memory");
 
@@ -143,20 +147,29 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
     const int b = c / kQ6SlotChunks, j = c - b * kQ6SlotChunks;
     // an odd block starts at 2 mod 4: its slot starts two bytes early.  The last chunk of an even block reads two
     // bytes into the next block of the row; the last chunk of an odd block ends with the block.
-    src_off[i] = (uint32_t)(row * kQ6RowBytes + b * 210 - 2 * (b & 1) + (j < kQ6SlotChunks - 1 ? 16 * j : kQ6TailAt));
+    src_off[i] = (uint32_t)row * row_bytes + (uint32_t)(b * 210 - 2 * (b & 1) + (j < kQ6SlotChunks - 1 ? 16 * j : kQ6TailAt));
   }
   const bool full = wave < kQ6FullWaves;
-  // round rr = 2 * (group - grp0) + (half of K)
-  auto request_round = [&](int rr, int buf) {
-    const uint8_t* src = w + (size_t)((uint32_t)(grp0 + (rr >> 1)) * (uint32_t)kQ6GroupBytes +
-                                      (uint32_t)((rr & 1) * (kQ6HalfBlocks * 210)));
-    uint8_t* dst = wbuf + buf * kQ6BufBytes + wave * 1024;
+  // rounds are requested in order: group by group, eight blocks by eight blocks
+  uint32_t req_src = (uint32_t)grp0 * 16u * row_bytes;    // byte offset of the next round to request
+  int req_kr = 0, req_buf = 0;
+  auto request_next = [&]() {
+    const uint8_t* src = w + (size_t)req_src;
+    uint8_t* dst = wbuf + req_buf * kQ6BufBytes + wave * 1024;
 #pragma unroll
     for (int i = 0; i < kQ6ReqMax - 1; i++)
       __builtin_amdgcn_global_load_lds((q6_gptr_t)(src + src_off[i]), (q6_lptr_t)(dst + i * (kQ6Waves * 1024)), 16, 0, 2);
     if (full)
       __builtin_amdgcn_global_load_lds((q6_gptr_t)(src + src_off[kQ6ReqMax - 1]),
                                        (q6_lptr_t)(dst + (kQ6ReqMax - 1) * (kQ6Waves * 1024)), 16, 0, 2);
+    req_buf = req_buf == kBufs - 1 ? 0 : req_buf + 1;
+    // the next eight blocks of the rows, or the first eight of the next group
+    req_kr++;
+    req_src += kQ6RoundBlocks * 210;
+    if (req_kr == rpg) {
+      req_kr = 0;
+      req_src += 15u * row_bytes;
+    }
   };
   // all but the youngest `rounds_after` rounds of requests of this wavefront have landed
   auto wait_rounds = [&](auto rounds_after) {
@@ -169,20 +182,21 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   using I2 = std::integral_constant<int, 2>;
   using I3 = std::integral_constant<int, 3>;
 #pragma unroll
-  for (int i = 0; i < kQ6Bufs; i++) request_round(i, i);      // nrounds >= 4
+  for (int i = 0; i < kBufs; i++) request_next();
 
   // ---- the raw activations back into registers, then into the two byte planes
-  float xf[8];
-  {
-    wait_rounds(std::integral_constant<int, kQ6Bufs>{});
-    const q6_u32x4 r = q6_read16(q6_lds(xstage) + (uint32_t)(tid * 16));
+  wait_rounds(std::integral_constant<int, kBufs>{});
+  if (tid < 4) reinterpret_cast<uint32_t*>(&xa[CFG::NBMAX * 32])[tid] = 0u;
+#pragma unroll
+  for (int i = 0; i < kXPasses; i++) {
+    const int k0 = 8 * tid + i * (8 * kQ6Threads);
+    if (k0 >= n_in) break;
+    float xf[8];
+    const q6_u32x4 r = q6_read16(q6_lds(xstage) + (uint32_t)(i * (16 * kQ6Threads) + tid * 16));
     widen8<XT>(make_uint4(r[0], r[1], r[2], r[3]), xf);
-  }
-  if (tid < 4) reinterpret_cast<uint32_t*>(&xa[kQ6Nb * 32])[tid] = 0u;
-  {
     float amax = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(xf[i]));
+    for (int j = 0; j < 8; j++) amax = fmaxf(amax, fabsf(xf[j]));
     // the eight threads of 64 values are an aligned octet
     amax = fmaxf(amax, dpp_quad<0xB1>(amax));
     amax = fmaxf(amax, dpp_quad<0x4E>(amax));
@@ -194,10 +208,10 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
     const float f = eb == 255u ? __uint_as_float(0x7FC00000u) : __uint_as_float((ec - 13u) << 23);
     int hi[8], lo[8];
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      const int v = (int)rintf(xf[i] * mul);
-      hi[i] = (v + 128) >> 8;
-      lo[i] = v;                     // only the low byte is used, as a signed byte
+    for (int j = 0; j < 8; j++) {
+      const int v = (int)rintf(xf[j] * mul);
+      hi[j] = (v + 128) >> 8;
+      lo[j] = v;                     // only the low byte is used, as a signed byte
     }
     // entry (k / 16, plane), 16 bytes; this thread's eight values are one half of it
     uint2* xa8 = reinterpret_cast<uint2*>(&xa[0]);
@@ -220,18 +234,18 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
     const int pos = c + n < kQ6RowChunks ? c + n : c + n - kQ6RowChunks;
     return (uint32_t)((n * kQ6RowChunks + pos) * 16);
   };
-  const int slot = wave * kQ6SlotChunks;                   // the wavefront's block of the half
+  const int slot = wave * kQ6SlotChunks;                   // the wavefront's block of the round
   // activation operand: lane (i, g) of the first MFMA holds something only if i < 8 and i % 4 == g, of the
   // second only if i >= 8 and i % 4 == g; plane (i / 4) % 2.  Unit u = 2 block + half starts at value 128 u.
   const uint32_t xa_base = q6_lds(&xa[0]);
-  const uint32_t zero_entry = xa_base + (uint32_t)(kQ6Nb * 32 * 16);
+  const uint32_t zero_entry = xa_base + (uint32_t)(CFG::NBMAX * 32 * 16);
   const bool mine = (n & 3) == g;
   const uint32_t plane16 = (uint32_t)(((n >> 2) & 1) * 16);
   const bool act1 = mine && n < 8, act2 = mine && n >= 8;
-  const uint32_t u0 = (uint32_t)(2 * wave);                // the wavefront's first unit of a first half of K
+  const uint32_t u0 = (uint32_t)(2 * wave);                // the wavefront's first unit of a group's first round
   const uint32_t a1_addr = act1 ? xa_base + 256u * u0 + 32u * (uint32_t)g + plane16 : zero_entry;
   const uint32_t a2_addr = act2 ? xa_base + 256u * u0 + 128u + 32u * (uint32_t)g + plane16 : zero_entry;
-  // per unit 256 bytes of table, per half of K 16 units
+  // per unit 256 bytes of table, per round 16 units
   const uint32_t a1_step = act1 ? 256u : 0u, a2_step = act2 ? 256u : 0u;
   const uint32_t fac_addr0 = q6_lds(&fac[0]) + 16u * u0 + 4u * (uint32_t)g;
   const uint32_t wbuf_base = q6_lds(wbuf);
@@ -257,12 +271,12 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
     const uint32_t d_off = chunk_at(slot + 13) + (uint32_t)(kQ6DAt + (ODD ? 2 : 0));
 
     struct Regs { q6_u32x4 ql, qh, a1, a2; uint32_t sc, d, f, qlx, qhx, scx; };
-    // unit hf of the round, k-half kh
-    auto issue = [&](auto hc, uint32_t buf, uint32_t kh, Regs& r) {
+    // unit hf of the round, round kr of the group
+    auto issue = [&](auto hc, uint32_t buf, uint32_t kr, Regs& r) {
       constexpr int hf = decltype(hc)::value;
       const uint32_t a_ql = buf + (hf ? ql_off1 : ql_off0), a_qh = buf + (hf ? qh_off1 : qh_off0);
       const uint32_t a_sc = buf + sc_off, a_d = buf + d_off;
-      const uint32_t ui = 16u * kh + (uint32_t)hf;
+      const uint32_t ui = 16u * kr + (uint32_t)hf;
       const uint32_t x1 = a1_addr + ui * a1_step, x2 = a2_addr + ui * a2_step;
       const uint32_t fa = fac_addr0 + 16u * ui;
       if constexpr (STAGE >= 2) return;
@@ -352,34 +366,35 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
 
     using U0 = std::integral_constant<int, 0>;
     using U1 = std::integral_constant<int, 1>;
-    int bufi = 0;
+    int bufi = 0, kr = 0, gi = 0;
     for (int rr = 0; rr < nrounds; rr++) {
       // the round's buffer: own requests landed, then everybody's
-      const int later = min(nrounds - 1 - rr, kQ6Bufs - 1);        // rounds requested after this one
+      const int later = min(nrounds - 1 - rr, kBufs - 1);          // rounds requested after this one
       if (later == 3) wait_rounds(I3{});
       else if (later == 2) wait_rounds(I2{});
       else if (later == 1) wait_rounds(I1{});
       else wait_rounds(I0{});
       q6_barrier();
       const uint32_t buf = wbuf_base + (uint32_t)(bufi * kQ6BufBytes);
-      const uint32_t kh = (uint32_t)(rr & 1);
       Regs ra, rb;
-      issue(U0{}, buf, kh, ra);
-      issue(U1{}, buf, kh, rb);
+      issue(U0{}, buf, (uint32_t)kr, ra);
+      issue(U1{}, buf, (uint32_t)kr, rb);
       settle(std::integral_constant<int, kReads>{}, ra);
       compute(ra);
       settle(I0{}, rb);
-      // every wavefront has read what it needs of the buffer: the round kQ6Bufs later may land there
+      // every wavefront has read what it needs of the buffer: a later round may land there
       q6_barrier();
-      if (rr + kQ6Bufs < nrounds) request_round(rr + kQ6Bufs, bufi);
-      bufi = bufi == kQ6Bufs - 1 ? 0 : bufi + 1;
+      if (rr + kBufs < nrounds) request_next();
+      bufi = bufi == kBufs - 1 ? 0 : bufi + 1;
       compute(rb);
-      if (kh) {
-        // the four accumulator lanes of a row
+      if (++kr == rpg) {
+        // the group is complete: the four accumulator lanes of a row
         acc += __shfl_xor(acc, 16, kWave);
         acc += __shfl_xor(acc, 32, kWave);
-        if (lane < 16) q6_write_f32(part_addr + (uint32_t)((rr >> 1) * (kQ6Waves * 16 * 4)), acc);
+        if (lane < 16) q6_write_f32(part_addr + (uint32_t)(gi * (kQ6Waves * 16 * 4)), acc);
         acc = 0.f;
+        kr = 0;
+        gi++;
       }
     }
   };
@@ -397,48 +412,72 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   }
 }
 
+// Which shape of the kernel takes (n_out, n_in), with how many workgroups; ok == false: neither.
+struct Q6Plan { bool ok, head; int num_wg; };
+Q6Plan q6_plan(int64_t n_out, int64_t n_in) {
+  Q6Plan p{false, false, 0};
+  const int64_t nb = n_in / 256;
+  // whole rounds of eight blocks, whole groups of 16 rows, 32-bit byte offsets into the weight buffer
+  if (n_in % (256 * kQ6RoundBlocks) != 0 || nb > Q6Wide::NBMAX || n_out % 16 != 0) return p;
+  if (n_out * nb * 210 >= ((int64_t)1 << 32)) return p;
+  const int64_t groups = n_out / 16;
+  const int cus = device_num_cus();
+  if (groups < cus) return p;                              // a group or more for every compute unit
+  int maxg;
+  if (nb == Q6Head::NBMAX && groups >= 2 * (int64_t)Q6Head::WGS * cus) {
+    // two workgroups per compute unit when each still gets two groups: their rounds interleave
+    p.head = true;
+    p.num_wg = Q6Head::WGS * cus;
+    maxg = Q6Head::MAXG;
+  } else {
+    p.num_wg = cus;
+    maxg = Q6Wide::MAXG;
+    if ((groups / cus) * (nb / kQ6RoundBlocks) < Q6Wide::BUFS) return p;   // every buffer is requested up front
+  }
+  if ((groups + p.num_wg - 1) / p.num_wg > maxg) p.num_wg = (int)((groups + maxg - 1) / maxg);
+  p.ok = true;
+  return p;
+}
+
 template <typename XT, typename YT>
 hipError_t q6_launch_xy(const void* w, const void* x, void* y, const void* bias, int bias_dtype, int64_t m, int64_t n_out,
-                        hipStream_t s) {
+                        int64_t n_in, hipStream_t s) {
+  const Q6Plan p = q6_plan(n_out, n_in);
+  if (!p.ok) return hipErrorInvalidValue;
   const int groups = (int)(n_out / 16);
-  // two workgroups per compute unit when every one of them still gets two groups: their rounds interleave
-  int num_wg = min(kQ6WgsPerCu * device_num_cus(), groups / kQ6MinGroups);
-  if ((groups + num_wg - 1) / num_wg > kQ6MaxGroups) num_wg = (groups + kQ6MaxGroups - 1) / kQ6MaxGroups;
-  const dim3 grid((unsigned)num_wg, (unsigned)m), block(kQ6Threads);
-  hipLaunchKernelGGL((gemv_q6k_stream_kernel<XT, YT>), grid, block, 0, s, static_cast<const uint8_t*>(w),
-                     static_cast<const uint16_t*>(x), static_cast<YT*>(y), bias, bias_dtype, (int)n_out, groups / num_wg,
-                     groups % num_wg);
+  const dim3 grid((unsigned)p.num_wg, (unsigned)m), block(kQ6Threads);
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, block, 0, s, static_cast<const uint8_t*>(w), static_cast<const uint16_t*>(x),
+                       static_cast<YT*>(y), bias, bias_dtype, (int)n_out, (int)(n_in / 256), groups / p.num_wg,
+                       groups % p.num_wg);
+  };
+  if (p.head) go(gemv_q6k_stream_kernel<XT, YT, Q6Head>);
+  else go(gemv_q6k_stream_kernel<XT, YT, Q6Wide>);
   return hipGetLastError();
 }
 
 template <typename XT>
 hipError_t q6_launch_x(const void* w, const void* x, void* y, int y_dtype, const void* bias, int bias_dtype, int64_t m,
-                       int64_t n_out, hipStream_t s) {
+                       int64_t n_out, int64_t n_in, hipStream_t s) {
   switch (y_dtype) {
-    case kF32: return q6_launch_xy<XT, float>(w, x, y, bias, bias_dtype, m, n_out, s);
-    case kF16: return q6_launch_xy<XT, f16_tag>(w, x, y, bias, bias_dtype, m, n_out, s);
-    case kBF16: return q6_launch_xy<XT, bf16_tag>(w, x, y, bias, bias_dtype, m, n_out, s);
+    case kF32: return q6_launch_xy<XT, float>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kF16: return q6_launch_xy<XT, f16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kBF16: return q6_launch_xy<XT, bf16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
     default: return hipErrorInvalidValue;
   }
 }
 
 }  // namespace
 
-// Whole groups of 16 rows, at least two per compute unit (the two LDS buffers are requested before anything
-// else), 32-bit byte offsets into the weight buffer.
 bool gemv_q6k_stream_supported(int format, int x_dtype, int64_t n_out, int64_t n_in) {
   if (format != kQ6_K || !(x_dtype == kBF16 || x_dtype == kF16)) return false;
-  if (n_in != kQ6Nb * 256 || n_out % 16 != 0) return false;
-  static const int off = dev_knob("TTQ_Q6K_STREAM_OFF", 0);
-  if (off) return false;
-  return n_out / 16 >= (int64_t)kQ6MinGroups * device_num_cus() && n_out * kQ6RowBytes < ((int64_t)1 << 32);
+  return q6_plan(n_out, n_in).ok;
 }
 
 hipError_t launch_gemv_q6k_stream(const void* w, const void* x, int x_dtype, void* y, int y_dtype, const void* bias,
                                   int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
-  (void)n_in;
-  if (x_dtype == kBF16) return q6_launch_x<bf16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, s);
-  if (x_dtype == kF16) return q6_launch_x<f16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, s);
+  if (x_dtype == kBF16) return q6_launch_x<bf16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  if (x_dtype == kF16) return q6_launch_x<f16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   return hipErrorInvalidValue;
 }
 

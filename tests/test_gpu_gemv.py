@@ -423,3 +423,27 @@ def test_q6_k_streamed_activation_extremes_bias_and_output_types():
         layer = QuantLinear.init(wd, F.Q6_K, n_in, n_out, bias=torch.from_numpy(bias).to(DEV))
         yy = layer.forward(xd1, out_dtype=out_dtype).float().cpu().numpy().reshape(-1)
         assert rel_l2(yy, want1) <= tol, out_dtype
+
+
+@pytest.mark.parametrize("xk", ["bf16", "f16"])
+@pytest.mark.parametrize("n_out,n_in", [(4096, 14336), (8192, 4096), (4096 + 16 * 5, 8192), (12288 + 48, 2048),
+                                        (4096 + 16, 6144), (4096, 12288)])
+def test_q6_k_streamed_other_row_lengths(xk, n_out, n_in):
+    """Rows of 2048 to 14336 values (one to seven rounds of eight blocks per group of 16 rows), one workgroup
+    per compute unit: normal activations against the float64 product, and unit vectors -- in the first and the
+    last round, in an odd and an even block -- against the canonical columns, bit for bit."""
+    p = random_blocks(F.Q6_K, n_out * (n_in // 256), seed=51 + n_in // 256)
+    what = oracle.dequant(F.Q6_K, p, n_out, n_in)
+    wd = packed_to_dev(p)
+    xd, xf = x_to_dev(Q.fill_normal(52, 1, 1.0, n_in), xk)
+    y = QL.gemv(F.Q6_K, wd, xd, n_out, n_in).cpu().numpy()[0]
+    assert rel_l2(y, oracle.linear_f64(what, xf)[0]) <= TOL
+    for c, s in ((0, 1.0), (255, -2.0), (256 + 97, 1.0), (2047, 0.5), (n_in - 2048 + 300, 1.0), (n_in - 1, 1.0)):
+        x = np.zeros((1, n_in), np.float32)
+        x[0, c] = s
+        xd, _ = x_to_dev(x, xk)
+        y = QL.gemv(F.Q6_K, wd, xd, n_out, n_in).cpu().numpy()[0]
+        col = what[:, c] * np.float32(s)
+        assert np.array_equal(y, col), c
+        nz = col != 0
+        assert np.array_equal(y[nz].view(np.uint32), col[nz].view(np.uint32)), c
