@@ -161,9 +161,12 @@ def test_packed_dot_few_rows(fmt, n_out, n_in, xk, m):
     want = oracle.linear_f64(what, xf)
     for r in range(m):
         assert rel_l2(y[r][rows], want[r]) <= TOL, r
+    # a single row of Q6_K with whole rounds of 2048 values and a row group per compute unit takes the streamed
+    # matrix-core kernel, whose activations are 15-bit block fixed point: same class, different rounding
+    same = 3e-4 if fmt == F.Q6_K and n_in % 2048 == 0 and n_in <= 14336 and n_out % 16 == 0 else 2e-6
     for r in {0, m - 1}:
         y1 = QL.gemv(fmt, wd, xd[r:r + 1], n_out, n_in).cpu().numpy()[0]
-        assert rel_l2(y[r], y1) <= 2e-6, r
+        assert rel_l2(y[r], y1) <= same, r
 
 
 @pytest.mark.parametrize("n_in", [1024, 8192])
