@@ -458,6 +458,10 @@ def main() -> int:
         timed("q6_k_gemv_down_4096x14336", F.Q6_K, 1,
               lambda ws, x, nc, y=y: (lambda i: QL.gemv(F.Q6_K, ws[i % nc], x, 4096, 14336, out=y)),
               n_out=4096, n_in=14336)
+        # Q8_0 decode on the headline shape (every projection of a Q8_0 file is a Q8_0 stream)
+        y = torch.empty((1, n_out), dtype=torch.float32, device=dev)
+        timed("q8_0_gemv_14336x4096", F.Q8_0, 1,
+              lambda ws, x, nc, y=y: (lambda i: QL.gemv(F.Q8_0, ws[i % nc], x, n_out, n_in, out=y)))
         for m in (8, 16):
             y = torch.empty((m, n_out), dtype=torch.float32, device=dev)
             timed("q4_k_gemv_m%d" % m, F.Q4_K, m,

@@ -341,6 +341,8 @@ hipError_t launch_gemv(int format, const void* w, const void* x, int x_dtype, vo
     return launch_gemv_q6k_stream(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   if (gemv_mfma_supported(format, x_dtype, n_out, n_in))
     return launch_gemv_mfma(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  if (m == 1 && gemv_q8_stream_supported(format, x_dtype, n_out, n_in))
+    return launch_gemv_q8_stream(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   if (gemv_q8_win_supported(format, n_out, n_in))
     return launch_gemv_q8_win(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   if (gemv_q8_mfma_supported(format, n_out, n_in))

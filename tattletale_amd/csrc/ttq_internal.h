@@ -66,6 +66,14 @@ hipError_t launch_gemv_q4k_stream(const void* w, const void* x, int x_dtype, voi
                                   const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                                   hipStream_t s);
 
+// Q8_0 through the int8 matrix cores with the raw bytes of the rows as the K dimension, streamed through three LDS
+// buffers (ttq_gemv_q8_stream.hip): n_in a multiple of 2048 up to 8192 (4096 for fp32 activations), whole groups of
+// 16 rows, at least one per compute unit.
+bool gemv_q8_stream_supported(int format, int x_dtype, int64_t n_out, int64_t n_in);
+hipError_t launch_gemv_q8_stream(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                                 const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                                 hipStream_t s);
+
 // Q6_K through the int8 matrix cores, 16 rows at a time streamed linearly through two LDS buffers
 // (ttq_gemv_q6k_stream.hip): 16-bit activations, n_in 4096, whole groups of 16 rows, at least two per compute unit.
 bool gemv_q6k_stream_supported(int format, int x_dtype, int64_t n_out, int64_t n_in);

@@ -447,3 +447,77 @@ def test_q6_k_streamed_other_row_lengths(xk, n_out, n_in):
         assert np.array_equal(y, col), c
         nz = col != 0
         assert np.array_equal(y[nz].view(np.uint32), col[nz].view(np.uint32)), c
+
+
+# ------------------------------------------------------------------- Q8_0, LDS-streamed kernel
+# (rows of 2048 .. 8192 values -- 4096 at most for fp32 activations --, whole groups of 16 rows, at least six
+# rounds of 2048 weights x 16 rows per compute unit; a single activation row)
+@pytest.mark.parametrize("xk", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("n_out,n_in", [(12288 + 16 * 5, 4096), (24576 + 16 * 3, 2048), (8192 + 16, 8192), (8192 + 16 * 7, 6144)])
+def test_q8_0_streamed_unit_vectors_and_random_activations(xk, n_out, n_in):
+    """Random block bytes (every weight value, negative and tiny scales).  Unit vectors, also scaled by a power
+    of two, reproduce the canonical column bit for bit: first and last weights of even and odd blocks, weights
+    whose byte is the first or the last of a 16-byte chunk, of a 64-byte MFMA, of a 2176-byte round, and the
+    first and last columns of every round.  Then normal activations against the float64 product, every row."""
+    p = random_blocks(F.Q8_0, n_out * (n_in // 32), seed=61 + n_in // 32)
+    what = oracle.dequant(F.Q8_0, p, n_out, n_in)
+    wd = packed_to_dev(p)
+    cols = [0, 1, 13, 14, 15, 29, 30, 31, 32, 33, 43, 44, 45, 46, 59, 60, 61, 62, 63, 64, 95, 96, 127, 128, 1023, 1024,
+            1054, 1055, 2046, 2047, n_in - 2049, n_in - 2048, n_in - 1025, n_in - 33, n_in - 32, n_in - 1]
+    cols = sorted({c for c in cols if 0 <= c < n_in})
+    for i, c in enumerate(cols):
+        s = (1.0, -0.5, 4.0)[i % 3]
+        x = np.zeros((1, n_in), np.float32)
+        x[0, c] = s
+        xd, _ = x_to_dev(x, xk)
+        y = QL.gemv(F.Q8_0, wd, xd, n_out, n_in).cpu().numpy()[0]
+        col = what[:, c] * np.float32(s)
+        assert np.array_equal(y, col), c
+        nz = col != 0
+        assert np.array_equal(y[nz].view(np.uint32), col[nz].view(np.uint32)), c
+    xd, xf = x_to_dev(Q.fill_normal(62, 1, 1.0, n_in), xk)
+    y = QL.gemv(F.Q8_0, wd, xd, n_out, n_in).cpu().numpy()[0]
+    assert rel_l2(y, oracle.linear_f64(what, xf)[0]) <= TOL
+
+
+@pytest.mark.parametrize("extra_groups", [0, 1, 255, 300, 1000])
+def test_q8_0_streamed_group_counts(extra_groups):
+    """Quantized normal weights; group counts that divide evenly among the compute units and ones that do not,
+    three to seven groups per workgroup."""
+    n_in = 4096
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    n_out = 16 * (3 * cus + extra_groups)
+    p, what = make(F.Q8_0, n_out, n_in, 400 + extra_groups)
+    xd, xf = x_to_dev(Q.fill_normal(401, 1, 1.0, n_in), "bf16")
+    y = QL.gemv(F.Q8_0, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()[0]
+    want = oracle.linear_f64(what, xf)[0]
+    assert rel_l2(y, want) <= TOL
+    assert np.max(np.abs(y - want)) <= 8e-3 * np.sqrt(np.mean(want ** 2))
+
+
+def test_q8_0_streamed_activation_extremes_bias_and_output_types():
+    n_in = 4096
+    n_out = 12288 + 16 * 5
+    p, what = make(F.Q8_0, n_out, n_in, 191)
+    wd = packed_to_dev(p)
+    x = np.zeros((4, n_in), np.float32)
+    x[1] = Q.fill_normal(192, 1, 1e-3, n_in)
+    x[1, 100] = 3.0e4
+    x[2] = Q.fill_normal(193, 1, 1.0, n_in)
+    x[2, 4095] = np.inf
+    x[3] = Q.fill_normal(194, 1, 1.0, n_in) * 1e-30
+    for xk in ("f32", "bf16"):
+        xd, xf = x_to_dev(x, xk)
+        y = gemv_row_by_row(F.Q8_0, wd, xd, n_out, n_in)
+        want = oracle.linear_f64(what, xf[[0, 1, 3]])
+        assert np.array_equal(y[0], np.zeros(n_out, np.float32))
+        assert rel_l2(y[1], want[1]) <= TOL
+        assert not np.any(np.isfinite(y[2]))
+        assert rel_l2(y[3], want[2]) <= TOL
+    bias = Q.fill_normal(195, 0, 0.5, n_out)
+    xd1, xf1 = x_to_dev(Q.fill_normal(196, 1, 1.0, n_in), "f16")
+    want1 = oracle.linear_f64(what, xf1).reshape(-1) + bias
+    for out_dtype, tol in ((torch.float32, TOL), (torch.bfloat16, 4e-3), (torch.float16, 1e-3)):
+        layer = QuantLinear.init(wd, F.Q8_0, n_in, n_out, bias=torch.from_numpy(bias).to(DEV))
+        yy = layer.forward(xd1, out_dtype=out_dtype).float().cpu().numpy().reshape(-1)
+        assert rel_l2(yy, want1) <= tol, out_dtype
