@@ -35,7 +35,7 @@
 // weigh.  Integer sums are exact; each (row, unit) then takes one float multiply by a power of two and one
 // fused multiply-add with d.  A unit-vector activation reproduces the canonical column bit for bit (d, scale
 // and q6 - 32 have 11 + 7 + 6 significant bits, so every order of the products is exact).
-#include "ttq_gemv_mfma_common.h"
+#include "ttq_stream_common.h"
 
 namespace ttq {
 
@@ -60,35 +60,6 @@ static_assert(kQ6RoundBlocks == kQ6Waves, "one block of the round per wavefront"
 // FIXED: the row length is NBMAX blocks, known at compile time.
 struct Q6Head { static constexpr int NBMAX = 16, BUFS = 2, WGS = 2, MAXG = 20; static constexpr bool FIXED = true; };    // rows of 4096, many rows
 struct Q6Wide { static constexpr int NBMAX = 56, BUFS = 3, WGS = 1, MAXG = 56; static constexpr bool FIXED = false; };   // rows up to 14336
-
-typedef const __attribute__((address_space(1))) void* q6_gptr_t;
-typedef __attribute__((address_space(3))) void* q6_lptr_t;
-typedef uint32_t q6_u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t q6_u32x2 __attribute__((ext_vector_type(2)));
-
-template <int N>
-__device__ __forceinline__ void q6_wait_vmcnt() {
-  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-  asm volatile("" ::: "memory");
-}
-// a barrier that leaves the outstanding requests alone
-__device__ __forceinline__ void q6_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-__device__ __forceinline__ uint32_t q6_lds(const void* p) { return (uint32_t)(size_t)(q6_lptr_t)(p); }
-// LDS accesses the compiler must not see: it cannot tell them from the asynchronous writes of the requests in
-// flight and would wait for every one of those first
-__device__ __forceinline__ q6_u32x4 q6_read16(uint32_t a) {
-  q6_u32x4 v;
-  asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(a) : "memory");
-  return v;
-}
-__device__ __forceinline__ float q6_read_f32(uint32_t a) {
-  float v;
-  asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(a) : "memory");
-  return v;
-}
-__device__ __forceinline__ void q6_write_f32(uint32_t a, float v) {
-  asm volatile("ds_write_b32 %0, %1" ::"v"(a), "v"(v) : "memory");
-}
 
 // XT: bf16 or fp16 activations.  The row groups are dealt out in runs: the first groups_rem workgroups take
 // groups_per_wg + 1 each, the others groups_per_wg.  nb: blocks per row, a multiple of eight.
@@ -130,7 +101,7 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   for (int i = 0; i < kXPasses; i++) {
     const int k0 = 8 * tid + i * (8 * kQ6Threads);
     if (k0 < n_in)                                        // whole wavefronts: n_in is a multiple of 512
-      __builtin_amdgcn_global_load_lds((q6_gptr_t)(xm + k0), (q6_lptr_t)(xstage + i * (16 * kQ6Threads) + wave * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((sm_gptr_t)(xm + k0), (sm_lptr_t)(xstage + i * (16 * kQ6Threads) + wave * 1024), 16, 0, 0);
   }
   // a compute unit serves its requests in the order they were made: every wavefront's activation requests are
   // queued before any weight request of the workgroup
@@ -158,10 +129,10 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
     uint8_t* dst = wbuf + req_buf * kQ6BufBytes + wave * 1024;
 #pragma unroll
     for (int i = 0; i < kQ6ReqMax - 1; i++)
-      __builtin_amdgcn_global_load_lds((q6_gptr_t)(src + src_off[i]), (q6_lptr_t)(dst + i * (kQ6Waves * 1024)), 16, 0, 2);
+      __builtin_amdgcn_global_load_lds((sm_gptr_t)(src + src_off[i]), (sm_lptr_t)(dst + i * (kQ6Waves * 1024)), 16, 0, 2);
     if (full)
-      __builtin_amdgcn_global_load_lds((q6_gptr_t)(src + src_off[kQ6ReqMax - 1]),
-                                       (q6_lptr_t)(dst + (kQ6ReqMax - 1) * (kQ6Waves * 1024)), 16, 0, 2);
+      __builtin_amdgcn_global_load_lds((sm_gptr_t)(src + src_off[kQ6ReqMax - 1]),
+                                       (sm_lptr_t)(dst + (kQ6ReqMax - 1) * (kQ6Waves * 1024)), 16, 0, 2);
     req_buf = req_buf == kBufs - 1 ? 0 : req_buf + 1;
     // the next eight blocks of the rows, or the first eight of the next group
     req_kr++;
@@ -174,8 +145,8 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   // all but the youngest `rounds_after` rounds of requests of this wavefront have landed
   auto wait_rounds = [&](auto rounds_after) {
     constexpr int A = decltype(rounds_after)::value;
-    if (full) q6_wait_vmcnt<A * kQ6ReqMax>();
-    else q6_wait_vmcnt<A * (kQ6ReqMax - 1)>();
+    if (full) sm_wait_vmcnt<A * kQ6ReqMax>();
+    else sm_wait_vmcnt<A * (kQ6ReqMax - 1)>();
   };
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
@@ -192,7 +163,7 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
     const int k0 = 8 * tid + i * (8 * kQ6Threads);
     if (k0 >= n_in) break;
     float xf[8];
-    const q6_u32x4 r = q6_read16(q6_lds(xstage) + (uint32_t)(i * (16 * kQ6Threads) + tid * 16));
+    const sm_u32x4 r = sm_read16(sm_lds(xstage) + (uint32_t)(i * (16 * kQ6Threads) + tid * 16));
     widen8<XT>(make_uint4(r[0], r[1], r[2], r[3]), xf);
     float amax = 0.f;
 #pragma unroll
@@ -237,7 +208,7 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   const int slot = wave * kQ6SlotChunks;                   // the wavefront's block of the round
   // activation operand: lane (i, g) of the first MFMA holds something only if i < 8 and i % 4 == g, of the
   // second only if i >= 8 and i % 4 == g; plane (i / 4) % 2.  Unit u = 2 block + half starts at value 128 u.
-  const uint32_t xa_base = q6_lds(&xa[0]);
+  const uint32_t xa_base = sm_lds(&xa[0]);
   const uint32_t zero_entry = xa_base + (uint32_t)(CFG::NBMAX * 32 * 16);
   const bool mine = (n & 3) == g;
   const uint32_t plane16 = (uint32_t)(((n >> 2) & 1) * 16);
@@ -247,12 +218,12 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   const uint32_t a2_addr = act2 ? xa_base + 256u * u0 + 128u + 32u * (uint32_t)g + plane16 : zero_entry;
   // per unit 256 bytes of table, per round 16 units
   const uint32_t a1_step = act1 ? 256u : 0u, a2_step = act2 ? 256u : 0u;
-  const uint32_t fac_addr0 = q6_lds(&fac[0]) + 16u * u0 + 4u * (uint32_t)g;
-  const uint32_t wbuf_base = q6_lds(wbuf);
+  const uint32_t fac_addr0 = sm_lds(&fac[0]) + 16u * u0 + 4u * (uint32_t)g;
+  const uint32_t wbuf_base = sm_lds(wbuf);
 
-  q6_barrier();                         // the plane table is complete
+  sm_barrier();                         // the plane table is complete
 
-  const uint32_t part_addr = q6_lds(&part[0][0][0]) + (uint32_t)((wave * 16 + n) * 4);
+  const uint32_t part_addr = sm_lds(&part[0][0][0]) + (uint32_t)((wave * 16 + n) * 4);
   // ODD: the wavefront's blocks sit two bytes into their slots
   auto run_rounds = [&](auto oddc) {
     constexpr bool ODD = decltype(oddc)::value;
@@ -270,7 +241,7 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
     const uint32_t scx_off1 = (g >> 1) ? chunk_at(slot + 13) + 12u : sc_off + 12u;
     const uint32_t d_off = chunk_at(slot + 13) + (uint32_t)(kQ6DAt + (ODD ? 2 : 0));
 
-    struct Regs { q6_u32x4 ql, qh, a1, a2; uint32_t sc, d, f, qlx, qhx, scx; };
+    struct Regs { sm_u32x4 ql, qh, a1, a2; uint32_t sc, d, f, qlx, qhx, scx; };
     // unit hf of the round, round kr of the group
     auto issue = [&](auto hc, uint32_t buf, uint32_t kr, Regs& r) {
       constexpr int hf = decltype(hc)::value;
@@ -374,7 +345,7 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
       else if (later == 2) wait_rounds(I2{});
       else if (later == 1) wait_rounds(I1{});
       else wait_rounds(I0{});
-      q6_barrier();
+      sm_barrier();
       const uint32_t buf = wbuf_base + (uint32_t)(bufi * kQ6BufBytes);
       Regs ra, rb;
       issue(U0{}, buf, (uint32_t)kr, ra);
@@ -383,7 +354,7 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
       compute(ra);
       settle(I0{}, rb);
       // every wavefront has read what it needs of the buffer: a later round may land there
-      q6_barrier();
+      sm_barrier();
       if (rr + kBufs < nrounds) request_next();
       bufi = bufi == kBufs - 1 ? 0 : bufi + 1;
       compute(rb);
@@ -391,7 +362,7 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
         // the group is complete: the four accumulator lanes of a row
         acc += __shfl_xor(acc, 16, kWave);
         acc += __shfl_xor(acc, 32, kWave);
-        if (lane < 16) q6_write_f32(part_addr + (uint32_t)(gi * (kQ6Waves * 16 * 4)), acc);
+        if (lane < 16) sm_write_f32(part_addr + (uint32_t)(gi * (kQ6Waves * 16 * 4)), acc);
         acc = 0.f;
         kr = 0;
         gi++;

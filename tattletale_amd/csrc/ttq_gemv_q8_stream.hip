@@ -21,7 +21,7 @@
 // waits for its own requests on its own counter, a barrier makes the buffer whole, a second one frees it.
 // Chunk c of row n lands at position 136 n + (c ^ (n / 2)): with the rows 8 chunks apart modulo 16, the 16 rows
 // of an operand read hit 16 different bank groups.  Wavefront w multiplies MFMAs w, w + 8, ... of the round's 34.
-#include "ttq_gemv_mfma_common.h"
+#include "ttq_stream_common.h"
 
 namespace ttq {
 
@@ -42,35 +42,12 @@ constexpr int kQ8MaxRounds = 4;                            // rounds per row: n_
 constexpr int kQ8MaxGroups = 32;                           // row groups of a workgroup; also 16 KiB of staging
 constexpr int kQ8EntriesPerMfma = 16;                      // (k-group 4) x (block slot 2) x (plane 2), 16 bytes each
 
-typedef const __attribute__((address_space(1))) void* q8_gptr_t;
-typedef __attribute__((address_space(3))) void* q8_lptr_t;
-typedef uint32_t q8_u32x4 __attribute__((ext_vector_type(4)));
-
-template <int N>
-__device__ __forceinline__ void q8_wait_vmcnt() {
-  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-  asm volatile("" ::: "memory");
-}
-// a barrier that leaves the outstanding requests alone
-__device__ __forceinline__ void q8_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-__device__ __forceinline__ uint32_t q8_lds(const void* p) { return (uint32_t)(size_t)(q8_lptr_t)(p); }
-// LDS accesses the compiler must not see: it cannot tell them from the asynchronous writes of the requests in
-// flight and would wait for every one of those first
-__device__ __forceinline__ q8_u32x4 q8_read16(uint32_t a) {
-  q8_u32x4 v;
-  asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(a) : "memory");
-  return v;
-}
-__device__ __forceinline__ void q8_write_f32(uint32_t a, float v) {
-  asm volatile("ds_write_b32 %0, %1" ::"v"(a), "v"(v) : "memory");
-}
-
 // eight activations of thread-owned positions k0 .. k0 + 7 from the staging area
 template <typename XT> struct Q8Stage;
 template <> struct Q8Stage<float> {
   static constexpr int kBytes = 32, kRequests = 2;
   static __device__ __forceinline__ void read(uint32_t a, uint32_t second, float (&f)[8]) {
-    const q8_u32x4 r0 = q8_read16(a), r1 = q8_read16(a + second);
+    const sm_u32x4 r0 = sm_read16(a), r1 = sm_read16(a + second);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       f[i] = __uint_as_float(r0[i]);
@@ -81,7 +58,7 @@ template <> struct Q8Stage<float> {
 template <typename XT> struct Q8Stage {
   static constexpr int kBytes = 16, kRequests = 1;
   static __device__ __forceinline__ void read(uint32_t a, uint32_t, float (&f)[8]) {
-    const q8_u32x4 r = q8_read16(a);
+    const sm_u32x4 r = sm_read16(a);
     widen8<XT>(make_uint4(r[0], r[1], r[2], r[3]), f);
   }
 };
@@ -126,8 +103,8 @@ gemv_q8_stream_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, Y
       const uint8_t* src = reinterpret_cast<const uint8_t*>(xm + k0);
 #pragma unroll
       for (int r = 0; r < ST::kRequests; r++)
-        __builtin_amdgcn_global_load_lds((q8_gptr_t)(src + 16 * r),
-                                         (q8_lptr_t)(xstage + i * kPassBytes + r * (16 * kQ8Threads) + wave * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((sm_gptr_t)(src + 16 * r),
+                                         (sm_lptr_t)(xstage + i * kPassBytes + r * (16 * kQ8Threads) + wave * 1024), 16, 0, 0);
     }
   }
   // a compute unit serves its requests in the order they were made: every wavefront's activation requests are
@@ -151,10 +128,10 @@ gemv_q8_stream_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, Y
     uint8_t* dst = wbuf + req_buf * kQ8BufBytes + wave * 1024;
 #pragma unroll
     for (int i = 0; i < kQ8ReqMax - 1; i++)
-      __builtin_amdgcn_global_load_lds((q8_gptr_t)(src + src_off[i]), (q8_lptr_t)(dst + i * (kQ8Waves * 1024)), 16, 0, 2);
+      __builtin_amdgcn_global_load_lds((sm_gptr_t)(src + src_off[i]), (sm_lptr_t)(dst + i * (kQ8Waves * 1024)), 16, 0, 2);
     if (full)
-      __builtin_amdgcn_global_load_lds((q8_gptr_t)(src + src_off[kQ8ReqMax - 1]),
-                                       (q8_lptr_t)(dst + (kQ8ReqMax - 1) * (kQ8Waves * 1024)), 16, 0, 2);
+      __builtin_amdgcn_global_load_lds((sm_gptr_t)(src + src_off[kQ8ReqMax - 1]),
+                                       (sm_lptr_t)(dst + (kQ8ReqMax - 1) * (kQ8Waves * 1024)), 16, 0, 2);
     req_buf = req_buf == kQ8Bufs - 1 ? 0 : req_buf + 1;
     req_kr++;
     req_src += kQ8RoundBytes;
@@ -166,15 +143,15 @@ gemv_q8_stream_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, Y
   // all but the youngest `rounds_after` rounds of requests of this wavefront have landed
   auto wait_rounds = [&](int rounds_after) {
     if (full) {
-      if (rounds_after >= 3) q8_wait_vmcnt<3 * kQ8ReqMax>();
-      else if (rounds_after == 2) q8_wait_vmcnt<2 * kQ8ReqMax>();
-      else if (rounds_after == 1) q8_wait_vmcnt<kQ8ReqMax>();
-      else q8_wait_vmcnt<0>();
+      if (rounds_after >= 3) sm_wait_vmcnt<3 * kQ8ReqMax>();
+      else if (rounds_after == 2) sm_wait_vmcnt<2 * kQ8ReqMax>();
+      else if (rounds_after == 1) sm_wait_vmcnt<kQ8ReqMax>();
+      else sm_wait_vmcnt<0>();
     } else {
-      if (rounds_after >= 3) q8_wait_vmcnt<3 * (kQ8ReqMax - 1)>();
-      else if (rounds_after == 2) q8_wait_vmcnt<2 * (kQ8ReqMax - 1)>();
-      else if (rounds_after == 1) q8_wait_vmcnt<kQ8ReqMax - 1>();
-      else q8_wait_vmcnt<0>();
+      if (rounds_after >= 3) sm_wait_vmcnt<3 * (kQ8ReqMax - 1)>();
+      else if (rounds_after == 2) sm_wait_vmcnt<2 * (kQ8ReqMax - 1)>();
+      else if (rounds_after == 1) sm_wait_vmcnt<kQ8ReqMax - 1>();
+      else sm_wait_vmcnt<0>();
     }
   };
   const int npre = min(nrounds, kQ8Bufs);
@@ -186,7 +163,7 @@ gemv_q8_stream_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, Y
     const int entries = rpg * (kQ8RoundMfma * kQ8EntriesPerMfma) + 1;
     for (int i = tid; i < entries; i += kQ8Threads) z[i] = make_uint4(0u, 0u, 0u, 0u);
   }
-  q8_barrier();
+  sm_barrier();
   // ---- the raw activations back into registers, then byte by byte into the operand table: weight e of block b
   // sits at byte 34 b + 2 + e of the row = byte P % 16 of chunk P / 16; MFMA = chunk / 4, k-group = chunk % 4,
   // and the block is the first (0) or second (1) one that has bytes in this chunk
@@ -198,7 +175,7 @@ gemv_q8_stream_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, Y
       const int k0 = 8 * tid + i * (8 * kQ8Threads);
       if (k0 >= n_in) break;
       float xf[8];
-      ST::read(q8_lds(xstage) + (uint32_t)(i * kPassBytes + tid * 16), 16u * kQ8Threads, xf);
+      ST::read(sm_lds(xstage) + (uint32_t)(i * kPassBytes + tid * 16), 16u * kQ8Threads, xf);
       float amax = 0.f;
 #pragma unroll
       for (int j = 0; j < 8; j++) amax = fmaxf(amax, fabsf(xf[j]));
@@ -232,7 +209,7 @@ gemv_q8_stream_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, Y
   // r / 8 == i % 2; it stands for block j0 + (r % 8) / 2 (j0: the first block with bytes in the MFMA) and plane r % 2.
   const uint32_t key = (uint32_t)(n >> 1);
   const uint32_t row_base = (uint32_t)(n * kQ8RoundBytes);
-  const uint32_t xa_base = q8_lds(&xa[0]);
+  const uint32_t xa_base = sm_lds(&xa[0]);
   constexpr int kPairs = (kQ8ReqMax + 1) / 2;               // two MFMAs share an accumulator
   uint32_t b_off[kQ8ReqMax], a_off[kQ8ReqMax];             // per MFMA of the wavefront: weight and activation operand
   bool a_used[kQ8ReqMax];
@@ -265,12 +242,12 @@ gemv_q8_stream_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, Y
     }
   }
   const uint32_t zero_entry = xa_base + (uint32_t)(rpg * (kQ8RoundMfma * kQ8EntriesPerMfma) * 16);
-  const uint32_t ftab_base = q8_lds(&ftab[0]);
-  const uint32_t wbuf_base = q8_lds(wbuf);
-  const uint32_t part_addr = q8_lds(&part[0][0][0]) + (uint32_t)((wave * 16 + n) * 4);
+  const uint32_t ftab_base = sm_lds(&ftab[0]);
+  const uint32_t wbuf_base = sm_lds(wbuf);
+  const uint32_t part_addr = sm_lds(&part[0][0][0]) + (uint32_t)((wave * 16 + n) * 4);
   const int nmf = full ? kQ8ReqMax : kQ8ReqMax - 1;        // MFMAs of this wavefront per round
 
-  q8_barrier();                         // the operand table is complete
+  sm_barrier();                         // the operand table is complete
   // (from here on the staging area is `part`)
 
   float acc = 0.f;
@@ -278,12 +255,12 @@ gemv_q8_stream_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, Y
   for (int rr = 0; rr < nrounds; rr++) {
     // the round's buffer: own requests landed, then everybody's
     wait_rounds(min(nrounds - 1 - rr, kQ8Bufs - 1));
-    q8_barrier();
+    sm_barrier();
     const uint32_t buf = wbuf_base + (uint32_t)(bufi * kQ8BufBytes);
     const uint32_t xa_round = xa_base + (uint32_t)(kr * (kQ8RoundMfma * kQ8EntriesPerMfma * 16));
     const uint32_t f_round = ftab_base + (uint32_t)(kr * (kQ8RoundBlocks * 4));
     // every operand of the round in one go: at most five MFMAs
-    q8_u32x4 bw[kQ8ReqMax], aw[kQ8ReqMax];
+    sm_u32x4 bw[kQ8ReqMax], aw[kQ8ReqMax];
     uint32_t dd[kPairs][2], ff[kPairs][2];
 #pragma unroll
     for (int i = 0; i < kQ8ReqMax; i++) {
@@ -307,7 +284,7 @@ gemv_q8_stream_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, Y
 #pragma unroll
     for (int p = 0; p < kPairs; p++) asm volatile("" : "+v"(dd[p][0]), "+v"(dd[p][1]), "+v"(ff[p][0]), "+v"(ff[p][1]));
     // every wavefront has read what it needs of the buffer: a later round may land there
-    q8_barrier();
+    sm_barrier();
     if (rr + kQ8Bufs < nrounds) request_next();
     bufi = bufi == kQ8Bufs - 1 ? 0 : bufi + 1;
 #pragma unroll
@@ -334,7 +311,7 @@ gemv_q8_stream_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, Y
       // the group is complete: the four accumulator lanes of a row
       acc += __shfl_xor(acc, 16, kWave);
       acc += __shfl_xor(acc, 32, kWave);
-      if (lane < 16) q8_write_f32(part_addr + (uint32_t)(gi * (kQ8Waves * 16 * 4)), acc);
+      if (lane < 16) sm_write_f32(part_addr + (uint32_t)(gi * (kQ8Waves * 16 * 4)), acc);
       acc = 0.f;
       kr = 0;
       gi++;
