@@ -27,7 +27,8 @@ M = 64 / 512 / 2048, attention-shaped GEMVs) under "extra", a roofline object fo
 for the GEMM, and a CPU baseline timed on this machine's host cores.
 
     python bench.py --only ladder     the roofline ladder of the headline kernel (see csrc/ttq_ladder.hip);
-                                      --only ladder_14336x4096 runs one shape (for a kernel trace)
+                                      --only ladder_14336x4096 runs one shape (for a kernel trace);
+                                      --only ladder_q6k the stages of the Q6_K streamed GEMV
 """
 from __future__ import annotations
 
@@ -599,6 +600,55 @@ def main() -> int:
             torch.cuda.empty_cache()
         return out
 
+    def run_ladder_q6k(steps: int, warmup: int, shapes=((128256, 4096), (4096, 14336))):
+        """The stages of the Q6_K streamed GEMV (tattletale_amd/csrc/ttq_gemv_q6k_stream.h): its requests, waits and
+        barriers alone; with the operand reads from LDS; the GEMV -- on the LM-head shape (two workgroups per
+        compute unit) and on a down projection (one workgroup, three buffers)."""
+        lad_path = os.path.join(ROOT, "tattletale_amd", "libttq_ladder.so")
+        if not os.path.exists(lad_path):
+            raise RuntimeError("%s not found: build it with `python -m tattletale_amd.build`" % lad_path)
+        LAD = C.CDLL(lad_path)
+        LAD.ttq_ladder_q6k_launch.restype = C.c_int
+        LAD.ttq_ladder_q6k_launch.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p]
+        L = _lib.lib()
+        rng = np.random.default_rng(98)
+        names = {2: "requests, waits and barriers", 1: "+ operand reads from LDS", 0: "GEMV (ttq_gemv_q6_k)"}
+        out = {}
+        for n_out, n_in in shapes:
+            st = steps if n_out < 100000 else max(20, steps // 4)
+            packed = random_packed(rng, F.Q6_K, n_out, n_in)
+            ncopies = rotated(packed.nbytes)
+            ws = [to_dev(packed) for _ in range(ncopies)]
+            x = torch.randn((1, n_in), device=dev).to(torch.bfloat16)
+            y = torch.empty((1, n_out), dtype=torch.float32, device=dev)
+            rows = []
+            for stage in (2, 1, 0):
+                if stage:
+                    def step(i, stage=stage):
+                        rc = LAD.ttq_ladder_q6k_launch(stage, ws[i % ncopies].data_ptr(), x.data_ptr(), y.data_ptr(), n_out,
+                                                       n_in, torch.cuda.current_stream(dev).cuda_stream)
+                        if rc != 0:
+                            raise RuntimeError("ttq_ladder_q6k_launch(%d) returned %d" % (stage, rc))
+                else:
+                    def step(i):
+                        _lib.check(L.ttq_gemv_q6_k(ws[i % ncopies].data_ptr(), x.data_ptr(), F.BF16, y.data_ptr(), 1,
+                                                   n_out, n_in, torch.cuda.current_stream(dev).cuda_stream),
+                                   "ttq_gemv_q6_k")
+                t = time_steps(step, st, warmup)
+                gbps = packed.nbytes / (t["ms"] * 1e-3) / 1e9
+                rows.append({"stage": names[stage], "us_per_launch": t["ms"] * 1e3, "us_min": t["ms_min"] * 1e3,
+                             "us_max": t["ms_max"] * 1e3, "weight_GBps": gbps, "hbm_frac": gbps / HBM_PEAK_GBPS})
+                log("[q6k stages %dx%d] %-32s %8.3f us  %.0f GB/s (%.3f of peak)"
+                    % (n_out, n_in, names[stage], t["ms"] * 1e3, gbps, gbps / HBM_PEAK_GBPS))
+            out["%dx%d" % (n_out, n_in)] = {"weight_bytes": int(packed.nbytes), "weight_copies": ncopies,
+                                           "steps": st, "stages": rows}
+            del ws
+            torch.cuda.empty_cache()
+        return out
+
+    if args.only == "ladder_q6k":
+        print(json.dumps(run_ladder_q6k(args.steps, args.warmup)), flush=True)
+        return 0
     if args.only == "ladder":
         print(json.dumps(run_ladder(args.steps, args.warmup)), flush=True)
         return 0

@@ -12,7 +12,12 @@
 //   rung 3  the GEMV without its arithmetic: request schedule, waits, operand reads from LDS and the
 //           activation prologue stay
 //   (rung 4, the GEMV itself, is ttq_gemv_q4_k of the product library)
+//
+// The Q6_K streamed GEMV (ttq_gemv_q6k_stream.h) has its stages built in: ttq_ladder_q6k_launch runs it without
+// the arithmetic on the operands (stage 1) or without the operand reads as well (stage 2: requests, waits and
+// barriers); the GEMV itself is ttq_gemv_q6_k of the product library.
 #include "ttq_gemv_q4k_stream.h"
+#include "ttq_gemv_q6k_stream.h"
 
 namespace ttq {
 
@@ -88,4 +93,14 @@ int ttq_ladder_launch(int rung, const void* w, const void* x_bf16, float* y, int
   if (rung == 1) hipLaunchKernelGGL((ladder_kernel<true, false>), grid, block, 0, s, wb, y, (int)n_out, (int)(n_in / 256), rows_per_wg);
   if (rung == 2) hipLaunchKernelGGL((ladder_kernel<true, true>), grid, block, 0, s, wb, y, (int)n_out, (int)(n_in / 256), rows_per_wg);
   return hipGetLastError() == hipSuccess ? 0 : -7;
+}
+
+extern "C" __attribute__((visibility("default")))
+int ttq_ladder_q6k_launch(int stage, const void* w, const void* x_bf16, float* y, int64_t n_out, int64_t n_in, void* stream) {
+  using namespace ttq;
+  if (!w || !x_bf16 || !y || stage < 1 || stage > 2 || !q6_plan(n_out, n_in).ok) return -1;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const hipError_t e = stage == 1 ? q6_launch_xy<bf16_tag, float, 1>(w, x_bf16, y, nullptr, 0, 1, n_out, n_in, s)
+                                  : q6_launch_xy<bf16_tag, float, 2>(w, x_bf16, y, nullptr, 0, 1, n_out, n_in, s);
+  return e == hipSuccess ? 0 : -7;
 }
