@@ -92,7 +92,7 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   const int bx = blockIdx.x;
   const int grp0 = bx * groups_per_wg + min(bx, groups_rem);
   const int ng = groups_per_wg + (bx < groups_rem ? 1 : 0);            // 1 .. CFG::MAXG
-  const int nrounds = rpg * ng;                                          // >= kBufs (the launcher sees to it)
+  const int nrounds = rpg * ng;
 
   // ---- the activations, as LDS requests too (a register load among the weight requests would make the
   // compiler wait for all of them at its first use): thread t stages x[8 t + 4096 i .. + 7]
@@ -152,11 +152,13 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   using I1 = std::integral_constant<int, 1>;
   using I2 = std::integral_constant<int, 2>;
   using I3 = std::integral_constant<int, 3>;
-#pragma unroll
-  for (int i = 0; i < kBufs; i++) request_next();
+  // One round is requested now, the others once the plane table is built: a compute unit takes about 64 KiB of
+  // outstanding requests, and a wavefront that asks for more sits in the request until earlier ones have landed --
+  // with the activations still unprocessed behind it.
+  if (nrounds > 0) request_next();      // (the launcher gives every workgroup a group; a request past the weights must never go out)
 
   // ---- the raw activations back into registers, then into the two byte planes
-  wait_rounds(std::integral_constant<int, kBufs>{});
+  wait_rounds(I1{});
   if (tid < 4) reinterpret_cast<uint32_t*>(&xa[CFG::NBMAX * 32])[tid] = 0u;
 #pragma unroll
   for (int i = 0; i < kXPasses; i++) {
@@ -222,6 +224,9 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   const uint32_t wbuf_base = sm_lds(wbuf);
 
   sm_barrier();                         // the plane table is complete
+#pragma unroll
+  for (int i = 1; i < kBufs; i++)
+    if (i < nrounds) request_next();
 
   const uint32_t part_addr = sm_lds(&part[0][0][0]) + (uint32_t)((wave * 16 + n) * 4);
   // ODD: the wavefront's blocks sit two bytes into their slots
@@ -394,6 +399,9 @@ inline Q6Plan q6_plan(int64_t n_out, int64_t n_in) {
   const int64_t groups = n_out / 16;
   const int cus = device_num_cus();
   if (groups < cus) return p;                              // a group or more for every compute unit
+  // between one and two groups per compute unit the uneven ones decide (6144x4096: 7.9 us against 7.7 of the
+  // packed-dot kernel, which deals rows out more finely)
+  if (groups < 2 * cus && groups % cus != 0) return p;
   int maxg;
   if (nb == Q6Head::NBMAX && groups >= 2 * (int64_t)Q6Head::WGS * cus) {
     // two workgroups per compute unit when each still gets two groups: their rounds interleave
@@ -403,7 +411,6 @@ inline Q6Plan q6_plan(int64_t n_out, int64_t n_in) {
   } else {
     p.num_wg = cus;
     maxg = Q6Wide::MAXG;
-    if ((groups / cus) * (nb / kQ6RoundBlocks) < Q6Wide::BUFS) return p;   // every buffer is requested up front
   }
   if ((groups + p.num_wg - 1) / p.num_wg > maxg) p.num_wg = (int)((groups + maxg - 1) / maxg);
   p.ok = true;

@@ -71,8 +71,9 @@ gemv_q8_stream_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, Y
                       const void* __restrict__ bias, int bias_dtype, int n_out, int rpg, int groups_per_wg,
                       int groups_rem) {
   __shared__ __attribute__((aligned(1024))) uint8_t wbuf[kQ8Bufs * kQ8BufBytes];
-  // the activation operand: per MFMA of the row 16 entries of 16 bytes, and one entry of zeros
-  __shared__ __attribute__((aligned(16))) v4i_t xa[kQ8MaxRounds * kQ8RoundMfma * kQ8EntriesPerMfma + 1];
+  // the activation operand: per MFMA of the row 16 entries of 16 bytes; then 64 entries of zeros, one per lane
+  // (lanes that all read one and the same entry are served one after the other: 1 us per launch)
+  __shared__ __attribute__((aligned(16))) v4i_t xa[kQ8MaxRounds * kQ8RoundMfma * kQ8EntriesPerMfma + 64];
   __shared__ float ftab[kQ8MaxRounds * kQ8RoundBlocks];    // per block: the scale of its fixed-point activations
   // (the raw activations land here first: the partial sums are written after they have been read back)
   __shared__ __attribute__((aligned(1024))) float part[kQ8MaxGroups][kQ8Waves][16];
@@ -154,55 +155,18 @@ gemv_q8_stream_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, Y
       else sm_wait_vmcnt<0>();
     }
   };
+  // One round is requested now, the others once the operand table is built: a compute unit takes about 64 KiB
+  // of outstanding requests, and a wavefront that asks for more sits in the request until earlier ones have
+  // landed -- with the activations still unprocessed behind it.
   const int npre = min(nrounds, kQ8Bufs);
-  for (int i = 0; i < npre; i++) request_next();
+  if (nrounds > 0) request_next();      // (the launcher gives every workgroup a group; a request past the weights must never go out)
 
   // ---- the operand table starts as zeros (scale bytes, other blocks' bytes, rows nobody uses)
   {
     uint4* z = reinterpret_cast<uint4*>(&xa[0]);
-    const int entries = rpg * (kQ8RoundMfma * kQ8EntriesPerMfma) + 1;
+    const int entries = rpg * (kQ8RoundMfma * kQ8EntriesPerMfma) + 64;
     for (int i = tid; i < entries; i += kQ8Threads) z[i] = make_uint4(0u, 0u, 0u, 0u);
   }
-  sm_barrier();
-  // ---- the raw activations back into registers, then byte by byte into the operand table: weight e of block b
-  // sits at byte 34 b + 2 + e of the row = byte P % 16 of chunk P / 16; MFMA = chunk / 4, k-group = chunk % 4,
-  // and the block is the first (0) or second (1) one that has bytes in this chunk
-  wait_rounds(npre);
-  {
-    uint8_t* xab = reinterpret_cast<uint8_t*>(&xa[0]);
-#pragma unroll
-    for (int i = 0; i < kXPasses; i++) {
-      const int k0 = 8 * tid + i * (8 * kQ8Threads);
-      if (k0 >= n_in) break;
-      float xf[8];
-      ST::read(sm_lds(xstage) + (uint32_t)(i * kPassBytes + tid * 16), 16u * kQ8Threads, xf);
-      float amax = 0.f;
-#pragma unroll
-      for (int j = 0; j < 8; j++) amax = fmaxf(amax, fabsf(xf[j]));
-      // the four threads of a block are an aligned quad
-      amax = fmaxf(amax, dpp_quad<0xB1>(amax));
-      amax = fmaxf(amax, dpp_quad<0x4E>(amax));
-      const uint32_t eb = __float_as_uint(amax) >> 23;       // biased exponent (amax >= 0)
-      const uint32_t ec = eb < 18u ? 18u : eb;
-      const float mul = __uint_as_float((267u - ec) << 23);  // 2^(13-E)
-      // non-finite activations poison their block instead of being clipped
-      const float f = eb == 255u ? __uint_as_float(0x7FC00000u) : __uint_as_float((ec - 13u) << 23);
-      const int b = k0 >> 5;
-      if ((tid & 3) == 0) ftab[b] = f;
-#pragma unroll
-      for (int j = 0; j < 8; j++) {
-        const int v = (int)rintf(xf[j] * mul);
-        const int hi = (v + 128) >> 8;                       // v = 256 hi + (signed low byte)
-        const int P = 34 * b + 2 + (k0 & 31) + j;
-        const int c = P >> 4;
-        const int first = (16 * c) / 34;                     // first block with bytes in this chunk
-        const int entry = c * 4 + (b - first) * 2;           // (MFMA, k-group) = chunk; then block slot, plane
-        xab[entry * 16 + (P & 15)] = (uint8_t)hi;
-        xab[(entry + 1) * 16 + (P & 15)] = (uint8_t)v;
-      }
-    }
-  }
-
   // ---- per-lane constants of the main loop.  MFMA t2 of a round (0..33) covers bytes 64 t2 .. 64 t2 + 63 of the
   // round's 2176; the wavefront takes t2 = wave + 8 i.  Operand lane (r, g): weight row n = r, k-group g (weights)
   // or selector row r, k-group g (activations).  Selector row r of the i-th MFMA of a wavefront is used if
@@ -241,41 +205,91 @@ gemv_q8_stream_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, Y
       f_off[p][e] = (uint32_t)(4 * jb);
     }
   }
-  const uint32_t zero_entry = xa_base + (uint32_t)(rpg * (kQ8RoundMfma * kQ8EntriesPerMfma) * 16);
+  const uint32_t zero_entry = xa_base + (uint32_t)((rpg * (kQ8RoundMfma * kQ8EntriesPerMfma) + lane) * 16);
   const uint32_t ftab_base = sm_lds(&ftab[0]);
   const uint32_t wbuf_base = sm_lds(wbuf);
   const uint32_t part_addr = sm_lds(&part[0][0][0]) + (uint32_t)((wave * 16 + n) * 4);
   const int nmf = full ? kQ8ReqMax : kQ8ReqMax - 1;        // MFMAs of this wavefront per round
 
+  // ---- the raw activations back into registers (they were requested before any weight, and the lane constants
+  // above were computed while they were on their way), then byte by byte into the operand table: weight e of
+  // block b sits at byte 34 b + 2 + e of the row = byte P % 16 of chunk P / 16; MFMA = chunk / 4, k-group =
+  // chunk % 4, and the block is the first (0) or second (1) one that has bytes in this chunk
+  sm_barrier();                         // the table is all zeros
+  wait_rounds(1);
+  {
+    uint8_t* xab = reinterpret_cast<uint8_t*>(&xa[0]);
+#pragma unroll
+    for (int i = 0; i < kXPasses; i++) {
+      const int k0 = 8 * tid + i * (8 * kQ8Threads);
+      if (k0 >= n_in) break;
+      float xf[8];
+      ST::read(sm_lds(xstage) + (uint32_t)(i * kPassBytes + tid * 16), 16u * kQ8Threads, xf);
+      float amax = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; j++) amax = fmaxf(amax, fabsf(xf[j]));
+      // the four threads of a block are an aligned quad
+      amax = fmaxf(amax, dpp_quad<0xB1>(amax));
+      amax = fmaxf(amax, dpp_quad<0x4E>(amax));
+      const uint32_t eb = __float_as_uint(amax) >> 23;       // biased exponent (amax >= 0)
+      const uint32_t ec = eb < 18u ? 18u : eb;
+      const float mul = __uint_as_float((267u - ec) << 23);  // 2^(13-E)
+      // non-finite activations poison their block instead of being clipped
+      const float f = eb == 255u ? __uint_as_float(0x7FC00000u) : __uint_as_float((ec - 13u) << 23);
+      const int b = k0 >> 5;
+      if ((tid & 3) == 0) ftab[b] = f;
+      // the thread's eight bytes start at byte P0 of the row and lie in chunk c0 or the one after it
+      const int P0 = 34 * b + 2 + (k0 & 31), c0 = P0 >> 4, e0 = P0 & 15;
+      const int base0 = ((c0 * 4 + (b - (16 * c0) / 34) * 2) * 16) + e0;
+      const int base1 = (((c0 + 1) * 4 + (b - (16 * (c0 + 1)) / 34) * 2) * 16) + e0 - 16;
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const int v = (int)rintf(xf[j] * mul);
+        const int hi = (v + 128) >> 8;                       // v = 256 hi + (signed low byte)
+        const int at = (e0 + j < 16 ? base0 : base1) + j;
+        xab[at] = (uint8_t)hi;
+        xab[at + 16] = (uint8_t)v;
+      }
+    }
+  }
+
+
   sm_barrier();                         // the operand table is complete
+  for (int i = 1; i < npre; i++) request_next();
   // (from here on the staging area is `part`)
 
   float acc = 0.f;
   int bufi = 0, kr = 0, gi = 0;
   for (int rr = 0; rr < nrounds; rr++) {
-    // the round's buffer: own requests landed, then everybody's
-    wait_rounds(min(nrounds - 1 - rr, kQ8Bufs - 1));
-    sm_barrier();
     const uint32_t buf = wbuf_base + (uint32_t)(bufi * kQ8BufBytes);
     const uint32_t xa_round = xa_base + (uint32_t)(kr * (kQ8RoundMfma * kQ8EntriesPerMfma * 16));
     const uint32_t f_round = ftab_base + (uint32_t)(kr * (kQ8RoundBlocks * 4));
-    // every operand of the round in one go: at most five MFMAs
+    // every operand of the round in one go, at most five MFMAs.  What does not depend on the landed bytes -- the
+    // activation operands and scales -- is asked for first, before the wait for the buffer
     sm_u32x4 bw[kQ8ReqMax], aw[kQ8ReqMax];
     uint32_t dd[kPairs][2], ff[kPairs][2];
 #pragma unroll
     for (int i = 0; i < kQ8ReqMax; i++) {
-      const uint32_t ab = buf + b_off[i];
       const uint32_t aa = a_used[i] ? xa_round + a_off[i] : zero_entry;
-      asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %3" : "=&v"(bw[i]), "=&v"(aw[i]) : "v"(ab), "v"(aa) : "memory");
+      asm volatile("ds_read_b128 %0, %1" : "=&v"(aw[i]) : "v"(aa) : "memory");
+    }
+#pragma unroll
+    for (int p = 0; p < kPairs; p++) {
+      const uint32_t fa0 = f_round + f_off[p][0], fa1 = f_round + f_off[p][1];
+      asm volatile("ds_read_b32 %0, %2\n\tds_read_b32 %1, %3" : "=&v"(ff[p][0]), "=&v"(ff[p][1]) : "v"(fa0), "v"(fa1) : "memory");
+    }
+    // the round's buffer: own requests landed, then everybody's
+    wait_rounds(min(nrounds - 1 - rr, kQ8Bufs - 1));
+    sm_barrier();
+#pragma unroll
+    for (int i = 0; i < kQ8ReqMax; i++) {
+      const uint32_t ab = buf + b_off[i];
+      asm volatile("ds_read_b128 %0, %1" : "=&v"(bw[i]) : "v"(ab) : "memory");
     }
 #pragma unroll
     for (int p = 0; p < kPairs; p++) {
       const uint32_t da0 = buf + d_off[p][0], da1 = buf + d_off[p][1];
-      const uint32_t fa0 = f_round + f_off[p][0], fa1 = f_round + f_off[p][1];
-      asm volatile("ds_read_u16 %0, %4\n\tds_read_u16 %1, %5\n\tds_read_b32 %2, %6\n\tds_read_b32 %3, %7"
-                   : "=&v"(dd[p][0]), "=&v"(dd[p][1]), "=&v"(ff[p][0]), "=&v"(ff[p][1])
-                   : "v"(da0), "v"(da1), "v"(fa0), "v"(fa1)
-                   : "memory");
+      asm volatile("ds_read_u16 %0, %2\n\tds_read_u16 %1, %3" : "=&v"(dd[p][0]), "=&v"(dd[p][1]) : "v"(da0), "v"(da1) : "memory");
     }
     // all of them have arrived (the asm statements tie every register to the wait)
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -333,14 +347,13 @@ gemv_q8_stream_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, Y
 int q8_plan(int x_dtype, int64_t n_out, int64_t n_in) {
   // whole rounds of 2048 weights, whole groups of 16 rows, tables and staging within LDS, 32-bit byte offsets
   if (n_in % 2048 != 0 || n_in > 2048 * kQ8MaxRounds || n_out % 16 != 0) return 0;
-  if (x_dtype == kF32 && n_in > 4096) return 0;
+  // fp32 activations keep the kernels whose activation planes carry 22 bits (two planes carry 15: 5e-5 on
+  // activations of uneven magnitude, where those deliver 1e-6)
+  if (x_dtype == kF32) return 0;
   if (n_out * (n_in / 32) * 34 >= ((int64_t)1 << 32)) return 0;
   const int64_t groups = n_out / 16;
   const int cus = device_num_cus();
-  // At least six rounds for every compute unit: below that the set-up of the operand table and the two barriers
-  // per round are not paid for (4096x4096, two rounds: 6.8 us against 6.5 of the aligned-window kernel;
-  // 6144x4096: 9.0 against 8.4; 14336x4096, seven rounds: 13.9 against 15.1).
-  if ((groups / cus) * (n_in / 2048) < 6) return 0;
+  if (groups < cus) return 0;                              // a group or more for every workgroup
   int num_wg = cus;
   if ((groups + num_wg - 1) / num_wg > kQ8MaxGroups) num_wg = (int)((groups + kQ8MaxGroups - 1) / kQ8MaxGroups);
   return num_wg;

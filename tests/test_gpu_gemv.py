@@ -426,8 +426,8 @@ def test_q6_k_streamed_activation_extremes_bias_and_output_types():
 
 
 @pytest.mark.parametrize("xk", ["bf16", "f16"])
-@pytest.mark.parametrize("n_out,n_in", [(4096, 14336), (8192, 4096), (4096 + 16 * 5, 8192), (12288 + 48, 2048),
-                                        (4096 + 16, 6144), (4096, 12288)])
+@pytest.mark.parametrize("n_out,n_in", [(4096, 14336), (8192, 4096), (8192 + 16 * 5, 8192), (12288 + 48, 2048),
+                                        (8192 + 16, 6144), (4096, 12288), (4096, 4096), (4096, 2048)])
 def test_q6_k_streamed_other_row_lengths(xk, n_out, n_in):
     """Rows of 2048 to 14336 values (one to seven rounds of eight blocks per group of 16 rows), one workgroup
     per compute unit: normal activations against the float64 product, and unit vectors -- in the first and the
@@ -450,10 +450,11 @@ def test_q6_k_streamed_other_row_lengths(xk, n_out, n_in):
 
 
 # ------------------------------------------------------------------- Q8_0, LDS-streamed kernel
-# (rows of 2048 .. 8192 values -- 4096 at most for fp32 activations --, whole groups of 16 rows, at least six
-# rounds of 2048 weights x 16 rows per compute unit; a single activation row)
+# (rows of 2048 .. 8192 values -- 4096 at most for fp32 activations --, whole groups of 16 rows, at least one
+# group per compute unit; a single activation row)
 @pytest.mark.parametrize("xk", ["f32", "bf16", "f16"])
-@pytest.mark.parametrize("n_out,n_in", [(12288 + 16 * 5, 4096), (24576 + 16 * 3, 2048), (8192 + 16, 8192), (8192 + 16 * 7, 6144)])
+@pytest.mark.parametrize("n_out,n_in", [(12288 + 16 * 5, 4096), (24576 + 16 * 3, 2048), (8192 + 16, 8192), (8192 + 16 * 7, 6144),
+                                        (4096, 4096), (4096 + 16 * 37, 2048), (4096 + 16, 6144)])
 def test_q8_0_streamed_unit_vectors_and_random_activations(xk, n_out, n_in):
     """Random block bytes (every weight value, negative and tiny scales).  Unit vectors, also scaled by a power
     of two, reproduce the canonical column bit for bit: first and last weights of even and odd blocks, weights
@@ -483,10 +484,10 @@ def test_q8_0_streamed_unit_vectors_and_random_activations(xk, n_out, n_in):
 @pytest.mark.parametrize("extra_groups", [0, 1, 255, 300, 1000])
 def test_q8_0_streamed_group_counts(extra_groups):
     """Quantized normal weights; group counts that divide evenly among the compute units and ones that do not,
-    three to seven groups per workgroup."""
+    one to five groups per workgroup."""
     n_in = 4096
     cus = torch.cuda.get_device_properties(0).multi_processor_count
-    n_out = 16 * (3 * cus + extra_groups)
+    n_out = 16 * (cus + extra_groups)
     p, what = make(F.Q8_0, n_out, n_in, 400 + extra_groups)
     xd, xf = x_to_dev(Q.fill_normal(401, 1, 1.0, n_in), "bf16")
     y = QL.gemv(F.Q8_0, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()[0]
