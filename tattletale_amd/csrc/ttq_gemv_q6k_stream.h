@@ -122,7 +122,9 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   }
   const bool full = wave < kQ6FullWaves;
   // rounds are requested in order: group by group, eight blocks by eight blocks
-  uint32_t req_src = (uint32_t)grp0 * 16u * row_bytes;    // byte offset of the next round to request
+  // (every workgroup has a group; a workgroup without one would ask for the matrix's last group: never past the end,
+  // and without a branch around the request, after which the compiler waits for every request in flight)
+  uint32_t req_src = (uint32_t)min(grp0, n_out / 16 - 1) * 16u * row_bytes;    // byte offset of the next round to request
   int req_kr = 0, req_buf = 0;
   auto request_next = [&]() {
     const uint8_t* src = w + (size_t)req_src;
@@ -155,7 +157,7 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   // One round is requested now, the others once the plane table is built: a compute unit takes about 64 KiB of
   // outstanding requests, and a wavefront that asks for more sits in the request until earlier ones have landed --
   // with the activations still unprocessed behind it.
-  if (nrounds > 0) request_next();      // (the launcher gives every workgroup a group; a request past the weights must never go out)
+  request_next();
 
   // ---- the raw activations back into registers, then into the two byte planes
   wait_rounds(I1{});
