@@ -337,6 +337,8 @@ hipError_t launch_gemv(int format, const void* w, const void* x, int x_dtype, vo
     return launch_gemv_dot2_multi(format, w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   if (gemv_q4k_stream_supported(format, x_dtype, n_out, n_in))
     return launch_gemv_q4k_stream(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  if (gemv_q4k_slice_supported(format, x_dtype, n_out, n_in))
+    return launch_gemv_q4k_slice(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   if (gemv_q6k_stream_supported(format, x_dtype, n_out, n_in))
     return launch_gemv_q6k_stream(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   if (gemv_mfma_supported(format, x_dtype, n_out, n_in))

@@ -66,6 +66,13 @@ hipError_t launch_gemv_q4k_stream(const void* w, const void* x, int x_dtype, voi
                                   const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                                   hipStream_t s);
 
+// The streamed kernel for long rows (ttq_gemv_q4k_slice.hip): n_in 6144 .. 14336 in steps of 2048, the K
+// dimension dealt to the wavefronts, each with its own activation tables.
+bool gemv_q4k_slice_supported(int format, int x_dtype, int64_t n_out, int64_t n_in);
+hipError_t launch_gemv_q4k_slice(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                                 const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                                 hipStream_t s);
+
 // Q8_0 through the int8 matrix cores with the raw bytes of the rows as the K dimension, streamed through three LDS
 // buffers (ttq_gemv_q8_stream.hip): n_in a multiple of 2048 up to 8192 (4096 for fp32 activations), whole groups of
 // 16 rows, at least one per compute unit.

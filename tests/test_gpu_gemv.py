@@ -449,6 +449,66 @@ def test_q6_k_streamed_other_row_lengths(xk, n_out, n_in):
         assert np.array_equal(y[nz].view(np.uint32), col[nz].view(np.uint32)), c
 
 
+# ------------------------------------------------------------------- Q4_K, long rows (K dealt to the wavefronts)
+# (rows of 6144 .. 14336 values, 16-bit activations, at least 16 rows per compute unit)
+@pytest.mark.parametrize("xk", ["bf16", "f16"])
+@pytest.mark.parametrize("n_out,n_in", [(4096, 14336), (4096 + 24, 14336), (8192 + 16 * 9, 14336), (4096 * 5, 14336),
+                                        (4096, 12288), (4096 + 16, 10240), (8192, 8192), (12288 + 40, 6144)])
+def test_q4_k_long_rows_unit_vectors_and_random_activations(xk, n_out, n_in):
+    """Three to seven slices of 2048 inputs, one to five row groups per workgroup (one or several blocks per
+    wavefront), ragged last groups.  Random block bytes: a unit vector -- in every slice, in even and odd
+    sub-blocks, scaled by a power of two -- reproduces the canonical column bit for bit; normal activations
+    with uneven magnitudes stay within 1e-3 of the float64 product on every row."""
+    p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=71 + n_in // 256)
+    what = oracle.dequant(F.Q4_K, p, n_out, n_in)
+    wd = packed_to_dev(p)
+    x = Q.fill_normal(72, 1, 1.0, n_in).reshape(1, n_in)
+    x[0, ::11] *= 29.0
+    xd, xf = x_to_dev(x, xk)
+    y = QL.gemv(F.Q4_K, wd, xd, n_out, n_in).cpu().numpy()[0]
+    assert rel_l2(y, oracle.linear_f64(what, xf)[0]) <= TOL
+    cols = [0, 31, 32, 255, 256 + 97, 2047] + [2048 * k + o for k in range(1, n_in // 2048) for o in (0, 1000 + 37 * k)]
+    cols += [n_in - 33, n_in - 1]
+    for i, c in enumerate(cols):
+        sc = (1.0, -0.5, 4.0)[i % 3]
+        x = np.zeros((1, n_in), np.float32)
+        x[0, c] = sc
+        xd, _ = x_to_dev(x, xk)
+        y = QL.gemv(F.Q4_K, wd, xd, n_out, n_in).cpu().numpy()[0]
+        col = what[:, c] * np.float32(sc)
+        assert np.array_equal(y, col), c
+        nz = col != 0
+        assert np.array_equal(y[nz].view(np.uint32), col[nz].view(np.uint32)), c
+
+
+def test_q4_k_long_rows_activation_extremes_bias_and_output_types():
+    """Zero activations, one huge value among tiny ones, non-finite values, tiny values; bias and 16-bit
+    outputs through the layer entry point."""
+    n_out, n_in = 4096 + 16, 14336
+    p, what = make(F.Q4_K, n_out, n_in, 81)
+    wd = packed_to_dev(p)
+    x = np.zeros((4, n_in), np.float32)
+    x[1] = Q.fill_normal(82, 1, 1e-3, n_in)
+    x[1, 9000] = 3.0e4
+    x[2] = Q.fill_normal(83, 1, 1.0, n_in)
+    x[2, n_in - 1] = np.inf
+    x[3] = Q.fill_normal(84, 1, 1.0, n_in) * 1e-30
+    xd, xf = x_to_dev(x, "bf16")
+    y = gemv_row_by_row(F.Q4_K, wd, xd, n_out, n_in)
+    want = oracle.linear_f64(what, xf[[0, 1, 3]])
+    assert np.array_equal(y[0], np.zeros(n_out, np.float32))
+    assert rel_l2(y[1], want[1]) <= TOL
+    assert not np.any(np.isfinite(y[2]))
+    assert rel_l2(y[3], want[2]) <= TOL
+    bias = Q.fill_normal(85, 0, 0.5, n_out)
+    xd1, xf1 = x_to_dev(Q.fill_normal(86, 1, 1.0, n_in), "f16")
+    want1 = oracle.linear_f64(what, xf1).reshape(-1) + bias
+    for out_dtype, tol in ((torch.float32, TOL), (torch.bfloat16, 4e-3), (torch.float16, 1e-3)):
+        layer = QuantLinear.init(wd, F.Q4_K, n_in, n_out, bias=torch.from_numpy(bias).to(DEV))
+        yy = layer.forward(xd1, out_dtype=out_dtype).float().cpu().numpy().reshape(-1)
+        assert rel_l2(yy, want1) <= tol, out_dtype
+
+
 # ------------------------------------------------------------------- Q8_0, LDS-streamed kernel
 # (rows of 2048 .. 8192 values -- 4096 at most for fp32 activations --, whole groups of 16 rows, at least one
 # group per compute unit; a single activation row)

@@ -43,10 +43,14 @@ def test_batch_random(xk, m, n_out, n_in):
     want = oracle.linear_f64(what, xf)
     for r in range(m):
         assert rel_l2(y[r][rows], want[r]) <= TOL, r
-    # the single-row kernel on three of the rows
+    # the single-row kernel on three of the rows.  With rows of 6144 .. 14336 values and a row group per
+    # compute unit that is the long-row kernel, which takes the sums of x of the mins term from the fixed-point
+    # values instead of the fp32 activations: both are within the bound above of the exact product, not of
+    # each other to the last bits
+    same = 3e-4 if n_in % 2048 == 0 and 6144 <= n_in <= 14336 and n_out >= 4096 else 2e-6
     for r in {0, m // 2, m - 1}:
         y1 = QL.gemv(F.Q4_K, wd, xd[r:r + 1], n_out, n_in).cpu().numpy()[0]
-        assert rel_l2(y[r], y1) <= 2e-6, r
+        assert rel_l2(y[r], y1) <= same, r
 
 
 @pytest.mark.parametrize("xk", ["bf16", "f16"])
