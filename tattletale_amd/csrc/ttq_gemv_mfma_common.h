@@ -70,6 +70,16 @@ __device__ __forceinline__ uint32_t pack_low_bytes(int a, int b, int c, int d) {
   return p01 | (p23 << 16);
 }
 
+// bytes 1 of a, b, c, d -> one dword (a lowest)
+__device__ __forceinline__ uint32_t pack_bytes1(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+  const uint32_t p01 = __builtin_amdgcn_perm(b, a, 0x0c0c0501u);
+  const uint32_t p23 = __builtin_amdgcn_perm(d, c, 0x0c0c0501u);
+  return p01 | (p23 << 16);
+}
+
+// 1.5 * 2^23: x + this, rounded to fp32, carries rint(x) in its low mantissa bits for |x| < 2^22
+constexpr uint32_t kRoundMagicBits = 0x4B400000u;
+
 // Optional RMSNorm in front of a GEMV: what the kernels that normalize the activation row themselves need.
 struct GemvNormArgs {
   const uint16_t* residual;     // (m, n_in) or null

@@ -29,13 +29,6 @@ constexpr int kSlConstBytes = 512;            // 8 super-blocks x 4 pairs of sub
 constexpr int kSlMaxBlocks = 38;              // (row groups of a workgroup) x (slices): their sums wait in LDS
 constexpr int kSlUpFirst = 4;                 // weight requests made before the activations are quantized
 
-// bytes 1 of a, b, c, d -> one dword (a lowest)
-__device__ __forceinline__ uint32_t pack_bytes1(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
-  const uint32_t p01 = __builtin_amdgcn_perm(b, a, 0x0c0c0501u);
-  const uint32_t p23 = __builtin_amdgcn_perm(d, c, 0x0c0c0501u);
-  return p01 | (p23 << 16);
-}
-
 __device__ __forceinline__ void sl_write16(uint32_t a, st_u32x4 v) {
   asm volatile("ds_write_b128 %0, %1" : : "v"(a), "v"(v) : "memory");
 }
@@ -138,14 +131,13 @@ gemv_q4k_slice_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
       const float f = eb == 255u ? __uint_as_float(0x7FC00000u) : __uint_as_float((ec - 13u) << 23);
       // v = rint(x * 2^(13-E)), |v| <= 2^14, read off the low bits of x * 2^(13-E) + 1.5 * 2^23 (one fused
       // multiply-add rounds to the integer grid, nearest-even like rintf; the product itself is exact)
-      constexpr uint32_t kMagicBits = 0x4B400000u;
       uint32_t vbits[32], vacc = 0u;
 #pragma unroll
       for (int i = 0; i < 32; i++) {
-        vbits[i] = __float_as_uint(fmaf_(xf[i], mul, __uint_as_float(kMagicBits)));
+        vbits[i] = __float_as_uint(fmaf_(xf[i], mul, __uint_as_float(kRoundMagicBits)));
         vacc += vbits[i];
       }
-      const int vsum = (int)(vacc - 32u * kMagicBits);      // modulo 2^32: the sum itself is below 2^19
+      const int vsum = (int)(vacc - 32u * kRoundMagicBits);      // modulo 2^32: the sum itself is below 2^19
       // sum(x) of the sub-block as the fixed-point values give it: the row sum is then exactly the dot
       // product of the dequantized weights with the quantized activations
       const float sum = (float)vsum * f;
