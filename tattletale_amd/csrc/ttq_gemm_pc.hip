@@ -204,6 +204,16 @@ template <> struct WFmt<kQ8_0> {
   }
 };
 
+// Split along K: copies of the tile grid, where the copies of a tile leave their partial sums, and the arrival
+// counters (zero between launches).
+struct PcSplit {
+  int splits;          // 1: none
+  int tile_wgs;        // workgroups of one copy of the tile grid
+  float* partials;
+  uint32_t* counters;
+};
+constexpr int kPcMaxCounters = 16384;     // (tile, consumer) pairs a split launch may have
+
 // W tile in LDS: [ksub 2][j NJ][g 4][n 16] units of 16 bytes (8 consecutive k of one column),
 // i.e. exactly the B operand of lane g*16+n for column block j.
 // FUSE: the weight holds gate rows [0, n_out) followed by up rows [n_out, 2*n_out), as GatedMLP
@@ -217,7 +227,7 @@ template <int NJ, int FMT, int MB, bool FUSE>
 __global__ void __launch_bounds__(kPcThreads)
 gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, void* __restrict__ yv,
                    int y_dtype, const void* __restrict__ bias, int bias_dtype, int m, int n_out, int n_in,
-                   int n_tiles, int m_tiles, int xcds_per_mtile) {
+                   int n_tiles, int m_tiles, int xcds_per_mtile, PcSplit sp) {
   constexpr int BN = NJ * 16;
   constexpr int kWUnits = 2 * NJ * 64;
   constexpr int kPcBM = pc_bm(MB), kXStage = pc_xstage(MB), kXRingBytes = 4 * kXStages * kXStage;
@@ -234,20 +244,26 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
   // Tile assignment.  Workgroups are dealt to the 8 XCDs round-robin (XCD = id % 8) and every XCD
   // has its own L2.  All workgroups of one row tile read the same 256 x n_in slab of X, so when
   // the row tiles divide the XCDs evenly each XCD is given workgroups of ONE row tile only.
+  // Split along K (sp.splits > 1): the grid holds sp.splits copies of the tile grid, copy c works on blocks
+  // [c, c + 1) * nblocks of every row and the copies of a tile add up in the epilogue.
+  const int ksplit = sp.splits > 1 ? (int)blockIdx.x / sp.tile_wgs : 0;
+  const int bid = (int)blockIdx.x - ksplit * sp.tile_wgs;
   int n_tile, m_tile;
   if (xcds_per_mtile > 0) {
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int xcd = bid & 7, slot = bid >> 3;
     m_tile = xcd / xcds_per_mtile;
     n_tile = slot * xcds_per_mtile + xcd % xcds_per_mtile;
   } else {
-    m_tile = blockIdx.x % m_tiles;
-    n_tile = blockIdx.x / m_tiles;
+    m_tile = bid % m_tiles;
+    n_tile = bid / m_tiles;
   }
   if (n_tile >= n_tiles) return;
   constexpr int BO = FUSE ? BN / 2 : BN;     // outputs per tile
   const int n0 = n_tile * BO;
-  const int ksteps = n_in >> 6;
-  const int nblocks = n_in >> 8;
+  const int row_blocks = n_in >> 8;                                  // super-blocks (256 k) in a row of W
+  const int nblocks = sp.splits > 1 ? row_blocks / sp.splits : row_blocks;   // this workgroup's share of them
+  const int block0 = ksplit * nblocks;
+  const int ksteps = nblocks * 4;
 
   // One barrier per 64-k step, numbered s = -1 .. ksteps-1.  Barrier s means: the data of step
   // s+1 is complete in LDS (W buffer (s+1)%2, X stage (s+1)%3) and every LDS read of step s has
@@ -281,12 +297,12 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
     const uint8_t* pf_row =
         xb + (size_t)min(m_tile * kPcBM + pc * (16 * MB) + (lane & (16 * MB - 1)), m - 1) * (size_t)(n_in * 2);
     auto dma_step = [&](int ks, int stage) {
-      const uint32_t koff = (uint32_t)ks * 128u;
+      const uint32_t koff = (uint32_t)(4 * block0 + ks) * 128u;
 #pragma unroll
       for (int i = 0; i < kDma; i++)
         __builtin_amdgcn_global_load_lds((gptr_t)(xb + (size_t)(xoff[i] + koff)),
                                          (lptr_t)(ring + stage * kXStage + i * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((gptr_t)(pf_row + (size_t)min(ks + kPf, ksteps - 1) * 128),
+      __builtin_amdgcn_global_load_lds((gptr_t)(pf_row + (size_t)(4 * block0 + min(ks + kPf, ksteps - 1)) * 128),
                                        (lptr_t)(pf_sink + pc * 64), 4, 0, 0);
     };
     // Requests complete in order, so "all but the youngest N have landed" is the only wait there
@@ -330,7 +346,7 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
                           : min(n0 + wr, n_out - 1);
     using WF = WFmt<FMT>;
     using WRaw = typename WF::Raw;
-    const uint8_t* wptr = w + (int64_t)nblocks * WF::kUnitBytes * (int64_t)wrow;
+    const uint8_t* wptr = w + (int64_t)row_blocks * WF::kUnitBytes * (int64_t)wrow + (int64_t)block0 * WF::kUnitBytes;
     const int wj = wr >> 4, wn = wr & 15;
     const uint32_t sw_addr = (uint32_t)(size_t)(lptr_t)(&sw[0]);
     auto load_w = [&](WRaw& dst, int b) {
@@ -465,6 +481,61 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
     step(std::integral_constant<int, ((3 * G) & 3)>{}, C3{}, C1{});   // after the last step: stale reads, never used
   }
 
+  // ---- split along K: this wavefront's 64 x BN partial sums go to the workspace (whole kilobytes per store
+  // instruction), a counter per (tile, consumer) says how many copies have arrived, and the wavefront that
+  // arrives last adds all copies in copy order -- the same sum whichever arrives last -- and carries on to the
+  // epilogue.  Nobody waits for anybody.  The eight L2 caches of the device are not coherent with each other:
+  // partial sums and counter are written and read as device-scope atomics (relaxed: they go through to the
+  // memory side and come from there), the stores are complete before the count, the loads are issued after
+  // it.  A release / acquire pair would do the same by writing back and invalidating a whole L2, under every
+  // other workgroup still running: 34 -> 88 us on 4096 x 4096 at 512 rows.
+  if constexpr (!FUSE) {
+    if (sp.splits > 1) {
+      constexpr int kPartFloats = MB * NJ * 256;
+      const int unit = (m_tile * n_tiles + n_tile) * 4 + wave;
+      float* all = sp.partials + (size_t)unit * (size_t)(sp.splits * kPartFloats);
+      uint64_t* mine = reinterpret_cast<uint64_t*>(all + ksplit * kPartFloats);
+#pragma unroll
+      for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+          uint64_t lo, hi;
+          const f32x4_t v = acc[i][j];
+          lo = (uint64_t)__float_as_uint(v[0]) | ((uint64_t)__float_as_uint(v[1]) << 32);
+          hi = (uint64_t)__float_as_uint(v[2]) | ((uint64_t)__float_as_uint(v[3]) << 32);
+          uint64_t* q = mine + ((i * NJ + j) * 64 + lane) * 2;
+          __hip_atomic_store(q, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(q + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      uint32_t arrived = 0;
+      if (lane == 0)
+        arrived = __hip_atomic_fetch_add(sp.counters + unit, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      arrived = (uint32_t)__builtin_amdgcn_readfirstlane((int)arrived);
+      if (arrived != (uint32_t)(sp.splits - 1)) return;
+      asm volatile("" ::: "memory");
+      // ready for the next launch on the stream
+      if (lane == 0) __hip_atomic_store(sp.counters + unit, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      // two copies: the other one is added to the registers (a + b = b + a); more: all in copy order
+      const bool two = sp.splits == 2;
+      for (int c = two ? 1 - ksplit : 0; c < (two ? 2 - ksplit : sp.splits); c++) {
+        const uint64_t* other = reinterpret_cast<const uint64_t*>(all + c * kPartFloats);
+#pragma unroll
+        for (int i = 0; i < MB; i++)
+#pragma unroll
+          for (int j = 0; j < NJ; j++) {
+            const uint64_t* q = other + ((i * NJ + j) * 64 + lane) * 2;
+            const uint64_t lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const uint64_t hi = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const f32x4_t v = {__uint_as_float((uint32_t)lo), __uint_as_float((uint32_t)(lo >> 32)),
+                               __uint_as_float((uint32_t)hi), __uint_as_float((uint32_t)(hi >> 32))};
+            if (c == 0 && !two) acc[i][j] = v;
+            else acc[i][j] += v;
+          }
+      }
+    }
+  }
+
   // ---- epilogue: lane holds Y[m0 + 16i + 4*(lane/16) + r][n0 + 16j + lane%16], r = 0..3
   const int cn = lane & 15, rb4 = (lane >> 4) * 4;
   if constexpr (FUSE) {
@@ -580,7 +651,7 @@ gemm_pc_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, vo
 
 template <int FMT, int MB, int NJ, bool FUSE>
 static hipError_t launch_pc_tile(const uint8_t* wb, const uint16_t* x, void* y, int y_dtype, const void* bias,
-                                 int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+                                 int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, int splits, hipStream_t s) {
   constexpr int BO = FUSE ? NJ * 8 : NJ * 16, BM = pc_bm(MB);
   const int n_tiles = (int)((n_out + BO - 1) / BO), m_tiles = (int)((m + BM - 1) / BM);
   int xcds_per_mtile = 0;
@@ -589,8 +660,21 @@ static hipError_t launch_pc_tile(const uint8_t* wb, const uint16_t* x, void* y, 
     xcds_per_mtile = 8 / m_tiles;
     nwg = (unsigned)(((n_tiles + xcds_per_mtile - 1) / xcds_per_mtile) * 8);
   }
-  hipLaunchKernelGGL((gemm_pc_kernel<NJ, FMT, MB, FUSE>), dim3(nwg), dim3(kPcThreads), 0, s, wb, x, y, y_dtype,
-                     bias, bias_dtype, (int)m, (int)n_out, (int)n_in, n_tiles, m_tiles, xcds_per_mtile);
+  PcSplit sp{1, (int)nwg, nullptr, nullptr};
+  if (!FUSE && splits > 1) {
+    // (the chooser has checked that the blocks of a row divide evenly and that the counters suffice)
+    const size_t units = (size_t)n_tiles * m_tiles * 4;
+    void* part = nullptr;
+    void* cnt = nullptr;
+    hipError_t e = stream_workspace(kWsGemmPartials, s, units * splits * (size_t)(MB * NJ * 1024), &part);
+    if (e == hipSuccess) e = stream_workspace(kWsGemmCounters, s, (size_t)kPcMaxCounters * 4, &cnt, true);
+    if (e != hipSuccess) return e;
+    sp.splits = splits;
+    sp.partials = static_cast<float*>(part);
+    sp.counters = static_cast<uint32_t*>(cnt);
+  }
+  hipLaunchKernelGGL((gemm_pc_kernel<NJ, FMT, MB, FUSE>), dim3(nwg * (unsigned)sp.splits), dim3(kPcThreads), 0, s, wb, x,
+                     y, y_dtype, bias, bias_dtype, (int)m, (int)n_out, (int)n_in, n_tiles, m_tiles, xcds_per_mtile, sp);
   return hipGetLastError();
 }
 
@@ -604,42 +688,66 @@ struct PcTile { int mb, nj; float step_us; };
 static const PcTile kPcTiles[] = {{4, 7, 0.87f}, {4, 4, 0.68f}, {2, 7, 0.585f}, {2, 4, 0.55f}, {1, 7, 0.46f}, {1, 4, 0.52f}};
 constexpr float kPcFixedUs = 6.f;
 
-static int pc_choose_tile(int64_t m, int64_t n_out, int64_t n_in, bool fuse, float* cost_us = nullptr) {
+// A grid that leaves most compute units idle (few columns x few rows: the attention output and down projections
+// at a few hundred rows) is also split along K, 2 / 4 / 7 / 8 ways while all copies still fit one round: the
+// length of a short round is the latency of its K loop.  What the meeting of the copies costs (measured, 1024 /
+// 4096 / 14336 columns x 4096 / 14336 inputs at 128 .. 1024 rows): a consumer stores its partial sums, counts,
+// and the last one loads the copies one after the other -- 2 + copies trips to the memory side (3 for two
+// copies), each the longer the more accumulators a lane holds -- and the partial sums cross the memory system
+// twice at about 4 TB/s.
+struct PcChoice { int tile, splits; float cost_us; };
+
+static float pc_split_us(const PcTile& t, int splits, int64_t padded_rows, int64_t padded_cols) {
+  const float trip = 0.9f + 0.06f * (float)(t.mb * t.nj);
+  const float trips = splits == 2 ? 3.f : 2.f + (float)splits;
+  return trips * trip + 2.f * (float)splits * (float)padded_rows * (float)padded_cols * 4.f / 4.0e6f;
+}
+
+static PcChoice pc_choose(int64_t m, int64_t n_out, int64_t n_in, bool fuse) {
   static const int forced = dev_knob("TTQ_GEMM_TILE", -1);
+  static const int forced_splits = dev_knob("TTQ_GEMM_SPLITS", 0);   // A/B: 1 = never split, n = n ways where possible
+  static const int kSplits[] = {1, 2, 4, 7, 8};
   const int cus = device_num_cus();
-  int best = 0;
-  float best_cost = 1e30f;
-  for (int i = 0; i < (int)(sizeof(kPcTiles) / sizeof(kPcTiles[0])); i++) {
-    if (forced >= 0 && forced < (int)(sizeof(kPcTiles) / sizeof(kPcTiles[0])) && i != forced) continue;
-    const PcTile& t = kPcTiles[i];
-    const int64_t bo = fuse ? t.nj * 8 : t.nj * 16, bm = pc_bm(t.mb);
-    const int64_t wgs = ((n_out + bo - 1) / bo) * ((m + bm - 1) / bm);
-    const int64_t rounds = (wgs + cus - 1) / cus;
-    const float cost = (float)rounds * ((float)(n_in / 64) * t.step_us + kPcFixedUs);
-    if (cost < best_cost * 0.999f) { best_cost = cost; best = i; }
+  const int64_t blocks = n_in / 256;
+  PcChoice best{0, 1, 1e30f};
+  for (int pass = 0; pass < 2 && best.cost_us > 1e29f; pass++) {
+    for (int i = 0; i < (int)(sizeof(kPcTiles) / sizeof(kPcTiles[0])); i++) {
+      if (forced >= 0 && forced < (int)(sizeof(kPcTiles) / sizeof(kPcTiles[0])) && i != forced) continue;
+      const PcTile& t = kPcTiles[i];
+      const int64_t bo = fuse ? t.nj * 8 : t.nj * 16, bm = pc_bm(t.mb);
+      const int64_t nt = (n_out + bo - 1) / bo, mt = (m + bm - 1) / bm, tiles = nt * mt;
+      for (int sp : kSplits) {
+        if (pass == 0 && forced_splits > 0 && sp != forced_splits) continue;
+        if (pass == 1 && sp != 1) continue;
+        if (sp > 1 && (fuse || blocks % sp != 0 || blocks / sp < 2 || tiles * sp > cus || tiles * 4 > kPcMaxCounters)) continue;
+        const int64_t rounds = (tiles * sp + cus - 1) / cus;
+        const float cost = (float)rounds * ((float)(n_in / 64 / sp) * t.step_us + kPcFixedUs) +
+                           (sp > 1 ? pc_split_us(t, sp, mt * bm, nt * bo) : 0.f);
+        if (cost < best.cost_us * 0.999f) best = PcChoice{i, sp, cost};
+      }
+    }
   }
-  if (cost_us) *cost_us = best_cost;
   return best;
 }
 
 // Rough time of the GEMM for this shape (microseconds), for callers that can also run the
 // operator as a few GEMV passes.  The Q6_K and Q8_0 producers are slower than the Q4_K one.
 float gemm_pc_estimate_us(int format, int64_t m, int64_t n_out, int64_t n_in) {
-  float c = 0.f;
-  pc_choose_tile(m, n_out, n_in, false, &c);
+  const float c = pc_choose(m, n_out, n_in, false).cost_us;
   return c * (format == kQ8_0 ? 1.9f : (format == kQ6_K ? 1.4f : 1.f)) + 2.f;
 }
 
 template <int FMT, bool FUSE>
 static hipError_t launch_pc_fmt(const uint8_t* wb, const uint16_t* x, void* y, int y_dtype, const void* bias,
                                 int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
-  switch (pc_choose_tile(m, n_out, n_in, FUSE)) {
-    case 0: return launch_pc_tile<FMT, 4, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-    case 1: return launch_pc_tile<FMT, 4, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-    case 2: return launch_pc_tile<FMT, 2, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-    case 3: return launch_pc_tile<FMT, 2, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-    case 4: return launch_pc_tile<FMT, 1, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-    default: return launch_pc_tile<FMT, 1, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  const PcChoice c = pc_choose(m, n_out, n_in, FUSE);
+  switch (c.tile) {
+    case 0: return launch_pc_tile<FMT, 4, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, s);
+    case 1: return launch_pc_tile<FMT, 4, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, s);
+    case 2: return launch_pc_tile<FMT, 2, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, s);
+    case 3: return launch_pc_tile<FMT, 2, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, s);
+    case 4: return launch_pc_tile<FMT, 1, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, s);
+    default: return launch_pc_tile<FMT, 1, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, s);
   }
 }
 

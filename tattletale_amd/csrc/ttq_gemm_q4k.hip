@@ -405,6 +405,23 @@ static bool prefer_skinny(int format, int64_t m, int64_t n_out, int64_t n_in) {
           gemm_skinny_estimate_us(format, m, n_out, n_in) < gemm_pc_estimate_us(format, m, n_out, n_in));
 }
 
+// 65 .. 256 rows on a matrix with few columns (attention output, down projection: 4096 columns are 37 tiles of
+// 112 for 256 compute units) leave the tiled kernel one short round whose length is the latency of its K loop.
+// It then splits K over copies of the grid (ttq_gemm_pc.hip); where the rows are too short for that, two or
+// three launches of the few-row kernel, 64 rows each, can still be faster.  The margin covers the tiled
+// kernel's estimate, which is fitted to full rounds and is about a third too high for a single short one.
+static float skinny_chunks_estimate_us(int format, int64_t m, int64_t n_out, int64_t n_in) {
+  const int64_t full = m / 64, rest = m % 64;
+  float us = (float)full * gemm_skinny_estimate_us(format, 64, n_out, n_in);
+  if (rest) us += gemm_skinny_estimate_us(format, rest, n_out, n_in);
+  return us;
+}
+static bool prefer_skinny_chunks(int format, int64_t m, int64_t n_out, int64_t n_in) {
+  if (m <= 64 || m > 256 || !gemm_skinny_supported(format, 64, n_out, n_in)) return false;
+  if (!gemm_pc_supported(format, m, n_out, n_in, 112)) return false;
+  return skinny_chunks_estimate_us(format, m, n_out, n_in) < 0.65f * gemm_pc_estimate_us(format, m, n_out, n_in);
+}
+
 bool gemm_supported(int format, int64_t m, int64_t n_out, int64_t n_in) {
   // Q4_K also has the single-role tiled kernel of this file, which takes any size
   return format == kQ4_K || gemm_skinny_supported(format, m, n_out, n_in) ||
@@ -422,6 +439,8 @@ hipError_t launch_gemm(int format, const void* w, const uint16_t* x_bf16, void* 
   if (m == 0 || n_out == 0) return hipSuccess;
   if (prefer_skinny(format, m, n_out, n_in))
     return launch_gemm_skinny(format, w, x_bf16, kBF16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  if (prefer_skinny_chunks(format, m, n_out, n_in))
+    return launch_gemm_skinny_chunked(format, w, x_bf16, kBF16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   if (format != kQ4_K) {
     if (!gemm_pc_supported(format, m, n_out, n_in, 112)) return hipErrorInvalidValue;
     return launch_gemm_pc(format, w, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);

@@ -198,8 +198,9 @@ hipError_t launch_hadamard128(float* v, const uint16_t* pre, const uint16_t* pos
                               hipStream_t s);
 
 // Workspaces the library keeps per (slot, device, stream), grown on demand (ttq_workspace.hip).
-constexpr int kWsExl3Rotated = 0, kWsBf16Activations = 1;
-hipError_t stream_workspace(int slot, hipStream_t s, size_t bytes, void** out);
+constexpr int kWsExl3Rotated = 0, kWsBf16Activations = 1, kWsGemmPartials = 2, kWsGemmCounters = 3;
+// zeroed: a newly allocated buffer is cleared (on the stream) before it is handed out
+hipError_t stream_workspace(int slot, hipStream_t s, size_t bytes, void** out, bool zeroed = false);
 // n fp16 or fp32 values (n a multiple of 8) rounded to bf16
 hipError_t launch_to_bf16(const void* x, int x_dtype, uint16_t* out, int64_t n, hipStream_t s);
 

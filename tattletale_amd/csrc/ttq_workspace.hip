@@ -16,7 +16,7 @@ std::mutex g_mutex;
 std::unordered_map<uint64_t, Buf> g_bufs;
 }  // namespace
 
-hipError_t stream_workspace(int slot, hipStream_t s, size_t bytes, void** out) {
+hipError_t stream_workspace(int slot, hipStream_t s, size_t bytes, void** out, bool zeroed) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
@@ -35,6 +35,14 @@ hipError_t stream_workspace(int slot, hipStream_t s, size_t bytes, void** out) {
     void* p = nullptr;
     e = hipMalloc(&p, bytes);
     if (e != hipSuccess) return e;
+    if (zeroed) {
+      // ordered before every launch that will use the buffer: they are all on this stream
+      e = hipMemsetAsync(p, 0, bytes, s);
+      if (e != hipSuccess) {
+        (void)hipFree(p);
+        return e;
+      }
+    }
     b.p = p;
     b.bytes = bytes;
   }

@@ -52,6 +52,67 @@ def test_gemm_identity_activations_give_bf16_weights_exactly(n_in):
     assert not (y[n_in:] & 0x7FFF).any()
 
 
+# Few tiles for 256 compute units (few columns x a few hundred rows) with a long K: the tiled kernel is launched
+# as 2 / 4 / 7 / 8 copies that split K and add their partial sums through a workspace.
+@pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
+@pytest.mark.parametrize("m,n_out,n_in", [(512, 4096, 4096), (256, 1024, 4096), (300, 1000, 2048), (130, 2048, 14336),
+                                          (192, 4096 + 40, 3584)])
+def test_gemm_split_along_k(fmt, m, n_out, n_in):
+    """Against the float64 product; three calls in a row give the same bits (the copies of a tile are added in a
+    fixed order, and the arrival counters are back at zero after every launch), also after a call with another
+    shape in between (the workspace grows)."""
+    w = Q.fill_normal(700 + m, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
+    p = Q.quantize(fmt, w)
+    what = oracle.dequant(fmt, p, n_out, n_in)
+    wd = packed_to_dev(p)
+    xd, xf = x_to_dev(Q.fill_normal(701 + m, 1, 1.0, m * n_in).reshape(m, n_in), "bf16")
+    y1 = dev_bits(QL.gemm(fmt, wd, xd, n_out, n_in))
+    want_r = oracle.linear_f64(oracle.bf16_to_f32(oracle.f32_to_bf16(what)), xf)
+    assert rel_l2(oracle.bf16_to_f32(y1), want_r) <= 4e-3
+    assert rel_l2(oracle.bf16_to_f32(y1), oracle.linear_f64(what, xf)) <= TOL
+    y2 = dev_bits(QL.gemm(fmt, wd, xd, n_out, n_in))
+    # another shape on the same stream
+    p3 = random_blocks(fmt, 512 * (1024 // BLOCK_WEIGHTS[fmt]), seed=5)
+    x3, _ = x_to_dev(Q.fill_normal(702, 1, 1.0, 384 * 1024).reshape(384, 1024), "bf16")
+    QL.gemm(fmt, packed_to_dev(p3), x3, 512, 1024)
+    y3 = dev_bits(QL.gemm(fmt, wd, xd, n_out, n_in))
+    assert np.array_equal(y1, y2) and np.array_equal(y1, y3)
+
+
+@pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
+def test_gemm_split_along_k_identity_activations_give_bf16_weights_exactly(fmt):
+    """X = [I; 0] over 2048 inputs (eight super-blocks, split four ways on a 256-CU device): every output is one
+    bf16-rounded weight plus zeros from the other copies."""
+    n_out, n_in = 192, 2048
+    p = random_blocks(fmt, n_out * (n_in // BLOCK_WEIGHTS[fmt]), seed=19)
+    what = oracle.dequant(fmt, p, n_out, n_in)
+    m = n_in + 32
+    x = np.zeros((m, n_in), np.float32)
+    x[np.arange(n_in), np.arange(n_in)] = 1.0
+    xd, _ = x_to_dev(x, "bf16")
+    y = dev_bits(QL.gemm(fmt, packed_to_dev(p), xd, n_out, n_in))
+    want = oracle.f32_to_bf16(what).T
+    # a weight that is -0 (Q6_K, Q8_0: q = 0 under a negative scale) comes out as +0: its copy's -0 meets the
+    # other copies' +0 in an fp32 addition
+    zero = (want & 0x7FFF) == 0
+    assert np.array_equal(y[:n_in][~zero], want[~zero])
+    assert not (y[:n_in][zero] & 0x7FFF).any()
+    assert not (y[n_in:] & 0x7FFF).any()
+
+
+def test_forward_split_along_k_f32_output_with_bias():
+    n_out, n_in, m = 1024 + 24, 4096, 200
+    w = Q.fill_normal(710, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
+    p = Q.quantize(F.Q4_K, w)
+    what = oracle.dequant(F.Q4_K, p, n_out, n_in)
+    bias = Q.fill_normal(711, 0, 0.5, n_out)
+    layer = QuantLinear.init(packed_to_dev(p), F.Q4_K, n_in, n_out, bias=torch.from_numpy(bias).to(DEV))
+    xd, xf = x_to_dev(Q.fill_normal(712, 1, 1.0, m * n_in).reshape(m, n_in), "bf16")
+    y = layer.forward(xd, out_dtype=torch.float32).cpu().numpy()
+    want = oracle.linear_f64(what, xf) + bias
+    assert rel_l2(y, want) <= TOL
+
+
 # Up to 64 activation rows take the kernel that dequantizes in registers (no W tile in LDS), with
 # 16, 32 or 64 weight rows per workgroup: n_out <= 4096 gives 16, 6144 gives 32, 12288 and up 64 on
 # a 256-CU device.  Token blocks of 16: m = 1..16, 17..32, 33..48, 49..64.  n_out not a multiple of
