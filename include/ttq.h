@@ -158,7 +158,12 @@ TTQ_API int ttq_gemv_exl3_noalloc(const uint16_t* trellis, const uint16_t* suh_f
  * multiplied with bf16 MFMA, fp32 accumulation.  Stands in for F.linear(x, weight) with a
  * (batch*seq, n_in) activation (neural_nets.nim:64; attn.nim:154-156 prefill case).
  * Up to 64 rows may run a kernel that dequantizes in registers instead of tiling W through LDS
- * (same arithmetic: weights rounded to bf16 once, fp32 accumulation); the library picks by shape. */
+ * (same arithmetic: weights rounded to bf16 once, fp32 accumulation); the library picks by shape.
+ * Shapes with few output tiles and a long K are computed as up to eight partial products over slices
+ * of K that meet in a workspace the library keeps per (device, stream) -- fp32, rows x columns x
+ * slices, allocated on first use and grown on demand, so the first call of such a shape on a stream
+ * must not happen under graph capture; the partial products are added in a fixed order (the same
+ * bits on every call).  The same holds for ttq_gemm_q6_k, ttq_gemm_q8_0 and ttq_linear_forward. */
 TTQ_API int ttq_gemm_q4_k(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m,
                   int64_t n_out, int64_t n_in, void* stream);
 /* The same operator for Q6_K and Q8_0 weights (a GGUF "Q4_K_M" file mixes Q4_K and Q6_K tensors;
