@@ -427,7 +427,8 @@ def main() -> int:
         sites workspace/transformers/src/layers/attn.nim:113-116,154-156,189), the LM-head-sized Q4_K
         stream, a Q6_K down projection (mlp.nim:60), the few-row decode GEMV (8 and 16 activation rows at once), the few-row form of the
         prefill operator (32 rows) and the prefill GEMM for Q6_K and Q8_0 weights, 14336 x 4096 unless
-        named otherwise; add + RMSNorm on rows of 4096."""
+        named otherwise; the down projection at 128 and 512 rows (K split over copies of the tile grid);
+        add + RMSNorm on rows of 4096."""
         n_out, n_in = 14336, 4096
         rng = np.random.default_rng(1234)
         res = {}
@@ -507,6 +508,12 @@ def main() -> int:
         timed("q4_k_gemm_m512_4096x4096", F.Q4_K, 512,
               lambda ws, x, nc, y=y: (lambda i: QL.gemm(F.Q4_K, ws[i % nc], x, 4096, 4096, out=y)),
               n_out=4096, n_in=4096, steps=max(20, steps // 4))
+        # the down projection of a prefill chunk: few output tiles, long K -- the launches that split K
+        for m in (128, 512):
+            y = torch.empty((m, 4096), dtype=torch.bfloat16, device=dev)
+            timed("q4_k_gemm_m%d_down_4096x14336" % m, F.Q4_K, m,
+                  lambda ws, x, nc, y=y: (lambda i: QL.gemm(F.Q4_K, ws[i % nc], x, 4096, 14336, out=y)),
+                  n_out=4096, n_in=14336, steps=max(20, steps // 4))
         # add + RMSNorm alone (ttq_rmsnorm with a residual): one decode row and a prefill block.
         # Algorithmic bytes: x and residual read, new residual and normalized row written.
         L = _lib.lib()
