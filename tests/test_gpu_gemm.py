@@ -56,11 +56,12 @@ def test_gemm_identity_activations_give_bf16_weights_exactly(n_in):
 # as 2 / 4 / 7 / 8 copies that split K and add their partial sums through a workspace.
 @pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
 @pytest.mark.parametrize("m,n_out,n_in", [(512, 4096, 4096), (256, 1024, 4096), (300, 1000, 2048), (130, 2048, 14336),
-                                          (192, 4096 + 40, 3584)])
+                                          (192, 4096 + 40, 3584), (300, 256, 6144), (300, 256, 5376)])
 def test_gemm_split_along_k(fmt, m, n_out, n_in):
     """Against the float64 product; three calls in a row give the same bits (the copies of a tile are added in a
     fixed order, and the arrival counters are back at zero after every launch), also after a call with another
-    shape in between (the workspace grows)."""
+    shape in between (the workspace grows).  On a 256-CU device the chooser takes two or four copies for the
+    first shapes, eight for 256 x 6144 and seven for 256 x 5376 (21 super-blocks)."""
     w = Q.fill_normal(700 + m, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
     p = Q.quantize(fmt, w)
     what = oracle.dequant(fmt, p, n_out, n_in)
