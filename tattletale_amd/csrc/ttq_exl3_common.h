@@ -69,6 +69,7 @@ __device__ __forceinline__ void load_x4(const bf16_tag* p, float (&v)[4]) {
 // Shared by the matrix-core trellis kernels (decode GEMV and prefill GEMM): workgroup shape, the
 // decode of a lane's four weights of a tile into an A fragment, and the LDS layout of a pass of tiles.
 typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 
 // 16 wavefronts: a wavefront issues one vector instruction about every five clocks however many others
 // share its SIMD, so the decode rate of a compute unit grows with the number of resident wavefronts.

@@ -7,7 +7,7 @@
 // pass of 64 rows would cost a workgroup more vector work than decoding the pass's weights.  The second
 // is the decode GEMV's workgroup (128 output channels, 16 wavefronts, weights staged through LDS as a
 // big-endian bit string, four weights per lane decoded into an A fragment) with 64 rows per workgroup:
-// each decoded fragment feeds four v_mfma_f32_16x16x16_f16, one per block of 16 rows, so the decode --
+// each pair of decoded fragments feeds four v_mfma_f32_16x16x32_f16, one per block of 16 rows, so the decode --
 // which bounds the single-row kernel -- is paid once per 64 rows; a wavefront takes two tile columns, so
 // that every activation fragment it reads from LDS serves two of them.  A workgroup covers the whole
 // reduction, rotates its 64 x 128 sums and writes y; no workspace is shared between workgroups.
@@ -147,19 +147,27 @@ gemm_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __re
 #pragma unroll
         for (int c = 0; c < kXpCols; c++) ln.fetch(wcol + ((gl * 8 + i) * 8 + c) * G::kTileStride, cw[buf][i][c]);
     };
+    // The wavefront's two k-tiles of a group go through one v_mfma_f32_16x16x32_f16: a lane's eight k positions
+    // are its four of the first tile followed by its four of the second -- any assignment of the 32 k's to
+    // (lane group, element) does, as long as the activation fragment uses the same one -- so the decode and the
+    // LDS reads are those of the 16-k form and there are half as many matrix instructions, each as long as
+    // one of those (measured: 19 ns per instruction and wavefront for either, all SIMDs busy).
     auto compute_group = [&](int gl, int buf) {
+      static_assert(kXpTiles == 2, "two k-tiles per matrix instruction");
+      f16x8_t a[kXpCols];
 #pragma unroll
-      for (int i = 0; i < kXpTiles; i++) {
-        f16x4_t a[kXpCols];
+      for (int c = 0; c < kXpCols; c++) {
+        const f16x4_t a0 = ln.template decode<CB>(cw[buf][0][c]), a1 = ln.template decode<CB>(cw[buf][1][c]);
+        a[c] = f16x8_t{a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+      }
+      const _Float16* xb = xcol + gl * 8 * 16;
 #pragma unroll
-        for (int c = 0; c < kXpCols; c++) a[c] = ln.template decode<CB>(cw[buf][i][c]);
-        const _Float16* xb = xcol + (gl * 8 + i) * 16;
+      for (int rb = 0; rb < kXpRowBlocks; rb++) {
+        const f16x4_t b0 = *reinterpret_cast<const f16x4_t*>(xb + rb * 16 * kXmColStride);
+        const f16x4_t b1 = *reinterpret_cast<const f16x4_t*>(xb + 16 + rb * 16 * kXmColStride);
+        const f16x8_t b = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
 #pragma unroll
-        for (int rb = 0; rb < kXpRowBlocks; rb++) {
-          const f16x4_t b = *reinterpret_cast<const f16x4_t*>(xb + rb * 16 * kXmColStride);
-#pragma unroll
-          for (int c = 0; c < kXpCols; c++) acc[c][rb] = __builtin_amdgcn_mfma_f32_16x16x16f16(a[c], b, acc[c][rb], 0, 0, 0);
-        }
+        for (int c = 0; c < kXpCols; c++) acc[c][rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[c], b, acc[c][rb], 0, 0, 0);
       }
     };
     fetch_group(0, 0);
