@@ -49,6 +49,7 @@ constexpr int kSkThreads = 512;
 constexpr int kSkWaves = kSkThreads / 64;
 // time per row block relative to Q4_K (cost model)
 constexpr float kSkQ6KWeightFactor = 1.2f, kSkQ8WeightFactor = 2.2f;
+constexpr float kSkSplitUs = 2.5f;     // a split launch: store, count and add the copies' sums (three trips to the memory side)
 
 __device__ __forceinline__ uint2 load8_a2(const uint8_t* p) {
   uint2 v;
@@ -302,6 +303,16 @@ struct SkQ8_0 {
   }
 };
 
+// Split along K: the grid holds `splits` copies of the row tiles, copy c works on super-blocks
+// [c, c + 1) * nsb / splits, and the copies of a tile add up through a workspace (see the epilogue).
+struct SkSplit {
+  int splits;          // 1: none
+  int tiles;           // workgroups of one copy
+  float* partials;
+  uint32_t* counters;  // one per tile, zero between launches
+};
+constexpr int kSkMaxCounters = 16384;
+
 // RB: blocks of 16 weight rows per workgroup; TB: blocks of 16 tokens (m <= 16 * TB); WD: ring of
 // (super-block, row block) items of packed weights per wavefront, WD - 1 of them in flight; XB:
 // buffers for a super-block's activations (2: the next super-block's are requested while this one
@@ -309,7 +320,8 @@ struct SkQ8_0 {
 template <class WF, class XT, int RB, int TB, int WD, int XB, bool FUSE>
 __global__ void __launch_bounds__(kSkThreads)
 gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, void* __restrict__ yv,
-                       int y_dtype, const void* __restrict__ bias, int bias_dtype, int m, int n_out, int n_in) {
+                       int y_dtype, const void* __restrict__ bias, int bias_dtype, int m, int n_out, int n_in,
+                       SkSplit sp) {
   static_assert((WD == 2 || WD == 4) && (2 * RB) % WD == 0 && (XB == 1 || XB == 2), "ring sizes");
   extern __shared__ float smem[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -322,7 +334,11 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
   // and the up rows of the same 16 outputs.
   static_assert(!FUSE || RB % 2 == 0, "a fused workgroup needs gate and up row blocks in pairs");
   constexpr int kOutPerWg = FUSE ? 8 * RB : 16 * RB;
-  const int n0 = blockIdx.x * kOutPerWg;
+  const int ksplit = sp.splits > 1 ? (int)blockIdx.x / sp.tiles : 0;
+  const int tile_id = (int)blockIdx.x - ksplit * sp.tiles;
+  const int n0 = tile_id * kOutPerWg;
+  // this workgroup's super-blocks
+  const int sb_lo = ksplit * (nsb / sp.splits), sb_hi = sb_lo + nsb / sp.splits;
 
   // byte offset of (row, super-block 0) and element offset of (token, k = 8*kg)
   uint32_t wofs[RB], xofs[TB];
@@ -373,7 +389,7 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
   auto super_block = [&](auto xi_c, int sb) {
     constexpr int XI = decltype(xi_c)::value;
     constexpr int kAhead = WD - 1;
-    const int sb_next = sb + kSkWaves < nsb ? sb + kSkWaves : sb;
+    const int sb_next = sb + kSkWaves < sb_hi ? sb + kSkWaves : sb;
     if constexpr (XB == 1) load_x(xfr[0], sb);
     // this super-block's activations into the operand layout (they were requested one super-block
     // ago when there are two buffers)
@@ -388,7 +404,7 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
         constexpr int kMaxOff = (RB - 1 + kAhead) / RB;
         const int off = (rb + kAhead) / RB;
         int sb_a = sb + off * kSkWaves;
-        if (kMaxOff > 1 || off > 0) sb_a = sb_a < nsb ? sb_a : sb;
+        if (kMaxOff > 1 || off > 0) sb_a = sb_a < sb_hi ? sb_a : sb;
         fetch(raw[(XI * RB + rb + kAhead) % WD], sb_a, (rb + kAhead) % RB);
       }
       typename WF::Raw& r = raw[(XI * RB + rb) % WD];
@@ -410,17 +426,17 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
     }
   };
 
-  if (wave < nsb) {
+  if (sb_lo + wave < sb_hi) {
 #pragma unroll
     for (int q = 0; q < WD - 1; q++) {
-      const int sb_q = wave + (q / RB) * kSkWaves;
-      fetch(raw[q % WD], sb_q < nsb ? sb_q : wave, q % RB);
+      const int sb_q = sb_lo + wave + (q / RB) * kSkWaves;
+      fetch(raw[q % WD], sb_q < sb_hi ? sb_q : sb_lo + wave, q % RB);
     }
-    if (XB == 2) load_x(xfr[0], wave);
+    if (XB == 2) load_x(xfr[0], sb_lo + wave);
   }
-  for (int sb = wave; sb < nsb; sb += 2 * kSkWaves) {
+  for (int sb = sb_lo + wave; sb < sb_hi; sb += 2 * kSkWaves) {
     super_block(std::integral_constant<int, 0>{}, sb);
-    if (sb + kSkWaves < nsb) super_block(std::integral_constant<int, 1>{}, sb + kSkWaves);
+    if (sb + kSkWaves < sb_hi) super_block(std::integral_constant<int, 1>{}, sb + kSkWaves);
   }
 
   // The wavefronts' partial sums: part[wave][rb][tb][r][lane]; element (rb, tb, r, lane) is weight
@@ -446,6 +462,35 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
     tile[tok * kTileLd + row] = s;
   }
   __syncthreads();
+  // ---- split along K: the tile of sums goes to the workspace, a counter per tile says how many copies have
+  // arrived, and the workgroup that arrives last adds all copies in copy order -- the same sum whichever
+  // arrives last -- and writes the outputs.  Nobody waits for anybody.  Sums and counter move as device-scope
+  // relaxed atomics (the L2 caches of the dies are not coherent with each other; these accesses go through to
+  // the memory side), the stores are complete before the count, the loads are issued after it.
+  if constexpr (!FUSE) {
+    if (sp.splits > 1) {
+      constexpr int kTileFloats = 16 * TB * kTileLd;
+      float* all = sp.partials + (size_t)tile_id * (size_t)(sp.splits * kTileFloats);
+      float* mine = all + ksplit * kTileFloats;
+      for (int e = tid; e < kTileFloats; e += kSkThreads)
+        __hip_atomic_store(mine + e, tile[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      uint32_t* flag = reinterpret_cast<uint32_t*>(part);          // the wavefronts' partial sums are done with
+      if (tid == 0)
+        flag[0] = __hip_atomic_fetch_add(sp.counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __syncthreads();
+      if (flag[0] != (uint32_t)(sp.splits - 1)) return;
+      if (tid == 0) __hip_atomic_store(sp.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int e = tid; e < kTileFloats; e += kSkThreads) {
+        float v = __hip_atomic_load(all + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int c = 1; c < sp.splits; c++)
+          v += __hip_atomic_load(all + c * kTileFloats + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        tile[e] = v;
+      }
+      __syncthreads();
+    }
+  }
   // 8 consecutive outputs of one token per thread
   constexpr int kGroups = kOutPerWg / 8;
   for (int t = tid; t < 16 * TB * kGroups; t += kSkThreads) {
@@ -485,7 +530,7 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
 // n_out counts outputs: weight rows, or gate/up pairs when fused.
 template <int RB, int TB, bool FUSE, class K>
 hipError_t launch_skinny_k(K kernel, const uint8_t* w, const uint16_t* x, void* y, int y_dtype, const void* bias,
-                           int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+                           int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, int splits, hipStream_t s) {
   const size_t lds = (size_t)(kSkWaves * RB * TB * 4 * 64 + 16 * TB * (16 * RB + 1)) * sizeof(float);
   static LargeLds configured;          // one per kernel instantiation: K is part of this function's type
   if (lds > 64 * 1024) {
@@ -493,16 +538,29 @@ hipError_t launch_skinny_k(K kernel, const uint8_t* w, const uint16_t* x, void* 
     if (e != hipSuccess) return e;
   }
   constexpr int kOutPerWg = FUSE ? 8 * RB : 16 * RB;
-  const dim3 grid((unsigned)((n_out + kOutPerWg - 1) / kOutPerWg)), block(kSkThreads);
-  hipLaunchKernelGGL(kernel, grid, block, lds, s, w, x, y, y_dtype, bias, bias_dtype, (int)m, (int)n_out, (int)n_in);
+  const int tiles = (int)((n_out + kOutPerWg - 1) / kOutPerWg);
+  SkSplit sp{1, tiles, nullptr, nullptr};
+  if (!FUSE && splits > 1) {
+    // (the chooser has checked that the super-blocks divide evenly and that the counters suffice)
+    void* part = nullptr;
+    void* cnt = nullptr;
+    hipError_t e = stream_workspace(kWsGemmPartials, s, (size_t)tiles * splits * (16 * TB * (16 * RB + 1)) * sizeof(float), &part);
+    if (e == hipSuccess) e = stream_workspace(kWsGemmCounters, s, (size_t)kSkMaxCounters * 4, &cnt, true);
+    if (e != hipSuccess) return e;
+    sp.splits = splits;
+    sp.partials = static_cast<float*>(part);
+    sp.counters = static_cast<uint32_t*>(cnt);
+  }
+  const dim3 grid((unsigned)(tiles * sp.splits)), block(kSkThreads);
+  hipLaunchKernelGGL(kernel, grid, block, lds, s, w, x, y, y_dtype, bias, bias_dtype, (int)m, (int)n_out, (int)n_in, sp);
   return hipGetLastError();
 }
 
 template <class WF, class XT, int RB, int TB, int WD, int XB, bool FUSE>
 hipError_t launch_skinny_tb(const uint8_t* w, const uint16_t* x, void* y, int y_dtype, const void* bias,
-                            int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+                            int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, int splits, hipStream_t s) {
   return launch_skinny_k<RB, TB, FUSE>(gemm_skinny_kernel<WF, XT, RB, TB, WD, XB, FUSE>, w, x, y, y_dtype, bias,
-                                       bias_dtype, m, n_out, n_in, s);
+                                       bias_dtype, m, n_out, n_in, splits, s);
 }
 
 // Cost model (microseconds), a least-squares fit to 4096 x 4096, 4096 x 14336 and 14336 x 4096 with
@@ -511,29 +569,46 @@ hipError_t launch_skinny_tb(const uint8_t* w, const uint16_t* x, void* y, int y_
 // 0.2 (the stream itself, about 5 TB/s).  The activations of a super-block are re-read from L2 by
 // every workgroup, which is what makes more rows per workgroup cheaper per row, as long as every
 // CU still gets a workgroup.  The weight term is scaled for the other formats.
-float skinny_cost_us(int format, int rb, int64_t m, int64_t n_out, int64_t n_in) {
+float skinny_cost_us(int format, int rb, int splits, int64_t m, int64_t n_out, int64_t n_in) {
   static const float kF0[4] = {1.95f, 2.78f, 2.11f, 2.51f}, kX[4] = {0.44f, 1.30f, 1.87f, 2.36f};
   static const float kW[4] = {0.97f, 0.88f, 1.10f, 1.31f};
   const float wf = format == kQ6_K ? kSkQ6KWeightFactor : (format == kQ8_0 ? kSkQ8WeightFactor : 1.f);
   const int64_t block_bytes = format == kQ4_K ? 144 : (format == kQ6_K ? 210 : 272);
   const float mb = (float)(n_out * (n_in >> 8) * block_bytes) * 1e-6f;
   const int t = (int)((m + 15) / 16) - 1;
-  const int64_t wgs = (n_out + 16 * rb - 1) / (16 * rb), cus = device_num_cus();
-  const int64_t iters = ((n_in >> 8) + kSkWaves - 1) / kSkWaves;
-  return (float)((wgs + cus - 1) / cus) * (kF0[t] + (float)iters * (kX[t] + rb * wf * kW[t])) + 0.2f * mb;
+  const int64_t wgs = splits * ((n_out + 16 * rb - 1) / (16 * rb)), cus = device_num_cus();
+  const int64_t iters = ((n_in >> 8) / splits + kSkWaves - 1) / kSkWaves;
+  return (float)((wgs + cus - 1) / cus) * (kF0[t] + (float)iters * (kX[t] + rb * wf * kW[t])) + 0.2f * mb +
+         (splits > 1 ? kSkSplitUs : 0.f);
 }
 
-// rows = weight rows (twice the outputs when fused, which also rules out single row blocks)
-int skinny_choose_rb(int format, int64_t m, int64_t rows, int64_t n_in, bool fuse, float* cost_us = nullptr) {
+// rows = weight rows (twice the outputs when fused, which also rules out single row blocks).  Few row tiles and a
+// long K: every workgroup re-reads all activations of its tokens, so more rows per workgroup are cheaper per
+// row, and a second copy of the grid along K gives the compute units those bigger tiles would leave idle
+// something to do (4096 x 14336, 64 rows: 16 rows per workgroup 35.6 us, 32 rows in two copies 27.2 us).  The
+// kernel takes any number of copies that divides the super-blocks; a sweep over 1 / 2 / 4 / 7 / 8 copies x 16 / 32
+// / 64 rows per workgroup on five shapes found nothing that beats two by more than the noise, and the cost
+// model above, fitted to full grids, misjudges the deeper splits, so two is what the chooser offers.
+struct SkChoice { int rb, splits; float cost_us; };
+SkChoice skinny_choose(int format, int64_t m, int64_t rows, int64_t n_in, bool fuse) {
   static const int forced_rb = dev_knob("TTQ_SK_RB", 0);
-  int best = 4;
-  float best_cost = 1e30f;
-  for (int rb = 4; rb >= (fuse ? 2 : 1); rb >>= 1) {
-    if (forced_rb > 0 && rb != forced_rb && !(fuse && forced_rb == 1)) continue;
-    const float c = skinny_cost_us(format, rb, m, rows, n_in);
-    if (c < best_cost) { best_cost = c; best = rb; }
+  static const int forced_splits = dev_knob("TTQ_SK_SPLITS", 0);
+  static const int kSplits[] = {1, 2};
+  const int64_t nsb = n_in >> 8, cus = device_num_cus();
+  SkChoice best{4, 1, 1e30f};
+  for (int pass = 0; pass < 2 && best.cost_us > 1e29f; pass++) {
+    for (int rb = 4; rb >= (fuse ? 2 : 1); rb >>= 1) {
+      if (forced_rb > 0 && rb != forced_rb && !(fuse && forced_rb == 1)) continue;
+      const int64_t tiles = (rows + 16 * rb - 1) / (16 * rb);
+      for (int sp : kSplits) {
+        if (pass == 0 && forced_splits > 0 && sp != forced_splits) continue;
+        if (pass == 1 && sp != 1) continue;
+        if (sp > 1 && (fuse || nsb % sp != 0 || tiles * sp > cus || tiles > kSkMaxCounters)) continue;
+        const float c = skinny_cost_us(format, rb, sp, m, rows, n_in);
+        if (c < best.cost_us) best = SkChoice{rb, sp, c};
+      }
+    }
   }
-  if (cost_us) *cost_us = best_cost;
   return best;
 }
 
@@ -542,11 +617,12 @@ template <class WF, class XT, bool FUSE>
 hipError_t launch_skinny_fmt(int format, const uint8_t* wb, const uint16_t* x_bf16, void* y, int y_dtype,
                              const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                              hipStream_t s) {
-  const int rb = skinny_choose_rb(format, m, FUSE ? 2 * n_out : n_out, n_in, FUSE);
+  const SkChoice ch = skinny_choose(format, m, FUSE ? 2 * n_out : n_out, n_in, FUSE);
+  const int rb = ch.rb;
   const int tb = (int)((m + 15) / 16);
 #define TTQ_SK_CASE(RBv, TBv, WDv, XBv) \
   if (rb == RBv && tb == TBv)            \
-    return launch_skinny_tb<WF, XT, RBv, TBv, WDv, XBv, FUSE>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    return launch_skinny_tb<WF, XT, RBv, TBv, WDv, XBv, FUSE>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, ch.splits, s);
   TTQ_SK_CASE(4, 1, 4, 2) TTQ_SK_CASE(4, 2, 4, 2) TTQ_SK_CASE(4, 3, 2, 1) TTQ_SK_CASE(4, 4, 2, 1)
   TTQ_SK_CASE(2, 1, 4, 2) TTQ_SK_CASE(2, 2, 4, 2) TTQ_SK_CASE(2, 3, 2, 1) TTQ_SK_CASE(2, 4, 2, 1)
   if constexpr (!FUSE) {
@@ -569,9 +645,7 @@ bool gemm_skinny_supported(int format, int64_t m, int64_t n_out, int64_t n_in) {
 }
 
 float gemm_skinny_estimate_us(int format, int64_t m, int64_t n_out, int64_t n_in) {
-  float c = 0.f;
-  skinny_choose_rb(format, m, n_out, n_in, false, &c);
-  return c;
+  return skinny_choose(format, m, n_out, n_in, false).cost_us;
 }
 
 // The fused gate||up + silu_and_mul form: n_ff outputs from 2 * n_ff weight rows (Q4_K).
@@ -580,9 +654,7 @@ bool gemm_skinny_silu_mul_supported(int64_t m, int64_t n_ff, int64_t n_in) {
 }
 
 float gemm_skinny_silu_mul_estimate_us(int64_t m, int64_t n_ff, int64_t n_in) {
-  float c = 0.f;
-  skinny_choose_rb(kQ4_K, m, 2 * n_ff, n_in, true, &c);
-  return c;
+  return skinny_choose(kQ4_K, m, 2 * n_ff, n_in, true).cost_us;
 }
 
 hipError_t launch_gemm_skinny_silu_mul(const void* w, const uint16_t* x_bf16, void* y, int y_dtype, const void* bias,

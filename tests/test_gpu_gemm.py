@@ -138,6 +138,32 @@ def test_gemm_few_rows(fmt, m, n_out, n_in):
         assert rel_l2(got[i], want_r[i]) <= 6e-3, i
 
 
+# Few rows x few row tiles x a long K: the few-row kernel takes more weight rows per workgroup (every workgroup
+# re-reads the activations of all its tokens) and runs two copies of the grid along K.
+@pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
+@pytest.mark.parametrize("m,n_out,n_in", [(64, 4096, 14336), (32, 1024, 8192), (48, 4096 + 40, 7168), (17, 512, 3584),
+                                          (5, 2048, 4096)])
+def test_gemm_few_rows_split_along_k(fmt, m, n_out, n_in):
+    """Against the float64 product, every token on its own; three calls give the same bits (fixed order of the
+    copies, counters back at zero), also with another split shape in between."""
+    p = random_blocks(fmt, n_out * (n_in // BLOCK_WEIGHTS[fmt]), seed=900 + m)
+    what_r = oracle.bf16_to_f32(oracle.f32_to_bf16(oracle.dequant(fmt, p, n_out, n_in)))
+    wd = packed_to_dev(p)
+    xd, xf = x_to_dev(Q.fill_normal(901 + m, 1, 1.0, m * n_in).reshape(m, n_in), "bf16")
+    y1 = dev_bits(QL.gemm(fmt, wd, xd, n_out, n_in))
+    got = oracle.bf16_to_f32(y1)
+    want_r = oracle.linear_f64(what_r, xf)
+    assert rel_l2(got, want_r) <= 4e-3
+    for i in range(m):
+        assert rel_l2(got[i], want_r[i]) <= 6e-3, i
+    y2 = dev_bits(QL.gemm(fmt, wd, xd, n_out, n_in))
+    p3 = random_blocks(fmt, 256 * (2048 // BLOCK_WEIGHTS[fmt]), seed=6)
+    x3, _ = x_to_dev(Q.fill_normal(902, 1, 1.0, 40 * 2048).reshape(40, 2048), "bf16")
+    QL.gemm(fmt, packed_to_dev(p3), x3, 256, 2048)
+    y3 = dev_bits(QL.gemm(fmt, wd, xd, n_out, n_in))
+    assert np.array_equal(y1, y2) and np.array_equal(y1, y3)
+
+
 @pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
 @pytest.mark.parametrize("m,n_out", [(64, 192), (40, 6144), (16, 12304)])
 def test_gemm_few_rows_unit_vectors_give_bf16_weights_exactly(fmt, m, n_out):
