@@ -425,7 +425,7 @@ def main() -> int:
         """Rows next to the headline ones, on random packed bytes with finite scale fields (timing
         only): the attention projections as decode GEMVs (q/o 4096x4096, k/v 1024x4096, reference call
         sites workspace/transformers/src/layers/attn.nim:113-116,154-156,189), the LM-head-sized Q4_K
-        stream, a Q6_K down projection (mlp.nim:60), the few-row decode GEMV (8 and 16 activation rows at once), the few-row form of the
+        stream, a Q6_K down projection (mlp.nim:60), the few-row decode GEMV (2, 4, 8 and 16 activation rows at once), the few-row form of the
         prefill operator (32 rows) and the prefill GEMM for Q6_K and Q8_0 weights, 14336 x 4096 unless
         named otherwise; the down projection at 128 and 512 rows (K split over copies of the tile grid);
         add + RMSNorm on rows of 4096."""
@@ -464,7 +464,7 @@ def main() -> int:
         y = torch.empty((1, n_out), dtype=torch.float32, device=dev)
         timed("q8_0_gemv_14336x4096", F.Q8_0, 1,
               lambda ws, x, nc, y=y: (lambda i: QL.gemv(F.Q8_0, ws[i % nc], x, n_out, n_in, out=y)))
-        for m in (8, 16):
+        for m in (2, 4, 8, 16):
             y = torch.empty((m, n_out), dtype=torch.float32, device=dev)
             timed("q4_k_gemv_m%d" % m, F.Q4_K, m,
                   lambda ws, x, nc, y=y: (lambda i: QL.gemv(F.Q4_K, ws[i % nc], x, n_out, n_in, out=y)))

@@ -326,6 +326,8 @@ hipError_t launch_gemv(int format, const void* w, const void* x, int x_dtype, vo
   if (m == 0 || n_out == 0) return hipSuccess;
   // a few rows at once: four per pass for up to four rows and for rows too long for the 8- and
   // 16-token tables, else eight or sixteen per pass
+  if (gemv_q4k_stream4_supported(format, x_dtype, m, n_out, n_in))
+    return launch_gemv_q4k_stream4(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   static const int batch4_max = dev_knob("TTQ_GEMV_BATCH4_MAX_ROWS", 4);
   const bool b4 = gemv_q4k_batch4_supported(format, x_dtype, m, n_out, n_in);
   if (b4 && m <= batch4_max)

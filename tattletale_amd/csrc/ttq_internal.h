@@ -73,6 +73,13 @@ hipError_t launch_gemv_q4k_slice(const void* w, const void* x, int x_dtype, void
                                  const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                                  hipStream_t s);
 
+// The streamed kernel for two to four activation rows (ttq_gemv_q4k_stream4.hip): the tokens share the matrix
+// instructions of a super-block; n_in 2048 or 4096, at least 16 rows per compute unit.
+bool gemv_q4k_stream4_supported(int format, int x_dtype, int64_t m, int64_t n_out, int64_t n_in);
+hipError_t launch_gemv_q4k_stream4(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                                   const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                                   hipStream_t s);
+
 // Q8_0 through the int8 matrix cores with the raw bytes of the rows as the K dimension, streamed through three LDS
 // buffers (ttq_gemv_q8_stream.hip): n_in a multiple of 2048 up to 8192 (4096 for fp32 activations), whole groups of
 // 16 rows, at least one per compute unit.
