@@ -248,6 +248,10 @@ int ttq_gemv_q4_k_silu_mul(const void* w, const void* x, int x_dtype, void* y, i
   if (m == 0 || n_ff == 0) return TTQ_OK;
   if (!w || !x || !y) return TTQ_ERR_NULL;
   if (!aligned16(w) || !aligned16(x) || !aligned16(y)) return TTQ_ERR_ALIGN;
+  // two to four rows: one pass over the weights for all of them
+  if (ttq::gemv_q4k_stream4_fused_supported(x_dtype, m, n_ff, n_in))
+    return hip_status(ttq::launch_gemv_q4k_stream4_fused(w, x, x_dtype, y, y_dtype, m, n_ff, n_in,
+                                                         static_cast<hipStream_t>(stream)));
   if (m <= 4 && ttq::gemv_q4k_stream_fused_supported(x_dtype, n_ff, n_in))
     return hip_status(ttq::launch_gemv_q4k_stream_fused(w, x, x_dtype, y, y_dtype, m, n_ff, n_in,
                                                         static_cast<hipStream_t>(stream)));

@@ -46,7 +46,12 @@ static_assert(2 * kS4XLine0 >= kS4Up + 2, "the landing slots are beyond the requ
 static_assert(kS4Up / 2 - kS4RingLines <= -2, "a top-up never overwrites a line that is still to be read");
 constexpr int s4_slot(int line) { return line % kS4RingLines; }
 
-template <typename XT, typename YT>
+// FUSE: the weight holds gate rows [0, n_out) followed by up rows [n_out, 2 n_out), as GatedMLP builds it
+// (workspace/transformers/src/layers/mlp.nim:39), and the kernel writes silu(gate . x) * (up . x), the silu_and_mul
+// of workspace/transformers/src/kernels/activations.nim:14-38: a workgroup takes the gate row groups of its
+// outputs, then the up row groups of the same outputs, and pairs their sums at the end.  n_out and rows_per_wg
+// count outputs.
+template <typename XT, typename YT, bool FUSE>
 __global__ void __launch_bounds__(kS4Threads)
 gemv_q4k_stream4_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
                         const void* __restrict__ bias, int bias_dtype, int m, int n_out, int nsb, int rows_per_wg) {
@@ -65,7 +70,7 @@ gemv_q4k_stream4_kernel(const uint8_t* __restrict__ w, const uint16_t* __restric
   const int wg_row_end = min(wg_row0 + rows_per_wg, n_out);
   const int last = wg_row_end - 1;
   const int ngroups = (wg_row_end - wg_row0 + 15) >> 4;
-  const int nblocks = ngroups << nks_log2;                // <= kS4MaxBlocks (the launcher sees to it)
+  const int nblocks = ((FUSE ? 2 : 1) * ngroups) << nks_log2;   // <= kS4MaxBlocks (the launcher sees to it)
   uint8_t* mybuf = wbuf + wave * kS4BufBytes;
   const int zero_entry = kS4Tok * kS4MaxSb * 32;
 
@@ -91,7 +96,14 @@ gemv_q4k_stream4_kernel(const uint8_t* __restrict__ w, const uint16_t* __restric
 #pragma unroll
     for (int o = 0; o < 2; o++) {
       const int row16 = 8 * o + r8;
-      const int row = min(wg_row0 + rg * 16 + row16, last);          // past the end: the last row again, never used
+      // past the end: the last row again, never used
+      int row;
+      if (FUSE) {
+        const int up = rg >= ngroups ? 1 : 0;
+        row = up * n_out + min(wg_row0 + (rg - up * ngroups) * 16 + row16, last);
+      } else {
+        row = min(wg_row0 + rg * 16 + row16, last);
+      }
       lane_off[o] = (uint32_t)row * rb + (uint32_t)(ks * kStSegBytes) + (uint32_t)(((lane & 7) ^ ((row16 >> 1) & 7)) * 16);
     }
   };
@@ -335,40 +347,49 @@ gemv_q4k_stream4_kernel(const uint8_t* __restrict__ w, const uint16_t* __restric
     float v = part[grp << nks_log2][tok * 16 + nn];
     if (nks_log2) v += part[(grp << 1) + 1][tok * 16 + nn];
     const int row = wg_row0 + r;
-    if (row < wg_row_end) YElem<YT>::store(y, (int64_t)tok * n_out + row, v + load_bias(bias, bias_dtype, row));
+    if (FUSE) {
+      float u = part[(ngroups + grp) << nks_log2][tok * 16 + nn];
+      if (nks_log2) u += part[((ngroups + grp) << 1) + 1][tok * 16 + nn];
+      if (row < wg_row_end) YElem<YT>::store(y, (int64_t)tok * n_out + row, (v / (1.f + expf(-v))) * u);
+    } else {
+      if (row < wg_row_end) YElem<YT>::store(y, (int64_t)tok * n_out + row, v + load_bias(bias, bias_dtype, row));
+    }
   }
 }
 
 struct S4Plan { bool ok; int num_wg, rows_per_wg; };
 
-S4Plan s4_plan(int64_t m, int64_t n_out, int64_t n_in) {
+// n_out counts outputs; a fused launch has twice as many weight rows and blocks
+S4Plan s4_plan(int64_t m, int64_t n_out, int64_t n_in, bool fuse) {
   S4Plan p{};
+  const int64_t parts = fuse ? 2 : 1;
   if (m < 2 || m > kS4Tok || (n_in != 4096 && n_in != 2048)) return p;
-  if (n_out < 16 * (int64_t)device_num_cus() || n_out * (n_in / 256) * 144 >= ((int64_t)1 << 32)) return p;
+  if (parts * n_out < 16 * (int64_t)device_num_cus() || parts * n_out * (n_in / 256) * 144 >= ((int64_t)1 << 32)) return p;
+  if (fuse && n_out % 8 != 0) return p;
   p.rows_per_wg = st_rows_per_wg(n_out, &p.num_wg);
-  if (((p.rows_per_wg + 15) / 16) * (n_in / 2048) > kS4MaxBlocks) return p;
+  if (parts * ((p.rows_per_wg + 15) / 16) * (n_in / 2048) > kS4MaxBlocks) return p;
   p.ok = true;
   return p;
 }
 
-template <typename XT, typename YT>
+template <typename XT, typename YT, bool FUSE>
 hipError_t s4_launch_xy(const void* w, const void* x, void* y, const void* bias, int bias_dtype, int64_t m,
                         int64_t n_out, int64_t n_in, hipStream_t s) {
-  const S4Plan p = s4_plan(m, n_out, n_in);
+  const S4Plan p = s4_plan(m, n_out, n_in, FUSE);
   if (!p.ok) return hipErrorInvalidValue;
-  hipLaunchKernelGGL((gemv_q4k_stream4_kernel<XT, YT>), dim3((unsigned)p.num_wg), dim3(kS4Threads), 0, s,
+  hipLaunchKernelGGL((gemv_q4k_stream4_kernel<XT, YT, FUSE>), dim3((unsigned)p.num_wg), dim3(kS4Threads), 0, s,
                      static_cast<const uint8_t*>(w), static_cast<const uint16_t*>(x), static_cast<YT*>(y), bias,
                      bias_dtype, (int)m, (int)n_out, (int)(n_in / 256), p.rows_per_wg);
   return hipGetLastError();
 }
 
-template <typename XT>
+template <typename XT, bool FUSE>
 hipError_t s4_launch_x(const void* w, const void* x, void* y, int y_dtype, const void* bias, int bias_dtype,
                        int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
   switch (y_dtype) {
-    case kF32: return s4_launch_xy<XT, float>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
-    case kF16: return s4_launch_xy<XT, f16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
-    case kBF16: return s4_launch_xy<XT, bf16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kF32: return s4_launch_xy<XT, float, FUSE>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kF16: return s4_launch_xy<XT, f16_tag, FUSE>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kBF16: return s4_launch_xy<XT, bf16_tag, FUSE>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
     default: return hipErrorInvalidValue;
   }
 }
@@ -378,13 +399,26 @@ hipError_t s4_launch_x(const void* w, const void* x, void* y, int y_dtype, const
 bool gemv_q4k_stream4_supported(int format, int x_dtype, int64_t m, int64_t n_out, int64_t n_in) {
   static const int disabled = dev_knob("TTQ_GEMV_NO_STREAM4", 0);
   if (disabled || format != kQ4_K || !(x_dtype == kBF16 || x_dtype == kF16)) return false;
-  return s4_plan(m, n_out, n_in).ok;
+  return s4_plan(m, n_out, n_in, false).ok;
 }
 
 hipError_t launch_gemv_q4k_stream4(const void* w, const void* x, int x_dtype, void* y, int y_dtype, const void* bias,
                                    int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
-  if (x_dtype == kBF16) return s4_launch_x<bf16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-  if (x_dtype == kF16) return s4_launch_x<f16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  if (x_dtype == kBF16) return s4_launch_x<bf16_tag, false>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  if (x_dtype == kF16) return s4_launch_x<f16_tag, false>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  return hipErrorInvalidValue;
+}
+
+// The gate || up form: n_ff outputs from 2 n_ff weight rows, two to four activation rows.
+bool gemv_q4k_stream4_fused_supported(int x_dtype, int64_t m, int64_t n_ff, int64_t n_in) {
+  if (!(x_dtype == kBF16 || x_dtype == kF16)) return false;
+  return s4_plan(m, n_ff, n_in, true).ok;
+}
+
+hipError_t launch_gemv_q4k_stream4_fused(const void* w, const void* x, int x_dtype, void* y, int y_dtype, int64_t m,
+                                         int64_t n_ff, int64_t n_in, hipStream_t s) {
+  if (x_dtype == kBF16) return s4_launch_x<bf16_tag, true>(w, x, y, y_dtype, nullptr, 0, m, n_ff, n_in, s);
+  if (x_dtype == kF16) return s4_launch_x<f16_tag, true>(w, x, y, y_dtype, nullptr, 0, m, n_ff, n_in, s);
   return hipErrorInvalidValue;
 }
 

@@ -79,6 +79,10 @@ bool gemv_q4k_stream4_supported(int format, int x_dtype, int64_t m, int64_t n_ou
 hipError_t launch_gemv_q4k_stream4(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
                                    const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                                    hipStream_t s);
+// gate || up + silu_and_mul on the same kernel: n_ff outputs from 2 n_ff weight rows
+bool gemv_q4k_stream4_fused_supported(int x_dtype, int64_t m, int64_t n_ff, int64_t n_in);
+hipError_t launch_gemv_q4k_stream4_fused(const void* w, const void* x, int x_dtype, void* y, int y_dtype, int64_t m,
+                                         int64_t n_ff, int64_t n_in, hipStream_t s);
 
 // Q8_0 through the int8 matrix cores with the raw bytes of the rows as the K dimension, streamed through three LDS
 // buffers (ttq_gemv_q8_stream.hip): n_in a multiple of 2048 up to 8192 (4096 for fp32 activations), whole groups of

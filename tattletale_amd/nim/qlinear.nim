@@ -162,7 +162,10 @@ proc forward*(self: QuantGatedMLP, x: TorchTensor): TorchTensor =
   let gu = self.gate_up_proj
   let nff = self.down_proj.in_features
   let m = x.numel() div gu.in_features
-  if gu.format == kQ4_K and gu.bias.isNone and m == 1:
+  # one row, or two to four rows on the shapes whose fused kernel reads the weights once for all of them
+  let few = m >= 2 and m <= 4 and (gu.in_features == 2048 or gu.in_features == 4096) and nff mod 8 == 0 and
+            nff >= 2048 and nff <= 16384
+  if gu.format == kQ4_K and gu.bias.isNone and (m == 1 or few):
     var shape = x.sizes().asNimView().toSeq()
     shape[^1] = nff
     let act = F.empty(shape, x.options())

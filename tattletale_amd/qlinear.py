@@ -406,15 +406,18 @@ class QuantGatedMLP:
     FUSED_FEW_ROWS = (17, 64)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        """x (..., hidden) -> (..., hidden)  (mlp.nim:43-60).  On Q4_K weights a single-token 16-bit
-        activation takes the fused GEMV + silu_and_mul kernel and a bf16 activation of 17 to 64 or at least
+        """x (..., hidden) -> (..., hidden)  (mlp.nim:43-60).  On Q4_K weights a 16-bit activation of one to
+        four tokens takes the fused GEMV + silu_and_mul kernel and a bf16 activation of 17 to 64 or at least
         ``FUSED_GEMM_MIN_ROWS`` rows the GEMM with silu_and_mul in its epilogue; everything else runs
         the projection, ``silu_and_mul`` and the down projection as three launches."""
         gu = self.gate_up_proj
         n_ff = self.down_proj.in_features
         m = x.numel() // gu.in_features
         act = None
-        if gu.format == _lib.Q4_K and gu.bias is None and m == 1 and x.dtype in (torch.bfloat16, torch.float16):
+        # one row, or two to four rows on the shapes whose fused kernel reads the weights once for all of them
+        # (rows of 2048 or 4096 values, 2 * n_ff from 4096 to 32768 weight rows)
+        few = 2 <= m <= 4 and gu.in_features in (2048, 4096) and n_ff % 8 == 0 and 2048 <= n_ff <= 16384
+        if gu.format == _lib.Q4_K and gu.bias is None and (m == 1 or few) and x.dtype in (torch.bfloat16, torch.float16):
             try:
                 act = gemv_q4_k_silu_mul(gu.qweight, x.reshape(m, gu.in_features), n_ff, gu.in_features,
                                          out_dtype=x.dtype).reshape(x.shape[:-1] + (n_ff,))

@@ -58,6 +58,30 @@ def test_fused_gate_up_silu_mul_gemv(xk, n_ff, n_in):
     assert rel_l2(y, sep) <= 2e-4
 
 
+@pytest.mark.parametrize("xk", ["bf16", "f16"])
+@pytest.mark.parametrize("m", [2, 3, 4])
+@pytest.mark.parametrize("n_ff,n_in", [(14336, 4096), (2048 + 8, 4096), (8192 + 16 * 5, 2048)])
+def test_fused_gate_up_silu_mul_two_to_four_rows(xk, m, n_ff, n_in):
+    """One pass over the weights for all rows (tokens share the matrix instructions): sampled outputs of every
+    row against the oracle, another magnitude per row; the whole result against the two separate kernels."""
+    rng = np.random.default_rng(n_ff + m)
+    p = random_blocks(F.Q4_K, 2 * n_ff * (n_in // 256), seed=n_ff + m)
+    outs = np.unique(np.concatenate([rng.integers(0, n_ff, 300), np.arange(n_ff - 40, n_ff), np.arange(40)]))
+    rows = np.concatenate([outs, n_ff + outs])
+    what = oracle.dequant(F.Q4_K, np.ascontiguousarray(p.reshape(2 * n_ff, -1)[rows]), rows.size, n_in)
+    x = Q.fill_normal(n_in + m, 1, 1.0, m * n_in).reshape(m, n_in) * np.float32(0.03)
+    for t in range(m):
+        x[t] *= (1.0, 0.1, 2.0, 0.5)[t]
+    xd, xf = x_to_dev(x, xk)
+    y = QL.gemv_q4_k_silu_mul(packed_to_dev(p), xd, n_ff, n_in).cpu().numpy()
+    assert y.shape == (m, n_ff) and np.all(np.isfinite(y))
+    want = oracle.silu_and_mul_f64(oracle.linear_f64(what, xf))
+    for r in range(m):
+        assert rel_l2(y[r][outs], want[r]) <= 1e-3, r
+    sep = QL.silu_and_mul(QL.gemv(F.Q4_K, packed_to_dev(p), xd, 2 * n_ff, n_in)).cpu().numpy()
+    assert rel_l2(y, sep) <= 2e-4
+
+
 def test_fused_gemv_output_dtypes_and_refusals():
     n_ff, n_in = 256, 1024
     p = random_blocks(F.Q4_K, 2 * n_ff * (n_in // 256), seed=3)
@@ -94,6 +118,31 @@ def test_gated_mlp_forward(shape):
     want = oracle.linear_f64(wdd, act16)
     got = oracle.bf16_to_f32(dev_bits(y)).reshape(-1, hidden)
     assert rel_l2(got, want) <= 2e-2
+
+
+@pytest.mark.parametrize("m", [2, 3, 4])
+def test_gated_mlp_forward_two_to_four_tokens(m):
+    """hidden 2048, intermediate 2048: the gate||up projection of two to four tokens is one launch of the fused
+    kernel that reads the weights once for all of them."""
+    hidden, inter = 2048, 2048
+    wg = Q.fill_normal(170, 0, 0.03, inter * hidden).reshape(inter, hidden)
+    wu = Q.fill_normal(171, 0, 0.03, inter * hidden).reshape(inter, hidden)
+    wd = Q.fill_normal(172, 0, 0.03, hidden * inter).reshape(hidden, inter)
+    pgu = np.concatenate([Q.quantize(F.Q4_K, wg), Q.quantize(F.Q4_K, wu)])
+    pd = Q.quantize(F.Q4_K, wd)
+    mlp = QuantGatedMLP.init(QuantLinear.init(packed_to_dev(pgu), F.Q4_K, hidden, 2 * inter),
+                             QuantLinear.init(packed_to_dev(pd), F.Q4_K, inter, hidden))
+    xd, xf = x_to_dev(Q.fill_normal(173, 1, 1.0, m * hidden).reshape(m, hidden), "bf16")
+    y = mlp.forward(xd)
+    assert y.shape == (m, hidden) and y.dtype == torch.bfloat16
+    wgu = oracle.dequant(F.Q4_K, pgu, 2 * inter, hidden)
+    wdd = oracle.dequant(F.Q4_K, pd, hidden, inter)
+    act = oracle.silu_and_mul_f64(oracle.linear_f64(wgu, xf))
+    act16 = oracle.bf16_to_f32(oracle.f32_to_bf16(act.astype(np.float32)))
+    want = oracle.linear_f64(wdd, act16)
+    got = oracle.bf16_to_f32(dev_bits(y))
+    for r in range(m):
+        assert rel_l2(got[r], want[r]) <= 2e-2, r
 
 
 def test_gated_mlp_rejects_mismatched_layers():
@@ -205,10 +254,11 @@ def test_fused_rmsnorm_gemv(xk, n_out, n_in, silu, with_residual):
     else:
         assert new_res is None
     # the same GEMV kernel on the row this kernel reported: identical arithmetic, identical bits
+    # (row by row: several rows in one call take the few-row kernels, which add in another order)
     if silu:
-        y_ref = QL.gemv_q4_k_silu_mul(packed_to_dev(p), normed, n_out, n_in)
+        y_ref = torch.cat([QL.gemv_q4_k_silu_mul(packed_to_dev(p), normed[r:r + 1], n_out, n_in)
+                           for r in range(normed.shape[0])])
     else:
-        # row by row: several rows in one call take the few-row kernel, which adds in another order
         y_ref = torch.cat([QL.gemv(F.Q4_K, packed_to_dev(p), normed[r:r + 1], n_out, n_in)
                            for r in range(normed.shape[0])])
     if n_out >= 2048 or silu:
