@@ -248,10 +248,23 @@ int ttq_gemv_q4_k_silu_mul(const void* w, const void* x, int x_dtype, void* y, i
   if (m == 0 || n_ff == 0) return TTQ_OK;
   if (!w || !x || !y) return TTQ_ERR_NULL;
   if (!aligned16(w) || !aligned16(x) || !aligned16(y)) return TTQ_ERR_ALIGN;
-  // two to four rows: one pass over the weights for all of them
-  if (ttq::gemv_q4k_stream4_fused_supported(x_dtype, m, n_ff, n_in))
-    return hip_status(ttq::launch_gemv_q4k_stream4_fused(w, x, x_dtype, y, y_dtype, m, n_ff, n_in,
-                                                         static_cast<hipStream_t>(stream)));
+  // two to four rows: one pass over the weights for all of them; more rows: four at a time
+  if (m >= 2 && ttq::gemv_q4k_stream4_fused_supported(x_dtype, m < 4 ? m : 4, n_ff, n_in) &&
+      ttq::gemv_q4k_stream_fused_supported(x_dtype, n_ff, n_in)) {
+    const char* xb = static_cast<const char*>(x);
+    char* yb = static_cast<char*>(y);
+    for (int64_t r0 = 0; r0 < m; r0 += 4) {
+      const int64_t rows = m - r0 < 4 ? m - r0 : 4;
+      const void* xr = xb + r0 * n_in * dtype_size(x_dtype);
+      void* yr = yb + r0 * n_ff * dtype_size(y_dtype);
+      const hipError_t e = rows >= 2 ? ttq::launch_gemv_q4k_stream4_fused(w, xr, x_dtype, yr, y_dtype, rows, n_ff, n_in,
+                                                                          static_cast<hipStream_t>(stream))
+                                     : ttq::launch_gemv_q4k_stream_fused(w, xr, x_dtype, yr, y_dtype, rows, n_ff, n_in,
+                                                                         static_cast<hipStream_t>(stream));
+      if (e != hipSuccess) return hip_status(e);
+    }
+    return TTQ_OK;
+  }
   if (m <= 4 && ttq::gemv_q4k_stream_fused_supported(x_dtype, n_ff, n_in))
     return hip_status(ttq::launch_gemv_q4k_stream_fused(w, x, x_dtype, y, y_dtype, m, n_ff, n_in,
                                                         static_cast<hipStream_t>(stream)));

@@ -59,7 +59,7 @@ def test_fused_gate_up_silu_mul_gemv(xk, n_ff, n_in):
 
 
 @pytest.mark.parametrize("xk", ["bf16", "f16"])
-@pytest.mark.parametrize("m", [2, 3, 4])
+@pytest.mark.parametrize("m", [2, 3, 4, 5, 9])
 @pytest.mark.parametrize("n_ff,n_in", [(14336, 4096), (2048 + 8, 4096), (8192 + 16 * 5, 2048)])
 def test_fused_gate_up_silu_mul_two_to_four_rows(xk, m, n_ff, n_in):
     """One pass over the weights for all rows (tokens share the matrix instructions): sampled outputs of every
@@ -71,9 +71,9 @@ def test_fused_gate_up_silu_mul_two_to_four_rows(xk, m, n_ff, n_in):
     what = oracle.dequant(F.Q4_K, np.ascontiguousarray(p.reshape(2 * n_ff, -1)[rows]), rows.size, n_in)
     x = Q.fill_normal(n_in + m, 1, 1.0, m * n_in).reshape(m, n_in) * np.float32(0.03)
     for t in range(m):
-        x[t] *= (1.0, 0.1, 2.0, 0.5)[t]
+        x[t] *= (1.0, 0.1, 2.0, 0.5)[t % 4]
     xd, xf = x_to_dev(x, xk)
-    y = QL.gemv_q4_k_silu_mul(packed_to_dev(p), xd, n_ff, n_in).cpu().numpy()
+    y = QL.gemv_q4_k_silu_mul(packed_to_dev(p), xd, n_ff, n_in).cpu().numpy()      # more than four rows: four at a time
     assert y.shape == (m, n_ff) and np.all(np.isfinite(y))
     want = oracle.silu_and_mul_f64(oracle.linear_f64(what, xf))
     for r in range(m):
