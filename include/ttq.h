@@ -236,7 +236,11 @@ TTQ_API int ttq_rmsnorm(const void* x, const void* residual, const void* gamma, 
  * GEMV.  With silu_mul != 0 the weight is the (2*n_out, n_in) gate/up matrix and y is
  * silu_and_mul of the projection (mlp.nim:56-59).  residual, new_residual_out and normed_out
  * may be NULL; normed_out receives the normalized row the GEMV consumed (other projections of
- * the same block read it).  Returns TTQ_ERR_UNSUPPORTED for fp32 activations or n_out < 16.
+ * the same block read it).  With two to four rows, normed_out given and a large matrix (rows of 2048 or
+ * 4096 values, 4096 weight rows or more) the call is two launches -- the normalization, then one pass
+ * over the weights for all rows -- which is faster than one weight pass per row; the results are those of
+ * ttq_rmsnorm followed by ttq_gemv_q4_k / ttq_gemv_q4_k_silu_mul on normed_out.
+ * Returns TTQ_ERR_UNSUPPORTED for fp32 activations or n_out < 16.
  * Out of place only: every workgroup re-reads x and residual while the outputs are written, so
  * new_residual_out and normed_out must not overlap x, residual or each other (TTQ_ERR_ALIAS);
  * use ttq_rmsnorm for the in-place form. */

@@ -307,6 +307,18 @@ int ttq_gemv_q4_k_rmsnorm(const void* w, const void* x, const void* residual, co
         overlaps(normed_out, nb, new_residual_out, nb))
       return TTQ_ERR_ALIAS;
   }
+  // two to four rows: the normalization as a launch of its own (it writes the rows the caller asked for anyway),
+  // then one pass over the weights for all rows -- the one-launch form below reads the weights once per row
+  if (m >= 2 && m <= 4 && normed_out &&
+      (silu_mul ? ttq::gemv_q4k_stream4_fused_supported(x_dtype, m, n_out, n_in)
+                : ttq::gemv_q4k_stream4_supported(TTQ_Q4_K, x_dtype, m, n_out, n_in))) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t e = ttq::launch_rmsnorm(x, residual, gamma, eps, x_dtype, new_residual_out, normed_out, m, n_in, s);
+    if (e != hipSuccess) return hip_status(e);
+    e = silu_mul ? ttq::launch_gemv_q4k_stream4_fused(w, normed_out, x_dtype, y, y_dtype, m, n_out, n_in, s)
+                 : ttq::launch_gemv_q4k_stream4(w, normed_out, x_dtype, y, y_dtype, nullptr, 0, m, n_out, n_in, s);
+    return hip_status(e);
+  }
   if (m <= 4 && (silu_mul ? ttq::gemv_q4k_stream_fused_supported(x_dtype, n_out, n_in)
                           : ttq::gemv_q4k_stream_supported(TTQ_Q4_K, x_dtype, n_out, n_in)))
     return hip_status(ttq::launch_gemv_q4k_stream_norm(w, x, x_dtype, y, y_dtype, m, n_out, n_in, silu_mul != 0, residual,

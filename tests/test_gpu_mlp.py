@@ -253,14 +253,19 @@ def test_fused_rmsnorm_gemv(xk, n_out, n_in, silu, with_residual):
         assert torch.equal(new_res, new_res_ref)
     else:
         assert new_res is None
-    # the same GEMV kernel on the row this kernel reported: identical arithmetic, identical bits
-    # (row by row: several rows in one call take the few-row kernels, which add in another order)
+    # the same GEMV kernel on the rows this call reported: identical arithmetic, identical bits.  Where the
+    # multi-row streamed kernel exists (rows of 2048 / 4096 values, 4096 weight rows or more) the call is the
+    # normalization followed by that kernel on both rows; elsewhere it is one kernel with the single-row
+    # arithmetic (several rows in one plain call would take the few-row kernels, which add in another order)
+    multi = n_in in (2048, 4096) and rows >= 4096 and (not silu or n_out % 8 == 0)
     if silu:
-        y_ref = torch.cat([QL.gemv_q4_k_silu_mul(packed_to_dev(p), normed[r:r + 1], n_out, n_in)
-                           for r in range(normed.shape[0])])
+        y_ref = (QL.gemv_q4_k_silu_mul(packed_to_dev(p), normed, n_out, n_in) if multi else
+                 torch.cat([QL.gemv_q4_k_silu_mul(packed_to_dev(p), normed[r:r + 1], n_out, n_in)
+                            for r in range(normed.shape[0])]))
     else:
-        y_ref = torch.cat([QL.gemv(F.Q4_K, packed_to_dev(p), normed[r:r + 1], n_out, n_in)
-                           for r in range(normed.shape[0])])
+        y_ref = (QL.gemv(F.Q4_K, packed_to_dev(p), normed, n_out, n_in) if multi else
+                 torch.cat([QL.gemv(F.Q4_K, packed_to_dev(p), normed[r:r + 1], n_out, n_in)
+                            for r in range(normed.shape[0])]))
     if n_out >= 2048 or silu:
         assert torch.equal(y, y_ref)
     # and against the oracle on a sample of outputs
