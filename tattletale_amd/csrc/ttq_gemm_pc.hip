@@ -165,26 +165,38 @@ template <> struct WFmt<kQ6_K> {
 
 // Q8_0: eight 34-byte blocks { d, q[32] } per 256 k; step C is blocks 2C and 2C+1.  Here a thread
 // takes the whole block 2C + whalf of every step (kWholeKsub: its 32 weights are k = 32*whalf + e,
-// `lo` the first 16, `hi` the last 16): one scale and three loads per block.
+// `lo` the first 16, `hi` the last 16): one scale per block.  Block i starts 34 i = 32 i + 2 i bytes into the
+// 272-byte unit, i.e. 2 i bytes into an aligned 16-byte chunk: the thread loads the three aligned chunks that
+// hold its block (loads at 2-byte alignment are served several times slower: the Q8_0 GEMM spent twice the
+// cycles of the Q4_K one waiting, with the same instruction counts) and shifts the bytes into place when it
+// dequantizes.
 template <> struct WFmt<kQ8_0> {
   static constexpr int kUnitBytes = 8 * 34;
   static constexpr bool kWholeKsub = true;
-  struct Raw { uint4 q[8]; uint32_t d[4]; };
+  struct Raw { uint4 ch[4][3]; };
   static __device__ __forceinline__ void load(Raw& dst, const uint8_t* p, int whalf) {
 #pragma unroll
     for (int c = 0; c < 4; c++) {
-      const uint8_t* blk = p + 34 * (2 * c + whalf);
-      dst.d[c] = load2(blk);
-      dst.q[2 * c] = load16_a2(blk + 2);
-      dst.q[2 * c + 1] = load16_a2(blk + 18);
+      const uint8_t* a = p + 32 * (2 * c + whalf);
+      dst.ch[c][0] = load16_a16(a);
+      dst.ch[c][1] = load16_a16(a + 16);
+      dst.ch[c][2] = load16_a16(a + 32);
     }
   }
   template <int C>
-  static __device__ __forceinline__ void dequant(const Raw& r, int, uint32_t (&lo)[8], uint32_t (&hi)[8]) {
-    const float d = f16_bits_to_f32((uint16_t)r.d[C]);
+  static __device__ __forceinline__ void dequant(const Raw& r, int whalf, uint32_t (&lo)[8], uint32_t (&hi)[8]) {
+    // the block starts 4 C + 2 whalf bytes into the three chunks
+    const uint32_t D[12] = {r.ch[C][0].x, r.ch[C][0].y, r.ch[C][0].z, r.ch[C][0].w, r.ch[C][1].x, r.ch[C][1].y,
+                            r.ch[C][1].z, r.ch[C][1].w, r.ch[C][2].x, r.ch[C][2].y, r.ch[C][2].z, r.ch[C][2].w};
+    const bool odd = whalf != 0;
+    const float d = f16_bits_to_f32((uint16_t)(odd ? D[C] >> 16 : D[C] & 0xFFFFu));
     const float md = -128.f * d;
-    const uint32_t a4[4] = {r.q[2 * C].x, r.q[2 * C].y, r.q[2 * C].z, r.q[2 * C].w};
-    const uint32_t b4[4] = {r.q[2 * C + 1].x, r.q[2 * C + 1].y, r.q[2 * C + 1].z, r.q[2 * C + 1].w};
+    uint32_t a4[4], b4[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      a4[j] = odd ? D[C + 1 + j] : __builtin_amdgcn_alignbyte(D[C + 1 + j], D[C + j], 2);
+      b4[j] = odd ? D[C + 5 + j] : __builtin_amdgcn_alignbyte(D[C + 5 + j], D[C + 4 + j], 2);
+    }
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       // q + 128 as an unsigned byte converts in one instruction; d * (u - 128) as one fused
