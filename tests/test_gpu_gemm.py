@@ -101,6 +101,22 @@ def test_gemm_split_along_k_identity_activations_give_bf16_weights_exactly(fmt):
     assert not (y[n_in:] & 0x7FFF).any()
 
 
+def test_split_launches_of_both_kernels_share_their_counters():
+    """The tiled and the few-row kernel keep their arrival counters in the same per-stream buffer and both leave
+    them at zero: calls of the two kinds, interleaved on one stream, reproduce their first results bit for bit."""
+    shapes = [(300, 1000, 2048), (64, 4096, 14336), (256, 1024, 4096), (32, 1024, 8192), (130, 2048, 14336)]
+    calls = []
+    for i, (m, n_out, n_in) in enumerate(shapes):
+        p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=950 + i)
+        xd, _ = x_to_dev(Q.fill_normal(960 + i, 1, 1.0, m * n_in).reshape(m, n_in), "bf16")
+        calls.append((packed_to_dev(p), xd, n_out, n_in))
+    first = [dev_bits(QL.gemm(F.Q4_K, *c)) for c in calls]
+    for order in ([4, 1, 0, 3, 2], [1, 1, 3, 3, 0, 4, 2]):
+        for i in order:
+            assert np.array_equal(dev_bits(QL.gemm(F.Q4_K, *calls[i])), first[i]), i
+    torch.cuda.synchronize()
+
+
 def test_forward_split_along_k_f32_output_with_bias():
     n_out, n_in, m = 1024 + 24, 4096, 200
     w = Q.fill_normal(710, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
