@@ -1,6 +1,7 @@
 // Device workspaces the library keeps for the paths that need one, one per (slot, device, stream): launches
 // on one stream run in order and can share a buffer; launches on different streams may overlap and get their
-// own.  Grown on demand and kept until the process ends.  Also here: the activation-type conversion that lets
+// own.  Grown on demand (by at least a factor of two; outgrown buffers stay allocated, because launches in
+// flight and captured graphs may still name them) and kept until the process ends.  Also here: the activation-type conversion that lets
 // fp16 and fp32 activations use the bf16 matrix-core GEMM.
 #include "ttq_device.h"
 #include "ttq_internal.h"
@@ -24,27 +25,29 @@ hipError_t stream_workspace(int slot, hipStream_t s, size_t bytes, void** out, b
   std::lock_guard<std::mutex> lock(g_mutex);
   Buf& b = g_bufs[key];
   if (b.bytes < bytes) {
-    if (b.p) {
-      // earlier launches on the stream may still use the old buffer
-      e = hipStreamSynchronize(s);
-      if (e != hipSuccess) return e;
-      (void)hipFree(b.p);
-      b.p = nullptr;
-      b.bytes = 0;
-    }
+    // A buffer that has become too small is kept, not freed: launches still in flight on the stream use it, and
+    // so does every HIP graph that was captured while it was current.  Growing by at least a factor of two
+    // bounds what the retired buffers hold to the size of the current one.
+    const size_t want = bytes > 2 * b.bytes ? bytes : 2 * b.bytes;
+    size_t got = want;
     void* p = nullptr;
-    e = hipMalloc(&p, bytes);
+    e = hipMalloc(&p, want);
+    if (e != hipSuccess && want > bytes) {        // no room for the spare half
+      (void)hipGetLastError();
+      got = bytes;
+      e = hipMalloc(&p, bytes);
+    }
     if (e != hipSuccess) return e;
     if (zeroed) {
       // ordered before every launch that will use the buffer: they are all on this stream
-      e = hipMemsetAsync(p, 0, bytes, s);
+      e = hipMemsetAsync(p, 0, got, s);
       if (e != hipSuccess) {
         (void)hipFree(p);
         return e;
       }
     }
     b.p = p;
-    b.bytes = bytes;
+    b.bytes = got;
   }
   *out = b.p;
   return hipSuccess;

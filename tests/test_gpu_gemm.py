@@ -117,6 +117,35 @@ def test_split_launches_of_both_kernels_share_their_counters():
     torch.cuda.synchronize()
 
 
+def test_split_launch_in_a_graph_survives_a_growing_workspace():
+    """A HIP graph of a split launch keeps naming the workspace that was current when it was captured; a later,
+    larger split launch on the same stream replaces that workspace without freeing it.  Replays, with eager
+    launches of both shapes in between, reproduce the eager result."""
+    small, big = (256, 1024, 4096), (512, 4096, 14336)
+    args = []
+    for i, (m, n_out, n_in) in enumerate((small, big)):
+        p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=970 + i)
+        xd, _ = x_to_dev(Q.fill_normal(980 + i, 1, 1.0, m * n_in).reshape(m, n_in), "bf16")
+        args.append((packed_to_dev(p), xd, n_out, n_in))
+    side = torch.cuda.Stream(DEV)
+    out = torch.empty((small[0], small[1]), dtype=torch.bfloat16, device=DEV)
+    with torch.cuda.stream(side):
+        want_small = dev_bits(QL.gemm(F.Q4_K, *args[0]))          # eager: allocates this stream's workspace
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            QL.gemm(F.Q4_K, *args[0], out=out)
+        torch.cuda.synchronize()
+        want_big = dev_bits(QL.gemm(F.Q4_K, *args[1]))            # grows the workspace of the same stream
+        for _ in range(3):
+            out.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert np.array_equal(dev_bits(out), want_small)
+            assert np.array_equal(dev_bits(QL.gemm(F.Q4_K, *args[1])), want_big)
+            assert np.array_equal(dev_bits(QL.gemm(F.Q4_K, *args[0])), want_small)
+    torch.cuda.synchronize()
+
+
 def test_forward_split_along_k_f32_output_with_bias():
     n_out, n_in, m = 1024 + 24, 4096, 200
     w = Q.fill_normal(710, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
