@@ -26,6 +26,7 @@ SOURCES = [
     "ttq_gemv_q4k_slice.hip",
     "ttq_gemv_q4k_stream4.hip",
     "ttq_gemv_q6k_stream.hip",
+    "ttq_gemv_q6k_stream4.hip",
     "ttq_gemv_q8_stream.hip",
     "ttq_gemv_q8_mfma.hip",
     "ttq_gemv_q8_win.hip",

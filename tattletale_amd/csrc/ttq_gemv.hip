@@ -335,6 +335,8 @@ hipError_t launch_gemv(int format, const void* w, const void* x, int x_dtype, vo
   if (gemv_q4k_batch_supported(format, x_dtype, m, n_out, n_in))
     return launch_gemv_q4k_batch(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   if (b4) return launch_gemv_q4k_batch4(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  if (gemv_q6k_stream4_supported(format, x_dtype, m, n_out, n_in))
+    return launch_gemv_q6k_stream4(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   if (gemv_dot2_multi_supported(format, x_dtype, m, n_in))
     return launch_gemv_dot2_multi(format, w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   if (gemv_q4k_stream_supported(format, x_dtype, n_out, n_in))
@@ -377,6 +379,12 @@ float gemv_estimate_us(int format, int x_dtype, int64_t m, int64_t n_out, int64_
     return (float)((m + tok - 1) / tok) * (tok == 16 ? mb / 2.7f + 7.5f : mb / 3.9f + 5.5f);
   }
   if (b4) return (float)((m + 3) / 4) * (mb / 2.4f + 2.f);
+  if (gemv_q6k_stream4_supported(format, x_dtype, m, n_out, n_in)) {
+    // measured at 13.8, 48 and 431 MB: two tokens 5.5 / 11.8 / 68.6 us, four tokens 6.5 / 13.6 / 75.4 us per pass;
+    // rows of 14336 values (two tokens a pass) 13.2 us at 48 MB
+    if (n_in > 4096) return (float)((m + 1) / 2) * (mb / 5.f + 3.5f);
+    return m == 2 ? mb / 6.4f + 3.5f : (float)((m + 3) / 4) * (mb / 5.8f + 4.f);
+  }
   if (gemv_dot2_multi_supported(format, x_dtype, m, n_in))
     return m <= 2 ? mb / 2.6f + 2.f : (float)((m + 3) / 4) * (mb / 1.7f + 2.f);
   if (gemv_q8_win_supported(format, n_out, n_in)) {

@@ -57,9 +57,13 @@ static_assert(kQ6RoundBlocks == kQ6Waves, "one block of the round per wavefront"
 // The two shapes of the kernel.  NBMAX: blocks per row it has tables for; BUFS: LDS buffers; WGS: workgroups per
 // compute unit; MAXG: row groups of a workgroup (their partial sums wait in LDS, in the space where the raw
 // activations land first).
-// FIXED: the row length is NBMAX blocks, known at compile time.
-struct Q6Head { static constexpr int NBMAX = 16, BUFS = 2, WGS = 2, MAXG = 20; static constexpr bool FIXED = true; };    // rows of 4096, many rows
-struct Q6Wide { static constexpr int NBMAX = 56, BUFS = 3, WGS = 1, MAXG = 56; static constexpr bool FIXED = false; };   // rows up to 14336
+// RPG: rounds per group when the kernel is built for one row length (2048 RPG values, NBMAX blocks), else 0.
+// rows of 4096, many rows
+struct Q6Head { static constexpr int NBMAX = 16, BUFS = 2, WGS = 2, MAXG = 20, RPG = 2; };
+// rows of 2048 or 4096, fewer rows
+template <int RPG_> struct Q6Short { static constexpr int NBMAX = 8 * RPG_, BUFS = 3, WGS = 1, MAXG = 56, RPG = RPG_; };
+// rows up to 14336
+struct Q6Wide { static constexpr int NBMAX = 56, BUFS = 3, WGS = 1, MAXG = 56, RPG = 0; };
 
 // XT: bf16 or fp16 activations.  The row groups are dealt out in runs: the first groups_rem workgroups take
 // groups_per_wg + 1 each, the others groups_per_wg.  nb: blocks per row, a multiple of eight.
@@ -70,8 +74,9 @@ __global__ void __launch_bounds__(kQ6Threads) __attribute__((amdgpu_waves_per_eu
 gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
                        const void* __restrict__ bias, int bias_dtype, int n_out, int nb_arg, int groups_per_wg,
                        int groups_rem) {
-  const int nb = CFG::FIXED ? CFG::NBMAX : nb_arg;
-  constexpr int kBufs = CFG::BUFS;
+  constexpr int kBufs = CFG::BUFS, RPG = CFG::RPG;
+  static_assert(RPG == 0 || CFG::NBMAX == 8 * RPG, "a fixed row length is the table's");
+  const int nb = RPG > 0 ? CFG::NBMAX : nb_arg;
   static_assert(kBufs >= 2 && kBufs <= 4, "the waits below count up to three later rounds");
   __shared__ __attribute__((aligned(1024))) uint8_t wbuf[kBufs * kQ6BufBytes];
   __shared__ __attribute__((aligned(16))) v4i_t xa[CFG::NBMAX * 32 + 1];   // (16 values, plane) entries + one of zeros
@@ -248,26 +253,40 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
     const uint32_t scx_off1 = (g >> 1) ? chunk_at(slot + 13) + 12u : sc_off + 12u;
     const uint32_t d_off = chunk_at(slot + 13) + (uint32_t)(kQ6DAt + (ODD ? 2 : 0));
 
-    struct Regs { sm_u32x4 ql, qh, a1, a2; uint32_t sc, d, f, qlx, qhx, scx; };
-    // unit hf of the round, round kr of the group
-    auto issue = [&](auto hc, uint32_t buf, uint32_t kr, Regs& r) {
+    // a unit's weights, and its activations: the two operands and the scale of the sums
+    struct Regs { sm_u32x4 ql, qh; uint32_t sc, d, qlx, qhx, scx; };
+    struct Acts { sm_u32x4 a1, a2; uint32_t f; };
+    // unit ui of a group (16 to a round)
+    auto issue_acts = [&](uint32_t ui, Acts& t) {
+      if constexpr (STAGE >= 2) return;
+      const uint32_t x1 = a1_addr + ui * a1_step, x2 = a2_addr + ui * a2_step;
+      const uint32_t fa = fac_addr0 + 16u * ui;
+      asm volatile(
+          "ds_read_b128 %0, %3\n\t"
+          "ds_read_b128 %1, %4\n\t"
+          "ds_read_b32 %2, %5"
+          : "=&v"(t.a1), "=&v"(t.a2), "=&v"(t.f)
+          : "v"(x1), "v"(x2), "v"(fa)
+          : "memory");
+    };
+    // (behind a wait) the registers hold what was read
+    auto settle_acts = [&](Acts& t) {
+      if constexpr (STAGE >= 2) return;
+      asm volatile("" : "+v"(t.a1), "+v"(t.a2), "+v"(t.f));
+    };
+    // unit hf of the round in `buf`
+    auto issue = [&](auto hc, uint32_t buf, Regs& r) {
       constexpr int hf = decltype(hc)::value;
       const uint32_t a_ql = buf + (hf ? ql_off1 : ql_off0), a_qh = buf + (hf ? qh_off1 : qh_off0);
       const uint32_t a_sc = buf + sc_off, a_d = buf + d_off;
-      const uint32_t ui = 16u * kr + (uint32_t)hf;
-      const uint32_t x1 = a1_addr + ui * a1_step, x2 = a2_addr + ui * a2_step;
-      const uint32_t fa = fac_addr0 + 16u * ui;
       if constexpr (STAGE >= 2) return;
       asm volatile(
-          "ds_read_b128 %0, %7\n\t"
-          "ds_read_b128 %1, %8\n\t"
-          "ds_read_b128 %2, %9\n\t"
-          "ds_read_b128 %3, %10\n\t"
-          "ds_read_b32 %4, %11 offset:%13\n\t"
-          "ds_read_u16 %5, %12\n\t"
-          "ds_read_b32 %6, %14"
-          : "=&v"(r.ql), "=&v"(r.qh), "=&v"(r.a1), "=&v"(r.a2), "=&v"(r.sc), "=&v"(r.d), "=&v"(r.f)
-          : "v"(a_ql), "v"(a_qh), "v"(x1), "v"(x2), "v"(a_sc), "v"(a_d), "n"(8 * hf), "v"(fa)
+          "ds_read_b128 %0, %4\n\t"
+          "ds_read_b128 %1, %5\n\t"
+          "ds_read_b32 %2, %6 offset:%8\n\t"
+          "ds_read_u16 %3, %7"
+          : "=&v"(r.ql), "=&v"(r.qh), "=&v"(r.sc), "=&v"(r.d)
+          : "v"(a_ql), "v"(a_qh), "v"(a_sc), "v"(a_d), "n"(8 * hf)
           : "memory");
       if constexpr (ODD) {
         const uint32_t a_qlx = buf + (hf ? qlx_off1 : qlx_off0), a_qhx = buf + (hf ? qhx_off1 : qhx_off0);
@@ -281,24 +300,15 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
             : "memory");
       }
     };
-    constexpr int kReads = ODD ? 10 : 7;                   // LDS reads of a unit
+    constexpr int kReads = 4 + (ODD ? 3 : 0) + (RPG > 0 ? 0 : 3);   // LDS reads of a unit
     auto settle = [&](auto pending, Regs& r) {
       constexpr int P = decltype(pending)::value;
       if constexpr (STAGE >= 2) return;
-      if constexpr (ODD)
-        asm volatile("s_waitcnt lgkmcnt(%10)"
-                     : "+v"(r.ql), "+v"(r.qh), "+v"(r.a1), "+v"(r.a2), "+v"(r.sc), "+v"(r.d), "+v"(r.f), "+v"(r.qlx),
-                       "+v"(r.qhx), "+v"(r.scx)
-                     : "n"(P)
-                     : "memory");
-      else
-        asm volatile("s_waitcnt lgkmcnt(%7)"
-                     : "+v"(r.ql), "+v"(r.qh), "+v"(r.a1), "+v"(r.a2), "+v"(r.sc), "+v"(r.d), "+v"(r.f)
-                     : "n"(P)
-                     : "memory");
+      asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(r.ql), "+v"(r.qh), "+v"(r.sc), "+v"(r.d) : "n"(P) : "memory");
+      if constexpr (ODD) asm volatile("" : "+v"(r.qlx), "+v"(r.qhx), "+v"(r.scx));
     };
     float acc = 0.f;
-    auto compute = [&](const Regs& r) {
+    auto compute = [&](const Regs& r, const Acts& t) {
       if constexpr (STAGE >= 1) return;
       uint32_t ql[4], qh[4], sc4;
       if constexpr (ODD) {
@@ -325,27 +335,45 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
         const uint32_t t2 = ((ql[i] >> 2) & 0x3C3C3C3Cu) | ((qh[i] << sh2) & ~0x3C3C3C3Cu);
         B1[i] = (int)((t1 & 0xFCFCFCFCu) ^ 0x80808080u);
         B2[i] = (int)((t2 & 0xFCFCFCFCu) ^ 0x80808080u);
-        A1[i] = (int)r.a1[i];
-        A2[i] = (int)r.a2[i];
+        A1[i] = (int)t.a1[i];
+        A2[i] = (int)t.a2[i];
       }
       const v4i_t zero = {0, 0, 0, 0};
       v4i_t C = __builtin_amdgcn_mfma_i32_16x16x64_i8(A1, B1, zero, 0, 0, 0);
       C = __builtin_amdgcn_mfma_i32_16x16x64_i8(A2, B2, C, 0, 0, 0);
       const int sc = (int)sc4;
-      int t = (int)(int8_t)(sc & 0xFF) * C[0];
-      t += (int)(int8_t)((sc >> 8) & 0xFF) * C[1];
-      t += (int)(int8_t)((sc >> 16) & 0xFF) * C[2];
-      t += (sc >> 24) * C[3];
+      // 24-bit multiplies (full rate; a 32-bit one takes four times as long): |C| <= 16 * 128 * 128
+      int ts = __mul24((int)(int8_t)(sc & 0xFF), C[0]);
+      ts += __mul24((int)(int8_t)((sc >> 8) & 0xFF), C[1]);
+      ts += __mul24((int)(int8_t)((sc >> 16) & 0xFF), C[2]);
+      ts += __mul24(sc >> 24, C[3]);
       const float d = f16_bits_to_f32((uint16_t)(r.d & 0xFFFFu));
-      acc = fmaf_((float)t * __uint_as_float(r.f), d, acc);
+      acc = fmaf_((float)ts * __uint_as_float(t.f), d, acc);
       // pins the arithmetic here: left alone the compiler moves it behind later waits
       asm volatile("" : "+v"(acc));
     };
 
     using U0 = std::integral_constant<int, 0>;
     using U1 = std::integral_constant<int, 1>;
-    int bufi = 0, kr = 0, gi = 0;
-    for (int rr = 0; rr < nrounds; rr++) {
+    // One row length (RPG rounds to a group, known at compile time): the wavefront's place in a group's rounds
+    // never changes, so neither do the activations it multiplies: they stay in registers for all its groups.
+    Acts held[RPG > 0 ? RPG : 1][2];
+    if constexpr (RPG > 0) {
+#pragma unroll
+      for (int kr = 0; kr < RPG; kr++) {
+        issue_acts(16u * (uint32_t)kr, held[kr][0]);
+        issue_acts(16u * (uint32_t)kr + 1u, held[kr][1]);
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int kr = 0; kr < RPG; kr++) {
+        settle_acts(held[kr][0]);
+        settle_acts(held[kr][1]);
+      }
+    }
+    int bufi = 0, rr = 0;
+    // round kr of its group; ta, tb: the activations of its two units
+    auto round = [&](uint32_t kr, Acts& ta, Acts& tb) {
       // the round's buffer: own requests landed, then everybody's
       const int later = min(nrounds - 1 - rr, kBufs - 1);          // rounds requested after this one
       if (later == 3) wait_rounds(I3{});
@@ -355,25 +383,37 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
       sm_barrier();
       const uint32_t buf = wbuf_base + (uint32_t)(bufi * kQ6BufBytes);
       Regs ra, rb;
-      issue(U0{}, buf, (uint32_t)kr, ra);
-      issue(U1{}, buf, (uint32_t)kr, rb);
+      issue(U0{}, buf, ra);
+      if constexpr (RPG == 0) issue_acts(16u * kr, ta);
+      issue(U1{}, buf, rb);
+      if constexpr (RPG == 0) issue_acts(16u * kr + 1u, tb);
       settle(std::integral_constant<int, kReads>{}, ra);
-      compute(ra);
+      if constexpr (RPG == 0) settle_acts(ta);
+      compute(ra, ta);
       settle(I0{}, rb);
+      if constexpr (RPG == 0) settle_acts(tb);
       // every wavefront has read what it needs of the buffer: a later round may land there
       sm_barrier();
       if (rr + kBufs < nrounds) request_next();
       bufi = bufi == kBufs - 1 ? 0 : bufi + 1;
-      compute(rb);
-      if (++kr == rpg) {
-        // the group is complete: the four accumulator lanes of a row
-        acc += __shfl_xor(acc, 16, kWave);
-        acc += __shfl_xor(acc, 32, kWave);
-        if (lane < 16) sm_write_f32(part_addr + (uint32_t)(gi * (kQ6Waves * 16 * 4)), acc);
-        acc = 0.f;
-        kr = 0;
-        gi++;
+      rr++;
+      compute(rb, tb);
+    };
+    for (int gi = 0; gi < ng; gi++) {
+      if constexpr (RPG > 0) {
+#pragma unroll
+        for (int kr = 0; kr < RPG; kr++) round((uint32_t)kr, held[kr][0], held[kr][1]);
+      } else {
+        for (int kr = 0; kr < rpg; kr++) {
+          Acts ta, tb;
+          round((uint32_t)kr, ta, tb);
+        }
       }
+      // the group is complete: the four accumulator lanes of a row
+      acc += __shfl_xor(acc, 16, kWave);
+      acc += __shfl_xor(acc, 32, kWave);
+      if (lane < 16) sm_write_f32(part_addr + (uint32_t)(gi * (kQ6Waves * 16 * 4)), acc);
+      acc = 0.f;
     }
   };
   if (wave & 1) run_rounds(std::true_type{});
@@ -391,9 +431,10 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
 }
 
 // Which shape of the kernel takes (n_out, n_in), with how many workgroups; ok == false: neither.
-struct Q6Plan { bool ok, head; int num_wg; };
+// rpg: 1 or 2 for rows of 2048 or 4096 values (the kernels built for one row length), else 0.
+struct Q6Plan { bool ok, head; int num_wg, rpg; };
 inline Q6Plan q6_plan(int64_t n_out, int64_t n_in) {
-  Q6Plan p{false, false, 0};
+  Q6Plan p{false, false, 0, 0};
   const int64_t nb = n_in / 256;
   // whole rounds of eight blocks, whole groups of 16 rows, 32-bit byte offsets into the weight buffer
   if (n_in % (256 * kQ6RoundBlocks) != 0 || nb > Q6Wide::NBMAX || n_out % 16 != 0) return p;
@@ -404,6 +445,7 @@ inline Q6Plan q6_plan(int64_t n_out, int64_t n_in) {
   // between one and two groups per compute unit the uneven ones decide (6144x4096: 7.9 us against 7.7 of the
   // packed-dot kernel, which deals rows out more finely)
   if (groups < 2 * cus && groups % cus != 0) return p;
+  p.rpg = nb <= 16 ? (int)(nb / 8) : 0;
   int maxg;
   if (nb == Q6Head::NBMAX && groups >= 2 * (int64_t)Q6Head::WGS * cus) {
     // two workgroups per compute unit when each still gets two groups: their rounds interleave
@@ -432,6 +474,8 @@ inline hipError_t q6_launch_xy(const void* w, const void* x, void* y, const void
                        groups % p.num_wg);
   };
   if (p.head) go(gemv_q6k_stream_kernel<XT, YT, Q6Head, STAGE>);
+  else if (p.rpg == 1) go(gemv_q6k_stream_kernel<XT, YT, Q6Short<1>, STAGE>);
+  else if (p.rpg == 2) go(gemv_q6k_stream_kernel<XT, YT, Q6Short<2>, STAGE>);
   else go(gemv_q6k_stream_kernel<XT, YT, Q6Wide, STAGE>);
   return hipGetLastError();
 }

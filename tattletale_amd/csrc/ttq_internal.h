@@ -99,6 +99,12 @@ hipError_t launch_gemv_q6k_stream(const void* w, const void* x, int x_dtype, voi
                                   const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                                   hipStream_t s);
 
+// The same stream for two to four activation rows in one pass (ttq_gemv_q6k_stream4.hip).
+bool gemv_q6k_stream4_supported(int format, int x_dtype, int64_t m, int64_t n_out, int64_t n_in);
+hipError_t launch_gemv_q6k_stream4(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                                   const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                                   hipStream_t s);
+
 // int8 matrix-core path for Q8_0, any activation dtype (ttq_gemv_q8_mfma.hip).
 // Q8_0 through the matrix cores, rows read as aligned 64-byte windows (ttq_gemv_q8_win.hip).
 bool gemv_q8_win_supported(int format, int64_t n_out, int64_t n_in);

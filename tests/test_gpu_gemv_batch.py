@@ -173,6 +173,81 @@ def test_streamed_two_to_four_rows_do_not_leak_and_output_types():
         assert rel_l2(yy, want3) <= tol, out_dtype
 
 
+# ------------------------------------------------------------------- Q6_K, two to four rows, streamed kernel
+# (whole rounds of 2048 values, a group of 16 weight rows or more per compute unit: a pair of tokens shares a
+# matrix instruction; rows of up to 4096 values take four tokens per pass, longer ones two)
+@pytest.mark.parametrize("xk", ["bf16", "f16"])
+@pytest.mark.parametrize("m", [2, 3, 4])
+@pytest.mark.parametrize("n_out,n_in", [(4096, 4096), (8192 + 16 * 37, 2048), (16384 + 16 * 5, 4096), (4096, 14336),
+                                        (4096 + 16 * 3, 6144), (164800, 2048)])
+def test_q6k_streamed_two_to_four_rows(xk, m, n_out, n_in):
+    """Random block bytes.  Normal activations with uneven magnitudes, another scale per token: every token
+    within 1e-3 of the float64 product and, to summation order, equal to the single-row kernel on that token.
+    Then unit vectors, a different column and power of two per token (both nibble planes, every bit pair, odd
+    and even blocks): the canonical columns bit for bit."""
+    rng = np.random.default_rng(n_out + n_in + m)
+    p = random_blocks(F.Q6_K, n_out * (n_in // 256), seed=70 + m)
+    rows = np.unique(np.concatenate([rng.integers(0, n_out, 600), np.arange(n_out - 48, n_out), np.arange(48)]))
+    what = oracle.dequant(F.Q6_K, np.ascontiguousarray(p.reshape(n_out, -1)[rows]), rows.size, n_in)
+    wd = packed_to_dev(p)
+    x = Q.fill_normal(71 + m, 1, 1.0, m * n_in).reshape(m, n_in)
+    for t in range(m):
+        x[t] *= (1.0, 1e-4, 300.0, 7.0)[t]
+        x[t, t::13] *= 31.0
+    xd, xf = x_to_dev(x, xk)
+    y = QL.gemv(F.Q6_K, wd, xd, n_out, n_in).cpu().numpy()
+    want = oracle.linear_f64(what, xf)
+    for t in range(m):
+        assert rel_l2(y[t][rows], want[t]) <= TOL, t
+        y1 = QL.gemv(F.Q6_K, wd, xd[t:t + 1], n_out, n_in).cpu().numpy()[0]
+        assert rel_l2(y[t], y1) <= 2e-6, t
+    col_sets = [(0, 33, 255, n_in - 1), (31 + 256, 32 + 64, 2047, n_in - 2048 + 300), (256 + 97, n_in - 33, 5, 1000),
+                (256 * 3 + 128 + 16, 256 * 5 + 64 + 15, 256 * 7 + 192 + 47, 256 * 6 + 100)]
+    for cols in col_sets:
+        x = np.zeros((m, n_in), np.float32)
+        sc = (1.0, -0.5, 4.0, 0.25)
+        for t in range(m):
+            x[t, cols[t]] = sc[t]
+        xd, _ = x_to_dev(x, xk)
+        y = QL.gemv(F.Q6_K, wd, xd, n_out, n_in).cpu().numpy()
+        for t in range(m):
+            col = what[:, cols[t]] * np.float32(sc[t])
+            assert np.array_equal(y[t][rows], col), (t, cols[t])
+            nz = col != 0
+            assert np.array_equal(y[t][rows][nz].view(np.uint32), col[nz].view(np.uint32)), (t, cols[t])
+
+
+def test_q6k_streamed_two_to_four_rows_do_not_leak_and_output_types():
+    """A row of zeros, a row with an Inf, a tiny row beside an ordinary one; bias and 16-bit outputs through the
+    layer entry point; quantized (not random) blocks."""
+    n_out, n_in = 4096 + 32, 4096
+    p = Q.quantize(F.Q6_K, Q.fill_normal(90, 0, 0.02, n_out * n_in).reshape(n_out, n_in))
+    what = oracle.dequant(F.Q6_K, p, n_out, n_in)
+    wd = packed_to_dev(p)
+    x = np.zeros((4, n_in), np.float32)
+    x[1] = Q.fill_normal(91, 1, 1.0, n_in)
+    x[1, n_in - 1] = np.inf
+    x[2] = Q.fill_normal(92, 1, 1.0, n_in) * 1e-30
+    x[3] = Q.fill_normal(93, 1, 1.0, n_in)
+    xd, xf = x_to_dev(x, "bf16")
+    y = QL.gemv(F.Q6_K, wd, xd, n_out, n_in).cpu().numpy()
+    want = oracle.linear_f64(what, xf[[2, 3]])
+    assert np.array_equal(y[0], np.zeros(n_out, np.float32))
+    assert not np.any(np.isfinite(y[1]))
+    assert rel_l2(y[2], want[0]) <= TOL
+    assert rel_l2(y[3], want[1]) <= TOL
+    y2 = QL.gemv(F.Q6_K, wd, xd[:2], n_out, n_in).cpu().numpy()          # the two-token shape
+    assert np.array_equal(y2[0], np.zeros(n_out, np.float32))
+    assert not np.any(np.isfinite(y2[1]))
+    bias = Q.fill_normal(94, 0, 0.5, n_out)
+    xd3, xf3 = x_to_dev(Q.fill_normal(95, 1, 1.0, 3 * n_in).reshape(3, n_in), "f16")
+    want3 = oracle.linear_f64(what, xf3) + bias
+    for out_dtype, tol in ((torch.float32, TOL), (torch.bfloat16, 4e-3), (torch.float16, 1e-3)):
+        layer = QuantLinear.init(wd, F.Q6_K, n_in, n_out, bias=torch.from_numpy(bias).to(DEV))
+        yy = layer.forward(xd3, out_dtype=out_dtype).float().cpu().numpy()
+        assert rel_l2(yy, want3) <= tol, out_dtype
+
+
 @pytest.mark.parametrize("m", [5, 20, 32])
 def test_forward_few_rows_bias_and_output_types(m):
     n_out, n_in = 2304, 1024
