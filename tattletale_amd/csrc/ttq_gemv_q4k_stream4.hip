@@ -36,7 +36,10 @@ constexpr int kS4BufBytes = 2 * kS4HalfBytes;              // 14336
 constexpr int kS4XPasses = 4;                  // activation requests per wavefront: 4 x 512 chunks of 8 values = 4 x 4096 / 8
 constexpr int kS4XLine0 = 4;                   // they land in the slots of lines 4 and 5
 constexpr int kS4MaxSb = 16;                   // n_in <= 4096
-constexpr int kS4MaxBlocks = 16;               // blocks of a workgroup (their sums wait in LDS)
+// Sums that wait in LDS for the end of the kernel: one per block of a workgroup, or -- when a workgroup has more
+// blocks than this and rows of 4096 values -- one per row group: a wavefront then takes both blocks of a group,
+// one after the other, and adds them in its accumulator.
+constexpr int kS4MaxPart = 40;
 constexpr int kS4CstDw = 20;                   // per (token, super-block): f[8], sum[8], kodd[4]
 static_assert(kS4XPasses * kS4Threads * 8 >= kS4Tok * kS4MaxSb * 256, "every activation has a thread");
 static_assert(kS4XLine0 + (kS4XPasses + 1) / 2 <= kS4RingLines, "the landing slots exist");
@@ -58,7 +61,7 @@ gemv_q4k_stream4_kernel(const uint8_t* __restrict__ w, const uint16_t* __restric
   __shared__ __attribute__((aligned(1024))) uint8_t wbuf[kS4Waves * kS4BufBytes];
   __shared__ __attribute__((aligned(16))) v4i_t xa[kS4Tok * kS4MaxSb * 32 + 1];      // plane tables + one zero entry
   __shared__ __attribute__((aligned(16))) uint32_t cst[kS4Tok * kS4MaxSb * kS4CstDw];
-  __shared__ float part[kS4MaxBlocks][64];
+  __shared__ float part[kS4MaxPart][64];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -70,7 +73,9 @@ gemv_q4k_stream4_kernel(const uint8_t* __restrict__ w, const uint16_t* __restric
   const int wg_row_end = min(wg_row0 + rows_per_wg, n_out);
   const int last = wg_row_end - 1;
   const int ngroups = (wg_row_end - wg_row0 + 15) >> 4;
-  const int nblocks = ((FUSE ? 2 : 1) * ngroups) << nks_log2;   // <= kS4MaxBlocks (the launcher sees to it)
+  const int nblocks = ((FUSE ? 2 : 1) * ngroups) << nks_log2;
+  // (the launcher sees to it that the blocks, or else the row groups, number kS4MaxPart at most)
+  const bool pair = nblocks > kS4MaxPart;
   uint8_t* mybuf = wbuf + wave * kS4BufBytes;
   const int zero_entry = kS4Tok * kS4MaxSb * 32;
 
@@ -112,10 +117,11 @@ gemv_q4k_stream4_kernel(const uint8_t* __restrict__ w, const uint16_t* __restric
     __builtin_amdgcn_global_load_lds((st_gptr_t)(w + (size_t)(lane_off[o] + (uint32_t)(line * 128))),
                                      (st_lptr_t)(mybuf + o * kS4HalfBytes + s4_slot(line) * 1024), 16, 0, 2);
   };
-  int blk = wave;
-  const bool have_block = blk < nblocks;
+  // the wavefront's blocks: wave, wave + 8, ..., or both blocks of row groups wave, wave + 8, ...
+  const int blk0 = pair ? 2 * wave : wave;
+  const bool have_block = blk0 < nblocks;
   if (have_block) {
-    set_block(blk);
+    set_block(blk0);
 #pragma unroll
     for (int i = 0; i < kS4UpFirst; i++) request(i);
     st_wait_vmcnt<kS4UpFirst>();
@@ -305,15 +311,16 @@ gemv_q4k_stream4_kernel(const uint8_t* __restrict__ w, const uint16_t* __restric
     asm volatile("" : "+v"(acc));       // keeps the arithmetic between the waits it was written between
   };
 
-  // ---- the wavefront's blocks: wave, wave + 8, ...  A block starts with UP requests outstanding.
-  auto run_block = [&](auto upc, const int b_) {
+  // ---- a block starts with UP requests outstanding.  next: the wavefront's block after it; reset: a new sum
+  // starts here; store >= 0: the sum is complete and goes there
+  auto run_block = [&](auto upc, const int b_, const int next, const bool reset, const int store) {
     constexpr int UP = decltype(upc)::value;
     using U = std::integral_constant<int, UP>;
     const int ks = b_ & ((1 << nks_log2) - 1);
 #pragma unroll
     for (int u = 0; u < 4; u++) a_addr[u] = a_addr0[u] + (uint32_t)ks * (kStBlockSb * a_step);
     cst_addr = cst_addr0 + (uint32_t)(ks * kStBlockSb * kS4CstDw * 4);
-    acc = 0.f;
+    if (reset) acc = 0.f;
     Regs ra, rb2;
     topup(U{}, std::integral_constant<int, 0>{}); issue(U{}, std::integral_constant<int, 0>{}, ra);
     topup(U{}, std::integral_constant<int, 1>{}); settle(ra); compute(ra); issue(U{}, std::integral_constant<int, 1>{}, rb2);
@@ -325,17 +332,31 @@ gemv_q4k_stream4_kernel(const uint8_t* __restrict__ w, const uint16_t* __restric
     topup(U{}, std::integral_constant<int, 7>{}); settle(ra); compute(ra); issue(U{}, std::integral_constant<int, 7>{}, rb2);
     settle(rb2);
     // every request of the block has landed and been read: the next block may use the buffer
-    const int next = b_ + kS4Waves;
     if (next < nblocks) {
       set_block(next);
 #pragma unroll
       for (int i = 0; i < kS4Up; i++) request(i);
     }
     compute(rb2);
-    part[b_][lane] = acc;               // (row n, token g): nothing to reduce across lanes
+    if (store >= 0) part[store][lane] = acc;               // (row n, token g): nothing to reduce across lanes
   };
-  for (; blk < nblocks; blk += kS4Waves) {
-    run_block(std::integral_constant<int, kS4Up>{}, blk);
+  for (int i = 0;; i++) {
+    int b_, next, store;
+    bool reset;
+    if (pair) {
+      const int rgi = wave + kS4Waves * (i >> 1), second = i & 1;
+      b_ = 2 * rgi + second;
+      next = second ? 2 * (rgi + kS4Waves) : b_ + 1;
+      reset = !second;
+      store = second ? rgi : -1;
+    } else {
+      b_ = wave + kS4Waves * i;
+      next = b_ + kS4Waves;
+      reset = true;
+      store = b_;
+    }
+    if (b_ >= nblocks) break;
+    run_block(std::integral_constant<int, kS4Up>{}, b_, next, reset, store);
   }
 
   // every request has landed; the blocks of a row group add up
@@ -344,12 +365,12 @@ gemv_q4k_stream4_kernel(const uint8_t* __restrict__ w, const uint16_t* __restric
   for (int t = tid; t < wg_rows16 * m; t += kS4Threads) {
     const int tok = t / wg_rows16, r = t - tok * wg_rows16;
     const int grp = r >> 4, nn = r & 15;
-    float v = part[grp << nks_log2][tok * 16 + nn];
-    if (nks_log2) v += part[(grp << 1) + 1][tok * 16 + nn];
+    float v = part[pair ? grp : grp << nks_log2][tok * 16 + nn];
+    if (nks_log2 && !pair) v += part[(grp << 1) + 1][tok * 16 + nn];
     const int row = wg_row0 + r;
     if (FUSE) {
-      float u = part[(ngroups + grp) << nks_log2][tok * 16 + nn];
-      if (nks_log2) u += part[((ngroups + grp) << 1) + 1][tok * 16 + nn];
+      float u = part[pair ? ngroups + grp : (ngroups + grp) << nks_log2][tok * 16 + nn];
+      if (nks_log2 && !pair) u += part[((ngroups + grp) << 1) + 1][tok * 16 + nn];
       if (row < wg_row_end) YElem<YT>::store(y, (int64_t)tok * n_out + row, (v / (1.f + expf(-v))) * u);
     } else {
       if (row < wg_row_end) YElem<YT>::store(y, (int64_t)tok * n_out + row, v + load_bias(bias, bias_dtype, row));
@@ -367,7 +388,9 @@ S4Plan s4_plan(int64_t m, int64_t n_out, int64_t n_in, bool fuse) {
   if (parts * n_out < 16 * (int64_t)device_num_cus() || parts * n_out * (n_in / 256) * 144 >= ((int64_t)1 << 32)) return p;
   if (fuse && n_out % 8 != 0) return p;
   p.rows_per_wg = st_rows_per_wg(n_out, &p.num_wg);
-  if (parts * ((p.rows_per_wg + 15) / 16) * (n_in / 2048) > kS4MaxBlocks) return p;
+  // the sums of a workgroup's blocks, or for rows of 4096 values else those of its row groups, fit LDS
+  const int64_t groups = parts * ((p.rows_per_wg + 15) / 16);
+  if (groups * (n_in / 2048) > kS4MaxPart && !(n_in == 4096 && groups <= kS4MaxPart)) return p;
   p.ok = true;
   return p;
 }

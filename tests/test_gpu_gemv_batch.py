@@ -145,6 +145,41 @@ def test_streamed_two_to_four_rows(xk, m, n_out, n_in):
             assert np.array_equal(y[t][nz].view(np.uint32), col[nz].view(np.uint32)), (t, cols[t])
 
 
+@pytest.mark.parametrize("m,n_out", [(2, 128256), (4, 128256 + 8), (3, 163840), (4, 81920 + 16)])
+def test_streamed_two_to_four_rows_many_weight_rows(m, n_out):
+    """More than 320 weight rows per compute unit (an LM head): a wavefront takes both halves of a row group
+    and keeps one sum per group.  Sampled rows against the float64 product and the single-row kernel; a unit
+    vector per token in either half of K bit for bit."""
+    n_in = 4096
+    rng = np.random.default_rng(n_out + m)
+    p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=50 + m)
+    rows = np.unique(np.concatenate([rng.integers(0, n_out, 800), np.arange(n_out - 48, n_out), np.arange(48),
+                                     np.arange(n_out // 2 - 300, n_out // 2 + 300)]))
+    what = oracle.dequant(F.Q4_K, np.ascontiguousarray(p.reshape(n_out, -1)[rows]), rows.size, n_in)
+    wd = packed_to_dev(p)
+    x = Q.fill_normal(51 + m, 1, 1.0, m * n_in).reshape(m, n_in)
+    for t in range(m):
+        x[t] *= (1.0, 1e-4, 300.0, 7.0)[t]
+        x[t, t::13] *= 31.0
+    xd, xf = x_to_dev(x, "bf16")
+    y = QL.gemv(F.Q4_K, wd, xd, n_out, n_in).cpu().numpy()
+    want = oracle.linear_f64(what, xf)
+    for t in range(m):
+        assert rel_l2(y[t][rows], want[t]) <= TOL, t
+        y1 = QL.gemv(F.Q4_K, wd, xd[t:t + 1], n_out, n_in).cpu().numpy()[0]
+        assert rel_l2(y[t], y1) <= 3e-4, t
+    cols = (33, 2048 + 255, 4095, 1000)
+    sc = (1.0, -0.5, 4.0, 0.25)
+    x = np.zeros((m, n_in), np.float32)
+    for t in range(m):
+        x[t, cols[t]] = sc[t]
+    xd, _ = x_to_dev(x, "bf16")
+    y = QL.gemv(F.Q4_K, wd, xd, n_out, n_in).cpu().numpy()
+    for t in range(m):
+        col = what[:, cols[t]] * np.float32(sc[t])
+        assert np.array_equal(y[t][rows], col), (t, cols[t])
+
+
 def test_streamed_two_to_four_rows_do_not_leak_and_output_types():
     """A row of zeros, a row with an Inf, a tiny row beside an ordinary one; bias and 16-bit outputs through the
     layer entry point."""
