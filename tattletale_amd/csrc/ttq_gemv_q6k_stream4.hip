@@ -28,24 +28,27 @@ typedef uint32_t sm_u32x2 __attribute__((ext_vector_type(2)));
 
 // TOK: activation rows of a pass (2 or 4); the other parameters as in the single-row kernel's shapes.
 // RPG: rounds per group (rows of 2048 RPG values) when the kernel is built for one row length, else 0.
-template <int TOK_, int NBMAX_, int BUFS_, int WGS_, int MAXG_, int RPG_>
+// KP: into how many parts of NBMAX blocks a row may fall; the parts are streamed one after the other, each with
+// its own plane tables (four tokens' tables of a row of 14336 values would not fit LDS).
+template <int TOK_, int NBMAX_, int BUFS_, int WGS_, int MAXG_, int RPG_, int KP_ = 1>
 struct Q6Multi {
-  static constexpr int TOK = TOK_, NBMAX = NBMAX_, BUFS = BUFS_, WGS = WGS_, MAXG = MAXG_, RPG = RPG_;
-  static_assert(RPG == 0 || NBMAX == 8 * RPG, "a fixed row length is the table's");
+  static constexpr int TOK = TOK_, NBMAX = NBMAX_, BUFS = BUFS_, WGS = WGS_, MAXG = MAXG_, RPG = RPG_, KP = KP_;
+  static_assert(RPG == 0 || (NBMAX == 8 * RPG && KP == 1), "a fixed row length is the table's");
 };
 // rows of 2048 RPG values (RPG 1 or 2), many of them, two tokens: two workgroups per compute unit
 template <int RPG> using Q6M2Head = Q6Multi<2, 8 * RPG, 2, 2, 20, RPG>;
 template <int RPG> using Q6M2One = Q6Multi<2, 8 * RPG, 3, 1, 56, RPG>;    // rows of 2048 RPG values, two tokens
 template <int RPG> using Q6M4One = Q6Multi<4, 8 * RPG, 3, 1, 56, RPG>;    // rows of 2048 RPG values, four tokens
 using Q6M2Wide = Q6Multi<2, 56, 3, 1, 24, 0>;                             // rows of up to 14336, two tokens
+using Q6M4Wide = Q6Multi<4, 32, 3, 1, 6, 0, 2>;                           // rows of up to 14336, four tokens, K in two parts
 
 template <typename XT, typename YT, typename CFG>
 __global__ void __launch_bounds__(kQ6Threads) __attribute__((amdgpu_waves_per_eu(2 * CFG::WGS, 2 * CFG::WGS)))
 gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
                       const void* __restrict__ bias, int bias_dtype, int m, int n_out, int nb_arg, int groups_per_wg,
                       int groups_rem) {
-  constexpr int TOK = CFG::TOK, kBufs = CFG::BUFS, kPairs = TOK / 2, RPG = CFG::RPG;
-  const int nb = RPG > 0 ? 8 * RPG : nb_arg;
+  constexpr int TOK = CFG::TOK, kBufs = CFG::BUFS, kPairs = TOK / 2, RPG = CFG::RPG, KP = CFG::KP;
+  const int nb = RPG > 0 ? 8 * RPG : nb_arg;              // blocks of a row: NBMAX KP at most
   static_assert(TOK == 2 || TOK == 4, "tokens come in pairs");
   static_assert(kBufs >= 2 && kBufs <= 3, "the waits below count up to two later rounds");
   // a token's plane table: kXaHead bytes of zeros, then (16 values, plane) entries of 16 bytes.  Consecutive tables
@@ -61,12 +64,13 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
   __shared__ __attribute__((aligned(16))) float fac[TOK * CFG::NBMAX * 8];
   __shared__ __attribute__((aligned(16))) float stage[2][kQ6Waves][TOK][16];
   __shared__ __attribute__((aligned(16))) float total[CFG::MAXG][TOK][16];
-  // the raw activations land in the buffers that the weights do not use before the plane tables are built
-  static_assert((kBufs - 1) * kQ6BufBytes >= TOK * CFG::NBMAX * 512, "room for the staged activations");
-  uint8_t* xstage = wbuf + kQ6BufBytes;
+  // The raw activations land in stream buffers.  One part: in those the first round does not use, which is
+  // requested before the tables are built.  Several parts: anywhere, and the stream starts behind the tables.
+  constexpr int kStageBufs = KP == 1 ? kBufs - 1 : kBufs;
+  static_assert(kStageBufs * kQ6BufBytes >= TOK * CFG::NBMAX * 512, "room for the staged activations");
+  uint8_t* xstage = wbuf + (kBufs - kStageBufs) * kQ6BufBytes;
 
   const int n_in = nb * 256;
-  const int rpg = nb >> 3;                                // rounds per group
   const uint32_t row_bytes = (uint32_t)nb * 210u;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -75,25 +79,6 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
   const int bx = blockIdx.x;
   const int grp0 = bx * groups_per_wg + min(bx, groups_rem);
   const int ng = groups_per_wg + (bx < groups_rem ? 1 : 0);            // 1 .. CFG::MAXG
-  const int nrounds = rpg * ng;
-
-  // ---- the activations, as LDS requests: thread t stages x[8 t + 4096 i .. + 7] of every token
-  constexpr int kXPasses = (CFG::NBMAX * 256 + 8 * kQ6Threads - 1) / (8 * kQ6Threads);
-#pragma unroll
-  for (int t = 0; t < TOK; t++) {
-    const uint16_t* xt = x + (int64_t)min(m0 + t, m - 1) * n_in;
-#pragma unroll
-    for (int i = 0; i < kXPasses; i++) {
-      const int k0 = 8 * tid + i * (8 * kQ6Threads);
-      if (k0 < n_in)                                      // whole wavefronts: n_in is a multiple of 512
-        __builtin_amdgcn_global_load_lds((sm_gptr_t)(xt + k0),
-                                         (sm_lptr_t)(xstage + t * (CFG::NBMAX * 512) + i * (16 * kQ6Threads) + wave * 1024),
-                                         16, 0, 0);
-    }
-  }
-  // a compute unit serves its requests in the order they were made: every wavefront's activation requests are
-  // queued before any weight request of the workgroup
-  asm volatile("s_barrier" ::: "memory");
 
   // ---- requests of a round, exactly as in the single-row kernel: request q = wave + 8 i fills LDS chunks
   // 64 q .. 64 q + 63 of the buffer; chunk position 112 n + (c + n) % 112 holds chunk c of row n's eight slots
@@ -107,7 +92,43 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
     src_off[i] = (uint32_t)row * row_bytes + (uint32_t)(b * 210 - 2 * (b & 1) + (j < kQ6SlotChunks - 1 ? 16 * j : kQ6TailAt));
   }
   const bool full = wave < kQ6FullWaves;
-  uint32_t req_src = (uint32_t)min(grp0, n_out / 16 - 1) * 16u * row_bytes;    // byte offset of the next round to request
+  // all but the youngest `rounds_after` rounds of requests of this wavefront have landed
+  auto wait_rounds = [&](auto rounds_after) {
+    constexpr int A = decltype(rounds_after)::value;
+    if (full) sm_wait_vmcnt<A * kQ6ReqMax>();
+    else sm_wait_vmcnt<A * (kQ6ReqMax - 1)>();
+  };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+
+  // ---- the parts of K (one, unless the configuration says otherwise): blocks kb0 .. kb0 + nbp - 1 of every row
+  for (int kp = 0, kb0 = 0; kp < KP && kb0 < nb; kp++, kb0 += CFG::NBMAX) {
+  const int nbp = min(nb - kb0, CFG::NBMAX);
+  const int n_in_p = nbp * 256;
+  const int rpg = nbp >> 3;                               // rounds per group
+  const int nrounds = rpg * ng;
+
+  // ---- the activations, as LDS requests: thread t stages values 8 t + 4096 i .. + 7 of every token's part
+  constexpr int kXPasses = (CFG::NBMAX * 256 + 8 * kQ6Threads - 1) / (8 * kQ6Threads);
+#pragma unroll
+  for (int t = 0; t < TOK; t++) {
+    const uint16_t* xt = x + (int64_t)min(m0 + t, m - 1) * n_in + kb0 * 256;
+#pragma unroll
+    for (int i = 0; i < kXPasses; i++) {
+      const int k0 = 8 * tid + i * (8 * kQ6Threads);
+      if (k0 < n_in_p)                                    // whole wavefronts: the part is a multiple of 512
+        __builtin_amdgcn_global_load_lds((sm_gptr_t)(xt + k0),
+                                         (sm_lptr_t)(xstage + t * (CFG::NBMAX * 512) + i * (16 * kQ6Threads) + wave * 1024),
+                                         16, 0, 0);
+    }
+  }
+  // a compute unit serves its requests in the order they were made: every wavefront's activation requests are
+  // queued before any weight request of the workgroup
+  asm volatile("s_barrier" ::: "memory");
+
+  // byte offset of the next round to request
+  uint32_t req_src = (uint32_t)min(grp0, n_out / 16 - 1) * 16u * row_bytes + (uint32_t)kb0 * 210u;
   int req_kr = 0, req_buf = 0;
   auto request_next = [&]() {
     const uint8_t* src = w + (size_t)req_src;
@@ -121,25 +142,20 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
     req_buf = req_buf == kBufs - 1 ? 0 : req_buf + 1;
     req_kr++;
     req_src += kQ6RoundBlocks * 210;
-    if (req_kr == rpg) {
+    if (req_kr == rpg) {                  // the same part of the next group's rows
       req_kr = 0;
-      req_src += 15u * row_bytes;
+      req_src += 16u * row_bytes - (uint32_t)rpg * (kQ6RoundBlocks * 210);
     }
   };
-  // all but the youngest `rounds_after` rounds of requests of this wavefront have landed
-  auto wait_rounds = [&](auto rounds_after) {
-    constexpr int A = decltype(rounds_after)::value;
-    if (full) sm_wait_vmcnt<A * kQ6ReqMax>();
-    else sm_wait_vmcnt<A * (kQ6ReqMax - 1)>();
-  };
-  using I0 = std::integral_constant<int, 0>;
-  using I1 = std::integral_constant<int, 1>;
-  using I2 = std::integral_constant<int, 2>;
-  // one round now (into the first buffer: the activations sit in the others), the rest once the tables are built
-  request_next();
+  if constexpr (KP == 1) {
+    // one round now (into the first buffer: the activations sit in the others), the rest once the tables are built
+    request_next();
+    wait_rounds(I1{});
+  } else {
+    wait_rounds(I0{});
+  }
 
   // ---- the raw activations back into registers (each wavefront reads what it asked for), then into byte planes
-  wait_rounds(I1{});
   if (tid < 128) {
 #pragma unroll
     for (int t = 0; t < TOK; t++) reinterpret_cast<uint32_t*>(xa + t * kXaTok)[tid] = 0u;
@@ -149,7 +165,7 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
 #pragma unroll
     for (int i = 0; i < kXPasses; i++) {
       const int k0 = 8 * tid + i * (8 * kQ6Threads);
-      if (k0 >= n_in) break;
+      if (k0 >= n_in_p) break;
       float xf[8];
       const sm_u32x4 r = sm_read16(sm_lds(xstage) + (uint32_t)(t * (CFG::NBMAX * 512) + i * (16 * kQ6Threads) + tid * 16));
       widen8<XT>(make_uint4(r[0], r[1], r[2], r[3]), xf);
@@ -215,7 +231,7 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
 
   sm_barrier();                         // the plane tables are complete, the staged activations read
 #pragma unroll
-  for (int i = 1; i < kBufs; i++)
+  for (int i = KP == 1 ? 1 : 0; i < kBufs; i++)
     if (i < nrounds) request_next();
 
   // the eight wavefronts' sums of group `grp` (complete since a barrier) -> its totals, in wavefront order
@@ -240,7 +256,13 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
       float sum = v[0];
 #pragma unroll
       for (int wv = 1; wv < kQ6Waves; wv++) sum += v[wv];
-      sm_write_f32(total_base + (uint32_t)(grp * (TOK * 64) + 4 * lane), sum);
+      const uint32_t ta = total_base + (uint32_t)(grp * (TOK * 64) + 4 * lane);
+      if (KP > 1 && kp > 0) {             // on top of the earlier parts of K
+        float before;
+        asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(before) : "v"(ta) : "memory");
+        sum += before;
+      }
+      sm_write_f32(ta, sum);
     }
   };
 
@@ -450,8 +472,10 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
   };
   if (blk & 1) run_rounds(std::true_type{});
   else run_rounds(std::false_type{});
+  // every wavefront has left its last sums and is done with the buffers and the tables
   sm_barrier();
   if (wave == ((ng - 1) & 7)) reduce_group(ng - 1);
+  }   // parts of K
   // every request has landed (plain loads are safe again)
   __syncthreads();
   for (int t = tid; t < ng * TOK * 16; t += kQ6Threads) {
@@ -463,15 +487,16 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
   }
 }
 
-// Which shape takes (m, n_out, n_in): 0 none, else 1 Q6M2Head, 2 Q6M2One, 3 Q6M4One, 4 Q6M2Wide.
+// Which shape takes (m, n_out, n_in): 0 none, else 1 Q6M2Head, 2 Q6M2One, 3 Q6M4One, 4 Q6M2Wide, 5 Q6M4Wide.
 struct Q6MultiPlan { int kind, tok, num_wg; };
 Q6MultiPlan q6_multi_plan(int64_t m, int64_t n_out, int64_t n_in) {
   Q6MultiPlan p{0, 0, 0};
   const Q6Plan single = q6_plan(n_out, n_in);              // the stream's own limits
   const int64_t nb = n_in / 256, groups = n_out / 16;
-  // two passes at most: eight rows of up to 4096 values, four longer ones
+  // two passes of four rows at most
   static const int max_rows = dev_knob("TTQ_Q6_MULTI_MAX_ROWS", 8);
-  if (!single.ok || m < 2 || m > (nb <= 16 ? max_rows : std::min(max_rows, 4))) return p;
+  if (!single.ok || m < 2 || m > max_rows) return p;
+  static_assert(Q6M4Wide::NBMAX * Q6M4Wide::KP >= Q6Wide::NBMAX && Q6M2Wide::NBMAX >= Q6Wide::NBMAX, "every row length of the stream");
   const int cus = device_num_cus();
   int maxg, wgs = 1;
   if (nb <= 16) {
@@ -489,10 +514,14 @@ Q6MultiPlan q6_multi_plan(int64_t m, int64_t n_out, int64_t n_in) {
       p.kind = 2;
       maxg = Q6M2One<1>::MAXG;
     }
-  } else {
+  } else if (m == 2) {
     p.kind = 4;
     p.tok = 2;
     maxg = Q6M2Wide::MAXG;
+  } else {
+    p.kind = 5;
+    p.tok = 4;
+    maxg = Q6M4Wide::MAXG;
   }
   p.num_wg = (int)std::min<int64_t>(groups, (int64_t)wgs * cus);
   if ((groups + p.num_wg - 1) / p.num_wg > maxg) p.num_wg = (int)((groups + maxg - 1) / maxg);
@@ -516,7 +545,8 @@ hipError_t q6_multi_launch_xy(const void* w, const void* x, void* y, const void*
     case 1: one ? go(gemv_q6k_multi_kernel<XT, YT, Q6M2Head<1>>) : go(gemv_q6k_multi_kernel<XT, YT, Q6M2Head<2>>); break;
     case 2: one ? go(gemv_q6k_multi_kernel<XT, YT, Q6M2One<1>>) : go(gemv_q6k_multi_kernel<XT, YT, Q6M2One<2>>); break;
     case 3: one ? go(gemv_q6k_multi_kernel<XT, YT, Q6M4One<1>>) : go(gemv_q6k_multi_kernel<XT, YT, Q6M4One<2>>); break;
-    default: go(gemv_q6k_multi_kernel<XT, YT, Q6M2Wide>); break;
+    case 4: go(gemv_q6k_multi_kernel<XT, YT, Q6M2Wide>); break;
+    default: go(gemv_q6k_multi_kernel<XT, YT, Q6M4Wide>); break;
   }
   return hipGetLastError();
 }

@@ -214,7 +214,7 @@ def test_streamed_two_to_four_rows_do_not_leak_and_output_types():
 @pytest.mark.parametrize("xk", ["bf16", "f16"])
 @pytest.mark.parametrize("m", [2, 3, 4])
 @pytest.mark.parametrize("n_out,n_in", [(4096, 4096), (8192 + 16 * 37, 2048), (16384 + 16 * 5, 4096), (4096, 14336),
-                                        (4096 + 16 * 3, 6144), (164800, 2048)])
+                                        (4096 + 16 * 3, 6144), (164800, 2048), (8192 + 16 * 5, 14336)])
 def test_q6k_streamed_two_to_four_rows(xk, m, n_out, n_in):
     """Random block bytes.  Normal activations with uneven magnitudes, another scale per token: every token
     within 1e-3 of the float64 product and, to summation order, equal to the single-row kernel on that token.
