@@ -252,6 +252,31 @@ def test_q6k_streamed_two_to_four_rows(xk, m, n_out, n_in):
             assert np.array_equal(y[t][rows][nz].view(np.uint32), col[nz].view(np.uint32)), (t, cols[t])
 
 
+@pytest.mark.parametrize("m,n_out,n_in", [(5, 4096 + 16, 4096), (8, 16384 + 16 * 5, 4096), (7, 8192 + 16, 2048),
+                                         (6, 4096, 14336), (4, 24576 + 16 * 9, 14336), (2, 24576 + 16 * 9, 14336)])
+def test_q6k_streamed_more_rows_and_more_groups(m, n_out, n_in):
+    """Five to eight rows (two passes of four, the second one ragged) and more row groups than a workgroup keeps
+    totals for (more workgroups than compute units): sampled rows against the float64 product and against the
+    single-row kernel."""
+    rng = np.random.default_rng(n_out + n_in + m)
+    p = random_blocks(F.Q6_K, n_out * (n_in // 256), seed=80 + m)
+    rows = np.unique(np.concatenate([rng.integers(0, n_out, 600), np.arange(n_out - 48, n_out), np.arange(48)]))
+    what = oracle.dequant(F.Q6_K, np.ascontiguousarray(p.reshape(n_out, -1)[rows]), rows.size, n_in)
+    wd = packed_to_dev(p)
+    x = Q.fill_normal(81 + m, 1, 1.0, m * n_in).reshape(m, n_in)
+    for t in range(m):
+        x[t] *= (1.0, 1e-4, 300.0, 7.0, 0.03, 55.0, 1e3, 2.0)[t]
+        x[t, t::13] *= 31.0
+    xd, xf = x_to_dev(x, "bf16")
+    y = QL.gemv(F.Q6_K, wd, xd, n_out, n_in).cpu().numpy()
+    want = oracle.linear_f64(what, xf)
+    for t in range(m):
+        assert rel_l2(y[t][rows], want[t]) <= TOL, t
+    for t in {0, m // 2, m - 1}:
+        y1 = QL.gemv(F.Q6_K, wd, xd[t:t + 1], n_out, n_in).cpu().numpy()[0]
+        assert rel_l2(y[t], y1) <= 2e-6, t
+
+
 def test_q6k_streamed_two_to_four_rows_do_not_leak_and_output_types():
     """A row of zeros, a row with an Inf, a tiny row beside an ordinary one; bias and 16-bit outputs through the
     layer entry point; quantized (not random) blocks."""
