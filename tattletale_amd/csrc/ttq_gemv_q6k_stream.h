@@ -25,7 +25,9 @@
 //   * along K a round is split: wavefront w multiplies block w of the eight for all 16 rows, two units of
 //     16 rows x 128 weights, two v_mfma_i32_16x16x64_i8 each;
 //   * rows of 4096 values and many of them (the LM head): two workgroups per compute unit with two buffers
-//     each, so that one's arithmetic falls into the other's waits; otherwise one workgroup with three buffers.
+//     each, so that one's arithmetic falls into the other's waits; otherwise one workgroup with three buffers;
+//   * rows of 2048 or 4096 values: a group is one or two rounds and a wavefront's place in them never changes, so
+//     the activation operands and scales of its two or four units are read into registers once, not per unit.
 // Arithmetic.  The activations are block fixed point, 15 bits in two byte planes with one power-of-two scale
 // per 64 values.  A weight reaches the matrix core as the signed byte 4 * (q6 - 32) = ((q6 << 2) ^ 0x80), built
 // from the nibble and the bit pair with four instructions per dword.  The 16 columns of the MFMA that a GEMV

@@ -1,16 +1,16 @@
-// Decode GEMV for Q6_K weights and two to four activation rows at once (a few sequences, or the tokens a speculative
-// step verifies) on gfx950: one pass over the weight stream of the single-row kernel (ttq_gemv_q6k_stream.h) serves
-// all of them.
+// Decode GEMV for Q6_K weights and two to eight activation rows at once (a few sequences, or the tokens a
+// speculative step verifies) on gfx950: one pass over the weight stream of the single-row kernel
+// (ttq_gemv_q6k_stream.h) serves two or four of them.
 //
-// Operator: F.linear with a (2..4, n_in) activation (workspace/libtorch/src/abi/neural_nets.nim:64-81) over a weight
+// Operator: F.linear with a (2..8, n_in) activation (workspace/libtorch/src/abi/neural_nets.nim:64-81) over a weight
 // of GGUF Q6_K blocks.
 //
 // The stream is the single-row kernel's: rounds of eight blocks of one group of 16 rows land in LDS buffers as 28
-// requests of 1 KiB, every block moved to a 16-byte boundary and the rows rotated against each other; wavefront w
-// multiplies block w of the round.  What changes is the activation operand.  The single-row kernel spends the 16
-// rows of a v_mfma_i32_16x16x64_i8 on (k-set, plane, sub-block) and adds the two k-sets of a unit into one
-// accumulator.  Here a row is (token of a pair, plane, sub-block): each of a unit's two MFMAs covers one k-set for
-// two tokens, and a second pair of tokens takes two MFMAs more.  Accumulator lane (n, g) then holds the four
+// requests of 1 KiB, every block moved to a 16-byte boundary and the rows rotated against each other; every
+// wavefront multiplies one block of the round.  What changes is the activation operand.  The single-row kernel
+// spends the 16 rows of a v_mfma_i32_16x16x64_i8 on (k-set, plane, sub-block) and adds the two k-sets of a unit into
+// one accumulator.  Here a row is (token of a pair, plane, sub-block): each of a unit's two MFMAs covers one k-set
+// for two tokens, and a second pair of tokens takes two MFMAs more.  Accumulator lane (n, g) then holds the four
 // sub-block sums of weight row n, token g / 2 of the pair, plane g % 2 -- the four that the k-set's four scale bytes
 // weigh -- so the weights are unpacked once for all tokens and only the short scale arithmetic is per token.
 //
@@ -18,6 +18,11 @@
 // LDS beside the tokens' plane tables, so they are added up on the way: at the end of a group every wavefront leaves
 // its sums in one of two small exchange areas, and at the end of the next group -- two or more barriers later -- one
 // wavefront (they take turns) adds the eight in a fixed order into the group's totals.
+//
+// Rows of 2048 or 4096 values: a wavefront's place in a group's rounds never changes, so its activation operands
+// live in registers.  Longer rows read them from LDS every unit; with four tokens their tables do not fit for a
+// whole row, and K is streamed in parts of 8192 values, each with tables of its own, one part on top of the other
+// in the totals.
 #include "ttq_gemv_q6k_stream.h"
 
 namespace ttq {
