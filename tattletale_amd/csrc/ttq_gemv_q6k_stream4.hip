@@ -69,11 +69,10 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
   __shared__ __attribute__((aligned(16))) float fac[TOK * CFG::NBMAX * 8];
   __shared__ __attribute__((aligned(16))) float stage[2][kQ6Waves][TOK][16];
   __shared__ __attribute__((aligned(16))) float total[CFG::MAXG][TOK][16];
-  // The raw activations land in stream buffers.  One part: in those the first round does not use, which is
-  // requested before the tables are built.  Several parts: anywhere, and the stream starts behind the tables.
-  constexpr int kStageBufs = KP == 1 ? kBufs - 1 : kBufs;
-  static_assert(kStageBufs * kQ6BufBytes >= TOK * CFG::NBMAX * 512, "room for the staged activations");
-  uint8_t* xstage = wbuf + (kBufs - kStageBufs) * kQ6BufBytes;
+  // The raw activations land where their planes will be: 16 values are 32 bytes either way, and the two threads
+  // that turn them into two entries of 16 bytes are neighbours in one wavefront, which has read before it writes.
+  // So the stream buffers are free from the start.  (The tables are written from inline asm like everything else
+  // that requests land in: the compiler would wait for every request in flight first.)
 
   const int n_in = nb * 256;
   const uint32_t row_bytes = (uint32_t)nb * 210u;
@@ -124,7 +123,7 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
       const int k0 = 8 * tid + i * (8 * kQ6Threads);
       if (k0 < n_in_p)                                    // whole wavefronts: the part is a multiple of 512
         __builtin_amdgcn_global_load_lds((sm_gptr_t)(xt + k0),
-                                         (sm_lptr_t)(xstage + t * (CFG::NBMAX * 512) + i * (16 * kQ6Threads) + wave * 1024),
+                                         (sm_lptr_t)(xa + t * kXaTok + kXaHead + i * (16 * kQ6Threads) + wave * 1024),
                                          16, 0, 0);
     }
   }
@@ -152,18 +151,15 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
       req_src += 16u * row_bytes - (uint32_t)rpg * (kQ6RoundBlocks * 210);
     }
   };
-  if constexpr (KP == 1) {
-    // one round now (into the first buffer: the activations sit in the others), the rest once the tables are built
-    request_next();
-    wait_rounds(I1{});
-  } else {
-    wait_rounds(I0{});
-  }
+  // One round now, the others once the tables are built: a compute unit takes about 64 KiB of outstanding requests,
+  // and a wavefront that asks for more sits in the request -- with the activations still unprocessed behind it.
+  request_next();
+  wait_rounds(I1{});
 
   // ---- the raw activations back into registers (each wavefront reads what it asked for), then into byte planes
   if (tid < 128) {
 #pragma unroll
-    for (int t = 0; t < TOK; t++) reinterpret_cast<uint32_t*>(xa + t * kXaTok)[tid] = 0u;
+    for (int t = 0; t < TOK; t++) sm_write_b32(sm_lds(xa) + (uint32_t)(t * kXaTok + 4 * tid), 0u);
   }
 #pragma unroll
   for (int t = 0; t < TOK; t++) {
@@ -172,7 +168,8 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
       const int k0 = 8 * tid + i * (8 * kQ6Threads);
       if (k0 >= n_in_p) break;
       float xf[8];
-      const sm_u32x4 r = sm_read16(sm_lds(xstage) + (uint32_t)(t * (CFG::NBMAX * 512) + i * (16 * kQ6Threads) + tid * 16));
+      const uint32_t tab = sm_lds(xa) + (uint32_t)(t * kXaTok + kXaHead);
+      const sm_u32x4 r = sm_read16(tab + (uint32_t)(i * (16 * kQ6Threads) + tid * 16));
       widen8<XT>(make_uint4(r[0], r[1], r[2], r[3]), xf);
       float amax = 0.f;
 #pragma unroll
@@ -194,10 +191,9 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
         lo[j] = v;                     // only the low byte is used, as a signed byte
       }
       // entry (k / 16, plane), 16 bytes; this thread's eight values are one half of it
-      uint2* xa8 = reinterpret_cast<uint2*>(xa + t * kXaTok + kXaHead);
-      const int e = (k0 >> 4) * 4 + ((k0 >> 3) & 1);
-      xa8[e] = make_uint2(pack_low_bytes(hi[0], hi[1], hi[2], hi[3]), pack_low_bytes(hi[4], hi[5], hi[6], hi[7]));
-      xa8[e + 2] = make_uint2(pack_low_bytes(lo[0], lo[1], lo[2], lo[3]), pack_low_bytes(lo[4], lo[5], lo[6], lo[7]));
+      const uint32_t e = tab + (uint32_t)((k0 >> 4) * 32 + ((k0 >> 3) & 1) * 8);
+      sm_write_b64(e, pack_low_bytes(hi[0], hi[1], hi[2], hi[3]), pack_low_bytes(hi[4], hi[5], hi[6], hi[7]));
+      sm_write_b64(e + 16u, pack_low_bytes(lo[0], lo[1], lo[2], lo[3]), pack_low_bytes(lo[4], lo[5], lo[6], lo[7]));
       // the weights arrive as 4 * (q - 32): a quarter of the scale; the high plane counts 256
       if ((tid & 7) == 0) {
         const int k64 = k0 >> 6;       // unit k64 / 2, k-set k64 % 2
@@ -234,9 +230,9 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
   const uint32_t total_base = sm_lds(&total[0][0][0]);
   const uint32_t stage_addr = stage_base + (uint32_t)((wave * TOK + (g >> 1)) * 64 + 4 * n);
 
-  sm_barrier();                         // the plane tables are complete, the staged activations read
+  sm_barrier();                         // the plane tables are complete
 #pragma unroll
-  for (int i = KP == 1 ? 1 : 0; i < kBufs; i++)
+  for (int i = 1; i < kBufs; i++)
     if (i < nrounds) request_next();
 
   // the eight wavefronts' sums of group `grp` (complete since a barrier) -> its totals, in wavefront order

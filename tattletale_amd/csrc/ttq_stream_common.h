@@ -28,6 +28,14 @@ __device__ __forceinline__ sm_u32x4 sm_read16(uint32_t a) {
   asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(a) : "memory");
   return v;
 }
+__device__ __forceinline__ void sm_write_b32(uint32_t a, uint32_t v) {
+  asm volatile("ds_write_b32 %0, %1" ::"v"(a), "v"(v) : "memory");
+}
+__device__ __forceinline__ void sm_write_b64(uint32_t a, uint32_t lo, uint32_t hi) {
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+  const u32x2 v = {lo, hi};
+  asm volatile("ds_write_b64 %0, %1" ::"v"(a), "v"(v) : "memory");
+}
 __device__ __forceinline__ void sm_write_f32(uint32_t a, float v) {
   asm volatile("ds_write_b32 %0, %1" ::"v"(a), "v"(v) : "memory");
 }
