@@ -155,6 +155,10 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
   // and a wavefront that asks for more sits in the request -- with the activations still unprocessed behind it.
   request_next();
   wait_rounds(I1{});
+  // Long rows: the activations have landed, and their share of what the compute unit has in flight goes to a
+  // second round (measured on short rows, whose activations are a quarter of a round: slower by 0.2 - 0.4 us).
+  constexpr int kEarlyRounds = RPG == 0 && kBufs > 2 ? 2 : 1;
+  if (kEarlyRounds > 1 && 1 < nrounds) request_next();
 
   // ---- the raw activations back into registers (each wavefront reads what it asked for), then into byte planes
   if (tid < 128) {
@@ -232,7 +236,7 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
 
   sm_barrier();                         // the plane tables are complete
 #pragma unroll
-  for (int i = 1; i < kBufs; i++)
+  for (int i = kEarlyRounds; i < kBufs; i++)
     if (i < nrounds) request_next();
 
   // the eight wavefronts' sums of group `grp` (complete since a barrier) -> its totals, in wavefront order
