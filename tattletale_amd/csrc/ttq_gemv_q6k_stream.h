@@ -192,18 +192,18 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
     const float mul = __uint_as_float((267u - ec) << 23);  // 2^(13-E)
     // non-finite activations poison their 64 values instead of being clipped
     const float f = eb == 255u ? __uint_as_float(0x7FC00000u) : __uint_as_float((ec - 13u) << 23);
-    int hi[8], lo[8];
+    // v = rint(x * 2^(13-E)) read off the low bits of x * 2^(13-E) + 1.5 * 2^23; the planes are byte 1 of
+    // v + 128 (the high one: (v + 128) >> 8) and byte 0 of v (the low one, a signed byte)
+    uint32_t vb[8];
 #pragma unroll
-    for (int j = 0; j < 8; j++) {
-      const int v = (int)rintf(xf[j] * mul);
-      hi[j] = (v + 128) >> 8;
-      lo[j] = v;                     // only the low byte is used, as a signed byte
-    }
+    for (int j = 0; j < 8; j++) vb[j] = __float_as_uint(fmaf_(xf[j], mul, __uint_as_float(kRoundMagicBits)));
     // entry (k / 16, plane), 16 bytes; this thread's eight values are one half of it
     uint2* xa8 = reinterpret_cast<uint2*>(&xa[0]);
     const int e = (k0 >> 4) * 4 + ((k0 >> 3) & 1);
-    xa8[e] = make_uint2(pack_low_bytes(hi[0], hi[1], hi[2], hi[3]), pack_low_bytes(hi[4], hi[5], hi[6], hi[7]));
-    xa8[e + 2] = make_uint2(pack_low_bytes(lo[0], lo[1], lo[2], lo[3]), pack_low_bytes(lo[4], lo[5], lo[6], lo[7]));
+    xa8[e] = make_uint2(pack_bytes1(vb[0] + 128u, vb[1] + 128u, vb[2] + 128u, vb[3] + 128u),
+                        pack_bytes1(vb[4] + 128u, vb[5] + 128u, vb[6] + 128u, vb[7] + 128u));
+    xa8[e + 2] = make_uint2(pack_low_bytes((int)vb[0], (int)vb[1], (int)vb[2], (int)vb[3]),
+                            pack_low_bytes((int)vb[4], (int)vb[5], (int)vb[6], (int)vb[7]));
     // the weights arrive as 4 * (q - 32): a quarter of the scale; the high plane counts 256
     if ((tid & 7) == 0) {
       fac[(k0 >> 6) * 2] = f * 64.f;
