@@ -25,6 +25,29 @@ __device__ __forceinline__ float dpp_quad(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
 }
 
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_quad_u32(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, false);
+}
+// lane i of every eight gets lane 7 - i (row_half_mirror): with quads that already agree, the other quad's value
+__device__ __forceinline__ uint32_t dpp_other_quad_u32(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xF, 0xF, false);
+}
+
+// max |f| as the bit pattern of a non-negative float.  Integer compares on purpose: a NaN, which fmaxf would
+// drop, counts as larger than infinity, so its exponent field (255) poisons the block as infinity's does.
+template <int N>
+__device__ __forceinline__ uint32_t amax_bits(const float (&f)[N]) {
+  uint32_t a = 0u;
+#pragma unroll
+  for (int i = 0; i < N; i++) {
+    const uint32_t b = __float_as_uint(f[i]) & 0x7FFFFFFFu;
+    a = a > b ? a : b;
+  }
+  return a;
+}
+__device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
+
 template <typename XT> __device__ __forceinline__ void widen8(const uint4& v, float (&f)[8]);
 template <> __device__ __forceinline__ void widen8<bf16_tag>(const uint4& v, float (&f)[8]) {
   const uint32_t d[4] = {v.x, v.y, v.z, v.w};

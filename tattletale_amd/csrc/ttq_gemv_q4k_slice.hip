@@ -121,10 +121,7 @@ gemv_q4k_slice_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
 #pragma unroll
         for (int i = 0; i < 8; i++) xf[8 * c + i] = t[i];
       }
-      float amax = 0.f;
-#pragma unroll
-      for (int i = 0; i < 32; i++) amax = fmaxf(amax, fabsf(xf[i]));
-      const uint32_t eb = __float_as_uint(amax) >> 23;      // biased exponent (amax >= 0)
+      const uint32_t eb = amax_bits(xf) >> 23;              // biased exponent of max |x|; 255 for Inf and NaN
       const uint32_t ec = eb < 18u ? 18u : eb;              // 2^(E-13) / 16 stays a normal number
       const float mul = __uint_as_float((267u - ec) << 23);  // 2^(13-E)
       // non-finite activations poison the sub-block instead of being clipped

@@ -142,13 +142,11 @@ gemv_q4k_stream4_kernel(const uint8_t* __restrict__ w, const uint16_t* __restric
       const st_u32x4 r = st_read1((uint32_t)(size_t)(st_lptr_t)(land(p)) + (uint32_t)(lane * 16));
       float xf[8];
       widen8<XT>(make_uint4(r[0], r[1], r[2], r[3]), xf);
-      float amax = 0.f;
-#pragma unroll
-      for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(xf[i]));
+      uint32_t amax = amax_bits(xf);
       // the four threads of a sub-block are an aligned quad
-      amax = fmaxf(amax, dpp_quad<0xB1>(amax));
-      amax = fmaxf(amax, dpp_quad<0x4E>(amax));
-      const uint32_t eb = __float_as_uint(amax) >> 23;      // biased exponent (amax >= 0)
+      amax = umax(amax, dpp_quad_u32<0xB1>(amax));
+      amax = umax(amax, dpp_quad_u32<0x4E>(amax));
+      const uint32_t eb = amax >> 23;                       // biased exponent of max |x|; 255 for Inf and NaN
       const uint32_t ec = eb < 18u ? 18u : eb;              // 2^(E-13) / 16 stays a normal number
       const float mul = __uint_as_float((267u - ec) << 23);  // 2^(13-E)
       // non-finite activations poison the sub-block instead of being clipped

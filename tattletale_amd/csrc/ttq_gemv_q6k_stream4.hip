@@ -175,14 +175,12 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
       const uint32_t tab = sm_lds(xa) + (uint32_t)(t * kXaTok + kXaHead);
       const sm_u32x4 r = sm_read16(tab + (uint32_t)(i * (16 * kQ6Threads) + tid * 16));
       widen8<XT>(make_uint4(r[0], r[1], r[2], r[3]), xf);
-      float amax = 0.f;
-#pragma unroll
-      for (int j = 0; j < 8; j++) amax = fmaxf(amax, fabsf(xf[j]));
+      uint32_t amax = amax_bits(xf);
       // the eight threads of 64 values are an aligned octet
-      amax = fmaxf(amax, dpp_quad<0xB1>(amax));
-      amax = fmaxf(amax, dpp_quad<0x4E>(amax));
-      amax = fmaxf(amax, __shfl_xor(amax, 4, kWave));
-      const uint32_t eb = __float_as_uint(amax) >> 23;       // biased exponent (amax >= 0)
+      amax = umax(amax, dpp_quad_u32<0xB1>(amax));
+      amax = umax(amax, dpp_quad_u32<0x4E>(amax));
+      amax = umax(amax, dpp_other_quad_u32(amax));
+      const uint32_t eb = amax >> 23;                        // biased exponent of max |x|; 255 for Inf and NaN
       const uint32_t ec = eb < 18u ? 18u : eb;               // 2^(E-13) / 4 stays a normal number
       const float mul = __uint_as_float((267u - ec) << 23);  // 2^(13-E)
       // non-finite activations poison their 64 values instead of being clipped

@@ -252,13 +252,11 @@ gemv_q8_stream_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, Y
       if (k0 >= n_in) break;
       float xf[8];
       ST::read(sm_lds(xstage) + (uint32_t)(i * kPassBytes + tid * 16), 16u * kQ8Threads, xf);
-      float amax = 0.f;
-#pragma unroll
-      for (int j = 0; j < 8; j++) amax = fmaxf(amax, fabsf(xf[j]));
+      uint32_t amax = amax_bits(xf);
       // the four threads of a block are an aligned quad
-      amax = fmaxf(amax, dpp_quad<0xB1>(amax));
-      amax = fmaxf(amax, dpp_quad<0x4E>(amax));
-      const uint32_t eb = __float_as_uint(amax) >> 23;       // biased exponent (amax >= 0)
+      amax = umax(amax, dpp_quad_u32<0xB1>(amax));
+      amax = umax(amax, dpp_quad_u32<0x4E>(amax));
+      const uint32_t eb = amax >> 23;                        // biased exponent of max |x|; 255 for Inf and NaN
       // |v| < 2^(S+1) with S = 13 (two planes) or 21 (three); the scale 2^(E-S) stays a normal number
       constexpr uint32_t kS = kPlanes == 3 ? 21u : 13u;
       const uint32_t ec = eb < kS + 5u ? kS + 5u : eb;

@@ -162,13 +162,11 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
   for (int p = 0; p < XP; p++) {
     const int k0 = 8 * (tid + p * kMfmaThreads);
     if (k0 < n_in) {
-      float amax = 0.f;
-#pragma unroll
-      for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(xf[t][p][i]));
+      uint32_t amax = amax_bits(xf[t][p]);
       // the four threads of a block are an aligned quad
-      amax = fmaxf(amax, dpp_quad<0xB1>(amax));
-      amax = fmaxf(amax, dpp_quad<0x4E>(amax));
-      const uint32_t eb = __float_as_uint(amax) >> 23;            // biased exponent (amax >= 0)
+      amax = umax(amax, dpp_quad_u32<0xB1>(amax));
+      amax = umax(amax, dpp_quad_u32<0x4E>(amax));
+      const uint32_t eb = amax >> 23;                             // biased exponent of max |x|; 255 for Inf and NaN
       const uint32_t ec = eb < (uint32_t)(X::kShift + 1) ? (uint32_t)(X::kShift + 1) : eb;
       const float mul = __uint_as_float((254u + (uint32_t)X::kShift - ec) << 23);   // 2^(shift-E)
       // non-finite activations poison the block instead of being clipped

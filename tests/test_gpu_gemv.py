@@ -588,3 +588,23 @@ def test_q8_0_streamed_activation_extremes_bias_and_output_types():
         layer = QuantLinear.init(wd, F.Q8_0, n_in, n_out, bias=torch.from_numpy(bias).to(DEV))
         yy = layer.forward(xd1, out_dtype=out_dtype).float().cpu().numpy().reshape(-1)
         assert rel_l2(yy, want1) <= tol, out_dtype
+
+
+# ------------------------------------------------------------------- non-finite activations
+@pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
+@pytest.mark.parametrize("n_out,n_in", [(14336, 4096), (4096, 14336), (1024, 4096), (304, 1280), (32768 + 16, 2048)])
+def test_nan_and_inf_activations_make_their_row_non_finite_and_no_other(fmt, n_out, n_in):
+    """F.linear gives a row of NaN for an activation row that holds a NaN or an infinity.  The kernels that turn
+    activations into block fixed point take the block's exponent from max |x|: an infinity and -- which a
+    floating-point max would drop -- a NaN must both poison their block, for every kernel the shapes, the
+    activation types and the row counts below reach; the rows beside it stay finite."""
+    wd = packed_to_dev(random_blocks(fmt, n_out * (n_in // (32 if fmt == F.Q8_0 else 256)), seed=900 + n_in))
+    for xk in ("bf16", "f16", "f32"):
+        for m in (1, 2, 3, 4, 8):
+            for bad, col in ((np.nan, 777), (-np.inf, n_in - 1), (np.nan, 0)):
+                x = Q.fill_normal(901 + m, 1, 1.0, m * n_in).reshape(m, n_in)
+                x[m - 1, col] = bad
+                xd, _ = x_to_dev(x, xk)
+                y = QL.gemv(fmt, wd, xd, n_out, n_in).cpu().numpy()
+                assert not np.any(np.isfinite(y[m - 1])), (xk, m, bad, col)
+                assert np.all(np.isfinite(y[:m - 1])), (xk, m, bad, col)

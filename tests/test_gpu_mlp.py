@@ -361,3 +361,23 @@ def test_fused_gemm_full_shape_llama3_8b_ffn():
     want = oracle.silu_and_mul_f64(oracle.linear_f64(what, xf[tok]))
     got = oracle.bf16_to_f32(dev_bits(y[torch.from_numpy(tok).to(DEV)][:, torch.from_numpy(outs).to(DEV)]))
     assert rel_l2(got, want) <= 2e-2
+
+
+@pytest.mark.parametrize("n_ff,n_in", [(14336, 4096), (2048, 2048), (1000, 1280)])
+def test_fused_gate_up_non_finite_activations(n_ff, n_in):
+    """A NaN or an infinity among the activations of a row: that row of silu(gate) * up is not finite, the rows
+    beside it are (one to five rows: the single-row, the two-to-four-row and the leftover forms)."""
+    wd = packed_to_dev(random_blocks(F.Q4_K, 2 * n_ff * (n_in // 256), seed=77))
+    for xk in ("bf16", "f16"):
+        for m in (1, 2, 4, 5):
+            for bad in (np.nan, np.inf):
+                x = Q.fill_normal(78 + m, 1, 1.0, m * n_in).reshape(m, n_in)
+                x[m - 1, 300] = bad
+                xd, _ = x_to_dev(x, xk)
+                try:
+                    y = QL.gemv_q4_k_silu_mul(wd, xd, n_ff, n_in).float().cpu().numpy()
+                except TtqError as e:
+                    assert e.status == F.ERR_UNSUPPORTED
+                    continue
+                assert not np.any(np.isfinite(y[m - 1])), (xk, m, bad)
+                assert np.all(np.isfinite(y[:m - 1])), (xk, m, bad)
