@@ -608,3 +608,25 @@ def test_nan_and_inf_activations_make_their_row_non_finite_and_no_other(fmt, n_o
                 y = QL.gemv(fmt, wd, xd, n_out, n_in).cpu().numpy()
                 assert not np.any(np.isfinite(y[m - 1])), (xk, m, bad, col)
                 assert np.all(np.isfinite(y[:m - 1])), (xk, m, bad, col)
+
+
+@pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
+@pytest.mark.parametrize("n_out,n_in", [(14336, 4096), (4096, 14336), (1024, 4096)])
+def test_non_finite_block_scale_reaches_its_output_row_only(fmt, n_out, n_in):
+    """A block whose fp16 scale d is an infinity or a NaN (a damaged file): the dequantized weights of that block
+    are not finite, so F.linear's output for that weight row is not finite -- and every other output is.  Decode
+    kernels for one to eight activation rows and the prefill kernels for 40."""
+    nbytes, per = {F.Q8_0: (34, 32), F.Q4_K: (144, 256), F.Q6_K: (210, 256)}[fmt]
+    row = 37
+    for hi_byte in (0x7C, 0xFE):                   # +inf, a NaN
+        p = random_blocks(fmt, n_out * (n_in // per), seed=910).reshape(-1, nbytes).copy()
+        blk = row * (n_in // per) + 3
+        off = 208 if fmt == F.Q6_K else 0
+        p[blk, off], p[blk, off + 1] = 0, hi_byte
+        wd = packed_to_dev(p.reshape(-1))
+        for m in (1, 2, 4, 8, 40):
+            xd, _ = x_to_dev(Q.fill_normal(911 + m, 1, 1.0, m * n_in).reshape(m, n_in), "bf16")
+            y = (QL.gemv(fmt, wd, xd, n_out, n_in) if m <= 8 else QL.gemm(fmt, wd, xd, n_out, n_in).float()).cpu().numpy()
+            bad = np.nonzero(~np.isfinite(y).all(axis=0))[0]
+            assert bad.tolist() == [row], (hex(hi_byte), m)
+            assert not np.any(np.isfinite(y[:, row])), (hex(hi_byte), m)
