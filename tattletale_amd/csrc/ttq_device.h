@@ -112,10 +112,25 @@ __device__ __forceinline__ uint16_t load2(const uint8_t* p) {
   return v;
 }
 
+// v[i] + v[i ^ 16] and v[i] + v[i ^ 32] in every lane i, by gfx950's row swaps (v_permlane16_swap_b32,
+// v_permlane32_swap_b32: with the same register on both sides one result holds the even rows' -- the lower
+// half's -- values in every row, the other the odd rows' -- the upper half's): two vector-ALU instructions in
+// place of a trip through the LDS crossbar (__shfl_xor is ds_bpermute_b32), same sums bit for bit.
+__device__ __forceinline__ float add_xor16(float v) {
+  const auto s = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(s[0]) + __uint_as_float(s[1]);
+}
+__device__ __forceinline__ float add_xor32(float v) {
+  const auto s = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(s[0]) + __uint_as_float(s[1]);
+}
+
 // Sum over the 64 lanes of a wavefront; every lane gets the total.
 __device__ __forceinline__ float wave_sum(float v) {
+  v = add_xor32(v);
+  v = add_xor16(v);
 #pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+  for (int off = 8; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
   return v;
 }
 

@@ -200,8 +200,8 @@ gemv_exl3_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __restric
 #pragma unroll
   for (int t = 0; t < TOK; t++) {
     float a = acc[t][0] + acc[t][1];
-    a += __shfl_xor(a, 16, kWave);
-    a += __shfl_xor(a, 32, kWave);
+    a = add_xor16(a);
+    a = add_xor32(a);
     if (lane < 16) red[(t * kExl3Waves + wave) * 16 + lane] = a;
   }
   __syncthreads();

@@ -379,8 +379,8 @@ gemv_q4k_mfma_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__
     if (++csi == S) {
       // the row group is finished for this wavefront's slice: add the four k-groups
       float v = acc;
-      v += __shfl_xor(v, 16, kWave);
-      v += __shfl_xor(v, 32, kWave);
+      v = add_xor16(v);
+      v = add_xor32(v);
       if constexpr (FUSE) {
         // every wavefront ends its round after the same number of steps
         if (lane < 16) part[wave * 16 + n] = v;

@@ -293,8 +293,8 @@ gemv_q4k_slice_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
         for (int i = 0; i < UP; i++) request(i);
       }
       compute(rb2);
-      acc += __shfl_xor(acc, 16, kWave);
-      acc += __shfl_xor(acc, 32, kWave);
+      acc = add_xor16(acc);
+      acc = add_xor32(acc);
       if (lane < 16) part[rg * nks + ks][lane] = acc;
     };
     int rg = rg0;

@@ -417,8 +417,8 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
     }
     compute(rb2);
     // the four k-groups of a row
-    acc += __shfl_xor(acc, 16, kWave);
-    acc += __shfl_xor(acc, 32, kWave);
+    acc = add_xor16(acc);
+    acc = add_xor32(acc);
     if (lane < 16) part[blk][lane] = acc;
   };
   // (the first block apart from the loop: the compiler schedules the straight-line copy better)

@@ -465,7 +465,7 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
       // the group is complete: the two planes of a (row, token) are 16 lanes apart
 #pragma unroll
       for (int q = 0; q < kPairs; q++) {
-        acc[q] += __shfl_xor(acc[q], 16, kWave);
+        acc[q] = add_xor16(acc[q]);
         if ((g & 1) == 0) sm_write_f32(stage_addr + (uint32_t)((gi & 1) * kStageHalf + q * 128), acc[q]);
         acc[q] = 0.f;
       }

@@ -192,8 +192,8 @@ gemv_q8_mfma_kernel(const uint8_t* __restrict__ w, const typename Q8X<XT>::elem_
     }
     if (++csi == S) {
       float v = acc;
-      v += __shfl_xor(v, 16, kWave);
-      v += __shfl_xor(v, 32, kWave);
+      v = add_xor16(v);
+      v = add_xor32(v);
       if (cr < rounds) {
         if (sl_log2 == 0) {
           const int row = wg_row0 + (cr * G + gi) * 16 + n;

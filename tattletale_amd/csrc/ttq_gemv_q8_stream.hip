@@ -386,8 +386,8 @@ gemv_q8_stream_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, Y
     }
     if (++kr == rpg) {
       // the group is complete: the four accumulator lanes of a row
-      acc += __shfl_xor(acc, 16, kWave);
-      acc += __shfl_xor(acc, 32, kWave);
+      acc = add_xor16(acc);
+      acc = add_xor32(acc);
       if (lane < 16) sm_write_f32(part_addr + (uint32_t)(gi * (kQ8Waves * 16 * 4)), acc);
       acc = 0.f;
       kr = 0;

@@ -315,8 +315,8 @@ gemv_q8_win_kernel(const uint8_t* __restrict__ w, const typename Q8WX<XT>::elem_
 #pragma unroll
       for (int t = 0; t < TOK; t++) {
         float v = acc[t];
-        v += __shfl_xor(v, 16, kWave);
-        v += __shfl_xor(v, 32, kWave);
+        v = add_xor16(v);
+        v = add_xor32(v);
         if (cr < rounds) {
           if (sl_log2 == 0) {
             if (lane < 16) store_row(wg_row0 + (cr * G + gi) * 16 + n, t, v);
