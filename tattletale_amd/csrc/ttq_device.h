@@ -125,12 +125,41 @@ __device__ __forceinline__ float add_xor32(float v) {
   return __uint_as_float(s[0]) + __uint_as_float(s[1]);
 }
 
+// The value of lane (lane ^ D), D a power of two up to 32, without the LDS crossbar that __shfl_xor
+// (ds_bpermute_b32) goes through: DPP moves inside a row of 16 lanes -- quad permutes for 1 and 2, a reversal
+// of eight lanes followed by a reversal of each quad for 4, a rotation by 8 for 8 -- and gfx950's row swaps
+// for 16 and 32.  (Each form was checked against __shfl_xor on the GPU.)
+template <int D>
+__device__ __forceinline__ float lane_xor(float v, int lane) {
+  static_assert(D == 1 || D == 2 || D == 4 || D == 8 || D == 16 || D == 32, "a power of two inside the wavefront");
+  const int b = __float_as_int(v);
+  if constexpr (D == 1) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(b, b, 0xB1, 0xF, 0xF, false));      // quad_perm [1, 0, 3, 2]
+  } else if constexpr (D == 2) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(b, b, 0x4E, 0xF, 0xF, false));      // quad_perm [2, 3, 0, 1]
+  } else if constexpr (D == 4) {
+    const int t = __builtin_amdgcn_update_dpp(b, b, 0x141, 0xF, 0xF, false);              // row_half_mirror: i -> 7 - i
+    return __int_as_float(__builtin_amdgcn_update_dpp(t, t, 0x1B, 0xF, 0xF, false));      // quad_perm [3, 2, 1, 0]
+  } else if constexpr (D == 8) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(b, b, 0x128, 0xF, 0xF, false));     // row_ror:8
+  } else if constexpr (D == 16) {
+    const auto s = __builtin_amdgcn_permlane16_swap((unsigned)b, (unsigned)b, false, false);
+    return __uint_as_float((lane & 16) ? s[0] : s[1]);
+  } else {
+    const auto s = __builtin_amdgcn_permlane32_swap((unsigned)b, (unsigned)b, false, false);
+    return __uint_as_float((lane & 32) ? s[0] : s[1]);
+  }
+}
+
 // Sum over the 64 lanes of a wavefront; every lane gets the total.
 __device__ __forceinline__ float wave_sum(float v) {
+  const int lane = (int)(threadIdx.x & 63u);
   v = add_xor32(v);
   v = add_xor16(v);
-#pragma unroll
-  for (int off = 8; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+  v += lane_xor<8>(v, lane);
+  v += lane_xor<4>(v, lane);
+  v += lane_xor<2>(v, lane);
+  v += lane_xor<1>(v, lane);
   return v;
 }
 

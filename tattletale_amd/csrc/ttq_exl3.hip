@@ -236,15 +236,12 @@ hadamard128_kernel(float* __restrict__ v, const uint16_t* __restrict__ pre,
     a[h] = v[idx];
     if (pre) a[h] *= f16_bits_to_f32(pre[ch[h]]);
   }
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const bool upper = (lane & d) != 0;
-#pragma unroll
-    for (int h = 0; h < 2; h++) {
-      const float o = __shfl_xor(a[h], d, kWave);
-      a[h] = upper ? (o - a[h]) : (a[h] + o);
-    }
-  }
+  fwht_lane_stage<1>(a, lane);
+  fwht_lane_stage<2>(a, lane);
+  fwht_lane_stage<4>(a, lane);
+  fwht_lane_stage<8>(a, lane);
+  fwht_lane_stage<16>(a, lane);
+  fwht_lane_stage<32>(a, lane);
   const float lo = a[0] + a[1], hi = a[0] - a[1];
   a[0] = lo;
   a[1] = hi;

@@ -30,21 +30,26 @@ struct Codebook {
 // (value index = 4*lane + i): stages 1 and 2 inside the lane, stages 4..64 against the lane
 // 1, 2, 4, 8, 16 away.  Same stage order and operand order as the textbook loop
 // (lower index gets a+b, upper a-b), so the results do not depend on how it is laid out.
+template <int D, int N>
+__device__ __forceinline__ void fwht_lane_stage(float (&v)[N], int lane) {
+  const bool upper = (lane & D) != 0;
+#pragma unroll
+  for (int i = 0; i < N; i++) {
+    const float o = lane_xor<D>(v[i], lane);
+    v[i] = upper ? (o - v[i]) : (v[i] + o);
+  }
+}
 __device__ __forceinline__ void fwht128_quad(float (&v)[4], int lane) {
   float t;
   t = v[0]; v[0] = t + v[1]; v[1] = t - v[1];
   t = v[2]; v[2] = t + v[3]; v[3] = t - v[3];
   t = v[0]; v[0] = t + v[2]; v[2] = t - v[2];
   t = v[1]; v[1] = t + v[3]; v[3] = t - v[3];
-#pragma unroll
-  for (int d = 1; d < 32; d <<= 1) {
-    const bool upper = (lane & d) != 0;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const float o = __shfl_xor(v[i], d, kWave);
-      v[i] = upper ? (o - v[i]) : (v[i] + o);
-    }
-  }
+  fwht_lane_stage<1>(v, lane);
+  fwht_lane_stage<2>(v, lane);
+  fwht_lane_stage<4>(v, lane);
+  fwht_lane_stage<8>(v, lane);
+  fwht_lane_stage<16>(v, lane);
 }
 
 // Four consecutive activations (a multiple of four elements from the row start) as floats.

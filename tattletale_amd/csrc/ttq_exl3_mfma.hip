@@ -115,8 +115,11 @@ gemv_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __re
         v[3] *= f16_bits_to_f32((uint16_t)(sv[it].y >> 16));
         fwht128_quad(v, lane);
         float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
-#pragma unroll
-        for (int d = 1; d < 32; d <<= 1) amax = fmaxf(amax, __shfl_xor(amax, d, kWave));
+        amax = fmaxf(amax, lane_xor<1>(amax, lane));
+        amax = fmaxf(amax, lane_xor<2>(amax, lane));
+        amax = fmaxf(amax, lane_xor<4>(amax, lane));
+        amax = fmaxf(amax, lane_xor<8>(amax, lane));
+        amax = fmaxf(amax, lane_xor<16>(amax, lane));
         // scale 2^(14 - exponent of amax); all-zero groups get the largest scale, which changes nothing
         int se = 268 - (int)((__float_as_uint(amax) >> 23) & 0xFF);
         se = se > 254 ? 254 : se;
@@ -210,7 +213,7 @@ gemv_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __re
   // is there (a bounded number of times: rows it gave up on come out as NaN), adds everything in a
   // fixed order, and leaves the words at zero for the next launch on the stream.
 #pragma unroll
-  for (int r = 0; r < 4; r++) acc[r] += __shfl_xor(acc[r], 1, kWave);
+  for (int r = 0; r < 4; r++) acc[r] += lane_xor<1>(acc[r], lane);
   const int tcol = wave & 7, kpart = wave >> 3;
   const bool owner = (col & 1) == 0 && (col >> 1) < ntok;      // this lane holds 4 channel sums of row col / 2
   constexpr int kPartWords = kXmTok * 128;                        // words per (slice, k part)
