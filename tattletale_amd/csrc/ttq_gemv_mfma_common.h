@@ -22,16 +22,17 @@ constexpr int kMaxWideSb = 32;                  // up to here the 4 KiB-per-supe
 
 template <int CTRL>
 __device__ __forceinline__ float dpp_quad(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
+  // (the lane's own value as the "old" operand: every lane has a source, and the compiler need not clear a register)
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, 0xF, 0xF, false));
 }
 
 template <int CTRL>
 __device__ __forceinline__ uint32_t dpp_quad_u32(uint32_t v) {
-  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, false);
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, 0xF, 0xF, false);
 }
 // lane i of every eight gets lane 7 - i (row_half_mirror): with quads that already agree, the other quad's value
 __device__ __forceinline__ uint32_t dpp_other_quad_u32(uint32_t v) {
-  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xF, 0xF, false);
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, 0x141, 0xF, 0xF, false);
 }
 
 // max |f| as the bit pattern of a non-negative float.  Integer compares on purpose: a NaN, which fmaxf would

@@ -236,8 +236,8 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
       lo[i] = v;                     // only the low byte is used
       vsum += v;
     }
-    vsum += __builtin_amdgcn_update_dpp(0, vsum, 0xB1, 0xF, 0xF, false);
-    vsum += __builtin_amdgcn_update_dpp(0, vsum, 0x4E, 0xF, 0xF, false);
+    vsum += __builtin_amdgcn_update_dpp(vsum, vsum, 0xB1, 0xF, 0xF, false);
+    vsum += __builtin_amdgcn_update_dpp(vsum, vsum, 0x4E, 0xF, 0xF, false);
     const int b = k0 >> 8, j = (k0 >> 5) & 7, h = (k0 >> 4) & 1, half8 = (k0 >> 3) & 1;
     const int e_hi = (b * 32 + 4 * j + h) * 2 + half8;
     uint2* xa8 = reinterpret_cast<uint2*>(&xa[0]);

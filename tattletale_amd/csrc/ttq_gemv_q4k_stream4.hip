@@ -159,8 +159,8 @@ gemv_q4k_stream4_kernel(const uint8_t* __restrict__ w, const uint16_t* __restric
         vacc += vb[i];
       }
       int vsum = (int)(vacc - 8u * kRoundMagicBits);
-      vsum += __builtin_amdgcn_update_dpp(0, vsum, 0xB1, 0xF, 0xF, false);
-      vsum += __builtin_amdgcn_update_dpp(0, vsum, 0x4E, 0xF, 0xF, false);
+      vsum += __builtin_amdgcn_update_dpp(vsum, vsum, 0xB1, 0xF, 0xF, false);
+      vsum += __builtin_amdgcn_update_dpp(vsum, vsum, 0x4E, 0xF, 0xF, false);
       // sum(x) as the fixed-point values give it: a row sum is the dot product with the quantized activations
       const float sum = (float)vsum * f;
       const int k0 = kc * 8;
