@@ -127,7 +127,9 @@ TTQ_API int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dt
  * (1, n_in) activation (neural_nets.nim:64).  n_in <= 32768 for Q4_K / Q6_K with 16-bit
  * activations, <= 16384 otherwise.  Two to four rows (a speculative step, a few sequences) of
  * 16-bit activations over a large Q4_K or Q6_K matrix cost about one pass over the weights, not
- * one per row; every row's result stays within the 1e-3 class of the single-row call. */
+ * one per row; every row's result stays within the 1e-3 class of the single-row call.  A NaN or
+ * an infinity among a row's activations, or in a block scale of a weight row, makes the outputs
+ * they reach non-finite, as F.linear on the dequantized weight would; other outputs are unaffected. */
 TTQ_API int ttq_gemv_q8_0(const void* w, const void* x, int x_dtype, float* y, int64_t m,
                   int64_t n_out, int64_t n_in, void* stream);
 TTQ_API int ttq_gemv_q4_k(const void* w, const void* x, int x_dtype, float* y, int64_t m,
