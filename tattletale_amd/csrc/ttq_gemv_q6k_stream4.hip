@@ -1,8 +1,8 @@
-// Decode GEMV for Q6_K weights and two to eight activation rows at once (a few sequences, or the tokens a
+// Decode GEMV for Q6_K weights and two or more activation rows at once (a few sequences, or the tokens a
 // speculative step verifies) on gfx950: one pass over the weight stream of the single-row kernel
-// (ttq_gemv_q6k_stream.h) serves two or four of them.
+// (ttq_gemv_q6k_stream.h) serves two or four of them; more rows take more passes.
 //
-// Operator: F.linear with a (2..8, n_in) activation (workspace/libtorch/src/abi/neural_nets.nim:64-81) over a weight
+// Operator: F.linear with a (2.., n_in) activation (workspace/libtorch/src/abi/neural_nets.nim:64-81) over a weight
 // of GGUF Q6_K blocks.
 //
 // The stream is the single-row kernel's: rounds of eight blocks of one group of 16 rows land in LDS buffers as 28
@@ -496,8 +496,8 @@ Q6MultiPlan q6_multi_plan(int64_t m, int64_t n_out, int64_t n_in) {
   Q6MultiPlan p{0, 0, 0};
   const Q6Plan single = q6_plan(n_out, n_in);              // the stream's own limits
   const int64_t nb = n_in / 256, groups = n_out / 16;
-  // two passes of four rows at most
-  static const int max_rows = dev_knob("TTQ_Q6_MULTI_MAX_ROWS", 8);
+  // (more than four rows: passes of four on gridDim.y; the entry points hand over 65535 rows at most)
+  static const int max_rows = dev_knob("TTQ_Q6_MULTI_MAX_ROWS", 65535);
   if (!single.ok || m < 2 || m > max_rows) return p;
   static_assert(Q6M4Wide::NBMAX * Q6M4Wide::KP >= Q6Wide::NBMAX && Q6M2Wide::NBMAX >= Q6Wide::NBMAX, "every row length of the stream");
   const int cus = device_num_cus();

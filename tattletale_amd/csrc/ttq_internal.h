@@ -99,7 +99,7 @@ hipError_t launch_gemv_q6k_stream(const void* w, const void* x, int x_dtype, voi
                                   const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                                   hipStream_t s);
 
-// The same stream for two to eight activation rows, two or four to a pass (ttq_gemv_q6k_stream4.hip).
+// The same stream for two or more activation rows, two or four to a pass (ttq_gemv_q6k_stream4.hip).
 bool gemv_q6k_stream4_supported(int format, int x_dtype, int64_t m, int64_t n_out, int64_t n_in);
 hipError_t launch_gemv_q6k_stream4(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
                                    const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,

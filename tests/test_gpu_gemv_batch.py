@@ -253,6 +253,7 @@ def test_q6k_streamed_two_to_four_rows(xk, m, n_out, n_in):
 
 
 @pytest.mark.parametrize("m,n_out,n_in", [(5, 4096 + 16, 4096), (8, 16384 + 16 * 5, 4096), (7, 8192 + 16, 2048),
+                                         (21, 4096 + 32, 4096), (13, 4096, 8192),
                                          (6, 4096, 14336), (4, 24576 + 16 * 9, 14336), (2, 24576 + 16 * 9, 14336)])
 def test_q6k_streamed_more_rows_and_more_groups(m, n_out, n_in):
     """Five to eight rows (two passes of four, the second one ragged) and more row groups than a workgroup keeps
@@ -265,7 +266,7 @@ def test_q6k_streamed_more_rows_and_more_groups(m, n_out, n_in):
     wd = packed_to_dev(p)
     x = Q.fill_normal(81 + m, 1, 1.0, m * n_in).reshape(m, n_in)
     for t in range(m):
-        x[t] *= (1.0, 1e-4, 300.0, 7.0, 0.03, 55.0, 1e3, 2.0)[t]
+        x[t] *= (1.0, 1e-4, 300.0, 7.0, 0.03, 55.0, 1e3, 2.0)[t % 8]
         x[t, t::13] *= 31.0
     xd, xf = x_to_dev(x, "bf16")
     y = QL.gemv(F.Q6_K, wd, xd, n_out, n_in).cpu().numpy()
