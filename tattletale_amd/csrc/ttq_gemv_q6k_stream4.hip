@@ -113,7 +113,7 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
   const int rpg = nbp >> 3;                               // rounds per group
   const int nrounds = rpg * ng;
 
-  // ---- the activations, as LDS requests: thread t stages values 8 t + 4096 i .. + 7 of every token's part
+  // ---- the activations, as LDS requests: thread t fetches values 8 t + 4096 i .. + 7 of every token's part
   constexpr int kXPasses = (CFG::NBMAX * 256 + 8 * kQ6Threads - 1) / (8 * kQ6Threads);
 #pragma unroll
   for (int t = 0; t < TOK; t++) {
