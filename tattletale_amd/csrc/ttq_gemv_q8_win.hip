@@ -418,8 +418,7 @@ bool gemv_q8_win_supported(int format, int64_t n_out, int64_t n_in) {
   static const int disabled = mfma_env_int("TTQ_GEMV_NO_MFMA", 0) || mfma_env_int("TTQ_GEMV_NO_Q8_WIN", 0);
   // whole chunks of 8 blocks (rows then start 16-byte aligned); plane tables within LDS; byte
   // offsets into the weight buffer are 32-bit in the kernel
-  // (from 1024 weight rows on: measured against the generic kernel at 1024x4096 5.3 / 6.0 us, 2000x4096 5.3 / 6.7,
-  // 1024x14336 12.4 / 17.7 and with four rows 13.6 / 38.0; at 512 rows the generic kernel wins with two rows or more)
+  // (from 1024 weight rows on; the dispatch sends small matrices with up to four activation rows elsewhere)
   return !disabled && format == kQ8_0 && n_out >= 1024 && n_in % 256 == 0 && n_in / 256 <= kQ8WinMaxChunks &&
          n_out * (n_in / 32) * 34 < ((int64_t)1 << 32);
 }
