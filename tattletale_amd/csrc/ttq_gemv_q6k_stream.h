@@ -75,7 +75,7 @@ template <typename XT, typename YT, typename CFG, int STAGE = 0>
 __global__ void __launch_bounds__(kQ6Threads) __attribute__((amdgpu_waves_per_eu(2 * CFG::WGS, 2 * CFG::WGS)))
 gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
                        const void* __restrict__ bias, int bias_dtype, int n_out, int nb_arg, int groups_per_wg,
-                       int groups_rem) {
+                       int groups_rem, int fold_log2) {
   constexpr int kBufs = CFG::BUFS, RPG = CFG::RPG;
   static_assert(RPG == 0 || CFG::NBMAX == 8 * RPG, "a fixed row length is the table's");
   const int nb = RPG > 0 ? CFG::NBMAX : nb_arg;
@@ -94,8 +94,13 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 15, g = lane >> 4;
-  const uint16_t* xm = x + (int64_t)blockIdx.y * n_in;
-  YT* ym = y + (int64_t)blockIdx.y * n_out;
+  // Folded rows (fold_log2 > 0): the matrix really has 2^fold_log2 times as many rows, of 2048 >> fold_log2 values
+  // each; consecutive rows are contiguous in memory, so 2^fold_log2 of them are streamed as one row of eight
+  // blocks against the activations repeated that often, and the wavefronts' sums are added per real row at the end.
+  const int x_len = n_in >> fold_log2;
+  const int x_mask = fold_log2 ? x_len - 1 : -1;          // (a folded length is a power of two)
+  const uint16_t* xm = x + (int64_t)blockIdx.y * x_len;
+  YT* ym = y + (((int64_t)blockIdx.y * n_out) << fold_log2);
   const int bx = blockIdx.x;
   const int grp0 = bx * groups_per_wg + min(bx, groups_rem);
   const int ng = groups_per_wg + (bx < groups_rem ? 1 : 0);            // 1 .. CFG::MAXG
@@ -108,7 +113,8 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   for (int i = 0; i < kXPasses; i++) {
     const int k0 = 8 * tid + i * (8 * kQ6Threads);
     if (k0 < n_in)                                        // whole wavefronts: n_in is a multiple of 512
-      __builtin_amdgcn_global_load_lds((sm_gptr_t)(xm + k0), (sm_lptr_t)(xstage + i * (16 * kQ6Threads) + wave * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((sm_gptr_t)(xm + (k0 & x_mask)),
+                                       (sm_lptr_t)(xstage + i * (16 * kQ6Threads) + wave * 1024), 16, 0, 0);
   }
   // a compute unit serves its requests in the order they were made: every wavefront's activation requests are
   // queued before any weight request of the workgroup
@@ -424,21 +430,41 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   else run_rounds(std::false_type{});
   // every request has landed (plain loads are safe again); the eight K-slices of a row add up in a fixed order
   __syncthreads();
-  for (int t = tid; t < ng * 16; t += kQ6Threads) {
-    const int grp = t >> 4, nn = t & 15;
-    float v = 0.f;
+  if (fold_log2 == 0) {
+    for (int t = tid; t < ng * 16; t += kQ6Threads) {
+      const int grp = t >> 4, nn = t & 15;
+      float v = 0.f;
 #pragma unroll
-    for (int wv = 0; wv < kQ6Waves; wv++) v += part[grp][wv][nn];
-    const int row = (grp0 + grp) * 16 + nn;
-    YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
+      for (int wv = 0; wv < kQ6Waves; wv++) v += part[grp][wv][nn];
+      const int row = (grp0 + grp) * 16 + nn;
+      YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
+    }
+  } else {
+    // real row fs of streamed row nn: the blocks of wavefronts fs * (8 >> fold_log2) ...
+    const int per = kQ6Waves >> fold_log2;
+    for (int t = tid; t < (ng * 16) << fold_log2; t += kQ6Threads) {
+      const int grp = t >> (4 + fold_log2), rem = t & ((16 << fold_log2) - 1);
+      const int nn = rem >> fold_log2, fs = rem & ((1 << fold_log2) - 1);
+      float v = 0.f;
+      for (int wv = fs * per; wv < (fs + 1) * per; wv++) v += part[grp][wv][nn];
+      const int row = (((grp0 + grp) * 16 + nn) << fold_log2) + fs;
+      YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
+    }
   }
 }
 
 // Which shape of the kernel takes (n_out, n_in), with how many workgroups; ok == false: neither.
 // rpg: 1 or 2 for rows of 2048 or 4096 values (the kernels built for one row length), else 0.
-struct Q6Plan { bool ok, head; int num_wg, rpg; };
+// fold_log2: rows of 1024 / 512 / 256 values are streamed two / four / eight at a time as rows of 2048.
+struct Q6Plan { bool ok, head; int num_wg, rpg, fold_log2; };
 inline Q6Plan q6_plan(int64_t n_out, int64_t n_in) {
-  Q6Plan p{false, false, 0, 0};
+  Q6Plan p{false, false, 0, 0, 0};
+  if (n_in == 1024 || n_in == 512 || n_in == 256) {
+    p.fold_log2 = n_in == 1024 ? 1 : (n_in == 512 ? 2 : 3);
+    if (n_out % (16 << p.fold_log2) != 0) return p;
+    n_out >>= p.fold_log2;
+    n_in = 2048;
+  }
   const int64_t nb = n_in / 256;
   // whole rounds of eight blocks, whole groups of 16 rows, 32-bit byte offsets into the weight buffer
   if (n_in % (256 * kQ6RoundBlocks) != 0 || nb > Q6Wide::NBMAX || n_out % 16 != 0) return p;
@@ -470,12 +496,14 @@ inline hipError_t q6_launch_xy(const void* w, const void* x, void* y, const void
                         int64_t n_in, hipStream_t s) {
   const Q6Plan p = q6_plan(n_out, n_in);
   if (!p.ok) return hipErrorInvalidValue;
-  const int groups = (int)(n_out / 16);
+  // (folded rows: the kernel sees the streamed shape)
+  const int64_t rows = n_out >> p.fold_log2, nb = (n_in << p.fold_log2) / 256;
+  const int groups = (int)(rows / 16);
   const dim3 grid((unsigned)p.num_wg, (unsigned)m), block(kQ6Threads);
   auto go = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, block, 0, s, static_cast<const uint8_t*>(w), static_cast<const uint16_t*>(x),
-                       static_cast<YT*>(y), bias, bias_dtype, (int)n_out, (int)(n_in / 256), groups / p.num_wg,
-                       groups % p.num_wg);
+                       static_cast<YT*>(y), bias, bias_dtype, (int)rows, (int)nb, groups / p.num_wg,
+                       groups % p.num_wg, p.fold_log2);
   };
   if (p.head) go(gemv_q6k_stream_kernel<XT, YT, Q6Head, STAGE>);
   else if (p.rpg == 1) go(gemv_q6k_stream_kernel<XT, YT, Q6Short<1>, STAGE>);

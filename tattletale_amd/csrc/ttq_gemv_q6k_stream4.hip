@@ -51,7 +51,7 @@ template <typename XT, typename YT, typename CFG>
 __global__ void __launch_bounds__(kQ6Threads) __attribute__((amdgpu_waves_per_eu(2 * CFG::WGS, 2 * CFG::WGS)))
 gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
                       const void* __restrict__ bias, int bias_dtype, int m, int n_out, int nb_arg, int groups_per_wg,
-                      int groups_rem) {
+                      int groups_rem, int fold_log2) {
   constexpr int TOK = CFG::TOK, kBufs = CFG::BUFS, kPairs = TOK / 2, RPG = CFG::RPG, KP = CFG::KP;
   const int nb = RPG > 0 ? 8 * RPG : nb_arg;              // blocks of a row: NBMAX KP at most
   static_assert(TOK == 2 || TOK == 4, "tokens come in pairs");
@@ -75,6 +75,10 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
   // that requests land in: the compiler would wait for every request in flight first.)
 
   const int n_in = nb * 256;
+  // Folded rows (fold_log2 > 0, as in the single-row kernel): 2^fold_log2 consecutive real rows of 2048 >> fold_log2
+  // values are streamed as one row of eight blocks against the activations repeated; n_out counts streamed rows.
+  const int x_len = n_in >> fold_log2;
+  const int x_mask = fold_log2 ? x_len - 1 : -1;          // (a folded length is a power of two)
   const uint32_t row_bytes = (uint32_t)nb * 210u;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -117,12 +121,12 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
   constexpr int kXPasses = (CFG::NBMAX * 256 + 8 * kQ6Threads - 1) / (8 * kQ6Threads);
 #pragma unroll
   for (int t = 0; t < TOK; t++) {
-    const uint16_t* xt = x + (int64_t)min(m0 + t, m - 1) * n_in + kb0 * 256;
+    const uint16_t* xt = x + (int64_t)min(m0 + t, m - 1) * x_len + kb0 * 256;
 #pragma unroll
     for (int i = 0; i < kXPasses; i++) {
       const int k0 = 8 * tid + i * (8 * kQ6Threads);
       if (k0 < n_in_p)                                    // whole wavefronts: the part is a multiple of 512
-        __builtin_amdgcn_global_load_lds((sm_gptr_t)(xt + k0),
+        __builtin_amdgcn_global_load_lds((sm_gptr_t)(xt + (k0 & x_mask)),
                                          (sm_lptr_t)(xa + t * kXaTok + kXaHead + i * (16 * kQ6Threads) + wave * 1024),
                                          16, 0, 0);
     }
@@ -256,16 +260,30 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
           : "v"(a), "n"(TOK * 64), "n"(2 * TOK * 64), "n"(3 * TOK * 64), "n"(4 * TOK * 64), "n"(5 * TOK * 64),
             "n"(6 * TOK * 64), "n"(7 * TOK * 64)
           : "memory");
-      float sum = v[0];
+      if (fold_log2 == 0) {
+        float sum = v[0];
 #pragma unroll
-      for (int wv = 1; wv < kQ6Waves; wv++) sum += v[wv];
-      const uint32_t ta = total_base + (uint32_t)(grp * (TOK * 64) + 4 * lane);
-      if (KP > 1 && kp > 0) {             // on top of the earlier parts of K
-        float before;
-        asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(before) : "v"(ta) : "memory");
-        sum += before;
+        for (int wv = 1; wv < kQ6Waves; wv++) sum += v[wv];
+        const uint32_t ta = total_base + (uint32_t)(grp * (TOK * 64) + 4 * lane);
+        if (KP > 1 && kp > 0) {             // on top of the earlier parts of K
+          float before;
+          asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(before) : "v"(ta) : "memory");
+          sum += before;
+        }
+        sm_write_f32(ta, sum);
+      } else {
+        // folded rows: the wavefronts whose blocks belong to real row fs of the streamed one (wavefront wv has
+        // block wv < 4 ? 2 wv : 2 wv - 7), in wavefront order; a group's totals are 2^fold_log2 sets
+        for (int fs = 0; fs < (1 << fold_log2); fs++) {
+          float sum = 0.f;
+#pragma unroll
+          for (int wv = 0; wv < kQ6Waves; wv++) {
+            const int b = wv < 4 ? 2 * wv : 2 * wv - 7;
+            if ((b >> (3 - fold_log2)) == fs) sum += v[wv];
+          }
+          sm_write_f32(total_base + (uint32_t)(((grp << fold_log2) + fs) * (TOK * 64) + 4 * lane), sum);
+        }
       }
-      sm_write_f32(ta, sum);
     }
   };
 
@@ -481,21 +499,26 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
   }   // parts of K
   // every request has landed (plain loads are safe again)
   __syncthreads();
-  for (int t = tid; t < ng * TOK * 16; t += kQ6Threads) {
-    const int grp = t / (TOK * 16), tok = (t >> 4) % TOK, nn = t & 15;
+  for (int t = tid; t < (ng * TOK * 16) << fold_log2; t += kQ6Threads) {
+    // set gs = (group, real row of the streamed row); folded launches keep ng << fold_log2 <= MAXG
+    const int gs = t / (TOK * 16), tok = (t >> 4) % TOK, nn = t & 15;
+    const int grp = gs >> fold_log2, fs = gs & ((1 << fold_log2) - 1);
     if (m0 + tok < m) {
-      const int row = (grp0 + grp) * 16 + nn;
-      YElem<YT>::store(y + (int64_t)(m0 + tok) * n_out, row, total[grp][tok][nn] + load_bias(bias, bias_dtype, row));
+      const int row = (((grp0 + grp) * 16 + nn) << fold_log2) + fs;
+      YElem<YT>::store(y + (((int64_t)(m0 + tok) * n_out) << fold_log2), row,
+                       total[gs][tok][nn] + load_bias(bias, bias_dtype, row));
     }
   }
 }
 
 // Which shape takes (m, n_out, n_in): 0 none, else 1 Q6M2Head, 2 Q6M2One, 3 Q6M4One, 4 Q6M2Wide, 5 Q6M4Wide.
-struct Q6MultiPlan { int kind, tok, num_wg; };
+struct Q6MultiPlan { int kind, tok, num_wg, fold_log2; };
 Q6MultiPlan q6_multi_plan(int64_t m, int64_t n_out, int64_t n_in) {
-  Q6MultiPlan p{0, 0, 0};
+  Q6MultiPlan p{0, 0, 0, 0};
   const Q6Plan single = q6_plan(n_out, n_in);              // the stream's own limits
-  const int64_t nb = n_in / 256, groups = n_out / 16;
+  // (folded rows: the streamed shape)
+  p.fold_log2 = single.fold_log2;
+  const int64_t nb = (n_in << p.fold_log2) / 256, groups = (n_out >> p.fold_log2) / 16;
   // (more than four rows: passes of four on gridDim.y; the entry points hand over 65535 rows at most)
   static const int max_rows = dev_knob("TTQ_Q6_MULTI_MAX_ROWS", 65535);
   if (!single.ok || m < 2 || m > max_rows) return p;
@@ -526,6 +549,7 @@ Q6MultiPlan q6_multi_plan(int64_t m, int64_t n_out, int64_t n_in) {
     p.tok = 4;
     maxg = Q6M4Wide::MAXG;
   }
+  maxg >>= p.fold_log2;                                      // a folded group has that many sets of totals
   p.num_wg = (int)std::min<int64_t>(groups, (int64_t)wgs * cus);
   if ((groups + p.num_wg - 1) / p.num_wg > maxg) p.num_wg = (int)((groups + maxg - 1) / maxg);
   return p;
@@ -536,14 +560,15 @@ hipError_t q6_multi_launch_xy(const void* w, const void* x, void* y, const void*
                               int64_t n_out, int64_t n_in, hipStream_t s) {
   const Q6MultiPlan p = q6_multi_plan(m, n_out, n_in);
   if (!p.kind) return hipErrorInvalidValue;
-  const int groups = (int)(n_out / 16);
+  const int64_t rows = n_out >> p.fold_log2, nb = (n_in << p.fold_log2) / 256;      // the streamed shape
+  const int groups = (int)(rows / 16);
   const dim3 grid((unsigned)p.num_wg, (unsigned)((m + p.tok - 1) / p.tok)), block(kQ6Threads);
   auto go = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, block, 0, s, static_cast<const uint8_t*>(w), static_cast<const uint16_t*>(x),
-                       static_cast<YT*>(y), bias, bias_dtype, (int)m, (int)n_out, (int)(n_in / 256), groups / p.num_wg,
-                       groups % p.num_wg);
+                       static_cast<YT*>(y), bias, bias_dtype, (int)m, (int)rows, (int)nb, groups / p.num_wg,
+                       groups % p.num_wg, p.fold_log2);
   };
-  const bool one = n_in == 2048;                             // else, for kinds 1 to 3, 4096
+  const bool one = nb == 8;                                  // else, for kinds 1 to 3, 16
   switch (p.kind) {
     case 1: one ? go(gemv_q6k_multi_kernel<XT, YT, Q6M2Head<1>>) : go(gemv_q6k_multi_kernel<XT, YT, Q6M2Head<2>>); break;
     case 2: one ? go(gemv_q6k_multi_kernel<XT, YT, Q6M2One<1>>) : go(gemv_q6k_multi_kernel<XT, YT, Q6M2One<2>>); break;

@@ -630,3 +630,31 @@ def test_non_finite_block_scale_reaches_its_output_row_only(fmt, n_out, n_in):
             bad = np.nonzero(~np.isfinite(y).all(axis=0))[0]
             assert bad.tolist() == [row], (hex(hi_byte), m)
             assert not np.any(np.isfinite(y[:, row])), (hex(hi_byte), m)
+
+
+@pytest.mark.parametrize("xk", ["bf16", "f16"])
+@pytest.mark.parametrize("n_out,n_in", [(8192, 1024), (16384 + 32 * 7, 1024), (16384 + 64 * 3, 512), (32768 + 128 * 5, 256),
+                                        (151936, 1024)])
+def test_q6_k_streamed_short_rows(xk, n_out, n_in):
+    """Rows of 1024 / 512 / 256 values: two / four / eight consecutive rows are streamed as one row of 2048 against
+    the activations repeated, and the wavefronts' sums go to the real rows.  Sampled rows against the float64
+    product; unit vectors (each real row of a streamed one, first and last blocks) bit for bit; bias."""
+    rng = np.random.default_rng(n_out + n_in)
+    p = random_blocks(F.Q6_K, n_out * (n_in // 256), seed=n_out % 1000 + n_in)
+    rows = np.unique(np.concatenate([rng.integers(0, n_out, 600), np.arange(n_out - 40, n_out), np.arange(40)]))
+    what = oracle.dequant(F.Q6_K, np.ascontiguousarray(p.reshape(n_out, -1)[rows]), rows.size, n_in)
+    wd = packed_to_dev(p)
+    x = Q.fill_normal(n_in + 3, 1, 1.0, n_in).reshape(1, n_in)
+    x[0, ::9] *= 27.0
+    xd, xf = x_to_dev(x, xk)
+    bias = Q.fill_normal(n_in + 4, 0, 3.0, n_out)
+    layer = QuantLinear.init(wd, F.Q6_K, n_in, n_out, bias=torch.from_numpy(bias).to(DEV))
+    y = layer.forward(xd, out_dtype=torch.float32).cpu().numpy()[0]
+    want = oracle.linear_f64(what, xf)[0] + bias[rows]
+    assert rel_l2(y[rows], want) <= 1e-3
+    for col, sc in ((0, 1.0), (n_in - 1, -0.5), (n_in // 2 + 17, 4.0), (255, 0.25)):
+        x = np.zeros((1, n_in), np.float32)
+        x[0, col] = sc
+        xd, _ = x_to_dev(x, xk)
+        y = QL.gemv(F.Q6_K, wd, xd, n_out, n_in).cpu().numpy()[0]
+        assert np.array_equal(y[rows], what[:, col] * np.float32(sc)), col
