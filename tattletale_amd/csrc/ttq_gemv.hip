@@ -376,7 +376,9 @@ hipError_t launch_gemv(int format, const void* w, const void* x, int x_dtype, vo
   // prologue; it re-reads the weights per activation row, so the more rows, the smaller the matrix it wins on.
   // Measured against the matrix-core kernels: 1024x4096 3.9 / 4.8 / 6.3 us for 1 / 2 / 4 rows against 5.3 / 6.5 /
   // 8.5, 2048x4096 5.0 / 6.6 / 10.3 against 5.6 / 6.9 / 8.8, 1024x14336 9.3 / 11.8 / 20.4 against 12.3 / 13.9 / 13.5.
-  if (format == kQ8_0 && m <= 4) {
+  // (Up to 2048 weight rows, two per wavefront: with short rows its lanes are mostly idle, and more rows of them
+  // are the matrix-core kernels' again -- 16384x256 9.2 us against 3.8.)
+  if (format == kQ8_0 && m <= 4 && n_out <= 2048) {
     const float mb = (float)(n_out * (n_in / 32) * 34) * 1e-6f;
     const float limit = n_in <= 4096 ? (m == 1 ? 12.f : (m == 2 ? 8.5f : 6.f)) : (m <= 2 ? 16.f : 0.f);
     if (mb <= limit) return launch_generic_xy<FmtQ8_0>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);

@@ -423,7 +423,7 @@ def test_q8_0_few_rows(n_out, n_in, xk, m):
     mb = n_out * (n_in // 32) * 34 * 1e-6
 
     def small(rows_):
-        if rows_ > 4:
+        if rows_ > 4 or n_out > 2048:
             return False
         return mb <= ((12.0 if rows_ == 1 else 8.5 if rows_ == 2 else 6.0) if n_in <= 4096 else (16.0 if rows_ <= 2 else 0.0))
     for r in {0, m - 1}:
