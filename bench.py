@@ -425,7 +425,7 @@ def main() -> int:
         """Rows next to the headline ones, on random packed bytes with finite scale fields (timing
         only): the attention projections as decode GEMVs (q/o 4096x4096, k/v 1024x4096, reference call
         sites workspace/transformers/src/layers/attn.nim:113-116,154-156,189), the LM-head-sized Q4_K
-        stream, a Q6_K down projection (mlp.nim:60), the Q6_K LM head for 1, 2 and 4 tokens, the few-row decode GEMV (2, 4, 8 and 16 activation rows at once), the few-row form of the
+        stream, a Q6_K down projection (mlp.nim:60), the Q6_K LM head for 1, 2 and 4 tokens (128256x4096) and for 1 and 4 (151936x1024), the few-row decode GEMV (2, 4, 8 and 16 activation rows at once), the few-row form of the
         prefill operator (32 rows) and the prefill GEMM for Q6_K and Q8_0 weights, 14336 x 4096 unless
         named otherwise; the down projection at 128 and 512 rows (K split over copies of the tile grid);
         add + RMSNorm on rows of 4096."""
@@ -467,6 +467,12 @@ def main() -> int:
             timed("q6_k_gemv_lm_head_128256x4096" + ("" if m == 1 else "_m%d" % m), F.Q6_K, m,
                   lambda ws, x, nc, y=y: (lambda i: QL.gemv(F.Q6_K, ws[i % nc], x, 128256, 4096, out=y)),
                   n_out=128256, n_in=4096, steps=max(20, steps // 10))
+        # the same for a small model (hidden size 1024, vocabulary 151936): rows of 1024 values, streamed two at a time
+        for m in (1, 4):
+            y = torch.empty((m, 151936), dtype=torch.float32, device=dev)
+            timed("q6_k_gemv_lm_head_151936x1024" + ("" if m == 1 else "_m%d" % m), F.Q6_K, m,
+                  lambda ws, x, nc, y=y: (lambda i: QL.gemv(F.Q6_K, ws[i % nc], x, 151936, 1024, out=y)),
+                  n_out=151936, n_in=1024, steps=max(20, steps // 4))
         # Q8_0 decode on the headline shape (every projection of a Q8_0 file is a Q8_0 stream)
         y = torch.empty((1, n_out), dtype=torch.float32, device=dev)
         timed("q8_0_gemv_14336x4096", F.Q8_0, 1,
