@@ -75,7 +75,7 @@ template <typename XT, typename YT, typename CFG, int STAGE = 0>
 __global__ void __launch_bounds__(kQ6Threads) __attribute__((amdgpu_waves_per_eu(2 * CFG::WGS, 2 * CFG::WGS)))
 gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
                        const void* __restrict__ bias, int bias_dtype, int n_out, int nb_arg, int groups_per_wg,
-                       int groups_rem, int fold_log2) {
+                       int groups_rem, int fold_log2, int fold_nb) {
   constexpr int kBufs = CFG::BUFS, RPG = CFG::RPG;
   static_assert(RPG == 0 || CFG::NBMAX == 8 * RPG, "a fixed row length is the table's");
   const int nb = RPG > 0 ? CFG::NBMAX : nb_arg;
@@ -97,8 +97,12 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   // Folded rows (fold_log2 > 0): the matrix really has 2^fold_log2 times as many rows, of 2048 >> fold_log2 values
   // each; consecutive rows are contiguous in memory, so 2^fold_log2 of them are streamed as one row of eight
   // blocks against the activations repeated that often, and the wavefronts' sums are added per real row at the end.
+  // fold_nb > 0: the real rows have fold_nb blocks, not a divisor of eight (1536, 2560, 3584, 5120 values ...), and
+  // 2^fold_log2 = 8 / gcd(fold_nb, 8) of them make whole rounds.  A round's blocks then belong to different real
+  // rows from one round to the next, so the wavefronts leave their sums after every round, not after every group,
+  // and the end adds the (round, wavefront) sums of each real row's blocks.
   const int x_len = n_in >> fold_log2;
-  const int x_mask = fold_log2 ? x_len - 1 : -1;          // (a folded length is a power of two)
+  const int x_mask = fold_log2 ? x_len - 1 : -1;          // (fold_nb == 0: a folded length is a power of two)
   const uint16_t* xm = x + (int64_t)blockIdx.y * x_len;
   YT* ym = y + (((int64_t)blockIdx.y * n_out) << fold_log2);
   const int bx = blockIdx.x;
@@ -113,7 +117,7 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   for (int i = 0; i < kXPasses; i++) {
     const int k0 = 8 * tid + i * (8 * kQ6Threads);
     if (k0 < n_in)                                        // whole wavefronts: n_in is a multiple of 512
-      __builtin_amdgcn_global_load_lds((sm_gptr_t)(xm + (k0 & x_mask)),
+      __builtin_amdgcn_global_load_lds((sm_gptr_t)(xm + (fold_nb ? k0 % x_len : (k0 & x_mask))),
                                        (sm_lptr_t)(xstage + i * (16 * kQ6Threads) + wave * 1024), 16, 0, 0);
   }
   // a compute unit serves its requests in the order they were made: every wavefront's activation requests are
@@ -409,21 +413,30 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
       rr++;
       compute(rb, tb);
     };
+    // the four accumulator lanes of a row -> the wavefront's sums, set `slot`
+    auto leave_sums = [&](int slot) {
+      acc = add_xor16(acc);
+      acc = add_xor32(acc);
+      if (lane < 16) sm_write_f32(part_addr + (uint32_t)(slot * (kQ6Waves * 16 * 4)), acc);
+      acc = 0.f;
+    };
+    const bool per_round = fold_nb != 0;
     for (int gi = 0; gi < ng; gi++) {
       if constexpr (RPG > 0) {
 #pragma unroll
-        for (int kr = 0; kr < RPG; kr++) round((uint32_t)kr, held[kr][0], held[kr][1]);
+        for (int kr = 0; kr < RPG; kr++) {
+          round((uint32_t)kr, held[kr][0], held[kr][1]);
+          if (per_round) leave_sums(gi * RPG + kr);
+        }
       } else {
         for (int kr = 0; kr < rpg; kr++) {
           Acts ta, tb;
           round((uint32_t)kr, ta, tb);
+          if (per_round) leave_sums(gi * rpg + kr);
         }
       }
-      // the group is complete: the four accumulator lanes of a row
-      acc = add_xor16(acc);
-      acc = add_xor32(acc);
-      if (lane < 16) sm_write_f32(part_addr + (uint32_t)(gi * (kQ6Waves * 16 * 4)), acc);
-      acc = 0.f;
+      // the group is complete
+      if (!per_round) leave_sums(gi);
     }
   };
   if (wave & 1) run_rounds(std::true_type{});
@@ -437,6 +450,17 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
 #pragma unroll
       for (int wv = 0; wv < kQ6Waves; wv++) v += part[grp][wv][nn];
       const int row = (grp0 + grp) * 16 + nn;
+      YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
+    }
+  } else if (fold_nb != 0) {
+    // real row fs of streamed row nn: blocks fs * fold_nb ... of the streamed row; block b was wavefront b % 8's
+    // in round b / 8
+    for (int t = tid; t < (ng * 16) << fold_log2; t += kQ6Threads) {
+      const int grp = t >> (4 + fold_log2), rem = t & ((16 << fold_log2) - 1);
+      const int nn = rem >> fold_log2, fs = rem & ((1 << fold_log2) - 1);
+      float v = 0.f;
+      for (int b = fs * fold_nb; b < (fs + 1) * fold_nb; b++) v += part[grp * rpg + (b >> 3)][b & 7][nn];
+      const int row = (((grp0 + grp) * 16 + nn) << fold_log2) + fs;
       YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
     }
   } else {
@@ -456,14 +480,25 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
 // Which shape of the kernel takes (n_out, n_in), with how many workgroups; ok == false: neither.
 // rpg: 1 or 2 for rows of 2048 or 4096 values (the kernels built for one row length), else 0.
 // fold_log2: rows of 1024 / 512 / 256 values are streamed two / four / eight at a time as rows of 2048.
-struct Q6Plan { bool ok, head; int num_wg, rpg, fold_log2; };
+// fold_nb: other row lengths that are not whole rounds (fold_nb blocks): 8 / gcd(fold_nb, 8) rows at a time.
+struct Q6Plan { bool ok, head; int num_wg, rpg, fold_log2, fold_nb; };
 inline Q6Plan q6_plan(int64_t n_out, int64_t n_in) {
-  Q6Plan p{false, false, 0, 0, 0};
+  Q6Plan p{false, false, 0, 0, 0, 0};
   if (n_in == 1024 || n_in == 512 || n_in == 256) {
     p.fold_log2 = n_in == 1024 ? 1 : (n_in == 512 ? 2 : 3);
     if (n_out % (16 << p.fold_log2) != 0) return p;
     n_out >>= p.fold_log2;
     n_in = 2048;
+  } else if (n_in % 256 == 0 && n_in % 2048 != 0 && n_in > 0) {
+    const int64_t nbr = n_in / 256;
+    p.fold_log2 = nbr % 4 == 0 ? 1 : (nbr % 2 == 0 ? 2 : 3);
+    if (n_out % (16 << p.fold_log2) != 0 || (nbr << p.fold_log2) > Q6Wide::NBMAX) {
+      p.fold_log2 = 0;
+      return p;
+    }
+    p.fold_nb = (int)nbr;
+    n_out >>= p.fold_log2;
+    n_in <<= p.fold_log2;
   }
   const int64_t nb = n_in / 256;
   // whole rounds of eight blocks, whole groups of 16 rows, 32-bit byte offsets into the weight buffer
@@ -486,7 +521,10 @@ inline Q6Plan q6_plan(int64_t n_out, int64_t n_in) {
     p.num_wg = cus;
     maxg = Q6Wide::MAXG;
   }
-  if ((groups + p.num_wg - 1) / p.num_wg > maxg) p.num_wg = (int)((groups + maxg - 1) / maxg);
+  if (p.fold_nb) maxg /= (int)(nb / 8);                    // sums are kept per round there
+  // more groups than one workgroup per slot keeps sums for: whole waves of workgroups (a last wave with a few
+  // workgroups in it would take as long as a full one)
+  if ((groups + p.num_wg - 1) / p.num_wg > maxg) p.num_wg *= (int)((groups + (int64_t)p.num_wg * maxg - 1) / ((int64_t)p.num_wg * maxg));
   p.ok = true;
   return p;
 }
@@ -503,7 +541,7 @@ inline hipError_t q6_launch_xy(const void* w, const void* x, void* y, const void
   auto go = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, block, 0, s, static_cast<const uint8_t*>(w), static_cast<const uint16_t*>(x),
                        static_cast<YT*>(y), bias, bias_dtype, (int)rows, (int)nb, groups / p.num_wg,
-                       groups % p.num_wg, p.fold_log2);
+                       groups % p.num_wg, p.fold_log2, p.fold_nb);
   };
   if (p.head) go(gemv_q6k_stream_kernel<XT, YT, Q6Head, STAGE>);
   else if (p.rpg == 1) go(gemv_q6k_stream_kernel<XT, YT, Q6Short<1>, STAGE>);

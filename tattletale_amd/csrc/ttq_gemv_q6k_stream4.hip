@@ -521,7 +521,7 @@ Q6MultiPlan q6_multi_plan(int64_t m, int64_t n_out, int64_t n_in) {
   const int64_t nb = (n_in << p.fold_log2) / 256, groups = (n_out >> p.fold_log2) / 16;
   // (more than four rows: passes of four on gridDim.y; the entry points hand over 65535 rows at most)
   static const int max_rows = dev_knob("TTQ_Q6_MULTI_MAX_ROWS", 65535);
-  if (!single.ok || m < 2 || m > max_rows) return p;
+  if (!single.ok || single.fold_nb != 0 || m < 2 || m > max_rows) return p;
   static_assert(Q6M4Wide::NBMAX * Q6M4Wide::KP >= Q6Wide::NBMAX && Q6M2Wide::NBMAX >= Q6Wide::NBMAX, "every row length of the stream");
   const int cus = device_num_cus();
   int maxg, wgs = 1;
@@ -551,7 +551,8 @@ Q6MultiPlan q6_multi_plan(int64_t m, int64_t n_out, int64_t n_in) {
   }
   maxg >>= p.fold_log2;                                      // a folded group has that many sets of totals
   p.num_wg = (int)std::min<int64_t>(groups, (int64_t)wgs * cus);
-  if ((groups + p.num_wg - 1) / p.num_wg > maxg) p.num_wg = (int)((groups + maxg - 1) / maxg);
+  // (whole waves of workgroups, as in the single-row plan)
+  if ((groups + p.num_wg - 1) / p.num_wg > maxg) p.num_wg *= (int)((groups + (int64_t)p.num_wg * maxg - 1) / ((int64_t)p.num_wg * maxg));
   return p;
 }
 

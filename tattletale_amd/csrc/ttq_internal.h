@@ -93,8 +93,8 @@ hipError_t launch_gemv_q8_stream(const void* w, const void* x, int x_dtype, void
                                  hipStream_t s);
 
 // Q6_K through the int8 matrix cores, 16 rows at a time streamed linearly through two or three LDS buffers
-// (ttq_gemv_q6k_stream.hip): 16-bit activations, n_in a multiple of 2048 up to 14336 (or 256 / 512 / 1024: eight /
-// four / two consecutive rows streamed as one), whole groups of 16 rows, at least one per compute unit.
+// (ttq_gemv_q6k_stream.hip): 16-bit activations, n_in a multiple of 2048 up to 14336 (or another multiple of 256:
+// two, four or eight consecutive rows streamed as one), whole groups of 16 rows, at least one per compute unit.
 bool gemv_q6k_stream_supported(int format, int x_dtype, int64_t n_out, int64_t n_in);
 hipError_t launch_gemv_q6k_stream(const void* w, const void* x, int x_dtype, void* y, int y_dtype,
                                   const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,

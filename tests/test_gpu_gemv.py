@@ -634,11 +634,16 @@ def test_non_finite_block_scale_reaches_its_output_row_only(fmt, n_out, n_in):
 
 @pytest.mark.parametrize("xk", ["bf16", "f16"])
 @pytest.mark.parametrize("n_out,n_in", [(8192, 1024), (16384 + 32 * 7, 1024), (16384 + 64 * 3, 512), (32768 + 128 * 5, 256),
-                                        (151936, 1024)])
+                                        (151936, 1024),
+                                        (16384 + 64 * 3, 1536), (16384 + 64 * 5, 2560), (152064, 3584), (8192 + 32, 5120),
+                                        (8192 + 32 * 9, 3072), (32768 + 128, 768), (32768 + 128 * 3, 1280), (32768, 1792),
+                                        (65536 + 64 * 7, 3584)])
 def test_q6_k_streamed_short_rows(xk, n_out, n_in):
-    """Rows of 1024 / 512 / 256 values: two / four / eight consecutive rows are streamed as one row of 2048 against
-    the activations repeated, and the wavefronts' sums go to the real rows.  Sampled rows against the float64
-    product; unit vectors (each real row of a streamed one, first and last blocks) bit for bit; bias."""
+    """Rows that are not whole rounds of 2048 values.  1024 / 512 / 256 values: two / four / eight consecutive rows
+    are streamed as one row of 2048 against the activations repeated, and the wavefronts' sums go to the real
+    rows.  Other multiples of 256 (1536, 2560, 3584, 5120 ...): two, four or eight rows make whole rounds, a
+    round's blocks belong to different real rows, and the sums are kept per round.  Sampled rows against the
+    float64 product; unit vectors (first, last and middle blocks of a row) bit for bit; bias."""
     rng = np.random.default_rng(n_out + n_in)
     p = random_blocks(F.Q6_K, n_out * (n_in // 256), seed=n_out % 1000 + n_in)
     rows = np.unique(np.concatenate([rng.integers(0, n_out, 600), np.arange(n_out - 40, n_out), np.arange(40)]))
