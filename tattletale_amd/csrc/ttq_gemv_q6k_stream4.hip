@@ -51,7 +51,7 @@ template <typename XT, typename YT, typename CFG>
 __global__ void __launch_bounds__(kQ6Threads) __attribute__((amdgpu_waves_per_eu(2 * CFG::WGS, 2 * CFG::WGS)))
 gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
                       const void* __restrict__ bias, int bias_dtype, int m, int n_out, int nb_arg, int groups_per_wg,
-                      int groups_rem, int fold_log2) {
+                      int groups_rem, int fold_log2, int fold_nb) {
   constexpr int TOK = CFG::TOK, kBufs = CFG::BUFS, kPairs = TOK / 2, RPG = CFG::RPG, KP = CFG::KP;
   const int nb = RPG > 0 ? 8 * RPG : nb_arg;              // blocks of a row: NBMAX KP at most
   static_assert(TOK == 2 || TOK == 4, "tokens come in pairs");
@@ -77,8 +77,11 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
   const int n_in = nb * 256;
   // Folded rows (fold_log2 > 0, as in the single-row kernel): 2^fold_log2 consecutive real rows of 2048 >> fold_log2
   // values are streamed as one row of eight blocks against the activations repeated; n_out counts streamed rows.
+  // fold_nb > 0: real rows of fold_nb blocks, not a divisor of eight; a round's blocks belong to different real rows
+  // from round to round, and the sums are handed over after every round (single part of K only).
   const int x_len = n_in >> fold_log2;
-  const int x_mask = fold_log2 ? x_len - 1 : -1;          // (a folded length is a power of two)
+  const int x_mask = fold_log2 ? x_len - 1 : -1;          // (fold_nb == 0: a folded length is a power of two)
+  const bool per_round = fold_nb != 0;
   const uint32_t row_bytes = (uint32_t)nb * 210u;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -126,7 +129,7 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
     for (int i = 0; i < kXPasses; i++) {
       const int k0 = 8 * tid + i * (8 * kQ6Threads);
       if (k0 < n_in_p)                                    // whole wavefronts: the part is a multiple of 512
-        __builtin_amdgcn_global_load_lds((sm_gptr_t)(xt + (k0 & x_mask)),
+        __builtin_amdgcn_global_load_lds((sm_gptr_t)(xt + (per_round ? k0 % x_len : (k0 & x_mask))),
                                          (sm_lptr_t)(xa + t * kXaTok + kXaHead + i * (16 * kQ6Threads) + wave * 1024),
                                          16, 0, 0);
     }
@@ -236,12 +239,17 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
   const uint32_t total_base = sm_lds(&total[0][0][0]);
   const uint32_t stage_addr = stage_base + (uint32_t)((wave * TOK + (g >> 1)) * 64 + 4 * n);
 
+  if (per_round) {                      // sums are added to the totals round by round there
+    float* tz = &total[0][0][0];
+    for (int i = tid; i < CFG::MAXG * TOK * 16; i += kQ6Threads) tz[i] = 0.f;
+  }
   sm_barrier();                         // the plane tables are complete
 #pragma unroll
   for (int i = kEarlyRounds; i < kBufs; i++)
     if (i < nrounds) request_next();
 
   // the eight wavefronts' sums of group `grp` (complete since a barrier) -> its totals, in wavefront order
+  // (per_round: `grp` counts rounds, rpg to a group)
   auto reduce_group = [&](int grp) {
     if (lane < TOK * 16) {
       const uint32_t a = stage_base + (uint32_t)((grp & 1) * kStageHalf + 4 * lane);
@@ -260,7 +268,48 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
           : "v"(a), "n"(TOK * 64), "n"(2 * TOK * 64), "n"(3 * TOK * 64), "n"(4 * TOK * 64), "n"(5 * TOK * 64),
             "n"(6 * TOK * 64), "n"(7 * TOK * 64)
           : "memory");
-      if (fold_log2 == 0) {
+      if (per_round) {
+        // round kr of group gg: wavefront wv had block 8 kr + (wv < 4 ? 2 wv : 2 wv - 7) of the streamed row, which
+        // belongs to real row (that block) / fold_nb; rounds come in order, wavefronts in order within a round
+        // (two divisions per hand-over; a real row has three blocks or more, so a round's eight touch four at most)
+        const int gg = grp / rpg, kr = grp - gg * rpg;
+        const int f0 = (8 * kr) / fold_nb, r0 = 8 * kr - f0 * fold_nb;
+        int fsw[kQ6Waves];
+#pragma unroll
+        for (int wv = 0; wv < kQ6Waves; wv++) {
+          const int t = r0 + (wv < 4 ? 2 * wv : 2 * wv - 7);
+          fsw[wv] = f0 + (t >= fold_nb) + (t >= 2 * fold_nb) + (t >= 3 * fold_nb);
+        }
+        // the (up to four) totals first, in one trip; then the sums on top, where a row had blocks in this round
+        const int last_set = (1 << fold_log2) - 1;
+        uint32_t ta[4];
+        float before[4];
+#pragma unroll
+        for (int d = 0; d < 4; d++)
+          ta[d] = total_base + (uint32_t)(((gg << fold_log2) + min(f0 + d, last_set)) * (TOK * 64) + 4 * lane);
+        asm volatile(
+            "ds_read_b32 %0, %4\n\t"
+            "ds_read_b32 %1, %5\n\t"
+            "ds_read_b32 %2, %6\n\t"
+            "ds_read_b32 %3, %7\n\t"
+            "s_waitcnt lgkmcnt(0)"
+            : "=&v"(before[0]), "=&v"(before[1]), "=&v"(before[2]), "=&v"(before[3])
+            : "v"(ta[0]), "v"(ta[1]), "v"(ta[2]), "v"(ta[3])
+            : "memory");
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+          float sum = 0.f;
+          bool any = false;
+#pragma unroll
+          for (int wv = 0; wv < kQ6Waves; wv++) {
+            if (fsw[wv] == f0 + d) {
+              sum += v[wv];
+              any = true;
+            }
+          }
+          if (any) sm_write_f32(ta[d], before[d] + sum);
+        }
+      } else if (fold_log2 == 0) {
         float sum = v[0];
 #pragma unroll
         for (int wv = 1; wv < kQ6Waves; wv++) sum += v[wv];
@@ -470,32 +519,42 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
       rr++;
       compute(rb, tb);
     };
+    // the wavefront's sums of hand-over `idx` (a group, or a round): the two planes of a (row, token) are 16 lanes
+    // apart; then the hand-over before it, which every wavefront completed before the barriers since
+    auto hand_over = [&](int idx) {
+#pragma unroll
+      for (int q = 0; q < kPairs; q++) {
+        acc[q] = add_xor16(acc[q]);
+        if ((g & 1) == 0) sm_write_f32(stage_addr + (uint32_t)((idx & 1) * kStageHalf + q * 128), acc[q]);
+        acc[q] = 0.f;
+      }
+      if (idx > 0 && wave == ((idx - 1) & 7)) reduce_group(idx - 1);
+    };
     for (int gi = 0; gi < ng; gi++) {
       if constexpr (RPG > 0) {
 #pragma unroll
-        for (int kr = 0; kr < RPG; kr++) round((uint32_t)kr, held[kr][0], held[kr][1]);
+        for (int kr = 0; kr < RPG; kr++) {
+          round((uint32_t)kr, held[kr][0], held[kr][1]);
+          if (per_round) hand_over(gi * RPG + kr);
+        }
       } else {
         for (int kr = 0; kr < rpg; kr++) {
           Acts ta, tb;
           round((uint32_t)kr, ta, tb);
+          if (per_round) hand_over(gi * rpg + kr);
         }
       }
-      // the group is complete: the two planes of a (row, token) are 16 lanes apart
-#pragma unroll
-      for (int q = 0; q < kPairs; q++) {
-        acc[q] = add_xor16(acc[q]);
-        if ((g & 1) == 0) sm_write_f32(stage_addr + (uint32_t)((gi & 1) * kStageHalf + q * 128), acc[q]);
-        acc[q] = 0.f;
-      }
-      // the group before: every wavefront left its sums before this group's barriers
-      if (gi > 0 && wave == ((gi - 1) & 7)) reduce_group(gi - 1);
+      if (!per_round) hand_over(gi);     // the group is complete
     }
   };
   if (blk & 1) run_rounds(std::true_type{});
   else run_rounds(std::false_type{});
   // every wavefront has left its last sums and is done with the buffers and the tables
   sm_barrier();
-  if (wave == ((ng - 1) & 7)) reduce_group(ng - 1);
+  {
+    const int last = (per_round ? nrounds : ng) - 1;
+    if (wave == (last & 7)) reduce_group(last);
+  }
   }   // parts of K
   // every request has landed (plain loads are safe again)
   __syncthreads();
@@ -512,16 +571,17 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
 }
 
 // Which shape takes (m, n_out, n_in): 0 none, else 1 Q6M2Head, 2 Q6M2One, 3 Q6M4One, 4 Q6M2Wide, 5 Q6M4Wide.
-struct Q6MultiPlan { int kind, tok, num_wg, fold_log2; };
+struct Q6MultiPlan { int kind, tok, num_wg, fold_log2, fold_nb; };
 Q6MultiPlan q6_multi_plan(int64_t m, int64_t n_out, int64_t n_in) {
-  Q6MultiPlan p{0, 0, 0, 0};
+  Q6MultiPlan p{0, 0, 0, 0, 0};
   const Q6Plan single = q6_plan(n_out, n_in);              // the stream's own limits
   // (folded rows: the streamed shape)
   p.fold_log2 = single.fold_log2;
   const int64_t nb = (n_in << p.fold_log2) / 256, groups = (n_out >> p.fold_log2) / 16;
   // (more than four rows: passes of four on gridDim.y; the entry points hand over 65535 rows at most)
   static const int max_rows = dev_knob("TTQ_Q6_MULTI_MAX_ROWS", 65535);
-  if (!single.ok || single.fold_nb != 0 || m < 2 || m > max_rows) return p;
+  if (!single.ok || m < 2 || m > max_rows) return p;
+  p.fold_nb = single.fold_nb;
   static_assert(Q6M4Wide::NBMAX * Q6M4Wide::KP >= Q6Wide::NBMAX && Q6M2Wide::NBMAX >= Q6Wide::NBMAX, "every row length of the stream");
   const int cus = device_num_cus();
   int maxg, wgs = 1;
@@ -540,7 +600,7 @@ Q6MultiPlan q6_multi_plan(int64_t m, int64_t n_out, int64_t n_in) {
       p.kind = 2;
       maxg = Q6M2One<1>::MAXG;
     }
-  } else if (m == 2) {
+  } else if (m == 2 || p.fold_nb) {      // (unevenly folded rows: two tokens a pass, one part of K)
     p.kind = 4;
     p.tok = 2;
     maxg = Q6M2Wide::MAXG;
@@ -567,7 +627,7 @@ hipError_t q6_multi_launch_xy(const void* w, const void* x, void* y, const void*
   auto go = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, block, 0, s, static_cast<const uint8_t*>(w), static_cast<const uint16_t*>(x),
                        static_cast<YT*>(y), bias, bias_dtype, (int)m, (int)rows, (int)nb, groups / p.num_wg,
-                       groups % p.num_wg, p.fold_log2);
+                       groups % p.num_wg, p.fold_log2, p.fold_nb);
   };
   const bool one = nb == 8;                                  // else, for kinds 1 to 3, 16
   switch (p.kind) {

@@ -256,11 +256,14 @@ def test_q6k_streamed_two_to_four_rows(xk, m, n_out, n_in):
                                          (21, 4096 + 32, 4096), (13, 4096, 8192),
                                          (2, 8192, 1024), (4, 16384 + 32 * 7, 1024), (3, 16384 + 64 * 3, 512),
                                          (7, 32768 + 128 * 5, 256), (2, 151936, 1024), (4, 151936, 1024),
+                                         (2, 16384 + 64 * 3, 1536), (4, 16384 + 64 * 5, 2560), (3, 8192 + 32 * 9, 3072),
+                                         (2, 152064, 3584), (4, 32768 + 128, 768), (5, 32768, 1792), (4, 65536 + 64, 3584),
                                          (6, 4096, 14336), (4, 24576 + 16 * 9, 14336), (2, 24576 + 16 * 9, 14336)])
 def test_q6k_streamed_more_rows_and_more_groups(m, n_out, n_in):
     """Five to eight rows (two passes of four, the second one ragged), more row groups than a workgroup keeps
-    totals for (more workgroups than compute units), and rows of 1024 / 512 / 256 values (two / four / eight real
-    rows streamed as one): sampled rows against the float64 product and against the single-row kernel."""
+    totals for (more workgroups than compute units), rows of 1024 / 512 / 256 values (two / four / eight real
+    rows streamed as one) and other row lengths that are not whole rounds (sums handed over round by round):
+    sampled rows against the float64 product and against the single-row kernel."""
     rng = np.random.default_rng(n_out + n_in + m)
     p = random_blocks(F.Q6_K, n_out * (n_in // 256), seed=80 + m)
     rows = np.unique(np.concatenate([rng.integers(0, n_out, 600), np.arange(n_out - 48, n_out), np.arange(48)]))
