@@ -35,16 +35,18 @@ typedef uint32_t sm_u32x2 __attribute__((ext_vector_type(2)));
 // RPG: rounds per group (rows of 2048 RPG values) when the kernel is built for one row length, else 0.
 // KP: into how many parts of NBMAX blocks a row may fall; the parts are streamed one after the other, each with
 // its own plane tables (four tokens' tables of a row of 14336 values would not fit LDS).
-template <int TOK_, int NBMAX_, int BUFS_, int WGS_, int MAXG_, int RPG_, int KP_ = 1>
+// SETS: real rows of a streamed row whose sums a wavefront can keep apart (unevenly folded rows: up to four).
+template <int TOK_, int NBMAX_, int BUFS_, int WGS_, int MAXG_, int RPG_, int KP_ = 1, int SETS_ = 1>
 struct Q6Multi {
   static constexpr int TOK = TOK_, NBMAX = NBMAX_, BUFS = BUFS_, WGS = WGS_, MAXG = MAXG_, RPG = RPG_, KP = KP_;
+  static constexpr int SETS = SETS_;
   static_assert(RPG == 0 || (NBMAX == 8 * RPG && KP == 1), "a fixed row length is the table's");
 };
 // rows of 2048 RPG values (RPG 1 or 2), many of them, two tokens: two workgroups per compute unit
 template <int RPG> using Q6M2Head = Q6Multi<2, 8 * RPG, 2, 2, 20, RPG>;
 template <int RPG> using Q6M2One = Q6Multi<2, 8 * RPG, 3, 1, 56, RPG>;    // rows of 2048 RPG values, two tokens
 template <int RPG> using Q6M4One = Q6Multi<4, 8 * RPG, 3, 1, 56, RPG>;    // rows of 2048 RPG values, four tokens
-using Q6M2Wide = Q6Multi<2, 56, 3, 1, 24, 0>;                             // rows of up to 14336, two tokens
+using Q6M2Wide = Q6Multi<2, 56, 3, 1, 24, 0, 1, 4>;                       // rows of up to 14336, two tokens
 using Q6M4Wide = Q6Multi<4, 32, 3, 1, 6, 0, 2>;                           // rows of up to 14336, four tokens, K in two parts
 
 template <typename XT, typename YT, typename CFG>
@@ -63,11 +65,13 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
   constexpr int kXaTok = kXaHead + CFG::NBMAX * 512 + 64;
   // a token's scales of the integer sums: (unit, plane, k-set) floats
   constexpr int kFacTok = CFG::NBMAX * 32;
-  constexpr int kStageHalf = kQ6Waves * TOK * 64;            // bytes of one exchange area
+  constexpr int SETS = CFG::SETS;
+  constexpr int kStageWave = SETS * TOK * 64;                // bytes of a wavefront's sums in an exchange area
+  constexpr int kStageHalf = kQ6Waves * kStageWave;          // bytes of one exchange area
   __shared__ __attribute__((aligned(1024))) uint8_t wbuf[kBufs * kQ6BufBytes];
   __shared__ __attribute__((aligned(16))) uint8_t xa[TOK * kXaTok];
   __shared__ __attribute__((aligned(16))) float fac[TOK * CFG::NBMAX * 8];
-  __shared__ __attribute__((aligned(16))) float stage[2][kQ6Waves][TOK][16];
+  __shared__ __attribute__((aligned(16))) float stage[2][kQ6Waves][SETS][TOK][16];
   __shared__ __attribute__((aligned(16))) float total[CFG::MAXG][TOK][16];
   // The raw activations land where their planes will be: 16 values are 32 bytes either way, and the two threads
   // that turn them into two entries of 16 bytes are neighbours in one wavefront, which has read before it writes.
@@ -78,7 +82,8 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
   // Folded rows (fold_log2 > 0, as in the single-row kernel): 2^fold_log2 consecutive real rows of 2048 >> fold_log2
   // values are streamed as one row of eight blocks against the activations repeated; n_out counts streamed rows.
   // fold_nb > 0: real rows of fold_nb blocks, not a divisor of eight; a round's blocks belong to different real rows
-  // from round to round, and the sums are handed over after every round (single part of K only).
+  // from round to round, so a wavefront keeps one sum per real row of the streamed row (SETS of them at most) and
+  // hands all of them over at the end of the group (single part of K only).
   const int x_len = n_in >> fold_log2;
   const int x_mask = fold_log2 ? x_len - 1 : -1;          // (fold_nb == 0: a folded length is a power of two)
   const bool per_round = fold_nb != 0;
@@ -235,102 +240,67 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
   // accumulator lane (n, g): token g / 2 of the pair, plane g % 2; its scales for the two k-sets are neighbours
   const uint32_t fac_addr0 = sm_lds(fac) + (uint32_t)((g >> 1) * kFacTok + 8 * (g & 1)) + 16u * u0;
   const uint32_t wbuf_base = sm_lds(wbuf);
-  const uint32_t stage_base = sm_lds(&stage[0][0][0][0]);
+  const uint32_t stage_base = sm_lds(&stage[0][0][0][0][0]);
   const uint32_t total_base = sm_lds(&total[0][0][0]);
-  const uint32_t stage_addr = stage_base + (uint32_t)((wave * TOK + (g >> 1)) * 64 + 4 * n);
+  const uint32_t stage_addr = stage_base + (uint32_t)(wave * kStageWave + (g >> 1) * 64 + 4 * n);
 
-  if (per_round) {                      // sums are added to the totals round by round there
-    float* tz = &total[0][0][0];
-    for (int i = tid; i < CFG::MAXG * TOK * 16; i += kQ6Threads) tz[i] = 0.f;
-  }
   sm_barrier();                         // the plane tables are complete
 #pragma unroll
   for (int i = kEarlyRounds; i < kBufs; i++)
     if (i < nrounds) request_next();
 
   // the eight wavefronts' sums of group `grp` (complete since a barrier) -> its totals, in wavefront order
-  // (per_round: `grp` counts rounds, rpg to a group)
+  // the eight wavefronts' sums of group `grp` (complete since a barrier) -> its totals, in wavefront order
   auto reduce_group = [&](int grp) {
     if (lane < TOK * 16) {
-      const uint32_t a = stage_base + (uint32_t)((grp & 1) * kStageHalf + 4 * lane);
-      float v[kQ6Waves];
-      asm volatile(
-          "ds_read_b32 %0, %8\n\t"
-          "ds_read_b32 %1, %8 offset:%9\n\t"
-          "ds_read_b32 %2, %8 offset:%10\n\t"
-          "ds_read_b32 %3, %8 offset:%11\n\t"
-          "ds_read_b32 %4, %8 offset:%12\n\t"
-          "ds_read_b32 %5, %8 offset:%13\n\t"
-          "ds_read_b32 %6, %8 offset:%14\n\t"
-          "ds_read_b32 %7, %8 offset:%15\n\t"
-          "s_waitcnt lgkmcnt(0)"
-          : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7])
-          : "v"(a), "n"(TOK * 64), "n"(2 * TOK * 64), "n"(3 * TOK * 64), "n"(4 * TOK * 64), "n"(5 * TOK * 64),
-            "n"(6 * TOK * 64), "n"(7 * TOK * 64)
-          : "memory");
-      if (per_round) {
-        // round kr of group gg: wavefront wv had block 8 kr + (wv < 4 ? 2 wv : 2 wv - 7) of the streamed row, which
-        // belongs to real row (that block) / fold_nb; rounds come in order, wavefronts in order within a round
-        // (two divisions per hand-over; a real row has three blocks or more, so a round's eight touch four at most)
-        const int gg = grp / rpg, kr = grp - gg * rpg;
-        const int f0 = (8 * kr) / fold_nb, r0 = 8 * kr - f0 * fold_nb;
-        int fsw[kQ6Waves];
-#pragma unroll
-        for (int wv = 0; wv < kQ6Waves; wv++) {
-          const int t = r0 + (wv < 4 ? 2 * wv : 2 * wv - 7);
-          fsw[wv] = f0 + (t >= fold_nb) + (t >= 2 * fold_nb) + (t >= 3 * fold_nb);
-        }
-        // the (up to four) totals first, in one trip; then the sums on top, where a row had blocks in this round
-        const int last_set = (1 << fold_log2) - 1;
-        uint32_t ta[4];
-        float before[4];
-#pragma unroll
-        for (int d = 0; d < 4; d++)
-          ta[d] = total_base + (uint32_t)(((gg << fold_log2) + min(f0 + d, last_set)) * (TOK * 64) + 4 * lane);
+      // one set of sums, or with unevenly folded rows one per real row of the streamed row
+      const int sets = per_round ? (1 << fold_log2) : 1;
+      for (int r = 0; r < sets; r++) {
+        const uint32_t a = stage_base + (uint32_t)((grp & 1) * kStageHalf + r * (TOK * 64) + 4 * lane);
+        float v[kQ6Waves];
         asm volatile(
-            "ds_read_b32 %0, %4\n\t"
-            "ds_read_b32 %1, %5\n\t"
-            "ds_read_b32 %2, %6\n\t"
-            "ds_read_b32 %3, %7\n\t"
+            "ds_read_b32 %0, %8\n\t"
+            "ds_read_b32 %1, %8 offset:%9\n\t"
+            "ds_read_b32 %2, %8 offset:%10\n\t"
+            "ds_read_b32 %3, %8 offset:%11\n\t"
+            "ds_read_b32 %4, %8 offset:%12\n\t"
+            "ds_read_b32 %5, %8 offset:%13\n\t"
+            "ds_read_b32 %6, %8 offset:%14\n\t"
+            "ds_read_b32 %7, %8 offset:%15\n\t"
             "s_waitcnt lgkmcnt(0)"
-            : "=&v"(before[0]), "=&v"(before[1]), "=&v"(before[2]), "=&v"(before[3])
-            : "v"(ta[0]), "v"(ta[1]), "v"(ta[2]), "v"(ta[3])
+            : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7])
+            : "v"(a), "n"(kStageWave), "n"(2 * kStageWave), "n"(3 * kStageWave), "n"(4 * kStageWave), "n"(5 * kStageWave),
+              "n"(6 * kStageWave), "n"(7 * kStageWave)
             : "memory");
+        if (per_round) {
+          // (a wavefront without a block of real row r in this group left a zero)
+          float sum = v[0];
 #pragma unroll
-        for (int d = 0; d < 4; d++) {
-          float sum = 0.f;
-          bool any = false;
+          for (int wv = 1; wv < kQ6Waves; wv++) sum += v[wv];
+          sm_write_f32(total_base + (uint32_t)(((grp << fold_log2) + r) * (TOK * 64) + 4 * lane), sum);
+        } else if (fold_log2 == 0) {
+          float sum = v[0];
 #pragma unroll
-          for (int wv = 0; wv < kQ6Waves; wv++) {
-            if (fsw[wv] == f0 + d) {
-              sum += v[wv];
-              any = true;
+          for (int wv = 1; wv < kQ6Waves; wv++) sum += v[wv];
+          const uint32_t ta = total_base + (uint32_t)(grp * (TOK * 64) + 4 * lane);
+          if (KP > 1 && kp > 0) {             // on top of the earlier parts of K
+            float before;
+            asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(before) : "v"(ta) : "memory");
+            sum += before;
+          }
+          sm_write_f32(ta, sum);
+        } else {
+          // folded rows: the wavefronts whose blocks belong to real row fs of the streamed one (wavefront wv has
+          // block wv < 4 ? 2 wv : 2 wv - 7), in wavefront order; a group's totals are 2^fold_log2 sets
+          for (int fs = 0; fs < (1 << fold_log2); fs++) {
+            float sum = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < kQ6Waves; wv++) {
+              const int b = wv < 4 ? 2 * wv : 2 * wv - 7;
+              if ((b >> (3 - fold_log2)) == fs) sum += v[wv];
             }
+            sm_write_f32(total_base + (uint32_t)(((grp << fold_log2) + fs) * (TOK * 64) + 4 * lane), sum);
           }
-          if (any) sm_write_f32(ta[d], before[d] + sum);
-        }
-      } else if (fold_log2 == 0) {
-        float sum = v[0];
-#pragma unroll
-        for (int wv = 1; wv < kQ6Waves; wv++) sum += v[wv];
-        const uint32_t ta = total_base + (uint32_t)(grp * (TOK * 64) + 4 * lane);
-        if (KP > 1 && kp > 0) {             // on top of the earlier parts of K
-          float before;
-          asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(before) : "v"(ta) : "memory");
-          sum += before;
-        }
-        sm_write_f32(ta, sum);
-      } else {
-        // folded rows: the wavefronts whose blocks belong to real row fs of the streamed one (wavefront wv has
-        // block wv < 4 ? 2 wv : 2 wv - 7), in wavefront order; a group's totals are 2^fold_log2 sets
-        for (int fs = 0; fs < (1 << fold_log2); fs++) {
-          float sum = 0.f;
-#pragma unroll
-          for (int wv = 0; wv < kQ6Waves; wv++) {
-            const int b = wv < 4 ? 2 * wv : 2 * wv - 7;
-            if ((b >> (3 - fold_log2)) == fs) sum += v[wv];
-          }
-          sm_write_f32(total_base + (uint32_t)(((grp << fold_log2) + fs) * (TOK * 64) + 4 * lane), sum);
         }
       }
     }
@@ -519,42 +489,73 @@ gemv_q6k_multi_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
       rr++;
       compute(rb, tb);
     };
-    // the wavefront's sums of hand-over `idx` (a group, or a round): the two planes of a (row, token) are 16 lanes
-    // apart; then the hand-over before it, which every wavefront completed before the barriers since
-    auto hand_over = [&](int idx) {
+    // Unevenly folded rows: the sums per real row of the streamed row.  The real row of the wavefront's block in
+    // round kr is (8 kr + blk) / fold_nb, the same for all lanes: a quotient and a remainder that advance by eight
+    // blocks per round.
+    float accf[kPairs][SETS];
+#pragma unroll
+    for (int q = 0; q < kPairs; q++)
+#pragma unroll
+      for (int r = 0; r < SETS; r++) accf[q][r] = 0.f;
+    const int fq0 = per_round ? blk / fold_nb : 0, fr0 = per_round ? blk - fq0 * fold_nb : 0;
+    int fq = fq0, fr = fr0;
+    auto to_real_row = [&]() {
 #pragma unroll
       for (int q = 0; q < kPairs; q++) {
-        acc[q] = add_xor16(acc[q]);
-        if ((g & 1) == 0) sm_write_f32(stage_addr + (uint32_t)((idx & 1) * kStageHalf + q * 128), acc[q]);
+#pragma unroll
+        for (int r = 0; r < SETS; r++)
+          if (fq == r) accf[q][r] += acc[q];
         acc[q] = 0.f;
+      }
+      fr += 8;
+      while (fr >= fold_nb) {
+        fr -= fold_nb;
+        fq++;
+      }
+    };
+    // the wavefront's sums of group `idx`: the two planes of a (row, token) are 16 lanes apart; then the group
+    // before it, which every wavefront handed over before the barriers since
+    auto hand_over = [&](int idx) {
+      if (per_round) {
+#pragma unroll
+        for (int q = 0; q < kPairs; q++)
+#pragma unroll
+          for (int r = 0; r < SETS; r++) {
+            const float v = add_xor16(accf[q][r]);
+            if ((g & 1) == 0) sm_write_f32(stage_addr + (uint32_t)((idx & 1) * kStageHalf + r * (TOK * 64) + q * 128), v);
+            accf[q][r] = 0.f;
+          }
+        fq = fq0;
+        fr = fr0;
+      } else {
+#pragma unroll
+        for (int q = 0; q < kPairs; q++) {
+          acc[q] = add_xor16(acc[q]);
+          if ((g & 1) == 0) sm_write_f32(stage_addr + (uint32_t)((idx & 1) * kStageHalf + q * 128), acc[q]);
+          acc[q] = 0.f;
+        }
       }
       if (idx > 0 && wave == ((idx - 1) & 7)) reduce_group(idx - 1);
     };
     for (int gi = 0; gi < ng; gi++) {
       if constexpr (RPG > 0) {
 #pragma unroll
-        for (int kr = 0; kr < RPG; kr++) {
-          round((uint32_t)kr, held[kr][0], held[kr][1]);
-          if (per_round) hand_over(gi * RPG + kr);
-        }
+        for (int kr = 0; kr < RPG; kr++) round((uint32_t)kr, held[kr][0], held[kr][1]);
       } else {
         for (int kr = 0; kr < rpg; kr++) {
           Acts ta, tb;
           round((uint32_t)kr, ta, tb);
-          if (per_round) hand_over(gi * rpg + kr);
+          if (per_round) to_real_row();
         }
       }
-      if (!per_round) hand_over(gi);     // the group is complete
+      hand_over(gi);     // the group is complete
     }
   };
   if (blk & 1) run_rounds(std::true_type{});
   else run_rounds(std::false_type{});
   // every wavefront has left its last sums and is done with the buffers and the tables
   sm_barrier();
-  {
-    const int last = (per_round ? nrounds : ng) - 1;
-    if (wave == (last & 7)) reduce_group(last);
-  }
+  if (wave == ((ng - 1) & 7)) reduce_group(ng - 1);
   }   // parts of K
   // every request has landed (plain loads are safe again)
   __syncthreads();
@@ -582,6 +583,7 @@ Q6MultiPlan q6_multi_plan(int64_t m, int64_t n_out, int64_t n_in) {
   static const int max_rows = dev_knob("TTQ_Q6_MULTI_MAX_ROWS", 65535);
   if (!single.ok || m < 2 || m > max_rows) return p;
   p.fold_nb = single.fold_nb;
+  if (p.fold_nb && (1 << single.fold_log2) > Q6M2Wide::SETS) return p;     // (rows of an odd number of blocks)
   static_assert(Q6M4Wide::NBMAX * Q6M4Wide::KP >= Q6Wide::NBMAX && Q6M2Wide::NBMAX >= Q6Wide::NBMAX, "every row length of the stream");
   const int cus = device_num_cus();
   int maxg, wgs = 1;

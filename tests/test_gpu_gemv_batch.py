@@ -278,9 +278,12 @@ def test_q6k_streamed_more_rows_and_more_groups(m, n_out, n_in):
     want = oracle.linear_f64(what, xf)
     for t in range(m):
         assert rel_l2(y[t][rows], want[t]) <= TOL, t
+    # rows of an odd number of blocks (768, 1792 values): eight rows at a time for a single activation row, the
+    # packed-dot kernel for several -- both within the bound above of the exact product, not of each other to 2e-6
+    same = 3e-4 if (n_in // 256) % 2 == 1 and n_in > 256 else 2e-6
     for t in {0, m // 2, m - 1}:
         y1 = QL.gemv(F.Q6_K, wd, xd[t:t + 1], n_out, n_in).cpu().numpy()[0]
-        assert rel_l2(y[t], y1) <= 2e-6, t
+        assert rel_l2(y[t], y1) <= same, t
 
 
 def test_q6k_streamed_two_to_four_rows_do_not_leak_and_output_types():
