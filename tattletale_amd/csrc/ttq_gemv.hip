@@ -419,9 +419,9 @@ float gemv_estimate_us(int format, int x_dtype, int64_t m, int64_t n_out, int64_
     // measured at 13.8, 48 and 431 MB: two tokens 5.5 / 11.8 / 68.6 us, four tokens 6.5 / 13.6 / 75.4 us per pass;
     // longer rows: two tokens 13.2 us at 48 MB; four tokens a pass, K streamed in one (up to 8192 values) or two
     // parts, each with its own activation tables: 11.9 us at 27.5 MB, 19.2 at 48, 27.4 at 96
-    if (n_in > 4096) return m == 2 ? mb / 5.f + 3.5f : (float)((m + 3) / 4) * (mb / 5.8f + (n_in > 8192 ? 11.f : 7.2f));
     // rows that are not whole rounds nor 256 / 512 / 1024 values: two tokens a pass (152064x3584: 89.6 us at 447 MB)
     if (n_in % 2048 != 0 && n_in != 1024 && n_in != 512 && n_in != 256) return (float)((m + 1) / 2) * (mb / 5.2f + 4.f);
+    if (n_in > 4096) return m == 2 ? mb / 5.f + 3.5f : (float)((m + 3) / 4) * (mb / 5.8f + (n_in > 8192 ? 11.f : 7.2f));
     return m == 2 ? mb / 6.4f + 3.5f : (float)((m + 3) / 4) * (mb / 5.8f + 4.f);
   }
   if (gemv_dot2_multi_supported(format, x_dtype, m, n_in))
