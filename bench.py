@@ -28,7 +28,9 @@ for the GEMM, and a CPU baseline timed on this machine's host cores.
 
     python bench.py --only ladder     the roofline ladder of the headline kernel (see csrc/ttq_ladder.hip);
                                       --only ladder_14336x4096 runs one shape (for a kernel trace);
-                                      --only ladder_q6k the stages of the Q6_K streamed GEMV
+                                      --only ladder_q6k the stages of the Q6_K streamed GEMV;
+                                      --only ladder_gemm the roles of the prefill GEMM kernel, alone and together
+                                      (the ladder kernels are compiled on demand into libttq_ladder.so)
 """
 from __future__ import annotations
 
@@ -571,14 +573,16 @@ def main() -> int:
         torch.cuda.empty_cache()
         return res
 
+    def ladder_lib():
+        """libttq_ladder.so, compiled on demand (measurement-only kernels, not part of the product build)."""
+        from tattletale_amd import build as B
+        return C.CDLL(B.build_ladder())
+
     def run_ladder(steps: int, warmup: int, shapes=((14336, 4096), (128256, 4096))):
         """What each stage of the headline kernel costs on its own (tattletale_amd/csrc/ttq_ladder.hip):
         empty launch, the kernel's requests alone, + the y store, the kernel without arithmetic, the
         kernel; at the headline shape and on a 295 MB Q4_K matrix (128256 x 4096)."""
-        lad_path = os.path.join(ROOT, "tattletale_amd", "libttq_ladder.so")
-        if not os.path.exists(lad_path):
-            raise RuntimeError("%s not found: build it with `python -m tattletale_amd.build`" % lad_path)
-        LAD = C.CDLL(lad_path)
+        LAD = ladder_lib()
         LAD.ttq_ladder_launch.restype = C.c_int
         LAD.ttq_ladder_launch.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p]
         L = _lib.lib()
@@ -624,10 +628,7 @@ def main() -> int:
         """The stages of the Q6_K streamed GEMV (tattletale_amd/csrc/ttq_gemv_q6k_stream.h): its requests, waits and
         barriers alone; with the operand reads from LDS; the GEMV -- on the LM-head shape (two workgroups per
         compute unit) and on a down projection (one workgroup, three buffers)."""
-        lad_path = os.path.join(ROOT, "tattletale_amd", "libttq_ladder.so")
-        if not os.path.exists(lad_path):
-            raise RuntimeError("%s not found: build it with `python -m tattletale_amd.build`" % lad_path)
-        LAD = C.CDLL(lad_path)
+        LAD = ladder_lib()
         LAD.ttq_ladder_q6k_launch.restype = C.c_int
         LAD.ttq_ladder_q6k_launch.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p]
         L = _lib.lib()
@@ -666,6 +667,71 @@ def main() -> int:
             torch.cuda.empty_cache()
         return out
 
+    def run_ladder_gemm(steps: int, warmup: int, ms_=(512, 2048), n_out=14336, n_in=4096):
+        """What each role of the prefill GEMM kernel costs alone and together
+        (tattletale_amd/csrc/ttq_ladder_gemm.hip), 256 x 112 tiles, Q4_K 14336 x 4096."""
+        LAD = ladder_lib()
+        LAD.ttq_ladder_gemm_launch.restype = C.c_int
+        LAD.ttq_ladder_gemm_launch.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
+                                               C.c_int64, C.c_int64, C.c_void_p]
+        rng = np.random.default_rng(97)
+        # (kernel, ABL, what runs); kernel 0 = X straight into the consumers' registers, 1 = X staged through LDS
+        rungs = [(0, 31, "barriers, prologue, epilogue only"),
+                 (0, 4124, "consumers alone (A requests, B reads, MFMA; real values in the W tile)"),
+                 (0, 4104, "+ W loads and LDS stores, no dequantization"),
+                 (0, 0, "whole kernel"),
+                 (0, 3, "W producers alone"),
+                 (0, 2, "consumers without A requests + W producers"),
+                 (0, 1024, "whole kernel without barriers (roles free-running)"),
+                 (2, 31, "8 consumers of 32 rows: barriers, prologue, epilogue only"),
+                 (2, 4124, "8 consumers of 32 rows: consumers alone"),
+                 (2, 0, "8 consumers of 32 rows: whole kernel"),
+                 (2, 2, "8 consumers of 32 rows: consumers without A requests + W producers"),
+                 (2, 1024, "8 consumers of 32 rows: whole kernel without barriers"),
+                 (0, 8192 + 4124, "4 consumers alone, addresses as if X were packed in fragment order"),
+                 (0, 8192, "4 consumers, whole kernel, addresses as if X were packed in fragment order"),
+                 (0, 8192 + 1024, "4 consumers, whole kernel, packed-order addresses, no barriers"),
+                 (0, 8192 + 8, "4 consumers, packed-order addresses, producers without dequantization"),
+                 (0, 8192 + 4, "4 consumers, packed-order addresses, producers without LDS stores"),
+                 (0, 8192 + 64, "4 consumers, whole kernel, packed-order addresses, consumers at priority 3"),
+                 (0, 8192 + 128, "4 consumers, whole kernel, packed-order addresses, producers at priority 3"),
+                 (2, 8192 + 4124, "8 consumers alone, addresses as if X were packed in fragment order"),
+                 (2, 8192, "8 consumers, whole kernel, addresses as if X were packed in fragment order"),
+                 (1, 31, "LDS-staged X: barriers, prologue, epilogue only"),
+                 (1, 4126, "LDS-staged X: consumers alone (real values in LDS)"),
+                 (1, 4124, "LDS-staged X: consumers + X movers"),
+                 (1, 0, "LDS-staged X: whole kernel"),
+                 (1, 29, "LDS-staged X: X movers alone"),
+                 (1, 1024, "LDS-staged X: whole kernel without barriers"),
+                 (1, 2048, "LDS-staged X by global_load_lds: whole kernel")]
+        packed = random_packed(rng, F.Q4_K, n_out, n_in)
+        ncopies = rotated(packed.nbytes)
+        ws = [to_dev(packed) for _ in range(ncopies)]
+        out = {}
+        for m in ms_:
+            x = torch.randn((m, n_in), device=dev).to(torch.bfloat16)
+            y = torch.empty((m, n_out), dtype=torch.bfloat16, device=dev)
+            flop = 2.0 * m * n_out * n_in
+            rows = []
+            for kern, abl, what in rungs:
+                def step(i, kern=kern, abl=abl):
+                    rc = LAD.ttq_ladder_gemm_launch(kern, abl, ws[i % ncopies].data_ptr(), x.data_ptr(), y.data_ptr(), m,
+                                                    n_out, n_in, torch.cuda.current_stream(dev).cuda_stream)
+                    if rc != 0:
+                        raise RuntimeError("ttq_ladder_gemm_launch(%d, %d) returned %d" % (kern, abl, rc))
+                t = time_steps(step, max(20, steps // (10 if m <= 512 else 40)), max(3, warmup // 10))
+                rows.append({"kernel": kern, "abl": abl, "rung": what, "us_per_launch": t["ms"] * 1e3,
+                             "us_min": t["ms_min"] * 1e3, "us_max": t["ms_max"] * 1e3,
+                             "mfma_frac_if_full_flops": flop / (t["ms"] * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS})
+                log("[ladder gemm m=%d] k%d abl %-5d %-72s %8.2f us" % (m, kern, abl, what, t["ms"] * 1e3))
+            out["m%d" % m] = {"n_out": n_out, "n_in": n_in, "flop": flop, "rungs": rows}
+        del ws
+        torch.cuda.empty_cache()
+        return out
+
+    if args.only == "ladder_gemm":
+        print(json.dumps(run_ladder_gemm(args.steps, args.warmup)), flush=True)
+        return 0
     if args.only == "ladder_q6k":
         print(json.dumps(run_ladder_q6k(args.steps, args.warmup)), flush=True)
         return 0

@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libttq_hip.so")
-LADDER_LIB = os.path.join(HERE, "libttq_ladder.so")      # bench.py's roofline ladder, not the product
+LADDER_LIB = os.path.join(HERE, "libttq_ladder.so")      # bench.py's measurement ladders, built on demand
 
 SOURCES = [
     "ttq_api.hip",
@@ -88,17 +88,35 @@ def build_library(force: bool = True, verbose: bool = False) -> str:
         raise RuntimeError("link failed:\n%s\n%s" % (r.stdout, r.stderr))
     if verbose:
         print("built", LIB)
-    # the measurement-only ladder kernels (bench.py --only ladder)
-    lobj = os.path.join(objdir, "ttq_ladder.hip.o")
-    _compile(os.path.join(CSRC, "ttq_ladder.hip"), lobj)
-    r = subprocess.run([hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LADDER_LIB, lobj],
+    return LIB
+
+
+LADDER_SOURCES = ["ttq_ladder.hip", "ttq_ladder_gemm.hip"]
+
+
+def build_ladder(force: bool = False, verbose: bool = False) -> str:
+    """Compile the measurement-only ladder kernels (bench.py --only ladder*) into ``libttq_ladder.so``.
+    Not part of the product library and not built by ``build_library``."""
+    srcs = [os.path.join(CSRC, s) for s in LADDER_SOURCES]
+    deps = srcs + [os.path.join(CSRC, h) for h in os.listdir(CSRC) if h.endswith(".h")]
+    if not force and os.path.exists(LADDER_LIB) and os.path.getmtime(LADDER_LIB) >= max(os.path.getmtime(d) for d in deps):
+        return LADDER_LIB
+    objdir = os.path.join(CSRC, "build")
+    os.makedirs(objdir, exist_ok=True)
+    objs = [os.path.join(objdir, os.path.basename(s) + ".o") for s in srcs]
+    with ThreadPoolExecutor(max_workers=len(srcs)) as ex:
+        list(ex.map(lambda so: _compile(*so), zip(srcs, objs)))
+    r = subprocess.run([hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LADDER_LIB] + objs,
                        capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n%s\n%s" % (r.stdout, r.stderr))
     if verbose:
         print("built", LADDER_LIB)
-    return LIB
+    return LADDER_LIB
 
 
 if __name__ == "__main__":
+    if "--ladder" in sys.argv:
+        build_ladder(force=True, verbose=True)
+        sys.exit(0)
     build_library(force="--if-stale" not in sys.argv, verbose=True)

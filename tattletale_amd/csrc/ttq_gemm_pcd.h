@@ -1,0 +1,246 @@
+// Prefill GEMM for Q4_K, Q6_K and Q8_0 weights on gfx950, producer/consumer form with the activations read
+// straight from global memory into the consumers' registers: Y (m, n_out) = X (m, n_in) * W^T.
+//
+// Replaces F.linear(x, weight) for a multi-row bf16 activation
+// (workspace/libtorch/src/abi/neural_nets.nim:64-81; the prefill case of
+//  workspace/transformers/src/layers/attn.nim:154-156).
+//
+// A workgroup of eight wavefronts (two per SIMD) owns a (64 * MB) x BN tile of Y:
+//   consumers (wavefronts 0-3, 16 * MB rows of the tile each): v_mfma_f32_16x16x32_bf16, B fragments from the W
+//       tile in LDS, A fragments by buffer loads from X itself.  Lane (r, g) of a 16 x 32 A fragment holds eight
+//       consecutive k of row r: 16 bytes of the row-major activation, so a fragment is one 16-byte load per lane
+//       and needs no LDS at all.  The fragments of step s+2 are requested during step s into one of three register
+//       sets that rotate by name.
+//   producers (wavefronts 4-7): pc_produce_w of ttq_gemm_pc.h -- packed blocks, canonical dequantization, bf16
+//       nearest-even, B fragments into the double-buffered W tile.
+// One barrier per 64-k step.
+//
+// Why X bypasses LDS: every byte written to LDS goes through one port of about 85 bytes per cycle and compute unit,
+// whoever writes (ds_write or global_load_lds), and LDS reads queue behind waiting ds_writes.  With X staged through
+// LDS a step writes 32 KB of X and 14 KB of W and reads 88 KB of fragments; here it writes 14 KB and reads 56 KB.
+//
+// ABL (a bit mask, 0 in the product) switches stages off for the measurement ladder of ttq_ladder_gemm.hip:
+// 1 the consumers' MFMAs and B reads, 2 their A requests, 4 / 8 / 16 the producers' LDS stores / arithmetic / global
+// loads, 512 cycle counts around the barriers, 1024 no barriers, 4096 real values in the W tile at the start.
+#pragma once
+
+#include "ttq_gemm_pc.h"
+
+namespace ttq {
+
+constexpr int pcd_threads(int nc) { return (nc + 4) * 64; }   // NC consumers, 4 W producers
+
+// 16-byte buffer load the compiler neither moves nor waits for: left to itself it sinks the requests of the next
+// steps down to their first use (to save registers) and then waits for each of them in turn.  The caller counts
+// outstanding requests itself (wait_vmcnt) before it touches the result.
+template <int IMM>
+__device__ __forceinline__ void buffer_load16_async(u32x4_t& dst, u32x4_t rsrc, int voffset, int soffset) {
+  asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4"
+               : "=v"(dst) : "v"(voffset), "s"(rsrc), "s"(soffset), "n"(IMM) : "memory");
+}
+
+template <int NJ, int FMT, int MB, bool FUSE, int ABL = 0, int NC = 4>
+__global__ void __launch_bounds__(pcd_threads(NC))
+gemm_pcd_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, void* __restrict__ yv,
+                int y_dtype, const void* __restrict__ bias, int bias_dtype, int m, int n_out, int n_in,
+                int n_tiles, int m_tiles, int xcds_per_mtile, PcSplit sp) {
+  constexpr int BN = NJ * 16;
+  constexpr int kWUnits = 2 * NJ * 64;
+  constexpr int kPcBM = NC * 16 * MB;
+  constexpr int kPcdThreads = pcd_threads(NC);
+  constexpr int kStgBytes = 16 * MB * (BN * 2 + 16);      // a consumer's epilogue staging area
+  __shared__ uint4 sw[2 * kWUnits];
+  __shared__ __attribute__((aligned(16))) uint8_t stg[NC * kStgBytes];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  [[maybe_unused]] uint32_t t_bar = 0;
+  [[maybe_unused]] const uint64_t t_begin = (ABL & 512) ? __builtin_readcyclecounter() : 0;
+  [[maybe_unused]] const uint64_t rt_begin = (ABL & 512) ? __builtin_amdgcn_s_memrealtime() : 0;
+  auto bar = [&]() {
+    if constexpr ((ABL & 1024) != 0) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // ladder: every role at its own pace (results are garbage)
+    } else if constexpr ((ABL & 512) != 0) {
+      const uint64_t t0 = __builtin_readcyclecounter();
+      lds_barrier();
+      t_bar += (uint32_t)(__builtin_readcyclecounter() - t0);
+    } else {
+      lds_barrier();
+    }
+  };
+  auto trace_out = [&]() {
+    if constexpr ((ABL & 512) != 0) {
+      if (lane == 0) {
+        uint32_t* t = sp.counters + ((size_t)blockIdx.x * 12 + wave) * 4;
+        t[0] = (uint32_t)(__builtin_readcyclecounter() - t_begin);
+        t[1] = t_bar;
+        t[2] = 0;
+        t[3] = (uint32_t)(__builtin_amdgcn_s_memrealtime() - rt_begin);     // 100 MHz ticks
+      }
+    }
+  };
+  // Tile assignment: as in gemm_pc_kernel (one X slab per XCD L2 when the row tiles divide the XCDs evenly; copies
+  // of the tile grid when the launch is split along K).
+  const int ksplit = sp.splits > 1 ? (int)blockIdx.x / sp.tile_wgs : 0;
+  const int bid = (int)blockIdx.x - ksplit * sp.tile_wgs;
+  int n_tile, m_tile;
+  if (xcds_per_mtile > 0) {
+    const int xcd = bid & 7, slot = bid >> 3;
+    m_tile = xcd / xcds_per_mtile;
+    n_tile = slot * xcds_per_mtile + xcd % xcds_per_mtile;
+  } else {
+    m_tile = bid % m_tiles;
+    n_tile = bid / m_tiles;
+  }
+  if (n_tile >= n_tiles) return;
+  constexpr int BO = FUSE ? BN / 2 : BN;     // outputs per tile
+  const int n0 = n_tile * BO;
+  const int row_blocks = n_in >> 8;                                  // super-blocks (256 k) in a row of W
+  const int nblocks = sp.splits > 1 ? row_blocks / sp.splits : row_blocks;   // this workgroup's share of them
+  const int block0 = ksplit * nblocks;
+  const int ksteps = nblocks * 4;
+
+  if constexpr ((ABL & 4096) != 0) {
+    const uint4* src = reinterpret_cast<const uint4*>(x);
+    const int lim = min(m, 256) * n_in / 8;
+    for (int i = tid; i < 2 * kWUnits; i += kPcdThreads) sw[i] = src[(i * 5 + (int)blockIdx.x * 32 + 4096) % lim];
+    __syncthreads();
+  }
+
+  // One barrier per 64-k step, numbered s = -1 .. ksteps-1.  Barrier s means: the W fragments of step s+1 are
+  // complete in LDS (buffer (s+1) % 2) and every LDS read of step s has finished.  The consumers pass it near the
+  // end of step s, the producers after preparing step s+1.
+  if (wave >= NC) {
+    if constexpr ((ABL & 128) != 0) __builtin_amdgcn_s_setprio(3);
+    pc_produce_w<NJ, FMT, FUSE, ABL>(w, tid - NC * 64, n0, n_out, row_blocks, block0, nblocks,
+                                     (uint32_t)(size_t)(lptr_t)(&sw[0]), bar);
+    trace_out();
+    return;
+  }
+
+  // -------------------------------------------------------------------- consumer
+  if constexpr ((ABL & 64) != 0) __builtin_amdgcn_s_setprio(3);
+  const int m0 = m_tile * kPcBM + wave * (16 * MB);
+  const int fr = lane & 15, fg = lane >> 4;
+  // A fragment (row block ib, half h of step ks): row m0 + 16 ib + fr, bytes 128 ks + 64 h + 16 fg .. + 16 of it.
+  // Buffer loads take the per-lane offset (loop-invariant), the uniform offset of the step and the half as an
+  // immediate: no address arithmetic per request.  Rows past the end are clamped (never stored to Y).
+  const uint8_t* xb = reinterpret_cast<const uint8_t*>(x);
+  // raw buffer descriptor: base, stride 0, bytes (< 4 GiB: the launcher checks), 32-bit untyped data
+  const uint64_t xaddr = (uint64_t)(size_t)xb;
+  u32x4_t xrsrc = {(uint32_t)xaddr, (uint32_t)(xaddr >> 32) & 0xFFFFu, (uint32_t)m * (uint32_t)(n_in * 2), 0x00020000u};
+#pragma unroll
+  for (int q = 0; q < 4; q++) xrsrc[q] = (uint32_t)__builtin_amdgcn_readfirstlane((int)xrsrc[q]);
+  int aoff[MB];
+#pragma unroll
+  for (int ib = 0; ib < MB; ib++)
+    aoff[ib] = (ABL & 8192) ? (m_tile * (n_in / 64) * (kPcBM * 128) + wave * (16 * MB * 128) + ib * 2048 + lane * 16)   // ladder: as if X were packed in fragment order
+                            : (int)((uint32_t)min(m0 + 16 * ib + fr, m - 1) * (uint32_t)(n_in * 2) + (uint32_t)(fg * 16));
+  struct ASet { u32x4_t v[2][MB]; };
+  auto request_one = [&](ASet& dst, int koff, int h, int ib) {   // koff: byte offset of the step in a row
+    if constexpr ((ABL & 2) != 0) return;
+    if (h == 0) buffer_load16_async<0>(dst.v[0][ib], xrsrc, aoff[ib], koff);
+    else buffer_load16_async<(ABL & 8192) ? 1024 : 64>(dst.v[1][ib], xrsrc, aoff[ib], koff);
+  };
+  auto step_koff = [&](int ks) { return (4 * block0 + min(ks, ksteps - 1)) * ((ABL & 8192) ? kPcBM * 128 : 128); };   // past the end: a harmless re-read
+  // A step is 2*NJ groups of MB MFMAs: group g uses the A fragments of half g/NJ and the B fragment of column block
+  // g%NJ.  B fragments are read two groups ahead into a ring of four, the A fragments of step ks+2 are requested one
+  // per group at the start of step ks, and __builtin_amdgcn_sched_barrier pins that order.
+  constexpr int G = 2 * NJ;
+  static_assert(2 * MB <= G, "one A request per group");
+  bf16x8_t bring[4];
+  auto read_b = [&](bf16x8_t& dst, int buf, int g) {   // g = half * NJ + j
+    const uint4 v = sw[buf * kWUnits + g * 64 + lane];
+    __builtin_memcpy(&dst, &v, 16);
+  };
+
+  f32x4_t acc[MB][NJ];
+#pragma unroll
+  for (int i = 0; i < MB; i++)
+#pragma unroll
+    for (int j = 0; j < NJ; j++) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  // one step: `cur` holds its A fragments, `into` receives those of step ks+2; BUF is its W buffer and fixes the
+  // ring slot of its first group (2*NJ is 2 mod 4 for the tiles built here, or 0).
+  auto step = [&](const ASet& cur, ASet& into, auto bufc, int ks) {
+    constexpr int BUF = decltype(bufc)::value;
+    constexpr int SO = (BUF * G) & 3;
+    if constexpr ((ABL & 1) != 0) { bar(); return; }
+    // Requests complete in order: all but the youngest 2 * MB (those of step ks+1) have landed, `cur` among them.
+    wait_vmcnt<2 * MB>();
+    const int koff2 = step_koff(ks + 2);
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+      if (g == G - 2) bar();     // barrier ks: step ks+1 is in LDS, reads of step ks done
+      if (g + 2 < G) read_b(bring[(g + 2 + SO) & 3], BUF, g + 2);
+      else read_b(bring[(g + 2 + SO) & 3], BUF ^ 1, g + 2 - G);
+      // request r of the step (row block r / 2, half r % 2: the two halves of a 128-byte line one after the other,
+      // so that the second finds the line in the vector cache) goes out with group r * G / (2 * MB)
+#pragma unroll
+      for (int r = 0; r < 2 * MB; r++)
+        if (r * G / (2 * MB) == g) request_one(into, koff2, r % 2, r / 2);
+      __builtin_amdgcn_sched_barrier(0);
+      const int half = g / NJ, j = g % NJ;
+#pragma unroll
+      for (int i = 0; i < MB; i++) {
+        bf16x8_t a;
+        __builtin_memcpy(&a, &cur.v[half][i], 16);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bring[(g + SO) & 3], acc[i][j], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  ASet a0{}, a1{}, a2{};
+#pragma unroll
+  for (int h = 0; h < 2; h++)
+#pragma unroll
+    for (int ib = 0; ib < MB; ib++) request_one(a0, step_koff(0), h, ib);
+#pragma unroll
+  for (int h = 0; h < 2; h++)
+#pragma unroll
+    for (int ib = 0; ib < MB; ib++) request_one(a1, step_koff(1), h, ib);
+  bar();                         // barrier -1: the W fragments of step 0 are in LDS
+  read_b(bring[0], 0, 0);
+  read_b(bring[1], 0, 1);
+  using C0 = std::integral_constant<int, 0>;
+  using C1 = std::integral_constant<int, 1>;
+  static_assert(((2 * G) & 3) == 0, "two steps bring the B ring back to slot 0");
+  // (ksteps is a multiple of four; the register sets rotate with period three, the W buffers with period two)
+  for (int ks = 0; ks < ksteps; ks += 6) {
+    step(a0, a2, C0{}, ks);
+    step(a1, a0, C1{}, ks + 1);
+    if (ks + 2 >= ksteps) break;
+    step(a2, a1, C0{}, ks + 2);
+    step(a0, a2, C1{}, ks + 3);
+    if (ks + 4 >= ksteps) break;
+    step(a1, a0, C0{}, ks + 4);
+    step(a2, a1, C1{}, ks + 5);
+  }
+  wait_vmcnt<0>();               // the re-reads past the last step
+  trace_out();
+
+  pc_epilogue<NJ, MB, FUSE, NC>(acc, PcEpi{sp, ksplit, m_tile, n_tile, n_tiles, wave, lane, stg + wave * kStgBytes, yv,
+                                       y_dtype, bias, bias_dtype, m, n_out, n0, m0});
+}
+
+// The caller owns the split-K workspace: sp.splits == 1 (no partials, no counters) or a prepared PcSplit whose
+// tile_wgs this function fills in.
+template <int FMT, int MB, int NJ, bool FUSE, int ABL = 0, int NC = 4>
+static hipError_t launch_pcd_grid(const uint8_t* wb, const uint16_t* x, void* y, int y_dtype, const void* bias,
+                                  int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, PcSplit sp, hipStream_t s) {
+  constexpr int BO = FUSE ? NJ * 8 : NJ * 16, BM = NC * 16 * MB;
+  const int n_tiles = (int)((n_out + BO - 1) / BO), m_tiles = (int)((m + BM - 1) / BM);
+  int xcds_per_mtile = 0;
+  unsigned nwg = (unsigned)(n_tiles * m_tiles);
+  if (m_tiles >= 2 && m_tiles <= 8 && 8 % m_tiles == 0) {
+    xcds_per_mtile = 8 / m_tiles;
+    nwg = (unsigned)(((n_tiles + xcds_per_mtile - 1) / xcds_per_mtile) * 8);
+  }
+  sp.tile_wgs = (int)nwg;
+  hipLaunchKernelGGL((gemm_pcd_kernel<NJ, FMT, MB, FUSE, ABL, NC>), dim3(nwg * (unsigned)sp.splits), dim3(pcd_threads(NC)), 0, s,
+                     wb, x, y, y_dtype, bias, bias_dtype, (int)m, (int)n_out, (int)n_in, n_tiles, m_tiles, xcds_per_mtile, sp);
+  return hipGetLastError();
+}
+
+}  // namespace ttq
