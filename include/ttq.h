@@ -15,7 +15,18 @@
  *
  * Conventions
  *   - All device pointers are HIP device memory on the current device; the library keeps
- *     no pointer after a call returns (work may still be in flight on `stream`).
+ *     no pointer to a caller's buffer after a call returns (work may still be in flight on `stream`).
+ *   - Workspaces.  A few paths need device memory beyond inputs and outputs (partial sums of a
+ *     launch split along K, the trellis GEMV's hand-off words, a bf16 or rotated copy of the
+ *     activations).  The ttq_*_ws entry points take it from the caller -- the reference's
+ *     convention, where the caller makes every tensor with from_blob / empty
+ *     (workspace/libtorch/src/abi/torch_tensors.nim:250-289) -- allocate nothing, and can be
+ *     captured into a HIP graph the first time they run.  The entry points without a workspace
+ *     argument are the convenience form: the library allocates what the call needs on first use,
+ *     one buffer per (device, stream), keeps it until ttq_release_workspaces, and such a first call
+ *     must not happen under capture.  A graph captured with a library-owned workspace must be
+ *     replayed on the stream it was captured on (another stream's launches use another buffer and
+ *     would overlap it), and one host thread at a time may issue calls on a given stream.
  *   - `stream` is a hipStream_t passed as void*; NULL = the default stream.  Launches are
  *     asynchronous; the caller synchronises (same contract as a torch tensor op).
  *   - Return value: 0 on success, a negative ttq_status otherwise.  No C++ exception
@@ -33,7 +44,7 @@
 extern "C" {
 #endif
 
-#define TTQ_VERSION 110 /* 0.1.1 */
+#define TTQ_VERSION 120 /* 0.1.2 */
 
 /* Exported symbols: the library is built with hidden visibility by default. */
 #if defined(TTQ_BUILD)
@@ -51,7 +62,8 @@ typedef enum {
   TTQ_ERR_FORMAT = -5,      /* unknown format / bits / codebook */
   TTQ_ERR_UNSUPPORTED = -6, /* valid request outside what the kernels cover (size limits) */
   TTQ_ERR_HIP = -7,         /* a HIP runtime call failed; see ttq_last_hip_error() */
-  TTQ_ERR_ALIAS = -8        /* an output overlaps an input in a call that must run out of place */
+  TTQ_ERR_ALIAS = -8,       /* an output overlaps an input in a call that must run out of place */
+  TTQ_ERR_WORKSPACE = -9    /* caller-owned workspace NULL, misaligned or smaller than ttq_workspace_bytes says */
 } ttq_status;
 
 /* Element types of activation / output / bias buffers.  They correspond to the
@@ -63,8 +75,9 @@ typedef enum { TTQ_Q8_0 = 0, TTQ_Q4_K = 1, TTQ_Q6_K = 2, TTQ_EXL3 = 3 } ttq_form
 
 /* How ttq_linear_forward may trade accuracy for speed when there are several activation rows. */
 typedef enum {
-  TTQ_PRECISION_AUTO = 0,       /* from five rows on, whichever kernel the shape makes cheaper */
-  TTQ_PRECISION_F32_SCALES = 1  /* always the decode kernels: fp32 scales, rel-L2 <= 1e-3 whatever m is */
+  TTQ_PRECISION_AUTO = 0,       /* from five rows on, whichever kernel of the activations' own type the shape makes cheaper */
+  TTQ_PRECISION_F32_SCALES = 1, /* always the decode kernels: fp32 scales, rel-L2 <= 1e-3 whatever m is */
+  TTQ_PRECISION_BF16_OK = 2     /* as AUTO, and fp16 / fp32 activations may be rounded to bf16 for the matrix-core GEMM */
 } ttq_precision;
 
 /* Codebook functions of the trellis format. */
@@ -112,15 +125,73 @@ typedef struct ttq_qlinear {
  * run matrix-core kernels that round each dequantized weight once to bf16 (fp16) -- the 2e-2 class
  * of the GEMM entry points -- when its cost estimate prefers them for the shape.  A layer with
  * precision == TTQ_PRECISION_F32_SCALES keeps the decode kernels, and with them the 1e-3 class,
- * for every m.  From 256 rows of fp16 / fp32 activations on (GGUF formats, no F32_SCALES), the rows
- * are first rounded to bf16 into a workspace the library keeps per (device, stream) -- allocated on
- * first use and grown on demand, so that first call must not happen under graph capture -- and the
- * bf16 matrix-core GEMM runs on the copy.
+ * for every m.  The operator computes in the type of x (linear.nim:45-57): fp32 activations always
+ * take the decode kernels (1e-3 class), fp16 activations those or the fp16 few-row matrix-core
+ * kernel.  Only a layer with precision == TTQ_PRECISION_BF16_OK lets the library round 256 or more
+ * rows of fp16 / fp32 activations to bf16 (into a workspace) and run the bf16 matrix-core GEMM on
+ * the copy (2e-2 class).
  * Limits (TTQ_ERR_UNSUPPORTED beyond): the decode kernels take n_in <= 32768 for Q4_K / Q6_K with
  * 16-bit activations and n_in <= 16384 otherwise; any m (rows are taken 65535 at a time where a
  * kernel needs that).  m == 0 or n_out == 0 returns TTQ_OK without touching a pointer. */
 TTQ_API int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int64_t m,
                        void* y, int y_dtype, void* stream);
+
+/* Bytes of caller-owned workspace that ttq_linear_forward_ws needs for this layer, row count and
+ * activation type (0: none; negative status on bad arguments).  An upper bound that depends on the
+ * device's compute-unit count; a pure host function.  No counterpart in the reference, where
+ * F.linear allocates what it needs inside libtorch; the caller makes the buffer as it makes every
+ * tensor (F.zeros / from_blob, torch_tensors.nim:250-289). */
+TTQ_API int64_t ttq_workspace_bytes(const ttq_qlinear* layer, int64_t m, int x_dtype);
+
+/* ttq_linear_forward with the workspace in the caller's hands: never allocates, safe to capture on
+ * its first call.  `ws` is 16-byte aligned device memory of at least ttq_workspace_bytes(layer, m,
+ * x_dtype) bytes (TTQ_ERR_WORKSPACE otherwise; ws may be NULL when that is 0), CLEARED TO ZERO ONCE
+ * before its first use: the library keeps arrival counters and a generation count in its first
+ * bytes and leaves them ready for the next call.  One workspace serves any sequence of calls for
+ * any layers on one stream (each call sized by its own ttq_workspace_bytes); calls that may
+ * overlap -- different streams -- need different workspaces. */
+TTQ_API int ttq_linear_forward_ws(const ttq_qlinear* layer, const void* x, int x_dtype, int64_t m,
+                          void* y, int y_dtype, void* ws, int64_t ws_bytes, void* stream);
+
+/* Frees every workspace the library allocated for the entry points without a workspace argument.
+ * Only when nothing that could use one is in flight, and no captured graph that was recorded
+ * through such an entry point will be replayed again: synchronize the device first. */
+TTQ_API int ttq_release_workspaces(void);
+
+/* Which kernel family ttq_linear_forward launches for this layer, row count and types: a
+ * ttq_route_id (>= 0) or a negative status.  It runs the dispatch code of ttq_linear_forward itself
+ * with the launches switched off, touches no buffer and no device memory, and depends only on its
+ * arguments and the current device's compute-unit count (256 when no device is visible).  No
+ * counterpart in the reference: there F.linear chooses inside libtorch. */
+typedef enum {
+  TTQ_ROUTE_NONE = 0,
+  TTQ_ROUTE_GEMV_Q4K_STREAM = 1,     /* Q4_K, weights streamed HBM -> LDS as whole cache lines */
+  TTQ_ROUTE_GEMV_Q4K_STREAM4 = 2,    /* ... two to four activation rows per pass */
+  TTQ_ROUTE_GEMV_Q4K_SLICE = 3,      /* ... long rows, K dealt to the wavefronts */
+  TTQ_ROUTE_GEMV_Q4K_BATCH4 = 4,
+  TTQ_ROUTE_GEMV_Q4K_BATCH = 5,
+  TTQ_ROUTE_GEMV_Q4K_MFMA = 6,       /* register-streamed int8 matrix-core kernel */
+  TTQ_ROUTE_GEMV_Q6K_STREAM = 7,
+  TTQ_ROUTE_GEMV_Q6K_STREAM4 = 8,
+  TTQ_ROUTE_GEMV_Q8_STREAM = 9,
+  TTQ_ROUTE_GEMV_Q8_WIN = 10,
+  TTQ_ROUTE_GEMV_Q8_MFMA = 11,
+  TTQ_ROUTE_GEMV_DOT2 = 12,
+  TTQ_ROUTE_GEMV_DOT2_MULTI = 13,
+  TTQ_ROUTE_GEMV_GENERIC = 14,
+  TTQ_ROUTE_GEMM_PC = 20,            /* producer / consumer prefill GEMM */
+  TTQ_ROUTE_GEMM_PC_SPLIT_K = 21,    /* ... in several copies along K (takes a workspace) */
+  TTQ_ROUTE_GEMM_SKINNY = 22,        /* 17-64 rows */
+  TTQ_ROUTE_GEMM_SKINNY_CHUNKED = 23,
+  TTQ_ROUTE_GEMM_Q4K_TILES = 24,     /* single-role tiled kernel (128-column tiles, activations beyond 4 GiB) */
+  TTQ_ROUTE_GEMM_PC_BF16_COPY = 25,  /* TTQ_PRECISION_BF16_OK: bf16 copy of fp16 / fp32 activations, then GEMM_PC */
+  TTQ_ROUTE_EXL3_GEMV = 30,
+  TTQ_ROUTE_EXL3_GEMV_SLICED = 31,   /* K sliced over workgroups that meet in a workspace */
+  TTQ_ROUTE_EXL3_GEMM = 32,
+  TTQ_ROUTE_EXL3_GEMV_TWO_LAUNCHES = 33
+} ttq_route_id;
+TTQ_API int ttq_route(const ttq_qlinear* layer, int64_t m, int x_dtype, int y_dtype);
+TTQ_API const char* ttq_route_name(int route);
 
 /* ---- decode GEMV, one entry per block format (m rows of x, normally m == 1) -------- */
 /* y[m][n_out] (fp32) = x[m][n_in] * W^T.  Stand in for F.linear(x, weight) with a
@@ -151,8 +222,9 @@ TTQ_API int ttq_gemv_exl3(const uint16_t* trellis, const uint16_t* suh_f16, cons
  * call there until the process ends.  It calls no allocating routine.  Returns TTQ_ERR_UNSUPPORTED
  * for m > 8 and for a launch that would need more than the 4 MiB (a device with more than 256
  * compute units).  All calls on one GPU share the array: calls that may overlap there (different
- * streams, different threads) race; calls on one stream do not.  Every call leaves the words it used
- * at zero, which is what the next call expects. */
+ * streams, different threads) race; calls on one stream do not.  Nothing is cleared between calls:
+ * the words carry the tag of the launch that wrote them (the array's generation count + 1), and
+ * every launch advances the count when its last group is done. */
 TTQ_API int ttq_gemv_exl3_noalloc(const uint16_t* trellis, const uint16_t* suh_f16, const uint16_t* svh_f16,
                   const uint16_t* x_f16, float* y, int64_t m, int64_t n_out, int64_t n_in,
                   int bits, int codebook, void* stream);
@@ -177,6 +249,15 @@ TTQ_API int ttq_gemm_q6_k(const void* w, const uint16_t* x_bf16, uint16_t* y_bf1
                   int64_t n_out, int64_t n_in, void* stream);
 TTQ_API int ttq_gemm_q8_0(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m,
                   int64_t n_out, int64_t n_in, void* stream);
+/* The three above with the workspace in the caller's hands (see ttq_linear_forward_ws for the
+ * contract: cleared once, never allocates, capturable on the first call).  Size: ttq_workspace_bytes
+ * of a ttq_qlinear with this format and shape, m and TTQ_BF16.  No counterpart in the reference. */
+TTQ_API int ttq_gemm_q4_k_ws(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m,
+                     int64_t n_out, int64_t n_in, void* ws, int64_t ws_bytes, void* stream);
+TTQ_API int ttq_gemm_q6_k_ws(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m,
+                     int64_t n_out, int64_t n_in, void* ws, int64_t ws_bytes, void* stream);
+TTQ_API int ttq_gemm_q8_0_ws(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m,
+                     int64_t n_out, int64_t n_in, void* ws, int64_t ws_bytes, void* stream);
 /* The operator for a trellis-coded weight and many activation rows (prefill: seq_len > 1 at every
  * projection, attn.nim:154-156): y (m, n_out) fp32 = svh o H( T * H(suh o x) ) for x (m, n_in) of any
  * dtype.  The activations are rotated once and rounded to fp16 (rel-L2 <= 2e-2 class, about 3e-4 in
@@ -188,6 +269,20 @@ TTQ_API int ttq_gemm_q8_0(const void* w, const uint16_t* x_bf16, uint16_t* y_bf1
 TTQ_API int ttq_gemm_exl3(const uint16_t* trellis, const uint16_t* suh_f16, const uint16_t* svh_f16,
                   const void* x, int x_dtype, float* y, int64_t m, int64_t n_out, int64_t n_in,
                   int bits, int codebook, void* stream);
+/* ttq_gemm_exl3 and ttq_gemv_exl3 with the workspace in the caller's hands (contract of
+ * ttq_linear_forward_ws; size: ttq_workspace_bytes of a TTQ_EXL3 ttq_qlinear of this shape).  No
+ * counterpart in the reference. */
+TTQ_API int ttq_gemm_exl3_ws(const uint16_t* trellis, const uint16_t* suh_f16, const uint16_t* svh_f16,
+                     const void* x, int x_dtype, float* y, int64_t m, int64_t n_out, int64_t n_in,
+                     int bits, int codebook, void* ws, int64_t ws_bytes, void* stream);
+TTQ_API int ttq_gemv_exl3_ws(const uint16_t* trellis, const uint16_t* suh_f16, const uint16_t* svh_f16,
+                     const uint16_t* x_f16, float* y, int64_t m, int64_t n_out, int64_t n_in,
+                     int bits, int codebook, void* ws, int64_t ws_bytes, void* stream);
+/* Diagnostics: how many times the last slice of a sliced trellis GEMV looks at a hand-off word
+ * that has not arrived before it gives the row up and writes NaN (default 65536; 0 = look once).
+ * Process-wide; returns the previous value.  Exists so that the give-up path can be exercised from
+ * the host with every kernel exiting normally.  No counterpart in the reference. */
+TTQ_API int ttq_debug_set_exl3_poll_limit(int limit);
 /* Prefill half of GatedMLP.forward in one kernel: y (m, n_ff) = silu(x Wg^T) * (x Wu^T) with the
  * fused gate||up weight of mlp.nim:39 (2*n_ff rows, gate rows first) -- gate_up_proj.forward
  * followed by silu_and_mul (mlp.nim:56-59, activations.nim:14-38), silu(g)*u formed in fp32 from

@@ -14,10 +14,19 @@ LIB_PATH = os.path.join(HERE, "libttq_hip.so")
 # status / dtype / format codes (include/ttq.h)
 OK = 0
 ERR_NULL, ERR_SHAPE, ERR_ALIGN, ERR_DTYPE, ERR_FORMAT, ERR_UNSUPPORTED, ERR_HIP, ERR_ALIAS = -1, -2, -3, -4, -5, -6, -7, -8
+ERR_WORKSPACE = -9
 F32, F16, BF16 = 0, 1, 2
 Q8_0, Q4_K, Q6_K, EXL3 = 0, 1, 2, 3
 CB_3INST, CB_MCG = 0, 1
-PRECISION_AUTO, PRECISION_F32_SCALES = 0, 1
+PRECISION_AUTO, PRECISION_F32_SCALES, PRECISION_BF16_OK = 0, 1, 2
+# ttq_route_id
+ROUTE = {
+    "none": 0, "gemv_q4k_stream": 1, "gemv_q4k_stream4": 2, "gemv_q4k_slice": 3, "gemv_q4k_batch4": 4,
+    "gemv_q4k_batch": 5, "gemv_q4k_mfma": 6, "gemv_q6k_stream": 7, "gemv_q6k_stream4": 8, "gemv_q8_stream": 9,
+    "gemv_q8_win": 10, "gemv_q8_mfma": 11, "gemv_dot2": 12, "gemv_dot2_multi": 13, "gemv_generic": 14,
+    "gemm_pc": 20, "gemm_pc_split_k": 21, "gemm_skinny": 22, "gemm_skinny_chunked": 23, "gemm_q4k_tiles": 24,
+    "gemm_pc_bf16_copy": 25, "exl3_gemv": 30, "exl3_gemv_sliced": 31, "exl3_gemm": 32, "exl3_gemv_two_launches": 33,
+}
 
 
 class TtqLibraryError(RuntimeError):
@@ -52,6 +61,17 @@ SIGNATURES = {
     "ttq_last_hip_error": (_i32, []),
     "ttq_packed_nbytes": (_i64, [_i32, _i64, _i64, _i32]),
     "ttq_linear_forward": (_i32, [C.POINTER(QLinearStruct), _vp, _i32, _i64, _vp, _i32, _vp]),
+    "ttq_workspace_bytes": (_i64, [C.POINTER(QLinearStruct), _i64, _i32]),
+    "ttq_linear_forward_ws": (_i32, [C.POINTER(QLinearStruct), _vp, _i32, _i64, _vp, _i32, _vp, _i64, _vp]),
+    "ttq_release_workspaces": (_i32, []),
+    "ttq_route": (_i32, [C.POINTER(QLinearStruct), _i64, _i32, _i32]),
+    "ttq_route_name": (C.c_char_p, [_i32]),
+    "ttq_gemm_q4_k_ws": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp]),
+    "ttq_gemm_q6_k_ws": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp]),
+    "ttq_gemm_q8_0_ws": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp]),
+    "ttq_gemm_exl3_ws": (_i32, [_vp, _vp, _vp, _vp, _i32, _vp, _i64, _i64, _i64, _i32, _i32, _vp, _i64, _vp]),
+    "ttq_gemv_exl3_ws": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32, _vp, _i64, _vp]),
+    "ttq_debug_set_exl3_poll_limit": (_i32, [_i32]),
     "ttq_gemv_q8_0": (_i32, [_vp, _vp, _i32, _vp, _i64, _i64, _i64, _vp]),
     "ttq_gemv_q4_k": (_i32, [_vp, _vp, _i32, _vp, _i64, _i64, _i64, _vp]),
     "ttq_gemv_q6_k": (_i32, [_vp, _vp, _i32, _vp, _i64, _i64, _i64, _vp]),

@@ -26,6 +26,8 @@ int device_num_cus() {
   return cus;
 }
 
+thread_local RouteProbe* t_route_probe = nullptr;
+
 hipError_t allow_large_lds(const void* kernel, LargeLds& state) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
@@ -84,6 +86,10 @@ int check_gemv_limits(int format, int x_dtype, int64_t n_in) {
   const int64_t lim = long_rows ? ttq::kMaxGemvIn16 : ttq::kMaxGemvInF32;
   return n_in <= lim ? TTQ_OK : TTQ_ERR_UNSUPPORTED;
 }
+
+// grid dimensions y and z end at 65535: the trellis GEMV puts groups of 8 activation rows on z, the fused decode
+// kernels and RMSNorm one row per workgroup on y
+constexpr int64_t kMaxExl3GemvRows = 8 * 65535, kMaxGridRows = 65535;
 
 // launch_gemv puts the activation rows (or passes over them) on gridDim.y, which ends at 65535
 hipError_t launch_gemv_any_m(int format, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
@@ -147,6 +153,7 @@ const char* ttq_strerror(int status) {
     case TTQ_ERR_UNSUPPORTED: return "request outside the supported size limits";
     case TTQ_ERR_HIP: return "HIP runtime error (see ttq_last_hip_error)";
     case TTQ_ERR_ALIAS: return "output buffer overlaps an input where that is not allowed";
+    case TTQ_ERR_WORKSPACE: return "caller-owned workspace is NULL, misaligned or smaller than ttq_workspace_bytes says";
     default: return "unknown status";
   }
 }
@@ -187,7 +194,7 @@ int ttq_gemv_exl3(const uint16_t* trellis, const uint16_t* suh_f16, const uint16
   if (!trellis || !suh_f16 || !svh_f16 || !x_f16 || !y) return TTQ_ERR_NULL;
   if (!aligned16(trellis) || !aligned16(x_f16) || !aligned16(y) || !aligned8(suh_f16) || !aligned8(svh_f16))
     return TTQ_ERR_ALIGN;
-  if (n_in > ttq::kMaxGemvInF32) return TTQ_ERR_UNSUPPORTED;
+  if (n_in > ttq::kMaxGemvInF32 || m > kMaxExl3GemvRows) return TTQ_ERR_UNSUPPORTED;
   return hip_status(ttq::launch_gemv_exl3(trellis, suh_f16, svh_f16, x_f16, TTQ_F16, y, TTQ_F32,
                                           nullptr, 0, m, n_out, n_in, bits, codebook,
                                           static_cast<hipStream_t>(stream)));
@@ -268,7 +275,7 @@ int ttq_gemv_q4_k_silu_mul(const void* w, const void* x, int x_dtype, void* y, i
   if (m <= 4 && ttq::gemv_q4k_stream_fused_supported(x_dtype, n_ff, n_in))
     return hip_status(ttq::launch_gemv_q4k_stream_fused(w, x, x_dtype, y, y_dtype, m, n_ff, n_in,
                                                         static_cast<hipStream_t>(stream)));
-  if (!ttq::gemv_fused_supported(TTQ_Q4_K, x_dtype, n_ff, n_in, true)) return TTQ_ERR_UNSUPPORTED;
+  if (!ttq::gemv_fused_supported(TTQ_Q4_K, x_dtype, n_ff, n_in, true) || m > kMaxGridRows) return TTQ_ERR_UNSUPPORTED;
   return hip_status(ttq::launch_gemv_fused(w, x, x_dtype, y, y_dtype, nullptr, 0, m, n_ff, n_in, true, nullptr,
                                            nullptr, 0.f, nullptr, nullptr, static_cast<hipStream_t>(stream)));
 }
@@ -278,6 +285,7 @@ int ttq_rmsnorm(const void* x, const void* residual, const void* gamma, float ep
   if (!valid_dtype(dtype)) return TTQ_ERR_DTYPE;
   if (m < 0 || n < 0 || !(eps >= 0.f)) return TTQ_ERR_SHAPE;
   if (m == 0 || n == 0) return TTQ_OK;
+  if (m > kMaxGridRows) return TTQ_ERR_UNSUPPORTED;
   if (!x || !gamma || !normed_out) return TTQ_ERR_NULL;
   if (!aligned16(x) || !aligned16(gamma) || !aligned16(normed_out) || (residual && !aligned16(residual)) ||
       (new_residual_out && !aligned16(new_residual_out)))
@@ -324,7 +332,7 @@ int ttq_gemv_q4_k_rmsnorm(const void* w, const void* x, const void* residual, co
     return hip_status(ttq::launch_gemv_q4k_stream_norm(w, x, x_dtype, y, y_dtype, m, n_out, n_in, silu_mul != 0, residual,
                                                        gamma, eps, new_residual_out, normed_out,
                                                        static_cast<hipStream_t>(stream)));
-  if (!ttq::gemv_fused_supported(TTQ_Q4_K, x_dtype, n_out, n_in, silu_mul != 0)) return TTQ_ERR_UNSUPPORTED;
+  if (!ttq::gemv_fused_supported(TTQ_Q4_K, x_dtype, n_out, n_in, silu_mul != 0) || m > kMaxGridRows) return TTQ_ERR_UNSUPPORTED;
   return hip_status(ttq::launch_gemv_fused(w, x, x_dtype, y, y_dtype, nullptr, 0, m, n_out, n_in, silu_mul != 0,
                                            residual, gamma, eps, new_residual_out, normed_out,
                                            static_cast<hipStream_t>(stream)));
@@ -407,7 +415,9 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
   if (!layer) return TTQ_ERR_NULL;
   if (!valid_dtype(x_dtype) || !valid_dtype(y_dtype)) return TTQ_ERR_DTYPE;
   if (layer->bias && !valid_dtype(layer->bias_dtype)) return TTQ_ERR_DTYPE;
-  if (layer->precision != TTQ_PRECISION_AUTO && layer->precision != TTQ_PRECISION_F32_SCALES) return TTQ_ERR_FORMAT;
+  if (layer->precision != TTQ_PRECISION_AUTO && layer->precision != TTQ_PRECISION_F32_SCALES &&
+      layer->precision != TTQ_PRECISION_BF16_OK)
+    return TTQ_ERR_FORMAT;
   const int rc = check_shape(layer->format, m, layer->n_out, layer->n_in, layer->bits, layer->codebook);
   if (rc != TTQ_OK) return rc;
   if (m == 0 || layer->n_out == 0) return TTQ_OK;   // an empty batch gives an empty output, as F.linear does
@@ -426,6 +436,7 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
           static_cast<const uint16_t*>(layer->qweight), static_cast<const uint16_t*>(layer->suh),
           static_cast<const uint16_t*>(layer->svh), x, x_dtype, y, y_dtype, layer->bias, layer->bias_dtype, m, n_out,
           n_in, layer->bits, layer->codebook, s));
+    if (m > kMaxExl3GemvRows) return TTQ_ERR_UNSUPPORTED;
     return hip_status(ttq::launch_gemv_exl3(
         static_cast<const uint16_t*>(layer->qweight), static_cast<const uint16_t*>(layer->suh),
         static_cast<const uint16_t*>(layer->svh), x, x_dtype, y, y_dtype, layer->bias,
@@ -448,12 +459,15 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
       return hip_status(ttq::launch_gemm(layer->format, layer->qweight, static_cast<const uint16_t*>(x), y, y_dtype,
                                          layer->bias, layer->bias_dtype, m, n_out, n_in, s));
   }
-  // fp16 / fp32 activations, 256 rows or more (four launches of the few-row kernel): round them to bf16 into the library's
-  // workspace (4096 rows at a time) and run the bf16 matrix-core GEMM (weights and activations rounded to bf16:
-  // the 2e-2 class, like the GEMM entry points)
+  // fp16 / fp32 activations, 256 rows or more, and only where the layer says that bf16 activations will do
+  // (TTQ_PRECISION_BF16_OK; the operator computes in the type of x otherwise): round them to bf16 into a workspace
+  // (4096 rows at a time) and run the bf16 matrix-core GEMM (weights and activations rounded to bf16: the 2e-2
+  // class, like the GEMM entry points)
   const bool block_fmt = layer->format == TTQ_Q4_K || layer->format == TTQ_Q6_K || layer->format == TTQ_Q8_0;
   if ((x_dtype == TTQ_F16 || x_dtype == TTQ_F32) && block_fmt && m >= 256 && route != 1 && n_in % 8 == 0 &&
+      layer->precision == TTQ_PRECISION_BF16_OK &&
       ttq::gemm_pc_supported(layer->format, m < 4096 ? m : 4096, n_out, n_in, 112)) {
+    if (ttq::route_probe(ttq::kRouteGemmPcBf16Copy)) return TTQ_OK;
     constexpr int64_t kRows = 4096;
     void* ws = nullptr;
     const int64_t block_rows = m < kRows ? m : kRows;
@@ -479,15 +493,154 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
     float us = (float)full * ttq::gemm_skinny_estimate_us(layer->format, 64, n_out, n_in);
     if (rest) us += ttq::gemm_skinny_estimate_us(layer->format, rest, n_out, n_in);
     const bool gemv_ok = check_gemv_limits(layer->format, x_dtype, n_in) == TTQ_OK;
-    if (!gemv_ok || route == 2 || us < ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in))
+    if (!gemv_ok || route == 2 || us < ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in)) {
+      if (ttq::route_probe(ttq::kRouteGemmSkinnyChunked)) return TTQ_OK;
       return hip_status(ttq::launch_gemm_skinny_chunked(layer->format, layer->qweight, static_cast<const uint16_t*>(x),
                                                         x_dtype, y, y_dtype, layer->bias, layer->bias_dtype, m, n_out,
                                                         n_in, s));
+    }
   }
   const int lim = check_gemv_limits(layer->format, x_dtype, n_in);
   if (lim != TTQ_OK) return lim;
   return hip_status(launch_gemv_any_m(layer->format, layer->qweight, x, x_dtype, y, y_dtype, layer->bias,
                                       layer->bias_dtype, m, n_out, n_in, s));
 }
+
+// ---- which kernel family ttq_linear_forward would launch
+int ttq_route(const ttq_qlinear* layer, int64_t m, int x_dtype, int y_dtype) {
+  if (!layer) return TTQ_ERR_NULL;
+  // the dispatch itself, with a probe bound to this thread (nothing is launched, allocated or dereferenced) and
+  // stand-ins for the buffers
+  ttq_qlinear probe_layer = *layer;
+  alignas(16) static char stand_in[16];
+  probe_layer.qweight = stand_in;
+  if (probe_layer.format == TTQ_EXL3) {
+    probe_layer.suh = stand_in;
+    probe_layer.svh = stand_in;
+  }
+  if (layer->bias) probe_layer.bias = stand_in;
+  ttq::RouteProbe probe{0};
+  ttq::t_route_probe = &probe;
+  const int rc = ttq_linear_forward(&probe_layer, stand_in, x_dtype, m, stand_in, y_dtype, nullptr);
+  ttq::t_route_probe = nullptr;
+  return rc != TTQ_OK ? rc : probe.route;
+}
+
+const char* ttq_route_name(int route) {
+  switch (route) {
+    case TTQ_ROUTE_NONE: return "none (empty call)";
+    case TTQ_ROUTE_GEMV_Q4K_STREAM: return "gemv_q4k_stream";
+    case TTQ_ROUTE_GEMV_Q4K_STREAM4: return "gemv_q4k_stream4";
+    case TTQ_ROUTE_GEMV_Q4K_SLICE: return "gemv_q4k_slice";
+    case TTQ_ROUTE_GEMV_Q4K_BATCH4: return "gemv_q4k_batch4";
+    case TTQ_ROUTE_GEMV_Q4K_BATCH: return "gemv_q4k_batch";
+    case TTQ_ROUTE_GEMV_Q4K_MFMA: return "gemv_q4k_mfma";
+    case TTQ_ROUTE_GEMV_Q6K_STREAM: return "gemv_q6k_stream";
+    case TTQ_ROUTE_GEMV_Q6K_STREAM4: return "gemv_q6k_stream4";
+    case TTQ_ROUTE_GEMV_Q8_STREAM: return "gemv_q8_stream";
+    case TTQ_ROUTE_GEMV_Q8_WIN: return "gemv_q8_win";
+    case TTQ_ROUTE_GEMV_Q8_MFMA: return "gemv_q8_mfma";
+    case TTQ_ROUTE_GEMV_DOT2: return "gemv_dot2";
+    case TTQ_ROUTE_GEMV_DOT2_MULTI: return "gemv_dot2_multi";
+    case TTQ_ROUTE_GEMV_GENERIC: return "gemv_generic";
+    case TTQ_ROUTE_GEMM_PC: return "gemm_pc";
+    case TTQ_ROUTE_GEMM_PC_SPLIT_K: return "gemm_pc_split_k";
+    case TTQ_ROUTE_GEMM_SKINNY: return "gemm_skinny";
+    case TTQ_ROUTE_GEMM_SKINNY_CHUNKED: return "gemm_skinny_chunked";
+    case TTQ_ROUTE_GEMM_Q4K_TILES: return "gemm_q4k_tiles";
+    case TTQ_ROUTE_GEMM_PC_BF16_COPY: return "gemm_pc_bf16_copy";
+    case TTQ_ROUTE_EXL3_GEMV: return "exl3_gemv";
+    case TTQ_ROUTE_EXL3_GEMV_SLICED: return "exl3_gemv_sliced";
+    case TTQ_ROUTE_EXL3_GEMM: return "exl3_gemm";
+    case TTQ_ROUTE_EXL3_GEMV_TWO_LAUNCHES: return "exl3_gemv_two_launches";
+    default: return "unknown route";
+  }
+}
+
+// ---- caller-owned workspaces
+int64_t ttq_workspace_bytes(const ttq_qlinear* layer, int64_t m, int x_dtype) {
+  if (!layer) return TTQ_ERR_NULL;
+  if (!valid_dtype(x_dtype)) return TTQ_ERR_DTYPE;
+  const int rc = check_shape(layer->format, m, layer->n_out, layer->n_in, layer->bits, layer->codebook);
+  if (rc != TTQ_OK) return rc;
+  if (m == 0 || layer->n_out == 0) return 0;
+  const int64_t n_out = layer->n_out, n_in = layer->n_in;
+  const int64_t header = (int64_t)ttq::caller_workspace_header_bytes();
+  constexpr int64_t kChunkRows = 4096;          // rows whose bf16 / rotated copy is in the workspace at a time
+  const int64_t block_rows = m < kChunkRows ? m : kChunkRows;
+  if (layer->format == TTQ_EXL3)                // hand-off words; the rotated activations of the many-row form
+    return header + ((block_rows * n_in * 2 + 255) & ~(int64_t)255);
+  if (m < 5) return 0;                          // the decode kernels take no workspace
+  // a bf16 copy of fp16 / fp32 activations, then the partial sums of a launch split along K: the prefill GEMM's
+  // exact size for every row count it can be called with here, and the few-row kernel's bound (one 64 x 64 tile
+  // of sums per compute unit)
+  int64_t scratch = 0;
+  if (x_dtype != TTQ_BF16 && m >= 256) scratch += (block_rows * n_in * 2 + 255) & ~(int64_t)255;
+  int64_t partials = (int64_t)ttq::device_num_cus() * (16 * 4 * (16 * 4 + 1) * 4);
+  const int64_t rows[3] = {m, block_rows, m % kChunkRows};
+  for (int64_t r : rows) {
+    if (r <= 0) continue;
+    const int64_t p = (int64_t)ttq::gemm_pc_partials_bytes(r, n_out, n_in);
+    if (p > partials) partials = p;
+  }
+  return header + scratch + ((partials + 255) & ~(int64_t)255);
+}
+
+static int ws_check(void* ws, int64_t ws_bytes) {
+  if (ws_bytes < 0 || (ws_bytes > 0 && (!ws || !aligned16(ws)))) return TTQ_ERR_WORKSPACE;
+  return TTQ_OK;
+}
+// the status of a call that ran with a caller-owned workspace bound
+static int ws_status(int rc, const ttq::CallerWsScope& scope) { return scope.too_small() ? TTQ_ERR_WORKSPACE : rc; }
+
+int ttq_linear_forward_ws(const ttq_qlinear* layer, const void* x, int x_dtype, int64_t m, void* y, int y_dtype,
+                          void* ws, int64_t ws_bytes, void* stream) {
+  const int rc = ws_check(ws, ws_bytes);
+  if (rc != TTQ_OK) return rc;
+  ttq::CallerWsScope scope(ws, (size_t)ws_bytes);
+  return ws_status(ttq_linear_forward(layer, x, x_dtype, m, y, y_dtype, stream), scope);
+}
+
+int ttq_gemm_q4_k_ws(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m, int64_t n_out,
+                     int64_t n_in, void* ws, int64_t ws_bytes, void* stream) {
+  const int rc = ws_check(ws, ws_bytes);
+  if (rc != TTQ_OK) return rc;
+  ttq::CallerWsScope scope(ws, (size_t)ws_bytes);
+  return ws_status(gemm_block(TTQ_Q4_K, w, x_bf16, y_bf16, m, n_out, n_in, stream), scope);
+}
+int ttq_gemm_q6_k_ws(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m, int64_t n_out,
+                     int64_t n_in, void* ws, int64_t ws_bytes, void* stream) {
+  const int rc = ws_check(ws, ws_bytes);
+  if (rc != TTQ_OK) return rc;
+  ttq::CallerWsScope scope(ws, (size_t)ws_bytes);
+  return ws_status(gemm_block(TTQ_Q6_K, w, x_bf16, y_bf16, m, n_out, n_in, stream), scope);
+}
+int ttq_gemm_q8_0_ws(const void* w, const uint16_t* x_bf16, uint16_t* y_bf16, int64_t m, int64_t n_out,
+                     int64_t n_in, void* ws, int64_t ws_bytes, void* stream) {
+  const int rc = ws_check(ws, ws_bytes);
+  if (rc != TTQ_OK) return rc;
+  ttq::CallerWsScope scope(ws, (size_t)ws_bytes);
+  return ws_status(gemm_block(TTQ_Q8_0, w, x_bf16, y_bf16, m, n_out, n_in, stream), scope);
+}
+int ttq_gemm_exl3_ws(const uint16_t* trellis, const uint16_t* suh_f16, const uint16_t* svh_f16, const void* x,
+                     int x_dtype, float* y, int64_t m, int64_t n_out, int64_t n_in, int bits, int codebook, void* ws,
+                     int64_t ws_bytes, void* stream) {
+  const int rc = ws_check(ws, ws_bytes);
+  if (rc != TTQ_OK) return rc;
+  ttq::CallerWsScope scope(ws, (size_t)ws_bytes);
+  return ws_status(ttq_gemm_exl3(trellis, suh_f16, svh_f16, x, x_dtype, y, m, n_out, n_in, bits, codebook, stream), scope);
+}
+int ttq_gemv_exl3_ws(const uint16_t* trellis, const uint16_t* suh_f16, const uint16_t* svh_f16, const uint16_t* x_f16,
+                     float* y, int64_t m, int64_t n_out, int64_t n_in, int bits, int codebook, void* ws,
+                     int64_t ws_bytes, void* stream) {
+  const int rc = ws_check(ws, ws_bytes);
+  if (rc != TTQ_OK) return rc;
+  ttq::CallerWsScope scope(ws, (size_t)ws_bytes);
+  return ws_status(ttq_gemv_exl3(trellis, suh_f16, svh_f16, x_f16, y, m, n_out, n_in, bits, codebook, stream), scope);
+}
+
+int ttq_release_workspaces(void) { return hip_status(ttq::release_stream_workspaces()); }
+
+int ttq_debug_set_exl3_poll_limit(int limit) { return ttq::exl3_set_poll_limit(limit); }
 
 }  // extern "C"

@@ -345,6 +345,7 @@ hipError_t launch_gemv_exl3(const uint16_t* trellis, const uint16_t* suh, const 
   static const int two_launches = dev_knob("TTQ_EXL3_TWO_LAUNCHES", 0);
   if (!two_launches) {
     const Exl3Plan plan = exl3_mfma_plan(m, n_out, n_in);
+    if (route_probe(plan.slices > 1 ? kRouteExl3GemvSliced : kRouteExl3Gemv)) return hipSuccess;
     unsigned long long* accum = nullptr;
     if (plan.slices > 1) {
       e = exl3_workspace(s, &accum);
@@ -353,6 +354,7 @@ hipError_t launch_gemv_exl3(const uint16_t* trellis, const uint16_t* suh, const 
     return launch_gemv_exl3_mfma(plan, trellis, suh, svh, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, bits,
                                  cb, accum, s);
   }
+  if (route_probe(kRouteExl3GemvTwoLaunches)) return hipSuccess;
   if (y_dtype != kF32) return hipErrorInvalidValue;     // the two-kernel form rotates an fp32 buffer in place
   float* yf = static_cast<float*>(y);
   switch (bits) {

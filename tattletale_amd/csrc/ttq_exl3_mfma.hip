@@ -5,7 +5,7 @@
 // Work split.  A workgroup owns one Hadamard group of 128 output channels (8 tiles across) and one
 // slice of the reduction dimension; its 8 wavefronts take one 16-channel tile column each.  The
 // slices of a group hand their sums to the group's last slice through tagged words in a workspace (one
-// store and one load, no counters); the last slice adds them in a fixed order, rotates the 128 sums of
+// store and one load each); the last slice adds them in a fixed order, rotates the 128 sums of
 // each row and writes y.  With one slice there is no workspace traffic.
 //
 // Weights.  For one k-tile the 8 tiles of the group are contiguous in trellis[k_tile][n_tile][16*bits],
@@ -38,7 +38,7 @@ __global__ void __launch_bounds__(kXmThreads)
 gemv_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __restrict__ suh,
                       const uint16_t* __restrict__ svh, const XT* __restrict__ x, void* __restrict__ y, int y_dtype,
                       const void* __restrict__ bias, int bias_dtype, int m, int n_out, int n_in, int slice_tiles,
-                      unsigned long long* __restrict__ accum) {
+                      unsigned long long* __restrict__ accum, int poll_limit) {
   using G = XmGeom<BITS>;
   __shared__ uint32_t slab[G::kSlabDw];
   __shared__ __attribute__((aligned(16))) _Float16 xs[2 * kXmTok * kXmColStride];
@@ -57,6 +57,12 @@ gemv_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __re
 
   XmLane<BITS> ln;
   ln.init(lane);
+
+  // The tag of this launch's hand-off words: the workspace's generation count + 1 (read now, needed at the end).
+  // accum[0] holds the generation, accum[1] the number of groups that have finished, the words start at accum + 8.
+  uint32_t tag = 0;
+  if (nslices > 1)
+    tag = __hip_atomic_load(reinterpret_cast<const uint32_t*>(accum), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
 
   // ---- weights: global -> registers, one pass ahead
   const char* wbase = reinterpret_cast<const char*>(trellis) + (int64_t)grp * 8 * (32 * BITS);
@@ -206,12 +212,16 @@ gemv_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __re
   }
 
   // ---- the two terms of each row.  Then, in a sliced launch, every slice but the last hands its sums
-  // to the last one straight from the registers, through tagged 64-bit words (tag 1 in the high half,
-  // the float in the low half) written and read with agent-scope accesses, which are coherent across
-  // the chip without cache maintenance.  The last slice has the highest workgroup index of its group,
-  // so the others were dispatched before it and finish without it; it polls each word until the tag
-  // is there (a bounded number of times: rows it gave up on come out as NaN), adds everything in a
-  // fixed order, and leaves the words at zero for the next launch on the stream.
+  // to the last one straight from the registers, through tagged 64-bit words (the launch's tag in the high
+  // half, the float in the low half) written and read with agent-scope accesses, which are coherent across
+  // the chip without cache maintenance.  The last slice polls each word until this launch's tag is there
+  // (a bounded number of times: rows it gave up on come out as NaN) and adds everything in a fixed order.
+  // Nothing is cleared: the tag is the workspace's generation count + 1, and the group that finishes last
+  // advances the count, so the words of this launch -- also those of a slice that arrives after its group
+  // gave up on it -- can never pass for words of a later one.  The count lives in the workspace and not in
+  // a kernel argument because a captured graph replays its arguments.  What remains: a slice that has not
+  // even begun when its group gives up reads the advanced count and tags its words like the next launch
+  // will; that takes a wavefront dispatch held back for poll_limit polls (tens of milliseconds by default).
 #pragma unroll
   for (int r = 0; r < 4; r++) acc[r] += lane_xor<1>(acc[r], lane);
   const int tcol = wave & 7, kpart = wave >> 3;
@@ -219,13 +229,14 @@ gemv_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __re
   constexpr int kPartWords = kXmTok * 128;                        // words per (slice, k part)
   unsigned long long* words = nullptr;
   if (nslices > 1) {
-    words = accum + (((int64_t)blockIdx.z * gridDim.x + grp) * nslices) * (kXmKSplit * kPartWords);
+    words = accum + 8 + (((int64_t)blockIdx.z * gridDim.x + grp) * nslices) * (kXmKSplit * kPartWords);
     if (slice != nslices - 1) {
       if (owner) {
         unsigned long long* dst = words + ((int64_t)slice * kXmKSplit + kpart) * kPartWords + (col >> 1) * 128 + tcol * 16 + 4 * q;
 #pragma unroll
         for (int r = 0; r < 4; r++)
-          __hip_atomic_store(dst + r, (1ull << 32) | __float_as_uint(acc[r]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(dst + r, ((unsigned long long)tag << 32) | __float_as_uint(acc[r]), __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
       }
       return;
     }
@@ -240,7 +251,6 @@ gemv_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __re
     // then this workgroup's own sums
     float s = 0.f;
     bool late = false;
-    constexpr int kPollLimit = 1 << 16;
     const int nparts = (nslices - 1) * kXmKSplit;
     for (int p0 = 0; p0 < nparts; p0 += 8) {
       unsigned long long w[8];
@@ -252,12 +262,11 @@ gemv_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __re
       for (int i = 0; i < 8; i++) {
         if (p0 + i < nparts) {
           unsigned long long* wp = words + (int64_t)(p0 + i) * kPartWords + e;
-          for (int polls = 0; (w[i] >> 32) != 1 && polls < kPollLimit; polls++) {
+          for (int polls = 0; (uint32_t)(w[i] >> 32) != tag && polls < poll_limit; polls++) {
             __builtin_amdgcn_s_sleep(2);
             w[i] = __hip_atomic_load(wp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
-          late |= (w[i] >> 32) != 1;
-          __hip_atomic_store(wp, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          late |= (uint32_t)(w[i] >> 32) != tag;
           s += __uint_as_float((uint32_t)w[i]);
         }
       }
@@ -267,6 +276,12 @@ gemv_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __re
     for (int k = 1; k < kXmKSplit; k++) s += yq[(k - 1) * kPartWords + e];
     yp[e] = late ? __uint_as_float(0x7FC00000u) : s;
   }
+  // Thread 0 has now seen (or given up on) a word of every other slice of its group, so each of them has read
+  // the generation count.  It counts its group in here and looks at the answer after the output phase: the group
+  // that is counted last advances the generation.
+  uint32_t counted = 0;
+  if (nslices > 1 && tid == 0)
+    counted = __hip_atomic_fetch_add(reinterpret_cast<uint32_t*>(accum) + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
 
   // ---- output side: rotate the 128 sums of each row, svh, bias
@@ -288,6 +303,11 @@ gemv_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __re
     }
     xm_store4(y, y_dtype, (int64_t)(t0 + hw) * n_out + n, o);
   }
+  if (nslices > 1 && tid == 0 && counted == gridDim.x * gridDim.z - 1) {
+    uint32_t* ctl = reinterpret_cast<uint32_t*>(accum);
+    __hip_atomic_store(ctl + 2, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(ctl, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
 }
 
 // ------------------------------------------------------------------------------ launch
@@ -305,9 +325,14 @@ Exl3Plan exl3_mfma_plan(int64_t m, int64_t n_out, int64_t n_in) {
   tiles = (tiles + 7) / 8 * 8;
   p.slice_tiles = tiles;
   p.slices = (kt_n + tiles - 1) / tiles;
-  p.accum_words = p.slices > 1 ? units * p.slices * kXmKSplit * kXmTok * 128 : 0;
+  p.accum_words = p.slices > 1 ? 8 + units * p.slices * kXmKSplit * kXmTok * 128 : 0;   // 8 control words in front
   return p;
 }
+
+// How often the last slice of a group looks at a word that has not arrived before it gives the row up (NaN).
+// A host-side setting so that the give-up path can be exercised without any kernel misbehaving.
+static std::atomic<int> g_exl3_poll_limit{1 << 16};
+int exl3_set_poll_limit(int limit) { return g_exl3_poll_limit.exchange(limit < 0 ? 0 : limit); }
 
 template <int BITS, int CB, typename XT>
 static hipError_t xm_launch(const Exl3Plan& p, const uint16_t* trellis, const uint16_t* suh, const uint16_t* svh,
@@ -316,7 +341,7 @@ static hipError_t xm_launch(const Exl3Plan& p, const uint16_t* trellis, const ui
   const dim3 grid((unsigned)p.groups, (unsigned)p.slices, (unsigned)p.row_groups), block(kXmThreads);
   hipLaunchKernelGGL((gemv_exl3_mfma_kernel<BITS, CB, XT>), grid, block, 0, s, trellis, suh, svh,
                      static_cast<const XT*>(x), y, y_dtype, bias, bias_dtype, (int)m, (int)n_out, (int)n_in, p.slice_tiles,
-                     accum);
+                     accum, g_exl3_poll_limit.load(std::memory_order_relaxed));
   return hipGetLastError();
 }
 
@@ -360,22 +385,28 @@ hipError_t launch_gemv_exl3_mfma(const Exl3Plan& p, const uint16_t* trellis, con
 }
 
 // ------------------------------------------------------------------------------ workspace
-// Sliced launches exchange their sums through 64-bit words that are zero before and after every launch.
-// The library keeps one array of them per (device, stream): launches on one stream run in order and can share it; launches
-// on different streams may overlap and get their own.  Sized for the largest plan: launches are sliced
-// only while there are fewer (group, row group) units than compute units.
+// Sliced launches exchange their sums through tagged 64-bit words behind eight control words (generation count,
+// groups finished), all zero before the first launch.  A caller-owned workspace (ttq_workspace.hip) supplies them
+// when one is bound; otherwise the library keeps one array per (device, stream): launches on one stream run in
+// order and can share it, launches on different streams may overlap and get their own.  Sized for the largest
+// plan: launches are sliced only while there are fewer (group, row group) units than compute units.
 namespace {
 std::mutex g_ws_mutex;
 std::unordered_map<uint64_t, unsigned long long*> g_ws;
 }  // namespace
 
 // units * slices <= compute units
-int64_t exl3_workspace_words() { return (int64_t)device_num_cus() * kXmKSplit * kXmTok * 128; }
+int64_t exl3_workspace_words() { return 8 + (int64_t)device_num_cus() * kXmKSplit * kXmTok * 128; }
 
 hipError_t exl3_workspace(hipStream_t s, unsigned long long** accum) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
+  void* bound = nullptr;
+  if (caller_workspace_region(kCwExl3Words, (size_t)exl3_workspace_words() * sizeof(unsigned long long), &bound, &e)) {
+    *accum = static_cast<unsigned long long*>(bound);
+    return e;
+  }
   const uint64_t key = ((uint64_t)(uint32_t)dev << 48) ^ (uint64_t)reinterpret_cast<uintptr_t>(s);
   std::lock_guard<std::mutex> lock(g_ws_mutex);
   auto it = g_ws.find(key);
@@ -384,7 +415,7 @@ hipError_t exl3_workspace(hipStream_t s, unsigned long long** accum) {
     void* p = nullptr;
     e = hipMalloc(&p, bytes);
     if (e != hipSuccess) return e;
-    e = hipMemset(p, 0, bytes);
+    e = hipMemsetAsync(p, 0, bytes, s);     // ordered before the launches that use it: they are all on this stream
     if (e != hipSuccess) {
       (void)hipFree(p);
       return e;
@@ -398,10 +429,10 @@ hipError_t exl3_workspace(hipStream_t s, unsigned long long** accum) {
 // ------------------------------------------------------------------------------ resident workspace
 // The same words as a file-scope array in device memory, for the entry point that must not allocate:
 // every GPU the library runs on holds its own copy from the moment the code object is loaded there
-// until the process ends, zero-initialised, and every launch leaves the words it used at zero again.
+// until the process ends, zero-initialised; the launches only ever advance its generation count.
 // The array's name is only a handle in host code; the address on a device comes from
 // hipGetSymbolAddress, asked once per device with that device current.
-constexpr int64_t kXmResidentWords = (int64_t)256 * kXmKSplit * kXmTok * 128;      // 4 MiB
+constexpr int64_t kXmResidentWords = 8 + (int64_t)256 * kXmKSplit * kXmTok * 128;      // 4 MiB
 static __device__ __align__(256) unsigned long long scratch[kXmResidentWords];
 
 namespace {
@@ -426,6 +457,18 @@ hipError_t exl3_resident_workspace(unsigned long long** accum) {
   }
   *accum = g_resident[dev];
   return hipSuccess;
+}
+
+// Frees the library-owned arrays (ttq_release_workspaces: nothing that uses them may be in flight or captured).
+hipError_t exl3_release_workspaces() {
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  hipError_t first = hipSuccess;
+  for (auto& kv : g_ws) {
+    const hipError_t e = hipFree(kv.second);
+    if (e != hipSuccess && first == hipSuccess) first = e;
+  }
+  g_ws.clear();
+  return first;
 }
 
 }  // namespace ttq

@@ -264,6 +264,7 @@ hipError_t launch_gemm_exl3(const uint16_t* trellis, const uint16_t* suh, const 
                             int x_dtype, void* y, int y_dtype, const void* bias, int bias_dtype, int64_t m,
                             int64_t n_out, int64_t n_in, int bits, int cb, hipStream_t s) {
   if (m == 0 || n_out == 0) return hipSuccess;
+  if (route_probe(kRouteExl3Gemm)) return hipSuccess;
   const int64_t block_rows = m < kXpMaxRows ? m : kXpMaxRows;
   void* ws = nullptr;
   hipError_t e = stream_workspace(kWsExl3Rotated, s, (size_t)block_rows * n_in * sizeof(uint16_t), &ws);

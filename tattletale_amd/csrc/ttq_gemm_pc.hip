@@ -76,6 +76,15 @@ static PcChoice pc_choose(int64_t m, int64_t n_out, int64_t n_in, bool fuse) {
   return best;
 }
 
+size_t gemm_pc_partials_bytes(int64_t m, int64_t n_out, int64_t n_in) {
+  if (m <= 0 || n_out <= 0 || n_in < 256) return 0;
+  const PcChoice c = pc_choose(m, n_out, n_in, false);
+  if (c.splits <= 1) return 0;
+  const PcTile& t = kPcTiles[c.tile];
+  const int64_t nt = (n_out + t.nj * 16 - 1) / (t.nj * 16), mt = (m + pc_bm(t.mb) - 1) / pc_bm(t.mb);
+  return (size_t)(nt * mt * 4) * (size_t)c.splits * (size_t)(t.mb * t.nj * 1024);
+}
+
 // Rough time of the GEMM for this shape (microseconds), for callers that can also run the
 // operator as a few GEMV passes.  The Q6_K and Q8_0 producers are slower than the Q4_K one.
 float gemm_pc_estimate_us(int format, int64_t m, int64_t n_out, int64_t n_in) {
@@ -112,6 +121,7 @@ hipError_t launch_gemm_pc(int format, const void* w, const uint16_t* x_bf16, voi
                           hipStream_t s) {
   if (m == 0 || n_out == 0) return hipSuccess;
   if (y_dtype != kBF16 && y_dtype != kF32 && y_dtype != kF16) return hipErrorInvalidValue;
+  if (route_probe(pc_choose(m, n_out, n_in, false).splits > 1 ? kRouteGemmPcSplitK : kRouteGemmPc)) return hipSuccess;
   const uint8_t* wb = static_cast<const uint8_t*>(w);
   switch (format) {
     case kQ4_K: return launch_pc_fmt<kQ4_K, false>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);

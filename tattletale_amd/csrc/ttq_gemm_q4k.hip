@@ -438,9 +438,10 @@ hipError_t launch_gemm(int format, const void* w, const uint16_t* x_bf16, void* 
                        int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
   if (m == 0 || n_out == 0) return hipSuccess;
   if (prefer_skinny(format, m, n_out, n_in))
-    return launch_gemm_skinny(format, w, x_bf16, kBF16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    TTQ_ROUTE(kRouteGemmSkinny, launch_gemm_skinny(format, w, x_bf16, kBF16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
   if (prefer_skinny_chunks(format, m, n_out, n_in))
-    return launch_gemm_skinny_chunked(format, w, x_bf16, kBF16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    TTQ_ROUTE(kRouteGemmSkinnyChunked,
+              launch_gemm_skinny_chunked(format, w, x_bf16, kBF16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
   if (format != kQ4_K) {
     if (!gemm_pc_supported(format, m, n_out, n_in, 112)) return hipErrorInvalidValue;
     return launch_gemm_pc(format, w, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
@@ -455,8 +456,8 @@ hipError_t launch_gemm(int format, const void* w, const uint16_t* x_bf16, void* 
   if (gemm_pc_supported(kQ4_K, m, n_out, n_in, use112 ? 112 : 128))
     return launch_gemm_pc(kQ4_K, w, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   const uint8_t* wb = static_cast<const uint8_t*>(w);
-  return use112 ? launch_nj<7>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s)
-                : launch_nj<8>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  TTQ_ROUTE(kRouteGemmQ4kTiles, (use112 ? launch_nj<7>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s)
+                                        : launch_nj<8>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s)));
 }
 
 }  // namespace ttq

@@ -352,26 +352,26 @@ hipError_t launch_gemv(int format, const void* w, const void* x, int x_dtype, vo
   // a few rows at once: four per pass for up to four rows and for rows too long for the 8- and
   // 16-token tables, else eight or sixteen per pass
   if (gemv_q4k_stream4_supported(format, x_dtype, m, n_out, n_in))
-    return launch_gemv_q4k_stream4(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    TTQ_ROUTE(kRouteGemvQ4kStream4, launch_gemv_q4k_stream4(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
   static const int batch4_max = dev_knob("TTQ_GEMV_BATCH4_MAX_ROWS", 4);
   const bool b4 = gemv_q4k_batch4_supported(format, x_dtype, m, n_out, n_in);
   if (b4 && m <= batch4_max)
-    return launch_gemv_q4k_batch4(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    TTQ_ROUTE(kRouteGemvQ4kBatch4, launch_gemv_q4k_batch4(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
   if (gemv_q4k_batch_supported(format, x_dtype, m, n_out, n_in))
-    return launch_gemv_q4k_batch(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-  if (b4) return launch_gemv_q4k_batch4(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    TTQ_ROUTE(kRouteGemvQ4kBatch, launch_gemv_q4k_batch(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
+  if (b4) TTQ_ROUTE(kRouteGemvQ4kBatch4, launch_gemv_q4k_batch4(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
   if (gemv_q6k_stream4_supported(format, x_dtype, m, n_out, n_in))
-    return launch_gemv_q6k_stream4(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    TTQ_ROUTE(kRouteGemvQ6kStream4, launch_gemv_q6k_stream4(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
   if (gemv_dot2_multi_supported(format, x_dtype, m, n_in))
-    return launch_gemv_dot2_multi(format, w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    TTQ_ROUTE(kRouteGemvDot2Multi, launch_gemv_dot2_multi(format, w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
   if (gemv_q4k_stream_supported(format, x_dtype, n_out, n_in))
-    return launch_gemv_q4k_stream(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    TTQ_ROUTE(kRouteGemvQ4kStream, launch_gemv_q4k_stream(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
   if (gemv_q4k_slice_supported(format, x_dtype, n_out, n_in))
-    return launch_gemv_q4k_slice(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    TTQ_ROUTE(kRouteGemvQ4kSlice, launch_gemv_q4k_slice(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
   if (gemv_q6k_stream_supported(format, x_dtype, n_out, n_in))
-    return launch_gemv_q6k_stream(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    TTQ_ROUTE(kRouteGemvQ6kStream, launch_gemv_q6k_stream(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
   if (gemv_mfma_supported(format, x_dtype, n_out, n_in))
-    return launch_gemv_mfma(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    TTQ_ROUTE(kRouteGemvQ4kMfma, launch_gemv_mfma(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
   // Q8_0 with few weights: the fp32 kernel (a wavefront per row, a row's activations in registers) has the shortest
   // prologue; it re-reads the weights per activation row, so the more rows, the smaller the matrix it wins on.
   // Measured against the matrix-core kernels: 1024x4096 3.9 / 4.8 / 6.3 us for 1 / 2 / 4 rows against 5.3 / 6.5 /
@@ -381,20 +381,20 @@ hipError_t launch_gemv(int format, const void* w, const void* x, int x_dtype, vo
   if (format == kQ8_0 && m <= 4 && n_out <= 2048) {
     const float mb = (float)(n_out * (n_in / 32) * 34) * 1e-6f;
     const float limit = n_in <= 4096 ? (m == 1 ? 12.f : (m == 2 ? 8.5f : 6.f)) : (m <= 2 ? 16.f : 0.f);
-    if (mb <= limit) return launch_generic_xy<FmtQ8_0>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    if (mb <= limit) TTQ_ROUTE(kRouteGemvGeneric, launch_generic_xy<FmtQ8_0>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
   }
   if (m == 1 && gemv_q8_stream_supported(format, x_dtype, n_out, n_in))
-    return launch_gemv_q8_stream(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    TTQ_ROUTE(kRouteGemvQ8Stream, launch_gemv_q8_stream(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
   if (gemv_q8_win_supported(format, n_out, n_in))
-    return launch_gemv_q8_win(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    TTQ_ROUTE(kRouteGemvQ8Win, launch_gemv_q8_win(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
   if (gemv_q8_mfma_supported(format, n_out, n_in))
-    return launch_gemv_q8_mfma(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    TTQ_ROUTE(kRouteGemvQ8Mfma, launch_gemv_q8_mfma(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
   if (gemv_dot2_supported(format, x_dtype, n_in))
-    return launch_gemv_dot2(format, w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    TTQ_ROUTE(kRouteGemvDot2, launch_gemv_dot2(format, w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
   switch (format) {
-    case kQ8_0: return launch_generic_xy<FmtQ8_0>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-    case kQ4_K: return launch_generic_xy<FmtQ4_K>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-    case kQ6_K: return launch_generic_xy<FmtQ6_K>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kQ8_0: TTQ_ROUTE(kRouteGemvGeneric, launch_generic_xy<FmtQ8_0>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
+    case kQ4_K: TTQ_ROUTE(kRouteGemvGeneric, launch_generic_xy<FmtQ4_K>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
+    case kQ6_K: TTQ_ROUTE(kRouteGemvGeneric, launch_generic_xy<FmtQ6_K>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
     default: return hipErrorInvalidValue;
   }
 }

@@ -12,6 +12,50 @@
 
 namespace ttq {
 
+// Which kernel family a dispatcher picks (values as ttq_route_id in ttq.h).  ttq_route runs the dispatch code of
+// ttq_linear_forward itself with a probe bound to the calling thread: every dispatcher reports its choice through
+// route_probe and, when a probe is bound, returns instead of launching.
+enum : int {
+  kRouteNone = 0,
+  kRouteGemvQ4kStream = 1,
+  kRouteGemvQ4kStream4 = 2,
+  kRouteGemvQ4kSlice = 3,
+  kRouteGemvQ4kBatch4 = 4,
+  kRouteGemvQ4kBatch = 5,
+  kRouteGemvQ4kMfma = 6,
+  kRouteGemvQ6kStream = 7,
+  kRouteGemvQ6kStream4 = 8,
+  kRouteGemvQ8Stream = 9,
+  kRouteGemvQ8Win = 10,
+  kRouteGemvQ8Mfma = 11,
+  kRouteGemvDot2 = 12,
+  kRouteGemvDot2Multi = 13,
+  kRouteGemvGeneric = 14,
+  kRouteGemmPc = 20,
+  kRouteGemmPcSplitK = 21,
+  kRouteGemmSkinny = 22,
+  kRouteGemmSkinnyChunked = 23,
+  kRouteGemmQ4kTiles = 24,
+  kRouteGemmPcBf16Copy = 25,
+  kRouteExl3Gemv = 30,
+  kRouteExl3GemvSliced = 31,
+  kRouteExl3Gemm = 32,
+  kRouteExl3GemvTwoLaunches = 33,
+};
+struct RouteProbe { int route; };
+extern thread_local RouteProbe* t_route_probe;
+inline bool route_probe(int id) {
+  RouteProbe* p = t_route_probe;
+  if (!p) return false;
+  if (p->route == 0) p->route = id;
+  return true;
+}
+#define TTQ_ROUTE(id, call)                      \
+  do {                                           \
+    if (::ttq::route_probe(id)) return hipSuccess; \
+    return call;                                 \
+  } while (0)
+
 // Developer A/B switches.  They are read from the environment only in builds made with
 // -DTTQ_DEV_KNOBS; the product build (tattletale_amd/build.py) leaves that off, so what the library
 // does never depends on the process environment.
@@ -219,6 +263,31 @@ hipError_t launch_hadamard128(float* v, const uint16_t* pre, const uint16_t* pos
 constexpr int kWsExl3Rotated = 0, kWsBf16Activations = 1, kWsGemmPartials = 2, kWsGemmCounters = 3;
 // zeroed: a newly allocated buffer is cleared (on the stream) before it is handed out
 hipError_t stream_workspace(int slot, hipStream_t s, size_t bytes, void** out, bool zeroed = false);
+// Frees every library-owned workspace (nothing that uses one may be in flight or captured).
+hipError_t release_stream_workspaces();
+hipError_t exl3_release_workspaces();
+// A caller-owned workspace, bound to the calling thread while the object lives: stream_workspace and
+// exl3_workspace then serve every request from it and allocate nothing.
+constexpr int kCwCounters = 0, kCwExl3Words = 1, kCwScratch = 2;
+class CallerWsScope {
+ public:
+  CallerWsScope(void* ws, size_t bytes);
+  ~CallerWsScope();
+  CallerWsScope(const CallerWsScope&) = delete;
+  CallerWsScope& operator=(const CallerWsScope&) = delete;
+  bool too_small() const;      // some request did not fit (the call then failed with hipErrorOutOfMemory)
+ private:
+  alignas(8) unsigned char state_[40];
+};
+// false: no caller workspace is bound.  true: *out / *err say where the region lies or that it does not fit.
+bool caller_workspace_region(int region, size_t bytes, void** out, hipError_t* err);
+// bytes in front of the scratch part of a caller-owned workspace (arrival counters, trellis hand-off words)
+size_t caller_workspace_header_bytes();
+int64_t exl3_workspace_words();
+// exact size of the partial sums a split-K launch of the prefill GEMM takes for this shape (0: not split)
+size_t gemm_pc_partials_bytes(int64_t m, int64_t n_out, int64_t n_in);
+// how often the trellis GEMV's last slice polls a missing word before it gives the row up; returns the old value
+int exl3_set_poll_limit(int limit);
 // n fp16 or fp32 values (n a multiple of 8) rounded to bf16
 hipError_t launch_to_bf16(const void* x, int x_dtype, uint16_t* out, int64_t n, hipStream_t s);
 

@@ -18,7 +18,9 @@ type
   TtqDtype* {.size: sizeof(cint).} = enum
     kTtqF32 = 0, kTtqF16 = 1, kTtqBF16 = 2
   TtqPrecision* {.size: sizeof(cint).} = enum
-    kTtqAuto = 0, kTtqF32Scales = 1    ## kTtqF32Scales: decode kernels (fp32 scales) for every batch size
+    kTtqAuto = 0, kTtqF32Scales = 1, kTtqBf16Ok = 2
+      ## kTtqF32Scales: decode kernels (fp32 scales) for every batch size
+      ## kTtqBf16Ok: fp16 / fp32 activations may be rounded to bf16 for the matrix-core GEMM
   TtqQLinear* {.bycopy.} = object      ## struct ttq_qlinear
     format*, bits*, codebook*, bias_dtype*: int32
     precision*, reserved*: int32       ## ttq_precision, 0
@@ -32,6 +34,12 @@ proc last_hip_error*(): cint {.ttq.}
 proc packed_nbytes*(format: cint, n_out, n_in: int64, bits: cint): int64 {.ttq.}
 proc linear_forward*(layer: ptr TtqQLinear, x: pointer, x_dtype: cint, m: int64,
                      y: pointer, y_dtype: cint, stream: pointer): cint {.ttq.}
+proc workspace_bytes*(layer: ptr TtqQLinear, m: int64, x_dtype: cint): int64 {.ttq.}
+proc linear_forward_ws*(layer: ptr TtqQLinear, x: pointer, x_dtype: cint, m: int64,
+                        y: pointer, y_dtype: cint, ws: pointer, ws_bytes: int64, stream: pointer): cint {.ttq.}
+proc release_workspaces*(): cint {.ttq.}
+proc route*(layer: ptr TtqQLinear, m: int64, x_dtype, y_dtype: cint): cint {.ttq.}
+proc route_name*(route: cint): cstring {.ttq.}
 proc gemv_q8_0*(w, x: pointer, x_dtype: cint, y: ptr cfloat, m, n_out, n_in: int64, stream: pointer): cint {.ttq.}
 proc gemv_q4_k*(w, x: pointer, x_dtype: cint, y: ptr cfloat, m, n_out, n_in: int64, stream: pointer): cint {.ttq.}
 proc gemv_q6_k*(w, x: pointer, x_dtype: cint, y: ptr cfloat, m, n_out, n_in: int64, stream: pointer): cint {.ttq.}
@@ -41,6 +49,17 @@ proc gemv_exl3_noalloc*(trellis, suh, svh, x: ptr uint16, y: ptr cfloat, m, n_ou
                         bits, codebook: cint, stream: pointer): cint {.ttq.}
 proc gemm_exl3*(trellis, suh, svh: ptr uint16, x: pointer, x_dtype: cint, y: ptr cfloat, m, n_out, n_in: int64,
                 bits, codebook: cint, stream: pointer): cint {.ttq.}
+proc gemv_exl3_ws*(trellis, suh, svh, x: ptr uint16, y: ptr cfloat, m, n_out, n_in: int64,
+                   bits, codebook: cint, ws: pointer, ws_bytes: int64, stream: pointer): cint {.ttq.}
+proc gemm_exl3_ws*(trellis, suh, svh: ptr uint16, x: pointer, x_dtype: cint, y: ptr cfloat, m, n_out, n_in: int64,
+                   bits, codebook: cint, ws: pointer, ws_bytes: int64, stream: pointer): cint {.ttq.}
+proc debug_set_exl3_poll_limit*(limit: cint): cint {.ttq.}
+proc gemm_q4_k_ws*(w: pointer, x, y: ptr uint16, m, n_out, n_in: int64, ws: pointer, ws_bytes: int64,
+                   stream: pointer): cint {.ttq.}
+proc gemm_q6_k_ws*(w: pointer, x, y: ptr uint16, m, n_out, n_in: int64, ws: pointer, ws_bytes: int64,
+                   stream: pointer): cint {.ttq.}
+proc gemm_q8_0_ws*(w: pointer, x, y: ptr uint16, m, n_out, n_in: int64, ws: pointer, ws_bytes: int64,
+                   stream: pointer): cint {.ttq.}
 proc gemm_q4_k*(w: pointer, x, y: ptr uint16, m, n_out, n_in: int64, stream: pointer): cint {.ttq.}
 proc gemm_q6_k*(w: pointer, x, y: ptr uint16, m, n_out, n_in: int64, stream: pointer): cint {.ttq.}
 proc gemm_q8_0*(w: pointer, x, y: ptr uint16, m, n_out, n_in: int64, stream: pointer): cint {.ttq.}
@@ -105,13 +124,8 @@ func init*(_: type QuantLinear, qweight: TorchTensor, format: QuantFormat,
               codebook: codebook, in_features: in_features, out_features: out_features,
               precision: precision)
 
-proc forward*(self: QuantLinear, x: TorchTensor): TorchTensor =
-  ## x: (..., in_features) -> (..., out_features); launches on torch's current stream.
-  var shape = x.sizes().asNimView().toSeq()      # (..., in) -> (..., out)
-  shape[^1] = self.out_features
-  let m = x.numel() div self.in_features
-  result = F.empty(shape, x.options())
-  var desc = TtqQLinear(
+func descriptor(self: QuantLinear): TtqQLinear =
+  TtqQLinear(
     format: self.format.int32, bits: self.bits.int32, codebook: self.codebook.int32,
     bias_dtype: (if self.bias.isSome: ttqDtype(self.bias.get().scalarType()).int32 else: 0),
     precision: self.precision.int32, reserved: 0,
@@ -120,8 +134,31 @@ proc forward*(self: QuantLinear, x: TorchTensor): TorchTensor =
     suh: (if self.suh.isSome: self.suh.get().data_ptr(byte) else: nil),
     svh: (if self.svh.isSome: self.svh.get().data_ptr(byte) else: nil),
     bias: (if self.bias.isSome: self.bias.get().data_ptr(byte) else: nil))
-  let rc = linear_forward(addr desc, x.data_ptr(byte), ttqDtype(x.scalarType()), m,
-                          result.data_ptr(byte), ttqDtype(x.scalarType()), currentStream())
+
+proc workspaceBytes*(self: QuantLinear, m: int, dtype: ScalarKind): int64 =
+  ## What forward(x, workspace) needs for m rows: make it with F.zeros (cleared once, then reusable).
+  var desc = self.descriptor()
+  result = workspace_bytes(addr desc, m, ttqDtype(dtype))
+  if result < 0:
+    raise newException(QuantLinearError, "ttq_workspace_bytes: " & $strerror(result.cint))
+
+proc forward*(self: QuantLinear, x: TorchTensor, workspace = none(TorchTensor)): TorchTensor =
+  ## x: (..., in_features) -> (..., out_features); launches on torch's current stream.  With a workspace
+  ## (a kUint8 tensor from F.zeros of at least workspaceBytes, torch_tensors.nim:280-289) the library
+  ## allocates nothing and the call can be captured into a graph the first time it runs.
+  var shape = x.sizes().asNimView().toSeq()      # (..., in) -> (..., out)
+  shape[^1] = self.out_features
+  let m = x.numel() div self.in_features
+  result = F.empty(shape, x.options())
+  var desc = self.descriptor()
+  let rc =
+    if workspace.isSome:
+      linear_forward_ws(addr desc, x.data_ptr(byte), ttqDtype(x.scalarType()), m, result.data_ptr(byte),
+                        ttqDtype(x.scalarType()), workspace.get().data_ptr(byte), workspace.get().nbytes.int64,
+                        currentStream())
+    else:
+      linear_forward(addr desc, x.data_ptr(byte), ttqDtype(x.scalarType()), m,
+                     result.data_ptr(byte), ttqDtype(x.scalarType()), currentStream())
   if rc != 0:
     raise newException(QuantLinearError, "ttq_linear_forward: " & $strerror(rc))
 

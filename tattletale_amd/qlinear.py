@@ -69,7 +69,9 @@ class QuantLinear:
     svh: Optional[torch.Tensor] = None    # EXL3: (out_features,) float16
     bits: int = 0
     codebook: int = _lib.CB_MCG
-    precision: int = _lib.PRECISION_AUTO  # PRECISION_F32_SCALES keeps the decode kernels for every batch
+    # PRECISION_F32_SCALES keeps the decode kernels for every batch; PRECISION_BF16_OK lets fp16 / fp32
+    # activations be rounded to bf16 for the matrix-core GEMM
+    precision: int = _lib.PRECISION_AUTO
 
     @classmethod
     def init(cls, qweight: torch.Tensor, format: int, in_features: int, out_features: int,
@@ -105,11 +107,31 @@ class QuantLinear:
             n_out=self.out_features, n_in=self.in_features,
             qweight=_ptr(self.qweight), suh=_ptr(self.suh), svh=_ptr(self.svh), bias=_ptr(self.bias))
 
-    def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    def workspace_bytes(self, m: int, x_dtype: torch.dtype) -> int:
+        """Bytes of caller-owned workspace ``forward(..., workspace=...)`` needs for ``m`` rows
+        (``ttq_workspace_bytes``); make it with ``torch.zeros`` -- it must be clear before its first use."""
+        st = self._struct()
+        n = _lib.lib().ttq_workspace_bytes(C.byref(st), m, _code(x_dtype))
+        if n < 0:
+            raise TtqError(int(n), "ttq_workspace_bytes")
+        return int(n)
+
+    def route(self, m: int, x_dtype: torch.dtype, out_dtype: Optional[torch.dtype] = None) -> str:
+        """Name of the kernel family ``forward`` launches for ``m`` rows of ``x_dtype`` (``ttq_route``)."""
+        st = self._struct()
+        r = _lib.lib().ttq_route(C.byref(st), m, _code(x_dtype), _code(out_dtype or x_dtype))
+        if r < 0:
+            raise TtqError(int(r), "ttq_route")
+        return _lib.lib().ttq_route_name(r).decode()
+
+    def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+                workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
         """x (..., in_features) -> (..., out_features)  (linear.nim:45-57).
 
         ``out_dtype`` defaults to ``x.dtype`` (what ``F.linear`` returns); pass
-        ``torch.float32`` for fp32 logits from 16-bit activations."""
+        ``torch.float32`` for fp32 logits from 16-bit activations.  With ``workspace`` (a zero-filled
+        uint8 tensor of at least ``workspace_bytes`` bytes) the call allocates nothing inside the
+        library (``ttq_linear_forward_ws``)."""
         if x.shape[-1] != self.in_features:
             raise TtqError(_lib.ERR_SHAPE, "QuantLinear.forward: last dim %d != in_features %d"
                            % (x.shape[-1], self.in_features))
@@ -119,8 +141,14 @@ class QuantLinear:
         y = torch.empty(x.shape[:-1] + (self.out_features,), dtype=out_dtype, device=dev)
         st = self._struct()
         with torch.cuda.device(dev):
-            check(_lib.lib().ttq_linear_forward(C.byref(st), x.data_ptr(), _code(x.dtype), m, y.data_ptr(),
-                                                _code(out_dtype), _stream(dev)), "ttq_linear_forward")
+            if workspace is not None:
+                _require_device(self.qweight, workspace)
+                check(_lib.lib().ttq_linear_forward_ws(C.byref(st), x.data_ptr(), _code(x.dtype), m, y.data_ptr(),
+                                                       _code(out_dtype), workspace.data_ptr(), _nbytes(workspace),
+                                                       _stream(dev)), "ttq_linear_forward_ws")
+            else:
+                check(_lib.lib().ttq_linear_forward(C.byref(st), x.data_ptr(), _code(x.dtype), m, y.data_ptr(),
+                                                    _code(out_dtype), _stream(dev)), "ttq_linear_forward")
         return y
 
     __call__ = forward

@@ -30,9 +30,9 @@ def test_every_declared_symbol_is_exported_and_bound():
 
 def test_version_and_strerror():
     L = _lib.lib()
-    assert L.ttq_version() == 110
+    assert L.ttq_version() == 120
     assert L.ttq_strerror(0) == b"ok"
-    for code in range(-8, 0):
+    for code in range(-9, 0):
         assert len(L.ttq_strerror(code)) > 3
     assert L.ttq_strerror(-99) == b"unknown status"
 
@@ -197,3 +197,22 @@ def test_quantlinear_has_no_cpu_path():
     from tattletale_amd import QuantLinear, TtqError
     with pytest.raises(TtqError):
         QuantLinear.init(torch.zeros(144, dtype=torch.uint8), _lib.Q4_K, 256, 1)
+
+
+def test_row_counts_beyond_a_grid_dimension_are_refused_where_the_library_does_not_slice_them():
+    """Kernels that put activation rows on gridDim.y / gridDim.z (65535 at most) and are not called in slices
+    return a status instead of a failed launch."""
+    L = _lib.lib()
+    buf = np.zeros(1 << 12, np.uint8)
+    p = buf.ctypes.data
+    p += (-p) % 16
+    assert L.ttq_rmsnorm(p, None, p, 1e-6, _lib.BF16, None, p, 65536, 256, None) == _lib.ERR_UNSUPPORTED
+    assert L.ttq_gemv_exl3(p, p, p, p, p, 8 * 65535 + 1, 128, 128, 3, _lib.CB_MCG, None) == _lib.ERR_UNSUPPORTED
+    st = QLinearStruct(format=_lib.EXL3, n_out=128, n_in=128, bits=3, codebook=_lib.CB_MCG, qweight=p, suh=p, svh=p,
+                       precision=_lib.PRECISION_F32_SCALES)
+    assert L.ttq_linear_forward(C.byref(st), p, _lib.F16, 8 * 65535 + 1, p, _lib.F32, None) == _lib.ERR_UNSUPPORTED
+    # shapes outside the streamed fused kernels (n_in = 512) fall back to one row per workgroup on gridDim.y
+    assert L.ttq_gemv_q4_k_silu_mul(p, p, _lib.BF16, p, _lib.BF16, 65536, 64, 512, None) in (
+        _lib.ERR_UNSUPPORTED,)
+    assert L.ttq_gemv_q4_k_rmsnorm(p, p, None, p, 1e-6, _lib.BF16, None, None, p, _lib.F32, 65536, 64, 512, 0,
+                                   None) == _lib.ERR_UNSUPPORTED

@@ -398,14 +398,16 @@ def test_forward_fp16_unit_vectors_give_fp16_weights_exactly(fmt):
 @pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
 @pytest.mark.parametrize("xk", ["f16", "f32"])
 @pytest.mark.parametrize("m,n_out,n_in", [(256, 1048, 1024), (600, 4096, 512)])
-def test_forward_fp16_fp32_activations_many_rows_take_the_bf16_gemm(fmt, xk, m, n_out, n_in):
-    """From 256 rows on, fp16 and fp32 activations are rounded to bf16 into the library's workspace and run
-    the matrix-core GEMM (2e-2 class: weights and activations rounded to bf16 once); every output type."""
+def test_forward_fp16_fp32_activations_many_rows_take_the_bf16_gemm_only_when_allowed(fmt, xk, m, n_out, n_in):
+    """A layer with TTQ_PRECISION_BF16_OK: from 256 rows on, fp16 and fp32 activations are rounded to bf16 into a
+    workspace and run the matrix-core GEMM (2e-2 class: weights and activations rounded to bf16 once); every
+    output type.  The default layer computes in the activations' own type: fp32 rows stay in the 1e-3 class."""
     p = random_blocks(fmt, n_out * (n_in // BLOCK_WEIGHTS[fmt]), seed=900 + m)
     what = oracle.dequant(fmt, p, n_out, n_in)
     bd, bf = x_to_dev(Q.fill_normal(901, 2, 0.5, n_out), "f32")
     xd, xf = x_to_dev(Q.fill_normal(902 + m, 1, 1.0, m * n_in).reshape(m, n_in) * np.float32(0.02), xk)
-    layer = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out, bias=bd)
+    layer = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out, bias=bd, precision=F.PRECISION_BF16_OK)
+    assert layer.route(m, xd.dtype, torch.float32) == "gemm_pc_bf16_copy"
     want = oracle.linear_f64(what, xf, bf)
     y32 = layer.forward(xd, out_dtype=torch.float32).cpu().numpy()
     assert rel_l2(y32, want) <= TOL
@@ -419,3 +421,25 @@ def test_forward_fp16_fp32_activations_many_rows_take_the_bf16_gemm(fmt, xk, m, 
     exact = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out, bias=bd, precision=F.PRECISION_F32_SCALES)
     ye = exact.forward(xd, out_dtype=torch.float32).cpu().numpy()
     assert rel_l2(ye, want) <= 1e-3
+    # the default layer never narrows the activations: fp32 rows keep the 1e-3 class, fp16 rows their own kernels
+    auto = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out, bias=bd)
+    assert auto.route(m, xd.dtype, torch.float32) != "gemm_pc_bf16_copy"
+    ya = auto.forward(xd, out_dtype=torch.float32).cpu().numpy()
+    assert rel_l2(ya, want) <= (1e-3 if xk == "f32" else TOL)
+
+
+@pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
+@pytest.mark.parametrize("m", [255, 256, 600])
+def test_forward_default_precision_keeps_fp32_activations_in_the_decode_class(fmt, m):
+    """No accuracy step at 256 rows: fp32 activations through a default layer stay within 1e-3 of the oracle,
+    every row, below and above the row count where the bf16-copy route would start if the layer allowed it."""
+    n_out, n_in = 1048, 1024
+    p = random_blocks(fmt, n_out * (n_in // BLOCK_WEIGHTS[fmt]), seed=930 + m)
+    what = oracle.dequant(fmt, p, n_out, n_in)
+    xd, xf = x_to_dev(Q.fill_normal(931 + m, 1, 1.0, m * n_in).reshape(m, n_in), "f32")
+    layer = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out)
+    y = layer.forward(xd).cpu().numpy()
+    want = oracle.linear_f64(what, xf)
+    assert rel_l2(y, want) <= 1e-3
+    for i in (0, 1, 127, 254, m - 1):
+        assert rel_l2(y[i], want[i]) <= 1e-3, i

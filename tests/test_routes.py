@@ -1,0 +1,95 @@
+"""Which kernel family the dispatcher picks (``ttq_route``): the benchmark configurations, the gate||up shape and
+the attention projections reach the kernels built for them.  A pure host query: no GPU is needed (without a visible
+device the dispatcher assumes 256 compute units, the MI355X count)."""
+import ctypes as C
+
+import pytest
+
+from tattletale_amd import _lib
+from tattletale_amd._lib import QLinearStruct, F32, F16, BF16, Q8_0, Q4_K, Q6_K, EXL3
+
+
+def route(fmt, n_out, n_in, m, x_dtype, y_dtype, bits=0, precision=_lib.PRECISION_AUTO):
+    L = _lib.lib()
+    st = QLinearStruct(format=fmt, n_out=n_out, n_in=n_in, bits=bits, codebook=_lib.CB_MCG, precision=precision)
+    r = L.ttq_route(C.byref(st), m, x_dtype, y_dtype)
+    assert r >= 0, r
+    name = L.ttq_route_name(r).decode()
+    assert _lib.ROUTE[name] == r
+    return name
+
+
+# (what, format, n_out, n_in, m, x dtype, y dtype, bits, kernel family)
+PINNED = [
+    ("config 1: Q8_0 GEMV 4096x4096, fp32 x", Q8_0, 4096, 4096, 1, F32, F32, 0, "gemv_q8_stream"),
+    ("config 2: Q4_K GEMV 14336x4096 (headline)", Q4_K, 14336, 4096, 1, BF16, F32, 0, "gemv_q4k_stream"),
+    ("config 3: Q6_K GEMV 128256x4096 (LM head)", Q6_K, 128256, 4096, 1, BF16, F32, 0, "gemv_q6k_stream"),
+    ("config 4: Q4_K GEMM M=64", Q4_K, 14336, 4096, 64, BF16, BF16, 0, "gemm_skinny"),
+    ("config 4: Q4_K GEMM M=512 (headline)", Q4_K, 14336, 4096, 512, BF16, BF16, 0, "gemm_pc"),
+    ("config 4: Q4_K GEMM M=2048", Q4_K, 14336, 4096, 2048, BF16, BF16, 0, "gemm_pc"),
+    ("config 5: EXL3 3-bit GEMV 4096x4096", EXL3, 4096, 4096, 1, F16, F32, 3, "exl3_gemv_sliced"),
+    ("gate||up 28672x4096, decode", Q4_K, 28672, 4096, 1, BF16, F32, 0, "gemv_q4k_stream"),
+    ("q / o projection 4096x4096, decode", Q4_K, 4096, 4096, 1, BF16, F32, 0, "gemv_q4k_stream"),
+    ("k / v projection 1024x4096, decode", Q4_K, 1024, 4096, 1, BF16, F32, 0, "gemv_dot2"),
+    ("down projection 4096x14336, decode", Q4_K, 4096, 14336, 1, BF16, F32, 0, "gemv_q4k_slice"),
+    ("q / o projection, prefill 512 rows", Q4_K, 4096, 4096, 512, BF16, BF16, 0, "gemm_pc"),
+    ("down projection, prefill 512 rows", Q4_K, 4096, 14336, 512, BF16, BF16, 0, "gemm_pc_split_k"),
+    ("two rows of the headline shape", Q4_K, 14336, 4096, 2, BF16, F32, 0, "gemv_q4k_stream4"),
+    ("three rows of the LM head", Q6_K, 128256, 4096, 3, BF16, F32, 0, "gemv_q6k_stream4"),
+    ("trellis layer, prefill 512 rows", EXL3, 4096, 4096, 512, F16, F32, 3, "exl3_gemm"),
+]
+
+
+@pytest.mark.parametrize("what,fmt,n_out,n_in,m,xd,yd,bits,want", PINNED, ids=[p[0] for p in PINNED])
+def test_benchmark_and_model_shapes_reach_their_kernels(what, fmt, n_out, n_in, m, xd, yd, bits, want):
+    assert route(fmt, n_out, n_in, m, xd, yd, bits) == want
+
+
+def test_precision_flags_steer_the_route():
+    # fp32 activations never leave the decode kernels by default, whatever the row count
+    for m in (5, 255, 256, 600, 4096):
+        assert route(Q4_K, 14336, 4096, m, F32, F32).startswith("gemv_")
+    # fp16 activations: their own few-row matrix-core kernel, never a bf16 copy
+    assert route(Q4_K, 14336, 4096, 256, F16, F16) == "gemm_skinny_chunked"
+    # only a layer that allows it rounds fp16 / fp32 activations to bf16
+    for xd in (F16, F32):
+        assert route(Q4_K, 14336, 4096, 256, xd, F32, precision=_lib.PRECISION_BF16_OK) == "gemm_pc_bf16_copy"
+        assert route(Q4_K, 14336, 4096, 255, xd, F32, precision=_lib.PRECISION_BF16_OK) != "gemm_pc_bf16_copy"
+    # F32_SCALES pins the decode kernels for bf16 activations too
+    assert route(Q4_K, 14336, 4096, 512, BF16, BF16, precision=_lib.PRECISION_F32_SCALES).startswith("gemv_")
+    assert route(EXL3, 4096, 4096, 512, F16, F32, bits=3, precision=_lib.PRECISION_F32_SCALES).startswith("exl3_gemv")
+
+
+def test_route_is_a_pure_query():
+    L = _lib.lib()
+    st = QLinearStruct(format=Q4_K, n_out=14336, n_in=4096)
+    assert L.ttq_route(None, 1, BF16, F32) == _lib.ERR_NULL
+    assert L.ttq_route(C.byref(st), 1, 9, F32) == _lib.ERR_DTYPE
+    assert L.ttq_route(C.byref(st), -1, BF16, F32) == _lib.ERR_SHAPE
+    assert L.ttq_route(C.byref(st), 0, BF16, F32) == _lib.ROUTE["none"]         # an empty batch launches nothing
+    st.n_in = 100
+    assert L.ttq_route(C.byref(st), 1, BF16, F32) == _lib.ERR_SHAPE
+    assert L.ttq_route_name(12345) == b"unknown route"
+    # the same answer every time, with no buffer behind the layer
+    st.n_in = 4096
+    assert len({L.ttq_route(C.byref(st), 512, BF16, BF16) for _ in range(5)}) == 1
+
+
+def test_workspace_size_query_and_argument_checks():
+    L = _lib.lib()
+    q = QLinearStruct(format=Q4_K, n_out=4096, n_in=14336)
+    assert L.ttq_workspace_bytes(C.byref(q), 1, BF16) == 0                       # decode kernels take none
+    split = L.ttq_workspace_bytes(C.byref(q), 512, BF16)
+    assert split > (4 << 20)                                                     # header + partial sums
+    assert L.ttq_workspace_bytes(C.byref(q), 512, F32) > split                   # + the bf16 copy of the rows
+    assert L.ttq_workspace_bytes(C.byref(q), 0, BF16) == 0
+    assert L.ttq_workspace_bytes(None, 1, BF16) == _lib.ERR_NULL
+    assert L.ttq_workspace_bytes(C.byref(q), 1, 5) == _lib.ERR_DTYPE
+    t = QLinearStruct(format=EXL3, n_out=4096, n_in=4096, bits=3, codebook=_lib.CB_MCG)
+    assert L.ttq_workspace_bytes(C.byref(t), 1, F16) > (4 << 20)                 # hand-off words
+    # a workspace that cannot be one is refused before anything else happens
+    assert L.ttq_linear_forward_ws(C.byref(q), None, BF16, 512, None, BF16, None, 1024, None) == _lib.ERR_WORKSPACE
+    assert L.ttq_linear_forward_ws(C.byref(q), None, BF16, 512, None, BF16, 8, 1024, None) == _lib.ERR_WORKSPACE
+    assert L.ttq_linear_forward_ws(C.byref(q), None, BF16, 512, None, BF16, None, -1, None) == _lib.ERR_WORKSPACE
+    assert L.ttq_linear_forward_ws(C.byref(q), None, BF16, 0, None, BF16, None, 0, None) == _lib.OK
+    assert L.ttq_strerror(_lib.ERR_WORKSPACE) not in (b"unknown status", b"ok")
