@@ -676,27 +676,14 @@ def main() -> int:
                                                C.c_int64, C.c_int64, C.c_void_p]
         rng = np.random.default_rng(97)
         # (kernel, ABL, what runs); kernel 0 = X straight into the consumers' registers, 1 = X staged through LDS
-        rungs = [(0, 31, "barriers, prologue, epilogue only"),
-                 (0, 4124, "consumers alone (A requests, B reads, MFMA; real values in the W tile)"),
-                 (0, 4104, "+ W loads and LDS stores, no dequantization"),
-                 (0, 0, "whole kernel"),
-                 (0, 3, "W producers alone"),
-                 (0, 2, "consumers without A requests + W producers"),
-                 (0, 1024, "whole kernel without barriers (roles free-running)"),
-                 (2, 31, "8 consumers of 32 rows: barriers, prologue, epilogue only"),
-                 (2, 4124, "8 consumers of 32 rows: consumers alone"),
-                 (2, 0, "8 consumers of 32 rows: whole kernel"),
-                 (2, 2, "8 consumers of 32 rows: consumers without A requests + W producers"),
-                 (2, 1024, "8 consumers of 32 rows: whole kernel without barriers"),
-                 (0, 8192 + 4124, "4 consumers alone, addresses as if X were packed in fragment order"),
-                 (0, 8192, "4 consumers, whole kernel, addresses as if X were packed in fragment order"),
-                 (0, 8192 + 1024, "4 consumers, whole kernel, packed-order addresses, no barriers"),
-                 (0, 8192 + 8, "4 consumers, packed-order addresses, producers without dequantization"),
-                 (0, 8192 + 4, "4 consumers, packed-order addresses, producers without LDS stores"),
-                 (0, 8192 + 64, "4 consumers, whole kernel, packed-order addresses, consumers at priority 3"),
-                 (0, 8192 + 128, "4 consumers, whole kernel, packed-order addresses, producers at priority 3"),
-                 (2, 8192 + 4124, "8 consumers alone, addresses as if X were packed in fragment order"),
-                 (2, 8192, "8 consumers, whole kernel, addresses as if X were packed in fragment order"),
+        rungs = [(0, 31, "packed X: barriers, prologue, epilogue only"),
+                 (0, 4124, "packed X: consumers alone (A requests, B reads, MFMA; real values in the W tile)"),
+                 (0, 4104, "packed X: + W loads and LDS stores, no dequantization"),
+                 (0, 0, "packed X: whole kernel"),
+                 (0, 3, "packed X: W producers alone"),
+                 (0, 2, "packed X: consumers without A requests + W producers"),
+                 (0, 1024, "packed X: whole kernel without barriers (roles free-running)"),
+                 (-1, 0, "packed X: the packing pass alone"),
                  (1, 31, "LDS-staged X: barriers, prologue, epilogue only"),
                  (1, 4126, "LDS-staged X: consumers alone (real values in LDS)"),
                  (1, 4124, "LDS-staged X: consumers + X movers"),
@@ -704,6 +691,8 @@ def main() -> int:
                  (1, 29, "LDS-staged X: X movers alone"),
                  (1, 1024, "LDS-staged X: whole kernel without barriers"),
                  (1, 2048, "LDS-staged X by global_load_lds: whole kernel")]
+        LAD.ttq_ladder_gemm_pack.restype = C.c_int
+        LAD.ttq_ladder_gemm_pack.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p]
         packed = random_packed(rng, F.Q4_K, n_out, n_in)
         ncopies = rotated(packed.nbytes)
         ws = [to_dev(packed) for _ in range(ncopies)]
@@ -713,10 +702,17 @@ def main() -> int:
             y = torch.empty((m, n_out), dtype=torch.bfloat16, device=dev)
             flop = 2.0 * m * n_out * n_in
             rows = []
+            xp = torch.empty(((m + 15) // 16 * 16, n_in), dtype=torch.bfloat16, device=dev)
+            if LAD.ttq_ladder_gemm_pack(x.data_ptr(), xp.data_ptr(), m, n_in, torch.cuda.current_stream(dev).cuda_stream):
+                raise RuntimeError("ttq_ladder_gemm_pack failed")
             for kern, abl, what in rungs:
                 def step(i, kern=kern, abl=abl):
-                    rc = LAD.ttq_ladder_gemm_launch(kern, abl, ws[i % ncopies].data_ptr(), x.data_ptr(), y.data_ptr(), m,
-                                                    n_out, n_in, torch.cuda.current_stream(dev).cuda_stream)
+                    sh = torch.cuda.current_stream(dev).cuda_stream
+                    if kern < 0:
+                        rc = LAD.ttq_ladder_gemm_pack(x.data_ptr(), xp.data_ptr(), m, n_in, sh)
+                    else:
+                        rc = LAD.ttq_ladder_gemm_launch(kern, abl, ws[i % ncopies].data_ptr(),
+                                                        (xp if kern == 0 else x).data_ptr(), y.data_ptr(), m, n_out, n_in, sh)
                     if rc != 0:
                         raise RuntimeError("ttq_ladder_gemm_launch(%d, %d) returned %d" % (kern, abl, rc))
                 t = time_steps(step, max(20, steps // (10 if m <= 512 else 40)), max(3, warmup // 10))

@@ -184,7 +184,9 @@ typedef enum {
   TTQ_ROUTE_GEMM_SKINNY = 22,        /* 17-64 rows */
   TTQ_ROUTE_GEMM_SKINNY_CHUNKED = 23,
   TTQ_ROUTE_GEMM_Q4K_TILES = 24,     /* single-role tiled kernel (128-column tiles, activations beyond 4 GiB) */
-  TTQ_ROUTE_GEMM_PC_BF16_COPY = 25,  /* TTQ_PRECISION_BF16_OK: bf16 copy of fp16 / fp32 activations, then GEMM_PC */
+  TTQ_ROUTE_GEMM_PC_BF16_COPY = 25,  /* TTQ_PRECISION_BF16_OK: fp16 / fp32 activations rounded to bf16 by the packing pass */
+  TTQ_ROUTE_GEMM_PC_PACKED = 26,     /* long launches: activations packed in fragment order first (takes a workspace) */
+  TTQ_ROUTE_GEMM_PC_PACKED_SPLIT_K = 27,
   TTQ_ROUTE_EXL3_GEMV = 30,
   TTQ_ROUTE_EXL3_GEMV_SLICED = 31,   /* K sliced over workgroups that meet in a workspace */
   TTQ_ROUTE_EXL3_GEMM = 32,

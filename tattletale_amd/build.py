@@ -34,6 +34,7 @@ SOURCES = [
     "ttq_gemv_q4k_batch4.hip",
     "ttq_gemm_q4k.hip",
     "ttq_gemm_pc.hip",
+    "ttq_gemm_pcd.hip",
     "ttq_gemm_skinny.hip",
     "ttq_exl3.hip",
     "ttq_exl3_mfma.hip",

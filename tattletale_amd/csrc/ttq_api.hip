@@ -460,30 +460,15 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
                                          layer->bias, layer->bias_dtype, m, n_out, n_in, s));
   }
   // fp16 / fp32 activations, 256 rows or more, and only where the layer says that bf16 activations will do
-  // (TTQ_PRECISION_BF16_OK; the operator computes in the type of x otherwise): round them to bf16 into a workspace
-  // (4096 rows at a time) and run the bf16 matrix-core GEMM (weights and activations rounded to bf16: the 2e-2
-  // class, like the GEMM entry points)
+  // (TTQ_PRECISION_BF16_OK; the operator computes in the type of x otherwise): the prefill GEMM's packing pass rounds
+  // them to bf16 on the way into its workspace (weights and activations rounded to bf16: the 2e-2 class, like the
+  // GEMM entry points)
   const bool block_fmt = layer->format == TTQ_Q4_K || layer->format == TTQ_Q6_K || layer->format == TTQ_Q8_0;
   if ((x_dtype == TTQ_F16 || x_dtype == TTQ_F32) && block_fmt && m >= 256 && route != 1 && n_in % 8 == 0 &&
       layer->precision == TTQ_PRECISION_BF16_OK &&
-      ttq::gemm_pc_supported(layer->format, m < 4096 ? m : 4096, n_out, n_in, 112)) {
-    if (ttq::route_probe(ttq::kRouteGemmPcBf16Copy)) return TTQ_OK;
-    constexpr int64_t kRows = 4096;
-    void* ws = nullptr;
-    const int64_t block_rows = m < kRows ? m : kRows;
-    hipError_t e = ttq::stream_workspace(ttq::kWsBf16Activations, s, (size_t)block_rows * n_in * 2, &ws);
-    if (e != hipSuccess) return hip_status(e);
-    for (int64_t r0 = 0; r0 < m; r0 += kRows) {
-      const int64_t rows = m - r0 < kRows ? m - r0 : kRows;
-      e = ttq::launch_to_bf16(static_cast<const char*>(x) + r0 * n_in * dtype_size(x_dtype), x_dtype,
-                              static_cast<uint16_t*>(ws), rows * n_in, s);
-      if (e != hipSuccess) return hip_status(e);
-      e = ttq::launch_gemm_pc(layer->format, layer->qweight, static_cast<const uint16_t*>(ws),
-                              static_cast<char*>(y) + r0 * n_out * dtype_size(y_dtype), y_dtype, layer->bias,
-                              layer->bias_dtype, rows, n_out, n_in, s);
-      if (e != hipSuccess) return hip_status(e);
-    }
-    return TTQ_OK;
+      ttq::gemm_pc_supported(layer->format, m < 8192 ? m : 8192, n_out, n_in, 112)) {
+    return hip_status(ttq::launch_gemm_pc_x(layer->format, layer->qweight, x, x_dtype, y, y_dtype, layer->bias,
+                                            layer->bias_dtype, m, n_out, n_in, s));
   }
   // fp16 activations, up to 64 rows: the few-row kernel takes them as they are
   const bool block_format = layer->format == TTQ_Q4_K || layer->format == TTQ_Q6_K || layer->format == TTQ_Q8_0;
@@ -549,6 +534,8 @@ const char* ttq_route_name(int route) {
     case TTQ_ROUTE_GEMM_SKINNY_CHUNKED: return "gemm_skinny_chunked";
     case TTQ_ROUTE_GEMM_Q4K_TILES: return "gemm_q4k_tiles";
     case TTQ_ROUTE_GEMM_PC_BF16_COPY: return "gemm_pc_bf16_copy";
+    case TTQ_ROUTE_GEMM_PC_PACKED: return "gemm_pc_packed";
+    case TTQ_ROUTE_GEMM_PC_PACKED_SPLIT_K: return "gemm_pc_packed_split_k";
     case TTQ_ROUTE_EXL3_GEMV: return "exl3_gemv";
     case TTQ_ROUTE_EXL3_GEMV_SLICED: return "exl3_gemv_sliced";
     case TTQ_ROUTE_EXL3_GEMM: return "exl3_gemm";
@@ -566,18 +553,20 @@ int64_t ttq_workspace_bytes(const ttq_qlinear* layer, int64_t m, int x_dtype) {
   if (m == 0 || layer->n_out == 0) return 0;
   const int64_t n_out = layer->n_out, n_in = layer->n_in;
   const int64_t header = (int64_t)ttq::caller_workspace_header_bytes();
-  constexpr int64_t kChunkRows = 4096;          // rows whose bf16 / rotated copy is in the workspace at a time
-  const int64_t block_rows = m < kChunkRows ? m : kChunkRows;
-  if (layer->format == TTQ_EXL3)                // hand-off words; the rotated activations of the many-row form
+  constexpr int64_t kExl3Rows = 4096, kGemmRows = 8192;   // rows whose rotated / packed copy is in the workspace at a time
+  if (layer->format == TTQ_EXL3) {              // hand-off words; the rotated activations of the many-row form
+    const int64_t block_rows = m < kExl3Rows ? m : kExl3Rows;
     return header + ((block_rows * n_in * 2 + 255) & ~(int64_t)255);
+  }
   if (m < 5) return 0;                          // the decode kernels take no workspace
-  // a bf16 copy of fp16 / fp32 activations, then the partial sums of a launch split along K: the prefill GEMM's
-  // exact size for every row count it can be called with here, and the few-row kernel's bound (one 64 x 64 tile
-  // of sums per compute unit)
-  int64_t scratch = 0;
-  if (x_dtype != TTQ_BF16 && m >= 256) scratch += (block_rows * n_in * 2 + 255) & ~(int64_t)255;
+  // the packed bf16 copy of the activations where the prefill GEMM wants one, then the partial sums of a launch
+  // split along K: the prefill GEMM's exact size for every row count it can be called with here, and the few-row
+  // kernel's bound (one 64 x 64 tile of sums per compute unit)
+  const int64_t block_rows = m < kGemmRows ? m : kGemmRows;
+  const int copy_dtype = (x_dtype != TTQ_BF16 && layer->precision == TTQ_PRECISION_BF16_OK && m >= 256) ? x_dtype : TTQ_BF16;
+  int64_t scratch = ((int64_t)ttq::gemm_pc_packed_bytes(m, n_out, n_in, copy_dtype) + 255) & ~(int64_t)255;
   int64_t partials = (int64_t)ttq::device_num_cus() * (16 * 4 * (16 * 4 + 1) * 4);
-  const int64_t rows[3] = {m, block_rows, m % kChunkRows};
+  const int64_t rows[3] = {m, block_rows, m % kGemmRows};
   for (int64_t r : rows) {
     if (r <= 0) continue;
     const int64_t p = (int64_t)ttq::gemm_pc_partials_bytes(r, n_out, n_in);

@@ -242,6 +242,14 @@ struct PcSplit {
 };
 constexpr int kPcMaxCounters = 16384;     // (tile, consumer) pairs a split launch may have
 
+// The same GEMM over a copy of the activations in fragment order (ttq_gemm_pcd.h, instantiated in ttq_gemm_pcd.hip):
+// tile = index into launch_gemm_pc's table of tile shapes.
+hipError_t launch_gemm_packed(int format, bool fuse, int tile, const uint8_t* wb, const uint16_t* xp, void* y, int y_dtype,
+                              const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, PcSplit sp,
+                              hipStream_t s);
+size_t gemm_packed_activation_bytes(int64_t m, int64_t n_in);
+hipError_t launch_gemm_pack_activations(const void* x, int x_dtype, uint16_t* xp, int64_t m, int64_t n_in, hipStream_t s);
+
 // What a consumer wavefront does with its finished accumulators (shared by the kernels of this file and of
 // ttq_gemm_pcd.h): the meeting of the K copies, bias, silu_and_mul, rounding, and the store of Y.
 struct PcEpi {

@@ -4,9 +4,11 @@
 
 namespace ttq {
 
+// x: the activations, or (tile_if_packed >= 0) their packed copy and the tile's index for launch_gemm_packed
 template <int FMT, int MB, int NJ, bool FUSE>
 static hipError_t launch_pc_tile(const uint8_t* wb, const uint16_t* x, void* y, int y_dtype, const void* bias,
-                                 int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, int splits, hipStream_t s) {
+                                 int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, int splits, int tile_if_packed,
+                                 hipStream_t s) {
   PcSplit sp{1, 0, nullptr, nullptr};
   if (!FUSE && splits > 1) {
     // (the chooser has checked that the blocks of a row divide evenly and that the counters suffice)
@@ -21,6 +23,8 @@ static hipError_t launch_pc_tile(const uint8_t* wb, const uint16_t* x, void* y, 
     sp.partials = static_cast<float*>(part);
     sp.counters = static_cast<uint32_t*>(cnt);
   }
+  if (tile_if_packed >= 0)
+    return launch_gemm_packed(FMT, FUSE, tile_if_packed, wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
   return launch_pc_grid<FMT, MB, NJ, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
 }
 
@@ -92,18 +96,56 @@ float gemm_pc_estimate_us(int format, int64_t m, int64_t n_out, int64_t n_in) {
   return c * (format == kQ8_0 ? 1.9f : (format == kQ6_K ? 1.4f : 1.f)) + 2.f;
 }
 
+// Long launches read the activations from a copy in fragment order (ttq_gemm_pcd.h), made by one pass over X into
+// a workspace: the GEMM is then about a tenth faster (no X traffic through LDS), which pays for the pass (2.5 us + the
+// bytes at ~3 TB/s) from about 30 us of GEMM on.
+constexpr int64_t kPackRows = 8192;         // rows packed (and multiplied) at a time
+static bool pc_use_packed(const PcChoice& c, int64_t m, int64_t n_in) {
+  static const int knob = dev_knob("TTQ_GEMM_PACKED", -1);      // A/B: 0 never, 1 always
+  if (knob >= 0) return knob != 0;
+  return c.cost_us >= 30.f + (float)(m * n_in * 4) / 3.0e6f * 10.f;
+}
+
 template <int FMT, bool FUSE>
-static hipError_t launch_pc_fmt(const uint8_t* wb, const uint16_t* x, void* y, int y_dtype, const void* bias,
-                                int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
-  const PcChoice c = pc_choose(m, n_out, n_in, FUSE);
+static hipError_t launch_pc_rows(const PcChoice& c, int tile_if_packed, const uint8_t* wb, const uint16_t* x, void* y,
+                                 int y_dtype, const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
+                                 hipStream_t s) {
+  const int p = tile_if_packed;
   switch (c.tile) {
-    case 0: return launch_pc_tile<FMT, 4, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, s);
-    case 1: return launch_pc_tile<FMT, 4, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, s);
-    case 2: return launch_pc_tile<FMT, 2, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, s);
-    case 3: return launch_pc_tile<FMT, 2, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, s);
-    case 4: return launch_pc_tile<FMT, 1, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, s);
-    default: return launch_pc_tile<FMT, 1, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, s);
+    case 0: return launch_pc_tile<FMT, 4, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s);
+    case 1: return launch_pc_tile<FMT, 4, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s);
+    case 2: return launch_pc_tile<FMT, 2, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s);
+    case 3: return launch_pc_tile<FMT, 2, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s);
+    case 4: return launch_pc_tile<FMT, 1, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s);
+    default: return launch_pc_tile<FMT, 1, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s);
   }
+}
+
+// x in x_dtype: bf16 for the direct form; any type when the launch goes through the packed copy (the packing pass
+// rounds to bf16).
+template <int FMT, bool FUSE>
+static hipError_t launch_pc_fmt(const uint8_t* wb, const void* x, int x_dtype, void* y, int y_dtype, const void* bias,
+                                int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, bool force_packed, hipStream_t s) {
+  const PcChoice whole = pc_choose(m, n_out, n_in, FUSE);
+  if (!force_packed && !pc_use_packed(whole, m, n_in))
+    return launch_pc_rows<FMT, FUSE>(whole, -1, wb, static_cast<const uint16_t*>(x), y, y_dtype, bias, bias_dtype, m, n_out,
+                                     n_in, s);
+  const int64_t block_rows = m < kPackRows ? m : kPackRows;
+  void* ws = nullptr;
+  hipError_t e = stream_workspace(kWsPackedActivations, s, gemm_packed_activation_bytes(block_rows, n_in), &ws);
+  if (e != hipSuccess) return e;
+  const int64_t xsize = x_dtype == kF32 ? 4 : 2, ysize = y_dtype == kF32 ? 4 : 2;
+  for (int64_t r0 = 0; r0 < m; r0 += kPackRows) {
+    const int64_t rows = m - r0 < kPackRows ? m - r0 : kPackRows;
+    e = launch_gemm_pack_activations(static_cast<const char*>(x) + r0 * n_in * xsize, x_dtype, static_cast<uint16_t*>(ws),
+                                     rows, n_in, s);
+    if (e != hipSuccess) return e;
+    const PcChoice c = rows == m ? whole : pc_choose(rows, n_out, n_in, FUSE);
+    e = launch_pc_rows<FMT, FUSE>(c, c.tile, wb, static_cast<const uint16_t*>(ws), static_cast<char*>(y) + r0 * n_out * ysize,
+                                  y_dtype, bias, bias_dtype, rows, n_out, n_in, s);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
 }
 
 // 112- and 64-column tiles are built in this form: with 128 columns the consumers' 128
@@ -116,19 +158,39 @@ bool gemm_pc_supported(int format, int64_t m, int64_t n_out, int64_t n_in, int b
          m * n_in * 2 < ((int64_t)1 << 32) && n_out > 0 && n_in > 0 && n_in % 256 == 0;
 }
 
+// x: bf16 activations; or (x_dtype fp16 / fp32) activations that may be rounded to bf16: those always go through the
+// packed copy, whose packing pass does the rounding.
+hipError_t launch_gemm_pc_x(int format, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                            const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+  if (m == 0 || n_out == 0) return hipSuccess;
+  if (y_dtype != kBF16 && y_dtype != kF32 && y_dtype != kF16) return hipErrorInvalidValue;
+  const PcChoice c = pc_choose(m, n_out, n_in, false);
+  const bool packed = x_dtype != kBF16 || pc_use_packed(c, m, n_in);
+  if (route_probe(x_dtype != kBF16 ? kRouteGemmPcBf16Copy
+                                   : (c.splits > 1 ? (packed ? kRouteGemmPcPackedSplitK : kRouteGemmPcSplitK)
+                                                   : (packed ? kRouteGemmPcPacked : kRouteGemmPc))))
+    return hipSuccess;
+  const uint8_t* wb = static_cast<const uint8_t*>(w);
+  const bool force = x_dtype != kBF16;
+  switch (format) {
+    case kQ4_K: return launch_pc_fmt<kQ4_K, false>(wb, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, force, s);
+    case kQ6_K: return launch_pc_fmt<kQ6_K, false>(wb, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, force, s);
+    case kQ8_0: return launch_pc_fmt<kQ8_0, false>(wb, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, force, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
 hipError_t launch_gemm_pc(int format, const void* w, const uint16_t* x_bf16, void* y, int y_dtype,
                           const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                           hipStream_t s) {
-  if (m == 0 || n_out == 0) return hipSuccess;
-  if (y_dtype != kBF16 && y_dtype != kF32 && y_dtype != kF16) return hipErrorInvalidValue;
-  if (route_probe(pc_choose(m, n_out, n_in, false).splits > 1 ? kRouteGemmPcSplitK : kRouteGemmPc)) return hipSuccess;
-  const uint8_t* wb = static_cast<const uint8_t*>(w);
-  switch (format) {
-    case kQ4_K: return launch_pc_fmt<kQ4_K, false>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-    case kQ6_K: return launch_pc_fmt<kQ6_K, false>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-    case kQ8_0: return launch_pc_fmt<kQ8_0, false>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-    default: return hipErrorInvalidValue;
-  }
+  return launch_gemm_pc_x(format, w, x_bf16, kBF16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+}
+
+// bytes of the packed copy a launch of this shape takes from the workspace (0: it reads X itself)
+size_t gemm_pc_packed_bytes(int64_t m, int64_t n_out, int64_t n_in, int x_dtype) {
+  if (m <= 0 || n_out <= 0 || n_in < 256) return 0;
+  const bool packed = x_dtype != kBF16 || pc_use_packed(pc_choose(m, n_out, n_in, false), m, n_in);
+  return packed ? gemm_packed_activation_bytes(m < kPackRows ? m : kPackRows, n_in) : 0;
 }
 
 
@@ -138,8 +200,8 @@ hipError_t launch_gemm_pc_silu_mul(const void* w, const uint16_t* x_bf16, void* 
                                    int bias_dtype, int64_t m, int64_t n_ff, int64_t n_in, hipStream_t s) {
   if (m == 0 || n_ff == 0) return hipSuccess;
   if (y_dtype != kBF16 && y_dtype != kF32) return hipErrorInvalidValue;
-  return launch_pc_fmt<kQ4_K, true>(static_cast<const uint8_t*>(w), x_bf16, y, y_dtype, bias, bias_dtype, m, n_ff,
-                                    n_in, s);
+  return launch_pc_fmt<kQ4_K, true>(static_cast<const uint8_t*>(w), x_bf16, kBF16, y, y_dtype, bias, bias_dtype, m, n_ff,
+                                    n_in, false, s);
 }
 
 }  // namespace ttq

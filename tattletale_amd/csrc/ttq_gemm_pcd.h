@@ -7,13 +7,18 @@
 //
 // A workgroup of eight wavefronts (two per SIMD) owns a (64 * MB) x BN tile of Y:
 //   consumers (wavefronts 0-3, 16 * MB rows of the tile each): v_mfma_f32_16x16x32_bf16, B fragments from the W
-//       tile in LDS, A fragments by buffer loads from X itself.  Lane (r, g) of a 16 x 32 A fragment holds eight
-//       consecutive k of row r: 16 bytes of the row-major activation, so a fragment is one 16-byte load per lane
-//       and needs no LDS at all.  The fragments of step s+2 are requested during step s into one of three register
-//       sets that rotate by name.
+//       tile in LDS, A fragments by buffer loads, three steps' worth of registers rotating by name: the fragments
+//       of step s+2 are requested during step s.
 //   producers (wavefronts 4-7): pc_produce_w of ttq_gemm_pc.h -- packed blocks, canonical dequantization, bf16
 //       nearest-even, B fragments into the double-buffered W tile.
 // One barrier per 64-k step.
+//
+// The activations come from a copy of X in fragment order (pack_activations below, one pass over X per call):
+//     Xp[step ks][row block rb][half h][lane l] = 16 bytes: row 16 rb + l % 16, k = 64 ks + 32 h + 8 (l / 16) .. + 7
+// so that an A fragment is one load instruction over 1 KB of consecutive bytes.  Read from the row-major X itself
+// the same fragment is 16 bytes from each of 16 rows per quarter wavefront, the vector memory path then handles a
+// lane at a time, and the consumers wait for their requests longer than they multiply (measured: 65 us against 43
+// for the consumers alone at M = 512).
 //
 // Why X bypasses LDS: every byte written to LDS goes through one port of about 85 bytes per cycle and compute unit,
 // whoever writes (ds_write or global_load_lds), and LDS reads queue behind waiting ds_writes.  With X staged through
@@ -41,7 +46,7 @@ __device__ __forceinline__ void buffer_load16_async(u32x4_t& dst, u32x4_t rsrc, 
 
 template <int NJ, int FMT, int MB, bool FUSE, int ABL = 0, int NC = 4>
 __global__ void __launch_bounds__(pcd_threads(NC))
-gemm_pcd_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, void* __restrict__ yv,
+gemm_pcd_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ xp, void* __restrict__ yv,
                 int y_dtype, const void* __restrict__ bias, int bias_dtype, int m, int n_out, int n_in,
                 int n_tiles, int m_tiles, int xcds_per_mtile, PcSplit sp) {
   constexpr int BN = NJ * 16;
@@ -101,7 +106,7 @@ gemm_pcd_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, v
   const int ksteps = nblocks * 4;
 
   if constexpr ((ABL & 4096) != 0) {
-    const uint4* src = reinterpret_cast<const uint4*>(x);
+    const uint4* src = reinterpret_cast<const uint4*>(xp);
     const int lim = min(m, 256) * n_in / 8;
     for (int i = tid; i < 2 * kWUnits; i += kPcdThreads) sw[i] = src[(i * 5 + (int)blockIdx.x * 32 + 4096) % lim];
     __syncthreads();
@@ -111,7 +116,6 @@ gemm_pcd_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, v
   // complete in LDS (buffer (s+1) % 2) and every LDS read of step s has finished.  The consumers pass it near the
   // end of step s, the producers after preparing step s+1.
   if (wave >= NC) {
-    if constexpr ((ABL & 128) != 0) __builtin_amdgcn_s_setprio(3);
     pc_produce_w<NJ, FMT, FUSE, ABL>(w, tid - NC * 64, n0, n_out, row_blocks, block0, nblocks,
                                      (uint32_t)(size_t)(lptr_t)(&sw[0]), bar);
     trace_out();
@@ -119,30 +123,29 @@ gemm_pcd_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, v
   }
 
   // -------------------------------------------------------------------- consumer
-  if constexpr ((ABL & 64) != 0) __builtin_amdgcn_s_setprio(3);
   const int m0 = m_tile * kPcBM + wave * (16 * MB);
-  const int fr = lane & 15, fg = lane >> 4;
-  // A fragment (row block ib, half h of step ks): row m0 + 16 ib + fr, bytes 128 ks + 64 h + 16 fg .. + 16 of it.
-  // Buffer loads take the per-lane offset (loop-invariant), the uniform offset of the step and the half as an
-  // immediate: no address arithmetic per request.  Rows past the end are clamped (never stored to Y).
-  const uint8_t* xb = reinterpret_cast<const uint8_t*>(x);
+  // A fragment (row block ib of this consumer, half h of step ks): 1 KB at ((ks * RB + rb0 + ib) * 2 + h) * 1024 of
+  // the packed copy, RB = row blocks of the whole activation.  Buffer loads take the per-lane offset (loop-invariant),
+  // the uniform offset of the step and the half as an immediate: no address arithmetic per request.  Row blocks past
+  // the end are clamped (never stored to Y).
+  const int row_blocks_x = (m + 15) >> 4;
+  const uint64_t xaddr = (uint64_t)(size_t)xp;
   // raw buffer descriptor: base, stride 0, bytes (< 4 GiB: the launcher checks), 32-bit untyped data
-  const uint64_t xaddr = (uint64_t)(size_t)xb;
-  u32x4_t xrsrc = {(uint32_t)xaddr, (uint32_t)(xaddr >> 32) & 0xFFFFu, (uint32_t)m * (uint32_t)(n_in * 2), 0x00020000u};
+  u32x4_t xrsrc = {(uint32_t)xaddr, (uint32_t)(xaddr >> 32) & 0xFFFFu, (uint32_t)row_blocks_x * (uint32_t)(n_in * 32),
+                   0x00020000u};
 #pragma unroll
   for (int q = 0; q < 4; q++) xrsrc[q] = (uint32_t)__builtin_amdgcn_readfirstlane((int)xrsrc[q]);
   int aoff[MB];
 #pragma unroll
-  for (int ib = 0; ib < MB; ib++)
-    aoff[ib] = (ABL & 8192) ? (m_tile * (n_in / 64) * (kPcBM * 128) + wave * (16 * MB * 128) + ib * 2048 + lane * 16)   // ladder: as if X were packed in fragment order
-                            : (int)((uint32_t)min(m0 + 16 * ib + fr, m - 1) * (uint32_t)(n_in * 2) + (uint32_t)(fg * 16));
+  for (int ib = 0; ib < MB; ib++) aoff[ib] = min((m0 >> 4) + ib, row_blocks_x - 1) * 2048 + lane * 16;
   struct ASet { u32x4_t v[2][MB]; };
-  auto request_one = [&](ASet& dst, int koff, int h, int ib) {   // koff: byte offset of the step in a row
+  auto request_one = [&](ASet& dst, int koff, int h, int ib) {   // koff: byte offset of the step in the packed copy
     if constexpr ((ABL & 2) != 0) return;
     if (h == 0) buffer_load16_async<0>(dst.v[0][ib], xrsrc, aoff[ib], koff);
-    else buffer_load16_async<(ABL & 8192) ? 1024 : 64>(dst.v[1][ib], xrsrc, aoff[ib], koff);
+    else buffer_load16_async<1024>(dst.v[1][ib], xrsrc, aoff[ib], koff);
   };
-  auto step_koff = [&](int ks) { return (4 * block0 + min(ks, ksteps - 1)) * ((ABL & 8192) ? kPcBM * 128 : 128); };   // past the end: a harmless re-read
+  // (past the last step: a harmless re-read)
+  auto step_koff = [&](int ks) { return (4 * block0 + min(ks, ksteps - 1)) * (row_blocks_x * 2048); };
   // A step is 2*NJ groups of MB MFMAs: group g uses the A fragments of half g/NJ and the B fragment of column block
   // g%NJ.  B fragments are read two groups ahead into a ring of four, the A fragments of step ks+2 are requested one
   // per group at the start of step ks, and __builtin_amdgcn_sched_barrier pins that order.
@@ -174,8 +177,7 @@ gemm_pcd_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, v
       if (g == G - 2) bar();     // barrier ks: step ks+1 is in LDS, reads of step ks done
       if (g + 2 < G) read_b(bring[(g + 2 + SO) & 3], BUF, g + 2);
       else read_b(bring[(g + 2 + SO) & 3], BUF ^ 1, g + 2 - G);
-      // request r of the step (row block r / 2, half r % 2: the two halves of a 128-byte line one after the other,
-      // so that the second finds the line in the vector cache) goes out with group r * G / (2 * MB)
+      // request r of the step (row block r / 2, half r % 2) goes out with group r * G / (2 * MB)
 #pragma unroll
       for (int r = 0; r < 2 * MB; r++)
         if (r * G / (2 * MB) == g) request_one(into, koff2, r % 2, r / 2);
@@ -224,8 +226,64 @@ gemm_pcd_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, v
                                        y_dtype, bias, bias_dtype, m, n_out, n0, m0});
 }
 
-// The caller owns the split-K workspace: sp.splits == 1 (no partials, no counters) or a prepared PcSplit whose
-// tile_wgs this function fills in.
+// X (m, n_in) in any activation type -> its bf16 copy in fragment order (rows past m as zeros).  A workgroup moves
+// 16 rows x 256 k: whole 128-byte lines in, whole kilobytes out.
+template <typename XT>
+__global__ void __launch_bounds__(256) pack_activations_kernel(const XT* __restrict__ x, uint16_t* __restrict__ xp, int m,
+                                                               int n_in, int row_blocks) {
+  const int t = threadIdx.x;
+  const int rb = blockIdx.y, ks = blockIdx.x * 4 + (t >> 6);        // a wavefront per 64-k step
+  const int l = t & 63, r = l >> 2, c2 = l & 3;                     // lane: row r, chunks 2 c2 and 2 c2 + 1 of the step
+  const int row = rb * 16 + r;
+  if (ks * 64 >= n_in) return;
+  uint4 v[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+  if constexpr (std::is_same<XT, bf16_tag>::value) {
+    if (row < m) {
+      const uint4* src = reinterpret_cast<const uint4*>(x + (int64_t)row * n_in + ks * 64 + c2 * 16);
+      v[0] = src[0];
+      v[1] = src[1];
+    }
+  } else if (row < m) {
+    const XT* src = x + (int64_t)row * n_in + ks * 64 + c2 * 16;
+    float f[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) f[i] = XElem<XT>::load(src, i);
+    v[0] = make_uint4(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]), pack_bf16x2(f[6], f[7]));
+    v[1] = make_uint4(pack_bf16x2(f[8], f[9]), pack_bf16x2(f[10], f[11]), pack_bf16x2(f[12], f[13]), pack_bf16x2(f[14], f[15]));
+  }
+  uint8_t* dst = reinterpret_cast<uint8_t*>(xp) + ((int64_t)ks * row_blocks + rb) * 2048;
+#pragma unroll
+  for (int q = 0; q < 2; q++) {
+    const int chunk = 2 * c2 + q;                                   // 8 k of the row: half chunk / 4, k-group chunk % 4
+    *reinterpret_cast<uint4*>(dst + (chunk >> 2) * 1024 + ((chunk & 3) * 16 + r) * 16) = v[q];
+  }
+}
+
+inline size_t packed_activation_bytes(int64_t m, int64_t n_in) { return (size_t)((m + 15) / 16) * 16 * (size_t)n_in * 2; }
+
+inline hipError_t launch_pack_activations(const void* x, int x_dtype, uint16_t* xp, int64_t m, int64_t n_in, hipStream_t s) {
+  const int row_blocks = (int)((m + 15) / 16);
+  const dim3 grid((unsigned)((n_in / 64 + 3) / 4), (unsigned)row_blocks), block(256);
+  switch (x_dtype) {
+    case kBF16:
+      hipLaunchKernelGGL(pack_activations_kernel<bf16_tag>, grid, block, 0, s, static_cast<const bf16_tag*>(x), xp, (int)m,
+                         (int)n_in, row_blocks);
+      break;
+    case kF16:
+      hipLaunchKernelGGL(pack_activations_kernel<f16_tag>, grid, block, 0, s, static_cast<const f16_tag*>(x), xp, (int)m,
+                         (int)n_in, row_blocks);
+      break;
+    case kF32:
+      hipLaunchKernelGGL(pack_activations_kernel<float>, grid, block, 0, s, static_cast<const float*>(x), xp, (int)m,
+                         (int)n_in, row_blocks);
+      break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+// xp: the packed copy of the activations.  The caller owns the split-K workspace: sp.splits == 1 (no partials, no
+// counters) or a prepared PcSplit whose tile_wgs this function fills in.
 template <int FMT, int MB, int NJ, bool FUSE, int ABL = 0, int NC = 4>
 static hipError_t launch_pcd_grid(const uint8_t* wb, const uint16_t* x, void* y, int y_dtype, const void* bias,
                                   int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, PcSplit sp, hipStream_t s) {

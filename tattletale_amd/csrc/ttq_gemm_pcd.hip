@@ -1,0 +1,46 @@
+// Prefill GEMM over a packed copy of the activations (kernel: ttq_gemm_pcd.h): the instantiations behind
+// launch_gemm_pc's choice of tile, and the packing pass.
+#include "ttq_gemm_pcd.h"
+
+namespace ttq {
+
+namespace {
+
+template <int FMT, bool FUSE>
+hipError_t packed_fmt(int tile, const uint8_t* wb, const uint16_t* xp, void* y, int y_dtype, const void* bias,
+                      int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, PcSplit sp, hipStream_t s) {
+  switch (tile) {
+    case 0: return launch_pcd_grid<FMT, 4, 7, FUSE>(wb, xp, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
+    case 1: return launch_pcd_grid<FMT, 4, 4, FUSE>(wb, xp, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
+    case 2: return launch_pcd_grid<FMT, 2, 7, FUSE>(wb, xp, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
+    case 3: return launch_pcd_grid<FMT, 2, 4, FUSE>(wb, xp, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
+    case 4: return launch_pcd_grid<FMT, 1, 7, FUSE>(wb, xp, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
+    case 5: return launch_pcd_grid<FMT, 1, 4, FUSE>(wb, xp, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace
+
+hipError_t launch_gemm_packed(int format, bool fuse, int tile, const uint8_t* wb, const uint16_t* xp, void* y, int y_dtype,
+                              const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, PcSplit sp,
+                              hipStream_t s) {
+  if (fuse) {
+    if (format != kQ4_K) return hipErrorInvalidValue;
+    return packed_fmt<kQ4_K, true>(tile, wb, xp, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
+  }
+  switch (format) {
+    case kQ4_K: return packed_fmt<kQ4_K, false>(tile, wb, xp, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
+    case kQ6_K: return packed_fmt<kQ6_K, false>(tile, wb, xp, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
+    case kQ8_0: return packed_fmt<kQ8_0, false>(tile, wb, xp, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+size_t gemm_packed_activation_bytes(int64_t m, int64_t n_in) { return packed_activation_bytes(m, n_in); }
+
+hipError_t launch_gemm_pack_activations(const void* x, int x_dtype, uint16_t* xp, int64_t m, int64_t n_in, hipStream_t s) {
+  return launch_pack_activations(x, x_dtype, xp, m, n_in, s);
+}
+
+}  // namespace ttq

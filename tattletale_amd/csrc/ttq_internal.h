@@ -37,6 +37,8 @@ enum : int {
   kRouteGemmSkinnyChunked = 23,
   kRouteGemmQ4kTiles = 24,
   kRouteGemmPcBf16Copy = 25,
+  kRouteGemmPcPacked = 26,
+  kRouteGemmPcPackedSplitK = 27,
   kRouteExl3Gemv = 30,
   kRouteExl3GemvSliced = 31,
   kRouteExl3Gemm = 32,
@@ -260,7 +262,7 @@ hipError_t launch_hadamard128(float* v, const uint16_t* pre, const uint16_t* pos
                               hipStream_t s);
 
 // Workspaces the library keeps per (slot, device, stream), grown on demand (ttq_workspace.hip).
-constexpr int kWsExl3Rotated = 0, kWsBf16Activations = 1, kWsGemmPartials = 2, kWsGemmCounters = 3;
+constexpr int kWsExl3Rotated = 0, kWsGemmPartials = 2, kWsGemmCounters = 3, kWsPackedActivations = 4;
 // zeroed: a newly allocated buffer is cleared (on the stream) before it is handed out
 hipError_t stream_workspace(int slot, hipStream_t s, size_t bytes, void** out, bool zeroed = false);
 // Frees every library-owned workspace (nothing that uses one may be in flight or captured).
@@ -284,12 +286,16 @@ bool caller_workspace_region(int region, size_t bytes, void** out, hipError_t* e
 // bytes in front of the scratch part of a caller-owned workspace (arrival counters, trellis hand-off words)
 size_t caller_workspace_header_bytes();
 int64_t exl3_workspace_words();
+// the prefill GEMM for activations of any type (fp16 / fp32 are rounded to bf16 by its packing pass), and the bytes
+// of packed copy such a launch takes from the workspace
+hipError_t launch_gemm_pc_x(int format, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                            const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s);
+size_t gemm_pc_packed_bytes(int64_t m, int64_t n_out, int64_t n_in, int x_dtype);
 // exact size of the partial sums a split-K launch of the prefill GEMM takes for this shape (0: not split)
 size_t gemm_pc_partials_bytes(int64_t m, int64_t n_out, int64_t n_in);
 // how often the trellis GEMV's last slice polls a missing word before it gives the row up; returns the old value
 int exl3_set_poll_limit(int limit);
 // n fp16 or fp32 values (n a multiple of 8) rounded to bf16
-hipError_t launch_to_bf16(const void* x, int x_dtype, uint16_t* out, int64_t n, hipStream_t s);
 
 // Trellis layer for many activation rows (ttq_exl3_prefill.hip): activations rotated once into a workspace
 // the library keeps per (device, stream), then 64 rows per decoded weight.  y fp32.

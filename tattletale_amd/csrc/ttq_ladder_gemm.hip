@@ -4,7 +4,7 @@
 // Not part of libttq_hip.so.  bench.py --only ladder_gemm builds libttq_ladder.so on demand and times the rungs;
 // a rocprofv3 kernel trace of that command names every rung by its kernel and its ABL template argument.
 //
-// kernel 0: gemm_pcd_kernel (ttq_gemm_pcd.h; activations from global memory straight into the consumers' registers)
+// kernel 0: gemm_pcd_kernel (ttq_gemm_pcd.h; activations from their packed copy straight into the consumers' registers)
 //   ABL 31    barriers, prologue and epilogue only
 //   ABL 4124  consumers alone: A requests, B reads, MFMA (real values put in the W tile once, at the start)
 //   ABL 4104  ... and the W producers' global loads and LDS stores, without the dequantization arithmetic
@@ -20,6 +20,7 @@
 //   ABL 29    X movers alone
 //   ABL 1024  the whole kernel without its barriers
 //   ABL 2048  the whole kernel with X moved by global_load_lds into rings of four stages (+ an L2 prefetch)
+// ttq_ladder_gemm_pack is kernel 0's packing pass on its own.
 #include "ttq_gemm_pcd.h"
 
 namespace {
@@ -29,7 +30,6 @@ hipError_t rung(const uint8_t* wb, const uint16_t* x, void* y, int64_t m, int64_
                 hipStream_t s) {
   using namespace ttq;
   if (KERNEL == 0) return launch_pcd_grid<kQ4_K, 4, 7, false, ABL>(wb, x, y, kBF16, nullptr, 0, m, n_out, n_in, sp, s);
-  if (KERNEL == 2) return launch_pcd_grid<kQ4_K, 2, 7, false, ABL, 8>(wb, x, y, kBF16, nullptr, 0, m, n_out, n_in, sp, s);
   return launch_pc_grid<kQ4_K, 4, 7, false, ABL>(wb, x, y, kBF16, nullptr, 0, m, n_out, n_in, sp, s);
 }
 
@@ -45,14 +45,17 @@ bool args_ok(const void* w, const void* x, const void* y, int64_t m, int64_t n_o
     TTQ_RUNG(0, 3 + EXTRA) TTQ_RUNG(0, 2 + EXTRA) TTQ_RUNG(0, 1024 + EXTRA)                                   \
     TTQ_RUNG(1, 31 + EXTRA) TTQ_RUNG(1, 4126 + EXTRA) TTQ_RUNG(1, 4124 + EXTRA) TTQ_RUNG(1, 0 + EXTRA)        \
     TTQ_RUNG(1, 29 + EXTRA) TTQ_RUNG(1, 1024 + EXTRA) TTQ_RUNG(1, 2048 + EXTRA)                               \
-    TTQ_RUNG(2, 31 + EXTRA) TTQ_RUNG(2, 4124 + EXTRA) TTQ_RUNG(2, 0 + EXTRA) TTQ_RUNG(2, 2 + EXTRA)           \
-    TTQ_RUNG(2, 1024 + EXTRA) TTQ_RUNG(0, 8192 + 4124 + EXTRA) TTQ_RUNG(0, 8192 + EXTRA)                      \
-    TTQ_RUNG(2, 8192 + 4124 + EXTRA) TTQ_RUNG(2, 8192 + EXTRA)                                                \
-    TTQ_RUNG(0, 8192 + 1024 + EXTRA) TTQ_RUNG(0, 8192 + 8 + EXTRA) TTQ_RUNG(0, 8192 + 4 + EXTRA)             \
-    TTQ_RUNG(0, 8192 + 64 + EXTRA) TTQ_RUNG(0, 8192 + 128 + EXTRA)                                            \
     default: return -1;                                                                                       \
   }
 
+extern "C" __attribute__((visibility("default")))
+int ttq_ladder_gemm_pack(const void* x_bf16, void* xp, int64_t m, int64_t n_in, void* stream) {
+  if (!x_bf16 || !xp || m <= 0 || n_in <= 0 || n_in % 256 != 0) return -1;
+  return ttq::launch_pack_activations(x_bf16, ttq::kBF16, static_cast<uint16_t*>(xp), m, n_in,
+                                      static_cast<hipStream_t>(stream)) == hipSuccess ? 0 : -7;
+}
+
+// x_bf16: the activations for kernel 1, their packed copy (ttq_ladder_gemm_pack) for kernel 0
 extern "C" __attribute__((visibility("default")))
 int ttq_ladder_gemm_launch(int kernel, int abl, const void* w, const void* x_bf16, void* y_bf16, int64_t m, int64_t n_out,
                            int64_t n_in, void* stream) {

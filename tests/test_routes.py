@@ -25,8 +25,8 @@ PINNED = [
     ("config 2: Q4_K GEMV 14336x4096 (headline)", Q4_K, 14336, 4096, 1, BF16, F32, 0, "gemv_q4k_stream"),
     ("config 3: Q6_K GEMV 128256x4096 (LM head)", Q6_K, 128256, 4096, 1, BF16, F32, 0, "gemv_q6k_stream"),
     ("config 4: Q4_K GEMM M=64", Q4_K, 14336, 4096, 64, BF16, BF16, 0, "gemm_skinny"),
-    ("config 4: Q4_K GEMM M=512 (headline)", Q4_K, 14336, 4096, 512, BF16, BF16, 0, "gemm_pc"),
-    ("config 4: Q4_K GEMM M=2048", Q4_K, 14336, 4096, 2048, BF16, BF16, 0, "gemm_pc"),
+    ("config 4: Q4_K GEMM M=512 (headline)", Q4_K, 14336, 4096, 512, BF16, BF16, 0, "gemm_pc_packed"),
+    ("config 4: Q4_K GEMM M=2048", Q4_K, 14336, 4096, 2048, BF16, BF16, 0, "gemm_pc_packed"),
     ("config 5: EXL3 3-bit GEMV 4096x4096", EXL3, 4096, 4096, 1, F16, F32, 3, "exl3_gemv_sliced"),
     ("gate||up 28672x4096, decode", Q4_K, 28672, 4096, 1, BF16, F32, 0, "gemv_q4k_stream"),
     ("q / o projection 4096x4096, decode", Q4_K, 4096, 4096, 1, BF16, F32, 0, "gemv_q4k_stream"),
@@ -81,7 +81,10 @@ def test_workspace_size_query_and_argument_checks():
     assert L.ttq_workspace_bytes(C.byref(q), 1, BF16) == 0                       # decode kernels take none
     split = L.ttq_workspace_bytes(C.byref(q), 512, BF16)
     assert split > (4 << 20)                                                     # header + partial sums
-    assert L.ttq_workspace_bytes(C.byref(q), 512, F32) > split                   # + the bf16 copy of the rows
+    small = QLinearStruct(format=Q4_K, n_out=1024, n_in=1024)                    # a short GEMM reads X itself ...
+    ok = QLinearStruct(format=Q4_K, n_out=1024, n_in=1024, precision=_lib.PRECISION_BF16_OK)
+    assert (L.ttq_workspace_bytes(C.byref(ok), 512, F32) >=                      # ... unless its rows must be rounded
+            L.ttq_workspace_bytes(C.byref(small), 512, BF16) + 512 * 1024 * 2)
     assert L.ttq_workspace_bytes(C.byref(q), 0, BF16) == 0
     assert L.ttq_workspace_bytes(None, 1, BF16) == _lib.ERR_NULL
     assert L.ttq_workspace_bytes(C.byref(q), 1, 5) == _lib.ERR_DTYPE
