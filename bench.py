@@ -683,7 +683,10 @@ def main() -> int:
                  (0, 3, "packed X: W producers alone"),
                  (0, 2, "packed X: consumers without A requests + W producers"),
                  (0, 1024, "packed X: whole kernel without barriers (roles free-running)"),
+                 (2, 0, "packed X: whole kernel as a persistent workgroup per CU, LDS counters for barriers"),
                  (-1, 0, "packed X: the packing pass alone"),
+                 (-2, 0, "for scale: the vendor library's dense bf16 GEMM (torch F.linear), random bf16 W, same x"),
+                 (-3, 0, "for scale: the same with W = 0 and x = 0 (the matrix cores clock higher on zeros)"),
                  (1, 31, "LDS-staged X: barriers, prologue, epilogue only"),
                  (1, 4126, "LDS-staged X: consumers alone (real values in LDS)"),
                  (1, 4124, "LDS-staged X: consumers + X movers"),
@@ -696,9 +699,13 @@ def main() -> int:
         packed = random_packed(rng, F.Q4_K, n_out, n_in)
         ncopies = rotated(packed.nbytes)
         ws = [to_dev(packed) for _ in range(ncopies)]
+        w_dense = [torch.randn((n_out, n_in), device=dev).mul_(0.02).to(torch.bfloat16)
+                   for _ in range(rotated(n_out * n_in * 2))]
+        w_zero = torch.zeros((n_out, n_in), dtype=torch.bfloat16, device=dev)
         out = {}
         for m in ms_:
             x = torch.randn((m, n_in), device=dev).to(torch.bfloat16)
+            x_zero = torch.zeros_like(x)
             y = torch.empty((m, n_out), dtype=torch.bfloat16, device=dev)
             flop = 2.0 * m * n_out * n_in
             rows = []
@@ -708,11 +715,17 @@ def main() -> int:
             for kern, abl, what in rungs:
                 def step(i, kern=kern, abl=abl):
                     sh = torch.cuda.current_stream(dev).cuda_stream
-                    if kern < 0:
+                    if kern == -2:
+                        torch.matmul(x, w_dense[i % len(w_dense)].t(), out=y)
+                        rc = 0
+                    elif kern == -3:
+                        torch.matmul(x_zero, w_zero.t(), out=y)
+                        rc = 0
+                    elif kern < 0:
                         rc = LAD.ttq_ladder_gemm_pack(x.data_ptr(), xp.data_ptr(), m, n_in, sh)
                     else:
                         rc = LAD.ttq_ladder_gemm_launch(kern, abl, ws[i % ncopies].data_ptr(),
-                                                        (xp if kern == 0 else x).data_ptr(), y.data_ptr(), m, n_out, n_in, sh)
+                                                        (x if kern == 1 else xp).data_ptr(), y.data_ptr(), m, n_out, n_in, sh)
                     if rc != 0:
                         raise RuntimeError("ttq_ladder_gemm_launch(%d, %d) returned %d" % (kern, abl, rc))
                 t = time_steps(step, max(20, steps // (10 if m <= 512 else 40)), max(3, warmup // 10))
@@ -720,8 +733,17 @@ def main() -> int:
                              "us_min": t["ms_min"] * 1e3, "us_max": t["ms_max"] * 1e3,
                              "mfma_frac_if_full_flops": flop / (t["ms"] * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS})
                 log("[ladder gemm m=%d] k%d abl %-5d %-72s %8.2f us" % (m, kern, abl, what, t["ms"] * 1e3))
-            out["m%d" % m] = {"n_out": n_out, "n_in": n_in, "flop": flop, "rungs": rows}
-        del ws
+            # the persistent kernel is measured only: check here that it still computes what the product kernel does
+            sh = torch.cuda.current_stream(dev).cuda_stream
+            y2 = torch.empty_like(y)
+            rc0 = LAD.ttq_ladder_gemm_launch(0, 0, ws[0].data_ptr(), xp.data_ptr(), y.data_ptr(), m, n_out, n_in, sh)
+            rc2 = LAD.ttq_ladder_gemm_launch(2, 0, ws[0].data_ptr(), xp.data_ptr(), y2.data_ptr(), m, n_out, n_in, sh)
+            torch.cuda.synchronize(dev)
+            same = rc0 == 0 and rc2 == 0 and bool(torch.equal(y, y2))
+            log("[ladder gemm m=%d] persistent kernel output identical to the product kernel's: %s" % (m, same))
+            out["m%d" % m] = {"n_out": n_out, "n_in": n_in, "flop": flop, "rungs": rows,
+                              "persistent_kernel_matches_product_kernel": same}
+        del ws, w_dense, w_zero
         torch.cuda.empty_cache()
         return out
 

@@ -439,6 +439,48 @@ __device__ __forceinline__ void pc_epilogue(f32x4_t (&acc)[MB][NJ], const PcEpi&
   }
 }
 
+// 64 k of a producer thread's row (chunk C of the 256 k in `r`), dequantized, rounded to bf16 and stored as B
+// fragments into W stage `buf` of the tile at LDS address sw_addr.  whalf / wj / wn: the thread's half of every
+// 32-byte chunk, its column block and its column inside the block.
+template <int NJ, int FMT, int ABL, int C>
+__device__ __forceinline__ void pc_dequant_to_lds(const typename WFmt<FMT>::Raw& r, int buf, int whalf, int wj, int wn,
+                                                  uint32_t sw_addr) {
+  using WF = WFmt<FMT>;
+  using WRaw = typename WF::Raw;
+  constexpr int kWUnits = 2 * NJ * 64;
+  constexpr int c = C;
+  uint32_t lo[8], hi[8];
+  if constexpr ((ABL & 8) != 0) {
+    // ladder: the raw words instead of the dequantized ones
+    const uint32_t* raw = reinterpret_cast<const uint32_t*>(&r);
+#pragma unroll
+    for (int i = 0; i < 8; i++) { lo[i] = raw[(4 * c + i) % (sizeof(WRaw) / 4)]; hi[i] = raw[(4 * c + i + 4) % (sizeof(WRaw) / 4)]; }
+  } else {
+    WF::template dequant<c>(r, whalf, lo, hi);
+  }
+  if constexpr ((ABL & 4) != 0) {
+    // ladder: no LDS stores; keep the values alive
+    uint32_t keep = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) keep ^= lo[i] ^ hi[i];
+    asm volatile("" : : "v"(keep));
+  } else if constexpr (WF::kWholeKsub) {
+    // k = 32*half + e -> ksub `half`, groups 0..3
+    const uint32_t base = sw_addr + (uint32_t)(buf * kWUnits + whalf * (NJ * 64) + wj * 64 + wn) * 16u;
+    lds_store16(base, lo[0], lo[1], lo[2], lo[3]);
+    lds_store16(base + 256u, lo[4], lo[5], lo[6], lo[7]);
+    lds_store16(base + 512u, hi[0], hi[1], hi[2], hi[3]);
+    lds_store16(base + 768u, hi[4], hi[5], hi[6], hi[7]);
+  } else {
+    // k = 16*half + e  -> ksub 0, groups 2*half and 2*half+1; k = 32 + 16*half + e: ksub 1
+    const uint32_t base = sw_addr + (uint32_t)(buf * kWUnits + (wj * 4 + 2 * whalf) * 16 + wn) * 16u;
+    lds_store16(base, lo[0], lo[1], lo[2], lo[3]);
+    lds_store16(base + 256u, lo[4], lo[5], lo[6], lo[7]);
+    lds_store16(base + NJ * 1024u, hi[0], hi[1], hi[2], hi[3]);
+    lds_store16(base + NJ * 1024u + 256u, hi[4], hi[5], hi[6], hi[7]);
+  }
+}
+
 // The W producer role (wavefronts 4-7 of either kernel): thread pt (0..255) owns one row of the tile and half of
 // every 32-byte chunk; it loads the packed blocks, dequantizes 64 k per step and writes the B fragments into the
 // double-buffered W tile at LDS address sw_addr, keeping the step barrier `bar`.
@@ -468,38 +510,8 @@ __device__ __forceinline__ void pc_produce_w(const uint8_t* __restrict__ w, int 
     WF::load(dst, wptr + WF::kUnitBytes * (int64_t)min(b, nblocks - 1), whalf);
   };
   auto dequant_to_lds = [&](const WRaw& r, auto cc, int buf) {
-    constexpr int c = decltype(cc)::value;
     if (widle) return;
-    uint32_t lo[8], hi[8];
-    if constexpr ((ABL & 8) != 0) {
-      // ladder: the raw words instead of the dequantized ones
-      const uint32_t* raw = reinterpret_cast<const uint32_t*>(&r);
-#pragma unroll
-      for (int i = 0; i < 8; i++) { lo[i] = raw[(4 * c + i) % (sizeof(WRaw) / 4)]; hi[i] = raw[(4 * c + i + 4) % (sizeof(WRaw) / 4)]; }
-    } else {
-      WF::template dequant<c>(r, whalf, lo, hi);
-    }
-    if constexpr ((ABL & 4) != 0) {
-      // ladder: no LDS stores; keep the values alive
-      uint32_t keep = 0;
-#pragma unroll
-      for (int i = 0; i < 8; i++) keep ^= lo[i] ^ hi[i];
-      asm volatile("" : : "v"(keep));
-    } else if constexpr (WF::kWholeKsub) {
-      // k = 32*half + e -> ksub `half`, groups 0..3
-      const uint32_t base = sw_addr + (uint32_t)(buf * kWUnits + whalf * (NJ * 64) + wj * 64 + wn) * 16u;
-      lds_store16(base, lo[0], lo[1], lo[2], lo[3]);
-      lds_store16(base + 256u, lo[4], lo[5], lo[6], lo[7]);
-      lds_store16(base + 512u, hi[0], hi[1], hi[2], hi[3]);
-      lds_store16(base + 768u, hi[4], hi[5], hi[6], hi[7]);
-    } else {
-      // k = 16*half + e  -> ksub 0, groups 2*half and 2*half+1; k = 32 + 16*half + e: ksub 1
-      const uint32_t base = sw_addr + (uint32_t)(buf * kWUnits + (wj * 4 + 2 * whalf) * 16 + wn) * 16u;
-      lds_store16(base, lo[0], lo[1], lo[2], lo[3]);
-      lds_store16(base + 256u, lo[4], lo[5], lo[6], lo[7]);
-      lds_store16(base + NJ * 1024u, hi[0], hi[1], hi[2], hi[3]);
-      lds_store16(base + NJ * 1024u + 256u, hi[4], hi[5], hi[6], hi[7]);
-    }
+    pc_dequant_to_lds<NJ, FMT, ABL, decltype(cc)::value>(r, buf, whalf, wj, wn, sw_addr);
   };
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;

@@ -20,8 +20,11 @@
 //   ABL 29    X movers alone
 //   ABL 1024  the whole kernel without its barriers
 //   ABL 2048  the whole kernel with X moved by global_load_lds into rings of four stages (+ an L2 prefetch)
-// ttq_ladder_gemm_pack is kernel 0's packing pass on its own.
-#include "ttq_gemm_pcd.h"
+// kernel 2: gemm_pcr_kernel (ttq_gemm_pcr.h; kernel 0 as a persistent workgroup per compute unit, a ring of W stages
+//   with counters in LDS in place of the step barrier)
+//   ABL 0     the whole kernel
+// ttq_ladder_gemm_pack is the packing pass of kernels 0 and 2 on its own.
+#include "ttq_gemm_pcr.h"
 
 namespace {
 
@@ -29,6 +32,11 @@ template <int KERNEL, int ABL>
 hipError_t rung(const uint8_t* wb, const uint16_t* x, void* y, int64_t m, int64_t n_out, int64_t n_in, ttq::PcSplit sp,
                 hipStream_t s) {
   using namespace ttq;
+  if (KERNEL == 2) {
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    return launch_pcr_grid<kQ4_K, 4, 7, false>(wb, x, y, kBF16, nullptr, 0, m, n_out, n_in, cus, s);
+  }
   if (KERNEL == 0) return launch_pcd_grid<kQ4_K, 4, 7, false, ABL>(wb, x, y, kBF16, nullptr, 0, m, n_out, n_in, sp, s);
   return launch_pc_grid<kQ4_K, 4, 7, false, ABL>(wb, x, y, kBF16, nullptr, 0, m, n_out, n_in, sp, s);
 }
@@ -55,7 +63,7 @@ int ttq_ladder_gemm_pack(const void* x_bf16, void* xp, int64_t m, int64_t n_in, 
                                       static_cast<hipStream_t>(stream)) == hipSuccess ? 0 : -7;
 }
 
-// x_bf16: the activations for kernel 1, their packed copy (ttq_ladder_gemm_pack) for kernel 0
+// x_bf16: the activations for kernel 1, their packed copy (ttq_ladder_gemm_pack) for kernels 0 and 2
 extern "C" __attribute__((visibility("default")))
 int ttq_ladder_gemm_launch(int kernel, int abl, const void* w, const void* x_bf16, void* y_bf16, int64_t m, int64_t n_out,
                            int64_t n_in, void* stream) {
@@ -67,6 +75,11 @@ int ttq_ladder_gemm_launch(int kernel, int abl, const void* w, const void* x_bf1
     e = rung<K, (A)>(static_cast<const uint8_t*>(w), static_cast<const uint16_t*>(x_bf16), y_bf16, m, n_out, n_in, sp, \
                      static_cast<hipStream_t>(stream));                                                                \
     break;
+  if (kernel == 2 && abl == 0) {
+    e = rung<2, 0>(static_cast<const uint8_t*>(w), static_cast<const uint16_t*>(x_bf16), y_bf16, m, n_out, n_in, sp,
+                   static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? 0 : -7;
+  }
   TTQ_RUNGS(0)
 #undef TTQ_RUNG
   return e == hipSuccess ? 0 : -7;
