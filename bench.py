@@ -80,7 +80,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--replays", type=int, default=7, help="timed replays of the K-step graph (median reported)")
     ap.add_argument("--only", default=None, help="run a single configuration (name in tattletale_amd.configs), "
-                                                 "or one of: ladder, widened, q4_k_gate_up_silu_gemv, dense_reference")
+                                                 "or one of: ladder, ladder_<n_out>x<n_in>, ladder_q6k, ladder_gemm, "
+                                                 "ladder_gemm_m<rows>, widened, q4_k_gate_up_silu_gemv, dense_reference")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-extra", action="store_true", help="headline workload only")
     ap.add_argument("--eager", action="store_true", help="always time plain launches")
@@ -749,6 +750,9 @@ def main() -> int:
 
     if args.only == "ladder_gemm":
         print(json.dumps(run_ladder_gemm(args.steps, args.warmup)), flush=True)
+        return 0
+    if args.only and args.only.startswith("ladder_gemm_m"):      # one row count (for a kernel trace)
+        print(json.dumps(run_ladder_gemm(args.steps, args.warmup, ms_=(int(args.only[len("ladder_gemm_m"):]),))), flush=True)
         return 0
     if args.only == "ladder_q6k":
         print(json.dumps(run_ladder_q6k(args.steps, args.warmup)), flush=True)
