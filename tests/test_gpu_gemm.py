@@ -443,3 +443,23 @@ def test_forward_default_precision_keeps_fp32_activations_in_the_decode_class(fm
     assert rel_l2(y, want) <= 1e-3
     for i in (0, 1, 127, 254, m - 1):
         assert rel_l2(y[i], want[i]) <= 1e-3, i
+
+
+@pytest.mark.parametrize("xk", ["f16", "bf16"])
+def test_packed_activations_in_chunks_of_8192_rows(xk):
+    """More rows than one packed copy holds (8192): the operator packs and multiplies chunk after chunk through the
+    same workspace.  Rows on both sides of the seam and in the short last chunk against the oracle; fp16 rows
+    reach the path through a BF16_OK layer, bf16 rows by the cost estimate of a long launch."""
+    m, n_out, n_in = 8192 + 130, (512 if xk == "f16" else 14336), (512 if xk == "f16" else 1024)
+    p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=955)
+    what = oracle.dequant(F.Q4_K, p, n_out, n_in)
+    xd, xf = x_to_dev(Q.fill_normal(956, 1, 1.0, m * n_in).reshape(m, n_in) * np.float32(0.05), xk)
+    layer = QuantLinear.init(packed_to_dev(p), F.Q4_K, n_in, n_out,
+                             precision=F.PRECISION_BF16_OK if xk == "f16" else F.PRECISION_AUTO)
+    assert layer.route(m, xd.dtype, torch.float32) in ("gemm_pc_bf16_copy", "gemm_pc_packed")
+    y = layer.forward(xd, out_dtype=torch.float32).cpu().numpy()
+    rows = [0, 1, 4095, 8190, 8191, 8192, 8193, 8192 + 64, m - 2, m - 1]
+    want = oracle.linear_f64(what, xf[rows])
+    for j, i in enumerate(rows):
+        assert rel_l2(y[i], want[j]) <= TOL, i
+    assert np.isfinite(y).all()
