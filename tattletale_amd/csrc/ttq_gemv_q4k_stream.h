@@ -46,6 +46,15 @@ constexpr int kStUpFront = 6;                             // requests before the
 // the landed super-blocks among all 8 wavefronts after a wait-for-all and a barrier was measured too: slower
 // (4.54 us; 6144x4096 4.77 -> 6.03 us), the pipelined consumption by the owners wins.
 constexpr int kStUpFrontFew = 16;
+// With at most two blocks per workgroup (one row group of rows of 2048 or 4096 values: the attention output
+// projection 4096x4096) four wavefronts share a block instead: wavefront 4 b + p takes super-blocks 2 p and 2 p + 1 of
+// block b.  The block lands in one buffer (that of wavefront 4 b), every line requested once: wavefront p asks for
+// lines 2 p + 1 and 2 p + 2 of both row halves (p = 0 also for line 0), multiplies super-block 2 p + 1, which lies in
+// its own lines, as soon as they have landed, and super-block 2 p, which begins in its neighbour's last line, after
+// a barrier that every wavefront reaches with its own lines landed.  After a stream of little more than a
+// microsecond eight wavefronts multiply two super-blocks each instead of two multiplying eight.  The raw activations
+// land in the buffer of wavefront 1, which holds no block in this form.  (kStQuad as the UP argument.)
+constexpr int kStQuad = -1;
 constexpr int kStMaxSb = 16;                              // n_in <= 4096: one staging pass, 8 KiB table
 constexpr int kStMaxBlocks = 80;                          // blocks of a workgroup (their row sums wait in LDS)
 
@@ -116,7 +125,9 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   // request will: that one is made long after the activations have been read back.
   const int k0 = 8 * tid;
   const bool xok = k0 < n_in;                             // whole wavefronts: n_in is a multiple of 512
-  uint8_t* xland = mybuf + kStHalfBytes + (kStLines - 1) * 1024;
+  constexpr bool kQuad = UP == kStQuad;
+  static_assert(!kQuad || (!FUSE && !NORM), "four wavefronts per block: the plain form only");
+  uint8_t* xland = kQuad ? wbuf + kStBlockBytes + wave * 1024 : mybuf + kStHalfBytes + (kStLines - 1) * 1024;
   if (xok) __builtin_amdgcn_global_load_lds((st_gptr_t)(xm + k0), (st_lptr_t)xland, 16, 0, 0);
   uint8_t* rland = mybuf + (kStLines - 1) * 1024;                      // request 16's slot
   uint8_t* gland = mybuf + kStHalfBytes + (kStLines - 2) * 1024;       // request 15's slot
@@ -152,25 +163,37 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
       lane_off[o] = (uint32_t)row * rb + (uint32_t)(ks * kStSegBytes) + (uint32_t)(((lane & 7) ^ ((row16 >> 1) & 7)) * 16);
     }
   };
+  uint8_t* blockbuf = kQuad ? wbuf + (wave >> 2) * (4 * kStBlockBytes) : mybuf;
   auto request = [&](int i) {
     const int line = i >> 1, o = i & 1;
     // non-temporal: every line is used once
     __builtin_amdgcn_global_load_lds((st_gptr_t)(w + (size_t)(lane_off[o] + (uint32_t)(line * 128))),
-                                     (st_lptr_t)(mybuf + o * kStHalfBytes + line * 1024), 16, 0, 2);
+                                     (st_lptr_t)(blockbuf + o * kStHalfBytes + line * 1024), 16, 0, 2);
   };
-  int blk = wave;
+  int blk = kQuad ? wave >> 2 : wave;
+  const int quad_p = wave & 3;                            // (kQuad) which quarter of the block
   const bool have_block = blk < nblocks;
   if (have_block) {
     set_block(blk);
+    if constexpr (kQuad) {
+      if (quad_p == 0) {
+        request(0);
+        request(1);
+      }
 #pragma unroll
-    for (int i = 0; i < UP; i++) request(i);
+      for (int i = 2; i < 6; i++) request(4 * quad_p + i);
+    } else {
+#pragma unroll
+      for (int i = 0; i < UP; i++) request(i);
+    }
   }
 
   // ---- the raw activations back into registers
   float xf[8];
   if (xok) {
-    if (have_block) st_wait_vmcnt<UP>();
-    else st_wait_vmcnt<0>();
+    if (!have_block) st_wait_vmcnt<0>();
+    else if (kQuad && quad_p == 0) st_wait_vmcnt<6>();
+    else st_wait_vmcnt<(kQuad ? 4 : UP)>();
     const st_u32x4 r = st_read1((uint32_t)(size_t)(st_lptr_t)(xland) + (uint32_t)(lane * 16));
     widen8<XT>(make_uint4(r[0], r[1], r[2], r[3]), xf);
   }
@@ -281,7 +304,7 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   // operand reads: row n of the block, chunk 9 s + c of its 72, c = 0 (header), 1 + g, 5 + g:
   // line s + (s + c) / 8, slot ((s + c) % 8) ^ key
   const uint32_t key = (uint32_t)(n >> 1) & 7u;
-  const uint32_t rowbase = (uint32_t)(size_t)(st_lptr_t)(mybuf) + (uint32_t)((n >> 3) * kStHalfBytes + (n & 7) * 128);
+  const uint32_t rowbase = (uint32_t)(size_t)(st_lptr_t)(blockbuf) + (uint32_t)((n >> 3) * kStHalfBytes + (n & 7) * 128);
 
   st_barrier();                         // the plane table is complete
 
@@ -292,7 +315,7 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   uint32_t a_addr[4], tab_addr = tab_addr0;
   auto topup = [&](auto sc) {
     constexpr int s = decltype(sc)::value;
-    if constexpr (UP + 2 * s < kStBlockRequests) {
+    if constexpr (!kQuad && UP + 2 * s < kStBlockRequests) {
       request(UP + 2 * s);
       request(UP + 2 * s + 1);
     }
@@ -300,8 +323,12 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
   auto issue = [&](auto sc, Regs& r) {
     constexpr int s = decltype(sc)::value;
     // super-block s needs requests 0 .. 2 s + 3 (its two top-up requests have been made by now)
-    constexpr int kIssued = UP + 2 * (s + 1) < kStBlockRequests ? UP + 2 * (s + 1) : kStBlockRequests;
-    st_wait_vmcnt<kIssued - (2 * s + 4)>();
+    if constexpr (kQuad) {
+      // (the caller has waited: its own lines have landed, and after the barrier everybody's)
+    } else {
+      constexpr int kIssued = UP + 2 * (s + 1) < kStBlockRequests ? UP + 2 * (s + 1) : kStBlockRequests;
+      st_wait_vmcnt<kIssued - (2 * s + 4)>();
+    }
     const uint32_t ta = tab_addr;
     // (s + c) ^ key, c = 1 + g or 5 + g: bits 0-2 are the slot, bit 3 says "next line"
     const uint32_t e0 = ((1u + (uint32_t)g + (uint32_t)s) ^ key), e1 = ((5u + (uint32_t)g + (uint32_t)s) ^ key);
@@ -372,6 +399,48 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
     // pins the arithmetic here: left alone the compiler moves it behind every wait of the block
     asm volatile("" : "+v"(acc));
   };
+
+  // ---- four wavefronts per block: this one's two super-blocks
+  if constexpr (kQuad) {
+    if (have_block) {
+      const int ks = blk & ((1 << nks_log2) - 1);
+#pragma unroll
+      for (int q = 0; q < 4; q++) a_addr[q] = a_addr0[q] + (uint32_t)ks * (kStBlockSb * a_step[q]);
+      tab_addr = tab_addr0 + (uint32_t)(ks * kStBlockSb * 128);
+      Regs ra, rb2;
+      st_wait_vmcnt<0>();                  // this wavefront's lines
+      auto two = [&](auto pc) {
+        constexpr int p2 = 2 * decltype(pc)::value;
+        issue(std::integral_constant<int, p2 + 1>{}, ra);
+        st_barrier();                      // every wavefront's lines (and ra's reads)
+        issue(std::integral_constant<int, p2>{}, rb2);
+        settle(std::integral_constant<int, 9>{}, ra);
+        compute(ra);
+        settle(std::integral_constant<int, 0>{}, rb2);
+        compute(rb2);
+      };
+      switch (quad_p) {
+        case 0: two(std::integral_constant<int, 0>{}); break;
+        case 1: two(std::integral_constant<int, 1>{}); break;
+        case 2: two(std::integral_constant<int, 2>{}); break;
+        default: two(std::integral_constant<int, 3>{}); break;
+      }
+      acc = add_xor16(acc);
+      acc = add_xor32(acc);
+      if (lane < 16) part[wave][lane] = acc;
+    } else {
+      st_barrier();
+    }
+    __syncthreads();
+    // one row group: its (block, quarter) sums in order
+    if (tid < 16) {
+      float v = 0.f;
+      for (int k = 0; k < 4 * nblocks; k++) v += part[k][tid];
+      const int row = wg_row0 + tid;
+      if (row < wg_row_end) YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
+    }
+    return;
+  }
 
   // ---- the wavefront's blocks: wave, wave + 8, ...  A block starts with nothing outstanding.
   auto run_block = [&](const int blk) {
@@ -466,6 +535,12 @@ inline hipError_t st_launch_xy(const void* w, const void* x, void* y, const void
                        static_cast<YT*>(y), bias, bias_dtype, (int)n_out, (int)(n_in / 256), rows_per_wg, na);
   };
   // (the normalizing form keeps three request slots free for x, residual and gamma)
+  if constexpr (!FUSE && !NORM) {
+    if (blocks <= 2 && rows_per_wg <= 16) {
+      go(gemv_q4k_stream_kernel<XT, YT, STAGE, false, kStQuad, false>);
+      return hipGetLastError();
+    }
+  }
   if (blocks <= 2 && !NORM) go(gemv_q4k_stream_kernel<XT, YT, STAGE, FUSE, NORM ? 12 : kStUpFrontFew, NORM>);
   else if (blocks <= 4) go(gemv_q4k_stream_kernel<XT, YT, STAGE, FUSE, 12, NORM>);
   else go(gemv_q4k_stream_kernel<XT, YT, STAGE, FUSE, kStUpFront, NORM>);
