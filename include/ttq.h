@@ -263,11 +263,13 @@ TTQ_API int ttq_gemm_q8_0_ws(const void* w, const uint16_t* x_bf16, uint16_t* y_
 /* The operator for a trellis-coded weight and many activation rows (prefill: seq_len > 1 at every
  * projection, attn.nim:154-156): y (m, n_out) fp32 = svh o H( T * H(suh o x) ) for x (m, n_in) of any
  * dtype.  The activations are rotated once and rounded to fp16 (rel-L2 <= 2e-2 class, about 3e-4 in
- * practice); every weight is decoded once per 64 rows.  The rotated activations live in a workspace
+ * practice); every weight is decoded once per 128 rows (tiled GEMM, split along K while compute
+ * units are free).  The rotated activations and the partial sums of a split launch live in a workspace
  * the library allocates per (device, stream) on first use and grows on demand (up to 4096 rows of
  * n_in fp16 values), so the first call, and a call with more rows than any before, must not happen
- * under graph capture.  ttq_linear_forward takes this path by itself when m is large enough to fill
- * the GPU with 64-row workgroups and the layer does not ask for TTQ_PRECISION_F32_SCALES. */
+ * under graph capture (ttq_gemm_exl3_ws has no such limit).  ttq_linear_forward takes this path by
+ * itself from 16 to 48 rows on, depending on the matrix, unless the layer asks for
+ * TTQ_PRECISION_F32_SCALES. */
 TTQ_API int ttq_gemm_exl3(const uint16_t* trellis, const uint16_t* suh_f16, const uint16_t* svh_f16,
                   const void* x, int x_dtype, float* y, int64_t m, int64_t n_out, int64_t n_in,
                   int bits, int codebook, void* stream);

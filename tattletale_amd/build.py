@@ -39,6 +39,7 @@ SOURCES = [
     "ttq_exl3.hip",
     "ttq_exl3_mfma.hip",
     "ttq_exl3_prefill.hip",
+    "ttq_gemm_exl3_pc.hip",
     "ttq_activations.hip",
     "ttq_workspace.hip",
     "ttq_host.cpp",

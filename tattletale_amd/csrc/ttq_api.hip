@@ -555,8 +555,9 @@ int64_t ttq_workspace_bytes(const ttq_qlinear* layer, int64_t m, int x_dtype) {
   const int64_t header = (int64_t)ttq::caller_workspace_header_bytes();
   constexpr int64_t kExl3Rows = 4096, kGemmRows = 8192;   // rows whose rotated / packed copy is in the workspace at a time
   if (layer->format == TTQ_EXL3) {              // hand-off words; the rotated activations of the many-row form
-    const int64_t block_rows = m < kExl3Rows ? m : kExl3Rows;
-    return header + ((block_rows * n_in * 2 + 255) & ~(int64_t)255);
+    const int64_t block_rows = ((m < kExl3Rows ? m : kExl3Rows) + 15) / 16 * 16;   // whole blocks of 16 rows
+    const int64_t partials = (int64_t)ttq::gemm_exl3_partials_bytes(m, n_out, n_in);
+    return header + ((block_rows * n_in * 2 + 255) & ~(int64_t)255) + ((partials + 255) & ~(int64_t)255);
   }
   if (m < 5) return 0;                          // the decode kernels take no workspace
   // the packed bf16 copy of the activations where the prefill GEMM wants one, then the partial sums of a launch

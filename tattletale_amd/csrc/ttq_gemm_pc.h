@@ -234,13 +234,6 @@ template <> struct WFmt<kQ8_0> {
 
 // Split along K: copies of the tile grid, where the copies of a tile leave their partial sums, and the arrival
 // counters (zero between launches).
-struct PcSplit {
-  int splits;          // 1: none
-  int tile_wgs;        // workgroups of one copy of the tile grid
-  float* partials;
-  uint32_t* counters;
-};
-constexpr int kPcMaxCounters = 16384;     // (tile, consumer) pairs a split launch may have
 
 // The same GEMM over a copy of the activations in fragment order (ttq_gemm_pcd.h, instantiated in ttq_gemm_pcd.hip):
 // tile = index into launch_gemm_pc's table of tile shapes.
@@ -260,9 +253,12 @@ struct PcEpi {
   int y_dtype;
   const void* bias;
   int bias_dtype, m, n_out, n0, m0;
+  const uint16_t* col_scale = nullptr;   // (ROT) fp16 scale per output column, applied after the rotation
 };
 
-template <int NJ, int MB, bool FUSE, int NC = 4>    // NC = consumer wavefronts per workgroup
+// ROT (tiles of 128 columns = one Hadamard group of output channels; the trellis layer): the 128 sums of every row
+// are rotated (Walsh-Hadamard butterfly, 1/sqrt(128)) and scaled per column before bias and store.
+template <int NJ, int MB, bool FUSE, int NC = 4, bool ROT = false>    // NC = consumer wavefronts per workgroup
 __device__ __forceinline__ void pc_epilogue(f32x4_t (&acc)[MB][NJ], const PcEpi& e) {
   constexpr int BN = NJ * 16;
   constexpr int BO = FUSE ? BN / 2 : BN;     // outputs per tile
@@ -328,6 +324,41 @@ __device__ __forceinline__ void pc_epilogue(f32x4_t (&acc)[MB][NJ], const PcEpi&
 
   // ---- epilogue: lane holds Y[m0 + 16i + 4*(lane/16) + r][n0 + 16j + lane%16], r = 0..3
   const int cn = lane & 15, rb4 = (lane >> 4) * 4;
+  if constexpr (ROT) {
+    static_assert(NJ == 8 && !FUSE, "one Hadamard group of 128 columns per tile");
+    // column 16 j + cn: bits 0-3 of the column index live in the lane (DPP moves inside a row of 16 lanes), bits 4-6
+    // in the register index j
+    float cs[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; j++) cs[j] = 0.08838834764831845f * f16_bits_to_f32(e.col_scale[n0 + 16 * j + cn]);
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        float v[NJ];
+#pragma unroll
+        for (int j = 0; j < NJ; j++) v[j] = acc[i][j][r];
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+          float o;
+          o = lane_xor<1>(v[j], lane); v[j] = (cn & 1) ? o - v[j] : v[j] + o;
+          o = lane_xor<2>(v[j], lane); v[j] = (cn & 2) ? o - v[j] : v[j] + o;
+          o = lane_xor<4>(v[j], lane); v[j] = (cn & 4) ? o - v[j] : v[j] + o;
+          o = lane_xor<8>(v[j], lane); v[j] = (cn & 8) ? o - v[j] : v[j] + o;
+        }
+#pragma unroll
+        for (int d = 1; d < NJ; d <<= 1)
+#pragma unroll
+          for (int j = 0; j < NJ; j++)
+            if ((j & d) == 0) {
+              const float a = v[j], b = v[j | d];
+              v[j] = a + b;
+              v[j | d] = a - b;
+            }
+#pragma unroll
+        for (int j = 0; j < NJ; j++) acc[i][j][r] = v[j] * cs[j];
+      }
+  }
   if constexpr (FUSE) {
     // gate in lanes cn < 8, the matching up eight lanes further; silu(g) * u in fp32, one rounding.
     const bool full = y_dtype == kBF16 && n0 + BO <= n_out && (n_out & 7) == 0;
@@ -388,7 +419,7 @@ __device__ __forceinline__ void pc_epilogue(f32x4_t (&acc)[MB][NJ], const PcEpi&
     }
     return;
   }
-  if (y_dtype == kBF16 && n0 + BN <= n_out && (n_out & 7) == 0) {
+  if ((y_dtype == kBF16 || (ROT && y_dtype == kF16)) && n0 + BN <= n_out && (n_out & 7) == 0) {
     // Full tile of bf16: transpose through the wavefront's own (now idle) X ring, so that global
     // memory sees 16-byte stores along the rows instead of 2-byte ones.  Row stride 240 bytes.
     constexpr int kRowBytes = BN * 2 + 16;
@@ -401,7 +432,7 @@ __device__ __forceinline__ void pc_epilogue(f32x4_t (&acc)[MB][NJ], const PcEpi&
 #pragma unroll
         for (int r = 0; r < 4; r++)
           *reinterpret_cast<uint16_t*>(stg + (16 * i + rb4 + r) * kRowBytes + (16 * j + cn) * 2) =
-              f32_to_bf16_bits(acc[i][j][r] + bv);
+              (ROT && y_dtype == kF16) ? f32_to_f16_bits(acc[i][j][r] + bv) : f32_to_bf16_bits(acc[i][j][r] + bv);
     }
     // same wavefront wrote and reads: LDS keeps program order, no barrier needed
     uint8_t* yb = static_cast<uint8_t*>(yv);
@@ -417,6 +448,41 @@ __device__ __forceinline__ void pc_epilogue(f32x4_t (&acc)[MB][NJ], const PcEpi&
         *reinterpret_cast<uint4*>(yb + ((int64_t)(m0 + row) * n_out + n0 + ch * 8) * 2) = v;
     }
     return;
+  }
+  if constexpr (ROT) {
+    if (y_dtype == kF32 && n0 + BN <= n_out && (n_out & 3) == 0) {
+      // Full tile of fp32: the same transpose, half of the columns at a time (64 floats and the padding are the 272
+      // bytes of a staged row), so that global memory sees 16-byte stores along the rows.
+      static_assert(NJ % 2 == 0, "two halves of whole column blocks");
+      constexpr int kRowBytes = BN * 2 + 16;
+      uint8_t* stg = e.stg;
+      uint8_t* yb = static_cast<uint8_t*>(yv);
+      constexpr int kChunks = BN / 8;      // 16-byte chunks per half row
+      constexpr int kSlots = 16 * MB * kChunks;
+#pragma unroll
+      for (int p = 0; p < 2; p++) {
+#pragma unroll
+        for (int jj = 0; jj < NJ / 2; jj++) {
+          const int j = p * (NJ / 2) + jj;
+          const float bv = load_bias(bias, bias_dtype, n0 + 16 * j + cn);
+#pragma unroll
+          for (int i = 0; i < MB; i++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+              *reinterpret_cast<float*>(stg + (16 * i + rb4 + r) * kRowBytes + (16 * jj + cn) * 4) = acc[i][j][r] + bv;
+        }
+#pragma unroll
+        for (int t = 0; t < (kSlots + 63) / 64; t++) {
+          const int c = t * 64 + lane;
+          const int row = c / kChunks, ch = c - row * kChunks;
+          if (c >= kSlots) break;
+          const uint4 v = *reinterpret_cast<const uint4*>(stg + row * kRowBytes + ch * 16);
+          if (m0 + row < m)
+            *reinterpret_cast<uint4*>(yb + ((int64_t)(m0 + row) * n_out + n0 + p * (BN / 2) + ch * 4) * 4) = v;
+        }
+      }
+      return;
+    }
   }
 #pragma unroll
   for (int j = 0; j < NJ; j++) {

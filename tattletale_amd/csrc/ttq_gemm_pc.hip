@@ -127,7 +127,9 @@ template <int FMT, bool FUSE>
 static hipError_t launch_pc_fmt(const uint8_t* wb, const void* x, int x_dtype, void* y, int y_dtype, const void* bias,
                                 int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, bool force_packed, hipStream_t s) {
   const PcChoice whole = pc_choose(m, n_out, n_in, FUSE);
-  if (!force_packed && !pc_use_packed(whole, m, n_in))
+  // (the fused gate||up form keeps the LDS-staged kernel: beside the packed kernel's three steps of A fragments its
+  // epilogue does not fit the registers, and a kernel that requests registers asynchronously must never spill them)
+  if (FUSE || (!force_packed && !pc_use_packed(whole, m, n_in)))
     return launch_pc_rows<FMT, FUSE>(whole, -1, wb, static_cast<const uint16_t*>(x), y, y_dtype, bias, bias_dtype, m, n_out,
                                      n_in, s);
   const int64_t block_rows = m < kPackRows ? m : kPackRows;

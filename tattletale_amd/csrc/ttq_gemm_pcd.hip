@@ -25,10 +25,9 @@ hipError_t packed_fmt(int tile, const uint8_t* wb, const uint16_t* xp, void* y, 
 hipError_t launch_gemm_packed(int format, bool fuse, int tile, const uint8_t* wb, const uint16_t* xp, void* y, int y_dtype,
                               const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, PcSplit sp,
                               hipStream_t s) {
-  if (fuse) {
-    if (format != kQ4_K) return hipErrorInvalidValue;
-    return packed_fmt<kQ4_K, true>(tile, wb, xp, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
-  }
+  // (no fused gate||up form here: its epilogue does not fit beside three steps of A fragments, and registers that
+  // are the target of asynchronous requests must not be spilled)
+  if (fuse) return hipErrorInvalidValue;
   switch (format) {
     case kQ4_K: return packed_fmt<kQ4_K, false>(tile, wb, xp, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
     case kQ6_K: return packed_fmt<kQ6_K, false>(tile, wb, xp, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);

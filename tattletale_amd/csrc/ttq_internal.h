@@ -300,6 +300,19 @@ int exl3_set_poll_limit(int limit);
 // Trellis layer for many activation rows (ttq_exl3_prefill.hip): activations rotated once into a workspace
 // the library keeps per (device, stream), then 64 rows per decoded weight.  y fp32.
 bool gemm_exl3_preferred(int64_t m, int64_t n_out, int64_t n_in);
+// a prefill GEMM launch split along K: copies of the tile grid that meet in a workspace (ttq_gemm_pc.h)
+struct PcSplit {
+  int splits;          // 1: none
+  int tile_wgs;        // workgroups of one copy of the tile grid
+  float* partials;
+  uint32_t* counters;
+};
+constexpr int kPcMaxCounters = 16384;     // (tile, consumer) pairs a split launch may have
+// bytes of partial sums the many-row trellis GEMM keeps in the workspace for this call (0: not split along K)
+size_t gemm_exl3_partials_bytes(int64_t m, int64_t n_out, int64_t n_in);
+hipError_t launch_gemm_exl3_pc(int bits, int cb, int mb, const uint16_t* trellis, const uint16_t* svh, const uint16_t* xp,
+                               void* y, int y_dtype, const void* bias, int bias_dtype, int64_t m, int64_t n_out,
+                               int64_t n_in, PcSplit sp, hipStream_t s);
 hipError_t launch_gemm_exl3(const uint16_t* trellis, const uint16_t* suh, const uint16_t* svh, const void* x,
                             int x_dtype, void* y, int y_dtype, const void* bias, int bias_dtype, int64_t m,
                             int64_t n_out, int64_t n_in, int bits, int cb, hipStream_t s);

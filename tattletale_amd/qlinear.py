@@ -233,7 +233,7 @@ def gemv_exl3(trellis: torch.Tensor, suh: torch.Tensor, svh: torch.Tensor, x: to
 def gemm_exl3(trellis: torch.Tensor, suh: torch.Tensor, svh: torch.Tensor, x: torch.Tensor,
               n_out: int, n_in: int, bits: int, codebook: int = _lib.CB_MCG) -> torch.Tensor:
     """fp32 y (m, n_out) for many activation rows through ``ttq_gemm_exl3`` (activations rotated once,
-    rounded to float16; every weight decoded once per 64 rows)."""
+    rounded to float16; every weight decoded once per 128 rows)."""
     dev = _require_device(trellis, suh, svh, x)
     if suh.dtype != torch.float16 or svh.dtype != torch.float16:
         raise TtqError(_lib.ERR_DTYPE, "ttq_gemm_exl3: suh/svh must be float16")

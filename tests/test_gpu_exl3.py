@@ -159,10 +159,11 @@ def _exl3_f64_rows(T_bits, suh_bits, svh_bits, xf):
 
 
 @pytest.mark.parametrize("bits,cb", [(3, F.CB_MCG), (2, F.CB_3INST), (4, F.CB_MCG), (6, F.CB_3INST), (8, F.CB_MCG)])
-@pytest.mark.parametrize("n_out,n_in,m", [(256, 512, 16), (384, 1024 + 128, 70), (1024, 2048, 333)])
+@pytest.mark.parametrize("n_out,n_in,m", [(256, 512, 16), (384, 1024 + 128, 70), (1024, 2048, 333), (128, 256, 4096 + 70)])
 def test_exl3_prefill_rows(bits, cb, n_out, n_in, m):
     """Many activation rows through ttq_gemm_exl3 (activations rotated once and rounded to fp16: the
-    2e-2 class, in practice below 1e-3), row by row against the oracle."""
+    2e-2 class, in practice below 1e-3), row by row against the oracle.  The shapes take tiles of 64 rows, tiles of
+    128 rows with a ragged last tile, a launch split four ways along K, and two chunks of rows through one workspace."""
     w = Q.fill_normal(800 + bits, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
     tr, suh, svh = Q.quantize_exl3(w, bits, cb, seed=bits)
     T = oracle.exl3_decode(tr, n_out, n_in, bits, cb)
@@ -197,6 +198,8 @@ def test_exl3_forward_takes_the_prefill_path_and_the_flag_pins_the_decode_class(
     assert not np.array_equal(y, ye)                                          # the two paths really differ
     y16 = auto.forward(xd, out_dtype=torch.bfloat16)                           # prefill path, 16-bit output
     assert torch.equal(y16, torch.from_numpy(y).to(DEV).to(torch.bfloat16))
+    y16h = auto.forward(xd, out_dtype=torch.float16)
+    assert torch.equal(y16h, torch.from_numpy(y).to(DEV).to(torch.float16))
 
 
 def test_exl3_prefill_full_shape_4096x4096_m512_sampled_rows():
