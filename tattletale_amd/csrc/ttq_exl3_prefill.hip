@@ -17,37 +17,46 @@
 
 namespace ttq {
 
-// ---- pass one for the producer/consumer GEMM (ttq_gemm_exl3_pc.h): the same values, stored in fragment order,
+// ---- pass one: Xp = fp16( H(x o suh) / sqrt(128) ) in the fragment order of the matrix cores,
 //   Xp[step of 64 k][block of 16 rows][half of 32 k][lane 64] x 16 bytes: row 16 rb + lane % 16, k = 64 ks + 32 h + 8 (lane / 16) .. + 7,
-// so that an A fragment of v_mfma_f32_16x16x32_f16 is one kilobyte of consecutive bytes.  Rows past the end of the last
-// block are left as they are (their products are never stored).
+// so that an A fragment of v_mfma_f32_16x16x32_f16 is one kilobyte of consecutive bytes.  A workgroup takes a block of
+// 16 rows and one 128-group of k: a half wavefront per row rotates its 128 values in registers (four per lane), the
+// 4 KB of results are put in fragment order in LDS and leave as two runs of 2 KB (steps 2 G and 2 G + 1 of the row
+// block).  Rows past the end are written as zeros.
 template <typename XT>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(512)
 exl3_rotate_pack_kernel(const XT* __restrict__ x, const uint16_t* __restrict__ suh, uint16_t* __restrict__ xp,
-                        int64_t items, int groups_per_row, int64_t n_in, int row_blocks) {
-  const int lane = threadIdx.x & 63, l32 = threadIdx.x & 31;
-  const int64_t item = (int64_t)blockIdx.x * (256 / 32) + (threadIdx.x >> 5);
-  if (item >= items) return;
-  const int64_t row = item / groups_per_row;
-  const int64_t k = (item - row * groups_per_row) * 128 + 4 * l32;
-  uint2 sraw;
-  __builtin_memcpy(&sraw, __builtin_assume_aligned(suh + k, 8), 8);
-  float v[4];
-  load_x4(x + row * n_in + k, v);
-  v[0] *= f16_bits_to_f32((uint16_t)sraw.x);
-  v[1] *= f16_bits_to_f32((uint16_t)(sraw.x >> 16));
-  v[2] *= f16_bits_to_f32((uint16_t)sraw.y);
-  v[3] *= f16_bits_to_f32((uint16_t)(sraw.y >> 16));
-  fwht128_quad(v, lane);
-  uint2 o;
-  o.x = (uint32_t)f32_to_f16_bits(v[0] * 0.08838834764831845f) | ((uint32_t)f32_to_f16_bits(v[1] * 0.08838834764831845f) << 16);
-  o.y = (uint32_t)f32_to_f16_bits(v[2] * 0.08838834764831845f) | ((uint32_t)f32_to_f16_bits(v[3] * 0.08838834764831845f) << 16);
-  const int64_t ks = k >> 6;
-  const int h = (int)(k >> 5) & 1, g = (int)(k >> 3) & 3, e = (int)k & 7;
-  const int64_t rb = row >> 4;
-  const int r = (int)row & 15;
-  uint8_t* dst = reinterpret_cast<uint8_t*>(xp) + ((ks * row_blocks + rb) * 2 + h) * 1024 + (g * 16 + r) * 16 + e * 2;
-  __builtin_memcpy(__builtin_assume_aligned(dst, 8), &o, 8);
+                        int64_t rows, int64_t n_in, int row_blocks) {
+  __shared__ __attribute__((aligned(16))) uint8_t blk[4096];
+  const int tid = threadIdx.x, lane = tid & 63, l32 = tid & 31;
+  const int r = tid >> 5;                                    // row of the block
+  const int64_t rb = blockIdx.y, grp = blockIdx.x;
+  const int64_t row = rb * 16 + r;
+  const int64_t k = grp * 128 + 4 * l32;
+  uint2 o = make_uint2(0u, 0u);
+  if (row < rows) {
+    uint2 sraw;
+    __builtin_memcpy(&sraw, __builtin_assume_aligned(suh + k, 8), 8);
+    float v[4];
+    load_x4(x + row * n_in + k, v);
+    v[0] *= f16_bits_to_f32((uint16_t)sraw.x);
+    v[1] *= f16_bits_to_f32((uint16_t)(sraw.x >> 16));
+    v[2] *= f16_bits_to_f32((uint16_t)sraw.y);
+    v[3] *= f16_bits_to_f32((uint16_t)(sraw.y >> 16));
+    fwht128_quad(v, lane);
+    o.x = (uint32_t)f32_to_f16_bits(v[0] * 0.08838834764831845f) | ((uint32_t)f32_to_f16_bits(v[1] * 0.08838834764831845f) << 16);
+    o.y = (uint32_t)f32_to_f16_bits(v[2] * 0.08838834764831845f) | ((uint32_t)f32_to_f16_bits(v[3] * 0.08838834764831845f) << 16);
+  }
+  // k inside the group: 4 * l32 = 64 * step + 32 * half + 8 * g + e
+  const int kk = 4 * l32;
+  const int st = kk >> 6, h = (kk >> 5) & 1, g = (kk >> 3) & 3, e = kk & 7;
+  *reinterpret_cast<uint2*>(blk + (st * 2 + h) * 1024 + (g * 16 + r) * 16 + e * 2) = o;
+  __syncthreads();
+  // thread t moves bytes 8 t .. 8 t + 7 of the block: the first 2 KB are step 2 grp, the others step 2 grp + 1
+  const uint2 v8 = *reinterpret_cast<const uint2*>(blk + tid * 8);
+  const int st2 = tid >> 8;
+  uint8_t* dst = reinterpret_cast<uint8_t*>(xp) + (((2 * grp + st2) * row_blocks + rb) * 2) * 1024 + (tid & 255) * 8;
+  *reinterpret_cast<uint2*>(dst) = v8;
 }
 
 // ------------------------------------------------------------------------------ launch
@@ -114,24 +123,22 @@ hipError_t launch_gemm_exl3(const uint16_t* trellis, const uint16_t* suh, const 
   for (int64_t r0 = 0; r0 < m; r0 += kXpMaxRows) {
     const int64_t rows = m - r0 < kXpMaxRows ? m - r0 : kXpMaxRows;
     const char* xb = static_cast<const char*>(x) + r0 * n_in * xsize;
-    const int groups_per_row = (int)(n_in / 128);
-    const int64_t items = rows * groups_per_row;
-    const dim3 rgrid((unsigned)((items + 7) / 8)), rblock(256);
     // rotated activations in fragment order, then the tiled GEMM (n_in is a whole number of Hadamard groups, i.e. an
     // even number of 64-k steps)
     const int row_blocks = (int)((rows + 15) / 16);
+    const dim3 rgrid((unsigned)(n_in / 128), (unsigned)row_blocks), rblock(512);
     switch (x_dtype) {
       case kF32:
         hipLaunchKernelGGL(exl3_rotate_pack_kernel<float>, rgrid, rblock, 0, s, reinterpret_cast<const float*>(xb), suh,
-                           xr, items, groups_per_row, n_in, row_blocks);
+                           xr, rows, n_in, row_blocks);
         break;
       case kF16:
         hipLaunchKernelGGL(exl3_rotate_pack_kernel<f16_tag>, rgrid, rblock, 0, s, reinterpret_cast<const f16_tag*>(xb),
-                           suh, xr, items, groups_per_row, n_in, row_blocks);
+                           suh, xr, rows, n_in, row_blocks);
         break;
       case kBF16:
         hipLaunchKernelGGL(exl3_rotate_pack_kernel<bf16_tag>, rgrid, rblock, 0, s, reinterpret_cast<const bf16_tag*>(xb),
-                           suh, xr, items, groups_per_row, n_in, row_blocks);
+                           suh, xr, rows, n_in, row_blocks);
         break;
       default: return hipErrorInvalidValue;
     }
