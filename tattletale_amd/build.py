@@ -60,14 +60,45 @@ def hipcc() -> str:
     return exe
 
 
+# Kernels whose consumers request registers asynchronously (inline-asm buffer loads that the compiler takes for
+# complete): a register the compiler spills is stored before its data has landed, so these must not spill at all.
+# The build reads the compiler's own resource report for them and fails otherwise.
+NO_SPILL_KERNELS = {
+    "ttq_gemm_pcd.hip": ("gemm_pcd_kernel",),
+    "ttq_gemm_exl3_pc.hip": ("gemm_exl3_pc_kernel",),
+}
+
+
+def spilling_kernels(report: str, names) -> list:
+    """Kernels named in `names` for which a -Rpass-analysis=kernel-resource-usage report shows vector register
+    spills, as (mangled name, spilled registers) pairs."""
+    bad, current = [], None
+    for line in report.splitlines():
+        if "Function Name:" in line:
+            current = line.split("Function Name:")[1].split()[0]
+        elif "VGPRs Spill:" in line and current is not None:
+            n = int(line.split("VGPRs Spill:")[1].split()[0])
+            if n > 0 and any(k in current for k in names):
+                bad.append((current, n))
+    return bad
+
+
 def _compile(src: str, obj: str) -> None:
     cmd = [hipcc()] + COMMON
     if src.endswith(".hip"):
         cmd += DEVICE
+    watched = NO_SPILL_KERNELS.get(os.path.basename(src))
+    if watched:
+        cmd += ["-Rpass-analysis=kernel-resource-usage"]
     cmd += ["-DTTQ_BUILD", "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))
+    if watched:
+        bad = spilling_kernels(r.stderr, watched)
+        if bad:
+            raise RuntimeError("%s: kernels with asynchronously loaded registers must not spill: %s"
+                               % (os.path.basename(src), ", ".join("%s (%d)" % b for b in bad)))
 
 
 def build_library(force: bool = True, verbose: bool = False) -> str:

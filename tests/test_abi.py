@@ -216,3 +216,21 @@ def test_row_counts_beyond_a_grid_dimension_are_refused_where_the_library_does_n
         _lib.ERR_UNSUPPORTED,)
     assert L.ttq_gemv_q4_k_rmsnorm(p, p, None, p, 1e-6, _lib.BF16, None, None, p, _lib.F32, 65536, 64, 512, 0,
                                    None) == _lib.ERR_UNSUPPORTED
+
+
+def test_build_rejects_spills_in_kernels_with_asynchronous_register_loads():
+    """The compiler's resource report, as the build reads it: a watched kernel that spills vector registers is
+    named, others and clean ones are not."""
+    from tattletale_amd import build as B
+    report = """x.h:1:1: remark: Function Name: _ZN3ttq15gemm_pcd_kernelILi7ELi1ELi4ELb0ELi0ELi4EEEvPKh [-Rpass-analysis=kernel-resource-usage]
+x.h:1:1: remark:     VGPRs: 256 [-Rpass-analysis=kernel-resource-usage]
+x.h:1:1: remark:     SGPRs Spill: 3 [-Rpass-analysis=kernel-resource-usage]
+x.h:1:1: remark:     VGPRs Spill: 12 [-Rpass-analysis=kernel-resource-usage]
+x.h:2:1: remark: Function Name: _ZN3ttq15gemm_pcd_kernelILi4ELi1ELi2ELb0ELi0ELi4EEEvPKh [-Rpass-analysis=kernel-resource-usage]
+x.h:2:1: remark:     VGPRs Spill: 0 [-Rpass-analysis=kernel-resource-usage]
+x.h:3:1: remark: Function Name: _ZN3ttq23pack_activations_kernelIfEEvPKT_Ptiii [-Rpass-analysis=kernel-resource-usage]
+x.h:3:1: remark:     VGPRs Spill: 5 [-Rpass-analysis=kernel-resource-usage]
+"""
+    bad = B.spilling_kernels(report, B.NO_SPILL_KERNELS["ttq_gemm_pcd.hip"])
+    assert bad == [("_ZN3ttq15gemm_pcd_kernelILi7ELi1ELi4ELb0ELi0ELi4EEEvPKh", 12)]
+    assert B.spilling_kernels(report, ("gemm_exl3_pc_kernel",)) == []
