@@ -178,6 +178,21 @@ def test_exl3_prefill_rows(bits, cb, n_out, n_in, m):
     assert worst <= 1.5e-3                # what the fp16 rounding of the rotated activations costs
 
 
+@pytest.mark.parametrize("n_out,n_in,m", [(128, 128, 1), (128, 128, 17), (256, 256, 130), (128, 384, 64), (128, 1024, 65)])
+def test_exl3_prefill_smallest_shapes(n_out, n_in, m):
+    """The many-row entry point on the smallest legal matrices (two 64-k steps, one tile column) and on row counts
+    around the tile heights."""
+    bits, cb = 3, F.CB_MCG
+    w = Q.fill_normal(830 + m, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
+    tr, suh, svh = Q.quantize_exl3(w, bits, cb, seed=m)
+    T = oracle.exl3_decode(tr, n_out, n_in, bits, cb)
+    x = Q.f32_to_f16(Q.fill_normal(831, 1, 1.0, m * n_in).reshape(m, n_in))
+    y = QL.gemm_exl3(packed_to_dev(tr), bits_to_dev(suh, "f16"), bits_to_dev(svh, "f16"), bits_to_dev(x, "f16"),
+                     n_out, n_in, bits, cb).cpu().numpy()
+    want = _exl3_f64_rows(T, suh, svh, oracle.f16_to_f32(x))
+    assert max(rel_l2(y[i], want[i]) for i in range(m)) <= 1.5e-3
+
+
 @pytest.mark.parametrize("xk", ["bf16", "f32", "f16"])
 def test_exl3_forward_takes_the_prefill_path_and_the_flag_pins_the_decode_class(xk):
     from util import x_to_dev
