@@ -71,16 +71,19 @@ bool gemm_exl3_preferred(int64_t m, int64_t n_out, int64_t n_in) {
 
 constexpr int64_t kXpMaxRows = 4096;       // rows rotated into the workspace at a time
 
-// The producer/consumer form: tiles of 128 rows x 128 columns (64 rows when there are no more), and -- while all
+// The producer/consumer form: tiles of 128 rows x 128 columns (64 rows when there are no more; 256 for launches that
+// are large enough), and -- while all
 // copies of the tile grid fit one round of workgroups -- 2, 4 or 8 copies along K, each with an even number of at
 // least eight 64-k steps: the decode of a tile is paid once per 128 rows, and every compute unit gets a share of it.
 struct XgChoice { int mb, splits; int64_t tiles; };
 static XgChoice xg_choose(int64_t rows, int64_t n_out, int64_t n_in) {
   XgChoice c;
-  c.mb = rows > 64 ? 2 : 1;
+  const int64_t steps = n_in / 64, cus = device_num_cus();
+  // 256-row tiles (every tile decoded once per 256 rows, by four producers instead of eight) where they alone give
+  // every compute unit a workgroup
+  c.mb = (n_out / 128) * ((rows + 255) / 256) >= cus ? 4 : (rows > 64 ? 2 : 1);
   c.tiles = (n_out / 128) * ((rows + 64 * c.mb - 1) / (64 * c.mb));
   c.splits = 1;
-  const int64_t steps = n_in / 64, cus = device_num_cus();
   for (int sp = 2; sp <= 8; sp *= 2)
     if (c.tiles * sp <= cus && steps % sp == 0 && (steps / sp) % 2 == 0 && steps / sp >= 8 && c.tiles * 4 <= kPcMaxCounters)
       c.splits = sp;

@@ -13,7 +13,8 @@
 //       come by LDS DMA into a ring of eight steps private to the wavefront (3 us ahead of their use, no registers
 //       held), a lane reads the two dwords that hold its four windows, swaps their halves (MSB-first 16-bit words -> a
 //       big-endian bit string), decodes four weights as in the decode GEMV (XmLane) and stores them as half of a B
-//       fragment unit.  A decoded tile thus serves every row of the tile (64 * MB) instead of 64.
+//       fragment unit.  A decoded tile thus serves every row of the tile (64 * MB) instead of 64.  (Tiles of 256 rows:
+//       four producers with eight column blocks each, see xg_producers.)
 //   epilogue: after the copies of a launch split along K have met, a consumer rotates the 128 sums of each of its
 //       rows in registers (butterflies over the column blocks in place, over the columns of a block by DPP moves),
 //       applies svh and the bias and stores.
@@ -24,24 +25,27 @@
 
 namespace ttq {
 
-constexpr int kXgAhead = 8;              // steps the producers' requests run ahead (a ring slot per step)
+// Two shapes of workgroup.  Tiles of 64 or 128 rows (MB = 1, 2): eight producers and four consumers, 168 registers
+// each.  Tiles of 256 rows (MB = 4; for launches whose 256-row tiles alone fill the compute units): the consumers
+// need 256 registers, which leaves room for four producers only, two k-tiles' worth of column blocks each -- the
+// decode is slower per step, but it is paid once per 256 rows.
+constexpr int xg_producers(int mb) { return mb == 4 ? 4 : 8; }
+constexpr int xg_threads(int mb) { return (4 + xg_producers(mb)) * 64; }
+// steps the producers' requests run ahead (a ring slot per step): about 3 us either way
+constexpr int xg_ahead(int mb) { return mb == 4 ? 4 : 8; }
 
-constexpr int kXgProducers = 8;          // producer wavefronts
-constexpr int kXgTiles = 32 / kXgProducers;   // tiles (column blocks of one k-tile) a producer decodes per step
-static_assert(kXgTiles == 4, "four tiles per producer and step");
-constexpr int xg_threads() { return (4 + kXgProducers) * 64; }
-
-// bytes of LDS a producer wavefront's ring takes
-template <int BITS>
+// what a producer wavefront handles per step, and the LDS its ring takes
+template <int BITS, int MB>
 struct XgGeom {
-  static constexpr int kRunBytes = kXgTiles * 32 * BITS;             // the wavefront's tiles of one k-tile
+  static constexpr int kTiles = 32 / xg_producers(MB);               // tiles (column blocks of one k-tile) per step
+  static constexpr int kRunBytes = kTiles * 32 * BITS;               // consecutive in trellis[k_tile][n_tile]
   static constexpr int kReq = (kRunBytes + 1023) / 1024;             // requests of 64 x 16 bytes
   static constexpr int kSlotBytes = kReq * 1024;
-  static constexpr int kRingBytes = kXgAhead * kSlotBytes;
+  static constexpr int kRingBytes = xg_ahead(MB) * kSlotBytes;
 };
 
 template <int BITS, int CB, int MB>
-__global__ void __launch_bounds__(xg_threads())
+__global__ void __launch_bounds__(xg_threads(MB))
 gemm_exl3_pc_kernel(const uint8_t* __restrict__ trellis, const uint16_t* __restrict__ svh, const uint16_t* __restrict__ xp,
                     void* __restrict__ yv, int y_dtype, const void* __restrict__ bias, int bias_dtype, int m, int n_out,
                     int n_in, int n_tiles, int m_tiles, int xcds_per_mtile, PcSplit sp) {
@@ -50,7 +54,9 @@ gemm_exl3_pc_kernel(const uint8_t* __restrict__ trellis, const uint16_t* __restr
   constexpr int kWUnits = 2 * NJ * 64;
   constexpr int kPcBM = NC * 16 * MB;
   constexpr int kStgBytes = 16 * MB * (BN * 2 + 16);      // a consumer's epilogue staging area
-  using RG = XgGeom<BITS>;
+  using RG = XgGeom<BITS, MB>;
+  constexpr int kXgProducers = xg_producers(MB), kXgTiles = RG::kTiles, kXgAhead = xg_ahead(MB);
+  static_assert(kXgTiles == 4 || kXgTiles == 8, "tiles in groups of four");
   __shared__ uint4 sw[2 * kWUnits];
   __shared__ __attribute__((aligned(16))) uint8_t stg[NC * kStgBytes];
   __shared__ __attribute__((aligned(1024))) uint8_t raw[kXgProducers * RG::kRingBytes];
@@ -170,8 +176,17 @@ gemm_exl3_pc_kernel(const uint8_t* __restrict__ trellis, const uint16_t* __restr
       const uint32_t dst = sw_addr + (uint32_t)(buf * kWUnits * 16) + unit0;
       Win4 ra;
       read4(slot, std::integral_constant<int, 0>{}, ra);
-      settle4(ra);
-      decode4(dst, std::integral_constant<int, 0>{}, ra);
+      if constexpr (kXgTiles == 8) {
+        Win4 rb;
+        read4(slot, std::integral_constant<int, 4>{}, rb);
+        settle4(ra);                     // (waits for rb's reads too: they are issued, and complete in order)
+        decode4(dst, std::integral_constant<int, 0>{}, ra);
+        settle4(rb);
+        decode4(dst, std::integral_constant<int, 4>{}, rb);
+      } else {
+        settle4(ra);
+        decode4(dst, std::integral_constant<int, 0>{}, ra);
+      }
     };
     // requests complete in order: all but the youngest kXgAhead - 1 steps' worth have landed
     auto wait_step = [&]() { wait_vmcnt<(kXgAhead - 1) * RG::kReq>(); };
@@ -202,13 +217,88 @@ gemm_exl3_pc_kernel(const uint8_t* __restrict__ trellis, const uint16_t* __restr
   int aoff[MB];
 #pragma unroll
   for (int ib = 0; ib < MB; ib++) aoff[ib] = min((m0 >> 4) + ib, row_blocks_x - 1) * 2048 + lane * 16;
+  auto step_koff = [&](int ks) { return (step0 + min(ks, ksteps - 1)) * (row_blocks_x * 2048); };
+  constexpr int G = 2 * NJ;
+  f32x4_t acc[MB][NJ];
+#pragma unroll
+  for (int i = 0; i < MB; i++)
+#pragma unroll
+    for (int jj = 0; jj < NJ; jj++) acc[i][jj] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  auto finish = [&]() {
+    wait_vmcnt<0>();               // the re-reads past the last step
+    PcEpi epi{sp, ksplit, m_tile, n_tile, n_tiles, wave, lane, stg + wave * kStgBytes, yv, y_dtype, bias, bias_dtype, m,
+              n_out, n0, m0};
+    epi.col_scale = svh;
+    pc_epilogue<NJ, MB, false, NC, true>(acc, epi);
+  };
+
+  if constexpr (MB == 4) {
+    // 256-row tiles: 128 accumulators leave room for the A fragments of four half steps (32 k: MB requests, 4 MB
+    // registers each) rotating by position: the fragments of half step q + 3 are requested during half step q.  A
+    // group is four matrix instructions, so B fragments two groups ahead in a ring of four are enough.
+    struct AHalf { u32x4_t v[MB]; };
+    auto request_half = [&](AHalf& dst, int koff, auto hc, int ib) {
+      if constexpr (decltype(hc)::value == 0) buffer_load16_async<0>(dst.v[ib], xrsrc, aoff[ib], koff);
+      else buffer_load16_async<1024>(dst.v[ib], xrsrc, aoff[ib], koff);
+    };
+    f16x8_t bring[4];
+    auto read_b = [&](f16x8_t& dst, int buf, int g) {
+      const uint4 v = sw[buf * kWUnits + g * 64 + lane];
+      __builtin_memcpy(&dst, &v, 16);
+    };
+    static_assert((G & 3) == 0 && MB <= NJ, "a step brings the B ring back to slot 0; one A request per group");
+    using H0 = std::integral_constant<int, 0>;
+    using H1 = std::integral_constant<int, 1>;
+    auto half_step = [&](const AHalf& cur, AHalf& into, auto bufc, auto hc, int ks) {
+      constexpr int BUF = decltype(bufc)::value, HALF = decltype(hc)::value;
+      // requests complete in order: all but those of the next two half steps have landed, `cur` among them
+      wait_vmcnt<2 * MB>();
+      const int koff3 = step_koff(ks + (HALF + 3) / 2);
+#pragma unroll
+      for (int j = 0; j < NJ; j++) {
+        const int g = HALF * NJ + j;
+        if (g == G - 2) bar();     // barrier ks: step ks+1 is in LDS, reads of step ks done
+        if (g + 2 < G) read_b(bring[(g + 2) & 3], BUF, g + 2);
+        else read_b(bring[(g + 2) & 3], BUF ^ 1, g + 2 - G);
+#pragma unroll
+        for (int r = 0; r < MB; r++)
+          if (r * NJ / MB == j) request_half(into, koff3, std::integral_constant<int, (HALF + 3) & 1>{}, r);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < MB; i++) {
+          f16x8_t a;
+          __builtin_memcpy(&a, &cur.v[i], 16);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bring[g & 3], acc[i][j], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    AHalf h0{}, h1{}, h2{}, h3{};
+#pragma unroll
+    for (int ib = 0; ib < MB; ib++) request_half(h0, step_koff(0), H0{}, ib);
+#pragma unroll
+    for (int ib = 0; ib < MB; ib++) request_half(h1, step_koff(0), H1{}, ib);
+#pragma unroll
+    for (int ib = 0; ib < MB; ib++) request_half(h2, step_koff(1), H0{}, ib);
+    bar();                         // barrier -1: the W fragments of step 0 are in LDS
+    read_b(bring[0], 0, 0);
+    read_b(bring[1], 0, 1);
+    // (the number of steps is even: the half-step sets and the W buffers both come round after two steps)
+    for (int ks = 0; ks < ksteps; ks += 2) {
+      half_step(h0, h3, H0{}, H0{}, ks);
+      half_step(h1, h0, H0{}, H1{}, ks);
+      half_step(h2, h1, H1{}, H0{}, ks + 1);
+      half_step(h3, h2, H1{}, H1{}, ks + 1);
+    }
+    finish();
+    return;
+  }
+
   struct ASet { u32x4_t v[2][MB]; };
   auto request_one = [&](ASet& dst, int koff, int h, int ib) {
     if (h == 0) buffer_load16_async<0>(dst.v[0][ib], xrsrc, aoff[ib], koff);
     else buffer_load16_async<1024>(dst.v[1][ib], xrsrc, aoff[ib], koff);
   };
-  auto step_koff = [&](int ks) { return (step0 + min(ks, ksteps - 1)) * (row_blocks_x * 2048); };
-  constexpr int G = 2 * NJ;
   static_assert(2 * MB <= G, "one A request per group");
   // B fragments are read kAheadB groups ahead of their use into a ring of kRing: a group is only MB matrix
   // instructions (16 clocks each), and an LDS read takes more than a hundred clocks to come back
@@ -219,11 +309,6 @@ gemm_exl3_pc_kernel(const uint8_t* __restrict__ trellis, const uint16_t* __restr
     const uint4 v = sw[buf * kWUnits + g * 64 + lane];
     __builtin_memcpy(&dst, &v, 16);
   };
-  f32x4_t acc[MB][NJ];
-#pragma unroll
-  for (int i = 0; i < MB; i++)
-#pragma unroll
-    for (int jj = 0; jj < NJ; jj++) acc[i][jj] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   // A fragments run kDepth - 1 steps ahead of their use: the copy of Xr was written by the pass before this one, so a
   // step's fragments come from the memory side of the L2 (more than a microsecond away) for the first workgroup of
   // an XCD that asks, and steps are short here (a third of a microsecond with 64-row tiles).
@@ -274,12 +359,7 @@ gemm_exl3_pc_kernel(const uint8_t* __restrict__ trellis, const uint16_t* __restr
       step(sets[(u + 1) % kDepth], sets[u % kDepth], C1{}, ks + u + 1);
     }
   }
-  wait_vmcnt<0>();               // the re-reads past the last step
-
-  PcEpi epi{sp, ksplit, m_tile, n_tile, n_tiles, wave, lane, stg + wave * kStgBytes, yv, y_dtype, bias, bias_dtype, m,
-            n_out, n0, m0};
-  epi.col_scale = svh;
-  pc_epilogue<NJ, MB, false, NC, true>(acc, epi);
+  finish();
 }
 
 template <int BITS, int CB, int MB>
@@ -295,7 +375,7 @@ static hipError_t launch_exl3_pc_grid(const uint8_t* trellis, const uint16_t* sv
     nwg = (unsigned)(((n_tiles + xcds_per_mtile - 1) / xcds_per_mtile) * 8);
   }
   sp.tile_wgs = (int)nwg;
-  hipLaunchKernelGGL((gemm_exl3_pc_kernel<BITS, CB, MB>), dim3(nwg * (unsigned)sp.splits), dim3(xg_threads()), 0, s,
+  hipLaunchKernelGGL((gemm_exl3_pc_kernel<BITS, CB, MB>), dim3(nwg * (unsigned)sp.splits), dim3(xg_threads(MB)), 0, s,
                      trellis, svh, xp, y, y_dtype, bias, bias_dtype, (int)m, (int)n_out, (int)n_in, n_tiles, m_tiles,
                      xcds_per_mtile, sp);
   return hipGetLastError();

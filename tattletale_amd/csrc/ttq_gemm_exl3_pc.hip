@@ -10,6 +10,7 @@ template <int BITS, int CB>
 hipError_t xg_mb(int mb, const uint8_t* trellis, const uint16_t* svh, const uint16_t* xp, void* y, int y_dtype,
                  const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, PcSplit sp, hipStream_t s) {
   if (mb == 1) return launch_exl3_pc_grid<BITS, CB, 1>(trellis, svh, xp, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
+  if (mb == 4) return launch_exl3_pc_grid<BITS, CB, 4>(trellis, svh, xp, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
   return launch_exl3_pc_grid<BITS, CB, 2>(trellis, svh, xp, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
 }
 
@@ -22,7 +23,7 @@ hipError_t xg_cb(int cb, int mb, const uint8_t* trellis, const uint16_t* svh, co
 
 }  // namespace
 
-// xp: the rotated activations (fp16) in fragment order; mb: 16-row blocks per consumer (1 or 2: tiles of 64 or 128 rows)
+// xp: the rotated activations (fp16) in fragment order; mb: 16-row blocks per consumer (1, 2 or 4: tiles of 64, 128 or 256 rows)
 hipError_t launch_gemm_exl3_pc(int bits, int cb, int mb, const uint16_t* trellis, const uint16_t* svh, const uint16_t* xp,
                                void* y, int y_dtype, const void* bias, int bias_dtype, int64_t m, int64_t n_out,
                                int64_t n_in, PcSplit sp, hipStream_t s) {

@@ -193,6 +193,23 @@ def test_exl3_prefill_smallest_shapes(n_out, n_in, m):
     assert max(rel_l2(y[i], want[i]) for i in range(m)) <= 1.5e-3
 
 
+@pytest.mark.parametrize("bits,cb", [(3, F.CB_MCG), (6, F.CB_3INST)])
+def test_exl3_prefill_256_row_tiles(bits, cb):
+    """A launch large enough for tiles of 256 rows (32 column groups x 9 row tiles, the last one ragged): four producer
+    wavefronts with eight tiles each, A fragments by half steps.  Sampled rows of every tile against the oracle."""
+    n_out, n_in, m = 4096, 256, 2048 + 40
+    w = Q.fill_normal(840 + bits, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
+    tr, suh, svh = Q.quantize_exl3(w, bits, cb, seed=40 + bits)
+    T = oracle.exl3_decode(tr, n_out, n_in, bits, cb)
+    x = Q.f32_to_f16(Q.fill_normal(841, 1, 1.0, m * n_in).reshape(m, n_in))
+    y = QL.gemm_exl3(packed_to_dev(tr), bits_to_dev(suh, "f16"), bits_to_dev(svh, "f16"), bits_to_dev(x, "f16"),
+                     n_out, n_in, bits, cb).cpu().numpy()
+    assert np.all(np.isfinite(y))
+    rows = sorted(set(list(range(0, m, 37)) + [63, 64, 127, 128, 255, 256, 2047, 2048, m - 1]))
+    want = _exl3_f64_rows(T, suh, svh, oracle.f16_to_f32(x[rows]))
+    assert max(rel_l2(y[i], want[j]) for j, i in enumerate(rows)) <= 1.5e-3
+
+
 @pytest.mark.parametrize("xk", ["bf16", "f32", "f16"])
 def test_exl3_forward_takes_the_prefill_path_and_the_flag_pins_the_decode_class(xk):
     from util import x_to_dev
