@@ -5,8 +5,9 @@
 // Two launches.  The first rotates the activations once -- x o suh, the 128-group butterfly, 1/sqrt(128),
 // rounded to fp16 -- into a workspace, in the fragment order of the matrix cores: every output group needs every
 // rotated row, and rotating inside each workgroup would cost more vector work than decoding its weights.  The
-// second is the producer/consumer GEMM of ttq_gemm_exl3_pc.h (tiles of 128 x 128 or 64 x 128, split along K while
-// the compute units are not all taken), whose epilogue rotates the 128 sums of each row and applies svh and the bias.
+// second is the producer/consumer GEMM of ttq_gemm_exl3_pc.h (tiles of 64, 128 or 256 rows x 128 columns, split along K
+// while the compute units are not all taken), whose epilogue rotates the 128 sums of each row and applies svh and the
+// bias.
 //
 // Accuracy: the rotated activations are rounded to fp16 once (2^-11 relative per element, about 3e-4
 // on a row product); weights are exact fp16, sums fp32.  The decode kernel's two-term split is for
@@ -72,9 +73,9 @@ bool gemm_exl3_preferred(int64_t m, int64_t n_out, int64_t n_in) {
 constexpr int64_t kXpMaxRows = 4096;       // rows rotated into the workspace at a time
 
 // The producer/consumer form: tiles of 128 rows x 128 columns (64 rows when there are no more; 256 for launches that
-// are large enough), and -- while all
-// copies of the tile grid fit one round of workgroups -- 2, 4 or 8 copies along K, each with an even number of at
-// least eight 64-k steps: the decode of a tile is paid once per 128 rows, and every compute unit gets a share of it.
+// are large enough), and -- while all copies of the tile grid fit one round of workgroups -- 2, 4 or 8 copies along K,
+// each with an even number of at least eight 64-k steps: the decode of a tile is paid once per 128 rows, and every
+// compute unit gets a share of it.
 struct XgChoice { int mb, splits; int64_t tiles; };
 static XgChoice xg_choose(int64_t rows, int64_t n_out, int64_t n_in) {
   XgChoice c;
