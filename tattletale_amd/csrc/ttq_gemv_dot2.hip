@@ -413,7 +413,7 @@ gemv_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, 
 #pragma unroll
       for (int r = 0; r < kN; r++) {
         const int row = base + r;
-        if (row < row_end) YElem<YT>::store(ym, row, acc[r] + load_bias(bias, bias_dtype, row));
+        if (row < row_end) YElem<YT>::store_through(ym, row, acc[r] + load_bias(bias, bias_dtype, row));
       }
     }
   };

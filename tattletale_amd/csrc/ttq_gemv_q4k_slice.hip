@@ -309,7 +309,7 @@ gemv_q4k_slice_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict_
     float v = part[grp * nks][nn];
     for (int k = 1; k < nks; k++) v += part[grp * nks + k][nn];
     const int row = wg_row0 + t;
-    if (row < wg_row_end) YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
+    if (row < wg_row_end) YElem<YT>::store_through(ym, row, v + load_bias(bias, bias_dtype, row));
   }
 }
 

@@ -437,7 +437,7 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
       float v = 0.f;
       for (int k = 0; k < 4 * nblocks; k++) v += part[k][tid];
       const int row = wg_row0 + tid;
-      if (row < wg_row_end) YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
+      if (row < wg_row_end) YElem<YT>::store_through(ym, row, v + load_bias(bias, bias_dtype, row));
     }
     return;
   }
@@ -506,9 +506,9 @@ gemv_q4k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
     if (FUSE) {
       float u = part[(ngroups + grp) << nks_log2][nn];
       if (nks_log2) u += part[((ngroups + grp) << 1) + 1][nn];
-      if (row < wg_row_end) YElem<YT>::store(ym, row, (v / (1.f + expf(-v))) * u);
+      if (row < wg_row_end) YElem<YT>::store_through(ym, row, (v / (1.f + expf(-v))) * u);
     } else {
-      if (row < wg_row_end) YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
+      if (row < wg_row_end) YElem<YT>::store_through(ym, row, v + load_bias(bias, bias_dtype, row));
     }
   }
 }

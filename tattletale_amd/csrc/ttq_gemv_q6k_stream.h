@@ -450,7 +450,7 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
 #pragma unroll
       for (int wv = 0; wv < kQ6Waves; wv++) v += part[grp][wv][nn];
       const int row = (grp0 + grp) * 16 + nn;
-      YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
+      YElem<YT>::store_through(ym, row, v + load_bias(bias, bias_dtype, row));
     }
   } else if (fold_nb != 0) {
     // real row fs of streamed row nn: blocks fs * fold_nb ... of the streamed row; block b was wavefront b % 8's
@@ -461,7 +461,7 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
       float v = 0.f;
       for (int b = fs * fold_nb; b < (fs + 1) * fold_nb; b++) v += part[grp * rpg + (b >> 3)][b & 7][nn];
       const int row = (((grp0 + grp) * 16 + nn) << fold_log2) + fs;
-      YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
+      YElem<YT>::store_through(ym, row, v + load_bias(bias, bias_dtype, row));
     }
   } else {
     // real row fs of streamed row nn: the blocks of wavefronts fs * (8 >> fold_log2) ...
@@ -472,7 +472,7 @@ gemv_q6k_stream_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict
       float v = 0.f;
       for (int wv = fs * per; wv < (fs + 1) * per; wv++) v += part[grp][wv][nn];
       const int row = (((grp0 + grp) * 16 + nn) << fold_log2) + fs;
-      YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
+      YElem<YT>::store_through(ym, row, v + load_bias(bias, bias_dtype, row));
     }
   }
 }

@@ -402,7 +402,7 @@ gemv_q8_stream_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, Y
 #pragma unroll
     for (int wv = 0; wv < kQ8Waves; wv++) v += part[grp][wv][nn];
     const int row = (grp0 + grp) * 16 + nn;
-    YElem<YT>::store(ym, row, v + load_bias(bias, bias_dtype, row));
+    YElem<YT>::store_through(ym, row, v + load_bias(bias, bias_dtype, row));
   }
 }
 
