@@ -246,20 +246,27 @@ gemv_exl3_mfma_kernel(const uint16_t* __restrict__ trellis, const uint16_t* __re
     if (owner) *reinterpret_cast<float4*>(dst + (col >> 1) * 128 + tcol * 16 + 4 * q) = make_float4(acc[0], acc[1], acc[2], acc[3]);
   }
   __syncthreads();
+  constexpr int kHandoffBatch = 16;
   for (int e = tid; e < ntok * 128; e += kXmThreads) {
-    // the other slices' words for this output (eight loads in flight before the first is looked at),
+    // the other slices' words for this output (sixteen loads in flight before the first is looked at: the fourteen
+    // words of a launch in eight slices in one round trip to the memory side),
     // then this workgroup's own sums
     float s = 0.f;
     bool late = false;
     const int nparts = (nslices - 1) * kXmKSplit;
-    for (int p0 = 0; p0 < nparts; p0 += 8) {
-      unsigned long long w[8];
+    // The slices of a group finish their decode within a fraction of a microsecond of each other, and a word asked for
+    // before it has reached the memory side costs a second round trip (about 0.9 us); 256 clocks of patience before
+    // the first look make the first look the only one (4096 x 4096, one row: 9.1 -> 8.8 us; two to six units of 64
+    // clocks measure the same).
+    if (nparts > 0) __builtin_amdgcn_s_sleep(4);
+    for (int p0 = 0; p0 < nparts; p0 += kHandoffBatch) {
+      unsigned long long w[kHandoffBatch];
 #pragma unroll
-      for (int i = 0; i < 8; i++)
+      for (int i = 0; i < kHandoffBatch; i++)
         w[i] = __hip_atomic_load(words + (int64_t)min(p0 + i, nparts - 1) * kPartWords + e, __ATOMIC_RELAXED,
                                  __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
-      for (int i = 0; i < 8; i++) {
+      for (int i = 0; i < kHandoffBatch; i++) {
         if (p0 + i < nparts) {
           unsigned long long* wp = words + (int64_t)(p0 + i) * kPartWords + e;
           for (int polls = 0; (uint32_t)(w[i] >> 32) != tag && polls < poll_limit; polls++) {
