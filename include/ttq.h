@@ -130,9 +130,10 @@ typedef struct ttq_qlinear {
  * kernel.  Only a layer with precision == TTQ_PRECISION_BF16_OK lets the library round 256 or more
  * rows of fp16 / fp32 activations to bf16 (into a workspace) and run the bf16 matrix-core GEMM on
  * the copy (2e-2 class).
- * Limits (TTQ_ERR_UNSUPPORTED beyond): the decode kernels take n_in <= 32768 for Q4_K / Q6_K with
- * 16-bit activations and n_in <= 16384 otherwise; any m (rows are taken 65535 at a time where a
- * kernel needs that).  m == 0 or n_out == 0 returns TTQ_OK without touching a pointer. */
+ * Limits (TTQ_ERR_UNSUPPORTED beyond): TTQ_EXL3 layers take n_in <= 16384; the block formats take
+ * any n_in (rows beyond 32768 values for Q4_K / Q6_K with 16-bit activations, beyond 16384 otherwise,
+ * run a decode kernel that stages nothing in LDS: correct, not tuned); any m (rows are taken 65535
+ * at a time where a kernel needs that).  m == 0 or n_out == 0 returns TTQ_OK without touching a pointer. */
 TTQ_API int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int64_t m,
                        void* y, int y_dtype, void* stream);
 
@@ -179,6 +180,7 @@ typedef enum {
   TTQ_ROUTE_GEMV_DOT2 = 12,
   TTQ_ROUTE_GEMV_DOT2_MULTI = 13,
   TTQ_ROUTE_GEMV_GENERIC = 14,
+  TTQ_ROUTE_GEMV_LONG = 15,          /* rows longer than the staged kernels take: nothing staged in LDS */
   TTQ_ROUTE_GEMM_PC = 20,            /* producer / consumer prefill GEMM */
   TTQ_ROUTE_GEMM_PC_SPLIT_K = 21,    /* ... in several copies along K (takes a workspace) */
   TTQ_ROUTE_GEMM_SKINNY = 22,        /* 17-64 rows */
@@ -197,8 +199,8 @@ TTQ_API const char* ttq_route_name(int route);
 
 /* ---- decode GEMV, one entry per block format (m rows of x, normally m == 1) -------- */
 /* y[m][n_out] (fp32) = x[m][n_in] * W^T.  Stand in for F.linear(x, weight) with a
- * (1, n_in) activation (neural_nets.nim:64).  n_in <= 32768 for Q4_K / Q6_K with 16-bit
- * activations, <= 16384 otherwise.  Two to four rows (a speculative step, a few sequences) of
+ * (1, n_in) activation (neural_nets.nim:64).  Any n_in (rows beyond 32768 values for Q4_K / Q6_K
+ * with 16-bit activations, beyond 16384 otherwise, take an untuned kernel).  Two to four rows (a speculative step, a few sequences) of
  * 16-bit activations over a large Q4_K or Q6_K matrix cost about one pass over the weights, not
  * one per row; every row's result stays within the 1e-3 class of the single-row call.  A NaN or
  * an infinity among a row's activations, or in a block scale of a weight row, makes the outputs

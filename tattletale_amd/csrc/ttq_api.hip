@@ -79,13 +79,6 @@ int check_shape(int format, int64_t m, int64_t n_out, int64_t n_in, int bits, in
   }
 }
 
-// Longest row the decode kernels take: the packed-dot kernel (Q4_K / Q6_K, 16-bit activations)
-// stages 32768 activations in 64 KiB of LDS, everything else 16384.
-int check_gemv_limits(int format, int x_dtype, int64_t n_in) {
-  const bool long_rows = (format == TTQ_Q4_K || format == TTQ_Q6_K) && (x_dtype == TTQ_F16 || x_dtype == TTQ_BF16);
-  const int64_t lim = long_rows ? ttq::kMaxGemvIn16 : ttq::kMaxGemvInF32;
-  return n_in <= lim ? TTQ_OK : TTQ_ERR_UNSUPPORTED;
-}
 
 // grid dimensions y and z end at 65535: the trellis GEMV puts groups of 8 activation rows on z, the fused decode
 // kernels and RMSNorm one row per workgroup on y
@@ -118,8 +111,6 @@ int gemv_block(int format, const void* w, const void* x, int x_dtype, void* y, i
   if (m == 0 || n_out == 0) return TTQ_OK;  // empty output: nothing to read or write
   if (!w || !x || !y) return TTQ_ERR_NULL;
   if (!aligned16(w) || !aligned16(x) || !aligned16(y)) return TTQ_ERR_ALIGN;
-  rc = check_gemv_limits(format, x_dtype, n_in);
-  if (rc != TTQ_OK) return rc;
   return hip_status(launch_gemv_any_m(format, w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in,
                                       static_cast<hipStream_t>(stream)));
 }
@@ -445,7 +436,7 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
 
   // Several rows of bf16 activations: the prefill GEMM (weights rounded to bf16) or a few passes of
   // the decode kernels (fp32 scales), whichever the shape makes cheaper.  Up to four rows always
-  // decode; a GEMV that the row length rules out leaves only the GEMM.
+  // decode.
   const bool gemm_ok = x_dtype == TTQ_BF16 && (y_dtype == TTQ_BF16 || y_dtype == TTQ_F32) &&
                        (layer->format == TTQ_Q4_K || layer->format == TTQ_Q6_K || layer->format == TTQ_Q8_0) &&
                        ttq::gemm_supported(layer->format, m, n_out, n_in);
@@ -453,8 +444,7 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
   static const int knob = ttq::dev_knob("TTQ_FORWARD_ROUTE", 0);
   const int route = layer->precision == TTQ_PRECISION_F32_SCALES ? 1 : knob;
   if (gemm_ok && m >= 5 && route != 1) {
-    const bool gemv_ok = check_gemv_limits(layer->format, x_dtype, n_in) == TTQ_OK;
-    if (!gemv_ok || route == 2 ||
+    if (route == 2 ||
         ttq::gemm_estimate_us(layer->format, m, n_out, n_in) < ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in))
       return hip_status(ttq::launch_gemm(layer->format, layer->qweight, static_cast<const uint16_t*>(x), y, y_dtype,
                                          layer->bias, layer->bias_dtype, m, n_out, n_in, s));
@@ -477,16 +467,13 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
     const int64_t full = m / 64, rest = m % 64;
     float us = (float)full * ttq::gemm_skinny_estimate_us(layer->format, 64, n_out, n_in);
     if (rest) us += ttq::gemm_skinny_estimate_us(layer->format, rest, n_out, n_in);
-    const bool gemv_ok = check_gemv_limits(layer->format, x_dtype, n_in) == TTQ_OK;
-    if (!gemv_ok || route == 2 || us < ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in)) {
+    if (route == 2 || us < ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in)) {
       if (ttq::route_probe(ttq::kRouteGemmSkinnyChunked)) return TTQ_OK;
       return hip_status(ttq::launch_gemm_skinny_chunked(layer->format, layer->qweight, static_cast<const uint16_t*>(x),
                                                         x_dtype, y, y_dtype, layer->bias, layer->bias_dtype, m, n_out,
                                                         n_in, s));
     }
   }
-  const int lim = check_gemv_limits(layer->format, x_dtype, n_in);
-  if (lim != TTQ_OK) return lim;
   return hip_status(launch_gemv_any_m(layer->format, layer->qweight, x, x_dtype, y, y_dtype, layer->bias,
                                       layer->bias_dtype, m, n_out, n_in, s));
 }
@@ -528,6 +515,7 @@ const char* ttq_route_name(int route) {
     case TTQ_ROUTE_GEMV_DOT2: return "gemv_dot2";
     case TTQ_ROUTE_GEMV_DOT2_MULTI: return "gemv_dot2_multi";
     case TTQ_ROUTE_GEMV_GENERIC: return "gemv_generic";
+    case TTQ_ROUTE_GEMV_LONG: return "gemv_long";
     case TTQ_ROUTE_GEMM_PC: return "gemm_pc";
     case TTQ_ROUTE_GEMM_PC_SPLIT_K: return "gemm_pc_split_k";
     case TTQ_ROUTE_GEMM_SKINNY: return "gemm_skinny";

@@ -44,6 +44,8 @@ struct FmtQ8_0 {
   static __device__ __forceinline__ int units(int n_in) { return (n_in + 63) >> 6; }
   static __device__ __forceinline__ int64_t row_bytes(int n_in) { return (int64_t)(n_in >> 5) * 34; }
   static __device__ __forceinline__ void kmap(int k, int& u, int& p) { u = k >> 6; p = k & 63; }
+  // first k of activation slots 16 q .. 16 q + 15 of unit u (consecutive k)
+  static __device__ __forceinline__ int64_t kbase(int u, int q) { return 64 * (int64_t)u + 16 * q; }
   struct Raw { uint4 a0, a1, b0, b1; uint32_t d0, d1; };
   static __device__ __forceinline__ Raw load(const uint8_t* row, int u, int n_in) {
     Raw r;
@@ -89,6 +91,7 @@ struct FmtQ4_K {
   static __device__ __forceinline__ int units(int n_in) { return n_in >> 6; }
   static __device__ __forceinline__ int64_t row_bytes(int n_in) { return (int64_t)(n_in >> 8) * 144; }
   static __device__ __forceinline__ void kmap(int k, int& u, int& p) { u = k >> 6; p = k & 63; }
+  static __device__ __forceinline__ int64_t kbase(int u, int q) { return 64 * (int64_t)u + 16 * q; }
   struct Raw { uint4 hdr, q0, q1; int c; };
   static __device__ __forceinline__ Raw load(const uint8_t* row, int u, int) {
     Raw r;
@@ -135,6 +138,10 @@ struct FmtQ6_K {
     const int j = rr >> 5, l = rr & 31;
     u = 4 * b + 2 * h + (l >> 4);
     p = 16 * j + (l & 15);
+  }
+  // slots 16 j .. 16 j + 15 of unit 4 b + 2 h + s: k = 256 b + 128 h + 32 j + 16 s + i
+  static __device__ __forceinline__ int64_t kbase(int u, int q) {
+    return 256 * (int64_t)(u >> 2) + 128 * ((u >> 1) & 1) + 32 * q + 16 * (u & 1);
   }
   struct Raw { uint4 a, b, h; uint32_t sc0, sc1; uint32_t d; int s; };
   static __device__ __forceinline__ Raw load(const uint8_t* row, int u, int) {
@@ -345,10 +352,100 @@ static hipError_t launch_generic_xy(const void* w, const void* x, int x_dtype, v
   }
 }
 
+// ---------------------------------------------------------------------- rows of any length
+// Rows longer than the staged kernels hold in LDS (F.linear has no such limit: the down projection of the
+// largest dense models has 53248 inputs).  Nothing is staged: a wavefront owns a weight row, its lanes walk the
+// row's units 64 apart, and every lane reads the 64 activations of its unit straight from memory in four runs of
+// 16 consecutive values (the activation row stays in L2, and the weights are read once).  Same arithmetic as the
+// generic kernel (fp32, scales applied once per sub-block).
+template <class F, typename XT, typename YT>
+__global__ void __launch_bounds__(kGemvThreads)
+gemv_long_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, YT* __restrict__ y,
+                 const void* __restrict__ bias, int bias_dtype, int n_out, int n_in) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const XT* xm = x + (int64_t)blockIdx.y * n_in;
+  YT* ym = y + (int64_t)blockIdx.y * n_out;
+  const int units = F::units(n_in);
+  const int64_t rb = F::row_bytes(n_in);
+  constexpr int kVec = 16 / (int)sizeof(XT);           // activations per 16-byte load
+  for (int row = blockIdx.x * kGemvWaves + wave; row < n_out; row += gridDim.x * kGemvWaves) {
+    float acc = 0.f;
+    for (int u = lane; u < units; u += 64) {
+      const typename F::Raw r = F::load(w + rb * row, u, n_in);
+      float xr[64];
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const int64_t k0 = F::kbase(u, q);
+        if (k0 + 16 <= n_in) {
+#pragma unroll
+          for (int v = 0; v < 16 / kVec; v++) {
+            XT raw[kVec];
+            const uint4 t = *reinterpret_cast<const uint4*>(__builtin_assume_aligned(xm + k0 + kVec * v, 16));
+            __builtin_memcpy(raw, &t, 16);
+#pragma unroll
+            for (int i = 0; i < kVec; i++) xr[16 * q + kVec * v + i] = XElem<XT>::load(raw, i);
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < 16; i++) xr[16 * q + i] = 0.f;      // past the end of a Q8_0 row of an odd number of blocks
+        }
+      }
+      acc += F::dot(r, xr);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) YElem<YT>::store(ym, row, acc + load_bias(bias, bias_dtype, row));
+  }
+}
+
+template <class F, typename XT, typename YT>
+static hipError_t launch_long(const void* w, const void* x, void* y, const void* bias, int bias_dtype, int64_t m,
+                              int64_t n_out, int64_t n_in, hipStream_t s) {
+  const int64_t need = (n_out + kGemvWaves - 1) / kGemvWaves, most = (int64_t)device_num_cus() * 8;
+  const dim3 grid((unsigned)(need < most ? need : most), (unsigned)m), block(kGemvThreads);
+  hipLaunchKernelGGL((gemv_long_kernel<F, XT, YT>), grid, block, 0, s, static_cast<const uint8_t*>(w),
+                     static_cast<const XT*>(x), static_cast<YT*>(y), bias, bias_dtype, (int)n_out, (int)n_in);
+  return hipGetLastError();
+}
+template <class F, typename XT>
+static hipError_t launch_long_y(const void* w, const void* x, void* y, int y_dtype, const void* bias, int bias_dtype,
+                                int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+  switch (y_dtype) {
+    case kF32: return launch_long<F, XT, float>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kF16: return launch_long<F, XT, f16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    case kBF16: return launch_long<F, XT, bf16_tag>(w, x, y, bias, bias_dtype, m, n_out, n_in, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+template <class F>
+static hipError_t launch_long_xy(const void* w, const void* x, int x_dtype, void* y, int y_dtype, const void* bias,
+                                 int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+  switch (x_dtype) {
+    case kF32: return launch_long_y<F, float>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kF16: return launch_long_y<F, f16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    case kBF16: return launch_long_y<F, bf16_tag>(w, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+// Longest row the staged decode kernels take: the packed-dot kernel (Q4_K / Q6_K, 16-bit activations) stages 32768
+// activations in 64 KiB of LDS, everything else 16384.
+bool gemv_row_is_long(int format, int x_dtype, int64_t n_in) {
+  const bool dot2 = (format == kQ4_K || format == kQ6_K) && (x_dtype == kF16 || x_dtype == kBF16);
+  return n_in > (dot2 ? kMaxGemvIn16 : kMaxGemvInF32);
+}
+
 hipError_t launch_gemv(int format, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
                        const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
                        hipStream_t s) {
   if (m == 0 || n_out == 0) return hipSuccess;
+  if (gemv_row_is_long(format, x_dtype, n_in)) {
+    switch (format) {
+      case kQ8_0: TTQ_ROUTE(kRouteGemvLong, launch_long_xy<FmtQ8_0>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
+      case kQ4_K: TTQ_ROUTE(kRouteGemvLong, launch_long_xy<FmtQ4_K>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
+      case kQ6_K: TTQ_ROUTE(kRouteGemvLong, launch_long_xy<FmtQ6_K>(w, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s));
+      default: return hipErrorInvalidValue;
+    }
+  }
   // a few rows at once: four per pass for up to four rows and for rows too long for the 8- and
   // 16-token tables, else eight or sixteen per pass
   if (gemv_q4k_stream4_supported(format, x_dtype, m, n_out, n_in))
@@ -406,6 +503,8 @@ hipError_t launch_gemv(int format, const void* w, const void* x, int x_dtype, vo
 float gemv_estimate_us(int format, int x_dtype, int64_t m, int64_t n_out, int64_t n_in) {
   const int64_t per = format == kQ8_0 ? 32 : 256, blk = format == kQ8_0 ? 34 : (format == kQ4_K ? 144 : 210);
   const float mb = (float)(n_out * (n_in / per) * blk) * 1e-6f;
+  // rows of any length: a pass over the weights per activation row, not measured beyond a few shapes
+  if (gemv_row_is_long(format, x_dtype, n_in)) return (float)m * (mb / 2.f + 3.f);
   const bool b4 = gemv_q4k_batch4_supported(format, x_dtype, m, n_out, n_in);
   if (b4 && m <= 4) return mb / 2.75f + 2.f;
   if (gemv_q4k_batch_supported(format, x_dtype, m, n_out, n_in)) {

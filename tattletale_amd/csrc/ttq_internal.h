@@ -31,6 +31,7 @@ enum : int {
   kRouteGemvDot2 = 12,
   kRouteGemvDot2Multi = 13,
   kRouteGemvGeneric = 14,
+  kRouteGemvLong = 15,
   kRouteGemmPc = 20,
   kRouteGemmPcSplitK = 21,
   kRouteGemmSkinny = 22,
@@ -78,6 +79,8 @@ enum : int { kQ8_0 = 0, kQ4_K = 1, kQ6_K = 2, kEXL3 = 3 };
 
 constexpr int64_t kMaxGemvInF32 = 16384;    // activations staged in 64 KiB of LDS
 constexpr int64_t kMaxGemvIn16 = 32768;
+// rows beyond what the staged decode kernels take (they go to the unstaged kernel of ttq_gemv.hip)
+bool gemv_row_is_long(int format, int x_dtype, int64_t n_in);
 
 hipError_t launch_dequant(int format, const void* w, void* out, int out_dtype, int64_t n_out,
                           int64_t n_in, hipStream_t s);

@@ -55,7 +55,7 @@ def test_gemv_validation_order(name):
     assert fn(p, p, _lib.F32, p, 1, 4, 100, None) == _lib.ERR_SHAPE
     assert fn(p, p, _lib.F32, p, -1, 4, 256, None) == _lib.ERR_SHAPE
     assert fn(p + 2, p, _lib.F32, p, 1, 4, 256, None) == _lib.ERR_ALIGN
-    assert fn(p, p, _lib.F32, p, 1, 4, 1 << 20, None) == _lib.ERR_UNSUPPORTED
+    assert fn(p, p, _lib.F32, p, 1, 4, 1 << 32, None) == _lib.ERR_UNSUPPORTED       # sizes are 31-bit inside the kernels
 
 
 def test_other_entry_points_validate():
@@ -142,13 +142,13 @@ def test_row_length_limits():
     buf = np.zeros(4096, np.uint8)
     p = buf.ctypes.data
     p += (-p) % 16
-    # 16-bit activations on the K-quants: 32768; everything else 16384 (misalignment answers when the
-    # limit lets the call through)
+    # the block formats take rows of any length (misalignment answers when the limits let the call through);
+    # the trellis format ends at 16384 values
     assert L.ttq_gemv_q4_k(p, p + 2, _lib.BF16, p, 1, 16, 32768, None) == _lib.ERR_ALIGN
     assert L.ttq_gemv_q6_k(p, p + 2, _lib.F16, p, 1, 16, 28672, None) == _lib.ERR_ALIGN
-    assert L.ttq_gemv_q4_k(p, p, _lib.BF16, p, 1, 16, 32768 + 256, None) == _lib.ERR_UNSUPPORTED
-    assert L.ttq_gemv_q4_k(p, p, _lib.F32, p, 1, 16, 16384 + 256, None) == _lib.ERR_UNSUPPORTED
-    assert L.ttq_gemv_q8_0(p, p, _lib.BF16, p, 1, 16, 16384 + 256, None) == _lib.ERR_UNSUPPORTED
+    assert L.ttq_gemv_q4_k(p, p + 2, _lib.BF16, p, 1, 16, 32768 + 256, None) == _lib.ERR_ALIGN
+    assert L.ttq_gemv_q4_k(p, p + 2, _lib.F32, p, 1, 16, 16384 + 256, None) == _lib.ERR_ALIGN
+    assert L.ttq_gemv_q8_0(p, p + 2, _lib.BF16, p, 1, 16, 16384 + 256, None) == _lib.ERR_ALIGN
     st = QLinearStruct(format=_lib.EXL3, bits=3, codebook=1, n_out=128, n_in=16384 + 128, qweight=p, suh=p, svh=p)
     assert L.ttq_linear_forward(C.byref(st), p, _lib.F16, 1, p, _lib.F32, None) == _lib.ERR_UNSUPPORTED
 

@@ -36,6 +36,37 @@ def test_k_quant_rows_up_to_32768_with_16bit_activations(fmt, xk, n_out, n_in, m
     assert sampled_rows_error(fmt, p, y, xf, n_out, n_in, 41) <= TOL
 
 
+@pytest.mark.parametrize("fmt,xk,n_out,n_in", [(F.Q4_K, "bf16", 1024, 53248), (F.Q4_K, "f32", 515, 16384 + 256),
+                                               (F.Q6_K, "f16", 300, 32768 + 512), (F.Q6_K, "f32", 200, 20480),
+                                               (F.Q8_0, "bf16", 257, 16384 + 32), (F.Q8_0, "f32", 64, 40000 - 32)])
+@pytest.mark.parametrize("m", [1, 3])
+def test_rows_beyond_what_the_staged_kernels_take(fmt, xk, n_out, n_in, m):
+    """F.linear has no row-length limit (53248 inputs: the down projection of the largest dense models).  Rows beyond
+    the LDS-staged kernels take the unstaged one; a Q8_0 row of an odd number of blocks ends in half a unit."""
+    per = 32 if fmt == F.Q8_0 else 256
+    p = random_blocks(fmt, n_out * (n_in // per), seed=n_in + fmt)
+    xd, xf = x_to_dev(Q.fill_normal(78, m, 1.0, m * n_in).reshape(m, n_in), xk)
+    wd = packed_to_dev(p)
+    y = QL.gemv(fmt, wd, xd, n_out, n_in).cpu().numpy()
+    assert np.all(np.isfinite(y))
+    assert sampled_rows_error(fmt, p, y, xf, n_out, n_in, 7) <= TOL
+    layer = QuantLinear.init(wd, fmt, n_in, n_out)
+    assert layer.route(m, xd.dtype) == "gemv_long"
+    yl = layer.forward(xd, out_dtype=torch.float32).cpu().numpy()
+    assert np.array_equal(yl, y)
+    # unit vectors reproduce the canonical column bit for bit, also in the last block of the row
+    cols = [0, 16384, n_in - 33, n_in - 1]
+    sub = np.ascontiguousarray(p.reshape(n_out, -1)[:16])
+    what = oracle.dequant(fmt, sub.reshape(-1), 16, n_in)
+    x1 = np.zeros((len(cols), n_in), np.float32)
+    for i, c in enumerate(cols):
+        x1[i, c] = 1.0
+    x1d, _ = x_to_dev(x1, xk)
+    y1 = QL.gemv(fmt, wd, x1d, n_out, n_in).cpu().numpy()
+    for i, c in enumerate(cols):
+        assert np.array_equal(y1[i][:16], what[:, c]), c
+
+
 def test_long_rows_unit_vectors_bit_exact():
     n_out, n_in = 512, 28672
     p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=5)

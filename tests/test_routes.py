@@ -37,6 +37,8 @@ PINNED = [
     ("two rows of the headline shape", Q4_K, 14336, 4096, 2, BF16, F32, 0, "gemv_q4k_stream4"),
     ("three rows of the LM head", Q6_K, 128256, 4096, 3, BF16, F32, 0, "gemv_q6k_stream4"),
     ("trellis layer, prefill 512 rows", EXL3, 4096, 4096, 512, F16, F32, 3, "exl3_gemm"),
+    ("down projection of a 53248-wide MLP, decode", Q4_K, 16384, 53248, 1, BF16, F32, 0, "gemv_long"),
+    ("fp32 activations beyond 16384 values", Q8_0, 4096, 16384 + 32, 1, F32, F32, 0, "gemv_long"),
 ]
 
 
