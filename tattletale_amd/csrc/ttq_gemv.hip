@@ -354,10 +354,12 @@ static hipError_t launch_generic_xy(const void* w, const void* x, int x_dtype, v
 
 // ---------------------------------------------------------------------- rows of any length
 // Rows longer than the staged kernels hold in LDS (F.linear has no such limit: the down projection of the
-// largest dense models has 53248 inputs).  Nothing is staged: a wavefront owns a weight row, its lanes walk the
-// row's units 64 apart, and every lane reads the 64 activations of its unit straight from memory in four runs of
-// 16 consecutive values (the activation row stays in L2, and the weights are read once).  Same arithmetic as the
-// generic kernel (fp32, scales applied once per sub-block).
+// largest dense models has 53248 inputs).  Nothing is staged: a wavefront owns kLongRows consecutive weight rows,
+// its lanes walk the rows' units 64 apart, and every lane reads the 64 activations of its unit straight from
+// memory in four runs of 16 consecutive values, once for all of its rows (the activation row stays in L2, the
+// weights are read once).  Same arithmetic as the generic kernel (fp32, scales applied once per sub-block).
+constexpr int kLongRows = 8;
+
 template <class F, typename XT, typename YT>
 __global__ void __launch_bounds__(kGemvThreads)
 gemv_long_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, YT* __restrict__ y,
@@ -368,10 +370,13 @@ gemv_long_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, YT* __
   const int units = F::units(n_in);
   const int64_t rb = F::row_bytes(n_in);
   constexpr int kVec = 16 / (int)sizeof(XT);           // activations per 16-byte load
-  for (int row = blockIdx.x * kGemvWaves + wave; row < n_out; row += gridDim.x * kGemvWaves) {
-    float acc = 0.f;
+  const int groups = (n_out + kLongRows - 1) / kLongRows;
+  for (int g = blockIdx.x * kGemvWaves + wave; g < groups; g += gridDim.x * kGemvWaves) {
+    const int row0 = g * kLongRows;
+    float acc[kLongRows];
+#pragma unroll
+    for (int r = 0; r < kLongRows; r++) acc[r] = 0.f;
     for (int u = lane; u < units; u += 64) {
-      const typename F::Raw r = F::load(w + rb * row, u, n_in);
       float xr[64];
 #pragma unroll
       for (int q = 0; q < 4; q++) {
@@ -390,17 +395,24 @@ gemv_long_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, YT* __
           for (int i = 0; i < 16; i++) xr[16 * q + i] = 0.f;      // past the end of a Q8_0 row of an odd number of blocks
         }
       }
-      acc += F::dot(r, xr);
+      // (rows past the end repeat the last one; their sums are not stored)
+#pragma unroll
+      for (int r = 0; r < kLongRows; r++)
+        acc[r] += F::dot(F::load(w + rb * min(row0 + r, n_out - 1), u, n_in), xr);
     }
-    acc = wave_sum(acc);
-    if (lane == 0) YElem<YT>::store(ym, row, acc + load_bias(bias, bias_dtype, row));
+#pragma unroll
+    for (int r = 0; r < kLongRows; r++) {
+      const float sum = wave_sum(acc[r]);
+      if (lane == 0 && row0 + r < n_out) YElem<YT>::store(ym, row0 + r, sum + load_bias(bias, bias_dtype, row0 + r));
+    }
   }
 }
 
 template <class F, typename XT, typename YT>
 static hipError_t launch_long(const void* w, const void* x, void* y, const void* bias, int bias_dtype, int64_t m,
                               int64_t n_out, int64_t n_in, hipStream_t s) {
-  const int64_t need = (n_out + kGemvWaves - 1) / kGemvWaves, most = (int64_t)device_num_cus() * 8;
+  const int64_t per_wg = (int64_t)kGemvWaves * kLongRows;
+  const int64_t need = (n_out + per_wg - 1) / per_wg, most = (int64_t)device_num_cus() * 8;
   const dim3 grid((unsigned)(need < most ? need : most), (unsigned)m), block(kGemvThreads);
   hipLaunchKernelGGL((gemv_long_kernel<F, XT, YT>), grid, block, 0, s, static_cast<const uint8_t*>(w),
                      static_cast<const XT*>(x), static_cast<YT*>(y), bias, bias_dtype, (int)n_out, (int)n_in);
