@@ -272,11 +272,12 @@ def test_q8_0_unit_vectors_and_extremes_many_rows(xk, n_in):
         assert rel_l2(y[-1], want[1]) <= TOL
 
 
-def test_gemv_rejects_oversized_rows():
-    with pytest.raises(TtqError) as e:
-        QL.gemv(F.Q4_K, torch.zeros(144 * 128, dtype=torch.uint8, device=DEV),
-                torch.zeros(32768, dtype=torch.float32, device=DEV), 1, 32768)
-    assert e.value.status == F.ERR_UNSUPPORTED
+def test_gemv_takes_rows_beyond_the_staged_kernels():
+    """fp32 activations of 32768 values are more than the staged kernels hold; the call runs all the same
+    (tests/test_gpu_limits.py checks the values of such rows against the oracle)."""
+    y = QL.gemv(F.Q4_K, torch.zeros(144 * 128, dtype=torch.uint8, device=DEV),
+                torch.ones(32768, dtype=torch.float32, device=DEV), 1, 32768)
+    assert y.shape == (1, 1) and float(y[0, 0]) == 0.0
 
 
 # ------------------------------------------------------------------- full benchmark shapes
