@@ -77,7 +77,7 @@ typedef enum { TTQ_Q8_0 = 0, TTQ_Q4_K = 1, TTQ_Q6_K = 2, TTQ_EXL3 = 3 } ttq_form
 typedef enum {
   TTQ_PRECISION_AUTO = 0,       /* from five rows on, whichever kernel of the activations' own type the shape makes cheaper */
   TTQ_PRECISION_F32_SCALES = 1, /* always the decode kernels: fp32 scales, rel-L2 <= 1e-3 whatever m is */
-  TTQ_PRECISION_BF16_OK = 2     /* as AUTO, and fp16 / fp32 activations may be rounded to bf16 for the matrix-core GEMM */
+  TTQ_PRECISION_BF16_OK = 2     /* as AUTO, and fp32 activations may be rounded to bf16 for the matrix-core GEMM */
 } ttq_precision;
 
 /* Codebook functions of the trellis format. */
@@ -126,10 +126,12 @@ typedef struct ttq_qlinear {
  * of the GEMM entry points -- when its cost estimate prefers them for the shape.  A layer with
  * precision == TTQ_PRECISION_F32_SCALES keeps the decode kernels, and with them the 1e-3 class,
  * for every m.  The operator computes in the type of x (linear.nim:45-57): fp32 activations always
- * take the decode kernels (1e-3 class), fp16 activations those or the fp16 few-row matrix-core
- * kernel.  Only a layer with precision == TTQ_PRECISION_BF16_OK lets the library round 256 or more
- * rows of fp16 / fp32 activations to bf16 (into a workspace) and run the bf16 matrix-core GEMM on
- * the copy (2e-2 class).
+ * take the decode kernels (1e-3 class); fp16 activations those, the fp16 few-row matrix-core kernel
+ * or, beyond 64 rows, the fp16 form of the prefill GEMM (a packed fp16 copy of x in a workspace,
+ * weights rounded once to fp16, fp16 matrix cores: about 2e-4 measured, inside the 1e-3 class; a
+ * dequantized weight beyond the fp16 range becomes an infinity there).  Only a layer with
+ * precision == TTQ_PRECISION_BF16_OK lets the library round 256 or more rows of fp32 activations
+ * to bf16 (into a workspace) and run the bf16 matrix-core GEMM on the copy (2e-2 class).
  * Limits (TTQ_ERR_UNSUPPORTED beyond): TTQ_EXL3 layers take n_in <= 16384; the block formats take
  * any n_in (rows beyond 32768 values for Q4_K / Q6_K with 16-bit activations, beyond 16384 otherwise,
  * run a decode kernel that stages nothing in LDS: correct, not tuned); any m (rows are taken 65535
@@ -186,9 +188,10 @@ typedef enum {
   TTQ_ROUTE_GEMM_SKINNY = 22,        /* 17-64 rows */
   TTQ_ROUTE_GEMM_SKINNY_CHUNKED = 23,
   TTQ_ROUTE_GEMM_Q4K_TILES = 24,     /* single-role tiled kernel (128-column tiles, activations beyond 4 GiB) */
-  TTQ_ROUTE_GEMM_PC_BF16_COPY = 25,  /* TTQ_PRECISION_BF16_OK: fp16 / fp32 activations rounded to bf16 by the packing pass */
+  TTQ_ROUTE_GEMM_PC_BF16_COPY = 25,  /* TTQ_PRECISION_BF16_OK: fp32 activations rounded to bf16 by the packing pass */
   TTQ_ROUTE_GEMM_PC_PACKED = 26,     /* long launches: activations packed in fragment order first (takes a workspace) */
   TTQ_ROUTE_GEMM_PC_PACKED_SPLIT_K = 27,
+  TTQ_ROUTE_GEMM_PC_F16 = 28,        /* fp16 activations: packed fp16 copy, weights rounded to fp16, fp16 matrix cores */
   TTQ_ROUTE_EXL3_GEMV = 30,
   TTQ_ROUTE_EXL3_GEMV_SLICED = 31,   /* K sliced over workgroups that meet in a workspace */
   TTQ_ROUTE_EXL3_GEMM = 32,

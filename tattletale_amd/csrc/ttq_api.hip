@@ -449,30 +449,40 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
       return hip_status(ttq::launch_gemm(layer->format, layer->qweight, static_cast<const uint16_t*>(x), y, y_dtype,
                                          layer->bias, layer->bias_dtype, m, n_out, n_in, s));
   }
-  // fp16 / fp32 activations, 256 rows or more, and only where the layer says that bf16 activations will do
-  // (TTQ_PRECISION_BF16_OK; the operator computes in the type of x otherwise): the prefill GEMM's packing pass rounds
-  // them to bf16 on the way into its workspace (weights and activations rounded to bf16: the 2e-2 class, like the
-  // GEMM entry points)
   const bool block_fmt = layer->format == TTQ_Q4_K || layer->format == TTQ_Q6_K || layer->format == TTQ_Q8_0;
-  if ((x_dtype == TTQ_F16 || x_dtype == TTQ_F32) && block_fmt && m >= 256 && route != 1 && n_in % 8 == 0 &&
-      layer->precision == TTQ_PRECISION_BF16_OK &&
-      ttq::gemm_pc_supported(layer->format, m < 8192 ? m : 8192, n_out, n_in, 112)) {
-    return hip_status(ttq::launch_gemm_pc_x(layer->format, layer->qweight, x, x_dtype, y, y_dtype, layer->bias,
-                                            layer->bias_dtype, m, n_out, n_in, s));
-  }
-  // fp16 activations, up to 64 rows: the few-row kernel takes them as they are
-  const bool block_format = layer->format == TTQ_Q4_K || layer->format == TTQ_Q6_K || layer->format == TTQ_Q8_0;
-  if (x_dtype == TTQ_F16 && block_format && m >= 5 && route != 1 &&
-      ttq::gemm_skinny_supported(layer->format, m < 64 ? m : 64, n_out, n_in)) {
-    const int64_t full = m / 64, rest = m % 64;
-    float us = (float)full * ttq::gemm_skinny_estimate_us(layer->format, 64, n_out, n_in);
-    if (rest) us += ttq::gemm_skinny_estimate_us(layer->format, rest, n_out, n_in);
-    if (route == 2 || us < ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in)) {
+  // fp16 activations, five rows or more: the operator computes in the type of x, so the weights are rounded to fp16
+  // (11 bits: the result stays in the 1e-3 class of the decode kernels) and multiplied on the fp16 matrix cores --
+  // by the few-row kernel (64 rows per launch) or, from where it is cheaper, by the prefill GEMM over a packed fp16
+  // copy of the activations -- unless passes of the decode kernels are cheaper still.
+  if (x_dtype == TTQ_F16 && block_fmt && m >= 5 && route != 1) {
+    float us_few = 1e30f, us_gemm = 1e30f;
+    if (ttq::gemm_skinny_supported(layer->format, m < 64 ? m : 64, n_out, n_in)) {
+      const int64_t full = m / 64, rest = m % 64;
+      us_few = (float)full * ttq::gemm_skinny_estimate_us(layer->format, 64, n_out, n_in);
+      if (rest) us_few += ttq::gemm_skinny_estimate_us(layer->format, rest, n_out, n_in);
+    }
+    if (m > 64 && ttq::gemm_pc_supported(layer->format, m < 8192 ? m : 8192, n_out, n_in, 112))
+      us_gemm = ttq::gemm_pc_estimate_us(layer->format, m, n_out, n_in) + 2.5f + (float)(m * n_in * 4) / 3.0e6f;
+    const float us_gemv = ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in);
+    if (us_gemm < us_few && (route == 2 || us_gemm < us_gemv))
+      return hip_status(ttq::launch_gemm_pc_x(layer->format, layer->qweight, x, x_dtype, y, y_dtype, layer->bias,
+                                              layer->bias_dtype, m, n_out, n_in, s, true));
+    if (us_few < 1e29f && (route == 2 || us_few < us_gemv)) {
       if (ttq::route_probe(ttq::kRouteGemmSkinnyChunked)) return TTQ_OK;
       return hip_status(ttq::launch_gemm_skinny_chunked(layer->format, layer->qweight, static_cast<const uint16_t*>(x),
                                                         x_dtype, y, y_dtype, layer->bias, layer->bias_dtype, m, n_out,
                                                         n_in, s));
     }
+  }
+  // fp32 activations, 256 rows or more, and only where the layer says that bf16 activations will do
+  // (TTQ_PRECISION_BF16_OK; the operator computes in the type of x otherwise): the prefill GEMM's packing pass rounds
+  // them to bf16 on the way into its workspace (weights and activations rounded to bf16: the 2e-2 class, like the
+  // GEMM entry points)
+  if (x_dtype == TTQ_F32 && block_fmt && m >= 256 && route != 1 && n_in % 8 == 0 &&
+      layer->precision == TTQ_PRECISION_BF16_OK &&
+      ttq::gemm_pc_supported(layer->format, m < 8192 ? m : 8192, n_out, n_in, 112)) {
+    return hip_status(ttq::launch_gemm_pc_x(layer->format, layer->qweight, x, x_dtype, y, y_dtype, layer->bias,
+                                            layer->bias_dtype, m, n_out, n_in, s));
   }
   return hip_status(launch_gemv_any_m(layer->format, layer->qweight, x, x_dtype, y, y_dtype, layer->bias,
                                       layer->bias_dtype, m, n_out, n_in, s));
@@ -523,6 +533,7 @@ const char* ttq_route_name(int route) {
     case TTQ_ROUTE_GEMM_Q4K_TILES: return "gemm_q4k_tiles";
     case TTQ_ROUTE_GEMM_PC_BF16_COPY: return "gemm_pc_bf16_copy";
     case TTQ_ROUTE_GEMM_PC_PACKED: return "gemm_pc_packed";
+    case TTQ_ROUTE_GEMM_PC_F16: return "gemm_pc_f16";
     case TTQ_ROUTE_GEMM_PC_PACKED_SPLIT_K: return "gemm_pc_packed_split_k";
     case TTQ_ROUTE_EXL3_GEMV: return "exl3_gemv";
     case TTQ_ROUTE_EXL3_GEMV_SLICED: return "exl3_gemv_sliced";
@@ -552,7 +563,11 @@ int64_t ttq_workspace_bytes(const ttq_qlinear* layer, int64_t m, int x_dtype) {
   // split along K: the prefill GEMM's exact size for every row count it can be called with here, and the few-row
   // kernel's bound (one 64 x 64 tile of sums per compute unit)
   const int64_t block_rows = m < kGemmRows ? m : kGemmRows;
-  const int copy_dtype = (x_dtype != TTQ_BF16 && layer->precision == TTQ_PRECISION_BF16_OK && m >= 256) ? x_dtype : TTQ_BF16;
+  // (fp16 activations beyond 64 rows may take the prefill GEMM over a packed fp16 copy; fp32 ones a bf16 copy where
+  // the layer allows it)
+  const int copy_dtype = (x_dtype == TTQ_F16 && m > 64) ||
+                                 (x_dtype == TTQ_F32 && layer->precision == TTQ_PRECISION_BF16_OK && m >= 256)
+                             ? x_dtype : TTQ_BF16;
   int64_t scratch = ((int64_t)ttq::gemm_pc_packed_bytes(m, n_out, n_in, copy_dtype) + 255) & ~(int64_t)255;
   int64_t partials = (int64_t)ttq::device_num_cus() * (16 * 4 * (16 * 4 + 1) * 4);
   const int64_t rows[3] = {m, block_rows, m % kGemmRows};

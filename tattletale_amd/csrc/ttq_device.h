@@ -49,6 +49,22 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return u;
 }
 
+// Two floats -> one dword of fp16 halves, one rounding (to nearest even) each.  The values are made opaque first:
+// otherwise the compiler folds a fused multiply-add that produced them into the conversion (v_fma_mix*), which rounds
+// the exact sum straight to fp16 instead of rounding the fp32 value -- a different result on ties of the fp32 value.
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+  asm("" : "+v"(lo));
+  asm("" : "+v"(hi));
+  f16x2_t r;
+  r[0] = (_Float16)lo;
+  r[1] = (_Float16)hi;
+  uint32_t u;
+  __builtin_memcpy(&u, &r, 4);
+  return u;
+}
+
 // Activation element -> float, by buffer element type.
 template <typename T> struct XElem;
 template <> struct XElem<float> {
@@ -62,6 +78,12 @@ template <> struct XElem<f16_tag> {
 template <> struct XElem<bf16_tag> {
   static __device__ __forceinline__ float load(const bf16_tag* p, int64_t i) { return bf16_bits_to_f32(p[i].v); }
 };
+
+// two floats -> one dword of the 16-bit type XT (bf16_tag / f16_tag), one rounding each
+template <class XT> __device__ __forceinline__ uint32_t pack_x2(float lo, float hi) {
+  if constexpr (__is_same(XT, f16_tag)) return pack_f16x2(lo, hi);
+  else return pack_bf16x2(lo, hi);
+}
 
 // Output element <- float.
 // store_through: the same store written through to memory (a relaxed store at system scope).  For the last

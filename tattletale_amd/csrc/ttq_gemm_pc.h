@@ -94,7 +94,7 @@ template <> struct WFmt<kQ4_K> {
 #pragma unroll
     for (int c = 0; c < 4; c++) dst.q[c] = load16_a16(p + 16 + 32 * c + 16 * whalf);
   }
-  template <int C>
+  template <int C, class XT = bf16_tag>
   static __device__ __forceinline__ void dequant(const Raw& r, int, uint32_t (&lo)[8], uint32_t (&hi)[8]) {
     const float d = f16_bits_to_f32((uint16_t)(r.hdr.x & 0xFFFF));
     const float dmin = f16_bits_to_f32((uint16_t)(r.hdr.x >> 16));
@@ -119,10 +119,10 @@ template <> struct WFmt<kQ4_K> {
       // fused multiply-add == canonical two-step form here (the product is exact)
       const float fl[4] = {fmaf_(e1, la[0], nm1), fmaf_(e1, la[1], nm1), fmaf_(e1, lb[0], nm1), fmaf_(e1, lb[1], nm1)};
       const float fh[4] = {fmaf_(e2, ha[0], nm2), fmaf_(e2, ha[1], nm2), fmaf_(e2, hb[0], nm2), fmaf_(e2, hb[1], nm2)};
-      lo[2 * i] = pack_bf16x2(fl[0], fl[1]);
-      lo[2 * i + 1] = pack_bf16x2(fl[2], fl[3]);
-      hi[2 * i] = pack_bf16x2(fh[0], fh[1]);
-      hi[2 * i + 1] = pack_bf16x2(fh[2], fh[3]);
+      lo[2 * i] = pack_x2<XT>(fl[0], fl[1]);
+      lo[2 * i + 1] = pack_x2<XT>(fl[2], fl[3]);
+      hi[2 * i] = pack_x2<XT>(fh[0], fh[1]);
+      hi[2 * i + 1] = pack_x2<XT>(fh[2], fh[3]);
     }
   }
 };
@@ -147,7 +147,7 @@ template <> struct WFmt<kQ6_K> {
     dst.sc = load16_a2(p + 192);
     dst.d = load2(p + 208);
   }
-  template <int C>
+  template <int C, class XT = bf16_tag>
   static __device__ __forceinline__ void dequant(const Raw& r, int whalf, uint32_t (&lo)[8], uint32_t (&hi)[8]) {
     constexpr int H = C >> 1, ODD = C & 1;
     const float d = f16_bits_to_f32((uint16_t)r.d);
@@ -171,10 +171,10 @@ template <> struct WFmt<kQ6_K> {
         fl[k] = fmaf_(s1, (float)((qa >> (8 * k)) & 0xFFu), m1);
         fh[k] = fmaf_(s2, (float)((qb >> (8 * k)) & 0xFFu), m2);
       }
-      lo[2 * i] = pack_bf16x2(fl[0], fl[1]);
-      lo[2 * i + 1] = pack_bf16x2(fl[2], fl[3]);
-      hi[2 * i] = pack_bf16x2(fh[0], fh[1]);
-      hi[2 * i + 1] = pack_bf16x2(fh[2], fh[3]);
+      lo[2 * i] = pack_x2<XT>(fl[0], fl[1]);
+      lo[2 * i + 1] = pack_x2<XT>(fl[2], fl[3]);
+      hi[2 * i] = pack_x2<XT>(fh[0], fh[1]);
+      hi[2 * i + 1] = pack_x2<XT>(fh[2], fh[3]);
     }
   }
 };
@@ -199,7 +199,7 @@ template <> struct WFmt<kQ8_0> {
       dst.ch[c][2] = load16_a16(a + 32);
     }
   }
-  template <int C>
+  template <int C, class XT = bf16_tag>
   static __device__ __forceinline__ void dequant(const Raw& r, int whalf, uint32_t (&lo)[8], uint32_t (&hi)[8]) {
     // the block starts 4 C + 2 whalf bytes into the three chunks
     const uint32_t D[12] = {r.ch[C][0].x, r.ch[C][0].y, r.ch[C][0].z, r.ch[C][0].w, r.ch[C][1].x, r.ch[C][1].y,
@@ -224,10 +224,10 @@ template <> struct WFmt<kQ8_0> {
         fl[k] = fmaf_(d, (float)((ua >> (8 * k)) & 0xFFu), md);
         fh[k] = fmaf_(d, (float)((ub >> (8 * k)) & 0xFFu), md);
       }
-      lo[2 * i] = pack_bf16x2(fl[0], fl[1]);
-      lo[2 * i + 1] = pack_bf16x2(fl[2], fl[3]);
-      hi[2 * i] = pack_bf16x2(fh[0], fh[1]);
-      hi[2 * i + 1] = pack_bf16x2(fh[2], fh[3]);
+      lo[2 * i] = pack_x2<XT>(fl[0], fl[1]);
+      lo[2 * i + 1] = pack_x2<XT>(fl[2], fl[3]);
+      hi[2 * i] = pack_x2<XT>(fh[0], fh[1]);
+      hi[2 * i + 1] = pack_x2<XT>(fh[2], fh[3]);
     }
   }
 };
@@ -239,9 +239,10 @@ template <> struct WFmt<kQ8_0> {
 // tile = index into launch_gemm_pc's table of tile shapes.
 hipError_t launch_gemm_packed(int format, bool fuse, int tile, const uint8_t* wb, const uint16_t* xp, void* y, int y_dtype,
                               const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, PcSplit sp,
-                              hipStream_t s);
+                              hipStream_t s, bool x_f16 = false);
 size_t gemm_packed_activation_bytes(int64_t m, int64_t n_in);
-hipError_t launch_gemm_pack_activations(const void* x, int x_dtype, uint16_t* xp, int64_t m, int64_t n_in, hipStream_t s);
+hipError_t launch_gemm_pack_activations(const void* x, int x_dtype, uint16_t* xp, int64_t m, int64_t n_in, hipStream_t s,
+                                        bool keep_f16 = false);
 
 // What a consumer wavefront does with its finished accumulators (shared by the kernels of this file and of
 // ttq_gemm_pcd.h): the meeting of the K copies, bias, silu_and_mul, rounding, and the store of Y.
@@ -419,7 +420,7 @@ __device__ __forceinline__ void pc_epilogue(f32x4_t (&acc)[MB][NJ], const PcEpi&
     }
     return;
   }
-  if ((y_dtype == kBF16 || (ROT && y_dtype == kF16)) && n0 + BN <= n_out && (n_out & 7) == 0) {
+  if ((y_dtype == kBF16 || y_dtype == kF16) && n0 + BN <= n_out && (n_out & 7) == 0) {
     // Full tile of bf16: transpose through the wavefront's own (now idle) X ring, so that global
     // memory sees 16-byte stores along the rows instead of 2-byte ones.  Row stride 240 bytes.
     constexpr int kRowBytes = BN * 2 + 16;
@@ -432,7 +433,7 @@ __device__ __forceinline__ void pc_epilogue(f32x4_t (&acc)[MB][NJ], const PcEpi&
 #pragma unroll
         for (int r = 0; r < 4; r++)
           *reinterpret_cast<uint16_t*>(stg + (16 * i + rb4 + r) * kRowBytes + (16 * j + cn) * 2) =
-              (ROT && y_dtype == kF16) ? f32_to_f16_bits(acc[i][j][r] + bv) : f32_to_bf16_bits(acc[i][j][r] + bv);
+              y_dtype == kF16 ? f32_to_f16_bits(acc[i][j][r] + bv) : f32_to_bf16_bits(acc[i][j][r] + bv);
     }
     // same wavefront wrote and reads: LDS keeps program order, no barrier needed
     uint8_t* yb = static_cast<uint8_t*>(yv);
@@ -508,7 +509,7 @@ __device__ __forceinline__ void pc_epilogue(f32x4_t (&acc)[MB][NJ], const PcEpi&
 // 64 k of a producer thread's row (chunk C of the 256 k in `r`), dequantized, rounded to bf16 and stored as B
 // fragments into W stage `buf` of the tile at LDS address sw_addr.  whalf / wj / wn: the thread's half of every
 // 32-byte chunk, its column block and its column inside the block.
-template <int NJ, int FMT, int ABL, int C>
+template <int NJ, int FMT, int ABL, int C, class XT = bf16_tag>
 __device__ __forceinline__ void pc_dequant_to_lds(const typename WFmt<FMT>::Raw& r, int buf, int whalf, int wj, int wn,
                                                   uint32_t sw_addr) {
   using WF = WFmt<FMT>;
@@ -522,7 +523,7 @@ __device__ __forceinline__ void pc_dequant_to_lds(const typename WFmt<FMT>::Raw&
 #pragma unroll
     for (int i = 0; i < 8; i++) { lo[i] = raw[(4 * c + i) % (sizeof(WRaw) / 4)]; hi[i] = raw[(4 * c + i + 4) % (sizeof(WRaw) / 4)]; }
   } else {
-    WF::template dequant<c>(r, whalf, lo, hi);
+    WF::template dequant<c, XT>(r, whalf, lo, hi);
   }
   if constexpr ((ABL & 4) != 0) {
     // ladder: no LDS stores; keep the values alive
@@ -550,7 +551,7 @@ __device__ __forceinline__ void pc_dequant_to_lds(const typename WFmt<FMT>::Raw&
 // The W producer role (wavefronts 4-7 of either kernel): thread pt (0..255) owns one row of the tile and half of
 // every 32-byte chunk; it loads the packed blocks, dequantizes 64 k per step and writes the B fragments into the
 // double-buffered W tile at LDS address sw_addr, keeping the step barrier `bar`.
-template <int NJ, int FMT, bool FUSE, int ABL, typename Bar>
+template <int NJ, int FMT, bool FUSE, int ABL, class XT = bf16_tag, typename Bar>
 __device__ __forceinline__ void pc_produce_w(const uint8_t* __restrict__ w, int pt, int n0, int n_out, int row_blocks,
                                              int block0, int nblocks, uint32_t sw_addr, Bar&& bar) {
   constexpr int BN = NJ * 16;
@@ -577,7 +578,7 @@ __device__ __forceinline__ void pc_produce_w(const uint8_t* __restrict__ w, int 
   };
   auto dequant_to_lds = [&](const WRaw& r, auto cc, int buf) {
     if (widle) return;
-    pc_dequant_to_lds<NJ, FMT, ABL, decltype(cc)::value>(r, buf, whalf, wj, wn, sw_addr);
+    pc_dequant_to_lds<NJ, FMT, ABL, decltype(cc)::value, XT>(r, buf, whalf, wj, wn, sw_addr);
   };
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;

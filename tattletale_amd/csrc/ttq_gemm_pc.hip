@@ -8,7 +8,7 @@ namespace ttq {
 template <int FMT, int MB, int NJ, bool FUSE>
 static hipError_t launch_pc_tile(const uint8_t* wb, const uint16_t* x, void* y, int y_dtype, const void* bias,
                                  int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, int splits, int tile_if_packed,
-                                 hipStream_t s) {
+                                 hipStream_t s, bool x_f16 = false) {
   PcSplit sp{1, 0, nullptr, nullptr};
   if (!FUSE && splits > 1) {
     // (the chooser has checked that the blocks of a row divide evenly and that the counters suffice)
@@ -24,7 +24,7 @@ static hipError_t launch_pc_tile(const uint8_t* wb, const uint16_t* x, void* y, 
     sp.counters = static_cast<uint32_t*>(cnt);
   }
   if (tile_if_packed >= 0)
-    return launch_gemm_packed(FMT, FUSE, tile_if_packed, wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
+    return launch_gemm_packed(FMT, FUSE, tile_if_packed, wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s, x_f16);
   return launch_pc_grid<FMT, MB, NJ, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
 }
 
@@ -109,23 +109,24 @@ static bool pc_use_packed(const PcChoice& c, int64_t m, int64_t n_in) {
 template <int FMT, bool FUSE>
 static hipError_t launch_pc_rows(const PcChoice& c, int tile_if_packed, const uint8_t* wb, const uint16_t* x, void* y,
                                  int y_dtype, const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
-                                 hipStream_t s) {
+                                 hipStream_t s, bool x_f16 = false) {
   const int p = tile_if_packed;
   switch (c.tile) {
-    case 0: return launch_pc_tile<FMT, 4, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s);
-    case 1: return launch_pc_tile<FMT, 4, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s);
-    case 2: return launch_pc_tile<FMT, 2, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s);
-    case 3: return launch_pc_tile<FMT, 2, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s);
-    case 4: return launch_pc_tile<FMT, 1, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s);
-    default: return launch_pc_tile<FMT, 1, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s);
+    case 0: return launch_pc_tile<FMT, 4, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s, x_f16);
+    case 1: return launch_pc_tile<FMT, 4, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s, x_f16);
+    case 2: return launch_pc_tile<FMT, 2, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s, x_f16);
+    case 3: return launch_pc_tile<FMT, 2, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s, x_f16);
+    case 4: return launch_pc_tile<FMT, 1, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s, x_f16);
+    default: return launch_pc_tile<FMT, 1, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s, x_f16);
   }
 }
 
 // x in x_dtype: bf16 for the direct form; any type when the launch goes through the packed copy (the packing pass
-// rounds to bf16).
+// rounds to bf16, or -- keep_f16 -- leaves fp16 activations as they are for the fp16 form of the kernel).
 template <int FMT, bool FUSE>
 static hipError_t launch_pc_fmt(const uint8_t* wb, const void* x, int x_dtype, void* y, int y_dtype, const void* bias,
-                                int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, bool force_packed, hipStream_t s) {
+                                int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, bool force_packed, hipStream_t s,
+                                bool keep_f16 = false) {
   const PcChoice whole = pc_choose(m, n_out, n_in, FUSE);
   // (the fused gate||up form keeps the LDS-staged kernel: beside the packed kernel's three steps of A fragments its
   // epilogue does not fit the registers, and a kernel that requests registers asynchronously must never spill them)
@@ -140,11 +141,11 @@ static hipError_t launch_pc_fmt(const uint8_t* wb, const void* x, int x_dtype, v
   for (int64_t r0 = 0; r0 < m; r0 += kPackRows) {
     const int64_t rows = m - r0 < kPackRows ? m - r0 : kPackRows;
     e = launch_gemm_pack_activations(static_cast<const char*>(x) + r0 * n_in * xsize, x_dtype, static_cast<uint16_t*>(ws),
-                                     rows, n_in, s);
+                                     rows, n_in, s, keep_f16);
     if (e != hipSuccess) return e;
     const PcChoice c = rows == m ? whole : pc_choose(rows, n_out, n_in, FUSE);
     e = launch_pc_rows<FMT, FUSE>(c, c.tile, wb, static_cast<const uint16_t*>(ws), static_cast<char*>(y) + r0 * n_out * ysize,
-                                  y_dtype, bias, bias_dtype, rows, n_out, n_in, s);
+                                  y_dtype, bias, bias_dtype, rows, n_out, n_in, s, keep_f16);
     if (e != hipSuccess) return e;
   }
   return hipSuccess;
@@ -161,23 +162,27 @@ bool gemm_pc_supported(int format, int64_t m, int64_t n_out, int64_t n_in, int b
 }
 
 // x: bf16 activations; or (x_dtype fp16 / fp32) activations that may be rounded to bf16: those always go through the
-// packed copy, whose packing pass does the rounding.
+// packed copy, whose packing pass does the rounding; or (f16_native) fp16 activations that stay fp16: the packed copy
+// keeps them as they are and the kernel rounds the weights to fp16 and multiplies on the fp16 matrix cores.
 hipError_t launch_gemm_pc_x(int format, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
-                            const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+                            const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s,
+                            bool f16_native) {
   if (m == 0 || n_out == 0) return hipSuccess;
   if (y_dtype != kBF16 && y_dtype != kF32 && y_dtype != kF16) return hipErrorInvalidValue;
+  if (f16_native && x_dtype != kF16) return hipErrorInvalidValue;
   const PcChoice c = pc_choose(m, n_out, n_in, false);
   const bool packed = x_dtype != kBF16 || pc_use_packed(c, m, n_in);
-  if (route_probe(x_dtype != kBF16 ? kRouteGemmPcBf16Copy
-                                   : (c.splits > 1 ? (packed ? kRouteGemmPcPackedSplitK : kRouteGemmPcSplitK)
-                                                   : (packed ? kRouteGemmPcPacked : kRouteGemmPc))))
+  if (route_probe(f16_native ? kRouteGemmPcF16
+                             : (x_dtype != kBF16 ? kRouteGemmPcBf16Copy
+                                                 : (c.splits > 1 ? (packed ? kRouteGemmPcPackedSplitK : kRouteGemmPcSplitK)
+                                                                 : (packed ? kRouteGemmPcPacked : kRouteGemmPc)))))
     return hipSuccess;
   const uint8_t* wb = static_cast<const uint8_t*>(w);
   const bool force = x_dtype != kBF16;
   switch (format) {
-    case kQ4_K: return launch_pc_fmt<kQ4_K, false>(wb, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, force, s);
-    case kQ6_K: return launch_pc_fmt<kQ6_K, false>(wb, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, force, s);
-    case kQ8_0: return launch_pc_fmt<kQ8_0, false>(wb, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, force, s);
+    case kQ4_K: return launch_pc_fmt<kQ4_K, false>(wb, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, force, s, f16_native);
+    case kQ6_K: return launch_pc_fmt<kQ6_K, false>(wb, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, force, s, f16_native);
+    case kQ8_0: return launch_pc_fmt<kQ8_0, false>(wb, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, force, s, f16_native);
     default: return hipErrorInvalidValue;
   }
 }

@@ -44,7 +44,9 @@ __device__ __forceinline__ void buffer_load16_async(u32x4_t& dst, u32x4_t rsrc, 
                : "=v"(dst) : "v"(voffset), "s"(rsrc), "s"(soffset), "n"(IMM) : "memory");
 }
 
-template <int NJ, int FMT, int MB, bool FUSE, int ABL = 0, int NC = 4>
+// XT: the 16-bit type of the packed activations, and the type the producers round the weights to (bf16, or fp16
+// for fp16 activations: the operator then computes in the activations' own type, with weights that keep 11 bits).
+template <int NJ, int FMT, int MB, bool FUSE, int ABL = 0, int NC = 4, class XT = bf16_tag>
 __global__ void __launch_bounds__(pcd_threads(NC))
 gemm_pcd_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ xp, void* __restrict__ yv,
                 int y_dtype, const void* __restrict__ bias, int bias_dtype, int m, int n_out, int n_in,
@@ -116,7 +118,7 @@ gemm_pcd_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ xp, 
   // complete in LDS (buffer (s+1) % 2) and every LDS read of step s has finished.  The consumers pass it near the
   // end of step s, the producers after preparing step s+1.
   if (wave >= NC) {
-    pc_produce_w<NJ, FMT, FUSE, ABL>(w, tid - NC * 64, n0, n_out, row_blocks, block0, nblocks,
+    pc_produce_w<NJ, FMT, FUSE, ABL, XT>(w, tid - NC * 64, n0, n_out, row_blocks, block0, nblocks,
                                      (uint32_t)(size_t)(lptr_t)(&sw[0]), bar);
     trace_out();
     return;
@@ -185,9 +187,16 @@ gemm_pcd_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ xp, 
       const int half = g / NJ, j = g % NJ;
 #pragma unroll
       for (int i = 0; i < MB; i++) {
-        bf16x8_t a;
-        __builtin_memcpy(&a, &cur.v[half][i], 16);
-        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bring[(g + SO) & 3], acc[i][j], 0, 0, 0);
+        if constexpr (__is_same(XT, f16_tag)) {
+          f16x8_t a, b;
+          __builtin_memcpy(&a, &cur.v[half][i], 16);
+          __builtin_memcpy(&b, &bring[(g + SO) & 3], 16);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[i][j], 0, 0, 0);
+        } else {
+          bf16x8_t a;
+          __builtin_memcpy(&a, &cur.v[half][i], 16);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bring[(g + SO) & 3], acc[i][j], 0, 0, 0);
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -226,9 +235,9 @@ gemm_pcd_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ xp, 
                                        y_dtype, bias, bias_dtype, m, n_out, n0, m0});
 }
 
-// X (m, n_in) in any activation type -> its bf16 copy in fragment order (rows past m as zeros).  A workgroup moves
-// 16 rows x 256 k: whole 128-byte lines in, whole kilobytes out.
-template <typename XT>
+// X (m, n_in) in any activation type -> its copy in fragment order as DT (bf16, or fp16 for the fp16 GEMM; rows past
+// m as zeros).  A workgroup moves 16 rows x 256 k: whole 128-byte lines in, whole kilobytes out.
+template <typename XT, typename DT = bf16_tag>
 __global__ void __launch_bounds__(256) pack_activations_kernel(const XT* __restrict__ x, uint16_t* __restrict__ xp, int m,
                                                                int n_in, int row_blocks) {
   const int t = threadIdx.x;
@@ -237,7 +246,7 @@ __global__ void __launch_bounds__(256) pack_activations_kernel(const XT* __restr
   const int row = rb * 16 + r;
   if (ks * 64 >= n_in) return;
   uint4 v[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
-  if constexpr (std::is_same<XT, bf16_tag>::value) {
+  if constexpr (std::is_same<XT, DT>::value) {
     if (row < m) {
       const uint4* src = reinterpret_cast<const uint4*>(x + (int64_t)row * n_in + ks * 64 + c2 * 16);
       v[0] = src[0];
@@ -248,8 +257,8 @@ __global__ void __launch_bounds__(256) pack_activations_kernel(const XT* __restr
     float f[16];
 #pragma unroll
     for (int i = 0; i < 16; i++) f[i] = XElem<XT>::load(src, i);
-    v[0] = make_uint4(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]), pack_bf16x2(f[6], f[7]));
-    v[1] = make_uint4(pack_bf16x2(f[8], f[9]), pack_bf16x2(f[10], f[11]), pack_bf16x2(f[12], f[13]), pack_bf16x2(f[14], f[15]));
+    v[0] = make_uint4(pack_x2<DT>(f[0], f[1]), pack_x2<DT>(f[2], f[3]), pack_x2<DT>(f[4], f[5]), pack_x2<DT>(f[6], f[7]));
+    v[1] = make_uint4(pack_x2<DT>(f[8], f[9]), pack_x2<DT>(f[10], f[11]), pack_x2<DT>(f[12], f[13]), pack_x2<DT>(f[14], f[15]));
   }
   uint8_t* dst = reinterpret_cast<uint8_t*>(xp) + ((int64_t)ks * row_blocks + rb) * 2048;
 #pragma unroll
@@ -261,9 +270,17 @@ __global__ void __launch_bounds__(256) pack_activations_kernel(const XT* __restr
 
 inline size_t packed_activation_bytes(int64_t m, int64_t n_in) { return (size_t)((m + 15) / 16) * 16 * (size_t)n_in * 2; }
 
-inline hipError_t launch_pack_activations(const void* x, int x_dtype, uint16_t* xp, int64_t m, int64_t n_in, hipStream_t s) {
+// keep_f16: fp16 activations stay fp16 (for the fp16 GEMM); everything else becomes bf16
+inline hipError_t launch_pack_activations(const void* x, int x_dtype, uint16_t* xp, int64_t m, int64_t n_in, hipStream_t s,
+                                          bool keep_f16 = false) {
   const int row_blocks = (int)((m + 15) / 16);
   const dim3 grid((unsigned)((n_in / 64 + 3) / 4), (unsigned)row_blocks), block(256);
+  if (keep_f16) {
+    if (x_dtype != kF16) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((pack_activations_kernel<f16_tag, f16_tag>), grid, block, 0, s, static_cast<const f16_tag*>(x), xp,
+                       (int)m, (int)n_in, row_blocks);
+    return hipGetLastError();
+  }
   switch (x_dtype) {
     case kBF16:
       hipLaunchKernelGGL(pack_activations_kernel<bf16_tag>, grid, block, 0, s, static_cast<const bf16_tag*>(x), xp, (int)m,
@@ -284,7 +301,7 @@ inline hipError_t launch_pack_activations(const void* x, int x_dtype, uint16_t* 
 
 // xp: the packed copy of the activations.  The caller owns the split-K workspace: sp.splits == 1 (no partials, no
 // counters) or a prepared PcSplit whose tile_wgs this function fills in.
-template <int FMT, int MB, int NJ, bool FUSE, int ABL = 0, int NC = 4>
+template <int FMT, int MB, int NJ, bool FUSE, int ABL = 0, int NC = 4, class XT = bf16_tag>
 static hipError_t launch_pcd_grid(const uint8_t* wb, const uint16_t* x, void* y, int y_dtype, const void* bias,
                                   int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, PcSplit sp, hipStream_t s) {
   constexpr int BO = FUSE ? NJ * 8 : NJ * 16, BM = NC * 16 * MB;
@@ -296,7 +313,7 @@ static hipError_t launch_pcd_grid(const uint8_t* wb, const uint16_t* x, void* y,
     nwg = (unsigned)(((n_tiles + xcds_per_mtile - 1) / xcds_per_mtile) * 8);
   }
   sp.tile_wgs = (int)nwg;
-  hipLaunchKernelGGL((gemm_pcd_kernel<NJ, FMT, MB, FUSE, ABL, NC>), dim3(nwg * (unsigned)sp.splits), dim3(pcd_threads(NC)), 0, s,
+  hipLaunchKernelGGL((gemm_pcd_kernel<NJ, FMT, MB, FUSE, ABL, NC, XT>), dim3(nwg * (unsigned)sp.splits), dim3(pcd_threads(NC)), 0, s,
                      wb, x, y, y_dtype, bias, bias_dtype, (int)m, (int)n_out, (int)n_in, n_tiles, m_tiles, xcds_per_mtile, sp);
   return hipGetLastError();
 }

@@ -100,21 +100,6 @@ __device__ __forceinline__ void fma_nibbles(uint32_t q0, uint32_t q1, float scal
   f[6] = fmaf_(s, d[0], offset); f[7] = fmaf_(s, d[1], offset);
 }
 
-typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
-typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
-__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
-  f16x2_t r;
-  r[0] = (_Float16)lo;      // round-to-nearest-even
-  r[1] = (_Float16)hi;
-  uint32_t u;
-  __builtin_memcpy(&u, &r, 4);
-  return u;
-}
-// two floats -> one dword of the activation type XT (bf16_tag / f16_tag), one rounding each
-template <class XT> __device__ __forceinline__ uint32_t pack_x2(float lo, float hi) {
-  if constexpr (std::is_same<XT, f16_tag>::value) return pack_f16x2(lo, hi);
-  else return pack_bf16x2(lo, hi);
-}
 // acc += A(16 x 32) * B(32 x 16) with both operands of the activation type
 template <class XT>
 __device__ __forceinline__ f32x4_t mfma_16x16x32(const uint32_t (&a)[4], const uint4& b, f32x4_t acc) {

@@ -40,6 +40,7 @@ enum : int {
   kRouteGemmPcBf16Copy = 25,
   kRouteGemmPcPacked = 26,
   kRouteGemmPcPackedSplitK = 27,
+  kRouteGemmPcF16 = 28,
   kRouteExl3Gemv = 30,
   kRouteExl3GemvSliced = 31,
   kRouteExl3Gemm = 32,
@@ -292,7 +293,7 @@ int64_t exl3_workspace_words();
 // the prefill GEMM for activations of any type (fp16 / fp32 are rounded to bf16 by its packing pass), and the bytes
 // of packed copy such a launch takes from the workspace
 hipError_t launch_gemm_pc_x(int format, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
-                            const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s);
+                            const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s, bool f16_native = false);
 size_t gemm_pc_packed_bytes(int64_t m, int64_t n_out, int64_t n_in, int x_dtype);
 // exact size of the partial sums a split-K launch of the prefill GEMM takes for this shape (0: not split)
 size_t gemm_pc_partials_bytes(int64_t m, int64_t n_out, int64_t n_in);

@@ -69,7 +69,7 @@ class QuantLinear:
     svh: Optional[torch.Tensor] = None    # EXL3: (out_features,) float16
     bits: int = 0
     codebook: int = _lib.CB_MCG
-    # PRECISION_F32_SCALES keeps the decode kernels for every batch; PRECISION_BF16_OK lets fp16 / fp32
+    # PRECISION_F32_SCALES keeps the decode kernels for every batch; PRECISION_BF16_OK lets fp32
     # activations be rounded to bf16 for the matrix-core GEMM
     precision: int = _lib.PRECISION_AUTO
 

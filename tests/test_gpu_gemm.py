@@ -350,9 +350,9 @@ def test_full_shape_other_formats_sampled_columns(name, n_out):
     assert rel_l2(got, want) <= TOL
 
 
-# fp16 activations have no tiled GEMM; from five rows on the operator may run the few-row kernel on
-# them, 64 rows per launch, with the weights rounded once to fp16 (11 significant bits: closer to the
-# canonical weights than the bf16 kernels).
+# fp16 activations stay fp16: from five rows on the operator may run the few-row kernel on them, 64 rows
+# per launch, and beyond 64 rows the prefill GEMM over a packed fp16 copy, both with the weights rounded once
+# to fp16 (11 significant bits: closer to the canonical weights than the bf16 kernels).
 @pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
 @pytest.mark.parametrize("m,n_out,n_in", [(5, 200, 768), (17, 4096, 512), (64, 12296, 256), (100, 1048, 1024),
                                           (200, 6144, 256)])
@@ -399,15 +399,16 @@ def test_forward_fp16_unit_vectors_give_fp16_weights_exactly(fmt):
 @pytest.mark.parametrize("xk", ["f16", "f32"])
 @pytest.mark.parametrize("m,n_out,n_in", [(256, 1048, 1024), (600, 4096, 512)])
 def test_forward_fp16_fp32_activations_many_rows_take_the_bf16_gemm_only_when_allowed(fmt, xk, m, n_out, n_in):
-    """A layer with TTQ_PRECISION_BF16_OK: from 256 rows on, fp16 and fp32 activations are rounded to bf16 into a
+    """A layer with TTQ_PRECISION_BF16_OK: from 256 rows on, fp32 activations are rounded to bf16 into a
     workspace and run the matrix-core GEMM (2e-2 class: weights and activations rounded to bf16 once); every
-    output type.  The default layer computes in the activations' own type: fp32 rows stay in the 1e-3 class."""
+    output type.  fp16 activations take the fp16 form of that GEMM whatever the layer says (nothing of them is
+    rounded).  The default layer computes in the activations' own type: fp32 rows stay in the 1e-3 class."""
     p = random_blocks(fmt, n_out * (n_in // BLOCK_WEIGHTS[fmt]), seed=900 + m)
     what = oracle.dequant(fmt, p, n_out, n_in)
     bd, bf = x_to_dev(Q.fill_normal(901, 2, 0.5, n_out), "f32")
     xd, xf = x_to_dev(Q.fill_normal(902 + m, 1, 1.0, m * n_in).reshape(m, n_in) * np.float32(0.02), xk)
     layer = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out, bias=bd, precision=F.PRECISION_BF16_OK)
-    assert layer.route(m, xd.dtype, torch.float32) == "gemm_pc_bf16_copy"
+    assert layer.route(m, xd.dtype, torch.float32) == ("gemm_pc_bf16_copy" if xk == "f32" else "gemm_pc_f16")
     want = oracle.linear_f64(what, xf, bf)
     y32 = layer.forward(xd, out_dtype=torch.float32).cpu().numpy()
     assert rel_l2(y32, want) <= TOL
@@ -426,6 +427,48 @@ def test_forward_fp16_fp32_activations_many_rows_take_the_bf16_gemm_only_when_al
     assert auto.route(m, xd.dtype, torch.float32) != "gemm_pc_bf16_copy"
     ya = auto.forward(xd, out_dtype=torch.float32).cpu().numpy()
     assert rel_l2(ya, want) <= (1e-3 if xk == "f32" else TOL)
+
+
+@pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
+@pytest.mark.parametrize("m,n_out,n_in", [(65, 1048, 1024), (300, 4096, 1024), (512, 14336, 512), (1000, 2040, 2048),
+                                          (513, 232, 4096)])
+def test_forward_fp16_activations_many_rows_fp16_gemm(fmt, m, n_out, n_in):
+    """The prefill GEMM in the activations' own type: a packed fp16 copy of X, weights rounded once to fp16, fp16
+    matrix cores, fp32 sums.  The result stays in the decode kernels' accuracy class (1e-3), every output type,
+    with bias; ragged tiles in both directions."""
+    p = random_blocks(fmt, n_out * (n_in // BLOCK_WEIGHTS[fmt]), seed=960 + m)
+    what = oracle.dequant(fmt, p, n_out, n_in)
+    bd, bf = x_to_dev(Q.fill_normal(961, 2, 0.5, n_out), "f32")
+    xd, xf = x_to_dev(Q.fill_normal(962 + m, 1, 1.0, m * n_in).reshape(m, n_in) * np.float32(0.02), "f16")
+    layer = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out, bias=bd)
+    assert layer.route(m, xd.dtype, torch.float32) in ("gemm_pc_f16", "gemm_skinny_chunked")
+    want = oracle.linear_f64(what, xf, bf)
+    y32 = layer.forward(xd, out_dtype=torch.float32).cpu().numpy()
+    assert np.isfinite(y32).all()
+    assert rel_l2(y32, want) <= 1e-3
+    for i in (0, 15, 16, 63, 64, m // 2, m - 2, m - 1):
+        assert rel_l2(y32[i], want[i]) <= 2e-3, i
+    y16 = layer.forward(xd)
+    assert y16.dtype == torch.float16 and rel_l2(oracle.f16_to_f32(dev_bits(y16)), want) <= 2e-3
+    ybf = layer.forward(xd, out_dtype=torch.bfloat16)
+    assert rel_l2(oracle.bf16_to_f32(dev_bits(ybf)), want) <= TOL
+
+
+@pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
+def test_forward_fp16_gemm_identity_activations_give_fp16_weights_exactly(fmt):
+    """X = [I; 0] through the fp16 GEMM returns every weight rounded once to fp16, bit for bit."""
+    n_in, n_out, m = 512, 1144, 512 + 40
+    p = random_blocks(fmt, n_out * (n_in // BLOCK_WEIGHTS[fmt]), seed=977)
+    what = oracle.dequant(fmt, p, n_out, n_in)
+    x = np.zeros((m, n_in), np.float32)
+    x[np.arange(n_in), np.arange(n_in)] = 1.0
+    xd, _ = x_to_dev(x, "f16")
+    layer = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out)
+    assert layer.route(m, xd.dtype, torch.float32) == "gemm_pc_f16"
+    y = layer.forward(xd, out_dtype=torch.float32).cpu().numpy()
+    want = oracle.f16_to_f32(oracle.f32_to_f16(what)).T
+    assert np.array_equal(y[:n_in], want)
+    assert not y[n_in:].any()
 
 
 @pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
@@ -449,14 +492,14 @@ def test_forward_default_precision_keeps_fp32_activations_in_the_decode_class(fm
 def test_packed_activations_in_chunks_of_8192_rows(xk):
     """More rows than one packed copy holds (8192): the operator packs and multiplies chunk after chunk through the
     same workspace.  Rows on both sides of the seam and in the short last chunk against the oracle; fp16 rows
-    reach the path through a BF16_OK layer, bf16 rows by the cost estimate of a long launch."""
+    (kept fp16 in the copy) always take a packed copy, bf16 rows by the cost estimate of a long launch."""
     m, n_out, n_in = 8192 + 130, (512 if xk == "f16" else 14336), (512 if xk == "f16" else 1024)
     p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=955)
     what = oracle.dequant(F.Q4_K, p, n_out, n_in)
     xd, xf = x_to_dev(Q.fill_normal(956, 1, 1.0, m * n_in).reshape(m, n_in) * np.float32(0.05), xk)
     layer = QuantLinear.init(packed_to_dev(p), F.Q4_K, n_in, n_out,
                              precision=F.PRECISION_BF16_OK if xk == "f16" else F.PRECISION_AUTO)
-    assert layer.route(m, xd.dtype, torch.float32) in ("gemm_pc_bf16_copy", "gemm_pc_packed")
+    assert layer.route(m, xd.dtype, torch.float32) in ("gemm_pc_f16", "gemm_pc_packed")
     y = layer.forward(xd, out_dtype=torch.float32).cpu().numpy()
     rows = [0, 1, 4095, 8190, 8191, 8192, 8193, 8192 + 64, m - 2, m - 1]
     want = oracle.linear_f64(what, xf[rows])

@@ -37,6 +37,8 @@ PINNED = [
     ("two rows of the headline shape", Q4_K, 14336, 4096, 2, BF16, F32, 0, "gemv_q4k_stream4"),
     ("three rows of the LM head", Q6_K, 128256, 4096, 3, BF16, F32, 0, "gemv_q6k_stream4"),
     ("trellis layer, prefill 512 rows", EXL3, 4096, 4096, 512, F16, F32, 3, "exl3_gemm"),
+    ("fp16 activations, prefill 512 rows of the headline shape", Q4_K, 14336, 4096, 512, F16, F16, 0, "gemm_pc_f16"),
+    ("fp16 activations, 64 rows", Q4_K, 14336, 4096, 64, F16, F16, 0, "gemm_skinny_chunked"),
     ("down projection of a 53248-wide MLP, decode", Q4_K, 16384, 53248, 1, BF16, F32, 0, "gemv_long"),
     ("fp32 activations beyond 16384 values", Q8_0, 4096, 16384 + 32, 1, F32, F32, 0, "gemv_long"),
 ]
@@ -51,12 +53,15 @@ def test_precision_flags_steer_the_route():
     # fp32 activations never leave the decode kernels by default, whatever the row count
     for m in (5, 255, 256, 600, 4096):
         assert route(Q4_K, 14336, 4096, m, F32, F32).startswith("gemv_")
-    # fp16 activations: their own few-row matrix-core kernel, never a bf16 copy
-    assert route(Q4_K, 14336, 4096, 256, F16, F16) == "gemm_skinny_chunked"
-    # only a layer that allows it rounds fp16 / fp32 activations to bf16
-    for xd in (F16, F32):
-        assert route(Q4_K, 14336, 4096, 256, xd, F32, precision=_lib.PRECISION_BF16_OK) == "gemm_pc_bf16_copy"
-        assert route(Q4_K, 14336, 4096, 255, xd, F32, precision=_lib.PRECISION_BF16_OK) != "gemm_pc_bf16_copy"
+    # fp16 activations: their own matrix-core kernels (few rows; the fp16 form of the prefill GEMM), never a bf16
+    # copy, whatever the layer allows
+    assert route(Q4_K, 14336, 4096, 40, F16, F16) == "gemm_skinny_chunked"
+    for prec in (_lib.PRECISION_AUTO, _lib.PRECISION_BF16_OK):
+        assert route(Q4_K, 14336, 4096, 256, F16, F16, precision=prec) == "gemm_pc_f16"
+    assert route(Q4_K, 14336, 4096, 256, F16, F16, precision=_lib.PRECISION_F32_SCALES).startswith("gemv_")
+    # only a layer that allows it rounds fp32 activations to bf16
+    assert route(Q4_K, 14336, 4096, 256, F32, F32, precision=_lib.PRECISION_BF16_OK) == "gemm_pc_bf16_copy"
+    assert route(Q4_K, 14336, 4096, 255, F32, F32, precision=_lib.PRECISION_BF16_OK) != "gemm_pc_bf16_copy"
     # F32_SCALES pins the decode kernels for bf16 activations too
     assert route(Q4_K, 14336, 4096, 512, BF16, BF16, precision=_lib.PRECISION_F32_SCALES).startswith("gemv_")
     assert route(EXL3, 4096, 4096, 512, F16, F32, bits=3, precision=_lib.PRECISION_F32_SCALES).startswith("exl3_gemv")
