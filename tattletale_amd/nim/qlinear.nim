@@ -20,7 +20,7 @@ type
   TtqPrecision* {.size: sizeof(cint).} = enum
     kTtqAuto = 0, kTtqF32Scales = 1, kTtqBf16Ok = 2
       ## kTtqF32Scales: decode kernels (fp32 scales) for every batch size
-      ## kTtqBf16Ok: fp16 / fp32 activations may be rounded to bf16 for the matrix-core GEMM
+      ## kTtqBf16Ok: fp32 activations may be rounded to bf16 for the matrix-core GEMM (fp16 ones have their own)
   TtqQLinear* {.bycopy.} = object      ## struct ttq_qlinear
     format*, bits*, codebook*, bias_dtype*: int32
     precision*, reserved*: int32       ## ttq_precision, 0
