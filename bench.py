@@ -433,7 +433,7 @@ def main() -> int:
         only): the attention projections as decode GEMVs (q/o 4096x4096, k/v 1024x4096, reference call
         sites workspace/transformers/src/layers/attn.nim:113-116,154-156,189), the LM-head-sized Q4_K
         stream, a Q6_K down projection (mlp.nim:60), the Q6_K LM head for 1, 2 and 4 tokens (128256x4096) and for 1 and 4 (151936x1024), the few-row decode GEMV (2, 4, 8 and 16 activation rows at once), the few-row form of the
-        prefill operator (32 rows) and the prefill GEMM for Q6_K and Q8_0 weights, 14336 x 4096 unless
+        prefill operator (32 rows), the prefill GEMM for Q6_K and Q8_0 weights and for fp16 activations, 14336 x 4096 unless
         named otherwise; the down projection at 128 and 512 rows (K split over copies of the tile grid);
         add + RMSNorm on rows of 4096."""
         n_out, n_in = 14336, 4096
@@ -500,6 +500,13 @@ def main() -> int:
             timed(nm, fmt, 512,
                   lambda ws, x, nc, y=y, fmt=fmt: (lambda i: QL.gemm(fmt, ws[i % nc], x, n_out, n_in, out=y)),
                   steps=max(20, steps // 4))
+        # fp16 activations through the operator (ttq_linear_forward): the fp16 form of the prefill GEMM -- a packed
+        # fp16 copy of the activations, weights rounded once to fp16, fp16 matrix cores
+        def f16_forward(ws, x, nc):
+            xh = (x.float() * 0.05).to(torch.float16)
+            layers = [QL.QuantLinear.init(w, F.Q4_K, n_in, n_out) for w in ws]
+            return lambda i: layers[i % nc].forward(xh)
+        timed("q4_k_forward_f16_m512", F.Q4_K, 512, f16_forward, steps=max(20, steps // 4))
         # trellis weights, 4096 x 4096 at 3 bits: 8 rows through the decode kernel (one decode of the weights
         # for all 8), 512 rows through the prefill path, and the Q4_K GEMM at the same shape beside it
         ecfg = CFG.CONFIGS["exl3_gemv"]
