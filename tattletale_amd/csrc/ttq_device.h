@@ -57,9 +57,9 @@ typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
 __device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
   asm("" : "+v"(lo));
   asm("" : "+v"(hi));
-  f16x2_t r;
-  r[0] = (_Float16)lo;
-  r[1] = (_Float16)hi;
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  const f32x2_t v = {lo, hi};
+  const f16x2_t r = __builtin_convertvector(v, f16x2_t);      // one v_cvt_pk_f16_f32
   uint32_t u;
   __builtin_memcpy(&u, &r, 4);
   return u;
