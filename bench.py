@@ -507,6 +507,13 @@ def main() -> int:
             layers = [QL.QuantLinear.init(w, F.Q4_K, n_in, n_out) for w in ws]
             return lambda i: layers[i % nc].forward(xh)
         timed("q4_k_forward_f16_m512", F.Q4_K, 512, f16_forward, steps=max(20, steps // 4))
+
+        # fp32 activations through the operator: the same GEMM over a copy scaled row by row and rounded to fp16
+        def f32_forward(ws, x, nc):
+            xf = x.float() * 0.05
+            layers = [QL.QuantLinear.init(w, F.Q4_K, n_in, n_out) for w in ws]
+            return lambda i: layers[i % nc].forward(xf)
+        timed("q4_k_forward_f32_m512", F.Q4_K, 512, f32_forward, steps=max(20, steps // 4))
         # trellis weights, 4096 x 4096 at 3 bits: 8 rows through the decode kernel (one decode of the weights
         # for all 8), 512 rows through the prefill path, and the Q4_K GEMM at the same shape beside it
         ecfg = CFG.CONFIGS["exl3_gemv"]

@@ -125,13 +125,17 @@ typedef struct ttq_qlinear {
  * run matrix-core kernels that round each dequantized weight once to bf16 (fp16) -- the 2e-2 class
  * of the GEMM entry points -- when its cost estimate prefers them for the shape.  A layer with
  * precision == TTQ_PRECISION_F32_SCALES keeps the decode kernels, and with them the 1e-3 class,
- * for every m.  The operator computes in the type of x (linear.nim:45-57): fp32 activations always
- * take the decode kernels (1e-3 class); fp16 activations those, the fp16 few-row matrix-core kernel
- * or, beyond 64 rows, the fp16 form of the prefill GEMM (a packed fp16 copy of x in a workspace,
- * weights rounded once to fp16, fp16 matrix cores: about 2e-4 measured, inside the 1e-3 class; a
- * dequantized weight beyond the fp16 range becomes an infinity there).  Only a layer with
- * precision == TTQ_PRECISION_BF16_OK lets the library round 256 or more rows of fp32 activations
- * to bf16 (into a workspace) and run the bf16 matrix-core GEMM on the copy (2e-2 class).
+ * for every m.  fp16 and fp32 activations stay in that 1e-3 class for every m by default: fp16
+ * activations take the decode kernels, the fp16 few-row matrix-core kernel or, beyond 64 rows, the
+ * fp16 form of the prefill GEMM (a packed fp16 copy of x in a workspace, weights rounded once to
+ * fp16, fp16 matrix cores: about 2e-4 measured; a dequantized weight beyond the fp16 range becomes
+ * an infinity there); fp32 activations take the decode kernels (which read them as 15-bit block
+ * fixed point) or, from five rows on, the same fp16 GEMM over a copy in which every row has been
+ * scaled by its own power of two (largest magnitude to 2^14) and rounded to fp16, the factor undone
+ * on the sums (about 2e-4 measured for rows of any magnitude; a non-finite value makes its own
+ * output row non-finite and no other).  Only a layer with precision == TTQ_PRECISION_BF16_OK lets
+ * the library round 256 or more rows of fp32 activations to bf16 and run the bf16 GEMM on the copy
+ * (2e-2 class).
  * Limits (TTQ_ERR_UNSUPPORTED beyond): TTQ_EXL3 layers take n_in <= 16384; the block formats take
  * any n_in (rows beyond 32768 values for Q4_K / Q6_K with 16-bit activations, beyond 16384 otherwise,
  * run a decode kernel that stages nothing in LDS: correct, not tuned); any m (rows are taken 65535
@@ -192,6 +196,7 @@ typedef enum {
   TTQ_ROUTE_GEMM_PC_PACKED = 26,     /* long launches: activations packed in fragment order first (takes a workspace) */
   TTQ_ROUTE_GEMM_PC_PACKED_SPLIT_K = 27,
   TTQ_ROUTE_GEMM_PC_F16 = 28,        /* fp16 activations: packed fp16 copy, weights rounded to fp16, fp16 matrix cores */
+  TTQ_ROUTE_GEMM_PC_F32_SCALED_F16 = 29, /* fp32 activations: the same over a copy scaled row by row and rounded to fp16 */
   TTQ_ROUTE_EXL3_GEMV = 30,
   TTQ_ROUTE_EXL3_GEMV_SLICED = 31,   /* K sliced over workgroups that meet in a workspace */
   TTQ_ROUTE_EXL3_GEMM = 32,

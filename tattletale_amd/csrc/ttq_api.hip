@@ -475,14 +475,25 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
     }
   }
   // fp32 activations, 256 rows or more, and only where the layer says that bf16 activations will do
-  // (TTQ_PRECISION_BF16_OK; the operator computes in the type of x otherwise): the prefill GEMM's packing pass rounds
-  // them to bf16 on the way into its workspace (weights and activations rounded to bf16: the 2e-2 class, like the
-  // GEMM entry points)
+  // (TTQ_PRECISION_BF16_OK): the prefill GEMM's packing pass rounds them to bf16 on the way into its workspace
+  // (weights and activations rounded to bf16: the 2e-2 class, like the GEMM entry points)
   if (x_dtype == TTQ_F32 && block_fmt && m >= 256 && route != 1 && n_in % 8 == 0 &&
       layer->precision == TTQ_PRECISION_BF16_OK &&
       ttq::gemm_pc_supported(layer->format, m < 8192 ? m : 8192, n_out, n_in, 112)) {
     return hip_status(ttq::launch_gemm_pc_x(layer->format, layer->qweight, x, x_dtype, y, y_dtype, layer->bias,
                                             layer->bias_dtype, m, n_out, n_in, s));
+  }
+  // fp32 activations, five rows or more: the fp16 form of the prefill GEMM over a copy in which every row has been
+  // scaled by a power of two (its largest magnitude to 2^14) and rounded to fp16, the factor undone on the sums.
+  // With the weights rounded to fp16 as well the result stays in the 1e-3 class of the decode kernels (about 2e-4
+  // measured), which take these activations as 15-bit block fixed point themselves, at a fraction of the time of
+  // their passes (14336 x 4096 at 512 rows: 2.2 ms in passes of four rows).
+  if (x_dtype == TTQ_F32 && block_fmt && m >= 5 && route != 1 &&
+      ttq::gemm_pc_supported(layer->format, m < 8192 ? m : 8192, n_out, n_in, 112)) {
+    const float us_gemm = ttq::gemm_pc_estimate_us(layer->format, m, n_out, n_in) + 5.f + (float)(m * n_in * 10) / 3.0e6f;
+    if (route == 2 || us_gemm < ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in))
+      return hip_status(ttq::launch_gemm_pc_x(layer->format, layer->qweight, x, x_dtype, y, y_dtype, layer->bias,
+                                              layer->bias_dtype, m, n_out, n_in, s, true));
   }
   return hip_status(launch_gemv_any_m(layer->format, layer->qweight, x, x_dtype, y, y_dtype, layer->bias,
                                       layer->bias_dtype, m, n_out, n_in, s));
@@ -534,6 +545,7 @@ const char* ttq_route_name(int route) {
     case TTQ_ROUTE_GEMM_PC_BF16_COPY: return "gemm_pc_bf16_copy";
     case TTQ_ROUTE_GEMM_PC_PACKED: return "gemm_pc_packed";
     case TTQ_ROUTE_GEMM_PC_F16: return "gemm_pc_f16";
+    case TTQ_ROUTE_GEMM_PC_F32_SCALED_F16: return "gemm_pc_f32_scaled_f16";
     case TTQ_ROUTE_GEMM_PC_PACKED_SPLIT_K: return "gemm_pc_packed_split_k";
     case TTQ_ROUTE_EXL3_GEMV: return "exl3_gemv";
     case TTQ_ROUTE_EXL3_GEMV_SLICED: return "exl3_gemv_sliced";
@@ -563,11 +575,9 @@ int64_t ttq_workspace_bytes(const ttq_qlinear* layer, int64_t m, int x_dtype) {
   // split along K: the prefill GEMM's exact size for every row count it can be called with here, and the few-row
   // kernel's bound (one 64 x 64 tile of sums per compute unit)
   const int64_t block_rows = m < kGemmRows ? m : kGemmRows;
-  // (fp16 activations beyond 64 rows may take the prefill GEMM over a packed fp16 copy; fp32 ones a bf16 copy where
-  // the layer allows it)
-  const int copy_dtype = (x_dtype == TTQ_F16 && m > 64) ||
-                                 (x_dtype == TTQ_F32 && layer->precision == TTQ_PRECISION_BF16_OK && m >= 256)
-                             ? x_dtype : TTQ_BF16;
+  // (fp16 activations beyond 64 rows may take the prefill GEMM over a packed fp16 copy; fp32 ones over a scaled
+  // fp16 copy, or a bf16 copy where the layer allows it)
+  const int copy_dtype = (x_dtype == TTQ_F16 && m > 64) || x_dtype == TTQ_F32 ? x_dtype : TTQ_BF16;
   int64_t scratch = ((int64_t)ttq::gemm_pc_packed_bytes(m, n_out, n_in, copy_dtype) + 255) & ~(int64_t)255;
   int64_t partials = (int64_t)ttq::device_num_cus() * (16 * 4 * (16 * 4 + 1) * 4);
   const int64_t rows[3] = {m, block_rows, m % kGemmRows};

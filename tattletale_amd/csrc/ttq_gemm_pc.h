@@ -239,10 +239,14 @@ template <> struct WFmt<kQ8_0> {
 // tile = index into launch_gemm_pc's table of tile shapes.
 hipError_t launch_gemm_packed(int format, bool fuse, int tile, const uint8_t* wb, const uint16_t* xp, void* y, int y_dtype,
                               const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, PcSplit sp,
-                              hipStream_t s, bool x_f16 = false);
+                              hipStream_t s, bool x_f16 = false, const float* row_scale = nullptr);
 size_t gemm_packed_activation_bytes(int64_t m, int64_t n_in);
 hipError_t launch_gemm_pack_activations(const void* x, int x_dtype, uint16_t* xp, int64_t m, int64_t n_in, hipStream_t s,
                                         bool keep_f16 = false);
+// fp32 activations -> fp16 in fragment order, every row scaled by a power of two that brings its largest magnitude to
+// 2^14; row_scale[row] receives the inverse factor
+hipError_t launch_gemm_pack_activations_scaled(const float* x, uint16_t* xp, float* row_scale, int64_t m, int64_t n_in,
+                                               hipStream_t s);
 
 // What a consumer wavefront does with its finished accumulators (shared by the kernels of this file and of
 // ttq_gemm_pcd.h): the meeting of the K copies, bias, silu_and_mul, rounding, and the store of Y.
@@ -255,6 +259,7 @@ struct PcEpi {
   const void* bias;
   int bias_dtype, m, n_out, n0, m0;
   const uint16_t* col_scale = nullptr;   // (ROT) fp16 scale per output column, applied after the rotation
+  const float* row_scale = nullptr;      // a factor per row of Y (the activations were scaled row by row), or none
 };
 
 // ROT (tiles of 128 columns = one Hadamard group of output channels; the trellis layer): the 128 sums of every row
@@ -268,6 +273,19 @@ __device__ __forceinline__ void pc_epilogue(f32x4_t (&acc)[MB][NJ], const PcEpi&
   void* yv = e.yv;
   const int y_dtype = e.y_dtype, bias_dtype = e.bias_dtype, m = e.m, n_out = e.n_out, n0 = e.n0, m0 = e.m0;
   const void* bias = e.bias;
+  // rows whose activations were scaled before they were rounded (fp32 activations as scaled fp16): undo it on the
+  // sums, before the copies along K meet and before the bias
+  if (e.row_scale != nullptr) {
+    const int rs4 = (lane >> 4) * 4;
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const float f = e.row_scale[min(m0 + 16 * i + rs4 + r, m - 1)];
+#pragma unroll
+        for (int j = 0; j < NJ; j++) acc[i][j][r] *= f;
+      }
+  }
   // ---- split along K: this wavefront's 64 x BN partial sums go to the workspace (whole kilobytes per store
   // instruction), a counter per (tile, consumer) says how many copies have arrived, and the wavefront that
   // arrives last adds all copies in copy order -- the same sum whichever arrives last -- and carries on to the

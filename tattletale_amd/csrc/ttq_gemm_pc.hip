@@ -8,7 +8,7 @@ namespace ttq {
 template <int FMT, int MB, int NJ, bool FUSE>
 static hipError_t launch_pc_tile(const uint8_t* wb, const uint16_t* x, void* y, int y_dtype, const void* bias,
                                  int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, int splits, int tile_if_packed,
-                                 hipStream_t s, bool x_f16 = false) {
+                                 hipStream_t s, bool x_f16 = false, const float* row_scale = nullptr) {
   PcSplit sp{1, 0, nullptr, nullptr};
   if (!FUSE && splits > 1) {
     // (the chooser has checked that the blocks of a row divide evenly and that the counters suffice)
@@ -24,7 +24,7 @@ static hipError_t launch_pc_tile(const uint8_t* wb, const uint16_t* x, void* y, 
     sp.counters = static_cast<uint32_t*>(cnt);
   }
   if (tile_if_packed >= 0)
-    return launch_gemm_packed(FMT, FUSE, tile_if_packed, wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s, x_f16);
+    return launch_gemm_packed(FMT, FUSE, tile_if_packed, wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s, x_f16, row_scale);
   return launch_pc_grid<FMT, MB, NJ, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, sp, s);
 }
 
@@ -109,15 +109,15 @@ static bool pc_use_packed(const PcChoice& c, int64_t m, int64_t n_in) {
 template <int FMT, bool FUSE>
 static hipError_t launch_pc_rows(const PcChoice& c, int tile_if_packed, const uint8_t* wb, const uint16_t* x, void* y,
                                  int y_dtype, const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
-                                 hipStream_t s, bool x_f16 = false) {
+                                 hipStream_t s, bool x_f16 = false, const float* row_scale = nullptr) {
   const int p = tile_if_packed;
   switch (c.tile) {
-    case 0: return launch_pc_tile<FMT, 4, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s, x_f16);
-    case 1: return launch_pc_tile<FMT, 4, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s, x_f16);
-    case 2: return launch_pc_tile<FMT, 2, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s, x_f16);
-    case 3: return launch_pc_tile<FMT, 2, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s, x_f16);
-    case 4: return launch_pc_tile<FMT, 1, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s, x_f16);
-    default: return launch_pc_tile<FMT, 1, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s, x_f16);
+    case 0: return launch_pc_tile<FMT, 4, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s, x_f16, row_scale);
+    case 1: return launch_pc_tile<FMT, 4, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s, x_f16, row_scale);
+    case 2: return launch_pc_tile<FMT, 2, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s, x_f16, row_scale);
+    case 3: return launch_pc_tile<FMT, 2, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s, x_f16, row_scale);
+    case 4: return launch_pc_tile<FMT, 1, 7, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s, x_f16, row_scale);
+    default: return launch_pc_tile<FMT, 1, 4, FUSE>(wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, c.splits, p, s, x_f16, row_scale);
   }
 }
 
@@ -126,7 +126,7 @@ static hipError_t launch_pc_rows(const PcChoice& c, int tile_if_packed, const ui
 template <int FMT, bool FUSE>
 static hipError_t launch_pc_fmt(const uint8_t* wb, const void* x, int x_dtype, void* y, int y_dtype, const void* bias,
                                 int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, bool force_packed, hipStream_t s,
-                                bool keep_f16 = false) {
+                                int f16_mode = 0) {      // 1: fp16 activations stay fp16; 2: fp32 activations as scaled fp16
   const PcChoice whole = pc_choose(m, n_out, n_in, FUSE);
   // (the fused gate||up form keeps the LDS-staged kernel: beside the packed kernel's three steps of A fragments its
   // epilogue does not fit the registers, and a kernel that requests registers asynchronously must never spill them)
@@ -135,17 +135,24 @@ static hipError_t launch_pc_fmt(const uint8_t* wb, const void* x, int x_dtype, v
                                      n_in, s);
   const int64_t block_rows = m < kPackRows ? m : kPackRows;
   void* ws = nullptr;
-  hipError_t e = stream_workspace(kWsPackedActivations, s, gemm_packed_activation_bytes(block_rows, n_in), &ws);
+  // (fp32 activations as scaled fp16: the rows' inverse factors follow the packed copy)
+  const size_t copy_bytes = (gemm_packed_activation_bytes(block_rows, n_in) + 255) & ~(size_t)255;
+  hipError_t e = stream_workspace(kWsPackedActivations, s, copy_bytes + (f16_mode == 2 ? (size_t)block_rows * 4 : 0), &ws);
   if (e != hipSuccess) return e;
+  float* row_scale = f16_mode == 2 ? reinterpret_cast<float*>(static_cast<char*>(ws) + copy_bytes) : nullptr;
   const int64_t xsize = x_dtype == kF32 ? 4 : 2, ysize = y_dtype == kF32 ? 4 : 2;
   for (int64_t r0 = 0; r0 < m; r0 += kPackRows) {
     const int64_t rows = m - r0 < kPackRows ? m - r0 : kPackRows;
-    e = launch_gemm_pack_activations(static_cast<const char*>(x) + r0 * n_in * xsize, x_dtype, static_cast<uint16_t*>(ws),
-                                     rows, n_in, s, keep_f16);
+    if (f16_mode == 2)
+      e = launch_gemm_pack_activations_scaled(static_cast<const float*>(x) + r0 * n_in, static_cast<uint16_t*>(ws), row_scale,
+                                              rows, n_in, s);
+    else
+      e = launch_gemm_pack_activations(static_cast<const char*>(x) + r0 * n_in * xsize, x_dtype, static_cast<uint16_t*>(ws),
+                                       rows, n_in, s, f16_mode == 1);
     if (e != hipSuccess) return e;
     const PcChoice c = rows == m ? whole : pc_choose(rows, n_out, n_in, FUSE);
     e = launch_pc_rows<FMT, FUSE>(c, c.tile, wb, static_cast<const uint16_t*>(ws), static_cast<char*>(y) + r0 * n_out * ysize,
-                                  y_dtype, bias, bias_dtype, rows, n_out, n_in, s, keep_f16);
+                                  y_dtype, bias, bias_dtype, rows, n_out, n_in, s, f16_mode != 0, row_scale);
     if (e != hipSuccess) return e;
   }
   return hipSuccess;
@@ -162,17 +169,18 @@ bool gemm_pc_supported(int format, int64_t m, int64_t n_out, int64_t n_in, int b
 }
 
 // x: bf16 activations; or (x_dtype fp16 / fp32) activations that may be rounded to bf16: those always go through the
-// packed copy, whose packing pass does the rounding; or (f16_native) fp16 activations that stay fp16: the packed copy
-// keeps them as they are and the kernel rounds the weights to fp16 and multiplies on the fp16 matrix cores.
+// packed copy, whose packing pass does the rounding; or (f16_native) the fp16 form of the kernel, which rounds the
+// weights to fp16 and multiplies on the fp16 matrix cores: fp16 activations stay as they are in the packed copy, fp32
+// activations become fp16 there after every row has been scaled by a power of two (undone in the epilogue).
 hipError_t launch_gemm_pc_x(int format, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
                             const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s,
                             bool f16_native) {
   if (m == 0 || n_out == 0) return hipSuccess;
   if (y_dtype != kBF16 && y_dtype != kF32 && y_dtype != kF16) return hipErrorInvalidValue;
-  if (f16_native && x_dtype != kF16) return hipErrorInvalidValue;
+  if (f16_native && x_dtype != kF16 && x_dtype != kF32) return hipErrorInvalidValue;
   const PcChoice c = pc_choose(m, n_out, n_in, false);
   const bool packed = x_dtype != kBF16 || pc_use_packed(c, m, n_in);
-  if (route_probe(f16_native ? kRouteGemmPcF16
+  if (route_probe(f16_native ? (x_dtype == kF32 ? kRouteGemmPcF32ScaledF16 : kRouteGemmPcF16)
                              : (x_dtype != kBF16 ? kRouteGemmPcBf16Copy
                                                  : (c.splits > 1 ? (packed ? kRouteGemmPcPackedSplitK : kRouteGemmPcSplitK)
                                                                  : (packed ? kRouteGemmPcPacked : kRouteGemmPc)))))
@@ -180,9 +188,9 @@ hipError_t launch_gemm_pc_x(int format, const void* w, const void* x, int x_dtyp
   const uint8_t* wb = static_cast<const uint8_t*>(w);
   const bool force = x_dtype != kBF16;
   switch (format) {
-    case kQ4_K: return launch_pc_fmt<kQ4_K, false>(wb, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, force, s, f16_native);
-    case kQ6_K: return launch_pc_fmt<kQ6_K, false>(wb, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, force, s, f16_native);
-    case kQ8_0: return launch_pc_fmt<kQ8_0, false>(wb, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, force, s, f16_native);
+    case kQ4_K: return launch_pc_fmt<kQ4_K, false>(wb, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, force, s, f16_native ? (x_dtype == kF32 ? 2 : 1) : 0);
+    case kQ6_K: return launch_pc_fmt<kQ6_K, false>(wb, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, force, s, f16_native ? (x_dtype == kF32 ? 2 : 1) : 0);
+    case kQ8_0: return launch_pc_fmt<kQ8_0, false>(wb, x, x_dtype, y, y_dtype, bias, bias_dtype, m, n_out, n_in, force, s, f16_native ? (x_dtype == kF32 ? 2 : 1) : 0);
     default: return hipErrorInvalidValue;
   }
 }
@@ -197,7 +205,10 @@ hipError_t launch_gemm_pc(int format, const void* w, const uint16_t* x_bf16, voi
 size_t gemm_pc_packed_bytes(int64_t m, int64_t n_out, int64_t n_in, int x_dtype) {
   if (m <= 0 || n_out <= 0 || n_in < 256) return 0;
   const bool packed = x_dtype != kBF16 || pc_use_packed(pc_choose(m, n_out, n_in, false), m, n_in);
-  return packed ? gemm_packed_activation_bytes(m < kPackRows ? m : kPackRows, n_in) : 0;
+  if (!packed) return 0;
+  const int64_t rows = m < kPackRows ? m : kPackRows;
+  // (fp32 activations: room for a factor per row behind the copy, whichever way they are narrowed)
+  return ((gemm_packed_activation_bytes(rows, n_in) + 255) & ~(size_t)255) + (x_dtype == kF32 ? (size_t)rows * 4 : 0);
 }
 
 

@@ -50,7 +50,7 @@ template <int NJ, int FMT, int MB, bool FUSE, int ABL = 0, int NC = 4, class XT 
 __global__ void __launch_bounds__(pcd_threads(NC))
 gemm_pcd_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ xp, void* __restrict__ yv,
                 int y_dtype, const void* __restrict__ bias, int bias_dtype, int m, int n_out, int n_in,
-                int n_tiles, int m_tiles, int xcds_per_mtile, PcSplit sp) {
+                int n_tiles, int m_tiles, int xcds_per_mtile, PcSplit sp, const float* __restrict__ row_scale) {
   constexpr int BN = NJ * 16;
   constexpr int kWUnits = 2 * NJ * 64;
   constexpr int kPcBM = NC * 16 * MB;
@@ -231,8 +231,10 @@ gemm_pcd_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ xp, 
   wait_vmcnt<0>();               // the re-reads past the last step
   trace_out();
 
-  pc_epilogue<NJ, MB, FUSE, NC>(acc, PcEpi{sp, ksplit, m_tile, n_tile, n_tiles, wave, lane, stg + wave * kStgBytes, yv,
-                                       y_dtype, bias, bias_dtype, m, n_out, n0, m0});
+  PcEpi epi{sp, ksplit, m_tile, n_tile, n_tiles, wave, lane, stg + wave * kStgBytes, yv, y_dtype, bias, bias_dtype, m, n_out,
+            n0, m0};
+  epi.row_scale = row_scale;
+  pc_epilogue<NJ, MB, FUSE, NC>(acc, epi);
 }
 
 // X (m, n_in) in any activation type -> its copy in fragment order as DT (bf16, or fp16 for the fp16 GEMM; rows past
@@ -266,6 +268,87 @@ __global__ void __launch_bounds__(256) pack_activations_kernel(const XT* __restr
     const int chunk = 2 * c2 + q;                                   // 8 k of the row: half chunk / 4, k-group chunk % 4
     *reinterpret_cast<uint4*>(dst + (chunk >> 2) * 1024 + ((chunk & 3) * 16 + r) * 16) = v[q];
   }
+}
+
+// fp32 X (m, n_in) -> fp16 in fragment order with a power-of-two factor per row: the row's largest magnitude lands in
+// [2^14, 2^15), so that any finite row fits fp16 and keeps its 11 bits whatever its size; inv[row] = 1 / factor for the
+// GEMM's epilogue.  A row with a non-finite value, or of zeros, is not scaled (factor 1): its non-finite values
+// convert as they are and poison that row's outputs only.  Two launches: a workgroup per row finds the factor, then
+// the packing pass of pack_activations_kernel multiplies by it.
+static __global__ void __launch_bounds__(256) row_scale_factors_kernel(const float* __restrict__ x, float* __restrict__ inv,
+                                                                       int n_in) {
+  __shared__ float part[2][4];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const float4* src = reinterpret_cast<const float4*>(x + (int64_t)blockIdx.x * n_in);
+  float amax = 0.f, bad = 0.f;
+  for (int k4 = t; k4 < n_in / 4; k4 += 256) {
+    const float4 v = src[k4];
+    const float a = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    // (fmaxf drops NaNs: look at them separately)
+    const bool ok = (__float_as_uint(a) < 0x7F800000u) && (v.x == v.x) && (v.y == v.y) && (v.z == v.z) && (v.w == v.w);
+    bad = ok ? bad : 1.f;
+    amax = fmaxf(amax, a);
+  }
+  amax = fmaxf(amax, lane_xor<1>(amax, lane)); bad = fmaxf(bad, lane_xor<1>(bad, lane));
+  amax = fmaxf(amax, lane_xor<2>(amax, lane)); bad = fmaxf(bad, lane_xor<2>(bad, lane));
+  amax = fmaxf(amax, lane_xor<4>(amax, lane)); bad = fmaxf(bad, lane_xor<4>(bad, lane));
+  amax = fmaxf(amax, lane_xor<8>(amax, lane)); bad = fmaxf(bad, lane_xor<8>(bad, lane));
+  amax = fmaxf(amax, lane_xor<16>(amax, lane)); bad = fmaxf(bad, lane_xor<16>(bad, lane));
+  amax = fmaxf(amax, lane_xor<32>(amax, lane)); bad = fmaxf(bad, lane_xor<32>(bad, lane));
+  if (lane == 0) { part[0][wave] = amax; part[1][wave] = bad; }
+  __syncthreads();
+  if (t == 0) {
+    amax = fmaxf(fmaxf(part[0][0], part[0][1]), fmaxf(part[0][2], part[0][3]));
+    bad = fmaxf(fmaxf(part[1][0], part[1][1]), fmaxf(part[1][2], part[1][3]));
+    // factor = 2^(14 - E), E the exponent of the largest magnitude (subnormal maxima count as 2^-126): biased exponent
+    // 268 - (E + 127); it stops at 2^126, so that its inverse stays a normal number: rows of tiny values are simply
+    // scaled a little less
+    const uint32_t eb = __float_as_uint(amax) >> 23, ec = eb < 1u ? 1u : eb;
+    float fi = 1.f;
+    if (bad == 0.f && amax > 0.f) {
+      const uint32_t fe = 268u - ec > 253u ? 253u : 268u - ec;
+      fi = __uint_as_float((254u - fe) << 23);
+    }
+    inv[blockIdx.x] = fi;
+  }
+}
+
+static __global__ void __launch_bounds__(256) pack_activations_scaled_kernel(const float* __restrict__ x, uint16_t* __restrict__ xp,
+                                                                             const float* __restrict__ inv, int m, int n_in,
+                                                                             int row_blocks) {
+  const int t = threadIdx.x;
+  const int rb = blockIdx.y, ks = blockIdx.x * 4 + (t >> 6);        // a wavefront per 64-k step
+  const int l = t & 63, r = l >> 2, c2 = l & 3;                     // lane: row r, chunks 2 c2 and 2 c2 + 1 of the step
+  const int row = rb * 16 + r;
+  if (ks * 64 >= n_in) return;
+  uint4 v[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+  if (row < m) {
+    // the factor from its inverse: both are powers of two
+    const float f = __uint_as_float((254u - (__float_as_uint(inv[row]) >> 23)) << 23);
+    const float4* src = reinterpret_cast<const float4*>(x + (int64_t)row * n_in + ks * 64 + c2 * 16);
+    const float4 a = src[0], b = src[1], c = src[2], d = src[3];
+    v[0] = make_uint4(pack_f16x2(a.x * f, a.y * f), pack_f16x2(a.z * f, a.w * f), pack_f16x2(b.x * f, b.y * f),
+                      pack_f16x2(b.z * f, b.w * f));
+    v[1] = make_uint4(pack_f16x2(c.x * f, c.y * f), pack_f16x2(c.z * f, c.w * f), pack_f16x2(d.x * f, d.y * f),
+                      pack_f16x2(d.z * f, d.w * f));
+  }
+  uint8_t* dst = reinterpret_cast<uint8_t*>(xp) + ((int64_t)ks * row_blocks + rb) * 2048;
+#pragma unroll
+  for (int q = 0; q < 2; q++) {
+    const int chunk = 2 * c2 + q;                                   // 8 k of the row: half chunk / 4, k-group chunk % 4
+    *reinterpret_cast<uint4*>(dst + (chunk >> 2) * 1024 + ((chunk & 3) * 16 + r) * 16) = v[q];
+  }
+}
+
+inline hipError_t launch_pack_activations_scaled(const float* x, uint16_t* xp, float* inv, int64_t m, int64_t n_in,
+                                                 hipStream_t s) {
+  const int row_blocks = (int)((m + 15) / 16);
+  hipLaunchKernelGGL(row_scale_factors_kernel, dim3((unsigned)m), dim3(256), 0, s, x, inv, (int)n_in);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  const dim3 grid((unsigned)((n_in / 64 + 3) / 4), (unsigned)row_blocks), block(256);
+  hipLaunchKernelGGL(pack_activations_scaled_kernel, grid, block, 0, s, x, xp, inv, (int)m, (int)n_in, row_blocks);
+  return hipGetLastError();
 }
 
 inline size_t packed_activation_bytes(int64_t m, int64_t n_in) { return (size_t)((m + 15) / 16) * 16 * (size_t)n_in * 2; }
@@ -303,7 +386,8 @@ inline hipError_t launch_pack_activations(const void* x, int x_dtype, uint16_t* 
 // counters) or a prepared PcSplit whose tile_wgs this function fills in.
 template <int FMT, int MB, int NJ, bool FUSE, int ABL = 0, int NC = 4, class XT = bf16_tag>
 static hipError_t launch_pcd_grid(const uint8_t* wb, const uint16_t* x, void* y, int y_dtype, const void* bias,
-                                  int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, PcSplit sp, hipStream_t s) {
+                                  int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, PcSplit sp, hipStream_t s,
+                                  const float* row_scale = nullptr) {
   constexpr int BO = FUSE ? NJ * 8 : NJ * 16, BM = NC * 16 * MB;
   const int n_tiles = (int)((n_out + BO - 1) / BO), m_tiles = (int)((m + BM - 1) / BM);
   int xcds_per_mtile = 0;
@@ -314,7 +398,8 @@ static hipError_t launch_pcd_grid(const uint8_t* wb, const uint16_t* x, void* y,
   }
   sp.tile_wgs = (int)nwg;
   hipLaunchKernelGGL((gemm_pcd_kernel<NJ, FMT, MB, FUSE, ABL, NC, XT>), dim3(nwg * (unsigned)sp.splits), dim3(pcd_threads(NC)), 0, s,
-                     wb, x, y, y_dtype, bias, bias_dtype, (int)m, (int)n_out, (int)n_in, n_tiles, m_tiles, xcds_per_mtile, sp);
+                     wb, x, y, y_dtype, bias, bias_dtype, (int)m, (int)n_out, (int)n_in, n_tiles, m_tiles, xcds_per_mtile, sp,
+                     row_scale);
   return hipGetLastError();
 }
 

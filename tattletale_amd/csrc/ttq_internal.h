@@ -41,6 +41,7 @@ enum : int {
   kRouteGemmPcPacked = 26,
   kRouteGemmPcPackedSplitK = 27,
   kRouteGemmPcF16 = 28,
+  kRouteGemmPcF32ScaledF16 = 29,
   kRouteExl3Gemv = 30,
   kRouteExl3GemvSliced = 31,
   kRouteExl3Gemm = 32,

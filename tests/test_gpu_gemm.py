@@ -472,6 +472,57 @@ def test_forward_fp16_gemm_identity_activations_give_fp16_weights_exactly(fmt):
 
 
 @pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
+@pytest.mark.parametrize("m,n_out,n_in", [(8, 4096, 4096), (65, 1048, 1024), (300, 4096, 1024), (513, 232, 4096)])
+def test_forward_fp32_activations_as_row_scaled_fp16(fmt, m, n_out, n_in):
+    """fp32 activations through the fp16 form of the prefill GEMM: every row scaled by its own power of two before it
+    is rounded to fp16, the factor undone on the sums.  Rows of very different magnitudes (1e-30 .. 1e+32) each keep
+    the 1e-3 class; a row of zeros gives zeros; a non-finite value poisons its own row and no other.  (No bias here:
+    it would swallow the rows of tiny values; test_forward_default_precision... and the fp16 tests cover it.)"""
+    p = random_blocks(fmt, n_out * (n_in // BLOCK_WEIGHTS[fmt]), seed=980 + m)
+    what = oracle.dequant(fmt, p, n_out, n_in)
+    x = Q.fill_normal(982 + m, 1, 1.0, m * n_in).reshape(m, n_in)
+    mags = np.array([1.0, 1e-30, 1e30, 3e-5, 7e4, 1e-28, 1e32, 1.0], np.float32)
+    x *= mags[np.arange(m) % 8][:, None]
+    x[1 % m, ::3] *= np.float32(1e-6)              # a wide range inside one row
+    zero_row, bad_row = 2 % m, 3 % m
+    x[zero_row] = 0.0
+    xd, xf = x_to_dev(x, "f32")
+    layer = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out)
+    routes = {layer.route(m, torch.float32, torch.float32)}
+    y = layer.forward(xd).cpu().numpy()
+    assert y.dtype == np.float32 and np.isfinite(y).all()
+    # sums of rows at 1e30 with weights of a few hundred overflow nowhere near: compare row by row, each against its own norm
+    for i in range(m):
+        want = oracle.linear_f64(what, xf[i:i + 1], None)[0]
+        got = y[i].astype(np.float64)
+        assert rel_l2(got, want) <= 1e-3 or (i == zero_row and not got.any()), (i, routes)
+    xb = x.copy()
+    xb[bad_row, 5] = np.inf
+    xb[(bad_row + 2) % m, 7] = np.nan
+    yb = layer.forward(x_to_dev(xb, "f32")[0]).cpu().numpy()
+    for i in range(m):
+        if i in (bad_row, (bad_row + 2) % m):
+            assert not np.isfinite(yb[i]).any(), i
+        else:
+            assert np.array_equal(yb[i], y[i]), i
+
+
+@pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
+def test_forward_fp32_identity_activations_give_fp16_weights_exactly(fmt):
+    n_in, n_out, m = 512, 1144, 512 + 40
+    p = random_blocks(fmt, n_out * (n_in // BLOCK_WEIGHTS[fmt]), seed=987)
+    what = oracle.dequant(fmt, p, n_out, n_in)
+    x = np.zeros((m, n_in), np.float32)
+    x[np.arange(n_in), np.arange(n_in)] = 1.0
+    xd, _ = x_to_dev(x, "f32")
+    layer = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out)
+    assert layer.route(m, torch.float32, torch.float32) == "gemm_pc_f32_scaled_f16"
+    y = layer.forward(xd).cpu().numpy()
+    assert np.array_equal(y[:n_in], oracle.f16_to_f32(oracle.f32_to_f16(what)).T)
+    assert not y[n_in:].any()
+
+
+@pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
 @pytest.mark.parametrize("m", [255, 256, 600])
 def test_forward_default_precision_keeps_fp32_activations_in_the_decode_class(fmt, m):
     """No accuracy step at 256 rows: fp32 activations through a default layer stay within 1e-3 of the oracle,

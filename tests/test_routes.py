@@ -38,6 +38,7 @@ PINNED = [
     ("three rows of the LM head", Q6_K, 128256, 4096, 3, BF16, F32, 0, "gemv_q6k_stream4"),
     ("trellis layer, prefill 512 rows", EXL3, 4096, 4096, 512, F16, F32, 3, "exl3_gemm"),
     ("fp16 activations, prefill 512 rows of the headline shape", Q4_K, 14336, 4096, 512, F16, F16, 0, "gemm_pc_f16"),
+    ("fp32 activations, prefill 512 rows of the headline shape", Q4_K, 14336, 4096, 512, F32, F32, 0, "gemm_pc_f32_scaled_f16"),
     ("fp16 activations, 64 rows", Q4_K, 14336, 4096, 64, F16, F16, 0, "gemm_skinny_chunked"),
     ("down projection of a 53248-wide MLP, decode", Q4_K, 16384, 53248, 1, BF16, F32, 0, "gemv_long"),
     ("fp32 activations beyond 16384 values", Q8_0, 4096, 16384 + 32, 1, F32, F32, 0, "gemv_long"),
@@ -50,9 +51,13 @@ def test_benchmark_and_model_shapes_reach_their_kernels(what, fmt, n_out, n_in, 
 
 
 def test_precision_flags_steer_the_route():
-    # fp32 activations never leave the decode kernels by default, whatever the row count
-    for m in (5, 255, 256, 600, 4096):
+    # fp32 activations: decode kernels for a handful of rows, then the fp16 form of the prefill GEMM over a copy
+    # scaled row by row (the 1e-3 class either way), never a bf16 copy by default
+    for m in (1, 2, 4):
         assert route(Q4_K, 14336, 4096, m, F32, F32).startswith("gemv_")
+    for m in (64, 255, 256, 600, 4096):
+        assert route(Q4_K, 14336, 4096, m, F32, F32) == "gemm_pc_f32_scaled_f16"
+        assert route(Q4_K, 14336, 4096, m, F32, F32, precision=_lib.PRECISION_F32_SCALES).startswith("gemv_")
     # fp16 activations: their own matrix-core kernels (few rows; the fp16 form of the prefill GEMM), never a bf16
     # copy, whatever the layer allows
     assert route(Q4_K, 14336, 4096, 40, F16, F16) == "gemm_skinny_chunked"
