@@ -133,21 +133,24 @@ def test_bf16_copy_route_with_a_caller_workspace():
     assert rel_l2(y.cpu().numpy(), oracle.linear_f64(oracle.dequant(F.Q4_K, p, n_out, n_in), xf)) <= 2e-2
 
 
+@pytest.mark.parametrize("xk", ["f16", "f32"])
 @pytest.mark.parametrize("m,n_out,n_in", [(300, 1048, 1024), (384, 1024, 6144)])
-def test_fp16_gemm_with_a_caller_workspace(m, n_out, n_in):
-    """fp16 activations beyond 64 rows: the packed fp16 copy (and the partial sums of a launch split along K) come out
-    of the caller's buffer; same bits as with the library's own workspace; a buffer too small for the fixed regions is refused."""
+def test_fp16_gemm_with_a_caller_workspace(m, n_out, n_in, xk):
+    """fp16 activations beyond 64 rows, fp32 activations: the packed fp16 copy (with the fp32 rows' factors behind it,
+    and the partial sums of a launch split along K) come out of the caller's buffer; same bits as with the library's
+    own workspace; a buffer too small for the fixed regions is refused."""
     p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=4500 + m)
-    xd, xf = x_to_dev(Q.fill_normal(4501, 1, 1.0, m * n_in).reshape(m, n_in) * np.float32(0.05), "f16")
+    xd, xf = x_to_dev(Q.fill_normal(4501, 1, 1.0, m * n_in).reshape(m, n_in) * np.float32(0.05), xk)
     layer = QuantLinear.init(packed_to_dev(p), F.Q4_K, n_in, n_out)
-    assert layer.route(m, torch.float16) == "gemm_pc_f16"
-    need = layer.workspace_bytes(m, torch.float16)
-    assert need >= m * n_in * 2
+    assert layer.route(m, xd.dtype) == ("gemm_pc_f16" if xk == "f16" else "gemm_pc_f32_scaled_f16")
+    need = layer.workspace_bytes(m, xd.dtype)
+    assert need >= m * n_in * 2 + (4 * m if xk == "f32" else 0)
     ws = zeros_ws(need)
     y = layer.forward(xd, workspace=ws)
     assert torch.equal(y, layer.forward(xd))
     want = oracle.linear_f64(oracle.dequant(F.Q4_K, p, n_out, n_in), xf)
-    assert rel_l2(oracle.f16_to_f32(dev_bits(y)), want) <= 2e-3
+    got = oracle.f16_to_f32(dev_bits(y)) if xk == "f16" else y.cpu().numpy()
+    assert rel_l2(got, want) <= (2e-3 if xk == "f16" else 1e-3)
     with pytest.raises(QL.TtqError) as e:
         layer.forward(xd, workspace=zeros_ws(1 << 20))
     assert e.value.status == F.ERR_WORKSPACE
