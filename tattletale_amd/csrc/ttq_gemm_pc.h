@@ -260,6 +260,7 @@ struct PcEpi {
   int bias_dtype, m, n_out, n0, m0;
   const uint16_t* col_scale = nullptr;   // (ROT) fp16 scale per output column, applied after the rotation
   const float* row_scale = nullptr;      // a factor per row of Y (the activations were scaled row by row), or none
+  bool f16_rows = false;                 // fp16 outputs leave through the staged 16-byte row stores too (the fp16 kernels)
 };
 
 // ROT (tiles of 128 columns = one Hadamard group of output channels; the trellis layer): the 128 sums of every row
@@ -438,7 +439,7 @@ __device__ __forceinline__ void pc_epilogue(f32x4_t (&acc)[MB][NJ], const PcEpi&
     }
     return;
   }
-  if ((y_dtype == kBF16 || y_dtype == kF16) && n0 + BN <= n_out && (n_out & 7) == 0) {
+  if ((y_dtype == kBF16 || ((ROT || e.f16_rows) && y_dtype == kF16)) && n0 + BN <= n_out && (n_out & 7) == 0) {
     // Full tile of bf16: transpose through the wavefront's own (now idle) X ring, so that global
     // memory sees 16-byte stores along the rows instead of 2-byte ones.  Row stride 240 bytes.
     constexpr int kRowBytes = BN * 2 + 16;
@@ -451,7 +452,7 @@ __device__ __forceinline__ void pc_epilogue(f32x4_t (&acc)[MB][NJ], const PcEpi&
 #pragma unroll
         for (int r = 0; r < 4; r++)
           *reinterpret_cast<uint16_t*>(stg + (16 * i + rb4 + r) * kRowBytes + (16 * j + cn) * 2) =
-              y_dtype == kF16 ? f32_to_f16_bits(acc[i][j][r] + bv) : f32_to_bf16_bits(acc[i][j][r] + bv);
+              ((ROT || e.f16_rows) && y_dtype == kF16) ? f32_to_f16_bits(acc[i][j][r] + bv) : f32_to_bf16_bits(acc[i][j][r] + bv);
     }
     // same wavefront wrote and reads: LDS keeps program order, no barrier needed
     uint8_t* yb = static_cast<uint8_t*>(yv);

@@ -233,7 +233,11 @@ gemm_pcd_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ xp, 
 
   PcEpi epi{sp, ksplit, m_tile, n_tile, n_tiles, wave, lane, stg + wave * kStgBytes, yv, y_dtype, bias, bias_dtype, m, n_out,
             n0, m0};
-  epi.row_scale = row_scale;
+  // (constants in the bf16 kernels, whose epilogue stays what it was)
+  if constexpr (__is_same(XT, f16_tag)) {
+    epi.row_scale = row_scale;
+    epi.f16_rows = true;
+  }
   pc_epilogue<NJ, MB, FUSE, NC>(acc, epi);
 }
 
