@@ -439,8 +439,8 @@ static hipError_t launch_long_xy(const void* w, const void* x, int x_dtype, void
   }
 }
 
-// Longest row the staged decode kernels take: the packed-dot kernel (Q4_K / Q6_K, 16-bit activations) stages 32768
-// activations in 64 KiB of LDS, everything else 16384.
+// Longest row the staged decode kernels take: the packed-dot kernel (Q4_K / Q6_K, 16-bit activations) stages 65536
+// activations in 128 KiB of LDS, everything else 16384.
 bool gemv_row_is_long(int format, int x_dtype, int64_t n_in) {
   const bool dot2 = (format == kQ4_K || format == kQ6_K) && (x_dtype == kF16 || x_dtype == kBF16);
   return n_in > (dot2 ? kMaxGemvIn16 : kMaxGemvInF32);

@@ -324,7 +324,9 @@ __device__ __forceinline__ void load_x_regs(const uint32_t* xs, int it, int lane
   }
 }
 
-template <class F, class Ops, typename YT, bool XREG>
+// BIG: rows of more than 32768 values (16 staging passes instead of 8; shorter rows keep the form with half the
+// staging registers).
+template <class F, class Ops, typename YT, bool XREG, bool BIG = false>
 __global__ void __launch_bounds__(kFastThreads)
 gemv_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, YT* __restrict__ y,
                  const void* __restrict__ bias, int bias_dtype, int n_out, int n_in, int rows_per_wave,
@@ -367,7 +369,7 @@ gemv_dot2_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x, 
   // stage x as permuted pairs: one 16-byte load (8 activations) per thread and pass,
   // all passes requested before the first is consumed
   {
-    constexpr int kMaxChunks = XREG ? 1 : (int)(kMaxGemvIn16 / kStageChunk);
+    constexpr int kMaxChunks = XREG ? 1 : (int)((BIG ? kMaxGemvIn16 : kMaxGemvIn16 / 2) / kStageChunk);
     uint4 xv[kMaxChunks];
 #pragma unroll
     for (int ch = 0; ch < kMaxChunks; ch++) {
@@ -686,10 +688,11 @@ static hipError_t launch_fmt_t(const void* w, const void* x, void* y, const void
     hipLaunchKernelGGL((gemv_dot2_kernel<F, Ops, YT, true>), grid, block, lds, s, wb, xb,
                        static_cast<YT*>(y), bias, bias_dtype, (int)n_out, (int)n_in, rows_per_wave, 0);
   else {
-    auto kernel = gemv_dot2_kernel<F, Ops, YT, false>;
-    static LargeLds configured;
+    const bool big = n_in > kMaxGemvIn16 / 2;
+    auto kernel = big ? gemv_dot2_kernel<F, Ops, YT, false, true> : gemv_dot2_kernel<F, Ops, YT, false, false>;
+    static LargeLds configured[2];
     if (lds > 64 * 1024) {
-      const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), configured);
+      const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), configured[big ? 1 : 0]);
       if (e != hipSuccess) return e;
     }
     hipLaunchKernelGGL(kernel, grid, block, lds, s, wb, xb, static_cast<YT*>(y), bias, bias_dtype, (int)n_out,

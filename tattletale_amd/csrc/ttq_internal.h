@@ -80,7 +80,7 @@ enum : int { kF32 = 0, kF16 = 1, kBF16 = 2 };
 enum : int { kQ8_0 = 0, kQ4_K = 1, kQ6_K = 2, kEXL3 = 3 };
 
 constexpr int64_t kMaxGemvInF32 = 16384;    // activations staged in 64 KiB of LDS
-constexpr int64_t kMaxGemvIn16 = 32768;
+constexpr int64_t kMaxGemvIn16 = 65536;   // 16-bit activations as staged pairs: 128 KiB of the 160 KiB of LDS
 // rows beyond what the staged decode kernels take (they go to the unstaged kernel of ttq_gemv.hip)
 bool gemv_row_is_long(int format, int x_dtype, int64_t n_in);
 

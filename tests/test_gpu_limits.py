@@ -26,9 +26,11 @@ def sampled_rows_error(fmt, p, y, xf, n_out, n_in, step, tail=64):
 
 
 @pytest.mark.parametrize("fmt,xk,n_out,n_in", [(F.Q4_K, "bf16", 8192, 28672), (F.Q4_K, "f16", 2048, 32768),
-                                               (F.Q6_K, "bf16", 4096, 28672), (F.Q6_K, "f16", 1024, 32768)])
+                                               (F.Q6_K, "bf16", 4096, 28672), (F.Q6_K, "f16", 1024, 32768),
+                                               (F.Q4_K, "bf16", 1024, 53248), (F.Q6_K, "f16", 520, 65536),
+                                               (F.Q4_K, "f16", 300, 32768 + 256)])
 @pytest.mark.parametrize("m", [1, 3])
-def test_k_quant_rows_up_to_32768_with_16bit_activations(fmt, xk, n_out, n_in, m):
+def test_k_quant_rows_up_to_65536_with_16bit_activations(fmt, xk, n_out, n_in, m):
     p = random_blocks(fmt, n_out * (n_in // 256), seed=n_in + fmt)
     xd, xf = x_to_dev(Q.fill_normal(77, m, 1.0, m * n_in).reshape(m, n_in), xk)
     y = QL.gemv(fmt, packed_to_dev(p), xd, n_out, n_in).cpu().numpy()
@@ -36,13 +38,13 @@ def test_k_quant_rows_up_to_32768_with_16bit_activations(fmt, xk, n_out, n_in, m
     assert sampled_rows_error(fmt, p, y, xf, n_out, n_in, 41) <= TOL
 
 
-@pytest.mark.parametrize("fmt,xk,n_out,n_in", [(F.Q4_K, "bf16", 1024, 53248), (F.Q4_K, "f32", 515, 16384 + 256),
-                                               (F.Q6_K, "f16", 300, 32768 + 512), (F.Q6_K, "f32", 200, 20480),
+@pytest.mark.parametrize("fmt,xk,n_out,n_in", [(F.Q4_K, "bf16", 520, 65536 + 2048), (F.Q4_K, "f32", 515, 16384 + 256),
+                                               (F.Q6_K, "f16", 300, 65536 + 512), (F.Q6_K, "f32", 200, 20480),
                                                (F.Q8_0, "bf16", 257, 16384 + 32), (F.Q8_0, "f32", 64, 40000 - 32)])
 @pytest.mark.parametrize("m", [1, 3])
 def test_rows_beyond_what_the_staged_kernels_take(fmt, xk, n_out, n_in, m):
-    """F.linear has no row-length limit (53248 inputs: the down projection of the largest dense models).  Rows beyond
-    the LDS-staged kernels take the unstaged one; a Q8_0 row of an odd number of blocks ends in half a unit."""
+    """F.linear has no row-length limit.  Rows beyond the LDS-staged kernels (65536 values for the K-quants with 16-bit
+    activations, 16384 otherwise) take the unstaged one; a Q8_0 row of an odd number of blocks ends in half a unit."""
     per = 32 if fmt == F.Q8_0 else 256
     p = random_blocks(fmt, n_out * (n_in // per), seed=n_in + fmt)
     xd, xf = x_to_dev(Q.fill_normal(78, m, 1.0, m * n_in).reshape(m, n_in), xk)

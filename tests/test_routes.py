@@ -40,7 +40,8 @@ PINNED = [
     ("fp16 activations, prefill 512 rows of the headline shape", Q4_K, 14336, 4096, 512, F16, F16, 0, "gemm_pc_f16"),
     ("fp32 activations, prefill 512 rows of the headline shape", Q4_K, 14336, 4096, 512, F32, F32, 0, "gemm_pc_f32_scaled_f16"),
     ("fp16 activations, 64 rows", Q4_K, 14336, 4096, 64, F16, F16, 0, "gemm_skinny_chunked"),
-    ("down projection of a 53248-wide MLP, decode", Q4_K, 16384, 53248, 1, BF16, F32, 0, "gemv_long"),
+    ("down projection of a 53248-wide MLP, decode", Q4_K, 16384, 53248, 1, BF16, F32, 0, "gemv_dot2"),
+    ("rows beyond 65536 values", Q4_K, 4096, 65536 + 256, 1, BF16, F32, 0, "gemv_long"),
     ("fp32 activations beyond 16384 values", Q8_0, 4096, 16384 + 32, 1, F32, F32, 0, "gemv_long"),
 ]
 
