@@ -136,10 +136,10 @@ typedef struct ttq_qlinear {
  * output row non-finite and no other).  Only a layer with precision == TTQ_PRECISION_BF16_OK lets
  * the library round 256 or more rows of fp32 activations to bf16 and run the bf16 GEMM on the copy
  * (2e-2 class).
- * Limits (TTQ_ERR_UNSUPPORTED beyond): TTQ_EXL3 layers take n_in <= 16384; the block formats take
- * any n_in (rows beyond 65536 values for Q4_K / Q6_K with 16-bit activations, beyond 16384 otherwise,
- * run a decode kernel that stages nothing in LDS: correct, not tuned); any m (rows are taken 65535
- * at a time where a kernel needs that).  m == 0 or n_out == 0 returns TTQ_OK without touching a pointer. */
+ * Limits (TTQ_ERR_UNSUPPORTED beyond): every format takes any n_in (block formats: rows beyond
+ * 65536 values for Q4_K / Q6_K with 16-bit activations, beyond 16384 otherwise, run a decode kernel
+ * that stages nothing in LDS: correct, not tuned); any m (rows are taken 65535 at a time where a
+ * kernel needs that).  m == 0 or n_out == 0 returns TTQ_OK without touching a pointer. */
 TTQ_API int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int64_t m,
                        void* y, int y_dtype, void* stream);
 

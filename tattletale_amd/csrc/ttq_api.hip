@@ -185,7 +185,7 @@ int ttq_gemv_exl3(const uint16_t* trellis, const uint16_t* suh_f16, const uint16
   if (!trellis || !suh_f16 || !svh_f16 || !x_f16 || !y) return TTQ_ERR_NULL;
   if (!aligned16(trellis) || !aligned16(x_f16) || !aligned16(y) || !aligned8(suh_f16) || !aligned8(svh_f16))
     return TTQ_ERR_ALIGN;
-  if (n_in > ttq::kMaxGemvInF32 || m > kMaxExl3GemvRows) return TTQ_ERR_UNSUPPORTED;
+  if (m > kMaxExl3GemvRows) return TTQ_ERR_UNSUPPORTED;
   return hip_status(ttq::launch_gemv_exl3(trellis, suh_f16, svh_f16, x_f16, TTQ_F16, y, TTQ_F32,
                                           nullptr, 0, m, n_out, n_in, bits, codebook,
                                           static_cast<hipStream_t>(stream)));
@@ -200,7 +200,6 @@ int ttq_gemv_exl3_noalloc(const uint16_t* trellis, const uint16_t* suh_f16, cons
   if (!trellis || !suh_f16 || !svh_f16 || !x_f16 || !y) return TTQ_ERR_NULL;
   if (!aligned16(trellis) || !aligned16(x_f16) || !aligned16(y) || !aligned8(suh_f16) || !aligned8(svh_f16))
     return TTQ_ERR_ALIGN;
-  if (n_in > ttq::kMaxGemvInF32) return TTQ_ERR_UNSUPPORTED;
   if (m > 8) return TTQ_ERR_UNSUPPORTED;        // one group of activation rows: the decode case
   const ttq::Exl3Plan plan = ttq::exl3_mfma_plan(m, n_out, n_in);
   if (plan.accum_words > ttq::exl3_resident_words()) return TTQ_ERR_UNSUPPORTED;
@@ -420,7 +419,6 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
   if (layer->format == TTQ_EXL3) {
     if (!layer->suh || !layer->svh) return TTQ_ERR_NULL;
     if (!aligned8(layer->suh) || !aligned8(layer->svh)) return TTQ_ERR_ALIGN;
-    if (n_in > ttq::kMaxGemvInF32) return TTQ_ERR_UNSUPPORTED;
     // many rows: rotate the activations once (rounded to fp16) and decode every weight once per 64 rows
     if (layer->precision != TTQ_PRECISION_F32_SCALES && ttq::gemm_exl3_preferred(m, n_out, n_in))
       return hip_status(ttq::launch_gemm_exl3(

@@ -142,15 +142,15 @@ def test_row_length_limits():
     buf = np.zeros(4096, np.uint8)
     p = buf.ctypes.data
     p += (-p) % 16
-    # the block formats take rows of any length (misalignment answers when the limits let the call through);
-    # the trellis format ends at 16384 values
+    # every format takes rows of any length (misalignment answers when the limits let the call through)
     assert L.ttq_gemv_q4_k(p, p + 2, _lib.BF16, p, 1, 16, 32768, None) == _lib.ERR_ALIGN
     assert L.ttq_gemv_q6_k(p, p + 2, _lib.F16, p, 1, 16, 28672, None) == _lib.ERR_ALIGN
     assert L.ttq_gemv_q4_k(p, p + 2, _lib.BF16, p, 1, 16, 32768 + 256, None) == _lib.ERR_ALIGN
     assert L.ttq_gemv_q4_k(p, p + 2, _lib.F32, p, 1, 16, 16384 + 256, None) == _lib.ERR_ALIGN
     assert L.ttq_gemv_q8_0(p, p + 2, _lib.BF16, p, 1, 16, 16384 + 256, None) == _lib.ERR_ALIGN
     st = QLinearStruct(format=_lib.EXL3, bits=3, codebook=1, n_out=128, n_in=16384 + 128, qweight=p, suh=p, svh=p)
-    assert L.ttq_linear_forward(C.byref(st), p, _lib.F16, 1, p, _lib.F32, None) == _lib.ERR_UNSUPPORTED
+    assert L.ttq_linear_forward(C.byref(st), p + 2, _lib.F16, 1, p, _lib.F32, None) == _lib.ERR_ALIGN
+    assert L.ttq_gemv_exl3(p, p, p, p + 2, p, 1, 128, 16384 + 128, 3, 1, None) == _lib.ERR_ALIGN
 
 
 def test_fused_rmsnorm_gemv_rejects_in_place_outputs():

@@ -102,6 +102,25 @@ def test_exl3_gemv_slicing_of_the_reduction(bits, cb, n_out, n_in, m):
         assert torch.equal(QL.gemv_exl3(*args, n_out, n_in, bits, cb), y)
 
 
+@pytest.mark.parametrize("n_out,n_in,m", [(256, 28672, 1), (128, 16384 + 128, 3), (256, 28672, 80)])
+def test_exl3_rows_beyond_16384_values(n_out, n_in, m):
+    """Rows of any length (28672: the down projection of a 70B-sized MLP): the decode kernel's slices walk them a
+    pass of 512 values at a time, the many-row form a K step at a time; no limit on n_in."""
+    bits, cb = 3, F.CB_MCG
+    w = Q.fill_normal(620, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
+    tr, suh, svh = Q.quantize_exl3(w, bits, cb, seed=5)
+    T = oracle.exl3_decode(tr, n_out, n_in, bits, cb)
+    x = Q.f32_to_f16(Q.fill_normal(621, 1, 1.0, m * n_in).reshape(m, n_in))
+    trd, sud, svd, xd = packed_to_dev(tr), bits_to_dev(suh, "f16"), bits_to_dev(svh, "f16"), bits_to_dev(x, "f16")
+    layer = QuantLinear.init(trd, F.EXL3, n_in, n_out, bits=bits, codebook=cb, suh=sud, svh=svd)
+    y = layer.forward(xd, out_dtype=torch.float32).cpu().numpy()
+    for i in sorted({0, m // 2, m - 1}):
+        assert rel_l2(y[i], oracle.exl3_gemv_f64(T, suh, svh, x[i])) <= (TOL if m <= 8 else 2e-3), i
+    if m <= 8:
+        yd = QL.gemv_exl3(trd, sud, svd, xd, n_out, n_in, bits, cb)
+        assert np.array_equal(yd.cpu().numpy(), y)
+
+
 def test_exl3_many_rows_take_whole_slices():
     """Enough (output group, row group) units to fill the GPU: no slicing, eight LDS passes per workgroup."""
     n_out, n_in, bits, m = 1024, 4096, 2, 8 * 33 + 5
