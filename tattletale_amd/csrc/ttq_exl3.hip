@@ -343,7 +343,7 @@ hipError_t launch_gemv_exl3(const uint16_t* trellis, const uint16_t* suh, const 
   if (m == 0 || n_out == 0) return hipSuccess;
   hipError_t e;
   static const int two_launches = dev_knob("TTQ_EXL3_TWO_LAUNCHES", 0);
-  if (!two_launches) {
+  if (!two_launches || n_in > kMaxGemvInF32) {      // (the two-launch form stages a whole row of activations in LDS)
     const Exl3Plan plan = exl3_mfma_plan(m, n_out, n_in);
     if (route_probe(plan.slices > 1 ? kRouteExl3GemvSliced : kRouteExl3Gemv)) return hipSuccess;
     unsigned long long* accum = nullptr;
