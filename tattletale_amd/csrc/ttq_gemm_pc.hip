@@ -96,14 +96,19 @@ float gemm_pc_estimate_us(int format, int64_t m, int64_t n_out, int64_t n_in) {
   return c * (format == kQ8_0 ? 1.9f : (format == kQ6_K ? 1.4f : 1.f)) + 2.f;
 }
 
-// Long launches read the activations from a copy in fragment order (ttq_gemm_pcd.h), made by one pass over X into
-// a workspace: the GEMM is then about a tenth faster (no X traffic through LDS), which pays for the pass (2.5 us + the
-// bytes at ~3 TB/s) from about 30 us of GEMM on.
+// Launches of 256-row tiles read the activations from a copy in fragment order (ttq_gemm_pcd.h), made by one pass
+// over X into a workspace: with no X traffic through LDS their K loop is 6 % (64-column tiles) to 15 % (112-column
+// tiles) shorter, which pays for the pass (2.5 us + the bytes at about 7 TB/s, they come out of the caches) on every
+// shape measured from 50 us of GEMM on: 4096 x 14336 at 512 rows 90.4 -> 84.6 us, at 1024 rows 150.7 -> 142.2 us,
+// 5120 x 13824 at 512 rows 102.1 -> 94.2 us, 4096 x 4096 at 1024 rows 53.8 -> 51.6 us.  Tiles of 128 and 64 rows
+// move a half and a quarter of the activation bytes per step through LDS and gain nothing from the copy (-0.5 to
+// -6 us on seven shapes, split along K or not).
 constexpr int64_t kPackRows = 8192;         // rows packed (and multiplied) at a time
 static bool pc_use_packed(const PcChoice& c, int64_t m, int64_t n_in) {
   static const int knob = dev_knob("TTQ_GEMM_PACKED", -1);      // A/B: 0 never, 1 always
   if (knob >= 0) return knob != 0;
-  return c.cost_us >= 30.f + (float)(m * n_in * 4) / 3.0e6f * 10.f;
+  (void)m; (void)n_in;
+  return kPcTiles[c.tile].mb == 4 && c.cost_us >= 45.f;
 }
 
 template <int FMT, bool FUSE>

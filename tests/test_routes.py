@@ -33,7 +33,7 @@ PINNED = [
     ("k / v projection 1024x4096, decode", Q4_K, 1024, 4096, 1, BF16, F32, 0, "gemv_dot2"),
     ("down projection 4096x14336, decode", Q4_K, 4096, 14336, 1, BF16, F32, 0, "gemv_q4k_slice"),
     ("q / o projection, prefill 512 rows", Q4_K, 4096, 4096, 512, BF16, BF16, 0, "gemm_pc"),
-    ("down projection, prefill 512 rows", Q4_K, 4096, 14336, 512, BF16, BF16, 0, "gemm_pc_split_k"),
+    ("down projection, prefill 512 rows", Q4_K, 4096, 14336, 512, BF16, BF16, 0, "gemm_pc_packed_split_k"),
     ("two rows of the headline shape", Q4_K, 14336, 4096, 2, BF16, F32, 0, "gemv_q4k_stream4"),
     ("three rows of the LM head", Q6_K, 128256, 4096, 3, BF16, F32, 0, "gemv_q6k_stream4"),
     ("trellis layer, prefill 512 rows", EXL3, 4096, 4096, 512, F16, F32, 3, "exl3_gemm"),
