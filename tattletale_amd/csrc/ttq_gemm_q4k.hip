@@ -446,15 +446,18 @@ hipError_t launch_gemm(int format, const void* w, const uint16_t* x_bf16, void* 
     if (!gemm_pc_supported(format, m, n_out, n_in, 112)) return hipErrorInvalidValue;
     return launch_gemm_pc(format, w, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   }
-  // Pick the tile width that needs the least time: rounds of tiles over the CUs times tile width.
+  // The producer/consumer kernel (ttq_gemm_pc.hip, 112- and 64-column tiles) wherever it takes the shape: it is
+  // faster than this file's single-role kernel also where 128-column tiles would save a round of workgroups
+  // (28672 x 4096 at 2048 rows: 547 us here, 420 us there).
+  if (gemm_pc_supported(kQ4_K, m, n_out, n_in, 112))
+    return launch_gemm_pc(kQ4_K, w, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+  // What is left (activations beyond 4 GiB): the tile width that needs the least time, rounds of tiles over the
+  // CUs times tile width.
   const int64_t cus = device_num_cus();
   const int64_t mt = (m + kGemmBM - 1) / kGemmBM;
   auto cost = [&](int64_t bn) { return ((((n_out + bn - 1) / bn) * mt + cus - 1) / cus) * bn; };
   static const int forced = dev_knob("TTQ_GEMM_BN", 0);
   const bool use112 = forced ? forced == 112 : cost(112) < cost(128);
-  // the producer/consumer kernel (ttq_gemm_pc.hip) exists for the 112-column tile
-  if (gemm_pc_supported(kQ4_K, m, n_out, n_in, use112 ? 112 : 128))
-    return launch_gemm_pc(kQ4_K, w, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
   const uint8_t* wb = static_cast<const uint8_t*>(w);
   TTQ_ROUTE(kRouteGemmQ4kTiles, (use112 ? launch_nj<7>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s)
                                         : launch_nj<8>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s)));

@@ -424,10 +424,12 @@ class QuantGatedMLP:
             raise TtqError(_lib.ERR_SHAPE, "QuantGatedMLP.init: hidden sizes differ")
         return cls(gate_up_proj, down_proj)
 
-    # The fused GEMM pays for the activation with quarter-rate exp2 / reciprocal in its epilogue and
-    # wins once the (rows, 2 * intermediate) tensor it saves no longer fits the caches: at
-    # 28672 x 4096 it breaks even at 512 rows and is 15 % faster at 2048.
-    FUSED_GEMM_MIN_ROWS = 512
+    # The fused GEMM saves the (rows, 2 * intermediate) tensor and its round trip, but pays for the activation
+    # with quarter-rate exp2 / reciprocal in its epilogue and reads its activations through LDS, where the
+    # plain GEMM reads a packed copy: at 28672 x 4096 the three launches are 4 to 6 % faster from 512 to
+    # 1792 rows (128 against 136 us at 512, 340 against 356 at 1536), level at 2048 (452 / 454 us), and the fused
+    # GEMM is 4 % faster at 4096 (879 against 912 us), with 235 MB less to allocate.
+    FUSED_GEMM_MIN_ROWS = 2048
     # 17..64 rows: the same entry point runs the few-row kernel with the activation in its epilogue (one
     # launch and one (rows, 2 * intermediate) round trip less); up to 16 rows the few-row GEMV passes
     # plus silu_and_mul are faster.

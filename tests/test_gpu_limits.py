@@ -104,6 +104,36 @@ def test_more_rows_than_one_grid_dimension(fmt, xk):
         assert rel_l2(yl[r], want[r]) <= 2e-2, r
 
 
+def test_gemm_on_activations_beyond_4_gib():
+    """The producer/consumer GEMM addresses the activations with 32-bit byte offsets; a Q4_K GEMM on more than 4 GiB
+    of them runs the single-role tiled kernel (64-bit row offsets).  Rows on both sides of the 4 GiB mark, the first
+    and last rows and blocks of rows in between, against float64 products on the canonical weights."""
+    n_out, n_in = 48, 256
+    mark = (1 << 32) // (n_in * 2)
+    m = mark + 300
+    p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=4096)
+    wd = packed_to_dev(p)
+    layer = QuantLinear.init(wd, F.Q4_K, n_in, n_out)
+    assert layer.route(m, torch.bfloat16) == "gemm_q4k_tiles"
+    assert layer.route(mark - 1, torch.bfloat16).startswith("gemm_pc")
+    x = torch.empty((m, n_in), dtype=torch.bfloat16, device=DEV)
+    g = torch.Generator(device=DEV).manual_seed(4097)
+    for r0 in range(0, m, 1 << 21):
+        x[r0:r0 + (1 << 21)].normal_(generator=g)
+    y = QL.gemm_q4_k(wd, x, n_out, n_in)
+    torch.cuda.synchronize()
+    w64 = torch.from_numpy(oracle.dequant(F.Q4_K, p, n_out, n_in).astype(np.float64)).to(DEV)
+    starts = [0, 256, 1 << 20, 3_000_001, mark - 300, mark - 3, mark + 40, m - 256]
+    for r0 in starts:
+        r1 = min(r0 + 256, m)
+        want = x[r0:r1].double() @ w64.T
+        got = y[r0:r1].double()
+        # (weights and sums rounded to bf16: the 2e-2 class of the GEMM entry points, row by row)
+        err = ((got - want).norm(dim=1) / want.norm(dim=1)).max().item()
+        assert err <= 2e-2, (r0, err)
+        assert ((got - want).norm() / want.norm()).item() <= 6e-3, r0
+
+
 @pytest.mark.parametrize("fmt", [F.Q8_0, F.Q4_K, F.Q6_K])
 def test_forward_of_an_empty_batch_is_an_empty_tensor(fmt):
     n_out, n_in = 64, 256
