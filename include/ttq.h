@@ -130,10 +130,10 @@ typedef struct ttq_qlinear {
  * fp16 form of the prefill GEMM (a packed fp16 copy of x in a workspace, weights rounded once to
  * fp16, fp16 matrix cores: about 2e-4 measured; a dequantized weight beyond the fp16 range becomes
  * an infinity there); fp32 activations take the decode kernels (which read them as 15-bit block
- * fixed point) or, from five rows on, the same fp16 GEMM over a copy in which every row has been
- * scaled by its own power of two (largest magnitude to 2^14) and rounded to fp16, the factor undone
- * on the sums (about 2e-4 measured for rows of any magnitude; a non-finite value makes its own
- * output row non-finite and no other).  Only a layer with precision == TTQ_PRECISION_BF16_OK lets
+ * fixed point) or, from five rows on, the same fp16 kernels (the few-row kernel, then the GEMM) over
+ * a copy in which every row has been scaled by its own power of two (largest magnitude to 2^14) and
+ * rounded to fp16, the factor undone on the sums (about 2e-4 measured for rows of any magnitude; a
+ * non-finite value makes its own output row non-finite and no other).  Only a layer with precision == TTQ_PRECISION_BF16_OK lets
  * the library round 256 or more rows of fp32 activations to bf16 and run the bf16 GEMM on the copy
  * (2e-2 class).
  * Limits (TTQ_ERR_UNSUPPORTED beyond): every format takes any n_in (block formats: rows beyond
@@ -187,11 +187,12 @@ typedef enum {
   TTQ_ROUTE_GEMV_DOT2_MULTI = 13,
   TTQ_ROUTE_GEMV_GENERIC = 14,
   TTQ_ROUTE_GEMV_LONG = 15,          /* rows longer than the staged kernels take: nothing staged in LDS */
+  TTQ_ROUTE_GEMM_SKINNY_F32_SCALED_F16 = 19, /* fp32 activations, few rows: the few-row kernel in fp16 over a copy scaled row by row */
   TTQ_ROUTE_GEMM_PC = 20,            /* producer / consumer prefill GEMM */
   TTQ_ROUTE_GEMM_PC_SPLIT_K = 21,    /* ... in several copies along K (takes a workspace) */
   TTQ_ROUTE_GEMM_SKINNY = 22,        /* 17-64 rows */
   TTQ_ROUTE_GEMM_SKINNY_CHUNKED = 23,
-  TTQ_ROUTE_GEMM_Q4K_TILES = 24,     /* single-role tiled kernel (128-column tiles, activations beyond 4 GiB) */
+  TTQ_ROUTE_GEMM_Q4K_TILES = 24,     /* single-role tiled kernel: more than 4 GiB of activations */
   TTQ_ROUTE_GEMM_PC_BF16_COPY = 25,  /* TTQ_PRECISION_BF16_OK: fp32 activations rounded to bf16 by the packing pass */
   TTQ_ROUTE_GEMM_PC_PACKED = 26,     /* long launches: activations packed in fragment order first (takes a workspace) */
   TTQ_ROUTE_GEMM_PC_PACKED_SPLIT_K = 27,

@@ -24,6 +24,7 @@ ROUTE = {
     "none": 0, "gemv_q4k_stream": 1, "gemv_q4k_stream4": 2, "gemv_q4k_slice": 3, "gemv_q4k_batch4": 4,
     "gemv_q4k_batch": 5, "gemv_q4k_mfma": 6, "gemv_q6k_stream": 7, "gemv_q6k_stream4": 8, "gemv_q8_stream": 9,
     "gemv_q8_win": 10, "gemv_q8_mfma": 11, "gemv_dot2": 12, "gemv_dot2_multi": 13, "gemv_generic": 14, "gemv_long": 15,
+    "gemm_skinny_f32_scaled_f16": 19,
     "gemm_pc": 20, "gemm_pc_split_k": 21, "gemm_skinny": 22, "gemm_skinny_chunked": 23, "gemm_q4k_tiles": 24,
     "gemm_pc_bf16_copy": 25, "gemm_pc_packed": 26, "gemm_pc_packed_split_k": 27, "gemm_pc_f16": 28, "gemm_pc_f32_scaled_f16": 29, "exl3_gemv": 30, "exl3_gemv_sliced": 31, "exl3_gemm": 32, "exl3_gemv_two_launches": 33,
 }

@@ -462,7 +462,9 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
     if (m > 64 && ttq::gemm_pc_supported(layer->format, m < 8192 ? m : 8192, n_out, n_in, 112))
       us_gemm = ttq::gemm_pc_estimate_us(layer->format, m, n_out, n_in) + 2.5f + (float)(m * n_in * 4) / 3.0e6f;
     const float us_gemv = ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in);
-    if (us_gemm < us_few && (route == 2 || us_gemm < us_gemv))
+    // (several launches of the few-row kernel against one short round of the tiled kernel: the margin of the bf16
+    // chooser, whose estimate for the tiled kernel is fitted to full rounds and about a third too high for a short one)
+    if (us_gemm < (m > 64 ? us_few / 0.65f : us_few) && (route == 2 || us_gemm < us_gemv))
       return hip_status(ttq::launch_gemm_pc_x(layer->format, layer->qweight, x, x_dtype, y, y_dtype, layer->bias,
                                               layer->bias_dtype, m, n_out, n_in, s, true));
     if (us_few < 1e29f && (route == 2 || us_few < us_gemv)) {
@@ -486,10 +488,24 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
   // With the weights rounded to fp16 as well the result stays in the 1e-3 class of the decode kernels (about 2e-4
   // measured), which take these activations as 15-bit block fixed point themselves, at a fraction of the time of
   // their passes (14336 x 4096 at 512 rows: 2.2 ms in passes of four rows).
-  if (x_dtype == TTQ_F32 && block_fmt && m >= 5 && route != 1 &&
-      ttq::gemm_pc_supported(layer->format, m < 8192 ? m : 8192, n_out, n_in, 112)) {
-    const float us_gemm = ttq::gemm_pc_estimate_us(layer->format, m, n_out, n_in) + 5.f + (float)(m * n_in * 10) / 3.0e6f;
-    if (route == 2 || us_gemm < ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in))
+  // A few rows take the few-row kernel in fp16 over a row-major copy scaled the same way (one pass of a workgroup
+  // per row, 2.5 us), as fp16 activations do: 14336 x 4096 at 8 rows 15 us against 28 us of the GEMM.
+  if (x_dtype == TTQ_F32 && block_fmt && m >= 5 && route != 1) {
+    float us_few = 1e30f, us_gemm = 1e30f;
+    if (ttq::gemm_skinny_supported(layer->format, m < 64 ? m : 64, n_out, n_in)) {
+      const int64_t full = m / 64, rest = m % 64;
+      us_few = (float)full * ttq::gemm_skinny_estimate_us(layer->format, 64, n_out, n_in) + 2.5f + (float)(m * n_in * 6) / 3.0e6f;
+      if (rest) us_few += ttq::gemm_skinny_estimate_us(layer->format, rest, n_out, n_in);
+    }
+    if (ttq::gemm_pc_supported(layer->format, m < 8192 ? m : 8192, n_out, n_in, 112))
+      us_gemm = ttq::gemm_pc_estimate_us(layer->format, m, n_out, n_in) + 5.f + (float)(m * n_in * 10) / 3.0e6f;
+    const float us_gemv = ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in);
+    if ((m > 64 ? us_few / 0.65f : us_few) < us_gemm && (route == 2 || us_few < us_gemv)) {
+      if (ttq::route_probe(ttq::kRouteGemmSkinnyF32ScaledF16)) return TTQ_OK;
+      return hip_status(ttq::launch_gemm_skinny_f32(layer->format, layer->qweight, static_cast<const float*>(x), y, y_dtype,
+                                                    layer->bias, layer->bias_dtype, m, n_out, n_in, s));
+    }
+    if (us_gemm < 1e29f && (route == 2 || us_gemm < us_gemv))
       return hip_status(ttq::launch_gemm_pc_x(layer->format, layer->qweight, x, x_dtype, y, y_dtype, layer->bias,
                                               layer->bias_dtype, m, n_out, n_in, s, true));
   }
@@ -535,6 +551,7 @@ const char* ttq_route_name(int route) {
     case TTQ_ROUTE_GEMV_DOT2_MULTI: return "gemv_dot2_multi";
     case TTQ_ROUTE_GEMV_GENERIC: return "gemv_generic";
     case TTQ_ROUTE_GEMV_LONG: return "gemv_long";
+    case TTQ_ROUTE_GEMM_SKINNY_F32_SCALED_F16: return "gemm_skinny_f32_scaled_f16";
     case TTQ_ROUTE_GEMM_PC: return "gemm_pc";
     case TTQ_ROUTE_GEMM_PC_SPLIT_K: return "gemm_pc_split_k";
     case TTQ_ROUTE_GEMM_SKINNY: return "gemm_skinny";

@@ -197,6 +197,53 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// fp32 activations for the fp16 matrix cores: the power of two that brings a row's largest magnitude to 2^14 (the row
+// then fits fp16 with room for sums of its neighbours, and values down to 2^-38 of the largest stay normal numbers).
+// Called by all 256 threads of a workgroup with the row (n_in a multiple of 4, 16-byte aligned) and 9 floats of LDS;
+// returns the INVERSE of the factor to every thread.  A row with a non-finite value, or of zeros, is not scaled (1):
+// its non-finite values convert as they are and poison that row's outputs only.
+__device__ __forceinline__ float block_row_inverse_factor(const float* __restrict__ row, int n_in, float* part) {
+  const int t = (int)threadIdx.x, lane = t & 63, wave = t >> 6;
+  const float4* src = reinterpret_cast<const float4*>(row);
+  float amax = 0.f, bad = 0.f;
+  for (int k4 = t; k4 < n_in / 4; k4 += 256) {
+    const float4 v = src[k4];
+    const float a = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    // (fmaxf drops NaNs: look at them separately)
+    const bool ok = (__float_as_uint(a) < 0x7F800000u) && (v.x == v.x) && (v.y == v.y) && (v.z == v.z) && (v.w == v.w);
+    bad = ok ? bad : 1.f;
+    amax = fmaxf(amax, a);
+  }
+  amax = fmaxf(amax, lane_xor<1>(amax, lane)); bad = fmaxf(bad, lane_xor<1>(bad, lane));
+  amax = fmaxf(amax, lane_xor<2>(amax, lane)); bad = fmaxf(bad, lane_xor<2>(bad, lane));
+  amax = fmaxf(amax, lane_xor<4>(amax, lane)); bad = fmaxf(bad, lane_xor<4>(bad, lane));
+  amax = fmaxf(amax, lane_xor<8>(amax, lane)); bad = fmaxf(bad, lane_xor<8>(bad, lane));
+  amax = fmaxf(amax, lane_xor<16>(amax, lane)); bad = fmaxf(bad, lane_xor<16>(bad, lane));
+  amax = fmaxf(amax, lane_xor<32>(amax, lane)); bad = fmaxf(bad, lane_xor<32>(bad, lane));
+  if (lane == 0) { part[wave] = amax; part[4 + wave] = bad; }
+  __syncthreads();
+  if (t == 0) {
+    amax = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
+    bad = fmaxf(fmaxf(part[4], part[5]), fmaxf(part[6], part[7]));
+    // factor = 2^(14 - E), E the exponent of the largest magnitude (subnormal maxima count as 2^-126): biased exponent
+    // 268 - (E + 127); it stops at 2^126, so that its inverse stays a normal number: rows of tiny values are simply
+    // scaled a little less
+    const uint32_t eb = __float_as_uint(amax) >> 23, ec = eb < 1u ? 1u : eb;
+    float fi = 1.f;
+    if (bad == 0.f && amax > 0.f) {
+      const uint32_t fe = 268u - ec > 253u ? 253u : 268u - ec;
+      fi = __uint_as_float((254u - fe) << 23);
+    }
+    part[8] = fi;
+  }
+  __syncthreads();
+  return part[8];
+}
+// the factor from its inverse: both are powers of two
+__device__ __forceinline__ float row_factor_of_inverse(float inv) {
+  return __uint_as_float((254u - (__float_as_uint(inv) >> 23)) << 23);
+}
+
 // Q4_K: 6-bit scale and min of sub-block j (0..7) from the 12 packed bytes held as three
 // little-endian dwords s0 (bytes 0-3), s1 (4-7), s2 (8-11).
 __device__ __forceinline__ void q4k_scale_min(uint32_t s0, uint32_t s1, uint32_t s2, int j,

@@ -281,40 +281,9 @@ __global__ void __launch_bounds__(256) pack_activations_kernel(const XT* __restr
 // the packing pass of pack_activations_kernel multiplies by it.
 static __global__ void __launch_bounds__(256) row_scale_factors_kernel(const float* __restrict__ x, float* __restrict__ inv,
                                                                        int n_in) {
-  __shared__ float part[2][4];
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  const float4* src = reinterpret_cast<const float4*>(x + (int64_t)blockIdx.x * n_in);
-  float amax = 0.f, bad = 0.f;
-  for (int k4 = t; k4 < n_in / 4; k4 += 256) {
-    const float4 v = src[k4];
-    const float a = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    // (fmaxf drops NaNs: look at them separately)
-    const bool ok = (__float_as_uint(a) < 0x7F800000u) && (v.x == v.x) && (v.y == v.y) && (v.z == v.z) && (v.w == v.w);
-    bad = ok ? bad : 1.f;
-    amax = fmaxf(amax, a);
-  }
-  amax = fmaxf(amax, lane_xor<1>(amax, lane)); bad = fmaxf(bad, lane_xor<1>(bad, lane));
-  amax = fmaxf(amax, lane_xor<2>(amax, lane)); bad = fmaxf(bad, lane_xor<2>(bad, lane));
-  amax = fmaxf(amax, lane_xor<4>(amax, lane)); bad = fmaxf(bad, lane_xor<4>(bad, lane));
-  amax = fmaxf(amax, lane_xor<8>(amax, lane)); bad = fmaxf(bad, lane_xor<8>(bad, lane));
-  amax = fmaxf(amax, lane_xor<16>(amax, lane)); bad = fmaxf(bad, lane_xor<16>(bad, lane));
-  amax = fmaxf(amax, lane_xor<32>(amax, lane)); bad = fmaxf(bad, lane_xor<32>(bad, lane));
-  if (lane == 0) { part[0][wave] = amax; part[1][wave] = bad; }
-  __syncthreads();
-  if (t == 0) {
-    amax = fmaxf(fmaxf(part[0][0], part[0][1]), fmaxf(part[0][2], part[0][3]));
-    bad = fmaxf(fmaxf(part[1][0], part[1][1]), fmaxf(part[1][2], part[1][3]));
-    // factor = 2^(14 - E), E the exponent of the largest magnitude (subnormal maxima count as 2^-126): biased exponent
-    // 268 - (E + 127); it stops at 2^126, so that its inverse stays a normal number: rows of tiny values are simply
-    // scaled a little less
-    const uint32_t eb = __float_as_uint(amax) >> 23, ec = eb < 1u ? 1u : eb;
-    float fi = 1.f;
-    if (bad == 0.f && amax > 0.f) {
-      const uint32_t fe = 268u - ec > 253u ? 253u : 268u - ec;
-      fi = __uint_as_float((254u - fe) << 23);
-    }
-    inv[blockIdx.x] = fi;
-  }
+  __shared__ float part[9];
+  const float fi = block_row_inverse_factor(x + (int64_t)blockIdx.x * n_in, n_in, part);
+  if (threadIdx.x == 0) inv[blockIdx.x] = fi;
 }
 
 static __global__ void __launch_bounds__(256) pack_activations_scaled_kernel(const float* __restrict__ x, uint16_t* __restrict__ xp,
@@ -327,8 +296,7 @@ static __global__ void __launch_bounds__(256) pack_activations_scaled_kernel(con
   if (ks * 64 >= n_in) return;
   uint4 v[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
   if (row < m) {
-    // the factor from its inverse: both are powers of two
-    const float f = __uint_as_float((254u - (__float_as_uint(inv[row]) >> 23)) << 23);
+    const float f = row_factor_of_inverse(inv[row]);
     const float4* src = reinterpret_cast<const float4*>(x + (int64_t)row * n_in + ks * 64 + c2 * 16);
     const float4 a = src[0], b = src[1], c = src[2], d = src[3];
     v[0] = make_uint4(pack_f16x2(a.x * f, a.y * f), pack_f16x2(a.z * f, a.w * f), pack_f16x2(b.x * f, b.y * f),

@@ -295,6 +295,7 @@ struct SkSplit {
   int tiles;           // workgroups of one copy
   float* partials;
   uint32_t* counters;  // one per tile, zero between launches
+  const float* row_scale;   // or null: a factor per token on the sums, before the bias (activations that were scaled row by row)
 };
 constexpr int kSkMaxCounters = 16384;
 
@@ -483,6 +484,7 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
     const int col = n0 + 8 * g;
     if (tok >= m || col >= n_out) continue;      // n_out is a multiple of 8: a group is all in or all out
     float v[8];
+    const float rs = !FUSE && sp.row_scale ? sp.row_scale[tok] : 1.f;
     if constexpr (FUSE) {
       // outputs 8g .. 8g+7 of the workgroup: gate in row block 2 * (g / 2), up in the next one
       const int lr = 32 * (g >> 1) + 8 * (g & 1);
@@ -495,7 +497,7 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
       }
     } else {
 #pragma unroll
-      for (int k = 0; k < 8; k++) v[k] = tile[tok * kTileLd + 8 * g + k] + load_bias(bias, bias_dtype, col + k);
+      for (int k = 0; k < 8; k++) v[k] = tile[tok * kTileLd + 8 * g + k] * rs + load_bias(bias, bias_dtype, col + k);
     }
     const int64_t o = (int64_t)tok * n_out + col;
     if (y_dtype == kBF16) {
@@ -515,7 +517,8 @@ gemm_skinny_kernel(const uint8_t* __restrict__ w, const uint16_t* __restrict__ x
 // n_out counts outputs: weight rows, or gate/up pairs when fused.
 template <int RB, int TB, bool FUSE, class K>
 hipError_t launch_skinny_k(K kernel, const uint8_t* w, const uint16_t* x, void* y, int y_dtype, const void* bias,
-                           int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, int splits, hipStream_t s) {
+                           int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, int splits, hipStream_t s,
+                           const float* row_scale) {
   const size_t lds = (size_t)(kSkWaves * RB * TB * 4 * 64 + 16 * TB * (16 * RB + 1)) * sizeof(float);
   static LargeLds configured;          // one per kernel instantiation: K is part of this function's type
   if (lds > 64 * 1024) {
@@ -524,7 +527,7 @@ hipError_t launch_skinny_k(K kernel, const uint8_t* w, const uint16_t* x, void* 
   }
   constexpr int kOutPerWg = FUSE ? 8 * RB : 16 * RB;
   const int tiles = (int)((n_out + kOutPerWg - 1) / kOutPerWg);
-  SkSplit sp{1, tiles, nullptr, nullptr};
+  SkSplit sp{1, tiles, nullptr, nullptr, row_scale};
   if (!FUSE && splits > 1) {
     // (the chooser has checked that the super-blocks divide evenly and that the counters suffice)
     void* part = nullptr;
@@ -543,9 +546,10 @@ hipError_t launch_skinny_k(K kernel, const uint8_t* w, const uint16_t* x, void* 
 
 template <class WF, class XT, int RB, int TB, int WD, int XB, bool FUSE>
 hipError_t launch_skinny_tb(const uint8_t* w, const uint16_t* x, void* y, int y_dtype, const void* bias,
-                            int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, int splits, hipStream_t s) {
+                            int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, int splits, hipStream_t s,
+                            const float* row_scale) {
   return launch_skinny_k<RB, TB, FUSE>(gemm_skinny_kernel<WF, XT, RB, TB, WD, XB, FUSE>, w, x, y, y_dtype, bias,
-                                       bias_dtype, m, n_out, n_in, splits, s);
+                                       bias_dtype, m, n_out, n_in, splits, s, row_scale);
 }
 
 // Cost model (microseconds), a least-squares fit to 4096 x 4096, 4096 x 14336 and 14336 x 4096 with
@@ -601,13 +605,13 @@ SkChoice skinny_choose(int format, int64_t m, int64_t rows, int64_t n_in, bool f
 template <class WF, class XT, bool FUSE>
 hipError_t launch_skinny_fmt(int format, const uint8_t* wb, const uint16_t* x_bf16, void* y, int y_dtype,
                              const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
-                             hipStream_t s) {
+                             hipStream_t s, const float* row_scale = nullptr) {
   const SkChoice ch = skinny_choose(format, m, FUSE ? 2 * n_out : n_out, n_in, FUSE);
   const int rb = ch.rb;
   const int tb = (int)((m + 15) / 16);
 #define TTQ_SK_CASE(RBv, TBv, WDv, XBv) \
   if (rb == RBv && tb == TBv)            \
-    return launch_skinny_tb<WF, XT, RBv, TBv, WDv, XBv, FUSE>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, ch.splits, s);
+    return launch_skinny_tb<WF, XT, RBv, TBv, WDv, XBv, FUSE>(wb, x_bf16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, ch.splits, s, row_scale);
   TTQ_SK_CASE(4, 1, 4, 2) TTQ_SK_CASE(4, 2, 4, 2) TTQ_SK_CASE(4, 3, 2, 1) TTQ_SK_CASE(4, 4, 2, 1)
   TTQ_SK_CASE(2, 1, 4, 2) TTQ_SK_CASE(2, 2, 4, 2) TTQ_SK_CASE(2, 3, 2, 1) TTQ_SK_CASE(2, 4, 2, 1)
   if constexpr (!FUSE) {
@@ -652,11 +656,12 @@ hipError_t launch_gemm_skinny_silu_mul(const void* w, const uint16_t* x_bf16, vo
 
 hipError_t launch_gemm_skinny(int format, const void* w, const uint16_t* x, int x_dtype, void* y, int y_dtype,
                               const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
-                              hipStream_t s) {
+                              hipStream_t s, const float* row_scale) {
   if (m == 0 || n_out == 0) return hipSuccess;
   if (y_dtype != kBF16 && y_dtype != kF32 && y_dtype != kF16) return hipErrorInvalidValue;
   const uint8_t* wb = static_cast<const uint8_t*>(w);
   if (x_dtype == kBF16) {
+    if (row_scale) return hipErrorInvalidValue;      // (row factors come with the scaled fp16 copy of fp32 activations)
     switch (format) {
       case kQ4_K: return launch_skinny_fmt<SkQ4K, bf16_tag, false>(format, wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
       case kQ6_K: return launch_skinny_fmt<SkQ6K, bf16_tag, false>(format, wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
@@ -666,28 +671,60 @@ hipError_t launch_gemm_skinny(int format, const void* w, const uint16_t* x, int 
   }
   if (x_dtype == kF16) {
     switch (format) {
-      case kQ4_K: return launch_skinny_fmt<SkQ4K, f16_tag, false>(format, wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-      case kQ6_K: return launch_skinny_fmt<SkQ6K, f16_tag, false>(format, wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
-      case kQ8_0: return launch_skinny_fmt<SkQ8_0, f16_tag, false>(format, wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s);
+      case kQ4_K: return launch_skinny_fmt<SkQ4K, f16_tag, false>(format, wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s, row_scale);
+      case kQ6_K: return launch_skinny_fmt<SkQ6K, f16_tag, false>(format, wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s, row_scale);
+      case kQ8_0: return launch_skinny_fmt<SkQ8_0, f16_tag, false>(format, wb, x, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s, row_scale);
       default: return hipErrorInvalidValue;
     }
   }
   return hipErrorInvalidValue;
 }
 
-// More than 64 rows of fp16 activations, for which no tiled GEMM exists: one launch per 64 rows.
+// More than 64 rows: one launch per 64 rows.
 hipError_t launch_gemm_skinny_chunked(int format, const void* w, const uint16_t* x, int x_dtype, void* y, int y_dtype,
                                       const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
-                                      hipStream_t s) {
+                                      hipStream_t s, const float* row_scale) {
   const int64_t ysize = y_dtype == kF32 ? 4 : 2;
   for (int64_t r0 = 0; r0 < m; r0 += 64) {
     const int64_t rows = m - r0 < 64 ? m - r0 : 64;
     const hipError_t e = launch_gemm_skinny(format, w, x + r0 * n_in, x_dtype,
                                             static_cast<uint8_t*>(y) + r0 * n_out * ysize, y_dtype, bias, bias_dtype,
-                                            rows, n_out, n_in, s);
+                                            rows, n_out, n_in, s, row_scale ? row_scale + r0 : nullptr);
     if (e != hipSuccess) return e;
   }
   return hipSuccess;
+}
+
+// fp32 activations: every row scaled by a power of two (its largest magnitude to 2^14) and rounded to fp16, row-major,
+// with the inverse factors behind the copy; the fp16 kernel multiplies its sums by them.  One workgroup per row.
+static __global__ void __launch_bounds__(256) scale_rows_f16_kernel(const float* __restrict__ x, uint16_t* __restrict__ xs,
+                                                                    float* __restrict__ inv, int n_in) {
+  __shared__ float part[9];
+  const float* row = x + (int64_t)blockIdx.x * n_in;
+  const float fi = block_row_inverse_factor(row, n_in, part);
+  const float f = row_factor_of_inverse(fi);
+  const float4* src = reinterpret_cast<const float4*>(row);
+  uint2* dst = reinterpret_cast<uint2*>(xs + (int64_t)blockIdx.x * n_in);
+  for (int k4 = (int)threadIdx.x; k4 < n_in / 4; k4 += 256) {
+    const float4 v = src[k4];
+    dst[k4] = make_uint2(pack_f16x2(v.x * f, v.y * f), pack_f16x2(v.z * f, v.w * f));
+  }
+  if (threadIdx.x == 0) inv[blockIdx.x] = fi;
+}
+
+hipError_t launch_gemm_skinny_f32(int format, const void* w, const float* x, void* y, int y_dtype, const void* bias,
+                                  int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s) {
+  if (m == 0 || n_out == 0) return hipSuccess;
+  void* ws = nullptr;
+  const size_t copy_bytes = ((size_t)m * (size_t)n_in * 2 + 255) & ~(size_t)255;
+  hipError_t e = stream_workspace(kWsPackedActivations, s, copy_bytes + (size_t)m * 4, &ws);
+  if (e != hipSuccess) return e;
+  uint16_t* xs = static_cast<uint16_t*>(ws);
+  float* inv = reinterpret_cast<float*>(static_cast<char*>(ws) + copy_bytes);
+  hipLaunchKernelGGL(scale_rows_f16_kernel, dim3((unsigned)m), dim3(256), 0, s, x, xs, inv, (int)n_in);
+  e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  return launch_gemm_skinny_chunked(format, w, xs, kF16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s, inv);
 }
 
 }  // namespace ttq

@@ -32,6 +32,7 @@ enum : int {
   kRouteGemvDot2Multi = 13,
   kRouteGemvGeneric = 14,
   kRouteGemvLong = 15,
+  kRouteGemmSkinnyF32ScaledF16 = 19,
   kRouteGemmPc = 20,
   kRouteGemmPcSplitK = 21,
   kRouteGemmSkinny = 22,
@@ -224,13 +225,18 @@ hipError_t allow_large_lds(const void* kernel, LargeLds& state);
 bool gemm_skinny_supported(int format, int64_t m, int64_t n_out, int64_t n_in);
 float gemm_skinny_estimate_us(int format, int64_t m, int64_t n_out, int64_t n_in);
 // x: bf16 or fp16 activations (the weights are rounded once to the same type); y: bf16, fp16 or fp32.
+// row_scale (fp16 activations only): a factor per row on the sums, before the bias.
 hipError_t launch_gemm_skinny(int format, const void* w, const uint16_t* x, int x_dtype, void* y, int y_dtype,
                               const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
-                              hipStream_t s);
-// Any number of rows, 64 per launch (fp16 activations have no tiled GEMM).
+                              hipStream_t s, const float* row_scale = nullptr);
+// Any number of rows, 64 per launch.
 hipError_t launch_gemm_skinny_chunked(int format, const void* w, const uint16_t* x, int x_dtype, void* y, int y_dtype,
                                       const void* bias, int bias_dtype, int64_t m, int64_t n_out, int64_t n_in,
-                                      hipStream_t s);
+                                      hipStream_t s, const float* row_scale = nullptr);
+// fp32 activations: a copy scaled row by row to fp16 range (a power of two per row, undone on the sums) in the
+// stream's workspace, then the fp16 kernel, 64 rows per launch.
+hipError_t launch_gemm_skinny_f32(int format, const void* w, const float* x, void* y, int y_dtype, const void* bias,
+                                  int bias_dtype, int64_t m, int64_t n_out, int64_t n_in, hipStream_t s);
 
 // The same kernel with the fused gate||up weight (2 * n_ff rows, gate rows first) and silu_and_mul
 // in its epilogue: y is (m, n_ff).  Q4_K.

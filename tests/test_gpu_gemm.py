@@ -23,7 +23,7 @@ BLOCK_WEIGHTS = {F.Q8_0: 32, F.Q4_K: 256, F.Q6_K: 256}      # weights per packed
 @pytest.mark.parametrize("m,n_out,n_in", [(64, 256, 1024), (128, 128, 256), (16, 384, 512), (100, 200, 768),
                                           (257, 130, 1024), (512, 512, 4096), (300, 16384, 256)])
 def test_gemm_random(m, n_out, n_in):
-    # (300, 16384, 256) is the one shape here for which the 128-column tile is chosen
+    # (300, 16384, 256): many column tiles of a single super-block
     w = Q.fill_normal(300 + m, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
     p = Q.quantize(F.Q4_K, w)
     what = oracle.dequant(F.Q4_K, p, n_out, n_in)
@@ -472,9 +472,11 @@ def test_forward_fp16_gemm_identity_activations_give_fp16_weights_exactly(fmt):
 
 
 @pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
-@pytest.mark.parametrize("m,n_out,n_in", [(8, 4096, 4096), (65, 1048, 1024), (300, 4096, 1024), (513, 232, 4096)])
+@pytest.mark.parametrize("m,n_out,n_in", [(8, 4096, 4096), (65, 1048, 1024), (300, 4096, 1024), (513, 232, 4096),
+                                          (5, 4096, 4096), (33, 4096, 1024), (64, 2048, 4096), (100, 1024, 4096)])
 def test_forward_fp32_activations_as_row_scaled_fp16(fmt, m, n_out, n_in):
-    """fp32 activations through the fp16 form of the prefill GEMM: every row scaled by its own power of two before it
+    """fp32 activations through the fp16 matrix-core kernels (the few-row kernel for a few rows, then the fp16 form of
+    the prefill GEMM): every row scaled by its own power of two before it
     is rounded to fp16, the factor undone on the sums.  Rows of very different magnitudes (1e-30 .. 1e+32) each keep
     the 1e-3 class; a row of zeros gives zeros; a non-finite value poisons its own row and no other.  (No bias here:
     it would swallow the rows of tiny values; test_forward_default_precision... and the fp16 tests cover it.)"""
@@ -489,6 +491,7 @@ def test_forward_fp32_activations_as_row_scaled_fp16(fmt, m, n_out, n_in):
     xd, xf = x_to_dev(x, "f32")
     layer = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out)
     routes = {layer.route(m, torch.float32, torch.float32)}
+    assert routes <= {"gemm_skinny_f32_scaled_f16", "gemm_pc_f32_scaled_f16"}
     y = layer.forward(xd).cpu().numpy()
     assert y.dtype == np.float32 and np.isfinite(y).all()
     # sums of rows at 1e30 with weights of a few hundred overflow nowhere near: compare row by row, each against its own norm
@@ -505,6 +508,41 @@ def test_forward_fp32_activations_as_row_scaled_fp16(fmt, m, n_out, n_in):
             assert not np.isfinite(yb[i]).any(), i
         else:
             assert np.array_equal(yb[i], y[i]), i
+
+
+@pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
+@pytest.mark.parametrize("m", [17, 40, 64, 80])
+def test_forward_few_fp32_unit_rows_give_fp16_weights_exactly(fmt, m):
+    """A few fp32 rows (the few-row kernel over the scaled fp16 copy): a row that is a power of two at one position
+    returns that column of the weights, rounded once to fp16, times the power of two -- exactly, whatever the power;
+    with a bias and fp32 / bf16 / fp16 outputs."""
+    n_in, n_out = 1024, 1048
+    p = random_blocks(fmt, n_out * (n_in // BLOCK_WEIGHTS[fmt]), seed=991 + m)
+    what = oracle.dequant(fmt, p, n_out, n_in)
+    w16 = oracle.f16_to_f32(oracle.f32_to_f16(what))
+    rng = np.random.default_rng(992 + m)
+    cols = rng.choice(n_in, size=m, replace=False)
+    powers = np.array([0, -20, 30, -60, 7, 60, -3, 1], np.int64)[np.arange(m) % 8]
+    x = np.zeros((m, n_in), np.float32)
+    x[np.arange(m), cols] = np.ldexp(np.float32(1.0), powers).astype(np.float32)
+    xd, _ = x_to_dev(x, "f32")
+    layer = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out)
+    assert layer.route(m, torch.float32, torch.float32) == "gemm_skinny_f32_scaled_f16"
+    y = layer.forward(xd).cpu().numpy()
+    want = np.ldexp(w16[:, cols].T.astype(np.float64), powers[:, None]).astype(np.float32)
+    assert np.array_equal(y, want)
+    # moderate rows with a bias, every output type
+    xm = np.zeros((m, n_in), np.float32)
+    xm[np.arange(m), cols] = np.ldexp(np.float32(1.0), powers % 4).astype(np.float32)
+    bias = Q.fill_normal(993, 1, 1.0, n_out)
+    lb = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out, bias=torch.from_numpy(bias).to(DEV))
+    want_b = np.ldexp(w16[:, cols].T.astype(np.float64), (powers % 4)[:, None]).astype(np.float32) + bias[None, :]
+    xmd, _ = x_to_dev(xm, "f32")
+    assert np.array_equal(lb.forward(xmd).cpu().numpy(), want_b)
+    yb = lb.forward(xmd, out_dtype=torch.bfloat16)
+    assert np.array_equal(dev_bits(yb), oracle.f32_to_bf16(want_b))
+    yh = lb.forward(xmd, out_dtype=torch.float16)
+    assert np.array_equal(dev_bits(yh), oracle.f32_to_f16(want_b))
 
 
 @pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])

@@ -156,6 +156,29 @@ def test_fp16_gemm_with_a_caller_workspace(m, n_out, n_in, xk):
     assert e.value.status == F.ERR_WORKSPACE
 
 
+@pytest.mark.parametrize("m", [16, 80])
+def test_few_fp32_rows_with_a_caller_workspace(m):
+    """fp32 activations of a few rows: the scaled fp16 copy and its row factors (and the partial sums of a launch
+    split along K) come out of the caller's buffer; same bits as with the library's own workspace."""
+    n_out, n_in = 4096, 4096
+    p = random_blocks(F.Q4_K, n_out * (n_in // 256), seed=4600 + m)
+    xd, xf = x_to_dev(Q.fill_normal(4601, 1, 1.0, m * n_in).reshape(m, n_in) * np.float32(0.05), "f32")
+    layer = QuantLinear.init(packed_to_dev(p), F.Q4_K, n_in, n_out)
+    assert layer.route(m, xd.dtype) == "gemm_skinny_f32_scaled_f16"
+    need = layer.workspace_bytes(m, xd.dtype)
+    assert need >= m * n_in * 2 + 4 * m
+    ws = zeros_ws(need)
+    y = layer.forward(xd, workspace=ws)
+    y2 = layer.forward(xd, workspace=ws)
+    torch.cuda.synchronize()
+    assert torch.equal(y, y2)
+    assert torch.equal(y, layer.forward(xd))
+    assert rel_l2(y.cpu().numpy(), oracle.linear_f64(oracle.dequant(F.Q4_K, p, n_out, n_in), xf)) <= 1e-3
+    with pytest.raises(QL.TtqError) as e:
+        layer.forward(xd, workspace=zeros_ws(1 << 16))
+    assert e.value.status == F.ERR_WORKSPACE
+
+
 def exl3_case(n_out, n_in, bits, m, seed):
     w = Q.fill_normal(seed, 0, 0.02, n_out * n_in).reshape(n_out, n_in)
     tr, suh, svh = Q.quantize_exl3(w, bits, F.CB_MCG, seed=seed)

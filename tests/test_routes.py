@@ -40,6 +40,8 @@ PINNED = [
     ("fp16 activations, prefill 512 rows of the headline shape", Q4_K, 14336, 4096, 512, F16, F16, 0, "gemm_pc_f16"),
     ("fp32 activations, prefill 512 rows of the headline shape", Q4_K, 14336, 4096, 512, F32, F32, 0, "gemm_pc_f32_scaled_f16"),
     ("fp16 activations, 64 rows", Q4_K, 14336, 4096, 64, F16, F16, 0, "gemm_skinny_chunked"),
+    ("fp32 activations, 8 rows of the headline shape", Q4_K, 14336, 4096, 8, F32, F32, 0, "gemm_skinny_f32_scaled_f16"),
+    ("fp32 activations, 64 rows of the down projection", Q6_K, 4096, 14336, 64, F32, F32, 0, "gemm_skinny_f32_scaled_f16"),
     ("down projection of a 53248-wide MLP, decode", Q4_K, 16384, 53248, 1, BF16, F32, 0, "gemv_dot2"),
     ("rows beyond 65536 values", Q4_K, 4096, 65536 + 256, 1, BF16, F32, 0, "gemv_long"),
     ("fp32 activations beyond 16384 values", Q8_0, 4096, 16384 + 32, 1, F32, F32, 0, "gemv_long"),
@@ -52,11 +54,14 @@ def test_benchmark_and_model_shapes_reach_their_kernels(what, fmt, n_out, n_in, 
 
 
 def test_precision_flags_steer_the_route():
-    # fp32 activations: decode kernels for a handful of rows, then the fp16 form of the prefill GEMM over a copy
-    # scaled row by row (the 1e-3 class either way), never a bf16 copy by default
+    # fp32 activations: decode kernels for a handful of rows, then the fp16 matrix-core kernels over a copy scaled
+    # row by row -- the few-row kernel, then the prefill GEMM -- (the 1e-3 class either way), never a bf16 copy by default
     for m in (1, 2, 4):
         assert route(Q4_K, 14336, 4096, m, F32, F32).startswith("gemv_")
-    for m in (64, 255, 256, 600, 4096):
+    for m in (5, 16, 64):
+        assert route(Q4_K, 14336, 4096, m, F32, F32) == "gemm_skinny_f32_scaled_f16"
+        assert route(Q4_K, 14336, 4096, m, F32, F32, precision=_lib.PRECISION_F32_SCALES).startswith("gemv_")
+    for m in (65, 255, 256, 600, 4096):
         assert route(Q4_K, 14336, 4096, m, F32, F32) == "gemm_pc_f32_scaled_f16"
         assert route(Q4_K, 14336, 4096, m, F32, F32, precision=_lib.PRECISION_F32_SCALES).startswith("gemv_")
     # fp16 activations: their own matrix-core kernels (few rows; the fp16 form of the prefill GEMM), never a bf16
