@@ -130,7 +130,7 @@ typedef struct ttq_qlinear {
  * fp16 form of the prefill GEMM (a packed fp16 copy of x in a workspace, weights rounded once to
  * fp16, fp16 matrix cores: about 2e-4 measured; a dequantized weight beyond the fp16 range becomes
  * an infinity there); fp32 activations take the decode kernels (which read them as 15-bit block
- * fixed point) or, from five rows on, the same fp16 kernels (the few-row kernel, then the GEMM) over
+ * fixed point) or, from two rows on where that is cheaper, the same fp16 kernels (the few-row kernel, then the GEMM) over
  * a copy in which every row has been scaled by its own power of two (largest magnitude to 2^14) and
  * rounded to fp16, the factor undone on the sums (about 2e-4 measured for rows of any magnitude; a
  * non-finite value makes its own output row non-finite and no other).  Only a layer with precision == TTQ_PRECISION_BF16_OK lets

@@ -489,15 +489,18 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
   // measured), which take these activations as 15-bit block fixed point themselves, at a fraction of the time of
   // their passes (14336 x 4096 at 512 rows: 2.2 ms in passes of four rows).
   // A few rows take the few-row kernel in fp16 over a row-major copy scaled the same way (one pass of a workgroup
-  // per row, 2.5 us), as fp16 activations do: 14336 x 4096 at 8 rows 15 us against 28 us of the GEMM.
-  if (x_dtype == TTQ_F32 && block_fmt && m >= 5 && route != 1) {
+  // per row), as fp16 activations do: 14336 x 4096 at 8 rows 17 us against 28 us of the GEMM.  From two rows on
+  // that also beats passes of the decode kernels where those have no kernel of several rows for fp32 activations
+  // (Q6_K 14336 x 4096 at four rows: 20 us against 49; the 128256 x 4096 head 149 against 408).
+  if (x_dtype == TTQ_F32 && block_fmt && m >= 2 && route != 1) {
     float us_few = 1e30f, us_gemm = 1e30f;
     if (ttq::gemm_skinny_supported(layer->format, m < 64 ? m : 64, n_out, n_in)) {
+      // (the scaling pass: a workgroup per row walks it twice -- 3.3 us on rows of 4096 values, 8.7 us on 14336)
       const int64_t full = m / 64, rest = m % 64;
-      us_few = (float)full * ttq::gemm_skinny_estimate_us(layer->format, 64, n_out, n_in) + 2.5f + (float)(m * n_in * 6) / 3.0e6f;
+      us_few = (float)full * ttq::gemm_skinny_estimate_us(layer->format, 64, n_out, n_in) + 1.5f + (float)n_in * 0.5e-3f;
       if (rest) us_few += ttq::gemm_skinny_estimate_us(layer->format, rest, n_out, n_in);
     }
-    if (ttq::gemm_pc_supported(layer->format, m < 8192 ? m : 8192, n_out, n_in, 112))
+    if (m >= 5 && ttq::gemm_pc_supported(layer->format, m < 8192 ? m : 8192, n_out, n_in, 112))
       us_gemm = ttq::gemm_pc_estimate_us(layer->format, m, n_out, n_in) + 5.f + (float)(m * n_in * 10) / 3.0e6f;
     const float us_gemv = ttq::gemv_estimate_us(layer->format, x_dtype, m, n_out, n_in);
     if ((m > 64 ? us_few / 0.65f : us_few) < us_gemm && (route == 2 || us_few < us_gemv)) {
@@ -585,7 +588,9 @@ int64_t ttq_workspace_bytes(const ttq_qlinear* layer, int64_t m, int x_dtype) {
     const int64_t partials = (int64_t)ttq::gemm_exl3_partials_bytes(m, n_out, n_in);
     return header + ((block_rows * n_in * 2 + 255) & ~(int64_t)255) + ((partials + 255) & ~(int64_t)255);
   }
-  if (m < 5) return 0;                          // the decode kernels take no workspace
+  // the decode kernels take no workspace (two to four rows of fp32 activations may take the few-row kernel over a
+  // scaled fp16 copy)
+  if (m < 5 && !(x_dtype == TTQ_F32 && m >= 2)) return 0;
   // the packed bf16 copy of the activations where the prefill GEMM wants one, then the partial sums of a launch
   // split along K: the prefill GEMM's exact size for every row count it can be called with here, and the few-row
   // kernel's bound (one 64 x 64 tile of sums per compute unit)

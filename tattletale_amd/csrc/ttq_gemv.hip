@@ -537,11 +537,16 @@ float gemv_estimate_us(int format, int x_dtype, int64_t m, int64_t n_out, int64_
   }
   if (gemv_dot2_multi_supported(format, x_dtype, m, n_in))
     return m <= 2 ? mb / 2.6f + 2.f : (float)((m + 3) / 4) * (mb / 1.7f + 2.f);
+  // the register-streamed int8 matrix-core kernel (Q4_K with fp32 activations): a pass per row; measured at 9.4 / 33 /
+  // 295 MB: 4.3 / 6.8 / 53 us for one row, 2.4 / 5.0 / 46.5 us for every further one
+  if (gemv_mfma_supported(format, x_dtype, n_out, n_in)) return 2.f + (float)m * (mb / 6.8f + 0.8f);
   if (gemv_q8_win_supported(format, n_out, n_in)) {
     const int tok = gemv_q8_win_tokens(x_dtype, m, n_in);
     return (float)((m + tok - 1) / tok) * (mb / (tok == 4 ? 3.1f : 3.6f) + 2.f);
   }
-  return (float)m * (mb / 3.2f + 3.f);
+  // the generic kernel, a pass per row (Q6_K with fp32 activations, 3.4 / 13.8 / 48 MB: 4.1 / 7.5 / 16.2 us for one
+  // row, 1.2 / 4.5 / 11 us for every further one; rows of 14336 values take twice that)
+  return 3.f + (float)m * (mb / 3.3f + 0.3f);
 }
 
 }  // namespace ttq

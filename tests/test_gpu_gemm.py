@@ -510,6 +510,31 @@ def test_forward_fp32_activations_as_row_scaled_fp16(fmt, m, n_out, n_in):
             assert np.array_equal(yb[i], y[i]), i
 
 
+@pytest.mark.parametrize("m", [2, 3, 4])
+@pytest.mark.parametrize("n_out,n_in", [(4096, 4096), (4096, 14336)])
+def test_forward_two_to_four_fp32_rows_on_q6_k(m, n_out, n_in):
+    """Q6_K has no decode kernel of several fp32 rows: from two rows on the operator takes the few-row kernel over the
+    row-scaled fp16 copy (the 1e-3 class, rows of any magnitude, with a bias), with the library's workspace or the
+    caller's; one row stays on the decode kernel."""
+    p = random_blocks(F.Q6_K, n_out * (n_in // 256), seed=1200 + m)
+    what = oracle.dequant(F.Q6_K, p, n_out, n_in)
+    x = Q.fill_normal(1201 + m, 1, 1.0, m * n_in).reshape(m, n_in)
+    x *= np.array([1.0, 1e-12, 3e9, 0.02], np.float32)[:m, None]
+    bias = Q.fill_normal(1202, 1, 1e-14, n_out)
+    xd, xf = x_to_dev(x, "f32")
+    layer = QuantLinear.init(packed_to_dev(p), F.Q6_K, n_in, n_out, bias=torch.from_numpy(bias).to(DEV))
+    assert layer.route(m, torch.float32) == "gemm_skinny_f32_scaled_f16"
+    assert layer.route(1, torch.float32).startswith("gemv_")
+    y = layer.forward(xd)
+    for i in range(m):
+        want = oracle.linear_f64(what, xf[i:i + 1], bias)[0]
+        assert rel_l2(y[i].cpu().numpy().astype(np.float64), want) <= 1e-3, i
+    need = layer.workspace_bytes(m, torch.float32)
+    assert need >= m * n_in * 2 + 4 * m
+    ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
+    assert torch.equal(layer.forward(xd, workspace=ws), y)
+
+
 @pytest.mark.parametrize("fmt", [F.Q4_K, F.Q6_K, F.Q8_0])
 @pytest.mark.parametrize("m", [17, 40, 64, 80])
 def test_forward_few_fp32_unit_rows_give_fp16_weights_exactly(fmt, m):

@@ -56,9 +56,11 @@ def test_benchmark_and_model_shapes_reach_their_kernels(what, fmt, n_out, n_in, 
 def test_precision_flags_steer_the_route():
     # fp32 activations: decode kernels for a handful of rows, then the fp16 matrix-core kernels over a copy scaled
     # row by row -- the few-row kernel, then the prefill GEMM -- (the 1e-3 class either way), never a bf16 copy by default
-    for m in (1, 2, 4):
+    for m in (1, 2):
         assert route(Q4_K, 14336, 4096, m, F32, F32).startswith("gemv_")
-    for m in (5, 16, 64):
+    assert route(Q6_K, 14336, 4096, 1, F32, F32).startswith("gemv_")             # a single row always decodes
+    assert route(Q6_K, 14336, 4096, 2, F32, F32) == "gemm_skinny_f32_scaled_f16"  # no decode kernel of several fp32 rows
+    for m in (4, 5, 16, 64):
         assert route(Q4_K, 14336, 4096, m, F32, F32) == "gemm_skinny_f32_scaled_f16"
         assert route(Q4_K, 14336, 4096, m, F32, F32, precision=_lib.PRECISION_F32_SCALES).startswith("gemv_")
     for m in (65, 255, 256, 600, 4096):
