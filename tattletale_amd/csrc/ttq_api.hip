@@ -495,9 +495,9 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
   if (x_dtype == TTQ_F32 && block_fmt && m >= 2 && route != 1) {
     float us_few = 1e30f, us_gemm = 1e30f;
     if (ttq::gemm_skinny_supported(layer->format, m < 64 ? m : 64, n_out, n_in)) {
-      // (the scaling pass: a workgroup per row walks it twice -- 3.3 us on rows of 4096 values, 8.7 us on 14336)
+      // (the scaling pass: a workgroup per row walks it twice -- 3 us on rows of 4096 values, 4.3 us on 14336)
       const int64_t full = m / 64, rest = m % 64;
-      us_few = (float)full * ttq::gemm_skinny_estimate_us(layer->format, 64, n_out, n_in) + 1.5f + (float)n_in * 0.5e-3f;
+      us_few = (float)full * ttq::gemm_skinny_estimate_us(layer->format, 64, n_out, n_in) + 2.5f + (float)n_in * 0.13e-3f;
       if (rest) us_few += ttq::gemm_skinny_estimate_us(layer->format, rest, n_out, n_in);
     }
     if (m >= 5 && ttq::gemm_pc_supported(layer->format, m < 8192 ? m : 8192, n_out, n_in, 112))

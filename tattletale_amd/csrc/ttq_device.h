@@ -199,14 +199,15 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 // fp32 activations for the fp16 matrix cores: the power of two that brings a row's largest magnitude to 2^14 (the row
 // then fits fp16 with room for sums of its neighbours, and values down to 2^-38 of the largest stay normal numbers).
-// Called by all 256 threads of a workgroup with the row (n_in a multiple of 4, 16-byte aligned) and 9 floats of LDS;
-// returns the INVERSE of the factor to every thread.  A row with a non-finite value, or of zeros, is not scaled (1):
+// Called by all 64 * NW threads of a workgroup with the row (n_in a multiple of 4, 16-byte aligned) and 2 * NW + 1
+// floats of LDS; returns the INVERSE of the factor to every thread.  A row with a non-finite value, or of zeros, is not scaled (1):
 // its non-finite values convert as they are and poison that row's outputs only.
+template <int NW = 4>
 __device__ __forceinline__ float block_row_inverse_factor(const float* __restrict__ row, int n_in, float* part) {
   const int t = (int)threadIdx.x, lane = t & 63, wave = t >> 6;
   const float4* src = reinterpret_cast<const float4*>(row);
   float amax = 0.f, bad = 0.f;
-  for (int k4 = t; k4 < n_in / 4; k4 += 256) {
+  for (int k4 = t; k4 < n_in / 4; k4 += 64 * NW) {
     const float4 v = src[k4];
     const float a = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
     // (fmaxf drops NaNs: look at them separately)
@@ -220,11 +221,13 @@ __device__ __forceinline__ float block_row_inverse_factor(const float* __restric
   amax = fmaxf(amax, lane_xor<8>(amax, lane)); bad = fmaxf(bad, lane_xor<8>(bad, lane));
   amax = fmaxf(amax, lane_xor<16>(amax, lane)); bad = fmaxf(bad, lane_xor<16>(bad, lane));
   amax = fmaxf(amax, lane_xor<32>(amax, lane)); bad = fmaxf(bad, lane_xor<32>(bad, lane));
-  if (lane == 0) { part[wave] = amax; part[4 + wave] = bad; }
+  if (lane == 0) { part[wave] = amax; part[NW + wave] = bad; }
   __syncthreads();
   if (t == 0) {
-    amax = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
-    bad = fmaxf(fmaxf(part[4], part[5]), fmaxf(part[6], part[7]));
+    amax = part[0];
+    bad = part[NW];
+#pragma unroll
+    for (int v = 1; v < NW; v++) { amax = fmaxf(amax, part[v]); bad = fmaxf(bad, part[NW + v]); }
     // factor = 2^(14 - E), E the exponent of the largest magnitude (subnormal maxima count as 2^-126): biased exponent
     // 268 - (E + 127); it stops at 2^126, so that its inverse stays a normal number: rows of tiny values are simply
     // scaled a little less
@@ -234,10 +237,10 @@ __device__ __forceinline__ float block_row_inverse_factor(const float* __restric
       const uint32_t fe = 268u - ec > 253u ? 253u : 268u - ec;
       fi = __uint_as_float((254u - fe) << 23);
     }
-    part[8] = fi;
+    part[2 * NW] = fi;
   }
   __syncthreads();
-  return part[8];
+  return part[2 * NW];
 }
 // the factor from its inverse: both are powers of two
 __device__ __forceinline__ float row_factor_of_inverse(float inv) {

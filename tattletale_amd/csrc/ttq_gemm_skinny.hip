@@ -697,15 +697,17 @@ hipError_t launch_gemm_skinny_chunked(int format, const void* w, const uint16_t*
 
 // fp32 activations: every row scaled by a power of two (its largest magnitude to 2^14) and rounded to fp16, row-major,
 // with the inverse factors behind the copy; the fp16 kernel multiplies its sums by them.  One workgroup per row.
-static __global__ void __launch_bounds__(256) scale_rows_f16_kernel(const float* __restrict__ x, uint16_t* __restrict__ xs,
-                                                                    float* __restrict__ inv, int n_in) {
-  __shared__ float part[9];
+constexpr int kScaleWaves = 16;      // a row of 14336 values is 3.5 loads per thread: the pass is two trips to memory
+static __global__ void __launch_bounds__(64 * kScaleWaves) scale_rows_f16_kernel(const float* __restrict__ x,
+                                                                                 uint16_t* __restrict__ xs,
+                                                                                 float* __restrict__ inv, int n_in) {
+  __shared__ float part[2 * kScaleWaves + 1];
   const float* row = x + (int64_t)blockIdx.x * n_in;
-  const float fi = block_row_inverse_factor(row, n_in, part);
+  const float fi = block_row_inverse_factor<kScaleWaves>(row, n_in, part);
   const float f = row_factor_of_inverse(fi);
   const float4* src = reinterpret_cast<const float4*>(row);
   uint2* dst = reinterpret_cast<uint2*>(xs + (int64_t)blockIdx.x * n_in);
-  for (int k4 = (int)threadIdx.x; k4 < n_in / 4; k4 += 256) {
+  for (int k4 = (int)threadIdx.x; k4 < n_in / 4; k4 += 64 * kScaleWaves) {
     const float4 v = src[k4];
     dst[k4] = make_uint2(pack_f16x2(v.x * f, v.y * f), pack_f16x2(v.z * f, v.w * f));
   }
@@ -721,7 +723,7 @@ hipError_t launch_gemm_skinny_f32(int format, const void* w, const float* x, voi
   if (e != hipSuccess) return e;
   uint16_t* xs = static_cast<uint16_t*>(ws);
   float* inv = reinterpret_cast<float*>(static_cast<char*>(ws) + copy_bytes);
-  hipLaunchKernelGGL(scale_rows_f16_kernel, dim3((unsigned)m), dim3(256), 0, s, x, xs, inv, (int)n_in);
+  hipLaunchKernelGGL(scale_rows_f16_kernel, dim3((unsigned)m), dim3(64 * kScaleWaves), 0, s, x, xs, inv, (int)n_in);
   e = hipGetLastError();
   if (e != hipSuccess) return e;
   return launch_gemm_skinny_chunked(format, w, xs, kF16, y, y_dtype, bias, bias_dtype, m, n_out, n_in, s, inv);
