@@ -435,7 +435,12 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
   // Several rows of bf16 activations: the prefill GEMM (weights rounded to bf16) or a few passes of
   // the decode kernels (fp32 scales), whichever the shape makes cheaper.  Up to four rows always
   // decode.
-  const bool gemm_ok = x_dtype == TTQ_BF16 && (y_dtype == TTQ_BF16 || y_dtype == TTQ_F32) &&
+  // (fp16 outputs from bf16 activations: every GEMM kernel but the single-role one, which only more than 4 GiB of
+  // activations reach, stores them)
+  const bool gemm_ok = x_dtype == TTQ_BF16 &&
+                       (y_dtype == TTQ_BF16 || y_dtype == TTQ_F32 ||
+                        (y_dtype == TTQ_F16 && (ttq::gemm_skinny_supported(layer->format, m, n_out, n_in) ||
+                                                ttq::gemm_pc_supported(layer->format, m, n_out, n_in, 112)))) &&
                        (layer->format == TTQ_Q4_K || layer->format == TTQ_Q6_K || layer->format == TTQ_Q8_0) &&
                        ttq::gemm_supported(layer->format, m, n_out, n_in);
   // TTQ_FORWARD_ROUTE (developer builds, A/B measurements): 1 = always the decode kernels, 2 = the GEMM whenever it exists

@@ -510,6 +510,28 @@ def test_forward_fp32_activations_as_row_scaled_fp16(fmt, m, n_out, n_in):
             assert np.array_equal(yb[i], y[i]), i
 
 
+@pytest.mark.parametrize("fmt,m,n_out,n_in", [(f, *c) for f in (F.Q4_K, F.Q6_K, F.Q8_0)
+                                              for c in ((40, 2048, 1024), (100, 1048, 2048), (512, 1160, 1024))] +
+                         [(F.Q4_K, 300, 14336, 4096)])
+def test_forward_bf16_activations_fp16_outputs_take_the_gemm(fmt, m, n_out, n_in):
+    """bf16 activations with fp16 outputs (an out_dtype of the caller's choice) run the same matrix-core kernels as
+    with bf16 outputs, not passes of the decode kernels; the sums are rounded to fp16 instead."""
+    p = random_blocks(fmt, n_out * (n_in // BLOCK_WEIGHTS[fmt]), seed=1300 + m)
+    xd, xf = x_to_dev(Q.fill_normal(1301 + m, 1, 1.0, m * n_in).reshape(m, n_in) * np.float32(0.01), "bf16")
+    bias = Q.fill_normal(1302, 1, 1.0, n_out)
+    layer = QuantLinear.init(packed_to_dev(p), fmt, n_in, n_out, bias=torch.from_numpy(bias).to(DEV))
+    assert layer.route(m, torch.bfloat16, torch.float16) == layer.route(m, torch.bfloat16, torch.bfloat16)
+    assert layer.route(m, torch.bfloat16, torch.float16).startswith("gemm_")
+    y16 = layer.forward(xd, out_dtype=torch.float16)
+    y32 = layer.forward(xd, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    assert y16.dtype == torch.float16
+    # the same sums, rounded once to fp16
+    assert np.array_equal(dev_bits(y16), oracle.f32_to_f16(y32.cpu().numpy()))
+    want = oracle.linear_f64(oracle.dequant(fmt, p, n_out, n_in), xf, bias)
+    assert rel_l2(y32.cpu().numpy(), want) <= TOL
+
+
 @pytest.mark.parametrize("m", [2, 3, 4])
 @pytest.mark.parametrize("n_out,n_in", [(4096, 4096), (4096, 14336)])
 def test_forward_two_to_four_fp32_rows_on_q6_k(m, n_out, n_in):
