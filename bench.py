@@ -514,6 +514,15 @@ def main() -> int:
             layers = [QL.QuantLinear.init(w, F.Q4_K, n_in, n_out) for w in ws]
             return lambda i: layers[i % nc].forward(xf)
         timed("q4_k_forward_f32_m512", F.Q4_K, 512, f32_forward, steps=max(20, steps // 4))
+        # a few fp32 rows through the operator: the few-row kernel in fp16 over a row-major copy scaled the same way
+        # (Q6_K has no decode kernel of several fp32 rows: four rows take it as well)
+        timed("q4_k_forward_f32_m8", F.Q4_K, 8, f32_forward)
+
+        def f32_forward_q6(ws, x, nc):
+            xf = x.float() * 0.05
+            layers = [QL.QuantLinear.init(w, F.Q6_K, n_in, n_out) for w in ws]
+            return lambda i: layers[i % nc].forward(xf)
+        timed("q6_k_forward_f32_m4", F.Q6_K, 4, f32_forward_q6)
         # trellis weights, 4096 x 4096 at 3 bits: 8 rows through the decode kernel (one decode of the weights
         # for all 8), 512 rows through the prefill path, and the Q4_K GEMM at the same shape beside it
         ecfg = CFG.CONFIGS["exl3_gemv"]
@@ -542,6 +551,13 @@ def main() -> int:
         timed("q4_k_gemm_m512_4096x4096", F.Q4_K, 512,
               lambda ws, x, nc, y=y: (lambda i: QL.gemm(F.Q4_K, ws[i % nc], x, 4096, 4096, out=y)),
               n_out=4096, n_in=4096, steps=max(20, steps // 4))
+        # the fused gate||up weight as a plain GEMM at 2048 rows: eight full rounds of 256 x 112 tiles
+        y = torch.empty((2048, 2 * n_out), dtype=torch.bfloat16, device=dev)
+        timed("q4_k_gemm_m2048_gate_up_28672x4096", F.Q4_K, 2048,
+              lambda ws, x, nc, y=y: (lambda i: QL.gemm(F.Q4_K, ws[i % nc], x, 2 * n_out, n_in, out=y)),
+              n_out=2 * n_out, n_in=n_in, steps=max(10, steps // 10))
+        del y
+        torch.cuda.empty_cache()
         # the down projection of a prefill chunk: few output tiles, long K -- the launches that split K
         for m in (128, 512):
             y = torch.empty((m, 4096), dtype=torch.bfloat16, device=dev)
