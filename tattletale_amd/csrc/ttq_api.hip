@@ -499,7 +499,8 @@ int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int
   // (Q6_K 14336 x 4096 at four rows: 20 us against 49; the 128256 x 4096 head 149 against 408).
   if (x_dtype == TTQ_F32 && block_fmt && m >= 2 && route != 1) {
     float us_few = 1e30f, us_gemm = 1e30f;
-    if (ttq::gemm_skinny_supported(layer->format, m < 64 ? m : 64, n_out, n_in)) {
+    // (up to 8192 rows: the scaled copy of all rows sits in the workspace at once)
+    if (m <= 8192 && ttq::gemm_skinny_supported(layer->format, m < 64 ? m : 64, n_out, n_in)) {
       // (the scaling pass: a workgroup per row walks it twice -- 3 us on rows of 4096 values, 4.3 us on 14336)
       const int64_t full = m / 64, rest = m % 64;
       us_few = (float)full * ttq::gemm_skinny_estimate_us(layer->format, 64, n_out, n_in) + 2.5f + (float)n_in * 0.13e-3f;
