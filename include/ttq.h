@@ -138,7 +138,7 @@ typedef struct ttq_qlinear {
  * (2e-2 class).
  * Limits (TTQ_ERR_UNSUPPORTED beyond): every format takes any n_in (block formats: rows beyond
  * 65536 values for Q4_K / Q6_K with 16-bit activations, beyond 16384 otherwise, run a decode kernel
- * that stages nothing in LDS: correct, not tuned); any m (rows are taken 65535 at a time where a
+ * that stages nothing in LDS, at about half the rate of the staged ones); any m (rows are taken 65535 at a time where a
  * kernel needs that).  m == 0 or n_out == 0 returns TTQ_OK without touching a pointer. */
 TTQ_API int ttq_linear_forward(const ttq_qlinear* layer, const void* x, int x_dtype, int64_t m,
                        void* y, int y_dtype, void* stream);
@@ -209,7 +209,7 @@ TTQ_API const char* ttq_route_name(int route);
 /* ---- decode GEMV, one entry per block format (m rows of x, normally m == 1) -------- */
 /* y[m][n_out] (fp32) = x[m][n_in] * W^T.  Stand in for F.linear(x, weight) with a
  * (1, n_in) activation (neural_nets.nim:64).  Any n_in (rows beyond 65536 values for Q4_K / Q6_K
- * with 16-bit activations, beyond 16384 otherwise, take an untuned kernel).  Two to four rows (a speculative step, a few sequences) of
+ * with 16-bit activations, beyond 16384 otherwise, take the unstaged kernel).  Two to four rows (a speculative step, a few sequences) of
  * 16-bit activations over a large Q4_K or Q6_K matrix cost about one pass over the weights, not
  * one per row; every row's result stays within the 1e-3 class of the single-row call.  A NaN or
  * an infinity among a row's activations, or in a block scale of a weight row, makes the outputs

@@ -354,16 +354,19 @@ static hipError_t launch_generic_xy(const void* w, const void* x, int x_dtype, v
 
 // ---------------------------------------------------------------------- rows of any length
 // Rows longer than the staged kernels hold in LDS (F.linear has no such limit: the down projection of the
-// largest dense models has 53248 inputs).  Nothing is staged: a wavefront owns kLongRows consecutive weight rows,
-// its lanes walk the rows' units 64 apart, and every lane reads the 64 activations of its unit straight from
-// memory in four runs of 16 consecutive values, once for all of its rows (the activation row stays in L2, the
-// weights are read once).  Same arithmetic as the generic kernel (fp32, scales applied once per sub-block).
+// largest dense models has 53248 inputs).  Nothing is staged: a workgroup owns kLongRows consecutive weight rows,
+// its 256 threads walk the rows' units 256 apart, and every thread reads the 64 activations of its unit straight
+// from memory in four runs of 16 consecutive values, once for all of the rows (the activation row stays in L2, the
+// weights are read once); the wavefronts' sums meet in LDS.  (A wavefront per group of rows left most compute
+// units idle on matrices of a few thousand rows: Q8_0 3584 x 18944 48 us.)  Same arithmetic as the generic kernel
+// (fp32, scales applied once per sub-block).
 constexpr int kLongRows = 8;
 
 template <class F, typename XT, typename YT>
 __global__ void __launch_bounds__(kGemvThreads)
 gemv_long_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, YT* __restrict__ y,
                  const void* __restrict__ bias, int bias_dtype, int n_out, int n_in) {
+  __shared__ float part[kGemvWaves][kLongRows];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const XT* xm = x + (int64_t)blockIdx.y * n_in;
   YT* ym = y + (int64_t)blockIdx.y * n_out;
@@ -371,12 +374,12 @@ gemv_long_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, YT* __
   const int64_t rb = F::row_bytes(n_in);
   constexpr int kVec = 16 / (int)sizeof(XT);           // activations per 16-byte load
   const int groups = (n_out + kLongRows - 1) / kLongRows;
-  for (int g = blockIdx.x * kGemvWaves + wave; g < groups; g += gridDim.x * kGemvWaves) {
+  for (int g = blockIdx.x; g < groups; g += gridDim.x) {
     const int row0 = g * kLongRows;
     float acc[kLongRows];
 #pragma unroll
     for (int r = 0; r < kLongRows; r++) acc[r] = 0.f;
-    for (int u = lane; u < units; u += 64) {
+    for (int u = tid; u < units; u += kGemvThreads) {
       float xr[64];
 #pragma unroll
       for (int q = 0; q < 4; q++) {
@@ -403,16 +406,23 @@ gemv_long_kernel(const uint8_t* __restrict__ w, const XT* __restrict__ x, YT* __
 #pragma unroll
     for (int r = 0; r < kLongRows; r++) {
       const float sum = wave_sum(acc[r]);
-      if (lane == 0 && row0 + r < n_out) YElem<YT>::store(ym, row0 + r, sum + load_bias(bias, bias_dtype, row0 + r));
+      if (lane == 0) part[wave][r] = sum;
     }
+    __syncthreads();
+    if (tid < kLongRows && row0 + tid < n_out) {
+      float sum = part[0][tid];
+#pragma unroll
+      for (int v = 1; v < kGemvWaves; v++) sum += part[v][tid];
+      YElem<YT>::store(ym, row0 + tid, sum + load_bias(bias, bias_dtype, row0 + tid));
+    }
+    __syncthreads();      // part is written again in the next round
   }
 }
 
 template <class F, typename XT, typename YT>
 static hipError_t launch_long(const void* w, const void* x, void* y, const void* bias, int bias_dtype, int64_t m,
                               int64_t n_out, int64_t n_in, hipStream_t s) {
-  const int64_t per_wg = (int64_t)kGemvWaves * kLongRows;
-  const int64_t need = (n_out + per_wg - 1) / per_wg, most = (int64_t)device_num_cus() * 8;
+  const int64_t need = (n_out + kLongRows - 1) / kLongRows, most = (int64_t)device_num_cus() * 8;
   const dim3 grid((unsigned)(need < most ? need : most), (unsigned)m), block(kGemvThreads);
   hipLaunchKernelGGL((gemv_long_kernel<F, XT, YT>), grid, block, 0, s, static_cast<const uint8_t*>(w),
                      static_cast<const XT*>(x), static_cast<YT*>(y), bias, bias_dtype, (int)n_out, (int)n_in);
@@ -515,8 +525,8 @@ hipError_t launch_gemv(int format, const void* w, const void* x, int x_dtype, vo
 float gemv_estimate_us(int format, int x_dtype, int64_t m, int64_t n_out, int64_t n_in) {
   const int64_t per = format == kQ8_0 ? 32 : 256, blk = format == kQ8_0 ? 34 : (format == kQ4_K ? 144 : 210);
   const float mb = (float)(n_out * (n_in / per) * blk) * 1e-6f;
-  // rows of any length: a pass over the weights per activation row, not measured beyond a few shapes
-  if (gemv_row_is_long(format, x_dtype, n_in)) return (float)m * (mb / 2.f + 3.f);
+  // rows of any length: a pass over the weights per activation row (72 MB in 24.6 us, 155 MB in 51 us, 463 MB in 122 us)
+  if (gemv_row_is_long(format, x_dtype, n_in)) return (float)m * (mb / 3.5f + 3.f);
   const bool b4 = gemv_q4k_batch4_supported(format, x_dtype, m, n_out, n_in);
   if (b4 && m <= 4) return mb / 2.75f + 2.f;
   if (gemv_q4k_batch_supported(format, x_dtype, m, n_out, n_in)) {
