@@ -1,4 +1,7 @@
-// Prefill GEMM for Q4_K weights on gfx950:  Y (m, n_out) = X (m, n_in) * W^T.
+// Prefill GEMM for Q4_K weights on gfx950:  Y (m, n_out) = X (m, n_in) * W^T -- the dispatch of the GEMM entry
+// points (launch_gemm, at the end of this file) and the single-role tiled kernel, which serves activation matrices
+// of more than 4 GiB (64-bit row offsets); everything smaller runs the few-row kernel (ttq_gemm_skinny.hip) or the
+// producer/consumer kernels (ttq_gemm_pc.hip, ttq_gemm_pcd.hip).
 //
 // Replaces F.linear(x, weight) for a multi-row bf16 activation
 // (workspace/libtorch/src/abi/neural_nets.nim:64-81; the prefill case of
