@@ -34,6 +34,9 @@ PINNED = [
     ("down projection 4096x14336, decode", Q4_K, 4096, 14336, 1, BF16, F32, 0, "gemv_q4k_slice"),
     ("q / o projection, prefill 512 rows", Q4_K, 4096, 4096, 512, BF16, BF16, 0, "gemm_pc"),
     ("down projection, prefill 512 rows", Q4_K, 4096, 14336, 512, BF16, BF16, 0, "gemm_pc_packed_split_k"),
+    ("gate||up weight as a plain GEMM, 2048 rows (eight full rounds of tiles)", Q4_K, 28672, 4096, 2048, BF16, BF16, 0, "gemm_pc_packed"),
+    ("headline shape, 4096 rows", Q4_K, 14336, 4096, 4096, BF16, BF16, 0, "gemm_pc_packed"),
+    ("down projection, prefill 1024 rows", Q4_K, 4096, 14336, 1024, BF16, BF16, 0, "gemm_pc_packed"),
     ("two rows of the headline shape", Q4_K, 14336, 4096, 2, BF16, F32, 0, "gemv_q4k_stream4"),
     ("three rows of the LM head", Q6_K, 128256, 4096, 3, BF16, F32, 0, "gemv_q6k_stream4"),
     ("trellis layer, prefill 512 rows", EXL3, 4096, 4096, 512, F16, F32, 3, "exl3_gemm"),
@@ -78,6 +81,15 @@ def test_precision_flags_steer_the_route():
     # F32_SCALES pins the decode kernels for bf16 activations too
     assert route(Q4_K, 14336, 4096, 512, BF16, BF16, precision=_lib.PRECISION_F32_SCALES).startswith("gemv_")
     assert route(EXL3, 4096, 4096, 512, F16, F32, bits=3, precision=_lib.PRECISION_F32_SCALES).startswith("exl3_gemv")
+
+
+def test_the_single_role_gemm_serves_only_activations_beyond_4_gib():
+    # every row count of every shape below reaches the few-row or the producer/consumer kernels
+    for n_out, n_in in ((28672, 4096), (14336, 4096), (4096, 14336), (128256, 4096), (16384, 256)):
+        for m in (65, 300, 1024, 2048, 4096, 8192, 8200, 100000):
+            if m * n_in * 2 < (1 << 32):
+                assert route(Q4_K, n_out, n_in, m, BF16, BF16) != "gemm_q4k_tiles", (n_out, n_in, m)
+    assert route(Q4_K, 48, 256, (1 << 32) // 512, BF16, BF16) == "gemm_q4k_tiles"
 
 
 def test_route_is_a_pure_query():
