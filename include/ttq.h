@@ -279,7 +279,7 @@ TTQ_API int ttq_gemm_q8_0_ws(const void* w, const uint16_t* x_bf16, uint16_t* y_
  * the library allocates per (device, stream) on first use and grows on demand (up to 4096 rows of
  * n_in fp16 values), so the first call, and a call with more rows than any before, must not happen
  * under graph capture (ttq_gemm_exl3_ws has no such limit).  ttq_linear_forward takes this path by
- * itself from 16 to 48 rows on, depending on the matrix, unless the layer asks for
+ * itself from 9 to 48 rows on, depending on the matrix, unless the layer asks for
  * TTQ_PRECISION_F32_SCALES. */
 TTQ_API int ttq_gemm_exl3(const uint16_t* trellis, const uint16_t* suh_f16, const uint16_t* svh_f16,
                   const void* x, int x_dtype, float* y, int64_t m, int64_t n_out, int64_t n_in,

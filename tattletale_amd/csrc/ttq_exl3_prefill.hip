@@ -63,11 +63,11 @@ exl3_rotate_pack_kernel(const XT* __restrict__ x, const uint16_t* __restrict__ s
 // ------------------------------------------------------------------------------ launch
 bool gemm_exl3_preferred(int64_t m, int64_t n_out, int64_t n_in) {
   // Measured against passes of the decode kernel (8 rows each; 4096 x 4096, 14336 x 4096, 4096 x 14336, 1024 x 4096 at
-  // 8 .. 64 rows): the tiled form wins from 24 rows on matrices of 2048 output channels or more, from 16 rows on the
-  // largest ones, from 48 rows on short ones.
-  if (n_in % 128 != 0 || m < 16) return false;
+  // 8 .. 64 rows): the tiled form wins from the third pass (17 rows) on matrices of 2048 output channels or more, from
+  // the second (9 rows: 30.5 against 37 us) on the largest ones, from 48 rows on short ones.
+  if (n_in % 128 != 0 || m < 9) return false;
   if (n_out * n_in >= ((int64_t)48 << 20)) return true;
-  return m >= 48 || (m >= 24 && n_out >= 2048);
+  return m >= 48 || (m >= 17 && n_out >= 2048);
 }
 
 constexpr int64_t kXpMaxRows = 4096;       // rows rotated into the workspace at a time
