@@ -104,10 +104,9 @@ float gemm_pc_estimate_us(int format, int64_t m, int64_t n_out, int64_t n_in) {
 // move a half and a quarter of the activation bytes per step through LDS and gain nothing from the copy (-0.5 to
 // -6 us on seven shapes, split along K or not).
 constexpr int64_t kPackRows = 8192;         // rows packed (and multiplied) at a time
-static bool pc_use_packed(const PcChoice& c, int64_t m, int64_t n_in) {
+static bool pc_use_packed(const PcChoice& c) {
   static const int knob = dev_knob("TTQ_GEMM_PACKED", -1);      // A/B: 0 never, 1 always
   if (knob >= 0) return knob != 0;
-  (void)m; (void)n_in;
   return kPcTiles[c.tile].mb == 4 && c.cost_us >= 45.f;
 }
 
@@ -135,7 +134,7 @@ static hipError_t launch_pc_fmt(const uint8_t* wb, const void* x, int x_dtype, v
   const PcChoice whole = pc_choose(m, n_out, n_in, FUSE);
   // (the fused gate||up form keeps the LDS-staged kernel: beside the packed kernel's three steps of A fragments its
   // epilogue does not fit the registers, and a kernel that requests registers asynchronously must never spill them)
-  if (FUSE || (!force_packed && !pc_use_packed(whole, m, n_in)))
+  if (FUSE || (!force_packed && !pc_use_packed(whole)))
     return launch_pc_rows<FMT, FUSE>(whole, -1, wb, static_cast<const uint16_t*>(x), y, y_dtype, bias, bias_dtype, m, n_out,
                                      n_in, s);
   const int64_t block_rows = m < kPackRows ? m : kPackRows;
@@ -184,7 +183,7 @@ hipError_t launch_gemm_pc_x(int format, const void* w, const void* x, int x_dtyp
   if (y_dtype != kBF16 && y_dtype != kF32 && y_dtype != kF16) return hipErrorInvalidValue;
   if (f16_native && x_dtype != kF16 && x_dtype != kF32) return hipErrorInvalidValue;
   const PcChoice c = pc_choose(m, n_out, n_in, false);
-  const bool packed = x_dtype != kBF16 || pc_use_packed(c, m, n_in);
+  const bool packed = x_dtype != kBF16 || pc_use_packed(c);
   if (route_probe(f16_native ? (x_dtype == kF32 ? kRouteGemmPcF32ScaledF16 : kRouteGemmPcF16)
                              : (x_dtype != kBF16 ? kRouteGemmPcBf16Copy
                                                  : (c.splits > 1 ? (packed ? kRouteGemmPcPackedSplitK : kRouteGemmPcSplitK)
@@ -209,7 +208,7 @@ hipError_t launch_gemm_pc(int format, const void* w, const uint16_t* x_bf16, voi
 // bytes of the packed copy a launch of this shape takes from the workspace (0: it reads X itself)
 size_t gemm_pc_packed_bytes(int64_t m, int64_t n_out, int64_t n_in, int x_dtype) {
   if (m <= 0 || n_out <= 0 || n_in < 256) return 0;
-  const bool packed = x_dtype != kBF16 || pc_use_packed(pc_choose(m, n_out, n_in, false), m, n_in);
+  const bool packed = x_dtype != kBF16 || pc_use_packed(pc_choose(m, n_out, n_in, false));
   if (!packed) return 0;
   const int64_t rows = m < kPackRows ? m : kPackRows;
   // (fp32 activations: room for a factor per row behind the copy, whichever way they are narrowed)
