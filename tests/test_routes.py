@@ -118,6 +118,12 @@ def test_workspace_size_query_and_argument_checks():
     assert (L.ttq_workspace_bytes(C.byref(ok), 512, F32) >=                      # ... unless its rows must be rounded
             L.ttq_workspace_bytes(C.byref(small), 512, BF16) + 512 * 1024 * 2)
     assert L.ttq_workspace_bytes(C.byref(q), 0, BF16) == 0
+    # two to four rows decode without a workspace, except fp32 ones, which may take the few-row kernel over a scaled
+    # fp16 copy (the copy and a factor per row)
+    for m in (2, 3, 4):
+        assert L.ttq_workspace_bytes(C.byref(q), m, BF16) == 0 and L.ttq_workspace_bytes(C.byref(q), m, F16) == 0
+        assert L.ttq_workspace_bytes(C.byref(q), m, F32) >= m * 14336 * 2 + 4 * m
+    assert L.ttq_workspace_bytes(C.byref(q), 1, F32) == 0
     assert L.ttq_workspace_bytes(None, 1, BF16) == _lib.ERR_NULL
     assert L.ttq_workspace_bytes(C.byref(q), 1, 5) == _lib.ERR_DTYPE
     t = QLinearStruct(format=EXL3, n_out=4096, n_in=4096, bits=3, codebook=_lib.CB_MCG)
